@@ -1,0 +1,19 @@
+"""Shared pytest configuration.
+
+``gpu``-marked tests need a real MI355X and the built HIP library; everything
+else runs on the CPU (oracle against golden vectors, host logic, symbol
+export checks).
+"""
+
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
