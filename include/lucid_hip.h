@@ -1,0 +1,138 @@
+/*
+ * lucid_hip.h - C ABI of the MI355X (gfx950) backend for Lucid's int8
+ * quantized-inference path.
+ *
+ * The library is the drop-in for the part of Lucid's backend seam
+ * (lucid/_C/backend/IBackend.h:226-2239, selected through
+ * lucid/_C/backend/Dispatcher.h:90-94) that lucid.quantization and
+ * lucid.nn.quantized reach.  Lucid composes quantize / dequantize /
+ * fake_quantize out of five to seven elementwise virtuals and runs quantized
+ * Linear / Conv2d as dequantize + float GEMM + fake_quantize; this ABI exposes
+ * each of those composites as ONE fused entry point instead, which is what a
+ * HIP backend registered beside CpuBackend (CpuBackend.h:13835-13842) and
+ * GpuBackend (GpuBackend.h:7782-7787) would bind.
+ *
+ * Conventions
+ *   - every function returns an lq_status (0 = ok); lq_last_error() returns the
+ *     thread-local message of the last failure.  Status values mirror Lucid's
+ *     exception family (lucid/_C/core/Error.h:63-495).
+ *   - all tensor pointers are DEVICE pointers to contiguous row-major data
+ *     unless a parameter is documented as host memory.
+ *   - lq_dtype values equal Lucid's Dtype enum order (lucid/_C/core/Dtype.h).
+ *   - a tensor is described around its channel axis as [outer][C][inner]
+ *     (the broadcast of lucid/quantization/_functional.py:45-54); per-tensor
+ *     parameters use C = 1.
+ *   - launches are asynchronous on `stream` (a hipStream_t; NULL = the default
+ *     stream).  lq_sync / lq_d2h synchronise.
+ *   - reductions and the split-K GEMM use a per-device workspace owned by the
+ *     library; calls that overlap on one device on different streams race on it.
+ */
+#ifndef LUCID_HIP_H
+#define LUCID_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LQ_VERSION 1
+
+typedef enum {
+    LQ_OK = 0,
+    LQ_ERR_VALUE = 1,            /* ValueError: bad argument value            */
+    LQ_ERR_SHAPE = 2,            /* ShapeMismatch      (Error.h)              */
+    LQ_ERR_DTYPE = 3,            /* DtypeMismatch                             */
+    LQ_ERR_DEVICE = 4,           /* DeviceMismatch                            */
+    LQ_ERR_OOM = 5,              /* OutOfMemory                               */
+    LQ_ERR_GPU_NOT_AVAILABLE = 6,/* GpuNotAvailable                           */
+    LQ_ERR_NOT_IMPLEMENTED = 7,  /* NotImplementedError                       */
+    LQ_ERR_INTERNAL = 8          /* LucidError (any other HIP failure)        */
+} lq_status;
+
+/* lucid/_C/core/Dtype.h enum order */
+typedef enum {
+    LQ_BOOL = 0, LQ_I8 = 1, LQ_I16 = 2, LQ_I32 = 3, LQ_I64 = 4,
+    LQ_F16 = 5, LQ_F32 = 6, LQ_F64 = 7, LQ_C64 = 8, LQ_BF16 = 9, LQ_C128 = 10
+} lq_dtype;
+
+typedef void* lq_stream; /* hipStream_t */
+typedef void* lq_event;  /* hipEvent_t  */
+
+/* ------------------------------------------------------------------ runtime */
+/* Storage / transfer: IBackend::from_cpu (IBackend.h:259), to_cpu (:1370),
+ * and the allocator (lucid/_C/core/Allocator.h). */
+int lq_version(void);
+const char* lq_last_error(void);
+int lq_device_count(int* count);
+int lq_init(int device);
+int lq_device_name(char* buf, size_t buflen);
+int lq_alloc(void** ptr, size_t nbytes);
+int lq_free(void* ptr);
+int lq_h2d(void* dst_dev, const void* src_host, size_t nbytes, lq_stream stream);
+int lq_d2h(void* dst_host, const void* src_dev, size_t nbytes, lq_stream stream);
+int lq_d2d(void* dst_dev, const void* src_dev, size_t nbytes, lq_stream stream);
+int lq_fill_bytes(void* dst_dev, int value, size_t nbytes, lq_stream stream);
+int lq_sync(lq_stream stream);
+int lq_stream_create(lq_stream* stream);
+int lq_stream_destroy(lq_stream stream);
+int lq_event_create(lq_event* ev);
+int lq_event_destroy(lq_event ev);
+int lq_event_record(lq_event ev, lq_stream stream);
+int lq_event_sync(lq_event ev);
+int lq_event_elapsed_ms(lq_event start, lq_event stop, float* ms);
+
+/* Op registry: OpSchema{name, version, deterministic}
+ * (lucid/_C/core/OpSchema.h, OpRegistry.h:55,158-164). */
+int lq_op_count(void);
+int lq_op_info(int index, const char** name, int* version, int* deterministic);
+
+/* Synthetic-data helper for benchmarks: fills x[n] with N(0,1) samples from a
+ * counter-based generator; a fraction `outlier_prob` of them is multiplied by
+ * `outlier_gain`.  No counterpart in Lucid (its RNG is off this path). */
+int lq_fill_normal(float* x, size_t n, uint64_t seed, float outlier_prob, float outlier_gain,
+                   lq_stream stream);
+int lq_fill_uniform_i8(int8_t* x, size_t n, uint64_t seed, int lo, int hi, lq_stream stream);
+/* Plain device copy kernel (n bytes, 16-byte vectors): the calibration
+ * workload for hardware-counter scaling. */
+int lq_copy_kernel(void* dst, const void* src, size_t nbytes, lq_stream stream);
+
+/* ------------------------------------------------------------ quantize family */
+/* min and max over everything but the channel axis, NaN-propagating.
+ * Replaces reduce_min/reduce_max (IBackend.h:689-692; CpuBackend.h:12012,
+ * Reduce.cpp:87-125) as used by MinMaxObserver / PerChannelMinMaxObserver
+ * (lucid/quantization/observer.py:363-375,634-653) and nnqd.Linear
+ * (lucid/nn/quantized/dynamic/linear.py:87-89).  mn, mx: device f32[C]. */
+int lq_minmax(const float* x, size_t outer, size_t C, size_t inner, float* mn, float* mx,
+              lq_stream stream);
+
+/* calculate_qparams (lucid/quantization/_qparams.py:190-215) over C channels,
+ * entirely on the device.  scale, zp: device f32[C]. */
+int lq_calc_qparams(const float* mn, const float* mx, size_t C, int symmetric, int qmin, int qmax,
+                    int is_signed, float eps, float* scale, float* zp, lq_stream stream);
+
+/* quantize (lucid/quantization/_functional.py:164-182):
+ *   code = clip(rint(x / s) + z, qmin, qmax), stored as q_dtype (LQ_I8 or
+ *   LQ_I16) after adding code_offset (0 = Lucid's storage; -128 keeps a quint8
+ *   code in an int8 for the signed MFMA operand).
+ * scale, zp: f32[C]; device memory, or host memory when qparams_on_host != 0
+ * (C must be 1 then: Lucid's Python-float scale). */
+int lq_quantize(const float* x, void* q, int q_dtype, int code_offset, size_t outer, size_t C,
+                size_t inner, const float* scale, const float* zp, int qparams_on_host, int qmin,
+                int qmax, lq_stream stream);
+
+/* dequantize (_functional.py:269-281): out = (f32(code) - z) * s. */
+int lq_dequantize(const void* q, int q_dtype, int code_offset, float* out, size_t outer, size_t C,
+                  size_t inner, const float* scale, const float* zp, int qparams_on_host,
+                  lq_stream stream);
+
+/* fake_quantize forward (_functional.py:299-313): (clip(rint(x/s)+z) - z) * s. */
+int lq_fake_quantize(const float* x, float* out, size_t outer, size_t C, size_t inner,
+                     const float* scale, const float* zp, int qparams_on_host, int qmin, int qmax,
+                     lq_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LUCID_HIP_H */

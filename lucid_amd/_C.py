@@ -1,0 +1,179 @@
+"""ctypes binding of ``liblucid_hip.so`` - the only crossing point between the
+Python host code and HIP.
+
+Plays the role of Lucid's pybind11 boundary (``lucid/_C/bindings/bind.cpp``):
+one thin layer, no tensor logic.  Status codes are turned into exception
+classes named after Lucid's own (``lucid/_C/core/Error.h:63-495``,
+``lucid/_C/bindings/bind_errors.cpp``).
+
+There is no CPU fallback: if the library is missing or no gfx950 device is
+visible, loading / initialising raises.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "liblucid_hip.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "lucid_hip.h")
+
+
+# ---------------------------------------------------------------- errors
+class LucidError(RuntimeError):
+    """Base of every error raised by the backend."""
+
+
+class OutOfMemory(LucidError):
+    pass
+
+
+class ShapeMismatch(LucidError):
+    pass
+
+
+class DtypeMismatch(LucidError):
+    pass
+
+
+class DeviceMismatch(LucidError):
+    pass
+
+
+class GpuNotAvailable(LucidError):
+    pass
+
+
+_STATUS_TO_EXC = {
+    1: ValueError,
+    2: ShapeMismatch,
+    3: DtypeMismatch,
+    4: DeviceMismatch,
+    5: OutOfMemory,
+    6: GpuNotAvailable,
+    7: NotImplementedError,
+    8: LucidError,
+}
+
+# lucid/_C/core/Dtype.h enum order
+BOOL, I8, I16, I32, I64, F16, F32, F64, C64, BF16, C128 = range(11)
+
+OUT_ACC_I32, OUT_F32, OUT_F16, OUT_REQUANT_I8, OUT_FAKEQUANT_F32 = range(5)
+
+_vp, _sz, _i, _f, _u64 = C.c_void_p, C.c_size_t, C.c_int, C.c_float, C.c_uint64
+
+# name -> argtypes; every function returns int status unless listed in _RESTYPE
+_SIGNATURES = {
+    "lq_version": [],
+    "lq_last_error": [],
+    "lq_device_count": [C.POINTER(_i)],
+    "lq_init": [_i],
+    "lq_device_name": [C.c_char_p, _sz],
+    "lq_alloc": [C.POINTER(_vp), _sz],
+    "lq_free": [_vp],
+    "lq_h2d": [_vp, _vp, _sz, _vp],
+    "lq_d2h": [_vp, _vp, _sz, _vp],
+    "lq_d2d": [_vp, _vp, _sz, _vp],
+    "lq_fill_bytes": [_vp, _i, _sz, _vp],
+    "lq_sync": [_vp],
+    "lq_stream_create": [C.POINTER(_vp)],
+    "lq_stream_destroy": [_vp],
+    "lq_event_create": [C.POINTER(_vp)],
+    "lq_event_destroy": [_vp],
+    "lq_event_record": [_vp, _vp],
+    "lq_event_sync": [_vp],
+    "lq_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
+    "lq_op_count": [],
+    "lq_op_info": [_i, C.POINTER(C.c_char_p), C.POINTER(_i), C.POINTER(_i)],
+    "lq_fill_normal": [_vp, _sz, _u64, _f, _f, _vp],
+    "lq_fill_uniform_i8": [_vp, _sz, _u64, _i, _i, _vp],
+    "lq_copy_kernel": [_vp, _vp, _sz, _vp],
+    "lq_minmax": [_vp, _sz, _sz, _sz, _vp, _vp, _vp],
+    "lq_calc_qparams": [_vp, _vp, _sz, _i, _i, _i, _i, _f, _vp, _vp, _vp],
+    "lq_quantize": [_vp, _vp, _i, _i, _sz, _sz, _sz, _vp, _vp, _i, _i, _i, _vp],
+    "lq_dequantize": [_vp, _i, _i, _vp, _sz, _sz, _sz, _vp, _vp, _i, _vp],
+    "lq_fake_quantize": [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _i, _i, _i, _vp],
+}
+_RESTYPE = {"lq_last_error": C.c_char_p}
+_NO_STATUS = {"lq_version", "lq_last_error", "lq_op_count"}
+
+_lib = None
+_initialised_device = None
+
+
+def load() -> C.CDLL:
+    """dlopen the library and declare every signature.  Does not touch the GPU."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise GpuNotAvailable(
+                f"{LIB_PATH} is missing: build it with `make -C lucid_amd/csrc` "
+                "(hipcc --offload-arch=gfx950).  There is no CPU fallback."
+            )
+        lib = C.CDLL(LIB_PATH)
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+            fn.argtypes = argtypes
+            fn.restype = _RESTYPE.get(name, C.c_int)
+        _lib = lib
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        msg = load().lq_last_error().decode("utf-8", "replace")
+        raise _STATUS_TO_EXC.get(status, LucidError)(msg)
+
+
+def call(name: str, *args):
+    """Call an ABI function and raise on a non-zero status."""
+    fn = getattr(load(), name)
+    rc = fn(*args)
+    if name not in _NO_STATUS:
+        check(rc)
+    return rc
+
+
+def init(device: int = 0) -> None:
+    """Select the device and allocate the library workspace (idempotent)."""
+    global _initialised_device
+    if _initialised_device != device:
+        call("lq_init", device)
+        _initialised_device = device
+
+
+def is_available() -> bool:
+    """True when the library loads and sees at least one device."""
+    try:
+        n = C.c_int(0)
+        rc = load().lq_device_count(C.byref(n))
+        return rc == 0 and n.value > 0
+    except (OSError, LucidError):
+        return False
+
+
+def device_name() -> str:
+    buf = C.create_string_buffer(256)
+    call("lq_device_name", buf, 256)
+    return buf.value.decode()
+
+
+def op_registry() -> list[tuple[str, int, bool]]:
+    """``(name, version, deterministic)`` rows, as ``op_registry_all`` in Lucid
+    (``lucid/_C/bindings/bind_op_registry.cpp``)."""
+    out = []
+    for i in range(load().lq_op_count()):
+        name, ver, det = C.c_char_p(), C.c_int(), C.c_int()
+        call("lq_op_info", i, C.byref(name), C.byref(ver), C.byref(det))
+        out.append((name.value.decode(), ver.value, bool(det.value)))
+    return out
+
+
+def declared_symbols() -> list[str]:
+    """Function names declared in ``include/lucid_hip.h``."""
+    import re
+
+    text = open(HEADER_PATH).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lq_[a-z0-9_]+)\s*\(", text)))

@@ -1,0 +1,229 @@
+"""Minimal tensor handle for the ``hip`` device.
+
+Lucid's ``Tensor`` wraps a C++ ``TensorImpl`` whose ``Storage`` is a variant of
+CPU / GPU / shared storage (``lucid/_C/core/Storage.h:334``).  This package
+adds a third storage kind - a HIP device allocation - and only what the
+quantized-inference path needs around it: shape, dtype, upload / download.
+
+A ``"cpu"`` tensor here is a host container (numpy array) used to stage data
+in and out; every compute entry point requires ``device == "hip"`` and raises
+``DeviceMismatch`` otherwise, so nothing ever computes on the host.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import weakref
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _C
+
+
+# ---------------------------------------------------------------- dtypes
+@dataclass(frozen=True)
+class dtype:
+    """Element type; ``code`` is Lucid's ``Dtype`` enum value (``core/Dtype.h``)."""
+
+    name: str
+    code: int
+    itemsize: int
+    np: object
+
+    def __repr__(self) -> str:
+        return f"lucid.{self.name}"
+
+
+bool_ = dtype("bool", _C.BOOL, 1, np.bool_)
+int8 = dtype("int8", _C.I8, 1, np.int8)
+int16 = dtype("int16", _C.I16, 2, np.int16)
+int32 = dtype("int32", _C.I32, 4, np.int32)
+int64 = dtype("int64", _C.I64, 8, np.int64)
+float16 = dtype("float16", _C.F16, 2, np.float16)
+float32 = dtype("float32", _C.F32, 4, np.float32)
+float64 = dtype("float64", _C.F64, 8, np.float64)
+
+_ALL = (bool_, int8, int16, int32, int64, float16, float32, float64)
+_BY_NP = {np.dtype(d.np): d for d in _ALL}
+_BY_NAME = {d.name: d for d in _ALL}
+
+
+def as_dtype(d) -> dtype:
+    if isinstance(d, dtype):
+        return d
+    if isinstance(d, str):
+        return _BY_NAME[d]
+    return _BY_NP[np.dtype(d)]
+
+
+# ---------------------------------------------------------------- devices
+# lucid/_device.py:21-22 knows "cpu" and "metal"; this backend adds "hip".
+_KNOWN_DEVICES = ("cpu", "hip")
+
+
+def _norm_device(device) -> str:
+    d = str(device).split(":")[0]
+    if d not in _KNOWN_DEVICES:
+        raise ValueError(f"unknown device {device!r}; expected one of {_KNOWN_DEVICES}")
+    return d
+
+
+class DeviceBuffer:
+    """Owns one ``lq_alloc`` allocation; freed when the last reference dies."""
+
+    __slots__ = ("ptr", "nbytes", "_fin", "__weakref__")
+
+    def __init__(self, nbytes: int) -> None:
+        _C.init()
+        p = C.c_void_p()
+        _C.call("lq_alloc", C.byref(p), int(nbytes))
+        self.ptr = p.value
+        self.nbytes = int(nbytes)
+        self._fin = weakref.finalize(self, _free, self.ptr)
+
+
+def _free(ptr) -> None:
+    try:
+        _C.load().lq_free(ptr)
+    except Exception:  # interpreter shutdown
+        pass
+
+
+class Tensor:
+    """Contiguous row-major tensor on ``"hip"`` (device memory) or ``"cpu"``
+    (host staging)."""
+
+    __slots__ = ("shape", "dtype", "device", "_buf", "_host", "_offset", "_grid", "__weakref__")
+
+    def __init__(self, shape, dt, device, buf=None, host=None, offset=0) -> None:
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = as_dtype(dt)
+        self.device = _norm_device(device)
+        self._buf = buf
+        self._host = host
+        self._offset = int(offset)
+        self._grid = None  # set by ops whose result lies on a quantization grid
+
+    # -- construction
+    @staticmethod
+    def empty(shape, dt=float32, device="hip") -> "Tensor":
+        dt = as_dtype(dt)
+        shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+        n = int(np.prod(shape, dtype=np.int64))
+        if _norm_device(device) == "cpu":
+            return Tensor(shape, dt, "cpu", host=np.empty(shape, dt.np))
+        return Tensor(shape, dt, "hip", buf=DeviceBuffer(n * dt.itemsize))
+
+    @staticmethod
+    def from_numpy(a, device="hip") -> "Tensor":
+        a = np.ascontiguousarray(a)
+        dt = as_dtype(a.dtype)
+        if _norm_device(device) == "cpu":
+            return Tensor(a.shape, dt, "cpu", host=a)
+        t = Tensor.empty(a.shape, dt, "hip")
+        _C.call("lq_h2d", t.data_ptr, a.ctypes.data, a.nbytes, None)
+        return t
+
+    # -- properties
+    @property
+    def ndim(self) -> int:
+        return len(self.shape)
+
+    @property
+    def numel(self) -> int:
+        return int(np.prod(self.shape, dtype=np.int64))
+
+    @property
+    def nbytes(self) -> int:
+        return self.numel * self.dtype.itemsize
+
+    @property
+    def data_ptr(self) -> int:
+        if self.device != "hip":
+            raise _C.DeviceMismatch("data_ptr: tensor is not on the hip device")
+        return self._buf.ptr + self._offset
+
+    @property
+    def is_hip(self) -> bool:
+        return self.device == "hip"
+
+    def size(self, dim=None):
+        return self.shape if dim is None else self.shape[dim]
+
+    def __len__(self) -> int:
+        return self.shape[0]
+
+    def __repr__(self) -> str:
+        return f"Tensor(shape={self.shape}, dtype={self.dtype.name}, device='{self.device}')"
+
+    # -- movement
+    def numpy(self) -> np.ndarray:
+        if self.device == "cpu":
+            return self._host
+        out = np.empty(self.shape, self.dtype.np)
+        if out.nbytes:
+            _C.call("lq_d2h", out.ctypes.data, self.data_ptr, out.nbytes, None)
+        return out
+
+    def to(self, target) -> "Tensor":
+        """``.to("hip")`` / ``.to("cpu")`` (``lucid/_tensor/_to.py:125-199``).
+        Dtype conversion is not part of this path and is rejected."""
+        if isinstance(target, dtype):
+            if target == self.dtype:
+                return self
+            raise NotImplementedError("dtype conversion is outside the hip quantized path")
+        dev = _norm_device(target)
+        if dev == self.device:
+            return self
+        if dev == "hip":
+            t = Tensor.from_numpy(self._host, "hip")
+        else:
+            t = Tensor.from_numpy(self.numpy(), "cpu")
+        return t
+
+    def cpu(self) -> "Tensor":
+        return self.to("cpu")
+
+    def item(self):
+        if self.numel != 1:
+            raise ValueError("item() needs a one-element tensor")
+        return self.numpy().reshape(()).item()
+
+    def tolist(self):
+        return self.numpy().tolist()
+
+    def reshape(self, *shape) -> "Tensor":
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
+            shape = tuple(shape[0])
+        shape = list(shape)
+        if -1 in shape:
+            known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
+            shape[shape.index(-1)] = self.numel // max(known, 1)
+        if int(np.prod(shape, dtype=np.int64)) != self.numel:
+            raise _C.ShapeMismatch(f"cannot reshape {self.shape} to {tuple(shape)}")
+        if self.device == "cpu":
+            return Tensor(shape, self.dtype, "cpu", host=self._host.reshape(shape))
+        return Tensor(shape, self.dtype, "hip", buf=self._buf, offset=self._offset)
+
+    def detach(self) -> "Tensor":
+        return self
+
+
+def tensor(data, dtype=None, device="cpu") -> Tensor:
+    """``lucid.tensor``: Python floats become float32, ints int64 - unless
+    ``dtype`` says otherwise."""
+    a = np.asarray(data)
+    if dtype is not None:
+        a = a.astype(as_dtype(dtype).np)
+    elif a.dtype == np.float64:
+        a = a.astype(np.float32)
+    return Tensor.from_numpy(a, device)
+
+
+def is_floating_point(t: Tensor) -> bool:
+    return t.dtype in (float16, float32, float64)
+
+
+def synchronize() -> None:
+    _C.call("lq_sync", None)

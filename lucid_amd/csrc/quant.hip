@@ -1,0 +1,557 @@
+// quantize / dequantize / fake_quantize / min-max / calculate_qparams for
+// gfx950.  All of them are HBM-bound: the kernels issue 128-bit loads that a
+// wavefront covers contiguously, keep several loads in flight per lane, and
+// do the arithmetic in the order Lucid's CPU path does it
+// (lucid/quantization/_functional.py:180, 281, 311-313): IEEE division,
+// round-half-even, add zero point, clamp, cast.  No reciprocal, no FMA.
+#include "common.hpp"
+
+using namespace lq;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// ---------------------------------------------------------------- element math
+// clip keeps NaN (CpuBackend.h:6880-6891); the float->int cast maps NaN to 0.
+__device__ __forceinline__ float q_core(float x, float s, float z, float lo, float hi) {
+    float t = x / s;
+    float r = __builtin_rintf(t);
+    float u = r + z;
+    u = (u < lo) ? lo : ((u > hi) ? hi : u);
+    return u;
+}
+
+__device__ __forceinline__ int to_code(float c) { return (c != c) ? 0 : int(c); }
+
+struct alignas(4) Code8x4 {
+    int8_t v[4];
+};
+struct alignas(8) Code16x4 {
+    int16_t v[4];
+};
+
+template <typename CodeT>
+struct CodeVec;
+template <>
+struct CodeVec<int8_t> {
+    using type = Code8x4;
+};
+template <>
+struct CodeVec<int16_t> {
+    using type = Code16x4;
+};
+
+// ---------------------------------------------------------------- segment ops
+// Each op works on groups of four consecutive elements ("quads") that share
+// one (scale, zero_point).
+template <typename CodeT>
+struct QuantizeOp {
+    using In = float4;
+    using Vec = typename CodeVec<CodeT>::type;
+    const float4* __restrict__ x;
+    Vec* __restrict__ q;
+    float lo, hi;
+    int off;
+    __device__ __forceinline__ In load(size_t i) const { return x[i]; }
+    __device__ __forceinline__ void store(size_t i, In v, float s, float z) const {
+        Vec o;
+        o.v[0] = CodeT(to_code(q_core(v.x, s, z, lo, hi)) + off);
+        o.v[1] = CodeT(to_code(q_core(v.y, s, z, lo, hi)) + off);
+        o.v[2] = CodeT(to_code(q_core(v.z, s, z, lo, hi)) + off);
+        o.v[3] = CodeT(to_code(q_core(v.w, s, z, lo, hi)) + off);
+        q[i] = o;
+    }
+    // scalar tail / generic path
+    __device__ __forceinline__ void scalar(size_t e, float s, float z) const {
+        const float* xs = reinterpret_cast<const float*>(x);
+        CodeT* qs = reinterpret_cast<CodeT*>(q);
+        qs[e] = CodeT(to_code(q_core(xs[e], s, z, lo, hi)) + off);
+    }
+};
+
+template <typename CodeT>
+struct DequantizeOp {
+    using Vec = typename CodeVec<CodeT>::type;
+    using In = Vec;
+    const Vec* __restrict__ q;
+    float4* __restrict__ out;
+    int off;
+    __device__ __forceinline__ In load(size_t i) const { return q[i]; }
+    __device__ __forceinline__ void store(size_t i, In v, float s, float z) const {
+        float4 o;
+        o.x = (float(int(v.v[0]) - off) - z) * s;
+        o.y = (float(int(v.v[1]) - off) - z) * s;
+        o.z = (float(int(v.v[2]) - off) - z) * s;
+        o.w = (float(int(v.v[3]) - off) - z) * s;
+        out[i] = o;
+    }
+    __device__ __forceinline__ void scalar(size_t e, float s, float z) const {
+        const CodeT* qs = reinterpret_cast<const CodeT*>(q);
+        float* os = reinterpret_cast<float*>(out);
+        os[e] = (float(int(qs[e]) - off) - z) * s;
+    }
+};
+
+struct FakeQuantizeOp {
+    using In = float4;
+    const float4* __restrict__ x;
+    float4* __restrict__ out;
+    float lo, hi;
+    __device__ __forceinline__ In load(size_t i) const { return x[i]; }
+    __device__ __forceinline__ void store(size_t i, In v, float s, float z) const {
+        float4 o;
+        o.x = (q_core(v.x, s, z, lo, hi) - z) * s;
+        o.y = (q_core(v.y, s, z, lo, hi) - z) * s;
+        o.z = (q_core(v.z, s, z, lo, hi) - z) * s;
+        o.w = (q_core(v.w, s, z, lo, hi) - z) * s;
+        out[i] = o;
+    }
+    __device__ __forceinline__ void scalar(size_t e, float s, float z) const {
+        const float* xs = reinterpret_cast<const float*>(x);
+        float* os = reinterpret_cast<float*>(out);
+        os[e] = (q_core(xs[e], s, z, lo, hi) - z) * s;
+    }
+};
+
+struct QParams {
+    const float* scale;  // device, length C, or nullptr -> use the by-value pair
+    const float* zp;
+    float s_host, z_host;
+};
+
+// One block = one chunk of U*256 quads inside one [outer][C] segment, so the
+// (scale, zero_point) pair is uniform across the block.  All U loads are
+// issued before the first store.
+template <typename Op, int U>
+__global__ __launch_bounds__(kThreads) void seg_kernel(Op op, size_t inner4,
+                                                       unsigned chunks_per_seg, size_t C,
+                                                       QParams qp) {
+    const size_t seg = blockIdx.x / chunks_per_seg;
+    const unsigned chunk = blockIdx.x - unsigned(seg * chunks_per_seg);
+    float s, z;
+    if (qp.scale) {
+        const size_t c = seg % C;
+        s = qp.scale[c];
+        z = qp.zp[c];
+    } else {
+        s = qp.s_host;
+        z = qp.z_host;
+    }
+    const size_t base = seg * inner4;
+    const size_t i0 = size_t(chunk) * (U * kThreads) + threadIdx.x;
+    typename Op::In v[U];
+    if (size_t(chunk + 1) * (U * kThreads) <= inner4) {  // whole chunk in range: no predicates
+#pragma unroll
+        for (int j = 0; j < U; ++j) v[j] = op.load(base + i0 + size_t(j) * kThreads);
+#pragma unroll
+        for (int j = 0; j < U; ++j) op.store(base + i0 + size_t(j) * kThreads, v[j], s, z);
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+        size_t i = i0 + size_t(j) * kThreads;
+        if (i < inner4) v[j] = op.load(base + i);
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+        size_t i = i0 + size_t(j) * kThreads;
+        if (i < inner4) op.store(base + i, v[j], s, z);
+    }
+}
+
+// Any shape, any alignment: one element per thread, channel looked up per
+// element.  Used for small or oddly shaped tensors (e.g. a 7x7x3 kernel).
+template <typename Op>
+__global__ __launch_bounds__(kThreads) void generic_kernel(Op op, size_t n, size_t C, size_t inner,
+                                                           QParams qp) {
+    size_t e = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t stride = size_t(gridDim.x) * kThreads;
+    for (; e < n; e += stride) {
+        float s, z;
+        if (qp.scale) {
+            const size_t c = (e / inner) % C;
+            s = qp.scale[c];
+            z = qp.zp[c];
+        } else {
+            s = qp.s_host;
+            z = qp.z_host;
+        }
+        op.scalar(e, s, z);
+    }
+}
+
+template <typename Op>
+int launch_elementwise(Op op, size_t outer, size_t C, size_t inner, QParams qp, bool vec_ok,
+                       hipStream_t st, const char* name) {
+    const size_t n = outer * C * inner;
+    if (n == 0) return LQ_OK;
+    const size_t segs = outer * C;
+    if (vec_ok && inner % 4 == 0 && inner >= 256) {
+        const size_t inner4 = inner / 4;
+        int U = inner4 >= 8 * kThreads ? 8 : (inner4 >= 4 * kThreads ? 4 : (inner4 >= 2 * kThreads ? 2 : 1));
+        const size_t per_block = size_t(U) * kThreads;
+        const size_t chunks = (inner4 + per_block - 1) / per_block;
+        const size_t blocks = chunks * segs;
+        LQ_REQUIRE(blocks <= 0x7fffffffull && chunks <= 0xffffffffull, LQ_ERR_SHAPE,
+                   "%s: tensor too large for one launch (%zu blocks)", name, blocks);
+        dim3 grid{unsigned(blocks)}, block{kThreads};
+        switch (U) {
+        case 8: hipLaunchKernelGGL((seg_kernel<Op, 8>), grid, block, 0, st, op, inner4, unsigned(chunks), C, qp); break;
+        case 4: hipLaunchKernelGGL((seg_kernel<Op, 4>), grid, block, 0, st, op, inner4, unsigned(chunks), C, qp); break;
+        case 2: hipLaunchKernelGGL((seg_kernel<Op, 2>), grid, block, 0, st, op, inner4, unsigned(chunks), C, qp); break;
+        default: hipLaunchKernelGGL((seg_kernel<Op, 1>), grid, block, 0, st, op, inner4, unsigned(chunks), C, qp); break;
+        }
+    } else {
+        size_t blocks = (n + kThreads - 1) / kThreads;
+        if (blocks > 262144) blocks = 262144;
+        hipLaunchKernelGGL((generic_kernel<Op>), dim3(unsigned(blocks)), dim3(kThreads), 0, st, op, n, C,
+                           inner, qp);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, name);
+    return LQ_OK;
+}
+
+int make_qparams(const float* scale, const float* zp, int on_host, size_t C, QParams* qp,
+                 const char* name) {
+    LQ_REQUIRE(scale && zp, LQ_ERR_VALUE, "%s: scale / zero_point is NULL", name);
+    if (on_host) {
+        LQ_REQUIRE(C == 1, LQ_ERR_VALUE, "%s: host qparams are per-tensor only (C = %zu)", name, C);
+        *qp = QParams{nullptr, nullptr, scale[0], zp[0]};
+    } else {
+        *qp = QParams{scale, zp, 0.f, 0.f};
+    }
+    return LQ_OK;
+}
+
+// ---------------------------------------------------------------- min / max
+struct MinMax {
+    float lo, hi;
+    int nan;
+};
+
+__device__ __forceinline__ void mm_update(MinMax& m, float v) {
+    m.nan |= (v != v);
+    m.lo = fminf(m.lo, v);  // fminf/fmaxf drop NaN; the flag carries it
+    m.hi = fmaxf(m.hi, v);
+}
+
+__device__ __forceinline__ MinMax mm_block_reduce(MinMax m) {
+    // wavefront (64 lanes) butterfly, then across the block's waves via LDS
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        m.lo = fminf(m.lo, __shfl_xor(m.lo, d, 64));
+        m.hi = fmaxf(m.hi, __shfl_xor(m.hi, d, 64));
+        m.nan |= __shfl_xor(m.nan, d, 64);
+    }
+    __shared__ float s_lo[kThreads / 64], s_hi[kThreads / 64];
+    __shared__ int s_nan[kThreads / 64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nwaves = (blockDim.x + 63) >> 6;
+    if (lane == 0) {
+        s_lo[wave] = m.lo;
+        s_hi[wave] = m.hi;
+        s_nan[wave] = m.nan;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < nwaves; ++w) {
+            m.lo = fminf(m.lo, s_lo[w]);
+            m.hi = fmaxf(m.hi, s_hi[w]);
+            m.nan |= s_nan[w];
+        }
+    }
+    return m;
+}
+
+__device__ __forceinline__ void mm_write(MinMax m, float* mn, float* mx, size_t idx) {
+    const float qnan = __builtin_nanf("");
+    mn[idx] = m.nan ? qnan : m.lo;
+    mx[idx] = m.nan ? qnan : m.hi;
+}
+
+// Channel elements lie in `outer` contiguous runs of `inner`.  Block
+// (c, split) scans its slice of every run.  Partials are laid out
+// [split][c]; with splits == 1 they are the final answer.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void minmax_seg_kernel(const float* __restrict__ x,
+                                                              size_t outer, size_t C, size_t inner,
+                                                              unsigned splits, float* pmin,
+                                                              float* pmax) {
+    const size_t c = blockIdx.x / splits;
+    const unsigned sp = blockIdx.x - unsigned(c * splits);
+    MinMax m{__builtin_inff(), -__builtin_inff(), 0};
+    if (VEC) {
+        const size_t inner4 = inner / 4;
+        const size_t per = (inner4 + splits - 1) / splits;
+        const size_t lo4 = size_t(sp) * per;
+        const size_t hi4 = lo4 + per < inner4 ? lo4 + per : inner4;
+        for (size_t o = 0; o < outer; ++o) {
+            const float4* p = reinterpret_cast<const float4*>(x + (o * C + c) * inner);
+            size_t i = lo4 + threadIdx.x;
+            // four independent loads in flight per lane
+            for (; i + 3 * kThreads < hi4; i += 4 * kThreads) {
+                float4 a = p[i], b = p[i + kThreads], d = p[i + 2 * kThreads], e = p[i + 3 * kThreads];
+                mm_update(m, a.x); mm_update(m, a.y); mm_update(m, a.z); mm_update(m, a.w);
+                mm_update(m, b.x); mm_update(m, b.y); mm_update(m, b.z); mm_update(m, b.w);
+                mm_update(m, d.x); mm_update(m, d.y); mm_update(m, d.z); mm_update(m, d.w);
+                mm_update(m, e.x); mm_update(m, e.y); mm_update(m, e.z); mm_update(m, e.w);
+            }
+            for (; i < hi4; i += kThreads) {
+                float4 a = p[i];
+                mm_update(m, a.x); mm_update(m, a.y); mm_update(m, a.z); mm_update(m, a.w);
+            }
+        }
+    } else {
+        const size_t per = (inner + splits - 1) / splits;
+        const size_t lo = size_t(sp) * per;
+        const size_t hi = lo + per < inner ? lo + per : inner;
+        for (size_t o = 0; o < outer; ++o) {
+            const float* p = x + (o * C + c) * inner;
+            for (size_t i = lo + threadIdx.x; i < hi; i += kThreads) mm_update(m, p[i]);
+        }
+    }
+    m = mm_block_reduce(m);
+    if (threadIdx.x == 0) mm_write(m, pmin, pmax, size_t(sp) * C + c);
+}
+
+// Short runs (inner < 64, e.g. a channel-last tensor): view x as
+// [outer][C*inner]; a thread owns one column and walks down a slice of rows,
+// so a wavefront reads contiguous memory.  Partials [split][C*inner].
+__global__ __launch_bounds__(kThreads) void minmax_col_kernel(const float* __restrict__ x,
+                                                              size_t outer, size_t cols,
+                                                              unsigned splits, float* pmin,
+                                                              float* pmax) {
+    const size_t col = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    const unsigned sp = blockIdx.y;
+    if (col >= cols) return;
+    const size_t per = (outer + splits - 1) / splits;
+    const size_t lo = size_t(sp) * per;
+    const size_t hi = lo + per < outer ? lo + per : outer;
+    MinMax m{__builtin_inff(), -__builtin_inff(), 0};
+    for (size_t r = lo; r < hi; ++r) mm_update(m, x[r * cols + col]);
+    mm_write(m, pmin, pmax, size_t(sp) * cols + col);
+}
+
+// Folds partials [groups][C][inner_cols] into mn[C], mx[C]; one wavefront
+// per channel.
+__global__ __launch_bounds__(64) void minmax_finalize_kernel(const float* __restrict__ pmin,
+                                                             const float* __restrict__ pmax,
+                                                             size_t C, unsigned groups,
+                                                             unsigned inner_cols, float* mn,
+                                                             float* mx) {
+    const size_t c = blockIdx.x;
+    MinMax m{__builtin_inff(), -__builtin_inff(), 0};
+    const size_t per_c = size_t(groups) * inner_cols;
+    for (size_t t = threadIdx.x; t < per_c; t += 64) {
+        const size_t g = t / inner_cols, i = t - g * inner_cols;
+        const size_t idx = (g * C + c) * inner_cols + i;
+        float a = pmin[idx], b = pmax[idx];
+        m.nan |= (a != a) | (b != b);
+        m.lo = fminf(m.lo, a);
+        m.hi = fmaxf(m.hi, b);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        m.lo = fminf(m.lo, __shfl_xor(m.lo, d, 64));
+        m.hi = fmaxf(m.hi, __shfl_xor(m.hi, d, 64));
+        m.nan |= __shfl_xor(m.nan, d, 64);
+    }
+    if (threadIdx.x == 0) mm_write(m, mn, mx, c);
+}
+
+__global__ void minmax_identity_kernel(float* mn, float* mx, size_t C) {
+    size_t c = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c < C) {
+        mn[c] = __builtin_inff();
+        mx[c] = -__builtin_inff();
+    }
+}
+
+// ---------------------------------------------------------------- qparams
+// vDSP_vmax / vDSP_vmin single precision propagate NaN (Vdsp.cpp:140-151).
+__device__ __forceinline__ float vmaxf(float a, float b) {
+    if (a != a || b != b) return __builtin_nanf("");
+    return a > b ? a : b;
+}
+__device__ __forceinline__ float vminf(float a, float b) {
+    if (a != a || b != b) return __builtin_nanf("");
+    return a < b ? a : b;
+}
+
+// lucid/quantization/_qparams.py:198-215, float32 throughout.
+__global__ void calc_qparams_kernel(const float* __restrict__ mn, const float* __restrict__ mx,
+                                    size_t C, int symmetric, int qmin, int qmax, int is_signed,
+                                    float eps, float half_range, float* scale, float* zp) {
+    size_t c = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    float lo = vminf(mn[c], 0.0f);
+    float hi = vmaxf(mx[c], 0.0f);
+    if (symmetric) {
+        float max_abs = vmaxf(fabsf(lo), fabsf(hi));
+        scale[c] = vmaxf(max_abs / half_range, eps);
+        zp[c] = is_signed ? 0.0f : float((qmax + qmin + 1) >> 1);
+    } else {
+        float s = vmaxf((hi - lo) / float(qmax - qmin), eps);
+        float z = float(qmin) - __builtin_rintf(lo / s);
+        float qlo = float(qmin), qhi = float(qmax);
+        z = (z < qlo) ? qlo : ((z > qhi) ? qhi : z);
+        scale[c] = s;
+        zp[c] = z;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int lq_minmax(const float* x, size_t outer, size_t C, size_t inner, float* mn, float* mx,
+              lq_stream stream) {
+    LQ_REQUIRE(mn && mx, LQ_ERR_VALUE, "minmax: output pointer is NULL");
+    LQ_REQUIRE(C >= 1, LQ_ERR_SHAPE, "minmax: C must be >= 1");
+    hipStream_t st = as_stream(stream);
+    const size_t per_channel = outer * inner;
+    if (per_channel == 0) {  // empty reduction: identities (Reduce.cpp:95,107)
+        hipLaunchKernelGGL(minmax_identity_kernel, dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, mn,
+                           mx, C);
+        LQ_CHECK_LAUNCH("minmax_identity");
+        return LQ_OK;
+    }
+    LQ_REQUIRE(x, LQ_ERR_VALUE, "minmax: x is NULL");
+    LQ_REQUIRE(C <= 0x3fffffffull, LQ_ERR_SHAPE, "minmax: too many channels (%zu)", C);
+
+    if (inner < 64 && C > 1) {
+        const size_t cols = C * inner;
+        // enough row slices to occupy the chip, at least 32 rows each
+        size_t col_blocks = (cols + kThreads - 1) / kThreads;
+        size_t splits = 2048 / col_blocks;
+        if (splits > outer / 32) splits = outer / 32;
+        if (splits < 1) splits = 1;
+        if (splits > 65535) splits = 65535;
+        void* ws = nullptr;
+        int rc = workspace(2 * splits * cols * sizeof(float), &ws);
+        if (rc) return rc;
+        float* pmin = static_cast<float*>(ws);
+        float* pmax = pmin + splits * cols;
+        hipLaunchKernelGGL(minmax_col_kernel, dim3(unsigned(col_blocks), unsigned(splits)),
+                           dim3(kThreads), 0, st, x, outer, cols, unsigned(splits), pmin, pmax);
+        LQ_CHECK_LAUNCH("minmax_col");
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(64), 0, st, pmin, pmax, C,
+                           unsigned(splits), unsigned(inner), mn, mx);
+        LQ_CHECK_LAUNCH("minmax_finalize");
+        return LQ_OK;
+    }
+
+    // contiguous runs: aim for ~2048 blocks, each slice at least 4096 elements
+    size_t splits = 1;
+    if (C < 2048) {
+        splits = 2048 / C;
+        size_t max_splits = inner / 4096;
+        if (splits > max_splits) splits = max_splits;
+        if (splits < 1) splits = 1;
+    }
+    const bool vec = (inner % 4 == 0) && aligned16(x);
+    float *pmin = mn, *pmax = mx;
+    if (splits > 1) {
+        void* ws = nullptr;
+        int rc = workspace(2 * splits * C * sizeof(float), &ws);
+        if (rc) return rc;
+        pmin = static_cast<float*>(ws);
+        pmax = pmin + splits * C;
+    }
+    dim3 grid{unsigned(C * splits)}, block{kThreads};
+    if (vec)
+        hipLaunchKernelGGL((minmax_seg_kernel<true>), grid, block, 0, st, x, outer, C, inner,
+                           unsigned(splits), pmin, pmax);
+    else
+        hipLaunchKernelGGL((minmax_seg_kernel<false>), grid, block, 0, st, x, outer, C, inner,
+                           unsigned(splits), pmin, pmax);
+    LQ_CHECK_LAUNCH("minmax_seg");
+    if (splits > 1) {
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(64), 0, st, pmin, pmax, C,
+                           unsigned(splits), 1u, mn, mx);
+        LQ_CHECK_LAUNCH("minmax_finalize");
+    }
+    return LQ_OK;
+}
+
+int lq_calc_qparams(const float* mn, const float* mx, size_t C, int symmetric, int qmin, int qmax,
+                    int is_signed, float eps, float* scale, float* zp, lq_stream stream) {
+    if (C == 0) return LQ_OK;
+    LQ_REQUIRE(mn && mx && scale && zp, LQ_ERR_VALUE, "calc_qparams: NULL pointer");
+    LQ_REQUIRE(qmax > qmin, LQ_ERR_VALUE, "calc_qparams: empty grid [%d,%d]", qmin, qmax);
+    // (quant_max - quant_min) / 2.0 is a Python float promoted to float32
+    const float half_range = float((double(qmax) - double(qmin)) / 2.0);
+    hipLaunchKernelGGL(calc_qparams_kernel, dim3(unsigned((C + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), mn, mx, C, symmetric, qmin, qmax, is_signed, eps, half_range,
+                       scale, zp);
+    LQ_CHECK_LAUNCH("calc_qparams");
+    return LQ_OK;
+}
+
+int lq_quantize(const float* x, void* q, int q_dtype, int code_offset, size_t outer, size_t C,
+                size_t inner, const float* scale, const float* zp, int qparams_on_host, int qmin,
+                int qmax, lq_stream stream) {
+    if (outer * C * inner == 0) return LQ_OK;
+    LQ_REQUIRE(x && q, LQ_ERR_VALUE, "quantize: NULL tensor pointer");
+    LQ_REQUIRE(q_dtype == LQ_I8 || q_dtype == LQ_I16, LQ_ERR_DTYPE,
+               "quantize: code storage must be int8 or int16 (got dtype %d)", q_dtype);
+    const int lim_lo = q_dtype == LQ_I8 ? -128 : -32768, lim_hi = q_dtype == LQ_I8 ? 127 : 32767;
+    LQ_REQUIRE(qmin <= qmax && qmin + code_offset >= lim_lo && qmax + code_offset <= lim_hi,
+               LQ_ERR_VALUE, "quantize: grid [%d,%d] + offset %d does not fit the code storage", qmin,
+               qmax, code_offset);
+    QParams qp;
+    int rc = make_qparams(scale, zp, qparams_on_host, C, &qp, "quantize");
+    if (rc) return rc;
+    const float lo = float(double(qmin)), hi = float(double(qmax));
+    if (q_dtype == LQ_I8) {
+        QuantizeOp<int8_t> op{reinterpret_cast<const float4*>(x), reinterpret_cast<Code8x4*>(q), lo, hi,
+                              code_offset};
+        return launch_elementwise(op, outer, C, inner, qp, aligned16(x) && aligned16(q),
+                                  as_stream(stream), "quantize");
+    }
+    QuantizeOp<int16_t> op{reinterpret_cast<const float4*>(x), reinterpret_cast<Code16x4*>(q), lo, hi,
+                           code_offset};
+    return launch_elementwise(op, outer, C, inner, qp, aligned16(x) && aligned16(q), as_stream(stream),
+                              "quantize");
+}
+
+int lq_dequantize(const void* q, int q_dtype, int code_offset, float* out, size_t outer, size_t C,
+                  size_t inner, const float* scale, const float* zp, int qparams_on_host,
+                  lq_stream stream) {
+    if (outer * C * inner == 0) return LQ_OK;
+    LQ_REQUIRE(q && out, LQ_ERR_VALUE, "dequantize: NULL tensor pointer");
+    LQ_REQUIRE(q_dtype == LQ_I8 || q_dtype == LQ_I16, LQ_ERR_DTYPE,
+               "dequantize: code storage must be int8 or int16 (got dtype %d)", q_dtype);
+    QParams qp;
+    int rc = make_qparams(scale, zp, qparams_on_host, C, &qp, "dequantize");
+    if (rc) return rc;
+    if (q_dtype == LQ_I8) {
+        DequantizeOp<int8_t> op{reinterpret_cast<const Code8x4*>(q), reinterpret_cast<float4*>(out),
+                                code_offset};
+        return launch_elementwise(op, outer, C, inner, qp, aligned16(q) && aligned16(out),
+                                  as_stream(stream), "dequantize");
+    }
+    DequantizeOp<int16_t> op{reinterpret_cast<const Code16x4*>(q), reinterpret_cast<float4*>(out),
+                             code_offset};
+    return launch_elementwise(op, outer, C, inner, qp, aligned16(q) && aligned16(out),
+                              as_stream(stream), "dequantize");
+}
+
+int lq_fake_quantize(const float* x, float* out, size_t outer, size_t C, size_t inner,
+                     const float* scale, const float* zp, int qparams_on_host, int qmin, int qmax,
+                     lq_stream stream) {
+    if (outer * C * inner == 0) return LQ_OK;
+    LQ_REQUIRE(x && out, LQ_ERR_VALUE, "fake_quantize: NULL tensor pointer");
+    LQ_REQUIRE(qmin <= qmax, LQ_ERR_VALUE, "fake_quantize: empty grid [%d,%d]", qmin, qmax);
+    QParams qp;
+    int rc = make_qparams(scale, zp, qparams_on_host, C, &qp, "fake_quantize");
+    if (rc) return rc;
+    FakeQuantizeOp op{reinterpret_cast<const float4*>(x), reinterpret_cast<float4*>(out),
+                      float(double(qmin)), float(double(qmax))};
+    return launch_elementwise(op, outer, C, inner, qp, aligned16(x) && aligned16(out),
+                              as_stream(stream), "fake_quantize");
+}
+
+}  // extern "C"

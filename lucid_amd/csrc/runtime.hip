@@ -1,0 +1,331 @@
+// Runtime entry points of the C ABI: device selection, storage, transfers,
+// events, the op registry and synthetic-data fills.
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "common.hpp"
+
+namespace lq {
+
+std::string& last_error() {
+    thread_local std::string msg;
+    return msg;
+}
+
+int fail(int status, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    last_error() = buf;
+    return status;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    int status = LQ_ERR_INTERNAL;
+    if (e == hipErrorOutOfMemory) status = LQ_ERR_OOM;
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice) status = LQ_ERR_GPU_NOT_AVAILABLE;
+    return fail(status, "%s: %s", what, hipGetErrorString(e));
+}
+
+namespace {
+constexpr int kMaxDevices = 16;
+struct Workspace {
+    void* ptr = nullptr;
+    size_t size = 0;
+};
+Workspace g_ws[kMaxDevices];
+std::mutex g_ws_mutex;
+}  // namespace
+
+int workspace(size_t nbytes, void** ptr) {
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    LQ_REQUIRE(dev >= 0 && dev < kMaxDevices, LQ_ERR_DEVICE, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Workspace& w = g_ws[dev];
+    if (w.size < nbytes) {
+        // finish whatever still reads the old block before it goes away
+        LQ_HIP(hipDeviceSynchronize());
+        if (w.ptr) LQ_HIP(hipFree(w.ptr));
+        w.ptr = nullptr;
+        w.size = 0;
+        size_t want = nbytes < (size_t(4) << 20) ? (size_t(4) << 20) : nbytes;
+        LQ_HIP(hipMalloc(&w.ptr, want));
+        w.size = want;
+    }
+    *ptr = w.ptr;
+    return LQ_OK;
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" {
+
+int lq_version(void) { return LQ_VERSION; }
+
+const char* lq_last_error(void) { return last_error().c_str(); }
+
+int lq_device_count(int* count) {
+    LQ_REQUIRE(count, LQ_ERR_VALUE, "count is NULL");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *count = 0;
+        return hip_fail(e, "hipGetDeviceCount");
+    }
+    *count = n;
+    return LQ_OK;
+}
+
+int lq_init(int device) {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0)
+        return fail(LQ_ERR_GPU_NOT_AVAILABLE, "no HIP device is visible (%s)",
+                    e == hipSuccess ? "count = 0" : hipGetErrorString(e));
+    LQ_REQUIRE(device >= 0 && device < n, LQ_ERR_DEVICE, "device %d out of range [0,%d)", device, n);
+    LQ_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    LQ_HIP(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(LQ_ERR_GPU_NOT_AVAILABLE, "device %d is %s; this library is built for gfx950 only",
+                    device, prop.gcnArchName);
+    void* ws = nullptr;
+    return workspace(size_t(4) << 20, &ws);
+}
+
+int lq_device_name(char* buf, size_t buflen) {
+    LQ_REQUIRE(buf && buflen > 0, LQ_ERR_VALUE, "buf is NULL");
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    LQ_HIP(hipGetDeviceProperties(&prop, dev));
+    snprintf(buf, buflen, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    return LQ_OK;
+}
+
+int lq_alloc(void** ptr, size_t nbytes) {
+    LQ_REQUIRE(ptr, LQ_ERR_VALUE, "ptr is NULL");
+    *ptr = nullptr;
+    if (nbytes == 0) nbytes = 16;  // a distinct, freeable address for empty tensors
+    LQ_HIP(hipMalloc(ptr, nbytes));
+    return LQ_OK;
+}
+
+int lq_free(void* ptr) {
+    if (ptr) LQ_HIP(hipFree(ptr));
+    return LQ_OK;
+}
+
+int lq_h2d(void* dst, const void* src, size_t nbytes, lq_stream stream) {
+    if (nbytes == 0) return LQ_OK;
+    LQ_REQUIRE(dst && src, LQ_ERR_VALUE, "NULL pointer in h2d");
+    LQ_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, as_stream(stream)));
+    LQ_HIP(hipStreamSynchronize(as_stream(stream)));  // pageable source may be reused at once
+    return LQ_OK;
+}
+
+int lq_d2h(void* dst, const void* src, size_t nbytes, lq_stream stream) {
+    if (nbytes == 0) return LQ_OK;
+    LQ_REQUIRE(dst && src, LQ_ERR_VALUE, "NULL pointer in d2h");
+    LQ_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    LQ_HIP(hipStreamSynchronize(as_stream(stream)));
+    return LQ_OK;
+}
+
+int lq_d2d(void* dst, const void* src, size_t nbytes, lq_stream stream) {
+    if (nbytes == 0) return LQ_OK;
+    LQ_REQUIRE(dst && src, LQ_ERR_VALUE, "NULL pointer in d2d");
+    LQ_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return LQ_OK;
+}
+
+int lq_sync(lq_stream stream) {
+    LQ_HIP(hipStreamSynchronize(as_stream(stream)));
+    return LQ_OK;
+}
+
+int lq_stream_create(lq_stream* stream) {
+    LQ_REQUIRE(stream, LQ_ERR_VALUE, "stream is NULL");
+    hipStream_t s;
+    LQ_HIP(hipStreamCreate(&s));  // default priority only
+    *stream = s;
+    return LQ_OK;
+}
+
+int lq_stream_destroy(lq_stream stream) {
+    if (stream) LQ_HIP(hipStreamDestroy(as_stream(stream)));
+    return LQ_OK;
+}
+
+int lq_event_create(lq_event* ev) {
+    LQ_REQUIRE(ev, LQ_ERR_VALUE, "ev is NULL");
+    hipEvent_t e;
+    LQ_HIP(hipEventCreate(&e));
+    *ev = e;
+    return LQ_OK;
+}
+
+int lq_event_destroy(lq_event ev) {
+    if (ev) LQ_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(ev)));
+    return LQ_OK;
+}
+
+int lq_event_record(lq_event ev, lq_stream stream) {
+    LQ_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(ev), as_stream(stream)));
+    return LQ_OK;
+}
+
+int lq_event_sync(lq_event ev) {
+    LQ_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(ev)));
+    return LQ_OK;
+}
+
+int lq_event_elapsed_ms(lq_event start, lq_event stop, float* ms) {
+    LQ_REQUIRE(ms, LQ_ERR_VALUE, "ms is NULL");
+    LQ_HIP(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start),
+                               reinterpret_cast<hipEvent_t>(stop)));
+    return LQ_OK;
+}
+
+// ------------------------------------------------------------------ op registry
+namespace {
+struct OpSchema {
+    const char* name;
+    int version;
+    int deterministic;
+};
+// Integer accumulation is order-independent, so every op here is
+// deterministic, the split-K GEMM included.
+const OpSchema kOps[] = {
+    {"minmax", 1, 1},        {"calc_qparams", 1, 1}, {"quantize", 1, 1},
+    {"dequantize", 1, 1},    {"fake_quantize", 1, 1},
+};
+}  // namespace
+
+int lq_op_count(void) { return int(sizeof kOps / sizeof kOps[0]); }
+
+int lq_op_info(int index, const char** name, int* version, int* deterministic) {
+    LQ_REQUIRE(index >= 0 && index < lq_op_count(), LQ_ERR_VALUE, "op index %d out of range", index);
+    if (name) *name = kOps[index].name;
+    if (version) *version = kOps[index].version;
+    if (deterministic) *deterministic = kOps[index].deterministic;
+    return LQ_OK;
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------ fills / copy
+namespace {
+
+__device__ inline uint64_t splitmix64(uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+// Two normals per counter (Box-Muller).  Quality is that of a benchmark
+// input generator, nothing more.
+__global__ void fill_normal_kernel(float* x, size_t n, uint64_t seed, float outlier_prob,
+                                   float outlier_gain) {
+    size_t pair = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (; pair * 2 < n; pair += stride) {
+        uint64_t r = splitmix64(seed ^ (pair * 0xD1342543DE82EF95ull));
+        uint64_t r2 = splitmix64(r);
+        float u1 = (float((r >> 40) + 1)) * (1.0f / 16777217.0f);
+        float u2 = float(r & 0xFFFFFF) * (1.0f / 16777216.0f);
+        float rad = sqrtf(-2.0f * logf(u1));
+        float s, c;
+        sincosf(6.28318530718f * u2, &s, &c);
+        float a = rad * c, b = rad * s;
+        float p1 = float(r2 >> 40) * (1.0f / 16777216.0f);
+        float p2 = float(r2 & 0xFFFFFF) * (1.0f / 16777216.0f);
+        if (p1 < outlier_prob) a *= outlier_gain;
+        if (p2 < outlier_prob) b *= outlier_gain;
+        x[pair * 2] = a;
+        if (pair * 2 + 1 < n) x[pair * 2 + 1] = b;
+    }
+}
+
+__global__ void fill_uniform_i8_kernel(int8_t* x, size_t n, uint64_t seed, int lo, int span) {
+    size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (; i < n; i += stride) {
+        uint64_t r = splitmix64(seed ^ (i * 0xD1342543DE82EF95ull));
+        x[i] = int8_t(lo + int((r >> 33) % uint64_t(span)));
+    }
+}
+
+__global__ void fill_bytes_kernel(uint8_t* x, size_t n, uint8_t v) {
+    size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (; i < n; i += stride) x[i] = v;
+}
+
+__global__ void copy16_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n16) {
+    size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+inline unsigned blocks_for(size_t work, unsigned per_block, unsigned cap) {
+    size_t b = (work + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    return unsigned(b > cap ? cap : b);
+}
+
+}  // namespace
+
+extern "C" {
+
+int lq_fill_normal(float* x, size_t n, uint64_t seed, float outlier_prob, float outlier_gain,
+                   lq_stream stream) {
+    if (n == 0) return LQ_OK;
+    LQ_REQUIRE(x, LQ_ERR_VALUE, "x is NULL");
+    hipLaunchKernelGGL(fill_normal_kernel, dim3(blocks_for((n + 1) / 2, 256, 65536)), dim3(256), 0,
+                       as_stream(stream), x, n, seed, outlier_prob, outlier_gain);
+    LQ_CHECK_LAUNCH("fill_normal");
+    return LQ_OK;
+}
+
+int lq_fill_uniform_i8(int8_t* x, size_t n, uint64_t seed, int lo, int hi, lq_stream stream) {
+    if (n == 0) return LQ_OK;
+    LQ_REQUIRE(x, LQ_ERR_VALUE, "x is NULL");
+    LQ_REQUIRE(lo >= -128 && hi <= 127 && lo <= hi, LQ_ERR_VALUE, "bad int8 range [%d,%d]", lo, hi);
+    hipLaunchKernelGGL(fill_uniform_i8_kernel, dim3(blocks_for(n, 256, 65536)), dim3(256), 0,
+                       as_stream(stream), x, n, seed, lo, hi - lo + 1);
+    LQ_CHECK_LAUNCH("fill_uniform_i8");
+    return LQ_OK;
+}
+
+// A fill kernel rather than hipMemsetAsync so that callers may capture it in
+// a HIP graph.
+int lq_fill_bytes(void* dst, int value, size_t nbytes, lq_stream stream) {
+    if (nbytes == 0) return LQ_OK;
+    LQ_REQUIRE(dst, LQ_ERR_VALUE, "dst is NULL");
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3(blocks_for(nbytes, 256, 65536)), dim3(256), 0,
+                       as_stream(stream), static_cast<uint8_t*>(dst), nbytes, uint8_t(value));
+    LQ_CHECK_LAUNCH("fill_bytes");
+    return LQ_OK;
+}
+
+int lq_copy_kernel(void* dst, const void* src, size_t nbytes, lq_stream stream) {
+    LQ_REQUIRE(dst && src, LQ_ERR_VALUE, "NULL pointer");
+    LQ_REQUIRE(nbytes % 16 == 0 && aligned16(dst) && aligned16(src), LQ_ERR_VALUE,
+               "copy kernel needs 16-byte aligned pointers and size");
+    if (nbytes == 0) return LQ_OK;
+    hipLaunchKernelGGL(copy16_kernel, dim3(blocks_for(nbytes / 16, 256, 1 << 20)), dim3(256), 0,
+                       as_stream(stream), static_cast<uint4*>(dst), static_cast<const uint4*>(src),
+                       nbytes / 16);
+    LQ_CHECK_LAUNCH("copy16");
+    return LQ_OK;
+}
+
+}  // extern "C"
