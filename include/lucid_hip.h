@@ -132,6 +132,54 @@ int lq_fake_quantize(const float* x, float* out, size_t outer, size_t C, size_t 
                      const float* scale, const float* zp, int qparams_on_host, int qmin, int qmax,
                      lq_stream stream);
 
+/* ------------------------------------------------------- quantized Linear */
+/* Output forms of the fused GEMM epilogue. */
+#define LQ_OUT_ACC_I32 0       /* raw int32 accumulators                         */
+#define LQ_OUT_F32 1           /* dequantized float32 (nnqd.Linear's result)     */
+#define LQ_OUT_F16 2           /* dequantized float16, RNE (core/Half.h:80-110)  */
+#define LQ_OUT_REQUANT_I8 3    /* code on the output grid, stored + out_offset   */
+#define LQ_OUT_FAKEQUANT_F32 4 /* float-carried value on the output grid         */
+
+/* sum_k w[n,k] for every weight row: the zero-point correction term, computed
+ * once when a module is converted (from_float, lucid/nn/quantized/linear.py:217-236). */
+int lq_rowsum_i8(const int8_t* w, int32_t* out, int N, int K, lq_stream stream);
+
+/* Quantized Linear forward.  Replaces the composite that
+ * lucid/nn/quantized/linear.py:199-215 (static), intrinsic.py:131-133 (fused
+ * ReLU) and dynamic/linear.py:84-99 (dynamic) build from dequantize +
+ * IBackend::linear (IBackend.h:960-966; CpuBackend.h:4525-4569) +
+ * fake_quantize, by its exact integer identity:
+ *     acc[m,n] = sum_k a[m,k] * w[n,k]                              (int32)
+ *     y = f32(acc - a_zp*wsum[n]) * (a_scale[m|0] * w_scale[n]) + bias[n]
+ *     y = relu(y) if relu
+ *     out = per out_mode
+ * a: int8 [M,K] activation codes as stored (a quint8 code c is stored as
+ * c - 128, and a_zp is then Z - 128); w: int8 [N,K].  All pointers are device
+ * pointers; scales and output qparams are read on the device so no host
+ * synchronisation is needed between layers. */
+typedef struct {
+    const int8_t* a;
+    const int8_t* w;
+    int M, N, K;
+    const int32_t* wsum;   /* [N], required when a_zp != 0                   */
+    int a_zp;
+    const float* a_scale;  /* [M] when a_scale_per_row, else [1]             */
+    int a_scale_per_row;
+    const float* w_scale;  /* [N]                                            */
+    const void* bias;      /* [N] or NULL                                    */
+    int bias_dtype;        /* LQ_F32 or LQ_F16                               */
+    int relu;
+    int out_mode;          /* LQ_OUT_*                                       */
+    const float* out_scale;/* [1], modes REQUANT_I8 / FAKEQUANT_F32          */
+    const float* out_zp;   /* [1]                                            */
+    int out_qmin, out_qmax, out_offset;
+    void* out;             /* [M, ldo] in the type out_mode implies          */
+    long ldo;              /* output row stride in elements; 0 means N       */
+    int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
+} lq_qlinear_args;
+
+int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -95,6 +95,25 @@ _SIGNATURES = {
     "lq_dequantize": [_vp, _i, _i, _vp, _sz, _sz, _sz, _vp, _vp, _i, _vp],
     "lq_fake_quantize": [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _i, _i, _i, _vp],
 }
+
+
+class QLinearArgs(C.Structure):
+    """``lq_qlinear_args`` of ``include/lucid_hip.h``."""
+
+    _fields_ = [
+        ("a", _vp), ("w", _vp), ("M", _i), ("N", _i), ("K", _i),
+        ("wsum", _vp), ("a_zp", _i),
+        ("a_scale", _vp), ("a_scale_per_row", _i), ("w_scale", _vp),
+        ("bias", _vp), ("bias_dtype", _i), ("relu", _i), ("out_mode", _i),
+        ("out_scale", _vp), ("out_zp", _vp),
+        ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
+        ("out", _vp), ("ldo", C.c_long), ("force_path", _i),
+    ]
+
+
+_SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
+_SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
+
 _RESTYPE = {"lq_last_error": C.c_char_p}
 _NO_STATUS = {"lq_version", "lq_last_error", "lq_op_count"}
 

@@ -1,0 +1,76 @@
+"""Thin argument marshalling for the fused GEMM / conv entry points.
+
+These helpers only fill the C structs of ``include/lucid_hip.h`` from
+``Tensor`` handles and validate devices; the quantized modules build on them.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+
+from . import _C
+from . import _tensor as T
+from ._tensor import Tensor
+
+OUT_ACC_I32, OUT_F32, OUT_F16, OUT_REQUANT_I8, OUT_FAKEQUANT_F32 = range(5)
+_OUT_DTYPE = {OUT_ACC_I32: T.int32, OUT_F32: T.float32, OUT_F16: T.float16,
+              OUT_REQUANT_I8: T.int8, OUT_FAKEQUANT_F32: T.float32}
+PATH_AUTO, PATH_TILE, PATH_SKINNY, PATH_NAIVE = range(4)
+
+
+def _ptr(t: Tensor | None, what: str, dt=None):
+    if t is None:
+        return None
+    if not isinstance(t, Tensor) or t.device != "hip":
+        raise _C.DeviceMismatch(f"{what} must be a tensor on the 'hip' device")
+    if dt is not None and t.dtype not in (dt if isinstance(dt, tuple) else (dt,)):
+        raise _C.DtypeMismatch(f"{what} has dtype {t.dtype}, expected {dt}")
+    return t.data_ptr
+
+
+def rowsum_i8(w: Tensor) -> Tensor:
+    """``sum_k w[n, k]`` as int32, over everything but the first axis."""
+    N = w.shape[0]
+    K = w.numel // max(N, 1)
+    out = Tensor.empty((N,), T.int32, "hip")
+    _C.call("lq_rowsum_i8", _ptr(w, "w", T.int8), out.data_ptr, N, K, None)
+    return out
+
+
+def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_scale: Tensor | None = None,
+               w_scale: Tensor | None = None, wsum: Tensor | None = None,
+               bias: Tensor | None = None, relu: bool = False, out_mode: int = OUT_F32,
+               out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
+               out_qmax: int = 255, out_offset: int = 0, path: int = PATH_AUTO,
+               out: Tensor | None = None) -> Tensor:
+    """Fused int8 GEMM + epilogue; see ``lq_qlinear_i8`` in ``lucid_hip.h``.
+    ``a`` is int8 ``[M, K]``, ``w`` int8 ``[N, K]``; the result is ``[M, N]``."""
+    if a.ndim != 2 or w.ndim != 2 or a.shape[1] != w.shape[1]:
+        raise _C.ShapeMismatch(f"qlinear_i8: a {a.shape} and w {w.shape} do not form a GEMM")
+    M, K = a.shape
+    N = w.shape[0]
+    if out is None:
+        out = Tensor.empty((M, N), _OUT_DTYPE[out_mode], "hip")
+    args = _C.QLinearArgs()
+    args.a, args.w = _ptr(a, "a", T.int8), _ptr(w, "w", T.int8)
+    args.M, args.N, args.K = M, N, K
+    args.wsum = _ptr(wsum, "wsum", T.int32)
+    args.a_zp = int(a_zp)
+    args.a_scale = _ptr(a_scale, "a_scale", T.float32)
+    args.a_scale_per_row = int(a_scale is not None and a_scale.numel != 1)
+    if a_scale is not None and a_scale.numel not in (1, M):
+        raise _C.ShapeMismatch(f"a_scale has {a_scale.numel} entries for M = {M}")
+    if w_scale is not None and w_scale.numel != N:
+        raise _C.ShapeMismatch(f"w_scale has {w_scale.numel} entries for N = {N}")
+    args.w_scale = _ptr(w_scale, "w_scale", T.float32)
+    args.bias = _ptr(bias, "bias", (T.float32, T.float16))
+    args.bias_dtype = bias.dtype.code if bias is not None else 0
+    if bias is not None and bias.numel != N:
+        raise _C.ShapeMismatch(f"bias has {bias.numel} entries for N = {N}")
+    args.relu, args.out_mode = int(relu), int(out_mode)
+    args.out_scale = _ptr(out_scale, "out_scale", T.float32)
+    args.out_zp = _ptr(out_zp, "out_zp", T.float32)
+    args.out_qmin, args.out_qmax, args.out_offset = int(out_qmin), int(out_qmax), int(out_offset)
+    args.out, args.ldo, args.force_path = out.data_ptr, 0, int(path)
+    _C.call("lq_qlinear_i8", C.byref(args), None)
+    return out

@@ -204,7 +204,8 @@ struct OpSchema {
 // deterministic, the split-K GEMM included.
 const OpSchema kOps[] = {
     {"minmax", 1, 1},        {"calc_qparams", 1, 1}, {"quantize", 1, 1},
-    {"dequantize", 1, 1},    {"fake_quantize", 1, 1},
+    {"dequantize", 1, 1},    {"fake_quantize", 1, 1}, {"rowsum_i8", 1, 1},
+    {"qlinear_i8", 1, 1},
 };
 }  // namespace
 

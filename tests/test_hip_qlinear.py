@@ -1,0 +1,155 @@
+"""GPU parity of the int8 GEMM + fused epilogue (``lq_qlinear_i8``) against
+the CPU oracle: int32 accumulators and requantized codes bit for bit, float
+outputs bit for bit as well (same float steps in the same order), on all three
+kernels (tile / skinny / naive), ragged shapes and every output form."""
+
+import numpy as np
+import pytest
+
+import lucid_amd as L
+from lucid_amd import _ops
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TILE, SKINNY, NAIVE = _ops.PATH_TILE, _ops.PATH_SKINNY, _ops.PATH_NAIVE
+
+
+def hip(a):
+    return L.tensor(np.ascontiguousarray(a), device="hip")
+
+
+def codes(rng, shape, lo=-128, hi=127):
+    return rng.integers(lo, hi + 1, shape).astype(np.int8)
+
+
+ACC_CASES = [
+    # M, N, K, path
+    (256, 256, 128, TILE), (256, 256, 256, TILE), (512, 512, 4096, TILE), (300, 260, 144, TILE),
+    (1, 16, 16, TILE), (129, 77, 784, TILE), (700, 1000, 576, TILE), (64, 256, 784, TILE),
+    (1, 11008, 4096, SKINNY), (16, 11008, 4096, SKINNY), (16, 1024, 4096, SKINNY),
+    (3, 50, 48, SKINNY), (17, 33, 784, SKINNY), (33, 100, 272, SKINNY), (64, 256, 784, SKINNY),
+    (64, 10, 256, SKINNY), (5, 7, 16, SKINNY),
+    (5, 7, 3, NAIVE), (17, 33, 147, NAIVE), (64, 10, 250, NAIVE),
+]
+
+
+@pytest.mark.parametrize("M,N,K,path", ACC_CASES)
+def test_accumulators_exact(M, N, K, path):
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    acc = _ops.qlinear_i8(hip(a), hip(w), out_mode=_ops.OUT_ACC_I32, path=path).numpy()
+    assert np.array_equal(acc, O.igemm(a, w))
+
+
+@pytest.mark.parametrize("path,M", [(TILE, 300), (SKINNY, 16), (NAIVE, 9)])
+def test_extreme_codes(path, M):
+    K, N = 4096, 48
+    a = np.full((M, K), -128, np.int8)
+    w = np.full((N, K), -128, np.int8)
+    acc = _ops.qlinear_i8(hip(a), hip(w), out_mode=_ops.OUT_ACC_I32, path=path).numpy()
+    assert (acc == 128 * 128 * K).all()
+
+
+def test_auto_path_matches_forced_paths():
+    rng = np.random.default_rng(0)
+    for M in (1, 16, 64, 65, 200):
+        a, w = codes(rng, (M, 512)), codes(rng, (96, 512))
+        ref = O.igemm(a, w)
+        assert np.array_equal(_ops.qlinear_i8(hip(a), hip(w), out_mode=0).numpy(), ref)
+    a, w = codes(rng, (20, 50)), codes(rng, (9, 50))     # K % 16 != 0 -> naive
+    assert np.array_equal(_ops.qlinear_i8(hip(a), hip(w), out_mode=0).numpy(), O.igemm(a, w))
+
+
+def _epilogue_case(rng, M, N, K, per_row, bias_kind):
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    a_scale = rng.uniform(0.005, 0.05, M if per_row else 1).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = None
+    if bias_kind == "f32":
+        bias = rng.standard_normal(N).astype(np.float32)
+    elif bias_kind == "f16":
+        bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    a_zp = 0 if per_row else int(rng.integers(-128, 127))
+    return a, w, a_scale, w_scale, bias, a_zp
+
+
+MODES = [_ops.OUT_F32, _ops.OUT_F16, _ops.OUT_REQUANT_I8, _ops.OUT_FAKEQUANT_F32]
+
+
+@pytest.mark.parametrize("path,M,N,K", [(TILE, 300, 260, 144), (TILE, 64, 256, 784),
+                                         (SKINNY, 16, 272, 4096), (SKINNY, 37, 50, 64),
+                                         (NAIVE, 9, 21, 30)])
+@pytest.mark.parametrize("per_row,bias_kind,relu", [(False, "f32", False), (False, "f32", True),
+                                                    (True, "f16", False), (False, None, True),
+                                                    (True, None, False)])
+def test_epilogue_bit_exact(path, M, N, K, per_row, bias_kind, relu):
+    rng = np.random.default_rng(M + 13 * N + K + int(per_row) + int(relu))
+    a, w, a_scale, w_scale, bias, a_zp = _epilogue_case(rng, M, N, K, per_row, bias_kind)
+    wsum = _ops.rowsum_i8(hip(w))
+    assert np.array_equal(wsum.numpy(), O.rowsum_i8(w))
+    y = O.qlinear(a, w, a_zp, a_scale, w_scale, bias=bias, relu=relu, out_mode=O.OUT_F32)
+    S = np.float32(np.abs(y).max() / 200 + 1e-6)
+    Z = np.float32(0.0 if relu else 128.0)
+    for mode in MODES:
+        got = _ops.qlinear_i8(hip(a), hip(w), a_zp=a_zp, a_scale=hip(a_scale),
+                              w_scale=hip(w_scale), wsum=wsum,
+                              bias=None if bias is None else hip(bias), relu=relu, out_mode=mode,
+                              out_scale=hip(S), out_zp=hip(Z), out_qmin=0, out_qmax=255,
+                              out_offset=-128, path=path).numpy()
+        exp = O.qlinear(a, w, a_zp, a_scale, w_scale, bias=bias, relu=relu, out_mode=mode,
+                        out_scale=S, out_zp=Z, out_qmin=0, out_qmax=255, out_offset=-128)
+        if mode == _ops.OUT_F16:
+            assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+        elif mode == _ops.OUT_REQUANT_I8:
+            assert np.array_equal(got, exp)
+        else:
+            assert np.array_equal(got.view(np.uint32), exp.view(np.uint32))
+
+
+def test_llm_shape_f16_output_matches_oracle_on_sampled_rows():
+    """K=4096, N=11008 with per-token activation scales, per-row weight scales,
+    fp16 bias, fp16 output - the benchmark's Linear, M = 2048 on the tile
+    kernel and M = 1, 16 on the skinny kernel."""
+    rng = np.random.default_rng(42)
+    K, N = 4096, 11008
+    wf = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    mn, mx = O.minmax(wf, ch_axis=0)
+    ws, wz = O.calc_qparams(mn, mx, True, -128, 127, True)
+    wq = O.quantize(wf, ws, wz, -128, 127, ch_axis=0)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    w_dev, ws_dev, b_dev = hip(wq), hip(ws), hip(bias)
+    for M in (1, 16, 2048):
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        mn, mx = O.minmax(x, ch_axis=0)
+        xs, xz = O.calc_qparams(mn, mx, True, -128, 127, True)
+        xq = O.quantize(x, xs, xz, -128, 127, ch_axis=0)
+        got = _ops.qlinear_i8(hip(xq), w_dev, a_scale=hip(xs), w_scale=ws_dev, bias=b_dev,
+                              out_mode=_ops.OUT_F16).numpy()
+        rows = np.unique(rng.integers(0, M, 24))
+        exp = O.qlinear(xq[rows], wq, 0, xs[rows], ws, bias=bias, out_mode=O.OUT_F16)
+        assert np.array_equal(got[rows].view(np.uint16), exp.view(np.uint16))
+        # linearity of the exact accumulators at full size: acc(x, w) + acc(x', w) == acc(x + x', w)
+        if M == 2048:
+            xa = codes(rng, (M, K), -60, 60)
+            xb = codes(rng, (M, K), -60, 60)
+            acc = lambda t: _ops.qlinear_i8(hip(t), w_dev, out_mode=_ops.OUT_ACC_I32).numpy()
+            assert np.array_equal(acc(xa) + acc(xb), acc((xa + xb).astype(np.int8)))
+
+
+def test_argument_validation():
+    a, w = hip(np.zeros((4, 32), np.int8)), hip(np.zeros((8, 32), np.int8))
+    with pytest.raises(L.ShapeMismatch):
+        _ops.qlinear_i8(a, hip(np.zeros((8, 16), np.int8)))
+    with pytest.raises(ValueError):      # a_zp without the weight row sums
+        _ops.qlinear_i8(a, w, a_zp=3, a_scale=hip(np.ones(1, np.float32)),
+                        w_scale=hip(np.ones(8, np.float32)))
+    with pytest.raises(L.DtypeMismatch):
+        _ops.qlinear_i8(hip(np.zeros((4, 32), np.float32)), w)
+    with pytest.raises(L.DeviceMismatch):
+        _ops.qlinear_i8(L.tensor(np.zeros((4, 32), np.int8)), w)
+    with pytest.raises(L.ShapeMismatch):  # skinny path forced on a tall problem
+        _ops.qlinear_i8(hip(np.zeros((100, 32), np.int8)), w, out_mode=0, path=SKINNY)
+    with pytest.raises(ValueError):       # MFMA path on K % 16 != 0
+        _ops.qlinear_i8(hip(np.zeros((4, 30), np.int8)), hip(np.zeros((8, 30), np.int8)),
+                        out_mode=0, path=TILE)
