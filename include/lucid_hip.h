@@ -176,6 +176,7 @@ typedef struct {
     void* out;             /* [M, ldo] in the type out_mode implies          */
     long ldo;              /* output row stride in elements; 0 means N       */
     int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
+    int tile_config;       /* 0 = choose; 1..5 = a specific tile shape (tuning) */
 } lq_qlinear_args;
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);

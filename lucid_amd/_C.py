@@ -107,7 +107,7 @@ class QLinearArgs(C.Structure):
         ("bias", _vp), ("bias_dtype", _i), ("relu", _i), ("out_mode", _i),
         ("out_scale", _vp), ("out_zp", _vp),
         ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
-        ("out", _vp), ("ldo", C.c_long), ("force_path", _i),
+        ("out", _vp), ("ldo", C.c_long), ("force_path", _i), ("tile_config", _i),
     ]
 
 

@@ -78,46 +78,103 @@ __device__ __forceinline__ float q_core(float x, float s, float z, float lo, flo
 }
 
 // One output element.  Float steps are separate (no FMA) and in the order the
-// CPU restatement uses, so results are bit-identical to it.
-__device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, int32_t acc,
-                                               float as, const ColParams& c, float S, float Z) {
-    const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
-    if (g.out_mode == OUT_ACC_I32) {
-        static_cast<int32_t*>(g.out)[idx] = acc;
-        return;
-    }
+// CPU restatement uses, so results are bit-identical to it.  MODE is a
+// compile-time constant so that each output form gets a tight loop.
+// epilogue_value returns the element as 32 bits (float bits, or the integer
+// for the accumulator / requantized-code forms); store_* narrows and writes.
+template <int MODE>
+__device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t acc, float as,
+                                                   const ColParams& c, float S, float Z) {
+    if (MODE == OUT_ACC_I32) return uint32_t(acc);
     float f = float(acc - c.corr);
     float sc = as * c.ws;
     float y = f * sc;
     if (g.bias) y = y + c.bias;
     if (g.relu) y = (y < 0.0f) ? 0.0f : y;
-    switch (g.out_mode) {
-    case OUT_F32:
-        static_cast<float*>(g.out)[idx] = y;
-        break;
-    case OUT_F16:
-        static_cast<_Float16*>(g.out)[idx] = _Float16(y);
-        break;
-    case OUT_REQUANT_I8: {
-        float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
+    if (MODE == OUT_F32 || MODE == OUT_F16) return __float_as_uint(y);
+    float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
+    if (MODE == OUT_REQUANT_I8) {
         int code = (qv != qv) ? 0 : int(qv);
-        static_cast<int8_t*>(g.out)[idx] = int8_t(code + g.out_offset);
-        break;
+        return uint32_t(code + g.out_offset);
     }
-    default: {  // OUT_FAKEQUANT_F32
-        float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
-        static_cast<float*>(g.out)[idx] = (qv - Z) * S;
-        break;
+    return __float_as_uint((qv - Z) * S);  // OUT_FAKEQUANT_F32
+}
+
+template <int MODE>
+__device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint32_t v) {
+    if (MODE == OUT_F16)
+        static_cast<_Float16*>(g.out)[idx] = _Float16(__uint_as_float(v));
+    else if (MODE == OUT_REQUANT_I8)
+        static_cast<int8_t*>(g.out)[idx] = int8_t(int(v));
+    else
+        static_cast<uint32_t*>(g.out)[idx] = v;  // f32 / i32 bit patterns
+}
+
+// four consecutive elements; idx is a multiple of 4 and the row is 4-aligned
+template <int MODE>
+__device__ __forceinline__ void store_vec4(const GemmArgs& g, size_t idx, uint4 v) {
+    if (MODE == OUT_F16) {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        h4 h = {_Float16(__uint_as_float(v.x)), _Float16(__uint_as_float(v.y)),
+                _Float16(__uint_as_float(v.z)), _Float16(__uint_as_float(v.w))};
+        *reinterpret_cast<h4*>(static_cast<_Float16*>(g.out) + idx) = h;
+    } else if (MODE == OUT_REQUANT_I8) {
+        uint32_t packed = (v.x & 0xffu) | ((v.y & 0xffu) << 8) | ((v.z & 0xffu) << 16) | (v.w << 24);
+        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(g.out) + idx) = packed;
+    } else {
+        *reinterpret_cast<uint4*>(static_cast<uint32_t*>(g.out) + idx) = v;
     }
+}
+
+template <int MODE>
+__device__ __forceinline__ void epilogue_store_t(const GemmArgs& g, int m, int n, int32_t acc,
+                                                 float as, const ColParams& c, float S, float Z) {
+    store_scalar<MODE>(g, size_t(m) * size_t(g.ldo) + size_t(n),
+                       epilogue_value<MODE>(g, acc, as, c, S, Z));
+}
+
+__device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, int32_t acc,
+                                               float as, const ColParams& c, float S, float Z) {
+    switch (g.out_mode) {
+    case OUT_ACC_I32: epilogue_store_t<OUT_ACC_I32>(g, m, n, acc, as, c, S, Z); break;
+    case OUT_F32: epilogue_store_t<OUT_F32>(g, m, n, acc, as, c, S, Z); break;
+    case OUT_F16: epilogue_store_t<OUT_F16>(g, m, n, acc, as, c, S, Z); break;
+    case OUT_REQUANT_I8: epilogue_store_t<OUT_REQUANT_I8>(g, m, n, acc, as, c, S, Z); break;
+    default: epilogue_store_t<OUT_FAKEQUANT_F32>(g, m, n, acc, as, c, S, Z); break;
     }
 }
 
 // ---------------------------------------------------------------- tile kernel
-constexpr int BM = 256, BN = 256, BK = 128;
-constexpr int kTileThreads = 256;
-constexpr int kChunksPerRow = BK / 16;                 // 8 sixteen-byte chunks per tile row
-constexpr int kStageBytes = (BM + BN) * BK;            // 64 KiB
-constexpr int kTileSmem = 2 * kStageBytes;             // double buffered: 128 KiB of 160 KiB
+// Compile-time shape of one tile kernel.
+//   BM x BN x BK : block tile (BK bytes of k per LDS stage)
+//   WM x WN      : wavefront grid; each wavefront owns (BM/WM) x (BN/WN) outputs
+//                  as TM x TN MFMA tiles of 32 x 32
+//   STAGES       : LDS stages; STAGES-1 of them are in flight from global memory
+//   MINWAVES     : wavefronts per SIMD the register budget must allow
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int MINWAVES_>
+struct TileCfg {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
+    static constexpr int MINWAVES = MINWAVES_;
+    static constexpr int THREADS = WM * WN * 64;
+    static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    static constexpr int C = BK / 16;              // 16-byte chunks per LDS row
+    static constexpr int R = 16 / C;               // LDS rows per 256 bytes (one pass over 64 banks)
+    static constexpr int ROWS_PER_PASS = THREADS / C;
+    static constexpr int PA = BM / ROWS_PER_PASS, PB = BN / ROWS_PER_PASS;
+    static constexpr int KSTEPS = BK / 32;
+    static constexpr int STAGE_BYTES = (BM + BN) * BK;
+    static constexpr int STAGE_STRIDE = TN * 32 + 4;   // words per staged output row
+    static constexpr int STAGE_WORDS = 32 * STAGE_STRIDE;
+    static constexpr int EPI_BYTES = 4 * BM + THREADS / 64 * STAGE_WORDS * 4;
+    static constexpr int SMEM = STAGES * STAGE_BYTES > EPI_BYTES ? STAGES * STAGE_BYTES : EPI_BYTES;
+    static_assert(BK == 64 || BK == 128, "BK is 64 or 128 bytes");
+    static_assert(ROWS_PER_PASS % 16 == 0 && BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "");
+    static_assert((STAGES - 2) * (PA + PB) <= 63, "vmcnt is a 6-bit counter");
+};
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding:
+// vmcnt in bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8]).
+constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
 // Blocks are handed to the 8 XCDs round-robin.  Give every XCD one contiguous
 // range of logical tile ids so that the tiles sharing an L2 also share
@@ -137,59 +194,119 @@ __device__ __forceinline__ void tile_coords(int bid, int nblk, int tiles_m, int 
     *tn = in_group / gsz;
 }
 
-// LDS tile layout: row-major rows of BK bytes; the 16-byte chunk kc of row r
-// sits at physical chunk kc ^ (r & 7), which makes both the 1 KiB
-// wavefront-wide direct loads and the ds_read_b128 fragment reads free of
-// bank conflicts.
-__global__ __launch_bounds__(kTileThreads, 1) void qgemm_tile_kernel(GemmArgs g) {
+// Epilogue of one wavefront's sub-tile, in 32-row bands.  The MFMA result
+// layout gives a lane one column and sixteen scattered rows; the band is
+// turned through LDS so that a lane ends up with four consecutive columns of
+// one row and the wavefront writes contiguous row segments.
+template <class Cfg, int MODE>
+__device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg::TM][Cfg::TN],
+                                              const ColParams (&cp)[Cfg::TN], const float* s_as,
+                                              uint32_t* stage, int m0, int n0, int wm, int wn,
+                                              int lane, float S, float Z) {
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, STRIDE = Cfg::STAGE_STRIDE;
+    constexpr int QUADS_PER_ROW = TN * 8;            // four-column groups per staged row
+    constexpr int PASSES = 32 * QUADS_PER_ROW / 64;
+    const int esize = MODE == OUT_F16 ? 2 : (MODE == OUT_REQUANT_I8 ? 1 : 4);
+    const bool vec_ok = (g.ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int band = wm * (TM * 32) + i * 32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const float as = s_as[band + row];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                stage[row * STRIDE + j * 32 + (lane & 31)] =
+                    epilogue_value<MODE>(g, acc[i][j][r], as, cp[j], S, Z);
+            __builtin_amdgcn_sched_barrier(0);  // keep the unrolled rows from piling up live registers
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int p = 0; p < PASSES; ++p) {
+            const int q = p * 64 + lane;
+            const int row = q / QUADS_PER_ROW, cq = (q % QUADS_PER_ROW) * 4;
+            const uint4 v = *reinterpret_cast<const uint4*>(stage + row * STRIDE + cq);
+            const int m = m0 + band + row, n = n0 + wn * (TN * 32) + cq;
+            if (m < g.M && n < g.N) {
+                const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
+                if (vec_ok && n + 4 <= g.N) {
+                    store_vec4<MODE>(g, idx, v);
+                } else {
+                    store_scalar<MODE>(g, idx, v.x);
+                    if (n + 1 < g.N) store_scalar<MODE>(g, idx + 1, v.y);
+                    if (n + 2 < g.N) store_scalar<MODE>(g, idx + 2, v.z);
+                    if (n + 3 < g.N) store_scalar<MODE>(g, idx + 3, v.w);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// LDS stage layout: BM rows of A then BN rows of B, each row BK bytes; the
+// 16-byte chunk kc of row r sits at physical chunk kc ^ ((r / R) % C).  With
+// 64 LDS banks a ds_read_b128 serves 16 lanes per pass; under this swizzle the
+// 16 fragment rows of a pass fall on 16 different bank groups.  A wavefront's
+// direct global->LDS load writes 1 KiB of consecutive slots, so the swizzle is
+// applied on the global side: a lane fetches the chunk that belongs in its slot.
+template <class Cfg, int MODE>
+__global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel(GemmArgs g) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
+    constexpr int C = Cfg::C, R = Cfg::R, PA = Cfg::PA, PB = Cfg::PB, STAGES = Cfg::STAGES;
+    constexpr int THREADS = Cfg::THREADS, KSTEPS = Cfg::KSTEPS;
     extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     int tm, tn;
     tile_coords(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * BM, n0 = tn * BN;
-    const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 wavefronts, 128 x 128 each
+    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
 
-    // ---- global -> LDS addressing.  Slot s = it*256 + tid holds row s/8,
-    // physical chunk s%8.  (s/8) & 7 == (tid/8) & 7 for every it, so the
-    // logical chunk a lane fetches is the same in all iterations.
-    const int row_in_pass = tid >> 3;                      // 0..31
-    const int kc = (tid & 7) ^ (row_in_pass & 7);          // logical chunk this lane fetches
-    constexpr int kPasses = BM * kChunksPerRow / kTileThreads;  // 8 (BM == BN)
-    unsigned a_off[kPasses], b_off[kPasses];
-    const int a_rows = g.M - m0, b_rows = g.N - n0;        // valid rows in this tile (>= 1)
+    // ---- global -> LDS addressing.  In pass `it` this lane fills the slot of
+    // row it*ROWS_PER_PASS + tid/C, physical chunk tid%C.  ROWS_PER_PASS is a
+    // multiple of 16, so the swizzle term - and with it the logical chunk the
+    // lane fetches - is the same in every pass.
+    const int row_in_pass = tid / C;
+    const int kc = (tid % C) ^ ((row_in_pass / R) % C);
+    unsigned a_off[PA], b_off[PB];
+    const int a_rows = g.M - m0, b_rows = g.N - n0;  // valid rows in this tile (>= 1)
 #pragma unroll
-    for (int it = 0; it < kPasses; ++it) {
-        int r = it * 32 + row_in_pass;
-        int ra = r < a_rows ? r : a_rows - 1;              // clamp: reads stay in bounds,
-        int rb = r < b_rows ? r : b_rows - 1;              // the rows are masked at the store
-        a_off[it] = unsigned(ra) * unsigned(g.K) + unsigned(kc * 16);
-        b_off[it] = unsigned(rb) * unsigned(g.K) + unsigned(kc * 16);
+    for (int it = 0; it < PA; ++it) {
+        int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
+        r = r < a_rows ? r : a_rows - 1;  // clamp: reads stay in bounds, rows are masked at the store
+        a_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
+    }
+#pragma unroll
+    for (int it = 0; it < PB; ++it) {
+        int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
+        r = r < b_rows ? r : b_rows - 1;
+        b_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
     }
     const int8_t* a_tile = g.a + size_t(m0) * g.K;
     const int8_t* b_tile = g.w + size_t(n0) * g.K;
 
     auto load_stage = [&](int k0, int8_t* stage) {
-        const bool in_k = (k0 + kc * 16) < g.K;
+        const bool in_k = (k0 + kc * 16) < g.K;  // K-tail chunks and look-ahead stages: zeros
         int8_t* sa = stage + wave * 1024;
         int8_t* sb = stage + BM * BK + wave * 1024;
 #pragma unroll
-        for (int it = 0; it < kPasses; ++it) {
+        for (int it = 0; it < PA; ++it) {
             const int8_t* src = in_k ? a_tile + k0 + a_off[it] : g.zeros;
-            __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * 4096), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
         }
 #pragma unroll
-        for (int it = 0; it < kPasses; ++it) {
+        for (int it = 0; it < PB; ++it) {
             const int8_t* src = in_k ? b_tile + k0 + b_off[it] : g.zeros;
-            __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sb + it * 4096), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sb + it * (THREADS * 16)), 16, 0, 0);
         }
     };
 
-    v16i acc[4][4];
+    v16i acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
@@ -197,62 +314,134 @@ __global__ __launch_bounds__(kTileThreads, 1) void qgemm_tile_kernel(GemmArgs g)
     // 2*kk + (lane >> 5) of the current 32-wide k step
     const int frag_row = lane & 31;
     const int frag_half = lane >> 5;
-    const int a_row_base = (wm * 128 + frag_row) * BK;
-    const int b_row_base = BM * BK + (wn * 128 + frag_row) * BK;
-    const int sw = frag_row & 7;
+    const int a_row_base = (wm * (TM * 32) + frag_row) * BK;
+    const int b_row_base = BM * BK + (wn * (TN * 32) + frag_row) * BK;
+    const int sw = (frag_row / R) % C;
 
+    auto read_frags = [&](const int8_t* stage, int kk, v4i (&af)[TM], v4i (&bf)[TN]) {
+        const int pc = ((kk * 2 + frag_half) ^ sw) * 16;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            af[i] = *reinterpret_cast<const v4i*>(stage + a_row_base + i * 32 * BK + pc);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            bf[j] = *reinterpret_cast<const v4i*>(stage + b_row_base + j * 32 * BK + pc);
+    };
+
+    // ---- main loop.  All STAGES buffers are kept in flight.  The fragments
+    // of k step kk+1 are fetched from LDS while the MFMAs of step kk run; the
+    // hand-over to the next stage (wait for its data, barrier, fetch its first
+    // fragments, refill the buffer just drained) sits inside the last k step
+    // of the current stage, so its latency is covered by that step's MFMAs.
+    // Stages past the end of K are loaded from the block of zeros, which keeps
+    // the number of outstanding loads - and so the vmcnt to wait for - constant.
     const int nk = (g.K + BK - 1) / BK;
-    load_stage(0, smem);
-    __builtin_amdgcn_s_waitcnt(0);
+#pragma unroll
+    for (int s = 0; s < STAGES; ++s) load_stage(s * BK, smem + s * Cfg::STAGE_BYTES);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 1) * (PA + PB)));
     __syncthreads();
 
-    for (int t = 0; t < nk; ++t) {
-        int8_t* cur = smem + (t & 1) * kStageBytes;
-        if (t + 1 < nk) load_stage((t + 1) * BK, smem + ((t + 1) & 1) * kStageBytes);
-#pragma unroll
-        for (int kk = 0; kk < BK / 32; ++kk) {
-            const int pc = ((kk * 2 + frag_half) ^ sw) * 16;
-            v4i af[4], bf[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                af[i] = *reinterpret_cast<const v4i*>(cur + a_row_base + i * 32 * BK + pc);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                bf[j] = *reinterpret_cast<const v4i*>(cur + b_row_base + j * 32 * BK + pc);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-    }
+    v4i af[2][TM], bf[2][TN];
+    read_frags(smem, 0, af[0], bf[0]);
 
-    // ---- epilogue.  acc[i][j][r] is row 8*(r/4) + 4*(lane>>5) + r%4, column lane&31
+    auto k_steps = [&](int t, bool last_stage) {
+        const int slot = t % STAGES;
+        int8_t* cur = smem + slot * Cfg::STAGE_BYTES;
+        const int8_t* nxt = smem + (slot + 1 == STAGES ? 0 : slot + 1) * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < KSTEPS; ++kk) {
+            if (kk + 1 < KSTEPS) {
+                read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+            } else if (!last_stage) {
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * (PA + PB)));
+                __syncthreads();  // stage t+1 is complete in LDS; nobody reads stage t any more
+                read_frags(nxt, 0, af[0], bf[0]);
+                load_stage((t + STAGES) * BK, cur);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[kk & 1][i], bf[kk & 1][j],
+                                                                      acc[i][j], 0, 0, 0);
+            // issue order inside the step: one MFMA, one LDS read, ... then the rest of the
+            // MFMAs.  The MFMA goes first so that the wait for the previous step's
+            // fragments is not held up by a read issued just before it.
+            if (kk + 1 < KSTEPS || !last_stage) {
+#pragma unroll
+                for (int x = 0; x < TM + TN; ++x) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for (int t = 0; t + 1 < nk; ++t) k_steps(t, false);
+    k_steps(nk - 1, true);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the zero-filled look-ahead stages
+    __syncthreads();                            // all fragment reads done before LDS is reused below
+
+    // ---- epilogue.  Row scales are staged in LDS and column parameters are
+    // loaded before the first store, so no global load sits between the stores.
+    float* s_as = reinterpret_cast<float*>(smem);
+    uint32_t* stage = reinterpret_cast<uint32_t*>(smem + 4 * BM) + wave * Cfg::STAGE_WORDS;
+    for (int rr = tid; rr < BM; rr += THREADS) {
+        const int m = m0 + rr;
+        float v = 1.0f;
+        if (g.a_scale) v = g.a_scale[(g.a_scale_per_row && m < g.M) ? m : 0];
+        s_as[rr] = v;
+    }
     float S = 1.0f, Z = 0.0f;
-    if (g.out_mode == OUT_REQUANT_I8 || g.out_mode == OUT_FAKEQUANT_F32) {
+    if (MODE == OUT_REQUANT_I8 || MODE == OUT_FAKEQUANT_F32) {
         S = g.out_scale[0];
         Z = g.out_zp[0];
     }
-    const float as_uniform = g.a_scale ? g.a_scale[0] : 1.0f;
+    ColParams cp[TN];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int n = n0 + wn * 128 + j * 32 + (lane & 31);
-        if (n >= g.N) continue;
-        const ColParams c = load_col(g, n);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int mb = m0 + wm * 128 + i * 32 + 4 * (lane >> 5);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = mb + 8 * (r >> 2) + (r & 3);
-                if (m < g.M) {
-                    const float as = g.a_scale_per_row ? g.a_scale[m] : as_uniform;
-                    epilogue_store(g, m, n, acc[i][j][r], as, c, S, Z);
-                }
-            }
-        }
+    for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+        cp[j] = load_col(g, n < g.N ? n : g.N - 1);
+    }
+    __syncthreads();
+    tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, wm, wn, lane, S, Z);
+}
+
+// Tile shapes.  "big" keeps LDS traffic per MFMA lowest (one block per CU);
+// "wide" and "mid" let two or more blocks share a CU so one block's barrier
+// and epilogue overlap another's MFMAs, and waste less on ragged M / N.
+using CfgBig = TileCfg<256, 256, 128, 2, 2, 2, 1>;
+using CfgBig64 = TileCfg<256, 256, 64, 2, 2, 4, 1>;
+using CfgWide = TileCfg<256, 128, 64, 2, 2, 3, 2>;
+using CfgTall = TileCfg<128, 256, 64, 2, 2, 3, 2>;
+using CfgMid = TileCfg<128, 128, 64, 2, 2, 4, 2>;
+
+template <class Cfg, int MODE>
+int launch_tile_mode(const GemmArgs& g, hipStream_t st) {
+    const void* fn = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE>);
+    static bool attr_set = false;
+    if (!attr_set) {
+        LQ_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
+        attr_set = true;
+    }
+    const int tiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
+    GemmArgs copy = g;
+    void* kargs[] = {&copy};
+    LQ_HIP(hipLaunchKernel(fn, dim3(tiles), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
+    return LQ_OK;
+}
+
+template <class Cfg>
+int launch_tile(const GemmArgs& g, hipStream_t st) {
+    LQ_REQUIRE(size_t(Cfg::BM > Cfg::BN ? Cfg::BM : Cfg::BN) * g.K < 0xffffffffull, LQ_ERR_SHAPE,
+               "qlinear_i8: K too large");
+    switch (g.out_mode) {
+    case OUT_ACC_I32: return launch_tile_mode<Cfg, OUT_ACC_I32>(g, st);
+    case OUT_F32: return launch_tile_mode<Cfg, OUT_F32>(g, st);
+    case OUT_F16: return launch_tile_mode<Cfg, OUT_F16>(g, st);
+    case OUT_REQUANT_I8: return launch_tile_mode<Cfg, OUT_REQUANT_I8>(g, st);
+    default: return launch_tile_mode<Cfg, OUT_FAKEQUANT_F32>(g, st);
     }
 }
 
@@ -454,18 +643,25 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
     LQ_REQUIRE(path == 3 || vec_ok, LQ_ERR_VALUE,
                "qlinear_i8: MFMA paths need K %% 16 == 0 and 16-byte aligned operands");
     if (path == 1) {
-        LQ_REQUIRE(size_t(BM) * p->K < 0xffffffffull, LQ_ERR_SHAPE, "qlinear_i8: K too large");
         int rc = zero_block(&g.zeros);
         if (rc) return rc;
-        static bool attr_set = false;
-        if (!attr_set) {
-            LQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(qgemm_tile_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kTileSmem));
-            attr_set = true;
+        int cfg = p->tile_config;
+        if (cfg == 0) {
+            // 128 x 256 tiles keep two blocks per CU busy and measured fastest from
+            // M = 2048 to 8192 at N = 11008; fall back to 128 x 128 when that would
+            // leave most of the 256 CUs without a tile.
+            const long tiles_tall = long((p->M + 127) / 128) * ((p->N + 255) / 256);
+            cfg = tiles_tall >= 256 ? 4 : 5;
         }
-        const int tiles = ((p->M + BM - 1) / BM) * ((p->N + BN - 1) / BN);
-        hipLaunchKernelGGL(qgemm_tile_kernel, dim3(tiles), dim3(kTileThreads), kTileSmem, st, g);
-        LQ_CHECK_LAUNCH("qgemm_tile");
+        switch (cfg) {
+        case 1: rc = launch_tile<CfgBig>(g, st); break;
+        case 2: rc = launch_tile<CfgBig64>(g, st); break;
+        case 3: rc = launch_tile<CfgWide>(g, st); break;
+        case 4: rc = launch_tile<CfgTall>(g, st); break;
+        case 5: rc = launch_tile<CfgMid>(g, st); break;
+        default: rc = launch_tile<CfgBig>(g, st); break;
+        }
+        if (rc) return rc;
     } else if (path == 2) {
         LQ_REQUIRE(p->M <= 64, LQ_ERR_SHAPE, "qlinear_i8: skinny path needs M <= 64 (M = %d)", p->M);
         dim3 grid{unsigned((p->N + 15) / 16)}, block{256};

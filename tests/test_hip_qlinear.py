@@ -42,6 +42,24 @@ def test_accumulators_exact(M, N, K, path):
     assert np.array_equal(acc, O.igemm(a, w))
 
 
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 260, 144), (129, 77, 784), (513, 1000, 576),
+                                   (2048, 512, 4096), (1, 16, 16), (700, 130, 64)])
+def test_every_tile_shape_exact(cfg, M, N, K):
+    rng = np.random.default_rng(cfg * 1000 + M + N + K)
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    acc = _ops.qlinear_i8(hip(a), hip(w), out_mode=_ops.OUT_ACC_I32, path=TILE,
+                          tile_config=cfg).numpy()
+    assert np.array_equal(acc, O.igemm(a, w))
+    a_scale = rng.uniform(0.005, 0.05, M).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    got = _ops.qlinear_i8(hip(a), hip(w), a_scale=hip(a_scale), w_scale=hip(w_scale),
+                          bias=hip(bias), out_mode=_ops.OUT_F16, path=TILE, tile_config=cfg).numpy()
+    exp = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, out_mode=O.OUT_F16)
+    assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+
+
 @pytest.mark.parametrize("path,M", [(TILE, 300), (SKINNY, 16), (NAIVE, 9)])
 def test_extreme_codes(path, M):
     K, N = 4096, 48
