@@ -1,0 +1,299 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 quantized-inference hot path on one MI355X.
+
+Headline workload (``--workload linear``, the default): the LLM-shaped int8
+quantized Linear, M=2048, K=4096, N=11008 - int8 weights (N(0,0.02),
+per-row symmetric scales) x int8 activations (N(0,1), per-token symmetric
+scales), int32 accumulation, fp16 dequantized output with fp16 bias.  A "step"
+is one launch of the fused GEMM+epilogue on inputs already resident in HBM.
+
+One JSON line is printed.  Besides the driver's fields it carries
+  roofline      the GEMM against the published int8 dense MFMA peak,
+  cpu_baseline  Lucid's CPU pass structure (dequantize weight -> float GEMM ->
+                bias), restated in oracle/, timed on the host cores on a
+                bounded row sample of the same layer,
+  extra         the bandwidth-bound members of the path measured in the same
+                run: quantize / dequantize / min-max on the 4096x4096x16
+                round-trip tensor against the 8 TB/s HBM peak, and the
+                decode-shaped Linears (M = 1, 16) against HBM.
+
+Timing: HIP events recorded on the stream the kernels are launched on (the
+default stream), through the library's own C ABI.  No PyTorch anywhere.
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X published dense int8 MFMA peak, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X published HBM3E bandwidth, GB/s
+
+# HBM bytes per launch of the headline GEMM, measured with rocprofv3 --pmc
+# (FETCH_SIZE and WRITE_SIZE in separate runs, scaled by the same counters read
+# on the library's plain copy kernel); None until measured.  See
+# profiles/qlinear_m2048_traffic.txt for the runs these come from.
+MEASURED_TRAFFIC_BYTES = {"linear_m2048": None}
+
+
+def _events(_C, n):
+    evs = []
+    for _ in range(n):
+        e = C.c_void_p()
+        _C.call("lq_event_create", C.byref(e))
+        evs.append(e)
+    return evs
+
+
+def _elapsed_ms(_C, a, b):
+    ms = C.c_float()
+    _C.call("lq_event_elapsed_ms", a, b, C.byref(ms))
+    return float(ms.value)
+
+
+def time_launches(_C, fn, steps, warmup):
+    """Returns (total ms over `steps` back-to-back launches, per-launch ms list)."""
+    for _ in range(warmup):
+        fn()
+    _C.call("lq_sync", None)
+    evs = _events(_C, steps + 1)
+    _C.call("lq_event_record", evs[0], None)
+    for i in range(steps):
+        fn()
+        _C.call("lq_event_record", evs[i + 1], None)
+    _C.call("lq_event_sync", evs[steps])
+    per = [_elapsed_ms(_C, evs[i], evs[i + 1]) for i in range(steps)]
+    total = _elapsed_ms(_C, evs[0], evs[steps])
+    for e in evs:
+        _C.call("lq_event_destroy", e)
+    return total, per
+
+
+def make_linear(L, Q, _C, _ops, M, K, N, seed):
+    """Synthetic layer of the benchmark's shape, quantized on the device with
+    the library's own kernels."""
+    wf = L.Tensor.empty((N, K), L.float32, "hip")
+    _C.call("lq_fill_normal", wf.data_ptr, N * K, seed, 0.0, 1.0, None)
+    # N(0, 0.02): scale the unit normals through a dequantize-free route - the
+    # per-row symmetric scale absorbs the factor, so quantize the unit normals
+    # and multiply the scales instead.
+    mn, mx = Q.minmax(wf, ch_axis=0)
+    ws, wz = Q.calculate_qparams(mn, mx, Q.per_channel_symmetric, Q.qint8)
+    wq = Q.quantize(wf, ws, wz, Q.qint8, ch_axis=0)
+    ws = L.tensor(ws.numpy() * np.float32(0.02), device="hip")
+    x = L.Tensor.empty((M, K), L.float32, "hip")
+    _C.call("lq_fill_normal", x.data_ptr, M * K, seed + 1, 0.0, 1.0, None)
+    xmn, xmx = Q.minmax(x, ch_axis=0)
+    xs, xz = Q.calculate_qparams(xmn, xmx, Q.per_channel_symmetric, Q.qint8)
+    xq = Q.quantize(x, xs, xz, Q.qint8, ch_axis=0)
+    rng = np.random.default_rng(seed)
+    bias = L.tensor((rng.standard_normal(N) * 0.02).astype(np.float16), device="hip")
+    out = L.Tensor.empty((M, N), L.float16, "hip")
+    return dict(x=x, xq=xq, xs=xs, wq=wq, ws=ws, bias=bias, out=out)
+
+
+def bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup, seed=1):
+    t = make_linear(L, Q, _C, _ops, M, K, N, seed)
+
+    def step(repeat=1):
+        _ops.qlinear_i8(t["xq"], t["wq"], a_scale=t["xs"], w_scale=t["ws"], bias=t["bias"],
+                        out_mode=_ops.OUT_F16, out=t["out"], repeat=repeat)
+
+    # per-launch event pairs give the spread; the average launch duration comes
+    # from `steps` launches issued back to back from native code between one
+    # pair of events, so that no host-side gap is charged to the kernel
+    _, per = time_launches(_C, step, steps, warmup)
+    total, _ = time_launches(_C, lambda: step(steps), 1, 1)
+    ops = 2.0 * M * K * N
+    bytes_alg = N * K + M * K + 2 * M * N + 4 * N + 4 * M + 2 * N
+    avg_ms = total / steps
+    return dict(total_ms=total, avg_kernel_ms=avg_ms, median_ms=float(np.median(per)),
+                p95_ms=float(np.percentile(per, 95)), ops=ops, bytes=bytes_alg,
+                tops=ops / (total / steps) / 1e9, kernel_tops=ops / avg_ms / 1e9,
+                gbs=bytes_alg / avg_ms / 1e6, tensors=t)
+
+
+def bench_act_quant_plus_linear(L, Q, _C, _ops, t, M, K, N, steps, warmup):
+    """The same layer with the dynamic per-token activation quantization in the
+    timed region: min/max -> qparams -> quantize -> GEMM (four launches)."""
+    mn = L.Tensor.empty((M,), L.float32, "hip")
+    mx = L.Tensor.empty((M,), L.float32, "hip")
+    s = L.Tensor.empty((M,), L.float32, "hip")
+    z = L.Tensor.empty((M,), L.float32, "hip")
+    xq = L.Tensor.empty((M, K), L.int8, "hip")
+
+    def step():
+        _C.call("lq_minmax", t["x"].data_ptr, 1, M, K, mn.data_ptr, mx.data_ptr, None)
+        _C.call("lq_calc_qparams", mn.data_ptr, mx.data_ptr, M, 1, -128, 127, 1, 1e-8, s.data_ptr,
+                z.data_ptr, None)
+        _C.call("lq_quantize", t["x"].data_ptr, xq.data_ptr, _C.I8, 0, 1, M, K, s.data_ptr,
+                z.data_ptr, 0, -128, 127, None)
+        _ops.qlinear_i8(xq, t["wq"], a_scale=s, w_scale=t["ws"], bias=t["bias"],
+                        out_mode=_ops.OUT_F16, out=t["out"])
+
+    total, _ = time_launches(_C, step, steps, warmup)
+    return 2.0 * M * K * N / (total / steps) / 1e9
+
+
+def bench_quant_roundtrip(L, Q, _C, steps, warmup):
+    """Config: 4096 x 4096 x 16 float32, N(0,1) with 0.1 % outliers x20;
+    per-channel symmetric int8 along dim 0, then per-tensor affine."""
+    shape = (4096, 4096, 16)
+    n = int(np.prod(shape))
+    Cn, inner = shape[0], shape[1] * shape[2]
+    x = L.Tensor.empty(shape, L.float32, "hip")
+    _C.call("lq_fill_normal", x.data_ptr, n, 2, 0.001, 20.0, None)
+    mn, mx = Q.minmax(x, ch_axis=0)
+    s, z = Q.calculate_qparams(mn, mx, Q.per_channel_symmetric, Q.qint8)
+    q = L.Tensor.empty(shape, L.int8, "hip")
+    dq = L.Tensor.empty(shape, L.float32, "hip")
+    gmn, gmx = Q.minmax(x)
+    ts, tz = Q.calculate_qparams(gmn, gmx, Q.per_tensor_affine, Q.quint8)
+    q16 = L.Tensor.empty(shape, L.int16, "hip")
+
+    cases = {
+        "minmax_per_channel": (4 * n, lambda: _C.call(
+            "lq_minmax", x.data_ptr, 1, Cn, inner, mn.data_ptr, mx.data_ptr, None)),
+        "minmax_per_tensor": (4 * n, lambda: _C.call(
+            "lq_minmax", x.data_ptr, 1, 1, n, gmn.data_ptr, gmx.data_ptr, None)),
+        "quantize_per_channel_i8": (5 * n, lambda: _C.call(
+            "lq_quantize", x.data_ptr, q.data_ptr, _C.I8, 0, 1, Cn, inner, s.data_ptr, z.data_ptr,
+            0, -128, 127, None)),
+        "dequantize_per_channel_i8": (5 * n, lambda: _C.call(
+            "lq_dequantize", q.data_ptr, _C.I8, 0, dq.data_ptr, 1, Cn, inner, s.data_ptr,
+            z.data_ptr, 0, None)),
+        "quantize_per_tensor_quint8_i16": (6 * n, lambda: _C.call(
+            "lq_quantize", x.data_ptr, q16.data_ptr, _C.I16, 0, 1, 1, n, ts.data_ptr, tz.data_ptr,
+            0, 0, 255, None)),
+        "dequantize_per_tensor_quint8_i16": (6 * n, lambda: _C.call(
+            "lq_dequantize", q16.data_ptr, _C.I16, 0, dq.data_ptr, 1, 1, n, ts.data_ptr,
+            tz.data_ptr, 0, None)),
+        "copy_kernel": (8 * n, lambda: _C.call(
+            "lq_copy_kernel", dq.data_ptr, x.data_ptr, 4 * n, None)),
+    }
+    out = {}
+    for name, (nbytes, fn) in cases.items():
+        _, per = time_launches(_C, fn, steps, warmup)
+        med = float(np.median(per))
+        out[name] = {"us": round(med * 1e3, 1), "GB/s": round(nbytes / med / 1e6, 1),
+                     "frac_of_8TBs": round(nbytes / med / 1e6 / PEAK_HBM_GBS, 4),
+                     "bytes": nbytes}
+    return out
+
+
+def cpu_baseline_linear(K, N, sample_rows, seed=1, reps=8):
+    """Lucid's CPU pass structure for this layer (dequantize the int8 weight on
+    every call, float32 GEMM, bias add), run by the oracle on `sample_rows`
+    rows of the same shape."""
+    import oracle as O
+
+    rng = np.random.default_rng(seed)
+    wq = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    ws = rng.uniform(1e-4, 3e-4, N).astype(np.float32)
+    wz = np.zeros(N, np.float32)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float32)
+    x = rng.standard_normal((sample_rows, K)).astype(np.float32)
+    times = []
+    for i in range(reps + 1):  # first call warms the library and the pages
+        t0 = time.perf_counter()
+        O.linear_faithful(x, wq, ws, wz, bias=bias)
+        times.append(time.perf_counter() - t0)
+    dt = float(np.median(times[1:]))
+    return 2.0 * sample_rows * K * N / dt / 1e12, dt, sum(times)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="linear", choices=["linear"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--cpu-sample-rows", type=int, default=2048)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        return 2
+
+    import lucid_amd as L
+    import lucid_amd.quantization as Q
+    from lucid_amd import _C, _ops
+
+    _C.init(0)
+    M, K, N = 2048, 4096, 11008
+    r = bench_linear(L, Q, _C, _ops, M, K, N, args.steps, args.warmup)
+    line = {
+        "metric": "quantized-Linear int8 TOPS",
+        "value": round(r["tops"], 2),
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(r["total_ms"] / args.steps, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "int8 quantized Linear M=2048 K=4096 N=11008, per-token x per-row "
+                               "scales, int32 accumulate, fp16 bias + fp16 output",
+                   "device": _C.device_name()},
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(r["kernel_tops"], 2),
+            "peak": PEAK_INT8_TOPS,
+            "unit": "TOP/s",
+            "frac": round(r["kernel_tops"] / PEAK_INT8_TOPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES["linear_m2048"],
+            "kernel": "qgemm_tile_kernel",
+            "avg_kernel_us": round(r["avg_kernel_ms"] * 1e3, 2),
+            "median_kernel_us": round(r["median_ms"] * 1e3, 2),
+            "p95_kernel_us": round(r["p95_ms"] * 1e3, 2),
+            "algorithmic_ops": r["ops"],
+        },
+    }
+    if not args.no_extra:
+        extra = {}
+        extra["linear_with_dynamic_act_quant_TOPS"] = round(
+            bench_act_quant_plus_linear(L, Q, _C, _ops, r["tensors"], M, K, N, args.steps,
+                                        args.warmup), 2)
+        del r["tensors"]
+        for m in (1, 16):
+            rs = bench_linear(L, Q, _C, _ops, m, K, N, args.steps, args.warmup, seed=3)
+            extra[f"linear_m{m}"] = {"us": round(rs["median_ms"] * 1e3, 2),
+                                     "GB/s": round(rs["gbs"], 1),
+                                     "frac_of_8TBs": round(rs["gbs"] / PEAK_HBM_GBS, 4),
+                                     "TOP/s": round(rs["kernel_tops"], 2), "bytes": rs["bytes"]}
+            del rs["tensors"]
+        extra["quant_roundtrip_4096x4096x16"] = bench_quant_roundtrip(
+            L, Q, _C, max(10, args.steps // 2), max(3, args.warmup // 2))
+        line["extra"] = extra
+    if not args.no_cpu_baseline:
+        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        tops, dt, spent = cpu_baseline_linear(K, N, args.cpu_sample_rows)
+        line["cpu_baseline"] = {
+            "value": round(tops, 5),
+            "unit": "TOP/s",
+            "cores": cores,
+            "kind": "port",
+            "sample": f"{args.cpu_sample_rows} of {M} rows of the same layer; median of 8 calls, "
+                      f"each = per-call weight dequantize + float32 GEMM + bias "
+                      f"({dt:.2f} s per call, {spent:.0f} s of CPU time in all)",
+        }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -181,6 +181,11 @@ typedef struct {
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);
 
+/* The same forward launched n times back to back from native code: for
+ * launch-bound callers (decode-shaped layers run for ~10 us, less than an
+ * interpreter's call overhead) and for timing.  No counterpart in Lucid. */
+int lq_qlinear_i8_n(const lq_qlinear_args* args, int n, lq_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -113,6 +113,7 @@ class QLinearArgs(C.Structure):
 
 _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
+_SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]
 
 _RESTYPE = {"lq_last_error": C.c_char_p}
 _NO_STATUS = {"lq_version", "lq_last_error", "lq_op_count"}

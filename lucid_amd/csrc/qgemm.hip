@@ -597,6 +597,15 @@ int lq_rowsum_i8(const int8_t* w, int32_t* out, int N, int K, lq_stream stream) 
     return LQ_OK;
 }
 
+int lq_qlinear_i8_n(const lq_qlinear_args* p, int n, lq_stream stream) {
+    LQ_REQUIRE(n >= 0, LQ_ERR_VALUE, "qlinear_i8_n: negative repeat count");
+    for (int i = 0; i < n; ++i) {
+        int rc = lq_qlinear_i8(p, stream);
+        if (rc) return rc;
+    }
+    return LQ_OK;
+}
+
 int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
     LQ_REQUIRE(p, LQ_ERR_VALUE, "qlinear_i8: args is NULL");
     LQ_REQUIRE(p->M >= 0 && p->N >= 0 && p->K >= 0, LQ_ERR_SHAPE, "qlinear_i8: negative extent");
