@@ -132,6 +132,27 @@ int lq_fake_quantize(const float* x, float* out, size_t outer, size_t C, size_t 
                      const float* scale, const float* zp, int qparams_on_host, int qmin, int qmax,
                      lq_stream stream);
 
+/* ------------------------------------------------------- elementwise members */
+/* ReLU on float32 (IBackend::relu; CpuBackend vrelu_f32, Vdsp.cpp:130-133):
+ * the activation between dynamic-quantized layers, whose outputs are float. */
+int lq_relu_f32(const float* x, float* out, size_t n, lq_stream stream);
+
+/* Observer state update: out_min = minimum(run_min, cur_min), out_max =
+ * maximum(run_max, cur_max) over C channels (observer.py:370-371,652-653;
+ * IBackend::minimum/maximum, CpuBackend.h:828-864).  run_* may be the scalar
+ * +-inf seed broadcast over C (run_is_scalar != 0).  out_* may alias cur_*. */
+int lq_minmax_fold(const float* run_min, const float* run_max, const float* cur_min,
+                   const float* cur_max, size_t C, int run_is_scalar, float* out_min,
+                   float* out_max, lq_stream stream);
+
+/* QFunctional.add / add_relu on codes (nn/quantized/functional_module.py:216-230):
+ * out = quantize(relu?((qa - za)*sa + (qb - zb)*sb)) with every qparam a device
+ * scalar.  Codes are int8 as stored (code + offset). */
+int lq_add_requant_i8(const int8_t* qa, int a_offset, const float* a_scale, const float* a_zp,
+                      const int8_t* qb, int b_offset, const float* b_scale, const float* b_zp,
+                      size_t n, int relu, const float* out_scale, const float* out_zp, int out_qmin,
+                      int out_qmax, int out_offset, int8_t* out, lq_stream stream);
+
 /* ------------------------------------------------------- quantized Linear */
 /* Output forms of the fused GEMM epilogue. */
 #define LQ_OUT_ACC_I32 0       /* raw int32 accumulators                         */
@@ -162,7 +183,10 @@ typedef struct {
     const int8_t* w;
     int M, N, K;
     const int32_t* wsum;   /* [N], required when a_zp != 0                   */
-    int a_zp;
+    int a_zp;              /* zero point of the stored codes (host value)       */
+    const float* a_zp_dev; /* optional device scalar (a zero point computed on the
+                              device, as in nnqd.Linear): the effective zero
+                              point is (int)*a_zp_dev + a_zp                    */
     const float* a_scale;  /* [M] when a_scale_per_row, else [1]             */
     int a_scale_per_row;
     const float* w_scale;  /* [N]                                            */

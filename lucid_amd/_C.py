@@ -102,7 +102,7 @@ class QLinearArgs(C.Structure):
 
     _fields_ = [
         ("a", _vp), ("w", _vp), ("M", _i), ("N", _i), ("K", _i),
-        ("wsum", _vp), ("a_zp", _i),
+        ("wsum", _vp), ("a_zp", _i), ("a_zp_dev", _vp),
         ("a_scale", _vp), ("a_scale_per_row", _i), ("w_scale", _vp),
         ("bias", _vp), ("bias_dtype", _i), ("relu", _i), ("out_mode", _i),
         ("out_scale", _vp), ("out_zp", _vp),
@@ -111,6 +111,10 @@ class QLinearArgs(C.Structure):
     ]
 
 
+_SIGNATURES["lq_relu_f32"] = [_vp, _vp, _sz, _vp]
+_SIGNATURES["lq_minmax_fold"] = [_vp, _vp, _vp, _vp, _sz, _i, _vp, _vp, _vp]
+_SIGNATURES["lq_add_requant_i8"] = [_vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _sz, _i, _vp, _vp, _i, _i,
+                                    _i, _vp, _vp]
 _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
 _SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]

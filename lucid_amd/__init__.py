@@ -32,6 +32,8 @@ from ._tensor import (
     tensor,
 )
 from . import quantization
+from . import nn
+from . import backends
 
 __version__ = "0.1.0"
 

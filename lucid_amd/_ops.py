@@ -37,7 +37,8 @@ def rowsum_i8(w: Tensor) -> Tensor:
     return out
 
 
-def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_scale: Tensor | None = None,
+def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None = None,
+               a_scale: Tensor | None = None,
                w_scale: Tensor | None = None, wsum: Tensor | None = None,
                bias: Tensor | None = None, relu: bool = False, out_mode: int = OUT_F32,
                out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
@@ -56,6 +57,7 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_scale: Tensor | None = 
     args.M, args.N, args.K = M, N, K
     args.wsum = _ptr(wsum, "wsum", T.int32)
     args.a_zp = int(a_zp)
+    args.a_zp_dev = _ptr(a_zp_dev, "a_zp_dev", T.float32)
     args.a_scale = _ptr(a_scale, "a_scale", T.float32)
     args.a_scale_per_row = int(a_scale is not None and a_scale.numel != 1)
     if a_scale is not None and a_scale.numel not in (1, M):

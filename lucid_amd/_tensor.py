@@ -69,6 +69,26 @@ def _norm_device(device) -> str:
     return d
 
 
+class Grid:
+    """Quantization-grid tag of an activation.
+
+    Lucid carries a quantized activation as a *float* tensor that happens to
+    lie on its grid (``lucid/nn/quantized/linear.py:207-215``).  Here the same
+    value is carried as its int8 codes plus ``(scale, zero_point)``; the float
+    view ``(code - Z) * S`` is produced by ``lq_dequantize`` only when somebody
+    asks for it.  ``offset`` is what was added to the code when storing it
+    (-128 for ``quint8``, so the codes are valid signed MFMA operands).
+    ``layout`` is "plain" (same element order as the float view) or "nhwc"
+    (codes of an NCHW float tensor kept channel-last for the conv kernels).
+    """
+
+    __slots__ = ("codes", "scale", "zero_point", "qdtype", "offset", "zp_host", "layout")
+
+    def __init__(self, codes, scale, zero_point, qdtype, offset, zp_host=None, layout="plain"):
+        self.codes, self.scale, self.zero_point = codes, scale, zero_point
+        self.qdtype, self.offset, self.zp_host, self.layout = qdtype, offset, zp_host, layout
+
+
 class DeviceBuffer:
     """Owns one ``lq_alloc`` allocation; freed when the last reference dies."""
 
@@ -142,7 +162,32 @@ class Tensor:
     def data_ptr(self) -> int:
         if self.device != "hip":
             raise _C.DeviceMismatch("data_ptr: tensor is not on the hip device")
+        if self._buf is None:
+            self._materialize()
         return self._buf.ptr + self._offset
+
+    @staticmethod
+    def on_grid(shape, grid: "Grid") -> "Tensor":
+        """A float32 tensor whose value is given by codes on a grid; the float
+        storage is created on first use."""
+        t = Tensor(shape, float32, "hip", buf=None)
+        t._grid = grid
+        return t
+
+    def _materialize(self) -> None:
+        g = self._grid
+        if g is None:
+            raise _C.LucidError("tensor has no storage")
+        n = self.numel
+        buf = DeviceBuffer(n * 4)
+        if g.layout == "nhwc" and len(self.shape) == 4:
+            B, Cc, H, W = self.shape
+            _C.call("lq_dequantize_nhwc_to_nchw", g.codes.data_ptr, g.offset, buf.ptr, B, Cc, H, W,
+                    g.scale.data_ptr, g.zero_point.data_ptr, None)
+        else:
+            _C.call("lq_dequantize", g.codes.data_ptr, _C.I8, g.offset, buf.ptr, 1, 1, n,
+                    g.scale.data_ptr, g.zero_point.data_ptr, 0, None)
+        self._buf = buf
 
     @property
     def is_hip(self) -> bool:
@@ -204,10 +249,31 @@ class Tensor:
             raise _C.ShapeMismatch(f"cannot reshape {self.shape} to {tuple(shape)}")
         if self.device == "cpu":
             return Tensor(shape, self.dtype, "cpu", host=self._host.reshape(shape))
+        g = self._grid
+        if g is not None and g.layout == "plain":
+            # keep the grid tag: the codes are reshaped the same way
+            out = Tensor(shape, self.dtype, "hip", buf=self._buf, offset=self._offset)
+            out._grid = Grid(g.codes.reshape(shape), g.scale, g.zero_point, g.qdtype, g.offset,
+                             g.zp_host, "plain")
+            return out
+        if self._buf is None:
+            self._materialize()
         return Tensor(shape, self.dtype, "hip", buf=self._buf, offset=self._offset)
 
     def detach(self) -> "Tensor":
         return self
+
+    def clone(self) -> "Tensor":
+        if self.device == "cpu":
+            return Tensor(self.shape, self.dtype, "cpu", host=self._host.copy())
+        out = Tensor.empty(self.shape, self.dtype, "hip")
+        if self.nbytes:
+            _C.call("lq_d2d", out.data_ptr, self.data_ptr, self.nbytes, None)
+        return out
+
+    def __deepcopy__(self, memo) -> "Tensor":
+        # a device allocation has exactly one owner: copy the bytes, not the handle
+        return self.clone()
 
 
 def tensor(data, dtype=None, device="cpu") -> Tensor:

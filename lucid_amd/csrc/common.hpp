@@ -41,6 +41,6 @@ int workspace(size_t nbytes, void** ptr);
 
 inline hipStream_t as_stream(lq_stream s) { return reinterpret_cast<hipStream_t>(s); }
 
-inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+__host__ __device__ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace lq

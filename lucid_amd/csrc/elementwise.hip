@@ -1,0 +1,140 @@
+// Small elementwise members of the quantized path: float ReLU between
+// dynamic-quantized layers, running min/max folding for observers, and the
+// residual join on codes.
+#include "common.hpp"
+
+using namespace lq;
+
+namespace {
+
+// vrelu_f32 (lucid/_C/backend/cpu/Vdsp.cpp:130-133): (x < 0) ? 0 : x, NaN passes.
+__global__ __launch_bounds__(256) void relu_f32_kernel(const float* __restrict__ x,
+                                                       float* __restrict__ out, size_t n) {
+    size_t i = (size_t(blockIdx.x) * 256 + threadIdx.x) * 4;
+    const size_t stride = size_t(gridDim.x) * 256 * 4;
+    const bool vec = aligned16(x) && aligned16(out);
+    for (; i < n; i += stride) {
+        if (vec && i + 4 <= n) {
+            float4 v = *reinterpret_cast<const float4*>(x + i);
+            v.x = v.x < 0.0f ? 0.0f : v.x;
+            v.y = v.y < 0.0f ? 0.0f : v.y;
+            v.z = v.z < 0.0f ? 0.0f : v.z;
+            v.w = v.w < 0.0f ? 0.0f : v.w;
+            *reinterpret_cast<float4*>(out + i) = v;
+        } else {
+            for (size_t e = i; e < n && e < i + 4; ++e) out[e] = x[e] < 0.0f ? 0.0f : x[e];
+        }
+    }
+}
+
+// running = minimum(running, current), running = maximum(running, current)
+// with vDSP_vmin / vDSP_vmax semantics (NaN propagates, Vdsp.cpp:140-151);
+// `current` may be a single value broadcast over C (scalar seed, observer.py:649-651).
+__global__ void minmax_fold_kernel(float* run_min, float* run_max, const float* cur_min,
+                                   const float* cur_max, size_t C, int run_is_scalar,
+                                   float* out_min, float* out_max) {
+    size_t c = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const float rmn = run_min[run_is_scalar ? 0 : c], rmx = run_max[run_is_scalar ? 0 : c];
+    const float cmn = cur_min[c], cmx = cur_max[c];
+    const float qnan = __builtin_nanf("");
+    out_min[c] = (rmn != rmn || cmn != cmn) ? qnan : (rmn < cmn ? rmn : cmn);
+    out_max[c] = (rmx != rmx || cmx != cmx) ? qnan : (rmx > cmx ? rmx : cmx);
+}
+
+__device__ __forceinline__ float q_core(float x, float s, float z, float lo, float hi) {
+    float t = x / s;
+    float r = __builtin_rintf(t);
+    float u = r + z;
+    u = (u < lo) ? lo : ((u > hi) ? hi : u);
+    return u;
+}
+
+// fq(relu(x + y)) on codes (lucid/nn/quantized/functional_module.py:224-230):
+// x = (qa - za)*sa, y = (qb - zb)*sb, each a float32 step, then the usual requantize.
+__global__ __launch_bounds__(256) void add_requant_kernel(const int8_t* __restrict__ qa, int a_off,
+                                                          const float* sa, const float* za,
+                                                          const int8_t* __restrict__ qb, int b_off,
+                                                          const float* sb, const float* zb,
+                                                          size_t n, int relu, const float* S_,
+                                                          const float* Z_, float lo, float hi,
+                                                          int out_off, int8_t* __restrict__ out) {
+    const float s_a = sa[0], z_a = za[0], s_b = sb[0], z_b = zb[0], S = S_[0], Z = Z_[0];
+    size_t i = (size_t(blockIdx.x) * 256 + threadIdx.x) * 4;
+    const size_t stride = size_t(gridDim.x) * 256 * 4;
+    const bool vec = (reinterpret_cast<uintptr_t>(qa) | reinterpret_cast<uintptr_t>(qb) |
+                      reinterpret_cast<uintptr_t>(out)) % 4 == 0;
+    for (; i < n; i += stride) {
+        int8_t a[4], b[4], o[4];
+        const int cnt = n - i < 4 ? int(n - i) : 4;
+        if (vec && cnt == 4) {
+            *reinterpret_cast<uint32_t*>(a) = *reinterpret_cast<const uint32_t*>(qa + i);
+            *reinterpret_cast<uint32_t*>(b) = *reinterpret_cast<const uint32_t*>(qb + i);
+        } else {
+            for (int e = 0; e < cnt; ++e) { a[e] = qa[i + e]; b[e] = qb[i + e]; }
+        }
+        for (int e = 0; e < cnt; ++e) {
+            float xa = (float(int(a[e]) - a_off) - z_a) * s_a;
+            float xb = (float(int(b[e]) - b_off) - z_b) * s_b;
+            float y = xa + xb;
+            if (relu) y = (y < 0.0f) ? 0.0f : y;
+            float qv = q_core(y, S, Z, lo, hi);
+            o[e] = int8_t(((qv != qv) ? 0 : int(qv)) + out_off);
+        }
+        if (vec && cnt == 4)
+            *reinterpret_cast<uint32_t*>(out + i) = *reinterpret_cast<const uint32_t*>(o);
+        else
+            for (int e = 0; e < cnt; ++e) out[i + e] = o[e];
+    }
+}
+
+inline unsigned grid_for(size_t n, size_t per_block) {
+    size_t b = (n + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    return unsigned(b > 65536 ? 65536 : b);
+}
+
+}  // namespace
+
+extern "C" {
+
+int lq_relu_f32(const float* x, float* out, size_t n, lq_stream stream) {
+    if (n == 0) return LQ_OK;
+    LQ_REQUIRE(x && out, LQ_ERR_VALUE, "relu_f32: NULL pointer");
+    hipLaunchKernelGGL(relu_f32_kernel, dim3(grid_for(n, 1024)), dim3(256), 0, as_stream(stream), x, out,
+                       n);
+    LQ_CHECK_LAUNCH("relu_f32");
+    return LQ_OK;
+}
+
+int lq_minmax_fold(const float* run_min, const float* run_max, const float* cur_min,
+                   const float* cur_max, size_t C, int run_is_scalar, float* out_min,
+                   float* out_max, lq_stream stream) {
+    if (C == 0) return LQ_OK;
+    LQ_REQUIRE(run_min && run_max && cur_min && cur_max && out_min && out_max, LQ_ERR_VALUE,
+               "minmax_fold: NULL pointer");
+    hipLaunchKernelGGL(minmax_fold_kernel, dim3(unsigned((C + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), const_cast<float*>(run_min), const_cast<float*>(run_max),
+                       cur_min, cur_max, C, run_is_scalar, out_min, out_max);
+    LQ_CHECK_LAUNCH("minmax_fold");
+    return LQ_OK;
+}
+
+int lq_add_requant_i8(const int8_t* qa, int a_offset, const float* a_scale, const float* a_zp,
+                      const int8_t* qb, int b_offset, const float* b_scale, const float* b_zp,
+                      size_t n, int relu, const float* out_scale, const float* out_zp, int out_qmin,
+                      int out_qmax, int out_offset, int8_t* out, lq_stream stream) {
+    if (n == 0) return LQ_OK;
+    LQ_REQUIRE(qa && qb && out && a_scale && a_zp && b_scale && b_zp && out_scale && out_zp,
+               LQ_ERR_VALUE, "add_requant_i8: NULL pointer");
+    LQ_REQUIRE(out_qmin <= out_qmax && out_qmin + out_offset >= -128 && out_qmax + out_offset <= 127,
+               LQ_ERR_VALUE, "add_requant_i8: output grid [%d,%d] + offset %d does not fit int8",
+               out_qmin, out_qmax, out_offset);
+    hipLaunchKernelGGL(add_requant_kernel, dim3(grid_for(n, 1024)), dim3(256), 0, as_stream(stream), qa,
+                       a_offset, a_scale, a_zp, qb, b_offset, b_scale, b_zp, n, relu, out_scale, out_zp,
+                       float(out_qmin), float(out_qmax), out_offset, out);
+    LQ_CHECK_LAUNCH("add_requant_i8");
+    return LQ_OK;
+}
+
+}  // extern "C"

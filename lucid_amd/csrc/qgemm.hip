@@ -35,6 +35,7 @@ struct GemmArgs {
     int M, N, K;
     const int32_t* wsum;  // [N] sum_k w[n,k]; may be null when a_zp == 0
     int a_zp;             // zero point of the stored activation codes
+    const float* a_zp_dev; // optional device scalar: effective zero point = int(*a_zp_dev) + a_zp
     const float* a_scale; // [M] or [1]
     int a_scale_per_row;
     const float* w_scale; // [N]
@@ -59,7 +60,8 @@ struct ColParams {
 __device__ __forceinline__ ColParams load_col(const GemmArgs& g, int n) {
     ColParams c;
     c.ws = g.w_scale ? g.w_scale[n] : 1.0f;
-    c.corr = (g.wsum && g.a_zp != 0) ? g.a_zp * g.wsum[n] : 0;
+    const int zp = g.a_zp_dev ? int(g.a_zp_dev[0]) + g.a_zp : g.a_zp;
+    c.corr = (g.wsum && zp != 0) ? zp * g.wsum[n] : 0;
     if (g.bias == nullptr)
         c.bias = 0.0f;
     else if (g.bias_dtype == LQ_F16)
@@ -621,8 +623,8 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
     LQ_REQUIRE(ldo >= p->N, LQ_ERR_SHAPE, "qlinear_i8: ldo %ld < N %d", ldo, p->N);
     if (p->out_mode != OUT_ACC_I32) {
         LQ_REQUIRE(p->w_scale && p->a_scale, LQ_ERR_VALUE, "qlinear_i8: scale pointer is NULL");
-        LQ_REQUIRE(p->a_zp == 0 || p->wsum, LQ_ERR_VALUE,
-                   "qlinear_i8: a_zp = %d needs the weight row sums", p->a_zp);
+        LQ_REQUIRE((p->a_zp == 0 && p->a_zp_dev == nullptr) || p->wsum, LQ_ERR_VALUE,
+                   "qlinear_i8: a non-zero activation zero point needs the weight row sums");
         LQ_REQUIRE(p->bias == nullptr || p->bias_dtype == LQ_F32 || p->bias_dtype == LQ_F16,
                    LQ_ERR_DTYPE, "qlinear_i8: bias must be float32 or float16 (dtype %d)",
                    p->bias_dtype);
@@ -638,7 +640,7 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
 
     GemmArgs g;
     g.a = p->a; g.w = p->w; g.M = p->M; g.N = p->N; g.K = p->K;
-    g.wsum = p->wsum; g.a_zp = p->a_zp;
+    g.wsum = p->wsum; g.a_zp = p->a_zp; g.a_zp_dev = p->a_zp_dev;
     g.a_scale = p->a_scale; g.a_scale_per_row = p->a_scale_per_row; g.w_scale = p->w_scale;
     g.bias = p->bias; g.bias_dtype = p->bias_dtype; g.relu = p->relu; g.out_mode = p->out_mode;
     g.out_scale = p->out_scale; g.out_zp = p->out_zp;

@@ -1,0 +1,121 @@
+"""The slice of ``lucid.nn`` that the quantized-inference path touches.
+
+Float ``Linear`` / ``Conv2d`` here are parameter holders that ``from_float`` /
+``quantize_dynamic`` / ``convert`` read; their float forward is Lucid's CPU /
+Metal business and is not part of this backend (calling it raises).  ``ReLU``
+does compute: it sits between dynamic-quantized layers, whose outputs are float.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+from .. import _C
+from .. import _tensor as T
+from .._tensor import Tensor
+from .module import Module
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, int) else tuple(v)
+
+
+class Identity(Module):
+    def forward(self, x):
+        return x
+
+
+class Sequential(Module):
+    def __init__(self, *mods) -> None:
+        super().__init__()
+        for i, m in enumerate(mods):
+            self._modules[str(i)] = m
+
+    def __getitem__(self, i):
+        return list(self._modules.values())[i]
+
+    def __len__(self):
+        return len(self._modules)
+
+    def forward(self, x):
+        for m in self._modules.values():
+            x = m(x)
+        return x
+
+
+class Linear(Module):
+    """Float Linear as a parameter holder (``weight`` (out,in), ``bias`` (out,))."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True) -> None:
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        bound = 1.0 / np.sqrt(in_features)
+        rng = np.random.default_rng(in_features * 7919 + out_features)
+        self.register_buffer("weight", T.tensor(
+            rng.uniform(-bound, bound, (out_features, in_features)).astype(np.float32)))
+        self.register_buffer("bias", T.tensor(
+            rng.uniform(-bound, bound, out_features).astype(np.float32)) if bias else None)
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.Linear.forward is not part of the hip quantized-inference backend; "
+            "quantize the model (quantize_dynamic / convert) first")
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}"
+
+
+class Conv2d(Module):
+    """Float Conv2d as a parameter holder (``weight`` OIHW, ``bias`` (O,))."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, padding_mode="zeros") -> None:
+        super().__init__()
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride = _pair(kernel_size), _pair(stride)
+        self.dilation, self.groups = _pair(dilation), groups
+        self._padding_str = padding if isinstance(padding, str) else None
+        self.padding = (0, 0) if isinstance(padding, str) else _pair(padding)
+        self.padding_mode = padding_mode
+        fan_in = in_channels // groups * self.kernel_size[0] * self.kernel_size[1]
+        bound = 1.0 / np.sqrt(fan_in)
+        rng = np.random.default_rng(fan_in * 7919 + out_channels)
+        self.register_buffer("weight", T.tensor(rng.uniform(
+            -bound, bound, (out_channels, in_channels // groups, *self.kernel_size)).astype(np.float32)))
+        self.register_buffer("bias", T.tensor(
+            rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.Conv2d.forward is not part of the hip quantized-inference backend; "
+            "quantize the model (convert) first")
+
+
+def relu(x: Tensor) -> Tensor:
+    """``F.relu``.  On a grid-carried activation with a non-negative grid the
+    codes are clamped at the zero point instead of touching floats."""
+    if not isinstance(x, Tensor) or x.device != "hip":
+        raise _C.DeviceMismatch("relu: expected a tensor on the 'hip' device")
+    if x.dtype != T.float32:
+        raise _C.DtypeMismatch(f"relu expects float32, got {x.dtype}")
+    out = Tensor.empty(x.shape, T.float32, "hip")
+    _C.call("lq_relu_f32", x.data_ptr, out.data_ptr, x.numel, None)
+    return out
+
+
+class ReLU(Module):
+    def forward(self, x):
+        return relu(x)
+
+
+class Flatten(Module):
+    def __init__(self, start_dim: int = 1) -> None:
+        super().__init__()
+        self.start_dim = start_dim
+
+    def forward(self, x):
+        lead = x.shape[: self.start_dim]
+        return x.reshape(*lead, -1)
+
+
+from . import intrinsic, quantized  # noqa: E402  (sub-packages need the classes above)

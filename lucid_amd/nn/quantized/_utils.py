@@ -1,0 +1,89 @@
+"""Helpers shared by the quantized modules (``lucid/nn/quantized/_utils.py``)."""
+
+from __future__ import annotations
+
+import warnings
+
+import numpy as np
+
+from ... import _C, _ops
+from ... import _tensor as T
+from ..._tensor import Grid, Tensor
+from ...quantization._functional import quantize
+from ...quantization._qscheme import QDtype
+
+
+def storage_offset(qdtype: QDtype) -> int:
+    """What is added to a code so that it fits a signed int8 MFMA operand."""
+    if qdtype.bits > 8:
+        raise NotImplementedError(f"{qdtype!r} activations do not fit the int8 kernels")
+    return 0 if qdtype.signed else -(1 << (qdtype.bits - 1))
+
+
+def quantize_weight(mod) -> tuple[Tensor, Tensor, Tensor, int]:
+    """``(codes, scale, zero_point, ch_axis)`` of a float module's weight
+    (``_utils.py:27-55``): run the qconfig's weight observer over the static
+    weight, then ``quantize`` along its channel axis."""
+    weight = mod.weight.to("hip")
+    wobs = mod.qconfig.weight()
+    wobs(weight)
+    scale, zero_point = wobs.calculate_qparams()
+    qdtype, ch_axis = wobs.qdtype, wobs.ch_axis
+    axis = ch_axis if ch_axis is not None else 0
+    if qdtype.storage != "int8":
+        raise NotImplementedError(f"weights must quantize to int8 storage, got {qdtype!r}")
+    codes = quantize(weight, scale, zero_point, qdtype, ch_axis=ch_axis)
+    if ch_axis is None:  # per-tensor weight qparams: broadcast to one entry per output row
+        n = weight.shape[0]
+        scale = T.tensor(np.full(n, scale.item(), np.float32), device="hip")
+        zero_point = T.tensor(np.full(n, zero_point.item(), np.float32), device="hip")
+    return codes, scale, zero_point, axis
+
+
+def activation_qparams(mod) -> tuple[Tensor, Tensor, QDtype]:
+    """Output ``(scale, zero_point, qdtype)`` from a module's activation
+    observer (``_utils.py:58-79``), with Lucid's uncalibrated-observer warning."""
+    obs = mod.activation_post_process
+    min_val = getattr(obs, "min_val", None)
+    if min_val is not None and bool(np.isinf(min_val.numpy()).any()):
+        warnings.warn(
+            f"Quantizing {type(mod).__name__} whose activation observer never saw "
+            "data — run calibration through the prepared model before convert(), "
+            "or the quantized output collapses to a near-zero grid.",
+            stacklevel=3,
+        )
+    scale, zero_point = obs.calculate_qparams()
+    return scale.to("hip"), zero_point.to("hip"), obs.qdtype
+
+
+def require_symmetric_weight(zero_point: Tensor, what: str) -> None:
+    """The int8 kernels fold the activation zero point only; a non-zero weight
+    zero point would also need activation row sums."""
+    if np.any(zero_point.numpy() != 0):
+        raise NotImplementedError(
+            f"{what}: affine (non-zero zero_point) weights are not supported by the hip int8 "
+            "kernels; use a symmetric weight observer (Lucid's default)")
+
+
+def input_grid(x: Tensor, what: str) -> Grid:
+    if not isinstance(x, Tensor) or x.device != "hip":
+        raise _C.DeviceMismatch(f"{what}: input must be a tensor on the 'hip' device")
+    if x._grid is None:
+        raise NotImplementedError(
+            f"{what}: the input is a plain float tensor, not an activation on a quantization "
+            "grid. Feed it through nn.quantized.Quantize (QuantStub) first; the float-input "
+            "form of this layer is Lucid's dequantize-to-float path, which this backend does "
+            "not provide.")
+    return x._grid
+
+
+def zp_args(g: Grid) -> tuple[int, Tensor | None]:
+    """``(a_zp, a_zp_dev)`` for the GEMM / conv entry points: a host zero point
+    when it is known, otherwise the device scalar plus the storage offset."""
+    if g.zp_host is not None:
+        return int(g.zp_host) + g.offset, None
+    return g.offset, g.zero_point
+
+
+def host_scalar(t: Tensor) -> float:
+    return float(t.numpy().reshape(-1)[0])

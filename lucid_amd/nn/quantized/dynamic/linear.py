@@ -1,0 +1,92 @@
+"""Dynamic-quantized ``Linear`` on the hip int8 GEMM.
+
+Mirrors ``lucid/nn/quantized/dynamic/linear.py:64-124``: buffers
+``weight_int8`` / ``weight_scale`` / ``weight_zero_point`` / ``bias``,
+attribute ``act_qdtype = quint8``, ``from_float(mod, dtype=qint8)``.  Per
+forward: global min / max of the input -> affine qparams -> activation codes
+-> int8 GEMM -> float32 output (not requantized).  All four steps are device
+kernels; the activation zero point is read by the GEMM from device memory, so
+the forward never waits for the host.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+from .... import _C, _ops
+from .... import _tensor as T
+from ...._tensor import Tensor
+from ....quantization._functional import minmax, quantize
+from ....quantization._qparams import calculate_qparams
+from ....quantization._qscheme import QDtype, per_channel_symmetric, per_tensor_affine, qint8, quint8
+from ...module import Module
+from .._utils import require_symmetric_weight, storage_offset
+
+
+class Linear(Module):
+    def __init__(self, in_features: int, out_features: int, bias: bool = True) -> None:
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight_ch_axis = 0
+        self.act_qdtype: QDtype = quint8
+        self.register_buffer("weight_int8", T.tensor(
+            np.zeros((out_features, in_features), np.int8), device="hip"))
+        self.register_buffer("weight_scale", T.tensor(np.ones(out_features, np.float32), device="hip"))
+        self.register_buffer("weight_zero_point", T.tensor(
+            np.zeros(out_features, np.float32), device="hip"))
+        self.register_buffer("bias", T.tensor(np.zeros(out_features, np.float32), device="hip")
+                             if bias else None)
+        self._wsum = None
+
+    def _state_loaded(self, name: str) -> None:
+        if name == "weight_int8":
+            self._wsum = None
+        if name == "weight_zero_point":
+            require_symmetric_weight(self.weight_zero_point, "dynamic.Linear")
+
+    def forward(self, x: Tensor) -> Tensor:
+        if not isinstance(x, Tensor) or x.device != "hip":
+            raise _C.DeviceMismatch("dynamic.Linear: input must be a tensor on the 'hip' device")
+        if x.dtype != T.float32:
+            raise _C.DtypeMismatch(f"dynamic.Linear expects float32 input, got {x.dtype}")
+        K, N = self.in_features, self.out_features
+        if x.shape[-1] != K:
+            raise _C.ShapeMismatch(f"expected last dim {K}, got {x.shape}")
+        M = x.numel // K
+        qd = self.act_qdtype
+        mn, mx = minmax(x)
+        x_scale, x_zp = calculate_qparams(mn, mx, per_tensor_affine, qd)
+        off = storage_offset(qd)
+        xq = Tensor.empty((M, K), T.int8, "hip")
+        _C.call("lq_quantize", x.data_ptr, xq.data_ptr, _C.I8, off, 1, 1, x.numel,
+                x_scale.data_ptr, x_zp.data_ptr, 0, qd.quant_min, qd.quant_max, None)
+        if self._wsum is None:
+            self._wsum = _ops.rowsum_i8(self.weight_int8)
+        y = _ops.qlinear_i8(xq, self.weight_int8, a_zp=off, a_zp_dev=x_zp, a_scale=x_scale,
+                            w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias,
+                            out_mode=_ops.OUT_F32)
+        return y.reshape(*x.shape[:-1], N)
+
+    @classmethod
+    def from_float(cls, mod, dtype: QDtype = qint8) -> "Linear":
+        """Quantize a float ``Linear``'s weight, no calibration
+        (``dynamic/linear.py:101-120``)."""
+        from ....quantization.observer import PerChannelMinMaxObserver
+
+        qmod = cls(mod.in_features, mod.out_features, bias=mod.bias is not None)
+        weight = mod.weight.to("hip")
+        obs = PerChannelMinMaxObserver(ch_axis=0, qscheme=per_channel_symmetric, qdtype=dtype)
+        obs(weight)
+        scale, zero_point = obs.calculate_qparams()
+        if dtype.storage != "int8":
+            raise NotImplementedError(f"dynamic.Linear weights must use int8 storage, got {dtype!r}")
+        qmod.register_buffer("weight_int8", quantize(weight, scale, zero_point, dtype, ch_axis=0))
+        qmod.register_buffer("weight_scale", scale)
+        qmod.register_buffer("weight_zero_point", zero_point)
+        if mod.bias is not None:
+            qmod.register_buffer("bias", mod.bias.to("hip"))
+        return qmod
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, dynamic=True"

@@ -1,0 +1,25 @@
+"""Fused quantized layers (``lucid/nn/quantized/intrinsic.py``): the ReLU runs
+before the output requantize, inside the kernel epilogue."""
+
+from __future__ import annotations
+
+from .linear import Linear
+
+
+class LinearReLU(Linear):
+    """Quantized ``Linear`` + ``ReLU`` (``intrinsic.py:23-37,131-138``)."""
+
+    _fused_relu = True
+
+    def _activation(self, y):
+        from .. import relu
+        return relu(y)
+
+    @classmethod
+    def from_float(cls, mod) -> "LinearReLU":
+        # an nni.LinearReLU is a Sequential(Linear, ReLU) that carries the qconfig
+        # and the activation observer of the fused pair
+        inner = mod[0]
+        inner.qconfig = mod.qconfig
+        inner.activation_post_process = mod.activation_post_process
+        return super().from_float(inner)

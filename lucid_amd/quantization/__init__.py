@@ -18,7 +18,22 @@ from ._qscheme import (
     quint8,
 )
 
+from .observer import (FixedQParamsObserver, MinMaxObserver, ObserverBase,
+                       PerChannelMinMaxObserver)
+from .qconfig import QConfig, get_default_qconfig
+
+
+def __getattr__(name):
+    # the workflow functions import lucid_amd.nn, which imports this package
+    if name in ("prepare", "convert", "quantize_dynamic"):
+        from . import _quantize
+        return getattr(_quantize, name)
+    raise AttributeError(name)
+
+
 __all__ = [
+    "ObserverBase", "MinMaxObserver", "PerChannelMinMaxObserver", "FixedQParamsObserver",
+    "QConfig", "get_default_qconfig", "prepare", "convert", "quantize_dynamic",
     "QScheme", "per_tensor_affine", "per_tensor_symmetric", "per_channel_affine",
     "per_channel_symmetric", "QDtype", "qint8", "quint8", "qint32", "qint4", "QParams",
     "calculate_qparams", "quantize", "dequantize", "fake_quantize", "minmax",

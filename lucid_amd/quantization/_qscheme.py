@@ -44,6 +44,13 @@ class QDtype:
     def __repr__(self) -> str:
         return f"lucid.quantization.{self.name}"
 
+    # grid descriptors are singletons (code compares them with ``is``)
+    def __copy__(self) -> "QDtype":
+        return self
+
+    def __deepcopy__(self, memo) -> "QDtype":
+        return self
+
 
 qint8: QDtype = QDtype("qint8", 8, True, -128, 127, "int8")
 quint8: QDtype = QDtype("quint8", 8, False, 0, 255, "int16")

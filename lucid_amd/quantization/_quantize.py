@@ -1,0 +1,125 @@
+"""Model-level workflow: ``prepare`` / ``convert`` / ``quantize_dynamic``
+(``lucid/quantization/_quantize.py:204-311,314-419,429-554,684-699``).
+
+Same control flow and warning texts as Lucid.  ``convert`` installs the hip
+int8 modules; calibration itself (a float forward through the prepared model)
+belongs to Lucid's float backends, so observers here are fed either by that
+float model's activations moved to ``"hip"`` or through fixed qparams.
+"""
+
+from __future__ import annotations
+
+import copy
+import warnings
+
+from .. import nn
+from ..nn import intrinsic as nni
+from ..nn import quantized as nnq
+from ..nn.quantized import dynamic as nnqd
+from ._qscheme import QDtype, qint8
+from .qconfig import QConfig, get_default_qconfig
+
+
+def _observed_types() -> tuple[type, ...]:
+    return (nn.Linear, nn.Conv2d, nni.LinearReLU, nni.ConvReLU2d, nnq.QuantStub,
+            nnq.FloatFunctional)
+
+
+def _quant_mapping() -> dict[type, object]:
+    m = {
+        nn.Linear: nnq.Linear.from_float,
+        nni.LinearReLU: nnq.LinearReLU.from_float,
+        nnq.QuantStub: nnq.Quantize.from_float,
+        nnq.DeQuantStub: nnq.DeQuantize.from_float,
+        nnq.FloatFunctional: nnq.QFunctional.from_float,
+    }
+    if hasattr(nnq, "Conv2d"):
+        m[nn.Conv2d] = nnq.Conv2d.from_float
+        m[nni.ConvReLU2d] = nnq.ConvReLU2d.from_float
+    return m
+
+
+def _dynamic_mapping() -> dict[type, object]:
+    return {nn.Linear: nnqd.Linear.from_float}
+
+
+def _make_observer_hook(obs):
+    def hook(_module, _args, output):
+        obs(output)
+    return hook
+
+
+def prepare(model, qconfig: QConfig | None = None, inplace: bool = False):
+    """Attach an activation observer (as a forward hook) and the ``qconfig`` to
+    every quantizable module (``_quantize.py:204-311``)."""
+    qcfg = qconfig if qconfig is not None else get_default_qconfig()
+    model = model if inplace else copy.deepcopy(model)
+    model.eval()
+    observed = _observed_types()
+    n_matched = 0
+    for _name, mod in model.named_modules():
+        if not isinstance(mod, observed):
+            continue
+        # the Linear / Conv inside a fused pair is observed through the pair
+        mod.qconfig = qcfg
+        obs = qcfg.activation()
+        mod.activation_post_process = obs
+        mod.register_forward_hook(_make_observer_hook(obs))
+        n_matched += 1
+    if n_matched == 0:
+        warnings.warn(
+            "prepare(): the QConfigMapping matched no quantizable modules — "
+            "convert() will leave this model unchanged.",
+            stacklevel=2,
+        )
+    return model
+
+
+def _convert_recursive(module, mapping, always) -> None:
+    for name, child in list(module.named_children()):
+        build = mapping.get(type(child))
+        convertible = build is not None and (
+            isinstance(child, always) or hasattr(child, "activation_post_process"))
+        if convertible:
+            module._modules[name] = build(child)  # keep the child's position
+        else:
+            _convert_recursive(child, mapping, always)
+
+
+def convert(model, inplace: bool = False):
+    """Swap every calibrated module for its quantized form
+    (``_quantize.py:314-419``)."""
+    model = model if inplace else copy.deepcopy(model)
+    _convert_recursive(model, _quant_mapping(), always=(nnq.DeQuantStub,))
+    model.eval()
+    return model
+
+
+def _swap_dynamic(module, mapping, types, dtype) -> None:
+    for name, child in list(module.named_children()):
+        build = mapping.get(type(child))
+        if build is not None and type(child) in types:
+            module._modules[name] = build(child, dtype)
+        else:
+            _swap_dynamic(child, mapping, types, dtype)
+
+
+def quantize_dynamic(model, qconfig_spec=None, dtype: QDtype = qint8, inplace: bool = False):
+    """Calibration-free dynamic quantization of every ``nn.Linear``
+    (``_quantize.py:429-539``)."""
+    model = model if inplace else copy.deepcopy(model)
+    model.eval()
+    mapping = _dynamic_mapping()
+    types = qconfig_spec if qconfig_spec is not None else set(mapping)
+    if not any(type(m) in types for m in model.modules()):
+        warnings.warn(
+            "quantize_dynamic(): no module of a targeted type "
+            f"({', '.join(sorted(t.__name__ for t in types))}) found — "
+            "the model is returned unchanged.",
+            stacklevel=2,
+        )
+    build = mapping.get(type(model))
+    if build is not None and type(model) in types:
+        return build(model, dtype)
+    _swap_dynamic(model, mapping, types, dtype)
+    return model

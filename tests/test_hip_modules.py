@@ -1,0 +1,308 @@
+"""GPU tests of the module layer: ``quantize_dynamic`` / ``convert`` install
+hip int8 modules whose results are bit-exact against the oracle's integer
+formulation and within tolerance of Lucid's float pass structure.
+
+The structure follows the reference's own suites
+(lucid/test/unit/quantization/test_dynamic_ptq.py, test_static_ptq.py,
+test_functional_module.py, test_real_gemm.py:148-157)."""
+
+import warnings
+
+import numpy as np
+import pytest
+
+import lucid_amd as L
+import lucid_amd.backends as backends
+import lucid_amd.nn as nn
+import lucid_amd.nn.intrinsic as nni
+import lucid_amd.nn.quantized as nnq
+import lucid_amd.nn.quantized.dynamic as nnqd
+import lucid_amd.quantization as Q
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def hip(a):
+    return L.tensor(np.ascontiguousarray(a), device="hip")
+
+
+def _set(linear, w, b):
+    linear.register_buffer("weight", L.tensor(w))
+    linear.register_buffer("bias", L.tensor(b))
+
+
+def _mlp(rng, sizes=(784, 256, 10), std=0.05):
+    layers, params = [], []
+    for i in range(len(sizes) - 1):
+        lin = nn.Linear(sizes[i], sizes[i + 1])
+        w = (rng.standard_normal((sizes[i + 1], sizes[i])) * std).astype(np.float32)
+        b = (rng.standard_normal(sizes[i + 1]) * std).astype(np.float32)
+        _set(lin, w, b)
+        params.append((w, b))
+        layers.append(lin)
+        if i < len(sizes) - 2:
+            layers.append(nn.ReLU())
+    return nn.Sequential(*layers), params
+
+
+def _oracle_weight(w):
+    mn, mx = O.minmax(w, ch_axis=0)
+    ws, wz = O.calc_qparams(mn, mx, True, -128, 127, True)
+    return O.quantize(w, ws, wz, -128, 127, ch_axis=0), ws, wz
+
+
+def _oracle_dynamic_linear(x, w, b):
+    """nnqd.Linear (dynamic/linear.py:84-99) in the integer formulation, plus
+    the reference's float pass structure for the tolerance check."""
+    wq, ws, wz = _oracle_weight(w)
+    mn, mx = O.minmax(x)
+    xs, xz = O.calc_qparams(mn, mx, False, 0, 255, False)
+    xq = O.quantize(x, xs, xz, 0, 255, code_offset=-128)
+    y_int = O.qlinear(xq, wq, int(xz[0]) - 128, xs, ws, bias=b, out_mode=O.OUT_F32)
+    y_float = O.linear_faithful(O.fake_quantize(x, xs, xz, 0, 255), wq, ws, wz, bias=b)
+    return y_int, y_float
+
+
+# ------------------------------------------------------------------ dynamic PTQ
+class TestDynamicPTQ:
+    def test_swaps_linear_and_keeps_int8_weight(self):
+        # test_dynamic_ptq.py:34-38
+        model, _ = _mlp(np.random.default_rng(0), (32, 64, 64, 10))
+        qm = Q.quantize_dynamic(model)
+        assert isinstance(qm[0], nnqd.Linear) and isinstance(qm[2], nnqd.Linear)
+        assert isinstance(model[0], nn.Linear)          # not in place
+        assert qm[0].weight_int8.dtype is L.int8 and qm[0].weight_int8.shape == (64, 32)
+        assert qm[0].act_qdtype is Q.quint8
+
+    def test_mlp_config_bit_exact_and_within_tolerance(self):
+        """Linear(784,256)-ReLU-Linear(256,10), batch 64, seeded."""
+        rng = np.random.default_rng(1)
+        model, params = _mlp(rng)
+        x = rng.standard_normal((64, 784)).astype(np.float32)
+        qm = Q.quantize_dynamic(model)
+        y = qm(hip(x))
+        assert y.shape == (64, 10) and y.dtype is L.float32 and y._grid is None
+
+        (w1, b1), (w2, b2) = params
+        h_int, h_float = _oracle_dynamic_linear(x, w1, b1)
+        h_int, h_float = np.maximum(h_int, 0), np.maximum(h_float, 0)
+        y_int, _ = _oracle_dynamic_linear(h_int, w2, b2)
+        _, y_float = _oracle_dynamic_linear(h_float, w2, b2)
+        # every stage is bit-exact against the integer formulation
+        wq1, ws1, _ = _oracle_weight(w1)
+        assert np.array_equal(qm[0].weight_int8.numpy(), wq1)
+        assert np.array_equal(qm[0].weight_scale.numpy(), ws1)
+        h = qm[1](qm[0](hip(x)))
+        assert np.array_equal(h.numpy().view(np.uint32), h_int.view(np.uint32))
+        assert np.array_equal(y.numpy().view(np.uint32), y_int.view(np.uint32))
+        # and within 1e-3 relative of the reference's float pass structure
+        assert np.abs(y.numpy() - y_float).max() <= 1e-3 * np.abs(y_float).max()
+        # quality bound of the reference's own test (test_dynamic_ptq.py:40-46)
+        y_fp = np.maximum(x @ w1.T + b1, 0) @ w2.T + b2
+        assert np.abs(y.numpy() - y_fp).mean() / np.abs(y_fp).mean() < 0.05
+
+    def test_leading_dims_are_flattened(self):
+        rng = np.random.default_rng(2)
+        lin = nn.Linear(48, 24)
+        w = (rng.standard_normal((24, 48)) * 0.1).astype(np.float32)
+        b = rng.standard_normal(24).astype(np.float32)
+        _set(lin, w, b)
+        q = nnqd.Linear.from_float(lin)
+        x = rng.standard_normal((3, 5, 48)).astype(np.float32)
+        y = q(hip(x))
+        assert y.shape == (3, 5, 24)
+        y_int, _ = _oracle_dynamic_linear(x.reshape(15, 48), w, b)
+        assert np.array_equal(y.numpy().reshape(15, 24).view(np.uint32), y_int.view(np.uint32))
+
+    def test_no_target_warns(self):
+        with pytest.warns(UserWarning, match="no module of a targeted type"):
+            Q.quantize_dynamic(nn.Sequential(nn.ReLU()))
+
+    def test_state_dict_round_trip_is_bit_equal(self):
+        # test_static_ptq.py:132-145 (checkpoint round trip)
+        rng = np.random.default_rng(3)
+        model, _ = _mlp(rng, (64, 32, 8))
+        qa, qb = Q.quantize_dynamic(model), Q.quantize_dynamic(_mlp(np.random.default_rng(9), (64, 32, 8))[0])
+        sd = qa.state_dict()
+        assert set(sd) == {"0.weight_int8", "0.weight_scale", "0.weight_zero_point", "0.bias",
+                           "2.weight_int8", "2.weight_scale", "2.weight_zero_point", "2.bias"}
+        host = {k: L.tensor(v.numpy()) for k, v in sd.items()}      # as if loaded from disk
+        qb.load_state_dict({k: v.to("hip") for k, v in host.items()})
+        x = hip(rng.standard_normal((16, 64)).astype(np.float32))
+        assert np.array_equal(qa(x).numpy().view(np.uint32), qb(x).numpy().view(np.uint32))
+
+
+# ------------------------------------------------------------------ static PTQ
+def _static_model(rng):
+    class MLP(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.quant = nnq.QuantStub()
+            self.fc1 = nni.LinearReLU(nn.Linear(16, 32), nn.ReLU())
+            self.fc2 = nn.Linear(32, 8)
+            self.dequant = nnq.DeQuantStub()
+
+        def forward(self, x):
+            return self.dequant(self.fc2(self.fc1(self.quant(x))))
+
+    m = MLP()
+    w1 = (rng.standard_normal((32, 16)) * 0.3).astype(np.float32)
+    b1 = (rng.standard_normal(32) * 0.1).astype(np.float32)
+    w2 = (rng.standard_normal((8, 32)) * 0.3).astype(np.float32)
+    b2 = (rng.standard_normal(8) * 0.1).astype(np.float32)
+    _set(m.fc1[0], w1, b1)
+    _set(m.fc2, w2, b2)
+    return m, (w1, b1, w2, b2)
+
+
+def _calibrate(prepared, params, rng, batches=20):
+    """Feeds the observers what a float forward of the model would show them
+    (the float forward itself is Lucid's CPU / Metal job)."""
+    w1, b1, w2, b2 = params
+    for _ in range(batches):
+        x = rng.standard_normal((64, 16)).astype(np.float32)
+        h = np.maximum(x @ w1.T + b1, 0)
+        y = h @ w2.T + b2
+        prepared.quant.activation_post_process(hip(x))
+        prepared.fc1.activation_post_process(hip(h))
+        prepared.fc2.activation_post_process(hip(y))
+
+
+class TestStaticPTQ:
+    def test_convert_structure_and_numerics(self):
+        rng = np.random.default_rng(0)
+        m, params = _static_model(rng)
+        prepared = Q.prepare(m, Q.get_default_qconfig())
+        _calibrate(prepared, params, rng)
+        qm = Q.convert(prepared)
+        # test_static_ptq.py:66-76
+        assert isinstance(qm.fc1, nnq.LinearReLU) and isinstance(qm.fc2, nnq.Linear)
+        assert isinstance(qm.quant, nnq.Quantize) and isinstance(qm.dequant, nnq.DeQuantize)
+        assert qm.fc1.weight_int8.dtype is L.int8 and qm.fc2.weight_int8.dtype is L.int8
+        assert qm.fc1.out_qdtype is Q.quint8 and qm.fc1.scale.shape == ()
+
+        w1, b1, w2, b2 = params
+        x = rng.standard_normal((64, 16)).astype(np.float32)
+        y = qm(hip(x))
+        assert y._grid is None and y.dtype is L.float32
+
+        # oracle, integer formulation, stage by stage
+        s0, z0 = qm.quant.scale.item(), qm.quant.zero_point.item()
+        s1, z1 = qm.fc1.scale.item(), qm.fc1.zero_point.item()
+        s2, z2 = qm.fc2.scale.item(), qm.fc2.zero_point.item()
+        xq = O.quantize(x, s0, z0, 0, 255, code_offset=-128)
+        wq1, ws1, wz1 = _oracle_weight(w1)
+        wq2, ws2, wz2 = _oracle_weight(w2)
+        h = O.qlinear(xq, wq1, int(z0) - 128, s0, ws1, bias=b1, relu=True,
+                      out_mode=O.OUT_REQUANT_I8, out_scale=s1, out_zp=z1, out_offset=-128)
+        yq = O.qlinear(h, wq2, int(z1) - 128, s1, ws2, bias=b2, out_mode=O.OUT_REQUANT_I8,
+                       out_scale=s2, out_zp=z2, out_offset=-128)
+        inner = qm.fc2(qm.fc1(qm.quant(hip(x))))
+        assert np.array_equal(inner._grid.codes.numpy(), yq)
+        assert np.array_equal(y.numpy().view(np.uint32),
+                              O.dequantize(yq, s2, z2, code_offset=-128).view(np.uint32))
+
+        # Lucid's float pass structure: codes agree up to +-1 on rounding ties
+        xf = O.fake_quantize(x, s0, z0, 0, 255)
+        hf = O.linear_faithful(xf, wq1, ws1, wz1, bias=b1, relu=True, fq=(s1, z1, 0, 255))
+        yf = O.linear_faithful(hf, wq2, ws2, wz2, bias=b2, fq=(s2, z2, 0, 255))
+        assert np.abs(y.numpy() - yf).max() <= s2 * 1.001
+        assert (y.numpy() != yf).mean() < 0.02
+        # quality bound of the reference's own test (test_static_ptq.py:78-86)
+        y_fp = np.maximum(x @ w1.T + b1, 0) @ w2.T + b2
+        assert np.abs(y.numpy() - y_fp).mean() / np.abs(y_fp).mean() < 0.05
+
+    def test_uncalibrated_convert_warns(self):
+        # lucid/test/unit/quantization/test_safety.py (warning text "never saw")
+        m, _ = _static_model(np.random.default_rng(1))
+        prepared = Q.prepare(m)
+        with pytest.warns(UserWarning, match="never saw"):
+            Q.convert(prepared)
+
+    def test_prepare_without_targets_warns(self):
+        with pytest.warns(UserWarning, match="matched no quantizable"):
+            Q.prepare(nn.Sequential(nn.ReLU()))
+
+    def test_plain_float_input_is_rejected_loudly(self):
+        rng = np.random.default_rng(2)
+        m, params = _static_model(rng)
+        prepared = Q.prepare(m)
+        _calibrate(prepared, params, rng, batches=2)
+        qm = Q.convert(prepared)
+        with pytest.raises(NotImplementedError, match="quantization grid"):
+            qm.fc1(hip(np.zeros((4, 16), np.float32)))
+        with pytest.raises(L.DeviceMismatch):
+            qm(L.tensor(np.zeros((4, 16), np.float32)))
+
+    def test_quantize_passes_integer_inputs_through(self):
+        # lucid/test/unit/quantization/test_breadth.py:38-46
+        q = nnq.Quantize(hip(np.float32(0.1)), hip(np.float32(0.0)))
+        idx = hip(np.arange(6, dtype=np.int64))
+        assert q(idx) is idx
+
+
+# ------------------------------------------------------------------ residual join
+def test_qfunctional_add_relu_matches_oracle():
+    rng = np.random.default_rng(5)
+    a = (rng.standard_normal((4, 500)) * 2).astype(np.float32)
+    b = (rng.standard_normal((4, 500)) * 3).astype(np.float32)
+    qa = nnq.Quantize(hip(np.float32(0.05)), hip(np.float32(120.0)))
+    qb = nnq.Quantize(hip(np.float32(0.07)), hip(np.float32(131.0)))
+    f = nnq.QFunctional(hip(np.float32(0.06)), hip(np.float32(0.0)))
+    out = f.add_relu(qa(hip(a)), qb(hip(b)))
+    ca = O.quantize(a, 0.05, 120.0, 0, 255, code_offset=-128)
+    cb = O.quantize(b, 0.07, 131.0, 0, 255, code_offset=-128)
+    exp = O.add_requant(ca, -128, np.float32(0.05), 120.0, cb, -128, np.float32(0.07), 131.0, True,
+                        np.float32(0.06), 0.0, 0, 255, -128)
+    assert np.array_equal(out._grid.codes.numpy(), exp)
+    # float view equals Lucid's composition fq(relu(x + y)) on the float-carried operands
+    xa, xb = O.fake_quantize(a, 0.05, 120.0, 0, 255), O.fake_quantize(b, 0.07, 131.0, 0, 255)
+    ref = O.fake_quantize(np.maximum(xa + xb, 0), 0.06, 0.0, 0, 255)
+    assert np.array_equal(out.numpy().view(np.uint32), ref.view(np.uint32))
+    out2 = nnq.QFunctional(hip(np.float32(0.06)), hip(np.float32(128.0))).add(qa(hip(a)), qb(hip(b)))
+    ref2 = O.fake_quantize(xa + xb, 0.06, 128.0, 0, 255)
+    assert np.array_equal(out2.numpy().view(np.uint32), ref2.view(np.uint32))
+
+
+def test_observers_known_answers_on_device():
+    # lucid/test/unit/quantization/test_observer.py:12-17,43-50
+    obs = Q.MinMaxObserver()
+    obs(hip([[-1.0, 2.0], [0.5, 3.0]]))
+    obs(hip([[-2.0, 1.0]]))
+    assert obs.min_val.item() == -2.0 and obs.max_val.item() == 3.0
+    scale, zp = obs.calculate_qparams()
+    assert scale.item() == pytest.approx(5.0 / 255.0, rel=1e-5) and 0 <= zp.item() <= 255
+    pc = Q.PerChannelMinMaxObserver(ch_axis=0)
+    pc(hip([[1.0, 2.0, 3.0], [-4.0, 0.5, 0.1]]))
+    assert pc.min_val.numpy().tolist() == [1.0, -4.0] and pc.max_val.numpy().tolist() == [3.0, 0.5]
+    s, z = pc.calculate_qparams()
+    assert s.shape == (2,) and z.numpy().tolist() == [0.0, 0.0]
+    pc(hip([[5.0, -9.0, 0.0], [0.0, 0.0, 7.0]]))
+    assert pc.min_val.numpy().tolist() == [-9.0, -4.0] and pc.max_val.numpy().tolist() == [5.0, 7.0]
+    fx = Q.FixedQParamsObserver(1.0 / 256, 0)
+    assert fx.calculate_qparams()[0].item() == 1.0 / 256
+
+
+def test_relu_kernel():
+    x = np.array([-1.0, -0.0, 0.0, 2.5, np.nan, -np.inf, np.inf] * 37, np.float32)
+    y = nn.relu(hip(x)).numpy()
+    exp = np.where(x < 0, np.float32(0), x)
+    assert np.array_equal(y.view(np.uint32)[~np.isnan(x)], exp.view(np.uint32)[~np.isnan(x)])
+    assert np.isnan(y[np.isnan(x)]).all()
+
+
+def test_engine_toggle():
+    # lucid/test/unit/quantization/test_real_gemm.py:148-157
+    prev = backends.quantized.engine
+    try:
+        for v in ("auto", "reference", "mlx_group", "hip"):
+            backends.quantized.engine = v
+            assert backends.quantized.engine == v
+        with pytest.raises(ValueError):
+            backends.quantized.engine = "cuda"
+        backends.quantized.engine = "hip"
+        assert backends.quantized.available and backends.quantized.use_hip()
+        assert not backends.quantized.use_mlx()
+    finally:
+        backends.quantized.engine = prev
