@@ -210,6 +210,61 @@ int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);
  * interpreter's call overhead) and for timing.  No counterpart in Lucid. */
 int lq_qlinear_i8_n(const lq_qlinear_args* args, int n, lq_stream stream);
 
+/* ------------------------------------------------------- quantized Conv2d */
+/* Quantized Conv2d forward.  Replaces the composite of
+ * lucid/nn/quantized/conv.py:168-184 (+ intrinsic.py:334-336 for the fused
+ * ReLU): dequantize kernel -> IBackend::conv_nd_forward (IBackend.h:1469-1482;
+ * per-image im2col + sgemm, CpuBackend.h:8124-8257) -> per-channel bias ->
+ * fake_quantize, by the same integer identity as lq_qlinear_i8 with
+ *     m = (b, oh, ow),  n = cout,  k = (kh, kw, cin_in_group).
+ * Layouts differ from Lucid's NCHW / OIHW on purpose: activation codes are
+ * NHWC [B,H,W,Cin] and weight codes [Cout,KH,KW,Cin/groups], so that k runs
+ * over contiguous bytes (use lq_quantize_nchw_to_nhwc, lq_repack_oihw_to_ohwi_i8
+ * and lq_dequantize_nhwc_to_nchw at the model boundary).  Zero padding of the
+ * float image (Im2Col.cpp:59-100) becomes padding with the code a_zp.
+ * Output: NHWC [B,OH,OW,Cout], OH/OW per lucid/_C/nn/ConvNd.cpp:56-59 with
+ * separate low/high pads ("same" padding can be asymmetric,
+ * lucid/nn/modules/conv.py:44-55). */
+typedef struct {
+    const int8_t* x;       /* NHWC codes as stored                           */
+    const int8_t* w;       /* [Cout,KH,KW,Cin/groups] codes                  */
+    int B, H, W, Cin, Cout, KH, KW;
+    int stride_h, stride_w, pad_h_lo, pad_h_hi, pad_w_lo, pad_w_hi, dil_h, dil_w, groups;
+    const int32_t* wsum;   /* [Cout] sum of each filter's codes              */
+    int a_zp;              /* zero point of the stored codes; also the pad code */
+    const float* a_scale;  /* [1]                                            */
+    const float* w_scale;  /* [Cout]                                         */
+    const void* bias;      /* [Cout] or NULL                                 */
+    int bias_dtype;
+    int relu;
+    int out_mode;          /* LQ_OUT_*                                       */
+    const float* out_scale;
+    const float* out_zp;
+    int out_qmin, out_qmax, out_offset;
+    void* out;             /* NHWC [B,OH,OW,Cout]                            */
+    int force_path;        /* 0 = choose; 1 = gemm (1x1), 2 = implicit GEMM,
+                              3 = explicit im2col + GEMM, 4 = naive          */
+    int tile_config;
+} lq_qconv2d_args;
+
+int lq_qconv2d_i8(const lq_qconv2d_args* args, lq_stream stream);
+
+/* Model-boundary layout helpers (per-tensor qparams as device scalars):
+ * quantize float32 NCHW into int8 NHWC codes; the inverse float view; and the
+ * one-time repack of weight codes from Lucid's OIHW buffer. */
+int lq_quantize_nchw_to_nhwc(const float* x, int8_t* q, int code_offset, int B, int C, int H, int W,
+                             const float* scale, const float* zp, int qmin, int qmax,
+                             lq_stream stream);
+int lq_dequantize_nhwc_to_nchw(const int8_t* q, int code_offset, float* out, int B, int C, int H,
+                               int W, const float* scale, const float* zp, lq_stream stream);
+int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH, int KW,
+                              lq_stream stream);
+
+/* Max-pool on NHWC codes (F.max_pool2d between quantized layers of a ResNet
+ * stem): quantisation is monotone, so pooling codes equals pooling values. */
+int lq_maxpool2d_nhwc_i8(const int8_t* x, int8_t* out, int B, int H, int W, int C, int KH, int KW,
+                         int stride_h, int stride_w, int pad_h, int pad_w, lq_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -119,6 +119,30 @@ _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
 _SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]
 
+
+
+class QConv2dArgs(C.Structure):
+    """``lq_qconv2d_args`` of ``include/lucid_hip.h``."""
+
+    _fields_ = [
+        ("x", _vp), ("w", _vp),
+        ("B", _i), ("H", _i), ("W", _i), ("Cin", _i), ("Cout", _i), ("KH", _i), ("KW", _i),
+        ("stride_h", _i), ("stride_w", _i), ("pad_h_lo", _i), ("pad_h_hi", _i), ("pad_w_lo", _i),
+        ("pad_w_hi", _i), ("dil_h", _i), ("dil_w", _i), ("groups", _i),
+        ("wsum", _vp), ("a_zp", _i), ("a_scale", _vp), ("w_scale", _vp),
+        ("bias", _vp), ("bias_dtype", _i), ("relu", _i), ("out_mode", _i),
+        ("out_scale", _vp), ("out_zp", _vp),
+        ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
+        ("out", _vp), ("force_path", _i), ("tile_config", _i),
+    ]
+
+
+_SIGNATURES["lq_qconv2d_i8"] = [C.POINTER(QConv2dArgs), _vp]
+_SIGNATURES["lq_quantize_nchw_to_nhwc"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]
+_SIGNATURES["lq_dequantize_nhwc_to_nchw"] = [_vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp]
+_SIGNATURES["lq_repack_oihw_to_ohwi_i8"] = [_vp, _vp, _i, _i, _i, _i, _vp]
+_SIGNATURES["lq_maxpool2d_nhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
+
 _RESTYPE = {"lq_last_error": C.c_char_p}
 _NO_STATUS = {"lq_version", "lq_last_error", "lq_op_count"}
 

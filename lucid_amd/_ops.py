@@ -80,3 +80,48 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
     else:
         _C.call("lq_qlinear_i8_n", C.byref(args), int(repeat), None)
     return out
+
+
+CONV_AUTO, CONV_GEMM, CONV_IMPLICIT, CONV_IM2COL, CONV_NAIVE = range(5)
+
+
+def conv_out_size(size: int, k: int, stride: int, pad_lo: int, pad_hi: int, dil: int) -> int:
+    """Output extent of one spatial axis (``lucid/_C/nn/ConvNd.cpp:56-59``)."""
+    return (size + pad_lo + pad_hi - dil * (k - 1) - 1) // stride + 1
+
+
+def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None,
+               w_scale: Tensor | None = None, wsum: Tensor | None = None,
+               bias: Tensor | None = None, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1),
+               groups: int = 1, relu: bool = False, out_mode: int = OUT_F32,
+               out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
+               out_qmax: int = 255, out_offset: int = 0, path: int = CONV_AUTO,
+               tile_config: int = 0) -> Tensor:
+    """Fused int8 convolution; see ``lq_qconv2d_i8``.  ``x`` int8 NHWC, ``w``
+    int8 ``[Cout, KH, KW, Cin/groups]``, ``pad`` = (h_lo, h_hi, w_lo, w_hi).
+    Returns NHWC ``[B, OH, OW, Cout]``."""
+    if x.ndim != 4 or w.ndim != 4:
+        raise _C.ShapeMismatch(f"qconv2d_i8: expected 4-d x and w, got {x.shape} and {w.shape}")
+    B, H, W, Cin = x.shape
+    Cout, KH, KW, Cg = w.shape
+    if Cg * groups != Cin:
+        raise _C.ShapeMismatch(f"qconv2d_i8: weight {w.shape} does not match Cin={Cin}, groups={groups}")
+    OH = conv_out_size(H, KH, stride[0], pad[0], pad[1], dilation[0])
+    OW = conv_out_size(W, KW, stride[1], pad[2], pad[3], dilation[1])
+    out = Tensor.empty((B, max(OH, 0), max(OW, 0), Cout), _OUT_DTYPE[out_mode], "hip")
+    a = _C.QConv2dArgs()
+    a.x, a.w = _ptr(x, "x", T.int8), _ptr(w, "w", T.int8)
+    a.B, a.H, a.W, a.Cin, a.Cout, a.KH, a.KW = B, H, W, Cin, Cout, KH, KW
+    a.stride_h, a.stride_w = int(stride[0]), int(stride[1])
+    a.pad_h_lo, a.pad_h_hi, a.pad_w_lo, a.pad_w_hi = (int(v) for v in pad)
+    a.dil_h, a.dil_w, a.groups = int(dilation[0]), int(dilation[1]), int(groups)
+    a.wsum, a.a_zp = _ptr(wsum, "wsum", T.int32), int(a_zp)
+    a.a_scale, a.w_scale = _ptr(a_scale, "a_scale", T.float32), _ptr(w_scale, "w_scale", T.float32)
+    a.bias = _ptr(bias, "bias", (T.float32, T.float16))
+    a.bias_dtype = bias.dtype.code if bias is not None else 0
+    a.relu, a.out_mode = int(relu), int(out_mode)
+    a.out_scale, a.out_zp = _ptr(out_scale, "out_scale", T.float32), _ptr(out_zp, "out_zp", T.float32)
+    a.out_qmin, a.out_qmax, a.out_offset = int(out_qmin), int(out_qmax), int(out_offset)
+    a.out, a.force_path, a.tile_config = out.data_ptr, int(path), int(tile_config)
+    _C.call("lq_qconv2d_i8", C.byref(a), None)
+    return out

@@ -1,0 +1,391 @@
+// Quantized Conv2d forward for gfx950: convolution lowered to the int8 MFMA
+// GEMM, plus the layout helpers around it.
+//
+// Activations are int8 codes in NHWC, weights int8 [Cout][KH][KW][Cin/groups],
+// the result is NHWC in the form the epilogue mode asks for.  The GEMM view is
+// M = B*OH*OW, N = Cout/groups, K = KH*KW*Cin/groups.  Out-of-image taps read
+// the activation zero-point code: Lucid pads the float image with 0.0
+// (lucid/_C/backend/cpu/Im2Col.cpp:59-100), which on the activation grid is
+// the code Z.  Three routes:
+//   gemm     : 1x1, stride 1, no padding -> the NHWC tensor IS the A matrix
+//   implicit : Cin/groups % 16 == 0 -> the tile kernel gathers A on the fly
+//   im2col   : anything else (e.g. a 7x7x3 stem) -> explicit int8 im2col into
+//              the workspace with K padded to a multiple of 16, then the GEMM
+//   naive    : one output per lane, any shape (checking aid)
+#include "common.hpp"
+#include "qepilogue.hpp"
+#include "qgemm.hpp"
+
+using namespace lq;
+
+namespace {
+
+struct ConvShape {
+    int B, H, W, Cin, Cout, KH, KW, OH, OW;
+    int sh, sw, ph, pw, dh, dw, groups;
+};
+
+// ---------------------------------------------------------------- naive
+__global__ __launch_bounds__(256) void qconv_naive_kernel(GemmArgs g, ConvShape c, const int8_t* x,
+                                                          const int8_t* w) {
+    const int Cg = c.Cin / c.groups, Og = c.Cout / c.groups;
+    const size_t total = size_t(c.B) * c.OH * c.OW * c.Cout;
+    float S = 1.0f, Z = 0.0f;
+    if (g.out_mode == OUT_REQUANT_I8 || g.out_mode == OUT_FAKEQUANT_F32) {
+        S = g.out_scale[0];
+        Z = g.out_zp[0];
+    }
+    const float as = g.a_scale ? g.a_scale[0] : 1.0f;
+    for (size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * 256) {
+        const int co = int(idx % c.Cout);
+        size_t p = idx / c.Cout;
+        const int ow = int(p % c.OW);
+        p /= c.OW;
+        const int oh = int(p % c.OH);
+        const int b = int(p / c.OH);
+        const int grp = co / Og;
+        int32_t acc = 0;
+        for (int kh = 0; kh < c.KH; ++kh)
+            for (int kw = 0; kw < c.KW; ++kw) {
+                const int ih = oh * c.sh - c.ph + kh * c.dh, iw = ow * c.sw - c.pw + kw * c.dw;
+                const int8_t* wr = w + ((size_t(co) * c.KH + kh) * c.KW + kw) * Cg;
+                if (ih < 0 || ih >= c.H || iw < 0 || iw >= c.W) {
+                    int ws = 0;
+                    for (int ci = 0; ci < Cg; ++ci) ws += wr[ci];
+                    acc += g.a_zp * ws;
+                } else {
+                    const int8_t* xr = x + ((size_t(b) * c.H + ih) * c.W + iw) * c.Cin + grp * Cg;
+                    for (int ci = 0; ci < Cg; ++ci) acc += int(xr[ci]) * int(wr[ci]);
+                }
+            }
+        const int m = int(idx / c.Cout);
+        epilogue_store(g, m, co, acc, as, load_col(g, co), S, Z);
+    }
+}
+
+// ---------------------------------------------------------------- explicit im2col
+// cols[m][k], k = (kh*KW + kw)*Cg + ci for k < K, zero for K <= k < Kp.
+__global__ __launch_bounds__(256) void im2col_i8_kernel(const int8_t* __restrict__ x,
+                                                        int8_t* __restrict__ cols, ConvShape c,
+                                                        int grp, int K, int Kp, int8_t pad_code) {
+    const int Cg = c.Cin / c.groups;
+    const size_t total = size_t(c.B) * c.OH * c.OW * Kp;
+    for (size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * 256) {
+        const int k = int(idx % Kp);
+        size_t m = idx / Kp;
+        int8_t v = 0;
+        if (k < K) {
+            const int ci = k % Cg, tap = k / Cg;
+            const int kw = tap % c.KW, kh = tap / c.KW;
+            const int ow = int(m % c.OW);
+            size_t q = m / c.OW;
+            const int oh = int(q % c.OH), b = int(q / c.OH);
+            const int ih = oh * c.sh - c.ph + kh * c.dh, iw = ow * c.sw - c.pw + kw * c.dw;
+            v = (ih < 0 || ih >= c.H || iw < 0 || iw >= c.W)
+                    ? pad_code
+                    : x[((size_t(b) * c.H + ih) * c.W + iw) * c.Cin + grp * Cg + ci];
+        }
+        cols[idx] = v;
+    }
+}
+
+// weight rows of one group, K bytes each, copied into rows of Kp bytes (zero tail)
+__global__ void pad_rows_kernel(const int8_t* __restrict__ w, int8_t* __restrict__ out, int rows,
+                                int K, int Kp) {
+    const size_t total = size_t(rows) * Kp;
+    for (size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * blockDim.x) {
+        const int k = int(idx % Kp);
+        const size_t r = idx / Kp;
+        out[idx] = k < K ? w[r * K + k] : int8_t(0);
+    }
+}
+
+// ---------------------------------------------------------------- layout helpers
+__device__ __forceinline__ float q_core_local(float x, float s, float z, float lo, float hi) {
+    float t = x / s;
+    float r = __builtin_rintf(t);
+    float u = r + z;
+    u = (u < lo) ? lo : ((u > hi) ? hi : u);
+    return u;
+}
+
+// float32 NCHW -> int8 NHWC codes (per-tensor qparams): the entry Quantize of a
+// convolutional model.  A block transposes a [C-tile][W-tile] patch through LDS.
+__global__ __launch_bounds__(256) void quantize_nchw_to_nhwc_kernel(
+    const float* __restrict__ x, int8_t* __restrict__ q, int B, int C, int HW, const float* scale,
+    const float* zp, float lo, float hi, int off) {
+    __shared__ int8_t tile[32][33];
+    const float s = scale[0], z = zp[0];
+    const int b = blockIdx.z, c0 = blockIdx.y * 32, p0 = blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int j = ty; j < 32; j += 8) {
+        const int c = c0 + j, p = p0 + tx;
+        int8_t v = 0;
+        if (c < C && p < HW) {
+            float u = q_core_local(x[(size_t(b) * C + c) * HW + p], s, z, lo, hi);
+            v = int8_t(((u != u) ? 0 : int(u)) + off);
+        }
+        tile[j][tx] = v;
+    }
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8) {
+        const int p = p0 + j, c = c0 + tx;
+        if (c < C && p < HW) q[(size_t(b) * HW + p) * C + c] = tile[tx][j];
+    }
+}
+
+// int8 NHWC codes -> float32 NCHW: the float view of a convolutional activation
+__global__ __launch_bounds__(256) void dequantize_nhwc_to_nchw_kernel(
+    const int8_t* __restrict__ q, int off, float* __restrict__ out, int B, int C, int HW,
+    const float* scale, const float* zp) {
+    __shared__ float tile[32][33];
+    const float s = scale[0], z = zp[0];
+    const int b = blockIdx.z, c0 = blockIdx.y * 32, p0 = blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int j = ty; j < 32; j += 8) {
+        const int p = p0 + j, c = c0 + tx;
+        float v = 0.0f;
+        if (c < C && p < HW) v = (float(int(q[(size_t(b) * HW + p) * C + c]) - off) - z) * s;
+        tile[j][tx] = v;
+    }
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8) {
+        const int c = c0 + j, p = p0 + tx;
+        if (c < C && p < HW) out[(size_t(b) * C + c) * HW + p] = tile[tx][j];
+    }
+}
+
+// weight codes OIHW -> O,KH,KW,I (the K order of the implicit GEMM); one-time
+__global__ void repack_oihw_to_ohwi_kernel(const int8_t* __restrict__ w, int8_t* __restrict__ out,
+                                           int O, int I, int KH, int KW) {
+    const size_t total = size_t(O) * I * KH * KW;
+    for (size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * blockDim.x) {
+        const int i = int(idx % I);
+        size_t r = idx / I;
+        const int kw = int(r % KW);
+        r /= KW;
+        const int kh = int(r % KH);
+        const int o = int(r / KH);
+        out[idx] = w[((size_t(o) * I + i) * KH + kh) * KW + kw];
+    }
+}
+
+// max-pool on codes, NHWC.  Quantisation is monotone, so the maximum of the
+// codes is the code of the maximum; padded taps never win.
+__global__ __launch_bounds__(256) void maxpool_nhwc_i8_kernel(const int8_t* __restrict__ x,
+                                                              int8_t* __restrict__ out, int B, int H,
+                                                              int W, int C, int KH, int KW, int sh,
+                                                              int sw, int ph, int pw, int OH, int OW) {
+    const size_t total = size_t(B) * OH * OW * C;
+    for (size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * 256) {
+        const int c = int(idx % C);
+        size_t p = idx / C;
+        const int ow = int(p % OW);
+        p /= OW;
+        const int oh = int(p % OH);
+        const int b = int(p / OH);
+        int best = -128;
+        for (int kh = 0; kh < KH; ++kh)
+            for (int kw = 0; kw < KW; ++kw) {
+                const int ih = oh * sh - ph + kh, iw = ow * sw - pw + kw;
+                if (ih < 0 || ih >= H || iw < 0 || iw >= W) continue;
+                const int v = x[((size_t(b) * H + ih) * W + iw) * C + c];
+                best = v > best ? v : best;
+            }
+        out[idx] = int8_t(best);
+    }
+}
+
+inline unsigned grid_1d(size_t n, unsigned per_block = 256) {
+    size_t b = (n + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    return unsigned(b > 262144 ? 262144 : b);
+}
+
+}  // namespace
+
+extern "C" {
+
+int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
+    LQ_REQUIRE(p, LQ_ERR_VALUE, "qconv2d_i8: args is NULL");
+    LQ_REQUIRE(p->B >= 0 && p->H > 0 && p->W > 0 && p->Cin > 0 && p->Cout > 0 && p->KH > 0 &&
+                   p->KW > 0,
+               LQ_ERR_SHAPE, "qconv2d_i8: non-positive extent");
+    LQ_REQUIRE(p->groups >= 1 && p->Cin % p->groups == 0 && p->Cout % p->groups == 0, LQ_ERR_SHAPE,
+               "qconv2d_i8: channels (%d -> %d) not divisible by groups %d", p->Cin, p->Cout,
+               p->groups);
+    LQ_REQUIRE(p->stride_h >= 1 && p->stride_w >= 1 && p->dil_h >= 1 && p->dil_w >= 1 &&
+                   p->pad_h_lo >= 0 && p->pad_h_hi >= 0 && p->pad_w_lo >= 0 && p->pad_w_hi >= 0,
+               LQ_ERR_VALUE, "qconv2d_i8: bad stride / dilation / padding");
+    // output extent, lucid/_C/nn/ConvNd.cpp:56-59
+    const int OH = (p->H + p->pad_h_lo + p->pad_h_hi - p->dil_h * (p->KH - 1) - 1) / p->stride_h + 1;
+    const int OW = (p->W + p->pad_w_lo + p->pad_w_hi - p->dil_w * (p->KW - 1) - 1) / p->stride_w + 1;
+    LQ_REQUIRE(OH > 0 && OW > 0, LQ_ERR_SHAPE, "qconv2d_i8: empty output (%d x %d)", OH, OW);
+    if (p->B == 0) return LQ_OK;
+    LQ_REQUIRE(p->x && p->w && p->out, LQ_ERR_VALUE, "qconv2d_i8: NULL tensor pointer");
+    LQ_REQUIRE(p->out_mode >= OUT_ACC_I32 && p->out_mode <= OUT_FAKEQUANT_F32, LQ_ERR_VALUE,
+               "qconv2d_i8: unknown out_mode %d", p->out_mode);
+    LQ_REQUIRE(p->a_zp >= -128 && p->a_zp <= 127, LQ_ERR_VALUE,
+               "qconv2d_i8: activation zero point %d is not an int8 code", p->a_zp);
+    const int Cg = p->Cin / p->groups, Og = p->Cout / p->groups;
+    const long K = long(p->KH) * p->KW * Cg;
+    LQ_REQUIRE(K <= 131071, LQ_ERR_SHAPE, "qconv2d_i8: K = %ld overflows the int32 accumulator", K);
+    const size_t M = size_t(p->B) * OH * OW;
+    LQ_REQUIRE(M <= 0x7fffffffull && size_t(p->B) * p->H * p->W * p->Cin < 0xffffffffull,
+               LQ_ERR_SHAPE, "qconv2d_i8: tensor too large for 32-bit indexing");
+    if (p->out_mode != OUT_ACC_I32) {
+        LQ_REQUIRE(p->w_scale && p->a_scale, LQ_ERR_VALUE, "qconv2d_i8: scale pointer is NULL");
+        LQ_REQUIRE(p->a_zp == 0 || p->wsum, LQ_ERR_VALUE,
+                   "qconv2d_i8: a non-zero activation zero point needs the filter sums");
+        LQ_REQUIRE(p->bias == nullptr || p->bias_dtype == LQ_F32 || p->bias_dtype == LQ_F16,
+                   LQ_ERR_DTYPE, "qconv2d_i8: bias must be float32 or float16");
+    }
+    if (p->out_mode == OUT_REQUANT_I8 || p->out_mode == OUT_FAKEQUANT_F32) {
+        LQ_REQUIRE(p->out_scale && p->out_zp, LQ_ERR_VALUE, "qconv2d_i8: output qparams are NULL");
+        if (p->out_mode == OUT_REQUANT_I8)
+            LQ_REQUIRE(p->out_qmin + p->out_offset >= -128 && p->out_qmax + p->out_offset <= 127,
+                       LQ_ERR_VALUE, "qconv2d_i8: output grid + offset does not fit int8");
+    }
+
+    hipStream_t st = as_stream(stream);
+    GemmArgs g{};
+    g.a = p->x; g.w = p->w; g.M = int(M); g.N = Og; g.K = int(K);
+    g.wsum = p->wsum; g.a_zp = p->a_zp; g.a_zp_dev = nullptr;
+    g.a_scale = p->a_scale; g.a_scale_per_row = 0; g.w_scale = p->w_scale;
+    g.bias = p->bias; g.bias_dtype = p->bias_dtype; g.relu = p->relu; g.out_mode = p->out_mode;
+    g.out_scale = p->out_scale; g.out_zp = p->out_zp;
+    g.out_qmin = p->out_qmin; g.out_qmax = p->out_qmax; g.out_offset = p->out_offset;
+    g.out = p->out; g.ldo = p->Cout;
+    g.cx = p->x; g.cH = p->H; g.cW = p->W; g.cCin = p->Cin; g.cOH = OH; g.cOW = OW; g.cKW = p->KW;
+    g.cCg = Cg; g.csh = p->stride_h; g.csw = p->stride_w; g.cph = p->pad_h_lo; g.cpw = p->pad_w_lo;
+    g.cdh = p->dil_h; g.cdw = p->dil_w;
+
+    const bool is_gemm = p->KH == 1 && p->KW == 1 && p->stride_h == 1 && p->stride_w == 1 &&
+                         p->pad_h_lo == 0 && p->pad_h_hi == 0 && p->pad_w_lo == 0 &&
+                         p->pad_w_hi == 0 && p->groups == 1;
+    const bool aligned = aligned16(p->x) && aligned16(p->w);
+    int path = p->force_path;  // 0 = choose, 1 = gemm, 2 = implicit, 3 = im2col, 4 = naive
+    if (path == 0) {
+        if (is_gemm && p->Cin % 16 == 0 && aligned)
+            path = 1;
+        else if (Cg % 16 == 0 && aligned)
+            path = 2;
+        else
+            path = 3;
+    }
+    if (path == 1) {
+        LQ_REQUIRE(is_gemm, LQ_ERR_VALUE, "qconv2d_i8: the gemm route needs a 1x1 stride-1 unpadded conv");
+        g.N = p->Cout;
+        return run_gemm(g, 0, p->tile_config, st);
+    }
+    if (path == 2) {
+        LQ_REQUIRE(Cg % 16 == 0 && aligned, LQ_ERR_VALUE,
+                   "qconv2d_i8: the implicit route needs Cin/groups %% 16 == 0 and aligned tensors");
+        return run_tile_kernel(g, true, p->groups, p->tile_config, st);
+    }
+    if (path == 4) {
+        ConvShape c{p->B, p->H, p->W, p->Cin, p->Cout, p->KH, p->KW, OH, OW, p->stride_h,
+                    p->stride_w, p->pad_h_lo, p->pad_w_lo, p->dil_h, p->dil_w, p->groups};
+        g.N = p->Cout;
+        hipLaunchKernelGGL(qconv_naive_kernel, dim3(grid_1d(M * p->Cout)), dim3(256), 0, st, g, c, p->x,
+                           p->w);
+        LQ_CHECK_LAUNCH("qconv_naive");
+        return LQ_OK;
+    }
+    LQ_REQUIRE(path == 3, LQ_ERR_VALUE, "qconv2d_i8: unknown force_path %d", path);
+    // explicit im2col, one group at a time
+    const int Kp = int((K + 15) / 16 * 16);
+    const size_t cols_bytes = (M * Kp + 255) / 256 * 256;
+    const size_t w_bytes = (size_t(Og) * Kp + 255) / 256 * 256;
+    void* ws = nullptr;
+    int rc = workspace(cols_bytes + w_bytes, &ws);
+    if (rc) return rc;
+    int8_t* cols = static_cast<int8_t*>(ws);
+    int8_t* wpad = cols + cols_bytes;
+    ConvShape c{p->B, p->H, p->W, p->Cin, p->Cout, p->KH, p->KW, OH, OW, p->stride_h, p->stride_w,
+                p->pad_h_lo, p->pad_w_lo, p->dil_h, p->dil_w, p->groups};
+    for (int grp = 0; grp < p->groups; ++grp) {
+        hipLaunchKernelGGL(im2col_i8_kernel, dim3(grid_1d(M * Kp)), dim3(256), 0, st, p->x, cols, c, grp,
+                           int(K), Kp, int8_t(p->a_zp));
+        LQ_CHECK_LAUNCH("im2col_i8");
+        hipLaunchKernelGGL(pad_rows_kernel, dim3(grid_1d(size_t(Og) * Kp)), dim3(256), 0, st,
+                           p->w + size_t(grp) * Og * K, wpad, Og, int(K), Kp);
+        LQ_CHECK_LAUNCH("pad_rows");
+        GemmArgs gg = g;
+        gg.a = cols; gg.w = wpad; gg.K = Kp; gg.N = Og;
+        const size_t col0 = size_t(grp) * Og;
+        gg.wsum = g.wsum ? g.wsum + col0 : nullptr;
+        gg.w_scale = g.w_scale ? g.w_scale + col0 : nullptr;
+        if (g.bias)
+            gg.bias = static_cast<const char*>(g.bias) + col0 * (g.bias_dtype == LQ_F16 ? 2 : 4);
+        const size_t esz = g.out_mode == OUT_F16 ? 2 : (g.out_mode == OUT_REQUANT_I8 ? 1 : 4);
+        gg.out = static_cast<char*>(g.out) + col0 * esz;
+        rc = run_gemm(gg, 0, p->tile_config, st);
+        if (rc) return rc;
+    }
+    return LQ_OK;
+}
+
+int lq_quantize_nchw_to_nhwc(const float* x, int8_t* q, int code_offset, int B, int C, int H, int W,
+                             const float* scale, const float* zp, int qmin, int qmax,
+                             lq_stream stream) {
+    if (size_t(B) * C * H * W == 0) return LQ_OK;
+    LQ_REQUIRE(x && q && scale && zp, LQ_ERR_VALUE, "quantize_nchw_to_nhwc: NULL pointer");
+    LQ_REQUIRE(qmin <= qmax && qmin + code_offset >= -128 && qmax + code_offset <= 127, LQ_ERR_VALUE,
+               "quantize_nchw_to_nhwc: grid [%d,%d] + offset %d does not fit int8", qmin, qmax,
+               code_offset);
+    LQ_REQUIRE(B <= 65535 && (C + 31) / 32 <= 65535, LQ_ERR_SHAPE, "quantize_nchw_to_nhwc: too large");
+    const int HW = H * W;
+    hipLaunchKernelGGL(quantize_nchw_to_nhwc_kernel, dim3((HW + 31) / 32, (C + 31) / 32, B), dim3(256), 0,
+                       as_stream(stream), x, q, B, C, HW, scale, zp, float(qmin), float(qmax),
+                       code_offset);
+    LQ_CHECK_LAUNCH("quantize_nchw_to_nhwc");
+    return LQ_OK;
+}
+
+int lq_dequantize_nhwc_to_nchw(const int8_t* q, int code_offset, float* out, int B, int C, int H,
+                               int W, const float* scale, const float* zp, lq_stream stream) {
+    if (size_t(B) * C * H * W == 0) return LQ_OK;
+    LQ_REQUIRE(q && out && scale && zp, LQ_ERR_VALUE, "dequantize_nhwc_to_nchw: NULL pointer");
+    LQ_REQUIRE(B <= 65535 && (C + 31) / 32 <= 65535, LQ_ERR_SHAPE, "dequantize_nhwc_to_nchw: too large");
+    const int HW = H * W;
+    hipLaunchKernelGGL(dequantize_nhwc_to_nchw_kernel, dim3((HW + 31) / 32, (C + 31) / 32, B), dim3(256),
+                       0, as_stream(stream), q, code_offset, out, B, C, HW, scale, zp);
+    LQ_CHECK_LAUNCH("dequantize_nhwc_to_nchw");
+    return LQ_OK;
+}
+
+int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH, int KW,
+                              lq_stream stream) {
+    const size_t total = size_t(O) * I * KH * KW;
+    if (total == 0) return LQ_OK;
+    LQ_REQUIRE(w && out, LQ_ERR_VALUE, "repack_oihw_to_ohwi_i8: NULL pointer");
+    hipLaunchKernelGGL(repack_oihw_to_ohwi_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream),
+                       w, out, O, I, KH, KW);
+    LQ_CHECK_LAUNCH("repack_oihw_to_ohwi");
+    return LQ_OK;
+}
+
+int lq_maxpool2d_nhwc_i8(const int8_t* x, int8_t* out, int B, int H, int W, int C, int KH, int KW,
+                         int stride_h, int stride_w, int pad_h, int pad_w, lq_stream stream) {
+    LQ_REQUIRE(KH > 0 && KW > 0 && stride_h > 0 && stride_w > 0 && pad_h >= 0 && pad_w >= 0,
+               LQ_ERR_VALUE, "maxpool2d_nhwc_i8: bad window");
+    LQ_REQUIRE(2 * pad_h <= KH && 2 * pad_w <= KW, LQ_ERR_VALUE,
+               "maxpool2d_nhwc_i8: padding larger than half the window");
+    const int OH = (H + 2 * pad_h - KH) / stride_h + 1, OW = (W + 2 * pad_w - KW) / stride_w + 1;
+    LQ_REQUIRE(OH > 0 && OW > 0, LQ_ERR_SHAPE, "maxpool2d_nhwc_i8: empty output");
+    const size_t total = size_t(B) * OH * OW * C;
+    if (total == 0) return LQ_OK;
+    LQ_REQUIRE(x && out, LQ_ERR_VALUE, "maxpool2d_nhwc_i8: NULL pointer");
+    hipLaunchKernelGGL(maxpool_nhwc_i8_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream), x,
+                       out, B, H, W, C, KH, KW, stride_h, stride_w, pad_h, pad_w, OH, OW);
+    LQ_CHECK_LAUNCH("maxpool2d_nhwc_i8");
+    return LQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,102 @@
+// Device-side epilogue shared by the GEMM and convolution kernels.
+#pragma once
+#include "qgemm.hpp"
+
+namespace lq {
+
+// ---------------------------------------------------------------- epilogue
+struct ColParams {
+    float ws, bias;
+    int32_t corr;  // a_zp * wsum[n]
+};
+
+__device__ __forceinline__ ColParams load_col(const GemmArgs& g, int n) {
+    ColParams c;
+    c.ws = g.w_scale ? g.w_scale[n] : 1.0f;
+    const int zp = g.a_zp_dev ? int(g.a_zp_dev[0]) + g.a_zp : g.a_zp;
+    c.corr = (g.wsum && zp != 0) ? zp * g.wsum[n] : 0;
+    if (g.bias == nullptr)
+        c.bias = 0.0f;
+    else if (g.bias_dtype == LQ_F16)
+        c.bias = float(static_cast<const _Float16*>(g.bias)[n]);
+    else
+        c.bias = static_cast<const float*>(g.bias)[n];
+    return c;
+}
+
+__device__ __forceinline__ float q_core(float x, float s, float z, float lo, float hi) {
+    float t = x / s;
+    float r = __builtin_rintf(t);
+    float u = r + z;
+    u = (u < lo) ? lo : ((u > hi) ? hi : u);
+    return u;
+}
+
+// One output element.  Float steps are separate (no FMA) and in the order the
+// CPU restatement uses, so results are bit-identical to it.  MODE is a
+// compile-time constant so that each output form gets a tight loop.
+// epilogue_value returns the element as 32 bits (float bits, or the integer
+// for the accumulator / requantized-code forms); store_* narrows and writes.
+template <int MODE>
+__device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t acc, float as,
+                                                   const ColParams& c, float S, float Z) {
+    if (MODE == OUT_ACC_I32) return uint32_t(acc);
+    float f = float(acc - c.corr);
+    float sc = as * c.ws;
+    float y = f * sc;
+    if (g.bias) y = y + c.bias;
+    if (g.relu) y = (y < 0.0f) ? 0.0f : y;
+    if (MODE == OUT_F32 || MODE == OUT_F16) return __float_as_uint(y);
+    float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
+    if (MODE == OUT_REQUANT_I8) {
+        int code = (qv != qv) ? 0 : int(qv);
+        return uint32_t(code + g.out_offset);
+    }
+    return __float_as_uint((qv - Z) * S);  // OUT_FAKEQUANT_F32
+}
+
+template <int MODE>
+__device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint32_t v) {
+    if (MODE == OUT_F16)
+        static_cast<_Float16*>(g.out)[idx] = _Float16(__uint_as_float(v));
+    else if (MODE == OUT_REQUANT_I8)
+        static_cast<int8_t*>(g.out)[idx] = int8_t(int(v));
+    else
+        static_cast<uint32_t*>(g.out)[idx] = v;  // f32 / i32 bit patterns
+}
+
+// four consecutive elements; idx is a multiple of 4 and the row is 4-aligned
+template <int MODE>
+__device__ __forceinline__ void store_vec4(const GemmArgs& g, size_t idx, uint4 v) {
+    if (MODE == OUT_F16) {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        h4 h = {_Float16(__uint_as_float(v.x)), _Float16(__uint_as_float(v.y)),
+                _Float16(__uint_as_float(v.z)), _Float16(__uint_as_float(v.w))};
+        *reinterpret_cast<h4*>(static_cast<_Float16*>(g.out) + idx) = h;
+    } else if (MODE == OUT_REQUANT_I8) {
+        uint32_t packed = (v.x & 0xffu) | ((v.y & 0xffu) << 8) | ((v.z & 0xffu) << 16) | (v.w << 24);
+        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(g.out) + idx) = packed;
+    } else {
+        *reinterpret_cast<uint4*>(static_cast<uint32_t*>(g.out) + idx) = v;
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ void epilogue_store_t(const GemmArgs& g, int m, int n, int32_t acc,
+                                                 float as, const ColParams& c, float S, float Z) {
+    store_scalar<MODE>(g, size_t(m) * size_t(g.ldo) + size_t(n),
+                       epilogue_value<MODE>(g, acc, as, c, S, Z));
+}
+
+__device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, int32_t acc,
+                                               float as, const ColParams& c, float S, float Z) {
+    switch (g.out_mode) {
+    case OUT_ACC_I32: epilogue_store_t<OUT_ACC_I32>(g, m, n, acc, as, c, S, Z); break;
+    case OUT_F32: epilogue_store_t<OUT_F32>(g, m, n, acc, as, c, S, Z); break;
+    case OUT_F16: epilogue_store_t<OUT_F16>(g, m, n, acc, as, c, S, Z); break;
+    case OUT_REQUANT_I8: epilogue_store_t<OUT_REQUANT_I8>(g, m, n, acc, as, c, S, Z); break;
+    default: epilogue_store_t<OUT_FAKEQUANT_F32>(g, m, n, acc, as, c, S, Z); break;
+    }
+}
+
+}  // namespace lq

@@ -16,6 +16,8 @@
 //            block's wavefronts and reduced in LDS.
 //   naive  : any shape / alignment, one output per lane.
 #include "common.hpp"
+#include "qgemm.hpp"
+#include "qepilogue.hpp"
 
 using namespace lq;
 
@@ -26,125 +28,6 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 #define LQ_GPTR(p) ((__attribute__((address_space(1))) void*)(p))
 #define LQ_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
-
-enum { OUT_ACC_I32 = 0, OUT_F32 = 1, OUT_F16 = 2, OUT_REQUANT_I8 = 3, OUT_FAKEQUANT_F32 = 4 };
-
-struct GemmArgs {
-    const int8_t* a;      // [M,K] activation codes as stored
-    const int8_t* w;      // [N,K] weight codes
-    int M, N, K;
-    const int32_t* wsum;  // [N] sum_k w[n,k]; may be null when a_zp == 0
-    int a_zp;             // zero point of the stored activation codes
-    const float* a_zp_dev; // optional device scalar: effective zero point = int(*a_zp_dev) + a_zp
-    const float* a_scale; // [M] or [1]
-    int a_scale_per_row;
-    const float* w_scale; // [N]
-    const void* bias;     // [N] f32 / f16, or null
-    int bias_dtype;
-    int relu;
-    int out_mode;
-    const float* out_scale;  // device scalars, used by the two requantizing modes
-    const float* out_zp;
-    int out_qmin, out_qmax, out_offset;
-    void* out;            // [M, ldo]
-    long ldo;
-    const int8_t* zeros;  // >= 16 zero bytes, source for K-tail chunks
-};
-
-// ---------------------------------------------------------------- epilogue
-struct ColParams {
-    float ws, bias;
-    int32_t corr;  // a_zp * wsum[n]
-};
-
-__device__ __forceinline__ ColParams load_col(const GemmArgs& g, int n) {
-    ColParams c;
-    c.ws = g.w_scale ? g.w_scale[n] : 1.0f;
-    const int zp = g.a_zp_dev ? int(g.a_zp_dev[0]) + g.a_zp : g.a_zp;
-    c.corr = (g.wsum && zp != 0) ? zp * g.wsum[n] : 0;
-    if (g.bias == nullptr)
-        c.bias = 0.0f;
-    else if (g.bias_dtype == LQ_F16)
-        c.bias = float(static_cast<const _Float16*>(g.bias)[n]);
-    else
-        c.bias = static_cast<const float*>(g.bias)[n];
-    return c;
-}
-
-__device__ __forceinline__ float q_core(float x, float s, float z, float lo, float hi) {
-    float t = x / s;
-    float r = __builtin_rintf(t);
-    float u = r + z;
-    u = (u < lo) ? lo : ((u > hi) ? hi : u);
-    return u;
-}
-
-// One output element.  Float steps are separate (no FMA) and in the order the
-// CPU restatement uses, so results are bit-identical to it.  MODE is a
-// compile-time constant so that each output form gets a tight loop.
-// epilogue_value returns the element as 32 bits (float bits, or the integer
-// for the accumulator / requantized-code forms); store_* narrows and writes.
-template <int MODE>
-__device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t acc, float as,
-                                                   const ColParams& c, float S, float Z) {
-    if (MODE == OUT_ACC_I32) return uint32_t(acc);
-    float f = float(acc - c.corr);
-    float sc = as * c.ws;
-    float y = f * sc;
-    if (g.bias) y = y + c.bias;
-    if (g.relu) y = (y < 0.0f) ? 0.0f : y;
-    if (MODE == OUT_F32 || MODE == OUT_F16) return __float_as_uint(y);
-    float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
-    if (MODE == OUT_REQUANT_I8) {
-        int code = (qv != qv) ? 0 : int(qv);
-        return uint32_t(code + g.out_offset);
-    }
-    return __float_as_uint((qv - Z) * S);  // OUT_FAKEQUANT_F32
-}
-
-template <int MODE>
-__device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint32_t v) {
-    if (MODE == OUT_F16)
-        static_cast<_Float16*>(g.out)[idx] = _Float16(__uint_as_float(v));
-    else if (MODE == OUT_REQUANT_I8)
-        static_cast<int8_t*>(g.out)[idx] = int8_t(int(v));
-    else
-        static_cast<uint32_t*>(g.out)[idx] = v;  // f32 / i32 bit patterns
-}
-
-// four consecutive elements; idx is a multiple of 4 and the row is 4-aligned
-template <int MODE>
-__device__ __forceinline__ void store_vec4(const GemmArgs& g, size_t idx, uint4 v) {
-    if (MODE == OUT_F16) {
-        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-        h4 h = {_Float16(__uint_as_float(v.x)), _Float16(__uint_as_float(v.y)),
-                _Float16(__uint_as_float(v.z)), _Float16(__uint_as_float(v.w))};
-        *reinterpret_cast<h4*>(static_cast<_Float16*>(g.out) + idx) = h;
-    } else if (MODE == OUT_REQUANT_I8) {
-        uint32_t packed = (v.x & 0xffu) | ((v.y & 0xffu) << 8) | ((v.z & 0xffu) << 16) | (v.w << 24);
-        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(g.out) + idx) = packed;
-    } else {
-        *reinterpret_cast<uint4*>(static_cast<uint32_t*>(g.out) + idx) = v;
-    }
-}
-
-template <int MODE>
-__device__ __forceinline__ void epilogue_store_t(const GemmArgs& g, int m, int n, int32_t acc,
-                                                 float as, const ColParams& c, float S, float Z) {
-    store_scalar<MODE>(g, size_t(m) * size_t(g.ldo) + size_t(n),
-                       epilogue_value<MODE>(g, acc, as, c, S, Z));
-}
-
-__device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, int32_t acc,
-                                               float as, const ColParams& c, float S, float Z) {
-    switch (g.out_mode) {
-    case OUT_ACC_I32: epilogue_store_t<OUT_ACC_I32>(g, m, n, acc, as, c, S, Z); break;
-    case OUT_F32: epilogue_store_t<OUT_F32>(g, m, n, acc, as, c, S, Z); break;
-    case OUT_F16: epilogue_store_t<OUT_F16>(g, m, n, acc, as, c, S, Z); break;
-    case OUT_REQUANT_I8: epilogue_store_t<OUT_REQUANT_I8>(g, m, n, acc, as, c, S, Z); break;
-    default: epilogue_store_t<OUT_FAKEQUANT_F32>(g, m, n, acc, as, c, S, Z); break;
-    }
-}
 
 // ---------------------------------------------------------------- tile kernel
 // Compile-time shape of one tile kernel.
@@ -203,8 +86,8 @@ __device__ __forceinline__ void tile_coords(int bid, int nblk, int tiles_m, int 
 template <class Cfg, int MODE>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg::TM][Cfg::TN],
                                               const ColParams (&cp)[Cfg::TN], const float* s_as,
-                                              uint32_t* stage, int m0, int n0, int wm, int wn,
-                                              int lane, float S, float Z) {
+                                              uint32_t* stage, int m0, int n0, int n_limit, int wm,
+                                              int wn, int lane, float S, float Z) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, STRIDE = Cfg::STAGE_STRIDE;
     constexpr int QUADS_PER_ROW = TN * 8;            // four-column groups per staged row
     constexpr int PASSES = 32 * QUADS_PER_ROW / 64;
@@ -230,15 +113,15 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
             const int row = q / QUADS_PER_ROW, cq = (q % QUADS_PER_ROW) * 4;
             const uint4 v = *reinterpret_cast<const uint4*>(stage + row * STRIDE + cq);
             const int m = m0 + band + row, n = n0 + wn * (TN * 32) + cq;
-            if (m < g.M && n < g.N) {
+            if (m < g.M && n < n_limit) {
                 const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
-                if (vec_ok && n + 4 <= g.N) {
+                if (vec_ok && n + 4 <= n_limit) {
                     store_vec4<MODE>(g, idx, v);
                 } else {
                     store_scalar<MODE>(g, idx, v.x);
-                    if (n + 1 < g.N) store_scalar<MODE>(g, idx + 1, v.y);
-                    if (n + 2 < g.N) store_scalar<MODE>(g, idx + 2, v.z);
-                    if (n + 3 < g.N) store_scalar<MODE>(g, idx + 3, v.w);
+                    if (n + 1 < n_limit) store_scalar<MODE>(g, idx + 1, v.y);
+                    if (n + 2 < n_limit) store_scalar<MODE>(g, idx + 2, v.z);
+                    if (n + 3 < n_limit) store_scalar<MODE>(g, idx + 3, v.w);
                 }
             }
         }
@@ -252,7 +135,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
 // 16 fragment rows of a pass fall on 16 different bank groups.  A wavefront's
 // direct global->LDS load writes 1 KiB of consecutive slots, so the swizzle is
 // applied on the global side: a lane fetches the chunk that belongs in its slot.
-template <class Cfg, int MODE>
+template <class Cfg, int MODE, bool CONV>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel(GemmArgs g) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
     constexpr int C = Cfg::C, R = Cfg::R, PA = Cfg::PA, PB = Cfg::PB, STAGES = Cfg::STAGES;
@@ -262,7 +145,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     int tm, tn;
     tile_coords(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int n_base = int(blockIdx.y) * g.N;  // first column of this group (0 for a plain GEMM)
+    const int n_limit = n_base + g.N;
+    const int m0 = tm * BM, n0 = n_base + tn * BN;
     const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
 
     // ---- global -> LDS addressing.  In pass `it` this lane fills the slot of
@@ -272,12 +157,27 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
     const int row_in_pass = tid / C;
     const int kc = (tid % C) ^ ((row_in_pass / R) % C);
     unsigned a_off[PA], b_off[PB];
-    const int a_rows = g.M - m0, b_rows = g.N - n0;  // valid rows in this tile (>= 1)
+    int a_hw[PA];  // CONV: top-left input coordinate of the pixel, (ih0 << 16) | (iw0 & 0xffff)
+    const int a_rows = g.M - m0, b_rows = n_limit - n0;  // valid rows in this tile (>= 1)
 #pragma unroll
     for (int it = 0; it < PA; ++it) {
         int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
         r = r < a_rows ? r : a_rows - 1;  // clamp: reads stay in bounds, rows are masked at the store
-        a_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
+        if (CONV) {
+            const int m = m0 + r;
+            const int pix = g.cOH * g.cOW;
+            const int b = m / pix, rem = m - b * pix;
+            const int oh = rem / g.cOW, ow = rem - oh * g.cOW;
+            const int ih0 = oh * g.csh - g.cph, iw0 = ow * g.csw - g.cpw;
+            a_hw[it] = (ih0 << 16) | (iw0 & 0xffff);
+            // may wrap for ih0 / iw0 < 0; it is only used after the bounds check,
+            // together with a tap offset that brings it back in range
+            a_off[it] = unsigned((b * g.cH + ih0) * g.cW + iw0) * unsigned(g.cCin) +
+                        unsigned(int(blockIdx.y) * g.cCg);
+        } else {
+            a_hw[it] = 0;
+            a_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
+        }
     }
 #pragma unroll
     for (int it = 0; it < PB; ++it) {
@@ -285,17 +185,34 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         r = r < b_rows ? r : b_rows - 1;
         b_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
     }
-    const int8_t* a_tile = g.a + size_t(m0) * g.K;
+    const int8_t* a_tile = CONV ? g.cx : g.a + size_t(m0) * g.K;
     const int8_t* b_tile = g.w + size_t(n0) * g.K;
 
     auto load_stage = [&](int k0, int8_t* stage) {
-        const bool in_k = (k0 + kc * 16) < g.K;  // K-tail chunks and look-ahead stages: zeros
+        const int k = k0 + kc * 16;
+        const bool in_k = k < g.K;  // K-tail chunks and look-ahead stages: zeros
         int8_t* sa = stage + wave * 1024;
         int8_t* sb = stage + BM * BK + wave * 1024;
+        if (CONV) {
+            // this lane's 16 bytes lie inside one filter tap (Cg % 16 == 0)
+            const int tap = k / g.cCg, ci0 = k - tap * g.cCg;
+            const int kh = tap / g.cKW, kw = tap - kh * g.cKW;
+            const int dh = kh * g.cdh, dw = kw * g.cdw;
+            const unsigned delta = unsigned(dh * g.cW + dw) * unsigned(g.cCin) + unsigned(ci0);
 #pragma unroll
-        for (int it = 0; it < PA; ++it) {
-            const int8_t* src = in_k ? a_tile + k0 + a_off[it] : g.zeros;
-            __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
+            for (int it = 0; it < PA; ++it) {
+                const int ih = (a_hw[it] >> 16) + dh;
+                const int iw = int(short(a_hw[it] & 0xffff)) + dw;
+                const bool ok = in_k && unsigned(ih) < unsigned(g.cH) && unsigned(iw) < unsigned(g.cW);
+                const int8_t* src = ok ? a_tile + (a_off[it] + delta) : g.pad_src;
+                __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < PA; ++it) {
+                const int8_t* src = in_k ? a_tile + k0 + a_off[it] : g.zeros;
+                __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
+            }
         }
 #pragma unroll
         for (int it = 0; it < PB; ++it) {
@@ -404,10 +321,10 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int n = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
-        cp[j] = load_col(g, n < g.N ? n : g.N - 1);
+        cp[j] = load_col(g, n < n_limit ? n : n_limit - 1);
     }
     __syncthreads();
-    tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, wm, wn, lane, S, Z);
+    tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z);
 }
 
 // Tile shapes.  "big" keeps LDS traffic per MFMA lowest (one block per CU);
@@ -418,10 +335,11 @@ using CfgBig64 = TileCfg<256, 256, 64, 2, 2, 4, 1>;
 using CfgWide = TileCfg<256, 128, 64, 2, 2, 3, 2>;
 using CfgTall = TileCfg<128, 256, 64, 2, 2, 3, 2>;
 using CfgMid = TileCfg<128, 128, 64, 2, 2, 4, 2>;
+using CfgN64 = TileCfg<256, 64, 64, 4, 1, 3, 2>;  // 64 output columns (early ResNet stages)
 
-template <class Cfg, int MODE>
-int launch_tile_mode(const GemmArgs& g, hipStream_t st) {
-    const void* fn = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE>);
+template <class Cfg, int MODE, bool CONV>
+int launch_tile_mode(const GemmArgs& g, int groups, hipStream_t st) {
+    const void* fn = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV>);
     static bool attr_set = false;
     if (!attr_set) {
         LQ_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
@@ -430,20 +348,46 @@ int launch_tile_mode(const GemmArgs& g, hipStream_t st) {
     const int tiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
     GemmArgs copy = g;
     void* kargs[] = {&copy};
-    LQ_HIP(hipLaunchKernel(fn, dim3(tiles), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
+    LQ_HIP(hipLaunchKernel(fn, dim3(tiles, groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
     return LQ_OK;
 }
 
-template <class Cfg>
-int launch_tile(const GemmArgs& g, hipStream_t st) {
+template <class Cfg, bool CONV>
+int launch_tile(const GemmArgs& g, int groups, hipStream_t st) {
     LQ_REQUIRE(size_t(Cfg::BM > Cfg::BN ? Cfg::BM : Cfg::BN) * g.K < 0xffffffffull, LQ_ERR_SHAPE,
-               "qlinear_i8: K too large");
+               "tile kernel: K too large");
     switch (g.out_mode) {
-    case OUT_ACC_I32: return launch_tile_mode<Cfg, OUT_ACC_I32>(g, st);
-    case OUT_F32: return launch_tile_mode<Cfg, OUT_F32>(g, st);
-    case OUT_F16: return launch_tile_mode<Cfg, OUT_F16>(g, st);
-    case OUT_REQUANT_I8: return launch_tile_mode<Cfg, OUT_REQUANT_I8>(g, st);
-    default: return launch_tile_mode<Cfg, OUT_FAKEQUANT_F32>(g, st);
+    case OUT_ACC_I32: return launch_tile_mode<Cfg, OUT_ACC_I32, CONV>(g, groups, st);
+    case OUT_F32: return launch_tile_mode<Cfg, OUT_F32, CONV>(g, groups, st);
+    case OUT_F16: return launch_tile_mode<Cfg, OUT_F16, CONV>(g, groups, st);
+    case OUT_REQUANT_I8: return launch_tile_mode<Cfg, OUT_REQUANT_I8, CONV>(g, groups, st);
+    default: return launch_tile_mode<Cfg, OUT_FAKEQUANT_F32, CONV>(g, groups, st);
+    }
+}
+
+// cfg: 0 = choose from the problem shape, 1..6 = a specific tile shape.
+template <bool CONV>
+int launch_tile_cfg(const GemmArgs& g, int groups, int cfg, hipStream_t st) {
+    if (cfg == 0) {
+        // 128 x 256 tiles keep two blocks per CU busy and measured fastest from
+        // M = 2048 to 8192 at N = 11008; narrower tiles when N is small or when
+        // the wide ones would leave most of the 256 CUs without work.
+        const long mt128 = (g.M + 127) / 128;
+        if (g.N <= 64)
+            cfg = 6;
+        else if (g.N <= 128 || mt128 * ((g.N + 255) / 256) * groups < 256)
+            cfg = 5;
+        else
+            cfg = 4;
+    }
+    switch (cfg) {
+    case 1: return launch_tile<CfgBig, CONV>(g, groups, st);
+    case 2: return launch_tile<CfgBig64, CONV>(g, groups, st);
+    case 3: return launch_tile<CfgWide, CONV>(g, groups, st);
+    case 4: return launch_tile<CfgTall, CONV>(g, groups, st);
+    case 5: return launch_tile<CfgMid, CONV>(g, groups, st);
+    case 6: return launch_tile<CfgN64, CONV>(g, groups, st);
+    default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
 
@@ -569,19 +513,64 @@ __global__ void rowsum_i8_kernel(const int8_t* __restrict__ w, int32_t* __restri
 // ---------------------------------------------------------------- host side
 namespace lq {
 
-// 16 zero bytes per device for K-tail chunks of the tile kernel.
-int zero_block(const int8_t** ptr) {
-    static void* zeros[16] = {nullptr};
+int pad_table(const int8_t** table) {
+    static void* tables[16] = {nullptr};
     int dev = 0;
     LQ_HIP(hipGetDevice(&dev));
     LQ_REQUIRE(dev >= 0 && dev < 16, LQ_ERR_DEVICE, "device index %d out of range", dev);
-    if (!zeros[dev]) {
+    if (!tables[dev]) {
+        uint8_t host[256 * 16];
+        for (int v = 0; v < 256; ++v)
+            for (int i = 0; i < 16; ++i) host[v * 16 + i] = uint8_t(v);
         void* p = nullptr;
-        LQ_HIP(hipMalloc(&p, 256));
-        LQ_HIP(hipMemset(p, 0, 256));
-        zeros[dev] = p;
+        LQ_HIP(hipMalloc(&p, sizeof host));
+        LQ_HIP(hipMemcpy(p, host, sizeof host, hipMemcpyHostToDevice));
+        tables[dev] = p;
     }
-    *ptr = static_cast<const int8_t*>(zeros[dev]);
+    *table = static_cast<const int8_t*>(tables[dev]);
+    return LQ_OK;
+}
+
+int run_tile_kernel(const GemmArgs& g_in, bool conv, int groups, int tile_config, hipStream_t st) {
+    GemmArgs g = g_in;
+    const int8_t* table = nullptr;
+    int rc = pad_table(&table);
+    if (rc) return rc;
+    g.zeros = table;
+    if (conv) {
+        const int zp = g.a_zp;  // the stored code of real 0.0
+        g.pad_src = table + size_t(uint8_t(int8_t(zp))) * 16;
+        return launch_tile_cfg<true>(g, groups, tile_config, st);
+    }
+    return launch_tile_cfg<false>(g, 1, tile_config, st);
+}
+
+int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t st) {
+    GemmArgs g = g_in;
+    const bool vec_ok = g.K % 16 == 0 && g.K > 0 && aligned16(g.a) && aligned16(g.w);
+    int path = force_path;  // 0 = choose, 1 = tile, 2 = skinny, 3 = naive
+    if (path == 0) path = !vec_ok ? 3 : (g.M <= 64 ? 2 : 1);
+    LQ_REQUIRE(path == 3 || vec_ok, LQ_ERR_VALUE,
+               "qlinear_i8: MFMA paths need K %% 16 == 0 and 16-byte aligned operands");
+    if (path == 1) {
+        int rc = run_tile_kernel(g, false, 1, tile_config, st);
+        if (rc) return rc;
+    } else if (path == 2) {
+        LQ_REQUIRE(g.M <= 64, LQ_ERR_SHAPE, "qlinear_i8: skinny path needs M <= 64 (M = %d)", g.M);
+        dim3 grid{unsigned((g.N + 15) / 16)}, block{256};
+        if (g.M <= 16)
+            hipLaunchKernelGGL((qgemm_skinny_kernel<1>), grid, block, 0, st, g);
+        else if (g.M <= 32)
+            hipLaunchKernelGGL((qgemm_skinny_kernel<2>), grid, block, 0, st, g);
+        else
+            hipLaunchKernelGGL((qgemm_skinny_kernel<4>), grid, block, 0, st, g);
+        LQ_CHECK_LAUNCH("qgemm_skinny");
+    } else {
+        size_t blocks = (size_t(g.M) * g.N + 255) / 256;
+        if (blocks > 65536) blocks = 65536;
+        hipLaunchKernelGGL(qgemm_naive_kernel, dim3(unsigned(blocks)), dim3(256), 0, st, g);
+        LQ_CHECK_LAUNCH("qgemm_naive");
+    }
     return LQ_OK;
 }
 
@@ -646,50 +635,9 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
     g.out_scale = p->out_scale; g.out_zp = p->out_zp;
     g.out_qmin = p->out_qmin; g.out_qmax = p->out_qmax; g.out_offset = p->out_offset;
     g.out = p->out; g.ldo = ldo; g.zeros = nullptr;
+    g.cx = nullptr; g.pad_src = nullptr;
 
-    hipStream_t st = as_stream(stream);
-    const bool vec_ok = p->K % 16 == 0 && p->K > 0 && aligned16(p->a) && aligned16(p->w);
-    int path = p->force_path;  // 0 = choose, 1 = tile, 2 = skinny, 3 = naive
-    if (path == 0) path = !vec_ok ? 3 : (p->M <= 64 ? 2 : 1);
-    LQ_REQUIRE(path == 3 || vec_ok, LQ_ERR_VALUE,
-               "qlinear_i8: MFMA paths need K %% 16 == 0 and 16-byte aligned operands");
-    if (path == 1) {
-        int rc = zero_block(&g.zeros);
-        if (rc) return rc;
-        int cfg = p->tile_config;
-        if (cfg == 0) {
-            // 128 x 256 tiles keep two blocks per CU busy and measured fastest from
-            // M = 2048 to 8192 at N = 11008; fall back to 128 x 128 when that would
-            // leave most of the 256 CUs without a tile.
-            const long tiles_tall = long((p->M + 127) / 128) * ((p->N + 255) / 256);
-            cfg = tiles_tall >= 256 ? 4 : 5;
-        }
-        switch (cfg) {
-        case 1: rc = launch_tile<CfgBig>(g, st); break;
-        case 2: rc = launch_tile<CfgBig64>(g, st); break;
-        case 3: rc = launch_tile<CfgWide>(g, st); break;
-        case 4: rc = launch_tile<CfgTall>(g, st); break;
-        case 5: rc = launch_tile<CfgMid>(g, st); break;
-        default: rc = launch_tile<CfgBig>(g, st); break;
-        }
-        if (rc) return rc;
-    } else if (path == 2) {
-        LQ_REQUIRE(p->M <= 64, LQ_ERR_SHAPE, "qlinear_i8: skinny path needs M <= 64 (M = %d)", p->M);
-        dim3 grid{unsigned((p->N + 15) / 16)}, block{256};
-        if (p->M <= 16)
-            hipLaunchKernelGGL((qgemm_skinny_kernel<1>), grid, block, 0, st, g);
-        else if (p->M <= 32)
-            hipLaunchKernelGGL((qgemm_skinny_kernel<2>), grid, block, 0, st, g);
-        else
-            hipLaunchKernelGGL((qgemm_skinny_kernel<4>), grid, block, 0, st, g);
-        LQ_CHECK_LAUNCH("qgemm_skinny");
-    } else {
-        size_t blocks = (size_t(p->M) * p->N + 255) / 256;
-        if (blocks > 65536) blocks = 65536;
-        hipLaunchKernelGGL(qgemm_naive_kernel, dim3(unsigned(blocks)), dim3(256), 0, st, g);
-        LQ_CHECK_LAUNCH("qgemm_naive");
-    }
-    return LQ_OK;
+    return run_gemm(g, p->force_path, p->tile_config, as_stream(stream));
 }
 
 }  // extern "C"

@@ -1,0 +1,53 @@
+// Internal interface between the GEMM / convolution translation units.
+#pragma once
+#include "common.hpp"
+
+namespace lq {
+
+enum { OUT_ACC_I32 = 0, OUT_F32 = 1, OUT_F16 = 2, OUT_REQUANT_I8 = 3, OUT_FAKEQUANT_F32 = 4 };
+
+struct GemmArgs {
+    const int8_t* a;      // [M,K] activation codes as stored
+    const int8_t* w;      // [N,K] weight codes
+    int M, N, K;
+    const int32_t* wsum;  // [N] sum_k w[n,k]; may be null when a_zp == 0
+    int a_zp;             // zero point of the stored activation codes
+    const float* a_zp_dev; // optional device scalar: effective zero point = int(*a_zp_dev) + a_zp
+    const float* a_scale; // [M] or [1]
+    int a_scale_per_row;
+    const float* w_scale; // [N]
+    const void* bias;     // [N] f32 / f16, or null
+    int bias_dtype;
+    int relu;
+    int out_mode;
+    const float* out_scale;  // device scalars, used by the two requantizing modes
+    const float* out_zp;
+    int out_qmin, out_qmax, out_offset;
+    void* out;            // [M, ldo]
+    long ldo;
+    const int8_t* zeros;  // >= 16 zero bytes, source for K-tail chunks
+    // Implicit-GEMM convolution (tile kernel instantiated with CONV = true): the
+    // A operand is gathered from NHWC activation codes; row m is output pixel
+    // (b, oh, ow), column k is ((kh*KW + kw)*Cg + ci).  N is then the output
+    // channels of ONE group and blockIdx.y selects the group.
+    const int8_t* cx;       // NHWC codes
+    const int8_t* pad_src;  // 16 bytes holding the zero-point code (out-of-image taps)
+    int cH, cW, cCin, cOH, cOW, cKW, cCg, csh, csw, cph, cpw, cdh, cdw;
+};
+
+
+// 256 blocks of 16 bytes; block v is filled with byte value v.  Block 0 is the
+// zero source for K-tail chunks, block (uint8)zp the source for out-of-image
+// convolution taps.
+int pad_table(const int8_t** table);
+
+// Launches the MFMA tile kernel on a filled-in GemmArgs.  conv = true gathers
+// the A operand from NHWC codes (cx / c* fields); `groups` becomes gridDim.y.
+int run_tile_kernel(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st);
+
+
+// Chooses between the tile, skinny and naive kernels (force_path: 0 = choose,
+// 1 = tile, 2 = skinny, 3 = naive) and launches.
+int run_gemm(const GemmArgs& g, int force_path, int tile_config, hipStream_t st);
+
+}  // namespace lq

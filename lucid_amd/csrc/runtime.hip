@@ -206,7 +206,7 @@ const OpSchema kOps[] = {
     {"minmax", 1, 1},        {"calc_qparams", 1, 1}, {"quantize", 1, 1},
     {"dequantize", 1, 1},    {"fake_quantize", 1, 1}, {"rowsum_i8", 1, 1},
     {"qlinear_i8", 1, 1},    {"relu", 1, 1},          {"minmax_fold", 1, 1},
-    {"add_requant_i8", 1, 1},
+    {"add_requant_i8", 1, 1}, {"qconv2d_i8", 1, 1},    {"maxpool2d_nhwc_i8", 1, 1},
 };
 }  // namespace
 

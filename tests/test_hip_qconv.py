@@ -1,0 +1,137 @@
+"""GPU parity of the quantized Conv2d forward (``lq_qconv2d_i8``) and its
+layout helpers against the CPU oracle: int32 accumulators and requantized
+codes bit for bit on every route (1x1-as-GEMM, implicit GEMM, explicit im2col,
+naive), including ResNet-50's layer shapes, asymmetric padding, dilation,
+groups and ragged extents."""
+
+import numpy as np
+import pytest
+
+import lucid_amd as L
+from lucid_amd import _C, _ops
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GEMM, IMPLICIT, IM2COL, NAIVE = _ops.CONV_GEMM, _ops.CONV_IMPLICIT, _ops.CONV_IM2COL, _ops.CONV_NAIVE
+
+
+def hip(a):
+    return L.tensor(np.ascontiguousarray(a), device="hip")
+
+
+def codes(rng, shape, lo=-128, hi=127):
+    return rng.integers(lo, hi + 1, shape).astype(np.int8)
+
+
+CASES = [
+    # B, H, W, Cin, Cout, KH, KW, stride, pad(hlo,hhi,wlo,whi), dil, groups, routes
+    (2, 9, 11, 16, 24, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1, (IMPLICIT, IM2COL, NAIVE)),
+    (1, 14, 14, 3, 16, 7, 7, (2, 2), (3, 3, 3, 3), (1, 1), 1, (IM2COL, NAIVE)),       # stem-like
+    (2, 8, 8, 32, 64, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), 1, (GEMM, IMPLICIT, IM2COL, NAIVE)),
+    (2, 8, 8, 64, 32, 1, 1, (2, 2), (0, 0, 0, 0), (1, 1), 1, (IMPLICIT, NAIVE)),       # downsample
+    (1, 10, 9, 32, 16, 3, 3, (2, 1), (0, 1, 1, 2), (1, 2), 2, (IMPLICIT, IM2COL, NAIVE)),
+    (1, 6, 6, 8, 8, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 4, (IM2COL, NAIVE)),
+    (3, 17, 13, 48, 70, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1, (IMPLICIT, NAIVE)),     # ragged M, N
+    (2, 28, 28, 128, 128, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1, (IMPLICIT,)),          # ResNet 3x3
+    (2, 14, 14, 256, 256, 3, 3, (2, 2), (1, 1, 1, 1), (1, 1), 1, (IMPLICIT,)),          # stride-2 3x3
+    (2, 14, 14, 1024, 256, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), 1, (GEMM,)),
+    (2, 56, 56, 64, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1, (IMPLICIT,)),            # N = 64 tile
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_accumulators_exact_on_every_route(case):
+    B, H, W, Cin, Cout, KH, KW, st, pad, dil, groups, routes = case
+    rng = np.random.default_rng(sum(case[:7]))
+    x = codes(rng, (B, H, W, Cin))
+    w = codes(rng, (Cout, KH, KW, Cin // groups))
+    a_zp = -17
+    exp = O.qconv2d(x, w, a_zp, 1.0, np.ones(Cout, np.float32), stride=st, pad=pad, dilation=dil,
+                    groups=groups, out_mode=O.OUT_ACC_I32)
+    xd, wd = hip(x), hip(w)
+    for route in routes:
+        got = _ops.qconv2d_i8(xd, wd, a_zp=a_zp, stride=st, pad=pad, dilation=dil, groups=groups,
+                              out_mode=_ops.OUT_ACC_I32, path=route).numpy()
+        assert got.shape == exp.shape and np.array_equal(got, exp), f"route {route}"
+    auto = _ops.qconv2d_i8(xd, wd, a_zp=a_zp, stride=st, pad=pad, dilation=dil, groups=groups,
+                           out_mode=_ops.OUT_ACC_I32).numpy()
+    assert np.array_equal(auto, exp)
+
+
+@pytest.mark.parametrize("case", [CASES[0], CASES[1], CASES[3], CASES[4], CASES[7]])
+@pytest.mark.parametrize("relu,bias_kind", [(True, "f32"), (False, "f32"), (True, None)])
+def test_epilogue_bit_exact(case, relu, bias_kind):
+    B, H, W, Cin, Cout, KH, KW, st, pad, dil, groups, routes = case
+    rng = np.random.default_rng(7 + sum(case[:7]))
+    x = codes(rng, (B, H, W, Cin))
+    w = codes(rng, (Cout, KH, KW, Cin // groups))
+    a_zp = int(rng.integers(-128, -60))
+    a_scale = np.float32(rng.uniform(0.005, 0.03))
+    w_scale = rng.uniform(0.0005, 0.004, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32) if bias_kind else None
+    kw = dict(stride=st, pad=pad, dilation=dil, groups=groups, bias=bias, relu=relu)
+    y = O.qconv2d(x, w, a_zp, a_scale, w_scale, out_mode=O.OUT_F32, **kw)
+    S = np.float32(np.abs(y).max() / 200 + 1e-6)
+    Z = np.float32(0.0 if relu else 128.0)
+    wsum = _ops.rowsum_i8(hip(w))
+    assert np.array_equal(wsum.numpy(), O.rowsum_i8(w))
+    dkw = dict(stride=st, pad=pad, dilation=dil, groups=groups, relu=relu, a_zp=a_zp,
+               a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=wsum,
+               bias=None if bias is None else hip(bias), out_scale=hip(S), out_zp=hip(Z),
+               out_qmin=0, out_qmax=255, out_offset=-128)
+    for route in routes:
+        for mode in (_ops.OUT_F32, _ops.OUT_REQUANT_I8, _ops.OUT_FAKEQUANT_F32):
+            got = _ops.qconv2d_i8(hip(x), hip(w), out_mode=mode, path=route, **dkw).numpy()
+            exp = O.qconv2d(x, w, a_zp, a_scale, w_scale, out_mode=mode, out_scale=S, out_zp=Z,
+                            out_qmin=0, out_qmax=255, out_offset=-128, **kw)
+            if mode == _ops.OUT_REQUANT_I8:
+                assert np.array_equal(got, exp), (route, mode)
+            else:
+                assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), (route, mode)
+
+
+def test_layout_helpers_round_trip():
+    rng = np.random.default_rng(3)
+    B, Cc, H, W = 2, 37, 9, 11
+    x = (rng.standard_normal((B, Cc, H, W)) * 2).astype(np.float32)
+    s, z = hip(np.float32(0.03)), hip(np.float32(120.0))
+    q = L.Tensor.empty((B, H, W, Cc), L.int8, "hip")
+    _C.call("lq_quantize_nchw_to_nhwc", hip(x).data_ptr, q.data_ptr, -128, B, Cc, H, W,
+            s.data_ptr, z.data_ptr, 0, 255, None)
+    exp_q = O.quantize(x.transpose(0, 2, 3, 1), 0.03, 120.0, 0, 255, code_offset=-128)
+    assert np.array_equal(q.numpy(), exp_q)
+    out = L.Tensor.empty((B, Cc, H, W), L.float32, "hip")
+    _C.call("lq_dequantize_nhwc_to_nchw", q.data_ptr, -128, out.data_ptr, B, Cc, H, W, s.data_ptr,
+            z.data_ptr, None)
+    exp = O.dequantize(exp_q, 0.03, 120.0, code_offset=-128).transpose(0, 3, 1, 2)
+    assert np.array_equal(out.numpy().view(np.uint32), np.ascontiguousarray(exp).view(np.uint32))
+    assert np.array_equal(out.numpy().view(np.uint32),
+                          O.fake_quantize(x, 0.03, 120.0, 0, 255).view(np.uint32))
+    w = codes(rng, (10, 6, 3, 5))
+    wo = L.Tensor.empty((10, 3, 5, 6), L.int8, "hip")
+    _C.call("lq_repack_oihw_to_ohwi_i8", hip(w).data_ptr, wo.data_ptr, 10, 6, 3, 5, None)
+    assert np.array_equal(wo.numpy(), w.transpose(0, 2, 3, 1))
+
+
+def test_maxpool_on_codes():
+    rng = np.random.default_rng(4)
+    x = codes(rng, (2, 13, 12, 70))
+    out = L.Tensor.empty((2, 7, 6, 70), L.int8, "hip")
+    _C.call("lq_maxpool2d_nhwc_i8", hip(x).data_ptr, out.data_ptr, 2, 13, 12, 70, 3, 3, 2, 2, 1, 1,
+            None)
+    assert np.array_equal(out.numpy(), O.maxpool2d_nhwc_i8(x, (3, 3), (2, 2), (1, 1)))
+
+
+def test_argument_validation():
+    x, w = hip(np.zeros((1, 4, 4, 16), np.int8)), hip(np.zeros((8, 3, 3, 16), np.int8))
+    with pytest.raises(L.ShapeMismatch):
+        _ops.qconv2d_i8(x, hip(np.zeros((8, 3, 3, 8), np.int8)), a_zp=0, out_mode=0)
+    with pytest.raises(L.ShapeMismatch):        # kernel larger than the padded image
+        _ops.qconv2d_i8(hip(np.zeros((1, 2, 2, 16), np.int8)), w, a_zp=0, out_mode=0)
+    with pytest.raises(ValueError):             # implicit route needs Cin/groups % 16 == 0
+        _ops.qconv2d_i8(hip(np.zeros((1, 4, 4, 8), np.int8)), hip(np.zeros((8, 3, 3, 8), np.int8)),
+                        a_zp=0, out_mode=0, path=IMPLICIT, pad=(1, 1, 1, 1))
+    with pytest.raises(ValueError):             # zero point without the filter sums
+        _ops.qconv2d_i8(x, w, a_zp=3, a_scale=hip(np.float32(1)), w_scale=hip(np.ones(8, np.float32)),
+                        pad=(1, 1, 1, 1))
