@@ -153,6 +153,21 @@ int lq_add_requant_i8(const int8_t* qa, int a_offset, const float* a_scale, cons
                       size_t n, int relu, const float* out_scale, const float* out_zp, int out_qmin,
                       int out_qmax, int out_offset, int8_t* out, lq_stream stream);
 
+/* F.adaptive_avg_pool2d(x, 1) on NHWC codes -> float32 [B, C]: Lucid pools the
+ * float-carried values, so the result leaves the grid (it feeds the float input
+ * of the classifier).  Exact integer sum of codes, then float32 scaling. */
+int lq_global_avgpool_nhwc_i8(const int8_t* q, int code_offset, int B, int H, int W, int C,
+                              const float* scale, const float* zp, float* out, lq_stream stream);
+
+/* Quantized Linear on a float activation that lies on no grid - literally
+ * lucid/nn/quantized/linear.py:199-215: dequantize(weight) -> x @ W^T + bias ->
+ * [relu] -> [fake_quantize].  float32 accumulation; for small layers (e.g. the
+ * classifier after global pooling), not a throughput path. */
+int lq_qlinear_w8a32(const float* x, const int8_t* w, const float* w_scale, const float* w_zp,
+                     const float* bias, int M, int N, int K, int relu, int fake_quantize_out,
+                     const float* out_scale, const float* out_zp, int out_qmin, int out_qmax,
+                     float* out, lq_stream stream);
+
 /* ------------------------------------------------------- quantized Linear */
 /* Output forms of the fused GEMM epilogue. */
 #define LQ_OUT_ACC_I32 0       /* raw int32 accumulators                         */

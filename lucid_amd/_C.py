@@ -115,6 +115,9 @@ _SIGNATURES["lq_relu_f32"] = [_vp, _vp, _sz, _vp]
 _SIGNATURES["lq_minmax_fold"] = [_vp, _vp, _vp, _vp, _sz, _i, _vp, _vp, _vp]
 _SIGNATURES["lq_add_requant_i8"] = [_vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _sz, _i, _vp, _vp, _i, _i,
                                     _i, _vp, _vp]
+_SIGNATURES["lq_global_avgpool_nhwc_i8"] = [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]
+_SIGNATURES["lq_qlinear_w8a32"] = [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp,
+                                   _vp]
 _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
 _SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]

@@ -88,6 +88,62 @@ __global__ __launch_bounds__(256) void add_requant_kernel(const int8_t* __restri
     }
 }
 
+// Global average pool of NHWC codes to float32 [B, C]: the exact integer sum of
+// the codes, then ((sum - HW*(Z + off)) * S) / HW in float32.
+__global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const int8_t* __restrict__ q, int off,
+                                                                  int B, int HW, int C,
+                                                                  const float* scale, const float* zp,
+                                                                  float* __restrict__ out) {
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63), b = blockIdx.y;
+    const int part = threadIdx.x >> 6;  // 4 slices of the pixels
+    __shared__ int red[4][64];
+    int s = 0;
+    if (c < C)
+        for (int p = part; p < HW; p += 4) s += q[(size_t(b) * HW + p) * C + c];
+    red[part][threadIdx.x & 63] = s;
+    __syncthreads();
+    if (part == 0 && c < C) {
+        s = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
+        const float total = float(s - off * HW) - float(HW) * zp[0];
+        out[size_t(b) * C + c] = (total * scale[0]) / float(HW);
+    }
+}
+
+// Quantized Linear on a float activation that is NOT on a grid (Lucid's own
+// formulation, lucid/nn/quantized/linear.py:199-215): y = x @ dequant(W)^T + b.
+// One wavefront per output; lanes stride over k and the partial sums are
+// folded by a butterfly, so the float summation order differs from a
+// sequential loop (Lucid's own order is Accelerate's and is not pinned either).
+__global__ __launch_bounds__(256) void qlinear_w8a32_kernel(
+    const float* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ w_scale,
+    const float* __restrict__ w_zp, const float* __restrict__ bias, int M, int N, int K, int relu,
+    int do_fq, const float* S_, const float* Z_, float lo, float hi, float* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const size_t o = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (o >= size_t(M) * N) return;
+    const int m = int(o / N), n = int(o % N);
+    const float ws = w_scale[n], wz = w_zp[n];
+    const float* xr = x + size_t(m) * K;
+    const int8_t* wr = w + size_t(n) * K;
+    float acc = 0.0f;
+    for (int k = lane; k < K; k += 64) {
+        const float wv = (float(int(wr[k])) - wz) * ws;  // dequantize, _functional.py:281
+        acc = acc + xr[k] * wv;
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) acc = acc + __shfl_xor(acc, d, 64);
+    if (lane != 0) return;
+    float y = acc;
+    if (bias) y = y + bias[n];
+    if (relu) y = (y < 0.0f) ? 0.0f : y;
+    if (do_fq) {
+        const float S = S_[0], Z = Z_[0];
+        const float qv = q_core(y, S, Z, lo, hi);
+        y = (qv - Z) * S;
+    }
+    out[o] = y;
+}
+
 inline unsigned grid_for(size_t n, size_t per_block) {
     size_t b = (n + per_block - 1) / per_block;
     if (b < 1) b = 1;
@@ -134,6 +190,38 @@ int lq_add_requant_i8(const int8_t* qa, int a_offset, const float* a_scale, cons
                        a_offset, a_scale, a_zp, qb, b_offset, b_scale, b_zp, n, relu, out_scale, out_zp,
                        float(out_qmin), float(out_qmax), out_offset, out);
     LQ_CHECK_LAUNCH("add_requant_i8");
+    return LQ_OK;
+}
+
+int lq_global_avgpool_nhwc_i8(const int8_t* q, int code_offset, int B, int H, int W, int C,
+                              const float* scale, const float* zp, float* out, lq_stream stream) {
+    if (size_t(B) * C == 0) return LQ_OK;
+    LQ_REQUIRE(q && scale && zp && out, LQ_ERR_VALUE, "global_avgpool_nhwc_i8: NULL pointer");
+    LQ_REQUIRE(H > 0 && W > 0 && size_t(H) * W < (1u << 23), LQ_ERR_SHAPE,
+               "global_avgpool_nhwc_i8: bad spatial extent %d x %d", H, W);
+    LQ_REQUIRE(B <= 65535, LQ_ERR_SHAPE, "global_avgpool_nhwc_i8: batch too large");
+    hipLaunchKernelGGL(global_avgpool_nhwc_kernel, dim3(unsigned((C + 63) / 64), unsigned(B)), dim3(256), 0,
+                       as_stream(stream), q, code_offset, B, H * W, C, scale, zp, out);
+    LQ_CHECK_LAUNCH("global_avgpool_nhwc_i8");
+    return LQ_OK;
+}
+
+int lq_qlinear_w8a32(const float* x, const int8_t* w, const float* w_scale, const float* w_zp,
+                     const float* bias, int M, int N, int K, int relu, int fake_quantize_out,
+                     const float* out_scale, const float* out_zp, int out_qmin, int out_qmax,
+                     float* out, lq_stream stream) {
+    LQ_REQUIRE(M >= 0 && N >= 0 && K >= 0, LQ_ERR_SHAPE, "qlinear_w8a32: negative extent");
+    if (size_t(M) * N == 0) return LQ_OK;
+    LQ_REQUIRE(out && w_scale && w_zp && (K == 0 || (x && w)), LQ_ERR_VALUE,
+               "qlinear_w8a32: NULL pointer");
+    LQ_REQUIRE(!fake_quantize_out || (out_scale && out_zp && out_qmin <= out_qmax), LQ_ERR_VALUE,
+               "qlinear_w8a32: output qparams missing");
+    const size_t outputs = size_t(M) * N;
+    LQ_REQUIRE((outputs + 3) / 4 <= 0x7fffffffull, LQ_ERR_SHAPE, "qlinear_w8a32: too many outputs");
+    hipLaunchKernelGGL(qlinear_w8a32_kernel, dim3(unsigned((outputs + 3) / 4)), dim3(256), 0,
+                       as_stream(stream), x, w, w_scale, w_zp, bias, M, N, K, relu, fake_quantize_out,
+                       out_scale, out_zp, float(out_qmin), float(out_qmax), out);
+    LQ_CHECK_LAUNCH("qlinear_w8a32");
     return LQ_OK;
 }
 

@@ -207,6 +207,7 @@ const OpSchema kOps[] = {
     {"dequantize", 1, 1},    {"fake_quantize", 1, 1}, {"rowsum_i8", 1, 1},
     {"qlinear_i8", 1, 1},    {"relu", 1, 1},          {"minmax_fold", 1, 1},
     {"add_requant_i8", 1, 1}, {"qconv2d_i8", 1, 1},    {"maxpool2d_nhwc_i8", 1, 1},
+    {"global_avgpool_nhwc_i8", 1, 1}, {"qlinear_w8a32", 1, 1},
 };
 }  // namespace
 

@@ -108,6 +108,52 @@ class ReLU(Module):
         return relu(x)
 
 
+class MaxPool2d(Module):
+    """``F.max_pool2d`` on a grid-carried NCHW activation: pooling the codes
+    equals pooling the values (quantization is monotone), so the result stays on
+    the input's grid."""
+
+    def __init__(self, kernel_size, stride=None, padding=0) -> None:
+        super().__init__()
+        self.kernel_size = _pair(kernel_size)
+        self.stride = _pair(stride if stride is not None else kernel_size)
+        self.padding = _pair(padding)
+
+    def forward(self, x: Tensor) -> Tensor:
+        g = x._grid if isinstance(x, Tensor) else None
+        if g is None or g.layout != "nhwc":
+            raise NotImplementedError("MaxPool2d: only grid-carried NCHW activations are supported")
+        B, H, W, Cc = g.codes.shape
+        (kh, kw), (sh, sw), (ph, pw) = self.kernel_size, self.stride, self.padding
+        OH, OW = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+        out = Tensor.empty((B, OH, OW, Cc), T.int8, "hip")
+        _C.call("lq_maxpool2d_nhwc_i8", g.codes.data_ptr, out.data_ptr, B, H, W, Cc, kh, kw, sh, sw,
+                ph, pw, None)
+        return Tensor.on_grid((B, Cc, OH, OW), T.Grid(out, g.scale, g.zero_point, g.qdtype, g.offset,
+                                                      g.zp_host, "nhwc"))
+
+
+class AdaptiveAvgPool2d(Module):
+    """``F.adaptive_avg_pool2d(x, 1)``: the mean of the float-carried values,
+    which leaves the grid - the result is an ordinary float tensor (B, C, 1, 1)."""
+
+    def __init__(self, output_size=1) -> None:
+        super().__init__()
+        if _pair(output_size) != (1, 1):
+            raise NotImplementedError("AdaptiveAvgPool2d: only global pooling (output_size=1)")
+
+    def forward(self, x: Tensor) -> Tensor:
+        g = x._grid if isinstance(x, Tensor) else None
+        if g is None or g.layout != "nhwc":
+            raise NotImplementedError(
+                "AdaptiveAvgPool2d: only grid-carried NCHW activations are supported")
+        B, H, W, Cc = g.codes.shape
+        out = Tensor.empty((B, Cc, 1, 1), T.float32, "hip")
+        _C.call("lq_global_avgpool_nhwc_i8", g.codes.data_ptr, g.offset, B, H, W, Cc,
+                g.scale.data_ptr, g.zero_point.data_ptr, out.data_ptr, None)
+        return out
+
+
 class Flatten(Module):
     def __init__(self, start_dim: int = 1) -> None:
         super().__init__()

@@ -3,9 +3,10 @@
 
 from . import dynamic
 from .functional_module import FloatFunctional, QFunctional
-from .intrinsic import LinearReLU
+from .conv import Conv2d
+from .intrinsic import ConvReLU2d, LinearReLU
 from .linear import Linear
 from .modules import DeQuantize, DeQuantStub, Quantize, QuantStub, QuantWrapper
 
-__all__ = ["Linear", "LinearReLU", "Quantize", "DeQuantize", "QuantStub", "DeQuantStub",
+__all__ = ["Linear", "LinearReLU", "Conv2d", "ConvReLU2d", "Quantize", "DeQuantize", "QuantStub", "DeQuantStub",
            "QuantWrapper", "QFunctional", "FloatFunctional", "dynamic"]

@@ -1,0 +1,148 @@
+"""Quantized ``Conv2d`` for static PTQ, on the hip implicit-GEMM int8 kernel.
+
+Mirrors ``lucid/nn/quantized/conv.py:75-229,388-542``: same constructor,
+buffers (``weight_int8`` int8 ``(Cout, Cin/groups, KH, KW)`` - Lucid's OIHW
+order is kept as the state-dict contract -, ``weight_scale`` /
+``weight_zero_point`` f32 ``(Cout,)``, ``bias``, ``scale``, ``zero_point``),
+attributes ``padding_str`` / ``padding_mode`` / ``weight_ch_axis`` /
+``out_qdtype``, ``from_float`` and the ``_activation`` hook.  The forward is
+one launch: activation codes (NHWC) x repacked weight codes through the MFMA
+GEMM with zero-point correction, scales, bias, optional ReLU and the output
+requantize in the epilogue.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+from ... import _C, _ops
+from ... import _tensor as T
+from ..._tensor import Grid, Tensor
+from ...quantization._qscheme import QDtype, quint8
+from ..module import Module
+from ._utils import (activation_qparams, host_scalar, input_grid, quantize_weight,
+                     require_symmetric_weight, storage_offset)
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, int) else tuple(v)
+
+
+def _same_pad_pair(in_size: int, kernel: int, stride: int, dilation: int) -> tuple[int, int]:
+    """``padding="same"`` amounts (``lucid/nn/modules/conv.py:44-55``): the odd
+    unit goes to the high side."""
+    out_size = (in_size + stride - 1) // stride
+    pad_total = max(0, (out_size - 1) * stride + (kernel - 1) * dilation + 1 - in_size)
+    return pad_total // 2, pad_total - pad_total // 2
+
+
+class Conv2d(Module):
+    _fused_relu = False
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size, stride=1, padding=0,
+                 dilation=1, groups: int = 1, bias: bool = True) -> None:
+        super().__init__()
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride = _pair(kernel_size), _pair(stride)
+        self.padding_str = padding if isinstance(padding, str) else None
+        self.padding = (0, 0) if isinstance(padding, str) else _pair(padding)
+        self.dilation, self.groups = _pair(dilation), groups
+        self.padding_mode = "zeros"
+        self.weight_ch_axis = 0
+        self.out_qdtype: QDtype = quint8
+        wshape = (out_channels, in_channels // groups, *self.kernel_size)
+        self.register_buffer("weight_int8", T.tensor(np.zeros(wshape, np.int8), device="hip"))
+        self.register_buffer("weight_scale", T.tensor(np.ones(out_channels, np.float32), device="hip"))
+        self.register_buffer("weight_zero_point", T.tensor(
+            np.zeros(out_channels, np.float32), device="hip"))
+        self.register_buffer("bias", T.tensor(np.zeros(out_channels, np.float32), device="hip")
+                             if bias else None)
+        self.register_buffer("scale", T.tensor(np.float32(1.0), device="hip"))
+        self.register_buffer("zero_point", T.tensor(np.float32(0.0), device="hip"))
+        self._w_ohwi = None   # weight codes repacked to (Cout, KH, KW, Cin/groups)
+        self._wsum = None
+        self._zp_host = None
+
+    def _state_loaded(self, name: str) -> None:
+        if name == "weight_int8":
+            self._w_ohwi = self._wsum = None
+        if name == "zero_point":
+            self._zp_host = None
+        if name == "weight_zero_point":
+            require_symmetric_weight(self.weight_zero_point, type(self).__name__)
+
+    def _resolve_pad(self, x: Tensor) -> tuple[int, int, int, int]:
+        """(h_lo, h_hi, w_lo, w_hi), as ``conv.py:119-141``."""
+        if self.padding_str == "valid":
+            return 0, 0, 0, 0
+        if self.padding_str == "same":
+            h = _same_pad_pair(x.shape[2], self.kernel_size[0], self.stride[0], self.dilation[0])
+            w = _same_pad_pair(x.shape[3], self.kernel_size[1], self.stride[1], self.dilation[1])
+            return h[0], h[1], w[0], w[1]
+        return self.padding[0], self.padding[0], self.padding[1], self.padding[1]
+
+    def _activation(self, y: Tensor) -> Tensor:
+        """Post-conv activation hook (identity; ReLU in the fused variant)."""
+        return y
+
+    def _prepare_weight(self) -> None:
+        O, I, KH, KW = self.weight_int8.shape
+        w = Tensor.empty((O, KH, KW, I), T.int8, "hip")
+        _C.call("lq_repack_oihw_to_ohwi_i8", self.weight_int8.data_ptr, w.data_ptr, O, I, KH, KW, None)
+        self._w_ohwi = w
+        self._wsum = _ops.rowsum_i8(w)
+
+    def forward(self, x: Tensor) -> Tensor:
+        name = type(self).__name__
+        g = input_grid(x, name)
+        if x.ndim != 4 or x.shape[1] != self.in_channels:
+            raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, H, W), got {x.shape}")
+        if self.padding_mode != "zeros":
+            raise NotImplementedError(
+                f"{name}: padding_mode={self.padding_mode!r} is not supported by the hip kernels")
+        if g.zp_host is None:
+            raise NotImplementedError(
+                f"{name}: the input zero point is only known on the device; convolution needs it "
+                "on the host for the padding code (static quantization provides it)")
+        if g.layout != "nhwc":
+            raise _C.LucidError(f"{name}: 4-d activation codes must be stored NHWC")
+        if self._w_ohwi is None:
+            self._prepare_weight()
+        if self._zp_host is None:
+            self._zp_host = int(host_scalar(self.zero_point))
+        off = storage_offset(self.out_qdtype)
+        codes = _ops.qconv2d_i8(
+            g.codes, self._w_ohwi, a_zp=int(g.zp_host) + g.offset, a_scale=g.scale,
+            w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias, stride=self.stride,
+            pad=self._resolve_pad(x), dilation=self.dilation, groups=self.groups,
+            relu=self._fused_relu, out_mode=_ops.OUT_REQUANT_I8, out_scale=self.scale,
+            out_zp=self.zero_point, out_qmin=self.out_qdtype.quant_min,
+            out_qmax=self.out_qdtype.quant_max, out_offset=off)
+        B, OH, OW, Co = codes.shape
+        return Tensor.on_grid((B, Co, OH, OW), Grid(codes, self.scale, self.zero_point,
+                                                    self.out_qdtype, off, self._zp_host, "nhwc"))
+
+    @classmethod
+    def from_float(cls, mod) -> "Conv2d":
+        """Quantize a calibrated float ``Conv2d`` (``conv.py:186-222``)."""
+        qmod = cls(mod.in_channels, mod.out_channels, mod.kernel_size, mod.stride, mod.padding,
+                   mod.dilation, mod.groups, bias=mod.bias is not None)
+        codes, w_scale, w_zp, ch_axis = quantize_weight(mod)
+        require_symmetric_weight(w_zp, cls.__name__)
+        qmod.register_buffer("weight_int8", codes)
+        qmod.register_buffer("weight_scale", w_scale)
+        qmod.register_buffer("weight_zero_point", w_zp)
+        qmod.weight_ch_axis = ch_axis
+        qmod.padding_str = getattr(mod, "_padding_str", None)
+        qmod.padding_mode = getattr(mod, "padding_mode", "zeros")
+        if mod.bias is not None:
+            qmod.register_buffer("bias", mod.bias.to("hip"))
+        a_scale, a_zp, a_qdtype = activation_qparams(mod)
+        qmod.register_buffer("scale", a_scale)
+        qmod.register_buffer("zero_point", a_zp)
+        qmod.out_qdtype = a_qdtype
+        return qmod
+
+    def extra_repr(self) -> str:
+        return (f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}, "
+                f"stride={self.stride}, qdtype={self.out_qdtype.name}")

@@ -3,6 +3,7 @@ before the output requantize, inside the kernel epilogue."""
 
 from __future__ import annotations
 
+from .conv import Conv2d
 from .linear import Linear
 
 
@@ -19,6 +20,23 @@ class LinearReLU(Linear):
     def from_float(cls, mod) -> "LinearReLU":
         # an nni.LinearReLU is a Sequential(Linear, ReLU) that carries the qconfig
         # and the activation observer of the fused pair
+        inner = mod[0]
+        inner.qconfig = mod.qconfig
+        inner.activation_post_process = mod.activation_post_process
+        return super().from_float(inner)
+
+
+class ConvReLU2d(Conv2d):
+    """Quantized ``Conv2d`` + ``ReLU`` (``intrinsic.py:334-341``)."""
+
+    _fused_relu = True
+
+    def _activation(self, y):
+        from .. import relu
+        return relu(y)
+
+    @classmethod
+    def from_float(cls, mod) -> "ConvReLU2d":
         inner = mod[0]
         inner.qconfig = mod.qconfig
         inner.activation_post_process = mod.activation_post_process

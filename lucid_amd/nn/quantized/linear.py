@@ -14,7 +14,7 @@ from __future__ import annotations
 
 import numpy as np
 
-from ... import _ops
+from ... import _C, _ops
 from ... import _tensor as T
 from ..._tensor import Grid, Tensor
 from ...quantization._qscheme import QDtype, quint8
@@ -57,11 +57,31 @@ class Linear(Module):
         Kept for API parity; the hip forward fuses the ReLU into the GEMM."""
         return y
 
-    def forward(self, x: Tensor) -> Tensor:
-        g = input_grid(x, type(self).__name__)
+    def _forward_float(self, x: Tensor) -> Tensor:
+        """Input is a float tensor on no grid (e.g. after global average
+        pooling): Lucid's own formulation - dequantized weight, float GEMM,
+        fake-quantized output - in one small kernel."""
         K, N = self.in_features, self.out_features
+        M = x.numel // K
+        y = Tensor.empty((M, N), T.float32, "hip")
+        _C.call("lq_qlinear_w8a32", x.data_ptr, self.weight_int8.data_ptr,
+                self.weight_scale.data_ptr, self.weight_zero_point.data_ptr,
+                self.bias.data_ptr if self.bias is not None else None, M, N, K,
+                int(self._fused_relu), 1, self.scale.data_ptr, self.zero_point.data_ptr,
+                self.out_qdtype.quant_min, self.out_qdtype.quant_max, y.data_ptr, None)
+        return y.reshape(*x.shape[:-1], N)
+
+    def forward(self, x: Tensor) -> Tensor:
+        K, N = self.in_features, self.out_features
+        if not isinstance(x, Tensor) or x.device != "hip":
+            raise _C.DeviceMismatch(f"{type(self).__name__}: input must be on the 'hip' device")
         if x.shape[-1] != K:
-            raise T._C.ShapeMismatch(f"expected last dim {K}, got {x.shape}")
+            raise _C.ShapeMismatch(f"expected last dim {K}, got {x.shape}")
+        if x._grid is None or x._grid.layout != "plain":
+            if x.dtype != T.float32:
+                raise _C.DtypeMismatch(f"{type(self).__name__} expects float32, got {x.dtype}")
+            return self._forward_float(x)
+        g = x._grid
         M = x.numel // K
         if self._wsum is None:
             self._wsum = _ops.rowsum_i8(self.weight_int8)

@@ -50,6 +50,15 @@ class Quantize(Module):
         if self._zp_host is None:
             self._zp_host = int(host_scalar(self.zero_point))
         off = storage_offset(self.qdtype)
+        if x.ndim == 4:
+            # an image batch: codes go channel-last, the layout of the conv kernels
+            B, Cc, H, W = x.shape
+            codes = Tensor.empty((B, H, W, Cc), T.int8, "hip")
+            _C.call("lq_quantize_nchw_to_nhwc", x.data_ptr, codes.data_ptr, off, B, Cc, H, W,
+                    self.scale.data_ptr, self.zero_point.data_ptr, self.qdtype.quant_min,
+                    self.qdtype.quant_max, None)
+            return Tensor.on_grid(x.shape, Grid(codes, self.scale, self.zero_point, self.qdtype,
+                                                off, self._zp_host, "nhwc"))
         codes = Tensor.empty(x.shape, T.int8, "hip")
         _C.call("lq_quantize", x.data_ptr, codes.data_ptr, _C.I8, off, 1, 1, x.numel,
                 self.scale.data_ptr, self.zero_point.data_ptr, 0, self.qdtype.quant_min,

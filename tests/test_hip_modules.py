@@ -224,14 +224,21 @@ class TestStaticPTQ:
         with pytest.warns(UserWarning, match="matched no quantizable"):
             Q.prepare(nn.Sequential(nn.ReLU()))
 
-    def test_plain_float_input_is_rejected_loudly(self):
+    def test_plain_float_input_runs_lucids_float_formulation(self):
+        """A float input that lies on no grid takes Lucid's own path
+        (linear.py:199-215): dequantized weight, float GEMM, fake-quantized output."""
         rng = np.random.default_rng(2)
         m, params = _static_model(rng)
         prepared = Q.prepare(m)
         _calibrate(prepared, params, rng, batches=2)
         qm = Q.convert(prepared)
-        with pytest.raises(NotImplementedError, match="quantization grid"):
-            qm.fc1(hip(np.zeros((4, 16), np.float32)))
+        x = rng.standard_normal((9, 16)).astype(np.float32)
+        y = qm.fc1(hip(x))
+        assert y._grid is None and y.shape == (9, 32)
+        wq1, ws1, wz1 = _oracle_weight(params[0])
+        s1, z1 = qm.fc1.scale.item(), qm.fc1.zero_point.item()
+        ref = O.linear_faithful(x, wq1, ws1, wz1, bias=params[1], relu=True, fq=(s1, z1, 0, 255))
+        assert np.abs(y.numpy() - ref).max() <= s1 * 1.001 and (y.numpy() != ref).mean() < 0.02
         with pytest.raises(L.DeviceMismatch):
             qm(L.tensor(np.zeros((4, 16), np.float32)))
 
