@@ -15,7 +15,8 @@ One JSON line is printed.  Besides the driver's fields it carries
   extra         the bandwidth-bound members of the path measured in the same
                 run: quantize / dequantize / min-max on the 4096x4096x16
                 round-trip tensor against the 8 TB/s HBM peak, and the
-                decode-shaped Linears (M = 1, 16) against HBM.
+                decode-shaped Linears (M = 1, 16) against HBM, and the int8
+                ResNet-50 (batch 32) in images/s.
 
 Timing: HIP events recorded on the stream the kernels are launched on (the
 default stream), through the library's own C ABI.  No PyTorch anywhere.
@@ -190,6 +191,31 @@ def bench_quant_roundtrip(L, Q, _C, steps, warmup):
     return out
 
 
+def bench_resnet50(L, _C, steps, warmup):
+    """int8 static-quantized ResNet-50, batch 32, 3x224x224 uniform[0,1] inputs,
+    random He-normal weights with BatchNorm folded, fixed calibration grids.  The
+    forward (53 convolutions, 16 residual joins, pooling, classifier: ~75
+    launches) is captured once into a HIP graph and replayed."""
+    import workloads as W
+
+    model = W.QResNet50()
+    rng = np.random.default_rng(0)
+    batch = 32
+    x = L.tensor(rng.uniform(0, 1, (batch, 3, 224, 224)).astype(np.float32), device="hip")
+    y = model(x)  # eager warm-up caches host-side scalars
+    with L.graph.capture() as g:
+        y = model(x)
+    total, per = time_launches(_C, g.replay, steps, warmup)
+    ms = total / steps
+    gmacs = W.resnet50_conv_gmacs(batch)
+    out = {"images_per_s": round(batch / ms * 1e3, 1), "ms_per_batch": round(ms, 4), "batch": batch,
+           "int8_TOP/s": round(2 * gmacs / ms, 2), "GMAC_per_batch": round(gmacs, 2),
+           "p95_ms": round(float(np.percentile(per, 95)), 4), "launch": "hip graph replay"}
+    assert np.isfinite(y.numpy()).all()
+    g.destroy()
+    return out
+
+
 def cpu_baseline_linear(K, N, sample_rows, seed=1, reps=8):
     """Lucid's CPU pass structure for this layer (dequantize the int8 weight on
     every call, float32 GEMM, bias add), run by the oracle on `sample_rows`
@@ -234,7 +260,7 @@ def main() -> int:
     M, K, N = 2048, 4096, 11008
     r = bench_linear(L, Q, _C, _ops, M, K, N, args.steps, args.warmup)
     line = {
-        "metric": "quantized-Linear int8 TOPS",
+        "metric": "quantized-Linear int8 TOPS & % MFMA peak; int8 ResNet-50 images/sec",
         "value": round(r["tops"], 2),
         "unit": "TOP/s",
         "n_gpus": 1,
@@ -278,6 +304,8 @@ def main() -> int:
             del rs["tensors"]
         extra["quant_roundtrip_4096x4096x16"] = bench_quant_roundtrip(
             L, Q, _C, max(10, args.steps // 2), max(3, args.warmup // 2))
+        extra["resnet50_int8_batch32"] = bench_resnet50(L, _C, max(10, args.steps // 2),
+                                                        max(3, args.warmup // 2))
         line["extra"] = extra
     if not args.no_cpu_baseline:
         cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))

@@ -72,6 +72,12 @@ _SIGNATURES = {
     "lq_device_name": [C.c_char_p, _sz],
     "lq_alloc": [C.POINTER(_vp), _sz],
     "lq_free": [_vp],
+    "lq_empty_cache": [],
+    "lq_memory_stats": [C.POINTER(_sz), C.POINTER(_sz)],
+    "lq_graph_begin": [_vp, C.POINTER(_i)],
+    "lq_graph_end": [_vp, _i],
+    "lq_graph_launch": [_i, _vp],
+    "lq_graph_destroy": [_i],
     "lq_h2d": [_vp, _vp, _sz, _vp],
     "lq_d2h": [_vp, _vp, _sz, _vp],
     "lq_d2d": [_vp, _vp, _sz, _vp],
@@ -177,9 +183,38 @@ def check(status: int) -> None:
         raise _STATUS_TO_EXC.get(status, LucidError)(msg)
 
 
+_current_stream = None  # lq_stream used when a caller passes None; None = the default stream
+
+
+def current_stream():
+    return _current_stream
+
+
+def set_current_stream(stream) -> None:
+    global _current_stream
+    _current_stream = stream
+
+
+def _stream_last() -> frozenset:
+    """Names of the entry points whose last parameter is the stream."""
+    global _STREAM_LAST
+    if _STREAM_LAST is None:
+        import re
+
+        text = re.sub(r"/\*.*?\*/", "", open(HEADER_PATH).read(), flags=re.S)
+        _STREAM_LAST = frozenset(re.findall(r"\b(lq_[a-z0-9_]+)\s*\([^;{}]*lq_stream\s+stream\s*\)", text))
+    return _STREAM_LAST
+
+
+_STREAM_LAST = None
+
+
 def call(name: str, *args):
-    """Call an ABI function and raise on a non-zero status."""
+    """Call an ABI function and raise on a non-zero status.  A ``None`` stream
+    argument means the current stream (see ``set_current_stream``)."""
     fn = getattr(load(), name)
+    if _current_stream is not None and args and args[-1] is None and name in _stream_last():
+        args = args[:-1] + (_current_stream,)
     rc = fn(*args)
     if name not in _NO_STATUS:
         check(rc)

@@ -34,6 +34,7 @@ from ._tensor import (
 from . import quantization
 from . import nn
 from . import backends
+from . import graph
 
 __version__ = "0.1.0"
 

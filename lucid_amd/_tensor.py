@@ -227,6 +227,18 @@ class Tensor:
             t = Tensor.from_numpy(self.numpy(), "cpu")
         return t
 
+    def copy_from(self, a) -> "Tensor":
+        """Overwrite this tensor's storage with a host array of the same shape
+        and dtype (the way to feed a new batch to a captured graph)."""
+        a = np.ascontiguousarray(a, dtype=self.dtype.np)
+        if a.shape != self.shape:
+            raise _C.ShapeMismatch(f"copy_from: {a.shape} into {self.shape}")
+        if self.device == "cpu":
+            self._host[...] = a
+        elif a.nbytes:
+            _C.call("lq_h2d", self.data_ptr, a.ctypes.data, a.nbytes, None)
+        return self
+
     def cpu(self) -> "Tensor":
         return self.to("cpu")
 

@@ -1,7 +1,9 @@
 // Runtime entry points of the C ABI: device selection, storage, transfers,
 // events, the op registry and synthetic-data fills.
 #include <cstring>
+#include <map>
 #include <mutex>
+#include <unordered_map>
 #include <vector>
 
 #include "common.hpp"
@@ -109,16 +111,189 @@ int lq_device_name(char* buf, size_t buflen) {
     return LQ_OK;
 }
 
-int lq_alloc(void** ptr, size_t nbytes) {
+// ------------------------------------------------------------------ caching allocator
+// hipMalloc / hipFree cost tens of microseconds and synchronise; a quantized
+// model allocates one output per layer.  Freed blocks are therefore kept in
+// per-device free lists keyed by their (rounded) size and handed out again.
+// Blocks are recycled in submission order, which is safe for work issued on
+// one stream; a caller that frees memory still in use on ANOTHER stream must
+// synchronise first (as with any pooled allocator).
+// While a graph is being captured (lq_graph_begin .. lq_graph_end) every block
+// allocated belongs to that graph: freeing it is deferred until the graph is
+// destroyed, so replays never write into memory that was handed to someone else.
+namespace {
+struct Pool {
+    std::multimap<size_t, void*> free_blocks;           // size -> block
+    std::unordered_map<void*, size_t> live;              // block -> size
+    std::unordered_map<void*, int> graph_owner;          // block -> graph id (while pinned)
+    size_t bytes_reserved = 0, bytes_in_use = 0;
+};
+Pool g_pool[kMaxDevices];
+std::mutex g_pool_mutex;
+int g_capturing_graph = 0;  // id of the graph being captured, 0 = none
+int g_next_graph_id = 1;
+std::unordered_map<int, std::vector<std::pair<int, void*>>> g_graph_blocks;  // id -> (dev, block)
+std::unordered_map<int, hipGraphExec_t> g_graph_exec;
+
+size_t round_size(size_t n) {
+    if (n < 512) return 512;
+    if (n < (size_t(1) << 20)) return (n + 511) / 512 * 512;
+    return (n + (size_t(2) << 20) - 1) / (size_t(2) << 20) * (size_t(2) << 20);  // 2 MiB granules
+}
+}  // namespace
+
+extern "C" int lq_alloc(void** ptr, size_t nbytes) {
     LQ_REQUIRE(ptr, LQ_ERR_VALUE, "ptr is NULL");
     *ptr = nullptr;
-    if (nbytes == 0) nbytes = 16;  // a distinct, freeable address for empty tensors
-    LQ_HIP(hipMalloc(ptr, nbytes));
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    LQ_REQUIRE(dev >= 0 && dev < kMaxDevices, LQ_ERR_DEVICE, "device index %d out of range", dev);
+    const size_t size = round_size(nbytes);
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    Pool& pool = g_pool[dev];
+    void* p = nullptr;
+    auto it = pool.free_blocks.lower_bound(size);
+    // reuse a cached block unless it would waste more than half of itself
+    if (it != pool.free_blocks.end() && it->first <= size * 2) {
+        p = it->second;
+        pool.live[p] = it->first;
+        pool.bytes_in_use += it->first;
+        pool.free_blocks.erase(it);
+    } else {
+        hipError_t e = hipMalloc(&p, size);
+        if (e == hipErrorOutOfMemory) {
+            // give cached blocks back to the driver and try once more
+            for (auto& kv : pool.free_blocks) (void)hipFree(kv.second);
+            for (auto& kv : pool.free_blocks) pool.bytes_reserved -= kv.first;
+            pool.free_blocks.clear();
+            (void)hipGetLastError();
+            e = hipMalloc(&p, size);
+        }
+        if (e != hipSuccess) return hip_fail(e, "hipMalloc");
+        pool.live[p] = size;
+        pool.bytes_reserved += size;
+        pool.bytes_in_use += size;
+    }
+    if (g_capturing_graph) {
+        pool.graph_owner[p] = g_capturing_graph;
+        g_graph_blocks[g_capturing_graph].push_back({dev, p});
+    }
+    *ptr = p;
     return LQ_OK;
 }
 
-int lq_free(void* ptr) {
-    if (ptr) LQ_HIP(hipFree(ptr));
+namespace {
+// caller holds g_pool_mutex
+void release_block(Pool& pool, void* p) {
+    auto it = pool.live.find(p);
+    if (it == pool.live.end()) return;
+    pool.bytes_in_use -= it->second;
+    pool.free_blocks.insert({it->second, p});
+    pool.live.erase(it);
+}
+}  // namespace
+
+extern "C" int lq_free(void* ptr) {
+    if (!ptr) return LQ_OK;
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    for (int dev = 0; dev < kMaxDevices; ++dev) {
+        Pool& pool = g_pool[dev];
+        if (!pool.live.count(ptr)) continue;
+        if (pool.graph_owner.count(ptr)) return LQ_OK;  // deferred until lq_graph_destroy
+        release_block(pool, ptr);
+        return LQ_OK;
+    }
+    return fail(LQ_ERR_VALUE, "lq_free: pointer %p was not allocated by lq_alloc", ptr);
+}
+
+extern "C" int lq_empty_cache(void) {
+    LQ_HIP(hipDeviceSynchronize());
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    Pool& pool = g_pool[dev];
+    for (auto& kv : pool.free_blocks) {
+        LQ_HIP(hipFree(kv.second));
+        pool.bytes_reserved -= kv.first;
+    }
+    pool.free_blocks.clear();
+    return LQ_OK;
+}
+
+extern "C" int lq_memory_stats(size_t* bytes_in_use, size_t* bytes_reserved) {
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    if (bytes_in_use) *bytes_in_use = g_pool[dev].bytes_in_use;
+    if (bytes_reserved) *bytes_reserved = g_pool[dev].bytes_reserved;
+    return LQ_OK;
+}
+
+// ------------------------------------------------------------------ graphs
+extern "C" int lq_graph_begin(lq_stream stream, int* graph_id) {
+    LQ_REQUIRE(stream, LQ_ERR_VALUE, "graph capture needs a created stream, not the default stream");
+    LQ_REQUIRE(graph_id, LQ_ERR_VALUE, "graph_id is NULL");
+    {
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        LQ_REQUIRE(g_capturing_graph == 0, LQ_ERR_VALUE, "a graph capture is already in progress");
+        g_capturing_graph = g_next_graph_id++;
+        *graph_id = g_capturing_graph;
+        g_graph_blocks[*graph_id];
+    }
+    hipError_t e = hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed);
+    if (e != hipSuccess) {
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        g_capturing_graph = 0;
+        return hip_fail(e, "hipStreamBeginCapture");
+    }
+    return LQ_OK;
+}
+
+extern "C" int lq_graph_end(lq_stream stream, int graph_id) {
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(as_stream(stream), &graph);
+    {
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        g_capturing_graph = 0;
+    }
+    if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture");
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    g_graph_exec[graph_id] = exec;
+    return LQ_OK;
+}
+
+extern "C" int lq_graph_launch(int graph_id, lq_stream stream) {
+    hipGraphExec_t exec = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        auto it = g_graph_exec.find(graph_id);
+        LQ_REQUIRE(it != g_graph_exec.end(), LQ_ERR_VALUE, "unknown graph id %d", graph_id);
+        exec = it->second;
+    }
+    LQ_HIP(hipGraphLaunch(exec, as_stream(stream)));
+    return LQ_OK;
+}
+
+extern "C" int lq_graph_destroy(int graph_id) {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    auto it = g_graph_exec.find(graph_id);
+    if (it != g_graph_exec.end()) {
+        LQ_HIP(hipGraphExecDestroy(it->second));
+        g_graph_exec.erase(it);
+    }
+    auto bt = g_graph_blocks.find(graph_id);
+    if (bt != g_graph_blocks.end()) {
+        for (auto& db : bt->second) {
+            Pool& pool = g_pool[db.first];
+            pool.graph_owner.erase(db.second);
+            release_block(pool, db.second);  // the Python owners are gone or will no-op
+        }
+        g_graph_blocks.erase(bt);
+    }
     return LQ_OK;
 }
 
