@@ -230,7 +230,9 @@ typedef struct {
     void* out;             /* [M, ldo] in the type out_mode implies          */
     long ldo;              /* output row stride in elements; 0 means N       */
     int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
-    int tile_config;       /* 0 = choose; 1..5 = a specific tile shape (tuning) */
+    int tile_config;       /* tuning: low byte 0 = choose, 1..6 = a tile shape;
+                              next byte 0 = choose, 1 = one block per tile,
+                              2 = stream-K work split                         */
 } lq_qlinear_args;
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);

@@ -135,100 +135,47 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
 // 16 fragment rows of a pass fall on 16 different bank groups.  A wavefront's
 // direct global->LDS load writes 1 KiB of consecutive slots, so the swizzle is
 // applied on the global side: a lane fetches the chunk that belongs in its slot.
-template <class Cfg, int MODE, bool CONV>
+// Balanced split of `total` k-iterations over `workers`: the first `rem` workers
+// take one iteration more.
+struct IterSplit {
+    int per, rem;
+    __host__ __device__ IterSplit(long total, int workers)
+        : per(int(total / workers)), rem(int(total % workers)) {}
+    __host__ __device__ long begin(int w) const { return long(w) * per + (w < rem ? w : rem); }
+    __host__ __device__ int owner(long it) const {
+        const long cut = long(rem) * (per + 1);
+        return it < cut ? int(it / (per + 1)) : rem + int((it - cut) / per);
+    }
+};
+
+// SK = false: one block per tile (blockIdx.x -> tile, blockIdx.y -> group).
+// SK = true ("stream-K"): gridDim.x workers split the tiles' k-iterations evenly;
+// a worker's range may start and end in the middle of a tile.  A tile touched by
+// several workers is finished without anybody waiting: every contributor stores
+// its int32 partial accumulators into its own slab, then bumps the tile's
+// arrival counter; whoever arrives last adds the other slabs to its registers
+// and runs the epilogue.  Integer partial sums add exactly, so the result does
+// not depend on who arrives when.
+template <class Cfg, int MODE, bool CONV, bool SK>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel(GemmArgs g) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
     constexpr int C = Cfg::C, R = Cfg::R, PA = Cfg::PA, PB = Cfg::PB, STAGES = Cfg::STAGES;
     constexpr int THREADS = Cfg::THREADS, KSTEPS = Cfg::KSTEPS;
     extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
+    __shared__ int s_flag;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    int tm, tn;
-    tile_coords(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
     const int n_base = int(blockIdx.y) * g.N;  // first column of this group (0 for a plain GEMM)
     const int n_limit = n_base + g.N;
-    const int m0 = tm * BM, n0 = n_base + tn * BN;
     const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+    const int nk = (g.K + BK - 1) / BK;
 
-    // ---- global -> LDS addressing.  In pass `it` this lane fills the slot of
-    // row it*ROWS_PER_PASS + tid/C, physical chunk tid%C.  ROWS_PER_PASS is a
-    // multiple of 16, so the swizzle term - and with it the logical chunk the
-    // lane fetches - is the same in every pass.
+    // global -> LDS addressing: in pass `it` this lane fills the slot of row
+    // it*ROWS_PER_PASS + tid/C, physical chunk tid%C.  ROWS_PER_PASS is a multiple
+    // of 16, so the swizzle term - and the logical chunk fetched - is the same in
+    // every pass.
     const int row_in_pass = tid / C;
     const int kc = (tid % C) ^ ((row_in_pass / R) % C);
-    unsigned a_off[PA], b_off[PB];
-    int a_hw[PA];  // CONV: top-left input coordinate of the pixel, (ih0 << 16) | (iw0 & 0xffff)
-    const int a_rows = g.M - m0, b_rows = n_limit - n0;  // valid rows in this tile (>= 1)
-#pragma unroll
-    for (int it = 0; it < PA; ++it) {
-        int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
-        r = r < a_rows ? r : a_rows - 1;  // clamp: reads stay in bounds, rows are masked at the store
-        if (CONV) {
-            const int m = m0 + r;
-            const int pix = g.cOH * g.cOW;
-            const int b = m / pix, rem = m - b * pix;
-            const int oh = rem / g.cOW, ow = rem - oh * g.cOW;
-            const int ih0 = oh * g.csh - g.cph, iw0 = ow * g.csw - g.cpw;
-            a_hw[it] = (ih0 << 16) | (iw0 & 0xffff);
-            // may wrap for ih0 / iw0 < 0; it is only used after the bounds check,
-            // together with a tap offset that brings it back in range
-            a_off[it] = unsigned((b * g.cH + ih0) * g.cW + iw0) * unsigned(g.cCin) +
-                        unsigned(int(blockIdx.y) * g.cCg);
-        } else {
-            a_hw[it] = 0;
-            a_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
-        }
-    }
-#pragma unroll
-    for (int it = 0; it < PB; ++it) {
-        int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
-        r = r < b_rows ? r : b_rows - 1;
-        b_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
-    }
-    const int8_t* a_tile = CONV ? g.cx : g.a + size_t(m0) * g.K;
-    const int8_t* b_tile = g.w + size_t(n0) * g.K;
-
-    auto load_stage = [&](int k0, int8_t* stage) {
-        const int k = k0 + kc * 16;
-        const bool in_k = k < g.K;  // K-tail chunks and look-ahead stages: zeros
-        int8_t* sa = stage + wave * 1024;
-        int8_t* sb = stage + BM * BK + wave * 1024;
-        if (CONV) {
-            // this lane's 16 bytes lie inside one filter tap (Cg % 16 == 0)
-            const int tap = k / g.cCg, ci0 = k - tap * g.cCg;
-            const int kh = tap / g.cKW, kw = tap - kh * g.cKW;
-            const int dh = kh * g.cdh, dw = kw * g.cdw;
-            const unsigned delta = unsigned(dh * g.cW + dw) * unsigned(g.cCin) + unsigned(ci0);
-#pragma unroll
-            for (int it = 0; it < PA; ++it) {
-                const int ih = (a_hw[it] >> 16) + dh;
-                const int iw = int(short(a_hw[it] & 0xffff)) + dw;
-                const bool ok = in_k && unsigned(ih) < unsigned(g.cH) && unsigned(iw) < unsigned(g.cW);
-                const int8_t* src = ok ? a_tile + (a_off[it] + delta) : g.pad_src;
-                __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
-            }
-        } else {
-#pragma unroll
-            for (int it = 0; it < PA; ++it) {
-                const int8_t* src = in_k ? a_tile + k0 + a_off[it] : g.zeros;
-                __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int it = 0; it < PB; ++it) {
-            const int8_t* src = in_k ? b_tile + k0 + b_off[it] : g.zeros;
-            __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sb + it * (THREADS * 16)), 16, 0, 0);
-        }
-    };
-
-    v16i acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
     // fragment addressing: lane holds row (lane & 31), 16 bytes of k at chunk
     // 2*kk + (lane >> 5) of the current 32-wide k step
     const int frag_row = lane & 31;
@@ -237,94 +184,258 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
     const int b_row_base = BM * BK + (wn * (TN * 32) + frag_row) * BK;
     const int sw = (frag_row / R) % C;
 
-    auto read_frags = [&](const int8_t* stage, int kk, v4i (&af)[TM], v4i (&bf)[TN]) {
-        const int pc = ((kk * 2 + frag_half) ^ sw) * 16;
+    v16i acc[TM][TN];
+
+    // k-iterations [kb, ke) of tile (tm, tn) into acc (zeroed first)
+    auto run_segment = [&](int tm, int tn, int kb, int ke) {
+        const int m0 = tm * BM, n0 = n_base + tn * BN;
+        unsigned a_off[PA], b_off[PB];
+        int a_hw[PA];  // CONV: top-left input coordinate of the pixel, (ih0 << 16) | (iw0 & 0xffff)
+        const int a_rows = g.M - m0, b_rows = n_limit - n0;  // valid rows in this tile (>= 1)
+#pragma unroll
+        for (int it = 0; it < PA; ++it) {
+            int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
+            r = r < a_rows ? r : a_rows - 1;  // clamp: reads stay in bounds, rows are masked at the store
+            if (CONV) {
+                const int m = m0 + r;
+                const int pix = g.cOH * g.cOW;
+                const int b = m / pix, rem = m - b * pix;
+                const int oh = rem / g.cOW, ow = rem - oh * g.cOW;
+                const int ih0 = oh * g.csh - g.cph, iw0 = ow * g.csw - g.cpw;
+                a_hw[it] = (ih0 << 16) | (iw0 & 0xffff);
+                // may wrap for ih0 / iw0 < 0; it is only used after the bounds check,
+                // together with a tap offset that brings it back in range
+                a_off[it] = unsigned((b * g.cH + ih0) * g.cW + iw0) * unsigned(g.cCin) +
+                            unsigned(int(blockIdx.y) * g.cCg);
+            } else {
+                a_hw[it] = 0;
+                a_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < PB; ++it) {
+            int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
+            r = r < b_rows ? r : b_rows - 1;
+            b_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
+        }
+        const int8_t* a_tile = CONV ? g.cx : g.a + size_t(m0) * g.K;
+        const int8_t* b_tile = g.w + size_t(n0) * g.K;
+        const int k_end = ke * BK < g.K ? ke * BK : g.K;  // nothing is fetched past the segment
+
+        auto load_stage = [&](int k0, int8_t* stage) {
+            const int k = k0 + kc * 16;
+            const bool in_k = k < k_end;  // K-tail chunks and look-ahead stages: zeros
+            int8_t* sa = stage + wave * 1024;
+            int8_t* sb = stage + BM * BK + wave * 1024;
+            if (CONV) {
+                // this lane's 16 bytes lie inside one filter tap (Cg % 16 == 0)
+                const int tap = k / g.cCg, ci0 = k - tap * g.cCg;
+                const int kh = tap / g.cKW, kw = tap - kh * g.cKW;
+                const int dh = kh * g.cdh, dw = kw * g.cdw;
+                const unsigned delta = unsigned(dh * g.cW + dw) * unsigned(g.cCin) + unsigned(ci0);
+#pragma unroll
+                for (int it = 0; it < PA; ++it) {
+                    const int ih = (a_hw[it] >> 16) + dh;
+                    const int iw = int(short(a_hw[it] & 0xffff)) + dw;
+                    const bool ok = in_k && unsigned(ih) < unsigned(g.cH) && unsigned(iw) < unsigned(g.cW);
+                    const int8_t* src = ok ? a_tile + (a_off[it] + delta) : g.pad_src;
+                    __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int it = 0; it < PA; ++it) {
+                    const int8_t* src = in_k ? a_tile + k0 + a_off[it] : g.zeros;
+                    __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < PB; ++it) {
+                const int8_t* src = in_k ? b_tile + k0 + b_off[it] : g.zeros;
+                __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sb + it * (THREADS * 16)), 16, 0, 0);
+            }
+        };
+
+        auto read_frags = [&](const int8_t* stage, int kk, v4i (&af)[TM], v4i (&bf)[TN]) {
+            const int pc = ((kk * 2 + frag_half) ^ sw) * 16;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                af[i] = *reinterpret_cast<const v4i*>(stage + a_row_base + i * 32 * BK + pc);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                bf[j] = *reinterpret_cast<const v4i*>(stage + b_row_base + j * 32 * BK + pc);
+        };
+
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-            af[i] = *reinterpret_cast<const v4i*>(stage + a_row_base + i * 32 * BK + pc);
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-            bf[j] = *reinterpret_cast<const v4i*>(stage + b_row_base + j * 32 * BK + pc);
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+        // All STAGES buffers are kept in flight.  The fragments of k step kk+1
+        // are fetched from LDS while the MFMAs of step kk run; the hand-over to
+        // the next stage (wait for its data, barrier, fetch its first fragments,
+        // refill the buffer just drained) sits inside the last k step of the
+        // current stage, so its latency is covered by that step's MFMAs.  Stages
+        // past the end are loaded from the block of zeros, which keeps the number
+        // of outstanding loads - and so the vmcnt to wait for - constant.
+#pragma unroll
+        for (int s = 0; s < STAGES; ++s) load_stage((kb + s) * BK, smem + s * Cfg::STAGE_BYTES);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 1) * (PA + PB)));
+        __syncthreads();
+
+        v4i af[2][TM], bf[2][TN];
+        read_frags(smem, 0, af[0], bf[0]);
+
+        auto k_steps = [&](int t, bool last_stage) {  // t counts from 0 within the segment
+            const int slot = t % STAGES;
+            int8_t* cur = smem + slot * Cfg::STAGE_BYTES;
+            const int8_t* nxt = smem + (slot + 1 == STAGES ? 0 : slot + 1) * Cfg::STAGE_BYTES;
+#pragma unroll
+            for (int kk = 0; kk < KSTEPS; ++kk) {
+                if (kk + 1 < KSTEPS) {
+                    read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+                } else if (!last_stage) {
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * (PA + PB)));
+                    __syncthreads();  // stage t+1 is complete in LDS; nobody reads stage t any more
+                    read_frags(nxt, 0, af[0], bf[0]);
+                    load_stage((kb + t + STAGES) * BK, cur);
+                }
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[kk & 1][i], bf[kk & 1][j],
+                                                                          acc[i][j], 0, 0, 0);
+                // issue order inside the step: one MFMA, one LDS read, ... then the rest of
+                // the MFMAs.  The MFMA goes first so that the wait for the previous step's
+                // fragments is not held up by a read issued just before it.
+                if (kk + 1 < KSTEPS || !last_stage) {
+#pragma unroll
+                    for (int x = 0; x < TM + TN; ++x) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        const int n_it = ke - kb;
+        for (int t = 0; t + 1 < n_it; ++t) k_steps(t, false);
+        k_steps(n_it - 1, true);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the zero-filled look-ahead stages
+        __syncthreads();                            // all fragment reads done before LDS is reused
     };
 
-    // ---- main loop.  All STAGES buffers are kept in flight.  The fragments
-    // of k step kk+1 are fetched from LDS while the MFMAs of step kk run; the
-    // hand-over to the next stage (wait for its data, barrier, fetch its first
-    // fragments, refill the buffer just drained) sits inside the last k step
-    // of the current stage, so its latency is covered by that step's MFMAs.
-    // Stages past the end of K are loaded from the block of zeros, which keeps
-    // the number of outstanding loads - and so the vmcnt to wait for - constant.
-    const int nk = (g.K + BK - 1) / BK;
+    // Row scales are staged in LDS and column parameters are loaded before the
+    // first store, so no global load sits between the stores.
+    auto run_epilogue = [&](int tm, int tn) {
+        const int m0 = tm * BM, n0 = n_base + tn * BN;
+        float* s_as = reinterpret_cast<float*>(smem);
+        uint32_t* stage = reinterpret_cast<uint32_t*>(smem + 4 * BM) + wave * Cfg::STAGE_WORDS;
+        for (int rr = tid; rr < BM; rr += THREADS) {
+            const int m = m0 + rr;
+            float v = 1.0f;
+            if (g.a_scale) v = g.a_scale[(g.a_scale_per_row && m < g.M) ? m : 0];
+            s_as[rr] = v;
+        }
+        float S = 1.0f, Z = 0.0f;
+        if (MODE == OUT_REQUANT_I8 || MODE == OUT_FAKEQUANT_F32) {
+            S = g.out_scale[0];
+            Z = g.out_zp[0];
+        }
+        ColParams cp[TN];
 #pragma unroll
-    for (int s = 0; s < STAGES; ++s) load_stage(s * BK, smem + s * Cfg::STAGE_BYTES);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 1) * (PA + PB)));
-    __syncthreads();
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+            cp[j] = load_col(g, n < n_limit ? n : n_limit - 1);
+        }
+        __syncthreads();
+        tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z);
+    };
 
-    v4i af[2][TM], bf[2][TN];
-    read_frags(smem, 0, af[0], bf[0]);
+    if (!SK) {
+        int tm, tn;
+        tile_coords(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
+        run_segment(tm, tn, 0, nk);
+        run_epilogue(tm, tn);
+        return;
+    }
 
-    auto k_steps = [&](int t, bool last_stage) {
-        const int slot = t % STAGES;
-        int8_t* cur = smem + slot * Cfg::STAGE_BYTES;
-        const int8_t* nxt = smem + (slot + 1 == STAGES ? 0 : slot + 1) * Cfg::STAGE_BYTES;
-#pragma unroll
-        for (int kk = 0; kk < KSTEPS; ++kk) {
-            if (kk + 1 < KSTEPS) {
-                read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-            } else if (!last_stage) {
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * (PA + PB)));
-                __syncthreads();  // stage t+1 is complete in LDS; nobody reads stage t any more
-                read_frags(nxt, 0, af[0], bf[0]);
-                load_stage((t + STAGES) * BK, cur);
-            }
+    // ---- stream-K
+    constexpr int kAccWords = TM * TN * 16;  // accumulator registers per lane
+    const int workers = gridDim.x;
+    const long total = long(tiles_m) * tiles_n * nk;
+    const IterSplit split(total, workers);
+    // give every XCD a contiguous range of workers (blocks are dealt round-robin)
+    const int wq = workers / 8, wr = workers % 8;
+    const int xcd = blockIdx.x % 8;
+    const int me = xcd * wq + (xcd < wr ? xcd : wr) + blockIdx.x / 8;
+    long it = split.begin(me);
+    const long it_end = split.begin(me + 1);
+    int* counters = g.sk_counters + size_t(blockIdx.y) * tiles_m * tiles_n;
+    int32_t* slabs = g.sk_slabs + size_t(blockIdx.y) * workers * 2 * size_t(kAccWords) * THREADS;
+    while (it < it_end) {
+        const int tile = int(it / nk);
+        const int kb = int(it - long(tile) * nk);
+        const int ke = (it_end - it) < (nk - kb) ? kb + int(it_end - it) : nk;
+        // same m-fastest walk in groups of 8 m-tiles as tile_coords
+        int tm, tn;
+        {
+            constexpr int GM = 8;
+            const int group_size = GM * tiles_n;
+            const int group = tile / group_size;
+            const int first_m = group * GM;
+            const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+            const int in_group = tile - group * group_size;
+            tm = first_m + in_group % gsz;
+            tn = in_group / gsz;
+        }
+        run_segment(tm, tn, kb, ke);
+        bool finish = true;
+        if (!(kb == 0 && ke == nk)) {
+            const int w_first = split.owner(long(tile) * nk);
+            const int w_last = split.owner(long(tile) * nk + nk - 1);
+            // slab 0 holds a worker's leading partial tile, slab 1 its trailing one
+            auto slab_of = [&](int w) {
+                const int first_tile = int(split.begin(w) / nk);
+                return slabs + (size_t(w) * 2 + (tile == first_tile ? 0 : 1)) * kAccWords * THREADS;
+            };
+            int32_t* mine = slab_of(me);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[kk & 1][i], bf[kk & 1][j],
-                                                                      acc[i][j], 0, 0, 0);
-            // issue order inside the step: one MFMA, one LDS read, ... then the rest of the
-            // MFMAs.  The MFMA goes first so that the wait for the previous step's
-            // fragments is not held up by a read issued just before it.
-            if (kk + 1 < KSTEPS || !last_stage) {
 #pragma unroll
-                for (int x = 0; x < TM + TN; ++x) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    for (int r = 0; r < 16; ++r)
+                        mine[((i * TN + j) * 16 + r) * THREADS + tid] = acc[i][j][r];
+            __threadfence();  // partials visible device-wide before the arrival is counted
+            __syncthreads();
+            if (tid == 0) s_flag = atomicAdd(&counters[tile], 1);
+            __syncthreads();
+            finish = s_flag == (w_last - w_first);  // the other contributors have all arrived
+            if (finish) {
+                __threadfence();
+                for (int w = w_first; w <= w_last; ++w) {
+                    if (w == me) continue;
+                    const int32_t* other = slab_of(w);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r)
+                                acc[i][j][r] += __builtin_nontemporal_load(
+                                    &other[((i * TN + j) * 16 + r) * THREADS + tid]);
                 }
-                __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+                if (tid == 0) counters[tile] = 0;  // ready for the next launch
             }
-            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
         }
-    };
-    for (int t = 0; t + 1 < nk; ++t) k_steps(t, false);
-    k_steps(nk - 1, true);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the zero-filled look-ahead stages
-    __syncthreads();                            // all fragment reads done before LDS is reused below
-
-    // ---- epilogue.  Row scales are staged in LDS and column parameters are
-    // loaded before the first store, so no global load sits between the stores.
-    float* s_as = reinterpret_cast<float*>(smem);
-    uint32_t* stage = reinterpret_cast<uint32_t*>(smem + 4 * BM) + wave * Cfg::STAGE_WORDS;
-    for (int rr = tid; rr < BM; rr += THREADS) {
-        const int m = m0 + rr;
-        float v = 1.0f;
-        if (g.a_scale) v = g.a_scale[(g.a_scale_per_row && m < g.M) ? m : 0];
-        s_as[rr] = v;
+        if (finish) run_epilogue(tm, tn);
+        it += ke - kb;
     }
-    float S = 1.0f, Z = 0.0f;
-    if (MODE == OUT_REQUANT_I8 || MODE == OUT_FAKEQUANT_F32) {
-        S = g.out_scale[0];
-        Z = g.out_zp[0];
-    }
-    ColParams cp[TN];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int n = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
-        cp[j] = load_col(g, n < n_limit ? n : n_limit - 1);
-    }
-    __syncthreads();
-    tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z);
 }
 
 // Tile shapes.  "big" keeps LDS traffic per MFMA lowest (one block per CU);
@@ -337,37 +448,102 @@ using CfgTall = TileCfg<128, 256, 64, 2, 2, 3, 2>;
 using CfgMid = TileCfg<128, 128, 64, 2, 2, 4, 2>;
 using CfgN64 = TileCfg<256, 64, 64, 4, 1, 3, 2>;  // 64 output columns (early ResNet stages)
 
+// Stream-K scratch per device: arrival counters (zero between launches: the
+// finisher of a tile resets its counter) and two accumulator slabs per worker.
+struct SkScratch {
+    int* counters = nullptr;
+    size_t counter_count = 0;
+    int32_t* slabs = nullptr;
+    size_t slab_bytes = 0;
+};
+SkScratch g_sk[16];
+
+int sk_scratch(size_t counters, size_t slab_bytes, SkScratch** out) {
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    LQ_REQUIRE(dev >= 0 && dev < 16, LQ_ERR_DEVICE, "device index %d out of range", dev);
+    SkScratch& s = g_sk[dev];
+    if (s.counter_count < counters) {
+        LQ_HIP(hipDeviceSynchronize());
+        if (s.counters) LQ_HIP(hipFree(s.counters));
+        s.counters = nullptr;
+        const size_t want = counters < 65536 ? 65536 : counters;
+        LQ_HIP(hipMalloc(&s.counters, want * sizeof(int)));
+        LQ_HIP(hipMemset(s.counters, 0, want * sizeof(int)));
+        s.counter_count = want;
+    }
+    if (s.slab_bytes < slab_bytes) {
+        LQ_HIP(hipDeviceSynchronize());
+        if (s.slabs) LQ_HIP(hipFree(s.slabs));
+        s.slabs = nullptr;
+        LQ_HIP(hipMalloc(&s.slabs, slab_bytes));
+        s.slab_bytes = slab_bytes;
+    }
+    *out = &s;
+    return LQ_OK;
+}
+
 template <class Cfg, int MODE, bool CONV>
-int launch_tile_mode(const GemmArgs& g, int groups, hipStream_t st) {
-    const void* fn = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV>);
+int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
+    const void* fn_dp = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV, false>);
+    const void* fn_sk = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV, true>);
     static bool attr_set = false;
     if (!attr_set) {
-        LQ_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
+        LQ_HIP(hipFuncSetAttribute(fn_dp, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
+        LQ_HIP(hipFuncSetAttribute(fn_sk, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
         attr_set = true;
     }
     const int tiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
+    const int nk = (g.K + Cfg::BK - 1) / Cfg::BK;
+    // blocks that fit on the chip at once: 256 CUs x blocks per CU (LDS-bound)
+    const int per_cu = (160 * 1024) / Cfg::SMEM < Cfg::MINWAVES ? (160 * 1024) / Cfg::SMEM : Cfg::MINWAVES;
+    const int slots = 256 * (per_cu < 1 ? 1 : per_cu);
+    // schedule: 0 = choose, 1 = one block per tile, 2 = stream-K.
+    // Stream-K pays when the tiles fill the last round of blocks badly and there
+    // are few rounds; every worker must get at least a few k-iterations.
+    // Stream-K is opt-in only.  Measured at M=2048, N=11008, K=4096 it loses to one
+    // block per tile (128x256 tiles: 116 us vs 371 us; 175 us even with the
+    // device-scope fences taken out): the 128 KiB partial slabs per worker and the
+    // L2 write-back / invalidate of the fences cost more than the idle tail they remove.
+    const bool sk = schedule == 2;
     GemmArgs copy = g;
     void* kargs[] = {&copy};
-    LQ_HIP(hipLaunchKernel(fn, dim3(tiles, groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
+    if (!sk) {
+        LQ_HIP(hipLaunchKernel(fn_dp, dim3(tiles, groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
+        return LQ_OK;
+    }
+    long workers = slots / groups;
+    if (workers < 1) workers = 1;
+    if (workers > long(tiles) * nk) workers = long(tiles) * nk;
+    SkScratch* s = nullptr;
+    const size_t slab_words = size_t(Cfg::TM) * Cfg::TN * 16 * Cfg::THREADS;
+    int rc = sk_scratch(size_t(tiles) * groups, size_t(groups) * workers * 2 * slab_words * 4, &s);
+    if (rc) return rc;
+    copy.sk_counters = s->counters;
+    copy.sk_slabs = s->slabs;
+    LQ_HIP(hipLaunchKernel(fn_sk, dim3(unsigned(workers), groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
     return LQ_OK;
 }
 
 template <class Cfg, bool CONV>
-int launch_tile(const GemmArgs& g, int groups, hipStream_t st) {
+int launch_tile(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
     LQ_REQUIRE(size_t(Cfg::BM > Cfg::BN ? Cfg::BM : Cfg::BN) * g.K < 0xffffffffull, LQ_ERR_SHAPE,
                "tile kernel: K too large");
     switch (g.out_mode) {
-    case OUT_ACC_I32: return launch_tile_mode<Cfg, OUT_ACC_I32, CONV>(g, groups, st);
-    case OUT_F32: return launch_tile_mode<Cfg, OUT_F32, CONV>(g, groups, st);
-    case OUT_F16: return launch_tile_mode<Cfg, OUT_F16, CONV>(g, groups, st);
-    case OUT_REQUANT_I8: return launch_tile_mode<Cfg, OUT_REQUANT_I8, CONV>(g, groups, st);
-    default: return launch_tile_mode<Cfg, OUT_FAKEQUANT_F32, CONV>(g, groups, st);
+    case OUT_ACC_I32: return launch_tile_mode<Cfg, OUT_ACC_I32, CONV>(g, groups, schedule, st);
+    case OUT_F32: return launch_tile_mode<Cfg, OUT_F32, CONV>(g, groups, schedule, st);
+    case OUT_F16: return launch_tile_mode<Cfg, OUT_F16, CONV>(g, groups, schedule, st);
+    case OUT_REQUANT_I8: return launch_tile_mode<Cfg, OUT_REQUANT_I8, CONV>(g, groups, schedule, st);
+    default: return launch_tile_mode<Cfg, OUT_FAKEQUANT_F32, CONV>(g, groups, schedule, st);
     }
 }
 
-// cfg: 0 = choose from the problem shape, 1..6 = a specific tile shape.
+// tile_config: low byte = tile shape (0 = choose from the problem shape, 1..6 =
+// a specific one), next byte = schedule (0 = choose, 1 = block per tile, 2 = stream-K).
 template <bool CONV>
-int launch_tile_cfg(const GemmArgs& g, int groups, int cfg, hipStream_t st) {
+int launch_tile_cfg(const GemmArgs& g, int groups, int tile_config, hipStream_t st) {
+    int cfg = tile_config & 0xff;
+    const int schedule = (tile_config >> 8) & 0xff;
     if (cfg == 0) {
         // 128 x 256 tiles keep two blocks per CU busy and measured fastest from
         // M = 2048 to 8192 at N = 11008; narrower tiles when N is small or when
@@ -381,12 +557,12 @@ int launch_tile_cfg(const GemmArgs& g, int groups, int cfg, hipStream_t st) {
             cfg = 4;
     }
     switch (cfg) {
-    case 1: return launch_tile<CfgBig, CONV>(g, groups, st);
-    case 2: return launch_tile<CfgBig64, CONV>(g, groups, st);
-    case 3: return launch_tile<CfgWide, CONV>(g, groups, st);
-    case 4: return launch_tile<CfgTall, CONV>(g, groups, st);
-    case 5: return launch_tile<CfgMid, CONV>(g, groups, st);
-    case 6: return launch_tile<CfgN64, CONV>(g, groups, st);
+    case 1: return launch_tile<CfgBig, CONV>(g, groups, schedule, st);
+    case 2: return launch_tile<CfgBig64, CONV>(g, groups, schedule, st);
+    case 3: return launch_tile<CfgWide, CONV>(g, groups, schedule, st);
+    case 4: return launch_tile<CfgTall, CONV>(g, groups, schedule, st);
+    case 5: return launch_tile<CfgMid, CONV>(g, groups, schedule, st);
+    case 6: return launch_tile<CfgN64, CONV>(g, groups, schedule, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -415,25 +591,37 @@ __global__ __launch_bounds__(256) void qgemm_skinny_kernel(GemmArgs g) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = v4i{0, 0, 0, 0};
 
+    // Weight bytes are streamed once, so memory-level parallelism is what counts:
+    // PF K blocks (4 KiB per wavefront each) are requested before the first MFMA.
+    constexpr int PF = 4;
     const int8_t* wrow = g.w + size_t(nr) * g.K;
-    for (int kb = kb0; kb < kb1; ++kb) {
-        const int kbase = kb * 256 + lg * 64;
-        v4i wf[4];
+    for (int kbc = kb0; kbc < kb1; kbc += PF) {
+        v4i wf[PF][4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int k = kbase + c * 16;
-            wf[c] = k < g.K ? *reinterpret_cast<const v4i*>(wrow + k) : v4i{0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            const int m = t * 16 + ln;
-            const int8_t* arow = g.a + size_t(m < g.M ? m : g.M - 1) * g.K;
+        for (int u = 0; u < PF; ++u) {
+            const int kbase = (kbc + u) * 256 + lg * 64;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const int k = kbase + c * 16;
-                v4i af = (k < g.K && m < g.M) ? *reinterpret_cast<const v4i*>(arow + k)
-                                              : v4i{0, 0, 0, 0};
-                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf[c], acc[t], 0, 0, 0);
+                wf[u][c] = (kbc + u < kb1 && k < g.K) ? *reinterpret_cast<const v4i*>(wrow + k)
+                                                     : v4i{0, 0, 0, 0};
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            if (kbc + u >= kb1) break;
+            const int kbase = (kbc + u) * 256 + lg * 64;
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const int m = t * 16 + ln;
+                const int8_t* arow = g.a + size_t(m < g.M ? m : g.M - 1) * g.K;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int k = kbase + c * 16;
+                    v4i af = (k < g.K && m < g.M) ? *reinterpret_cast<const v4i*>(arow + k)
+                                                  : v4i{0, 0, 0, 0};
+                    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf[u][c], acc[t], 0, 0, 0);
+                }
             }
         }
     }

@@ -33,6 +33,9 @@ struct GemmArgs {
     const int8_t* cx;       // NHWC codes
     const int8_t* pad_src;  // 16 bytes holding the zero-point code (out-of-image taps)
     int cH, cW, cCin, cOH, cOW, cKW, cCg, csh, csw, cph, cpw, cdh, cdw;
+    // stream-K scratch (set by the launcher)
+    int* sk_counters;
+    int32_t* sk_slabs;
 };
 
 

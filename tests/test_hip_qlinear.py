@@ -60,6 +60,30 @@ def test_every_tile_shape_exact(cfg, M, N, K):
     assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
 
 
+@pytest.mark.parametrize("cfg", [1, 3, 4, 5, 6])
+@pytest.mark.parametrize("M,N,K", [(300, 260, 144), (513, 1000, 576), (2048, 1100, 4096),
+                                   (256, 256, 128), (129, 77, 784), (1500, 3000, 1024)])
+def test_stream_k_schedule_exact(cfg, M, N, K):
+    """Forced stream-K work split: tiles shared between workers are finished by
+    whoever arrives last; integer partial sums make the result exact.  Launched
+    twice to show that the arrival counters are left reset."""
+    rng = np.random.default_rng(cfg * 31 + M + N + K)
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    ref = O.igemm(a, w)
+    ad, wd = hip(a), hip(w)
+    for _ in range(2):
+        acc = _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, path=TILE,
+                              tile_config=cfg | 0x200).numpy()
+        assert np.array_equal(acc, ref)
+    a_scale = rng.uniform(0.005, 0.05, M).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    got = _ops.qlinear_i8(ad, wd, a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias),
+                          out_mode=_ops.OUT_F16, path=TILE, tile_config=cfg | 0x200).numpy()
+    exp = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, out_mode=O.OUT_F16)
+    assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+
+
 @pytest.mark.parametrize("path,M", [(TILE, 300), (SKINNY, 16), (NAIVE, 9)])
 def test_extreme_codes(path, M):
     K, N = 4096, 48
