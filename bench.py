@@ -216,6 +216,74 @@ def bench_resnet50(L, _C, steps, warmup):
     return out
 
 
+def bench_dynamic_mlp(L, Q, _C, steps, warmup):
+    """Dynamic-quantized MLP Linear(784,256)-ReLU-Linear(256,10), batch 64
+    (launch-latency bound: 0.43 MOP).  Eager = one Python-driven forward (9
+    launches); graph = the same forward replayed from a HIP graph."""
+    import lucid_amd.nn as nn
+
+    rng = np.random.default_rng(1)
+    layers = []
+    for fin, fout in ((784, 256), (256, 10)):
+        lin = nn.Linear(fin, fout)
+        lin.register_buffer("weight", L.tensor((rng.standard_normal((fout, fin)) * 0.05).astype(np.float32)))
+        lin.register_buffer("bias", L.tensor((rng.standard_normal(fout) * 0.05).astype(np.float32)))
+        layers.append(lin)
+    model = Q.quantize_dynamic(nn.Sequential(layers[0], nn.ReLU(), layers[1]))
+    x = L.tensor(rng.standard_normal((64, 784)).astype(np.float32), device="hip")
+    y = model(x)
+    total, _ = time_launches(_C, lambda: model(x), steps, warmup)
+    eager_us = total / steps * 1e3
+    with L.graph.capture() as g:
+        y = model(x)
+    total, _ = time_launches(_C, g.replay, steps, warmup)
+    graph_us = total / steps * 1e3
+    assert np.isfinite(y.numpy()).all()
+    g.destroy()
+    return {"eager_us_per_forward": round(eager_us, 1), "graph_us_per_forward": round(graph_us, 1),
+            "launches_per_forward": 9}
+
+
+def bench_vit_linears(L, Q, _C, _ops, steps, warmup):
+    """The four Linear shapes of a ViT-B/16 encoder block at batch 64 (12 608
+    token rows), dynamic-quantized as nnqd.Linear does: per-tensor affine quint8
+    activations from the runtime min/max, per-row symmetric int8 weights, float32
+    output.  GEMM-only and whole-layer (min/max + qparams + quantize + GEMM) rates."""
+    M = 64 * 197
+    out = {}
+    for name, K, N in (("qkv", 768, 2304), ("proj", 768, 768), ("fc1", 768, 3072), ("fc2", 3072, 768)):
+        t = make_linear(L, Q, _C, _ops, M, K, N, seed=7)
+        x = t["x"]
+        wsum = _ops.rowsum_i8(t["wq"])
+        bias = L.tensor(np.zeros(N, np.float32), device="hip")
+        mn, mx = Q.minmax(x)
+        xs, xz = Q.calculate_qparams(mn, mx, Q.per_tensor_affine, Q.quint8)
+        xq = L.Tensor.empty((M, K), L.int8, "hip")
+        y = L.Tensor.empty((M, N), L.float32, "hip")
+
+        def quant():
+            _C.call("lq_minmax", x.data_ptr, 1, 1, M * K, mn.data_ptr, mx.data_ptr, None)
+            _C.call("lq_calc_qparams", mn.data_ptr, mx.data_ptr, 1, 0, 0, 255, 0, 1e-8, xs.data_ptr,
+                    xz.data_ptr, None)
+            _C.call("lq_quantize", x.data_ptr, xq.data_ptr, _C.I8, -128, 1, 1, M * K, xs.data_ptr,
+                    xz.data_ptr, 0, 0, 255, None)
+
+        def gemm(repeat=1):
+            _ops.qlinear_i8(xq, t["wq"], a_zp=-128, a_zp_dev=xz, a_scale=xs, w_scale=t["ws"],
+                            wsum=wsum, bias=bias, out_mode=_ops.OUT_F32, out=y, repeat=repeat)
+
+        quant()
+        total, _ = time_launches(_C, lambda: gemm(steps), 1, 1)
+        g_ms = total / steps
+        total, _ = time_launches(_C, lambda: (quant(), gemm()), steps, warmup)
+        l_ms = total / steps
+        ops = 2.0 * M * K * N
+        out[name] = {"M": M, "K": K, "N": N, "gemm_us": round(g_ms * 1e3, 1),
+                     "gemm_TOP/s": round(ops / g_ms / 1e9, 1),
+                     "layer_us": round(l_ms * 1e3, 1), "layer_TOP/s": round(ops / l_ms / 1e9, 1)}
+    return out
+
+
 def cpu_baseline_linear(K, N, sample_rows, seed=1, reps=8):
     """Lucid's CPU pass structure for this layer (dequantize the int8 weight on
     every call, float32 GEMM, bias add), run by the oracle on `sample_rows`
@@ -304,6 +372,9 @@ def main() -> int:
             del rs["tensors"]
         extra["quant_roundtrip_4096x4096x16"] = bench_quant_roundtrip(
             L, Q, _C, max(10, args.steps // 2), max(3, args.warmup // 2))
+        extra["dynamic_mlp_784_256_10_batch64"] = bench_dynamic_mlp(L, Q, _C, args.steps, args.warmup)
+        extra["vit_b16_linears_batch64"] = bench_vit_linears(L, Q, _C, _ops, max(10, args.steps // 2),
+                                                             max(3, args.warmup // 2))
         extra["resnet50_int8_batch32"] = bench_resnet50(L, _C, max(10, args.steps // 2),
                                                         max(3, args.warmup // 2))
         line["extra"] = extra
