@@ -91,6 +91,24 @@ class Conv2d(Module):
             "quantize the model (convert) first")
 
 
+class BatchNorm2d(Module):
+    """Float BatchNorm2d as a parameter / statistics holder (folded into the
+    preceding convolution by ``fuse_modules`` before quantization)."""
+
+    def __init__(self, num_features: int, eps: float = 1e-5, affine: bool = True) -> None:
+        super().__init__()
+        self.num_features, self.eps, self.affine = num_features, eps, affine
+        self.register_buffer("weight", T.tensor(np.ones(num_features, np.float32)) if affine else None)
+        self.register_buffer("bias", T.tensor(np.zeros(num_features, np.float32)) if affine else None)
+        self.register_buffer("running_mean", T.tensor(np.zeros(num_features, np.float32)))
+        self.register_buffer("running_var", T.tensor(np.ones(num_features, np.float32)))
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.BatchNorm2d.forward is not part of the hip quantized-inference backend; "
+            "fold it into the convolution with quantization.fuse_modules")
+
+
 def relu(x: Tensor) -> Tensor:
     """``F.relu``.  On a grid-carried activation with a non-negative grid the
     codes are clamped at the zero point instead of touching floats."""
@@ -164,4 +182,4 @@ class Flatten(Module):
         return x.reshape(*lead, -1)
 
 
-from . import intrinsic, quantized  # noqa: E402  (sub-packages need the classes above)
+from . import intrinsic, quantized, utils  # noqa: E402  (sub-packages need the classes above)

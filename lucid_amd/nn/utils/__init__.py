@@ -1,0 +1,3 @@
+from .fusion import fuse_conv_bn_eval
+
+__all__ = ["fuse_conv_bn_eval"]

@@ -28,12 +28,15 @@ def __getattr__(name):
     if name in ("prepare", "convert", "quantize_dynamic"):
         from . import _quantize
         return getattr(_quantize, name)
+    if name == "fuse_modules":
+        from ._fuse_modules import fuse_modules
+        return fuse_modules
     raise AttributeError(name)
 
 
 __all__ = [
     "ObserverBase", "MinMaxObserver", "PerChannelMinMaxObserver", "FixedQParamsObserver",
-    "QConfig", "get_default_qconfig", "prepare", "convert", "quantize_dynamic",
+    "QConfig", "get_default_qconfig", "prepare", "convert", "quantize_dynamic", "fuse_modules",
     "QScheme", "per_tensor_affine", "per_tensor_symmetric", "per_channel_affine",
     "per_channel_symmetric", "QDtype", "qint8", "quint8", "qint32", "qint4", "QParams",
     "calculate_qparams", "quantize", "dequantize", "fake_quantize", "minmax",

@@ -1,0 +1,54 @@
+"""``fuse_modules``: collapse Conv/BN/ReLU and Linear/ReLU runs before
+``prepare`` (``lucid/quantization/fuse_modules.py:92-185``).  The first member
+of each run is replaced by the fused module, the rest by ``Identity``."""
+
+from __future__ import annotations
+
+import copy
+from typing import Sequence
+
+from .. import nn
+from ..nn import intrinsic as nni
+from ..nn.utils.fusion import fuse_conv_bn_eval
+
+
+def _get(model, dotted: str):
+    mod = model
+    for part in dotted.split("."):
+        mod = mod._modules[part]
+    return mod
+
+
+def _set(model, dotted: str, new) -> None:
+    parts = dotted.split(".")
+    parent = model
+    for part in parts[:-1]:
+        parent = parent._modules[part]
+    parent._modules[parts[-1]] = new
+
+
+def _fuse_run(mods):
+    ids = [nn.Identity() for _ in range(len(mods) - 1)]
+    first = mods[0]
+    if isinstance(first, nn.Conv2d):
+        rest = list(mods[1:])
+        conv = first
+        if rest and isinstance(rest[0], nn.BatchNorm2d):
+            conv = fuse_conv_bn_eval(first, rest.pop(0))
+        if rest and isinstance(rest[0], nn.ReLU):
+            rest.pop(0)
+            conv = nni.ConvReLU2d(conv, nn.ReLU())
+        if not rest:
+            return [conv, *ids]
+    if isinstance(first, nn.Linear) and len(mods) == 2 and isinstance(mods[1], nn.ReLU):
+        return [nni.LinearReLU(first, nn.ReLU()), *ids]
+    raise ValueError(f"fuse_modules: unsupported pattern {[type(m).__name__ for m in mods]}")
+
+
+def fuse_modules(model, modules_to_fuse: Sequence[Sequence[str]], inplace: bool = False):
+    model = model if inplace else copy.deepcopy(model)
+    for group in modules_to_fuse:
+        mods = [_get(model, name) for name in group]
+        for name, new in zip(group, _fuse_run(mods)):
+            _set(model, name, new)
+    return model
