@@ -39,11 +39,16 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0   # MI355X published dense int8 MFMA peak, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X published HBM3E bandwidth, GB/s
 
-# HBM bytes per launch of the headline GEMM, measured with rocprofv3 --pmc
-# (FETCH_SIZE and WRITE_SIZE in separate runs, scaled by the same counters read
-# on the library's plain copy kernel); None until measured.  See
-# profiles/qlinear_m2048_traffic.txt for the runs these come from.
-MEASURED_TRAFFIC_BYTES = {"linear_m2048": None}
+# HBM bytes per launch, measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE
+# in separate runs, in KiB per dispatch, scaled by what the same counters read on
+# the library's plain 1 GiB copy kernel: fetch x2.000, write x1.000).  The runs
+# are summarised in profiles/hbm_traffic_qlinear_and_quantize.md.
+MEASURED_TRAFFIC_BYTES = {
+    "linear_m2048": int((2.0 * 95728 + 44032) * 1024),
+    "quantize_per_channel_i8": int((2.0 * 524577 + 262144) * 1024),
+    "dequantize_per_channel_i8": int((2.0 * 131350 + 1048712) * 1024),
+    "minmax_per_channel": int((2.0 * 524317 + 257) * 1024),
+}
 
 
 def _events(_C, n):
@@ -187,7 +192,7 @@ def bench_quant_roundtrip(L, Q, _C, steps, warmup):
         med = float(np.median(per))
         out[name] = {"us": round(med * 1e3, 1), "GB/s": round(nbytes / med / 1e6, 1),
                      "frac_of_8TBs": round(nbytes / med / 1e6 / PEAK_HBM_GBS, 4),
-                     "bytes": nbytes}
+                     "bytes": nbytes, "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
     return out
 
 
