@@ -150,6 +150,37 @@ def bench_act_quant_plus_linear(L, Q, _C, _ops, t, M, K, N, steps, warmup):
     return 2.0 * M * K * N / (total / steps) / 1e9
 
 
+def bench_linear_from_host(L, Q, _C, _ops, t, M, K, N, steps):
+    """The same layer when the caller holds host buffers: float32 activations
+    uploaded (pageable memory, as numpy hands them over), dynamic activation
+    quantization, GEMM, fp16 result downloaded.  Wall clock per call."""
+    rng = np.random.default_rng(7)
+    xh = rng.standard_normal((M, K)).astype(np.float32)
+    outh = np.empty((M, N), np.float16)
+    mn = L.Tensor.empty((M,), L.float32, "hip")
+    mx = L.Tensor.empty((M,), L.float32, "hip")
+    s = L.Tensor.empty((M,), L.float32, "hip")
+    z = L.Tensor.empty((M,), L.float32, "hip")
+    xq = L.Tensor.empty((M, K), L.int8, "hip")
+    times = []
+    for _ in range(steps + 2):
+        t0 = time.perf_counter()
+        _C.call("lq_h2d", t["x"].data_ptr, xh.ctypes.data, xh.nbytes, None)
+        _C.call("lq_minmax", t["x"].data_ptr, 1, M, K, mn.data_ptr, mx.data_ptr, None)
+        _C.call("lq_calc_qparams", mn.data_ptr, mx.data_ptr, M, 1, -128, 127, 1, 1e-8, s.data_ptr,
+                z.data_ptr, None)
+        _C.call("lq_quantize", t["x"].data_ptr, xq.data_ptr, _C.I8, 0, 1, M, K, s.data_ptr,
+                z.data_ptr, 0, -128, 127, None)
+        _ops.qlinear_i8(xq, t["wq"], a_scale=s, w_scale=t["ws"], bias=t["bias"],
+                        out_mode=_ops.OUT_F16, out=t["out"])
+        _C.call("lq_d2h", outh.ctypes.data, t["out"].data_ptr, outh.nbytes, None)
+        times.append(time.perf_counter() - t0)
+    dt = float(np.median(times[2:]))
+    return {"ms_per_call": round(dt * 1e3, 3), "TOP/s": round(2.0 * M * K * N / dt / 1e12, 2),
+            "host_bytes_moved": int(xh.nbytes + outh.nbytes),
+            "host_GB/s": round((xh.nbytes + outh.nbytes) / dt / 1e9, 2)}
+
+
 def bench_quant_roundtrip(L, Q, _C, steps, warmup):
     """Config: 4096 x 4096 x 16 float32, N(0,1) with 0.1 % outliers x20;
     per-channel symmetric int8 along dim 0, then per-tensor affine."""
@@ -307,7 +338,19 @@ def cpu_baseline_linear(K, N, sample_rows, seed=1, reps=8):
         O.linear_faithful(x, wq, ws, wz, bias=bias)
         times.append(time.perf_counter() - t0)
     dt = float(np.median(times[1:]))
-    return 2.0 * sample_rows * K * N / dt / 1e12, dt, sum(times)
+    # one core, on a slice of the rows (the per-call weight dequantize is the same)
+    rows1 = min(sample_rows, 128)
+    nthreads = O.set_threads(0)
+    O.set_threads(1)
+    t1 = []
+    for i in range(3):
+        t0 = time.perf_counter()
+        O.linear_faithful(x[:rows1], wq, ws, wz, bias=bias)
+        t1.append(time.perf_counter() - t0)
+    O.set_threads(nthreads)
+    single = {"value": round(2.0 * rows1 * K * N / float(np.median(t1)) / 1e12, 5), "unit": "TOP/s",
+              "cores": 1, "sample": f"{rows1} rows, median of 3 calls"}
+    return 2.0 * sample_rows * K * N / dt / 1e12, dt, sum(times) + sum(t1), nthreads, single
 
 
 def main() -> int:
@@ -367,6 +410,8 @@ def main() -> int:
         extra["linear_with_dynamic_act_quant_TOPS"] = round(
             bench_act_quant_plus_linear(L, Q, _C, _ops, r["tensors"], M, K, N, args.steps,
                                         args.warmup), 2)
+        extra["linear_m2048_host_buffers_in_and_out"] = bench_linear_from_host(
+            L, Q, _C, _ops, r["tensors"], M, K, N, 10)
         del r["tensors"]
         for m in (1, 16):
             rs = bench_linear(L, Q, _C, _ops, m, K, N, args.steps, args.warmup, seed=3)
@@ -384,8 +429,7 @@ def main() -> int:
                                                         max(3, args.warmup // 2))
         line["extra"] = extra
     if not args.no_cpu_baseline:
-        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-        tops, dt, spent = cpu_baseline_linear(K, N, args.cpu_sample_rows)
+        tops, dt, spent, cores, single = cpu_baseline_linear(K, N, args.cpu_sample_rows)
         line["cpu_baseline"] = {
             "value": round(tops, 5),
             "unit": "TOP/s",
@@ -394,6 +438,7 @@ def main() -> int:
             "sample": f"{args.cpu_sample_rows} of {M} rows of the same layer; median of 8 calls, "
                       f"each = per-call weight dequantize + float32 GEMM + bias "
                       f"({dt:.2f} s per call, {spent:.0f} s of CPU time in all)",
+            "single_thread": single,
         }
     print(json.dumps(line))
     return 0

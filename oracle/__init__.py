@@ -48,6 +48,11 @@ def lib() -> C.CDLL:
     return _lib
 
 
+def set_threads(n: int = 0) -> int:
+    """Set (n > 0) and return the OpenMP thread count the oracle's loops use."""
+    return int(lib().orc_set_threads(int(n)))
+
+
 def _p(a: np.ndarray | None):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 

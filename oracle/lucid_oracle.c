@@ -36,8 +36,24 @@
 #include <stdlib.h>
 #include <string.h>
 
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
 #define ORC_I8 1
 #define ORC_I16 2
+
+/* Thread count of the loops below (for timing the baseline on one core and on
+ * all of them); returns the count now in force. */
+int orc_set_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+    return omp_get_max_threads();
+#else
+    (void)n;
+    return 1;
+#endif
+}
 
 /* ------------------------------------------------------------------ */
 /* element arithmetic                                                  */
