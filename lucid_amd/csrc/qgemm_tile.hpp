@@ -1,0 +1,582 @@
+// MFMA tile kernel of the int8 GEMM / implicit-GEMM convolution: template and
+// launcher.  Included by one small translation unit per tile shape, so the
+// shapes compile in parallel.
+#pragma once
+#include "common.hpp"
+#include "qgemm.hpp"
+#include "qepilogue.hpp"
+
+#include <type_traits>
+
+namespace lq {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+#define LQ_GPTR(p) ((__attribute__((address_space(1))) void*)(p))
+#define LQ_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// ---------------------------------------------------------------- tile kernel
+// Compile-time shape of one tile kernel.
+//   BM x BN x BK : block tile (BK bytes of k per LDS stage)
+//   WM x WN      : wavefront grid; each wavefront owns (BM/WM) x (BN/WN) outputs
+//                  as TM x TN MFMA tiles of 32 x 32
+//   STAGES       : LDS stages; STAGES-1 of them are in flight from global memory
+//   MINWAVES     : wavefronts per SIMD the register budget must allow
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int MINWAVES_>
+struct TileCfg {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
+    static constexpr int MINWAVES = MINWAVES_;
+    static constexpr int THREADS = WM * WN * 64;
+    static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    static constexpr int C = BK / 16;              // 16-byte chunks per LDS row
+    static constexpr int R = 16 / C;               // LDS rows per 256 bytes (one pass over 64 banks)
+    static constexpr int ROWS_PER_PASS = THREADS / C;
+    static constexpr int PA = BM / ROWS_PER_PASS, PB = BN / ROWS_PER_PASS;
+    static constexpr int KSTEPS = BK / 32;
+    static constexpr int STAGE_BYTES = (BM + BN) * BK;
+    // Three blocks per CU leave 168 registers per lane and 53 KB of LDS per block:
+    // fragments are then read just before use (the other wavefronts cover the
+    // latency) and the epilogue stages 16 rows at a time.
+    static constexpr bool PIPE = MINWAVES_ < 3;
+    static constexpr int EPI_ROWS = MINWAVES_ < 3 ? 32 : 16;
+    static constexpr int STAGE_STRIDE = TN * 32 + 4;   // words per staged output row
+    static constexpr int STAGE_WORDS = EPI_ROWS * STAGE_STRIDE;
+    static constexpr int EPI_BYTES = 4 * BM + THREADS / 64 * STAGE_WORDS * 4;
+    static constexpr int SMEM = STAGES * STAGE_BYTES > EPI_BYTES ? STAGES * STAGE_BYTES : EPI_BYTES;
+    static_assert(BK == 64 || BK == 128, "BK is 64 or 128 bytes");
+    static_assert(ROWS_PER_PASS % 16 == 0 && BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "");
+    static_assert((STAGES - 2) * (PA + PB) <= 63, "vmcnt is a 6-bit counter");
+};
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding:
+// vmcnt in bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8]).
+constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+
+// Blocks are handed to the 8 XCDs round-robin.  Give every XCD one contiguous
+// range of logical tile ids so that the tiles sharing an L2 also share
+// operand rows, then walk tiles m-fastest inside groups of 8 m-tiles.
+__device__ __forceinline__ void tile_coords(int bid, int nblk, int tiles_m, int tiles_n, int* tm,
+                                            int* tn) {
+    const int q = nblk / 8, r = nblk % 8;
+    const int xcd = bid % 8, local = bid / 8;
+    const int lid = xcd * q + (xcd < r ? xcd : r) + local;
+    constexpr int GM = 8;
+    const int group_size = GM * tiles_n;
+    const int group = lid / group_size;
+    const int first_m = group * GM;
+    const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int in_group = lid - group * group_size;
+    *tm = first_m + in_group % gsz;
+    *tn = in_group / gsz;
+}
+
+// Epilogue of one wavefront's sub-tile, in 32-row bands.  The MFMA result
+// layout gives a lane one column and sixteen scattered rows; the band is
+// turned through LDS so that a lane ends up with four consecutive columns of
+// one row and the wavefront writes contiguous row segments.
+template <class Cfg, int MODE>
+__device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg::TM][Cfg::TN],
+                                              const ColParams (&cp)[Cfg::TN], const float* s_as,
+                                              uint32_t* stage, int m0, int n0, int n_limit, int wm,
+                                              int wn, int lane, float S, float Z) {
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, STRIDE = Cfg::STAGE_STRIDE;
+    constexpr int QUADS_PER_ROW = TN * 8;            // four-column groups per staged row
+    constexpr int EPI_ROWS = Cfg::EPI_ROWS;          // rows staged at a time (32 or 16)
+    constexpr int PARTS = 32 / EPI_ROWS, RPP = 16 / PARTS;
+    constexpr int PASSES = EPI_ROWS * QUADS_PER_ROW / 64;
+    const int esize = MODE == OUT_F16 ? 2 : (MODE == OUT_REQUANT_I8 ? 1 : 4);
+    const bool vec_ok = (g.ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int part = 0; part < PARTS; ++part) {
+            const int band = wm * (TM * 32) + i * 32 + part * EPI_ROWS;
+#pragma unroll
+            for (int rr = 0; rr < RPP; ++rr) {
+                const int r = part * RPP + rr;
+                const int row = 8 * (rr >> 2) + 4 * (lane >> 5) + (rr & 3);  // row within the staged part
+                const float as = s_as[band + row];
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    stage[row * STRIDE + j * 32 + (lane & 31)] =
+                        epilogue_value<MODE>(g, acc[i][j][r], as, cp[j], S, Z);
+                __builtin_amdgcn_sched_barrier(0);  // keep the unrolled rows from piling up live registers
+            }
+            __syncthreads();
+#pragma unroll 4
+            for (int p = 0; p < PASSES; ++p) {
+                const int q = p * 64 + lane;
+                const int row = q / QUADS_PER_ROW, cq = (q % QUADS_PER_ROW) * 4;
+                const uint4 v = *reinterpret_cast<const uint4*>(stage + row * STRIDE + cq);
+                const int m = m0 + band + row, n = n0 + wn * (TN * 32) + cq;
+                if (m < g.M && n < n_limit) {
+                    const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
+                    if (vec_ok && n + 4 <= n_limit) {
+                        store_vec4<MODE>(g, idx, v);
+                    } else {
+                        store_scalar<MODE>(g, idx, v.x);
+                        if (n + 1 < n_limit) store_scalar<MODE>(g, idx + 1, v.y);
+                        if (n + 2 < n_limit) store_scalar<MODE>(g, idx + 2, v.z);
+                        if (n + 3 < n_limit) store_scalar<MODE>(g, idx + 3, v.w);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// LDS stage layout: BM rows of A then BN rows of B, each row BK bytes; the
+// 16-byte chunk kc of row r sits at physical chunk kc ^ ((r / R) % C).  With
+// 64 LDS banks a ds_read_b128 serves 16 lanes per pass; under this swizzle the
+// 16 fragment rows of a pass fall on 16 different bank groups.  A wavefront's
+// direct global->LDS load writes 1 KiB of consecutive slots, so the swizzle is
+// applied on the global side: a lane fetches the chunk that belongs in its slot.
+// Balanced split of `total` k-iterations over `workers`: the first `rem` workers
+// take one iteration more.
+struct IterSplit {
+    int per, rem;
+    __host__ __device__ IterSplit(long total, int workers)
+        : per(int(total / workers)), rem(int(total % workers)) {}
+    __host__ __device__ long begin(int w) const { return long(w) * per + (w < rem ? w : rem); }
+    __host__ __device__ int owner(long it) const {
+        const long cut = long(rem) * (per + 1);
+        return it < cut ? int(it / (per + 1)) : rem + int((it - cut) / per);
+    }
+};
+
+// SK = false: one block per tile (blockIdx.x -> tile, blockIdx.y -> group).
+// SK = true ("stream-K"): gridDim.x workers split the tiles' k-iterations evenly;
+// a worker's range may start and end in the middle of a tile.  A tile touched by
+// several workers is finished without anybody waiting: every contributor stores
+// its int32 partial accumulators into its own slab, then bumps the tile's
+// arrival counter; whoever arrives last adds the other slabs to its registers
+// and runs the epilogue.  Integer partial sums add exactly, so the result does
+// not depend on who arrives when.
+template <class Cfg, int MODE, bool CONV, bool SK>
+__global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel(GemmArgs g) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
+    constexpr int C = Cfg::C, R = Cfg::R, PA = Cfg::PA, PB = Cfg::PB, STAGES = Cfg::STAGES;
+    constexpr int THREADS = Cfg::THREADS, KSTEPS = Cfg::KSTEPS;
+    extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
+    __shared__ int s_flag;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // wavefront index as a scalar: LDS stage addresses (the M0 operand of the direct
+    // loads) then need no per-load readfirstlane
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    const int n_base = int(blockIdx.y) * g.N;  // first column of this group (0 for a plain GEMM)
+    const int n_limit = n_base + g.N;
+    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+    const int nk = (g.K + BK - 1) / BK;
+
+    // global -> LDS addressing: in pass `it` this lane fills the slot of row
+    // it*ROWS_PER_PASS + tid/C, physical chunk tid%C.  ROWS_PER_PASS is a multiple
+    // of 16, so the swizzle term - and the logical chunk fetched - is the same in
+    // every pass.
+    const int row_in_pass = tid / C;
+    const int kc = (tid % C) ^ ((row_in_pass / R) % C);
+    // fragment addressing: lane holds row (lane & 31), 16 bytes of k at chunk
+    // 2*kk + (lane >> 5) of the current 32-wide k step
+    const int frag_row = lane & 31;
+    const int frag_half = lane >> 5;
+    const int a_row_base = (wm * (TM * 32) + frag_row) * BK;
+    const int b_row_base = BM * BK + (wn * (TN * 32) + frag_row) * BK;
+    const int sw = (frag_row / R) % C;
+
+    v16i acc[TM][TN];
+
+    // k-iterations [kb, ke) of tile (tm, tn) into acc (zeroed first)
+    auto run_segment = [&](int tm, int tn, int kb, int ke) {
+        const int m0 = tm * BM, n0 = n_base + tn * BN;
+        unsigned a_off[PA], b_off[PB];
+        int a_hw[PA];  // CONV: top-left input coordinate of the pixel, (ih0 << 16) | (iw0 & 0xffff)
+        const int a_rows = g.M - m0, b_rows = n_limit - n0;  // valid rows in this tile (>= 1)
+#pragma unroll
+        for (int it = 0; it < PA; ++it) {
+            int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
+            r = r < a_rows ? r : a_rows - 1;  // clamp: reads stay in bounds, rows are masked at the store
+            if (CONV) {
+                const int m = m0 + r;
+                const int pix = g.cOH * g.cOW;
+                const int b = m / pix, rem = m - b * pix;
+                const int oh = rem / g.cOW, ow = rem - oh * g.cOW;
+                const int ih0 = oh * g.csh - g.cph, iw0 = ow * g.csw - g.cpw;
+                a_hw[it] = (ih0 << 16) | (iw0 & 0xffff);
+                // may wrap for ih0 / iw0 < 0; it is only used after the bounds check,
+                // together with a tap offset that brings it back in range
+                a_off[it] = unsigned((b * g.cH + ih0) * g.cW + iw0) * unsigned(g.cCin) +
+                            unsigned(int(blockIdx.y) * g.cCg);
+            } else {
+                a_hw[it] = 0;
+                a_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < PB; ++it) {
+            int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
+            r = r < b_rows ? r : b_rows - 1;
+            b_off[it] = unsigned(r) * unsigned(g.K) + unsigned(kc * 16);
+        }
+        const int8_t* a_tile = CONV ? g.cx : g.a + size_t(m0) * g.K;
+        const int8_t* b_tile = g.w + size_t(n0) * g.K;
+        const int k_end = ke * BK < g.K ? ke * BK : g.K;  // nothing is fetched past the segment
+
+        // `full` (compile time): the whole stage lies inside K, so no lane needs the
+        // zero source and the address is a uniform base plus a per-lane offset
+        auto load_stage = [&](int k0, int8_t* stage, auto full) {
+            const int k = k0 + kc * 16;
+            const bool in_k = k < k_end;  // K-tail chunks and look-ahead stages: zeros
+            int8_t* sa = stage + wave * 1024;
+            int8_t* sb = stage + BM * BK + wave * 1024;
+            if (!CONV && decltype(full)::value) {
+                const int8_t* ab = a_tile + k0;
+                const int8_t* bb = b_tile + k0;
+#pragma unroll
+                for (int it = 0; it < PA; ++it)
+                    __builtin_amdgcn_global_load_lds(LQ_GPTR(ab + a_off[it]), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
+#pragma unroll
+                for (int it = 0; it < PB; ++it)
+                    __builtin_amdgcn_global_load_lds(LQ_GPTR(bb + b_off[it]), LQ_LPTR(sb + it * (THREADS * 16)), 16, 0, 0);
+                return;
+            }
+            if (CONV) {
+                // this lane's 16 bytes lie inside one filter tap (Cg % 16 == 0)
+                const int tap = k / g.cCg, ci0 = k - tap * g.cCg;
+                const int kh = tap / g.cKW, kw = tap - kh * g.cKW;
+                const int dh = kh * g.cdh, dw = kw * g.cdw;
+                const unsigned delta = unsigned(dh * g.cW + dw) * unsigned(g.cCin) + unsigned(ci0);
+#pragma unroll
+                for (int it = 0; it < PA; ++it) {
+                    const int ih = (a_hw[it] >> 16) + dh;
+                    const int iw = int(short(a_hw[it] & 0xffff)) + dw;
+                    const bool ok = in_k && unsigned(ih) < unsigned(g.cH) && unsigned(iw) < unsigned(g.cW);
+                    const int8_t* src = ok ? a_tile + (a_off[it] + delta) : g.pad_src;
+                    __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int it = 0; it < PA; ++it) {
+                    const int8_t* src = in_k ? a_tile + k0 + a_off[it] : g.zeros;
+                    __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < PB; ++it) {
+                const int8_t* src = in_k ? b_tile + k0 + b_off[it] : g.zeros;
+                __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sb + it * (THREADS * 16)), 16, 0, 0);
+            }
+        };
+
+        auto read_frags = [&](const int8_t* stage, int kk, v4i (&af)[TM], v4i (&bf)[TN]) {
+            const int pc = ((kk * 2 + frag_half) ^ sw) * 16;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                af[i] = *reinterpret_cast<const v4i*>(stage + a_row_base + i * 32 * BK + pc);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                bf[j] = *reinterpret_cast<const v4i*>(stage + b_row_base + j * 32 * BK + pc);
+        };
+
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+        // All STAGES buffers are kept in flight.  The fragments of k step kk+1
+        // are fetched from LDS while the MFMAs of step kk run; the hand-over to
+        // the next stage (wait for its data, barrier, fetch its first fragments,
+        // refill the buffer just drained) sits inside the last k step of the
+        // current stage, so its latency is covered by that step's MFMAs.  Stages
+        // past the end are loaded from the block of zeros, which keeps the number
+        // of outstanding loads - and so the vmcnt to wait for - constant.
+#pragma unroll
+        for (int s = 0; s < STAGES; ++s)
+            load_stage((kb + s) * BK, smem + s * Cfg::STAGE_BYTES, std::false_type{});
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 1) * (PA + PB)));
+        __syncthreads();
+
+        v4i af[2][TM], bf[2][TN];
+        if (Cfg::PIPE) read_frags(smem, 0, af[0], bf[0]);
+
+        auto k_steps = [&](int t, bool last_stage, auto full) {  // t counts from 0 within the segment
+            const int slot = t % STAGES;
+            int8_t* cur = smem + slot * Cfg::STAGE_BYTES;
+            const int8_t* nxt = smem + (slot + 1 == STAGES ? 0 : slot + 1) * Cfg::STAGE_BYTES;
+            if (!Cfg::PIPE) {
+                // fragments are read right before their MFMAs; the CU's other
+                // wavefronts fill the wait
+#pragma unroll
+                for (int kk = 0; kk < KSTEPS; ++kk) {
+                    read_frags(cur, kk, af[0], bf[0]);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[0][i], bf[0][j], acc[i][j], 0, 0, 0);
+                }
+                if (!last_stage) {
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * (PA + PB)));
+                    __syncthreads();  // stage t+1 is complete in LDS; nobody reads stage t any more
+                    load_stage((kb + t + STAGES) * BK, cur, full);
+                }
+                return;
+            }
+#pragma unroll
+            for (int kk = 0; kk < KSTEPS; ++kk) {
+                if (kk + 1 < KSTEPS) {
+                    read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+                } else if (!last_stage) {
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * (PA + PB)));
+                    __syncthreads();  // stage t+1 is complete in LDS; nobody reads stage t any more
+                    read_frags(nxt, 0, af[0], bf[0]);
+                    load_stage((kb + t + STAGES) * BK, cur, full);
+                }
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[kk & 1][i], bf[kk & 1][j],
+                                                                          acc[i][j], 0, 0, 0);
+                // issue order inside the step: one MFMA, then all LDS reads of the next
+                // step's fragments, then the other MFMAs.  The compiler waits for every
+                // outstanding LDS read before the first MFMA of a step, so the reads go
+                // out as early as possible; the MFMA goes first so that this wait is not
+                // held up by a read issued just before it.
+                if (kk + 1 < KSTEPS) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
+                } else if (!last_stage) {
+                    // hand-over step: the refill loads go out one per MFMA after the reads
+                    constexpr int NL = PA + PB < TM * TN - 1 ? PA + PB : TM * TN - 1;
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+                    for (int x = 0; x < NL; ++x) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x020, PA + PB - NL, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1 - NL, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        const int n_it = ke - kb;
+        // iterations whose refill stage (t + STAGES) lies wholly inside K come first
+        int n_full = (k_end / BK) - kb - STAGES;
+        n_full = n_full < 0 ? 0 : (n_full > n_it - 1 ? n_it - 1 : n_full);
+        int t = 0;
+        for (; t < n_full; ++t) k_steps(t, false, std::true_type{});
+        for (; t + 1 < n_it; ++t) k_steps(t, false, std::false_type{});
+        k_steps(n_it - 1, true, std::false_type{});
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the zero-filled look-ahead stages
+        __syncthreads();                            // all fragment reads done before LDS is reused
+    };
+
+    // Row scales are staged in LDS and column parameters are loaded before the
+    // first store, so no global load sits between the stores.
+    auto run_epilogue = [&](int tm, int tn) {
+        const int m0 = tm * BM, n0 = n_base + tn * BN;
+        float* s_as = reinterpret_cast<float*>(smem);
+        uint32_t* stage = reinterpret_cast<uint32_t*>(smem + 4 * BM) + wave * Cfg::STAGE_WORDS;
+        for (int rr = tid; rr < BM; rr += THREADS) {
+            const int m = m0 + rr;
+            float v = 1.0f;
+            if (g.a_scale) v = g.a_scale[(g.a_scale_per_row && m < g.M) ? m : 0];
+            s_as[rr] = v;
+        }
+        float S = 1.0f, Z = 0.0f;
+        if (MODE == OUT_REQUANT_I8 || MODE == OUT_FAKEQUANT_F32) {
+            S = g.out_scale[0];
+            Z = g.out_zp[0];
+        }
+        ColParams cp[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+            cp[j] = load_col(g, n < n_limit ? n : n_limit - 1);
+        }
+        __syncthreads();
+        tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z);
+    };
+
+    if (!SK) {
+        int tm, tn;
+        tile_coords(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
+        run_segment(tm, tn, 0, nk);
+        run_epilogue(tm, tn);
+        return;
+    }
+
+    // ---- stream-K
+    constexpr int kAccWords = TM * TN * 16;  // accumulator registers per lane
+    const int workers = gridDim.x;
+    const long total = long(tiles_m) * tiles_n * nk;
+    const IterSplit split(total, workers);
+    // give every XCD a contiguous range of workers (blocks are dealt round-robin)
+    const int wq = workers / 8, wr = workers % 8;
+    const int xcd = blockIdx.x % 8;
+    const int me = xcd * wq + (xcd < wr ? xcd : wr) + blockIdx.x / 8;
+    long it = split.begin(me);
+    const long it_end = split.begin(me + 1);
+    int* counters = g.sk_counters + size_t(blockIdx.y) * tiles_m * tiles_n;
+    int32_t* slabs = g.sk_slabs + size_t(blockIdx.y) * workers * 2 * size_t(kAccWords) * THREADS;
+    while (it < it_end) {
+        const int tile = int(it / nk);
+        const int kb = int(it - long(tile) * nk);
+        const int ke = (it_end - it) < (nk - kb) ? kb + int(it_end - it) : nk;
+        // same m-fastest walk in groups of 8 m-tiles as tile_coords
+        int tm, tn;
+        {
+            constexpr int GM = 8;
+            const int group_size = GM * tiles_n;
+            const int group = tile / group_size;
+            const int first_m = group * GM;
+            const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+            const int in_group = tile - group * group_size;
+            tm = first_m + in_group % gsz;
+            tn = in_group / gsz;
+        }
+        run_segment(tm, tn, kb, ke);
+        bool finish = true;
+        if (!(kb == 0 && ke == nk)) {
+            const int w_first = split.owner(long(tile) * nk);
+            const int w_last = split.owner(long(tile) * nk + nk - 1);
+            // slab 0 holds a worker's leading partial tile, slab 1 its trailing one
+            auto slab_of = [&](int w) {
+                const int first_tile = int(split.begin(w) / nk);
+                return slabs + (size_t(w) * 2 + (tile == first_tile ? 0 : 1)) * kAccWords * THREADS;
+            };
+            int32_t* mine = slab_of(me);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        mine[((i * TN + j) * 16 + r) * THREADS + tid] = acc[i][j][r];
+            __threadfence();  // partials visible device-wide before the arrival is counted
+            __syncthreads();
+            if (tid == 0) s_flag = atomicAdd(&counters[tile], 1);
+            __syncthreads();
+            finish = s_flag == (w_last - w_first);  // the other contributors have all arrived
+            if (finish) {
+                __threadfence();
+                for (int w = w_first; w <= w_last; ++w) {
+                    if (w == me) continue;
+                    const int32_t* other = slab_of(w);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r)
+                                acc[i][j][r] += __builtin_nontemporal_load(
+                                    &other[((i * TN + j) * 16 + r) * THREADS + tid]);
+                }
+                if (tid == 0) counters[tile] = 0;  // ready for the next launch
+            }
+            __syncthreads();
+        }
+        if (finish) run_epilogue(tm, tn);
+        it += ke - kb;
+    }
+}
+
+// Tile shapes.  "big" keeps LDS traffic per MFMA lowest (one block per CU);
+// "wide" and "mid" let two or more blocks share a CU so one block's barrier
+// and epilogue overlap another's MFMAs, and waste less on ragged M / N.
+using CfgBig = TileCfg<256, 256, 128, 2, 2, 2, 1>;
+using CfgBig64 = TileCfg<256, 256, 64, 2, 2, 4, 1>;
+using CfgWide = TileCfg<256, 128, 64, 2, 2, 3, 2>;
+using CfgTall = TileCfg<128, 256, 64, 2, 2, 3, 2>;
+using CfgMid = TileCfg<128, 128, 64, 2, 2, 4, 2>;
+using CfgN64 = TileCfg<256, 64, 64, 4, 1, 3, 2>;  // 64 output columns (early ResNet stages)
+using CfgTall3 = TileCfg<128, 256, 64, 2, 2, 2, 3>;  // three blocks per CU
+
+}  // namespace
+
+// Stream-K scratch per device: arrival counters (zero between launches: the
+// finisher of a tile resets its counter) and two accumulator slabs per worker.
+struct SkScratch {
+    int* counters = nullptr;
+    size_t counter_count = 0;
+    int32_t* slabs = nullptr;
+    size_t slab_bytes = 0;
+};
+int sk_scratch(size_t counters, size_t slab_bytes, SkScratch** out);
+
+namespace {
+
+template <class Cfg, int MODE, bool CONV>
+int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
+    const void* fn_dp = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV, false>);
+    const void* fn_sk = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV, true>);
+    static bool attr_set = false;
+    if (!attr_set) {
+        LQ_HIP(hipFuncSetAttribute(fn_dp, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
+        LQ_HIP(hipFuncSetAttribute(fn_sk, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
+        attr_set = true;
+    }
+    const int tiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
+    const int nk = (g.K + Cfg::BK - 1) / Cfg::BK;
+    // blocks that fit on the chip at once: 256 CUs x blocks per CU (LDS-bound)
+    const int per_cu = (160 * 1024) / Cfg::SMEM < Cfg::MINWAVES ? (160 * 1024) / Cfg::SMEM : Cfg::MINWAVES;
+    const int slots = 256 * (per_cu < 1 ? 1 : per_cu);
+    // schedule: 0 = choose, 1 = one block per tile, 2 = stream-K.
+    // Stream-K pays when the tiles fill the last round of blocks badly and there
+    // are few rounds; every worker must get at least a few k-iterations.
+    // Stream-K is opt-in only.  Measured at M=2048, N=11008, K=4096 it loses to one
+    // block per tile (128x256 tiles: 116 us vs 371 us; 175 us even with the
+    // device-scope fences taken out): the 128 KiB partial slabs per worker and the
+    // L2 write-back / invalidate of the fences cost more than the idle tail they remove.
+    const bool sk = schedule == 2;
+    GemmArgs copy = g;
+    void* kargs[] = {&copy};
+    if (!sk) {
+        LQ_HIP(hipLaunchKernel(fn_dp, dim3(tiles, groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
+        return LQ_OK;
+    }
+    long workers = slots / groups;
+    if (workers < 1) workers = 1;
+    if (workers > long(tiles) * nk) workers = long(tiles) * nk;
+    SkScratch* s = nullptr;
+    const size_t slab_words = size_t(Cfg::TM) * Cfg::TN * 16 * Cfg::THREADS;
+    int rc = sk_scratch(size_t(tiles) * groups, size_t(groups) * workers * 2 * slab_words * 4, &s);
+    if (rc) return rc;
+    copy.sk_counters = s->counters;
+    copy.sk_slabs = s->slabs;
+    LQ_HIP(hipLaunchKernel(fn_sk, dim3(unsigned(workers), groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
+    return LQ_OK;
+}
+
+template <class Cfg, bool CONV>
+int launch_tile(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
+    LQ_REQUIRE(size_t(Cfg::BM > Cfg::BN ? Cfg::BM : Cfg::BN) * g.K < 0xffffffffull, LQ_ERR_SHAPE,
+               "tile kernel: K too large");
+    switch (g.out_mode) {
+    case OUT_ACC_I32: return launch_tile_mode<Cfg, OUT_ACC_I32, CONV>(g, groups, schedule, st);
+    case OUT_F32: return launch_tile_mode<Cfg, OUT_F32, CONV>(g, groups, schedule, st);
+    case OUT_F16: return launch_tile_mode<Cfg, OUT_F16, CONV>(g, groups, schedule, st);
+    case OUT_REQUANT_I8: return launch_tile_mode<Cfg, OUT_REQUANT_I8, CONV>(g, groups, schedule, st);
+    default: return launch_tile_mode<Cfg, OUT_FAKEQUANT_F32, CONV>(g, groups, schedule, st);
+    }
+}
+
+}  // namespace
+}  // namespace lq
+
+// One per translation unit: the launcher of one tile shape.
+#define LQ_DEFINE_TILE_LAUNCHER(NAME, CFG)                                                      \
+    namespace lq {                                                                              \
+    int NAME(const GemmArgs& g, bool conv, int groups, int schedule, hipStream_t st) {          \
+        return conv ? launch_tile<CFG, true>(g, groups, schedule, st)                           \
+                    : launch_tile<CFG, false>(g, groups, schedule, st);                         \
+    }                                                                                           \
+    }

@@ -64,8 +64,9 @@ __device__ __forceinline__ float clamp_code(float r, float z, float lo, float hi
 __device__ __forceinline__ float4 rint_div4(float4 v, float s, float r) {
     float4 t = {v.x * r, v.y * r, v.z * r, v.w * r};
     float4 n = {__builtin_rintf(t.x), __builtin_rintf(t.y), __builtin_rintf(t.z), __builtin_rintf(t.w)};
-    const bool ok = rint_quotient_safe(t.x, n.x) & rint_quotient_safe(t.y, n.y) &
-                    rint_quotient_safe(t.z, n.z) & rint_quotient_safe(t.w, n.w);
+    // branch-free conjunction: the four tests are evaluated unconditionally
+    const bool ok = (int(rint_quotient_safe(t.x, n.x)) & int(rint_quotient_safe(t.y, n.y)) &
+                     int(rint_quotient_safe(t.z, n.z)) & int(rint_quotient_safe(t.w, n.w))) != 0;
     if (__builtin_expect(!ok, 0)) {
         n.x = __builtin_rintf(v.x / s);
         n.y = __builtin_rintf(v.y / s);
