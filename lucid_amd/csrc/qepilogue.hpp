@@ -10,18 +10,64 @@ struct ColParams {
     int32_t corr;  // a_zp * wsum[n]
 };
 
+// A missing bias is the additive identity -0.0f (y + -0.0f == y bit for bit,
+// signed zeros and NaNs included), so the add needs no per-element test.
 __device__ __forceinline__ ColParams load_col(const GemmArgs& g, int n) {
     ColParams c;
     c.ws = g.w_scale ? g.w_scale[n] : 1.0f;
     const int zp = g.a_zp_dev ? int(g.a_zp_dev[0]) + g.a_zp : g.a_zp;
     c.corr = (g.wsum && zp != 0) ? zp * g.wsum[n] : 0;
     if (g.bias == nullptr)
-        c.bias = 0.0f;
+        c.bias = -0.0f;
     else if (g.bias_dtype == LQ_F16)
         c.bias = float(static_cast<const _Float16*>(g.bias)[n]);
     else
         c.bias = static_cast<const float*>(g.bias)[n];
     return c;
+}
+
+// The same for T columns at once, with every load issued before the first
+// value is used (one memory round trip instead of one per load).
+template <int T>
+__device__ __forceinline__ void load_cols(const GemmArgs& g, const int (&n)[T], ColParams (&c)[T]) {
+    const int zp = g.a_zp_dev ? int(g.a_zp_dev[0]) + g.a_zp : g.a_zp;
+    int32_t wsum[T];
+    uint32_t braw[T];
+    if (g.w_scale) {
+#pragma unroll
+        for (int j = 0; j < T; ++j) c[j].ws = g.w_scale[n[j]];
+    } else {
+#pragma unroll
+        for (int j = 0; j < T; ++j) c[j].ws = 1.0f;
+    }
+    if (g.wsum) {
+#pragma unroll
+        for (int j = 0; j < T; ++j) wsum[j] = g.wsum[n[j]];
+    } else {
+#pragma unroll
+        for (int j = 0; j < T; ++j) wsum[j] = 0;
+    }
+    const bool f16 = g.bias != nullptr && g.bias_dtype == LQ_F16;
+    if (f16) {
+#pragma unroll
+        for (int j = 0; j < T; ++j) braw[j] = static_cast<const uint16_t*>(g.bias)[n[j]];
+    } else if (g.bias != nullptr) {
+#pragma unroll
+        for (int j = 0; j < T; ++j) braw[j] = static_cast<const uint32_t*>(g.bias)[n[j]];
+    } else {
+#pragma unroll
+        for (int j = 0; j < T; ++j) braw[j] = 0x80000000u;  // -0.0f
+    }
+#pragma unroll
+    for (int j = 0; j < T; ++j) {
+        c[j].corr = zp * wsum[j];
+        if (f16) {
+            const uint16_t h = uint16_t(braw[j]);
+            c[j].bias = float(__builtin_bit_cast(_Float16, h));
+        } else {
+            c[j].bias = __uint_as_float(braw[j]);
+        }
+    }
 }
 
 __device__ __forceinline__ float q_core(float x, float s, float z, float lo, float hi) {
@@ -44,8 +90,11 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
     float f = float(acc - c.corr);
     float sc = as * c.ws;
     float y = f * sc;
-    if (g.bias) y = y + c.bias;
-    if (g.relu) y = (y < 0.0f) ? 0.0f : y;
+    y = y + c.bias;
+    // ReLU as a floor of 0, no ReLU as a floor of -inf: one compare and select either
+    // way (a NaN fails the compare and passes through, as in the CPU formulation)
+    const float floor = g.relu ? 0.0f : -__builtin_inff();
+    y = (y < floor) ? floor : y;
     if (MODE == OUT_F32 || MODE == OUT_F16) return __float_as_uint(y);
     float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
     if (MODE == OUT_REQUANT_I8) {

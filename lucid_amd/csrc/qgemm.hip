@@ -26,11 +26,16 @@ using namespace lq;
 namespace lq {
 SkScratch g_sk[16];
 
-int sk_scratch(size_t counters, size_t slab_bytes, SkScratch** out) {
+// Returns in *out the device's scratch grown to the requested sizes, or null
+// when it would have to grow and may not (the stream is being captured into a
+// graph: growing synchronizes the device).
+int sk_scratch(size_t counters, size_t slab_bytes, bool may_grow, SkScratch** out) {
     int dev = 0;
     LQ_HIP(hipGetDevice(&dev));
     LQ_REQUIRE(dev >= 0 && dev < 16, LQ_ERR_DEVICE, "device index %d out of range", dev);
     SkScratch& s = g_sk[dev];
+    *out = nullptr;
+    if ((s.counter_count < counters || s.slab_bytes < slab_bytes) && !may_grow) return LQ_OK;
     if (s.counter_count < counters) {
         LQ_HIP(hipDeviceSynchronize());
         if (s.counters) LQ_HIP(hipFree(s.counters));

@@ -36,6 +36,7 @@ struct GemmArgs {
     // stream-K scratch (set by the launcher)
     int* sk_counters;
     int32_t* sk_slabs;
+    int sk_tiles;  // the last sk_tiles tile ids are shared between workers
 };
 
 

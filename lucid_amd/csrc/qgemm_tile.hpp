@@ -13,6 +13,7 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 #define LQ_GPTR(p) ((__attribute__((address_space(1))) void*)(p))
 #define LQ_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -41,7 +42,9 @@ struct TileCfg {
     // latency) and the epilogue stages 16 rows at a time.
     static constexpr bool PIPE = MINWAVES_ < 3;
     static constexpr int EPI_ROWS = MINWAVES_ < 3 ? 32 : 16;
-    static constexpr int STAGE_STRIDE = TN * 32 + 4;   // words per staged output row
+    // words per staged output row: a multiple of 4 (16-byte reads) that puts row
+    // r + 4 - the upper half-wavefront's row - 32 banks away from row r
+    static constexpr int STAGE_STRIDE = TN * 32 + 8;
     static constexpr int STAGE_WORDS = EPI_ROWS * STAGE_STRIDE;
     static constexpr int EPI_BYTES = 4 * BM + THREADS / 64 * STAGE_WORDS * 4;
     static constexpr int SMEM = STAGES * STAGE_BYTES > EPI_BYTES ? STAGES * STAGE_BYTES : EPI_BYTES;
@@ -72,58 +75,91 @@ __device__ __forceinline__ void tile_coords(int bid, int nblk, int tiles_m, int 
     *tn = in_group / gsz;
 }
 
-// Epilogue of one wavefront's sub-tile, in 32-row bands.  The MFMA result
-// layout gives a lane one column and sixteen scattered rows; the band is
-// turned through LDS so that a lane ends up with four consecutive columns of
-// one row and the wavefront writes contiguous row segments.
+// Wavefront-private LDS traffic needs no workgroup barrier: one wavefront's LDS
+// instructions execute in order.  This only keeps the compiler from moving
+// accesses across the point.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Epilogue of one wavefront's sub-tile, in 32-row bands (or half bands).  The
+// MFMA result layout gives a lane one column and sixteen scattered rows; the
+// band is turned through a wavefront-private LDS area so that a lane ends up
+// with four consecutive columns of one row and the wavefront writes contiguous
+// row segments.  `interior` (uniform): the whole tile lies inside the output
+// and rows are vector-aligned, so the stores need no per-lane tests.
 template <class Cfg, int MODE>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg::TM][Cfg::TN],
                                               const ColParams (&cp)[Cfg::TN], const float* s_as,
                                               uint32_t* stage, int m0, int n0, int n_limit, int wm,
-                                              int wn, int lane, float S, float Z) {
+                                              int wn, int lane, float S, float Z, bool interior) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, STRIDE = Cfg::STAGE_STRIDE;
     constexpr int QUADS_PER_ROW = TN * 8;            // four-column groups per staged row
     constexpr int EPI_ROWS = Cfg::EPI_ROWS;          // rows staged at a time (32 or 16)
     constexpr int PARTS = 32 / EPI_ROWS, RPP = 16 / PARTS;
     constexpr int PASSES = EPI_ROWS * QUADS_PER_ROW / 64;
+    constexpr int ROWS_PER_PASS = 64 / QUADS_PER_ROW;
+    static_assert(64 % QUADS_PER_ROW == 0 && RPP % 4 == 0, "");
     const int esize = MODE == OUT_F16 ? 2 : (MODE == OUT_REQUANT_I8 ? 1 : 4);
     const bool vec_ok = (g.ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0);
+    const int row0 = lane / QUADS_PER_ROW, cq = (lane % QUADS_PER_ROW) * 4;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int part = 0; part < PARTS; ++part) {
             const int band = wm * (TM * 32) + i * 32 + part * EPI_ROWS;
+            // this lane's rows of the part: groups of four consecutive rows
+            float as[RPP];
+#pragma unroll
+            for (int q = 0; q < RPP / 4; ++q) {
+                const float4 v = *reinterpret_cast<const float4*>(s_as + band + 8 * q + 4 * (lane >> 5));
+                as[4 * q] = v.x, as[4 * q + 1] = v.y, as[4 * q + 2] = v.z, as[4 * q + 3] = v.w;
+            }
 #pragma unroll
             for (int rr = 0; rr < RPP; ++rr) {
                 const int r = part * RPP + rr;
                 const int row = 8 * (rr >> 2) + 4 * (lane >> 5) + (rr & 3);  // row within the staged part
-                const float as = s_as[band + row];
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     stage[row * STRIDE + j * 32 + (lane & 31)] =
-                        epilogue_value<MODE>(g, acc[i][j][r], as, cp[j], S, Z);
-                __builtin_amdgcn_sched_barrier(0);  // keep the unrolled rows from piling up live registers
+                        epilogue_value<MODE>(g, acc[i][j][r], as[rr], cp[j], S, Z);
             }
-            __syncthreads();
+            wave_lds_sync();
+            const int m_first = m0 + band + row0, n = n0 + wn * (TN * 32) + cq;
+            const uint32_t* src = stage + row0 * STRIDE + cq;
+            if (interior) {
+                uint4 v[PASSES];
+#pragma unroll
+                for (int p = 0; p < PASSES; ++p)
+                    v[p] = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
+                size_t idx = size_t(m_first) * size_t(g.ldo) + size_t(n);
+                const size_t step = size_t(ROWS_PER_PASS) * size_t(g.ldo);
+#pragma unroll
+                for (int p = 0; p < PASSES; ++p) {
+                    store_vec4<MODE>(g, idx, v[p]);
+                    idx += step;
+                }
+            } else {
 #pragma unroll 4
-            for (int p = 0; p < PASSES; ++p) {
-                const int q = p * 64 + lane;
-                const int row = q / QUADS_PER_ROW, cq = (q % QUADS_PER_ROW) * 4;
-                const uint4 v = *reinterpret_cast<const uint4*>(stage + row * STRIDE + cq);
-                const int m = m0 + band + row, n = n0 + wn * (TN * 32) + cq;
-                if (m < g.M && n < n_limit) {
-                    const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
-                    if (vec_ok && n + 4 <= n_limit) {
-                        store_vec4<MODE>(g, idx, v);
-                    } else {
-                        store_scalar<MODE>(g, idx, v.x);
-                        if (n + 1 < n_limit) store_scalar<MODE>(g, idx + 1, v.y);
-                        if (n + 2 < n_limit) store_scalar<MODE>(g, idx + 2, v.z);
-                        if (n + 3 < n_limit) store_scalar<MODE>(g, idx + 3, v.w);
+                for (int p = 0; p < PASSES; ++p) {
+                    const uint4 v = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
+                    const int m = m_first + p * ROWS_PER_PASS;
+                    if (m < g.M && n < n_limit) {
+                        const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
+                        if (vec_ok && n + 4 <= n_limit) {
+                            store_vec4<MODE>(g, idx, v);
+                        } else {
+                            store_scalar<MODE>(g, idx, v.x);
+                            if (n + 1 < n_limit) store_scalar<MODE>(g, idx + 1, v.y);
+                            if (n + 2 < n_limit) store_scalar<MODE>(g, idx + 2, v.z);
+                            if (n + 3 < n_limit) store_scalar<MODE>(g, idx + 3, v.w);
+                        }
                     }
                 }
             }
-            __syncthreads();
+            wave_lds_sync();
         }
     }
 }
@@ -188,8 +224,30 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
 
     v16i acc[TM][TN];
 
-    // k-iterations [kb, ke) of tile (tm, tn) into acc (zeroed first)
+    // Epilogue operands of the current tile.  They are fetched while the last
+    // k-iteration of the tile runs, so their latency is paid under its MFMAs.
+    static_assert(BM <= THREADS, "one row scale per thread");
+    ColParams cp[TN];
+    float as_mine = 1.0f;  // a_scale of row m0 + tid
+    bool fetched = false;
+    auto fetch_params = [&](int tm, int tn) {
+        const int m0 = tm * BM, n0 = n_base + tn * BN;
+        int n[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            n[j] = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+            n[j] = n[j] < n_limit ? n[j] : n_limit - 1;
+        }
+        load_cols(g, n, cp);
+        const int m = m0 + tid;
+        as_mine = g.a_scale ? g.a_scale[(g.a_scale_per_row && m < g.M) ? m : 0] : 1.0f;
+        fetched = true;
+    };
+
+    // k-iterations [kb, ke) of tile (tm, tn) into acc (zeroed first); ke == nk
+    // also fetches the tile's epilogue operands
     auto run_segment = [&](int tm, int tn, int kb, int ke) {
+        fetched = false;
         const int m0 = tm * BM, n0 = n_base + tn * BN;
         unsigned a_off[PA], b_off[PB];
         int a_hw[PA];  // CONV: top-left input coordinate of the pixel, (ih0 << 16) | (iw0 & 0xffff)
@@ -374,6 +432,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         int t = 0;
         for (; t < n_full; ++t) k_steps(t, false, std::true_type{});
         for (; t + 1 < n_it; ++t) k_steps(t, false, std::false_type{});
+        if (ke == nk) fetch_params(tm, tn);
         k_steps(n_it - 1, true, std::false_type{});
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the zero-filled look-ahead stages
         __syncthreads();                            // all fragment reads done before LDS is reused
@@ -385,25 +444,19 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         const int m0 = tm * BM, n0 = n_base + tn * BN;
         float* s_as = reinterpret_cast<float*>(smem);
         uint32_t* stage = reinterpret_cast<uint32_t*>(smem + 4 * BM) + wave * Cfg::STAGE_WORDS;
-        for (int rr = tid; rr < BM; rr += THREADS) {
-            const int m = m0 + rr;
-            float v = 1.0f;
-            if (g.a_scale) v = g.a_scale[(g.a_scale_per_row && m < g.M) ? m : 0];
-            s_as[rr] = v;
-        }
+        if (!fetched) fetch_params(tm, tn);  // a shared tile finished by a worker that did not end it
+        if (tid < BM) s_as[tid] = as_mine;
         float S = 1.0f, Z = 0.0f;
         if (MODE == OUT_REQUANT_I8 || MODE == OUT_FAKEQUANT_F32) {
             S = g.out_scale[0];
             Z = g.out_zp[0];
         }
-        ColParams cp[TN];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int n = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
-            cp[j] = load_col(g, n < n_limit ? n : n_limit - 1);
-        }
+        const int esize = MODE == OUT_F16 ? 2 : (MODE == OUT_REQUANT_I8 ? 1 : 4);
+        const bool interior = m0 + BM <= g.M && n0 + BN <= n_limit && g.ldo % 4 == 0 &&
+                              reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0;
         __syncthreads();
-        tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z);
+        tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z, interior);
+        __syncthreads();  // the staging area is the next tile's first LDS stage
     };
 
     if (!SK) {
@@ -414,78 +467,140 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         return;
     }
 
-    // ---- stream-K
+    // ---- stream-K over the last g.sk_tiles tile ids, then the other tiles one
+    // block per tile (worker w takes tiles w, w + workers, ...).  The shared tiles
+    // come first: their partial sums are exchanged while every worker still has a
+    // whole tile of its own to compute, and nobody ever waits for anybody.
     constexpr int kAccWords = TM * TN * 16;  // accumulator registers per lane
     const int workers = gridDim.x;
-    const long total = long(tiles_m) * tiles_n * nk;
+    const int tiles = tiles_m * tiles_n;
+    const int dp_tiles = tiles - g.sk_tiles;
+    const long total = long(g.sk_tiles) * nk;
     const IterSplit split(total, workers);
     // give every XCD a contiguous range of workers (blocks are dealt round-robin)
     const int wq = workers / 8, wr = workers % 8;
     const int xcd = blockIdx.x % 8;
     const int me = xcd * wq + (xcd < wr ? xcd : wr) + blockIdx.x / 8;
+    // same m-fastest walk in groups of 8 m-tiles as tile_coords
+    auto coords = [&](int tile, int* tm, int* tn) {
+        constexpr int GM = 8;
+        const int group_size = GM * tiles_n;
+        const int group = tile / group_size;
+        const int first_m = group * GM;
+        const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+        const int in_group = tile - group * group_size;
+        *tm = first_m + in_group % gsz;
+        *tn = in_group / gsz;
+    };
     long it = split.begin(me);
     const long it_end = split.begin(me + 1);
-    int* counters = g.sk_counters + size_t(blockIdx.y) * tiles_m * tiles_n;
+    int dp_tile = me;
+    int* counters = g.sk_counters + size_t(blockIdx.y) * g.sk_tiles;
     int32_t* slabs = g.sk_slabs + size_t(blockIdx.y) * workers * 2 * size_t(kAccWords) * THREADS;
-    while (it < it_end) {
-        const int tile = int(it / nk);
-        const int kb = int(it - long(tile) * nk);
-        const int ke = (it_end - it) < (nk - kb) ? kb + int(it_end - it) : nk;
-        // same m-fastest walk in groups of 8 m-tiles as tile_coords
-        int tm, tn;
-        {
-            constexpr int GM = 8;
-            const int group_size = GM * tiles_n;
-            const int group = tile / group_size;
-            const int first_m = group * GM;
-            const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
-            const int in_group = tile - group * group_size;
-            tm = first_m + in_group % gsz;
-            tn = in_group / gsz;
+    // one loop over both kinds of work, so that the segment and the epilogue are
+    // instantiated once
+    for (;;) {
+        int tile, kb, ke, local = 0;
+        if (it < it_end) {
+            local = int(it / nk);  // index among the shared tiles
+            kb = int(it - long(local) * nk);
+            ke = (it_end - it) < (nk - kb) ? kb + int(it_end - it) : nk;
+            tile = dp_tiles + local;
+            it += ke - kb;
+        } else if (dp_tile < dp_tiles) {
+            tile = dp_tile;
+            kb = 0;
+            ke = nk;
+            dp_tile += workers;
+        } else {
+            break;
         }
+        int tm, tn;
+        coords(tile, &tm, &tn);
         run_segment(tm, tn, kb, ke);
         bool finish = true;
         if (!(kb == 0 && ke == nk)) {
-            const int w_first = split.owner(long(tile) * nk);
-            const int w_last = split.owner(long(tile) * nk + nk - 1);
+            const int w_first = split.owner(long(local) * nk);
+            const int w_last = split.owner(long(local) * nk + nk - 1);
             // slab 0 holds a worker's leading partial tile, slab 1 its trailing one
-            auto slab_of = [&](int w) {
-                const int first_tile = int(split.begin(w) / nk);
-                return slabs + (size_t(w) * 2 + (tile == first_tile ? 0 : 1)) * kAccWords * THREADS;
+            // (the address is the same in every lane; saying so keeps the buffer
+            // descriptor in scalar registers)
+            auto slab_of = [&](int w) -> int32_t* {
+                const int first_local = int(split.begin(w) / nk);
+                const uint64_t p = reinterpret_cast<uint64_t>(
+                    slabs + (size_t(w) * 2 + (local == first_local ? 0 : 1)) * kAccWords * THREADS);
+                const uint64_t lo = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(p))));
+                const uint64_t hi = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(p >> 32))));
+                return reinterpret_cast<int32_t*>((hi << 32) | lo);
             };
-            int32_t* mine = slab_of(me);
+            // The XCDs' L2 caches are not coherent with each other.  Instead of
+            // device-scope fences (which write back and invalidate a whole L2, under
+            // the feet of the 63 other blocks that share it), every access to a slab
+            // carries device scope itself: write-through stores, cache-bypassing loads.
+            // They are plain (non-atomic) buffer accesses with the device-scope bit, so
+            // the compiler keeps many of them in flight.
+            // 16 bytes per lane and access: chunk q of a lane's accumulators sits at
+            // (q * THREADS + tid) * 16 of the slab.
+            constexpr unsigned kScopeDevice = 16;  // "sc1" cache-policy bit of buffer accesses
+            constexpr unsigned kSlabBytes = kAccWords * THREADS * 4;
+            const unsigned lane_off = unsigned(tid) * 16;
+            {
+                const __amdgpu_buffer_rsrc_t mine =
+                    __builtin_amdgcn_make_buffer_rsrc(slab_of(me), 0, kSlabBytes, 0x00020000);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                    for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        mine[((i * TN + j) * 16 + r) * THREADS + tid] = acc[i][j][r];
-            __threadfence();  // partials visible device-wide before the arrival is counted
+                        for (int q = 0; q < 4; ++q) {
+                            const v4u v = {unsigned(acc[i][j][4 * q]), unsigned(acc[i][j][4 * q + 1]),
+                                           unsigned(acc[i][j][4 * q + 2]), unsigned(acc[i][j][4 * q + 3])};
+                            __builtin_amdgcn_raw_buffer_store_b128(
+                                v, mine, lane_off + unsigned(((i * TN + j) * 4 + q) * THREADS * 16), 0, kScopeDevice);
+                        }
+            }
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // this wavefront's partials have been written through
+            __syncthreads();                            // ... and so have the other wavefronts'
+            if (tid == 0)
+                s_flag = __hip_atomic_fetch_add(&counters[local], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
-            if (tid == 0) s_flag = atomicAdd(&counters[tile], 1);
-            __syncthreads();
-            finish = s_flag == (w_last - w_first);  // the other contributors have all arrived
+            // the other contributors have all arrived
+            finish = __builtin_amdgcn_readfirstlane(s_flag) == (w_last - w_first);
             if (finish) {
-                __threadfence();
                 for (int w = w_first; w <= w_last; ++w) {
                     if (w == me) continue;
-                    const int32_t* other = slab_of(w);
+                    const __amdgpu_buffer_rsrc_t other =
+                        __builtin_amdgcn_make_buffer_rsrc(slab_of(w), 0, kSlabBytes, 0x00020000);
+                    // eight 16-byte loads in flight per lane (the fragment registers of
+                    // the main loop are free here), then their 32 additions
+                    constexpr int kBatch = 8;
+                    static_assert((TM * TN * 4) % kBatch == 0, "");
 #pragma unroll
-                    for (int i = 0; i < TM; ++i)
+                    for (int c0 = 0; c0 < TM * TN * 4; c0 += kBatch) {
+                        v4u v[kBatch];
 #pragma unroll
-                        for (int j = 0; j < TN; ++j)
+                        for (int c = 0; c < kBatch; ++c)
+                            v[c] = __builtin_amdgcn_raw_buffer_load_b128(
+                                other, lane_off + unsigned((c0 + c) * THREADS * 16), 0, kScopeDevice);
 #pragma unroll
-                            for (int r = 0; r < 16; ++r)
-                                acc[i][j][r] += __builtin_nontemporal_load(
-                                    &other[((i * TN + j) * 16 + r) * THREADS + tid]);
+                        for (int c = 0; c < kBatch; ++c) {
+                            const int ij = (c0 + c) / 4, q = (c0 + c) % 4;
+                            v16i& a = acc[ij / TN][ij % TN];
+                            a[4 * q] += int(v[c].x);
+                            a[4 * q + 1] += int(v[c].y);
+                            a[4 * q + 2] += int(v[c].z);
+                            a[4 * q + 3] += int(v[c].w);
+                        }
+                        __builtin_amdgcn_sched_group_barrier(0x020, kBatch, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, kBatch * 4, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
-                if (tid == 0) counters[tile] = 0;  // ready for the next launch
+                if (tid == 0) counters[local] = 0;  // ready for the next launch
             }
             __syncthreads();
         }
         if (finish) run_epilogue(tm, tn);
-        it += ke - kb;
     }
 }
 
@@ -510,7 +625,7 @@ struct SkScratch {
     int32_t* slabs = nullptr;
     size_t slab_bytes = 0;
 };
-int sk_scratch(size_t counters, size_t slab_bytes, SkScratch** out);
+int sk_scratch(size_t counters, size_t slab_bytes, bool may_grow, SkScratch** out);
 
 namespace {
 
@@ -529,29 +644,48 @@ int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st
     // blocks that fit on the chip at once: 256 CUs x blocks per CU (LDS-bound)
     const int per_cu = (160 * 1024) / Cfg::SMEM < Cfg::MINWAVES ? (160 * 1024) / Cfg::SMEM : Cfg::MINWAVES;
     const int slots = 256 * (per_cu < 1 ? 1 : per_cu);
-    // schedule: 0 = choose, 1 = one block per tile, 2 = stream-K.
-    // Stream-K pays when the tiles fill the last round of blocks badly and there
-    // are few rounds; every worker must get at least a few k-iterations.
-    // Stream-K is opt-in only.  Measured at M=2048, N=11008, K=4096 it loses to one
-    // block per tile (128x256 tiles: 116 us vs 371 us; 175 us even with the
-    // device-scope fences taken out): the 128 KiB partial slabs per worker and the
-    // L2 write-back / invalidate of the fences cost more than the idle tail they remove.
-    const bool sk = schedule == 2;
+    // schedule: 0 = choose, 1 = one block per tile, 2 = stream-K over all tiles,
+    // 3 = hybrid: stream-K over the tiles that would form a badly filled last round
+    // of blocks (done first, so the partial sums are exchanged early), one block per
+    // tile for the rest.
+    // Both shared schedules are exact and tested, and both measured slower than one
+    // block per tile at M=2048, N=11008, K=4096 (111 us): 136 us for the hybrid,
+    // more for stream-K over everything.  The worker that finishes a shared tile
+    // pays a reduction and a second epilogue on top of its own whole tile, which
+    // costs more than the idle slots of the last round.  The automatic choice is
+    // therefore always one block per tile.
+    int sk_tiles = 0;
+    const int slots_g = slots / groups;
+    if (schedule == 2) {
+        sk_tiles = tiles;
+    } else if (schedule == 3) {
+        const int rem = slots_g > 0 ? tiles % slots_g : 0;
+        if (slots_g > 0 && rem > 0 && tiles > slots_g) sk_tiles = rem;
+    }
+    const bool sk = sk_tiles > 0;
     GemmArgs copy = g;
     void* kargs[] = {&copy};
     if (!sk) {
         LQ_HIP(hipLaunchKernel(fn_dp, dim3(tiles, groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
         return LQ_OK;
     }
-    long workers = slots / groups;
+    long workers = slots_g;
     if (workers < 1) workers = 1;
-    if (workers > long(tiles) * nk) workers = long(tiles) * nk;
+    if (workers > long(sk_tiles) * nk) workers = long(sk_tiles) * nk;
     SkScratch* s = nullptr;
     const size_t slab_words = size_t(Cfg::TM) * Cfg::TN * 16 * Cfg::THREADS;
-    int rc = sk_scratch(size_t(tiles) * groups, size_t(groups) * workers * 2 * slab_words * 4, &s);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    LQ_HIP(hipStreamIsCapturing(st, &capturing));
+    int rc = sk_scratch(size_t(sk_tiles) * groups, size_t(groups) * workers * 2 * slab_words * 4,
+                        capturing == hipStreamCaptureStatusNone, &s);
     if (rc) return rc;
+    if (!s) {  // scratch too small and the stream is being captured: one block per tile
+        LQ_HIP(hipLaunchKernel(fn_dp, dim3(tiles, groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
+        return LQ_OK;
+    }
     copy.sk_counters = s->counters;
     copy.sk_slabs = s->slabs;
+    copy.sk_tiles = sk_tiles;
     LQ_HIP(hipLaunchKernel(fn_sk, dim3(unsigned(workers), groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
     return LQ_OK;
 }

@@ -84,6 +84,30 @@ def test_stream_k_schedule_exact(cfg, M, N, K):
     assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
 
 
+@pytest.mark.parametrize("cfg,M,N,K", [(4, 2048, 11008, 512), (5, 3000, 3000, 256), (6, 4096, 2500, 320),
+                                       (3, 4096, 5000, 256), (4, 2100, 11000, 400), (1, 2048, 11008, 192)])
+def test_hybrid_schedule_exact(cfg, M, N, K):
+    """More tiles than fit on the chip at once: the leftover tiles of the last
+    round are shared between all workers (partial sums met by the last arriver),
+    the rest run one block per tile.  Launched twice: the arrival counters must
+    be left reset."""
+    rng = np.random.default_rng(cfg * 17 + M + N + K)
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    ref = O.igemm(a, w)
+    ad, wd = hip(a), hip(w)
+    tc = cfg | 0x300
+    for _ in range(2):
+        acc = _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, path=TILE, tile_config=tc).numpy()
+        assert np.array_equal(acc, ref)
+    a_scale = rng.uniform(0.005, 0.05, M).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    got = _ops.qlinear_i8(ad, wd, a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias),
+                          out_mode=_ops.OUT_F16, path=TILE, tile_config=tc).numpy()
+    exp = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, out_mode=O.OUT_F16)
+    assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+
+
 @pytest.mark.parametrize("path,M", [(TILE, 300), (SKINNY, 16), (NAIVE, 9)])
 def test_extreme_codes(path, M):
     K, N = 4096, 48
