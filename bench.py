@@ -44,7 +44,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X published HBM3E bandwidth, GB/s
 # the library's plain 1 GiB copy kernel: fetch x2.000, write x1.000).  The runs
 # are summarised in profiles/hbm_traffic_qlinear_and_quantize.md.
 MEASURED_TRAFFIC_BYTES = {
-    "linear_m2048": int((2.0 * 95728 + 44032) * 1024),
+    "linear_m2048": int((2.0 * 96636 + 44032) * 1024),
     "quantize_per_channel_i8": int((2.0 * 524577 + 262144) * 1024),
     "dequantize_per_channel_i8": int((2.0 * 131350 + 1048712) * 1024),
     "minmax_per_channel": int((2.0 * 524317 + 257) * 1024),
