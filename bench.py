@@ -252,6 +252,34 @@ def bench_resnet50(L, _C, steps, warmup):
     return out
 
 
+def bench_vit_b16(L, _C, steps, warmup):
+    """Dynamic-quantized ViT-B/16, batch 64, 3x224x224 uniform[0,1] inputs, random
+    N(0, 0.02) weights: all Linears W8A8 with runtime activation qparams; patch
+    embedding, LayerNorm, attention, GELU and residuals float32.  Captured once
+    into a HIP graph and replayed; eager time beside it."""
+    import workloads as W
+
+    model = W.QViT()
+    rng = np.random.default_rng(0)
+    batch = 64
+    x = L.tensor(rng.uniform(0, 1, (batch, 3, 224, 224)).astype(np.float32), device="hip")
+    y = model(x)
+    eager_total, _ = time_launches(_C, lambda: model(x), max(3, steps // 4), 1)
+    eager_ms = eager_total / max(3, steps // 4)
+    with L.graph.capture() as g:
+        y = model(x)
+    total, per = time_launches(_C, g.replay, steps, warmup)
+    ms = total / steps
+    gops = W.vit_linear_gops(batch=batch)
+    out = {"images_per_s": round(batch / ms * 1e3, 1), "ms_per_batch": round(ms, 4), "batch": batch,
+           "eager_ms_per_batch": round(eager_ms, 4),
+           "linear_int8_TOP/s_end_to_end": round(gops / ms, 2), "linear_GOP_per_batch": round(gops, 1),
+           "p95_ms": round(float(np.percentile(per, 95)), 4), "launch": "hip graph replay"}
+    assert np.isfinite(y.numpy()).all()
+    g.destroy()
+    return out
+
+
 def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     """Dynamic-quantized MLP Linear(784,256)-ReLU-Linear(256,10), batch 64
     (launch-latency bound: 0.43 MOP).  Eager = one Python-driven forward (9
@@ -425,6 +453,8 @@ def main() -> int:
         extra["dynamic_mlp_784_256_10_batch64"] = bench_dynamic_mlp(L, Q, _C, args.steps, args.warmup)
         extra["vit_b16_linears_batch64"] = bench_vit_linears(L, Q, _C, _ops, max(10, args.steps // 2),
                                                              max(3, args.warmup // 2))
+        extra["vit_b16_dynamic_int8_batch64"] = bench_vit_b16(L, _C, max(10, args.steps // 2),
+                                                              max(3, args.warmup // 2))
         extra["resnet50_int8_batch32"] = bench_resnet50(L, _C, max(10, args.steps // 2),
                                                         max(3, args.warmup // 2))
         line["extra"] = extra

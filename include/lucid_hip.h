@@ -174,6 +174,46 @@ int lq_add_requant_i8(const int8_t* qa, int a_offset, const float* a_scale, cons
 int lq_global_avgpool_nhwc_i8(const int8_t* q, int code_offset, int B, int H, int W, int C,
                               const float* scale, const float* zp, float* out, lq_stream stream);
 
+/* ------------------------------------------------- float32 steps of a ViT block */
+/* What Lucid's dynamic-quantized ViT keeps in float32 between its int8 Linears
+ * (lucid/models/vision/vit/_model.py:132-161,202-204,275-278,449-458).  Tolerance
+ * parity (1e-4 relative against a float32 CPU evaluation): summation orders differ. */
+
+/* LayerNorm over the last axis of [rows, cols] (IBackend::layer_norm_forward;
+ * lucid/_C/backend/cpu/Norm.cpp:35-65: mean, centred dot product / N,
+ * rstd = 1/sqrt(var + eps), (c * rstd) * gamma + beta). */
+int lq_layernorm_f32(const float* x, const float* gamma, const float* beta, float* out, long rows, int cols,
+                     float eps, lq_stream stream);
+
+/* GELU, exact erf form (lucid/nn/functional/activations.py:219, approximate="none"). */
+int lq_gelu_f32(const float* x, float* out, size_t n, lq_stream stream);
+
+/* out = a + b (IBackend::add on float32; the residual joins). */
+int lq_add_f32(const float* a, const float* b, float* out, size_t n, lq_stream stream);
+
+/* Scaled dot-product attention (IBackend::sdpa_forward, CpuBackend.h:7603-7730:
+ * softmax(scale * Q K^T) V, no mask, no dropout) read straight from the packed
+ * activation of the qkv Linear, [B, T, 3, H, D] (vit/_model.py:137-141), writing
+ * [B, T, H*D] (vit/_model.py:158).  D must be 64 and T <= 208 (ViT-B/16: T = 197);
+ * anything else returns LQ_ERR_NOT_IMPLEMENTED. */
+int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale, lq_stream stream);
+
+/* Patch embedding, a convolution whose stride equals its kernel
+ * (vit/_model.py:62-69), as im2col + GEMM: image [B,C,H,W] -> rows
+ * [B*(H/p)*(W/p), C*p*p] in (c, ph, pw) column order - the order of the conv
+ * weight [dim, C, p, p] flattened. */
+int lq_patchify_f32(const float* img, float* out, int B, int C, int H, int W, int patch, lq_stream stream);
+
+/* out[M,N] = a[M,K] . w[N,K]^T + bias[N] in float32 (IBackend::linear, CpuBackend.h:4525);
+ * bias may be null. */
+int lq_sgemm_nt_f32(const float* a, const float* w, const float* bias, float* out, int M, int N, int K,
+                    lq_stream stream);
+
+/* tokens[b,0,:] = cls + pos[0], tokens[b,1+i,:] = patches[b,i,:] + pos[1+i]
+ * (cat + position table, vit/_model.py:452-454); out is [B, T, D], patches [B, T-1, D]. */
+int lq_assemble_tokens_f32(const float* patches, const float* cls, const float* pos, float* out, int B, int T,
+                           int D, lq_stream stream);
+
 /* Quantized Linear on a float activation that lies on no grid - literally
  * lucid/nn/quantized/linear.py:199-215: dequantize(weight) -> x @ W^T + bias ->
  * [relu] -> [fake_quantize].  float32 accumulation; for small layers (e.g. the

@@ -124,6 +124,14 @@ _SIGNATURES["lq_add_requant_i8"] = [_vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _sz, _
 _SIGNATURES["lq_global_avgpool_nhwc_i8"] = [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]
 _SIGNATURES["lq_qlinear_w8a32"] = [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp,
                                    _vp]
+_l = C.c_long
+_SIGNATURES["lq_layernorm_f32"] = [_vp, _vp, _vp, _vp, _l, _i, _f, _vp]
+_SIGNATURES["lq_gelu_f32"] = [_vp, _vp, _sz, _vp]
+_SIGNATURES["lq_add_f32"] = [_vp, _vp, _vp, _sz, _vp]
+_SIGNATURES["lq_attention_f32"] = [_vp, _vp, _i, _i, _i, _i, _f, _vp]
+_SIGNATURES["lq_patchify_f32"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
+_SIGNATURES["lq_sgemm_nt_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
+_SIGNATURES["lq_assemble_tokens_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
 _SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]

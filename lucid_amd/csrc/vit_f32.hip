@@ -1,0 +1,454 @@
+// float32 companions of the int8 Linear path: what a ViT block does between its
+// quantized Linears.  Lucid's dynamic-quantized ViT keeps LayerNorm, attention,
+// GELU, the residual adds and the patch embedding in float32
+// (lucid/models/vision/vit/_model.py:132-161,202-204,275-278,449-458); these kernels
+// are those steps on gfx950, in float32 end to end:
+//
+//   lq_layernorm_f32        lucid/_C/backend/cpu/Norm.cpp:35-65
+//   lq_gelu_f32             lucid/nn/functional/activations.py:219 (approximate="none", erf)
+//   lq_add_f32              residual add
+//   lq_attention_f32        scaled dot-product attention, CpuBackend.h:7603-7730,
+//                           read straight from the packed qkv activation
+//   lq_patchify_f32 + lq_sgemm_nt_f32   the stride = kernel patch convolution as a GEMM
+//   lq_assemble_tokens_f32  class token + position table
+//
+// Matrix products use the float32 MFMA instructions; results agree with a CPU
+// float32 evaluation to rounding-order differences (tested to 1e-4 relative).
+#include "common.hpp"
+
+using namespace lq;
+
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// ---------------------------------------------------------------- LayerNorm
+// One wavefront per row; the row (a few KiB) is re-read from cache for the
+// variance and the output pass.  mean, centred values, var = dot(c,c)/N,
+// rstd = 1/sqrt(var+eps), y = (c*rstd)*gamma + beta: the reference's steps.
+__global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x,
+                                                        const float* __restrict__ gamma,
+                                                        const float* __restrict__ beta,
+                                                        float* __restrict__ out, long rows, int cols,
+                                                        float eps) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const long row = long(blockIdx.x) * 4 + wave;
+    if (row >= rows) return;
+    const float* xr = x + row * cols;
+    float* yr = out + row * cols;
+    const bool vec = (cols % 4 == 0) && aligned16(x) && aligned16(out) && aligned16(gamma) && aligned16(beta);
+    const float inv_n = 1.0f / float(cols);
+    float s = 0.0f;
+    if (vec) {
+        for (int c = lane * 4; c < cols; c += 256) {
+            const float4 v = *reinterpret_cast<const float4*>(xr + c);
+            s += (v.x + v.y) + (v.z + v.w);
+        }
+    } else {
+        for (int c = lane; c < cols; c += 64) s += xr[c];
+    }
+    const float mean = wave_sum(s) * inv_n;
+    float q = 0.0f;
+    if (vec) {
+        for (int c = lane * 4; c < cols; c += 256) {
+            const float4 v = *reinterpret_cast<const float4*>(xr + c);
+            const float a = v.x - mean, b = v.y - mean, cc = v.z - mean, d = v.w - mean;
+            q += (a * a + b * b) + (cc * cc + d * d);
+        }
+    } else {
+        for (int c = lane; c < cols; c += 64) {
+            const float a = xr[c] - mean;
+            q += a * a;
+        }
+    }
+    const float var = wave_sum(q) * inv_n;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    if (vec) {
+        for (int c = lane * 4; c < cols; c += 256) {
+            const float4 v = *reinterpret_cast<const float4*>(xr + c);
+            const float4 g = *reinterpret_cast<const float4*>(gamma + c);
+            const float4 b = *reinterpret_cast<const float4*>(beta + c);
+            float4 y;
+            y.x = ((v.x - mean) * rstd) * g.x + b.x;
+            y.y = ((v.y - mean) * rstd) * g.y + b.y;
+            y.z = ((v.z - mean) * rstd) * g.z + b.z;
+            y.w = ((v.w - mean) * rstd) * g.w + b.w;
+            *reinterpret_cast<float4*>(yr + c) = y;
+        }
+    } else {
+        for (int c = lane; c < cols; c += 64) yr[c] = ((xr[c] - mean) * rstd) * gamma[c] + beta[c];
+    }
+}
+
+// ---------------------------------------------------------------- elementwise
+__device__ __forceinline__ float gelu_erf(float x) {
+    return (0.5f * x) * (1.0f + erff(x * 0.70710678118654752440f));
+}
+
+__global__ __launch_bounds__(256) void gelu_kernel(const float* __restrict__ x, float* __restrict__ out,
+                                                   size_t n, int vec) {
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (vec) {
+        if (i * 4 >= n) return;
+        const float4 v = reinterpret_cast<const float4*>(x)[i];
+        float4 y = {gelu_erf(v.x), gelu_erf(v.y), gelu_erf(v.z), gelu_erf(v.w)};
+        reinterpret_cast<float4*>(out)[i] = y;
+    } else if (i < n) {
+        out[i] = gelu_erf(x[i]);
+    }
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                  float* __restrict__ out, size_t n, int vec) {
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (vec) {
+        if (i * 4 >= n) return;
+        const float4 u = reinterpret_cast<const float4*>(a)[i];
+        const float4 v = reinterpret_cast<const float4*>(b)[i];
+        float4 y = {u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w};
+        reinterpret_cast<float4*>(out)[i] = y;
+    } else if (i < n) {
+        out[i] = a[i] + b[i];
+    }
+}
+
+// image [B,C,H,W] -> patch rows [B*(H/p)*(W/p), C*p*p], column order (c, ph, pw):
+// the im2col of a convolution whose stride equals its kernel
+__global__ __launch_bounds__(256) void patchify_kernel(const float* __restrict__ img, float* __restrict__ out,
+                                                       int B, int C, int H, int W, int p) {
+    const int gh = H / p, gw = W / p, K = C * p * p;
+    const size_t total = size_t(B) * gh * gw * K;
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int k = int(i % K);
+    const size_t row = i / K;
+    const int pw = k % p, ph = (k / p) % p, c = k / (p * p);
+    const int gx = int(row % gw), gy = int((row / gw) % gh), b = int(row / (size_t(gw) * gh));
+    out[i] = img[((size_t(b) * C + c) * H + (gy * p + ph)) * W + (gx * p + pw)];
+}
+
+// tokens[b,0,:] = cls + pos[0]; tokens[b,1+i,:] = patches[b,i,:] + pos[1+i]
+__global__ __launch_bounds__(256) void assemble_tokens_kernel(const float* __restrict__ patches,
+                                                              const float* __restrict__ cls,
+                                                              const float* __restrict__ pos,
+                                                              float* __restrict__ out, int B, int T, int D) {
+    const size_t total = size_t(B) * T * D;
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int d = int(i % D);
+    const int t = int((i / D) % T);
+    const size_t b = i / (size_t(D) * T);
+    const float v = t == 0 ? cls[d] : patches[(b * (T - 1) + (t - 1)) * D + d];
+    out[i] = v + pos[size_t(t) * D + d];
+}
+
+// ---------------------------------------------------------------- float32 GEMM, out = a . w^T + bias
+// 128 x 128 x 16 block tile, 4 wavefronts of 64 x 64, v_mfma_f32_32x32x2_f32.
+// LDS tiles are k-major ([k][row], rows padded) so that a fragment read takes
+// consecutive words.
+constexpr int SG_BM = 128, SG_BN = 128, SG_BK = 16, SG_LD = 128 + 4;
+
+__global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__ a, const float* __restrict__ w,
+                                                       const float* __restrict__ bias, float* __restrict__ out,
+                                                       int M, int N, int K) {
+    __shared__ float sa[2][SG_BK][SG_LD];
+    __shared__ float sb[2][SG_BK][SG_LD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * SG_BM, n0 = blockIdx.x * SG_BN;
+    // loader: thread -> (row = tid / 4 (+64), 4 consecutive k at 4 * (tid % 4))
+    const int lrow = tid >> 2, lk = (tid & 3) * 4;
+    const bool vec = (K % 4 == 0) && aligned16(a) && aligned16(w);
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    float4 ra[2], rb[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int m = m0 + lrow + 64 * h, n = n0 + lrow + 64 * h, k = k0 + lk;
+            float4 va = {0.f, 0.f, 0.f, 0.f}, vb = {0.f, 0.f, 0.f, 0.f};
+            if (m < M) {
+                const float* p = a + size_t(m) * K + k;
+                if (vec && k + 3 < K) {
+                    va = *reinterpret_cast<const float4*>(p);
+                } else {
+                    if (k < K) va.x = p[0];
+                    if (k + 1 < K) va.y = p[1];
+                    if (k + 2 < K) va.z = p[2];
+                    if (k + 3 < K) va.w = p[3];
+                }
+            }
+            if (n < N) {
+                const float* p = w + size_t(n) * K + k;
+                if (vec && k + 3 < K) {
+                    vb = *reinterpret_cast<const float4*>(p);
+                } else {
+                    if (k < K) vb.x = p[0];
+                    if (k + 1 < K) vb.y = p[1];
+                    if (k + 2 < K) vb.z = p[2];
+                    if (k + 3 < K) vb.w = p[3];
+                }
+            }
+            ra[h] = va;
+            rb[h] = vb;
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int r = lrow + 64 * h;
+            sa[buf][lk][r] = ra[h].x, sa[buf][lk + 1][r] = ra[h].y, sa[buf][lk + 2][r] = ra[h].z,
+            sa[buf][lk + 3][r] = ra[h].w;
+            sb[buf][lk][r] = rb[h].x, sb[buf][lk + 1][r] = rb[h].y, sb[buf][lk + 2][r] = rb[h].z,
+            sb[buf][lk + 3][r] = rb[h].w;
+        }
+    };
+    const int nk = (K + SG_BK - 1) / SG_BK;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int t = 0; t < nk; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < nk) fetch((t + 1) * SG_BK);
+#pragma unroll
+        for (int kk = 0; kk < SG_BK; kk += 2) {
+            const int kr = kk + (lane >> 5);
+            float fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) fa[i] = sa[buf][kr][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fb[j] = sb[buf][kr][wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (t + 1 < nk) {
+            stash(buf ^ 1);  // the other buffer was last read one iteration ago, behind a barrier
+            __syncthreads();
+        }
+    }
+    // result layout of the 32x32 MFMA: column = lane % 32, row = 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+            if (n >= N) continue;
+            const float bv = bias ? bias[n] : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < M) out[size_t(m) * N + n] = acc[i][j][r] + bv;
+            }
+        }
+}
+
+// ---------------------------------------------------------------- attention
+// One block per (batch, head); one wavefront per 16 queries; head dim 64, at
+// most 208 tokens.  qkv is the packed activation [B, T, 3, H, 64] of the qkv
+// Linear; out is [B, T, H*64].
+//
+// Per wavefront: S^T = K . Q^T as 13 tiles of 16 keys x 16 queries
+// (v_mfma_f32_16x16x4_f32, accumulators stay in registers), softmax over the
+// keys of each query (a lane holds 52 of a query's keys, the other three lane
+// groups the rest), then O = P . V where the S^T accumulators ARE the A
+// operand: register r of a tile holds P[query = lane%16][key = 16t + 4*(lane/16) + r],
+// which is a valid k-slice assignment as long as V is read with the same one.
+constexpr int AT_D = 64, AT_TMAX = 208, AT_LD = AT_D + 4;  // row stride 68: 4*row + k hits all 64 banks
+
+__global__ __launch_bounds__(832) void attention_kernel(const float* __restrict__ qkv, float* __restrict__ out,
+                                                        int B, int T, int H, float scale) {
+    extern __shared__ __attribute__((aligned(16))) float at_smem[];
+    float (*sk)[AT_LD] = reinterpret_cast<float (*)[AT_LD]>(at_smem);
+    float (*sv)[AT_LD] = reinterpret_cast<float (*)[AT_LD]>(at_smem + AT_TMAX * AT_LD);
+    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nwaves = blockDim.x >> 6;
+    const size_t tok_stride = size_t(3) * H * AT_D;
+    const float* base = qkv + size_t(b) * T * tok_stride + size_t(h) * AT_D;
+    // K and V rows into LDS (rows past T are zero)
+    for (int i = tid; i < AT_TMAX * (AT_D / 4); i += blockDim.x) {
+        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        float4 kv = {0.f, 0.f, 0.f, 0.f}, vv = {0.f, 0.f, 0.f, 0.f};
+        if (row < T) {
+            const float* p = base + size_t(row) * tok_stride + c4;
+            kv = *reinterpret_cast<const float4*>(p + size_t(H) * AT_D);
+            vv = *reinterpret_cast<const float4*>(p + size_t(2) * H * AT_D);
+        }
+        *reinterpret_cast<float4*>(&sk[row][c4]) = kv;
+        *reinterpret_cast<float4*>(&sv[row][c4]) = vv;
+    }
+    __syncthreads();
+    const int q0 = wave * 16;
+    if (q0 >= T || wave >= nwaves) return;  // no barrier below this line
+    const int g = lane >> 4, c = lane & 15;
+    // B operand of S^T: Q[q0 + c][4*s + g], pre-scaled so that S = scale * Q.K^T
+    float qf[AT_D / 4];
+    {
+        const int q = q0 + c;
+        const float* qp = base + size_t(q < T ? q : T - 1) * tok_stride;
+#pragma unroll
+        for (int s = 0; s < AT_D / 4; ++s) qf[s] = qp[4 * s + g] * scale;
+    }
+    constexpr int NT = AT_TMAX / 16;
+    v4f st[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        v4f a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < AT_D / 4; ++s)
+            a = __builtin_amdgcn_mfma_f32_16x16x4f32(sk[16 * t + c][4 * s + g], qf[s], a, 0, 0, 0);
+        st[t] = a;
+    }
+    // st[t][r] = S[query q0 + c][key 16t + 4g + r]
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int key = 16 * t + 4 * g + r;
+            if (key >= T) st[t][r] = -__builtin_inff();
+            mx = fmaxf(mx, st[t][r]);
+        }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float sum = 0.0f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float e = expf(st[t][r] - mx);  // exp(-inf) = 0 for the padded keys
+            st[t][r] = e;
+            sum += e;
+        }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+    // O[q][n] = sum_key P[q][key] V[key][n], four 16-wide column tiles
+    v4f o[AT_D / 16];
+#pragma unroll
+    for (int j = 0; j < AT_D / 16; ++j) o[j] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float p = st[t][r] * inv;
+#pragma unroll
+            for (int j = 0; j < AT_D / 16; ++j)
+                o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, sv[16 * t + 4 * g + r][16 * j + c], o[j], 0, 0, 0);
+        }
+    // result layout of the 16x16 MFMA: column = lane % 16, row = 4*(lane/16) + r
+#pragma unroll
+    for (int j = 0; j < AT_D / 16; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int q = q0 + 4 * g + r;
+            if (q < T) out[(size_t(b) * T + q) * (size_t(H) * AT_D) + size_t(h) * AT_D + 16 * j + c] = o[j][r];
+        }
+}
+
+unsigned blocks_for(size_t n) { return unsigned((n + 255) / 256); }
+
+}  // namespace
+
+extern "C" {
+
+int lq_layernorm_f32(const float* x, const float* gamma, const float* beta, float* out, long rows, int cols,
+                     float eps, void* stream) {
+    LQ_REQUIRE(x && gamma && beta && out, LQ_ERR_VALUE, "layernorm: null pointer");
+    LQ_REQUIRE(rows >= 0 && cols > 0, LQ_ERR_SHAPE, "layernorm: bad shape (%ld, %d)", rows, cols);
+    if (rows == 0) return LQ_OK;
+    LQ_REQUIRE((rows + 3) / 4 < 0x7fffffffL, LQ_ERR_SHAPE, "layernorm: too many rows");
+    layernorm_kernel<<<unsigned((rows + 3) / 4), 256, 0, as_stream(stream)>>>(x, gamma, beta, out, rows, cols, eps);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_gelu_f32(const float* x, float* out, size_t n, void* stream) {
+    LQ_REQUIRE(x && out, LQ_ERR_VALUE, "gelu: null pointer");
+    if (n == 0) return LQ_OK;
+    const int vec = (n % 4 == 0) && aligned16(x) && aligned16(out);
+    gelu_kernel<<<blocks_for(vec ? n / 4 : n), 256, 0, as_stream(stream)>>>(x, out, n, vec);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_add_f32(const float* a, const float* b, float* out, size_t n, void* stream) {
+    LQ_REQUIRE(a && b && out, LQ_ERR_VALUE, "add: null pointer");
+    if (n == 0) return LQ_OK;
+    const int vec = (n % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(out);
+    add_kernel<<<blocks_for(vec ? n / 4 : n), 256, 0, as_stream(stream)>>>(a, b, out, n, vec);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_patchify_f32(const float* img, float* out, int B, int C, int H, int W, int patch, void* stream) {
+    LQ_REQUIRE(img && out, LQ_ERR_VALUE, "patchify: null pointer");
+    LQ_REQUIRE(B >= 0 && C > 0 && H > 0 && W > 0 && patch > 0 && H % patch == 0 && W % patch == 0, LQ_ERR_SHAPE,
+               "patchify: image %dx%dx%dx%d is not a whole number of %d-pixel patches", B, C, H, W, patch);
+    const size_t total = size_t(B) * C * H * W;
+    if (total == 0) return LQ_OK;
+    patchify_kernel<<<blocks_for(total), 256, 0, as_stream(stream)>>>(img, out, B, C, H, W, patch);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_assemble_tokens_f32(const float* patches, const float* cls, const float* pos, float* out, int B, int T,
+                           int D, void* stream) {
+    LQ_REQUIRE(patches && cls && pos && out, LQ_ERR_VALUE, "assemble_tokens: null pointer");
+    LQ_REQUIRE(B >= 0 && T >= 1 && D > 0, LQ_ERR_SHAPE, "assemble_tokens: bad shape");
+    const size_t total = size_t(B) * T * D;
+    if (total == 0) return LQ_OK;
+    assemble_tokens_kernel<<<blocks_for(total), 256, 0, as_stream(stream)>>>(patches, cls, pos, out, B, T, D);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_sgemm_nt_f32(const float* a, const float* w, const float* bias, float* out, int M, int N, int K,
+                    void* stream) {
+    LQ_REQUIRE(a && w && out, LQ_ERR_VALUE, "sgemm: null pointer");
+    LQ_REQUIRE(M >= 0 && N >= 0 && K > 0, LQ_ERR_SHAPE, "sgemm: bad shape (%d, %d, %d)", M, N, K);
+    if (M == 0 || N == 0) return LQ_OK;
+    dim3 grid((N + SG_BN - 1) / SG_BN, (M + SG_BM - 1) / SG_BM);
+    LQ_REQUIRE(grid.y < 65536, LQ_ERR_SHAPE, "sgemm: M too large");
+    sgemm_nt_kernel<<<grid, 256, 0, as_stream(stream)>>>(a, w, bias, out, M, N, K);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale, void* stream) {
+    LQ_REQUIRE(qkv && out, LQ_ERR_VALUE, "attention: null pointer");
+    LQ_REQUIRE(B >= 0 && T >= 1 && H >= 1, LQ_ERR_SHAPE, "attention: bad shape");
+    LQ_REQUIRE(D == AT_D && T <= AT_TMAX, LQ_ERR_NOT_IMPLEMENTED,
+               "attention: head dim %d / %d tokens; this kernel handles head dim 64 and up to 208 tokens", D, T);
+    LQ_REQUIRE(aligned16(qkv), LQ_ERR_VALUE, "attention: qkv must be 16-byte aligned");
+    if (B == 0) return LQ_OK;
+    const int waves = (T + 15) / 16;
+    constexpr size_t kSmem = size_t(2) * AT_TMAX * AT_LD * sizeof(float);
+    static bool attr_set = false;
+    if (!attr_set) {
+        LQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(kSmem)));
+        attr_set = true;
+    }
+    attention_kernel<<<unsigned(B) * H, waves * 64, kSmem, as_stream(stream)>>>(qkv, out, B, T, H, scale);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,81 @@
+"""float32 functional ops that sit between the quantized Linears of a
+transformer block (``lucid.nn.functional``: ``layer_norm``, ``gelu``,
+``scaled_dot_product_attention``) plus the residual add.  Each is one HIP
+kernel; inputs and outputs are float32 tensors on the ``hip`` device.
+"""
+
+from __future__ import annotations
+
+import math
+
+from .. import _C
+from .. import _tensor as T
+from .._tensor import Tensor
+
+
+def _require_f32_hip(name: str, *ts: Tensor) -> None:
+    for t in ts:
+        if not isinstance(t, Tensor) or t.device != "hip":
+            raise _C.DeviceMismatch(f"{name}: inputs must be tensors on the 'hip' device")
+        if t.dtype != T.float32:
+            raise _C.DtypeMismatch(f"{name} expects float32, got {t.dtype}")
+
+
+def layer_norm(x: Tensor, normalized_shape, weight: Tensor, bias: Tensor, eps: float = 1e-5) -> Tensor:
+    """``F.layer_norm`` over the last axis (``lucid/_C/backend/cpu/Norm.cpp:35-65``)."""
+    _require_f32_hip("layer_norm", x, weight, bias)
+    cols = normalized_shape if isinstance(normalized_shape, int) else int(normalized_shape[-1])
+    if x.shape[-1] != cols or weight.numel != cols or bias.numel != cols:
+        raise _C.ShapeMismatch(f"layer_norm: last dim {x.shape[-1]} vs normalized_shape {cols}")
+    out = Tensor.empty(x.shape, T.float32, "hip")
+    _C.call("lq_layernorm_f32", x.data_ptr, weight.data_ptr, bias.data_ptr, out.data_ptr,
+            x.numel // cols, cols, float(eps), None)
+    return out
+
+
+def gelu(x: Tensor, approximate: str = "none") -> Tensor:
+    """``F.gelu`` (``lucid/nn/functional/activations.py:219``), exact erf form."""
+    if approximate != "none":
+        raise NotImplementedError("gelu: only approximate='none' is built")
+    _require_f32_hip("gelu", x)
+    out = Tensor.empty(x.shape, T.float32, "hip")
+    _C.call("lq_gelu_f32", x.data_ptr, out.data_ptr, x.numel, None)
+    return out
+
+
+def add(a: Tensor, b: Tensor) -> Tensor:
+    _require_f32_hip("add", a, b)
+    if a.shape != b.shape:
+        raise _C.ShapeMismatch(f"add: {a.shape} vs {b.shape}")
+    out = Tensor.empty(a.shape, T.float32, "hip")
+    _C.call("lq_add_f32", a.data_ptr, b.data_ptr, out.data_ptr, a.numel, None)
+    return out
+
+
+def scaled_dot_product_attention_qkv(qkv: Tensor, num_heads: int, scale: float | None = None) -> Tensor:
+    """``F.scaled_dot_product_attention(q, k, v)`` on the packed output of a qkv
+    Linear: ``qkv`` is ``(B, T, 3*H*D)`` laid out ``(B, T, 3, H, D)`` as in
+    ``lucid/models/vision/vit/_model.py:137-141``; returns ``(B, T, H*D)``, the
+    ``permute(0, 2, 1, 3).reshape(B, T, C)`` of ``_model.py:158``."""
+    _require_f32_hip("scaled_dot_product_attention", qkv)
+    if qkv.ndim != 3 or qkv.shape[2] % (3 * num_heads):
+        raise _C.ShapeMismatch(f"attention: bad packed qkv shape {qkv.shape} for {num_heads} heads")
+    B, Tn, C3 = qkv.shape
+    D = C3 // (3 * num_heads)
+    s = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    out = Tensor.empty((B, Tn, num_heads * D), T.float32, "hip")
+    _C.call("lq_attention_f32", qkv.data_ptr, out.data_ptr, B, Tn, num_heads, D, s, None)
+    return out
+
+
+def linear_f32(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
+    """``F.linear`` in float32 (``CpuBackend.h:4525``): ``x @ weight.T + bias``."""
+    _require_f32_hip("linear", x, weight)
+    K = weight.shape[1]
+    if x.shape[-1] != K:
+        raise _C.ShapeMismatch(f"linear: {x.shape} @ {weight.shape}^T")
+    M, N = x.numel // K, weight.shape[0]
+    out = Tensor.empty((*x.shape[:-1], N), T.float32, "hip")
+    _C.call("lq_sgemm_nt_f32", x.data_ptr, weight.data_ptr, bias.data_ptr if bias is not None else None,
+            out.data_ptr, M, N, K, None)
+    return out

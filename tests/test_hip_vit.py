@@ -1,0 +1,152 @@
+"""float32 ViT kernels and the end-to-end dynamic-quantized ViT against the CPU
+restatement (oracle/vit.py).  float32 steps: 1e-4 relative (summation orders
+differ); the quantized Linears inside are bit-exact given equal inputs, but
+float32 noise ahead of a dynamic quantizer can move an activation across a
+rounding tie, so end-to-end agreement is stated as a tolerance."""
+
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import lucid_amd as L
+import lucid_amd.nn.functional as F
+import oracle.vit as V
+import workloads
+from lucid_amd import _C
+
+pytestmark = pytest.mark.gpu
+
+
+def hip(a):
+    return L.tensor(a, device="hip")
+
+
+def rel(a, b):
+    return float(np.max(np.abs(a.astype(np.float64) - b.astype(np.float64))) /
+                 max(1e-30, np.max(np.abs(b.astype(np.float64)))))
+
+
+@pytest.mark.parametrize("rows,cols", [(12608, 768), (7, 768), (5, 33), (1, 1), (64, 1000), (3, 4)])
+def test_layer_norm(rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(cols)).astype(np.float32)
+    got = F.layer_norm(hip(x), cols, hip(g), hip(b), 1e-6).numpy()
+    exp = V.layer_norm(x, g, b, 1e-6)
+    assert np.max(np.abs(got - exp)) <= 1e-4 * max(1.0, np.max(np.abs(exp)))
+
+
+@pytest.mark.parametrize("n", [1, 3, 1024, 12608 * 3072 // 8 + 5])
+def test_gelu_and_add(n):
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 2).astype(np.float32)
+    y = rng.standard_normal(n).astype(np.float32)
+    got = F.gelu(hip(x)).numpy()
+    exp = V.gelu(x)
+    assert np.max(np.abs(got - exp)) <= 2e-6
+    assert np.array_equal(F.add(hip(x), hip(y)).numpy(), x + y)
+
+
+@pytest.mark.parametrize("B,T,H", [(2, 197, 12), (1, 1, 1), (3, 16, 2), (2, 17, 3), (1, 208, 2), (4, 50, 12)])
+def test_attention_on_packed_qkv(B, T, H):
+    rng = np.random.default_rng(B * 1000 + T * 10 + H)
+    qkv = rng.standard_normal((B, T, 3 * H * 64)).astype(np.float32)
+    got = F.scaled_dot_product_attention_qkv(hip(qkv), H).numpy()
+    exp = V.attention_qkv(qkv, H)
+    assert rel(got, exp) < 1e-4
+
+
+def test_attention_rejects_what_the_kernel_does_not_cover():
+    with pytest.raises(NotImplementedError):
+        F.scaled_dot_product_attention_qkv(hip(np.zeros((1, 4, 3 * 2 * 32), np.float32)), 2)  # head dim 32
+    with pytest.raises(NotImplementedError):
+        F.scaled_dot_product_attention_qkv(hip(np.zeros((1, 209, 3 * 64), np.float32)), 1)  # 209 tokens
+
+
+@pytest.mark.parametrize("M,N,K", [(12544, 768, 768), (1, 1, 1), (130, 70, 19), (64, 200, 768), (257, 129, 33)])
+def test_float_linear(M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    got = F.linear_f32(hip(x), hip(w), hip(b)).numpy()
+    exp = x.astype(np.float64) @ w.astype(np.float64).T + b
+    assert rel(got, exp) < 1e-5
+    got = F.linear_f32(hip(x), hip(w)).numpy()
+    assert rel(got, x.astype(np.float64) @ w.astype(np.float64).T) < 1e-5
+
+
+def test_patchify_and_token_assembly_are_exact():
+    rng = np.random.default_rng(3)
+    img = rng.standard_normal((3, 3, 32, 48)).astype(np.float32)
+    rows = L.Tensor.empty((3 * 6, 3 * 256), L.float32, "hip")
+    _C.call("lq_patchify_f32", hip(img).data_ptr, rows.data_ptr, 3, 3, 32, 48, 16, None)
+    assert np.array_equal(rows.numpy(), V.patch_rows(img, 16))
+    emb = rng.standard_normal((3, 6, 40)).astype(np.float32)
+    cls = rng.standard_normal(40).astype(np.float32)
+    pos = rng.standard_normal((7, 40)).astype(np.float32)
+    out = L.Tensor.empty((3, 7, 40), L.float32, "hip")
+    _C.call("lq_assemble_tokens_f32", hip(emb).data_ptr, hip(cls).data_ptr, hip(pos).data_ptr,
+            out.data_ptr, 3, 7, 40, None)
+    exp = np.concatenate([np.broadcast_to(cls, (3, 1, 40)), emb], axis=1) + pos[None]
+    assert np.array_equal(out.numpy(), exp.astype(np.float32))
+
+
+SMALL = dict(image=64, patch=16, dim=128, depth=2, heads=2, mlp=256, classes=10)
+
+
+def test_vit_b16_block_stage_by_stage():
+    """Every step of a ViT-B/16 block fed with the CPU path's own input for that
+    step: the quantized Linears are bit-exact, the float32 steps agree to
+    rounding order."""
+    cfg = workloads.VIT_B16
+    p = workloads.vit_float_params(cfg, seed=4)
+    rng = np.random.default_rng(11)
+    images = rng.uniform(0, 1, (2, 3, 224, 224)).astype(np.float32)
+    model = workloads.QViT(cfg, params=p)
+    st = {}
+    V.vit_forward(p, images, cfg, stages=st)
+    blk = model.blocks[0]
+    tok, b = st["tokens"], "blocks.0."
+    h = V.layer_norm(tok, p[b + "norm1.weight"], p[b + "norm1.bias"], 1e-6)
+    assert rel(blk.norm1(hip(tok)).numpy(), h) < 1e-5
+    wq, ws = V.quantize_weight(p[b + "qkv.weight"])
+    assert np.array_equal(blk.qkv.weight_int8.numpy(), wq) and np.array_equal(blk.qkv.weight_scale.numpy(), ws)
+    qkv = V.dynamic_linear(h, wq, ws, p[b + "qkv.bias"])
+    assert np.array_equal(blk.qkv(hip(h)).numpy(), qkv)
+    a = V.attention_qkv(qkv, cfg["heads"])
+    assert rel(F.scaled_dot_product_attention_qkv(hip(qkv), cfg["heads"]).numpy(), a) < 1e-5
+    wq, ws = V.quantize_weight(p[b + "proj.weight"])
+    pr = V.dynamic_linear(a, wq, ws, p[b + "proj.bias"])
+    assert np.array_equal(blk.proj(hip(a)).numpy(), pr)
+    x1 = (tok + pr).astype(np.float32)
+    h2 = V.layer_norm(x1, p[b + "norm2.weight"], p[b + "norm2.bias"], 1e-6)
+    wq, ws = V.quantize_weight(p[b + "fc1.weight"])
+    f1 = V.dynamic_linear(h2, wq, ws, p[b + "fc1.bias"])
+    assert np.array_equal(blk.fc1(hip(h2)).numpy(), f1)
+    ge = V.gelu(f1)
+    assert np.max(np.abs(F.gelu(hip(f1)).numpy() - ge)) <= 2e-6
+    wq, ws = V.quantize_weight(p[b + "fc2.weight"])
+    assert np.array_equal(blk.fc2(hip(ge)).numpy(), V.dynamic_linear(ge, wq, ws, p[b + "fc2.bias"]))
+
+
+@pytest.mark.parametrize("cfg,batch", [(SMALL, 3), (workloads.VIT_B16, 2)])
+def test_vit_end_to_end_against_the_cpu_path(cfg, batch):
+    """Free-running comparison.  A dynamic quantizer turns an input difference d
+    (here float32 rounding order, 1e-7) into an RMS difference of sqrt(d * step)
+    on the elements that cross a rounding tie, so after a few layers two correct
+    implementations differ at the level of the quantization step itself
+    (~0.4 % of the activation range per layer); the bound below is that level,
+    not a rounding-error bound.  Stage-by-stage parity is the test above."""
+    p = workloads.vit_float_params(cfg, seed=4)
+    rng = np.random.default_rng(11)
+    images = rng.uniform(0, 1, (batch, 3, cfg["image"], cfg["image"])).astype(np.float32)
+    model = workloads.QViT(cfg, params=p)
+    got = model(hip(images)).numpy()
+    exp = V.vit_forward(p, images, cfg)
+    assert got.shape == exp.shape == (batch, cfg["classes"])
+    err = rel(got, exp)
+    print(f"ViT dim {cfg['dim']} depth {cfg['depth']} batch {batch}: end-to-end max error / max |logit| = {err:.2e}")
+    assert err < 4e-2

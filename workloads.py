@@ -1,5 +1,6 @@
 """Benchmark / test workloads built on the quantized modules: the int8
-static-quantized ResNet-50 of the benchmark configuration.
+static-quantized ResNet-50 and the dynamic-quantized ViT-B/16 of the benchmark
+configurations.
 
 Topology is torchvision-style ResNet-50 v1.5, as Lucid's zoo builds it
 (``lucid/models/vision/resnet/_model.py:109-210,255-299``): 7x7/2 stem,
@@ -180,3 +181,116 @@ def resnet50_conv_gmacs(batch: int, size: int = 224) -> float:
         total += out * out * cout * cin * k * k
     total += 2048 * 1000
     return batch * total / 1e9
+
+
+# ---------------------------------------------------------------- ViT-B/16, dynamic int8 Linears
+# Topology as Lucid's zoo builds it (``lucid/models/vision/vit/_model.py``): 16x16
+# patch convolution, class token + position table, pre-norm blocks (LayerNorm eps
+# 1e-6, packed qkv attention, 4x GELU MLP), final LayerNorm, class-token pooling,
+# Linear head.  Every ``nn.Linear`` goes through ``quantize_dynamic`` (W8A8: weights
+# per-output-channel symmetric qint8, activations per-tensor affine quint8 from the
+# runtime min / max); patch embedding, LayerNorm, attention, GELU and the residual
+# adds stay float32.
+VIT_B16 = dict(image=224, patch=16, dim=768, depth=12, heads=12, mlp=3072, classes=1000)
+
+
+def vit_float_params(cfg=VIT_B16, seed: int = 0) -> dict:
+    """Random N(0, 0.02) weights (biases too, so that every term is exercised),
+    LayerNorm at gamma = 1 + N(0, 0.02), beta = N(0, 0.02)."""
+    rng = np.random.default_rng(seed)
+    d, m = cfg["dim"], cfg["mlp"]
+    n = lambda *s: (rng.standard_normal(s) * 0.02).astype(np.float32)
+    tokens = (cfg["image"] // cfg["patch"]) ** 2 + 1
+    p = {"patch.weight": n(d, 3, cfg["patch"], cfg["patch"]), "patch.bias": n(d), "cls": n(d),
+         "pos": n(tokens, d), "norm.weight": 1 + n(d), "norm.bias": n(d),
+         "head.weight": n(cfg["classes"], d), "head.bias": n(cfg["classes"])}
+    for i in range(cfg["depth"]):
+        b = f"blocks.{i}."
+        p[b + "norm1.weight"], p[b + "norm1.bias"] = 1 + n(d), n(d)
+        p[b + "norm2.weight"], p[b + "norm2.bias"] = 1 + n(d), n(d)
+        p[b + "qkv.weight"], p[b + "qkv.bias"] = n(3 * d, d), n(3 * d)
+        p[b + "proj.weight"], p[b + "proj.bias"] = n(d, d), n(d)
+        p[b + "fc1.weight"], p[b + "fc1.bias"] = n(m, d), n(m)
+        p[b + "fc2.weight"], p[b + "fc2.bias"] = n(d, m), n(d)
+    return p
+
+
+def _float_linear(w, b):
+    lin = nn.Linear(w.shape[1], w.shape[0])
+    lin.register_buffer("weight", L.tensor(w))
+    lin.register_buffer("bias", L.tensor(b))
+    return lin
+
+
+def _layer_norm(w, b, eps=1e-6):
+    ln = nn.LayerNorm(w.shape[0], eps=eps)
+    ln.register_buffer("weight", L.tensor(w, device="hip"))
+    ln.register_buffer("bias", L.tensor(b, device="hip"))
+    return ln
+
+
+class ViTBlock(nn.Module):
+    def __init__(self, prefix, p, heads):
+        super().__init__()
+        self.heads = heads
+        self.norm1 = _layer_norm(p[prefix + "norm1.weight"], p[prefix + "norm1.bias"])
+        self.norm2 = _layer_norm(p[prefix + "norm2.weight"], p[prefix + "norm2.bias"])
+        self.qkv = _float_linear(p[prefix + "qkv.weight"], p[prefix + "qkv.bias"])
+        self.proj = _float_linear(p[prefix + "proj.weight"], p[prefix + "proj.bias"])
+        self.fc1 = _float_linear(p[prefix + "fc1.weight"], p[prefix + "fc1.bias"])
+        self.fc2 = _float_linear(p[prefix + "fc2.weight"], p[prefix + "fc2.bias"])
+
+    def forward(self, x):
+        import lucid_amd.nn.functional as F
+
+        a = F.scaled_dot_product_attention_qkv(self.qkv(self.norm1(x)), self.heads)
+        x = F.add(x, self.proj(a))
+        return F.add(x, self.fc2(F.gelu(self.fc1(self.norm2(x)))))
+
+
+class QViT(nn.Module):
+    """ViT for image classification with dynamic-quantized Linears; input float32
+    NCHW images on the hip device, output float32 logits."""
+
+    def __init__(self, cfg=VIT_B16, params=None, seed: int = 0):
+        super().__init__()
+        p = params if params is not None else vit_float_params(cfg, seed)
+        self.cfg = dict(cfg)
+        d = cfg["dim"]
+        self.register_buffer("patch_weight", L.tensor(p["patch.weight"].reshape(d, -1), device="hip"))
+        self.register_buffer("patch_bias", L.tensor(p["patch.bias"], device="hip"))
+        self.register_buffer("cls_token", L.tensor(p["cls"], device="hip"))
+        self.register_buffer("pos_embed", L.tensor(p["pos"], device="hip"))
+        self.blocks = nn.Sequential(*[ViTBlock(f"blocks.{i}.", p, cfg["heads"]) for i in range(cfg["depth"])])
+        self.norm = _layer_norm(p["norm.weight"], p["norm.bias"])
+        self.head = _float_linear(p["head.weight"], p["head.bias"])
+        Q.quantize_dynamic(self, inplace=True)
+
+    def forward(self, x):
+        from lucid_amd import _C
+        import lucid_amd.nn.functional as F
+
+        cfg = self.cfg
+        B, C, H, W = x.shape
+        ps, d = cfg["patch"], cfg["dim"]
+        n = (H // ps) * (W // ps)
+        rows = L.Tensor.empty((B * n, C * ps * ps), L.float32, "hip")
+        _C.call("lq_patchify_f32", x.data_ptr, rows.data_ptr, B, C, H, W, ps, None)
+        emb = F.linear_f32(rows, self.patch_weight, self.patch_bias)
+        tok = L.Tensor.empty((B, n + 1, d), L.float32, "hip")
+        _C.call("lq_assemble_tokens_f32", emb.data_ptr, self.cls_token.data_ptr, self.pos_embed.data_ptr,
+                tok.data_ptr, B, n + 1, d, None)
+        tok = self.norm(self.blocks(tok))
+        # class-token pooling: row 0 of every image
+        cls = L.Tensor.empty((B, d), L.float32, "hip")
+        for b in range(B):
+            _C.call("lq_d2d", cls.data_ptr + b * d * 4, tok.data_ptr + b * (n + 1) * d * 4, d * 4, None)
+        return self.head(cls)
+
+
+def vit_linear_gops(cfg=VIT_B16, batch: int = 1) -> float:
+    """int8 operations (2 per multiply-accumulate) of the quantized Linears, in 1e9."""
+    t = (cfg["image"] // cfg["patch"]) ** 2 + 1
+    d, m = cfg["dim"], cfg["mlp"]
+    per_block = 2.0 * t * (d * 3 * d + d * d + 2 * d * m)
+    return batch * (cfg["depth"] * per_block + 2.0 * d * cfg["classes"]) / 1e9
