@@ -174,19 +174,34 @@ int lq_add_requant_i8(const int8_t* qa, int a_offset, const float* a_scale, cons
 int lq_global_avgpool_nhwc_i8(const int8_t* q, int code_offset, int B, int H, int W, int C,
                               const float* scale, const float* zp, float* out, lq_stream stream);
 
+/* ------------------------------------------------- ranges kept by the producer */
+/* nnqd.Linear takes x.min() / x.max() of its input on every forward
+ * (lucid/nn/quantized/dynamic/linear.py:87-89): a full pass over a tensor some
+ * kernel has just written.  The float32 kernels below can keep that range as a
+ * by-product: pass them four 32-bit words initialised by lq_range_keys_init and
+ * they fold the min / max (and a NaN flag) of what they write into them with
+ * order-independent atomics.  lq_calc_qparams_from_keys then is
+ * calculate_qparams(min, max) on that range (_qparams.py:190-215), bit-identical
+ * to lq_minmax + lq_calc_qparams; mn_out / mx_out (optional) receive the range. */
+int lq_range_keys_init(uint32_t* keys, lq_stream stream);
+int lq_calc_qparams_from_keys(const uint32_t* keys, int symmetric, int qmin, int qmax, int is_signed,
+                              float eps, float* scale, float* zp, float* mn_out, float* mx_out,
+                              lq_stream stream);
+
 /* ------------------------------------------------- float32 steps of a ViT block */
 /* What Lucid's dynamic-quantized ViT keeps in float32 between its int8 Linears
  * (lucid/models/vision/vit/_model.py:132-161,202-204,275-278,449-458).  Tolerance
- * parity (1e-4 relative against a float32 CPU evaluation): summation orders differ. */
+ * parity (1e-4 relative against a float32 CPU evaluation): summation orders differ.
+ * range_keys, where present, may be null. */
 
 /* LayerNorm over the last axis of [rows, cols] (IBackend::layer_norm_forward;
  * lucid/_C/backend/cpu/Norm.cpp:35-65: mean, centred dot product / N,
  * rstd = 1/sqrt(var + eps), (c * rstd) * gamma + beta). */
 int lq_layernorm_f32(const float* x, const float* gamma, const float* beta, float* out, long rows, int cols,
-                     float eps, lq_stream stream);
+                     float eps, uint32_t* range_keys, lq_stream stream);
 
 /* GELU, exact erf form (lucid/nn/functional/activations.py:219, approximate="none"). */
-int lq_gelu_f32(const float* x, float* out, size_t n, lq_stream stream);
+int lq_gelu_f32(const float* x, float* out, size_t n, uint32_t* range_keys, lq_stream stream);
 
 /* out = a + b (IBackend::add on float32; the residual joins). */
 int lq_add_f32(const float* a, const float* b, float* out, size_t n, lq_stream stream);
@@ -196,7 +211,8 @@ int lq_add_f32(const float* a, const float* b, float* out, size_t n, lq_stream s
  * activation of the qkv Linear, [B, T, 3, H, D] (vit/_model.py:137-141), writing
  * [B, T, H*D] (vit/_model.py:158).  D must be 64 and T <= 208 (ViT-B/16: T = 197);
  * anything else returns LQ_ERR_NOT_IMPLEMENTED. */
-int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale, lq_stream stream);
+int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale,
+                     uint32_t* range_keys, lq_stream stream);
 
 /* Patch embedding, a convolution whose stride equals its kernel
  * (vit/_model.py:62-69), as im2col + GEMM: image [B,C,H,W] -> rows
@@ -208,6 +224,11 @@ int lq_patchify_f32(const float* img, float* out, int B, int C, int H, int W, in
  * bias may be null. */
 int lq_sgemm_nt_f32(const float* a, const float* w, const float* bias, float* out, int M, int N, int K,
                     lq_stream stream);
+
+/* dst[r, 0:cols] = src[r * src_row_stride + 0:cols]: strided row gather (class-token
+ * pooling x[:, 0], vit/_model.py `_pool`). */
+int lq_gather_rows_f32(const float* src, size_t src_row_stride, float* dst, size_t rows, size_t cols,
+                       lq_stream stream);
 
 /* tokens[b,0,:] = cls + pos[0], tokens[b,1+i,:] = patches[b,i,:] + pos[1+i]
  * (cat + position table, vit/_model.py:452-454); out is [B, T, D], patches [B, T-1, D]. */
@@ -243,6 +264,7 @@ int lq_rowsum_i8(const int8_t* w, int32_t* out, int N, int K, lq_stream stream);
  *     acc[m,n] = sum_k a[m,k] * w[n,k]                              (int32)
  *     y = f32(acc - a_zp*wsum[n]) * (a_scale[m|0] * w_scale[n]) + bias[n]
  *     y = relu(y) if relu
+ *     y = y + residual[m,n] if residual
  *     out = per out_mode
  * a: int8 [M,K] activation codes as stored (a quint8 code c is stored as
  * c - 128, and a_zp is then Z - 128); w: int8 [N,K].  All pointers are device
@@ -270,9 +292,15 @@ typedef struct {
     void* out;             /* [M, ldo] in the type out_mode implies          */
     long ldo;              /* output row stride in elements; 0 means N       */
     int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
-    int tile_config;       /* tuning: low byte 0 = choose, 1..6 = a tile shape;
+    int tile_config;       /* tuning: low byte 0 = choose, 1..7 = a tile shape;
                               next byte 0 = choose, 1 = one block per tile,
-                              2 = stream-K work split                         */
+                              2 = stream-K work split, 3 = stream-K over the
+                              leftover tiles of the last round only             */
+    const float* residual; /* optional float32 [M, ldr] added after the activation:
+                              out = act(y) + residual (x + linear(...), the
+                              residual joins of a transformer block,
+                              vit/_model.py:276-277); modes F32 / F16 only        */
+    long ldr;              /* residual row stride in elements; 0 means N     */
 } lq_qlinear_args;
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);

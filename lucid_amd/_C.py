@@ -114,6 +114,7 @@ class QLinearArgs(C.Structure):
         ("out_scale", _vp), ("out_zp", _vp),
         ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
         ("out", _vp), ("ldo", C.c_long), ("force_path", _i), ("tile_config", _i),
+        ("residual", _vp), ("ldr", C.c_long),
     ]
 
 
@@ -125,10 +126,13 @@ _SIGNATURES["lq_global_avgpool_nhwc_i8"] = [_vp, _i, _i, _i, _i, _i, _vp, _vp, _
 _SIGNATURES["lq_qlinear_w8a32"] = [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp,
                                    _vp]
 _l = C.c_long
-_SIGNATURES["lq_layernorm_f32"] = [_vp, _vp, _vp, _vp, _l, _i, _f, _vp]
-_SIGNATURES["lq_gelu_f32"] = [_vp, _vp, _sz, _vp]
+_SIGNATURES["lq_layernorm_f32"] = [_vp, _vp, _vp, _vp, _l, _i, _f, _vp, _vp]
+_SIGNATURES["lq_gelu_f32"] = [_vp, _vp, _sz, _vp, _vp]
 _SIGNATURES["lq_add_f32"] = [_vp, _vp, _vp, _sz, _vp]
-_SIGNATURES["lq_attention_f32"] = [_vp, _vp, _i, _i, _i, _i, _f, _vp]
+_SIGNATURES["lq_attention_f32"] = [_vp, _vp, _i, _i, _i, _i, _f, _vp, _vp]
+_SIGNATURES["lq_gather_rows_f32"] = [_vp, _sz, _vp, _sz, _sz, _vp]
+_SIGNATURES["lq_range_keys_init"] = [_vp, _vp]
+_SIGNATURES["lq_calc_qparams_from_keys"] = [_vp, _i, _i, _i, _i, _f, _vp, _vp, _vp, _vp, _vp]
 _SIGNATURES["lq_patchify_f32"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_sgemm_nt_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_assemble_tokens_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]

@@ -43,9 +43,11 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
                bias: Tensor | None = None, relu: bool = False, out_mode: int = OUT_F32,
                out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
                out_qmax: int = 255, out_offset: int = 0, path: int = PATH_AUTO,
-               tile_config: int = 0, out: Tensor | None = None, repeat: int = 1) -> Tensor:
+               tile_config: int = 0, out: Tensor | None = None, repeat: int = 1,
+               residual: Tensor | None = None) -> Tensor:
     """Fused int8 GEMM + epilogue; see ``lq_qlinear_i8`` in ``lucid_hip.h``.
-    ``a`` is int8 ``[M, K]``, ``w`` int8 ``[N, K]``; the result is ``[M, N]``."""
+    ``a`` is int8 ``[M, K]``, ``w`` int8 ``[N, K]``; the result is ``[M, N]``.
+    ``residual`` (float32, ``M*N`` elements) is added after the activation."""
     if a.ndim != 2 or w.ndim != 2 or a.shape[1] != w.shape[1]:
         raise _C.ShapeMismatch(f"qlinear_i8: a {a.shape} and w {w.shape} do not form a GEMM")
     M, K = a.shape
@@ -75,6 +77,9 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
     args.out_qmin, args.out_qmax, args.out_offset = int(out_qmin), int(out_qmax), int(out_offset)
     args.out, args.ldo, args.force_path = out.data_ptr, 0, int(path)
     args.tile_config = int(tile_config)
+    if residual is not None and residual.numel != M * N:
+        raise _C.ShapeMismatch(f"residual has {residual.numel} elements for an output of {M}x{N}")
+    args.residual, args.ldr = _ptr(residual, "residual", T.float32), 0
     if repeat == 1:
         _C.call("lq_qlinear_i8", C.byref(args), None)
     else:

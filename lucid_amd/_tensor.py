@@ -114,7 +114,7 @@ class Tensor:
     """Contiguous row-major tensor on ``"hip"`` (device memory) or ``"cpu"``
     (host staging)."""
 
-    __slots__ = ("shape", "dtype", "device", "_buf", "_host", "_offset", "_grid", "__weakref__")
+    __slots__ = ("shape", "dtype", "device", "_buf", "_host", "_offset", "_grid", "_range", "__weakref__")
 
     def __init__(self, shape, dt, device, buf=None, host=None, offset=0) -> None:
         self.shape = tuple(int(s) for s in shape)
@@ -124,6 +124,9 @@ class Tensor:
         self._host = host
         self._offset = int(offset)
         self._grid = None  # set by ops whose result lies on a quantization grid
+        # device min / max keys kept by the kernel that wrote this tensor
+        # (``lq_range_keys_init``), read by a dynamic quantizer downstream
+        self._range = None
 
     # -- construction
     @staticmethod

@@ -104,6 +104,15 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
     return __float_as_uint((qv - Z) * S);  // OUT_FAKEQUANT_F32
 }
 
+// y + residual[m, n] for the float output forms (x + linear(...), the residual
+// joins of a transformer block); the other forms ignore the operand.
+template <int MODE>
+__device__ __forceinline__ uint32_t add_residual(const GemmArgs& g, uint32_t bits, int m, int n) {
+    if ((MODE == OUT_F32 || MODE == OUT_F16) && g.residual)
+        return __float_as_uint(__uint_as_float(bits) + g.residual[size_t(m) * size_t(g.ldr) + size_t(n)]);
+    return bits;
+}
+
 template <int MODE>
 __device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint32_t v) {
     if (MODE == OUT_F16)
@@ -134,7 +143,7 @@ template <int MODE>
 __device__ __forceinline__ void epilogue_store_t(const GemmArgs& g, int m, int n, int32_t acc,
                                                  float as, const ColParams& c, float S, float Z) {
     store_scalar<MODE>(g, size_t(m) * size_t(g.ldo) + size_t(n),
-                       epilogue_value<MODE>(g, acc, as, c, S, Z));
+                       add_residual<MODE>(g, epilogue_value<MODE>(g, acc, as, c, S, Z), m, n));
 }
 
 __device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, int32_t acc,

@@ -344,7 +344,15 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
                        p->out_qmin, p->out_qmax, p->out_offset);
     }
 
-    GemmArgs g;
+    if (p->residual) {
+        LQ_REQUIRE(p->out_mode == OUT_F32 || p->out_mode == OUT_F16, LQ_ERR_VALUE,
+                   "qlinear_i8: a residual operand needs a float output mode");
+        LQ_REQUIRE((p->ldr ? p->ldr : p->N) >= p->N, LQ_ERR_SHAPE, "qlinear_i8: ldr %ld < N %d", p->ldr,
+                   p->N);
+    }
+
+    GemmArgs g{};
+    g.residual = p->residual; g.ldr = p->ldr ? p->ldr : p->N;
     g.a = p->a; g.w = p->w; g.M = p->M; g.N = p->N; g.K = p->K;
     g.wsum = p->wsum; g.a_zp = p->a_zp; g.a_zp_dev = p->a_zp_dev;
     g.a_scale = p->a_scale; g.a_scale_per_row = p->a_scale_per_row; g.w_scale = p->w_scale;

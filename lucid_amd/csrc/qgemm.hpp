@@ -25,6 +25,8 @@ struct GemmArgs {
     int out_qmin, out_qmax, out_offset;
     void* out;            // [M, ldo]
     long ldo;
+    const float* residual;  // optional [M, ldr] float32 added to y after the activation (float outputs only)
+    long ldr;
     const int8_t* zeros;  // >= 16 zero bytes, source for K-tail chunks
     // Implicit-GEMM convolution (tile kernel instantiated with CONV = true): the
     // A operand is gathered from NHWC activation codes; row m is output pixel

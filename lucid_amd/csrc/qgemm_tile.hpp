@@ -136,6 +136,21 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                     v[p] = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
                 size_t idx = size_t(m_first) * size_t(g.ldo) + size_t(n);
                 const size_t step = size_t(ROWS_PER_PASS) * size_t(g.ldo);
+                if ((MODE == OUT_F32 || MODE == OUT_F16) && g.residual) {
+                    // `interior` also vouches for the residual's alignment
+                    const float* rp = g.residual + size_t(m_first) * size_t(g.ldr) + size_t(n);
+                    float4 rv[PASSES];
+#pragma unroll
+                    for (int p = 0; p < PASSES; ++p)
+                        rv[p] = *reinterpret_cast<const float4*>(rp + size_t(p) * ROWS_PER_PASS * size_t(g.ldr));
+#pragma unroll
+                    for (int p = 0; p < PASSES; ++p) {
+                        v[p].x = __float_as_uint(__uint_as_float(v[p].x) + rv[p].x);
+                        v[p].y = __float_as_uint(__uint_as_float(v[p].y) + rv[p].y);
+                        v[p].z = __float_as_uint(__uint_as_float(v[p].z) + rv[p].z);
+                        v[p].w = __float_as_uint(__uint_as_float(v[p].w) + rv[p].w);
+                    }
+                }
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
                     store_vec4<MODE>(g, idx, v[p]);
@@ -144,9 +159,13 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
             } else {
 #pragma unroll 4
                 for (int p = 0; p < PASSES; ++p) {
-                    const uint4 v = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
+                    uint4 v = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
                     const int m = m_first + p * ROWS_PER_PASS;
                     if (m < g.M && n < n_limit) {
+                        v.x = add_residual<MODE>(g, v.x, m, n);
+                        if (n + 1 < n_limit) v.y = add_residual<MODE>(g, v.y, m, n + 1);
+                        if (n + 2 < n_limit) v.z = add_residual<MODE>(g, v.z, m, n + 2);
+                        if (n + 3 < n_limit) v.w = add_residual<MODE>(g, v.w, m, n + 3);
                         const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
                         if (vec_ok && n + 4 <= n_limit) {
                             store_vec4<MODE>(g, idx, v);
@@ -453,7 +472,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         }
         const int esize = MODE == OUT_F16 ? 2 : (MODE == OUT_REQUANT_I8 ? 1 : 4);
         const bool interior = m0 + BM <= g.M && n0 + BN <= n_limit && g.ldo % 4 == 0 &&
-                              reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0;
+                              reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0 &&
+                              (g.residual == nullptr ||
+                               (g.ldr % 4 == 0 && reinterpret_cast<uintptr_t>(g.residual) % 16 == 0));
         __syncthreads();
         tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z, interior);
         __syncthreads();  // the staging area is the next tile's first LDS stage

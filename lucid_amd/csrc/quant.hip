@@ -5,6 +5,7 @@
 // (lucid/quantization/_functional.py:180, 281, 311-313): IEEE division,
 // round-half-even, add zero point, clamp, cast.  No reciprocal, no FMA.
 #include "common.hpp"
+#include "range_keys.hpp"
 
 using namespace lq;
 
@@ -420,30 +421,36 @@ __global__ __launch_bounds__(kThreads) void minmax_col_kernel(const float* __res
     mm_write(m, pmin, pmax, size_t(sp) * cols + col);
 }
 
-// Folds partials [groups][C][inner_cols] into mn[C], mx[C]; one wavefront
-// per channel.
-__global__ __launch_bounds__(64) void minmax_finalize_kernel(const float* __restrict__ pmin,
-                                                             const float* __restrict__ pmax,
-                                                             size_t C, unsigned groups,
-                                                             unsigned inner_cols, float* mn,
-                                                             float* mx) {
+// Folds partials [groups][C][inner_cols] into mn[C], mx[C]; one block per
+// channel, four independent loads per thread in flight.
+__global__ __launch_bounds__(256) void minmax_finalize_kernel(const float* __restrict__ pmin,
+                                                              const float* __restrict__ pmax,
+                                                              size_t C, unsigned groups,
+                                                              unsigned inner_cols, float* mn,
+                                                              float* mx) {
     const size_t c = blockIdx.x;
     MinMax m{__builtin_inff(), -__builtin_inff(), 0};
     const size_t per_c = size_t(groups) * inner_cols;
-    for (size_t t = threadIdx.x; t < per_c; t += 64) {
-        const size_t g = t / inner_cols, i = t - g * inner_cols;
-        const size_t idx = (g * C + c) * inner_cols + i;
-        float a = pmin[idx], b = pmax[idx];
-        m.nan |= (a != a) | (b != b);
-        m.lo = fminf(m.lo, a);
-        m.hi = fmaxf(m.hi, b);
-    }
+    for (size_t t0 = threadIdx.x; t0 < per_c; t0 += 4 * 256) {
+        float a[4], b[4];
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-        m.lo = fminf(m.lo, __shfl_xor(m.lo, d, 64));
-        m.hi = fmaxf(m.hi, __shfl_xor(m.hi, d, 64));
-        m.nan |= __shfl_xor(m.nan, d, 64);
+        for (int u = 0; u < 4; ++u) {
+            const size_t t = t0 + size_t(u) * 256;
+            a[u] = __builtin_inff(), b[u] = -__builtin_inff();
+            if (t < per_c) {
+                const size_t g = t / inner_cols, i = t - g * inner_cols;
+                const size_t idx = (g * C + c) * inner_cols + i;
+                a[u] = pmin[idx], b[u] = pmax[idx];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            m.nan |= (a[u] != a[u]) | (b[u] != b[u]);
+            m.lo = fminf(m.lo, a[u]);
+            m.hi = fmaxf(m.hi, b[u]);
+        }
     }
+    m = mm_block_reduce(m);
     if (threadIdx.x == 0) mm_write(m, mn, mx, c);
 }
 
@@ -467,25 +474,50 @@ __device__ __forceinline__ float vminf(float a, float b) {
 }
 
 // lucid/quantization/_qparams.py:198-215, float32 throughout.
-__global__ void calc_qparams_kernel(const float* __restrict__ mn, const float* __restrict__ mx,
-                                    size_t C, int symmetric, int qmin, int qmax, int is_signed,
-                                    float eps, float half_range, float* scale, float* zp) {
-    size_t c = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (c >= C) return;
-    float lo = vminf(mn[c], 0.0f);
-    float hi = vmaxf(mx[c], 0.0f);
+__device__ __forceinline__ void qparams_of(float mn, float mx, int symmetric, int qmin, int qmax,
+                                           int is_signed, float eps, float half_range, float* scale,
+                                           float* zp) {
+    float lo = vminf(mn, 0.0f);
+    float hi = vmaxf(mx, 0.0f);
     if (symmetric) {
         float max_abs = vmaxf(fabsf(lo), fabsf(hi));
-        scale[c] = vmaxf(max_abs / half_range, eps);
-        zp[c] = is_signed ? 0.0f : float((qmax + qmin + 1) >> 1);
+        *scale = vmaxf(max_abs / half_range, eps);
+        *zp = is_signed ? 0.0f : float((qmax + qmin + 1) >> 1);
     } else {
         float s = vmaxf((hi - lo) / float(qmax - qmin), eps);
         float z = float(qmin) - __builtin_rintf(lo / s);
         float qlo = float(qmin), qhi = float(qmax);
         z = (z < qlo) ? qlo : ((z > qhi) ? qhi : z);
-        scale[c] = s;
-        zp[c] = z;
+        *scale = s;
+        *zp = z;
     }
+}
+
+__global__ void calc_qparams_kernel(const float* __restrict__ mn, const float* __restrict__ mx,
+                                    size_t C, int symmetric, int qmin, int qmax, int is_signed,
+                                    float eps, float half_range, float* scale, float* zp) {
+    size_t c = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    qparams_of(mn[c], mx[c], symmetric, qmin, qmax, is_signed, eps, half_range, &scale[c], &zp[c]);
+}
+
+__global__ void range_keys_init_kernel(uint32_t* keys) {
+    keys[0] = kRangeMinIdentity;
+    keys[1] = kRangeMaxIdentity;
+    keys[2] = 0;
+    keys[3] = 0;
+}
+
+// Per-tensor qparams from a range kept by the producing kernel; also writes
+// the range itself when asked.
+__global__ void calc_qparams_from_keys_kernel(const uint32_t* __restrict__ keys, int symmetric, int qmin,
+                                              int qmax, int is_signed, float eps, float half_range,
+                                              float* scale, float* zp, float* mn_out, float* mx_out) {
+    float mn = range_unkey(keys[0]), mx = range_unkey(keys[1]);
+    if (keys[2]) mn = mx = __builtin_nanf("");
+    if (mn_out) *mn_out = mn;
+    if (mx_out) *mx_out = mx;
+    qparams_of(mn, mx, symmetric, qmin, qmax, is_signed, eps, half_range, scale, zp);
 }
 
 }  // namespace
@@ -523,7 +555,7 @@ int lq_minmax(const float* x, size_t outer, size_t C, size_t inner, float* mn, f
         hipLaunchKernelGGL(minmax_col_kernel, dim3(unsigned(col_blocks), unsigned(splits)),
                            dim3(kThreads), 0, st, x, outer, cols, unsigned(splits), pmin, pmax);
         LQ_CHECK_LAUNCH("minmax_col");
-        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(64), 0, st, pmin, pmax, C,
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(256), 0, st, pmin, pmax, C,
                            unsigned(splits), unsigned(inner), mn, mx);
         LQ_CHECK_LAUNCH("minmax_finalize");
         return LQ_OK;
@@ -555,7 +587,7 @@ int lq_minmax(const float* x, size_t outer, size_t C, size_t inner, float* mn, f
                            unsigned(splits), pmin, pmax);
     LQ_CHECK_LAUNCH("minmax_seg");
     if (splits > 1) {
-        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(64), 0, st, pmin, pmax, C,
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(256), 0, st, pmin, pmax, C,
                            unsigned(splits), 1u, mn, mx);
         LQ_CHECK_LAUNCH("minmax_finalize");
     }
@@ -573,6 +605,25 @@ int lq_calc_qparams(const float* mn, const float* mx, size_t C, int symmetric, i
                        as_stream(stream), mn, mx, C, symmetric, qmin, qmax, is_signed, eps, half_range,
                        scale, zp);
     LQ_CHECK_LAUNCH("calc_qparams");
+    return LQ_OK;
+}
+
+int lq_range_keys_init(uint32_t* keys, lq_stream stream) {
+    LQ_REQUIRE(keys, LQ_ERR_VALUE, "range_keys_init: NULL pointer");
+    hipLaunchKernelGGL(range_keys_init_kernel, dim3(1), dim3(1), 0, as_stream(stream), keys);
+    LQ_CHECK_LAUNCH("range_keys_init");
+    return LQ_OK;
+}
+
+int lq_calc_qparams_from_keys(const uint32_t* keys, int symmetric, int qmin, int qmax, int is_signed,
+                              float eps, float* scale, float* zp, float* mn_out, float* mx_out,
+                              lq_stream stream) {
+    LQ_REQUIRE(keys && scale && zp, LQ_ERR_VALUE, "calc_qparams_from_keys: NULL pointer");
+    LQ_REQUIRE(qmax > qmin, LQ_ERR_VALUE, "calc_qparams_from_keys: empty grid [%d,%d]", qmin, qmax);
+    const float half_range = float((double(qmax) - double(qmin)) / 2.0);
+    hipLaunchKernelGGL(calc_qparams_from_keys_kernel, dim3(1), dim3(1), 0, as_stream(stream), keys,
+                       symmetric, qmin, qmax, is_signed, eps, half_range, scale, zp, mn_out, mx_out);
+    LQ_CHECK_LAUNCH("calc_qparams_from_keys");
     return LQ_OK;
 }
 

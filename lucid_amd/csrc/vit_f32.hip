@@ -15,6 +15,7 @@
 // Matrix products use the float32 MFMA instructions; results agree with a CPU
 // float32 evaluation to rounding-order differences (tested to 1e-4 relative).
 #include "common.hpp"
+#include "range_keys.hpp"
 
 using namespace lq;
 
@@ -33,58 +34,75 @@ __device__ __forceinline__ float wave_sum(float v) {
 // One wavefront per row; the row (a few KiB) is re-read from cache for the
 // variance and the output pass.  mean, centred values, var = dot(c,c)/N,
 // rstd = 1/sqrt(var+eps), y = (c*rstd)*gamma + beta: the reference's steps.
+constexpr int LN_ROWS_PER_WAVE = 4;
+
 __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x,
                                                         const float* __restrict__ gamma,
                                                         const float* __restrict__ beta,
                                                         float* __restrict__ out, long rows, int cols,
-                                                        float eps) {
+                                                        float eps, uint32_t* range_keys) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const long row = long(blockIdx.x) * 4 + wave;
-    if (row >= rows) return;
-    const float* xr = x + row * cols;
-    float* yr = out + row * cols;
     const bool vec = (cols % 4 == 0) && aligned16(x) && aligned16(out) && aligned16(gamma) && aligned16(beta);
     const float inv_n = 1.0f / float(cols);
-    float s = 0.0f;
-    if (vec) {
-        for (int c = lane * 4; c < cols; c += 256) {
-            const float4 v = *reinterpret_cast<const float4*>(xr + c);
-            s += (v.x + v.y) + (v.z + v.w);
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    int nan = 0;
+    auto track = [&](float y) {
+        nan |= (y != y);
+        lo = fminf(lo, y);
+        hi = fmaxf(hi, y);
+    };
+    for (int rr = 0; rr < LN_ROWS_PER_WAVE; ++rr) {
+        const long row = (long(blockIdx.x) * 4 + wave) * LN_ROWS_PER_WAVE + rr;
+        if (row >= rows) break;
+        const float* xr = x + row * cols;
+        float* yr = out + row * cols;
+        float s = 0.0f;
+        if (vec) {
+            for (int c = lane * 4; c < cols; c += 256) {
+                const float4 v = *reinterpret_cast<const float4*>(xr + c);
+                s += (v.x + v.y) + (v.z + v.w);
+            }
+        } else {
+            for (int c = lane; c < cols; c += 64) s += xr[c];
         }
-    } else {
-        for (int c = lane; c < cols; c += 64) s += xr[c];
+        const float mean = wave_sum(s) * inv_n;
+        float q = 0.0f;
+        if (vec) {
+            for (int c = lane * 4; c < cols; c += 256) {
+                const float4 v = *reinterpret_cast<const float4*>(xr + c);
+                const float a = v.x - mean, b = v.y - mean, cc = v.z - mean, d = v.w - mean;
+                q += (a * a + b * b) + (cc * cc + d * d);
+            }
+        } else {
+            for (int c = lane; c < cols; c += 64) {
+                const float a = xr[c] - mean;
+                q += a * a;
+            }
+        }
+        const float var = wave_sum(q) * inv_n;
+        const float rstd = 1.0f / sqrtf(var + eps);
+        if (vec) {
+            for (int c = lane * 4; c < cols; c += 256) {
+                const float4 v = *reinterpret_cast<const float4*>(xr + c);
+                const float4 g = *reinterpret_cast<const float4*>(gamma + c);
+                const float4 b = *reinterpret_cast<const float4*>(beta + c);
+                float4 y;
+                y.x = ((v.x - mean) * rstd) * g.x + b.x;
+                y.y = ((v.y - mean) * rstd) * g.y + b.y;
+                y.z = ((v.z - mean) * rstd) * g.z + b.z;
+                y.w = ((v.w - mean) * rstd) * g.w + b.w;
+                *reinterpret_cast<float4*>(yr + c) = y;
+                track(y.x), track(y.y), track(y.z), track(y.w);
+            }
+        } else {
+            for (int c = lane; c < cols; c += 64) {
+                const float y = ((xr[c] - mean) * rstd) * gamma[c] + beta[c];
+                yr[c] = y;
+                track(y);
+            }
+        }
     }
-    const float mean = wave_sum(s) * inv_n;
-    float q = 0.0f;
-    if (vec) {
-        for (int c = lane * 4; c < cols; c += 256) {
-            const float4 v = *reinterpret_cast<const float4*>(xr + c);
-            const float a = v.x - mean, b = v.y - mean, cc = v.z - mean, d = v.w - mean;
-            q += (a * a + b * b) + (cc * cc + d * d);
-        }
-    } else {
-        for (int c = lane; c < cols; c += 64) {
-            const float a = xr[c] - mean;
-            q += a * a;
-        }
-    }
-    const float var = wave_sum(q) * inv_n;
-    const float rstd = 1.0f / sqrtf(var + eps);
-    if (vec) {
-        for (int c = lane * 4; c < cols; c += 256) {
-            const float4 v = *reinterpret_cast<const float4*>(xr + c);
-            const float4 g = *reinterpret_cast<const float4*>(gamma + c);
-            const float4 b = *reinterpret_cast<const float4*>(beta + c);
-            float4 y;
-            y.x = ((v.x - mean) * rstd) * g.x + b.x;
-            y.y = ((v.y - mean) * rstd) * g.y + b.y;
-            y.z = ((v.z - mean) * rstd) * g.z + b.z;
-            y.w = ((v.w - mean) * rstd) * g.w + b.w;
-            *reinterpret_cast<float4*>(yr + c) = y;
-        }
-    } else {
-        for (int c = lane; c < cols; c += 64) yr[c] = ((xr[c] - mean) * rstd) * gamma[c] + beta[c];
-    }
+    if (range_keys) range_block_update(range_keys, lo, hi, nan);
 }
 
 // ---------------------------------------------------------------- elementwise
@@ -92,17 +110,42 @@ __device__ __forceinline__ float gelu_erf(float x) {
     return (0.5f * x) * (1.0f + erff(x * 0.70710678118654752440f));
 }
 
+// Grid-stride (a bounded number of blocks) so that the optional range
+// tracking costs a few thousand atomics at most.
 __global__ __launch_bounds__(256) void gelu_kernel(const float* __restrict__ x, float* __restrict__ out,
-                                                   size_t n, int vec) {
-    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+                                                   size_t n, int vec, uint32_t* range_keys) {
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    int nan = 0;
+    auto track = [&](float y) {
+        nan |= (y != y);
+        lo = fminf(lo, y);
+        hi = fmaxf(hi, y);
+    };
+    const size_t stride = size_t(gridDim.x) * 256;
     if (vec) {
-        if (i * 4 >= n) return;
-        const float4 v = reinterpret_cast<const float4*>(x)[i];
-        float4 y = {gelu_erf(v.x), gelu_erf(v.y), gelu_erf(v.z), gelu_erf(v.w)};
-        reinterpret_cast<float4*>(out)[i] = y;
-    } else if (i < n) {
-        out[i] = gelu_erf(x[i]);
+        for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i * 4 < n; i += stride) {
+            const float4 v = reinterpret_cast<const float4*>(x)[i];
+            float4 y = {gelu_erf(v.x), gelu_erf(v.y), gelu_erf(v.z), gelu_erf(v.w)};
+            reinterpret_cast<float4*>(out)[i] = y;
+            track(y.x), track(y.y), track(y.z), track(y.w);
+        }
+    } else {
+        for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+            const float y = gelu_erf(x[i]);
+            out[i] = y;
+            track(y);
+        }
     }
+    if (range_keys) range_block_update(range_keys, lo, hi, nan);
+}
+
+// dst[r, :] = src[r * src_row_stride : r * src_row_stride + cols]
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float* __restrict__ src, size_t src_row_stride,
+                                                          float* __restrict__ dst, size_t rows, size_t cols) {
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= rows * cols) return;
+    const size_t r = i / cols, c = i - r * cols;
+    dst[i] = src[r * src_row_stride + c];
 }
 
 __global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
@@ -272,7 +315,7 @@ __global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__
 constexpr int AT_D = 64, AT_TMAX = 208, AT_LD = AT_D + 4;  // row stride 68: 4*row + k hits all 64 banks
 
 __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict__ qkv, float* __restrict__ out,
-                                                        int B, int T, int H, float scale) {
+                                                        int B, int T, int H, float scale, uint32_t* range_keys) {
     extern __shared__ __attribute__((aligned(16))) float at_smem[];
     float (*sk)[AT_LD] = reinterpret_cast<float (*)[AT_LD]>(at_smem);
     float (*sv)[AT_LD] = reinterpret_cast<float (*)[AT_LD]>(at_smem + AT_TMAX * AT_LD);
@@ -294,8 +337,8 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
         *reinterpret_cast<float4*>(&sv[row][c4]) = vv;
     }
     __syncthreads();
-    const int q0 = wave * 16;
-    if (q0 >= T || wave >= nwaves) return;  // no barrier below this line
+    const int q0 = wave * 16;  // the launch has exactly ceil(T / 16) wavefronts, so q0 < T
+    (void)nwaves;
     const int g = lane >> 4, c = lane & 15;
     // B operand of S^T: Q[q0 + c][4*s + g], pre-scaled so that S = scale * Q.K^T
     float qf[AT_D / 4];
@@ -360,6 +403,20 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
             const int q = q0 + 4 * g + r;
             if (q < T) out[(size_t(b) * T + q) * (size_t(H) * AT_D) + size_t(h) * AT_D + 16 * j + c] = o[j][r];
         }
+    if (range_keys) {
+        float lo = __builtin_inff(), hi = -__builtin_inff();
+        int nan = 0;
+#pragma unroll
+        for (int j = 0; j < AT_D / 16; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (q0 + 4 * g + r < T) {
+                    nan |= (o[j][r] != o[j][r]);
+                    lo = fminf(lo, o[j][r]);
+                    hi = fmaxf(hi, o[j][r]);
+                }
+        range_block_update(range_keys, lo, hi, nan);
+    }
 }
 
 unsigned blocks_for(size_t n) { return unsigned((n + 255) / 256); }
@@ -369,21 +426,25 @@ unsigned blocks_for(size_t n) { return unsigned((n + 255) / 256); }
 extern "C" {
 
 int lq_layernorm_f32(const float* x, const float* gamma, const float* beta, float* out, long rows, int cols,
-                     float eps, void* stream) {
+                     float eps, uint32_t* range_keys, void* stream) {
     LQ_REQUIRE(x && gamma && beta && out, LQ_ERR_VALUE, "layernorm: null pointer");
     LQ_REQUIRE(rows >= 0 && cols > 0, LQ_ERR_SHAPE, "layernorm: bad shape (%ld, %d)", rows, cols);
     if (rows == 0) return LQ_OK;
-    LQ_REQUIRE((rows + 3) / 4 < 0x7fffffffL, LQ_ERR_SHAPE, "layernorm: too many rows");
-    layernorm_kernel<<<unsigned((rows + 3) / 4), 256, 0, as_stream(stream)>>>(x, gamma, beta, out, rows, cols, eps);
+    const long per_block = 4L * LN_ROWS_PER_WAVE;
+    LQ_REQUIRE((rows + per_block - 1) / per_block < 0x7fffffffL, LQ_ERR_SHAPE, "layernorm: too many rows");
+    layernorm_kernel<<<unsigned((rows + per_block - 1) / per_block), 256, 0, as_stream(stream)>>>(
+        x, gamma, beta, out, rows, cols, eps, range_keys);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }
 
-int lq_gelu_f32(const float* x, float* out, size_t n, void* stream) {
+int lq_gelu_f32(const float* x, float* out, size_t n, uint32_t* range_keys, void* stream) {
     LQ_REQUIRE(x && out, LQ_ERR_VALUE, "gelu: null pointer");
     if (n == 0) return LQ_OK;
     const int vec = (n % 4 == 0) && aligned16(x) && aligned16(out);
-    gelu_kernel<<<blocks_for(vec ? n / 4 : n), 256, 0, as_stream(stream)>>>(x, out, n, vec);
+    unsigned blocks = blocks_for(vec ? n / 4 : n);
+    if (blocks > 8192) blocks = 8192;
+    gelu_kernel<<<blocks, 256, 0, as_stream(stream)>>>(x, out, n, vec, range_keys);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }
@@ -431,7 +492,18 @@ int lq_sgemm_nt_f32(const float* a, const float* w, const float* bias, float* ou
     return LQ_OK;
 }
 
-int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale, void* stream) {
+int lq_gather_rows_f32(const float* src, size_t src_row_stride, float* dst, size_t rows, size_t cols,
+                       void* stream) {
+    LQ_REQUIRE(src && dst, LQ_ERR_VALUE, "gather_rows: null pointer");
+    LQ_REQUIRE(src_row_stride >= cols, LQ_ERR_SHAPE, "gather_rows: row stride smaller than the row");
+    if (rows * cols == 0) return LQ_OK;
+    gather_rows_kernel<<<blocks_for(rows * cols), 256, 0, as_stream(stream)>>>(src, src_row_stride, dst, rows, cols);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale, uint32_t* range_keys,
+                     void* stream) {
     LQ_REQUIRE(qkv && out, LQ_ERR_VALUE, "attention: null pointer");
     LQ_REQUIRE(B >= 0 && T >= 1 && H >= 1, LQ_ERR_SHAPE, "attention: bad shape");
     LQ_REQUIRE(D == AT_D && T <= AT_TMAX, LQ_ERR_NOT_IMPLEMENTED,
@@ -446,7 +518,8 @@ int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, f
                                    hipFuncAttributeMaxDynamicSharedMemorySize, int(kSmem)));
         attr_set = true;
     }
-    attention_kernel<<<unsigned(B) * H, waves * 64, kSmem, as_stream(stream)>>>(qkv, out, B, T, H, scale);
+    attention_kernel<<<unsigned(B) * H, waves * 64, kSmem, as_stream(stream)>>>(qkv, out, B, T, H, scale,
+                                                                                 range_keys);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }

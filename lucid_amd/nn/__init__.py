@@ -188,16 +188,17 @@ from . import intrinsic, quantized, utils  # noqa: E402  (sub-packages need the 
 class LayerNorm(Module):
     """``nn.LayerNorm`` over the last axis, float32, one HIP kernel."""
 
-    def __init__(self, normalized_shape: int, eps: float = 1e-5) -> None:
+    def __init__(self, normalized_shape: int, eps: float = 1e-5, track_range: bool = False) -> None:
         super().__init__()
         self.normalized_shape, self.eps = int(normalized_shape), float(eps)
+        self.track_range = track_range  # keep min / max of the output for a dynamic quantizer
         self.register_buffer("weight", T.tensor(np.ones(normalized_shape, np.float32)))
         self.register_buffer("bias", T.tensor(np.zeros(normalized_shape, np.float32)))
 
     def forward(self, x):
         from . import functional as F
 
-        return F.layer_norm(x, self.normalized_shape, self.weight, self.bias, self.eps)
+        return F.layer_norm(x, self.normalized_shape, self.weight, self.bias, self.eps, self.track_range)
 
 
 class GELU(Module):

@@ -21,25 +21,40 @@ def _require_f32_hip(name: str, *ts: Tensor) -> None:
             raise _C.DtypeMismatch(f"{name} expects float32, got {t.dtype}")
 
 
-def layer_norm(x: Tensor, normalized_shape, weight: Tensor, bias: Tensor, eps: float = 1e-5) -> Tensor:
-    """``F.layer_norm`` over the last axis (``lucid/_C/backend/cpu/Norm.cpp:35-65``)."""
+def _new_range() -> Tensor:
+    """Four device words holding a running (min, max, NaN flag) for the tensor a
+    kernel is about to write."""
+    keys = Tensor.empty((4,), T.int32, "hip")
+    _C.call("lq_range_keys_init", keys.data_ptr, None)
+    return keys
+
+
+def layer_norm(x: Tensor, normalized_shape, weight: Tensor, bias: Tensor, eps: float = 1e-5,
+               track_range: bool = False) -> Tensor:
+    """``F.layer_norm`` over the last axis (``lucid/_C/backend/cpu/Norm.cpp:35-65``).
+    ``track_range`` makes the kernel keep the min / max of its output, which a
+    dynamic-quantized Linear fed with the result then uses instead of a pass of
+    its own (same for ``gelu`` and the attention below)."""
     _require_f32_hip("layer_norm", x, weight, bias)
     cols = normalized_shape if isinstance(normalized_shape, int) else int(normalized_shape[-1])
     if x.shape[-1] != cols or weight.numel != cols or bias.numel != cols:
         raise _C.ShapeMismatch(f"layer_norm: last dim {x.shape[-1]} vs normalized_shape {cols}")
     out = Tensor.empty(x.shape, T.float32, "hip")
+    out._range = _new_range() if track_range else None
     _C.call("lq_layernorm_f32", x.data_ptr, weight.data_ptr, bias.data_ptr, out.data_ptr,
-            x.numel // cols, cols, float(eps), None)
+            x.numel // cols, cols, float(eps), out._range.data_ptr if track_range else None, None)
     return out
 
 
-def gelu(x: Tensor, approximate: str = "none") -> Tensor:
+def gelu(x: Tensor, approximate: str = "none", track_range: bool = False) -> Tensor:
     """``F.gelu`` (``lucid/nn/functional/activations.py:219``), exact erf form."""
     if approximate != "none":
         raise NotImplementedError("gelu: only approximate='none' is built")
     _require_f32_hip("gelu", x)
     out = Tensor.empty(x.shape, T.float32, "hip")
-    _C.call("lq_gelu_f32", x.data_ptr, out.data_ptr, x.numel, None)
+    out._range = _new_range() if track_range else None
+    _C.call("lq_gelu_f32", x.data_ptr, out.data_ptr, x.numel, out._range.data_ptr if track_range else None,
+            None)
     return out
 
 
@@ -52,7 +67,8 @@ def add(a: Tensor, b: Tensor) -> Tensor:
     return out
 
 
-def scaled_dot_product_attention_qkv(qkv: Tensor, num_heads: int, scale: float | None = None) -> Tensor:
+def scaled_dot_product_attention_qkv(qkv: Tensor, num_heads: int, scale: float | None = None,
+                                     track_range: bool = False) -> Tensor:
     """``F.scaled_dot_product_attention(q, k, v)`` on the packed output of a qkv
     Linear: ``qkv`` is ``(B, T, 3*H*D)`` laid out ``(B, T, 3, H, D)`` as in
     ``lucid/models/vision/vit/_model.py:137-141``; returns ``(B, T, H*D)``, the
@@ -64,7 +80,9 @@ def scaled_dot_product_attention_qkv(qkv: Tensor, num_heads: int, scale: float |
     D = C3 // (3 * num_heads)
     s = 1.0 / math.sqrt(D) if scale is None else float(scale)
     out = Tensor.empty((B, Tn, num_heads * D), T.float32, "hip")
-    _C.call("lq_attention_f32", qkv.data_ptr, out.data_ptr, B, Tn, num_heads, D, s, None)
+    out._range = _new_range() if track_range else None
+    _C.call("lq_attention_f32", qkv.data_ptr, out.data_ptr, B, Tn, num_heads, D, s,
+            out._range.data_ptr if track_range else None, None)
     return out
 
 

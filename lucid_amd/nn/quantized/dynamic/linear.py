@@ -45,7 +45,9 @@ class Linear(Module):
         if name == "weight_zero_point":
             require_symmetric_weight(self.weight_zero_point, "dynamic.Linear")
 
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, residual: Tensor | None = None) -> Tensor:
+        """``residual`` (optional, not in Lucid's signature) is added to the
+        output inside the GEMM epilogue: ``x_res + linear(x)`` in one kernel."""
         if not isinstance(x, Tensor) or x.device != "hip":
             raise _C.DeviceMismatch("dynamic.Linear: input must be a tensor on the 'hip' device")
         if x.dtype != T.float32:
@@ -55,8 +57,15 @@ class Linear(Module):
             raise _C.ShapeMismatch(f"expected last dim {K}, got {x.shape}")
         M = x.numel // K
         qd = self.act_qdtype
-        mn, mx = minmax(x)
-        x_scale, x_zp = calculate_qparams(mn, mx, per_tensor_affine, qd)
+        if x._range is not None:
+            # the kernel that wrote x kept its min / max: qparams straight from them
+            x_scale = Tensor.empty((), T.float32, "hip")
+            x_zp = Tensor.empty((), T.float32, "hip")
+            _C.call("lq_calc_qparams_from_keys", x._range.data_ptr, 0, qd.quant_min, qd.quant_max,
+                    int(qd.signed), 1e-8, x_scale.data_ptr, x_zp.data_ptr, None, None, None)
+        else:
+            mn, mx = minmax(x)
+            x_scale, x_zp = calculate_qparams(mn, mx, per_tensor_affine, qd)
         off = storage_offset(qd)
         xq = Tensor.empty((M, K), T.int8, "hip")
         _C.call("lq_quantize", x.data_ptr, xq.data_ptr, _C.I8, off, 1, 1, x.numel,
@@ -65,7 +74,7 @@ class Linear(Module):
             self._wsum = _ops.rowsum_i8(self.weight_int8)
         y = _ops.qlinear_i8(xq, self.weight_int8, a_zp=off, a_zp_dev=x_zp, a_scale=x_scale,
                             w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias,
-                            out_mode=_ops.OUT_F32)
+                            out_mode=_ops.OUT_F32, residual=residual)
         return y.reshape(*x.shape[:-1], N)
 
     @classmethod

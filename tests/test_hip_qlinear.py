@@ -219,3 +219,30 @@ def test_argument_validation():
     with pytest.raises(ValueError):       # MFMA path on K % 16 != 0
         _ops.qlinear_i8(hip(np.zeros((4, 30), np.int8)), hip(np.zeros((8, 30), np.int8)),
                         out_mode=0, path=TILE)
+
+
+@pytest.mark.parametrize("M,N,K,path", [(394, 768, 768, TILE), (300, 260, 144, TILE), (129, 77, 784, TILE),
+                                        (16, 256, 64, SKINNY), (9, 10, 7, NAIVE), (2048, 512, 256, TILE)])
+@pytest.mark.parametrize("mode", [_ops.OUT_F32, _ops.OUT_F16])
+def test_residual_joins_in_the_epilogue(M, N, K, path, mode):
+    """out = (acc * scales + bias) + residual, float32 add, then the store's
+    narrowing: x + linear(...) of a transformer block in one kernel."""
+    rng = np.random.default_rng(M + N + K + mode)
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    a_scale = rng.uniform(0.005, 0.05, M).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    got = _ops.qlinear_i8(hip(a), hip(w), a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias),
+                          out_mode=mode, path=path, residual=hip(res)).numpy()
+    y = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, out_mode=O.OUT_F32) + res
+    if mode == _ops.OUT_F16:
+        assert np.array_equal(got.view(np.uint16), O.f32_to_f16_bits(y))
+    else:
+        assert np.array_equal(got, y)
+
+
+def test_residual_needs_a_float_output():
+    a, w = hip(np.zeros((4, 16), np.int8)), hip(np.zeros((4, 16), np.int8))
+    with pytest.raises(ValueError):
+        _ops.qlinear_i8(a, w, out_mode=_ops.OUT_ACC_I32, residual=hip(np.zeros((4, 4), np.float32)))

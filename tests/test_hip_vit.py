@@ -150,3 +150,45 @@ def test_vit_end_to_end_against_the_cpu_path(cfg, batch):
     err = rel(got, exp)
     print(f"ViT dim {cfg['dim']} depth {cfg['depth']} batch {batch}: end-to-end max error / max |logit| = {err:.2e}")
     assert err < 4e-2
+
+
+def _range_of(t):
+    """(min, max) a dynamic quantizer would derive from the tensor's kept range."""
+    s = L.Tensor.empty((), L.float32, "hip")
+    z = L.Tensor.empty((), L.float32, "hip")
+    mn = L.Tensor.empty((), L.float32, "hip")
+    mx = L.Tensor.empty((), L.float32, "hip")
+    _C.call("lq_calc_qparams_from_keys", t._range.data_ptr, 0, 0, 255, 0, 1e-8, s.data_ptr, z.data_ptr,
+            mn.data_ptr, mx.data_ptr, None)
+    return mn.numpy(), mx.numpy(), s.numpy(), z.numpy()
+
+
+@pytest.mark.parametrize("rows,cols", [(12608, 768), (5, 33), (17, 1000)])
+def test_kept_ranges_equal_a_separate_minmax_pass(rows, cols):
+    import lucid_amd.quantization as Q
+
+    rng = np.random.default_rng(rows * 3 + cols)
+    x = (rng.standard_normal((rows, cols)) * 3 - 0.5).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(cols)).astype(np.float32)
+    for out in (F.layer_norm(hip(x), cols, hip(g), hip(b), 1e-6, track_range=True),
+                F.gelu(hip(x), track_range=True)):
+        mn, mx = Q.minmax(out)
+        s, z = Q.calculate_qparams(mn, mx, Q.per_tensor_affine, Q.quint8)
+        kmn, kmx, ks, kz = _range_of(out)
+        y = out.numpy()
+        assert kmn == y.min() == mn.numpy() and kmx == y.max() == mx.numpy()
+        assert ks.tobytes() == s.numpy().tobytes() and kz.tobytes() == z.numpy().tobytes()
+
+
+def test_kept_range_of_attention_and_nan_propagation():
+    rng = np.random.default_rng(2)
+    qkv = rng.standard_normal((3, 197, 3 * 12 * 64)).astype(np.float32)
+    out = F.scaled_dot_product_attention_qkv(hip(qkv), 12, track_range=True)
+    kmn, kmx, _, _ = _range_of(out)
+    y = out.numpy()
+    assert kmn == y.min() and kmx == y.max()
+    x = rng.standard_normal((64, 256)).astype(np.float32)
+    x[17, 5] = np.nan
+    kmn, kmx, ks, _ = _range_of(F.gelu(hip(x), track_range=True))
+    assert np.isnan(kmn) and np.isnan(kmx) and np.isnan(ks)  # Reduce.cpp:87-125 propagates NaN

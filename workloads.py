@@ -222,8 +222,8 @@ def _float_linear(w, b):
     return lin
 
 
-def _layer_norm(w, b, eps=1e-6):
-    ln = nn.LayerNorm(w.shape[0], eps=eps)
+def _layer_norm(w, b, eps=1e-6, track_range=True):
+    ln = nn.LayerNorm(w.shape[0], eps=eps, track_range=track_range)
     ln.register_buffer("weight", L.tensor(w, device="hip"))
     ln.register_buffer("bias", L.tensor(b, device="hip"))
     return ln
@@ -243,9 +243,11 @@ class ViTBlock(nn.Module):
     def forward(self, x):
         import lucid_amd.nn.functional as F
 
-        a = F.scaled_dot_product_attention_qkv(self.qkv(self.norm1(x)), self.heads)
-        x = F.add(x, self.proj(a))
-        return F.add(x, self.fc2(F.gelu(self.fc1(self.norm2(x)))))
+        # every float32 kernel that feeds a dynamic-quantized Linear keeps the range of
+        # what it writes; the residual adds ride in the epilogues of proj and fc2
+        a = F.scaled_dot_product_attention_qkv(self.qkv(self.norm1(x)), self.heads, track_range=True)
+        x = self.proj(a, residual=x)
+        return self.fc2(F.gelu(self.fc1(self.norm2(x)), track_range=True), residual=x)
 
 
 class QViT(nn.Module):
@@ -262,7 +264,7 @@ class QViT(nn.Module):
         self.register_buffer("cls_token", L.tensor(p["cls"], device="hip"))
         self.register_buffer("pos_embed", L.tensor(p["pos"], device="hip"))
         self.blocks = nn.Sequential(*[ViTBlock(f"blocks.{i}.", p, cfg["heads"]) for i in range(cfg["depth"])])
-        self.norm = _layer_norm(p["norm.weight"], p["norm.bias"])
+        self.norm = _layer_norm(p["norm.weight"], p["norm.bias"], track_range=False)
         self.head = _float_linear(p["head.weight"], p["head.bias"])
         Q.quantize_dynamic(self, inplace=True)
 
@@ -283,8 +285,7 @@ class QViT(nn.Module):
         tok = self.norm(self.blocks(tok))
         # class-token pooling: row 0 of every image
         cls = L.Tensor.empty((B, d), L.float32, "hip")
-        for b in range(B):
-            _C.call("lq_d2d", cls.data_ptr + b * d * 4, tok.data_ptr + b * (n + 1) * d * 4, d * 4, None)
+        _C.call("lq_gather_rows_f32", tok.data_ptr, (n + 1) * d, cls.data_ptr, B, d, None)
         return self.head(cls)
 
 
