@@ -178,30 +178,30 @@ int lq_global_avgpool_nhwc_i8(const int8_t* q, int code_offset, int B, int H, in
 /* nnqd.Linear takes x.min() / x.max() of its input on every forward
  * (lucid/nn/quantized/dynamic/linear.py:87-89): a full pass over a tensor some
  * kernel has just written.  The float32 kernels below can keep that range as a
- * by-product: pass them four 32-bit words initialised by lq_range_keys_init and
- * they fold the min / max (and a NaN flag) of what they write into them with
- * order-independent atomics.  lq_calc_qparams_from_keys then is
- * calculate_qparams(min, max) on that range (_qparams.py:190-215), bit-identical
- * to lq_minmax + lq_calc_qparams; mn_out / mx_out (optional) receive the range. */
-int lq_range_keys_init(uint32_t* keys, lq_stream stream);
-int lq_calc_qparams_from_keys(const uint32_t* keys, int symmetric, int qmin, int qmax, int is_signed,
-                              float eps, float* scale, float* zp, float* mn_out, float* mx_out,
-                              lq_stream stream);
+ * by-product: pass them a device buffer of lq_range_buffer_bytes() bytes (no
+ * initialisation needed) and every block stores the min / max of what it wrote
+ * into a slot of its own.  lq_calc_qparams_from_range reduces the slots and is
+ * then calculate_qparams(min, max) (_qparams.py:190-215), bit-identical to
+ * lq_minmax + lq_calc_qparams; mn_out / mx_out (optional) receive the range. */
+size_t lq_range_buffer_bytes(void);
+int lq_calc_qparams_from_range(const float* range, int symmetric, int qmin, int qmax, int is_signed,
+                               float eps, float* scale, float* zp, float* mn_out, float* mx_out,
+                               lq_stream stream);
 
 /* ------------------------------------------------- float32 steps of a ViT block */
 /* What Lucid's dynamic-quantized ViT keeps in float32 between its int8 Linears
  * (lucid/models/vision/vit/_model.py:132-161,202-204,275-278,449-458).  Tolerance
  * parity (1e-4 relative against a float32 CPU evaluation): summation orders differ.
- * range_keys, where present, may be null. */
+ * range, where present, may be null. */
 
 /* LayerNorm over the last axis of [rows, cols] (IBackend::layer_norm_forward;
  * lucid/_C/backend/cpu/Norm.cpp:35-65: mean, centred dot product / N,
  * rstd = 1/sqrt(var + eps), (c * rstd) * gamma + beta). */
 int lq_layernorm_f32(const float* x, const float* gamma, const float* beta, float* out, long rows, int cols,
-                     float eps, uint32_t* range_keys, lq_stream stream);
+                     float eps, float* range, lq_stream stream);
 
 /* GELU, exact erf form (lucid/nn/functional/activations.py:219, approximate="none"). */
-int lq_gelu_f32(const float* x, float* out, size_t n, uint32_t* range_keys, lq_stream stream);
+int lq_gelu_f32(const float* x, float* out, size_t n, float* range, lq_stream stream);
 
 /* out = a + b (IBackend::add on float32; the residual joins). */
 int lq_add_f32(const float* a, const float* b, float* out, size_t n, lq_stream stream);
@@ -212,7 +212,7 @@ int lq_add_f32(const float* a, const float* b, float* out, size_t n, lq_stream s
  * [B, T, H*D] (vit/_model.py:158).  D must be 64 and T <= 208 (ViT-B/16: T = 197);
  * anything else returns LQ_ERR_NOT_IMPLEMENTED. */
 int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale,
-                     uint32_t* range_keys, lq_stream stream);
+                     float* range, lq_stream stream);
 
 /* Patch embedding, a convolution whose stride equals its kernel
  * (vit/_model.py:62-69), as im2col + GEMM: image [B,C,H,W] -> rows

@@ -131,8 +131,8 @@ _SIGNATURES["lq_gelu_f32"] = [_vp, _vp, _sz, _vp, _vp]
 _SIGNATURES["lq_add_f32"] = [_vp, _vp, _vp, _sz, _vp]
 _SIGNATURES["lq_attention_f32"] = [_vp, _vp, _i, _i, _i, _i, _f, _vp, _vp]
 _SIGNATURES["lq_gather_rows_f32"] = [_vp, _sz, _vp, _sz, _sz, _vp]
-_SIGNATURES["lq_range_keys_init"] = [_vp, _vp]
-_SIGNATURES["lq_calc_qparams_from_keys"] = [_vp, _i, _i, _i, _i, _f, _vp, _vp, _vp, _vp, _vp]
+_SIGNATURES["lq_range_buffer_bytes"] = []
+_SIGNATURES["lq_calc_qparams_from_range"] = [_vp, _i, _i, _i, _i, _f, _vp, _vp, _vp, _vp, _vp]
 _SIGNATURES["lq_patchify_f32"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_sgemm_nt_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_assemble_tokens_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
@@ -164,8 +164,8 @@ _SIGNATURES["lq_dequantize_nhwc_to_nchw"] = [_vp, _i, _vp, _i, _i, _i, _i, _vp, 
 _SIGNATURES["lq_repack_oihw_to_ohwi_i8"] = [_vp, _vp, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_maxpool2d_nhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 
-_RESTYPE = {"lq_last_error": C.c_char_p}
-_NO_STATUS = {"lq_version", "lq_last_error", "lq_op_count"}
+_RESTYPE = {"lq_last_error": C.c_char_p, "lq_range_buffer_bytes": C.c_size_t}
+_NO_STATUS = {"lq_version", "lq_last_error", "lq_op_count", "lq_range_buffer_bytes"}
 
 _lib = None
 _initialised_device = None
@@ -249,6 +249,11 @@ def is_available() -> bool:
         return rc == 0 and n.value > 0
     except (OSError, LucidError):
         return False
+
+
+def range_buffer_words() -> int:
+    """float32 words of a kept-range buffer (``lq_range_buffer_bytes``)."""
+    return int(load().lq_range_buffer_bytes()) // 4
 
 
 def device_name() -> str:

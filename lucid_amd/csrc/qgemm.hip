@@ -21,6 +21,11 @@
 
 #include "qgemm_tile.hpp"
 
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
+
 using namespace lq;
 
 namespace lq {
@@ -67,23 +72,7 @@ int launch_tile_c7(const GemmArgs&, bool, int, int, hipStream_t);
 
 namespace {
 
-// tile_config: low byte = tile shape (0 = choose from the problem shape, 1..6 =
-// a specific one), next byte = schedule (0 = choose, 1 = block per tile, 2 = stream-K).
-int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st) {
-    int cfg = tile_config & 0xff;
-    const int schedule = (tile_config >> 8) & 0xff;
-    if (cfg == 0) {
-        // 128 x 256 tiles keep two blocks per CU busy and measured fastest from
-        // M = 2048 to 8192 at N = 11008; narrower tiles when N is small or when
-        // the wide ones would leave most of the 256 CUs without work.
-        const long mt128 = (g.M + 127) / 128;
-        if (g.N <= 64)
-            cfg = 6;
-        else if (g.N <= 128 || mt128 * ((g.N + 255) / 256) * groups < 256)
-            cfg = 5;
-        else
-            cfg = 4;
-    }
+int launch_tile_shape(const GemmArgs& g, bool conv, int groups, int cfg, int schedule, hipStream_t st) {
     switch (cfg) {
     case 1: return launch_tile_c1(g, conv, groups, schedule, st);
     case 2: return launch_tile_c2(g, conv, groups, schedule, st);
@@ -94,6 +83,117 @@ int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, h
     case 7: return launch_tile_c7(g, conv, groups, schedule, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
+}
+
+// Shape chosen from the problem size alone: 128 x 256 tiles keep two blocks per
+// CU busy; narrower tiles when N is small or when the wide ones would leave
+// most of the 256 CUs without work.
+int heuristic_tile_shape(const GemmArgs& g, int groups) {
+    const long mt128 = (g.M + 127) / 128;
+    if (g.N <= 64) return 6;
+    if (g.N <= 128 || mt128 * ((g.N + 255) / 256) * groups < 256) return 5;
+    return 4;
+}
+
+// The best tile shape depends on how the tile count falls on the 256 CUs and on
+// the epilogue's share, which no simple rule predicted well (at M = 12608 the
+// winner changes between K = 768 and K = 3072).  So the first launch of a problem
+// shape times each candidate on the caller's own operands (every shape gives
+// bit-identical results) and the choice is kept for the life of the process.
+// Not while the stream is being captured, and not when LQ_TILE_AUTOTUNE=0.
+struct TuneKey {
+    int M, N, K, mode, conv, groups, geom[8], flags;
+    bool operator==(const TuneKey& o) const { return std::memcmp(this, &o, sizeof(TuneKey)) == 0; }
+};
+struct TuneKeyHash {
+    size_t operator()(const TuneKey& k) const {
+        const unsigned char* p = reinterpret_cast<const unsigned char*>(&k);
+        size_t h = 1469598103934665603ull;
+        for (size_t i = 0; i < sizeof(TuneKey); ++i) h = (h ^ p[i]) * 1099511628211ull;
+        return h;
+    }
+};
+std::mutex g_tune_mu;
+std::unordered_map<TuneKey, int, TuneKeyHash> g_tune;
+
+bool autotune_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("LQ_TILE_AUTOTUNE");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, int* cfg_out) {
+    TuneKey key;
+    std::memset(&key, 0, sizeof(key));
+    key.M = g.M, key.N = g.N, key.K = g.K, key.mode = g.out_mode, key.conv = conv, key.groups = groups;
+    if (conv) {
+        const int geom[8] = {g.cH, g.cW, g.cCin, g.cKW, g.csh * 16 + g.csw, g.cph * 256 + g.cpw,
+                             g.cdh * 16 + g.cdw, g.cOW};
+        std::memcpy(key.geom, geom, sizeof(geom));
+    }
+    key.flags = (g.residual ? 1 : 0) | (g.a_scale_per_row ? 2 : 0) | (g.bias ? 4 : 0);
+    {
+        std::lock_guard<std::mutex> lock(g_tune_mu);
+        auto it = g_tune.find(key);
+        if (it != g_tune.end()) {
+            *cfg_out = it->second;
+            return LQ_OK;
+        }
+    }
+    const int fallback = heuristic_tile_shape(g, groups);
+    *cfg_out = fallback;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    LQ_HIP(hipStreamIsCapturing(st, &capturing));
+    // too little work to be worth timing: a handful of tiles whatever the shape
+    const double ops = 2.0 * g.M * double(g.N) * g.K * groups;
+    if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9) return LQ_OK;
+
+    int cands[6], n = 0;
+    if (g.N <= 64) cands[n++] = 6;
+    cands[n++] = 5;
+    if (g.N > 64) cands[n++] = 3, cands[n++] = 4;
+    if (g.N > 128 && g.M > 128) cands[n++] = 1;
+    hipEvent_t e0, e1;
+    LQ_HIP(hipEventCreate(&e0));
+    LQ_HIP(hipEventCreate(&e1));
+    float best = 1e30f;
+    int rc = LQ_OK;
+    bool timed = true;
+    for (int i = 0; i < n && rc == LQ_OK && timed; ++i) {
+        rc = launch_tile_shape(g, conv, groups, cands[i], 1, st);  // warm: code load, attributes
+        if (rc) break;
+        timed = hipEventRecord(e0, st) == hipSuccess;
+        for (int r = 0; r < 3 && rc == LQ_OK; ++r) rc = launch_tile_shape(g, conv, groups, cands[i], 1, st);
+        float ms = 0.0f;
+        timed = timed && rc == LQ_OK && hipEventRecord(e1, st) == hipSuccess &&
+                hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+        if (timed && ms < best) best = ms, *cfg_out = cands[i];
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (!timed && rc == LQ_OK) {  // timing unavailable: keep the rule-based choice, do not cache
+        *cfg_out = fallback;
+        return LQ_OK;
+    }
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lock(g_tune_mu);
+    g_tune[key] = *cfg_out;
+    return LQ_OK;
+}
+
+// tile_config: low byte = tile shape (0 = choose, 1..7 = a specific one), next
+// byte = schedule (0 = choose, 1 = block per tile, 2 = stream-K, 3 = stream-K over
+// the leftover tiles only).
+int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st) {
+    int cfg = tile_config & 0xff;
+    const int schedule = (tile_config >> 8) & 0xff;
+    if (cfg == 0) {
+        int rc = tuned_tile_shape(g, conv, groups, st, &cfg);
+        if (rc) return rc;
+    }
+    return launch_tile_shape(g, conv, groups, cfg, schedule, st);
 }
 
 // ---------------------------------------------------------------- skinny kernel

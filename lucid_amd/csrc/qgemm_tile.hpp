@@ -110,6 +110,18 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
 #pragma unroll
         for (int part = 0; part < PARTS; ++part) {
             const int band = wm * (TM * 32) + i * 32 + part * EPI_ROWS;
+            const int m_first = m0 + band + row0, n = n0 + wn * (TN * 32) + cq;
+            // residual rows of this part, requested before the arithmetic so that
+            // their latency is paid under it (`interior` vouches for alignment)
+            constexpr bool kFloatOut = MODE == OUT_F32 || MODE == OUT_F16;
+            const bool res_fast = kFloatOut && interior && g.residual != nullptr;
+            float4 rv[kFloatOut ? PASSES : 1];
+            if (kFloatOut && res_fast) {
+                const float* rp = g.residual + size_t(m_first) * size_t(g.ldr) + size_t(n);
+#pragma unroll
+                for (int p = 0; p < PASSES; ++p)
+                    rv[p] = *reinterpret_cast<const float4*>(rp + size_t(p) * ROWS_PER_PASS * size_t(g.ldr));
+            }
             // this lane's rows of the part: groups of four consecutive rows
             float as[RPP];
 #pragma unroll
@@ -127,7 +139,6 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                         epilogue_value<MODE>(g, acc[i][j][r], as[rr], cp[j], S, Z);
             }
             wave_lds_sync();
-            const int m_first = m0 + band + row0, n = n0 + wn * (TN * 32) + cq;
             const uint32_t* src = stage + row0 * STRIDE + cq;
             if (interior) {
                 uint4 v[PASSES];
@@ -136,13 +147,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                     v[p] = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
                 size_t idx = size_t(m_first) * size_t(g.ldo) + size_t(n);
                 const size_t step = size_t(ROWS_PER_PASS) * size_t(g.ldo);
-                if ((MODE == OUT_F32 || MODE == OUT_F16) && g.residual) {
-                    // `interior` also vouches for the residual's alignment
-                    const float* rp = g.residual + size_t(m_first) * size_t(g.ldr) + size_t(n);
-                    float4 rv[PASSES];
-#pragma unroll
-                    for (int p = 0; p < PASSES; ++p)
-                        rv[p] = *reinterpret_cast<const float4*>(rp + size_t(p) * ROWS_PER_PASS * size_t(g.ldr));
+                if (kFloatOut && res_fast) {
 #pragma unroll
                     for (int p = 0; p < PASSES; ++p) {
                         v[p].x = __float_as_uint(__uint_as_float(v[p].x) + rv[p].x);

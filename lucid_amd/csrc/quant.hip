@@ -5,7 +5,7 @@
 // (lucid/quantization/_functional.py:180, 281, 311-313): IEEE division,
 // round-half-even, add zero point, clamp, cast.  No reciprocal, no FMA.
 #include "common.hpp"
-#include "range_keys.hpp"
+#include "range_slots.hpp"
 
 using namespace lq;
 
@@ -331,8 +331,8 @@ __device__ __forceinline__ MinMax mm_block_reduce(MinMax m) {
         m.hi = fmaxf(m.hi, __shfl_xor(m.hi, d, 64));
         m.nan |= __shfl_xor(m.nan, d, 64);
     }
-    __shared__ float s_lo[kThreads / 64], s_hi[kThreads / 64];
-    __shared__ int s_nan[kThreads / 64];
+    __shared__ float s_lo[16], s_hi[16];  // up to 1024 threads
+    __shared__ int s_nan[16];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nwaves = (blockDim.x + 63) >> 6;
     if (lane == 0) {
@@ -501,23 +501,31 @@ __global__ void calc_qparams_kernel(const float* __restrict__ mn, const float* _
     qparams_of(mn[c], mx[c], symmetric, qmin, qmax, is_signed, eps, half_range, &scale[c], &zp[c]);
 }
 
-__global__ void range_keys_init_kernel(uint32_t* keys) {
-    keys[0] = kRangeMinIdentity;
-    keys[1] = kRangeMaxIdentity;
-    keys[2] = 0;
-    keys[3] = 0;
-}
-
-// Per-tensor qparams from a range kept by the producing kernel; also writes
-// the range itself when asked.
-__global__ void calc_qparams_from_keys_kernel(const uint32_t* __restrict__ keys, int symmetric, int qmin,
-                                              int qmax, int is_signed, float eps, float half_range,
-                                              float* scale, float* zp, float* mn_out, float* mx_out) {
-    float mn = range_unkey(keys[0]), mx = range_unkey(keys[1]);
-    if (keys[2]) mn = mx = __builtin_nanf("");
-    if (mn_out) *mn_out = mn;
-    if (mx_out) *mx_out = mx;
-    qparams_of(mn, mx, symmetric, qmin, qmax, is_signed, eps, half_range, scale, zp);
+// Per-tensor qparams from a range kept by the producing kernel (one block):
+// reduce the partial slots, then calculate_qparams; also writes the range
+// itself when asked.
+__global__ __launch_bounds__(1024) void calc_qparams_from_range_kernel(const float* __restrict__ range,
+                                                                        int symmetric, int qmin, int qmax,
+                                                                        int is_signed, float eps,
+                                                                        float half_range, float* scale,
+                                                                        float* zp, float* mn_out,
+                                                                        float* mx_out) {
+    const unsigned n = reinterpret_cast<const unsigned*>(range)[0];
+    MinMax m{__builtin_inff(), -__builtin_inff(), 0};
+    for (unsigned i = threadIdx.x; i < n; i += 1024) {
+        const float a = range[4 + i], b = range[4 + kRangeSlots + i];
+        m.nan |= (a != a) | (b != b);
+        m.lo = fminf(m.lo, a);
+        m.hi = fmaxf(m.hi, b);
+    }
+    m = mm_block_reduce(m);
+    if (threadIdx.x == 0) {
+        float mn = m.lo, mx = m.hi;
+        if (m.nan) mn = mx = __builtin_nanf("");
+        if (mn_out) *mn_out = mn;
+        if (mx_out) *mx_out = mx;
+        qparams_of(mn, mx, symmetric, qmin, qmax, is_signed, eps, half_range, scale, zp);
+    }
 }
 
 }  // namespace
@@ -608,22 +616,17 @@ int lq_calc_qparams(const float* mn, const float* mx, size_t C, int symmetric, i
     return LQ_OK;
 }
 
-int lq_range_keys_init(uint32_t* keys, lq_stream stream) {
-    LQ_REQUIRE(keys, LQ_ERR_VALUE, "range_keys_init: NULL pointer");
-    hipLaunchKernelGGL(range_keys_init_kernel, dim3(1), dim3(1), 0, as_stream(stream), keys);
-    LQ_CHECK_LAUNCH("range_keys_init");
-    return LQ_OK;
-}
+size_t lq_range_buffer_bytes(void) { return size_t(kRangeWords) * 4; }
 
-int lq_calc_qparams_from_keys(const uint32_t* keys, int symmetric, int qmin, int qmax, int is_signed,
-                              float eps, float* scale, float* zp, float* mn_out, float* mx_out,
-                              lq_stream stream) {
-    LQ_REQUIRE(keys && scale && zp, LQ_ERR_VALUE, "calc_qparams_from_keys: NULL pointer");
-    LQ_REQUIRE(qmax > qmin, LQ_ERR_VALUE, "calc_qparams_from_keys: empty grid [%d,%d]", qmin, qmax);
+int lq_calc_qparams_from_range(const float* range, int symmetric, int qmin, int qmax, int is_signed,
+                               float eps, float* scale, float* zp, float* mn_out, float* mx_out,
+                               lq_stream stream) {
+    LQ_REQUIRE(range && scale && zp, LQ_ERR_VALUE, "calc_qparams_from_range: NULL pointer");
+    LQ_REQUIRE(qmax > qmin, LQ_ERR_VALUE, "calc_qparams_from_range: empty grid [%d,%d]", qmin, qmax);
     const float half_range = float((double(qmax) - double(qmin)) / 2.0);
-    hipLaunchKernelGGL(calc_qparams_from_keys_kernel, dim3(1), dim3(1), 0, as_stream(stream), keys,
+    hipLaunchKernelGGL(calc_qparams_from_range_kernel, dim3(1), dim3(1024), 0, as_stream(stream), range,
                        symmetric, qmin, qmax, is_signed, eps, half_range, scale, zp, mn_out, mx_out);
-    LQ_CHECK_LAUNCH("calc_qparams_from_keys");
+    LQ_CHECK_LAUNCH("calc_qparams_from_range");
     return LQ_OK;
 }
 

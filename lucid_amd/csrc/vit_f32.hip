@@ -15,7 +15,7 @@
 // Matrix products use the float32 MFMA instructions; results agree with a CPU
 // float32 evaluation to rounding-order differences (tested to 1e-4 relative).
 #include "common.hpp"
-#include "range_keys.hpp"
+#include "range_slots.hpp"
 
 using namespace lq;
 
@@ -34,13 +34,13 @@ __device__ __forceinline__ float wave_sum(float v) {
 // One wavefront per row; the row (a few KiB) is re-read from cache for the
 // variance and the output pass.  mean, centred values, var = dot(c,c)/N,
 // rstd = 1/sqrt(var+eps), y = (c*rstd)*gamma + beta: the reference's steps.
-constexpr int LN_ROWS_PER_WAVE = 4;
+constexpr int LN_ROWS_PER_WAVE = 1;
 
 __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x,
                                                         const float* __restrict__ gamma,
                                                         const float* __restrict__ beta,
                                                         float* __restrict__ out, long rows, int cols,
-                                                        float eps, uint32_t* range_keys) {
+                                                        float eps, float* range) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const bool vec = (cols % 4 == 0) && aligned16(x) && aligned16(out) && aligned16(gamma) && aligned16(beta);
     const float inv_n = 1.0f / float(cols);
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
             }
         }
     }
-    if (range_keys) range_block_update(range_keys, lo, hi, nan);
+    if (range) range_block_store(range, lo, hi, nan);
 }
 
 // ---------------------------------------------------------------- elementwise
@@ -110,10 +110,12 @@ __device__ __forceinline__ float gelu_erf(float x) {
     return (0.5f * x) * (1.0f + erff(x * 0.70710678118654752440f));
 }
 
-// Grid-stride (a bounded number of blocks) so that the optional range
-// tracking costs a few thousand atomics at most.
+// Four float4 per thread (block-strided, so each access of a wavefront is
+// contiguous); the optional range costs one partial slot per block.
+constexpr int GELU_PER_THREAD = 4;
+
 __global__ __launch_bounds__(256) void gelu_kernel(const float* __restrict__ x, float* __restrict__ out,
-                                                   size_t n, int vec, uint32_t* range_keys) {
+                                                   size_t n, int vec, float* range) {
     float lo = __builtin_inff(), hi = -__builtin_inff();
     int nan = 0;
     auto track = [&](float y) {
@@ -121,22 +123,35 @@ __global__ __launch_bounds__(256) void gelu_kernel(const float* __restrict__ x, 
         lo = fminf(lo, y);
         hi = fmaxf(hi, y);
     };
-    const size_t stride = size_t(gridDim.x) * 256;
+    const size_t base = size_t(blockIdx.x) * (256 * GELU_PER_THREAD) + threadIdx.x;
     if (vec) {
-        for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i * 4 < n; i += stride) {
-            const float4 v = reinterpret_cast<const float4*>(x)[i];
-            float4 y = {gelu_erf(v.x), gelu_erf(v.y), gelu_erf(v.z), gelu_erf(v.w)};
-            reinterpret_cast<float4*>(out)[i] = y;
-            track(y.x), track(y.y), track(y.z), track(y.w);
+        float4 v[GELU_PER_THREAD];
+#pragma unroll
+        for (int u = 0; u < GELU_PER_THREAD; ++u) {
+            const size_t i = base + size_t(u) * 256;
+            if (i * 4 < n) v[u] = reinterpret_cast<const float4*>(x)[i];
+        }
+#pragma unroll
+        for (int u = 0; u < GELU_PER_THREAD; ++u) {
+            const size_t i = base + size_t(u) * 256;
+            if (i * 4 < n) {
+                float4 y = {gelu_erf(v[u].x), gelu_erf(v[u].y), gelu_erf(v[u].z), gelu_erf(v[u].w)};
+                reinterpret_cast<float4*>(out)[i] = y;
+                track(y.x), track(y.y), track(y.z), track(y.w);
+            }
         }
     } else {
-        for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
-            const float y = gelu_erf(x[i]);
-            out[i] = y;
-            track(y);
+#pragma unroll
+        for (int u = 0; u < GELU_PER_THREAD; ++u) {
+            const size_t i = base + size_t(u) * 256;
+            if (i < n) {
+                const float y = gelu_erf(x[i]);
+                out[i] = y;
+                track(y);
+            }
         }
     }
-    if (range_keys) range_block_update(range_keys, lo, hi, nan);
+    if (range) range_block_store(range, lo, hi, nan);
 }
 
 // dst[r, :] = src[r * src_row_stride : r * src_row_stride + cols]
@@ -315,7 +330,7 @@ __global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__
 constexpr int AT_D = 64, AT_TMAX = 208, AT_LD = AT_D + 4;  // row stride 68: 4*row + k hits all 64 banks
 
 __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict__ qkv, float* __restrict__ out,
-                                                        int B, int T, int H, float scale, uint32_t* range_keys) {
+                                                        int B, int T, int H, float scale, float* range) {
     extern __shared__ __attribute__((aligned(16))) float at_smem[];
     float (*sk)[AT_LD] = reinterpret_cast<float (*)[AT_LD]>(at_smem);
     float (*sv)[AT_LD] = reinterpret_cast<float (*)[AT_LD]>(at_smem + AT_TMAX * AT_LD);
@@ -403,7 +418,7 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
             const int q = q0 + 4 * g + r;
             if (q < T) out[(size_t(b) * T + q) * (size_t(H) * AT_D) + size_t(h) * AT_D + 16 * j + c] = o[j][r];
         }
-    if (range_keys) {
+    if (range) {
         float lo = __builtin_inff(), hi = -__builtin_inff();
         int nan = 0;
 #pragma unroll
@@ -415,7 +430,7 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
                     lo = fminf(lo, o[j][r]);
                     hi = fmaxf(hi, o[j][r]);
                 }
-        range_block_update(range_keys, lo, hi, nan);
+        range_block_store(range, lo, hi, nan);
     }
 }
 
@@ -426,25 +441,32 @@ unsigned blocks_for(size_t n) { return unsigned((n + 255) / 256); }
 extern "C" {
 
 int lq_layernorm_f32(const float* x, const float* gamma, const float* beta, float* out, long rows, int cols,
-                     float eps, uint32_t* range_keys, void* stream) {
+                     float eps, float* range, void* stream) {
     LQ_REQUIRE(x && gamma && beta && out, LQ_ERR_VALUE, "layernorm: null pointer");
     LQ_REQUIRE(rows >= 0 && cols > 0, LQ_ERR_SHAPE, "layernorm: bad shape (%ld, %d)", rows, cols);
     if (rows == 0) return LQ_OK;
     const long per_block = 4L * LN_ROWS_PER_WAVE;
     LQ_REQUIRE((rows + per_block - 1) / per_block < 0x7fffffffL, LQ_ERR_SHAPE, "layernorm: too many rows");
+    LQ_REQUIRE(range == nullptr || (rows + per_block - 1) / per_block <= kRangeSlots, LQ_ERR_SHAPE,
+               "layernorm: %ld rows are too many for a kept range (at most %ld)", rows,
+               long(kRangeSlots) * per_block);
     layernorm_kernel<<<unsigned((rows + per_block - 1) / per_block), 256, 0, as_stream(stream)>>>(
-        x, gamma, beta, out, rows, cols, eps, range_keys);
+        x, gamma, beta, out, rows, cols, eps, range);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }
 
-int lq_gelu_f32(const float* x, float* out, size_t n, uint32_t* range_keys, void* stream) {
+int lq_gelu_f32(const float* x, float* out, size_t n, float* range, void* stream) {
     LQ_REQUIRE(x && out, LQ_ERR_VALUE, "gelu: null pointer");
     if (n == 0) return LQ_OK;
     const int vec = (n % 4 == 0) && aligned16(x) && aligned16(out);
-    unsigned blocks = blocks_for(vec ? n / 4 : n);
-    if (blocks > 8192) blocks = 8192;
-    gelu_kernel<<<blocks, 256, 0, as_stream(stream)>>>(x, out, n, vec, range_keys);
+    const size_t units = vec ? n / 4 : n;
+    const size_t blocks = (units + 256 * GELU_PER_THREAD - 1) / (256 * GELU_PER_THREAD);
+    LQ_REQUIRE(blocks < 0x7fffffffull, LQ_ERR_SHAPE, "gelu: tensor too large");
+    LQ_REQUIRE(range == nullptr || blocks <= size_t(kRangeSlots), LQ_ERR_SHAPE,
+               "gelu: %zu elements are too many for a kept range (at most %zu)", n,
+               size_t(kRangeSlots) * 256 * GELU_PER_THREAD * 4);
+    gelu_kernel<<<unsigned(blocks), 256, 0, as_stream(stream)>>>(x, out, n, vec, range);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }
@@ -502,7 +524,7 @@ int lq_gather_rows_f32(const float* src, size_t src_row_stride, float* dst, size
     return LQ_OK;
 }
 
-int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale, uint32_t* range_keys,
+int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, float scale, float* range,
                      void* stream) {
     LQ_REQUIRE(qkv && out, LQ_ERR_VALUE, "attention: null pointer");
     LQ_REQUIRE(B >= 0 && T >= 1 && H >= 1, LQ_ERR_SHAPE, "attention: bad shape");
@@ -510,6 +532,8 @@ int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, f
                "attention: head dim %d / %d tokens; this kernel handles head dim 64 and up to 208 tokens", D, T);
     LQ_REQUIRE(aligned16(qkv), LQ_ERR_VALUE, "attention: qkv must be 16-byte aligned");
     if (B == 0) return LQ_OK;
+    LQ_REQUIRE(range == nullptr || long(B) * H <= kRangeSlots, LQ_ERR_SHAPE,
+               "attention: too many (batch, head) pairs for a kept range");
     const int waves = (T + 15) / 16;
     constexpr size_t kSmem = size_t(2) * AT_TMAX * AT_LD * sizeof(float);
     static bool attr_set = false;
@@ -519,7 +543,7 @@ int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, f
         attr_set = true;
     }
     attention_kernel<<<unsigned(B) * H, waves * 64, kSmem, as_stream(stream)>>>(qkv, out, B, T, H, scale,
-                                                                                 range_keys);
+                                                                                 range);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }

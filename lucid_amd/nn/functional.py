@@ -22,11 +22,10 @@ def _require_f32_hip(name: str, *ts: Tensor) -> None:
 
 
 def _new_range() -> Tensor:
-    """Four device words holding a running (min, max, NaN flag) for the tensor a
-    kernel is about to write."""
-    keys = Tensor.empty((4,), T.int32, "hip")
-    _C.call("lq_range_keys_init", keys.data_ptr, None)
-    return keys
+    """Device buffer into which a kernel stores the per-block min / max of the
+    tensor it is about to write (``lq_range_buffer_bytes``)."""
+    _C.init()
+    return Tensor.empty((_C.range_buffer_words(),), T.float32, "hip")
 
 
 def layer_norm(x: Tensor, normalized_shape, weight: Tensor, bias: Tensor, eps: float = 1e-5,

@@ -61,7 +61,7 @@ class Linear(Module):
             # the kernel that wrote x kept its min / max: qparams straight from them
             x_scale = Tensor.empty((), T.float32, "hip")
             x_zp = Tensor.empty((), T.float32, "hip")
-            _C.call("lq_calc_qparams_from_keys", x._range.data_ptr, 0, qd.quant_min, qd.quant_max,
+            _C.call("lq_calc_qparams_from_range", x._range.data_ptr, 0, qd.quant_min, qd.quant_max,
                     int(qd.signed), 1e-8, x_scale.data_ptr, x_zp.data_ptr, None, None, None)
         else:
             mn, mx = minmax(x)

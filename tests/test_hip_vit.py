@@ -158,7 +158,7 @@ def _range_of(t):
     z = L.Tensor.empty((), L.float32, "hip")
     mn = L.Tensor.empty((), L.float32, "hip")
     mx = L.Tensor.empty((), L.float32, "hip")
-    _C.call("lq_calc_qparams_from_keys", t._range.data_ptr, 0, 0, 255, 0, 1e-8, s.data_ptr, z.data_ptr,
+    _C.call("lq_calc_qparams_from_range", t._range.data_ptr, 0, 0, 255, 0, 1e-8, s.data_ptr, z.data_ptr,
             mn.data_ptr, mx.data_ptr, None)
     return mn.numpy(), mx.numpy(), s.numpy(), z.numpy()
 
