@@ -360,6 +360,14 @@ int lq_dequantize_nhwc_to_nchw(const int8_t* q, int code_offset, float* out, int
 int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH, int KW,
                               lq_stream stream);
 
+/* F.pad with mode reflect (1) / replicate (2) / circular (3) on NHWC codes: how a
+ * quantized convolution with padding_mode != "zeros" pads before convolving with
+ * padding 0 (lucid/nn/modules/conv.py:104-123).  The padded float image is a gather
+ * of the original, so the codes are gathered the same way; out is
+ * [B, H+top+bottom, W+left+right, C]. */
+int lq_pad_nhwc_i8(const int8_t* x, int8_t* out, int B, int H, int W, int C, int pad_top, int pad_bottom,
+                   int pad_left, int pad_right, int mode, lq_stream stream);
+
 /* Max-pool on NHWC codes (F.max_pool2d between quantized layers of a ResNet
  * stem): quantisation is monotone, so pooling codes equals pooling values. */
 int lq_maxpool2d_nhwc_i8(const int8_t* x, int8_t* out, int B, int H, int W, int C, int KH, int KW,

@@ -136,6 +136,7 @@ _SIGNATURES["lq_calc_qparams_from_range"] = [_vp, _i, _i, _i, _i, _f, _vp, _vp, 
 _SIGNATURES["lq_patchify_f32"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_sgemm_nt_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_assemble_tokens_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
+_SIGNATURES["lq_pad_nhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
 _SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]

@@ -174,6 +174,40 @@ __global__ void repack_oihw_to_ohwi_kernel(const int8_t* __restrict__ w, int8_t*
     }
 }
 
+// Non-zero padding modes of F.pad on NHWC codes (reflect / replicate / circular):
+// the padded float image is a gather of the original, so the padded code image is
+// the same gather of the codes.  One lane per 16 channels when C % 16 == 0, else per byte.
+__device__ __forceinline__ int pad_source(int i, int n, int mode) {
+    if (i >= 0 && i < n) return i;
+    if (mode == 1) {  // reflect: -1 -> 1, n -> n - 2 (no edge repeat)
+        i = i < 0 ? -i : 2 * (n - 1) - i;
+        return i;
+    }
+    if (mode == 2) return i < 0 ? 0 : n - 1;  // replicate
+    i %= n;                                   // circular
+    return i < 0 ? i + n : i;
+}
+
+__global__ __launch_bounds__(256) void pad_nhwc_i8_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ out,
+                                                          int B, int H, int W, int C, int pt, int pl, int OH,
+                                                          int OW, int mode, int vec) {
+    const int cunits = vec ? C / 16 : C;
+    const size_t total = size_t(B) * OH * OW * cunits;
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int cu = int(i % cunits);
+    const size_t pix = i / cunits;
+    const int ow = int(pix % OW), oh = int((pix / OW) % OH);
+    const size_t b = pix / (size_t(OW) * OH);
+    const int ih = pad_source(oh - pt, H, mode), iw = pad_source(ow - pl, W, mode);
+    const size_t src = ((b * H + ih) * W + iw) * C, dst = pix * C;
+    if (vec)
+        reinterpret_cast<uint4*>(out + dst)[cu] = reinterpret_cast<const uint4*>(x + src)[cu];
+    else
+        out[dst + cu] = x[src + cu];
+}
+
+
 // max-pool on codes, NHWC.  Quantisation is monotone, so the maximum of the
 // codes is the code of the maximum; padded taps never win.
 __global__ __launch_bounds__(256) void maxpool_nhwc_i8_kernel(const int8_t* __restrict__ x,
@@ -368,6 +402,30 @@ int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH
     hipLaunchKernelGGL(repack_oihw_to_ohwi_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream),
                        w, out, O, I, KH, KW);
     LQ_CHECK_LAUNCH("repack_oihw_to_ohwi");
+    return LQ_OK;
+}
+
+int lq_pad_nhwc_i8(const int8_t* x, int8_t* out, int B, int H, int W, int C, int pad_top, int pad_bottom,
+                   int pad_left, int pad_right, int mode, lq_stream stream) {
+    LQ_REQUIRE(x && out, LQ_ERR_VALUE, "pad: NULL pointer");
+    LQ_REQUIRE(B >= 0 && H > 0 && W > 0 && C > 0, LQ_ERR_SHAPE, "pad: bad shape");
+    LQ_REQUIRE(pad_top >= 0 && pad_bottom >= 0 && pad_left >= 0 && pad_right >= 0, LQ_ERR_VALUE,
+               "pad: negative padding");
+    LQ_REQUIRE(mode >= 1 && mode <= 3, LQ_ERR_VALUE, "pad: mode must be 1 (reflect), 2 (replicate) or 3 (circular)");
+    if (mode == 1)  // F.pad's rule for reflect: the pad must be smaller than the dimension
+        LQ_REQUIRE(pad_top < H && pad_bottom < H && pad_left < W && pad_right < W, LQ_ERR_VALUE,
+                   "pad: reflect padding must be smaller than the image");
+    if (mode == 3)
+        LQ_REQUIRE(pad_top <= H && pad_bottom <= H && pad_left <= W && pad_right <= W, LQ_ERR_VALUE,
+                   "pad: circular padding must not exceed the image");
+    const int OH = H + pad_top + pad_bottom, OW = W + pad_left + pad_right;
+    const int vec = (C % 16 == 0) && aligned16(x) && aligned16(out);
+    const size_t total = size_t(B) * OH * OW * (vec ? C / 16 : C);
+    if (total == 0) return LQ_OK;
+    LQ_REQUIRE((total + 255) / 256 < 0x7fffffffull, LQ_ERR_SHAPE, "pad: tensor too large");
+    hipLaunchKernelGGL(pad_nhwc_i8_kernel, dim3(unsigned((total + 255) / 256)), dim3(256), 0, as_stream(stream), x,
+                       out, B, H, W, C, pad_top, pad_left, OH, OW, mode, vec);
+    LQ_CHECK_LAUNCH("pad_nhwc_i8");
     return LQ_OK;
 }
 

@@ -24,6 +24,9 @@ from ._utils import (activation_qparams, host_scalar, input_grid, quantize_weigh
                      require_symmetric_weight, storage_offset)
 
 
+_PAD_MODES = {"zeros": 0, "reflect": 1, "replicate": 2, "circular": 3}
+
+
 def _pair(v):
     return (v, v) if isinstance(v, int) else tuple(v)
 
@@ -97,9 +100,8 @@ class Conv2d(Module):
         g = input_grid(x, name)
         if x.ndim != 4 or x.shape[1] != self.in_channels:
             raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, H, W), got {x.shape}")
-        if self.padding_mode != "zeros":
-            raise NotImplementedError(
-                f"{name}: padding_mode={self.padding_mode!r} is not supported by the hip kernels")
+        if self.padding_mode not in _PAD_MODES:
+            raise ValueError(f"{name}: unknown padding_mode {self.padding_mode!r}")
         if g.zp_host is None:
             raise NotImplementedError(
                 f"{name}: the input zero point is only known on the device; convolution needs it "
@@ -111,10 +113,18 @@ class Conv2d(Module):
         if self._zp_host is None:
             self._zp_host = int(host_scalar(self.zero_point))
         off = storage_offset(self.out_qdtype)
+        in_codes, pad = g.codes, self._resolve_pad(x)
+        if self.padding_mode != "zeros" and any(pad):
+            # pre-pad the codes, then convolve with padding 0 (nn/modules/conv.py:104-123)
+            B, H, W, Ci = in_codes.shape
+            padded = Tensor.empty((B, H + pad[0] + pad[1], W + pad[2] + pad[3], Ci), T.int8, "hip")
+            _C.call("lq_pad_nhwc_i8", in_codes.data_ptr, padded.data_ptr, B, H, W, Ci, pad[0], pad[1], pad[2],
+                    pad[3], _PAD_MODES[self.padding_mode], None)
+            in_codes, pad = padded, (0, 0, 0, 0)
         codes = _ops.qconv2d_i8(
-            g.codes, self._w_ohwi, a_zp=int(g.zp_host) + g.offset, a_scale=g.scale,
+            in_codes, self._w_ohwi, a_zp=int(g.zp_host) + g.offset, a_scale=g.scale,
             w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias, stride=self.stride,
-            pad=self._resolve_pad(x), dilation=self.dilation, groups=self.groups,
+            pad=pad, dilation=self.dilation, groups=self.groups,
             relu=self._fused_relu, out_mode=_ops.OUT_REQUANT_I8, out_scale=self.scale,
             out_zp=self.zero_point, out_qmin=self.out_qdtype.quant_min,
             out_qmax=self.out_qdtype.quant_max, out_offset=off)

@@ -135,3 +135,60 @@ def test_argument_validation():
     with pytest.raises(ValueError):             # zero point without the filter sums
         _ops.qconv2d_i8(x, w, a_zp=3, a_scale=hip(np.float32(1)), w_scale=hip(np.ones(8, np.float32)),
                         pad=(1, 1, 1, 1))
+
+
+_NP_MODE = {1: "reflect", 2: "edge", 3: "wrap"}
+
+
+@pytest.mark.parametrize("mode", [1, 2, 3])
+@pytest.mark.parametrize("shape,pad", [((2, 9, 11, 16), (1, 1, 1, 1)), ((1, 5, 7, 3), (2, 0, 1, 3)),
+                                        ((3, 8, 8, 64), (3, 3, 3, 3)), ((1, 4, 4, 20), (0, 0, 0, 0))])
+def test_padding_modes_on_codes(mode, shape, pad):
+    """F.pad reflect / replicate / circular gathers the image; on a tensor that lies
+    on a grid the codes are gathered the same way (torch's F.pad semantics are
+    numpy's reflect / edge / wrap)."""
+    rng = np.random.default_rng(sum(shape) + mode)
+    x = codes(rng, shape)
+    B, H, W, Cc = shape
+    out = L.Tensor.empty((B, H + pad[0] + pad[1], W + pad[2] + pad[3], Cc), L.int8, "hip")
+    _C.call("lq_pad_nhwc_i8", hip(x).data_ptr, out.data_ptr, B, H, W, Cc, *pad, mode, None)
+    exp = np.pad(x, ((0, 0), (pad[0], pad[1]), (pad[2], pad[3]), (0, 0)), mode=_NP_MODE[mode])
+    assert np.array_equal(out.numpy(), exp)
+    import torch
+
+    tmode = {1: "reflect", 2: "replicate", 3: "circular"}[mode]
+    t = torch.nn.functional.pad(torch.from_numpy(x.astype(np.float32)).permute(0, 3, 1, 2),
+                                (pad[2], pad[3], pad[0], pad[1]), mode=tmode)
+    assert np.array_equal(t.permute(0, 2, 3, 1).numpy().astype(np.int8), exp)
+
+
+@pytest.mark.parametrize("padding_mode", ["reflect", "replicate", "circular"])
+def test_conv_module_with_a_padding_mode(padding_mode):
+    """nnq.Conv2d with padding_mode != zeros: pre-pad, then convolve with padding 0
+    (lucid/nn/modules/conv.py:104-123)."""
+    import lucid_amd.nn.quantized as nnq
+    import lucid_amd.quantization as Q
+    from lucid_amd._tensor import Grid, Tensor
+
+    rng = np.random.default_rng(5)
+    B, H, W, Cin, Cout = 2, 9, 10, 16, 24
+    x = rng.integers(0, 256, (B, H, W, Cin)).astype(np.int16)
+    wq = codes(rng, (Cout, Cin, 3, 3), -127, 127)
+    ws = rng.uniform(0.001, 0.01, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    conv = nnq.Conv2d(Cin, Cout, 3, padding=1)
+    conv.padding_mode = padding_mode
+    state = {"weight_int8": wq, "weight_scale": ws, "weight_zero_point": np.zeros(Cout, np.float32),
+             "bias": bias, "scale": np.float32(0.05), "zero_point": np.float32(120.0)}
+    conv.load_state_dict({k: L.tensor(v, device="hip") for k, v in state.items()})
+    in_scale, in_zp = np.float32(0.02), 128
+    grid = Grid(hip((x - 128).astype(np.int8)), L.tensor(np.float32(in_scale), device="hip"),
+                L.tensor(np.float32(in_zp), device="hip"), Q.quint8, -128, in_zp, "nhwc")
+    y = conv(Tensor.on_grid((B, Cin, H, W), grid))
+    got = y._grid.codes.numpy()
+    xp = np.pad((x - 128).astype(np.int8), ((0, 0), (1, 1), (1, 1), (0, 0)),
+                mode={"reflect": "reflect", "replicate": "edge", "circular": "wrap"}[padding_mode])
+    exp = O.qconv2d(xp, np.ascontiguousarray(wq.transpose(0, 2, 3, 1)), in_zp - 128, in_scale, ws, bias=bias,
+                    out_mode=O.OUT_REQUANT_I8, out_scale=0.05, out_zp=120.0, out_qmin=0, out_qmax=255,
+                    out_offset=-128)
+    assert np.array_equal(got, exp)
