@@ -235,6 +235,23 @@ int lq_gather_rows_f32(const float* src, size_t src_row_stride, float* dst, size
 int lq_assemble_tokens_f32(const float* patches, const float* cls, const float* pos, float* out, int B, int T,
                            int D, lq_stream stream);
 
+/* The other merges of QFunctional (functional_module.py:220-246) on codes:
+ * fq(act(x OP y)), OP = add (0) or mul (1), y a second code tensor or - when qb is
+ * NULL - the float scalar (add_scalar / mul_scalar).  Each operand is dequantized
+ * with its own float32 steps, OP and the optional ReLU are float32, then the usual
+ * requantize. */
+int lq_binary_requant_i8(int op, const int8_t* qa, int a_offset, const float* a_scale, const float* a_zp,
+                         const int8_t* qb, int b_offset, const float* b_scale, const float* b_zp, float scalar,
+                         size_t n, int relu, const float* out_scale, const float* out_zp, int out_qmin,
+                         int out_qmax, int out_offset, int8_t* out, lq_stream stream);
+
+/* One operand of QFunctional.cat (functional_module.py:232-234): codes [rows, cols]
+ * on their own grid re-expressed on the output grid, written with row stride out_ld
+ * into the operand's column slot of the concatenated tensor. */
+int lq_requant_rows_i8(const int8_t* q, int q_offset, const float* scale, const float* zp, size_t rows,
+                       size_t cols, int8_t* out, size_t out_ld, const float* out_scale, const float* out_zp,
+                       int out_qmin, int out_qmax, int out_offset, lq_stream stream);
+
 /* Quantized Linear on a float activation that lies on no grid - literally
  * lucid/nn/quantized/linear.py:199-215: dequantize(weight) -> x @ W^T + bias ->
  * [relu] -> [fake_quantize].  float32 accumulation; for small layers (e.g. the

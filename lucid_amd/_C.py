@@ -137,6 +137,9 @@ _SIGNATURES["lq_patchify_f32"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_sgemm_nt_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_assemble_tokens_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_pad_nhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
+_SIGNATURES["lq_binary_requant_i8"] = [_i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _f, _sz, _i, _vp, _vp, _i, _i,
+                                       _i, _vp, _vp]
+_SIGNATURES["lq_requant_rows_i8"] = [_vp, _i, _vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
 _SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]

@@ -88,6 +88,47 @@ __global__ __launch_bounds__(256) void add_requant_kernel(const int8_t* __restri
     }
 }
 
+// fq(act(x OP y)) on codes with OP in {add, mul} and y either a second code tensor
+// or a float scalar (QFunctional.add / mul / add_relu / add_scalar / mul_scalar,
+// lucid/nn/quantized/functional_module.py:224-246): dequantize each operand with
+// its own float32 steps, apply OP in float32, requantize.
+__global__ __launch_bounds__(256) void binary_requant_kernel(int op, const int8_t* __restrict__ qa, int a_off,
+                                                             const float* sa, const float* za,
+                                                             const int8_t* __restrict__ qb, int b_off,
+                                                             const float* sb, const float* zb, float scalar,
+                                                             size_t n, int relu, const float* S_, const float* Z_,
+                                                             float lo, float hi, int out_off,
+                                                             int8_t* __restrict__ out) {
+    const float s_a = sa[0], z_a = za[0], S = S_[0], Z = Z_[0];
+    const float s_b = qb ? sb[0] : 1.0f, z_b = qb ? zb[0] : 0.0f;
+    const size_t stride = size_t(gridDim.x) * 256;
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+        const float xa = (float(int(qa[i]) - a_off) - z_a) * s_a;
+        const float xb = qb ? (float(int(qb[i]) - b_off) - z_b) * s_b : scalar;
+        float y = op == 0 ? xa + xb : xa * xb;
+        if (relu) y = (y < 0.0f) ? 0.0f : y;
+        const float qv = q_core(y, S, Z, lo, hi);
+        out[i] = int8_t(((qv != qv) ? 0 : int(qv)) + out_off);
+    }
+}
+
+// One operand of a quantized concatenation: codes [rows, cols] on their own grid
+// re-expressed on the output grid, written at row stride out_ld (the operand's
+// column slot inside the concatenated rows).
+__global__ __launch_bounds__(256) void requant_rows_kernel(const int8_t* __restrict__ q, int off, const float* s_,
+                                                           const float* z_, size_t rows, size_t cols,
+                                                           int8_t* __restrict__ out, size_t out_ld, const float* S_,
+                                                           const float* Z_, float lo, float hi, int out_off) {
+    const float s = s_[0], z = z_[0], S = S_[0], Z = Z_[0];
+    const size_t n = rows * cols, stride = size_t(gridDim.x) * 256;
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+        const size_t r = i / cols, c = i - r * cols;
+        const float x = (float(int(q[i]) - off) - z) * s;
+        const float qv = q_core(x, S, Z, lo, hi);
+        out[r * out_ld + c] = int8_t(((qv != qv) ? 0 : int(qv)) + out_off);
+    }
+}
+
 // Global average pool of NHWC codes to float32 [B, C]: the exact integer sum of
 // the codes, then ((sum - HW*(Z + off)) * S) / HW in float32.
 __global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const int8_t* __restrict__ q, int off,
@@ -190,6 +231,40 @@ int lq_add_requant_i8(const int8_t* qa, int a_offset, const float* a_scale, cons
                        a_offset, a_scale, a_zp, qb, b_offset, b_scale, b_zp, n, relu, out_scale, out_zp,
                        float(out_qmin), float(out_qmax), out_offset, out);
     LQ_CHECK_LAUNCH("add_requant_i8");
+    return LQ_OK;
+}
+
+int lq_binary_requant_i8(int op, const int8_t* qa, int a_offset, const float* a_scale, const float* a_zp,
+                         const int8_t* qb, int b_offset, const float* b_scale, const float* b_zp, float scalar,
+                         size_t n, int relu, const float* out_scale, const float* out_zp, int out_qmin,
+                         int out_qmax, int out_offset, int8_t* out, lq_stream stream) {
+    if (n == 0) return LQ_OK;
+    LQ_REQUIRE(op == 0 || op == 1, LQ_ERR_VALUE, "binary_requant_i8: op must be 0 (add) or 1 (mul)");
+    LQ_REQUIRE(qa && out && a_scale && a_zp && out_scale && out_zp && (!qb || (b_scale && b_zp)), LQ_ERR_VALUE,
+               "binary_requant_i8: NULL pointer");
+    LQ_REQUIRE(out_qmin <= out_qmax && out_qmin + out_offset >= -128 && out_qmax + out_offset <= 127,
+               LQ_ERR_VALUE, "binary_requant_i8: output grid [%d,%d] + offset %d does not fit int8", out_qmin,
+               out_qmax, out_offset);
+    hipLaunchKernelGGL(binary_requant_kernel, dim3(grid_for(n, 256)), dim3(256), 0, as_stream(stream), op, qa,
+                       a_offset, a_scale, a_zp, qb, b_offset, b_scale, b_zp, scalar, n, relu, out_scale, out_zp,
+                       float(out_qmin), float(out_qmax), out_offset, out);
+    LQ_CHECK_LAUNCH("binary_requant_i8");
+    return LQ_OK;
+}
+
+int lq_requant_rows_i8(const int8_t* q, int q_offset, const float* scale, const float* zp, size_t rows,
+                       size_t cols, int8_t* out, size_t out_ld, const float* out_scale, const float* out_zp,
+                       int out_qmin, int out_qmax, int out_offset, lq_stream stream) {
+    if (rows * cols == 0) return LQ_OK;
+    LQ_REQUIRE(q && out && scale && zp && out_scale && out_zp, LQ_ERR_VALUE, "requant_rows_i8: NULL pointer");
+    LQ_REQUIRE(out_ld >= cols, LQ_ERR_SHAPE, "requant_rows_i8: output row stride smaller than the row");
+    LQ_REQUIRE(out_qmin <= out_qmax && out_qmin + out_offset >= -128 && out_qmax + out_offset <= 127,
+               LQ_ERR_VALUE, "requant_rows_i8: output grid [%d,%d] + offset %d does not fit int8", out_qmin,
+               out_qmax, out_offset);
+    hipLaunchKernelGGL(requant_rows_kernel, dim3(grid_for(rows * cols, 256)), dim3(256), 0, as_stream(stream), q,
+                       q_offset, scale, zp, rows, cols, out, out_ld, out_scale, out_zp, float(out_qmin),
+                       float(out_qmax), out_offset);
+    LQ_CHECK_LAUNCH("requant_rows_i8");
     return LQ_OK;
 }
 

@@ -272,6 +272,35 @@ def test_qfunctional_add_relu_matches_oracle():
     assert np.array_equal(out2.numpy().view(np.uint32), ref2.view(np.uint32))
 
 
+def test_qfunctional_mul_scalars_and_cat_match_the_float_composition():
+    """functional_module.py:220-246: each merge is fake_quantize(op(x, y)) on
+    float-carried operands; on codes it must give the same bits."""
+    rng = np.random.default_rng(6)
+    a = (rng.standard_normal((4, 300)) * 2).astype(np.float32)
+    b = (rng.standard_normal((4, 300)) * 3).astype(np.float32)
+    qa = nnq.Quantize(hip(np.float32(0.05)), hip(np.float32(120.0)))
+    qb = nnq.Quantize(hip(np.float32(0.07)), hip(np.float32(131.0)))
+    xa, xb = O.fake_quantize(a, 0.05, 120.0, 0, 255), O.fake_quantize(b, 0.07, 131.0, 0, 255)
+    f = nnq.QFunctional(hip(np.float32(0.11)), hip(np.float32(125.0)))
+    same = lambda got, ref: np.array_equal(got.numpy().view(np.uint32), ref.view(np.uint32))
+    assert same(f.mul(qa(hip(a)), qb(hip(b))), O.fake_quantize(xa * xb, 0.11, 125.0, 0, 255))
+    assert same(f.add_scalar(qa(hip(a)), 0.3), O.fake_quantize(xa + np.float32(0.3), 0.11, 125.0, 0, 255))
+    assert same(f.mul_scalar(qa(hip(a)), -1.7), O.fake_quantize(xa * np.float32(-1.7), 0.11, 125.0, 0, 255))
+    got = f.cat([qa(hip(a)), qb(hip(b))], dim=1)
+    assert got.shape == (4, 600)
+    assert same(got, O.fake_quantize(np.concatenate([xa, xb], 1), 0.11, 125.0, 0, 255))
+    got0 = f.cat([qa(hip(a)), qb(hip(b))], dim=0)
+    assert got0.shape == (8, 300)
+    assert same(got0, O.fake_quantize(np.concatenate([xa, xb], 0), 0.11, 125.0, 0, 255))
+    # channel concatenation of 4-d activations (stored NHWC)
+    u = (rng.standard_normal((2, 5, 6, 7)) * 2).astype(np.float32)
+    v = (rng.standard_normal((2, 9, 6, 7)) * 2).astype(np.float32)
+    xu, xv = O.fake_quantize(u, 0.05, 120.0, 0, 255), O.fake_quantize(v, 0.07, 131.0, 0, 255)
+    got4 = f.cat([qa(hip(u)), qb(hip(v))], dim=1)
+    assert got4.shape == (2, 14, 6, 7)
+    assert same(got4, O.fake_quantize(np.concatenate([xu, xv], 1), 0.11, 125.0, 0, 255))
+
+
 def test_observers_known_answers_on_device():
     # lucid/test/unit/quantization/test_observer.py:12-17,43-50
     obs = Q.MinMaxObserver()
