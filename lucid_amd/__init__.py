@@ -35,6 +35,8 @@ from . import quantization
 from . import nn
 from . import backends
 from . import graph
+from . import serialization
+from .serialization import load, save
 
 __version__ = "0.1.0"
 

@@ -140,7 +140,9 @@ class Tensor:
 
     @staticmethod
     def from_numpy(a, device="hip") -> "Tensor":
-        a = np.ascontiguousarray(a)
+        a = np.asarray(a)
+        if not a.flags.c_contiguous:  # (np.ascontiguousarray would also turn 0-d into 1-d)
+            a = np.ascontiguousarray(a)
         dt = as_dtype(a.dtype)
         if _norm_device(device) == "cpu":
             return Tensor(a.shape, dt, "cpu", host=a)
@@ -233,7 +235,9 @@ class Tensor:
     def copy_from(self, a) -> "Tensor":
         """Overwrite this tensor's storage with a host array of the same shape
         and dtype (the way to feed a new batch to a captured graph)."""
-        a = np.ascontiguousarray(a, dtype=self.dtype.np)
+        a = np.asarray(a, dtype=self.dtype.np)
+        if not a.flags.c_contiguous:
+            a = np.ascontiguousarray(a)
         if a.shape != self.shape:
             raise _C.ShapeMismatch(f"copy_from: {a.shape} into {self.shape}")
         if self.device == "cpu":

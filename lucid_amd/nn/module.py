@@ -88,7 +88,11 @@ class Module:
             for bname in list(mod._buffers):
                 key = f"{name}.{bname}" if name else bname
                 if key in state:
-                    mod._buffers[bname] = state[key]
+                    old, new = mod._buffers[bname], state[key]
+                    # a checkpoint holds host tensors: keep each buffer on the device it lives on
+                    if old is not None and isinstance(new, Tensor) and new.device != old.device:
+                        new = new.to(old.device)
+                    mod._buffers[bname] = new
                     mod._state_loaded(bname)
 
     def _state_loaded(self, name: str) -> None:

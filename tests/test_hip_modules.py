@@ -213,6 +213,35 @@ class TestStaticPTQ:
         y_fp = np.maximum(x @ w1.T + b1, 0) @ w2.T + b2
         assert np.abs(y.numpy() - y_fp).mean() / np.abs(y_fp).mean() < 0.05
 
+    @pytest.mark.parametrize("ext", ["lucid", "safetensors"])
+    def test_checkpoint_file_round_trip_is_bit_equal(self, tmp_path, ext):
+        """test_static_ptq.py:132-145: save(state_dict) -> load -> load_state_dict into a
+        freshly calibrated twin gives the same output bits, and int8 stays int8."""
+        rng = np.random.default_rng(0)
+        m, params = _static_model(rng)
+        prepared = Q.prepare(m, Q.get_default_qconfig())
+        _calibrate(prepared, params, rng)
+        qm = Q.convert(prepared)
+        x = hip(rng.standard_normal((64, 16)).astype(np.float32))
+        before = qm(x).numpy()
+        path = str(tmp_path / f"qmodel.{ext}")
+        if ext == "lucid":
+            L.save(qm.state_dict(), path)
+        else:
+            L.serialization.save_safetensors(qm.state_dict(), path)
+        loaded = L.load(path)
+        assert loaded["fc1.weight_int8"].dtype is L.int8 and loaded["fc1.weight_int8"].device == "cpu"
+        assert loaded["fc1.scale"].shape == ()
+        rng2 = np.random.default_rng(77)  # a twin with other weights and another calibration
+        m2, params2 = _static_model(rng2)
+        prepared2 = Q.prepare(m2, Q.get_default_qconfig())
+        _calibrate(prepared2, params2, rng2)
+        qm2 = Q.convert(prepared2)
+        assert not np.array_equal(qm2(x).numpy(), before)
+        qm2.load_state_dict(loaded)
+        assert qm2.fc1.weight_int8.device == "hip"
+        assert np.array_equal(qm2(x).numpy().view(np.uint32), before.view(np.uint32))
+
     def test_uncalibrated_convert_warns(self):
         # lucid/test/unit/quantization/test_safety.py (warning text "never saw")
         m, _ = _static_model(np.random.default_rng(1))
