@@ -160,6 +160,22 @@ int lq_minmax_fold(const float* run_min, const float* run_max, const float* cur_
                    const float* cur_max, size_t C, int run_is_scalar, float* out_min,
                    float* out_max, lq_stream stream);
 
+/* Moving-average observers (lucid/quantization/observer.py:490-506 per tensor,
+ * :1000-1018 per channel): out = seed ? cur : run + c * (cur - run) in float32.
+ * Per tensor the seed test is isinf(run_min) elementwise; per channel everything is
+ * seeded when every running minimum is still infinite.  run_* hold one value when
+ * run_is_scalar (the +-inf start), else C. */
+int lq_minmax_ema(const float* run_min, const float* run_max, const float* cur_min, const float* cur_max,
+                  size_t C, int run_is_scalar, int per_channel, float averaging_constant, float* out_min,
+                  float* out_max, lq_stream stream);
+
+/* lucid.histc (IBackend::histogram_forward, CpuBackend.h:13276-13316) on float32
+ * input: `bins` equal-width buckets over [lo, hi], the bucket taken in double
+ * arithmetic as (int64)((v - lo) / ((hi - lo) / bins)), the right edge folded into
+ * the last bucket, values outside skipped; float32 counts out (HistogramObserver's
+ * running histogram, observer.py:819-838). */
+int lq_histc_f32(const float* x, size_t n, double lo, double hi, int bins, float* out, lq_stream stream);
+
 /* QFunctional.add / add_relu on codes (nn/quantized/functional_module.py:216-230):
  * out = quantize(relu?((qa - za)*sa + (qb - zb)*sb)) with every qparam a device
  * scalar.  Codes are int8 as stored (code + offset). */

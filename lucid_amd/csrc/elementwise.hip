@@ -42,6 +42,65 @@ __global__ void minmax_fold_kernel(float* run_min, float* run_max, const float* 
     out_max[c] = (rmx != rmx || cmx != cmx) ? qnan : (rmx > cmx ? rmx : cmx);
 }
 
+// Moving-average observers (lucid/quantization/observer.py:490-506,1000-1018):
+// new = seed ? cur : run + c * (cur - run), float32 steps in that order.
+// Per-tensor (mode 0): seed where the running minimum is infinite, elementwise.
+// Per-channel (mode 1): seed everything when EVERY running minimum is infinite
+// (the scalar +-inf start), else average everything.  One block.
+__global__ __launch_bounds__(1024) void minmax_ema_kernel(const float* run_min, const float* run_max,
+                                                          const float* cur_min, const float* cur_max, size_t C,
+                                                          int run_is_scalar, int mode, float c, float* out_min,
+                                                          float* out_max) {
+    __shared__ int s_not_inf;
+    if (threadIdx.x == 0) s_not_inf = 0;
+    __syncthreads();
+    if (mode == 1) {
+        const size_t nrun = run_is_scalar ? 1 : C;
+        int any = 0;
+        for (size_t i = threadIdx.x; i < nrun; i += 1024) any |= !isinf(run_min[i]);
+        if (any) atomicOr(&s_not_inf, 1);
+        __syncthreads();
+    }
+    const bool seed_all = mode == 1 && s_not_inf == 0;
+    for (size_t i = threadIdx.x; i < C; i += 1024) {
+        const float rmn = run_min[run_is_scalar ? 0 : i], rmx = run_max[run_is_scalar ? 0 : i];
+        const float cmn = cur_min[i], cmx = cur_max[i];
+        const bool seed = mode == 1 ? seed_all : isinf(rmn);
+        const float dmn = cmn - rmn, dmx = cmx - rmx;
+        const float emn = c * dmn, emx = c * dmx;
+        out_min[i] = seed ? cmn : rmn + emn;
+        out_max[i] = seed ? cmx : rmx + emx;
+    }
+}
+
+// lucid.histc (CpuBackend.h:13276-13316): `bins` equal-width buckets over
+// [lo, hi] in double arithmetic, bin = (int64)((v - lo) / step) with the right
+// edge folded into the last bin, values outside the range skipped.  Counts are
+// exact integers (LDS then global atomics) and leave as float32.
+__global__ __launch_bounds__(256) void histc_kernel(const float* __restrict__ x, size_t n, double lo, double hi,
+                                                    double step, int bins,
+                                                    unsigned long long* __restrict__ counts) {
+    extern __shared__ unsigned s_hist[];
+    for (int b = threadIdx.x; b < bins; b += 256) s_hist[b] = 0;
+    __syncthreads();
+    const size_t stride = size_t(gridDim.x) * 256;
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+        const double v = double(x[i]);
+        if (v < lo || v > hi) continue;  // NaN fails neither test in C++; see below
+        long long bin = (long long)((v - lo) / step);
+        if (bin >= bins) bin = bins - 1;
+        if (bin >= 0) atomicAdd(&s_hist[bin], 1u);
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < bins; b += 256)
+        if (s_hist[b]) atomicAdd(&counts[b], (unsigned long long)s_hist[b]);
+}
+
+__global__ void histc_finish_kernel(const unsigned long long* counts, int bins, float* out) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < bins) out[b] = float(double(counts[b]));  // the reference counts in double, then casts
+}
+
 __device__ __forceinline__ float q_core(float x, float s, float z, float lo, float hi) {
     float t = x / s;
     float r = __builtin_rintf(t);
@@ -214,6 +273,42 @@ int lq_minmax_fold(const float* run_min, const float* run_max, const float* cur_
                        as_stream(stream), const_cast<float*>(run_min), const_cast<float*>(run_max),
                        cur_min, cur_max, C, run_is_scalar, out_min, out_max);
     LQ_CHECK_LAUNCH("minmax_fold");
+    return LQ_OK;
+}
+
+int lq_minmax_ema(const float* run_min, const float* run_max, const float* cur_min, const float* cur_max,
+                  size_t C, int run_is_scalar, int per_channel, float averaging_constant, float* out_min,
+                  float* out_max, lq_stream stream) {
+    if (C == 0) return LQ_OK;
+    LQ_REQUIRE(run_min && run_max && cur_min && cur_max && out_min && out_max, LQ_ERR_VALUE,
+               "minmax_ema: NULL pointer");
+    hipLaunchKernelGGL(minmax_ema_kernel, dim3(1), dim3(1024), 0, as_stream(stream), run_min, run_max, cur_min,
+                       cur_max, C, run_is_scalar, per_channel ? 1 : 0, averaging_constant, out_min, out_max);
+    LQ_CHECK_LAUNCH("minmax_ema");
+    return LQ_OK;
+}
+
+int lq_histc_f32(const float* x, size_t n, double lo, double hi, int bins, float* out, lq_stream stream) {
+    LQ_REQUIRE(out, LQ_ERR_VALUE, "histc: NULL output");
+    LQ_REQUIRE(bins > 0 && bins <= 16384, LQ_ERR_VALUE, "histc: bins must be in 1..16384 (got %d)", bins);
+    LQ_REQUIRE(hi > lo, LQ_ERR_VALUE, "histc: hi must be > lo");  // Histogram.cpp:105-106
+    LQ_REQUIRE(n == 0 || x, LQ_ERR_VALUE, "histc: NULL input");
+    hipStream_t st = as_stream(stream);
+    void* ws = nullptr;
+    int rc = workspace(size_t(bins) * sizeof(unsigned long long), &ws);
+    if (rc) return rc;
+    auto* counts = static_cast<unsigned long long*>(ws);
+    rc = lq_fill_bytes(counts, 0, size_t(bins) * sizeof(unsigned long long), stream);
+    if (rc) return rc;
+    if (n) {
+        size_t blocks = (n + 256 * 16 - 1) / (256 * 16);
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(histc_kernel, dim3(unsigned(blocks)), dim3(256), size_t(bins) * sizeof(unsigned), st, x,
+                           n, lo, hi, (hi - lo) / double(bins), bins, counts);
+        LQ_CHECK_LAUNCH("histc");
+    }
+    hipLaunchKernelGGL(histc_finish_kernel, dim3(unsigned((bins + 255) / 256)), dim3(256), 0, st, counts, bins, out);
+    LQ_CHECK_LAUNCH("histc_finish");
     return LQ_OK;
 }
 

@@ -18,7 +18,8 @@ from ._qscheme import (
     quint8,
 )
 
-from .observer import (FixedQParamsObserver, MinMaxObserver, ObserverBase,
+from .observer import (FixedQParamsObserver, HistogramObserver, MinMaxObserver,
+                       MovingAverageMinMaxObserver, MovingAveragePerChannelMinMaxObserver, ObserverBase,
                        PerChannelMinMaxObserver)
 from .qconfig import QConfig, get_default_qconfig
 
@@ -36,6 +37,7 @@ def __getattr__(name):
 
 __all__ = [
     "ObserverBase", "MinMaxObserver", "PerChannelMinMaxObserver", "FixedQParamsObserver",
+    "MovingAverageMinMaxObserver", "MovingAveragePerChannelMinMaxObserver", "HistogramObserver",
     "QConfig", "get_default_qconfig", "prepare", "convert", "quantize_dynamic", "fuse_modules",
     "QScheme", "per_tensor_affine", "per_tensor_symmetric", "per_channel_affine",
     "per_channel_symmetric", "QDtype", "qint8", "quint8", "qint32", "qint4", "QParams",

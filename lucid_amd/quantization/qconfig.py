@@ -7,7 +7,7 @@ from dataclasses import dataclass
 from typing import Callable
 
 from ._qscheme import per_channel_symmetric, per_tensor_affine, qint8, quint8
-from .observer import MinMaxObserver, ObserverBase, PerChannelMinMaxObserver
+from .observer import HistogramObserver, ObserverBase, PerChannelMinMaxObserver
 
 
 @dataclass(frozen=True)
@@ -17,12 +17,10 @@ class QConfig:
 
 
 def get_default_qconfig() -> QConfig:
-    """quint8 affine activations, per-channel symmetric qint8 weights along
-    axis 0.  Lucid's default activation observer is the histogram one
-    (``qconfig.py``), which belongs to the calibration side that this backend
-    does not rebuild; the min/max observer is used here."""
+    """Histogram observer on quint8 affine activations, per-channel symmetric
+    qint8 weights along axis 0 (``qconfig.py:150-190``)."""
     return QConfig(
-        activation=MinMaxObserver.with_args(qscheme=per_tensor_affine, qdtype=quint8),
+        activation=HistogramObserver.with_args(qscheme=per_tensor_affine, qdtype=quint8),
         weight=PerChannelMinMaxObserver.with_args(ch_axis=0, qscheme=per_channel_symmetric,
                                                   qdtype=qint8),
     )
