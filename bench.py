@@ -448,6 +448,11 @@ def main() -> int:
                                      "frac_of_8TBs": round(rs["gbs"] / PEAK_HBM_GBS, 4),
                                      "TOP/s": round(rs["kernel_tops"], 2), "bytes": rs["bytes"]}
             del rs["tensors"]
+        # the same layer at a prefill-sized M: more tiles per CU, better-filled rounds
+        rl = bench_linear(L, Q, _C, _ops, 8192, K, N, max(10, args.steps // 2), max(3, args.warmup // 2), seed=5)
+        extra["linear_m8192"] = {"us": round(rl["avg_kernel_ms"] * 1e3, 2), "TOP/s": round(rl["kernel_tops"], 2),
+                                 "frac_of_int8_peak": round(rl["kernel_tops"] / PEAK_INT8_TOPS, 4)}
+        del rl["tensors"]
         extra["quant_roundtrip_4096x4096x16"] = bench_quant_roundtrip(
             L, Q, _C, max(10, args.steps // 2), max(3, args.warmup // 2))
         extra["dynamic_mlp_784_256_10_batch64"] = bench_dynamic_mlp(L, Q, _C, args.steps, args.warmup)

@@ -190,6 +190,32 @@ int lq_add_requant_i8(const int8_t* qa, int a_offset, const float* a_scale, cons
 int lq_global_avgpool_nhwc_i8(const int8_t* q, int code_offset, int B, int H, int W, int C,
                               const float* scale, const float* zp, float* out, lq_stream stream);
 
+/* ------------------------------------------------- group-wise weight-only path */
+/* engine.quantized.{quantize, dequantize, quantized_matmul}
+ * (lucid/_C/bindings/bind_quantized.cpp:18-25; lucid/_C/ops/quantized/QuantizedMatmul.cpp:47-115;
+ * lucid/quantization/_qgemm.py:69-320), which Lucid implements by calling MLX.  MLX is
+ * not part of the Lucid checkout; these follow the documented contract
+ * (_qgemm.py:84-97,167-171): per row and per group of group_size (32 / 64 / 128)
+ * consecutive elements, s = (max - min) / (2^bits - 1), beta = min,
+ * c = clip(round((w - beta) / s), 0, 2^bits - 1), w ~ c * s + beta; bits is 4 or 8;
+ * codes are packed little-endian into 32-bit words (code j at bits [j*bits, (j+1)*bits)):
+ * packed is [N, K*bits/32], scales and biases [N, K/group_size].  Decoding takes scales
+ * and biases as given, so weights packed elsewhere under this contract load unchanged.
+ * lq_wq_matmul: out[M,N] = x[M,K] . w_hat^T in float32 (transpose = True of
+ * _qgemm.quantized_matmul); M <= 16 streams the packed weight once per four rows,
+ * larger M decodes into the workspace and runs the float32 GEMM. */
+int lq_wq_quantize(const float* w, int N, int K, int group_size, int bits, uint32_t* packed, float* scales,
+                   float* biases, lq_stream stream);
+int lq_wq_dequantize(const uint32_t* packed, const float* scales, const float* biases, int N, int K, int group_size,
+                     int bits, float* out, lq_stream stream);
+int lq_wq_matmul(const float* x, const uint32_t* packed, const float* scales, const float* biases, int M, int N, int K,
+                 int group_size, int bits, float* out, lq_stream stream);
+
+/* y[m,n] = act(y[m,n] + bias[n]) in place on float32 [M,N]; bias may be NULL, act is
+ * ReLU when relu != 0: the float bias / fused ReLU after the weight-only matmul
+ * (lucid/nn/quantized/mlx_linear.py forward). */
+int lq_bias_act_f32(float* y, const float* bias, size_t M, int N, int relu, lq_stream stream);
+
 /* ------------------------------------------------- ranges kept by the producer */
 /* nnqd.Linear takes x.min() / x.max() of its input on every forward
  * (lucid/nn/quantized/dynamic/linear.py:87-89): a full pass over a tensor some

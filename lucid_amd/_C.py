@@ -142,6 +142,10 @@ _SIGNATURES["lq_binary_requant_i8"] = [_i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp,
 _SIGNATURES["lq_requant_rows_i8"] = [_vp, _i, _vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_minmax_ema"] = [_vp, _vp, _vp, _vp, _sz, _i, _i, _f, _vp, _vp, _vp]
 _SIGNATURES["lq_histc_f32"] = [_vp, _sz, C.c_double, C.c_double, _i, _vp, _vp]
+_SIGNATURES["lq_wq_quantize"] = [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp]
+_SIGNATURES["lq_wq_dequantize"] = [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]
+_SIGNATURES["lq_wq_matmul"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp]
+_SIGNATURES["lq_bias_act_f32"] = [_vp, _vp, _sz, _i, _i, _vp]
 _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
 _SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]

@@ -42,6 +42,18 @@ __global__ void minmax_fold_kernel(float* run_min, float* run_max, const float* 
     out_max[c] = (rmx != rmx || cmx != cmx) ? qnan : (rmx > cmx ? rmx : cmx);
 }
 
+// y[m, n] = act(y[m, n] + bias[n]) in place: the float bias and optional ReLU that
+// follow the weight-only matmul (lucid/nn/quantized/mlx_linear.py forward).
+__global__ __launch_bounds__(256) void bias_act_kernel(float* __restrict__ y, const float* __restrict__ bias,
+                                                       size_t total, int N, int relu) {
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    float v = y[i];
+    if (bias) v = v + bias[i % N];
+    if (relu) v = (v < 0.0f) ? 0.0f : v;
+    y[i] = v;
+}
+
 // Moving-average observers (lucid/quantization/observer.py:490-506,1000-1018):
 // new = seed ? cur : run + c * (cur - run), float32 steps in that order.
 // Per-tensor (mode 0): seed where the running minimum is infinite, elementwise.
@@ -273,6 +285,17 @@ int lq_minmax_fold(const float* run_min, const float* run_max, const float* cur_
                        as_stream(stream), const_cast<float*>(run_min), const_cast<float*>(run_max),
                        cur_min, cur_max, C, run_is_scalar, out_min, out_max);
     LQ_CHECK_LAUNCH("minmax_fold");
+    return LQ_OK;
+}
+
+int lq_bias_act_f32(float* y, const float* bias, size_t M, int N, int relu, lq_stream stream) {
+    if (M * size_t(N) == 0) return LQ_OK;
+    LQ_REQUIRE(y && N > 0, LQ_ERR_VALUE, "bias_act: bad arguments");
+    const size_t total = M * size_t(N);
+    LQ_REQUIRE((total + 255) / 256 < 0x7fffffffull, LQ_ERR_SHAPE, "bias_act: tensor too large");
+    hipLaunchKernelGGL(bias_act_kernel, dim3(unsigned((total + 255) / 256)), dim3(256), 0, as_stream(stream), y,
+                       bias, total, N, relu);
+    LQ_CHECK_LAUNCH("bias_act");
     return LQ_OK;
 }
 

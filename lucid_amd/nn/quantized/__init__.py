@@ -6,7 +6,8 @@ from .functional_module import FloatFunctional, QFunctional
 from .conv import Conv2d
 from .intrinsic import ConvReLU2d, LinearReLU
 from .linear import Linear
+from .mlx_linear import QuantizedLinearMLX
 from .modules import DeQuantize, DeQuantStub, Quantize, QuantStub, QuantWrapper
 
-__all__ = ["Linear", "LinearReLU", "Conv2d", "ConvReLU2d", "Quantize", "DeQuantize", "QuantStub", "DeQuantStub",
+__all__ = ["QuantizedLinearMLX", "Linear", "LinearReLU", "Conv2d", "ConvReLU2d", "Quantize", "DeQuantize", "QuantStub", "DeQuantStub",
            "QuantWrapper", "QFunctional", "FloatFunctional", "dynamic"]
