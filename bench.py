@@ -128,6 +128,34 @@ def bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup, seed=1):
                 gbs=bytes_alg / avg_ms / 1e6, tensors=t)
 
 
+def probe_mfma_ceiling(L, _C, xq, wq, ms_target=40.0):
+    """TOP/s of a loop of nothing but int8 MFMAs over register operands taken from
+    the benchmark's own activation and weight codes (two wavefronts per SIMD, eight
+    independent accumulators each): what the matrix cores sustain for this data under
+    the board's power limit, before any data movement.  Long enough (tens of ms) for
+    the clock to settle."""
+    sink = L.Tensor.empty((1,), L.int32, "hip")
+    ops = C.c_double()
+    nbytes = min(xq.numel, wq.numel)
+
+    def run(iters):
+        evs = _events(_C, 2)
+        _C.call("lq_event_record", evs[0], None)
+        _C.call("lq_probe_mfma_i8", xq.data_ptr, wq.data_ptr, nbytes, iters, sink.data_ptr, C.byref(ops), None)
+        _C.call("lq_event_record", evs[1], None)
+        _C.call("lq_event_sync", evs[1])
+        ms = _elapsed_ms(_C, evs[0], evs[1])
+        for e in evs:
+            _C.call("lq_event_destroy", e)
+        return ms
+
+    ms = run(2000)
+    iters = int(max(2000, min(2_000_000, 2000 * ms_target / max(ms, 1e-3))))
+    run(iters)
+    ms = run(iters)
+    return ops.value / ms / 1e9
+
+
 def bench_act_quant_plus_linear(L, Q, _C, _ops, t, M, K, N, steps, warmup):
     """The same layer with the dynamic per-token activation quantization in the
     timed region: min/max -> qparams -> quantize -> GEMM (four launches)."""
@@ -308,6 +336,29 @@ def bench_dynamic_mlp(L, Q, _C, steps, warmup):
             "launches_per_forward": 9}
 
 
+def bench_weight_only(L, _C, steps, warmup, K=4096, N=11008, gs=64):
+    """Group-wise weight-only Linear (float32 activations, int4 / int8 weights decoded
+    inside the product) at decode-sized M: the launch streams the packed weight once, so
+    the figure of merit is bytes of (codes + scales + biases) per second."""
+    from lucid_amd.quantization import _qgemm
+
+    rng = np.random.default_rng(9)
+    w = L.tensor((rng.standard_normal((N, K)) * 0.05).astype(np.float32), device="hip")
+    out = {}
+    for bits in (4, 8):
+        packed, scales, biases = _qgemm.quantize(w, gs, bits)
+        nbytes = N * K * bits // 8 + 2 * 4 * N * (K // gs)
+        for m in (1, 16):
+            x = L.tensor(rng.standard_normal((m, K)).astype(np.float32), device="hip")
+            fn = lambda: _qgemm.quantized_matmul(x, packed, scales, biases, True, gs, bits)
+            _, per = time_launches(_C, fn, steps, warmup)
+            us = float(np.median(per)) * 1e3
+            gbs = nbytes / (us * 1e-6) / 1e9
+            out[f"w{bits}_m{m}"] = {"us": round(us, 2), "GB/s": round(gbs, 1),
+                                    "frac_of_8TBs": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+    return out
+
+
 def bench_vit_linears(L, Q, _C, _ops, steps, warmup):
     """The four Linear shapes of a ViT-B/16 encoder block at batch 64 (12 608
     token rows), dynamic-quantized as nnqd.Linear does: per-tensor affine quint8
@@ -433,6 +484,10 @@ def main() -> int:
             "algorithmic_ops": r["ops"],
         },
     }
+    # the same operand codes through a loop of MFMAs alone: the data-dependent ceiling
+    ceiling = probe_mfma_ceiling(L, _C, r["tensors"]["xq"], r["tensors"]["wq"])
+    line["roofline"]["mfma_only_same_operands_tops"] = round(ceiling, 1)
+    line["roofline"]["frac_of_mfma_only"] = round(r["kernel_tops"] / ceiling, 4)
     if not args.no_extra:
         extra = {}
         extra["linear_with_dynamic_act_quant_TOPS"] = round(
@@ -453,6 +508,7 @@ def main() -> int:
         extra["linear_m8192"] = {"us": round(rl["avg_kernel_ms"] * 1e3, 2), "TOP/s": round(rl["kernel_tops"], 2),
                                  "frac_of_int8_peak": round(rl["kernel_tops"] / PEAK_INT8_TOPS, 4)}
         del rl["tensors"]
+        extra["weight_only_group64_k4096_n11008"] = bench_weight_only(L, _C, args.steps, args.warmup)
         extra["quant_roundtrip_4096x4096x16"] = bench_quant_roundtrip(
             L, Q, _C, max(10, args.steps // 2), max(3, args.warmup // 2))
         extra["dynamic_mlp_784_256_10_batch64"] = bench_dynamic_mlp(L, Q, _C, args.steps, args.warmup)

@@ -109,6 +109,17 @@ int lq_op_info(int index, const char** name, int* version, int* deterministic);
 int lq_fill_normal(float* x, size_t n, uint64_t seed, float outlier_prob, float outlier_gain,
                    lq_stream stream);
 int lq_fill_uniform_i8(int8_t* x, size_t n, uint64_t seed, int lo, int hi, lq_stream stream);
+/* Matrix-core rate probe for roofline accounting: 2 blocks per CU, each
+ * wavefront issuing `iters` rounds of eight v_mfma_i32_32x32x32_i8 on eight
+ * independent accumulators, operands taken from a[] / b[] (at least 32 KiB
+ * each, 16-byte aligned) and rotated so that operand bits toggle as they do in
+ * a GEMM over that data; no LDS or memory traffic in the loop.  *ops receives
+ * the integer operations launched (2*32*32*32 per instruction); time the call
+ * with events to get the rate the matrix cores sustain under the power limit
+ * for these operand statistics.  sink: one int of device memory.  No
+ * counterpart in Lucid. */
+int lq_probe_mfma_i8(const int8_t* a, const int8_t* b, size_t nbytes, int iters, int* sink,
+                     double* ops, lq_stream stream);
 /* Plain device copy kernel (n bytes, 16-byte vectors): the calibration
  * workload for hardware-counter scaling. */
 int lq_copy_kernel(void* dst, const void* src, size_t nbytes, lq_stream stream);

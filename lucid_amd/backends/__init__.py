@@ -3,9 +3,14 @@
 
 * ``"auto"``      - use the HIP int8 kernels when the library and a device are there.
 * ``"hip"``       - require them (raises ``GpuNotAvailable`` otherwise).
-* ``"reference"`` / ``"mlx_group"`` - Lucid's own engines; accepted as values so
-  that code written against Lucid keeps working, but they select paths that live
-  in Lucid, not here: modules built by this package always run the HIP kernels.
+* ``"mlx_group"`` - ``convert`` / ``quantize_dynamic`` build the group-wise
+  weight-only ``QuantizedLinearMLX`` (int4 / int8 weights, float activations) for
+  the Linear family, as Lucid does when its MLX engine is active; the kernels are
+  the HIP ones.  Unlike Lucid, ``"auto"`` does not pick this form: the default here
+  is the int8 x int8 integer GEMM.
+* ``"reference"`` - Lucid's dequantize-to-float engine; accepted so that code
+  written against Lucid keeps working, but modules built by this package always
+  run the HIP kernels.
 """
 
 from __future__ import annotations
@@ -33,7 +38,13 @@ class _QuantizedBackend:
         self._engine = value
 
     def use_mlx(self) -> bool:
-        return False  # no MLX on this platform
+        """Whether ``convert`` / ``quantize_dynamic`` route the Linear family to the
+        group-wise weight-only form (only when asked for by name)."""
+        if self._engine == "mlx_group":
+            if not self.available:
+                raise _C.GpuNotAvailable("quantized.engine = 'mlx_group' but no HIP device / library")
+            return True
+        return False
 
     def use_hip(self) -> bool:
         """Whether the HIP kernels should run given the current mode."""

@@ -441,6 +441,37 @@ __global__ void fill_uniform_i8_kernel(int8_t* x, size_t n, uint64_t seed, int l
     }
 }
 
+typedef int probe_v16i __attribute__((ext_vector_type(16)));
+typedef int probe_v4i __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void probe_mfma_i8_kernel(const int8_t* __restrict__ a,
+                                                            const int8_t* __restrict__ b, int iters,
+                                                            int* __restrict__ sink) {
+    probe_v16i acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0;
+    probe_v4i ra[8], rb[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        ra[i] = reinterpret_cast<const probe_v4i*>(a)[i * 256 + threadIdx.x];
+        rb[i] = reinterpret_cast<const probe_v4i*>(b)[i * 256 + threadIdx.x];
+    }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[i], rb[(i * 3 + 1) & 7], acc[i], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) s ^= acc[i][j];
+    // keeps the accumulators live; one word per block, written by one lane
+    if (threadIdx.x == 0) sink[0] = s;
+}
+
 __global__ void fill_bytes_kernel(uint8_t* x, size_t n, uint8_t v) {
     size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     size_t stride = size_t(gridDim.x) * blockDim.x;
@@ -480,6 +511,29 @@ int lq_fill_uniform_i8(int8_t* x, size_t n, uint64_t seed, int lo, int hi, lq_st
     hipLaunchKernelGGL(fill_uniform_i8_kernel, dim3(blocks_for(n, 256, 65536)), dim3(256), 0,
                        as_stream(stream), x, n, seed, lo, hi - lo + 1);
     LQ_CHECK_LAUNCH("fill_uniform_i8");
+    return LQ_OK;
+}
+
+// Matrix-core rate probe: every wavefront keeps eight 32x32 int32 accumulators
+// and issues `iters` rounds of eight v_mfma_i32_32x32x32_i8 whose operands
+// rotate over eight register sets taken from `a` and `b`, so operand bits
+// toggle between instructions the way they do in a GEMM over that data.  No
+// LDS or memory traffic inside the loop: the rate is what the matrix cores
+// sustain for these operand statistics under the board's power limit.
+int lq_probe_mfma_i8(const int8_t* a, const int8_t* b, size_t nbytes, int iters, int* sink, double* ops,
+                     lq_stream stream) {
+    LQ_REQUIRE(a && b && sink && ops, LQ_ERR_VALUE, "probe_mfma_i8: NULL pointer");
+    LQ_REQUIRE(iters > 0, LQ_ERR_VALUE, "probe_mfma_i8: iters must be positive");
+    LQ_REQUIRE(nbytes >= size_t(256) * 8 * 16, LQ_ERR_SHAPE, "probe_mfma_i8: need at least 32 KiB of operand data");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0, LQ_ERR_VALUE,
+               "probe_mfma_i8: operands must be 16-byte aligned");
+    int dev = 0, cus = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    LQ_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int blocks = 2 * cus;  // two wavefronts per SIMD
+    hipLaunchKernelGGL(probe_mfma_i8_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), a, b, iters, sink);
+    LQ_CHECK_LAUNCH("probe_mfma_i8");
+    *ops = double(blocks) * 4.0 * double(iters) * 8.0 * (2.0 * 32 * 32 * 32);
     return LQ_OK;
 }
 

@@ -12,7 +12,7 @@ from __future__ import annotations
 import copy
 import warnings
 
-from .. import nn
+from .. import backends, nn
 from ..nn import intrinsic as nni
 from ..nn import quantized as nnq
 from ..nn.quantized import dynamic as nnqd
@@ -41,6 +41,53 @@ def _quant_mapping() -> dict[type, object]:
 
 def _dynamic_mapping() -> dict[type, object]:
     return {nn.Linear: nnqd.Linear.from_float}
+
+
+def _mlx_weight_bits(mod) -> int:
+    """4 or 8, from the weight observer's dtype (``_quantize.py:116-123``)."""
+    qcfg = getattr(mod, "qconfig", None)
+    if qcfg is not None:
+        bits = getattr(getattr(qcfg.weight(), "qdtype", None), "bits", None)
+        if isinstance(bits, int) and bits in (4, 8):
+            return bits
+    return 8
+
+
+def _mlx_group_size(in_features: int):
+    """First of 64 / 128 / 32 that divides ``in_features``, else None
+    (``_quantize.py:126-137``)."""
+    for gs in (64, 128, 32):
+        if in_features % gs == 0:
+            return gs
+    return None
+
+
+def _mlx_linear_builder(relu: bool):
+    """``convert`` builder for the group-wise weight-only Linear
+    (``_quantize.py:140-163``); a layer no group size divides keeps the int8 form."""
+    fallback = nnq.LinearReLU.from_float if relu else nnq.Linear.from_float
+
+    def build(child):
+        inner = child[0] if relu else child
+        gs = _mlx_group_size(inner.in_features)
+        if gs is None:
+            return fallback(child)
+        return nnq.QuantizedLinearMLX.from_float(
+            inner, bits=_mlx_weight_bits(child), group_size=gs, relu=relu)
+
+    return build
+
+
+def _mlx_dynamic_builder():
+    """``quantize_dynamic`` builder for the same (``_quantize.py:166-179``)."""
+
+    def build(child, dtype):
+        gs = _mlx_group_size(child.in_features)
+        if gs is None:
+            return nnqd.Linear.from_float(child, dtype)
+        return nnq.QuantizedLinearMLX.from_float(child, bits=dtype.bits, group_size=gs, relu=False)
+
+    return build
 
 
 def _make_observer_hook(obs):
@@ -90,7 +137,11 @@ def convert(model, inplace: bool = False):
     """Swap every calibrated module for its quantized form
     (``_quantize.py:314-419``)."""
     model = model if inplace else copy.deepcopy(model)
-    _convert_recursive(model, _quant_mapping(), always=(nnq.DeQuantStub,))
+    mapping = _quant_mapping()
+    if backends.quantized.use_mlx():
+        mapping[nn.Linear] = _mlx_linear_builder(relu=False)
+        mapping[nni.LinearReLU] = _mlx_linear_builder(relu=True)
+    _convert_recursive(model, mapping, always=(nnq.DeQuantStub,))
     model.eval()
     return model
 
@@ -110,6 +161,8 @@ def quantize_dynamic(model, qconfig_spec=None, dtype: QDtype = qint8, inplace: b
     model = model if inplace else copy.deepcopy(model)
     model.eval()
     mapping = _dynamic_mapping()
+    if backends.quantized.use_mlx():
+        mapping[nn.Linear] = _mlx_dynamic_builder()
     types = qconfig_spec if qconfig_spec is not None else set(mapping)
     if not any(type(m) in types for m in model.modules()):
         warnings.warn(

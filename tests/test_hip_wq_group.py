@@ -105,3 +105,74 @@ def test_argument_validation():
 
 def _C_err():
     return L.ShapeMismatch
+
+
+class TestConvertRoutesToGroupWise:
+    """test_real_gemm.py:94-145, with the engine named explicitly: here ``"auto"``
+    builds the int8 x int8 modules and ``"mlx_group"`` the weight-only ones."""
+
+    @pytest.fixture(autouse=True)
+    def _engine(self):
+        L.backends.quantized.engine = "mlx_group"
+        yield
+        L.backends.quantized.engine = "auto"
+
+    @staticmethod
+    def _prepared(model, shapes_in, rng):
+        import lucid_amd.quantization as Q
+        prepared = Q.prepare(model, Q.get_default_qconfig())
+        for mod in prepared.modules():
+            if hasattr(mod, "activation_post_process"):
+                mod.activation_post_process(hip(rng.standard_normal(shapes_in).astype(np.float32)))
+        return prepared
+
+    def test_static_convert_routes_linear(self):
+        import lucid_amd.quantization as Q
+        rng = np.random.default_rng(0)
+        m = nn.Sequential(nn.Linear(128, 256), nn.ReLU(), nn.Linear(256, 64))
+        x = rng.standard_normal((16, 128)).astype(np.float32)
+        w0, b0, w2, b2 = (t.numpy() for t in (m[0].weight, m[0].bias, m[2].weight, m[2].bias))
+        yf = np.maximum(x @ w0.T + b0, 0) @ w2.T + b2
+        qm = Q.convert(self._prepared(m, (16, 64), rng))
+        assert isinstance(qm[0], nnq.QuantizedLinearMLX) and isinstance(qm[2], nnq.QuantizedLinearMLX)
+        assert qm[0].group_size == 64 and qm[0].bits == 8
+        yq = qm(hip(x)).numpy()
+        assert np.abs(yf - yq).max() / (np.abs(yf).max() + 1e-9) < 0.05
+
+    def test_dynamic_convert_routes_linear(self):
+        import lucid_amd.quantization as Q
+        m = nn.Sequential(nn.Linear(96, 256), nn.ReLU(), nn.Linear(256, 64))
+        qm = Q.quantize_dynamic(m)
+        assert isinstance(qm[0], nnq.QuantizedLinearMLX) and qm[0].group_size == 32
+        assert isinstance(qm[2], nnq.QuantizedLinearMLX) and qm[2].group_size == 64
+
+    def test_indivisible_dim_keeps_the_int8_form(self):
+        import lucid_amd.quantization as Q
+        rng = np.random.default_rng(2)
+        qm = Q.convert(self._prepared(nn.Sequential(nn.Linear(8, 16)), (4, 16), rng))
+        assert isinstance(qm[0], nnq.Linear) and not isinstance(qm[0], nnq.QuantizedLinearMLX)
+        import lucid_amd.nn.quantized.dynamic as nnqd
+        assert isinstance(Q.quantize_dynamic(nn.Sequential(nn.Linear(8, 16)))[0], nnqd.Linear)
+
+    def test_relu_fused_variant_routes(self):
+        import lucid_amd.nn.intrinsic as nni
+        import lucid_amd.quantization as Q
+        rng = np.random.default_rng(3)
+        m = nn.Sequential(nni.LinearReLU(nn.Linear(64, 128), nn.ReLU()))
+        qm = Q.convert(self._prepared(m, (8, 128), rng))
+        assert isinstance(qm[0], nnq.QuantizedLinearMLX) and qm[0].relu is True
+        y = qm(hip(rng.standard_normal((8, 64)).astype(np.float32))).numpy()
+        assert y.min() >= 0.0
+
+
+def test_backends_toggle():
+    # test_real_gemm.py:148-158
+    q = L.backends.quantized
+    assert q.engine == "auto" and not q.use_mlx()
+    q.engine = "mlx_group"
+    assert q.use_mlx()
+    q.engine = "reference"
+    assert not q.use_mlx()
+    q.engine = "auto"
+    with pytest.raises(ValueError):
+        q.engine = "nonsense"
