@@ -172,6 +172,166 @@ int launch_gemv(const float* x, const uint32_t* packed, const float* scales, con
     return LQ_OK;
 }
 
+// Small-batch matmul on the matrix cores: up to 16 activation rows against 32 weight
+// rows per block.  The weight is the A operand of v_mfma_f32_16x16x4_f32 and x^T the B
+// operand, so a lane holds one weight row r = lane % 16 (two row blocks) and one
+// activation row of the same index, and the four k slots of an instruction belong to
+// the four lane quarters q = lane / 16.  A quarter owns CODES consecutive k of a step -
+// exactly the codes of one 16-byte load, all in one group - so nothing is shuffled
+// between lanes: code j of the load meets x[k0 + j] in instruction j.  Weights are
+// decoded as c * s + b (the dequantize kernel's expression) right before use.  The four
+// eight wavefronts of a block take the k steps round-robin (two per SIMD, each with
+// four independent accumulator chains, so dependent MFMAs do not wait on each other)
+// and add their partial tiles through LDS in a fixed order.
+//
+// Read straight from x, a lane's 16-byte loads would touch 64 different cache lines per
+// instruction (16 rows x 4 quarters).  A pre-pass therefore lays x out in the order the
+// lanes consume it - float4 number (step * XV + j) * 64 + lane of a 16-row block - so
+// that every load of the main kernel is one contiguous KiB per wavefront; rows past M
+// are written as zeros there.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int BITS>
+__global__ __launch_bounds__(256) void wq_arrange_x_kernel(const float* __restrict__ x, int M, int K,
+                                                           float4* __restrict__ xt) {
+    constexpr int CODES = 128 / BITS, STEP = 4 * CODES, XV = CODES / 4;
+    const int per_block = K / STEP * XV * 64;  // float4 per 16-row block
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= per_block) return;
+    const int lane = idx & 63, sj = idx >> 6, j = sj % XV, step = sj / XV;
+    const int m = blockIdx.y * 16 + (lane & 15), k = step * STEP + (lane >> 4) * CODES + 4 * j;
+    float4 v = {0.f, 0.f, 0.f, 0.f};
+    if (m < M) v = *reinterpret_cast<const float4*>(x + size_t(m) * K + k);
+    xt[size_t(blockIdx.y) * per_block + idx] = v;
+}
+
+template <int BITS>
+__global__ __launch_bounds__(512) void wq_mfma_kernel(const float4* xt, const uint32_t* packed, const float* scales,
+                                                      const float* biases, int M, int N, int K, int gs, float* out) {
+    constexpr int CODES = 128 / BITS;  // codes per 16-byte load: 32 or 16
+    constexpr int STEP = 4 * CODES;    // k covered by one wavefront step
+    constexpr int XV = CODES / 4;      // float4 loads of x per step
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    constexpr int WAVES = 8;
+    __shared__ __attribute__((aligned(16))) float red[WAVES][2][64][4];
+    // the wavefront index as a scalar, so that the step loop branches uniformly
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, q = lane >> 4;
+    const int n_base = blockIdx.x * 32;
+    const int words_per_row = K * BITS / 32, groups_per_row = K / gs;
+    const int m0 = blockIdx.y * 16;
+    const float4* xblk = xt + size_t(blockIdx.y) * (K / STEP * XV * 64) + lane;
+    const uint32_t* wrow[2];
+    const float* srow[2];
+    const float* brow[2];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+        int n = n_base + rb * 16 + r;
+        n = n < N ? n : N - 1;  // clamped rows are computed and dropped at the store
+        wrow[rb] = packed + size_t(n) * words_per_row;
+        srow[rb] = scales + size_t(n) * groups_per_row;
+        brow[rb] = biases + size_t(n) * groups_per_row;
+    }
+    v4f acc[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
+    const int steps = K / STEP;
+
+    // Two register sets, named at compile time (a run-time buffer index would put the
+    // arrays in scratch memory): the loads of the next step are issued before this one
+    // is used.
+    struct Operands {
+        uint4 wv[2];
+        float sc[2], bi[2];
+        float4 xv[XV];
+    };
+    auto fetch = [&](int step, Operands& o) {
+        const int k0 = step * STEP + q * CODES;
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+            o.wv[rb] = *reinterpret_cast<const uint4*>(wrow[rb] + k0 * BITS / 32);
+            o.sc[rb] = srow[rb][k0 / gs];
+            o.bi[rb] = brow[rb][k0 / gs];
+        }
+#pragma unroll
+        for (int j = 0; j < XV; ++j) o.xv[j] = xblk[(step * XV + j) * 64];
+    };
+    auto compute = [&](const Operands& o) {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+            const uint32_t words[4] = {o.wv[rb].x, o.wv[rb].y, o.wv[rb].z, o.wv[rb].w};
+            const float s = o.sc[rb], b = o.bi[rb];
+#pragma unroll
+            for (int j = 0; j < CODES; ++j) {
+                const uint32_t code = (words[j * BITS / 32] >> ((j * BITS) % 32)) & MASK;
+                const float wval = float(code) * s + b;
+                const float4 xq = o.xv[j / 4];
+                const float xval = (j % 4) == 0 ? xq.x : ((j % 4) == 1 ? xq.y : ((j % 4) == 2 ? xq.z : xq.w));
+                acc[rb][j & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(wval, xval, acc[rb][j & 1], 0, 0, 0);
+            }
+        }
+    };
+    // The look-ahead fetch is unconditional (past the end it re-reads the last step and
+    // the result is dropped): a branch around it would make the compiler wait, at the
+    // join, as if the new loads had not been issued - that is, for them.
+    // keeps the look-ahead loads ahead of the MFMAs: neither the optimizer (memory clobber;
+    // the pointers are not __restrict__ for that reason) nor the instruction scheduler may
+    // move a load across this point
+    auto pin = [] {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    Operands o0, o1;
+    int step = wave;
+    const int last = steps - 1;
+    if (step < steps) {
+        fetch(step, o0);
+        for (;;) {
+            fetch(step + WAVES < steps ? step + WAVES : last, o1);
+            pin();
+            compute(o0);
+            pin();
+            step += WAVES;
+            if (step >= steps) break;
+            fetch(step + WAVES < steps ? step + WAVES : last, o0);
+            pin();
+            compute(o1);
+            pin();
+            step += WAVES;
+            if (step >= steps) break;
+        }
+    }
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) *reinterpret_cast<v4f*>(red[wave][rb][lane]) = acc[rb][0] + acc[rb][1];
+    __syncthreads();
+    // D[i][j]: lane holds i = 4 * (lane / 16) + t, j = lane % 16  ->  out[m0 + j][n_base + rb*16 + i]
+    {
+        const int e = threadIdx.x;  // 2 * 64 * 4 = 512 values, one per thread
+        const int rb = e >> 8, l = (e >> 2) & 63, t = e & 3;
+        float v = red[0][rb][l][t];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) v += red[w][rb][l][t];
+        const int n = n_base + rb * 16 + 4 * (l >> 4) + t, mm = m0 + (l & 15);
+        if (n < N && mm < M) out[size_t(mm) * N + n] = v;
+    }
+}
+
+template <int BITS>
+int launch_wq_mfma(const float* x, const uint32_t* packed, const float* scales, const float* biases, int M, int N,
+                   int K, int gs, float* out, hipStream_t st) {
+    constexpr int STEP = 512 / BITS;
+    const int mblocks = (M + 15) / 16;
+    void* ws = nullptr;
+    const int rc = workspace(size_t(mblocks) * 16 * K * sizeof(float), &ws);
+    if (rc) return rc;
+    const int per_block = K / STEP * (32 / BITS) * 64;
+    hipLaunchKernelGGL((wq_arrange_x_kernel<BITS>), dim3(unsigned((per_block + 255) / 256), unsigned(mblocks)),
+                       dim3(256), 0, st, x, M, K, static_cast<float4*>(ws));
+    LQ_CHECK_LAUNCH("wq_arrange_x");
+    hipLaunchKernelGGL((wq_mfma_kernel<BITS>), dim3(unsigned((N + 31) / 32), unsigned(mblocks)), dim3(512), 0, st,
+                       static_cast<const float4*>(ws), packed, scales, biases, M, N, K, gs, out);
+    LQ_CHECK_LAUNCH("wq_mfma");
+    return LQ_OK;
+}
+
 int check_group(const char* who, int K, int gs, int bits) {
     LQ_REQUIRE(bits == 4 || bits == 8, LQ_ERR_VALUE, "%s: bits must be 4 or 8 (got %d)", who, bits);
     LQ_REQUIRE(gs == 32 || gs == 64 || gs == 128, LQ_ERR_VALUE, "%s: group_size must be 32, 64 or 128 (got %d)", who,
@@ -227,6 +387,11 @@ int lq_wq_matmul(const float* x, const uint32_t* packed, const float* scales, co
     hipStream_t st = as_stream(stream);
     const bool fused_ok = aligned16(x) && aligned16(packed) && K % 4 == 0 && (K * bits / 8) % 16 == 0 &&
                           size_t(4) * K * sizeof(float) <= 64 * 1024;
+    // 16 activation rows per launch on the matrix cores; a step covers 512 / bits weights per row
+    const bool mfma_ok = aligned16(x) && aligned16(packed) && K % (512 / bits) == 0;
+    if (M > 1 && M <= 64 && mfma_ok)
+        return bits == 4 ? launch_wq_mfma<4>(x, packed, scales, biases, M, N, K, group_size, out, st)
+                         : launch_wq_mfma<8>(x, packed, scales, biases, M, N, K, group_size, out, st);
     if (M <= 16 && fused_ok) {
         // decode shapes: weights are read once per pass of up to four activation rows
         for (int m0 = 0; m0 < M; m0 += 4) {

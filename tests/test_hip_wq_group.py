@@ -37,7 +37,11 @@ def test_quantize_and_dequantize_bit_exact(bits, gs, N, K):
 
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("M,N,K,gs", [(1, 256, 512, 64), (3, 100, 256, 32), (4, 512, 4096, 128), (16, 64, 1024, 64),
-                                      (8, 128, 128, 64), (40, 96, 256, 64), (2, 64, 8192, 64)])
+                                      (8, 128, 128, 64), (40, 96, 256, 64), (2, 64, 8192, 64),
+                                      # matrix-core path: ragged M and N, several row blocks, k steps not a
+                                      # multiple of the four wavefronts, K too ragged for it (192 at 4 bits)
+                                      (5, 33, 640, 32), (16, 11008, 4096, 64), (17, 70, 1152, 128),
+                                      (64, 257, 2048, 64), (7, 48, 192, 32), (65, 64, 512, 64)])
 def test_matmul_against_the_dequantize_path(bits, M, N, K, gs):
     rng = np.random.default_rng(bits * 7 + M + N + K)
     w = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
