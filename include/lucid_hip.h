@@ -109,6 +109,60 @@ int lq_op_info(int index, const char** name, int* version, int* deterministic);
 int lq_fill_normal(float* x, size_t n, uint64_t seed, float outlier_prob, float outlier_gain,
                    lq_stream stream);
 int lq_fill_uniform_i8(int8_t* x, size_t n, uint64_t seed, int lo, int hi, lq_stream stream);
+/* ---- quantized module breadth (lucid/nn/quantized/{sparse,activation,conv_transpose}.py,
+ * dynamic/rnn.py) ---- */
+
+/* out2[0] = min, out2[1] = max of an int32 / int64 index tensor (n > 0): the range
+ * check of lucid/nn/functional/sparse.py:17-71 without a host copy of the indices. */
+int lq_index_minmax(const void* idx, int idx_is_64, size_t n, long long* out2, lq_stream stream);
+
+/* nnq.Embedding.forward (sparse.py:128-134 = dequantize + F.embedding,
+ * CpuBackend.h:8970-9010): out[i, :] = (table[idx[i], :] - zp[idx[i]]) * scale[idx[i]],
+ * zeros where idx[i] == padding_idx >= 0 (pass -1 for none).  table int8
+ * [num_embeddings, dim], per-row scale / zp; only the rows asked for are read.  Ids
+ * outside the table give zeros (callers check the range first, as Lucid does). */
+int lq_embedding_i8(const int8_t* table, const float* scale, const float* zp, int num_embeddings, int dim,
+                    const void* idx, int idx_is_64, size_t n_idx, int padding_idx, float* out,
+                    lq_stream stream);
+
+/* nnq.EmbeddingBag.forward (sparse.py:270-279 = dequantize + F.embedding_bag,
+ * CpuBackend.h:5989-6088): bag b pools the decoded rows of idx[offsets[b] .. offsets[b+1])
+ * (the last bag runs to n_idx); offsets == NULL: idx is bags x fixed_len, one bag per row.
+ * mode 0 sum (rows added in index order), 1 mean (divided by the rows added, if any),
+ * 2 max (an empty bag gives zeros); padding_idx (-1 for none) and ids outside the table
+ * are skipped.  out float32 [bags, dim]. */
+int lq_embedding_bag_i8(const int8_t* table, const float* scale, const float* zp, int num_embeddings, int dim,
+                        const void* idx, int idx_is_64, size_t n_idx, const void* offsets, int offsets_is_64,
+                        int fixed_len, int bags, int mode, int padding_idx, float* out, lq_stream stream);
+
+/* Activations of lucid/nn/quantized/activation.py: kind 0 sigmoid, 1 hardswish,
+ * 2 hardsigmoid, 3 tanh, 4 elu(alpha), 5 leaky_relu(alpha = negative slope); float32
+ * formulas of CpuBackend.h:1049-1060,1722-1723,1783-1785,2001-2002,2064-2065.
+ * lq_act_f32: out = act(x), then fake-quantized to (out_scale, out_zp, [qmin, qmax])
+ * when fake_quantize_out != 0 (_QuantizedActivation.forward, activation.py:44-53).
+ * lq_act_requant_i8: the same for an input carried as codes on a per-tensor grid,
+ * output as codes: out = requantize(act(dequantize(q))) element by element. */
+int lq_act_f32(int kind, float alpha, const float* x, float* out, size_t n, int fake_quantize_out,
+               const float* out_scale, const float* out_zp, int out_qmin, int out_qmax, lq_stream stream);
+int lq_act_requant_i8(int kind, float alpha, const int8_t* q, int q_offset, const float* scale, const float* zp,
+                      size_t n, const float* out_scale, const float* out_zp, int out_qmin, int out_qmax,
+                      int out_offset, int8_t* out, lq_stream stream);
+
+/* Zero insertion for nnq.ConvTranspose2d (conv_transpose.py): NHWC codes [B, H, W, C] ->
+ * [B, (H-1)*stride_h + 1 + extra_h, (W-1)*stride_w + 1 + extra_w, C]; input pixels land on
+ * multiples of the stride, every other byte is `fill` (the stored code of real zero).
+ * A stride-1 lq_qconv2d_i8 of the result with the flipped, transposed kernel and padding
+ * dilation*(k-1) - p is the transposed convolution (extra = output_padding). */
+int lq_dilate_nhwc_i8(const int8_t* x, int B, int H, int W, int C, int stride_h, int stride_w, int extra_h,
+                      int extra_w, int fill, int8_t* out, lq_stream stream);
+
+/* One LSTM time step after the two gate products (CpuBackend.h:13456-13506; gate order
+ * i, f, g, o): raw = gates_x + gates_h + bias (bias = b_ih + b_hh or NULL, [4*hidden]),
+ * c_out = sigmoid(f)*c_in + sigmoid(i)*tanh(g), h_out = sigmoid(o)*tanh(c_out); h is also
+ * written to y (row stride y_ld) when y != NULL.  gates_* float32 [batch, 4*hidden]. */
+int lq_lstm_cell_f32(const float* gates_x, const float* gates_h, const float* bias, const float* c_in, int batch,
+                     int hidden, float* h_out, float* c_out, float* y, size_t y_ld, lq_stream stream);
+
 /* Matrix-core rate probe for roofline accounting: 2 blocks per CU, each
  * wavefront issuing `iters` rounds of eight v_mfma_i32_32x32x32_i8 on eight
  * independent accumulators, operands taken from a[] / b[] (at least 32 KiB

@@ -206,3 +206,111 @@ class GELU(Module):
         from . import functional as F
 
         return F.gelu(x)
+
+
+class Embedding(Module):
+    """Float Embedding as a parameter holder (``weight`` (num_embeddings, embedding_dim))."""
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, padding_idx: int | None = None) -> None:
+        super().__init__()
+        self.num_embeddings, self.embedding_dim, self.padding_idx = num_embeddings, embedding_dim, padding_idx
+        rng = np.random.default_rng(num_embeddings * 7919 + embedding_dim)
+        w = rng.standard_normal((num_embeddings, embedding_dim)).astype(np.float32)
+        if padding_idx is not None:
+            w[padding_idx] = 0.0
+        self.register_buffer("weight", T.tensor(w))
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.Embedding.forward is not part of the hip quantized-inference backend; "
+            "convert the model first")
+
+    def extra_repr(self) -> str:
+        return f"{self.num_embeddings}, {self.embedding_dim}"
+
+
+class EmbeddingBag(Embedding):
+    """Float EmbeddingBag as a parameter holder; ``mode`` in ``sum`` / ``mean`` / ``max``."""
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, mode: str = "mean",
+                 padding_idx: int | None = None) -> None:
+        super().__init__(num_embeddings, embedding_dim, padding_idx)
+        if mode not in ("sum", "mean", "max"):
+            raise ValueError(f"EmbeddingBag: mode must be one of ['max', 'mean', 'sum'], got {mode!r}")
+        self.mode = mode
+
+
+class _FloatActivation(Module):
+    """Float activation evaluated by the same kernel as its quantized form, without the
+    output grid."""
+
+    _kind = -1
+
+    def _alpha(self) -> float:
+        return 0.0
+
+    def forward(self, x: Tensor) -> Tensor:
+        from .quantized.activation import apply_activation
+        return apply_activation(self._kind, self._alpha(), x, None)
+
+
+class Sigmoid(_FloatActivation):
+    _kind = 0
+
+
+class Hardswish(_FloatActivation):
+    _kind = 1
+
+
+class Hardsigmoid(_FloatActivation):
+    _kind = 2
+
+
+class Tanh(_FloatActivation):
+    _kind = 3
+
+
+class ELU(_FloatActivation):
+    _kind = 4
+
+    def __init__(self, alpha: float = 1.0) -> None:
+        super().__init__()
+        self.alpha = float(alpha)
+
+    def _alpha(self) -> float:
+        return self.alpha
+
+
+class LeakyReLU(_FloatActivation):
+    _kind = 5
+
+    def __init__(self, negative_slope: float = 0.01) -> None:
+        super().__init__()
+        self.negative_slope = float(negative_slope)
+
+    def _alpha(self) -> float:
+        return self.negative_slope
+
+
+class ConvTranspose2d(Module):
+    """Float ConvTranspose2d as a parameter holder (``weight`` (in, out/groups, kh, kw))."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, output_padding=0,
+                 groups=1, bias=True, dilation=1) -> None:
+        super().__init__()
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride = _pair(kernel_size), _pair(stride)
+        self.padding = padding if isinstance(padding, str) else _pair(padding)
+        self.output_padding, self.dilation, self.groups = _pair(output_padding), _pair(dilation), groups
+        fan_in = out_channels // groups * self.kernel_size[0] * self.kernel_size[1]
+        bound = 1.0 / np.sqrt(fan_in)
+        rng = np.random.default_rng(fan_in * 7919 + in_channels)
+        self.register_buffer("weight", T.tensor(rng.uniform(
+            -bound, bound, (in_channels, out_channels // groups, *self.kernel_size)).astype(np.float32)))
+        self.register_buffer("bias", T.tensor(
+            rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.ConvTranspose2d.forward is not part of the hip quantized-inference backend; "
+            "quantize the model (convert) first")

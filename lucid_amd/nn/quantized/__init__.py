@@ -4,10 +4,14 @@
 from . import dynamic
 from .functional_module import FloatFunctional, QFunctional
 from .conv import Conv2d
+from .conv_transpose import ConvTranspose2d
 from .intrinsic import ConvReLU2d, LinearReLU
 from .linear import Linear
 from .mlx_linear import QuantizedLinearMLX
 from .modules import DeQuantize, DeQuantStub, Quantize, QuantStub, QuantWrapper
+from .activation import ELU, Hardsigmoid, Hardswish, LeakyReLU, Sigmoid, Tanh
+from .sparse import Embedding, EmbeddingBag
 
 __all__ = ["QuantizedLinearMLX", "Linear", "LinearReLU", "Conv2d", "ConvReLU2d", "Quantize", "DeQuantize", "QuantStub", "DeQuantStub",
-           "QuantWrapper", "QFunctional", "FloatFunctional", "dynamic"]
+           "QuantWrapper", "QFunctional", "FloatFunctional", "dynamic", "Embedding", "EmbeddingBag", "ConvTranspose2d", "Sigmoid",
+           "Hardswish", "Hardsigmoid", "Tanh", "ELU", "LeakyReLU"]

@@ -22,7 +22,7 @@ from .qconfig import QConfig, get_default_qconfig
 
 def _observed_types() -> tuple[type, ...]:
     return (nn.Linear, nn.Conv2d, nni.LinearReLU, nni.ConvReLU2d, nnq.QuantStub,
-            nnq.FloatFunctional)
+            nnq.FloatFunctional, nn.ConvTranspose2d, nn.Sigmoid, nn.Hardswish, nn.Hardsigmoid, nn.Tanh, nn.ELU, nn.LeakyReLU)
 
 
 def _quant_mapping() -> dict[type, object]:
@@ -32,6 +32,15 @@ def _quant_mapping() -> dict[type, object]:
         nnq.QuantStub: nnq.Quantize.from_float,
         nnq.DeQuantStub: nnq.DeQuantize.from_float,
         nnq.FloatFunctional: nnq.QFunctional.from_float,
+        nn.ConvTranspose2d: nnq.ConvTranspose2d.from_float,
+        nn.Embedding: nnq.Embedding.from_float,
+        nn.EmbeddingBag: nnq.EmbeddingBag.from_float,
+        nn.Sigmoid: nnq.Sigmoid.from_float,
+        nn.Hardswish: nnq.Hardswish.from_float,
+        nn.Hardsigmoid: nnq.Hardsigmoid.from_float,
+        nn.Tanh: nnq.Tanh.from_float,
+        nn.ELU: nnq.ELU.from_float,
+        nn.LeakyReLU: nnq.LeakyReLU.from_float,
     }
     if hasattr(nnq, "Conv2d"):
         m[nn.Conv2d] = nnq.Conv2d.from_float
@@ -141,7 +150,8 @@ def convert(model, inplace: bool = False):
     if backends.quantized.use_mlx():
         mapping[nn.Linear] = _mlx_linear_builder(relu=False)
         mapping[nni.LinearReLU] = _mlx_linear_builder(relu=True)
-    _convert_recursive(model, mapping, always=(nnq.DeQuantStub,))
+    # DeQuantStub and the embedding tables convert without calibration (_quantize.py:414-417)
+    _convert_recursive(model, mapping, always=(nnq.DeQuantStub, nn.Embedding, nn.EmbeddingBag))
     model.eval()
     return model
 

@@ -1,0 +1,158 @@
+"""CPU restatement of the quantized module breadth: int8 embedding tables, activations
+that requantize their result, transposed convolution, the weight-only LSTM.
+
+TEST INFRASTRUCTURE ONLY, like the rest of ``oracle/``.  numpy float32, plain loops
+where the reference loops.
+
+* ``embedding``      ``lucid/nn/quantized/sparse.py:128-134`` (dequantize the table,
+                     ``F.embedding``) with ``CpuBackend.h:8970-9010`` (padding row = zeros)
+* ``embedding_bag``  ``sparse.py:270-279`` with ``CpuBackend.h:5989-6088`` (bag bounds,
+                     skipped ids, sum in index order, mean over the rows added, max from
+                     the lowest float, an empty bag gives zeros)
+* ``act``            ``CpuBackend.h:1049-1060`` sigmoid, ``:1722-1723`` leaky_relu,
+                     ``:1783-1785`` elu, ``:2001-2002`` hard_sigmoid, ``:2064-2065``
+                     hard_swish, tanh
+* ``quantized_act``  ``lucid/nn/quantized/activation.py:44-53`` (activation, then
+                     fake-quantize to the calibrated grid)
+* ``lstm``           ``CpuBackend.h:13394-13519`` on dequantized weights
+                     (``lucid/nn/quantized/dynamic/rnn.py``)
+
+PARITY UNPINNED at the bit level for sigmoid, tanh, elu (the reference evaluates exp /
+tanh through Accelerate's vForce, whose last-bit behaviour is not published) and for the
+LSTM's float32 GEMMs (``cblas_sgemm`` accumulation order).  ``tests/test_oracle_breadth.py``
+pins the formulas against float64 closed forms; hard_sigmoid, hard_swish, leaky_relu and
+the embedding lookups are exact arithmetic and compared bit for bit.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+import oracle as O
+
+SIGMOID, HARDSWISH, HARDSIGMOID, TANH, ELU, LEAKY_RELU = range(6)
+
+
+def dequantize_rows(codes, scale, zp):
+    codes = np.asarray(codes)
+    return ((codes.astype(np.float32) - np.asarray(zp, np.float32)[:, None]) *
+            np.asarray(scale, np.float32)[:, None]).astype(np.float32)
+
+
+def embedding(codes, scale, zp, idx, padding_idx=None):
+    table = dequantize_rows(codes, scale, zp)
+    idx = np.asarray(idx)
+    out = table[idx.reshape(-1)].reshape(idx.shape + (table.shape[1],)).copy()
+    if padding_idx is not None and padding_idx >= 0:
+        out[idx == padding_idx] = 0.0
+    return out
+
+
+def embedding_bag(codes, scale, zp, idx, offsets=None, mode="mean", padding_idx=None):
+    table = dequantize_rows(codes, scale, zp)
+    num, D = table.shape
+    idx = np.asarray(idx)
+    if idx.ndim == 2:
+        offsets = np.arange(0, idx.size, idx.shape[1])
+        idx = idx.reshape(-1)
+    offsets = np.asarray(offsets)
+    B, n = len(offsets), idx.size
+    pad = -1 if padding_idx is None else int(padding_idx)
+    out = np.zeros((B, D), np.float32)
+    for b in range(B):
+        s = int(offsets[b])
+        e = int(offsets[b + 1]) if b + 1 < B else n
+        row = np.full(D, np.finfo(np.float32).min, np.float32) if mode == "max" else np.zeros(D, np.float32)
+        count = 0
+        for k in range(s, e):
+            i = int(idx[k])
+            if i == pad or i < 0 or i >= num:
+                continue
+            if mode == "max":
+                row = np.where(table[i] > row, table[i], row)
+            else:
+                row = (row + table[i]).astype(np.float32)
+            count += 1
+        if mode == "max" and count == 0:
+            row = np.zeros(D, np.float32)
+        if mode == "mean" and count > 0:
+            row = (row / np.float32(count)).astype(np.float32)
+        out[b] = row
+    return out
+
+
+def act(kind, x, alpha=0.0):
+    x = np.asarray(x, np.float32)
+    one, alpha = np.float32(1.0), np.float32(alpha)
+    with np.errstate(over="ignore"):
+        if kind == SIGMOID:
+            return (one / (one + np.exp(-x).astype(np.float32))).astype(np.float32)
+        if kind in (HARDSWISH, HARDSIGMOID):
+            t = ((x + np.float32(3.0)) / np.float32(6.0)).astype(np.float32)
+            t = np.where(t < 0, np.float32(0.0), t)
+            t = np.where(one < t, one, t).astype(np.float32)
+            return (x * t).astype(np.float32) if kind == HARDSWISH else t
+        if kind == TANH:
+            return np.tanh(x).astype(np.float32)
+        if kind == ELU:
+            return np.where(x >= 0, x, alpha * (np.exp(x).astype(np.float32) - one)).astype(np.float32)
+        if kind == LEAKY_RELU:
+            return np.where(x >= 0, x, alpha * x).astype(np.float32)
+    raise ValueError(kind)
+
+
+def quantized_act(kind, x, alpha, S, Z, qmin, qmax):
+    """Float output of ``_QuantizedActivation.forward``."""
+    return O.fake_quantize(act(kind, x, alpha), S, Z, qmin, qmax)
+
+
+def quantized_act_codes(kind, q, in_offset, s, z, alpha, S, Z, qmin, qmax, out_offset):
+    """The same for an input carried as stored codes (``code + in_offset``), result as
+    stored codes."""
+    x = O.dequantize(np.asarray(q, np.int8), s, z, code_offset=in_offset)
+    return O.quantize(act(kind, x, alpha), S, Z, qmin, qmax, code_offset=out_offset)
+
+
+def lstm(x, h0, c0, w_ih, w_hh, b_ih, b_hh):
+    """One layer, one direction, time-major ``x`` (T, B, I); returns (y, h_n, c_n)."""
+    x = np.asarray(x, np.float32)
+    T, B, _ = x.shape
+    H = h0.shape[-1]
+    h, c = np.asarray(h0, np.float32).copy(), np.asarray(c0, np.float32).copy()
+    bias = (np.asarray(b_ih, np.float32) + np.asarray(b_hh, np.float32)).astype(np.float32)
+    y = np.zeros((T, B, H), np.float32)
+    sig = lambda v: (np.float32(1.0) / (np.float32(1.0) + np.exp(-v).astype(np.float32))).astype(np.float32)
+    for t in range(T):
+        raw = ((x[t] @ w_ih.T).astype(np.float32) + (h @ w_hh.T).astype(np.float32)).astype(np.float32)
+        raw = (raw + bias).astype(np.float32)
+        i, f = sig(raw[:, :H]), sig(raw[:, H:2 * H])
+        g, o = np.tanh(raw[:, 2 * H:3 * H]).astype(np.float32), sig(raw[:, 3 * H:])
+        c = (f * c + i * g).astype(np.float32)
+        h = (o * np.tanh(c).astype(np.float32)).astype(np.float32)
+        y[t] = h
+    return y, h, c
+
+
+def conv_transpose2d(x, w, bias, stride, padding, output_padding, dilation=(1, 1), groups=1):
+    """Float64 scatter form of a transposed convolution: ``x`` (B, Cin, H, W), ``w``
+    (Cin, Cout/groups, kh, kw)."""
+    x = np.asarray(x, np.float64)
+    w = np.asarray(w, np.float64)
+    B, Cin, H, W = x.shape
+    _, Cog, kh, kw = w.shape
+    (sh, sw), (ph, pw), (oph, opw), (dh, dw) = stride, padding, output_padding, dilation
+    OH = (H - 1) * sh - 2 * ph + dh * (kh - 1) + oph + 1
+    OW = (W - 1) * sw - 2 * pw + dw * (kw - 1) + opw + 1
+    full = np.zeros((B, Cog * groups, OH + 2 * ph, OW + 2 * pw), np.float64)
+    cig = Cin // groups
+    for g in range(groups):
+        for ci in range(g * cig, (g + 1) * cig):
+            for i in range(kh):
+                for j in range(kw):
+                    contrib = x[:, ci, :, :, None] * w[ci, :, i, j][None, None, None, :]  # B,H,W,Cog
+                    full[:, g * Cog:(g + 1) * Cog, i * dh:i * dh + (H - 1) * sh + 1:sh,
+                         j * dw:j * dw + (W - 1) * sw + 1:sw] += np.transpose(contrib, (0, 3, 1, 2))
+    out = full[:, :, ph:ph + OH, pw:pw + OW]
+    if bias is not None:
+        out = out + np.asarray(bias, np.float64)[None, :, None, None]
+    return out

@@ -1,0 +1,213 @@
+"""Quantized module breadth on the device against the restatement (oracle/breadth.py)
+and the reference's own tests (lucid/test/unit/quantization/test_breadth.py,
+test_module_breadth.py)."""
+
+import numpy as np
+import pytest
+
+import lucid_amd as L
+import lucid_amd.nn as nn
+import lucid_amd.nn.quantized as nnq
+import lucid_amd.quantization as Q
+import oracle as O
+import oracle.breadth as Br
+
+pytestmark = pytest.mark.gpu
+
+
+def hip(a, dtype=None):
+    return L.tensor(a, device="hip") if dtype is None else L.tensor(np.asarray(a, dtype), device="hip")
+
+
+# ---------------------------------------------------------------- embeddings
+@pytest.mark.parametrize("num,dim,idx_dtype", [(100, 32, np.int64), (257, 30, np.int32), (5000, 768, np.int64)])
+def test_embedding_bit_exact(num, dim, idx_dtype):
+    emb = nn.Embedding(num, dim, padding_idx=3)
+    q = nnq.Embedding.from_float(emb)
+    assert q.weight_int8.dtype is L.int8 and q.weight_int8.shape == (num, dim)
+    w = emb.weight.numpy()
+    mn, mx = O.minmax(w, ch_axis=0)
+    s, z = O.calc_qparams(mn, mx, True, -128, 127, True)
+    codes = O.quantize(w, s, z, -128, 127, ch_axis=0)
+    assert np.array_equal(q.weight_int8.numpy(), codes) and np.array_equal(q.weight_scale.numpy(), s)
+    rng = np.random.default_rng(num)
+    idx = rng.integers(0, num, (4, 37)).astype(idx_dtype)
+    idx[0, :5] = 3
+    y = q(hip(idx)).numpy()
+    want = Br.embedding(codes, s, z, idx, padding_idx=3)
+    assert y.shape == (4, 37, dim)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    # test_breadth.py:12-23
+    yf = np.where((idx == 3)[..., None], 0, w[idx])
+    assert np.abs(yf - y).mean() / (np.abs(yf).mean() + 1e-9) < 0.02
+    # test_breadth.py:25-30
+    assert q.weight_int8.numpy().nbytes + q.weight_scale.numpy().nbytes < num * dim * 4 / 2
+
+
+def test_embedding_index_checks():
+    q = nnq.Embedding.from_float(nn.Embedding(10, 8))
+    with pytest.raises(IndexError, match=r"index 10 is out of range for a table with 10 entries"):
+        q(hip(np.array([1, 10], np.int64)))
+    with pytest.raises(IndexError, match=r"index -1 is out of range"):
+        q(hip(np.array([-1, 2], np.int64)))
+    with pytest.raises(TypeError, match="indices must be an integer tensor"):
+        q(hip(np.array([1.0, 2.0], np.float32)))
+    assert q(hip(np.zeros((0,), np.int64))).shape == (0, 8)
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean", "max"])
+def test_embedding_bag_bit_exact(mode):
+    bag = nn.EmbeddingBag(50, 16, mode=mode, padding_idx=9)
+    q = nnq.EmbeddingBag.from_float(bag)
+    codes, s, z = q.weight_int8.numpy(), q.weight_scale.numpy(), q.weight_zero_point.numpy()
+    idx = np.array([1, 5, 9, 3, 7, 2, 8, 9, 9], np.int64)
+    off = np.array([0, 3, 5, 5], np.int64)
+    y = q(hip(idx), hip(off)).numpy()
+    want = Br.embedding_bag(codes, s, z, idx, off, mode, padding_idx=9)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(y[2], np.zeros(16, np.float32))  # the empty bag
+    # 2-d indices: every row a bag; int32 indices and offsets
+    idx2 = np.random.default_rng(0).integers(0, 50, (64, 11)).astype(np.int32)
+    y2 = q(hip(idx2)).numpy()
+    assert np.array_equal(y2.view(np.uint32),
+                          Br.embedding_bag(codes, s, z, idx2, None, mode, padding_idx=9).view(np.uint32))
+    with pytest.raises(ValueError, match="offsets required"):
+        q(hip(idx))
+
+
+def test_convert_installs_embeddings_without_calibration():
+    # test_breadth.py:32-35, test_module_breadth.py:91-104
+    qm = Q.convert(Q.prepare(nn.Sequential(nn.Embedding(50, 16))))
+    assert isinstance(qm[0], nnq.Embedding)
+    m = nn.Sequential(nn.EmbeddingBag(50, 16, mode="mean"))
+    w = m[0].weight.numpy()
+    qm = Q.convert(m)
+    assert isinstance(qm[0], nnq.EmbeddingBag) and qm[0].weight_int8.dtype is L.int8
+    idx, off = np.array([1, 5, 9, 3, 7, 2, 8], np.int64), np.array([0, 3, 5], np.int64)
+    yq = qm[0](hip(idx), hip(off)).numpy()
+    yf = np.stack([w[[1, 5, 9]].mean(0), w[[3, 7]].mean(0), w[[2, 8]].mean(0)])
+    assert np.abs(yf - yq).max() / (np.abs(yf).max() + 1e-9) < 0.05
+
+
+def test_integer_input_passes_through_quantize():
+    # test_breadth.py:38-47
+    idx = hip(np.array([1, 2, 3], np.int64))
+    quant = nnq.Quantize(hip(np.float32(0.05)), hip(np.float32(0.0)))
+    assert np.array_equal(quant(idx).numpy(), [1, 2, 3])
+
+
+# ---------------------------------------------------------------- activations
+_ACTS = [(nn.Sigmoid, nnq.Sigmoid, Br.SIGMOID, {}), (nn.Hardswish, nnq.Hardswish, Br.HARDSWISH, {}),
+         (nn.Hardsigmoid, nnq.Hardsigmoid, Br.HARDSIGMOID, {}), (nn.Tanh, nnq.Tanh, Br.TANH, {}),
+         (nn.ELU, nnq.ELU, Br.ELU, {"alpha": 0.7}), (nn.LeakyReLU, nnq.LeakyReLU, Br.LEAKY_RELU, {"negative_slope": 0.2})]
+_EXACT = (Br.HARDSWISH, Br.HARDSIGMOID, Br.LEAKY_RELU)
+
+
+@pytest.mark.parametrize("fcls,qcls,kind,kw", _ACTS)
+def test_float_activation(fcls, qcls, kind, kw):
+    x = (np.random.default_rng(kind).standard_normal(100003) * 3).astype(np.float32)
+    y = fcls(**kw)(hip(x)).numpy()
+    want = Br.act(kind, x, *kw.values())
+    if kind in _EXACT:
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    else:  # exp / tanh: library last bits differ
+        assert np.abs(y - want).max() <= 4e-7 * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("fcls,qcls,kind,kw", _ACTS)
+def test_quantized_activation_on_codes_and_on_floats(fcls, qcls, kind, kw):
+    rng = np.random.default_rng(10 + kind)
+    alpha = next(iter(kw.values()), 0.0)
+    x = (rng.standard_normal((8, 4099)) * 2).astype(np.float32)
+    s, z = np.float32(16 / 255), np.float32(128)
+    y_float = Br.act(kind, x, alpha)
+    S = np.float32((y_float.max() - min(y_float.min(), 0)) / 255)
+    Z = np.float32(np.rint(-min(y_float.min(), 0) / S))
+    act = qcls(hip(S), hip(Z), Q.quint8)
+    act._configure(fcls(**kw))
+    # on codes
+    xq = nnq.Quantize(hip(s), hip(z), Q.quint8)(hip(x))
+    out = act(xq)
+    assert out._grid is not None and out.shape == x.shape
+    stored = O.quantize(x, s, z, 0, 255, code_offset=-128)
+    want = Br.quantized_act_codes(kind, stored, -128, s, z, alpha, S, Z, 0, 255, -128)
+    got = out._grid.codes.numpy()
+    if kind in _EXACT:
+        assert np.array_equal(got, want)
+    else:
+        d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() < 1e-3
+    # on plain floats: activation + fake-quantize
+    yf = act(hip(x)).numpy()
+    want_f = Br.quantized_act(kind, x, alpha, S, Z, 0, 255)
+    if kind in _EXACT:
+        assert np.array_equal(yf.view(np.uint32), want_f.view(np.uint32))
+    else:
+        assert np.abs(yf - want_f).max() <= S * 1.001 and (yf != want_f).mean() < 1e-3
+
+
+@pytest.mark.parametrize("fcls,qcls,kind,kw", _ACTS)
+def test_convert_installs_quantized_activation(fcls, qcls, kind, kw):
+    # test_module_breadth.py:55-89
+    rng = np.random.default_rng(kind)
+    m = nn.Sequential(nnq.QuantStub(), nn.Linear(64, 64), fcls(**kw), nnq.DeQuantStub())
+    prepared = Q.prepare(m, Q.get_default_qconfig())
+    w, b = m[1].weight.numpy(), m[1].bias.numpy()
+    alpha = next(iter(kw.values()), 0.0)
+    for _ in range(5):
+        x = rng.standard_normal((8, 64)).astype(np.float32)
+        h = x @ w.T + b
+        prepared[0].activation_post_process(hip(x))
+        prepared[1].activation_post_process(hip(h))
+        prepared[2].activation_post_process(hip(Br.act(kind, h, alpha)))
+    qm = Q.convert(prepared)
+    assert isinstance(qm[2], qcls)
+    if kind == Br.LEAKY_RELU:
+        assert qm[2].negative_slope == pytest.approx(0.2)
+    x = rng.standard_normal((8, 64)).astype(np.float32)
+    yq = qm(hip(x)).numpy()
+    yf = Br.act(kind, x @ w.T + b, alpha)
+    assert np.abs(yf - yq).max() / (np.abs(yf).max() + 1e-9) < 0.1
+
+
+# ---------------------------------------------------------------- transposed convolution
+@pytest.mark.parametrize("cin,cout,k,stride,padding,output_padding,dilation,groups",
+                         [(8, 4, 3, 2, 1, 1, 1, 1),      # test_module_breadth.py:33-52
+                          (32, 48, (3, 2), (2, 3), (1, 0), (1, 2), 1, 1),
+                          (32, 32, 3, 1, 1, 0, 1, 2),     # stride 1: no zero insertion
+                          (16, 24, 2, 2, 0, 0, (2, 1), 1)])
+def test_conv_transpose2d(cin, cout, k, stride, padding, output_padding, dilation, groups):
+    pair = lambda v: (v, v) if isinstance(v, int) else v
+    rng = np.random.default_rng(cin + cout)
+    m = nn.Sequential(nnq.QuantStub(), nn.ConvTranspose2d(cin, cout, k, stride=stride, padding=padding,
+                                                          output_padding=output_padding, groups=groups,
+                                                          dilation=dilation), nnq.DeQuantStub())
+    w, b = m[1].weight.numpy(), m[1].bias.numpy()
+    args = (pair(stride), pair(padding), pair(output_padding), pair(dilation), groups)
+    prepared = Q.prepare(m, Q.get_default_qconfig())
+    for _ in range(6):
+        x = rng.standard_normal((2, cin, 8, 7)).astype(np.float32)
+        prepared[0].activation_post_process(hip(x))
+        prepared[1].activation_post_process(hip(Br.conv_transpose2d(x, w, b, *args).astype(np.float32)))
+    qm = Q.convert(prepared)
+    ct = qm[1]
+    assert isinstance(ct, nnq.ConvTranspose2d) and ct.weight_int8.dtype is L.int8
+    assert ct.weight_int8.shape == w.shape and ct.weight_scale.shape == (cout // groups,)
+    x = rng.standard_normal((2, cin, 8, 7)).astype(np.float32)
+    yf = Br.conv_transpose2d(x, w, b, *args)
+    out = ct(qm[0](hip(x)))
+    yq = qm(hip(x)).numpy()
+    assert yq.shape == yf.shape
+    assert np.abs(yf - yq).mean() / (np.abs(yf).mean() + 1e-9) < 0.05
+    # the float64 scatter form on the dequantized operands, requantized: codes agree up to
+    # one step on rounding ties
+    s0, z0 = qm[0].scale.item(), qm[0].zero_point.item()
+    xd = O.dequantize(O.quantize(x, s0, z0, 0, 255, code_offset=-128), s0, z0, code_offset=-128)
+    ws = ct.weight_scale.numpy()
+    wd = ct.weight_int8.numpy().astype(np.float32) * ws[None, :, None, None]
+    ref = Br.conv_transpose2d(xd, wd, b, *args)
+    S, Z = ct.scale.item(), ct.zero_point.item()
+    want = np.clip(np.rint(ref / np.float64(S)) + Z, 0, 255)
+    got = np.transpose(out._grid.codes.numpy().astype(np.int32) + 128, (0, 3, 1, 2))
+    d = np.abs(got - want)
+    assert d.max() <= 1 and (d != 0).mean() < 0.01

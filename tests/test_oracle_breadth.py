@@ -1,0 +1,139 @@
+"""The restatement of the module breadth (oracle/breadth.py) against what the mathematics
+fixes: float64 closed forms of the activations, brute-force lookups, a scatter-form
+transposed convolution against a direct sum, the LSTM against a float64 step."""
+
+import numpy as np
+import pytest
+
+import oracle as O
+import oracle.breadth as Br
+
+
+def _table(rng, n=50, d=16):
+    w = rng.standard_normal((n, d)).astype(np.float32)
+    mn, mx = O.minmax(w, ch_axis=0)
+    s, z = O.calc_qparams(mn, mx, True, -128, 127, True)
+    return w, O.quantize(w, s, z, -128, 127, ch_axis=0), s, z
+
+
+def test_embedding_is_a_row_gather_of_the_dequantized_table():
+    rng = np.random.default_rng(0)
+    w, q, s, z = _table(rng)
+    idx = rng.integers(0, 50, (3, 7))
+    out = Br.embedding(q, s, z, idx, padding_idx=4)
+    assert out.shape == (3, 7, 16)
+    for a in range(3):
+        for b in range(7):
+            i = idx[a, b]
+            want = np.zeros(16, np.float32) if i == 4 else (q[i].astype(np.float32) - z[i]) * s[i]
+            assert np.array_equal(out[a, b], want)
+    # test_breadth.py:12-23: mean relative error of the int8 table under 2 %
+    assert np.abs(out - np.where((idx == 4)[..., None], 0, w[idx])).mean() / np.abs(w[idx]).mean() < 0.02
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean", "max"])
+def test_embedding_bag_pools_in_float64_agreement(mode):
+    rng = np.random.default_rng(1)
+    w, q, s, z = _table(rng)
+    idx = np.array([1, 5, 9, 3, 7, 2, 8, 9, 9])
+    off = np.array([0, 3, 5, 5])  # third bag empty, fourth runs to the end
+    out = Br.embedding_bag(q, s, z, idx, off, mode, padding_idx=9)
+    table = Br.dequantize_rows(q, s, z).astype(np.float64)
+    bags = [[1, 5], [3, 7], [], [2, 8]]  # 9 is padding
+    for b, members in enumerate(bags):
+        if not members:
+            want = np.zeros(16)
+        elif mode == "sum":
+            want = table[members].sum(0)
+        elif mode == "mean":
+            want = table[members].mean(0)
+        else:
+            want = table[members].max(0)
+        assert np.allclose(out[b], want, rtol=1e-6, atol=1e-6)
+    # 2-d indices: one bag per row
+    out2 = Br.embedding_bag(q, s, z, np.array([[1, 5, 9], [3, 7, 2]]), None, mode, padding_idx=9)
+    assert np.array_equal(out2[0], out[0])
+
+
+def test_activation_formulas_against_float64():
+    x = np.linspace(-9, 9, 20001).astype(np.float32)
+    x64 = x.astype(np.float64)
+    hs = np.clip((x64 + 3) / 6, 0, 1)
+    want = {Br.SIGMOID: 1 / (1 + np.exp(-x64)), Br.HARDSWISH: x64 * hs, Br.HARDSIGMOID: hs,
+            Br.TANH: np.tanh(x64), Br.ELU: np.where(x64 >= 0, x64, 0.7 * np.expm1(x64)),
+            Br.LEAKY_RELU: np.where(x64 >= 0, x64, 0.2 * x64)}
+    alpha = {Br.ELU: 0.7, Br.LEAKY_RELU: 0.2}
+    for kind, ref in want.items():
+        got = Br.act(kind, x, alpha.get(kind, 0.0))
+        assert got.dtype == np.float32
+        assert np.abs(got - ref).max() < 2e-6, kind
+    # special values: the hard forms saturate, a NaN passes
+    assert Br.act(Br.HARDSIGMOID, np.float32([-3, 3, -100, 100])).tolist() == [0, 1, 0, 1]
+    assert np.isnan(Br.act(Br.HARDSWISH, np.float32([np.nan]))[0])
+    assert Br.act(Br.SIGMOID, np.float32([0]))[0] == 0.5
+
+
+def test_quantized_activation_on_codes_equals_the_float_formulation():
+    rng = np.random.default_rng(2)
+    s, z, S, Z = np.float32(0.05), np.float32(120), np.float32(1 / 255), np.float32(0)
+    q = rng.integers(-128, 128, 4096).astype(np.int8)  # stored quint8 codes (code - 128)
+    x = O.dequantize(q, s, z, code_offset=-128)
+    for kind in range(6):
+        codes = Br.quantized_act_codes(kind, q, -128, s, z, 0.3, S, Z, 0, 255, -128)
+        floats = Br.quantized_act(kind, x, 0.3, S, Z, 0, 255)
+        assert np.array_equal(O.dequantize(codes, S, Z, code_offset=-128), floats)
+
+
+def test_lstm_against_a_float64_recurrence():
+    rng = np.random.default_rng(3)
+    T, B, I, H = 5, 3, 8, 6
+    x = rng.standard_normal((T, B, I)).astype(np.float32)
+    wih, whh = (rng.standard_normal((4 * H, n)).astype(np.float32) * 0.3 for n in (I, H))
+    bih, bhh = (rng.standard_normal(4 * H).astype(np.float32) * 0.1 for _ in range(2))
+    h0, c0 = (rng.standard_normal((B, H)).astype(np.float32) for _ in range(2))
+    y, hn, cn = Br.lstm(x, h0, c0, wih, whh, bih, bhh)
+    h, c = h0.astype(np.float64), c0.astype(np.float64)
+    sig = lambda v: 1 / (1 + np.exp(-v))
+    for t in range(T):
+        raw = x[t].astype(np.float64) @ wih.T + h @ whh.T + bih + bhh
+        i, f, g, o = sig(raw[:, :H]), sig(raw[:, H:2 * H]), np.tanh(raw[:, 2 * H:3 * H]), sig(raw[:, 3 * H:])
+        c = f * c + i * g
+        h = o * np.tanh(c)
+        assert np.allclose(y[t], h, atol=1e-5)
+    assert np.allclose(hn, h, atol=1e-5) and np.allclose(cn, c, atol=1e-5)
+    assert np.array_equal(y[-1], hn)
+
+
+@pytest.mark.parametrize("stride,padding,output_padding,dilation,groups",
+                         [((2, 2), (1, 1), (1, 1), (1, 1), 1), ((1, 1), (0, 0), (0, 0), (1, 1), 1),
+                          ((3, 2), (2, 0), (2, 1), (1, 1), 1), ((2, 2), (1, 1), (0, 0), (2, 1), 2)])
+def test_conv_transpose_scatter_form_against_the_direct_sum(stride, padding, output_padding, dilation, groups):
+    rng = np.random.default_rng(4)
+    B, Cin, Cout, H, W, kh, kw = 2, 4, 6, 5, 4, 3, 2
+    x = rng.standard_normal((B, Cin, H, W))
+    w = rng.standard_normal((Cin, Cout // groups, kh, kw))
+    bias = rng.standard_normal(Cout)
+    out = Br.conv_transpose2d(x, w, bias, stride, padding, output_padding, dilation, groups)
+    (sh, sw), (ph, pw), (dh, dw) = stride, padding, dilation
+    OH = (H - 1) * sh - 2 * ph + dh * (kh - 1) + output_padding[0] + 1
+    OW = (W - 1) * sw - 2 * pw + dw * (kw - 1) + output_padding[1] + 1
+    assert out.shape == (B, Cout, OH, OW)
+    cig, cog = Cin // groups, Cout // groups
+    want = np.zeros_like(out)
+    for b in range(B):
+        for co in range(Cout):
+            g = co // cog
+            for oh in range(OH):
+                for ow in range(OW):
+                    acc = bias[co]
+                    for ci in range(g * cig, (g + 1) * cig):
+                        for i in range(kh):
+                            for j in range(kw):
+                                nh, nw = oh + ph - i * dh, ow + pw - j * dw
+                                if nh % sh or nw % sw:
+                                    continue
+                                h, wd = nh // sh, nw // sw
+                                if 0 <= h < H and 0 <= wd < W:
+                                    acc += x[b, ci, h, wd] * w[ci, co - g * cog, i, j]
+                    want[b, co, oh, ow] = acc
+    assert np.allclose(out, want, atol=1e-10)
