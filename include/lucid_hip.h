@@ -159,9 +159,12 @@ int lq_dilate_nhwc_i8(const int8_t* x, int B, int H, int W, int C, int stride_h,
 /* One LSTM time step after the two gate products (CpuBackend.h:13456-13506; gate order
  * i, f, g, o): raw = gates_x + gates_h + bias (bias = b_ih + b_hh or NULL, [4*hidden]),
  * c_out = sigmoid(f)*c_in + sigmoid(i)*tanh(g), h_out = sigmoid(o)*tanh(c_out); h is also
- * written to y (row stride y_ld) when y != NULL.  gates_* float32 [batch, 4*hidden]. */
-int lq_lstm_cell_f32(const float* gates_x, const float* gates_h, const float* bias, const float* c_in, int batch,
-                     int hidden, float* h_out, float* c_out, float* y, size_t y_ld, lq_stream stream);
+ * written to y (row stride y_ld) when y != NULL.  gates_x: this step's rows of x W_ih^T,
+ * row stride gates_x_ld floats (the product is taken once over all time steps);
+ * gates_h float32 [batch, 4*hidden] contiguous. */
+int lq_lstm_cell_f32(const float* gates_x, size_t gates_x_ld, const float* gates_h, const float* bias,
+                     const float* c_in, int batch, int hidden, float* h_out, float* c_out, float* y,
+                     size_t y_ld, lq_stream stream);
 
 /* Matrix-core rate probe for roofline accounting: 2 blocks per CU, each
  * wavefront issuing `iters` rounds of eight v_mfma_i32_32x32x32_i8 on eight

@@ -234,13 +234,13 @@ __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf
 
 __global__ __launch_bounds__(256) void lstm_cell_kernel(const float* __restrict__ gx, const float* __restrict__ gh,
                                                         const float* __restrict__ bias,
-                                                        const float* __restrict__ c_in, int B, int H,
+                                                        const float* __restrict__ c_in, int B, int H, size_t gx_ld,
                                                         float* __restrict__ h_out, float* __restrict__ c_out,
                                                         float* __restrict__ y, size_t y_ld) {
     const size_t n = size_t(B) * H, stride = size_t(gridDim.x) * 256;
     for (size_t e = size_t(blockIdx.x) * 256 + threadIdx.x; e < n; e += stride) {
         const size_t b = e / H, j = e - b * H;
-        const float* px = gx + b * 4 * size_t(H);
+        const float* px = gx + b * gx_ld;
         const float* ph = gh + b * 4 * size_t(H);
         const size_t H2 = 2 * size_t(H), H3 = 3 * size_t(H);
         const float bi = bias ? bias[j] : 0.0f, bf = bias ? bias[H + j] : 0.0f;
@@ -354,15 +354,16 @@ int lq_dilate_nhwc_i8(const int8_t* x, int B, int H, int W, int C, int stride_h,
     return LQ_OK;
 }
 
-int lq_lstm_cell_f32(const float* gates_x, const float* gates_h, const float* bias, const float* c_in, int batch,
-                     int hidden,
+int lq_lstm_cell_f32(const float* gates_x, size_t gates_x_ld, const float* gates_h, const float* bias,
+                     const float* c_in, int batch, int hidden,
                      float* h_out, float* c_out, float* y, size_t y_ld, lq_stream stream) {
     LQ_REQUIRE(batch >= 0 && hidden >= 0, LQ_ERR_SHAPE, "lstm_cell_f32: negative extent");
     if (size_t(batch) * hidden == 0) return LQ_OK;
     LQ_REQUIRE(gates_x && gates_h && c_in && h_out && c_out, LQ_ERR_VALUE, "lstm_cell_f32: NULL pointer");
     LQ_REQUIRE(!y || y_ld >= size_t(hidden), LQ_ERR_SHAPE, "lstm_cell_f32: output row stride smaller than hidden");
+    LQ_REQUIRE(gates_x_ld >= size_t(4) * hidden, LQ_ERR_SHAPE, "lstm_cell_f32: gate row stride smaller than 4 * hidden");
     hipLaunchKernelGGL(lstm_cell_kernel, dim3(grid_for(size_t(batch) * hidden, 256)), dim3(256), 0,
-                       as_stream(stream), gates_x, gates_h, bias, c_in, batch, hidden, h_out, c_out, y, y_ld);
+                       as_stream(stream), gates_x, gates_h, bias, c_in, batch, hidden, gates_x_ld, h_out, c_out, y, y_ld);
     LQ_CHECK_LAUNCH("lstm_cell_f32");
     return LQ_OK;
 }

@@ -314,3 +314,39 @@ class ConvTranspose2d(Module):
         raise NotImplementedError(
             "float nn.ConvTranspose2d.forward is not part of the hip quantized-inference backend; "
             "quantize the model (convert) first")
+
+
+class LSTM(Module):
+    """Float LSTM as a parameter holder: ``weight_ih_l{k}`` (4H, in), ``weight_hh_l{k}``
+    (4H, H), ``bias_ih_l{k}``, ``bias_hh_l{k}`` (and ``..._reverse`` when bidirectional),
+    gate order i, f, g, o."""
+
+    def __init__(self, input_size: int, hidden_size: int, num_layers: int = 1, bias: bool = True,
+                 batch_first: bool = False, dropout: float = 0.0, bidirectional: bool = False,
+                 proj_size: int = 0) -> None:
+        super().__init__()
+        if proj_size:
+            raise NotImplementedError("LSTM: proj_size is not supported on the hip backend")
+        self.input_size, self.hidden_size, self.num_layers = input_size, hidden_size, num_layers
+        self.bias, self.batch_first, self.dropout = bias, batch_first, dropout
+        self.bidirectional, self.proj_size = bidirectional, 0
+        bound = 1.0 / np.sqrt(hidden_size)
+        rng = np.random.default_rng(input_size * 7919 + hidden_size * 31 + num_layers)
+        dirs = 2 if bidirectional else 1
+        for k in range(num_layers):
+            fan = input_size if k == 0 else hidden_size * dirs
+            for suffix in ("", "_reverse")[:dirs]:
+                u = lambda *shape: T.tensor(rng.uniform(-bound, bound, shape).astype(np.float32))
+                self.register_buffer(f"weight_ih_l{k}{suffix}", u(4 * hidden_size, fan))
+                self.register_buffer(f"weight_hh_l{k}{suffix}", u(4 * hidden_size, hidden_size))
+                if bias:
+                    self.register_buffer(f"bias_ih_l{k}{suffix}", u(4 * hidden_size))
+                    self.register_buffer(f"bias_hh_l{k}{suffix}", u(4 * hidden_size))
+
+    def named_parameters(self):
+        return list(self.named_buffers())
+
+    def forward(self, x, hx=None):
+        raise NotImplementedError(
+            "float nn.LSTM.forward is not part of the hip quantized-inference backend; "
+            "quantize the model (quantize_dynamic) first")

@@ -49,7 +49,7 @@ def _quant_mapping() -> dict[type, object]:
 
 
 def _dynamic_mapping() -> dict[type, object]:
-    return {nn.Linear: nnqd.Linear.from_float}
+    return {nn.Linear: nnqd.Linear.from_float, nn.LSTM: nnqd.LSTM.from_float}
 
 
 def _mlx_weight_bits(mod) -> int:

@@ -211,3 +211,74 @@ def test_conv_transpose2d(cin, cout, k, stride, padding, output_padding, dilatio
     got = np.transpose(out._grid.codes.numpy().astype(np.int32) + 128, (0, 3, 1, 2))
     d = np.abs(got - want)
     assert d.max() <= 1 and (d != 0).mean() < 0.01
+
+
+# ---------------------------------------------------------------- dynamic LSTM
+def _oracle_lstm_stack(q, x, hx, batch_first):
+    """Layer by layer, direction by direction, with Br.lstm on the dequantized weights."""
+    import lucid_amd.nn.quantized.dynamic as nnqd  # noqa: F401
+    H, dirs = q.hidden_size, 2 if q.bidirectional else 1
+    xs = np.transpose(x, (1, 0, 2)) if batch_first else x
+    Tn, Bn, _ = xs.shape
+    hs, cs = [], []
+    for k in range(q.num_layers):
+        outs = []
+        for d, suffix in enumerate(("", "_reverse")[:dirs]):
+            def w(name):
+                return (getattr(q, name + "_int8").numpy().astype(np.float32) *
+                        getattr(q, name + "_scale").numpy()[:, None]).astype(np.float32)
+            wih, whh = w(f"weight_ih_l{k}{suffix}"), w(f"weight_hh_l{k}{suffix}")
+            if q.bias:
+                bih, bhh = (getattr(q, f"bias_{n}_l{k}{suffix}").numpy() for n in ("ih", "hh"))
+            else:
+                bih = bhh = np.zeros(4 * H, np.float32)
+            idx = k * dirs + d
+            h0 = hx[0][idx] if hx is not None else np.zeros((Bn, H), np.float32)
+            c0 = hx[1][idx] if hx is not None else np.zeros((Bn, H), np.float32)
+            seq = xs[::-1] if d == 1 else xs
+            y, hn, cn = Br.lstm(seq, h0, c0, wih, whh, bih, bhh)
+            outs.append(y[::-1] if d == 1 else y)
+            hs.append(hn)
+            cs.append(cn)
+        xs = np.concatenate(outs, axis=-1)
+    y = np.transpose(xs, (1, 0, 2)) if batch_first else xs
+    return y, np.stack(hs), np.stack(cs)
+
+
+@pytest.mark.parametrize("layers,bidir,batch_first,bias,with_state",
+                         [(1, False, True, True, False), (2, True, False, True, True), (2, False, True, False, True)])
+def test_dynamic_lstm(layers, bidir, batch_first, bias, with_state):
+    import lucid_amd.nn.quantized.dynamic as nnqd
+    rng = np.random.default_rng(layers * 7 + bidir)
+    I, H, Bn, Tn = 8, 16, 4, 5
+    lstm = nn.LSTM(I, H, num_layers=layers, bias=bias, batch_first=batch_first, bidirectional=bidir)
+    qm = Q.quantize_dynamic(lstm)
+    assert isinstance(qm, nnqd.LSTM) and qm.weight_ih_l0_int8.dtype is L.int8
+    # test_dynamic_ptq.py:55-64: the state dict holds the int8 form only
+    assert [k for k in qm.state_dict() if k.startswith("weight_ih_l0")][:2] == ["weight_ih_l0_int8", "weight_ih_l0_scale"]
+    assert not any(k in qm.state_dict() for k in ("weight_ih_l0", "weight_hh_l0"))
+    x = rng.standard_normal((Bn, Tn, I) if batch_first else (Tn, Bn, I)).astype(np.float32)
+    dirs = 2 if bidir else 1
+    hx = None
+    if with_state:
+        hx = tuple(rng.standard_normal((layers * dirs, Bn, H)).astype(np.float32) for _ in range(2))
+    y, (hn, cn) = qm(hip(x), None if hx is None else (hip(hx[0]), hip(hx[1])))
+    wy, wh, wc = _oracle_lstm_stack(qm, x, hx, batch_first)
+    assert y.shape == wy.shape and hn.shape == wh.shape
+    for got, want in ((y.numpy(), wy), (hn.numpy(), wh), (cn.numpy(), wc)):
+        assert np.abs(got - want).max() < 2e-5
+    # test_dynamic_ptq.py:66-75: close to the float LSTM (float weights through the same recurrence)
+    fl = {n: t.numpy() for n, t in lstm.named_parameters()}
+
+    class F:  # the float weights presented as a "quantized" module with unit scales
+        pass
+    f = F()
+    f.hidden_size, f.bidirectional, f.num_layers, f.bias = H, bidir, layers, bias
+    for n, v in fl.items():
+        if n.startswith("weight"):
+            setattr(f, n + "_int8", type("A", (), {"numpy": lambda self, v=v: v})())
+            setattr(f, n + "_scale", type("A", (), {"numpy": lambda self, v=v: np.ones(v.shape[0], np.float32)})())
+        else:
+            setattr(f, n, type("A", (), {"numpy": lambda self, v=v: v})())
+    yf, _, _ = _oracle_lstm_stack(f, x, hx, batch_first)
+    assert np.abs(yf - y.numpy()).mean() / (np.abs(yf).mean() + 1e-9) < 0.03

@@ -17,6 +17,9 @@ pytestmark = pytest.mark.gpu
 
 def test_allocator_reuses_and_reports():
     _C.init()
+    import gc
+    gc.collect()
+    _C.call("lq_empty_cache")                       # no cached block of this size left from earlier tests
     used0, res0 = C.c_size_t(), C.c_size_t()
     _C.call("lq_memory_stats", C.byref(used0), C.byref(res0))
     a = L.Tensor.empty((1 << 20,), L.float32, "hip")
