@@ -1,9 +1,10 @@
 """The slice of ``lucid.nn`` that the quantized-inference path touches.
 
-Float ``Linear`` / ``Conv2d`` here are parameter holders that ``from_float`` /
+Float ``Conv2d`` and friends here are parameter holders that ``from_float`` /
 ``quantize_dynamic`` / ``convert`` read; their float forward is Lucid's CPU /
-Metal business and is not part of this backend (calling it raises).  ``ReLU``
-does compute: it sits between dynamic-quantized layers, whose outputs are float.
+Metal business and is not part of this backend (calling it raises).  ``Linear``,
+``ReLU`` and the pointwise activations do compute in float32 on the device, so that
+a prepared MLP can be calibrated where it will run.
 """
 
 from __future__ import annotations
@@ -57,9 +58,17 @@ class Linear(Module):
             rng.uniform(-bound, bound, out_features).astype(np.float32)) if bias else None)
 
     def forward(self, x):
-        raise NotImplementedError(
-            "float nn.Linear.forward is not part of the hip quantized-inference backend; "
-            "quantize the model (quantize_dynamic / convert) first")
+        """``x @ weight.T + bias`` in float32 on the device - what a calibration pass
+        through a prepared model needs (observers are forward hooks)."""
+        if not isinstance(x, Tensor) or x.device != "hip":
+            raise NotImplementedError(
+                "float nn.Linear.forward runs on the 'hip' device only; the CPU float path is Lucid's")
+        from .functional import linear_f32
+        w = self.weight if self.weight.device == "hip" else self.weight.to("hip")
+        b = self.bias
+        if b is not None and b.device != "hip":
+            b = b.to("hip")
+        return linear_f32(x, w, b)
 
     def extra_repr(self) -> str:
         return f"in_features={self.in_features}, out_features={self.out_features}"

@@ -1,0 +1,80 @@
+"""prepare -> calibrate -> convert -> infer entirely on the device
+(lucid/test/unit/quantization/test_device_metal.py is the template: the same recipe,
+with "hip" in place of "metal" and a numpy float model in place of the CPU run)."""
+
+import numpy as np
+import pytest
+
+import lucid_amd as L
+import lucid_amd.nn as nn
+import lucid_amd.quantization as Q
+
+pytestmark = pytest.mark.gpu
+
+
+def hip(a):
+    return L.tensor(np.asarray(a, np.float32), device="hip")
+
+
+def _static_quant(qconfig):
+    rng = np.random.default_rng(0)
+    m = nn.Sequential(nn.Linear(16, 16), nn.ReLU(), nn.Linear(16, 8)).to("hip")
+    qm = Q.prepare(m, qconfig)
+    for _ in range(4):
+        qm(hip(rng.standard_normal((4, 16))))       # observers are fed by the float forward
+    cm = Q.convert(qm)
+    x = np.array([[0.1 * i - 0.8 for i in range(16)] for _ in range(4)], np.float32)
+    w0, b0, w2, b2 = (t.numpy() for t in (m[0].weight, m[0].bias, m[2].weight, m[2].bias))
+    return cm, cm(hip(x)), np.maximum(x @ w0.T + b0, 0) @ w2.T + b2
+
+
+def test_float_linear_forward_matches_numpy():
+    rng = np.random.default_rng(1)
+    lin = nn.Linear(48, 24).to("hip")
+    x = rng.standard_normal((5, 7, 48)).astype(np.float32)
+    y = lin(hip(x)).numpy()
+    want = x @ lin.weight.numpy().T + lin.bias.numpy()
+    assert y.shape == (5, 7, 24) and np.abs(y - want).max() < 1e-5
+
+
+def test_static_ptq_round_trip_on_device():
+    # test_device_metal.py:53-65: no crash, finite, and within quantization noise of the float model
+    cm, y, yf = _static_quant(Q.get_default_qconfig())
+    assert y.device == "hip"
+    out = y.numpy()
+    assert np.isfinite(out).all()
+    assert np.abs(out - yf).max() < 5e-2
+
+
+def test_observers_were_fed_by_the_forward_hooks():
+    rng = np.random.default_rng(2)
+    m = nn.Sequential(nn.Linear(16, 16), nn.ReLU(), nn.Linear(16, 8)).to("hip")
+    qm = Q.prepare(m, Q.QConfig(activation=Q.MinMaxObserver, weight=Q.get_default_qconfig().weight))
+    xs = [rng.standard_normal((4, 16)).astype(np.float32) for _ in range(3)]
+    for x in xs:
+        qm(hip(x))
+    w0, b0 = m[0].weight.numpy(), m[0].bias.numpy()
+    h = np.concatenate([x @ w0.T + b0 for x in xs])
+    obs = qm[0].activation_post_process
+    assert np.isclose(obs.min_val.numpy(), h.min(), atol=1e-5) and np.isclose(obs.max_val.numpy(), h.max(), atol=1e-5)
+
+
+@pytest.mark.parametrize("factory", [Q.MinMaxObserver, Q.MovingAverageMinMaxObserver,
+                                     lambda: Q.PerChannelMinMaxObserver(ch_axis=0),
+                                     lambda: Q.MovingAveragePerChannelMinMaxObserver(ch_axis=0),
+                                     Q.HistogramObserver])
+def test_observers_calibrate_on_device(factory):
+    # test_device_metal.py:75-95
+    obs = factory()
+    x = np.random.default_rng(3).standard_normal((4, 8)).astype(np.float32)
+    obs(hip(x))
+    obs(hip(x * 1.5))
+    scale, zero_point = obs.calculate_qparams()
+    assert np.isfinite(scale.numpy()).all() and np.isfinite(zero_point.numpy()).all()
+
+
+def test_fake_quantize_takes_cpu_qparams_on_a_device_input():
+    # test_device_metal.py:98-109
+    x = hip(np.random.default_rng(4).standard_normal((4, 8)))
+    out = Q.fake_quantize(x, L.tensor(np.float32(0.05)), L.tensor(np.float32(0.0)), -128, 127, None)
+    assert out.device == "hip" and np.isfinite(out.numpy()).all()
