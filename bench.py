@@ -359,6 +359,48 @@ def bench_weight_only(L, _C, steps, warmup, K=4096, N=11008, gs=64):
     return out
 
 
+def bench_breadth(L, Q, _C, steps, warmup):
+    """HBM-bound members of the module breadth against 8 TB/s: the int8 embedding lookup
+    (1 B read + 4 B written per element gathered, plus 8 B per row of scale / zero point)
+    and a quantized activation on codes (1 B read + 1 B written per element)."""
+    import lucid_amd.nn as nn
+    import lucid_amd.nn.quantized as nnq
+
+    rng = np.random.default_rng(11)
+    out = {}
+    num, dim, n_idx = 50_000, 768, 64 * 512
+    emb = nnq.Embedding.from_float(nn.Embedding(num, dim))
+    idx = L.tensor(rng.integers(0, num, (64, 512)).astype(np.int64), device="hip")
+    res = L.Tensor.empty((64, 512, dim), L.float32, "hip")
+
+    def lookup():
+        _C.call("lq_embedding_i8", emb.weight_int8.data_ptr, emb.weight_scale.data_ptr,
+                emb.weight_zero_point.data_ptr, num, dim, idx.data_ptr, 1, n_idx, -1, res.data_ptr, None)
+
+    _, per = time_launches(_C, lookup, steps, warmup)
+    nbytes = n_idx * (dim * 5 + 8 + 8)
+    us = float(np.median(per)) * 1e3
+    out["embedding_50000x768_32768_lookups"] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                                                "frac_of_8TBs": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4),
+                                                "bytes": nbytes}
+    n = 1 << 28
+    codes = L.Tensor.empty((n,), L.int8, "hip")
+    _C.call("lq_fill_uniform_i8", codes.data_ptr, n, 5, -128, 127, None)
+    dst = L.Tensor.empty((n,), L.int8, "hip")
+    s_in, z_in = L.tensor(np.float32(0.05), device="hip"), L.tensor(np.float32(128.0), device="hip")
+    s_out, z_out = L.tensor(np.float32(1 / 255), device="hip"), L.tensor(np.float32(0.0), device="hip")
+
+    def act():
+        _C.call("lq_act_requant_i8", 0, 0.0, codes.data_ptr, -128, s_in.data_ptr, z_in.data_ptr, n,
+                s_out.data_ptr, z_out.data_ptr, 0, 255, -128, dst.data_ptr, None)
+
+    _, per = time_launches(_C, act, max(5, steps // 5), 2)
+    us = float(np.median(per)) * 1e3
+    out["sigmoid_on_codes_256Mi"] = {"us": round(us, 2), "GB/s": round(2 * n / us / 1e3, 1),
+                                     "frac_of_8TBs": round(2 * n / us / 1e3 / PEAK_HBM_GBS, 4), "bytes": 2 * n}
+    return out
+
+
 def bench_vit_linears(L, Q, _C, _ops, steps, warmup):
     """The four Linear shapes of a ViT-B/16 encoder block at batch 64 (12 608
     token rows), dynamic-quantized as nnqd.Linear does: per-tensor affine quint8
@@ -509,6 +551,7 @@ def main() -> int:
                                  "frac_of_int8_peak": round(rl["kernel_tops"] / PEAK_INT8_TOPS, 4)}
         del rl["tensors"]
         extra["weight_only_group64_k4096_n11008"] = bench_weight_only(L, _C, args.steps, args.warmup)
+        extra["module_breadth"] = bench_breadth(L, Q, _C, args.steps, args.warmup)
         extra["quant_roundtrip_4096x4096x16"] = bench_quant_roundtrip(
             L, Q, _C, max(10, args.steps // 2), max(3, args.warmup // 2))
         extra["dynamic_mlp_784_256_10_batch64"] = bench_dynamic_mlp(L, Q, _C, args.steps, args.warmup)
