@@ -481,6 +481,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="linear", choices=["linear"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="only print the MFMA-only rate for several operand distributions")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--cpu-sample-rows", type=int, default=2048)
     args = ap.parse_args()
@@ -495,6 +497,20 @@ def main() -> int:
 
     _C.init(0)
     M, K, N = 2048, 4096, 11008
+    if args.mfma_probe:
+        # the matrix cores' sustained rate by operand statistics (no data movement at all)
+        res = {}
+        n = 1 << 22
+        a, b = L.Tensor.empty((n,), L.int8, "hip"), L.Tensor.empty((n,), L.int8, "hip")
+        for name, lo, hi in (("all_zero", 0, 0), ("uniform_-8..7", -8, 7), ("uniform_0..127", 0, 127),
+                             ("uniform_-127..127", -127, 127)):
+            _C.call("lq_fill_uniform_i8", a.data_ptr, n, 1, lo, hi, None)
+            _C.call("lq_fill_uniform_i8", b.data_ptr, n, 2, lo, hi, None)
+            res[name] = round(probe_mfma_ceiling(L, _C, a, b), 1)
+        t = make_linear(L, Q, _C, _ops, M, K, N, 1)
+        res["benchmark_codes"] = round(probe_mfma_ceiling(L, _C, t["xq"], t["wq"]), 1)
+        print(json.dumps({"mfma_only_tops_by_operand_data": res, "datasheet_peak_tops": PEAK_INT8_TOPS}))
+        return 0
     r = bench_linear(L, Q, _C, _ops, M, K, N, args.steps, args.warmup)
     line = {
         "metric": "quantized-Linear int8 TOPS & % MFMA peak; int8 ResNet-50 images/sec",
