@@ -397,6 +397,27 @@ int lq_rowsum_i8(const int8_t* w, int32_t* out, int N, int K, lq_stream stream);
  * c - 128, and a_zp is then Z - 128); w: int8 [N,K].  All pointers are device
  * pointers; scales and output qparams are read on the device so no host
  * synchronisation is needed between layers. */
+/* Optional residual join on codes, fused into the REQUANT_I8 epilogue: what
+ * QFunctional.add / add_relu (lucid/nn/quantized/functional_module.py:224-230) does to
+ * this layer's output and a second activation, without the layer's own output ever
+ * reaching memory.  With c1 the layer's code on (out_scale, out_zp):
+ *     x1 = (c1 - out_zp) * out_scale          x2 = (q[m,n] - offset - zp) * scale
+ *     y  = x1 + x2,  y = max(y, 0) if relu
+ *     out[m,n] = code of y on (out_scale', out_zp', [out_qmin', out_qmax']) + out_offset'
+ * (primed = the fields of this struct), bit for bit what lq_add_requant_i8 gives on
+ * the stored intermediate.  q == NULL: no join. */
+typedef struct {
+    const int8_t* q;        /* [M, ld] stored codes of the other operand          */
+    long ld;                /* row stride in elements; 0 means N (Cout)           */
+    int offset;             /* storage offset of q's codes                        */
+    const float* scale;     /* [1] grid of q                                      */
+    const float* zp;        /* [1]                                                */
+    int relu;
+    const float* out_scale; /* [1] grid of the joined result                      */
+    const float* out_zp;    /* [1]                                                */
+    int out_qmin, out_qmax, out_offset;
+} lq_join_args;
+
 typedef struct {
     const int8_t* a;
     const int8_t* w;
@@ -428,6 +449,7 @@ typedef struct {
                               residual joins of a transformer block,
                               vit/_model.py:276-277); modes F32 / F16 only        */
     long ldr;              /* residual row stride in elements; 0 means N     */
+    lq_join_args join;     /* optional join on codes; mode REQUANT_I8 only   */
 } lq_qlinear_args;
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);
@@ -470,8 +492,12 @@ typedef struct {
     int out_qmin, out_qmax, out_offset;
     void* out;             /* NHWC [B,OH,OW,Cout]                            */
     int force_path;        /* 0 = choose; 1 = gemm (1x1), 2 = implicit GEMM,
-                              3 = explicit im2col + GEMM, 4 = naive          */
+                              3 = explicit im2col + GEMM, 4 = naive,
+                              5 = packed 4-channel image (Cin <= 4)          */
     int tile_config;
+    lq_join_args join;     /* optional join on codes (NHWC, ld = Cout): the residual
+                              add of a bottleneck block fused into its last
+                              convolution; mode REQUANT_I8 only                  */
 } lq_qconv2d_args;
 
 int lq_qconv2d_i8(const lq_qconv2d_args* args, lq_stream stream);

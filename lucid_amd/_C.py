@@ -111,6 +111,15 @@ _SIGNATURES = {
 }
 
 
+class JoinArgs(C.Structure):
+    """``lq_join_args`` of ``include/lucid_hip.h``."""
+
+    _fields_ = [
+        ("q", _vp), ("ld", C.c_long), ("offset", _i), ("scale", _vp), ("zp", _vp), ("relu", _i),
+        ("out_scale", _vp), ("out_zp", _vp), ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
+    ]
+
+
 class QLinearArgs(C.Structure):
     """``lq_qlinear_args`` of ``include/lucid_hip.h``."""
 
@@ -122,7 +131,7 @@ class QLinearArgs(C.Structure):
         ("out_scale", _vp), ("out_zp", _vp),
         ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
         ("out", _vp), ("ldo", C.c_long), ("force_path", _i), ("tile_config", _i),
-        ("residual", _vp), ("ldr", C.c_long),
+        ("residual", _vp), ("ldr", C.c_long), ("join", JoinArgs),
     ]
 
 
@@ -172,7 +181,7 @@ class QConv2dArgs(C.Structure):
         ("bias", _vp), ("bias_dtype", _i), ("relu", _i), ("out_mode", _i),
         ("out_scale", _vp), ("out_zp", _vp),
         ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
-        ("out", _vp), ("force_path", _i), ("tile_config", _i),
+        ("out", _vp), ("force_path", _i), ("tile_config", _i), ("join", JoinArgs),
     ]
 
 

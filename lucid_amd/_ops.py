@@ -44,10 +44,11 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
                out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
                out_qmax: int = 255, out_offset: int = 0, path: int = PATH_AUTO,
                tile_config: int = 0, out: Tensor | None = None, repeat: int = 1,
-               residual: Tensor | None = None) -> Tensor:
+               residual: Tensor | None = None, join=None) -> Tensor:
     """Fused int8 GEMM + epilogue; see ``lq_qlinear_i8`` in ``lucid_hip.h``.
     ``a`` is int8 ``[M, K]``, ``w`` int8 ``[N, K]``; the result is ``[M, N]``.
-    ``residual`` (float32, ``M*N`` elements) is added after the activation."""
+    ``residual`` (float32, ``M*N`` elements) is added after the activation;
+    ``join`` fuses a residual add on codes after the requantize (see ``_fill_join``)."""
     if a.ndim != 2 or w.ndim != 2 or a.shape[1] != w.shape[1]:
         raise _C.ShapeMismatch(f"qlinear_i8: a {a.shape} and w {w.shape} do not form a GEMM")
     M, K = a.shape
@@ -80,6 +81,7 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
     if residual is not None and residual.numel != M * N:
         raise _C.ShapeMismatch(f"residual has {residual.numel} elements for an output of {M}x{N}")
     args.residual, args.ldr = _ptr(residual, "residual", T.float32), 0
+    _fill_join(args.join, join, (M, N))
     if repeat == 1:
         _C.call("lq_qlinear_i8", C.byref(args), None)
     else:
@@ -87,12 +89,28 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
     return out
 
 
-CONV_AUTO, CONV_GEMM, CONV_IMPLICIT, CONV_IM2COL, CONV_NAIVE = range(5)
+CONV_AUTO, CONV_GEMM, CONV_IMPLICIT, CONV_IM2COL, CONV_NAIVE, CONV_PACKED4 = range(6)
 
 
 def conv_out_size(size: int, k: int, stride: int, pad_lo: int, pad_hi: int, dil: int) -> int:
     """Output extent of one spatial axis (``lucid/_C/nn/ConvNd.cpp:56-59``)."""
     return (size + pad_lo + pad_hi - dil * (k - 1) - 1) // stride + 1
+
+
+def _fill_join(j, join, out_shape) -> None:
+    """``join`` = dict(q=codes tensor shaped like the output, offset, scale, zp, relu, out_scale,
+    out_zp, out_qmin, out_qmax, out_offset): the residual add on codes fused into the epilogue."""
+    if join is None:
+        return
+    q = join["q"]
+    if tuple(q.shape) != tuple(out_shape):
+        raise _C.ShapeMismatch(f"join operand {q.shape} does not match the output {tuple(out_shape)}")
+    j.q, j.ld, j.offset = _ptr(q, "join.q", T.int8), 0, int(join["offset"])
+    j.scale, j.zp = _ptr(join["scale"], "join.scale", T.float32), _ptr(join["zp"], "join.zp", T.float32)
+    j.relu = int(join.get("relu", False))
+    j.out_scale = _ptr(join["out_scale"], "join.out_scale", T.float32)
+    j.out_zp = _ptr(join["out_zp"], "join.out_zp", T.float32)
+    j.out_qmin, j.out_qmax, j.out_offset = int(join["out_qmin"]), int(join["out_qmax"]), int(join["out_offset"])
 
 
 def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None,
@@ -101,7 +119,7 @@ def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None
                groups: int = 1, relu: bool = False, out_mode: int = OUT_F32,
                out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
                out_qmax: int = 255, out_offset: int = 0, path: int = CONV_AUTO,
-               tile_config: int = 0) -> Tensor:
+               tile_config: int = 0, join=None) -> Tensor:
     """Fused int8 convolution; see ``lq_qconv2d_i8``.  ``x`` int8 NHWC, ``w``
     int8 ``[Cout, KH, KW, Cin/groups]``, ``pad`` = (h_lo, h_hi, w_lo, w_hi).
     Returns NHWC ``[B, OH, OW, Cout]``."""
@@ -128,5 +146,6 @@ def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None
     a.out_scale, a.out_zp = _ptr(out_scale, "out_scale", T.float32), _ptr(out_zp, "out_zp", T.float32)
     a.out_qmin, a.out_qmax, a.out_offset = int(out_qmin), int(out_qmax), int(out_offset)
     a.out, a.force_path, a.tile_config = out.data_ptr, int(path), int(tile_config)
+    _fill_join(a.join, join, out.shape)
     _C.call("lq_qconv2d_i8", C.byref(a), None)
     return out

@@ -9,8 +9,11 @@
 // the code Z.  Three routes:
 //   gemm     : 1x1, stride 1, no padding -> the NHWC tensor IS the A matrix
 //   implicit : Cin/groups % 16 == 0 -> the tile kernel gathers A on the fly
-//   im2col   : anything else (e.g. a 7x7x3 stem) -> explicit int8 im2col into
-//              the workspace with K padded to a multiple of 16, then the GEMM
+//   packed   : at most four input channels (an RGB stem) -> image repacked once to
+//              4 channels with the padding materialised; a filter row is then
+//              contiguous bytes and the tile kernel gathers it without im2col
+//   im2col   : anything else -> explicit int8 im2col into the workspace with K
+//              padded to a multiple of 16, then the GEMM
 //   naive    : one output per lane, any shape (checking aid)
 #include "common.hpp"
 #include "qepilogue.hpp"
@@ -100,6 +103,48 @@ __global__ void pad_rows_kernel(const int8_t* __restrict__ w, int8_t* __restrict
         const int k = int(idx % Kp);
         const size_t r = idx / Kp;
         out[idx] = k < K ? w[r * K + k] : int8_t(0);
+    }
+}
+
+// ---------------------------------------------------------------- few input channels
+// A convolution over at most four input channels (an RGB stem) as an implicit GEMM
+// without im2col: the image is copied once into a 4-channel, spatially pre-padded
+// buffer - padding and the spare channels hold the zero-point code -, so that four
+// neighbouring pixels of a row are one 16-byte chunk and a filter row of KWp = KW
+// rounded up to 4 taps is KWp * 4 contiguous bytes.  The tile kernel then gathers it as a
+// convolution over 16-byte "super pixels": KWp / 4 taps per filter row, each four real
+// pixels apart, no bounds to check.  The filter gets zeros in the added taps and channel.
+__global__ __launch_bounds__(256) void pack4_padded_kernel(const int8_t* __restrict__ x, int B, int H, int W, int C,
+                                                           int ph, int pw, int Hp, int Wp, int fill,
+                                                           uint32_t* __restrict__ out) {
+    const size_t n = size_t(B) * Hp * Wp, stride = size_t(gridDim.x) * 256;
+    const uint32_t f = uint32_t(uint8_t(fill));
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+        const int wp = int(i % Wp);
+        size_t r = i / Wp;
+        const int hp = int(r % Hp), b = int(r / Hp);
+        const int h = hp - ph, w = wp - pw;
+        uint32_t v = f | (f << 8) | (f << 16) | (f << 24);
+        if (h >= 0 && h < H && w >= 0 && w < W) {
+            const int8_t* src = x + ((size_t(b) * H + h) * W + w) * C;
+            v = 0;
+            for (int c = 0; c < 4; ++c) v |= (c < C ? uint32_t(uint8_t(src[c])) : f) << (8 * c);
+        }
+        out[i] = v;
+    }
+}
+
+// w [Cout, KH, KW, C] -> [Cout, KH, KWp, 4], zeros in the added taps and channels
+__global__ void pack4_filter_kernel(const int8_t* __restrict__ w, int Cout, int KH, int KW, int C, int KWp,
+                                    int8_t* __restrict__ out) {
+    const size_t total = size_t(Cout) * KH * KWp * 4;
+    for (size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * blockDim.x) {
+        const int c = int(idx % 4);
+        size_t r = idx / 4;
+        const int kw = int(r % KWp);
+        r /= KWp;  // = co * KH + kh
+        out[idx] = (c < C && kw < KW) ? w[(r * KW + kw) * C + c] : int8_t(0);
     }
 }
 
@@ -298,19 +343,54 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
     g.cx = p->x; g.cH = p->H; g.cW = p->W; g.cCin = p->Cin; g.cOH = OH; g.cOW = OW; g.cKW = p->KW;
     g.cCg = Cg; g.csh = p->stride_h; g.csw = p->stride_w; g.cph = p->pad_h_lo; g.cpw = p->pad_w_lo;
     g.cdh = p->dil_h; g.cdw = p->dil_w;
+    const int jrc = set_join(g, p->join, p->out_mode, p->Cout, "qconv2d_i8");
+    if (jrc) return jrc;
 
     const bool is_gemm = p->KH == 1 && p->KW == 1 && p->stride_h == 1 && p->stride_w == 1 &&
                          p->pad_h_lo == 0 && p->pad_h_hi == 0 && p->pad_w_lo == 0 &&
                          p->pad_w_hi == 0 && p->groups == 1;
     const bool aligned = aligned16(p->x) && aligned16(p->w);
-    int path = p->force_path;  // 0 = choose, 1 = gemm, 2 = implicit, 3 = im2col, 4 = naive
+    int path = p->force_path;  // 0 = choose, 1 = gemm, 2 = implicit, 3 = im2col, 4 = naive, 5 = packed 4-channel
+    const bool few_channels = p->Cin <= 4 && p->groups == 1 && p->dil_w == 1 && p->KH * ((p->KW + 3) / 4) * 16 <= 131071;
     if (path == 0) {
         if (is_gemm && p->Cin % 16 == 0 && aligned)
             path = 1;
         else if (Cg % 16 == 0 && aligned)
             path = 2;
+        else if (few_channels)
+            path = 5;
         else
             path = 3;
+    }
+    if (path == 5) {
+        LQ_REQUIRE(few_channels, LQ_ERR_VALUE,
+                   "qconv2d_i8: the packed route needs Cin <= 4, groups == 1 and dilation_w == 1");
+        const int KWp = (p->KW + 3) / 4 * 4;
+        const int Hp = p->H + p->pad_h_lo + p->pad_h_hi;
+        int Wp = p->W + p->pad_w_lo + p->pad_w_hi;
+        const int need = (OW - 1) * p->stride_w + KWp;  // the last output's window of KWp pixels
+        Wp = Wp > need ? Wp : need;
+        Wp = (Wp + 3) / 4 * 4;                          // rows start 16-byte aligned
+        const size_t img_bytes = (size_t(p->B) * Hp * Wp * 4 + 255) / 256 * 256;
+        const size_t flt_bytes = (size_t(p->Cout) * p->KH * KWp * 4 + 255) / 256 * 256;
+        LQ_REQUIRE(size_t(p->B) * Hp * Wp * 4 < 0xffffffffull, LQ_ERR_SHAPE, "qconv2d_i8: padded image too large");
+        void* ws = nullptr;
+        int rc = workspace(img_bytes + flt_bytes, &ws);
+        if (rc) return rc;
+        int8_t* img = static_cast<int8_t*>(ws);
+        int8_t* flt = img + img_bytes;
+        hipLaunchKernelGGL(pack4_padded_kernel, dim3(grid_1d(size_t(p->B) * Hp * Wp)), dim3(256), 0, st, p->x, p->B,
+                           p->H, p->W, p->Cin, p->pad_h_lo, p->pad_w_lo, Hp, Wp, p->a_zp,
+                           reinterpret_cast<uint32_t*>(img));
+        LQ_CHECK_LAUNCH("pack4_padded");
+        hipLaunchKernelGGL(pack4_filter_kernel, dim3(grid_1d(size_t(p->Cout) * p->KH * KWp * 4)), dim3(256), 0, st,
+                           p->w, p->Cout, p->KH, p->KW, p->Cin, KWp, flt);
+        LQ_CHECK_LAUNCH("pack4_filter");
+        GemmArgs gg = g;
+        gg.w = flt; gg.K = p->KH * KWp * 4; gg.N = p->Cout;
+        gg.cx = img; gg.cH = Hp; gg.cW = Wp; gg.cCin = 4; gg.cCg = 16; gg.cKW = KWp / 4;
+        gg.cph = 0; gg.cpw = 0; gg.cdw = 4;  // a tap of the gather = four real pixels
+        return run_tile_kernel(gg, true, 1, p->tile_config, st);
     }
     if (path == 1) {
         LQ_REQUIRE(is_gemm, LQ_ERR_VALUE, "qconv2d_i8: the gemm route needs a 1x1 stride-1 unpadded conv");
@@ -359,6 +439,7 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
             gg.bias = static_cast<const char*>(g.bias) + col0 * (g.bias_dtype == LQ_F16 ? 2 : 4);
         const size_t esz = g.out_mode == OUT_F16 ? 2 : (g.out_mode == OUT_REQUANT_I8 ? 1 : 4);
         gg.out = static_cast<char*>(g.out) + col0 * esz;
+        if (g.join_q) gg.join_q = g.join_q + col0;
         rc = run_gemm(gg, 0, p->tile_config, st);
         if (rc) return rc;
     }

@@ -113,6 +113,44 @@ __device__ __forceinline__ uint32_t add_residual(const GemmArgs& g, uint32_t bit
     return bits;
 }
 
+// The fused residual join on codes (lucid/nn/quantized/functional_module.py:224-230 applied
+// to this layer's output): both operands are dequantized in float32 with their own
+// grids, added, optionally clamped at zero, and requantized.
+struct JoinParams {
+    float S1, Z1;          // this layer's output grid
+    float s2, z2;          // the other operand's grid
+    float S, Z, lo, hi;    // the join's output grid
+};
+
+__device__ __forceinline__ JoinParams load_join(const GemmArgs& g, float S1, float Z1) {
+    JoinParams jp;
+    jp.S1 = S1, jp.Z1 = Z1;
+    jp.s2 = g.join_scale[0], jp.z2 = g.join_zp[0];
+    jp.S = g.join_out_scale[0], jp.Z = g.join_out_zp[0];
+    jp.lo = float(g.join_out_qmin), jp.hi = float(g.join_out_qmax);
+    return jp;
+}
+
+// bits: this layer's stored code (code + out_offset); other: the partner's stored code
+__device__ __forceinline__ uint32_t join_code(const GemmArgs& g, const JoinParams& jp, uint32_t bits, int other) {
+    const float x1 = (float(int(bits) - g.out_offset) - jp.Z1) * jp.S1;
+    const float x2 = (float(other - g.join_off) - jp.z2) * jp.s2;
+    float y = x1 + x2;
+    if (g.join_relu) y = (y < 0.0f) ? 0.0f : y;
+    const float qv = q_core(y, jp.S, jp.Z, jp.lo, jp.hi);
+    return uint32_t(((qv != qv) ? 0 : int(qv)) + g.join_out_offset);
+}
+
+// one element's residual step, whichever form the output mode has
+template <int MODE>
+__device__ __forceinline__ uint32_t finish_value(const GemmArgs& g, uint32_t bits, int m, int n, float S, float Z) {
+    if (MODE == OUT_REQUANT_I8 && g.join_q) {
+        const JoinParams jp = load_join(g, S, Z);
+        return join_code(g, jp, bits, int(g.join_q[size_t(m) * size_t(g.join_ld) + size_t(n)]));
+    }
+    return add_residual<MODE>(g, bits, m, n);
+}
+
 template <int MODE>
 __device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint32_t v) {
     if (MODE == OUT_F16)
@@ -143,7 +181,7 @@ template <int MODE>
 __device__ __forceinline__ void epilogue_store_t(const GemmArgs& g, int m, int n, int32_t acc,
                                                  float as, const ColParams& c, float S, float Z) {
     store_scalar<MODE>(g, size_t(m) * size_t(g.ldo) + size_t(n),
-                       add_residual<MODE>(g, epilogue_value<MODE>(g, acc, as, c, S, Z), m, n));
+                       finish_value<MODE>(g, epilogue_value<MODE>(g, acc, as, c, S, Z), m, n, S, Z));
 }
 
 __device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, int32_t acc,

@@ -133,7 +133,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
                              g.cdh * 16 + g.cdw, g.cOW};
         std::memcpy(key.geom, geom, sizeof(geom));
     }
-    key.flags = (g.residual ? 1 : 0) | (g.a_scale_per_row ? 2 : 0) | (g.bias ? 4 : 0);
+    key.flags = (g.residual ? 1 : 0) | (g.a_scale_per_row ? 2 : 0) | (g.bias ? 4 : 0) | (g.join_q ? 8 : 0);
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);
         auto it = g_tune.find(key);
@@ -461,6 +461,8 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
     g.out_qmin = p->out_qmin; g.out_qmax = p->out_qmax; g.out_offset = p->out_offset;
     g.out = p->out; g.ldo = ldo; g.zeros = nullptr;
     g.cx = nullptr; g.pad_src = nullptr;
+    const int jrc = set_join(g, p->join, p->out_mode, p->N, "qlinear_i8");
+    if (jrc) return jrc;
 
     return run_gemm(g, p->force_path, p->tile_config, as_stream(stream));
 }

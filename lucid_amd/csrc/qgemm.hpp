@@ -27,6 +27,18 @@ struct GemmArgs {
     long ldo;
     const float* residual;  // optional [M, ldr] float32 added to y after the activation (float outputs only)
     long ldr;
+    // Optional join on codes after the requantize (OUT_REQUANT_I8 only): the layer's code
+    // and join_q[m, n] are dequantized with their own grids, added, optionally clamped at
+    // zero, and requantized to (join_out_*): QFunctional.add / add_relu fused in.
+    const int8_t* join_q;   // [M, join_ld] stored codes, or null
+    long join_ld;
+    int join_off;           // storage offset of join_q's codes
+    const float* join_scale;
+    const float* join_zp;
+    int join_relu;
+    const float* join_out_scale;
+    const float* join_out_zp;
+    int join_out_qmin, join_out_qmax, join_out_offset;
     const int8_t* zeros;  // >= 16 zero bytes, source for K-tail chunks
     // Implicit-GEMM convolution (tile kernel instantiated with CONV = true): the
     // A operand is gathered from NHWC activation codes; row m is output pixel
@@ -41,6 +53,24 @@ struct GemmArgs {
     int sk_tiles;  // the last sk_tiles tile ids are shared between workers
 };
 
+
+// Validates a join description against the output mode and copies it into g
+// (ld 0 = n_cols).
+inline int set_join(GemmArgs& g, const lq_join_args& j, int out_mode, long n_cols, const char* who) {
+    g.join_q = nullptr;
+    if (j.q == nullptr) return LQ_OK;
+    LQ_REQUIRE(out_mode == OUT_REQUANT_I8, LQ_ERR_VALUE, "%s: a join on codes needs out_mode REQUANT_I8", who);
+    LQ_REQUIRE(j.scale && j.zp && j.out_scale && j.out_zp, LQ_ERR_VALUE, "%s: join qparams are NULL", who);
+    LQ_REQUIRE(j.out_qmin <= j.out_qmax && j.out_qmin + j.out_offset >= -128 && j.out_qmax + j.out_offset <= 127,
+               LQ_ERR_VALUE, "%s: join output grid [%d,%d] + offset %d does not fit int8", who, j.out_qmin,
+               j.out_qmax, j.out_offset);
+    const long ld = j.ld ? j.ld : n_cols;
+    LQ_REQUIRE(ld >= n_cols, LQ_ERR_SHAPE, "%s: join row stride %ld < %ld columns", who, ld, n_cols);
+    g.join_q = j.q; g.join_ld = ld; g.join_off = j.offset; g.join_scale = j.scale; g.join_zp = j.zp;
+    g.join_relu = j.relu; g.join_out_scale = j.out_scale; g.join_out_zp = j.out_zp;
+    g.join_out_qmin = j.out_qmin; g.join_out_qmax = j.out_qmax; g.join_out_offset = j.out_offset;
+    return LQ_OK;
+}
 
 // 256 blocks of 16 bytes; block v is filled with byte value v.  Block 0 is the
 // zero source for K-tail chunks, block (uint8)zp the source for out-of-image

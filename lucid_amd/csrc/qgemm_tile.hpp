@@ -122,6 +122,15 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                 for (int p = 0; p < PASSES; ++p)
                     rv[p] = *reinterpret_cast<const float4*>(rp + size_t(p) * ROWS_PER_PASS * size_t(g.ldr));
             }
+            // the other operand of a fused join on codes: four codes per row, requested early too
+            const bool join_fast = MODE == OUT_REQUANT_I8 && interior && g.join_q != nullptr;
+            uint32_t jv[MODE == OUT_REQUANT_I8 ? PASSES : 1];
+            if (MODE == OUT_REQUANT_I8 && join_fast) {
+                const int8_t* jq = g.join_q + size_t(m_first) * size_t(g.join_ld) + size_t(n);
+#pragma unroll
+                for (int p = 0; p < PASSES; ++p)
+                    jv[p] = *reinterpret_cast<const uint32_t*>(jq + size_t(p) * ROWS_PER_PASS * size_t(g.join_ld));
+            }
             // this lane's rows of the part: groups of four consecutive rows
             float as[RPP];
 #pragma unroll
@@ -156,6 +165,16 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                         v[p].w = __float_as_uint(__uint_as_float(v[p].w) + rv[p].w);
                     }
                 }
+                if (MODE == OUT_REQUANT_I8 && join_fast) {
+                    const JoinParams jp = load_join(g, S, Z);
+#pragma unroll
+                    for (int p = 0; p < PASSES; ++p) {
+                        v[p].x = join_code(g, jp, v[p].x, int(int8_t(jv[p] & 0xff)));
+                        v[p].y = join_code(g, jp, v[p].y, int(int8_t((jv[p] >> 8) & 0xff)));
+                        v[p].z = join_code(g, jp, v[p].z, int(int8_t((jv[p] >> 16) & 0xff)));
+                        v[p].w = join_code(g, jp, v[p].w, int(int8_t(jv[p] >> 24)));
+                    }
+                }
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
                     store_vec4<MODE>(g, idx, v[p]);
@@ -167,10 +186,10 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                     uint4 v = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
                     const int m = m_first + p * ROWS_PER_PASS;
                     if (m < g.M && n < n_limit) {
-                        v.x = add_residual<MODE>(g, v.x, m, n);
-                        if (n + 1 < n_limit) v.y = add_residual<MODE>(g, v.y, m, n + 1);
-                        if (n + 2 < n_limit) v.z = add_residual<MODE>(g, v.z, m, n + 2);
-                        if (n + 3 < n_limit) v.w = add_residual<MODE>(g, v.w, m, n + 3);
+                        v.x = finish_value<MODE>(g, v.x, m, n, S, Z);
+                        if (n + 1 < n_limit) v.y = finish_value<MODE>(g, v.y, m, n + 1, S, Z);
+                        if (n + 2 < n_limit) v.z = finish_value<MODE>(g, v.z, m, n + 2, S, Z);
+                        if (n + 3 < n_limit) v.w = finish_value<MODE>(g, v.w, m, n + 3, S, Z);
                         const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
                         if (vec_ok && n + 4 <= n_limit) {
                             store_vec4<MODE>(g, idx, v);
@@ -479,7 +498,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         const bool interior = m0 + BM <= g.M && n0 + BN <= n_limit && g.ldo % 4 == 0 &&
                               reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0 &&
                               (g.residual == nullptr ||
-                               (g.ldr % 4 == 0 && reinterpret_cast<uintptr_t>(g.residual) % 16 == 0));
+                               (g.ldr % 4 == 0 && reinterpret_cast<uintptr_t>(g.residual) % 16 == 0)) &&
+                              (g.join_q == nullptr ||
+                               (g.join_ld % 4 == 0 && reinterpret_cast<uintptr_t>(g.join_q) % 4 == 0));
         __syncthreads();
         tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z, interior);
         __syncthreads();  // the staging area is the next tile's first LDS stage

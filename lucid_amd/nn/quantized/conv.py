@@ -95,7 +95,10 @@ class Conv2d(Module):
         self._w_ohwi = w
         self._wsum = _ops.rowsum_i8(w)
 
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, join=None) -> Tensor:
+        """``join = (other, qfunctional, relu)`` fuses ``qfunctional.add[_relu](self(x), other)``
+        into this layer's epilogue: the result is on the functional's grid, bit for bit what
+        the two separate modules give, and the layer's own output is never stored."""
         name = type(self).__name__
         g = input_grid(x, name)
         if x.ndim != 4 or x.shape[1] != self.in_channels:
@@ -121,14 +124,29 @@ class Conv2d(Module):
             _C.call("lq_pad_nhwc_i8", in_codes.data_ptr, padded.data_ptr, B, H, W, Ci, pad[0], pad[1], pad[2],
                     pad[3], _PAD_MODES[self.padding_mode], None)
             in_codes, pad = padded, (0, 0, 0, 0)
+        jarg = out_grid = None
+        if join is not None:
+            other, fn, relu = join
+            go = input_grid(other, name)
+            if go.layout != "nhwc":
+                raise _C.LucidError(f"{name}: the joined operand's codes must be stored NHWC")
+            if fn._zp_host is None:
+                fn._zp_host = int(host_scalar(fn.zero_point))
+            foff = storage_offset(fn.qdtype)
+            jarg = dict(q=go.codes, offset=go.offset, scale=go.scale, zp=go.zero_point, relu=relu,
+                        out_scale=fn.scale, out_zp=fn.zero_point, out_qmin=fn.qdtype.quant_min,
+                        out_qmax=fn.qdtype.quant_max, out_offset=foff)
+            out_grid = (fn.scale, fn.zero_point, fn.qdtype, foff, fn._zp_host)
         codes = _ops.qconv2d_i8(
             in_codes, self._w_ohwi, a_zp=int(g.zp_host) + g.offset, a_scale=g.scale,
             w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias, stride=self.stride,
             pad=pad, dilation=self.dilation, groups=self.groups,
             relu=self._fused_relu, out_mode=_ops.OUT_REQUANT_I8, out_scale=self.scale,
             out_zp=self.zero_point, out_qmin=self.out_qdtype.quant_min,
-            out_qmax=self.out_qdtype.quant_max, out_offset=off)
+            out_qmax=self.out_qdtype.quant_max, out_offset=off, join=jarg)
         B, OH, OW, Co = codes.shape
+        if out_grid is not None:
+            return Tensor.on_grid((B, Co, OH, OW), Grid(codes, *out_grid, "nhwc"))
         return Tensor.on_grid((B, Co, OH, OW), Grid(codes, self.scale, self.zero_point,
                                                     self.out_qdtype, off, self._zp_host, "nhwc"))
 

@@ -192,3 +192,85 @@ def test_conv_module_with_a_padding_mode(padding_mode):
                     out_mode=O.OUT_REQUANT_I8, out_scale=0.05, out_zp=120.0, out_qmin=0, out_qmax=255,
                     out_offset=-128)
     assert np.array_equal(got, exp)
+
+
+@pytest.mark.parametrize("shape,path", [((2, 14, 14, 64, 256, 1, 1), 0), ((2, 14, 14, 64, 96, 3, 3), 0),
+                                        ((3, 9, 7, 32, 40, 3, 3), 0), ((2, 9, 7, 6, 10, 3, 3), 0),
+                                        ((2, 9, 7, 32, 40, 3, 3), 4)])
+def test_fused_join_equals_conv_then_add_requant(shape, path):
+    """The residual add on codes fused into the epilogue gives the bits of the two-kernel
+    form: conv -> stored codes -> lq_add_requant_i8 (functional_module.py:224-230)."""
+    from lucid_amd import _C, _ops
+    B, H, W, Cin, Cout, KH, KW = shape
+    rng = np.random.default_rng(sum(shape))
+    x = rng.integers(-128, 128, (B, H, W, Cin)).astype(np.int8)
+    w = rng.integers(-127, 128, (Cout, KH, KW, Cin)).astype(np.int8)
+    ws = (rng.random(Cout).astype(np.float32) + 0.5) * 1e-3
+    bias = rng.standard_normal(Cout).astype(np.float32) * 0.1
+    hip = lambda a: L.tensor(a, device="hip")
+    dw, dx = hip(w), hip(x)
+    common = dict(a_zp=-3, a_scale=hip(np.float32(0.02)), w_scale=hip(ws), wsum=_ops.rowsum_i8(dw),
+                  bias=hip(bias), pad=(1, 1, 1, 1) if KH == 3 else (0, 0, 0, 0), relu=False,
+                  out_mode=_ops.OUT_REQUANT_I8, out_scale=hip(np.float32(0.03)), out_zp=hip(np.float32(120.0)),
+                  out_qmin=0, out_qmax=255, out_offset=-128, path=path)
+    first = _ops.qconv2d_i8(dx, dw, **common)
+    other = rng.integers(-128, 128, first.shape).astype(np.int8)
+    d_other = hip(other)
+    s2, z2 = hip(np.float32(0.025)), hip(np.float32(131.0))
+    S, Z = hip(np.float32(0.04)), hip(np.float32(7.0))
+    for relu in (True, False):
+        want = L.Tensor.empty(first.shape, L.int8, "hip")
+        _C.call("lq_add_requant_i8", first.data_ptr, -128, common["out_scale"].data_ptr, common["out_zp"].data_ptr,
+                d_other.data_ptr, -128, s2.data_ptr, z2.data_ptr, first.numel, int(relu), S.data_ptr, Z.data_ptr,
+                0, 255, -128, want.data_ptr, None)
+        fused = _ops.qconv2d_i8(dx, dw, **common, join=dict(q=d_other, offset=-128, scale=s2, zp=z2, relu=relu,
+                                                             out_scale=S, out_zp=Z, out_qmin=0, out_qmax=255,
+                                                             out_offset=-128))
+        assert np.array_equal(fused.numpy(), want.numpy())
+    # the oracle's two steps, once
+    o1 = O.qconv2d(x, w, -3, 0.02, ws, pad=common["pad"], bias=bias, out_mode=O.OUT_REQUANT_I8, out_scale=0.03,
+                   out_zp=120.0, out_qmin=0, out_qmax=255, out_offset=-128)
+    o2 = O.add_requant(o1, -128, 0.03, 120.0, other, -128, 0.025, 131.0, False, 0.04, 7.0, 0, 255, -128)
+    assert np.array_equal(fused.numpy(), o2)
+
+
+def test_join_needs_the_requantizing_mode():
+    from lucid_amd import _ops
+    hip = lambda a: L.tensor(a, device="hip")
+    x, w = hip(np.zeros((1, 4, 4, 16), np.int8)), hip(np.zeros((16, 1, 1, 16), np.int8))
+    one = hip(np.float32(1.0))
+    j = dict(q=hip(np.zeros((1, 4, 4, 16), np.int8)), offset=0, scale=one, zp=one, relu=False, out_scale=one,
+             out_zp=one, out_qmin=-128, out_qmax=127, out_offset=0)
+    with pytest.raises(ValueError, match="REQUANT_I8"):
+        _ops.qconv2d_i8(x, w, a_zp=0, a_scale=one, w_scale=hip(np.ones(16, np.float32)), out_mode=_ops.OUT_F32,
+                        join=j)
+
+
+@pytest.mark.parametrize("B,H,W,Cin,Cout,KH,KW,stride,pad", [
+    (2, 224, 224, 3, 64, 7, 7, (2, 2), (3, 3, 3, 3)),   # the ResNet stem
+    (3, 17, 13, 3, 24, 3, 3, (1, 1), (1, 1, 1, 1)),
+    (2, 20, 9, 1, 16, 5, 2, (2, 1), (2, 1, 0, 1)),      # one channel, asymmetric padding, odd sizes
+    (2, 11, 11, 4, 40, 3, 5, (1, 3), (0, 0, 2, 2)),
+])
+def test_packed_route_for_few_input_channels(B, H, W, Cin, Cout, KH, KW, stride, pad):
+    """At most four input channels: the packed 4-channel gather gives the accumulators and codes of
+    the oracle (and so of the im2col route it replaces)."""
+    from lucid_amd import _ops
+    rng = np.random.default_rng(B + H + Cout)
+    x = rng.integers(-128, 128, (B, H, W, Cin)).astype(np.int8)
+    w = rng.integers(-127, 128, (Cout, KH, KW, Cin)).astype(np.int8)
+    ws = (rng.random(Cout).astype(np.float32) + 0.5) * 1e-3
+    bias = rng.standard_normal(Cout).astype(np.float32) * 0.1
+    hip = lambda a: L.tensor(a, device="hip")
+    dx, dw = hip(x), hip(w)
+    acc = _ops.qconv2d_i8(dx, dw, a_zp=0, stride=stride, pad=pad, out_mode=_ops.OUT_ACC_I32, path=_ops.CONV_PACKED4)
+    assert np.array_equal(acc.numpy(), O.qconv2d(x, w, 0, 1.0, np.ones(Cout, np.float32), stride=stride, pad=pad,
+                                                 out_mode=O.OUT_ACC_I32))
+    kw = dict(a_zp=-7, a_scale=hip(np.float32(0.02)), w_scale=hip(ws), wsum=_ops.rowsum_i8(dw), bias=hip(bias),
+              stride=stride, pad=pad, relu=True, out_mode=_ops.OUT_REQUANT_I8, out_scale=hip(np.float32(0.05)),
+              out_zp=hip(np.float32(0.0)), out_qmin=0, out_qmax=255, out_offset=-128)
+    auto = _ops.qconv2d_i8(dx, dw, **kw)                       # chooses the packed route
+    want = O.qconv2d(x, w, -7, 0.02, ws, stride=stride, pad=pad, bias=bias, relu=True, out_mode=O.OUT_REQUANT_I8,
+                     out_scale=0.05, out_zp=0.0, out_qmin=0, out_qmax=255, out_offset=-128)
+    assert np.array_equal(auto.numpy(), want)
+    assert np.array_equal(_ops.qconv2d_i8(dx, dw, **kw, path=_ops.CONV_IM2COL).numpy(), want)

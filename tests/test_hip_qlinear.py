@@ -246,3 +246,26 @@ def test_residual_needs_a_float_output():
     a, w = hip(np.zeros((4, 16), np.int8)), hip(np.zeros((4, 16), np.int8))
     with pytest.raises(ValueError):
         _ops.qlinear_i8(a, w, out_mode=_ops.OUT_ACC_I32, residual=hip(np.zeros((4, 4), np.float32)))
+
+
+@pytest.mark.parametrize("M,N,K,path", [(256, 512, 128, 1), (130, 72, 96, 1), (8, 64, 256, 2), (5, 33, 40, 3)])
+def test_fused_join_on_codes(M, N, K, path):
+    """qlinear with a join == qlinear to codes, then lq_add_requant_i8 (tile, skinny, naive)."""
+    from lucid_amd import _C, _ops
+    rng = np.random.default_rng(M + N + K)
+    hip = lambda a: L.tensor(a, device="hip")
+    a, w = hip(rng.integers(-128, 128, (M, K)).astype(np.int8)), hip(rng.integers(-127, 128, (N, K)).astype(np.int8))
+    common = dict(a_zp=5, a_scale=hip(np.float32(0.02)), w_scale=hip((rng.random(N).astype(np.float32) + 0.5) * 1e-3),
+                  wsum=_ops.rowsum_i8(w), bias=hip(rng.standard_normal(N).astype(np.float32) * 0.1),
+                  out_mode=_ops.OUT_REQUANT_I8, out_scale=hip(np.float32(0.03)), out_zp=hip(np.float32(-3.0)),
+                  out_qmin=-128, out_qmax=127, out_offset=0, path=path)
+    first = _ops.qlinear_i8(a, w, **common)
+    other = hip(rng.integers(-128, 128, (M, N)).astype(np.int8))
+    s2, z2, S, Z = (hip(np.float32(v)) for v in (0.025, 131.0, 0.04, 7.0))
+    want = L.Tensor.empty((M, N), L.int8, "hip")
+    _C.call("lq_add_requant_i8", first.data_ptr, 0, common["out_scale"].data_ptr, common["out_zp"].data_ptr,
+            other.data_ptr, -128, s2.data_ptr, z2.data_ptr, M * N, 1, S.data_ptr, Z.data_ptr, 0, 255, -128,
+            want.data_ptr, None)
+    fused = _ops.qlinear_i8(a, w, **common, join=dict(q=other, offset=-128, scale=s2, zp=z2, relu=True, out_scale=S,
+                                                       out_zp=Z, out_qmin=0, out_qmax=255, out_offset=-128))
+    assert np.array_equal(fused.numpy(), want.numpy())

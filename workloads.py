@@ -112,10 +112,14 @@ class QBottleneck(nn.Module):
                                   calib) if has_down else None)
         self.skip_add = _qfunctional(f"{prefix}.add", calib)
 
+    fuse_join = True  # conv3 applies skip_add.add_relu in its epilogue (same bits, one kernel less)
+
     def forward(self, x):
         identity = x if self.downsample is None else self.downsample(x)
-        out = self.conv3(self.conv2(self.conv1(x)))
-        return self.skip_add.add_relu(out, identity)
+        h = self.conv2(self.conv1(x))
+        if self.fuse_join:
+            return self.conv3(h, join=(identity, self.skip_add, True))
+        return self.skip_add.add_relu(self.conv3(h), identity)
 
 
 class QResNet50(nn.Module):
