@@ -280,6 +280,67 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_i8_kernel(const int8_t* __re
     }
 }
 
+// The same, sixteen channels per lane (C % 16 == 0, 16-byte aligned tensors): a lane
+// keeps a running per-byte maximum of 16-byte loads.
+__device__ __forceinline__ uint32_t max_i8x4(uint32_t a, uint32_t b) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int x = int(int8_t((a >> (8 * e)) & 0xff)), y = int(int8_t((b >> (8 * e)) & 0xff));
+        r |= uint32_t(uint8_t(x > y ? x : y)) << (8 * e);
+    }
+    return r;
+}
+
+__global__ __launch_bounds__(256) void maxpool_nhwc_i8x16_kernel(const uint4* __restrict__ x, uint4* __restrict__ out,
+                                                                 int B, int H, int W, int C16, int KH, int KW,
+                                                                 int sh, int sw, int ph, int pw, int OH, int OW) {
+    const size_t total = size_t(B) * OH * OW * C16;
+    for (size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += size_t(gridDim.x) * 256) {
+        const int c = int(idx % C16);
+        size_t p = idx / C16;
+        const int ow = int(p % OW);
+        p /= OW;
+        const int oh = int(p % OH), b = int(p / OH);
+        uint4 best = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};  // -128 in every byte
+        for (int kh = 0; kh < KH; ++kh) {
+            const int ih = oh * sh - ph + kh;
+            if (ih < 0 || ih >= H) continue;
+            for (int kw = 0; kw < KW; ++kw) {
+                const int iw = ow * sw - pw + kw;
+                if (iw < 0 || iw >= W) continue;
+                const uint4 v = x[((size_t(b) * H + ih) * W + iw) * C16 + c];
+                best.x = max_i8x4(best.x, v.x);
+                best.y = max_i8x4(best.y, v.y);
+                best.z = max_i8x4(best.z, v.z);
+                best.w = max_i8x4(best.w, v.w);
+            }
+        }
+        out[idx] = best;
+    }
+}
+
+// float32 NCHW -> int8 NHWC for at most four channels (an RGB image): one pixel per
+// lane, plane reads and pixel writes both contiguous across a wavefront.
+__global__ __launch_bounds__(256) void quantize_nchw_to_nhwc_small_c_kernel(
+    const float* __restrict__ x, int8_t* __restrict__ q, int C, size_t HW, const float* scale, const float* zp,
+    float lo, float hi, int off) {
+    const float s = scale[0], z = zp[0];
+    const size_t b = blockIdx.y;
+    for (size_t p = size_t(blockIdx.x) * 256 + threadIdx.x; p < HW; p += size_t(gridDim.x) * 256) {
+        int8_t v[4];
+        for (int c = 0; c < C; ++c) {
+            const float u = q_core_local(x[(b * C + c) * HW + p], s, z, lo, hi);
+            v[c] = int8_t(((u != u) ? 0 : int(u)) + off);
+        }
+        int8_t* dst = q + (b * HW + p) * C;
+        if (C == 4)
+            *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(v);
+        else
+            for (int c = 0; c < C; ++c) dst[c] = v[c];
+    }
+}
+
 inline unsigned grid_1d(size_t n, unsigned per_block = 256) {
     size_t b = (n + per_block - 1) / per_block;
     if (b < 1) b = 1;
@@ -456,6 +517,13 @@ int lq_quantize_nchw_to_nhwc(const float* x, int8_t* q, int code_offset, int B, 
                code_offset);
     LQ_REQUIRE(B <= 65535 && (C + 31) / 32 <= 65535, LQ_ERR_SHAPE, "quantize_nchw_to_nhwc: too large");
     const int HW = H * W;
+    if (C <= 4) {
+        const unsigned gx = unsigned((HW + 255) / 256 < 1024 ? (HW + 255) / 256 : 1024);
+        hipLaunchKernelGGL(quantize_nchw_to_nhwc_small_c_kernel, dim3(gx, B), dim3(256), 0, as_stream(stream), x, q, C,
+                           size_t(HW), scale, zp, float(qmin), float(qmax), code_offset);
+        LQ_CHECK_LAUNCH("quantize_nchw_to_nhwc");
+        return LQ_OK;
+    }
     hipLaunchKernelGGL(quantize_nchw_to_nhwc_kernel, dim3((HW + 31) / 32, (C + 31) / 32, B), dim3(256), 0,
                        as_stream(stream), x, q, B, C, HW, scale, zp, float(qmin), float(qmax),
                        code_offset);
@@ -521,6 +589,13 @@ int lq_maxpool2d_nhwc_i8(const int8_t* x, int8_t* out, int B, int H, int W, int 
     const size_t total = size_t(B) * OH * OW * C;
     if (total == 0) return LQ_OK;
     LQ_REQUIRE(x && out, LQ_ERR_VALUE, "maxpool2d_nhwc_i8: NULL pointer");
+    if (C % 16 == 0 && aligned16(x) && aligned16(out)) {
+        hipLaunchKernelGGL(maxpool_nhwc_i8x16_kernel, dim3(grid_1d(total / 16)), dim3(256), 0, as_stream(stream),
+                           reinterpret_cast<const uint4*>(x), reinterpret_cast<uint4*>(out), B, H, W, C / 16, KH, KW,
+                           stride_h, stride_w, pad_h, pad_w, OH, OW);
+        LQ_CHECK_LAUNCH("maxpool2d_nhwc_i8");
+        return LQ_OK;
+    }
     hipLaunchKernelGGL(maxpool_nhwc_i8_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream), x,
                        out, B, H, W, C, KH, KW, stride_h, stride_w, pad_h, pad_w, OH, OW);
     LQ_CHECK_LAUNCH("maxpool2d_nhwc_i8");
