@@ -719,6 +719,13 @@ int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st
     long workers = slots_g;
     if (workers < 1) workers = 1;
     if (workers > long(sk_tiles) * nk) workers = long(sk_tiles) * nk;
+    if (schedule == 2 && long(tiles) * 2 <= workers) {
+        // fewer tiles than block slots: a whole number of workers per tile, so that no
+        // worker's range straddles two tiles (plain split-K, each piece >= 4 iterations)
+        long split = workers / tiles;
+        if (split > nk / 4) split = nk / 4;
+        workers = long(tiles) * (split < 1 ? 1 : split);
+    }
     SkScratch* s = nullptr;
     const size_t slab_words = size_t(Cfg::TM) * Cfg::TN * 16 * Cfg::THREADS;
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
