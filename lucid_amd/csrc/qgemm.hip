@@ -68,6 +68,7 @@ int launch_tile_c4(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c5(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c6(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c7(const GemmArgs&, bool, int, int, hipStream_t);
+int launch_tile_c8(const GemmArgs&, bool, int, int, hipStream_t);
 }  // namespace lq
 
 namespace {
@@ -81,6 +82,7 @@ int launch_tile_shape(const GemmArgs& g, bool conv, int groups, int cfg, int sch
     case 5: return launch_tile_c5(g, conv, groups, schedule, st);
     case 6: return launch_tile_c6(g, conv, groups, schedule, st);
     case 7: return launch_tile_c7(g, conv, groups, schedule, st);
+    case 8: return launch_tile_c8(g, conv, groups, schedule, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -150,11 +152,16 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     const double ops = 2.0 * g.M * double(g.N) * g.K * groups;
     if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9) return LQ_OK;
 
-    int cands[6], n = 0;
+    // candidates are whole tile_config values (shape | schedule << 8)
+    int cands[8], n = 0;
     if (g.N <= 64) cands[n++] = 6;
     cands[n++] = 5;
+    if (g.K <= 256) cands[n++] = 8;  // one to four k-iterations: latency-bound tiles, four blocks per CU
     if (g.N > 64) cands[n++] = 3, cands[n++] = 4;
     if (g.N > 128 && g.M > 128) cands[n++] = 1;
+    // a long K over few tiles (late convolution stages): split K between the idle CUs
+    const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
+    if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
     hipEvent_t e0, e1;
     LQ_HIP(hipEventCreate(&e0));
     LQ_HIP(hipEventCreate(&e1));
@@ -162,10 +169,11 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     int rc = LQ_OK;
     bool timed = true;
     for (int i = 0; i < n && rc == LQ_OK && timed; ++i) {
-        rc = launch_tile_shape(g, conv, groups, cands[i], 1, st);  // warm: code load, attributes
+        const int shape = cands[i] & 0xff, sched = (cands[i] >> 8) ? (cands[i] >> 8) : 1;
+        rc = launch_tile_shape(g, conv, groups, shape, sched, st);  // warm: code load, attributes
         if (rc) break;
         timed = hipEventRecord(e0, st) == hipSuccess;
-        for (int r = 0; r < 3 && rc == LQ_OK; ++r) rc = launch_tile_shape(g, conv, groups, cands[i], 1, st);
+        for (int r = 0; r < 3 && rc == LQ_OK; ++r) rc = launch_tile_shape(g, conv, groups, shape, sched, st);
         float ms = 0.0f;
         timed = timed && rc == LQ_OK && hipEventRecord(e1, st) == hipSuccess &&
                 hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
@@ -183,15 +191,18 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     return LQ_OK;
 }
 
-// tile_config: low byte = tile shape (0 = choose, 1..7 = a specific one), next
+// tile_config: low byte = tile shape (0 = choose, 1..8 = a specific one), next
 // byte = schedule (0 = choose, 1 = block per tile, 2 = stream-K, 3 = stream-K over
 // the leftover tiles only).
 int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st) {
     int cfg = tile_config & 0xff;
-    const int schedule = (tile_config >> 8) & 0xff;
+    int schedule = (tile_config >> 8) & 0xff;
     if (cfg == 0) {
-        int rc = tuned_tile_shape(g, conv, groups, st, &cfg);
+        int tuned = 0;
+        int rc = tuned_tile_shape(g, conv, groups, st, &tuned);
         if (rc) return rc;
+        cfg = tuned & 0xff;
+        if (schedule == 0) schedule = (tuned >> 8) & 0xff;
     }
     return launch_tile_shape(g, conv, groups, cfg, schedule, st);
 }

@@ -661,6 +661,7 @@ using CfgTall = TileCfg<128, 256, 64, 2, 2, 3, 2>;
 using CfgMid = TileCfg<128, 128, 64, 2, 2, 4, 2>;
 using CfgN64 = TileCfg<256, 64, 64, 4, 1, 3, 2>;  // 64 output columns (early ResNet stages)
 using CfgTall3 = TileCfg<128, 256, 64, 2, 2, 2, 3>;  // three blocks per CU
+using CfgMid4 = TileCfg<128, 128, 64, 2, 2, 2, 4>;   // four blocks per CU: short K, latency-bound tiles
 
 }  // namespace
 

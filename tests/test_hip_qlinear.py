@@ -42,7 +42,7 @@ def test_accumulators_exact(M, N, K, path):
     assert np.array_equal(acc, O.igemm(a, w))
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 260, 144), (129, 77, 784), (513, 1000, 576),
                                    (2048, 512, 4096), (1, 16, 16), (700, 130, 64)])
 def test_every_tile_shape_exact(cfg, M, N, K):
@@ -60,7 +60,7 @@ def test_every_tile_shape_exact(cfg, M, N, K):
     assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
 
 
-@pytest.mark.parametrize("cfg", [1, 3, 4, 5, 6])
+@pytest.mark.parametrize("cfg", [1, 3, 4, 5, 6, 8])
 @pytest.mark.parametrize("M,N,K", [(300, 260, 144), (513, 1000, 576), (2048, 1100, 4096),
                                    (256, 256, 128), (129, 77, 784), (1500, 3000, 1024)])
 def test_stream_k_schedule_exact(cfg, M, N, K):
@@ -269,3 +269,17 @@ def test_fused_join_on_codes(M, N, K, path):
     fused = _ops.qlinear_i8(a, w, **common, join=dict(q=other, offset=-128, scale=s2, zp=z2, relu=True, out_scale=S,
                                                        out_zp=Z, out_qmin=0, out_qmax=255, out_offset=-128))
     assert np.array_equal(fused.numpy(), want.numpy())
+
+
+def test_split_k_over_few_tiles_exact():
+    """Fewer tiles than block slots and a long K (a late convolution stage as a GEMM): the
+    stream-K schedule gives every tile a whole number of workers; exact, like every schedule."""
+    M, N, K = 1568, 512, 4608
+    rng = np.random.default_rng(99)
+    a = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    w = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    hip = lambda t: L.tensor(t, device="hip")
+    acc = _ops.qlinear_i8(hip(a), hip(w), out_mode=_ops.OUT_ACC_I32, path=1, tile_config=5 | 0x200).numpy()
+    assert np.array_equal(acc, O.igemm(a, w))
+    # and through the automatic choice (which may pick that schedule for this shape)
+    assert np.array_equal(_ops.qlinear_i8(hip(a), hip(w), out_mode=_ops.OUT_ACC_I32, path=1).numpy(), acc)
