@@ -390,7 +390,7 @@ int lq_rowsum_i8(const int8_t* w, int32_t* out, int N, int K, lq_stream stream);
  * fake_quantize, by its exact integer identity:
  *     acc[m,n] = sum_k a[m,k] * w[n,k]                              (int32)
  *     y = f32(acc - a_zp*wsum[n]) * (a_scale[m|0] * w_scale[n]) + bias[n]
- *     y = relu(y) if relu
+ *     y = relu(y) if relu,  y = gelu(y) if gelu
  *     y = y + residual[m,n] if residual
  *     out = per out_mode
  * a: int8 [M,K] activation codes as stored (a quint8 code c is stored as
@@ -450,6 +450,14 @@ typedef struct {
                               vit/_model.py:276-277); modes F32 / F16 only        */
     long ldr;              /* residual row stride in elements; 0 means N     */
     lq_join_args join;     /* optional join on codes; mode REQUANT_I8 only   */
+    int gelu;              /* mode F32: exact-erf GELU
+                              (lucid/nn/functional/activations.py:219) applied to
+                              y after the bias / ReLU and before a residual - the
+                              fc1 -> GELU of a transformer MLP in one kernel   */
+    float* range;          /* optional range buffer (lq_range_buffer_bytes()) that
+                              receives the min / max of the stored output, for
+                              lq_calc_qparams_from_range of the next dynamic
+                              quantizer; mode F32, tile kernel only             */
 } lq_qlinear_args;
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);

@@ -131,7 +131,7 @@ class QLinearArgs(C.Structure):
         ("out_scale", _vp), ("out_zp", _vp),
         ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
         ("out", _vp), ("ldo", C.c_long), ("force_path", _i), ("tile_config", _i),
-        ("residual", _vp), ("ldr", C.c_long), ("join", JoinArgs),
+        ("residual", _vp), ("ldr", C.c_long), ("join", JoinArgs), ("gelu", _i), ("range", _vp),
     ]
 
 

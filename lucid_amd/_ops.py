@@ -44,7 +44,8 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
                out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
                out_qmax: int = 255, out_offset: int = 0, path: int = PATH_AUTO,
                tile_config: int = 0, out: Tensor | None = None, repeat: int = 1,
-               residual: Tensor | None = None, join=None) -> Tensor:
+               residual: Tensor | None = None, join=None, gelu: bool = False,
+               range_buf: Tensor | None = None) -> Tensor:
     """Fused int8 GEMM + epilogue; see ``lq_qlinear_i8`` in ``lucid_hip.h``.
     ``a`` is int8 ``[M, K]``, ``w`` int8 ``[N, K]``; the result is ``[M, N]``.
     ``residual`` (float32, ``M*N`` elements) is added after the activation;
@@ -82,6 +83,7 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
         raise _C.ShapeMismatch(f"residual has {residual.numel} elements for an output of {M}x{N}")
     args.residual, args.ldr = _ptr(residual, "residual", T.float32), 0
     _fill_join(args.join, join, (M, N))
+    args.gelu, args.range = int(gelu), _ptr(range_buf, "range", T.float32)
     if repeat == 1:
         _C.call("lq_qlinear_i8", C.byref(args), None)
     else:

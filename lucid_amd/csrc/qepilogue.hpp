@@ -96,6 +96,12 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
     const float floor = g.relu ? 0.0f : -__builtin_inff();
     y = (y < floor) ? floor : y;
     if (MODE == OUT_F32 || MODE == OUT_F16) return __float_as_uint(y);
+    if (MODE == OUT_F32X) {
+        // GELU, erf form (lucid/nn/functional/activations.py:219): the expression of the
+        // stand-alone kernel, so fusing it changes no bit
+        if (g.gelu) y = (0.5f * y) * (1.0f + erff(y * 0.70710678118654752440f));
+        return __float_as_uint(y);
+    }
     float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
     if (MODE == OUT_REQUANT_I8) {
         int code = (qv != qv) ? 0 : int(qv);
@@ -108,7 +114,7 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
 // joins of a transformer block); the other forms ignore the operand.
 template <int MODE>
 __device__ __forceinline__ uint32_t add_residual(const GemmArgs& g, uint32_t bits, int m, int n) {
-    if ((MODE == OUT_F32 || MODE == OUT_F16) && g.residual)
+    if ((MODE == OUT_F32 || MODE == OUT_F16 || MODE == OUT_F32X) && g.residual)
         return __float_as_uint(__uint_as_float(bits) + g.residual[size_t(m) * size_t(g.ldr) + size_t(n)]);
     return bits;
 }
@@ -188,7 +194,12 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, 
                                                float as, const ColParams& c, float S, float Z) {
     switch (g.out_mode) {
     case OUT_ACC_I32: epilogue_store_t<OUT_ACC_I32>(g, m, n, acc, as, c, S, Z); break;
-    case OUT_F32: epilogue_store_t<OUT_F32>(g, m, n, acc, as, c, S, Z); break;
+    case OUT_F32:
+        if (g.gelu)
+            epilogue_store_t<OUT_F32X>(g, m, n, acc, as, c, S, Z);
+        else
+            epilogue_store_t<OUT_F32>(g, m, n, acc, as, c, S, Z);
+        break;
     case OUT_F16: epilogue_store_t<OUT_F16>(g, m, n, acc, as, c, S, Z); break;
     case OUT_REQUANT_I8: epilogue_store_t<OUT_REQUANT_I8>(g, m, n, acc, as, c, S, Z); break;
     default: epilogue_store_t<OUT_FAKEQUANT_F32>(g, m, n, acc, as, c, S, Z); break;

@@ -135,7 +135,8 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
                              g.cdh * 16 + g.cdw, g.cOW};
         std::memcpy(key.geom, geom, sizeof(geom));
     }
-    key.flags = (g.residual ? 1 : 0) | (g.a_scale_per_row ? 2 : 0) | (g.bias ? 4 : 0) | (g.join_q ? 8 : 0);
+    key.flags = (g.residual ? 1 : 0) | (g.a_scale_per_row ? 2 : 0) | (g.bias ? 4 : 0) | (g.join_q ? 8 : 0) |
+                (g.gelu ? 16 : 0) | (g.range ? 32 : 0);
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);
         auto it = g_tune.find(key);
@@ -377,7 +378,10 @@ int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t 
     GemmArgs g = g_in;
     const bool vec_ok = g.K % 16 == 0 && g.K > 0 && aligned16(g.a) && aligned16(g.w);
     int path = force_path;  // 0 = choose, 1 = tile, 2 = skinny, 3 = naive
-    if (path == 0) path = !vec_ok ? 3 : (g.M <= 64 ? 2 : 1);
+    if (path == 0) path = !vec_ok ? 3 : (g.M <= 64 && g.range == nullptr ? 2 : 1);
+    // only the tile kernel keeps the range of what it writes
+    LQ_REQUIRE(g.range == nullptr || path == 1, LQ_ERR_NOT_IMPLEMENTED,
+               "qlinear_i8: a kept range needs the tile kernel (K %% 16 == 0, aligned operands)");
     LQ_REQUIRE(path == 3 || vec_ok, LQ_ERR_VALUE,
                "qlinear_i8: MFMA paths need K %% 16 == 0 and 16-byte aligned operands");
     if (path == 1) {
@@ -474,6 +478,11 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
     g.cx = nullptr; g.pad_src = nullptr;
     const int jrc = set_join(g, p->join, p->out_mode, p->N, "qlinear_i8");
     if (jrc) return jrc;
+    LQ_REQUIRE(p->gelu == 0 || p->out_mode == OUT_F32, LQ_ERR_VALUE, "qlinear_i8: GELU needs out_mode F32");
+    LQ_REQUIRE(p->range == nullptr || p->out_mode == OUT_F32, LQ_ERR_VALUE,
+               "qlinear_i8: a kept range needs out_mode F32");
+    g.gelu = p->gelu != 0;
+    g.range = p->range;
 
     return run_gemm(g, p->force_path, p->tile_config, as_stream(stream));
 }

@@ -5,6 +5,9 @@
 namespace lq {
 
 enum { OUT_ACC_I32 = 0, OUT_F32 = 1, OUT_F16 = 2, OUT_REQUANT_I8 = 3, OUT_FAKEQUANT_F32 = 4 };
+// Internal variant of OUT_F32 (never an ABI value): float32 output with a GELU and / or a
+// kept range.  A template mode of its own, so that the plain float epilogue carries neither.
+constexpr int OUT_F32X = 5;
 
 struct GemmArgs {
     const int8_t* a;      // [M,K] activation codes as stored
@@ -27,6 +30,9 @@ struct GemmArgs {
     long ldo;
     const float* residual;  // optional [M, ldr] float32 added to y after the activation (float outputs only)
     long ldr;
+    int gelu;             // OUT_F32: exact-erf GELU after the bias / ReLU (before a residual)
+    float* range;         // OUT_F32, one block per tile: min / max of the stored tile go to the block's slot
+                          // (either one selects the OUT_F32X instance of the kernels)
     // Optional join on codes after the requantize (OUT_REQUANT_I8 only): the layer's code
     // and join_q[m, n] are dequantized with their own grids, added, optionally clamped at
     // zero, and requantized to (join_out_*): QFunctional.add / add_relu fused in.

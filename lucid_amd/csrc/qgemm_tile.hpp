@@ -5,6 +5,7 @@
 #include "common.hpp"
 #include "qgemm.hpp"
 #include "qepilogue.hpp"
+#include "range_slots.hpp"
 
 #include <type_traits>
 
@@ -94,7 +95,8 @@ template <class Cfg, int MODE>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg::TM][Cfg::TN],
                                               const ColParams (&cp)[Cfg::TN], const float* s_as,
                                               uint32_t* stage, int m0, int n0, int n_limit, int wm,
-                                              int wn, int lane, float S, float Z, bool interior) {
+                                              int wn, int lane, float S, float Z, bool interior,
+                                              float& r_lo, float& r_hi, int& r_nan) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, STRIDE = Cfg::STAGE_STRIDE;
     constexpr int QUADS_PER_ROW = TN * 8;            // four-column groups per staged row
     constexpr int EPI_ROWS = Cfg::EPI_ROWS;          // rows staged at a time (32 or 16)
@@ -105,6 +107,14 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
     const int esize = MODE == OUT_F16 ? 2 : (MODE == OUT_REQUANT_I8 ? 1 : 4);
     const bool vec_ok = (g.ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0);
     const int row0 = lane / QUADS_PER_ROW, cq = (lane % QUADS_PER_ROW) * 4;
+    // running range of what this lane stores (float32 output with a kept range only)
+    const bool keep = MODE == OUT_F32X && g.range != nullptr;
+    auto track = [&](uint32_t bits) {
+        const float y = __uint_as_float(bits);
+        r_nan |= (y != y);
+        r_lo = fminf(r_lo, y);
+        r_hi = fmaxf(r_hi, y);
+    };
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -113,7 +123,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
             const int m_first = m0 + band + row0, n = n0 + wn * (TN * 32) + cq;
             // residual rows of this part, requested before the arithmetic so that
             // their latency is paid under it (`interior` vouches for alignment)
-            constexpr bool kFloatOut = MODE == OUT_F32 || MODE == OUT_F16;
+            constexpr bool kFloatOut = MODE == OUT_F32 || MODE == OUT_F16 || MODE == OUT_F32X;
             const bool res_fast = kFloatOut && interior && g.residual != nullptr;
             float4 rv[kFloatOut ? PASSES : 1];
             if (kFloatOut && res_fast) {
@@ -175,6 +185,10 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                         v[p].w = join_code(g, jp, v[p].w, int(int8_t(jv[p] >> 24)));
                     }
                 }
+                if (MODE == OUT_F32X && keep) {
+#pragma unroll
+                    for (int p = 0; p < PASSES; ++p) track(v[p].x), track(v[p].y), track(v[p].z), track(v[p].w);
+                }
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
                     store_vec4<MODE>(g, idx, v[p]);
@@ -190,6 +204,12 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                         if (n + 1 < n_limit) v.y = finish_value<MODE>(g, v.y, m, n + 1, S, Z);
                         if (n + 2 < n_limit) v.z = finish_value<MODE>(g, v.z, m, n + 2, S, Z);
                         if (n + 3 < n_limit) v.w = finish_value<MODE>(g, v.w, m, n + 3, S, Z);
+                        if (MODE == OUT_F32X && keep) {
+                            track(v.x);
+                            if (n + 1 < n_limit) track(v.y);
+                            if (n + 2 < n_limit) track(v.z);
+                            if (n + 3 < n_limit) track(v.w);
+                        }
                         const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
                         if (vec_ok && n + 4 <= n_limit) {
                             store_vec4<MODE>(g, idx, v);
@@ -502,8 +522,13 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
                               (g.join_q == nullptr ||
                                (g.join_ld % 4 == 0 && reinterpret_cast<uintptr_t>(g.join_q) % 4 == 0));
         __syncthreads();
-        tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z, interior);
+        float r_lo = __builtin_inff(), r_hi = -__builtin_inff();
+        int r_nan = 0;
+        tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z, interior, r_lo,
+                                 r_hi, r_nan);
         __syncthreads();  // the staging area is the next tile's first LDS stage
+        // one block per tile here (the launcher sees to it), so the block's slot is the tile's
+        if (MODE == OUT_F32X && !SK && g.range != nullptr) range_block_store(g.range, r_lo, r_hi, r_nan);
     };
 
     if (!SK) {
@@ -704,6 +729,11 @@ int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st
     // therefore always one block per tile.
     int sk_tiles = 0;
     const int slots_g = slots / groups;
+    if (g.range != nullptr) {
+        LQ_REQUIRE(long(tiles) * groups <= kRangeSlots, LQ_ERR_SHAPE,
+                   "tile kernel: %ld tiles are too many for a kept range", long(tiles) * groups);
+        schedule = 1;
+    }
     if (schedule == 2) {
         sk_tiles = tiles;
     } else if (schedule == 3) {
@@ -751,7 +781,12 @@ int launch_tile(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
                "tile kernel: K too large");
     switch (g.out_mode) {
     case OUT_ACC_I32: return launch_tile_mode<Cfg, OUT_ACC_I32, CONV>(g, groups, schedule, st);
-    case OUT_F32: return launch_tile_mode<Cfg, OUT_F32, CONV>(g, groups, schedule, st);
+    case OUT_F32:
+        if (g.gelu || g.range != nullptr) {
+            if (CONV) return fail(LQ_ERR_NOT_IMPLEMENTED, "tile kernel: GELU / kept range are not built for convolutions");
+            return launch_tile_mode<Cfg, OUT_F32X, false>(g, groups, schedule, st);
+        }
+        return launch_tile_mode<Cfg, OUT_F32, CONV>(g, groups, schedule, st);
     case OUT_F16: return launch_tile_mode<Cfg, OUT_F16, CONV>(g, groups, schedule, st);
     case OUT_REQUANT_I8: return launch_tile_mode<Cfg, OUT_REQUANT_I8, CONV>(g, groups, schedule, st);
     default: return launch_tile_mode<Cfg, OUT_FAKEQUANT_F32, CONV>(g, groups, schedule, st);

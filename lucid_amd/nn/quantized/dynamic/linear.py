@@ -45,9 +45,14 @@ class Linear(Module):
         if name == "weight_zero_point":
             require_symmetric_weight(self.weight_zero_point, "dynamic.Linear")
 
-    def forward(self, x: Tensor, residual: Tensor | None = None) -> Tensor:
-        """``residual`` (optional, not in Lucid's signature) is added to the
-        output inside the GEMM epilogue: ``x_res + linear(x)`` in one kernel."""
+    def forward(self, x: Tensor, residual: Tensor | None = None, activation: str | None = None,
+                track_range: bool = False) -> Tensor:
+        """Beyond Lucid's signature, all inside the GEMM epilogue: ``residual`` is added to
+        the output (``x_res + linear(x)`` in one kernel); ``activation="gelu"`` applies the
+        exact-erf GELU to it (``gelu(linear(x))``); ``track_range`` keeps the min / max of
+        what is written, for the next dynamic-quantized layer."""
+        if activation not in (None, "gelu"):
+            raise ValueError(f"dynamic.Linear: unknown fused activation {activation!r}")
         if not isinstance(x, Tensor) or x.device != "hip":
             raise _C.DeviceMismatch("dynamic.Linear: input must be a tensor on the 'hip' device")
         if x.dtype != T.float32:
@@ -72,10 +77,17 @@ class Linear(Module):
                 x_scale.data_ptr, x_zp.data_ptr, 0, qd.quant_min, qd.quant_max, None)
         if self._wsum is None:
             self._wsum = _ops.rowsum_i8(self.weight_int8)
+        rng = None
+        if track_range:
+            from ...functional import _new_range
+            rng = _new_range()
         y = _ops.qlinear_i8(xq, self.weight_int8, a_zp=off, a_zp_dev=x_zp, a_scale=x_scale,
                             w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias,
-                            out_mode=_ops.OUT_F32, residual=residual)
-        return y.reshape(*x.shape[:-1], N)
+                            out_mode=_ops.OUT_F32, residual=residual, gelu=activation == "gelu",
+                            range_buf=rng)
+        y = y.reshape(*x.shape[:-1], N)
+        y._range = rng
+        return y
 
     @classmethod
     def from_float(cls, mod, dtype: QDtype = qint8) -> "Linear":

@@ -11,6 +11,7 @@ import pytest
 
 import lucid_amd as L
 import lucid_amd.nn.functional as F
+import oracle as O
 import oracle.vit as V
 import workloads
 from lucid_amd import _C
@@ -192,3 +193,38 @@ def test_kept_range_of_attention_and_nan_propagation():
     x[17, 5] = np.nan
     kmn, kmx, ks, _ = _range_of(F.gelu(hip(x), track_range=True))
     assert np.isnan(kmn) and np.isnan(kmx) and np.isnan(ks)  # Reduce.cpp:87-125 propagates NaN
+
+
+@pytest.mark.parametrize("M,K,N", [(12608 // 8, 768, 3072), (300, 96, 200), (129, 64, 72)])
+def test_gelu_and_kept_range_in_the_gemm_epilogue(M, K, N):
+    """fc1 -> GELU fused: the bits of linear followed by the stand-alone GELU kernel, and the
+    kept range gives the qparams that min / max of the result give."""
+    import lucid_amd.nn as nn
+    import lucid_amd.nn.functional as F
+    import lucid_amd.quantization as Q
+    from lucid_amd import _C
+    rng = np.random.default_rng(M + N)
+    lin = nn.Linear(K, N)
+    q = Q.quantize_dynamic(nn.Sequential(lin))[0]
+    x = L.tensor(rng.standard_normal((M, K)).astype(np.float32), device="hip")
+    want = F.gelu(q(x)).numpy()
+    fused = q(x, activation="gelu", track_range=True)
+    got = fused.numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    s = L.Tensor.empty((), L.float32, "hip")
+    z = L.Tensor.empty((), L.float32, "hip")
+    _C.call("lq_calc_qparams_from_range", fused._range.data_ptr, 0, 0, 255, 0, 1e-8, s.data_ptr, z.data_ptr,
+            None, None, None)
+    ws, wz = O.calc_qparams(np.float32([want.min()]), np.float32([want.max()]), False, 0, 255, False)
+    assert s.numpy() == ws[0] and z.numpy() == wz[0]
+
+
+def test_vit_block_fused_and_unfused_gelu_agree(monkeypatch):
+    import workloads as W
+    cfg = dict(W.VIT_B16, depth=1, dim=192, heads=3, mlp=768)
+    model = W.QViT(cfg, seed=3)
+    x = L.tensor(np.random.default_rng(0).standard_normal((2, 3, 224, 224)).astype(np.float32), device="hip")
+    a = model(x).numpy()
+    monkeypatch.setattr(W.ViTBlock, "fuse_gelu", False)
+    b = model(x).numpy()
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))

@@ -234,6 +234,8 @@ def _layer_norm(w, b, eps=1e-6, track_range=True):
 
 
 class ViTBlock(nn.Module):
+    fuse_gelu = True
+
     def __init__(self, prefix, p, heads):
         super().__init__()
         self.heads = heads
@@ -251,7 +253,11 @@ class ViTBlock(nn.Module):
         # what it writes; the residual adds ride in the epilogues of proj and fc2
         a = F.scaled_dot_product_attention_qkv(self.qkv(self.norm1(x)), self.heads, track_range=True)
         x = self.proj(a, residual=x)
-        return self.fc2(F.gelu(self.fc1(self.norm2(x)), track_range=True), residual=x)
+        if self.fuse_gelu:  # GELU and the range of its result in fc1's epilogue (same bits, one kernel less)
+            h = self.fc1(self.norm2(x), activation="gelu", track_range=True)
+        else:
+            h = F.gelu(self.fc1(self.norm2(x)), track_range=True)
+        return self.fc2(h, residual=x)
 
 
 class QViT(nn.Module):
