@@ -103,7 +103,7 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
         return __float_as_uint(y);
     }
     float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
-    if (MODE == OUT_REQUANT_I8) {
+    if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) {
         int code = (qv != qv) ? 0 : int(qv);
         return uint32_t(code + g.out_offset);
     }
@@ -150,7 +150,7 @@ __device__ __forceinline__ uint32_t join_code(const GemmArgs& g, const JoinParam
 // one element's residual step, whichever form the output mode has
 template <int MODE>
 __device__ __forceinline__ uint32_t finish_value(const GemmArgs& g, uint32_t bits, int m, int n, float S, float Z) {
-    if (MODE == OUT_REQUANT_I8 && g.join_q) {
+    if (MODE == OUT_REQUANT_JOIN) {
         const JoinParams jp = load_join(g, S, Z);
         return join_code(g, jp, bits, int(g.join_q[size_t(m) * size_t(g.join_ld) + size_t(n)]));
     }
@@ -161,7 +161,7 @@ template <int MODE>
 __device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint32_t v) {
     if (MODE == OUT_F16)
         static_cast<_Float16*>(g.out)[idx] = _Float16(__uint_as_float(v));
-    else if (MODE == OUT_REQUANT_I8)
+    else if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN)
         static_cast<int8_t*>(g.out)[idx] = int8_t(int(v));
     else
         static_cast<uint32_t*>(g.out)[idx] = v;  // f32 / i32 bit patterns
@@ -175,7 +175,7 @@ __device__ __forceinline__ void store_vec4(const GemmArgs& g, size_t idx, uint4 
         h4 h = {_Float16(__uint_as_float(v.x)), _Float16(__uint_as_float(v.y)),
                 _Float16(__uint_as_float(v.z)), _Float16(__uint_as_float(v.w))};
         *reinterpret_cast<h4*>(static_cast<_Float16*>(g.out) + idx) = h;
-    } else if (MODE == OUT_REQUANT_I8) {
+    } else if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) {
         uint32_t packed = (v.x & 0xffu) | ((v.y & 0xffu) << 8) | ((v.z & 0xffu) << 16) | (v.w << 24);
         *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(g.out) + idx) = packed;
     } else {
@@ -201,7 +201,12 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, 
             epilogue_store_t<OUT_F32>(g, m, n, acc, as, c, S, Z);
         break;
     case OUT_F16: epilogue_store_t<OUT_F16>(g, m, n, acc, as, c, S, Z); break;
-    case OUT_REQUANT_I8: epilogue_store_t<OUT_REQUANT_I8>(g, m, n, acc, as, c, S, Z); break;
+    case OUT_REQUANT_I8:
+        if (g.join_q)
+            epilogue_store_t<OUT_REQUANT_JOIN>(g, m, n, acc, as, c, S, Z);
+        else
+            epilogue_store_t<OUT_REQUANT_I8>(g, m, n, acc, as, c, S, Z);
+        break;
     default: epilogue_store_t<OUT_FAKEQUANT_F32>(g, m, n, acc, as, c, S, Z); break;
     }
 }

@@ -8,6 +8,8 @@ enum { OUT_ACC_I32 = 0, OUT_F32 = 1, OUT_F16 = 2, OUT_REQUANT_I8 = 3, OUT_FAKEQU
 // Internal variant of OUT_F32 (never an ABI value): float32 output with a GELU and / or a
 // kept range.  A template mode of its own, so that the plain float epilogue carries neither.
 constexpr int OUT_F32X = 5;
+// Likewise OUT_REQUANT_I8 followed by the fused join on codes.
+constexpr int OUT_REQUANT_JOIN = 6;
 
 struct GemmArgs {
     const int8_t* a;      // [M,K] activation codes as stored

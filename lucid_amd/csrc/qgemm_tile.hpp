@@ -104,7 +104,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
     constexpr int PASSES = EPI_ROWS * QUADS_PER_ROW / 64;
     constexpr int ROWS_PER_PASS = 64 / QUADS_PER_ROW;
     static_assert(64 % QUADS_PER_ROW == 0 && RPP % 4 == 0, "");
-    const int esize = MODE == OUT_F16 ? 2 : (MODE == OUT_REQUANT_I8 ? 1 : 4);
+    const int esize = MODE == OUT_F16 ? 2 : ((MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) ? 1 : 4);
     const bool vec_ok = (g.ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0);
     const int row0 = lane / QUADS_PER_ROW, cq = (lane % QUADS_PER_ROW) * 4;
     // running range of what this lane stores (float32 output with a kept range only)
@@ -133,9 +133,9 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                     rv[p] = *reinterpret_cast<const float4*>(rp + size_t(p) * ROWS_PER_PASS * size_t(g.ldr));
             }
             // the other operand of a fused join on codes: four codes per row, requested early too
-            const bool join_fast = MODE == OUT_REQUANT_I8 && interior && g.join_q != nullptr;
-            uint32_t jv[MODE == OUT_REQUANT_I8 ? PASSES : 1];
-            if (MODE == OUT_REQUANT_I8 && join_fast) {
+            const bool join_fast = MODE == OUT_REQUANT_JOIN && interior;
+            uint32_t jv[MODE == OUT_REQUANT_JOIN ? PASSES : 1];
+            if (MODE == OUT_REQUANT_JOIN && join_fast) {
                 const int8_t* jq = g.join_q + size_t(m_first) * size_t(g.join_ld) + size_t(n);
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p)
@@ -175,7 +175,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                         v[p].w = __float_as_uint(__uint_as_float(v[p].w) + rv[p].w);
                     }
                 }
-                if (MODE == OUT_REQUANT_I8 && join_fast) {
+                if (MODE == OUT_REQUANT_JOIN && join_fast) {
                     const JoinParams jp = load_join(g, S, Z);
 #pragma unroll
                     for (int p = 0; p < PASSES; ++p) {
@@ -510,11 +510,11 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         if (!fetched) fetch_params(tm, tn);  // a shared tile finished by a worker that did not end it
         if (tid < BM) s_as[tid] = as_mine;
         float S = 1.0f, Z = 0.0f;
-        if (MODE == OUT_REQUANT_I8 || MODE == OUT_FAKEQUANT_F32) {
+        if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN || MODE == OUT_FAKEQUANT_F32) {
             S = g.out_scale[0];
             Z = g.out_zp[0];
         }
-        const int esize = MODE == OUT_F16 ? 2 : (MODE == OUT_REQUANT_I8 ? 1 : 4);
+        const int esize = MODE == OUT_F16 ? 2 : ((MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) ? 1 : 4);
         const bool interior = m0 + BM <= g.M && n0 + BN <= n_limit && g.ldo % 4 == 0 &&
                               reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0 &&
                               (g.residual == nullptr ||
@@ -788,7 +788,9 @@ int launch_tile(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
         }
         return launch_tile_mode<Cfg, OUT_F32, CONV>(g, groups, schedule, st);
     case OUT_F16: return launch_tile_mode<Cfg, OUT_F16, CONV>(g, groups, schedule, st);
-    case OUT_REQUANT_I8: return launch_tile_mode<Cfg, OUT_REQUANT_I8, CONV>(g, groups, schedule, st);
+    case OUT_REQUANT_I8:
+        if (g.join_q != nullptr) return launch_tile_mode<Cfg, OUT_REQUANT_JOIN, CONV>(g, groups, schedule, st);
+        return launch_tile_mode<Cfg, OUT_REQUANT_I8, CONV>(g, groups, schedule, st);
     default: return launch_tile_mode<Cfg, OUT_FAKEQUANT_F32, CONV>(g, groups, schedule, st);
     }
 }
