@@ -69,6 +69,7 @@ int launch_tile_c5(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c6(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c7(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c8(const GemmArgs&, bool, int, int, hipStream_t);
+int launch_tile_c9(const GemmArgs&, bool, int, int, hipStream_t);
 }  // namespace lq
 
 namespace {
@@ -83,6 +84,7 @@ int launch_tile_shape(const GemmArgs& g, bool conv, int groups, int cfg, int sch
     case 6: return launch_tile_c6(g, conv, groups, schedule, st);
     case 7: return launch_tile_c7(g, conv, groups, schedule, st);
     case 8: return launch_tile_c8(g, conv, groups, schedule, st);
+    case 9: return launch_tile_c9(g, conv, groups, schedule, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -154,7 +156,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9) return LQ_OK;
 
     // candidates are whole tile_config values (shape | schedule << 8)
-    int cands[8], n = 0;
+    int cands[10], n = 0;
     if (g.N <= 64) cands[n++] = 6;
     cands[n++] = 5;
     if (g.K <= 256) cands[n++] = 8;  // one to four k-iterations: latency-bound tiles, four blocks per CU
@@ -163,6 +165,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     // a long K over few tiles (late convolution stages): split K between the idle CUs
     const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
     if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
+    if (tiles128 < 256) cands[n++] = 9;  // ... or cover the chip with 64 x 64 tiles
     hipEvent_t e0, e1;
     LQ_HIP(hipEventCreate(&e0));
     LQ_HIP(hipEventCreate(&e1));
@@ -192,7 +195,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     return LQ_OK;
 }
 
-// tile_config: low byte = tile shape (0 = choose, 1..8 = a specific one), next
+// tile_config: low byte = tile shape (0 = choose, 1..9 = a specific one), next
 // byte = schedule (0 = choose, 1 = block per tile, 2 = stream-K, 3 = stream-K over
 // the leftover tiles only).
 int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st) {

@@ -645,7 +645,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
                         __builtin_amdgcn_make_buffer_rsrc(slab_of(w), 0, kSlabBytes, 0x00020000);
                     // eight 16-byte loads in flight per lane (the fragment registers of
                     // the main loop are free here), then their 32 additions
-                    constexpr int kBatch = 8;
+                    constexpr int kBatch = (TM * TN * 4) % 8 == 0 ? 8 : 4;
                     static_assert((TM * TN * 4) % kBatch == 0, "");
 #pragma unroll
                     for (int c0 = 0; c0 < TM * TN * 4; c0 += kBatch) {
@@ -687,6 +687,7 @@ using CfgMid = TileCfg<128, 128, 64, 2, 2, 4, 2>;
 using CfgN64 = TileCfg<256, 64, 64, 4, 1, 3, 2>;  // 64 output columns (early ResNet stages)
 using CfgTall3 = TileCfg<128, 256, 64, 2, 2, 2, 3>;  // three blocks per CU
 using CfgMid4 = TileCfg<128, 128, 64, 2, 2, 2, 4>;   // four blocks per CU: short K, latency-bound tiles
+using CfgSmall = TileCfg<64, 64, 64, 2, 2, 4, 4>;    // few rows (late convolution stages): more tiles than CUs
 
 }  // namespace
 
