@@ -156,6 +156,127 @@ __global__ __launch_bounds__(256) void wq_gemv_kernel(const float* __restrict__ 
     }
 }
 
+// One activation row (decode): the same scheme with the weight stream software-pipelined.
+// A wavefront owns four weight rows and walks K in steps of 64 * CODES; the 16-byte code
+// loads (and scale / bias) of all four rows for the next step are in flight while the current
+// step is multiplied, and the first step's loads are issued before x is staged, so the only
+// exposed memory latency is the first one.  K % (64 * CODES) == 0.
+template <int BITS>
+__global__ __launch_bounds__(256) void wq_gemv1_kernel(const float* x, const uint32_t* packed, const float* scales,
+                                                       const float* biases, int N, int K, int gs, float* out) {
+    extern __shared__ __attribute__((aligned(16))) float sx[];
+    constexpr int CODES = 128 / BITS, QUADS = CODES / 4, RW = WQ_ROWS / 4;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int chunks = K / CODES, steps = chunks / 64;
+    const int gs_shift = 31 - __builtin_clz(gs);
+    const int words_per_row = K * BITS / 32, groups_per_row = K >> gs_shift;
+    const uint4* wrow[RW];
+    const float* srow[RW];
+    const float* brow[RW];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        int n = blockIdx.x * WQ_ROWS + wave * RW + r;
+        n = n < N ? n : N - 1;  // clamped rows are computed and dropped at the store
+        wrow[r] = reinterpret_cast<const uint4*>(packed + size_t(n) * words_per_row);
+        srow[r] = scales + size_t(n) * groups_per_row;
+        brow[r] = biases + size_t(n) * groups_per_row;
+    }
+    struct Operands {
+        uint4 w[RW];
+        float s[RW], b[RW];
+    };
+    auto fetch = [&](int step, Operands& o) {
+        const int L = step * 64 + lane, g = (L * CODES) >> gs_shift;  // group sizes are powers of two
+#pragma unroll
+        for (int r = 0; r < RW; ++r) o.w[r] = wrow[r][L], o.s[r] = srow[r][g], o.b[r] = brow[r][g];
+    };
+    auto pin = [] {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    Operands o0, o1;
+    fetch(0, o0);
+    pin();
+    for (int i = tid * 4; i < K; i += 256 * 4) {
+        const float4 v = *reinterpret_cast<const float4*>(x + i);
+        const int L = i / CODES, j = (i % CODES) / 4;
+        *reinterpret_cast<float4*>(sx + (j * chunks + L) * 4) = v;
+    }
+    __syncthreads();
+    float acc[RW];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) acc[r] = 0.0f;
+    auto compute = [&](int step, const Operands& o) {
+        const int L = step * 64 + lane;
+        float dot[RW], sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < RW; ++r) dot[r] = 0.0f;
+#pragma unroll
+        for (int quad = 0; quad < QUADS; ++quad) {
+            const float4 xv = *reinterpret_cast<const float4*>(sx + (quad * chunks + L) * 4);
+            sum += (xv.x + xv.y) + (xv.z + xv.w);
+#pragma unroll
+            for (int r = 0; r < RW; ++r) {
+                const uint32_t words[4] = {o.w[r].x, o.w[r].y, o.w[r].z, o.w[r].w};
+                float c[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = quad * 4 + e;  // code index inside the 16-byte load
+                    c[e] = float((words[j * BITS / 32] >> ((j * BITS) % 32)) & MASK);
+                }
+                // fused multiply-adds by name (contraction is off for this library): the decode
+                // loop is bound by vector instructions, not by memory
+                dot[r] = __builtin_fmaf(c[0], xv.x, dot[r]);
+                dot[r] = __builtin_fmaf(c[1], xv.y, dot[r]);
+                dot[r] = __builtin_fmaf(c[2], xv.z, dot[r]);
+                dot[r] = __builtin_fmaf(c[3], xv.w, dot[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RW; ++r) acc[r] += o.s[r] * dot[r] + o.b[r] * sum;
+    };
+    const int last = steps - 1;
+    int step = 0;
+    for (;;) {
+        fetch(step + 1 < steps ? step + 1 : last, o1);
+        pin();
+        compute(step, o0);
+        pin();
+        if (++step >= steps) break;
+        fetch(step + 1 < steps ? step + 1 : last, o0);
+        pin();
+        compute(step, o1);
+        pin();
+        if (++step >= steps) break;
+    }
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        float v = acc[r];
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+        const int n = blockIdx.x * WQ_ROWS + wave * RW + r;
+        if (lane == 0 && n < N) out[n] = v;
+    }
+}
+
+template <int BITS>
+int launch_gemv1(const float* x, const uint32_t* packed, const float* scales, const float* biases, int N, int K,
+                 int gs, float* out, hipStream_t st) {
+    const size_t smem = size_t(K) * sizeof(float);
+    const void* fn = reinterpret_cast<const void*>(wq_gemv1_kernel<BITS>);
+    static size_t attr = 0;
+    if (smem > attr) {
+        LQ_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+        attr = smem;
+    }
+    hipLaunchKernelGGL((wq_gemv1_kernel<BITS>), dim3(unsigned((N + WQ_ROWS - 1) / WQ_ROWS)), dim3(256), smem, st, x,
+                       packed, scales, biases, N, K, gs, out);
+    LQ_CHECK_LAUNCH("wq_gemv1");
+    return LQ_OK;
+}
+
 template <int BITS, int MT>
 int launch_gemv(const float* x, const uint32_t* packed, const float* scales, const float* biases, int M, int N,
                 int K, int gs, int m0, float* out, hipStream_t st) {
@@ -219,6 +340,7 @@ __global__ __launch_bounds__(512) void wq_mfma_kernel(const float4* xt, const ui
     const int r = lane & 15, q = lane >> 4;
     const int n_base = blockIdx.x * 32;
     const int words_per_row = K * BITS / 32, groups_per_row = K / gs;
+    const int gs_shift = 31 - __builtin_clz(gs);  // group sizes are powers of two
     const int m0 = blockIdx.y * 16;
     const float4* xblk = xt + size_t(blockIdx.y) * (K / STEP * XV * 64) + lane;
     const uint32_t* wrow[2];
@@ -248,8 +370,8 @@ __global__ __launch_bounds__(512) void wq_mfma_kernel(const float4* xt, const ui
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             o.wv[rb] = *reinterpret_cast<const uint4*>(wrow[rb] + k0 * BITS / 32);
-            o.sc[rb] = srow[rb][k0 / gs];
-            o.bi[rb] = brow[rb][k0 / gs];
+            o.sc[rb] = srow[rb][k0 >> gs_shift];
+            o.bi[rb] = brow[rb][k0 >> gs_shift];
         }
 #pragma unroll
         for (int j = 0; j < XV; ++j) o.xv[j] = xblk[(step * XV + j) * 64];
@@ -392,6 +514,9 @@ int lq_wq_matmul(const float* x, const uint32_t* packed, const float* scales, co
     if (M > 1 && M <= 64 && mfma_ok)
         return bits == 4 ? launch_wq_mfma<4>(x, packed, scales, biases, M, N, K, group_size, out, st)
                          : launch_wq_mfma<8>(x, packed, scales, biases, M, N, K, group_size, out, st);
+    if (M == 1 && fused_ok && K % (8192 / bits) == 0)
+        return bits == 4 ? launch_gemv1<4>(x, packed, scales, biases, N, K, group_size, out, st)
+                         : launch_gemv1<8>(x, packed, scales, biases, N, K, group_size, out, st);
     if (M <= 16 && fused_ok) {
         // decode shapes: weights are read once per pass of up to four activation rows
         for (int m0 = 0; m0 < M; m0 += 4) {
