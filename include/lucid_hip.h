@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define LQ_VERSION 1
+#define LQ_VERSION 2
 
 typedef enum {
     LQ_OK = 0,

@@ -198,6 +198,9 @@ _lib = None
 _initialised_device = None
 
 
+ABI_VERSION = 2  # LQ_VERSION of include/lucid_hip.h this binding was written against
+
+
 def load() -> C.CDLL:
     """dlopen the library and declare every signature.  Does not touch the GPU."""
     global _lib
@@ -208,6 +211,11 @@ def load() -> C.CDLL:
                 "(hipcc --offload-arch=gfx950).  There is no CPU fallback."
             )
         lib = C.CDLL(LIB_PATH)
+        lib.lq_version.restype = C.c_int
+        if lib.lq_version() != ABI_VERSION:
+            raise GpuNotAvailable(
+                f"{LIB_PATH} has ABI version {lib.lq_version()}, this binding needs {ABI_VERSION}: "
+                "rebuild it with `make -C lucid_amd/csrc` (argument structs differ between versions)")
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(lib, name)  # AttributeError if the symbol is not exported
             fn.argtypes = argtypes
