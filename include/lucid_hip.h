@@ -443,7 +443,10 @@ typedef struct {
     int tile_config;       /* tuning: low byte 0 = choose, 1..9 = a tile shape;
                               next byte 0 = choose, 1 = one block per tile,
                               2 = stream-K work split, 3 = stream-K over the
-                              leftover tiles of the last round only             */
+                              leftover tiles of the last round only; bits 16..30
+                              = number of leading 256-column tiles computed with
+                              shape 1, the remaining columns as a problem of
+                              their own (0 = no split)                          */
     const float* residual; /* optional float32 [M, ldr] added after the activation:
                               out = act(y) + residual (x + linear(...), the
                               residual joins of a transformer block,
@@ -461,6 +464,11 @@ typedef struct {
 } lq_qlinear_args;
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);
+
+/* The tile_config (same encoding as the field above) that the calling thread's last
+ * tile-kernel launch resolved to - what the autotuner chose when 0 was passed.  For
+ * benchmarks and tests; 0 before the first such launch.  No counterpart in Lucid. */
+int lq_last_tile_config(void);
 
 /* The same forward launched n times back to back from native code: for
  * launch-bound callers (decode-shaped layers run for ~10 us, less than an

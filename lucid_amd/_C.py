@@ -66,6 +66,7 @@ _vp, _sz, _i, _f, _u64 = C.c_void_p, C.c_size_t, C.c_int, C.c_float, C.c_uint64
 # name -> argtypes; every function returns int status unless listed in _RESTYPE
 _SIGNATURES = {
     "lq_version": [],
+    "lq_last_tile_config": [],
     "lq_last_error": [],
     "lq_device_count": [C.POINTER(_i)],
     "lq_init": [_i],
@@ -192,7 +193,7 @@ _SIGNATURES["lq_repack_oihw_to_ohwi_i8"] = [_vp, _vp, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_maxpool2d_nhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 
 _RESTYPE = {"lq_last_error": C.c_char_p, "lq_range_buffer_bytes": C.c_size_t}
-_NO_STATUS = {"lq_version", "lq_last_error", "lq_op_count", "lq_range_buffer_bytes"}
+_NO_STATUS = {"lq_version", "lq_last_error", "lq_op_count", "lq_range_buffer_bytes", "lq_last_tile_config"}
 
 _lib = None
 _initialised_device = None

@@ -279,6 +279,15 @@ class Tensor:
             self._materialize()
         return Tensor(shape, self.dtype, "hip", buf=self._buf, offset=self._offset)
 
+    def narrow_rows(self, n: int) -> "Tensor":
+        """The first ``n`` entries along axis 0 as a view of the same storage (a prefix of a
+        contiguous tensor is contiguous)."""
+        if self.device != "hip" or self._grid is not None:
+            raise NotImplementedError("narrow_rows: plain device tensors only")
+        if not 0 <= n <= self.shape[0]:
+            raise _C.ShapeMismatch(f"narrow_rows: {n} rows of {self.shape[0]}")
+        return Tensor((n, *self.shape[1:]), self.dtype, "hip", buf=self._buf, offset=self._offset)
+
     def detach(self) -> "Tensor":
         return self
 

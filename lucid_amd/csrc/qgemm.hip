@@ -99,6 +99,34 @@ int heuristic_tile_shape(const GemmArgs& g, int groups) {
     return 4;
 }
 
+int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st);
+thread_local int t_last_tile_config = 0;  // what the last tile-kernel launch of this thread resolved to
+
+// Two regions of one GEMM: the first a_tiles * 256 output columns go to the 256 x 256 shape
+// (chosen so that its tiles fill whole rounds of the 256 CUs, one block each), the remaining
+// columns are a problem of their own with whatever shape suits it.  The 256 x 256 shape has
+// the best main loop (least LDS traffic per MFMA) but wastes most of a round when its tile
+// count is not a multiple of the CU count; this keeps the one and avoids the other.
+int launch_split(const GemmArgs& g, int a_tiles, hipStream_t st) {
+    const long NA = long(a_tiles) * 256;
+    if (NA <= 0 || NA >= g.N) return fail(LQ_ERR_VALUE, "tile split: %ld columns of %d", NA, g.N);
+    GemmArgs ga = g;
+    ga.N = int(NA);
+    int rc = launch_tile_shape(ga, false, 1, 1, 1, st);
+    if (rc) return rc;
+    GemmArgs gb = g;
+    gb.N = g.N - int(NA);
+    gb.w = g.w + size_t(NA) * g.K;
+    if (g.wsum) gb.wsum = g.wsum + NA;
+    if (g.w_scale) gb.w_scale = g.w_scale + NA;
+    if (g.bias) gb.bias = static_cast<const char*>(g.bias) + NA * (g.bias_dtype == LQ_F16 ? 2 : 4);
+    const size_t esz = g.out_mode == OUT_F16 ? 2 : (g.out_mode == OUT_REQUANT_I8 ? 1 : 4);
+    gb.out = static_cast<char*>(g.out) + NA * esz;
+    if (g.residual) gb.residual = g.residual + NA;
+    if (g.join_q) gb.join_q = g.join_q + NA;
+    return launch_tile_cfg(gb, false, 1, 0, st);
+}
+
 // The best tile shape depends on how the tile count falls on the 256 CUs and on
 // the epilogue's share, which no simple rule predicted well (at M = 12608 the
 // winner changes between K = 768 and K = 3072).  So the first launch of a problem
@@ -156,7 +184,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9) return LQ_OK;
 
     // candidates are whole tile_config values (shape | schedule << 8)
-    int cands[10], n = 0;
+    int cands[12], n = 0;
     if (g.N <= 64) cands[n++] = 6;
     cands[n++] = 5;
     if (g.K <= 256) cands[n++] = 8;  // one to four k-iterations: latency-bound tiles, four blocks per CU
@@ -166,6 +194,13 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
     if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
     if (tiles128 < 256) cands[n++] = 9;  // ... or cover the chip with 64 x 64 tiles
+    // whole rounds of 256 x 256 tiles plus a remainder (see launch_split)
+    if (!conv && groups == 1 && g.range == nullptr && g.M >= 256) {
+        const long tiles_m = (g.M + 255) / 256, tiles_n = g.N / 256;
+        const long rounds = tiles_m * tiles_n / 256;
+        const long a_tiles = rounds > 0 ? rounds * 256 / tiles_m : 0;
+        if (a_tiles > 0 && a_tiles * 256 < g.N && a_tiles < 32768) cands[n++] = 1 | (1 << 8) | int(a_tiles << 16);
+    }
     hipEvent_t e0, e1;
     LQ_HIP(hipEventCreate(&e0));
     LQ_HIP(hipEventCreate(&e1));
@@ -173,15 +208,32 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     int rc = LQ_OK;
     bool timed = true;
     for (int i = 0; i < n && rc == LQ_OK && timed; ++i) {
-        const int shape = cands[i] & 0xff, sched = (cands[i] >> 8) ? (cands[i] >> 8) : 1;
-        rc = launch_tile_shape(g, conv, groups, shape, sched, st);  // warm: code load, attributes
+        const int shape = cands[i] & 0xff, sched = ((cands[i] >> 8) & 0xff) ? ((cands[i] >> 8) & 0xff) : 1;
+        const int a_tiles = cands[i] >> 16;
+        auto launch = [&] {
+            return a_tiles ? launch_split(g, a_tiles, st) : launch_tile_shape(g, conv, groups, shape, sched, st);
+        };
+        rc = launch();  // warm: code load, attributes (and the remainder's own tuning)
         if (rc) break;
+        // Candidates can be within a few percent of each other and the clock takes a while
+        // to settle under load: every candidate runs for about a millisecond per timing (its
+        // own launches warm the chip up for it), and the better of two timings counts.
         timed = hipEventRecord(e0, st) == hipSuccess;
-        for (int r = 0; r < 3 && rc == LQ_OK; ++r) rc = launch_tile_shape(g, conv, groups, shape, sched, st);
-        float ms = 0.0f;
+        rc = launch();
+        float one = 0.0f;
         timed = timed && rc == LQ_OK && hipEventRecord(e1, st) == hipSuccess &&
-                hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
-        if (timed && ms < best) best = ms, *cfg_out = cands[i];
+                hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&one, e0, e1) == hipSuccess;
+        if (!timed || rc) break;
+        int reps = one > 0.0f ? int(1.0f / one) : 4;
+        reps = reps < 4 ? 4 : (reps > 40 ? 40 : reps);
+        for (int pass = 0; pass < 2 && timed && rc == LQ_OK; ++pass) {
+            timed = hipEventRecord(e0, st) == hipSuccess;
+            for (int r = 0; r < reps && rc == LQ_OK; ++r) rc = launch();
+            float ms = 0.0f;
+            timed = timed && rc == LQ_OK && hipEventRecord(e1, st) == hipSuccess &&
+                    hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+            if (timed && ms / reps < best) best = ms / reps, *cfg_out = cands[i];
+        }
     }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
@@ -197,17 +249,28 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
 
 // tile_config: low byte = tile shape (0 = choose, 1..9 = a specific one), next
 // byte = schedule (0 = choose, 1 = block per tile, 2 = stream-K, 3 = stream-K over
-// the leftover tiles only).
+// the leftover tiles only), bits 16..30 = number of leading 256-column tiles given to
+// shape 1 with the remaining columns tuned separately (0 = no split).
 int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st) {
     int cfg = tile_config & 0xff;
     int schedule = (tile_config >> 8) & 0xff;
+    int a_tiles = (tile_config >> 16) & 0x7fff;
     if (cfg == 0) {
         int tuned = 0;
         int rc = tuned_tile_shape(g, conv, groups, st, &tuned);
         if (rc) return rc;
         cfg = tuned & 0xff;
         if (schedule == 0) schedule = (tuned >> 8) & 0xff;
+        a_tiles = tuned >> 16;
     }
+    if (a_tiles > 0) {
+        LQ_REQUIRE(!conv && groups == 1 && g.range == nullptr, LQ_ERR_VALUE,
+                   "tile_config: a column split needs a plain GEMM without a kept range");
+        const int rc = launch_split(g, a_tiles, st);
+        t_last_tile_config = 1 | (1 << 8) | (a_tiles << 16);
+        return rc;
+    }
+    t_last_tile_config = cfg | ((schedule ? schedule : 1) << 8);
     return launch_tile_shape(g, conv, groups, cfg, schedule, st);
 }
 
@@ -412,6 +475,8 @@ int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t 
 }  // namespace lq
 
 extern "C" {
+
+int lq_last_tile_config(void) { return t_last_tile_config; }
 
 int lq_rowsum_i8(const int8_t* w, int32_t* out, int N, int K, lq_stream stream) {
     if (N == 0) return LQ_OK;

@@ -283,3 +283,32 @@ def test_split_k_over_few_tiles_exact():
     assert np.array_equal(acc, O.igemm(a, w))
     # and through the automatic choice (which may pick that schedule for this shape)
     assert np.array_equal(_ops.qlinear_i8(hip(a), hip(w), out_mode=_ops.OUT_ACC_I32, path=1).numpy(), acc)
+
+
+@pytest.mark.parametrize("M,N,K,a_tiles", [(2048, 11008, 256, 32), (300, 1000, 128, 2), (512, 800, 192, 1)])
+def test_column_split_between_two_tile_shapes_exact(M, N, K, a_tiles):
+    """tile_config bits 16+: the first a_tiles * 256 columns with 256x256 tiles, the rest as a problem
+    of its own - every per-column operand (weights, sums, scales, bias, residual, join, output) is offset."""
+    rng = np.random.default_rng(M + N + K)
+    a = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    w = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    ws = (rng.random(N).astype(np.float32) + 0.5) * 1e-3
+    bias = rng.standard_normal(N).astype(np.float32)
+    hip = lambda t: L.tensor(t, device="hip")
+    da, dw = hip(a), hip(w)
+    tc = 1 | (1 << 8) | (a_tiles << 16)
+    assert np.array_equal(_ops.qlinear_i8(da, dw, out_mode=_ops.OUT_ACC_I32, path=1, tile_config=tc).numpy(),
+                          O.igemm(a, w))
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    common = dict(a_zp=3, a_scale=hip(np.float32(0.02)), w_scale=hip(ws), wsum=_ops.rowsum_i8(dw), bias=hip(bias))
+    y = _ops.qlinear_i8(da, dw, **common, out_mode=_ops.OUT_F32, residual=hip(res), path=1, tile_config=tc).numpy()
+    want = _ops.qlinear_i8(da, dw, **common, out_mode=_ops.OUT_F32, residual=hip(res), path=1, tile_config=5 | 0x100)
+    assert np.array_equal(y.view(np.uint32), want.numpy().view(np.uint32))
+    other = hip(rng.integers(-128, 128, (M, N)).astype(np.int8))
+    one = lambda v: hip(np.float32(v))
+    jk = dict(out_mode=_ops.OUT_REQUANT_I8, out_scale=one(0.05), out_zp=one(3.0), out_qmin=-128, out_qmax=127,
+              join=dict(q=other, offset=-128, scale=one(0.02), zp=one(120.0), relu=True, out_scale=one(0.06),
+                        out_zp=one(0.0), out_qmin=0, out_qmax=255, out_offset=-128))
+    j1 = _ops.qlinear_i8(da, dw, **common, **jk, path=1, tile_config=tc).numpy()
+    j2 = _ops.qlinear_i8(da, dw, **common, **jk, path=1, tile_config=5 | 0x100).numpy()
+    assert np.array_equal(j1, j2)
