@@ -44,7 +44,9 @@ PEAK_HBM_GBS = 8000.0     # MI355X published HBM3E bandwidth, GB/s
 # the library's plain 1 GiB copy kernel: fetch x2.000, write x1.000).  The runs
 # are summarised in profiles/hbm_traffic_qlinear_and_quantize.md.
 MEASURED_TRAFFIC_BYTES = {
-    "linear_m2048": int((2.0 * 96636 + 44032) * 1024),
+    # one 128x256-tiled launch / the column split (256x256 tiles over 8192 columns + 128x256 over 2816)
+    "linear_m2048": int((2.0 * 96504 + 44032) * 1024),
+    "linear_m2048_split": int((2.0 * (49458.5 + 30888.25) + 32768 + 11264) * 1024),
     "quantize_per_channel_i8": int((2.0 * 524577 + 262144) * 1024),
     "dequantize_per_channel_i8": int((2.0 * 131350 + 1048712) * 1024),
     "minmax_per_channel": int((2.0 * 524317 + 257) * 1024),
@@ -554,7 +556,7 @@ def main() -> int:
             "peak": PEAK_INT8_TOPS,
             "unit": "TOP/s",
             "frac": round(r["kernel_tops"] / PEAK_INT8_TOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES["linear_m2048"],
+            "traffic": MEASURED_TRAFFIC_BYTES["linear_m2048_split" if r["split"] else "linear_m2048"],
             "kernel": "qgemm_tile_kernel",
             "avg_kernel_us": round(r["avg_kernel_ms"] * 1e3, 2),
             "median_kernel_us": round(r["median_ms"] * 1e3, 2),
