@@ -277,6 +277,26 @@ def bench_quant_roundtrip(L, Q, _C, steps, warmup):
     return out
 
 
+EAGER_ONLY = False  # --eager: time Python-driven launches where a graph replay is timed by default
+
+
+class _Replay:
+    """`fn` captured into a HIP graph (default), or `fn` itself under --eager."""
+
+    def __init__(self, L, fn):
+        self.graph = None
+        if EAGER_ONLY:
+            self.run, self.how = fn, "eager launches"
+        else:
+            with L.graph.capture() as g:
+                fn()
+            self.graph, self.run, self.how = g, g.replay, "hip graph replay"
+
+    def destroy(self):
+        if self.graph is not None:
+            self.graph.destroy()
+
+
 def bench_resnet50(L, _C, steps, warmup):
     """int8 static-quantized ResNet-50, batch 32, 3x224x224 uniform[0,1] inputs,
     random He-normal weights with BatchNorm folded, fixed calibration grids.  The
@@ -289,14 +309,13 @@ def bench_resnet50(L, _C, steps, warmup):
     batch = 32
     x = L.tensor(rng.uniform(0, 1, (batch, 3, 224, 224)).astype(np.float32), device="hip")
     y = model(x)  # eager warm-up caches host-side scalars
-    with L.graph.capture() as g:
-        y = model(x)
-    total, per = time_launches(_C, g.replay, steps, warmup)
+    g = _Replay(L, lambda: model(x))
+    total, per = time_launches(_C, g.run, steps, warmup)
     ms = total / steps
     gmacs = W.resnet50_conv_gmacs(batch)
     out = {"images_per_s": round(batch / ms * 1e3, 1), "ms_per_batch": round(ms, 4), "batch": batch,
            "int8_TOP/s": round(2 * gmacs / ms, 2), "GMAC_per_batch": round(gmacs, 2),
-           "p95_ms": round(float(np.percentile(per, 95)), 4), "launch": "hip graph replay"}
+           "p95_ms": round(float(np.percentile(per, 95)), 4), "launch": g.how}
     assert np.isfinite(y.numpy()).all()
     g.destroy()
     return out
@@ -316,15 +335,14 @@ def bench_vit_b16(L, _C, steps, warmup):
     y = model(x)
     eager_total, _ = time_launches(_C, lambda: model(x), max(3, steps // 4), 1)
     eager_ms = eager_total / max(3, steps // 4)
-    with L.graph.capture() as g:
-        y = model(x)
-    total, per = time_launches(_C, g.replay, steps, warmup)
+    g = _Replay(L, lambda: model(x))
+    total, per = time_launches(_C, g.run, steps, warmup)
     ms = total / steps
     gops = W.vit_linear_gops(batch=batch)
     out = {"images_per_s": round(batch / ms * 1e3, 1), "ms_per_batch": round(ms, 4), "batch": batch,
            "eager_ms_per_batch": round(eager_ms, 4),
            "linear_int8_TOP/s_end_to_end": round(gops / ms, 2), "linear_GOP_per_batch": round(gops, 1),
-           "p95_ms": round(float(np.percentile(per, 95)), 4), "launch": "hip graph replay"}
+           "p95_ms": round(float(np.percentile(per, 95)), 4), "launch": g.how}
     assert np.isfinite(y.numpy()).all()
     g.destroy()
     return out
@@ -348,9 +366,8 @@ def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     y = model(x)
     total, _ = time_launches(_C, lambda: model(x), steps, warmup)
     eager_us = total / steps * 1e3
-    with L.graph.capture() as g:
-        y = model(x)
-    total, _ = time_launches(_C, g.replay, steps, warmup)
+    g = _Replay(L, lambda: model(x))
+    total, _ = time_launches(_C, g.run, steps, warmup)
     graph_us = total / steps * 1e3
     assert np.isfinite(y.numpy()).all()
     g.destroy()
@@ -506,6 +523,8 @@ def main() -> int:
     ap.add_argument("--mfma-probe", action="store_true",
                     help="only print the MFMA-only rate for several operand distributions")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--eager", action="store_true",
+                    help="time Python-driven launches instead of HIP graph replays (for runs under a tracer)")
     ap.add_argument("--cpu-sample-rows", type=int, default=2048)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -518,6 +537,8 @@ def main() -> int:
     from lucid_amd import _C, _ops
 
     _C.init(0)
+    global EAGER_ONLY
+    EAGER_ONLY = args.eager
     M, K, N = 2048, 4096, 11008
     if args.mfma_probe:
         # the matrix cores' sustained rate by operand statistics (no data movement at all)
@@ -566,8 +587,9 @@ def main() -> int:
         },
     }
     if r["split"]:
-        # a step is two launches (column split); `achieved` above charges both,
-        # and the gap between them, to the step.  The dominant kernel on its own:
+        # a step is two launches (the tuner split the output columns between two tile shapes);
+        # `achieved` above charges both, and the gap between them, to the step.  The dominant
+        # kernel on its own:
         sp = r["split"]
         line["roofline"]["launches_per_step"] = 2
         line["roofline"]["dominant_kernel"] = {
