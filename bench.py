@@ -277,6 +277,73 @@ def bench_quant_roundtrip(L, Q, _C, steps, warmup):
     return out
 
 
+def _acc_digest(c):
+    """Two position-weighted int64 sums of an int32 matrix: equal digests = equal accumulators
+    (up to collisions no kernel bug would hit)."""
+    c = np.asarray(c).astype(np.int64)
+    wr = (np.arange(c.shape[0], dtype=np.int64) * 31 % 1009 + 1)[:, None]
+    wc = (np.arange(c.shape[1], dtype=np.int64) * 17 % 1013 + 1)[None, :]
+    return [int(c.sum()), int((c * wr * wc).sum())]
+
+
+def vendor_child(path, steps, warmup):
+    """Child process of --vendor-yardstick: torch only (its own copy of the HIP runtime cannot
+    share a process with this library's), operands from the .npz the parent wrote."""
+    import torch
+
+    z = np.load(path)
+    a, w = torch.from_numpy(z["a"]).cuda(), torch.from_numpy(z["w"]).cuda()
+    c = torch._int_mm(a, w.t())
+    digest = _acc_digest(c.cpu().numpy())
+    for _ in range(warmup):
+        torch._int_mm(a, w.t())
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(steps):
+        torch._int_mm(a, w.t())
+    e1.record()
+    torch.cuda.synchronize()
+    print(json.dumps({"ms": e0.elapsed_time(e1) / steps, "digest": digest}))
+    return 0
+
+
+def vendor_yardstick(L, Q, _C, _ops, steps, warmup):
+    """The vendor library's int8 x int8 -> int32 GEMM (hipBLASLt behind ``torch._int_mm``) on the
+    very codes this library's kernel is timed on: the matrix cores' clock depends on the operand
+    data, so only the same codes compare.  The vendor call writes raw int32 accumulators; this
+    library is timed both with its fused fp16 epilogue and writing the accumulators.  torch runs
+    in a child process; this process idles meanwhile."""
+    import subprocess
+    import tempfile
+
+    out = {}
+    for (M, K, N) in ((2048, 4096, 11008), (2048, 4096, 8192), (8192, 4096, 11008), (8192, 8192, 8192)):
+        r = bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup)
+        t = r["tensors"]
+        acc = L.Tensor.empty((M, N), L.int32, "hip")
+        _ops.qlinear_i8(t["xq"], t["wq"], out_mode=_ops.OUT_ACC_I32, out=acc)
+        tot, _ = time_launches(_C, lambda: _ops.qlinear_i8(t["xq"], t["wq"], out_mode=_ops.OUT_ACC_I32, out=acc,
+                                                           repeat=steps), 1, 1)
+        digest = _acc_digest(acc.numpy())
+        with tempfile.TemporaryDirectory() as d:
+            path = os.path.join(d, "operands.npz")
+            np.savez(path, a=t["xq"].numpy(), w=t["wq"].numpy())
+            child = subprocess.run([sys.executable, os.path.abspath(__file__), "--vendor-child", path,
+                                    "--steps", str(steps), "--warmup", str(warmup)],
+                                   capture_output=True, text=True, timeout=600)
+        if child.returncode != 0:
+            raise RuntimeError("vendor yardstick child failed: " + child.stderr[-2000:])
+        v = json.loads(child.stdout.strip().splitlines()[-1])
+        out[f"M{M}_K{K}_N{N}"] = {
+            "this_library_fp16_epilogue_TOP/s": round(r["kernel_tops"], 1),
+            "this_library_int32_accumulators_TOP/s": round(r["ops"] / (tot / steps) / 1e9, 1),
+            "vendor_int32_accumulators_TOP/s": round(r["ops"] / v["ms"] / 1e9, 1),
+            "vendor_us": round(v["ms"] * 1e3, 1), "accumulators_equal": v["digest"] == digest}
+        del r, t, acc
+    return out
+
+
 EAGER_ONLY = False  # --eager: time Python-driven launches where a graph replay is timed by default
 
 
@@ -522,6 +589,10 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="only print the MFMA-only rate for several operand distributions")
+    ap.add_argument("--vendor-yardstick", action="store_true",
+                    help="time the ROCm library's int8 GEMM (through torch._int_mm, if torch is importable) "
+                         "on the same operand codes beside this library's; a yardstick, not a dependency")
+    ap.add_argument("--vendor-child", default=None, help=argparse.SUPPRESS)
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--eager", action="store_true",
                     help="time Python-driven launches instead of HIP graph replays (for runs under a tracer)")
@@ -531,6 +602,9 @@ def main() -> int:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
         return 2
+
+    if args.vendor_child:
+        return vendor_child(args.vendor_child, args.steps, args.warmup)
 
     import lucid_amd as L
     import lucid_amd.quantization as Q
@@ -553,6 +627,9 @@ def main() -> int:
         t = make_linear(L, Q, _C, _ops, M, K, N, 1)
         res["benchmark_codes"] = round(probe_mfma_ceiling(L, _C, t["xq"], t["wq"]), 1)
         print(json.dumps({"mfma_only_tops_by_operand_data": res, "datasheet_peak_tops": PEAK_INT8_TOPS}))
+        return 0
+    if args.vendor_yardstick:
+        print(json.dumps(vendor_yardstick(L, Q, _C, _ops, args.steps, args.warmup)))
         return 0
     r = bench_linear(L, Q, _C, _ops, M, K, N, args.steps, args.warmup)
     line = {
