@@ -70,6 +70,7 @@ __device__ __forceinline__ void load_cols(const GemmArgs& g, const int (&n)[T], 
     }
 }
 
+// The plain form: one division per element (kernels that are bound by memory, not by it).
 __device__ __forceinline__ float q_core(float x, float s, float z, float lo, float hi) {
     float t = x / s;
     float r = __builtin_rintf(t);
@@ -78,14 +79,60 @@ __device__ __forceinline__ float q_core(float x, float s, float z, float lo, flo
     return u;
 }
 
+// One quantization grid, with the reciprocal of its scale (see quant_fast).
+struct QGrid {
+    float s, inv, z, lo, hi;
+};
+
+// `fast`: the kernel quantizes many elements per lane, so one division to get the
+// reciprocal pays.  A grid outside what quant_fast's argument covers (a scale outside a sane
+// range, a zero point or bounds beyond +-255) gets a NaN reciprocal, which sends every
+// element down the dividing branch.
+__device__ __forceinline__ QGrid make_qgrid(float s, float z, float lo, float hi, bool fast) {
+    QGrid G;
+    G.s = s, G.z = z, G.lo = lo, G.hi = hi;
+    const float a = __builtin_fabsf(s);
+    const bool ok = fast && a > 0x1p-60f && a < 0x1p60f && __builtin_fabsf(z) <= 255.0f &&
+                    __builtin_fabsf(lo) <= 255.0f && __builtin_fabsf(hi) <= 255.0f;
+    G.inv = ok ? 1.0f / s : __builtin_nanf("");
+    return G;
+}
+
+// clamp(rint(x / s) + z, lo, hi) with the correctly rounded IEEE quotient, bit for bit,
+// mostly without dividing; a NaN becomes KEEP_NAN ? NaN : 0.
+// tp = x * fl(1/s) is within 2^-22.9 relative of the exact quotient e, and fl(x / s) within
+// 2^-24.  rint only changes value at the half-integers.
+//  * |tp| < 512: tp is within 6.2e-5 of e and fl(x / s) within 3.1e-5; when tp is farther
+//    than 2^-12 = 2.4e-4 from every half-integer, both lie strictly between the same two of
+//    them and round to the same integer.
+//  * 512 <= |tp| < inf, with d passing the test: both rint(tp) and rint(fl(x / s)) are
+//    beyond +-511 with the same sign, and with |z|, |lo|, |hi| <= 255 both clamp to the
+//    same bound.
+// Otherwise (a few elements in ten thousand, and whatever is infinite or NaN: d = NaN
+// fails the test) the lane divides.
+template <bool KEEP_NAN>
+__device__ __forceinline__ float quant_fast(float x, const QGrid& G) {
+    const float tp = x * G.inv;
+    const float r = __builtin_rintf(tp);
+    const float d = tp - r;  // exact where it matters
+    float c = __builtin_amdgcn_fmed3f(r + G.z, G.lo, G.hi);
+    if (__builtin_expect(!(__builtin_fabsf(d) < 0.5f - 0x1p-12f), 0)) {
+        const float u = __builtin_rintf(x / G.s) + G.z;
+        c = (u != u) ? (KEEP_NAN ? u : 0.0f) : __builtin_amdgcn_fmed3f(u, G.lo, G.hi);
+    }
+    return c;
+}
+
 // One output element.  Float steps are separate (no FMA) and in the order the
 // CPU restatement uses, so results are bit-identical to it.  MODE is a
 // compile-time constant so that each output form gets a tight loop.
-// epilogue_value returns the element as 32 bits (float bits, or the integer
-// for the accumulator / requantized-code forms); store_* narrows and writes.
+// epilogue_value returns the element as 32 bits: float bits, the integer for the
+// accumulator / requantized-code forms, or - ahead of a fused join - the requantized
+// code still as a float (finish_value / join_code take it from there); store_*
+// narrows and writes.
 template <int MODE>
 __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t acc, float as,
-                                                   const ColParams& c, float S, float Z) {
+                                                   const ColParams& c, const QGrid& G) {
     if (MODE == OUT_ACC_I32) return uint32_t(acc);
     float f = float(acc - c.corr);
     float sc = as * c.ws;
@@ -102,12 +149,10 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
         if (g.gelu) y = (0.5f * y) * (1.0f + erff(y * 0.70710678118654752440f));
         return __float_as_uint(y);
     }
-    float qv = q_core(y, S, Z, float(g.out_qmin), float(g.out_qmax));
-    if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) {
-        int code = (qv != qv) ? 0 : int(qv);
-        return uint32_t(code + g.out_offset);
-    }
-    return __float_as_uint((qv - Z) * S);  // OUT_FAKEQUANT_F32
+    if (MODE == OUT_REQUANT_JOIN) return __float_as_uint(quant_fast<false>(y, G));
+    // the stored form adds out_offset: store_* does, on the packed bytes where it can
+    if (MODE == OUT_REQUANT_I8) return uint32_t(int(quant_fast<false>(y, G)));
+    return __float_as_uint((quant_fast<true>(y, G) - G.z) * G.s);  // OUT_FAKEQUANT_F32
 }
 
 // y + residual[m, n] for the float output forms (x + linear(...), the residual
@@ -123,38 +168,44 @@ __device__ __forceinline__ uint32_t add_residual(const GemmArgs& g, uint32_t bit
 // to this layer's output): both operands are dequantized in float32 with their own
 // grids, added, optionally clamped at zero, and requantized.
 struct JoinParams {
-    float S1, Z1;          // this layer's output grid
-    float s2, z2;          // the other operand's grid
-    float S, Z, lo, hi;    // the join's output grid
+    float S1, Z1;  // this layer's output grid
+    float s2, z2;  // the other operand's grid
+    QGrid out;     // the join's output grid
 };
 
-__device__ __forceinline__ JoinParams load_join(const GemmArgs& g, float S1, float Z1) {
+__device__ __forceinline__ JoinParams load_join(const GemmArgs& g, const QGrid& G, bool fast) {
     JoinParams jp;
-    jp.S1 = S1, jp.Z1 = Z1;
+    jp.S1 = G.s, jp.Z1 = G.z;
     jp.s2 = g.join_scale[0], jp.z2 = g.join_zp[0];
-    jp.S = g.join_out_scale[0], jp.Z = g.join_out_zp[0];
-    jp.lo = float(g.join_out_qmin), jp.hi = float(g.join_out_qmax);
+    jp.out = make_qgrid(g.join_out_scale[0], g.join_out_zp[0], float(g.join_out_qmin), float(g.join_out_qmax), fast);
     return jp;
 }
 
-// bits: this layer's stored code (code + out_offset); other: the partner's stored code
+// bits: this layer's requantized code as a float (what epilogue_value<OUT_REQUANT_JOIN>
+// returned); other: the partner's stored code
 __device__ __forceinline__ uint32_t join_code(const GemmArgs& g, const JoinParams& jp, uint32_t bits, int other) {
-    const float x1 = (float(int(bits) - g.out_offset) - jp.Z1) * jp.S1;
+    const float x1 = (__uint_as_float(bits) - jp.Z1) * jp.S1;
     const float x2 = (float(other - g.join_off) - jp.z2) * jp.s2;
     float y = x1 + x2;
     if (g.join_relu) y = (y < 0.0f) ? 0.0f : y;
-    const float qv = q_core(y, jp.S, jp.Z, jp.lo, jp.hi);
-    return uint32_t(((qv != qv) ? 0 : int(qv)) + g.join_out_offset);
+    return uint32_t(int(quant_fast<false>(y, jp.out)));  // store_* adds join_out_offset
 }
 
 // one element's residual step, whichever form the output mode has
 template <int MODE>
-__device__ __forceinline__ uint32_t finish_value(const GemmArgs& g, uint32_t bits, int m, int n, float S, float Z) {
+__device__ __forceinline__ uint32_t finish_value(const GemmArgs& g, uint32_t bits, int m, int n, const QGrid& G) {
     if (MODE == OUT_REQUANT_JOIN) {
-        const JoinParams jp = load_join(g, S, Z);
+        const JoinParams jp = load_join(g, G, false);
         return join_code(g, jp, bits, int(g.join_q[size_t(m) * size_t(g.join_ld) + size_t(n)]));
     }
     return add_residual<MODE>(g, bits, m, n);
+}
+
+// Codes leave epilogue_value / join_code without their storage offset (-128 for the quint8
+// form, else 0); it is added here, to four packed bytes at once where it is 0 or +-128.
+template <int MODE>
+__device__ __forceinline__ int code_offset(const GemmArgs& g) {
+    return MODE == OUT_REQUANT_JOIN ? g.join_out_offset : g.out_offset;
 }
 
 template <int MODE>
@@ -162,7 +213,7 @@ __device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint
     if (MODE == OUT_F16)
         static_cast<_Float16*>(g.out)[idx] = _Float16(__uint_as_float(v));
     else if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN)
-        static_cast<int8_t*>(g.out)[idx] = int8_t(int(v));
+        static_cast<int8_t*>(g.out)[idx] = int8_t(int(v) + code_offset<MODE>(g));
     else
         static_cast<uint32_t*>(g.out)[idx] = v;  // f32 / i32 bit patterns
 }
@@ -176,7 +227,17 @@ __device__ __forceinline__ void store_vec4(const GemmArgs& g, size_t idx, uint4 
                 _Float16(__uint_as_float(v.z)), _Float16(__uint_as_float(v.w))};
         *reinterpret_cast<h4*>(static_cast<_Float16*>(g.out) + idx) = h;
     } else if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) {
-        uint32_t packed = (v.x & 0xffu) | ((v.y & 0xffu) << 8) | ((v.z & 0xffu) << 16) | (v.w << 24);
+        // low bytes of x, y, z, w -> one dword (byte selectors 0-3: second operand, 4-7: first)
+        const uint32_t xy = __builtin_amdgcn_perm(v.y, v.x, 0x0c0c0400u);
+        const uint32_t zw = __builtin_amdgcn_perm(v.w, v.z, 0x0c0c0400u);
+        uint32_t packed = __builtin_amdgcn_perm(zw, xy, 0x05040100u);
+        const int off = code_offset<MODE>(g);
+        if ((off & 0x7f) == 0) {
+            if (off & 0x80) packed ^= 0x80808080u;  // +-128 modulo 256, byte by byte
+        } else {
+            const uint32_t o = uint32_t(off);
+            packed = ((v.x + o) & 0xffu) | (((v.y + o) & 0xffu) << 8) | (((v.z + o) & 0xffu) << 16) | ((v.w + o) << 24);
+        }
         *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(g.out) + idx) = packed;
     } else {
         *reinterpret_cast<uint4*>(static_cast<uint32_t*>(g.out) + idx) = v;
@@ -186,8 +247,10 @@ __device__ __forceinline__ void store_vec4(const GemmArgs& g, size_t idx, uint4 
 template <int MODE>
 __device__ __forceinline__ void epilogue_store_t(const GemmArgs& g, int m, int n, int32_t acc,
                                                  float as, const ColParams& c, float S, float Z) {
+    // one element per call: no reciprocal, the grid divides
+    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), false);
     store_scalar<MODE>(g, size_t(m) * size_t(g.ldo) + size_t(n),
-                       finish_value<MODE>(g, epilogue_value<MODE>(g, acc, as, c, S, Z), m, n, S, Z));
+                       finish_value<MODE>(g, epilogue_value<MODE>(g, acc, as, c, G), m, n, G));
 }
 
 __device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, int32_t acc,

@@ -70,6 +70,7 @@ int launch_tile_c6(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c7(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c8(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c9(const GemmArgs&, bool, int, int, hipStream_t);
+int launch_tile_c10(const GemmArgs&, bool, int, int, hipStream_t);
 }  // namespace lq
 
 namespace {
@@ -85,6 +86,7 @@ int launch_tile_shape(const GemmArgs& g, bool conv, int groups, int cfg, int sch
     case 7: return launch_tile_c7(g, conv, groups, schedule, st);
     case 8: return launch_tile_c8(g, conv, groups, schedule, st);
     case 9: return launch_tile_c9(g, conv, groups, schedule, st);
+    case 10: return launch_tile_c10(g, conv, groups, schedule, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -184,7 +186,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9) return LQ_OK;
 
     // candidates are whole tile_config values (shape | schedule << 8)
-    int cands[12], n = 0;
+    int cands[16], n = 0;
     if (g.N <= 64) cands[n++] = 6;
     cands[n++] = 5;
     if (g.K <= 256) cands[n++] = 8;  // one to four k-iterations: latency-bound tiles, four blocks per CU
@@ -194,6 +196,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
     if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
     if (tiles128 < 256) cands[n++] = 9;  // ... or cover the chip with 64 x 64 tiles
+    if (tiles128 < 256 && g.K >= 1024) cands[n++] = 10;  // ... with 128-byte k-iterations
     // whole rounds of 256 x 256 tiles plus a remainder (see launch_split)
     if (!conv && groups == 1 && g.range == nullptr && g.M >= 256) {
         const long tiles_m = (g.M + 255) / 256, tiles_n = g.N / 256;

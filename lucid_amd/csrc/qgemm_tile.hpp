@@ -107,6 +107,10 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
     const int esize = MODE == OUT_F16 ? 2 : ((MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) ? 1 : 4);
     const bool vec_ok = (g.ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0);
     const int row0 = lane / QUADS_PER_ROW, cq = (lane % QUADS_PER_ROW) * 4;
+    constexpr bool kRequant = MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN || MODE == OUT_FAKEQUANT_F32;
+    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), kRequant);
+    JoinParams jp;
+    if (MODE == OUT_REQUANT_JOIN) jp = load_join(g, G, true);
     // running range of what this lane stores (float32 output with a kept range only)
     const bool keep = MODE == OUT_F32X && g.range != nullptr;
     auto track = [&](uint32_t bits) {
@@ -155,7 +159,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     stage[row * STRIDE + j * 32 + (lane & 31)] =
-                        epilogue_value<MODE>(g, acc[i][j][r], as[rr], cp[j], S, Z);
+                        epilogue_value<MODE>(g, acc[i][j][r], as[rr], cp[j], G);
             }
             wave_lds_sync();
             const uint32_t* src = stage + row0 * STRIDE + cq;
@@ -176,7 +180,6 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                     }
                 }
                 if (MODE == OUT_REQUANT_JOIN && join_fast) {
-                    const JoinParams jp = load_join(g, S, Z);
 #pragma unroll
                     for (int p = 0; p < PASSES; ++p) {
                         v[p].x = join_code(g, jp, v[p].x, int(int8_t(jv[p] & 0xff)));
@@ -200,10 +203,10 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                     uint4 v = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
                     const int m = m_first + p * ROWS_PER_PASS;
                     if (m < g.M && n < n_limit) {
-                        v.x = finish_value<MODE>(g, v.x, m, n, S, Z);
-                        if (n + 1 < n_limit) v.y = finish_value<MODE>(g, v.y, m, n + 1, S, Z);
-                        if (n + 2 < n_limit) v.z = finish_value<MODE>(g, v.z, m, n + 2, S, Z);
-                        if (n + 3 < n_limit) v.w = finish_value<MODE>(g, v.w, m, n + 3, S, Z);
+                        v.x = finish_value<MODE>(g, v.x, m, n, G);
+                        if (n + 1 < n_limit) v.y = finish_value<MODE>(g, v.y, m, n + 1, G);
+                        if (n + 2 < n_limit) v.z = finish_value<MODE>(g, v.z, m, n + 2, G);
+                        if (n + 3 < n_limit) v.w = finish_value<MODE>(g, v.w, m, n + 3, G);
                         if (MODE == OUT_F32X && keep) {
                             track(v.x);
                             if (n + 1 < n_limit) track(v.y);
@@ -344,6 +347,18 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         const int8_t* a_tile = CONV ? g.cx : g.a + size_t(m0) * g.K;
         const int8_t* b_tile = g.w + size_t(n0) * g.K;
         const int k_end = ke * BK < g.K ? ke * BK : g.K;  // nothing is fetched past the segment
+        // CONV: filter tap (kh, kw) and channel offset of this lane's 16 bytes in the next stage
+        // to be loaded.  Stages are loaded in k order, BK bytes apart, so the position is found
+        // by division once per segment and then stepped (the divisions by run-time values cost
+        // more than the MFMAs of a small tile's k-iteration).
+        int c_ci0 = 0, c_kh = 0, c_kw = 0;
+        if (CONV) {
+            const int k = kb * BK + kc * 16;
+            const int tap = k / g.cCg;
+            c_ci0 = k - tap * g.cCg;
+            c_kh = tap / g.cKW;
+            c_kw = tap - c_kh * g.cKW;
+        }
 
         // `full` (compile time): the whole stage lies inside K, so no lane needs the
         // zero source and the address is a uniform base plus a per-lane offset
@@ -365,8 +380,12 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
             }
             if (CONV) {
                 // this lane's 16 bytes lie inside one filter tap (Cg % 16 == 0)
-                const int tap = k / g.cCg, ci0 = k - tap * g.cCg;
-                const int kh = tap / g.cKW, kw = tap - kh * g.cKW;
+                const int ci0 = c_ci0, kh = c_kh, kw = c_kw;
+                c_ci0 += BK;  // on to the next stage
+                while (c_ci0 >= g.cCg) {
+                    c_ci0 -= g.cCg;
+                    if (++c_kw == g.cKW) c_kw = 0, ++c_kh;
+                }
                 const int dh = kh * g.cdh, dw = kw * g.cdw;
                 const unsigned delta = unsigned(dh * g.cW + dw) * unsigned(g.cCin) + unsigned(ci0);
 #pragma unroll
@@ -638,7 +657,42 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
             __syncthreads();
             // the other contributors have all arrived
             finish = __builtin_amdgcn_readfirstlane(s_flag) == (w_last - w_first);
-            if (finish) {
+            if (finish && TM * TN * 4 <= 8) {
+                // small accumulators (64 x 64 tiles): the slabs of up to kGroup contributors
+                // are requested together, one memory round trip for all of them instead of
+                // one each.  A slot with no contributor re-reads this worker's own slab and
+                // is not added, so that the loads stay unconditional.
+                constexpr int kChunks = TM * TN * 4, kGroup = kChunks <= 8 ? 16 / kChunks : 1;
+                for (int w0 = w_first; w0 <= w_last; w0 += kGroup) {
+                    v4u v[kGroup][kChunks];
+#pragma unroll
+                    for (int x = 0; x < kGroup; ++x) {
+                        const int w = w0 + x;
+                        const bool use = w <= w_last && w != me;
+                        const __amdgpu_buffer_rsrc_t other =
+                            __builtin_amdgcn_make_buffer_rsrc(slab_of(use ? w : me), 0, kSlabBytes, 0x00020000);
+#pragma unroll
+                        for (int c = 0; c < kChunks; ++c)
+                            v[x][c] = __builtin_amdgcn_raw_buffer_load_b128(other, lane_off + unsigned(c * THREADS * 16),
+                                                                            0, kScopeDevice);
+                    }
+#pragma unroll
+                    for (int x = 0; x < kGroup; ++x) {
+                        const int w = w0 + x;
+                        if (w <= w_last && w != me) {
+#pragma unroll
+                            for (int c = 0; c < kChunks; ++c) {
+                                v16i& a = acc[(c / 4) / TN][(c / 4) % TN];
+                                a[4 * (c % 4)] += int(v[x][c].x);
+                                a[4 * (c % 4) + 1] += int(v[x][c].y);
+                                a[4 * (c % 4) + 2] += int(v[x][c].z);
+                                a[4 * (c % 4) + 3] += int(v[x][c].w);
+                            }
+                        }
+                    }
+                }
+                if (tid == 0) counters[local] = 0;  // ready for the next launch
+            } else if (finish) {
                 for (int w = w_first; w <= w_last; ++w) {
                     if (w == me) continue;
                     const __amdgpu_buffer_rsrc_t other =
@@ -688,6 +742,10 @@ using CfgN64 = TileCfg<256, 64, 64, 4, 1, 3, 2>;  // 64 output columns (early Re
 using CfgTall3 = TileCfg<128, 256, 64, 2, 2, 2, 3>;  // three blocks per CU
 using CfgMid4 = TileCfg<128, 128, 64, 2, 2, 2, 4>;   // four blocks per CU: short K, latency-bound tiles
 using CfgSmall = TileCfg<64, 64, 64, 2, 2, 4, 4>;    // few rows (late convolution stages): more tiles than CUs
+// the same tiles over a long K: half the k-iterations (and barriers) at twice the bytes each;
+// measured 27 -> 21 us on a 1568 x 512 x 4608 convolution, where a tile's time is the chain
+// wait - barrier - LDS read - MFMA of each k-iteration with nothing else on the CU to cover it
+using CfgSmallK = TileCfg<64, 64, 128, 2, 2, 4, 2>;
 
 }  // namespace
 

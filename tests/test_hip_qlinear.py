@@ -42,7 +42,7 @@ def test_accumulators_exact(M, N, K, path):
     assert np.array_equal(acc, O.igemm(a, w))
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 260, 144), (129, 77, 784), (513, 1000, 576),
                                    (2048, 512, 4096), (1, 16, 16), (700, 130, 64)])
 def test_every_tile_shape_exact(cfg, M, N, K):
@@ -60,7 +60,7 @@ def test_every_tile_shape_exact(cfg, M, N, K):
     assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
 
 
-@pytest.mark.parametrize("cfg", [1, 3, 4, 5, 6, 8, 9])
+@pytest.mark.parametrize("cfg", [1, 3, 4, 5, 6, 8, 9, 10])
 @pytest.mark.parametrize("M,N,K", [(300, 260, 144), (513, 1000, 576), (2048, 1100, 4096),
                                    (256, 256, 128), (129, 77, 784), (1500, 3000, 1024)])
 def test_stream_k_schedule_exact(cfg, M, N, K):
@@ -312,3 +312,64 @@ def test_column_split_between_two_tile_shapes_exact(M, N, K, a_tiles):
     j1 = _ops.qlinear_i8(da, dw, **common, **jk, path=1, tile_config=tc).numpy()
     j2 = _ops.qlinear_i8(da, dw, **common, **jk, path=1, tile_config=5 | 0x100).numpy()
     assert np.array_equal(j1, j2)
+
+
+@pytest.mark.parametrize("out_scale", [1.0, 0.5, 3.0, 0.1, 7.3e-4, 1e-30, 1e30])
+@pytest.mark.parametrize("relu", [False, True])
+def test_requantize_at_ties_near_ties_and_saturation(out_scale, relu):
+    """The tile kernel's epilogue avoids the division for most elements (a reciprocal multiply
+    with a guard band around the rounding boundaries, the IEEE quotient for the rest).  Power
+    of two scales put a large share of the quotients exactly on half-integers (ties to even),
+    bias values of +-1 ulp put them just off; tiny and huge scales saturate or zero everything
+    and fall outside what the reciprocal route accepts.  Codes must equal the oracle's."""
+    rng = np.random.default_rng(int(out_scale * 1000) % 977 + relu)
+    M, N, K = 384, 256, 64
+    a, w = codes(rng, (M, K), -3, 3), codes(rng, (N, K), -3, 3)
+    a_scale = np.float32(0.5)
+    w_scale = np.full(N, 0.5, np.float32)
+    w_scale[::3] = 0.25
+    # bias: zero, +-tiny (pushes exact ties just off the boundary), and halves
+    bias = rng.choice(np.array([0.0, 1e-7, -1e-7, 0.5, -0.5, 0.125], np.float32), N).astype(np.float32)
+    S, Z = np.float32(out_scale), np.float32(-5.0)
+    for mode in (_ops.OUT_REQUANT_I8, _ops.OUT_FAKEQUANT_F32):
+        got = _ops.qlinear_i8(hip(a), hip(w), a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias),
+                              relu=relu, out_mode=mode, out_scale=hip(S), out_zp=hip(Z), out_qmin=-128,
+                              out_qmax=127, out_offset=0, path=TILE).numpy()
+        exp = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, relu=relu, out_mode=mode, out_scale=S, out_zp=Z,
+                        out_qmin=-128, out_qmax=127, out_offset=0)
+        if mode == _ops.OUT_REQUANT_I8:
+            assert np.array_equal(got, exp)
+            if out_scale in (1.0, 0.5):  # the case is what it claims to be: many exact ties
+                t = (O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, relu=relu, out_mode=O.OUT_F32) / S)
+                assert (np.abs(t - np.floor(t) - 0.5) == 0).mean() > 0.02
+        else:
+            assert np.array_equal(got.view(np.uint32), exp.view(np.uint32))
+
+
+def test_fused_join_at_ties_and_with_odd_grids():
+    """The fused join on codes through the same guard-band route: power-of-two grids make the
+    joined sums land on half-integers; a zero point beyond +-255 switches the route off.  Equal
+    to the stand-alone lq_add_requant_i8 (itself checked against the oracle) bit for bit."""
+    from lucid_amd import _C
+    rng = np.random.default_rng(77)
+    M, N, K = 256, 384, 64
+    a, w = hip(codes(rng, (M, K), -4, 4)), hip(codes(rng, (N, K), -4, 4))
+    for (s1, z1, s2, z2, S, Z) in ((0.5, 0.0, 0.25, 3.0, 1.0, 0.0), (0.5, -3.0, 0.5, 0.0, 2.0, 10.0),
+                                    (0.03, 2.0, 0.025, 131.0, 0.04, 7.0), (0.5, 0.0, 0.5, 0.0, 1.0, 300.0)):
+        common = dict(a_scale=hip(np.float32(0.5)), w_scale=hip(np.full(N, 0.5, np.float32)),
+                      out_mode=_ops.OUT_REQUANT_I8, out_scale=hip(np.float32(s1)), out_zp=hip(np.float32(z1)),
+                      out_qmin=-128, out_qmax=127, out_offset=0, path=TILE)
+        first = _ops.qlinear_i8(a, w, **common)
+        other = hip(codes(rng, (M, N)))
+        s2t, z2t, St, Zt = (hip(np.float32(v)) for v in (s2, z2, S, Z))
+        want = L.Tensor.empty((M, N), L.int8, "hip")
+        _C.call("lq_add_requant_i8", first.data_ptr, 0, common["out_scale"].data_ptr, common["out_zp"].data_ptr,
+                other.data_ptr, -128, s2t.data_ptr, z2t.data_ptr, M * N, 0, St.data_ptr, Zt.data_ptr, 0, 255, -128,
+                want.data_ptr, None)
+        fused = _ops.qlinear_i8(a, w, **common, join=dict(q=other, offset=-128, scale=s2t, zp=z2t, relu=False,
+                                                           out_scale=St, out_zp=Zt, out_qmin=0, out_qmax=255,
+                                                           out_offset=-128))
+        assert np.array_equal(fused.numpy(), want.numpy())
+        exp = O.add_requant(first.numpy(), 0, np.float32(s1), np.float32(z1), other.numpy(), -128, np.float32(s2),
+                            np.float32(z2), False, np.float32(S), np.float32(Z), 0, 255, -128)
+        assert np.array_equal(fused.numpy(), exp.reshape(M, N))
