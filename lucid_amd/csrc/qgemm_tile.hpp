@@ -440,6 +440,60 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 1) * (PA + PB)));
         __syncthreads();
 
+        if constexpr (TM * TN == 1) {
+            // One MFMA per k step cannot cover the LDS latency of the next step's fragments, so
+            // a wavefront holds the fragments of a whole stage: the registers of step kk are
+            // refilled from the next stage right after the MFMA that consumed them, KSTEPS
+            // MFMAs ahead of their use.  Two accumulators (even / odd steps) keep consecutive
+            // MFMAs independent.  The hand-over (wait for the next stage's data, barrier) comes
+            // first in the iteration, the refill of the stage just drained last, its address
+            // arithmetic running beside the MFMAs.
+            v4i fa[KSTEPS], fb[KSTEPS];
+            v16i acc_odd;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc_odd[r] = 0;
+            auto read_step = [&](const int8_t* stage, int kk) {
+                const int pc = ((kk * 2 + frag_half) ^ sw) * 16;
+                fa[kk] = *reinterpret_cast<const v4i*>(stage + a_row_base + pc);
+                fb[kk] = *reinterpret_cast<const v4i*>(stage + b_row_base + pc);
+            };
+#pragma unroll
+            for (int kk = 0; kk < KSTEPS; ++kk) read_step(smem, kk);
+            auto stage_steps = [&](int t, bool last_stage, auto full) {
+                const int slot = t % STAGES;
+                int8_t* cur = smem + slot * Cfg::STAGE_BYTES;
+                const int8_t* nxt = smem + (slot + 1 == STAGES ? 0 : slot + 1) * Cfg::STAGE_BYTES;
+                if (!last_stage) {
+                    // lgkmcnt(0): this wavefront's reads of `cur` have landed in registers, so after
+                    // the barrier nobody still reads the buffer that is refilled below
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * (PA + PB)) & ~(0xF << 8));
+                    __syncthreads();
+                }
+#pragma unroll
+                for (int kk = 0; kk < KSTEPS; ++kk) {
+                    if (kk & 1)
+                        acc_odd = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[kk], fb[kk], acc_odd, 0, 0, 0);
+                    else
+                        acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[kk], fb[kk], acc[0][0], 0, 0, 0);
+                    if (!last_stage) read_step(nxt, kk);
+                }
+                if (!last_stage) load_stage((kb + t + STAGES) * BK, cur, full);
+            };
+            const int n_it = ke - kb;
+            int n_full = (k_end / BK) - kb - STAGES;
+            n_full = n_full < 0 ? 0 : (n_full > n_it - 1 ? n_it - 1 : n_full);
+            int t = 0;
+            for (; t < n_full; ++t) stage_steps(t, false, std::true_type{});
+            for (; t + 1 < n_it; ++t) stage_steps(t, false, std::false_type{});
+            if (ke == nk) fetch_params(tm, tn);
+            stage_steps(n_it - 1, true, std::false_type{});
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[0][0][r] += acc_odd[r];
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the zero-filled look-ahead stages
+            __syncthreads();                            // all fragment reads done before LDS is reused
+            return;
+        }
+
         v4i af[2][TM], bf[2][TN];
         if (Cfg::PIPE) read_frags(smem, 0, af[0], bf[0]);
 
