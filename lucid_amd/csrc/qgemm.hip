@@ -477,7 +477,50 @@ int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t 
 
 }  // namespace lq
 
+namespace {
+
+// x = every float32 bit pattern of [first, first + count): the tile epilogue's requantize
+// (quant_fast: reciprocal multiply with a guard band, division for the rest) against the plain
+// divide-round-add-clamp, compared as the codes the two would store.
+__global__ __launch_bounds__(256) void quant_route_check_kernel(float s, float z, float lo, float hi,
+                                                                unsigned long long first,
+                                                                unsigned long long count,
+                                                                unsigned long long* mismatches,
+                                                                unsigned long long* divided) {
+    const lq::QGrid G = lq::make_qgrid(s, z, lo, hi, true);
+    unsigned long long bad = 0, slow = 0;
+    for (unsigned long long i = blockIdx.x * 256ull + threadIdx.x; i < count; i += gridDim.x * 256ull) {
+        const float x = __uint_as_float(unsigned(first + i));
+        const float fast = lq::quant_fast<false>(x, G);
+        const float u = lq::q_core(x, s, z, lo, hi);
+        const float plain = (u != u) ? 0.0f : u;
+        bad += __float_as_uint(fast) != __float_as_uint(plain) && !(fast == 0.0f && plain == 0.0f);
+        const float tp = x * G.inv;
+        slow += !(__builtin_fabsf(tp - __builtin_rintf(tp)) < 0.5f - 0x1p-12f);
+    }
+    if (bad) atomicAdd(mismatches, bad);
+    if (slow) atomicAdd(divided, slow);
+}
+
+}  // namespace
+
 extern "C" {
+
+int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, unsigned long long first_bits,
+                              unsigned long long count, unsigned long long* mismatches,
+                              unsigned long long* divided, lq_stream stream) {
+    LQ_REQUIRE(mismatches && divided, LQ_ERR_VALUE, "selftest_requant_route: NULL counter");
+    LQ_REQUIRE(first_bits + count <= (1ull << 32), LQ_ERR_VALUE, "selftest_requant_route: range beyond 2^32");
+    hipStream_t st = as_stream(stream);
+    int rc = lq_fill_bytes(mismatches, 0, sizeof(unsigned long long), stream);
+    if (rc == LQ_OK) rc = lq_fill_bytes(divided, 0, sizeof(unsigned long long), stream);
+    if (rc) return rc;
+    if (count == 0) return LQ_OK;
+    hipLaunchKernelGGL(quant_route_check_kernel, dim3(4096), dim3(256), 0, st, scale, zp, float(qmin), float(qmax),
+                       first_bits, count, mismatches, divided);
+    LQ_CHECK_LAUNCH("selftest_requant_route");
+    return LQ_OK;
+}
 
 int lq_last_tile_config(void) { return t_last_tile_config; }
 
