@@ -279,8 +279,9 @@ int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, h
 
 // ---------------------------------------------------------------- skinny kernel
 // M <= 16*MT.  A block owns 16 weight rows; its 4 wavefronts each take a
-// quarter of K.  Lane (n = lane&15, g = lane>>4) reads 64 contiguous bytes of
-// weight row n per 256-byte K block; the activation operand uses the same
+// quarter of K.  In load c of a 256-byte K block, lane (n = lane&15, g = lane>>4) reads
+// bytes [64c + 16g, 64c + 16g + 16) of weight row n, so the four lanes of a row fetch one
+// whole 64-byte segment per instruction; the activation operand uses the same
 // byte -> k mapping, so the dot products are unchanged.
 template <int MT>
 __global__ __launch_bounds__(256) void qgemm_skinny_kernel(GemmArgs g) {
@@ -309,10 +310,10 @@ __global__ __launch_bounds__(256) void qgemm_skinny_kernel(GemmArgs g) {
         v4i wf[PF][4];
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
-            const int kbase = (kbc + u) * 256 + lg * 64;
+            const int kbase = (kbc + u) * 256 + lg * 16;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                const int k = kbase + c * 16;
+                const int k = kbase + c * 64;
                 wf[u][c] = (kbc + u < kb1 && k < g.K) ? *reinterpret_cast<const v4i*>(wrow + k)
                                                      : v4i{0, 0, 0, 0};
             }
@@ -320,14 +321,14 @@ __global__ __launch_bounds__(256) void qgemm_skinny_kernel(GemmArgs g) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
             if (kbc + u >= kb1) break;
-            const int kbase = (kbc + u) * 256 + lg * 64;
+            const int kbase = (kbc + u) * 256 + lg * 16;
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 const int m = t * 16 + ln;
                 const int8_t* arow = g.a + size_t(m < g.M ? m : g.M - 1) * g.K;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    const int k = kbase + c * 16;
+                    const int k = kbase + c * 64;
                     v4i af = (k < g.K && m < g.M) ? *reinterpret_cast<const v4i*>(arow + k)
                                                   : v4i{0, 0, 0, 0};
                     acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf[u][c], acc[t], 0, 0, 0);
