@@ -322,6 +322,75 @@ __global__ __launch_bounds__(256) void qlinear_w8a32_patch_kernel(
         }
 }
 
+// Long K: the block's four wavefronts share one 4-column x 8-row patch and take every fourth
+// 256-wide k step each (four times the loads in flight per output); partial sums meet in
+// LDS, then each wavefront folds and stores eight of the 32 outputs.
+__global__ __launch_bounds__(256) void qlinear_w8a32_patch_k4_kernel(
+    const float* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ w_scale,
+    const float* __restrict__ w_zp, const float* __restrict__ bias, int M, int N, int K, int relu,
+    int do_fq, const float* S_, const float* Z_, float lo, float hi, float* __restrict__ out) {
+    constexpr int NT = 4, MT = 8;
+    __shared__ float red[4][MT * NT][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * NT, m0 = blockIdx.y * MT;
+    float ws[NT], wz[NT];
+    const int8_t* wr[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int n = n0 + j < N ? n0 + j : N - 1;  // clamped columns are computed and dropped
+        ws[j] = w_scale[n], wz[j] = w_zp[n], wr[j] = w + size_t(n) * K;
+    }
+    const float* xr[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xr[i] = x + size_t(m0 + i < M ? m0 + i : M - 1) * K;
+    float acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = 0.0f;
+    for (int k = wave * 256 + lane * 4; k < K; k += 1024) {
+        float wv[NT][4];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const uint32_t c = *reinterpret_cast<const uint32_t*>(wr[j] + k);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                wv[j][e] = (float(int(int8_t((c >> (8 * e)) & 0xff))) - wz[j]) * ws[j];  // dequantize, _functional.py:281
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const float4 xv = *reinterpret_cast<const float4*>(xr[i] + k);
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                float a = acc[i][j];
+                a = a + xv.x * wv[j][0];
+                a = a + xv.y * wv[j][1];
+                a = a + xv.z * wv[j][2];
+                a = a + xv.w * wv[j][3];
+                acc[i][j] = a;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) red[wave][i * NT + j][lane] = acc[i][j];
+    __syncthreads();
+    const float S = do_fq ? S_[0] : 1.0f, Z = do_fq ? Z_[0] : 0.0f;
+#pragma unroll
+    for (int o = 0; o < 8; ++o) {
+        const int idx = wave * 8 + o, i = idx / NT, j = idx % NT;
+        float y = ((red[0][idx][lane] + red[1][idx][lane]) + red[2][idx][lane]) + red[3][idx][lane];
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) y = y + __shfl_xor(y, d, 64);
+        if (lane != 0 || m0 + i >= M || n0 + j >= N) continue;
+        if (bias) y = y + bias[n0 + j];
+        if (relu) y = (y < 0.0f) ? 0.0f : y;
+        if (do_fq) y = (q_core(y, S, Z, lo, hi) - Z) * S;
+        out[size_t(m0 + i) * N + n0 + j] = y;
+    }
+}
+
 inline unsigned grid_for(size_t n, size_t per_block) {
     size_t b = (n + per_block - 1) / per_block;
     if (b < 1) b = 1;
@@ -477,7 +546,17 @@ int lq_qlinear_w8a32(const float* x, const int8_t* w, const float* w_scale, cons
                "qlinear_w8a32: output qparams missing");
     const size_t outputs = size_t(M) * N;
     LQ_REQUIRE((outputs + 3) / 4 <= 0x7fffffffull, LQ_ERR_SHAPE, "qlinear_w8a32: too many outputs");
-    if (M >= 4 && K % 4 == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(w) & 3u) == 0 && (M + 7) / 8 <= 65535) {
+    const bool patch_ok = M >= 4 && K % 4 == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(w) & 3u) == 0 &&
+                          (M + 7) / 8 <= 65535;
+    // few patches and a long K: one patch per block, K split between its wavefronts
+    if (patch_ok && K >= 1024 && size_t((N + 3) / 4) * size_t((M + 7) / 8) <= 4096) {
+        hipLaunchKernelGGL(qlinear_w8a32_patch_k4_kernel, dim3(unsigned((N + 3) / 4), unsigned((M + 7) / 8)), dim3(256),
+                           0, as_stream(stream), x, w, w_scale, w_zp, bias, M, N, K, relu, fake_quantize_out,
+                           out_scale, out_zp, float(out_qmin), float(out_qmax), out);
+        LQ_CHECK_LAUNCH("qlinear_w8a32");
+        return LQ_OK;
+    }
+    if (patch_ok) {
         hipLaunchKernelGGL(qlinear_w8a32_patch_kernel, dim3(unsigned((N + 15) / 16), unsigned((M + 7) / 8)), dim3(256),
                            0, as_stream(stream), x, w, w_scale, w_zp, bias, M, N, K, relu, fake_quantize_out,
                            out_scale, out_zp, float(out_qmin), float(out_qmax), out);
