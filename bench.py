@@ -137,7 +137,8 @@ def bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup, seed=1):
             # the leading NA rows of the weight are a contiguous prefix, so the prefix of the
             # scale / bias arrays and a narrower output describe exactly region A
             _ops.qlinear_i8(t["xq"], t["wq_head"], a_scale=t["xs"], w_scale=t["ws_head"], bias=t["bias_head"],
-                            out_mode=_ops.OUT_F16, out=sub, repeat=repeat, path=1, tile_config=1 | 0x100)
+                            out_mode=_ops.OUT_F16, out=sub, repeat=repeat, path=1,
+                            tile_config=(tile_config & 0xff) | 0x100)
 
         t["wq_head"] = t["wq"].narrow_rows(NA)
         t["ws_head"], t["bias_head"] = t["ws"].narrow_rows(NA), t["bias"].narrow_rows(NA)

@@ -453,12 +453,12 @@ typedef struct {
     void* out;             /* [M, ldo] in the type out_mode implies          */
     long ldo;              /* output row stride in elements; 0 means N       */
     int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
-    int tile_config;       /* tuning: low byte 0 = choose, 1..10 = a tile shape;
+    int tile_config;       /* tuning: low byte 0 = choose, 1..12 = a tile shape;
                               next byte 0 = choose, 1 = one block per tile,
                               2 = stream-K work split, 3 = stream-K over the
                               leftover tiles of the last round only; bits 16..30
                               = number of leading 256-column tiles computed with
-                              shape 1, the remaining columns as a problem of
+                              256x256 tiles, the remaining columns as a problem of
                               their own (0 = no split)                          */
     const float* residual; /* optional float32 [M, ldr] added after the activation:
                               out = act(y) + residual (x + linear(...), the

@@ -71,6 +71,8 @@ int launch_tile_c7(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c8(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c9(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c10(const GemmArgs&, bool, int, int, hipStream_t);
+int launch_tile_c11(const GemmArgs&, bool, int, int, hipStream_t);
+int launch_tile_c12(const GemmArgs&, bool, int, int, hipStream_t);
 }  // namespace lq
 
 namespace {
@@ -87,6 +89,8 @@ int launch_tile_shape(const GemmArgs& g, bool conv, int groups, int cfg, int sch
     case 8: return launch_tile_c8(g, conv, groups, schedule, st);
     case 9: return launch_tile_c9(g, conv, groups, schedule, st);
     case 10: return launch_tile_c10(g, conv, groups, schedule, st);
+    case 11: return launch_tile_c11(g, conv, groups, schedule, st);
+    case 12: return launch_tile_c12(g, conv, groups, schedule, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -104,6 +108,8 @@ int heuristic_tile_shape(const GemmArgs& g, int groups) {
 int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st);
 thread_local int t_last_tile_config = 0;  // what the last tile-kernel launch of this thread resolved to
 
+constexpr int kSplitShape = 11;  // 256 x 256 x 128 tiles, eight wavefronts
+
 // Two regions of one GEMM: the first a_tiles * 256 output columns go to the 256 x 256 shape
 // (chosen so that its tiles fill whole rounds of the 256 CUs, one block each), the remaining
 // columns are a problem of their own with whatever shape suits it.  The 256 x 256 shape has
@@ -114,7 +120,7 @@ int launch_split(const GemmArgs& g, int a_tiles, hipStream_t st) {
     if (NA <= 0 || NA >= g.N) return fail(LQ_ERR_VALUE, "tile split: %ld columns of %d", NA, g.N);
     GemmArgs ga = g;
     ga.N = int(NA);
-    int rc = launch_tile_shape(ga, false, 1, 1, 1, st);
+    int rc = launch_tile_shape(ga, false, 1, kSplitShape, 1, st);
     if (rc) return rc;
     GemmArgs gb = g;
     gb.N = g.N - int(NA);
@@ -191,7 +197,8 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     cands[n++] = 5;
     if (g.K <= 256) cands[n++] = 8;  // one to four k-iterations: latency-bound tiles, four blocks per CU
     if (g.N > 64) cands[n++] = 3, cands[n++] = 4;
-    if (g.N > 128 && g.M > 128) cands[n++] = 1;
+    if (g.N > 128 && g.M > 128) cands[n++] = 1, cands[n++] = 11;
+    if (g.N > 128 && !conv) cands[n++] = 12;
     // a long K over few tiles (late convolution stages): split K between the idle CUs
     const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
     if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
@@ -202,7 +209,8 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
         const long tiles_m = (g.M + 255) / 256, tiles_n = g.N / 256;
         const long rounds = tiles_m * tiles_n / 256;
         const long a_tiles = rounds > 0 ? rounds * 256 / tiles_m : 0;
-        if (a_tiles > 0 && a_tiles * 256 < g.N && a_tiles < 32768) cands[n++] = 1 | (1 << 8) | int(a_tiles << 16);
+        if (a_tiles > 0 && a_tiles * 256 < g.N && a_tiles < 32768)
+            cands[n++] = kSplitShape | (1 << 8) | int(a_tiles << 16);
     }
     hipEvent_t e0, e1;
     LQ_HIP(hipEventCreate(&e0));
@@ -270,7 +278,7 @@ int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, h
         LQ_REQUIRE(!conv && groups == 1 && g.range == nullptr, LQ_ERR_VALUE,
                    "tile_config: a column split needs a plain GEMM without a kept range");
         const int rc = launch_split(g, a_tiles, st);
-        t_last_tile_config = 1 | (1 << 8) | (a_tiles << 16);
+        t_last_tile_config = kSplitShape | (1 << 8) | (a_tiles << 16);
         return rc;
     }
     t_last_tile_config = cfg | ((schedule ? schedule : 1) << 8);

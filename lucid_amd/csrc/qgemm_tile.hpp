@@ -536,6 +536,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
                     for (int j = 0; j < TN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[kk & 1][i], bf[kk & 1][j],
                                                                           acc[i][j], 0, 0, 0);
+
                 // issue order inside the step: one MFMA, then all LDS reads of the next
                 // step's fragments, then the other MFMAs.  The compiler waits for every
                 // outstanding LDS read before the first MFMA of a step, so the reads go
@@ -800,6 +801,14 @@ using CfgSmall = TileCfg<64, 64, 64, 2, 2, 4, 4>;    // few rows (late convoluti
 // measured 27 -> 21 us on a 1568 x 512 x 4608 convolution, where a tile's time is the chain
 // wait - barrier - LDS read - MFMA of each k-iteration with nothing else on the CU to cover it
 using CfgSmallK = TileCfg<64, 64, 128, 2, 2, 4, 2>;
+// Eight wavefronts (two per SIMD, wavefront tiles of 128 x 64 and 64 x 64): one wavefront's
+// barrier waits and LDS reads are covered by the other's MFMAs.  Measured against the
+// four-wavefront shapes of the same block tile: 256 x 256 x 128 +4 % (2.34 against 2.26 POP/s
+// at 8192 x 8192 x 4096), 128 x 256 x 64 +4 % on a 2816-column problem but -7 % on large ones.
+// (A 4 x 2 wavefront grid gained half as much; raising the wavefront priority around the MFMAs
+// lost 8 %; BK = 64 with four stages lost 7 %.)
+using CfgBig8 = TileCfg<256, 256, 128, 2, 4, 2, 1>;
+using CfgTall8 = TileCfg<128, 256, 64, 2, 4, 3, 2>;
 
 }  // namespace
 

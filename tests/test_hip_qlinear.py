@@ -42,7 +42,7 @@ def test_accumulators_exact(M, N, K, path):
     assert np.array_equal(acc, O.igemm(a, w))
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 260, 144), (129, 77, 784), (513, 1000, 576),
                                    (2048, 512, 4096), (1, 16, 16), (700, 130, 64)])
 def test_every_tile_shape_exact(cfg, M, N, K):
@@ -60,7 +60,7 @@ def test_every_tile_shape_exact(cfg, M, N, K):
     assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
 
 
-@pytest.mark.parametrize("cfg", [1, 3, 4, 5, 6, 8, 9, 10])
+@pytest.mark.parametrize("cfg", [1, 3, 4, 5, 6, 8, 9, 10, 11, 12])
 @pytest.mark.parametrize("M,N,K", [(300, 260, 144), (513, 1000, 576), (2048, 1100, 4096),
                                    (256, 256, 128), (129, 77, 784), (1500, 3000, 1024)])
 def test_stream_k_schedule_exact(cfg, M, N, K):
