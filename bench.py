@@ -46,7 +46,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X published HBM3E bandwidth, GB/s
 MEASURED_TRAFFIC_BYTES = {
     # one 128x256-tiled launch / the column split (256x256 tiles over 8192 columns + 128x256 over 2816)
     "linear_m2048": int((2.0 * 96504 + 44032) * 1024),
-    "linear_m2048_split": int((2.0 * (49458.5 + 30888.25) + 32768 + 11264) * 1024),
+    "linear_m2048_split": int((2.0 * (49357.0 + 30884.2) + 32768 + 11264) * 1024),
     "quantize_per_channel_i8": int((2.0 * 524577 + 262144) * 1024),
     "dequantize_per_channel_i8": int((2.0 * 131350 + 1048712) * 1024),
     "minmax_per_channel": int((2.0 * 524317 + 257) * 1024),

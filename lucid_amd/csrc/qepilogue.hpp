@@ -146,7 +146,7 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
     if (MODE == OUT_F32X) {
         // GELU, erf form (lucid/nn/functional/activations.py:219): the expression of the
         // stand-alone kernel, so fusing it changes no bit
-        if (g.gelu) y = (0.5f * y) * (1.0f + erff(y * 0.70710678118654752440f));
+        if (g.gelu) y = (0.5f * y) * (1.0f + erf_as(y * 0.70710678118654752440f));
         return __float_as_uint(y);
     }
     if (MODE == OUT_REQUANT_JOIN) return __float_as_uint(quant_fast<false>(y, G));

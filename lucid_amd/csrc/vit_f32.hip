@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
 
 // ---------------------------------------------------------------- elementwise
 __device__ __forceinline__ float gelu_erf(float x) {
-    return (0.5f * x) * (1.0f + erff(x * 0.70710678118654752440f));
+    return (0.5f * x) * (1.0f + lq::erf_as(x * 0.70710678118654752440f));
 }
 
 // Four float4 per thread (block-strided, so each access of a wavefront is
