@@ -298,6 +298,19 @@ int lq_wq_matmul(const float* x, const uint32_t* packed, const float* scales, co
 int lq_bias_act_f32(float* y, const float* bias, size_t M, int N, int relu, lq_stream stream);
 
 /* ------------------------------------------------- ranges kept by the producer */
+/* Dynamic per-row quantization in one pass: for every row of x [rows, cols],
+ * min / max of the row (PerChannelMinMaxObserver with ch_axis = 0,
+ * observer.py:634-653), its qparams (calculate_qparams, _qparams.py:198-215) and
+ * its int8 codes (quantize, _functional.py:164-182) - the results of lq_minmax +
+ * lq_calc_qparams + lq_quantize bit for bit, with x read once.  This is the
+ * per-token activation quantization in front of an LLM-shaped Linear.  scale,
+ * zp: [rows] out; mn_out, mx_out: optional [rows] out.  cols must be a multiple
+ * of 4, at most 16384, x 16-byte aligned (LQ_ERR_NOT_IMPLEMENTED otherwise: use
+ * the three calls). */
+int lq_quantize_rows_dynamic_i8(const float* x, size_t rows, size_t cols, int symmetric, int qmin, int qmax,
+                                int is_signed, float eps, int code_offset, float* scale, float* zp,
+                                float* mn_out, float* mx_out, int8_t* q, lq_stream stream);
+
 /* nnqd.Linear takes x.min() / x.max() of its input on every forward
  * (lucid/nn/quantized/dynamic/linear.py:87-89): a full pass over a tensor some
  * kernel has just written.  The float32 kernels below can keep that range as a

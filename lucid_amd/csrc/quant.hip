@@ -528,9 +528,83 @@ __global__ __launch_bounds__(1024) void calc_qparams_from_range_kernel(const flo
     }
 }
 
+// Dynamic per-row quantization in one pass over x: a block holds one row in registers, takes
+// its min / max (observer.py:634-653 with ch_axis = 0), turns them into the row's qparams
+// (qparams_of) and writes the row's codes with QuantizeOp's arithmetic - the three separate
+// launches' results, bit for bit, with x read once instead of twice.
+template <int R>  // float4 per lane: rows of up to 1024 * R floats
+__global__ __launch_bounds__(256) void quantize_rows_dynamic_kernel(
+    const float4* __restrict__ x, int quads, int symmetric, int qmin, int qmax, int is_signed, float eps,
+    float half_range, int off, float* __restrict__ scale, float* __restrict__ zp, float* __restrict__ mn_out,
+    float* __restrict__ mx_out, Code8x4* __restrict__ q) {
+    __shared__ float s_sz[2];
+    const size_t row = blockIdx.x;
+    const float4* xr = x + row * size_t(quads);
+    float4 v[R];
+    MinMax m{__builtin_inff(), -__builtin_inff(), 0};
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int i = u * 256 + int(threadIdx.x);
+        if (i < quads) {
+            v[u] = nt_load(&xr[i]);
+            mm_update(m, v[u].x), mm_update(m, v[u].y), mm_update(m, v[u].z), mm_update(m, v[u].w);
+        }
+    }
+    m = mm_block_reduce(m);
+    if (threadIdx.x == 0) {
+        const float qnan = __builtin_nanf("");
+        const float mn = m.nan ? qnan : m.lo, mx = m.nan ? qnan : m.hi;
+        float s, z;
+        qparams_of(mn, mx, symmetric, qmin, qmax, is_signed, eps, half_range, &s, &z);
+        scale[row] = s, zp[row] = z;
+        if (mn_out) mn_out[row] = mn;
+        if (mx_out) mx_out[row] = mx;
+        s_sz[0] = s, s_sz[1] = z;
+    }
+    __syncthreads();
+    const float s = s_sz[0], z = s_sz[1], r = 1.0f / s;
+    const QuantizeOp<int8_t> op{nullptr, nullptr, float(double(qmin)), float(double(qmax)), off};
+    Code8x4* qr = q + row * size_t(quads);
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int i = u * 256 + int(threadIdx.x);
+        if (i < quads) nt_store(&qr[i], op.pack(v[u], s, z, r));
+    }
+}
+
 }  // namespace
 
 extern "C" {
+
+int lq_quantize_rows_dynamic_i8(const float* x, size_t rows, size_t cols, int symmetric, int qmin, int qmax,
+                                int is_signed, float eps, int code_offset, float* scale, float* zp,
+                                float* mn_out, float* mx_out, int8_t* q, lq_stream stream) {
+    if (rows == 0) return LQ_OK;
+    LQ_REQUIRE(x && q && scale && zp, LQ_ERR_VALUE, "quantize_rows_dynamic: NULL pointer");
+    LQ_REQUIRE(qmax > qmin && qmin + code_offset >= -128 && qmax + code_offset <= 127, LQ_ERR_VALUE,
+               "quantize_rows_dynamic: grid [%d,%d] + offset %d does not fit int8", qmin, qmax, code_offset);
+    LQ_REQUIRE(cols >= 4 && cols % 4 == 0 && cols <= 16384 && aligned16(x) &&
+                   (reinterpret_cast<uintptr_t>(q) & 3u) == 0 && rows <= 0x7fffffffull,
+               LQ_ERR_NOT_IMPLEMENTED,
+               "quantize_rows_dynamic: rows of %zu floats (a multiple of 4, at most 16384, 16-byte aligned) "
+               "are what the one-pass kernel takes; use lq_minmax + lq_calc_qparams + lq_quantize", cols);
+    const float half_range = float((double(qmax) - double(qmin)) / 2.0);
+    const int quads = int(cols / 4);
+    hipStream_t st = as_stream(stream);
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    Code8x4* q4 = reinterpret_cast<Code8x4*>(q);
+#define LQ_ROWS_DYN(R)                                                                                      \
+    hipLaunchKernelGGL(quantize_rows_dynamic_kernel<R>, dim3(unsigned(rows)), dim3(256), 0, st, x4, quads,  \
+                       symmetric, qmin, qmax, is_signed, eps, half_range, code_offset, scale, zp, mn_out,   \
+                       mx_out, q4)
+    if (quads <= 256) LQ_ROWS_DYN(1);
+    else if (quads <= 1024) LQ_ROWS_DYN(4);
+    else if (quads <= 2048) LQ_ROWS_DYN(8);
+    else LQ_ROWS_DYN(16);
+#undef LQ_ROWS_DYN
+    LQ_CHECK_LAUNCH("quantize_rows_dynamic");
+    return LQ_OK;
+}
 
 int lq_minmax(const float* x, size_t outer, size_t C, size_t inner, float* mn, float* mx,
               lq_stream stream) {

@@ -3,7 +3,7 @@
 Names and signatures follow ``lucid/quantization/__init__.py:67-118``.
 """
 
-from ._functional import dequantize, fake_quantize, minmax, quantize
+from ._functional import dequantize, fake_quantize, minmax, quantize, quantize_rows_dynamic
 from ._qparams import QParams, calculate_qparams
 from ._qscheme import (
     QDtype,
@@ -41,5 +41,5 @@ __all__ = [
     "QConfig", "get_default_qconfig", "prepare", "convert", "quantize_dynamic", "fuse_modules",
     "QScheme", "per_tensor_affine", "per_tensor_symmetric", "per_channel_affine",
     "per_channel_symmetric", "QDtype", "qint8", "quint8", "qint32", "qint4", "QParams",
-    "calculate_qparams", "quantize", "dequantize", "fake_quantize", "minmax",
+    "calculate_qparams", "quantize", "dequantize", "fake_quantize", "minmax", "quantize_rows_dynamic",
 ]

@@ -128,6 +128,37 @@ def fake_quantize(x: Tensor, scale, zero_point, quant_min: int, quant_max: int,
     return out
 
 
+def quantize_rows_dynamic(x: Tensor, qscheme, qdtype: QDtype, eps: float = 1e-8
+                          ) -> tuple[Tensor, Tensor, Tensor]:
+    """Per-row ("per-token") dynamic quantization of a 2-d float32 tensor in one pass:
+    ``(codes, scale, zero_point)`` equal, bit for bit, to
+
+        mn, mx = minmax(x, ch_axis=0)
+        scale, zero_point = calculate_qparams(mn, mx, qscheme, qdtype, eps)
+        codes = quantize(x, scale, zero_point, qdtype, ch_axis=0)
+
+    (``observer.py:634-653``, ``_qparams.py:198-215``, ``_functional.py:164-182``) with ``x``
+    read once.  Rows the one-pass kernel does not take (longer than 16384, not a multiple
+    of 4, int16 storage) go through those three calls."""
+    from ._qparams import calculate_qparams
+    _require_hip(x, "quantize_rows_dynamic")
+    if x.dtype != T.float32 or x.ndim != 2:
+        raise _C.DtypeMismatch(f"quantize_rows_dynamic expects a 2-d float32 tensor, got {x.dtype} {x.shape}")
+    rows, cols = x.shape
+    storage = T.as_dtype(qdtype.storage)
+    if storage == T.int8 and cols % 4 == 0 and 4 <= cols <= 16384 and x.data_ptr % 16 == 0:
+        q = Tensor.empty(x.shape, T.int8, "hip")
+        scale = Tensor.empty((rows,), T.float32, "hip")
+        zp = Tensor.empty((rows,), T.float32, "hip")
+        _C.call("lq_quantize_rows_dynamic_i8", x.data_ptr, rows, cols, int(qscheme.is_symmetric),
+                qdtype.quant_min, qdtype.quant_max, int(qdtype.signed), float(eps), 0, scale.data_ptr,
+                zp.data_ptr, None, None, q.data_ptr, None)
+        return q, scale, zp
+    mn, mx = minmax(x, ch_axis=0)
+    scale, zp = calculate_qparams(mn, mx, qscheme, qdtype, eps)
+    return quantize(x, scale, zp, qdtype, ch_axis=0), scale, zp
+
+
 def minmax(x: Tensor, ch_axis: int | None = None) -> tuple[Tensor, Tensor]:
     """Min and max of ``x`` in one pass: global (0-d results) or per channel
     along ``ch_axis`` (length-C results).  NaN-propagating, as Lucid's

@@ -310,3 +310,37 @@ def _slice_to_host(t, sl, np_dtype):
     out = np.empty(sl.stop - sl.start, np_dtype)
     _C.call("lq_d2h", out.ctypes.data, t.data_ptr + sl.start * out.itemsize, out.nbytes, None)
     return out
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 4), (7, 784), (64, 1024), (33, 4096), (5, 16384), (3, 4100), (2, 20000)])
+@pytest.mark.parametrize("scheme", ["sym_i8", "affine_u8", "affine_i8"])
+def test_quantize_rows_dynamic_equals_the_three_calls_and_the_oracle(rows, cols, scheme):
+    """One pass per row (min / max -> qparams -> codes) against minmax + calculate_qparams +
+    quantize on the device and against the oracle; rows with outliers, constant rows, a NaN row."""
+    import oracle as O
+    rng = np.random.default_rng(rows * 31 + cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    x[rng.random((rows, cols)) < 0.001] *= 20
+    if rows > 2:
+        x[1] = 0.25          # a constant row
+        x[2, cols // 2] = np.nan
+    qscheme, qdtype = {"sym_i8": (Q.per_channel_symmetric, Q.qint8), "affine_u8": (Q.per_channel_affine, Q.quint8),
+                       "affine_i8": (Q.per_channel_affine, Q.qint8)}[scheme]
+    xt = L.tensor(x, device="hip")
+    if qdtype is Q.quint8:   # int16 storage: the wrapper takes the three-call route
+        q, s, z = Q.quantize_rows_dynamic(xt, qscheme, qdtype)
+    else:
+        q, s, z = Q.quantize_rows_dynamic(xt, qscheme, qdtype)
+    mn, mx = Q.minmax(xt, ch_axis=0)
+    s3, z3 = Q.calculate_qparams(mn, mx, qscheme, qdtype)
+    q3 = Q.quantize(xt, s3, z3, qdtype, ch_axis=0)
+    assert np.array_equal(s.numpy().view(np.uint32), s3.numpy().view(np.uint32))
+    assert np.array_equal(z.numpy().view(np.uint32), z3.numpy().view(np.uint32))
+    assert np.array_equal(q.numpy(), q3.numpy())
+    omn, omx = O.minmax(x, ch_axis=0)
+    os_, oz = O.calc_qparams(omn, omx, qscheme.is_symmetric, qdtype.quant_min, qdtype.quant_max, qdtype.signed)
+    ok = ~np.isnan(os_)
+    assert np.array_equal(s.numpy()[ok].view(np.uint32), os_[ok].view(np.uint32))
+    oq = O.quantize(x, os_, oz, qdtype.quant_min, qdtype.quant_max, ch_axis=0,
+                    q_dtype=O.I8 if qdtype.storage == "int8" else O.I16)
+    assert np.array_equal(q.numpy()[ok], oq[ok])
