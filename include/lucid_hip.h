@@ -298,6 +298,17 @@ int lq_wq_matmul(const float* x, const uint32_t* packed, const float* scales, co
 int lq_bias_act_f32(float* y, const float* bias, size_t M, int N, int relu, lq_stream stream);
 
 /* ------------------------------------------------- ranges kept by the producer */
+/* Dynamic per-tensor quantization of a small tensor (n <= 262144) in one launch:
+ * global min / max (MinMaxObserver, observer.py:363-375; x.min() / x.max() in
+ * nnqd.Linear, dynamic/linear.py:87-89), calculate_qparams (_qparams.py:198-215)
+ * and quantize (_functional.py:164-182) - the results of lq_minmax +
+ * lq_calc_qparams + lq_quantize bit for bit.  scale, zp: one float each (device);
+ * mn_out, mx_out optional.  Larger tensors: LQ_ERR_NOT_IMPLEMENTED (use the
+ * three calls, which are bandwidth-bound there). */
+int lq_quantize_tensor_dynamic_i8(const float* x, size_t n, int symmetric, int qmin, int qmax, int is_signed,
+                                  float eps, int code_offset, float* scale, float* zp, float* mn_out,
+                                  float* mx_out, int8_t* q, lq_stream stream);
+
 /* Dynamic per-row quantization in one pass: for every row of x [rows, cols],
  * min / max of the row (PerChannelMinMaxObserver with ch_axis = 0,
  * observer.py:634-653), its qparams (calculate_qparams, _qparams.py:198-215) and

@@ -572,9 +572,59 @@ __global__ __launch_bounds__(256) void quantize_rows_dynamic_kernel(
     }
 }
 
+// Dynamic per-tensor quantization of a small tensor in one launch (one block): global
+// min / max (observer.py:363-375), qparams, codes.  The second read of x comes from the L2.
+__global__ __launch_bounds__(1024) void quantize_tensor_dynamic_kernel(
+    const float* __restrict__ x, size_t n, int symmetric, int qmin, int qmax, int is_signed, float eps,
+    float half_range, int off, float* __restrict__ scale, float* __restrict__ zp, float* __restrict__ mn_out,
+    float* __restrict__ mx_out, int8_t* __restrict__ q) {
+    __shared__ float s_sz[2];
+    const bool vec = aligned16(x) && (reinterpret_cast<uintptr_t>(q) & 3u) == 0;
+    const size_t quads = vec ? n / 4 : 0;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    MinMax m{__builtin_inff(), -__builtin_inff(), 0};
+    for (size_t i = threadIdx.x; i < quads; i += 1024) {
+        const float4 v = x4[i];
+        mm_update(m, v.x), mm_update(m, v.y), mm_update(m, v.z), mm_update(m, v.w);
+    }
+    for (size_t e = quads * 4 + threadIdx.x; e < n; e += 1024) mm_update(m, x[e]);
+    m = mm_block_reduce(m);
+    if (threadIdx.x == 0) {
+        const float qnan = __builtin_nanf("");
+        const float mn = m.nan ? qnan : m.lo, mx = m.nan ? qnan : m.hi;
+        float s, z;
+        qparams_of(mn, mx, symmetric, qmin, qmax, is_signed, eps, half_range, &s, &z);
+        *scale = s, *zp = z;
+        if (mn_out) *mn_out = mn;
+        if (mx_out) *mx_out = mx;
+        s_sz[0] = s, s_sz[1] = z;
+    }
+    __syncthreads();
+    const float s = s_sz[0], z = s_sz[1], r = 1.0f / s;
+    const QuantizeOp<int8_t> op{x4, reinterpret_cast<Code8x4*>(q), float(double(qmin)), float(double(qmax)), off};
+    for (size_t i = threadIdx.x; i < quads; i += 1024) op.q[i] = op.pack(x4[i], s, z, r);
+    for (size_t e = quads * 4 + threadIdx.x; e < n; e += 1024) op.scalar(e, s, z);
+}
+
 }  // namespace
 
 extern "C" {
+
+int lq_quantize_tensor_dynamic_i8(const float* x, size_t n, int symmetric, int qmin, int qmax, int is_signed,
+                                  float eps, int code_offset, float* scale, float* zp, float* mn_out,
+                                  float* mx_out, int8_t* q, lq_stream stream) {
+    LQ_REQUIRE(scale && zp && (n == 0 || (x && q)), LQ_ERR_VALUE, "quantize_tensor_dynamic: NULL pointer");
+    LQ_REQUIRE(qmax > qmin && qmin + code_offset >= -128 && qmax + code_offset <= 127, LQ_ERR_VALUE,
+               "quantize_tensor_dynamic: grid [%d,%d] + offset %d does not fit int8", qmin, qmax, code_offset);
+    LQ_REQUIRE(n <= (size_t(1) << 18), LQ_ERR_NOT_IMPLEMENTED,
+               "quantize_tensor_dynamic: the one-launch form is for tensors of up to 262144 elements (got %zu); "
+               "use lq_minmax + lq_calc_qparams + lq_quantize", n);
+    const float half_range = float((double(qmax) - double(qmin)) / 2.0);
+    hipLaunchKernelGGL(quantize_tensor_dynamic_kernel, dim3(1), dim3(1024), 0, as_stream(stream), x, n, symmetric,
+                       qmin, qmax, is_signed, eps, half_range, code_offset, scale, zp, mn_out, mx_out, q);
+    LQ_CHECK_LAUNCH("quantize_tensor_dynamic");
+    return LQ_OK;
+}
 
 int lq_quantize_rows_dynamic_i8(const float* x, size_t rows, size_t cols, int symmetric, int qmin, int qmax,
                                 int is_signed, float eps, int code_offset, float* scale, float* zp,

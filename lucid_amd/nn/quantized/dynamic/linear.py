@@ -62,7 +62,17 @@ class Linear(Module):
             raise _C.ShapeMismatch(f"expected last dim {K}, got {x.shape}")
         M = x.numel // K
         qd = self.act_qdtype
-        if x._range is not None:
+        off = storage_offset(qd)
+        xq = Tensor.empty((M, K), T.int8, "hip")
+        small = x._range is None and x.numel <= (1 << 18)
+        if small:
+            # min / max, qparams and codes of a small activation in one launch (same bits)
+            x_scale = Tensor.empty((), T.float32, "hip")
+            x_zp = Tensor.empty((), T.float32, "hip")
+            _C.call("lq_quantize_tensor_dynamic_i8", x.data_ptr if x.numel else None, x.numel, 0, qd.quant_min,
+                    qd.quant_max, int(qd.signed), 1e-8, off, x_scale.data_ptr, x_zp.data_ptr, None, None,
+                    xq.data_ptr if x.numel else None, None)
+        elif x._range is not None:
             # the kernel that wrote x kept its min / max: qparams straight from them
             x_scale = Tensor.empty((), T.float32, "hip")
             x_zp = Tensor.empty((), T.float32, "hip")
@@ -71,10 +81,9 @@ class Linear(Module):
         else:
             mn, mx = minmax(x)
             x_scale, x_zp = calculate_qparams(mn, mx, per_tensor_affine, qd)
-        off = storage_offset(qd)
-        xq = Tensor.empty((M, K), T.int8, "hip")
-        _C.call("lq_quantize", x.data_ptr, xq.data_ptr, _C.I8, off, 1, 1, x.numel,
-                x_scale.data_ptr, x_zp.data_ptr, 0, qd.quant_min, qd.quant_max, None)
+        if not small:
+            _C.call("lq_quantize", x.data_ptr, xq.data_ptr, _C.I8, off, 1, 1, x.numel,
+                    x_scale.data_ptr, x_zp.data_ptr, 0, qd.quant_min, qd.quant_max, None)
         if self._wsum is None:
             self._wsum = _ops.rowsum_i8(self.weight_int8)
         rng = None

@@ -344,3 +344,43 @@ def test_quantize_rows_dynamic_equals_the_three_calls_and_the_oracle(rows, cols,
     oq = O.quantize(x, os_, oz, qdtype.quant_min, qdtype.quant_max, ch_axis=0,
                     q_dtype=O.I8 if qdtype.storage == "int8" else O.I16)
     assert np.array_equal(q.numpy()[ok], oq[ok])
+
+
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 1000, 64 * 784, 262144, 50177])
+@pytest.mark.parametrize("qd", ["quint8", "qint8"])
+def test_quantize_tensor_dynamic_equals_the_three_calls(n, qd):
+    """Global min / max, qparams and codes of a small tensor in one launch: the bits of
+    minmax + calculate_qparams + quantize (and so of the oracle, which those are tested against)."""
+    from lucid_amd import _C
+    rng = np.random.default_rng(n + len(qd))
+    x = (rng.standard_normal(n) * 3 + 0.5).astype(np.float32)
+    qdtype = getattr(Q, qd)
+    off = -128 if qd == "quint8" else 0
+    xt = L.tensor(x, device="hip")
+    q = L.Tensor.empty((n,), L.int8, "hip")
+    s, z = L.Tensor.empty((), L.float32, "hip"), L.Tensor.empty((), L.float32, "hip")
+    mn1, mx1 = L.Tensor.empty((), L.float32, "hip"), L.Tensor.empty((), L.float32, "hip")
+    _C.call("lq_quantize_tensor_dynamic_i8", xt.data_ptr if n else None, n, 0, qdtype.quant_min, qdtype.quant_max,
+            int(qdtype.signed), 1e-8, off, s.data_ptr, z.data_ptr, mn1.data_ptr, mx1.data_ptr,
+            q.data_ptr if n else None, None)
+    mn, mx = Q.minmax(xt)
+    s3, z3 = Q.calculate_qparams(mn, mx, Q.per_tensor_affine, qdtype)
+    assert np.array_equal(bits(mn1.numpy()), bits(mn.numpy())) and np.array_equal(bits(mx1.numpy()), bits(mx.numpy()))
+    assert np.array_equal(bits(s.numpy()), bits(s3.numpy())) and np.array_equal(bits(z.numpy()), bits(z3.numpy()))
+    if n:
+        q3 = L.Tensor.empty((n,), L.int8, "hip")
+        _C.call("lq_quantize", xt.data_ptr, q3.data_ptr, _C.I8, off, 1, 1, n, s3.data_ptr, z3.data_ptr, 0,
+                qdtype.quant_min, qdtype.quant_max, None)
+        assert np.array_equal(q.numpy(), q3.numpy())
+        exp = O.quantize(x, s3.numpy(), z3.numpy(), qdtype.quant_min, qdtype.quant_max, code_offset=off)
+        assert np.array_equal(q.numpy(), exp)
+
+
+def test_quantize_tensor_dynamic_refuses_large_tensors():
+    from lucid_amd import _C
+    x = L.Tensor.empty((262145,), L.float32, "hip")
+    q = L.Tensor.empty((262145,), L.int8, "hip")
+    s, z = L.Tensor.empty((), L.float32, "hip"), L.Tensor.empty((), L.float32, "hip")
+    with pytest.raises(NotImplementedError):
+        _C.call("lq_quantize_tensor_dynamic_i8", x.data_ptr, 262145, 0, 0, 255, 0, 1e-8, -128, s.data_ptr, z.data_ptr,
+                None, None, q.data_ptr, None)
