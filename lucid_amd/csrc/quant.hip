@@ -573,19 +573,44 @@ __global__ __launch_bounds__(256) void quantize_rows_dynamic_kernel(
 }
 
 // Dynamic per-tensor quantization of a small tensor in one launch (one block): global
-// min / max (observer.py:363-375), qparams, codes.  The second read of x comes from the L2.
+// min / max (observer.py:363-375), qparams, codes.  Up to 16 float4 per lane (65536
+// elements) stay in registers between the two phases, all their loads in flight at once;
+// beyond that the block works in batches of 8 and re-reads x (from the L2) for the codes.
 __global__ __launch_bounds__(1024) void quantize_tensor_dynamic_kernel(
     const float* __restrict__ x, size_t n, int symmetric, int qmin, int qmax, int is_signed, float eps,
     float half_range, int off, float* __restrict__ scale, float* __restrict__ zp, float* __restrict__ mn_out,
     float* __restrict__ mx_out, int8_t* __restrict__ q) {
     __shared__ float s_sz[2];
+    constexpr int kKeep = 16, kBatch = 8;
     const bool vec = aligned16(x) && (reinterpret_cast<uintptr_t>(q) & 3u) == 0;
     const size_t quads = vec ? n / 4 : 0;
+    const bool keep = quads <= size_t(kKeep) * 1024;
     const float4* x4 = reinterpret_cast<const float4*>(x);
     MinMax m{__builtin_inff(), -__builtin_inff(), 0};
-    for (size_t i = threadIdx.x; i < quads; i += 1024) {
-        const float4 v = x4[i];
-        mm_update(m, v.x), mm_update(m, v.y), mm_update(m, v.z), mm_update(m, v.w);
+    float4 v[kKeep];
+    if (keep) {
+#pragma unroll
+        for (int u = 0; u < kKeep; ++u) {
+            const size_t i = size_t(u) * 1024 + threadIdx.x;
+            if (i < quads) v[u] = x4[i];
+        }
+#pragma unroll
+        for (int u = 0; u < kKeep; ++u)
+            if (size_t(u) * 1024 + threadIdx.x < quads)
+                mm_update(m, v[u].x), mm_update(m, v[u].y), mm_update(m, v[u].z), mm_update(m, v[u].w);
+    } else {
+        for (size_t i0 = 0; i0 < quads; i0 += size_t(kBatch) * 1024) {
+            float4 w[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const size_t i = i0 + size_t(u) * 1024 + threadIdx.x;
+                if (i < quads) w[u] = x4[i];
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u)
+                if (i0 + size_t(u) * 1024 + threadIdx.x < quads)
+                    mm_update(m, w[u].x), mm_update(m, w[u].y), mm_update(m, w[u].z), mm_update(m, w[u].w);
+        }
     }
     for (size_t e = quads * 4 + threadIdx.x; e < n; e += 1024) mm_update(m, x[e]);
     m = mm_block_reduce(m);
@@ -602,7 +627,27 @@ __global__ __launch_bounds__(1024) void quantize_tensor_dynamic_kernel(
     __syncthreads();
     const float s = s_sz[0], z = s_sz[1], r = 1.0f / s;
     const QuantizeOp<int8_t> op{x4, reinterpret_cast<Code8x4*>(q), float(double(qmin)), float(double(qmax)), off};
-    for (size_t i = threadIdx.x; i < quads; i += 1024) op.q[i] = op.pack(x4[i], s, z, r);
+    if (keep) {
+#pragma unroll
+        for (int u = 0; u < kKeep; ++u) {
+            const size_t i = size_t(u) * 1024 + threadIdx.x;
+            if (i < quads) op.q[i] = op.pack(v[u], s, z, r);
+        }
+    } else {
+        for (size_t i0 = 0; i0 < quads; i0 += size_t(kBatch) * 1024) {
+            float4 w[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const size_t i = i0 + size_t(u) * 1024 + threadIdx.x;
+                if (i < quads) w[u] = x4[i];
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const size_t i = i0 + size_t(u) * 1024 + threadIdx.x;
+                if (i < quads) op.q[i] = op.pack(w[u], s, z, r);
+            }
+        }
+    }
     for (size_t e = quads * 4 + threadIdx.x; e < n; e += 1024) op.scalar(e, s, z);
 }
 
