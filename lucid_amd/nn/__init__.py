@@ -100,6 +100,33 @@ class Conv2d(Module):
             "quantize the model (convert) first")
 
 
+class Conv1d(Module):
+    """Float Conv1d as a parameter holder (``weight`` (O, I/groups, K), ``bias`` (O,))."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, padding_mode="zeros") -> None:
+        super().__init__()
+        one = lambda v: int(v[0]) if isinstance(v, (tuple, list)) else int(v)
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride = one(kernel_size), one(stride)
+        self.dilation, self.groups = one(dilation), groups
+        self._padding_str = padding if isinstance(padding, str) else None
+        self.padding = 0 if isinstance(padding, str) else one(padding)
+        self.padding_mode = padding_mode
+        fan_in = in_channels // groups * self.kernel_size
+        bound = 1.0 / np.sqrt(fan_in)
+        rng = np.random.default_rng(fan_in * 7919 + out_channels + 1)
+        self.register_buffer("weight", T.tensor(rng.uniform(
+            -bound, bound, (out_channels, in_channels // groups, self.kernel_size)).astype(np.float32)))
+        self.register_buffer("bias", T.tensor(
+            rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.Conv1d.forward is not part of the hip quantized-inference backend; "
+            "quantize the model (convert) first")
+
+
 class BatchNorm2d(Module):
     """Float BatchNorm2d as a parameter / statistics holder (folded into the
     preceding convolution by ``fuse_modules`` before quantization)."""
@@ -322,6 +349,31 @@ class ConvTranspose2d(Module):
     def forward(self, x):
         raise NotImplementedError(
             "float nn.ConvTranspose2d.forward is not part of the hip quantized-inference backend; "
+            "quantize the model (convert) first")
+
+
+class ConvTranspose1d(Module):
+    """Float ConvTranspose1d as a parameter holder (``weight`` (in, out/groups, k))."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, output_padding=0,
+                 groups=1, bias=True, dilation=1) -> None:
+        super().__init__()
+        one = lambda v: int(v[0]) if isinstance(v, (tuple, list)) else int(v)
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride = one(kernel_size), one(stride)
+        self.padding = padding if isinstance(padding, str) else one(padding)
+        self.output_padding, self.dilation, self.groups = one(output_padding), one(dilation), groups
+        fan_in = out_channels // groups * self.kernel_size
+        bound = 1.0 / np.sqrt(fan_in)
+        rng = np.random.default_rng(fan_in * 7919 + in_channels + 1)
+        self.register_buffer("weight", T.tensor(rng.uniform(
+            -bound, bound, (in_channels, out_channels // groups, self.kernel_size)).astype(np.float32)))
+        self.register_buffer("bias", T.tensor(
+            rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.ConvTranspose1d.forward is not part of the hip quantized-inference backend; "
             "quantize the model (convert) first")
 
 

@@ -174,3 +174,71 @@ class Conv2d(Module):
     def extra_repr(self) -> str:
         return (f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}, "
                 f"stride={self.stride}, qdtype={self.out_qdtype.name}")
+
+
+class Conv1d(Conv2d):
+    """Quantized ``Conv1d`` (``lucid/nn/quantized/conv.py:232-385``): the same buffers with a
+    three-dimensional kernel ``weight_int8`` ``(Cout, Cin/groups, K)``.  A 1-d convolution over
+    ``(B, C, L)`` is the 2-d one over ``(B, C, 1, L)``: the input codes are turned to
+    channel-last order, the implicit-GEMM kernel runs with a one-row image, and the result is
+    turned back to ``(B, Cout, L_out)`` codes."""
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size, stride=1, padding=0,
+                 dilation=1, groups: int = 1, bias: bool = True) -> None:
+        one = lambda v: int(v[0]) if isinstance(v, (tuple, list)) else int(v)
+        super().__init__(in_channels, out_channels, (1, one(kernel_size)), (1, one(stride)),
+                         padding if isinstance(padding, str) else (0, one(padding)), (1, one(dilation)), groups, bias)
+        self.register_buffer("weight_int8", T.tensor(
+            np.zeros((out_channels, in_channels // groups, one(kernel_size)), np.int8), device="hip"))
+
+    def _prepare_weight(self) -> None:
+        O, I, K = self.weight_int8.shape
+        w = Tensor.empty((O, 1, K, I), T.int8, "hip")
+        _C.call("lq_repack_oihw_to_ohwi_i8", self.weight_int8.data_ptr, w.data_ptr, O, I, 1, K, None)
+        self._w_ohwi = w
+        self._wsum = _ops.rowsum_i8(w)
+
+    def forward(self, x: Tensor) -> Tensor:
+        name = type(self).__name__
+        g = input_grid(x, name)
+        if x.ndim != 3 or x.shape[1] != self.in_channels:
+            raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, L), got {x.shape}")
+        if g.layout != "plain":
+            raise _C.LucidError(f"{name}: 3-d activation codes must be stored in their own (B, C, L) order")
+        B, Cc, Ln = x.shape
+        # (B, C, L) -> (B, 1, L, C): the weight repacker is a generic (O, I, K) -> (O, K, I) turn
+        nhwc = Tensor.empty((B, 1, Ln, Cc), T.int8, "hip")
+        _C.call("lq_repack_oihw_to_ohwi_i8", g.codes.data_ptr, nhwc.data_ptr, B, Cc, 1, Ln, None)
+        x4 = Tensor.on_grid((B, Cc, 1, Ln), Grid(nhwc, g.scale, g.zero_point, g.qdtype, g.offset, g.zp_host, "nhwc"))
+        y4 = super().forward(x4)
+        gy = y4._grid
+        _, Co, _, Lo = y4.shape
+        plain = Tensor.empty((B, Co, Lo), T.int8, "hip")
+        _C.call("lq_repack_oihw_to_ohwi_i8", gy.codes.data_ptr, plain.data_ptr, B, Lo, 1, Co, None)
+        return Tensor.on_grid((B, Co, Lo), Grid(plain, gy.scale, gy.zero_point, gy.qdtype, gy.offset, gy.zp_host,
+                                                "plain"))
+
+    @classmethod
+    def from_float(cls, mod) -> "Conv1d":
+        """Quantize a calibrated float ``Conv1d`` (``conv.py:186-222``)."""
+        qmod = cls(mod.in_channels, mod.out_channels, mod.kernel_size, mod.stride, mod.padding,
+                   mod.dilation, mod.groups, bias=mod.bias is not None)
+        codes, w_scale, w_zp, ch_axis = quantize_weight(mod)
+        require_symmetric_weight(w_zp, cls.__name__)
+        qmod.register_buffer("weight_int8", codes)
+        qmod.register_buffer("weight_scale", w_scale)
+        qmod.register_buffer("weight_zero_point", w_zp)
+        qmod.weight_ch_axis = ch_axis
+        qmod.padding_str = getattr(mod, "_padding_str", None)
+        qmod.padding_mode = getattr(mod, "padding_mode", "zeros")
+        if mod.bias is not None:
+            qmod.register_buffer("bias", mod.bias.to("hip"))
+        a_scale, a_zp, a_qdtype = activation_qparams(mod)
+        qmod.register_buffer("scale", a_scale)
+        qmod.register_buffer("zero_point", a_zp)
+        qmod.out_qdtype = a_qdtype
+        return qmod
+
+    def extra_repr(self) -> str:
+        return (f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size[1]}, "
+                f"stride={self.stride[1]}, qdtype={self.out_qdtype.name}")

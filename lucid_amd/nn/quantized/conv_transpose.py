@@ -128,3 +128,48 @@ class ConvTranspose2d(Module):
     def extra_repr(self) -> str:
         return (f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}, "
                 f"stride={self.stride}, qdtype={self.out_qdtype.name}")
+
+
+class ConvTranspose1d(ConvTranspose2d):
+    """Quantized ``ConvTranspose1d`` (``lucid/nn/quantized/conv_transpose.py:162-319``):
+    ``weight_int8`` ``(in, out/groups, k)``; computed as the 2-d layer over a one-row image
+    (codes turned to channel-last order and back)."""
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size, stride=1, padding=0,
+                 output_padding=0, dilation=1, groups: int = 1, bias: bool = True) -> None:
+        one = lambda v: int(v[0]) if isinstance(v, (tuple, list)) else int(v)
+        super().__init__(in_channels, out_channels, (1, one(kernel_size)), (1, one(stride)), (0, one(padding)),
+                         (0, one(output_padding)), (1, one(dilation)), groups, bias)
+        self.register_buffer("weight_int8", T.tensor(
+            np.zeros((in_channels, out_channels // groups, one(kernel_size)), np.int8), device="hip"))
+
+    def _prepare_weight(self) -> None:
+        w3 = self.weight_int8
+        try:  # the 2-d preparation on the kernel seen as (in, out/groups, 1, k)
+            self._buffers["weight_int8"] = w3.reshape(w3.shape[0], w3.shape[1], 1, w3.shape[2])
+            super()._prepare_weight()
+        finally:
+            self._buffers["weight_int8"] = w3
+
+    def forward(self, x: Tensor) -> Tensor:
+        name = type(self).__name__
+        g = input_grid(x, name)
+        if x.ndim != 3 or x.shape[1] != self.in_channels:
+            raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, L), got {x.shape}")
+        if g.layout != "plain":
+            raise _C.LucidError(f"{name}: 3-d activation codes must be stored in their own (B, C, L) order")
+        B, Cc, Ln = x.shape
+        nhwc = Tensor.empty((B, 1, Ln, Cc), T.int8, "hip")
+        _C.call("lq_repack_oihw_to_ohwi_i8", g.codes.data_ptr, nhwc.data_ptr, B, Cc, 1, Ln, None)
+        x4 = Tensor.on_grid((B, Cc, 1, Ln), Grid(nhwc, g.scale, g.zero_point, g.qdtype, g.offset, g.zp_host, "nhwc"))
+        y4 = super().forward(x4)
+        gy = y4._grid
+        _, Co, _, Lo = y4.shape
+        plain = Tensor.empty((B, Co, Lo), T.int8, "hip")
+        _C.call("lq_repack_oihw_to_ohwi_i8", gy.codes.data_ptr, plain.data_ptr, B, Lo, 1, Co, None)
+        return Tensor.on_grid((B, Co, Lo), Grid(plain, gy.scale, gy.zero_point, gy.qdtype, gy.offset, gy.zp_host,
+                                                "plain"))
+
+    def extra_repr(self) -> str:
+        return (f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size[1]}, "
+                f"stride={self.stride[1]}, qdtype={self.out_qdtype.name}")

@@ -282,3 +282,79 @@ def test_dynamic_lstm(layers, bidir, batch_first, bias, with_state):
             setattr(f, n, type("A", (), {"numpy": lambda self, v=v: v})())
     yf, _, _ = _oracle_lstm_stack(f, x, hx, batch_first)
     assert np.abs(yf - y.numpy()).mean() / (np.abs(yf).mean() + 1e-9) < 0.03
+
+
+# ---------------------------------------------------------------- Conv1d
+@pytest.mark.parametrize("cin,cout,k,stride,padding,dilation,groups,Ln",
+                         [(16, 32, 3, 1, 1, 1, 1, 50), (32, 48, 5, 2, 2, 1, 1, 37), (32, 32, 3, 1, "same", 2, 2, 64),
+                          (16, 16, 1, 1, 0, 1, 1, 9), (64, 64, 7, 3, "valid", 1, 4, 100)])
+def test_conv1d_bit_exact_against_the_oracle(cin, cout, k, stride, padding, dilation, groups, Ln):
+    """nnq.Conv1d == the oracle's integer convolution of the same codes as a one-row image
+    (conv.py:232-385 on the 2-d kernel), codes bit for bit; the float view within a step."""
+    rng = np.random.default_rng(cin * 3 + cout + k)
+    m = nn.Sequential(nnq.QuantStub(), nn.Conv1d(cin, cout, k, stride=stride, padding=padding, dilation=dilation,
+                                                 groups=groups), nnq.DeQuantStub())
+    prepared = Q.prepare(m, Q.get_default_qconfig())
+    for _ in range(4):
+        x = rng.standard_normal((3, cin, Ln)).astype(np.float32)
+        prepared[0].activation_post_process(hip(x))
+        prepared[1].activation_post_process(hip((rng.standard_normal((3, cout, 4)) * 2).astype(np.float32)))
+    qm = Q.convert(prepared)
+    c1 = qm[1]
+    assert isinstance(c1, nnq.Conv1d) and c1.weight_int8.shape == (cout, cin // groups, k)
+    x = rng.standard_normal((3, cin, Ln)).astype(np.float32)
+    xq = qm[0](hip(x))
+    out = c1(xq)
+    # the same layer through the oracle: NHWC codes of a (B, 1, L, C) image, OHWI weights
+    s0, z0 = qm[0].scale.item(), qm[0].zero_point.item()
+    codes = O.quantize(x, s0, z0, 0, 255, code_offset=-128)                      # (B, C, L)
+    x_nhwc = np.ascontiguousarray(np.transpose(codes, (0, 2, 1))[:, None, :, :])  # (B, 1, L, C)
+    w_ohwi = np.ascontiguousarray(np.transpose(c1.weight_int8.numpy(), (0, 2, 1))[:, None, :, :])
+    if padding == "same":
+        total = max(0, (-(-Ln // stride) - 1) * stride + (k - 1) * dilation + 1 - Ln)
+        pad = (0, 0, total // 2, total - total // 2)
+    elif padding == "valid":
+        pad = (0, 0, 0, 0)
+    else:
+        pad = (0, 0, padding, padding)
+    want = O.qconv2d(x_nhwc, w_ohwi, int(z0) - 128, np.float32(s0), c1.weight_scale.numpy(), stride=(1, stride),
+                     pad=pad, dilation=(1, dilation), groups=groups, bias=c1.bias.numpy(), out_mode=O.OUT_REQUANT_I8,
+                     out_scale=np.float32(c1.scale.item()), out_zp=np.float32(c1.zero_point.item()), out_qmin=0,
+                     out_qmax=255, out_offset=-128)                                # (B, 1, Lo, Cout)
+    got = out._grid.codes.numpy()                                                  # (B, Cout, Lo)
+    assert got.shape == (3, cout, want.shape[2])
+    assert np.array_equal(got, np.transpose(want[:, 0], (0, 2, 1)))
+    y = qm(hip(x)).numpy()
+    assert y.shape == got.shape and np.isfinite(y).all()
+
+
+@pytest.mark.parametrize("cin,cout,k,stride,padding,output_padding,dilation,groups",
+                         [(16, 32, 3, 2, 1, 1, 1, 1), (32, 32, 4, 3, 0, 2, 1, 2), (16, 16, 3, 1, 1, 0, 2, 1)])
+def test_conv_transpose1d(cin, cout, k, stride, padding, output_padding, dilation, groups):
+    """nnq.ConvTranspose1d == nnq.ConvTranspose2d on the same operands as a one-row image, codes
+    bit for bit (conv_transpose.py:162-319); the 2-d layer is checked against the oracle above."""
+    rng = np.random.default_rng(cin + cout + k)
+    m = nn.Sequential(nnq.QuantStub(), nn.ConvTranspose1d(cin, cout, k, stride=stride, padding=padding,
+                                                          output_padding=output_padding, groups=groups,
+                                                          dilation=dilation), nnq.DeQuantStub())
+    prepared = Q.prepare(m, Q.get_default_qconfig())
+    for _ in range(4):
+        prepared[0].activation_post_process(hip(rng.standard_normal((2, cin, 21)).astype(np.float32)))
+        prepared[1].activation_post_process(hip((rng.standard_normal((2, cout, 5)) * 0.7).astype(np.float32)))
+    qm = Q.convert(prepared)
+    c1 = qm[1]
+    assert isinstance(c1, nnq.ConvTranspose1d) and c1.weight_int8.shape == (cin, cout // groups, k)
+    c2 = nnq.ConvTranspose2d(cin, cout, (1, k), (1, stride), (0, padding), (0, output_padding), (1, dilation), groups)
+    c2.register_buffer("weight_int8", L.tensor(c1.weight_int8.numpy()[:, :, None, :], device="hip"))
+    for name in ("weight_scale", "weight_zero_point", "bias", "scale", "zero_point"):
+        c2.register_buffer(name, getattr(c1, name))
+    c2.out_qdtype = c1.out_qdtype
+    x = rng.standard_normal((2, cin, 21)).astype(np.float32)
+    y1 = c1(qm[0](hip(x)))
+    # the 2-d layer on the same codes: quantize the (B, C, 1, L) view with the same stub
+    y2 = c2(qm[0](hip(x[:, :, None, :])))
+    got = y1._grid.codes.numpy()                                   # (B, Cout, Lo)
+    want = np.transpose(y2._grid.codes.numpy()[:, 0], (0, 2, 1))   # NHWC (B, 1, Lo, Cout) -> (B, Cout, Lo)
+    lo = (21 - 1) * stride - 2 * padding + dilation * (k - 1) + output_padding + 1
+    assert got.shape == (2, cout, lo) and np.array_equal(got, want)
+    assert np.isfinite(qm(hip(x)).numpy()).all()
