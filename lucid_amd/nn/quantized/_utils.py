@@ -25,7 +25,9 @@ def quantize_weight(mod) -> tuple[Tensor, Tensor, Tensor, int]:
     (``_utils.py:27-55``): run the qconfig's weight observer over the static
     weight, then ``quantize`` along its channel axis."""
     weight = mod.weight.to("hip")
-    wobs = mod.qconfig.weight()
+    wobs = getattr(mod, "weight_fake_quant", None)  # a QAT layer: its FakeQuantize, refreshed
+    if wobs is None:
+        wobs = mod.qconfig.weight()
     wobs(weight)
     scale, zero_point = wobs.calculate_qparams()
     qdtype, ch_axis = wobs.qdtype, wobs.ch_axis

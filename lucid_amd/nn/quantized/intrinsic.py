@@ -20,6 +20,9 @@ class LinearReLU(Linear):
     def from_float(cls, mod) -> "LinearReLU":
         # an nni.LinearReLU is a Sequential(Linear, ReLU) that carries the qconfig
         # and the activation observer of the fused pair
+        # (a QAT LinearReLU is already a single weighted layer: intrinsic.py:23-37)
+        if not hasattr(mod, "__getitem__"):
+            return super().from_float(mod)
         inner = mod[0]
         inner.qconfig = mod.qconfig
         inner.activation_post_process = mod.activation_post_process

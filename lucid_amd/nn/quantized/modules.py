@@ -12,9 +12,15 @@ from ._utils import host_scalar, storage_offset
 
 
 class QuantStub(Module):
-    """Float-model entry marker; ``prepare`` attaches its observer."""
+    """Float-model entry marker; ``prepare`` attaches its observer (a forward hook: the stub
+    stays an identity), ``prepare_qat`` a ``FakeQuantize``, which the stub applies to a float
+    input (``modules.py:84-95``)."""
 
     def forward(self, x):
+        from ...quantization._fake_quantize import FakeQuantize
+        app = self.__dict__.get("_modules", {}).get("activation_post_process")
+        if isinstance(app, FakeQuantize) and getattr(x, "dtype", None) is T.float32:
+            return app(x)
         return x
 
 

@@ -21,12 +21,15 @@ from ._qscheme import (
 from .observer import (FixedQParamsObserver, HistogramObserver, MinMaxObserver,
                        MovingAverageMinMaxObserver, MovingAveragePerChannelMinMaxObserver, ObserverBase,
                        PerChannelMinMaxObserver)
-from .qconfig import QConfig, get_default_qconfig
+from .qconfig import QConfig, get_default_qat_qconfig, get_default_qconfig
 
 
 def __getattr__(name):
     # the workflow functions import lucid_amd.nn, which imports this package
-    if name in ("prepare", "convert", "quantize_dynamic"):
+    if name == "FakeQuantize":
+        from ._fake_quantize import FakeQuantize
+        return FakeQuantize
+    if name in ("prepare", "prepare_qat", "convert", "quantize_dynamic"):
         from . import _quantize
         return getattr(_quantize, name)
     if name == "fuse_modules":

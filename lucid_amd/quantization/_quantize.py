@@ -133,6 +133,42 @@ def prepare(model, qconfig: QConfig | None = None, inplace: bool = False):
     return model
 
 
+def _qat_mapping() -> dict[type, object]:
+    """Float module type -> its QAT form (``_quantize.py:557-573``); the convolutions' QAT
+    forms need a float convolution, which this backend does not have."""
+    import lucid_amd.nn.qat as nnqat
+    return {nn.Linear: nnqat.Linear.from_float, nni.LinearReLU: nnqat.LinearReLU.from_float}
+
+
+def _prepare_qat_recursive(module, qcfg, qat_map) -> int:
+    n = 0
+    for name, child in list(module.named_children()):
+        build = qat_map.get(type(child))
+        if build is not None:
+            child.qconfig = qcfg
+            module._modules[name] = build(child)
+            n += 1
+        elif isinstance(child, nnq.QuantStub):
+            child.qconfig = qcfg
+            child.activation_post_process = qcfg.activation()
+            n += 1
+        else:
+            n += _prepare_qat_recursive(child, qcfg, qat_map)
+    return n
+
+
+def prepare_qat(model, qconfig: QConfig | None = None, inplace: bool = False):
+    """Swap the weighted layers for their QAT forms and put a ``FakeQuantize`` on every
+    ``QuantStub`` (``_quantize.py:575-700``).  The result runs the simulated-quantization
+    forward on the device and converts with ``convert``; fine-tuning it is Lucid's job."""
+    from .qconfig import get_default_qat_qconfig
+    qcfg = qconfig if qconfig is not None else get_default_qat_qconfig()
+    model = model if inplace else copy.deepcopy(model)
+    if _prepare_qat_recursive(model, qcfg, _qat_mapping()) == 0:
+        warnings.warn("prepare_qat(): no module of this model has a QAT form here", stacklevel=2)
+    return model
+
+
 def _convert_recursive(module, mapping, always) -> None:
     for name, child in list(module.named_children()):
         build = mapping.get(type(child))
@@ -149,6 +185,9 @@ def convert(model, inplace: bool = False):
     (``_quantize.py:314-419``)."""
     model = model if inplace else copy.deepcopy(model)
     mapping = _quant_mapping()
+    import lucid_amd.nn.qat as nnqat
+    mapping[nnqat.Linear] = nnq.Linear.from_float
+    mapping[nnqat.LinearReLU] = nnq.LinearReLU.from_float
     if backends.quantized.use_mlx():
         mapping[nn.Linear] = _mlx_linear_builder(relu=False)
         mapping[nni.LinearReLU] = _mlx_linear_builder(relu=True)
