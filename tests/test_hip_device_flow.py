@@ -46,6 +46,13 @@ def test_static_ptq_round_trip_on_device():
     assert np.abs(out - yf).max() < 5e-2
 
 
+def test_qat_qconfig_static_quant_on_device():
+    # test_device_metal.py:65-68: the FakeQuantize-based qconfig through the same static flow
+    cm, y, yf = _static_quant(Q.get_default_qat_qconfig())
+    out = y.numpy()
+    assert np.isfinite(out).all() and np.abs(out - yf).max() < 1e-1
+
+
 def test_observers_were_fed_by_the_forward_hooks():
     rng = np.random.default_rng(2)
     m = nn.Sequential(nn.Linear(16, 16), nn.ReLU(), nn.Linear(16, 8)).to("hip")
