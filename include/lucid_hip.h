@@ -367,6 +367,16 @@ int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, f
  * weight [dim, C, p, p] flattened. */
 int lq_patchify_f32(const float* img, float* out, int B, int C, int H, int W, int patch, lq_stream stream);
 
+/* Float32 convolution of an NCHW image with an OIHW filter, zero padding (pad_h / pad_w
+ * on both sides), as im2col + GEMM (IBackend::conv_nd_forward, CpuBackend.h:8124-8257;
+ * Im2Col.cpp:59-100; output size ConvNd.cpp:56-59).  It is what a calibration pass
+ * through a prepared convolutional model and the forward of a QAT convolution run on;
+ * inference goes through lq_qconv2d_i8.  out: [B, Cout, OH, OW].  Synchronises the
+ * stream before it returns (its scratch comes from lq_alloc). */
+int lq_conv2d_f32(const float* x, const float* w, const float* bias, float* out, int B, int Cin, int H, int W, int Cout,
+                  int KH, int KW, int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, int groups,
+                  lq_stream stream);
+
 /* out[M,N] = a[M,K] . w[N,K]^T + bias[N] in float32 (IBackend::linear, CpuBackend.h:4525);
  * bias may be null. */
 int lq_sgemm_nt_f32(const float* a, const float* w, const float* bias, float* out, int M, int N, int K,

@@ -95,9 +95,28 @@ class Conv2d(Module):
             rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
 
     def forward(self, x):
-        raise NotImplementedError(
-            "float nn.Conv2d.forward is not part of the hip quantized-inference backend; "
-            "quantize the model (convert) first")
+        """Float32 convolution on the device (im2col + GEMM): what a calibration pass through a
+        prepared model needs.  Zero padding with symmetric amounts; inference is the quantized
+        module's business."""
+        if not isinstance(x, Tensor) or x.device != "hip":
+            raise NotImplementedError(
+                "float nn.Conv2d.forward runs on the 'hip' device only; the CPU float path is Lucid's")
+        if self.padding_mode != "zeros":
+            raise NotImplementedError(f"float nn.Conv2d.forward: padding_mode {self.padding_mode!r} is not built")
+        pad = self.padding
+        if self._padding_str == "same":
+            from .quantized.conv import _same_pad_pair
+            ph = _same_pad_pair(x.shape[2], self.kernel_size[0], self.stride[0], self.dilation[0])
+            pw = _same_pad_pair(x.shape[3], self.kernel_size[1], self.stride[1], self.dilation[1])
+            if ph[0] != ph[1] or pw[0] != pw[1]:
+                raise NotImplementedError("float nn.Conv2d.forward: asymmetric 'same' padding is not built")
+            pad = (ph[0], pw[0])
+        from .functional import conv2d_f32
+        w = self.weight if self.weight.device == "hip" else self.weight.to("hip")
+        b = self.bias
+        if b is not None and b.device != "hip":
+            b = b.to("hip")
+        return conv2d_f32(x, w, b, self.stride, pad, self.dilation, self.groups)
 
 
 class Conv1d(Module):

@@ -85,6 +85,24 @@ def scaled_dot_product_attention_qkv(qkv: Tensor, num_heads: int, scale: float |
     return out
 
 
+def conv2d_f32(x: Tensor, weight: Tensor, bias: Tensor | None = None, stride=(1, 1), padding=(0, 0),
+               dilation=(1, 1), groups: int = 1) -> Tensor:
+    """``F.conv2d`` in float32 with zero padding (``CpuBackend.h:8124-8257``): NCHW input, OIHW
+    weight, symmetric ``padding`` = (h, w).  Calibration and QAT forwards only."""
+    _require_f32_hip("conv2d", x, weight)
+    if x.ndim != 4 or weight.ndim != 4 or weight.shape[1] * groups != x.shape[1]:
+        raise _C.ShapeMismatch(f"conv2d: input {x.shape} and weight {weight.shape} (groups={groups}) do not match")
+    B, Cin, H, W = x.shape
+    Cout, _, KH, KW = weight.shape
+    OH = (H + 2 * padding[0] - dilation[0] * (KH - 1) - 1) // stride[0] + 1
+    OW = (W + 2 * padding[1] - dilation[1] * (KW - 1) - 1) // stride[1] + 1
+    out = Tensor.empty((B, Cout, max(OH, 0), max(OW, 0)), T.float32, "hip")
+    _C.call("lq_conv2d_f32", x.data_ptr, weight.data_ptr, bias.data_ptr if bias is not None else None, out.data_ptr,
+            B, Cin, H, W, Cout, KH, KW, int(stride[0]), int(stride[1]), int(padding[0]), int(padding[1]),
+            int(dilation[0]), int(dilation[1]), int(groups), None)
+    return out
+
+
 def linear_f32(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
     """``F.linear`` in float32 (``CpuBackend.h:4525``): ``x @ weight.T + bias``."""
     _require_f32_hip("linear", x, weight)

@@ -40,6 +40,8 @@ class ConvReLU2d(Conv2d):
 
     @classmethod
     def from_float(cls, mod) -> "ConvReLU2d":
+        if not hasattr(mod, "__getitem__"):  # a QAT ConvReLU2d is a single weighted layer
+            return super().from_float(mod)
         inner = mod[0]
         inner.qconfig = mod.qconfig
         inner.activation_post_process = mod.activation_post_process

@@ -134,10 +134,11 @@ def prepare(model, qconfig: QConfig | None = None, inplace: bool = False):
 
 
 def _qat_mapping() -> dict[type, object]:
-    """Float module type -> its QAT form (``_quantize.py:557-573``); the convolutions' QAT
-    forms need a float convolution, which this backend does not have."""
+    """Float module type -> its QAT form (``_quantize.py:557-573``): Linear and Conv2d, plain
+    and fused with ReLU."""
     import lucid_amd.nn.qat as nnqat
-    return {nn.Linear: nnqat.Linear.from_float, nni.LinearReLU: nnqat.LinearReLU.from_float}
+    return {nn.Linear: nnqat.Linear.from_float, nni.LinearReLU: nnqat.LinearReLU.from_float,
+            nn.Conv2d: nnqat.Conv2d.from_float, nni.ConvReLU2d: nnqat.ConvReLU2d.from_float}
 
 
 def _prepare_qat_recursive(module, qcfg, qat_map) -> int:
@@ -188,6 +189,8 @@ def convert(model, inplace: bool = False):
     import lucid_amd.nn.qat as nnqat
     mapping[nnqat.Linear] = nnq.Linear.from_float
     mapping[nnqat.LinearReLU] = nnq.LinearReLU.from_float
+    mapping[nnqat.Conv2d] = nnq.Conv2d.from_float
+    mapping[nnqat.ConvReLU2d] = nnq.ConvReLU2d.from_float
     if backends.quantized.use_mlx():
         mapping[nn.Linear] = _mlx_linear_builder(relu=False)
         mapping[nni.LinearReLU] = _mlx_linear_builder(relu=True)

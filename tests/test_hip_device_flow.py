@@ -85,3 +85,57 @@ def test_fake_quantize_takes_cpu_qparams_on_a_device_input():
     x = hip(np.random.default_rng(4).standard_normal((4, 8)))
     out = Q.fake_quantize(x, L.tensor(np.float32(0.05)), L.tensor(np.float32(0.0)), -128, 127, None)
     assert out.device == "hip" and np.isfinite(out.numpy()).all()
+
+
+def _conv2d_numpy(x, w, b, stride, pad, dil, groups):
+    B, C, H, W = x.shape
+    O, Cg, KH, KW = w.shape
+    xp = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (pad[0], pad[0]), (pad[1], pad[1])))
+    OH = (H + 2 * pad[0] - dil[0] * (KH - 1) - 1) // stride[0] + 1
+    OW = (W + 2 * pad[1] - dil[1] * (KW - 1) - 1) // stride[1] + 1
+    out = np.zeros((B, O, OH, OW))
+    og = O // groups
+    for o in range(O):
+        g = o // og
+        for kh in range(KH):
+            for kw in range(KW):
+                sl = xp[:, g * Cg:(g + 1) * Cg, kh * dil[0]:kh * dil[0] + (OH - 1) * stride[0] + 1:stride[0],
+                        kw * dil[1]:kw * dil[1] + (OW - 1) * stride[1] + 1:stride[1]]
+                out[:, o] += np.tensordot(sl, w[o, :, kh, kw].astype(np.float64), axes=([1], [0]))
+        if b is not None:
+            out[:, o] += b[o]
+    return out
+
+
+@pytest.mark.parametrize("cin,cout,k,stride,pad,dil,groups,hw", [
+    (3, 16, 7, 2, 3, 1, 1, (30, 29)), (16, 32, 3, 1, 1, 1, 1, (14, 14)), (32, 32, (3, 1), (2, 1), (1, 0), (1, 2), 4, (9, 11)),
+    (8, 24, 1, 1, 0, 1, 1, (5, 5)), (16, 16, 3, 1, 2, 2, 16, (12, 12))])
+def test_float_conv2d_forward_matches_numpy(cin, cout, k, stride, pad, dil, groups, hw):
+    pair = lambda v: (v, v) if isinstance(v, int) else v
+    rng = np.random.default_rng(cin + cout)
+    conv = nn.Conv2d(cin, cout, k, stride=stride, padding=pad, dilation=dil, groups=groups).to("hip")
+    x = rng.standard_normal((2, cin, *hw)).astype(np.float32)
+    y = conv(hip(x)).numpy()
+    want = _conv2d_numpy(x, conv.weight.numpy(), conv.bias.numpy(), pair(stride), pair(pad), pair(dil), groups)
+    assert y.shape == want.shape
+    assert np.abs(y - want).max() <= 1e-4 * (1 + np.abs(want).max())
+
+
+def test_conv_model_calibrates_and_converts_on_device():
+    """prepare -> calibrate (float convolutions on the device feed the observers) -> convert -> infer
+    for a small convolutional model, against its float forward."""
+    import lucid_amd.nn.quantized as nnq
+    rng = np.random.default_rng(5)
+    import lucid_amd.nn.intrinsic as nni
+    m = nn.Sequential(nnq.QuantStub(), nni.ConvReLU2d(nn.Conv2d(16, 32, 3, padding=1), nn.ReLU()),
+                      nn.Conv2d(32, 16, 1), nnq.DeQuantStub()).to("hip")
+    qm = Q.prepare(m, Q.get_default_qconfig())
+    for _ in range(4):
+        qm(hip(rng.standard_normal((2, 16, 12, 12))))
+    cm = Q.convert(qm)
+    assert isinstance(cm[1], nnq.ConvReLU2d) and isinstance(cm[2], nnq.Conv2d)
+    x = rng.standard_normal((2, 16, 12, 12)).astype(np.float32)
+    yf = m(hip(x)).numpy()
+    yq = cm(hip(x)).numpy()
+    assert yq.shape == yf.shape and np.isfinite(yq).all()
+    assert np.abs(yq - yf).mean() / np.abs(yf).mean() < 0.05

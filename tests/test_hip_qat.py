@@ -89,3 +89,36 @@ def test_prepare_qat_forward_and_convert():
     y8 = q8(hip(x)).numpy()
     d8 = np.abs(y8 - y)
     assert d8.max() <= step * 2.001 and (d8 > step * 0.01).mean() < 0.05
+
+
+def test_prepare_qat_convolutional_model_forward_and_convert():
+    rng = np.random.default_rng(3)
+    m = nn.Sequential(nnq.QuantStub(), nni.ConvReLU2d(nn.Conv2d(16, 32, 3, padding=1), nn.ReLU()),
+                      nn.Conv2d(32, 16, 1), nnq.DeQuantStub())
+    qat = Q.prepare_qat(m)
+    assert isinstance(qat[1], nnqat.ConvReLU2d) and isinstance(qat[2], nnqat.Conv2d)
+    for _ in range(5):
+        qat(hip(rng.standard_normal((2, 16, 10, 10)).astype(np.float32)))
+    for mod in qat.modules():
+        if type(mod).__name__ == "FakeQuantize":
+            mod.disable_observer()
+    x = rng.standard_normal((2, 16, 10, 10)).astype(np.float32)
+    y = qat(hip(x)).numpy()
+    # the forward is the float convolution of fake-quantized operands, fake-quantized
+    c1 = qat[1]
+    fq = lambda t, mm, ax=None: O.fake_quantize(t, mm.scale.numpy(), mm.zero_point.numpy(), mm.qdtype.quant_min,
+                                                mm.qdtype.quant_max, ch_axis=ax)
+    h = fq(x, qat[0].activation_post_process)
+    conv = nn.Conv2d(16, 32, 3, padding=1)
+    conv.register_buffer("weight", hip(fq(c1.weight.numpy(), c1.weight_fake_quant, 0)))
+    conv.register_buffer("bias", c1.bias)
+    h1 = fq(np.maximum(conv(hip(h)).numpy(), 0), c1.activation_post_process)
+    step1 = float(c1.activation_post_process.scale.numpy())
+    got1 = qat[1](qat[0](hip(x))).numpy()
+    assert np.abs(got1 - h1).max() <= step1 * 1.001
+    q8 = Q.convert(qat)
+    assert isinstance(q8[1], nnq.ConvReLU2d) and isinstance(q8[2], nnq.Conv2d)
+    y8 = q8(hip(x)).numpy()
+    step = float(qat[2].activation_post_process.scale.numpy())
+    d = np.abs(y8 - y)
+    assert d.max() <= step * 2.001 and (d > step * 0.01).mean() < 0.05
