@@ -35,6 +35,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // variance and the output pass.  mean, centred values, var = dot(c,c)/N,
 // rstd = 1/sqrt(var+eps), y = (c*rstd)*gamma + beta: the reference's steps.
 constexpr int LN_ROWS_PER_WAVE = 1;
+constexpr int LN_KEEP = 8;  // float4 per lane held in registers: rows of up to 2048 floats
 
 __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x,
                                                         const float* __restrict__ gamma,
@@ -56,6 +57,46 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
         if (row >= rows) break;
         const float* xr = x + row * cols;
         float* yr = out + row * cols;
+        if (vec && cols <= LN_KEEP * 256) {
+            // the row stays in registers (one trip to memory instead of three); the sums run
+            // over the same values in the same order as below
+            float4 v[LN_KEEP];
+#pragma unroll
+            for (int u = 0; u < LN_KEEP; ++u) {
+                const int c = lane * 4 + u * 256;
+                if (c < cols) v[u] = *reinterpret_cast<const float4*>(xr + c);
+            }
+            float s = 0.0f;
+#pragma unroll
+            for (int u = 0; u < LN_KEEP; ++u)
+                if (lane * 4 + u * 256 < cols) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+            const float mean = wave_sum(s) * inv_n;
+            float q = 0.0f;
+#pragma unroll
+            for (int u = 0; u < LN_KEEP; ++u)
+                if (lane * 4 + u * 256 < cols) {
+                    const float a = v[u].x - mean, b = v[u].y - mean, cc = v[u].z - mean, d = v[u].w - mean;
+                    q += (a * a + b * b) + (cc * cc + d * d);
+                }
+            const float var = wave_sum(q) * inv_n;
+            const float rstd = 1.0f / sqrtf(var + eps);
+#pragma unroll
+            for (int u = 0; u < LN_KEEP; ++u) {
+                const int c = lane * 4 + u * 256;
+                if (c < cols) {
+                    const float4 g = *reinterpret_cast<const float4*>(gamma + c);
+                    const float4 b = *reinterpret_cast<const float4*>(beta + c);
+                    float4 y;
+                    y.x = ((v[u].x - mean) * rstd) * g.x + b.x;
+                    y.y = ((v[u].y - mean) * rstd) * g.y + b.y;
+                    y.z = ((v[u].z - mean) * rstd) * g.z + b.z;
+                    y.w = ((v[u].w - mean) * rstd) * g.w + b.w;
+                    *reinterpret_cast<float4*>(yr + c) = y;
+                    track(y.x), track(y.y), track(y.z), track(y.w);
+                }
+            }
+            continue;
+        }
         float s = 0.0f;
         if (vec) {
             for (int c = lane * 4; c < cols; c += 256) {
