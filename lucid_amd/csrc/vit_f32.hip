@@ -396,13 +396,15 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
     const int q0 = wave * 16;  // the launch has exactly ceil(T / 16) wavefronts, so q0 < T
     (void)nwaves;
     const int g = lane >> 4, c = lane & 15;
-    // B operand of S^T: Q[q0 + c][4*s + g], pre-scaled so that S = scale * Q.K^T
+    // B operand of S^T: Q[q0 + c][4*s + g], pre-scaled so that S = scale * log2(e) * Q.K^T
     float qf[AT_D / 4];
     {
         const int q = q0 + c;
         const float* qp = base + size_t(q < T ? q : T - 1) * tok_stride;
 #pragma unroll
-        for (int s = 0; s < AT_D / 4; ++s) qf[s] = qp[4 * s + g] * scale;
+        // (scale * log2 e: the scores are kept in the base-2 domain, so that the softmax
+        // numerators are one v_exp_f32 each: 2^(s - max) = e^((s - max) ln 2))
+        for (int s = 0; s < AT_D / 4; ++s) qf[s] = qp[4 * s + g] * (scale * 1.4426950408889634f);
     }
     constexpr int NT = AT_TMAX / 16;
     v4f st[NT];
@@ -431,7 +433,7 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float e = expf(st[t][r] - mx);  // exp(-inf) = 0 for the padded keys
+            const float e = __builtin_amdgcn_exp2f(st[t][r] - mx);  // 2^(-inf) = 0 for the padded keys
             st[t][r] = e;
             sum += e;
         }
