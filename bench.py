@@ -622,6 +622,9 @@ def main() -> int:
     if args.vendor_child:
         return vendor_child(args.vendor_child, args.steps, args.warmup)
 
+    import __graft_entry__
+    __graft_entry__.ensure_built()  # loads what is built; compiles only if nothing is
+
     import lucid_amd as L
     import lucid_amd.quantization as Q
     from lucid_amd import _C, _ops
