@@ -347,6 +347,20 @@ int lq_calc_qparams_from_range(const float* range, int symmetric, int qmin, int 
 int lq_layernorm_f32(const float* x, const float* gamma, const float* beta, float* out, long rows, int cols,
                      float eps, float* range, lq_stream stream);
 
+/* LayerNorm in front of a dynamic-quantized Linear without the float32 round trip
+ * (nn.LayerNorm followed by nnqd.Linear: Norm.cpp:35-65, then dynamic/linear.py:87-92).
+ * lq_layernorm_stats_f32 writes each row's mean and rstd to stats [rows, 2] and keeps
+ * the min / max of the normalized values in `range` (lq_range_buffer_bytes() bytes);
+ * after lq_calc_qparams_from_range, lq_layernorm_quantize_i8 normalizes again with
+ * those statistics and writes the int8 codes - bit for bit the codes of
+ * lq_layernorm_f32 + lq_quantize.  Rows must be a multiple of 4 floats, at most
+ * 2048, 16-byte aligned (LQ_ERR_NOT_IMPLEMENTED otherwise). */
+int lq_layernorm_stats_f32(const float* x, const float* gamma, const float* beta, long rows, int cols, float eps,
+                           float* stats, float* range, lq_stream stream);
+int lq_layernorm_quantize_i8(const float* x, const float* gamma, const float* beta, const float* stats, long rows,
+                             int cols, const float* scale, const float* zp, int qmin, int qmax, int code_offset,
+                             int8_t* q, lq_stream stream);
+
 /* GELU, exact erf form (lucid/nn/functional/activations.py:219, approximate="none"). */
 int lq_gelu_f32(const float* x, float* out, size_t n, float* range, lq_stream stream);
 

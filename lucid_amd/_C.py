@@ -102,6 +102,8 @@ _SIGNATURES = {
     "lq_act_requant_i8": [_i, _f, _vp, _i, _vp, _vp, _sz, _vp, _vp, _i, _i, _i, _vp, _vp],
     "lq_dilate_nhwc_i8": [_vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp],
     "lq_lstm_cell_f32": [_vp, _sz, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _sz, _vp],
+    "lq_layernorm_stats_f32": [_vp, _vp, _vp, C.c_long, _i, C.c_float, _vp, _vp, _vp],
+    "lq_layernorm_quantize_i8": [_vp, _vp, _vp, _vp, C.c_long, _i, _vp, _vp, _i, _i, _i, _vp, _vp],
     "lq_conv2d_f32": [_vp, _vp, _vp, _vp] + [_i] * 14 + [_vp],
     "lq_quantize_tensor_dynamic_i8": [_vp, _sz, _i, _i, _i, _i, C.c_float, _i, _vp, _vp, _vp, _vp, _vp, _vp],
     "lq_quantize_rows_dynamic_i8": [_vp, _sz, _sz, _i, _i, _i, _i, C.c_float, _i, _vp, _vp, _vp, _vp, _vp, _vp],

@@ -15,6 +15,7 @@
 // Matrix products use the float32 MFMA instructions; results agree with a CPU
 // float32 evaluation to rounding-order differences (tested to 1e-4 relative).
 #include "common.hpp"
+#include "qepilogue.hpp"
 #include "range_slots.hpp"
 
 using namespace lq;
@@ -144,6 +145,96 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
         }
     }
     if (range) range_block_store(range, lo, hi, nan);
+}
+
+// LayerNorm feeding a dynamic quantizer without ever storing its float32 output: the first
+// kernel takes each row's mean and 1/sqrt(var + eps) and the range of the normalized values, the
+// second (after the qparams have been derived from that range) normalizes again - the same
+// expressions on the same inputs, so the same bits - and writes int8 codes.  x is read twice
+// and 1 byte per element written, where LayerNorm + quantize read it twice, write it once as
+// float32 and read that back.  Rows of up to 2048 floats, vector-aligned.
+__global__ __launch_bounds__(256) void layernorm_stats_kernel(const float* __restrict__ x,
+                                                              const float* __restrict__ gamma,
+                                                              const float* __restrict__ beta, long rows, int cols,
+                                                              float eps, float* __restrict__ stats, float* range) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const float inv_n = 1.0f / float(cols);
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    int nan = 0;
+    auto track = [&](float y) {
+        nan |= (y != y);
+        lo = fminf(lo, y);
+        hi = fmaxf(hi, y);
+    };
+    const long row = long(blockIdx.x) * 4 + wave;
+    if (row < rows) {
+        const float* xr = x + row * cols;
+        float4 v[LN_KEEP];
+#pragma unroll
+        for (int u = 0; u < LN_KEEP; ++u) {
+            const int c = lane * 4 + u * 256;
+            if (c < cols) v[u] = *reinterpret_cast<const float4*>(xr + c);
+        }
+        float s = 0.0f;
+#pragma unroll
+        for (int u = 0; u < LN_KEEP; ++u)
+            if (lane * 4 + u * 256 < cols) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+        const float mean = wave_sum(s) * inv_n;
+        float q = 0.0f;
+#pragma unroll
+        for (int u = 0; u < LN_KEEP; ++u)
+            if (lane * 4 + u * 256 < cols) {
+                const float a = v[u].x - mean, b = v[u].y - mean, cc = v[u].z - mean, d = v[u].w - mean;
+                q += (a * a + b * b) + (cc * cc + d * d);
+            }
+        const float var = wave_sum(q) * inv_n;
+        const float rstd = 1.0f / sqrtf(var + eps);
+        if (lane == 0) stats[2 * row] = mean, stats[2 * row + 1] = rstd;
+#pragma unroll
+        for (int u = 0; u < LN_KEEP; ++u) {
+            const int c = lane * 4 + u * 256;
+            if (c < cols) {
+                const float4 g = *reinterpret_cast<const float4*>(gamma + c);
+                const float4 b = *reinterpret_cast<const float4*>(beta + c);
+                track(((v[u].x - mean) * rstd) * g.x + b.x);
+                track(((v[u].y - mean) * rstd) * g.y + b.y);
+                track(((v[u].z - mean) * rstd) * g.z + b.z);
+                track(((v[u].w - mean) * rstd) * g.w + b.w);
+            }
+        }
+    }
+    range_block_store(range, lo, hi, nan);
+}
+
+__global__ __launch_bounds__(256) void layernorm_quantize_kernel(const float* __restrict__ x,
+                                                                 const float* __restrict__ gamma,
+                                                                 const float* __restrict__ beta,
+                                                                 const float* __restrict__ stats, long rows, int cols,
+                                                                 const float* __restrict__ scale,
+                                                                 const float* __restrict__ zp, float qlo, float qhi,
+                                                                 int off, int8_t* __restrict__ q) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const long row = long(blockIdx.x) * 4 + wave;
+    if (row >= rows) return;
+    const QGrid G = make_qgrid(scale[0], zp[0], qlo, qhi, true);
+    const float mean = stats[2 * row], rstd = stats[2 * row + 1];
+    const float* xr = x + row * cols;
+    int8_t* qr = q + row * cols;
+#pragma unroll
+    for (int u = 0; u < LN_KEEP; ++u) {
+        const int c = lane * 4 + u * 256;
+        if (c < cols) {
+            const float4 v = *reinterpret_cast<const float4*>(xr + c);
+            const float4 g = *reinterpret_cast<const float4*>(gamma + c);
+            const float4 b = *reinterpret_cast<const float4*>(beta + c);
+            const int c0 = int(quant_fast<false>(((v.x - mean) * rstd) * g.x + b.x, G)) + off;
+            const int c1 = int(quant_fast<false>(((v.y - mean) * rstd) * g.y + b.y, G)) + off;
+            const int c2 = int(quant_fast<false>(((v.z - mean) * rstd) * g.z + b.z, G)) + off;
+            const int c3 = int(quant_fast<false>(((v.w - mean) * rstd) * g.w + b.w, G)) + off;
+            *reinterpret_cast<uint32_t*>(qr + c) = uint32_t(c0 & 0xff) | (uint32_t(c1 & 0xff) << 8) |
+                                                   (uint32_t(c2 & 0xff) << 16) | (uint32_t(c3) << 24);
+        }
+    }
 }
 
 // ---------------------------------------------------------------- elementwise
@@ -495,6 +586,40 @@ int lq_layernorm_f32(const float* x, const float* gamma, const float* beta, floa
                long(kRangeSlots) * per_block);
     layernorm_kernel<<<unsigned((rows + per_block - 1) / per_block), 256, 0, as_stream(stream)>>>(
         x, gamma, beta, out, rows, cols, eps, range);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_layernorm_stats_f32(const float* x, const float* gamma, const float* beta, long rows, int cols, float eps,
+                           float* stats, float* range, void* stream) {
+    LQ_REQUIRE(x && gamma && beta && stats && range, LQ_ERR_VALUE, "layernorm_stats: null pointer");
+    LQ_REQUIRE(rows >= 0 && cols > 0, LQ_ERR_SHAPE, "layernorm_stats: bad shape (%ld, %d)", rows, cols);
+    LQ_REQUIRE(cols % 4 == 0 && cols <= LN_KEEP * 256 && aligned16(x) && aligned16(gamma) && aligned16(beta),
+               LQ_ERR_NOT_IMPLEMENTED,
+               "layernorm_stats: rows of %d floats; the fused form takes vector-aligned rows of a multiple of 4, "
+               "at most %d (use lq_layernorm_f32 + lq_quantize)", cols, LN_KEEP * 256);
+    if (rows == 0) return LQ_OK;
+    const long blocks = (rows + 3) / 4;
+    LQ_REQUIRE(blocks <= kRangeSlots, LQ_ERR_SHAPE, "layernorm_stats: %ld rows are too many for a kept range", rows);
+    layernorm_stats_kernel<<<unsigned(blocks), 256, 0, as_stream(stream)>>>(x, gamma, beta, rows, cols, eps, stats,
+                                                                             range);
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_layernorm_quantize_i8(const float* x, const float* gamma, const float* beta, const float* stats, long rows,
+                             int cols, const float* scale, const float* zp, int qmin, int qmax, int code_offset,
+                             int8_t* q, void* stream) {
+    LQ_REQUIRE(x && gamma && beta && stats && scale && zp && q, LQ_ERR_VALUE, "layernorm_quantize: null pointer");
+    LQ_REQUIRE(rows >= 0 && cols > 0, LQ_ERR_SHAPE, "layernorm_quantize: bad shape (%ld, %d)", rows, cols);
+    LQ_REQUIRE(cols % 4 == 0 && cols <= LN_KEEP * 256 && aligned16(x) && aligned16(gamma) && aligned16(beta) &&
+                   (reinterpret_cast<uintptr_t>(q) & 3u) == 0,
+               LQ_ERR_NOT_IMPLEMENTED, "layernorm_quantize: rows of %d floats are not what the fused form takes", cols);
+    LQ_REQUIRE(qmax > qmin && qmin + code_offset >= -128 && qmax + code_offset <= 127, LQ_ERR_VALUE,
+               "layernorm_quantize: grid [%d,%d] + offset %d does not fit int8", qmin, qmax, code_offset);
+    if (rows == 0) return LQ_OK;
+    layernorm_quantize_kernel<<<unsigned((rows + 3) / 4), 256, 0, as_stream(stream)>>>(
+        x, gamma, beta, stats, rows, cols, scale, zp, float(qmin), float(qmax), code_offset, q);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }

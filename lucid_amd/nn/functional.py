@@ -45,6 +45,33 @@ def layer_norm(x: Tensor, normalized_shape, weight: Tensor, bias: Tensor, eps: f
     return out
 
 
+def layer_norm_dynamic_quantize(x: Tensor, normalized_shape, weight: Tensor, bias: Tensor, eps: float, qdtype):
+    """``layer_norm`` followed by the per-tensor affine dynamic quantization of a
+    dynamic-quantized Linear (``dynamic/linear.py:87-92``), without storing the float32
+    result: ``(codes [rows, cols] int8, scale, zero_point)`` - the bits that ``layer_norm(...,
+    track_range=True)`` and the Linear's own quantization produce.  ``None`` when the rows are
+    not what the fused kernels take (the caller then takes the two-step route)."""
+    _require_f32_hip("layer_norm", x, weight, bias)
+    cols = normalized_shape if isinstance(normalized_shape, int) else int(normalized_shape[-1])
+    if x.shape[-1] != cols or weight.numel != cols or bias.numel != cols:
+        raise _C.ShapeMismatch(f"layer_norm: last dim {x.shape[-1]} vs normalized_shape {cols}")
+    rows = x.numel // cols
+    if cols % 4 or cols > 2048 or rows == 0 or (rows + 3) // 4 > 16384:
+        return None
+    from .quantized._utils import storage_offset
+    stats = Tensor.empty((rows, 2), T.float32, "hip")
+    rng = _new_range()
+    _C.call("lq_layernorm_stats_f32", x.data_ptr, weight.data_ptr, bias.data_ptr, rows, cols, float(eps),
+            stats.data_ptr, rng.data_ptr, None)
+    scale, zp = Tensor.empty((), T.float32, "hip"), Tensor.empty((), T.float32, "hip")
+    _C.call("lq_calc_qparams_from_range", rng.data_ptr, 0, qdtype.quant_min, qdtype.quant_max, int(qdtype.signed),
+            1e-8, scale.data_ptr, zp.data_ptr, None, None, None)
+    q = Tensor.empty((rows, cols), T.int8, "hip")
+    _C.call("lq_layernorm_quantize_i8", x.data_ptr, weight.data_ptr, bias.data_ptr, stats.data_ptr, rows, cols,
+            scale.data_ptr, zp.data_ptr, qdtype.quant_min, qdtype.quant_max, storage_offset(qdtype), q.data_ptr, None)
+    return q, scale, zp
+
+
 def gelu(x: Tensor, approximate: str = "none", track_range: bool = False) -> Tensor:
     """``F.gelu`` (``lucid/nn/functional/activations.py:219``), exact erf form."""
     if approximate != "none":

@@ -84,6 +84,16 @@ class Linear(Module):
         if not small:
             _C.call("lq_quantize", x.data_ptr, xq.data_ptr, _C.I8, off, 1, 1, x.numel,
                     x_scale.data_ptr, x_zp.data_ptr, 0, qd.quant_min, qd.quant_max, None)
+        return self.forward_quantized(xq, x_scale, x_zp, x.shape[:-1], residual, activation, track_range)
+
+    def forward_quantized(self, xq: Tensor, x_scale: Tensor, x_zp: Tensor, lead_shape, residual: Tensor | None = None,
+                          activation: str | None = None, track_range: bool = False) -> Tensor:
+        """The layer on an activation that is already quantized with this layer's activation
+        grid (``act_qdtype``, per-tensor affine, device-side ``x_scale`` / ``x_zp``): what
+        ``forward`` does after its own quantization, for a producer that writes codes directly
+        (``functional.layer_norm_dynamic_quantize``)."""
+        N = self.out_features
+        off = storage_offset(self.act_qdtype)
         if self._wsum is None:
             self._wsum = _ops.rowsum_i8(self.weight_int8)
         rng = None
@@ -94,7 +104,7 @@ class Linear(Module):
                             w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias,
                             out_mode=_ops.OUT_F32, residual=residual, gelu=activation == "gelu",
                             range_buf=rng)
-        y = y.reshape(*x.shape[:-1], N)
+        y = y.reshape(*lead_shape, N)
         y._range = rng
         return y
 

@@ -228,3 +228,47 @@ def test_vit_block_fused_and_unfused_gelu_agree(monkeypatch):
     monkeypatch.setattr(W.ViTBlock, "fuse_gelu", False)
     b = model(x).numpy()
     assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+@pytest.mark.parametrize("rows,cols", [(394, 768), (12608, 768), (5, 192), (7, 2048), (64, 4)])
+def test_layernorm_dynamic_quantize_equals_layernorm_then_quantize(rows, cols):
+    """LayerNorm that writes the next dynamic Linear's codes directly: codes, scale and zero
+    point are the bits of layer_norm(track_range) + calc_qparams_from_range + quantize."""
+    from lucid_amd import _C
+    import lucid_amd.quantization as Q
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.3).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(cols)).astype(np.float32)
+    xt, gt, bt = hip(x), hip(g), hip(b)
+    fused = F.layer_norm_dynamic_quantize(xt, cols, gt, bt, 1e-6, Q.quint8)
+    assert fused is not None
+    q, s, z = fused
+    y = F.layer_norm(xt, cols, gt, bt, 1e-6, track_range=True)
+    s2, z2 = L.Tensor.empty((), L.float32, "hip"), L.Tensor.empty((), L.float32, "hip")
+    _C.call("lq_calc_qparams_from_range", y._range.data_ptr, 0, 0, 255, 0, 1e-8, s2.data_ptr, z2.data_ptr, None, None,
+            None)
+    q2 = L.Tensor.empty((rows, cols), L.int8, "hip")
+    _C.call("lq_quantize", y.data_ptr, q2.data_ptr, _C.I8, -128, 1, 1, rows * cols, s2.data_ptr, z2.data_ptr, 0, 0, 255,
+            None)
+    assert np.array_equal(s.numpy().view(np.uint32), s2.numpy().view(np.uint32))
+    assert np.array_equal(z.numpy().view(np.uint32), z2.numpy().view(np.uint32))
+    assert np.array_equal(q.numpy(), q2.numpy())
+
+
+def test_layernorm_dynamic_quantize_declines_other_rows():
+    import lucid_amd.quantization as Q
+    x = hip(np.zeros((4, 2052), np.float32))
+    w = hip(np.ones(2052, np.float32))
+    assert F.layer_norm_dynamic_quantize(x, 2052, w, w, 1e-6, Q.quint8) is None
+
+
+def test_vit_block_with_and_without_fused_layernorm_quantize_agree(monkeypatch):
+    import workloads as W
+    cfg = dict(W.VIT_B16, depth=2, dim=192, heads=3, mlp=768)
+    model = W.QViT(cfg, seed=4)
+    x = L.tensor(np.random.default_rng(1).standard_normal((2, 3, 224, 224)).astype(np.float32), device="hip")
+    a = model(x).numpy()
+    monkeypatch.setattr(W.ViTBlock, "fuse_ln_quant", False)
+    b = model(x).numpy()
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))

@@ -235,6 +235,7 @@ def _layer_norm(w, b, eps=1e-6, track_range=True):
 
 class ViTBlock(nn.Module):
     fuse_gelu = True
+    fuse_ln_quant = True  # LayerNorm writes the next Linear's int8 codes, not float32 (same bits)
 
     def __init__(self, prefix, p, heads):
         super().__init__()
@@ -251,13 +252,26 @@ class ViTBlock(nn.Module):
 
         # every float32 kernel that feeds a dynamic-quantized Linear keeps the range of
         # what it writes; the residual adds ride in the epilogues of proj and fc2
-        a = F.scaled_dot_product_attention_qkv(self.qkv(self.norm1(x)), self.heads, track_range=True)
+        a = F.scaled_dot_product_attention_qkv(self._norm_linear(self.norm1, self.qkv, x), self.heads,
+                                               track_range=True)
         x = self.proj(a, residual=x)
         if self.fuse_gelu:  # GELU and the range of its result in fc1's epilogue (same bits, one kernel less)
-            h = self.fc1(self.norm2(x), activation="gelu", track_range=True)
+            h = self._norm_linear(self.norm2, self.fc1, x, activation="gelu", track_range=True)
         else:
-            h = F.gelu(self.fc1(self.norm2(x)), track_range=True)
+            h = F.gelu(self._norm_linear(self.norm2, self.fc1, x), track_range=True)
         return self.fc2(h, residual=x)
+
+    def _norm_linear(self, norm, lin, x, **kw):
+        """``lin(norm(x))``; with ``fuse_ln_quant`` the normalized activation goes to the Linear
+        as codes without a float32 copy in between."""
+        import lucid_amd.nn.functional as F
+
+        if self.fuse_ln_quant:
+            r = F.layer_norm_dynamic_quantize(x, norm.normalized_shape, norm.weight, norm.bias, norm.eps,
+                                              lin.act_qdtype)
+            if r is not None:
+                return lin.forward_quantized(r[0], r[1], r[2], x.shape[:-1], **kw)
+        return lin(norm(x), **kw)
 
 
 class QViT(nn.Module):
