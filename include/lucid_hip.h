@@ -169,15 +169,18 @@ int lq_lstm_cell_f32(const float* gates_x, size_t gates_x_ld, const float* gates
 /* Self-test of the tile kernels' requantize arithmetic.  Their epilogue computes
  * clamp(rint(x / scale) + zp, qmin, qmax) mostly without dividing (x * (1/scale),
  * accepted when it lies clear of every rounding boundary, the IEEE quotient
- * otherwise); this runs that routine and the plain divide-round-add-clamp of
- * quantize (lucid/quantization/_functional.py:164-182) on every float32 bit
- * pattern in [first_bits, first_bits + count) and counts the patterns whose
- * stored code would differ (*mismatches, must be 0) and those that took the
- * dividing branch (*divided).  Both counters are device memory (8 bytes each).
- * No counterpart in Lucid. */
-int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, unsigned long long first_bits,
-                              unsigned long long count, unsigned long long* mismatches,
-                              unsigned long long* divided, lq_stream stream);
+ * otherwise), with a ReLU directly before it (relu != 0) folded into the lower
+ * clamp bound, and ahead of a fused join as the code minus zp from shifted
+ * bounds.  This runs both forms of that routine and the plain [max(x, 0),]
+ * divide-round-add-clamp of quantize (lucid/quantization/_functional.py:164-182)
+ * on every float32 bit pattern in [first_bits, first_bits + count) and counts the
+ * patterns whose stored code would differ (*mismatches, must be 0) and those
+ * that took the dividing branch (*divided).  Both counters are device memory
+ * (8 bytes each).  No counterpart in Lucid. */
+int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, int relu,
+                              unsigned long long first_bits, unsigned long long count,
+                              unsigned long long* mismatches, unsigned long long* divided,
+                              lq_stream stream);
 
 /* Matrix-core rate probe for roofline accounting: 2 blocks per CU, each
  * wavefront issuing `iters` rounds of eight v_mfma_i32_32x32x32_i8 on eight

@@ -79,27 +79,41 @@ __device__ __forceinline__ float q_core(float x, float s, float z, float lo, flo
     return u;
 }
 
-// One quantization grid, with the reciprocal of its scale (see quant_fast).
+// One quantization grid, with the reciprocal of its scale (see quant_fast) and, when a ReLU
+// comes directly before the quantization, that floor folded into the bounds.
 struct QGrid {
     float s, inv, z, lo, hi;
+    float lof;       // lower bound of the multiplying route: max(lo, z) under a ReLU, else lo
+    float loc, hic;  // lof - z and hi - z: the bounds of a code taken relative to z
+    bool relu;
 };
 
 // `fast`: the kernel quantizes many elements per lane, so one division to get the
 // reciprocal pays.  A grid outside what quant_fast's argument covers (a scale outside a sane
-// range, a zero point or bounds beyond +-255) gets a NaN reciprocal, which sends every
-// element down the dividing branch.
-__device__ __forceinline__ QGrid make_qgrid(float s, float z, float lo, float hi, bool fast) {
+// range, a zero point that is not an integer, a zero point or bounds beyond +-255) gets a NaN
+// reciprocal, which sends every element down the dividing branch.
+// `relu`: the value is max(x, 0) (a NaN kept), quantized.  For s > 0 dividing and rounding are
+// monotone and take 0 to 0, so rint(max(x, 0) / s) = max(rint(x / s), 0): the floor becomes
+// the lower bound max(lo, z) of the clamp, which is right when lo <= z <= hi; any other grid
+// divides, and the dividing branch applies the floor as written.
+__device__ __forceinline__ QGrid make_qgrid(float s, float z, float lo, float hi, bool fast, bool relu = false) {
     QGrid G;
-    G.s = s, G.z = z, G.lo = lo, G.hi = hi;
+    G.s = s, G.z = z, G.lo = lo, G.hi = hi, G.relu = relu;
     const float a = __builtin_fabsf(s);
-    const bool ok = fast && a > 0x1p-60f && a < 0x1p60f && __builtin_fabsf(z) <= 255.0f &&
-                    __builtin_fabsf(lo) <= 255.0f && __builtin_fabsf(hi) <= 255.0f;
+    bool ok = fast && a > 0x1p-60f && a < 0x1p60f && __builtin_fabsf(z) <= 255.0f && z == __builtin_rintf(z) &&
+              __builtin_fabsf(lo) <= 255.0f && __builtin_fabsf(hi) <= 255.0f;
+    if (relu) ok = ok && s > 0.0f && lo <= z && z <= hi;
     G.inv = ok ? 1.0f / s : __builtin_nanf("");
+    G.lof = (relu && z > lo) ? z : lo;
+    G.loc = G.lof - z, G.hic = hi - z;
     return G;
 }
 
 // clamp(rint(x / s) + z, lo, hi) with the correctly rounded IEEE quotient, bit for bit,
-// mostly without dividing; a NaN becomes KEEP_NAN ? NaN : 0.
+// mostly without dividing; a NaN becomes KEEP_NAN ? NaN : 0.  CENTERED: the same code
+// minus z (what dequantizing it starts with), from clamp(rint(x / s), lo - z, hi - z):
+// all of these are integers far below 2^24, or the clamp decides.  (Its zero may be -0 where
+// the difference is +0: equal as a number, and the join that consumes it adds before it rounds.)
 // tp = x * fl(1/s) is within 2^-22.9 relative of the exact quotient e, and fl(x / s) within
 // 2^-24.  rint only changes value at the half-integers.
 //  * |tp| < 512: tp is within 6.2e-5 of e and fl(x / s) within 3.1e-5; when tp is farther
@@ -110,15 +124,17 @@ __device__ __forceinline__ QGrid make_qgrid(float s, float z, float lo, float hi
 //    same bound.
 // Otherwise (a few elements in ten thousand, and whatever is infinite or NaN: d = NaN
 // fails the test) the lane divides.
-template <bool KEEP_NAN>
+template <bool KEEP_NAN, bool CENTERED = false>
 __device__ __forceinline__ float quant_fast(float x, const QGrid& G) {
     const float tp = x * G.inv;
     const float r = __builtin_rintf(tp);
     const float d = tp - r;  // exact where it matters
-    float c = __builtin_amdgcn_fmed3f(r + G.z, G.lo, G.hi);
+    float c = CENTERED ? __builtin_amdgcn_fmed3f(r, G.loc, G.hic) : __builtin_amdgcn_fmed3f(r + G.z, G.lof, G.hi);
     if (__builtin_expect(!(__builtin_fabsf(d) < 0.5f - 0x1p-12f), 0)) {
-        const float u = __builtin_rintf(x / G.s) + G.z;
+        const float xr = (G.relu && x < 0.0f) ? 0.0f : x;
+        const float u = __builtin_rintf(xr / G.s) + G.z;
         c = (u != u) ? (KEEP_NAN ? u : 0.0f) : __builtin_amdgcn_fmed3f(u, G.lo, G.hi);
+        if (CENTERED) c = c - G.z;
     }
     return c;
 }
@@ -128,8 +144,9 @@ __device__ __forceinline__ float quant_fast(float x, const QGrid& G) {
 // compile-time constant so that each output form gets a tight loop.
 // epilogue_value returns the element as 32 bits: float bits, the integer for the
 // accumulator / requantized-code forms, or - ahead of a fused join - the requantized
-// code still as a float (finish_value / join_code take it from there); store_*
-// narrows and writes.
+// code minus its zero point, as a float (finish_value / join_code take it from there);
+// store_* narrows and writes.  G was made with relu = g.relu: the requantizing forms
+// leave the floor to it.
 template <int MODE>
 __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t acc, float as,
                                                    const ColParams& c, const QGrid& G) {
@@ -138,21 +155,21 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
     float sc = as * c.ws;
     float y = f * sc;
     y = y + c.bias;
+    if (MODE == OUT_REQUANT_JOIN) return __float_as_uint(quant_fast<false, true>(y, G));
+    // the stored form adds out_offset: store_* does, on the packed bytes where it can
+    if (MODE == OUT_REQUANT_I8) return uint32_t(int(quant_fast<false>(y, G)));
+    // not the centered form: its -0 (from rint(x / s) = -0) would survive the multiplication
+    if (MODE == OUT_FAKEQUANT_F32) return __float_as_uint((quant_fast<true>(y, G) - G.z) * G.s);
     // ReLU as a floor of 0, no ReLU as a floor of -inf: one compare and select either
     // way (a NaN fails the compare and passes through, as in the CPU formulation)
     const float floor = g.relu ? 0.0f : -__builtin_inff();
     y = (y < floor) ? floor : y;
-    if (MODE == OUT_F32 || MODE == OUT_F16) return __float_as_uint(y);
     if (MODE == OUT_F32X) {
         // GELU, erf form (lucid/nn/functional/activations.py:219): the expression of the
         // stand-alone kernel, so fusing it changes no bit
         if (g.gelu) y = (0.5f * y) * (1.0f + erf_as(y * 0.70710678118654752440f));
-        return __float_as_uint(y);
     }
-    if (MODE == OUT_REQUANT_JOIN) return __float_as_uint(quant_fast<false>(y, G));
-    // the stored form adds out_offset: store_* does, on the packed bytes where it can
-    if (MODE == OUT_REQUANT_I8) return uint32_t(int(quant_fast<false>(y, G)));
-    return __float_as_uint((quant_fast<true>(y, G) - G.z) * G.s);  // OUT_FAKEQUANT_F32
+    return __float_as_uint(y);
 }
 
 // y + residual[m, n] for the float output forms (x + linear(...), the residual
@@ -168,27 +185,38 @@ __device__ __forceinline__ uint32_t add_residual(const GemmArgs& g, uint32_t bit
 // to this layer's output): both operands are dequantized in float32 with their own
 // grids, added, optionally clamped at zero, and requantized.
 struct JoinParams {
-    float S1, Z1;  // this layer's output grid
-    float s2, z2;  // the other operand's grid
-    QGrid out;     // the join's output grid
+    float S1;       // this layer's output scale (its code arrives minus the zero point)
+    float s2, z2;   // the other operand's grid
+    float k2;       // 128 + join_off + z2: what takes a stored byte + 128 to code - z2
+    bool k2_exact;  // ... in one exact subtraction (an integer zero point of sane size)
+    QGrid out;      // the join's output grid, with the join's ReLU
 };
 
 __device__ __forceinline__ JoinParams load_join(const GemmArgs& g, const QGrid& G, bool fast) {
     JoinParams jp;
-    jp.S1 = G.s, jp.Z1 = G.z;
+    jp.S1 = G.s;
     jp.s2 = g.join_scale[0], jp.z2 = g.join_zp[0];
-    jp.out = make_qgrid(g.join_out_scale[0], g.join_out_zp[0], float(g.join_out_qmin), float(g.join_out_qmax), fast);
+    jp.k2 = float(128 + g.join_off) + jp.z2;
+    jp.k2_exact = jp.z2 == __builtin_rintf(jp.z2) && __builtin_fabsf(jp.z2) <= 0x1p20f && g.join_off >= -(1 << 20) &&
+                  g.join_off <= (1 << 20);
+    jp.out = make_qgrid(g.join_out_scale[0], g.join_out_zp[0], float(g.join_out_qmin), float(g.join_out_qmax), fast,
+                        g.join_relu != 0);
     return jp;
 }
 
-// bits: this layer's requantized code as a float (what epilogue_value<OUT_REQUANT_JOIN>
-// returned); other: the partner's stored code
+// bits: this layer's requantized code minus its zero point, as a float (what
+// epilogue_value<OUT_REQUANT_JOIN> returned); other: the partner's stored code
 __device__ __forceinline__ uint32_t join_code(const GemmArgs& g, const JoinParams& jp, uint32_t bits, int other) {
-    const float x1 = (__uint_as_float(bits) - jp.Z1) * jp.S1;
+    const float x1 = __uint_as_float(bits) * jp.S1;
     const float x2 = (float(other - g.join_off) - jp.z2) * jp.s2;
-    float y = x1 + x2;
-    if (g.join_relu) y = (y < 0.0f) ? 0.0f : y;
-    return uint32_t(int(quant_fast<false>(y, jp.out)));  // store_* adds join_out_offset
+    return uint32_t(int(quant_fast<false>(x1 + x2, jp.out)));  // store_* adds join_out_offset
+}
+
+// The same with the partner's stored byte + 128 (0..255) already a float; needs jp.k2_exact.
+__device__ __forceinline__ uint32_t join_code_biased(const JoinParams& jp, uint32_t bits, float other_biased) {
+    const float x1 = __uint_as_float(bits) * jp.S1;
+    const float x2 = (other_biased - jp.k2) * jp.s2;
+    return uint32_t(int(quant_fast<false>(x1 + x2, jp.out)));
 }
 
 // one element's residual step, whichever form the output mode has
@@ -248,7 +276,7 @@ template <int MODE>
 __device__ __forceinline__ void epilogue_store_t(const GemmArgs& g, int m, int n, int32_t acc,
                                                  float as, const ColParams& c, float S, float Z) {
     // one element per call: no reciprocal, the grid divides
-    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), false);
+    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), false, g.relu != 0);
     store_scalar<MODE>(g, size_t(m) * size_t(g.ldo) + size_t(n),
                        finish_value<MODE>(g, epilogue_value<MODE>(g, acc, as, c, G), m, n, G));
 }

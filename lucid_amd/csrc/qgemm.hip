@@ -489,21 +489,26 @@ int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t 
 namespace {
 
 // x = every float32 bit pattern of [first, first + count): the tile epilogue's requantize
-// (quant_fast: reciprocal multiply with a guard band, division for the rest) against the plain
+// (quant_fast: reciprocal multiply with a guard band, division for the rest), in both of its
+// forms (the code, and the code minus the zero point), against the plain [floor at zero,]
 // divide-round-add-clamp, compared as the codes the two would store.
-__global__ __launch_bounds__(256) void quant_route_check_kernel(float s, float z, float lo, float hi,
+__global__ __launch_bounds__(256) void quant_route_check_kernel(float s, float z, float lo, float hi, int relu,
                                                                 unsigned long long first,
                                                                 unsigned long long count,
                                                                 unsigned long long* mismatches,
                                                                 unsigned long long* divided) {
-    const lq::QGrid G = lq::make_qgrid(s, z, lo, hi, true);
+    const lq::QGrid G = lq::make_qgrid(s, z, lo, hi, true, relu != 0);
     unsigned long long bad = 0, slow = 0;
     for (unsigned long long i = blockIdx.x * 256ull + threadIdx.x; i < count; i += gridDim.x * 256ull) {
         const float x = __uint_as_float(unsigned(first + i));
         const float fast = lq::quant_fast<false>(x, G);
-        const float u = lq::q_core(x, s, z, lo, hi);
+        const float centered = lq::quant_fast<false, true>(x, G);
+        const float xr = (relu && x < 0.0f) ? 0.0f : x;
+        const float u = lq::q_core(xr, s, z, lo, hi);
         const float plain = (u != u) ? 0.0f : u;
-        bad += __float_as_uint(fast) != __float_as_uint(plain) && !(fast == 0.0f && plain == 0.0f);
+        const float plain_c = plain - z;
+        bad += (__float_as_uint(fast) != __float_as_uint(plain) && !(fast == 0.0f && plain == 0.0f)) ||
+               (__float_as_uint(centered) != __float_as_uint(plain_c) && !(centered == 0.0f && plain_c == 0.0f));
         const float tp = x * G.inv;
         slow += !(__builtin_fabsf(tp - __builtin_rintf(tp)) < 0.5f - 0x1p-12f);
     }
@@ -515,7 +520,7 @@ __global__ __launch_bounds__(256) void quant_route_check_kernel(float s, float z
 
 extern "C" {
 
-int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, unsigned long long first_bits,
+int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, int relu, unsigned long long first_bits,
                               unsigned long long count, unsigned long long* mismatches,
                               unsigned long long* divided, lq_stream stream) {
     LQ_REQUIRE(mismatches && divided, LQ_ERR_VALUE, "selftest_requant_route: NULL counter");
@@ -526,7 +531,7 @@ int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, unsigne
     if (rc) return rc;
     if (count == 0) return LQ_OK;
     hipLaunchKernelGGL(quant_route_check_kernel, dim3(4096), dim3(256), 0, st, scale, zp, float(qmin), float(qmax),
-                       first_bits, count, mismatches, divided);
+                       relu, first_bits, count, mismatches, divided);
     LQ_CHECK_LAUNCH("selftest_requant_route");
     return LQ_OK;
 }

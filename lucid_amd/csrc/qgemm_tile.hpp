@@ -108,9 +108,12 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
     const bool vec_ok = (g.ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0);
     const int row0 = lane / QUADS_PER_ROW, cq = (lane % QUADS_PER_ROW) * 4;
     constexpr bool kRequant = MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN || MODE == OUT_FAKEQUANT_F32;
-    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), kRequant);
+    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), kRequant, g.relu != 0);
     JoinParams jp;
-    if (MODE == OUT_REQUANT_JOIN) jp = load_join(g, G, true);
+    if (MODE == OUT_REQUANT_JOIN) {
+        jp = load_join(g, G, true);
+        interior = interior && jp.k2_exact;  // the vector path subtracts the partner's offsets in one step
+    }
     // running range of what this lane stores (float32 output with a kept range only)
     const bool keep = MODE == OUT_F32X && g.range != nullptr;
     auto track = [&](uint32_t bits) {
@@ -182,10 +185,11 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                 if (MODE == OUT_REQUANT_JOIN && join_fast) {
 #pragma unroll
                     for (int p = 0; p < PASSES; ++p) {
-                        v[p].x = join_code(g, jp, v[p].x, int(int8_t(jv[p] & 0xff)));
-                        v[p].y = join_code(g, jp, v[p].y, int(int8_t((jv[p] >> 8) & 0xff)));
-                        v[p].z = join_code(g, jp, v[p].z, int(int8_t((jv[p] >> 16) & 0xff)));
-                        v[p].w = join_code(g, jp, v[p].w, int(int8_t(jv[p] >> 24)));
+                        const uint32_t b = jv[p] ^ 0x80808080u;  // stored bytes + 128, all four
+                        v[p].x = join_code_biased(jp, v[p].x, float(b & 0xffu));
+                        v[p].y = join_code_biased(jp, v[p].y, float((b >> 8) & 0xffu));
+                        v[p].z = join_code_biased(jp, v[p].z, float((b >> 16) & 0xffu));
+                        v[p].w = join_code_biased(jp, v[p].w, float(b >> 24));
                     }
                 }
                 if (MODE == OUT_F32X && keep) {

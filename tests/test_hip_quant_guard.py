@@ -65,24 +65,33 @@ def test_scaled_normal_data_many_scales():
     assert np.array_equal(got, O.quantize(x, s, z, -128, 127, ch_axis=0))
 
 
+@pytest.mark.parametrize("relu", [0, 1])
 @pytest.mark.parametrize("scale,zp,qmin,qmax", [
     (0.05, 0.0, -128, 127), (0.037, 128.0, 0, 255), (1.0, -5.0, -128, 127), (0.5, 3.0, 0, 255),
     (3.0, 0.0, -128, 127), (0.1, 64.0, 0, 255), (7.3e-4, 17.0, 0, 255), (0.0314, 64.0, 0, 255),
-    (1e-30, 0.0, -128, 127), (1e30, 0.0, -128, 127), (0.02, 300.0, 0, 255), (-0.25, 0.0, -128, 127)])
-def test_tile_epilogue_requantize_route_on_every_float32(scale, zp, qmin, qmax):
+    (1e-30, 0.0, -128, 127), (1e30, 0.0, -128, 127), (0.02, 300.0, 0, 255), (-0.25, 0.0, -128, 127),
+    (0.04, -3.0, 0, 255), (0.04, 200.0, -128, 127), (0.04, 0.5, -128, 127), (0.04, 255.0, 0, 255),
+    (0.04, -128.0, -128, 127)])
+def test_tile_epilogue_requantize_route_on_every_float32(scale, zp, qmin, qmax, relu):
     """The GEMM / convolution epilogue requantizes through a reciprocal multiply where that is
-    provably the same and divides elsewhere.  Every one of the 2^32 float32 bit patterns (all
-    finite values, both zeros, subnormals, infinities, every NaN) must give the code that the
-    plain quantize arithmetic gives.  A tiny or huge scale and a zero point beyond 255 are
-    outside what the reciprocal route accepts: there every pattern must take the dividing
-    branch (a negative scale is accepted like a positive one)."""
+    provably the same and divides elsewhere; a ReLU directly before it is folded into the lower
+    clamp bound, and a fused join takes the code minus its zero point from shifted bounds.
+    Every one of the 2^32 float32 bit patterns (all finite values, both zeros, subnormals,
+    infinities, every NaN) must give, in both forms, the code that the plain [floor at zero,]
+    divide-round-add-clamp gives.  A tiny or huge scale, a zero point beyond 255 or not an
+    integer are outside what the reciprocal route accepts, and under a ReLU so are a negative
+    scale and a zero point outside the code range: there every pattern must take the dividing
+    branch (without a ReLU a negative scale is accepted like a positive one)."""
     from lucid_amd import _C
     bad = L.Tensor.empty((1,), L.int64, "hip")
     slow = L.Tensor.empty((1,), L.int64, "hip")
-    _C.call("lq_selftest_requant_route", scale, zp, qmin, qmax, 0, 1 << 32, bad.data_ptr, slow.data_ptr, None)
+    _C.call("lq_selftest_requant_route", scale, zp, qmin, qmax, relu, 0, 1 << 32, bad.data_ptr, slow.data_ptr, None)
     assert int(bad.numpy()[0]) == 0
     divided = int(slow.numpy()[0])
-    if abs(scale) < 1e-20 or abs(scale) > 1e20 or abs(zp) > 255:
+    refused = abs(scale) < 1e-20 or abs(scale) > 1e20 or abs(zp) > 255 or zp != round(zp)
+    if relu:
+        refused = refused or scale < 0 or not (qmin <= zp <= qmax)
+    if refused:
         assert divided == 1 << 32
     else:
         # NaNs, infinities and the huge-quotient tail always divide; of the rest only a sliver
@@ -91,7 +100,7 @@ def test_tile_epilogue_requantize_route_on_every_float32(scale, zp, qmin, qmax):
 
 def test_tile_epilogue_requantize_route_random_grids():
     """The same exhaustive comparison on 48 random grids (scales log-uniform in 1e-5..1e2,
-    integer zero points, both code ranges)."""
+    integer zero points, both code ranges, with and without the folded ReLU)."""
     from lucid_amd import _C
     rng = np.random.default_rng(2024)
     bad = L.Tensor.empty((1,), L.int64, "hip")
@@ -101,5 +110,7 @@ def test_tile_epilogue_requantize_route_random_grids():
         signed = bool(i % 2)
         qmin, qmax = (-128, 127) if signed else (0, 255)
         zp = float(rng.integers(qmin, qmax + 1))
-        _C.call("lq_selftest_requant_route", scale, zp, qmin, qmax, 0, 1 << 32, bad.data_ptr, slow.data_ptr, None)
-        assert int(bad.numpy()[0]) == 0, (scale, zp, qmin, qmax)
+        relu = (i // 2) % 2
+        _C.call("lq_selftest_requant_route", scale, zp, qmin, qmax, relu, 0, 1 << 32, bad.data_ptr, slow.data_ptr,
+                None)
+        assert int(bad.numpy()[0]) == 0, (scale, zp, qmin, qmax, relu)
