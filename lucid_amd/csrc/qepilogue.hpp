@@ -147,12 +147,13 @@ __device__ __forceinline__ float quant_fast(float x, const QGrid& G) {
 // code minus its zero point, as a float (finish_value / join_code take it from there);
 // store_* narrows and writes.  G was made with relu = g.relu: the requantizing forms
 // leave the floor to it.
-template <int MODE>
+// PRESCALED: c.ws already holds as * ws (one activation scale for all rows).
+template <int MODE, bool PRESCALED = false>
 __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t acc, float as,
                                                    const ColParams& c, const QGrid& G) {
     if (MODE == OUT_ACC_I32) return uint32_t(acc);
     float f = float(acc - c.corr);
-    float sc = as * c.ws;
+    float sc = PRESCALED ? c.ws : as * c.ws;
     float y = f * sc;
     y = y + c.bias;
     if (MODE == OUT_REQUANT_JOIN) return __float_as_uint(quant_fast<false, true>(y, G));

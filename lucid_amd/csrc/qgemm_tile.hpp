@@ -90,13 +90,14 @@ __device__ __forceinline__ void wave_lds_sync() {
 // band is turned through a wavefront-private LDS area so that a lane ends up
 // with four consecutive columns of one row and the wavefront writes contiguous
 // row segments.  `interior` (uniform): the whole tile lies inside the output
-// and rows are vector-aligned, so the stores need no per-lane tests.
+// and rows are vector-aligned, so the stores need no per-lane tests.  `prescaled`
+// (uniform): cp[].ws already carries the (single) activation scale, s_as is not read.
 template <class Cfg, int MODE>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg::TM][Cfg::TN],
                                               const ColParams (&cp)[Cfg::TN], const float* s_as,
                                               uint32_t* stage, int m0, int n0, int n_limit, int wm,
                                               int wn, int lane, float S, float Z, bool interior,
-                                              float& r_lo, float& r_hi, int& r_nan) {
+                                              bool prescaled, float& r_lo, float& r_hi, int& r_nan) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, STRIDE = Cfg::STAGE_STRIDE;
     constexpr int QUADS_PER_ROW = TN * 8;            // four-column groups per staged row
     constexpr int EPI_ROWS = Cfg::EPI_ROWS;          // rows staged at a time (32 or 16)
@@ -149,20 +150,32 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                     jv[p] = *reinterpret_cast<const uint32_t*>(jq + size_t(p) * ROWS_PER_PASS * size_t(g.join_ld));
             }
             // this lane's rows of the part: groups of four consecutive rows
-            float as[RPP];
+            if (prescaled) {
 #pragma unroll
-            for (int q = 0; q < RPP / 4; ++q) {
-                const float4 v = *reinterpret_cast<const float4*>(s_as + band + 8 * q + 4 * (lane >> 5));
-                as[4 * q] = v.x, as[4 * q + 1] = v.y, as[4 * q + 2] = v.z, as[4 * q + 3] = v.w;
-            }
+                for (int rr = 0; rr < RPP; ++rr) {
+                    const int r = part * RPP + rr;
+                    const int row = 8 * (rr >> 2) + 4 * (lane >> 5) + (rr & 3);  // row within the staged part
 #pragma unroll
-            for (int rr = 0; rr < RPP; ++rr) {
-                const int r = part * RPP + rr;
-                const int row = 8 * (rr >> 2) + 4 * (lane >> 5) + (rr & 3);  // row within the staged part
+                    for (int j = 0; j < TN; ++j)
+                        stage[row * STRIDE + j * 32 + (lane & 31)] =
+                            epilogue_value<MODE, true>(g, acc[i][j][r], 1.0f, cp[j], G);
+                }
+            } else {
+                float as[RPP];
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    stage[row * STRIDE + j * 32 + (lane & 31)] =
-                        epilogue_value<MODE>(g, acc[i][j][r], as[rr], cp[j], G);
+                for (int q = 0; q < RPP / 4; ++q) {
+                    const float4 v = *reinterpret_cast<const float4*>(s_as + band + 8 * q + 4 * (lane >> 5));
+                    as[4 * q] = v.x, as[4 * q + 1] = v.y, as[4 * q + 2] = v.z, as[4 * q + 3] = v.w;
+                }
+#pragma unroll
+                for (int rr = 0; rr < RPP; ++rr) {
+                    const int r = part * RPP + rr;
+                    const int row = 8 * (rr >> 2) + 4 * (lane >> 5) + (rr & 3);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        stage[row * STRIDE + j * 32 + (lane & 31)] =
+                            epilogue_value<MODE, false>(g, acc[i][j][r], as[rr], cp[j], G);
+                }
             }
             wave_lds_sync();
             const uint32_t* src = stage + row0 * STRIDE + cq;
@@ -602,8 +615,16 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         __syncthreads();
         float r_lo = __builtin_inff(), r_hi = -__builtin_inff();
         int r_nan = 0;
-        tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z, interior, r_lo,
-                                 r_hi, r_nan);
+        // one activation scale for all rows (always so for a convolution): the kernels that
+        // write codes fold it into the column scales (as * ws, the product every element would
+        // form) and save each element that multiplication
+        const bool prescaled = (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) && (CONV || !g.a_scale_per_row);
+        if (prescaled) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) cp[j].ws = as_mine * cp[j].ws;
+        }
+        tile_epilogue<Cfg, MODE>(g, acc, cp, s_as, stage, m0, n0, n_limit, wm, wn, lane, S, Z, interior, prescaled,
+                                 r_lo, r_hi, r_nan);
         __syncthreads();  // the staging area is the next tile's first LDS stage
         // one block per tile here (the launcher sees to it), so the block's slot is the tile's
         if (MODE == OUT_F32X && !SK && g.range != nullptr) range_block_store(g.range, r_lo, r_hi, r_nan);
