@@ -170,8 +170,9 @@ int lq_lstm_cell_f32(const float* gates_x, size_t gates_x_ld, const float* gates
  * clamp(rint(x / scale) + zp, qmin, qmax) mostly without dividing (x * (1/scale),
  * accepted when it lies clear of every rounding boundary, the IEEE quotient
  * otherwise), with a ReLU directly before it (relu != 0) folded into the lower
- * clamp bound, and ahead of a fused join as the code minus zp from shifted
- * bounds.  This runs both forms of that routine and the plain [max(x, 0),]
+ * clamp bound, ahead of a fused join as the code minus zp from shifted bounds,
+ * and for packing as the code shifted into 0..255.  This runs those forms of
+ * the routine and the plain [max(x, 0),]
  * divide-round-add-clamp of quantize (lucid/quantization/_functional.py:164-182)
  * on every float32 bit pattern in [first_bits, first_bits + count) and counts the
  * patterns whose stored code would differ (*mismatches, must be 0) and those

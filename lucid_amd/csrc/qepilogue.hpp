@@ -82,9 +82,11 @@ __device__ __forceinline__ float q_core(float x, float s, float z, float lo, flo
 // One quantization grid, with the reciprocal of its scale (see quant_fast) and, when a ReLU
 // comes directly before the quantization, that floor folded into the bounds.
 struct QGrid {
-    float s, inv, z, lo, hi;
+    float s, inv, z, lo, hi;  // z, lo, hi include `bias`
     float lof;       // lower bound of the multiplying route: max(lo, z) under a ReLU, else lo
     float loc, hic;  // lof - z and hi - z: the bounds of a code taken relative to z
+    float bias;      // 0, or 128 for a signed range: codes come out as code + bias, in 0..255
+    bool in_byte;    // ... so that four of them pack with v_cvt_pk_u8_f32 (see CodePack)
     bool relu;
 };
 
@@ -96,8 +98,18 @@ struct QGrid {
 // monotone and take 0 to 0, so rint(max(x, 0) / s) = max(rint(x / s), 0): the floor becomes
 // the lower bound max(lo, z) of the clamp, which is right when lo <= z <= hi; any other grid
 // divides, and the dividing branch applies the floor as written.
-__device__ __forceinline__ QGrid make_qgrid(float s, float z, float lo, float hi, bool fast, bool relu = false) {
+// `biased`: the codes are wanted as code + 128 (signed range) or code + 0, within 0..255, so
+// that they can be packed as unsigned bytes; the shift goes into z, lo and hi (small
+// integers: nothing rounds).  A range that does not fit a byte, or a zero point that is not a
+// small integer, stays unshifted with in_byte false.
+__device__ __forceinline__ QGrid make_qgrid(float s, float z, float lo, float hi, bool fast, bool relu = false,
+                                            bool biased = false) {
     QGrid G;
+    const bool z_int = z == __builtin_rintf(z) && __builtin_fabsf(z) <= 255.0f;
+    const float b = lo < 0.0f ? 128.0f : 0.0f;
+    G.in_byte = biased && z_int && lo <= hi && lo + b >= 0.0f && hi + b <= 255.0f;
+    G.bias = G.in_byte ? b : 0.0f;
+    z += G.bias, lo += G.bias, hi += G.bias;
     G.s = s, G.z = z, G.lo = lo, G.hi = hi, G.relu = relu;
     const float a = __builtin_fabsf(s);
     bool ok = fast && a > 0x1p-60f && a < 0x1p60f && __builtin_fabsf(z) <= 255.0f && z == __builtin_rintf(z) &&
@@ -110,7 +122,7 @@ __device__ __forceinline__ QGrid make_qgrid(float s, float z, float lo, float hi
 }
 
 // clamp(rint(x / s) + z, lo, hi) with the correctly rounded IEEE quotient, bit for bit,
-// mostly without dividing; a NaN becomes KEEP_NAN ? NaN : 0.  CENTERED: the same code
+// mostly without dividing; a NaN becomes KEEP_NAN ? NaN : 0 (all plus G.bias).  CENTERED: the same code
 // minus z (what dequantizing it starts with), from clamp(rint(x / s), lo - z, hi - z):
 // all of these are integers far below 2^24, or the clamp decides.  (Its zero may be -0 where
 // the difference is +0: equal as a number, and the join that consumes it adds before it rounds.)
@@ -133,7 +145,7 @@ __device__ __forceinline__ float quant_fast(float x, const QGrid& G) {
     if (__builtin_expect(!(__builtin_fabsf(d) < 0.5f - 0x1p-12f), 0)) {
         const float xr = (G.relu && x < 0.0f) ? 0.0f : x;
         const float u = __builtin_rintf(xr / G.s) + G.z;
-        c = (u != u) ? (KEEP_NAN ? u : 0.0f) : __builtin_amdgcn_fmed3f(u, G.lo, G.hi);
+        c = (u != u) ? (KEEP_NAN ? u : G.bias) : __builtin_amdgcn_fmed3f(u, G.lo, G.hi);
         if (CENTERED) c = c - G.z;
     }
     return c;
@@ -142,10 +154,10 @@ __device__ __forceinline__ float quant_fast(float x, const QGrid& G) {
 // One output element.  Float steps are separate (no FMA) and in the order the
 // CPU restatement uses, so results are bit-identical to it.  MODE is a
 // compile-time constant so that each output form gets a tight loop.
-// epilogue_value returns the element as 32 bits: float bits, the integer for the
-// accumulator / requantized-code forms, or - ahead of a fused join - the requantized
-// code minus its zero point, as a float (finish_value / join_code take it from there);
-// store_* narrows and writes.  G was made with relu = g.relu: the requantizing forms
+// epilogue_value returns the element as 32 bits: float bits, the integer accumulator,
+// the requantized code as a float (plus G.bias) or - ahead of a fused join - that code
+// minus its zero point (finish_value / join_code take it from there); store_* narrows
+// and writes.  G was made with relu = g.relu: the requantizing forms
 // leave the floor to it.
 // PRESCALED: c.ws already holds as * ws (one activation scale for all rows).
 template <int MODE, bool PRESCALED = false>
@@ -157,8 +169,8 @@ __device__ __forceinline__ uint32_t epilogue_value(const GemmArgs& g, int32_t ac
     float y = f * sc;
     y = y + c.bias;
     if (MODE == OUT_REQUANT_JOIN) return __float_as_uint(quant_fast<false, true>(y, G));
-    // the stored form adds out_offset: store_* does, on the packed bytes where it can
-    if (MODE == OUT_REQUANT_I8) return uint32_t(int(quant_fast<false>(y, G)));
+    // still a float (plus G.bias): store_* narrows it and adds out_offset
+    if (MODE == OUT_REQUANT_I8) return __float_as_uint(quant_fast<false>(y, G));
     // not the centered form: its -0 (from rint(x / s) = -0) would survive the multiplication
     if (MODE == OUT_FAKEQUANT_F32) return __float_as_uint((quant_fast<true>(y, G) - G.z) * G.s);
     // ReLU as a floor of 0, no ReLU as a floor of -inf: one compare and select either
@@ -201,7 +213,7 @@ __device__ __forceinline__ JoinParams load_join(const GemmArgs& g, const QGrid& 
     jp.k2_exact = jp.z2 == __builtin_rintf(jp.z2) && __builtin_fabsf(jp.z2) <= 0x1p20f && g.join_off >= -(1 << 20) &&
                   g.join_off <= (1 << 20);
     jp.out = make_qgrid(g.join_out_scale[0], g.join_out_zp[0], float(g.join_out_qmin), float(g.join_out_qmax), fast,
-                        g.join_relu != 0);
+                        g.join_relu != 0, fast);
     return jp;
 }
 
@@ -210,62 +222,74 @@ __device__ __forceinline__ JoinParams load_join(const GemmArgs& g, const QGrid& 
 __device__ __forceinline__ uint32_t join_code(const GemmArgs& g, const JoinParams& jp, uint32_t bits, int other) {
     const float x1 = __uint_as_float(bits) * jp.S1;
     const float x2 = (float(other - g.join_off) - jp.z2) * jp.s2;
-    return uint32_t(int(quant_fast<false>(x1 + x2, jp.out)));  // store_* adds join_out_offset
+    return __float_as_uint(quant_fast<false>(x1 + x2, jp.out));  // store_* narrows, adds join_out_offset
 }
 
 // The same with the partner's stored byte + 128 (0..255) already a float; needs jp.k2_exact.
 __device__ __forceinline__ uint32_t join_code_biased(const JoinParams& jp, uint32_t bits, float other_biased) {
     const float x1 = __uint_as_float(bits) * jp.S1;
     const float x2 = (other_biased - jp.k2) * jp.s2;
-    return uint32_t(int(quant_fast<false>(x1 + x2, jp.out)));
+    return __float_as_uint(quant_fast<false>(x1 + x2, jp.out));
 }
 
-// one element's residual step, whichever form the output mode has
+// one element's residual step, whichever form the output mode has (jp: read by the join only)
 template <int MODE>
-__device__ __forceinline__ uint32_t finish_value(const GemmArgs& g, uint32_t bits, int m, int n, const QGrid& G) {
-    if (MODE == OUT_REQUANT_JOIN) {
-        const JoinParams jp = load_join(g, G, false);
+__device__ __forceinline__ uint32_t finish_value(const GemmArgs& g, uint32_t bits, int m, int n, const JoinParams& jp) {
+    if (MODE == OUT_REQUANT_JOIN)
         return join_code(g, jp, bits, int(g.join_q[size_t(m) * size_t(g.join_ld) + size_t(n)]));
-    }
     return add_residual<MODE>(g, bits, m, n);
 }
 
-// Codes leave epilogue_value / join_code without their storage offset (-128 for the quint8
-// form, else 0); it is added here, to four packed bytes at once where it is 0 or +-128.
+// Codes leave epilogue_value / join_code as floats, plus the grid's bias and without their
+// storage offset (-128 for the quint8 form, else 0).  stored byte = (value - bias + offset)
+// mod 256: when the values lie in 0..255 and offset - bias is 0 or +-128 modulo 256, four of
+// them are converted and packed by v_cvt_pk_u8_f32 and the offset is an XOR on the dword.
+struct CodePack {
+    int add;        // offset - bias
+    uint32_t flip;  // 0x80808080 when add is 128 modulo 256
+    bool pk;        // the packed route applies
+};
+
 template <int MODE>
-__device__ __forceinline__ int code_offset(const GemmArgs& g) {
-    return MODE == OUT_REQUANT_JOIN ? g.join_out_offset : g.out_offset;
+__device__ __forceinline__ CodePack make_code_pack(const GemmArgs& g, const QGrid& G) {
+    CodePack c;
+    c.add = (MODE == OUT_REQUANT_JOIN ? g.join_out_offset : g.out_offset) - int(G.bias);
+    c.pk = G.in_byte && (c.add & 0x7f) == 0;
+    c.flip = (c.add & 0x80) ? 0x80808080u : 0u;
+    return c;
 }
 
 template <int MODE>
-__device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint32_t v) {
+__device__ __forceinline__ void store_scalar(const GemmArgs& g, size_t idx, uint32_t v, const CodePack& cpk) {
     if (MODE == OUT_F16)
         static_cast<_Float16*>(g.out)[idx] = _Float16(__uint_as_float(v));
     else if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN)
-        static_cast<int8_t*>(g.out)[idx] = int8_t(int(v) + code_offset<MODE>(g));
+        static_cast<int8_t*>(g.out)[idx] = int8_t(int(__uint_as_float(v)) + cpk.add);
     else
         static_cast<uint32_t*>(g.out)[idx] = v;  // f32 / i32 bit patterns
 }
 
 // four consecutive elements; idx is a multiple of 4 and the row is 4-aligned
 template <int MODE>
-__device__ __forceinline__ void store_vec4(const GemmArgs& g, size_t idx, uint4 v) {
+__device__ __forceinline__ void store_vec4(const GemmArgs& g, size_t idx, uint4 v, const CodePack& cpk) {
     if (MODE == OUT_F16) {
         typedef _Float16 h4 __attribute__((ext_vector_type(4)));
         h4 h = {_Float16(__uint_as_float(v.x)), _Float16(__uint_as_float(v.y)),
                 _Float16(__uint_as_float(v.z)), _Float16(__uint_as_float(v.w))};
         *reinterpret_cast<h4*>(static_cast<_Float16*>(g.out) + idx) = h;
     } else if (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) {
-        // low bytes of x, y, z, w -> one dword (byte selectors 0-3: second operand, 4-7: first)
-        const uint32_t xy = __builtin_amdgcn_perm(v.y, v.x, 0x0c0c0400u);
-        const uint32_t zw = __builtin_amdgcn_perm(v.w, v.z, 0x0c0c0400u);
-        uint32_t packed = __builtin_amdgcn_perm(zw, xy, 0x05040100u);
-        const int off = code_offset<MODE>(g);
-        if ((off & 0x7f) == 0) {
-            if (off & 0x80) packed ^= 0x80808080u;  // +-128 modulo 256, byte by byte
+        uint32_t packed;
+        if (cpk.pk) {
+            packed = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(v.x), 0, 0u);
+            packed = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(v.y), 1, packed);
+            packed = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(v.z), 2, packed);
+            packed = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(v.w), 3, packed);
+            packed ^= cpk.flip;
         } else {
-            const uint32_t o = uint32_t(off);
-            packed = ((v.x + o) & 0xffu) | (((v.y + o) & 0xffu) << 8) | (((v.z + o) & 0xffu) << 16) | ((v.w + o) << 24);
+            const uint32_t o = uint32_t(cpk.add);
+            const uint32_t x = uint32_t(int(__uint_as_float(v.x))), y = uint32_t(int(__uint_as_float(v.y)));
+            const uint32_t z = uint32_t(int(__uint_as_float(v.z))), w = uint32_t(int(__uint_as_float(v.w)));
+            packed = ((x + o) & 0xffu) | (((y + o) & 0xffu) << 8) | (((z + o) & 0xffu) << 16) | ((w + o) << 24);
         }
         *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(g.out) + idx) = packed;
     } else {
@@ -278,8 +302,11 @@ __device__ __forceinline__ void epilogue_store_t(const GemmArgs& g, int m, int n
                                                  float as, const ColParams& c, float S, float Z) {
     // one element per call: no reciprocal, the grid divides
     const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), false, g.relu != 0);
+    JoinParams jp;
+    if (MODE == OUT_REQUANT_JOIN) jp = load_join(g, G, false);
     store_scalar<MODE>(g, size_t(m) * size_t(g.ldo) + size_t(n),
-                       finish_value<MODE>(g, epilogue_value<MODE>(g, acc, as, c, G), m, n, G));
+                       finish_value<MODE>(g, epilogue_value<MODE>(g, acc, as, c, G), m, n, jp),
+                       make_code_pack<MODE>(g, MODE == OUT_REQUANT_JOIN ? jp.out : G));
 }
 
 __device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, int32_t acc,

@@ -489,8 +489,8 @@ int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t 
 namespace {
 
 // x = every float32 bit pattern of [first, first + count): the tile epilogue's requantize
-// (quant_fast: reciprocal multiply with a guard band, division for the rest), in both of its
-// forms (the code, and the code minus the zero point), against the plain [floor at zero,]
+// (quant_fast: reciprocal multiply with a guard band, division for the rest), in its three
+// forms (the code, the code minus the zero point, the code shifted into 0..255), against the plain [floor at zero,]
 // divide-round-add-clamp, compared as the codes the two would store.
 __global__ __launch_bounds__(256) void quant_route_check_kernel(float s, float z, float lo, float hi, int relu,
                                                                 unsigned long long first,
@@ -498,6 +498,7 @@ __global__ __launch_bounds__(256) void quant_route_check_kernel(float s, float z
                                                                 unsigned long long* mismatches,
                                                                 unsigned long long* divided) {
     const lq::QGrid G = lq::make_qgrid(s, z, lo, hi, true, relu != 0);
+    const lq::QGrid Gb = lq::make_qgrid(s, z, lo, hi, true, relu != 0, true);  // codes as unsigned bytes
     unsigned long long bad = 0, slow = 0;
     for (unsigned long long i = blockIdx.x * 256ull + threadIdx.x; i < count; i += gridDim.x * 256ull) {
         const float x = __uint_as_float(unsigned(first + i));
@@ -507,8 +508,10 @@ __global__ __launch_bounds__(256) void quant_route_check_kernel(float s, float z
         const float u = lq::q_core(xr, s, z, lo, hi);
         const float plain = (u != u) ? 0.0f : u;
         const float plain_c = plain - z;
+        const float biased = lq::quant_fast<false>(x, Gb);
         bad += (__float_as_uint(fast) != __float_as_uint(plain) && !(fast == 0.0f && plain == 0.0f)) ||
-               (__float_as_uint(centered) != __float_as_uint(plain_c) && !(centered == 0.0f && plain_c == 0.0f));
+               (__float_as_uint(centered) != __float_as_uint(plain_c) && !(centered == 0.0f && plain_c == 0.0f)) ||
+               !(biased == plain + Gb.bias) || (Gb.in_byte && !(biased >= 0.0f && biased <= 255.0f));
         const float tp = x * G.inv;
         slow += !(__builtin_fabsf(tp - __builtin_rintf(tp)) < 0.5f - 0x1p-12f);
     }

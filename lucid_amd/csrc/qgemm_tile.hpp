@@ -109,12 +109,14 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
     const bool vec_ok = (g.ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0);
     const int row0 = lane / QUADS_PER_ROW, cq = (lane % QUADS_PER_ROW) * 4;
     constexpr bool kRequant = MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN || MODE == OUT_FAKEQUANT_F32;
-    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), kRequant, g.relu != 0);
+    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), kRequant, g.relu != 0,
+                               MODE == OUT_REQUANT_I8);
     JoinParams jp;
     if (MODE == OUT_REQUANT_JOIN) {
         jp = load_join(g, G, true);
         interior = interior && jp.k2_exact;  // the vector path subtracts the partner's offsets in one step
     }
+    const CodePack cpk = make_code_pack<MODE>(g, MODE == OUT_REQUANT_JOIN ? jp.out : G);
     // running range of what this lane stores (float32 output with a kept range only)
     const bool keep = MODE == OUT_F32X && g.range != nullptr;
     auto track = [&](uint32_t bits) {
@@ -211,7 +213,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                 }
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
-                    store_vec4<MODE>(g, idx, v[p]);
+                    store_vec4<MODE>(g, idx, v[p], cpk);
                     idx += step;
                 }
             } else {
@@ -220,10 +222,10 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                     uint4 v = *reinterpret_cast<const uint4*>(src + p * ROWS_PER_PASS * STRIDE);
                     const int m = m_first + p * ROWS_PER_PASS;
                     if (m < g.M && n < n_limit) {
-                        v.x = finish_value<MODE>(g, v.x, m, n, G);
-                        if (n + 1 < n_limit) v.y = finish_value<MODE>(g, v.y, m, n + 1, G);
-                        if (n + 2 < n_limit) v.z = finish_value<MODE>(g, v.z, m, n + 2, G);
-                        if (n + 3 < n_limit) v.w = finish_value<MODE>(g, v.w, m, n + 3, G);
+                        v.x = finish_value<MODE>(g, v.x, m, n, jp);
+                        if (n + 1 < n_limit) v.y = finish_value<MODE>(g, v.y, m, n + 1, jp);
+                        if (n + 2 < n_limit) v.z = finish_value<MODE>(g, v.z, m, n + 2, jp);
+                        if (n + 3 < n_limit) v.w = finish_value<MODE>(g, v.w, m, n + 3, jp);
                         if (MODE == OUT_F32X && keep) {
                             track(v.x);
                             if (n + 1 < n_limit) track(v.y);
@@ -232,12 +234,12 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, v16i (&acc)[Cfg
                         }
                         const size_t idx = size_t(m) * size_t(g.ldo) + size_t(n);
                         if (vec_ok && n + 4 <= n_limit) {
-                            store_vec4<MODE>(g, idx, v);
+                            store_vec4<MODE>(g, idx, v, cpk);
                         } else {
-                            store_scalar<MODE>(g, idx, v.x);
-                            if (n + 1 < n_limit) store_scalar<MODE>(g, idx + 1, v.y);
-                            if (n + 2 < n_limit) store_scalar<MODE>(g, idx + 2, v.z);
-                            if (n + 3 < n_limit) store_scalar<MODE>(g, idx + 3, v.w);
+                            store_scalar<MODE>(g, idx, v.x, cpk);
+                            if (n + 1 < n_limit) store_scalar<MODE>(g, idx + 1, v.y, cpk);
+                            if (n + 2 < n_limit) store_scalar<MODE>(g, idx + 2, v.z, cpk);
+                            if (n + 3 < n_limit) store_scalar<MODE>(g, idx + 3, v.w, cpk);
                         }
                     }
                 }
