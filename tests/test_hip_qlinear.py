@@ -373,3 +373,76 @@ def test_fused_join_at_ties_and_with_odd_grids():
         exp = O.add_requant(first.numpy(), 0, np.float32(s1), np.float32(z1), other.numpy(), -128, np.float32(s2),
                             np.float32(z2), False, np.float32(S), np.float32(Z), 0, 255, -128)
         assert np.array_equal(fused.numpy(), exp.reshape(M, N))
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("zp,qmin,qmax,offset", [
+    (0.0, 0, 255, -128),      # unsigned codes stored signed: packed route, XOR
+    (128.0, 0, 255, -128),
+    (-7.0, -128, 127, 0),     # signed range: shifted by 128 for the packed route
+    (-128.0, -128, 127, 0),   # zero point on the lower bound
+    (127.0, -128, 127, 0),    # ... on the upper bound: a ReLU leaves one code
+    (10.0, 0, 100, -50),      # a storage offset that is no multiple of 128: the general narrowing
+    (3.0, 0, 127, 0),         # unsigned subrange stored as is
+    (-20.0, 0, 255, -128),    # zero point below the range: a ReLU cannot be folded, every element divides
+    (200.0, -128, 127, 0)])   # zero point above the range
+def test_requantize_grid_variants_through_the_tile_epilogue(zp, qmin, qmax, offset, relu):
+    """The tile epilogue folds the ReLU and the storage form into the clamp bounds where the
+    grid allows it and falls back to the plain arithmetic where it does not; both must give
+    the oracle's codes.  M is not a multiple of the tile height, so interior and edge tiles
+    (vector and scalar stores) both run."""
+    rng = np.random.default_rng(int(zp * 2) % 97 + qmax + relu)
+    M, N, K = 300, 260, 96
+    a, w, a_scale, w_scale, bias, a_zp = _epilogue_case(rng, M, N, K, False, "f32")
+    wsum = _ops.rowsum_i8(hip(w))
+    y = O.qlinear(a, w, a_zp, a_scale, w_scale, bias=bias, relu=relu, out_mode=O.OUT_F32)
+    S, Z = np.float32(np.abs(y).max() / 90 + 1e-6), np.float32(zp)
+    for mode in (_ops.OUT_REQUANT_I8, _ops.OUT_FAKEQUANT_F32):
+        got = _ops.qlinear_i8(hip(a), hip(w), a_zp=a_zp, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=wsum,
+                              bias=hip(bias), relu=relu, out_mode=mode, out_scale=hip(S), out_zp=hip(Z),
+                              out_qmin=qmin, out_qmax=qmax, out_offset=offset, path=TILE).numpy()
+        exp = O.qlinear(a, w, a_zp, a_scale, w_scale, bias=bias, relu=relu, out_mode=mode, out_scale=S, out_zp=Z,
+                        out_qmin=qmin, out_qmax=qmax, out_offset=offset)
+        if mode == _ops.OUT_REQUANT_I8:
+            assert np.array_equal(got, exp)
+            if qmin < zp < qmax:
+                assert len(np.unique(got)) > 20  # the case exercises the grid
+        else:
+            assert np.array_equal(got.view(np.uint32), exp.view(np.uint32))
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("z1,z2,off2,Zj,qmin,qmax,offj", [
+    (0.0, 0.0, -128, 0.0, 0, 255, -128),
+    (-3.0, 17.0, 0, -9.0, -128, 127, 0),       # every grid signed, partner stored as is
+    (5.0, 131.0, -128, 64.0, 0, 255, -128),
+    (2.0, 7.5, -128, 3.0, 0, 255, -128),       # partner zero point no integer: the general join
+    (2.0, 7.0, -128, 3.0, 0, 100, -50),        # join output with a storage offset that is no multiple of 128
+    (2.0, 7.0, -128, -4.0, 0, 255, -128)])     # join zero point below its range: its ReLU is not folded
+def test_fused_join_grid_variants(z1, z2, off2, Zj, qmin, qmax, offj, relu):
+    """The fused join takes this layer's code minus its zero point from shifted clamp bounds,
+    the partner's stored byte in one subtraction, and folds its ReLU and storage form like the
+    plain requantize; each has a fallback.  Equal to the oracle's two-step form (requantize,
+    then add_requant) on interior and edge tiles."""
+    rng = np.random.default_rng(int(z2 * 2) + qmax + relu)
+    M, N, K = 300, 260, 64
+    a, w = codes(rng, (M, K), -6, 6), codes(rng, (N, K), -6, 6)
+    a_scale, w_scale = np.float32(0.11), rng.uniform(0.05, 0.2, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    s1, s2, Sj = np.float32(0.31), np.float32(0.027), np.float32(0.35)
+    common = dict(a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias), out_mode=_ops.OUT_REQUANT_I8,
+                  out_scale=hip(s1), out_zp=hip(np.float32(z1)), out_qmin=-128, out_qmax=127, out_offset=0,
+                  path=TILE)
+    lo2, hi2 = (0, 255) if off2 else (-128, 127)
+    other = rng.integers(lo2, hi2 + 1, (M, N)).astype(np.int64)
+    other_stored = (other + off2).astype(np.int8)
+    fused = _ops.qlinear_i8(hip(a), hip(w), **common,
+                            join=dict(q=hip(other_stored), offset=off2, scale=hip(s2), zp=hip(np.float32(z2)),
+                                      relu=relu, out_scale=hip(Sj), out_zp=hip(np.float32(Zj)), out_qmin=qmin,
+                                      out_qmax=qmax, out_offset=offj)).numpy()
+    first = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, out_mode=O.OUT_REQUANT_I8, out_scale=s1,
+                      out_zp=np.float32(z1), out_qmin=-128, out_qmax=127, out_offset=0)
+    exp = O.add_requant(first, 0, s1, np.float32(z1), other_stored, off2, s2, np.float32(z2), relu, Sj,
+                        np.float32(Zj), qmin, qmax, offj)
+    assert np.array_equal(fused, exp.reshape(M, N))
+    assert len(np.unique(fused)) > 20
