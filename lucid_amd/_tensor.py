@@ -288,6 +288,18 @@ class Tensor:
             raise _C.ShapeMismatch(f"narrow_rows: {n} rows of {self.shape[0]}")
         return Tensor((n, *self.shape[1:]), self.dtype, "hip", buf=self._buf, offset=self._offset)
 
+    def row_range(self, lo: int, hi: int) -> "Tensor":
+        """Entries ``[lo, hi)`` along axis 0 as a view of the same storage."""
+        if self.device != "hip" or self._grid is not None:
+            raise NotImplementedError("row_range: plain device tensors only")
+        if not 0 <= lo <= hi <= self.shape[0]:
+            raise _C.ShapeMismatch(f"row_range: [{lo}, {hi}) of {self.shape[0]}")
+        if self._buf is None:
+            self._materialize()
+        row_bytes = self.nbytes // self.shape[0] if self.shape[0] else 0
+        return Tensor((hi - lo, *self.shape[1:]), self.dtype, "hip", buf=self._buf,
+                      offset=self._offset + lo * row_bytes)
+
     def detach(self) -> "Tensor":
         return self
 

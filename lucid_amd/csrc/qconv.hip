@@ -219,6 +219,63 @@ __global__ void repack_oihw_to_ohwi_kernel(const int8_t* __restrict__ w, int8_t*
     }
 }
 
+// Volumetric convolution as an explicit GEMM.  x: codes in Lucid's own (B, C, D, H, W)
+// order; cols: [B*OD*OH*OW, KD*KH*KW*Cg] with k = ((kd*KH + kh)*KW + kw)*Cg + c over the
+// channels [c0, c0 + Cg) of one group; taps in the padding read pad_code (the zero point's
+// stored code).  `ins` > 1 spreads the input over a grid with ins - 1 zero-point codes between
+// neighbours (the zero insertion of a transposed convolution) without materialising it.
+// One byte per lane: consecutive lanes write consecutive bytes.
+struct Vol3 {
+    int d, h, w;
+};
+
+__global__ void im2col_ncdhw_i8_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ cols, int C, Vol3 in,
+                                       int c0, int Cg, Vol3 kern, Vol3 stride, Vol3 pad, Vol3 dil, Vol3 ins,
+                                       Vol3 out, int pad_code, size_t total) {
+    const size_t K = size_t(kern.d) * kern.h * kern.w * Cg;
+    for (size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * blockDim.x) {
+        const size_t k = idx % K;
+        size_t m = idx / K;
+        const int c = int(k % Cg);
+        int tap = int(k / Cg);
+        const int kw = tap % kern.w;
+        tap /= kern.w;
+        const int kh = tap % kern.h, kd = tap / kern.h;
+        const int ow = int(m % out.w);
+        m /= out.w;
+        const int oh = int(m % out.h);
+        m /= out.h;
+        const int od = int(m % out.d);
+        const size_t b = m / out.d;
+        // coordinates on the spread grid; a real sample sits at every ins-th of them
+        const int vd = od * stride.d - pad.d + kd * dil.d;
+        const int vh = oh * stride.h - pad.h + kh * dil.h;
+        const int vw = ow * stride.w - pad.w + kw * dil.w;
+        int v = pad_code;
+        if (vd >= 0 && vh >= 0 && vw >= 0 && vd % ins.d == 0 && vh % ins.h == 0 && vw % ins.w == 0) {
+            const int id = vd / ins.d, ih = vh / ins.h, iw = vw / ins.w;
+            if (id < in.d && ih < in.h && iw < in.w)
+                v = x[(((b * C + c0 + c) * in.d + id) * in.h + ih) * size_t(in.w) + iw];
+        }
+        cols[idx] = int8_t(v);
+    }
+}
+
+// GEMM result rows [B*L, Ng] (position-major) into channels [c0, c0 + Ng) of a
+// channels-first tensor (B, Ctot, L): one byte per lane, consecutive lanes along L.
+__global__ void rows_to_channels_first_i8_kernel(const int8_t* __restrict__ rows, int8_t* __restrict__ dst,
+                                                 size_t L, int Ng, int c0, int Ctot, size_t total) {
+    for (size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * blockDim.x) {
+        const size_t l = idx % L;
+        const size_t r = idx / L;
+        const int n = int(r % Ng);
+        const size_t b = r / Ng;
+        dst[(b * Ctot + c0 + n) * L + l] = rows[(b * L + l) * Ng + n];
+    }
+}
+
 // Non-zero padding modes of F.pad on NHWC codes (reflect / replicate / circular):
 // the padded float image is a gather of the original, so the padded code image is
 // the same gather of the codes.  One lane per 16 channels when C % 16 == 0, else per byte.
@@ -551,6 +608,47 @@ int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH
     hipLaunchKernelGGL(repack_oihw_to_ohwi_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream),
                        w, out, O, I, KH, KW);
     LQ_CHECK_LAUNCH("repack_oihw_to_ohwi");
+    return LQ_OK;
+}
+
+int lq_im2col_ncdhw_i8(const int8_t* x, int8_t* cols, int B, int C, int D, int H, int W, int c0, int Cg,
+                       const int* kernel, const int* stride, const int* pad_lo, const int* dilation,
+                       const int* insert, const int* out_size, int pad_code, lq_stream stream) {
+    LQ_REQUIRE(kernel && stride && pad_lo && dilation && insert && out_size, LQ_ERR_VALUE,
+               "im2col_ncdhw: NULL geometry");
+    LQ_REQUIRE(B >= 0 && C > 0 && D > 0 && H > 0 && W > 0, LQ_ERR_SHAPE, "im2col_ncdhw: bad input shape");
+    LQ_REQUIRE(c0 >= 0 && Cg > 0 && c0 + Cg <= C, LQ_ERR_SHAPE, "im2col_ncdhw: channels [%d, %d) of %d", c0,
+               c0 + Cg, C);
+    LQ_REQUIRE(pad_code >= -128 && pad_code <= 127, LQ_ERR_VALUE, "im2col_ncdhw: padding code %d is no int8", pad_code);
+    // any tap outside the spread input reads the padding code, so out_size needs no upper bound:
+    // high-side padding, e.g. a transposed convolution's output_padding, is simply more outputs
+    for (int i = 0; i < 3; ++i)
+        LQ_REQUIRE(kernel[i] > 0 && stride[i] > 0 && dilation[i] > 0 && insert[i] > 0 && pad_lo[i] >= 0 &&
+                       out_size[i] >= 0,
+                   LQ_ERR_VALUE, "im2col_ncdhw: bad geometry in dimension %d", i);
+    const size_t M = size_t(B) * out_size[0] * out_size[1] * out_size[2];
+    const size_t total = M * kernel[0] * kernel[1] * kernel[2] * Cg;
+    if (total == 0) return LQ_OK;
+    LQ_REQUIRE(x && cols, LQ_ERR_VALUE, "im2col_ncdhw: NULL pointer");
+    hipLaunchKernelGGL(im2col_ncdhw_i8_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream), x, cols, C,
+                       Vol3{D, H, W}, c0, Cg, Vol3{kernel[0], kernel[1], kernel[2]},
+                       Vol3{stride[0], stride[1], stride[2]}, Vol3{pad_lo[0], pad_lo[1], pad_lo[2]},
+                       Vol3{dilation[0], dilation[1], dilation[2]}, Vol3{insert[0], insert[1], insert[2]},
+                       Vol3{out_size[0], out_size[1], out_size[2]}, pad_code, total);
+    LQ_CHECK_LAUNCH("im2col_ncdhw");
+    return LQ_OK;
+}
+
+int lq_rows_to_channels_first_i8(const int8_t* rows, int8_t* dst, int B, size_t L, int Ng, int c0, int Ctot,
+                                 lq_stream stream) {
+    LQ_REQUIRE(B >= 0 && Ng > 0 && c0 >= 0 && c0 + Ng <= Ctot, LQ_ERR_SHAPE,
+               "rows_to_channels_first: channels [%d, %d) of %d", c0, c0 + Ng, Ctot);
+    const size_t total = size_t(B) * L * Ng;
+    if (total == 0) return LQ_OK;
+    LQ_REQUIRE(rows && dst, LQ_ERR_VALUE, "rows_to_channels_first: NULL pointer");
+    hipLaunchKernelGGL(rows_to_channels_first_i8_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream), rows,
+                       dst, L, Ng, c0, Ctot, total);
+    LQ_CHECK_LAUNCH("rows_to_channels_first");
     return LQ_OK;
 }
 

@@ -146,6 +146,33 @@ class Conv1d(Module):
             "quantize the model (convert) first")
 
 
+class Conv3d(Module):
+    """Float Conv3d as a parameter holder (``weight`` (O, I/groups, KD, KH, KW), ``bias`` (O,))."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, padding_mode="zeros") -> None:
+        super().__init__()
+        three = lambda v: (int(v),) * 3 if isinstance(v, int) else tuple(int(e) for e in v)
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride = three(kernel_size), three(stride)
+        self.dilation, self.groups = three(dilation), groups
+        self._padding_str = padding if isinstance(padding, str) else None
+        self.padding = (0, 0, 0) if isinstance(padding, str) else three(padding)
+        self.padding_mode = padding_mode
+        fan_in = in_channels // groups * int(np.prod(self.kernel_size))
+        bound = 1.0 / np.sqrt(fan_in)
+        rng = np.random.default_rng(fan_in * 7919 + out_channels + 3)
+        self.register_buffer("weight", T.tensor(rng.uniform(
+            -bound, bound, (out_channels, in_channels // groups, *self.kernel_size)).astype(np.float32)))
+        self.register_buffer("bias", T.tensor(
+            rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.Conv3d.forward is not part of the hip quantized-inference backend; "
+            "quantize the model (convert) first")
+
+
 class BatchNorm2d(Module):
     """Float BatchNorm2d as a parameter / statistics holder (folded into the
     preceding convolution by ``fuse_modules`` before quantization)."""
@@ -393,6 +420,31 @@ class ConvTranspose1d(Module):
     def forward(self, x):
         raise NotImplementedError(
             "float nn.ConvTranspose1d.forward is not part of the hip quantized-inference backend; "
+            "quantize the model (convert) first")
+
+
+class ConvTranspose3d(Module):
+    """Float ConvTranspose3d as a parameter holder (``weight`` (in, out/groups, kd, kh, kw))."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, output_padding=0,
+                 groups=1, bias=True, dilation=1) -> None:
+        super().__init__()
+        three = lambda v: (int(v),) * 3 if isinstance(v, int) else tuple(int(e) for e in v)
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride = three(kernel_size), three(stride)
+        self.padding = padding if isinstance(padding, str) else three(padding)
+        self.output_padding, self.dilation, self.groups = three(output_padding), three(dilation), groups
+        fan_in = out_channels // groups * int(np.prod(self.kernel_size))
+        bound = 1.0 / np.sqrt(fan_in)
+        rng = np.random.default_rng(fan_in * 7919 + in_channels + 3)
+        self.register_buffer("weight", T.tensor(rng.uniform(
+            -bound, bound, (in_channels, out_channels // groups, *self.kernel_size)).astype(np.float32)))
+        self.register_buffer("bias", T.tensor(
+            rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
+
+    def forward(self, x):
+        raise NotImplementedError(
+            "float nn.ConvTranspose3d.forward is not part of the hip quantized-inference backend; "
             "quantize the model (convert) first")
 
 

@@ -3,8 +3,8 @@
 
 from . import dynamic
 from .functional_module import FloatFunctional, QFunctional
-from .conv import Conv1d, Conv2d
-from .conv_transpose import ConvTranspose1d, ConvTranspose2d
+from .conv import Conv1d, Conv2d, Conv3d
+from .conv_transpose import ConvTranspose1d, ConvTranspose2d, ConvTranspose3d
 from .intrinsic import ConvReLU2d, LinearReLU
 from .linear import Linear
 from .mlx_linear import QuantizedLinearMLX
@@ -12,6 +12,6 @@ from .modules import DeQuantize, DeQuantStub, Quantize, QuantStub, QuantWrapper
 from .activation import ELU, Hardsigmoid, Hardswish, LeakyReLU, Sigmoid, Tanh
 from .sparse import Embedding, EmbeddingBag
 
-__all__ = ["QuantizedLinearMLX", "Linear", "LinearReLU", "Conv1d", "Conv2d", "ConvReLU2d", "Quantize", "DeQuantize", "QuantStub", "DeQuantStub",
-           "QuantWrapper", "QFunctional", "FloatFunctional", "dynamic", "Embedding", "EmbeddingBag", "ConvTranspose1d", "ConvTranspose2d", "Sigmoid",
+__all__ = ["QuantizedLinearMLX", "Linear", "LinearReLU", "Conv1d", "Conv2d", "Conv3d", "ConvReLU2d", "Quantize", "DeQuantize", "QuantStub", "DeQuantStub",
+           "QuantWrapper", "QFunctional", "FloatFunctional", "dynamic", "Embedding", "EmbeddingBag", "ConvTranspose1d", "ConvTranspose2d", "ConvTranspose3d", "Sigmoid",
            "Hardswish", "Hardsigmoid", "Tanh", "ELU", "LeakyReLU"]

@@ -13,6 +13,8 @@ requantize in the epilogue.
 
 from __future__ import annotations
 
+import ctypes as C
+
 import numpy as np
 
 from ... import _C, _ops
@@ -242,3 +244,119 @@ class Conv1d(Conv2d):
     def extra_repr(self) -> str:
         return (f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size[1]}, "
                 f"stride={self.stride[1]}, qdtype={self.out_qdtype.name}")
+
+
+def _triple(v):
+    return (int(v),) * 3 if isinstance(v, int) else tuple(int(e) for e in v)
+
+
+def volumetric_gemm(name, x: Tensor, g, w_rows: Tensor, wsum: Tensor, w_scale: Tensor, bias, kernel, stride,
+                    pads, dilation, insert, groups: int, relu: bool, scale: Tensor, zero_point: Tensor,
+                    qdtype: QDtype, zp_host: int) -> Tensor:
+    """A 3-d convolution on codes as an explicit GEMM, group by group: gather the taps of
+    ``x``'s ``(B, C, D, H, W)`` codes (``insert`` > 1: as if zero-point codes stood between
+    neighbouring samples), multiply with the group's kernel rows ``[Cout/groups, taps * C/groups]``
+    through the fused int8 GEMM, write the result channels-first.  ``pads`` = ((lo, hi),) * 3."""
+    B, Cc, D, H, W = x.shape
+    spread = [(n - 1) * i + 1 for n, i in zip((D, H, W), insert)]
+    outs = [(n + lo + hi - d * (k - 1) - 1) // s + 1
+            for n, (lo, hi), k, s, d in zip(spread, pads, kernel, stride, dilation)]
+    if min(outs) < 1:
+        raise _C.ShapeMismatch(f"{name}: kernel {tuple(kernel)} does not fit input {x.shape}")
+    L = outs[0] * outs[1] * outs[2]
+    Co = w_rows.shape[0]
+    Cg, Og = Cc // groups, Co // groups
+    a_zp = int(g.zp_host) + g.offset
+    off = storage_offset(qdtype)
+    i3 = lambda v: (C.c_int * 3)(*[int(e) for e in v])
+    codes = Tensor.empty((B, Co, *outs), T.int8, "hip")
+    cols = Tensor.empty((B * L, Cg * kernel[0] * kernel[1] * kernel[2]), T.int8, "hip")
+    for grp in range(groups):
+        _C.call("lq_im2col_ncdhw_i8", g.codes.data_ptr, cols.data_ptr, B, Cc, D, H, W, grp * Cg, Cg, i3(kernel),
+                i3(stride), i3([p[0] for p in pads]), i3(dilation), i3(insert), i3(outs), a_zp, None)
+        part = lambda t: t.row_range(grp * Og, (grp + 1) * Og)
+        y = _ops.qlinear_i8(cols, part(w_rows), a_zp=a_zp, a_scale=g.scale, w_scale=part(w_scale), wsum=part(wsum),
+                            bias=None if bias is None else part(bias), relu=relu, out_mode=_ops.OUT_REQUANT_I8,
+                            out_scale=scale, out_zp=zero_point, out_qmin=qdtype.quant_min,
+                            out_qmax=qdtype.quant_max, out_offset=off)
+        _C.call("lq_rows_to_channels_first_i8", y.data_ptr, codes.data_ptr, B, L, Og, grp * Og, Co, None)
+    return Tensor.on_grid((B, Co, *outs), Grid(codes, scale, zero_point, qdtype, off, zp_host, "plain"))
+
+
+class Conv3d(Conv2d):
+    """Quantized ``Conv3d`` (``lucid/nn/quantized/conv.py:545-700``): the same buffers with a
+    five-dimensional kernel ``weight_int8`` ``(Cout, Cin/groups, KD, KH, KW)``.  The forward is
+    an explicit GEMM on codes: the taps of each group are gathered from the ``(B, C, D, H, W)``
+    codes into a matrix (padding taps hold the input zero point's code), multiplied with the
+    group's kernel rows by the int8 GEMM with the usual fused epilogue (zero-point correction,
+    scales, bias, optional ReLU, requantize) and written back channels-first.  Zero padding
+    only (numbers, ``"same"`` or ``"valid"``)."""
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size, stride=1, padding=0,
+                 dilation=1, groups: int = 1, bias: bool = True) -> None:
+        super().__init__(in_channels, out_channels, (1, 1), (1, 1), 0, (1, 1), groups, bias)
+        self.kernel_size, self.stride = _triple(kernel_size), _triple(stride)
+        self.padding_str = padding if isinstance(padding, str) else None
+        self.padding = (0, 0, 0) if isinstance(padding, str) else _triple(padding)
+        self.dilation = _triple(dilation)
+        self.register_buffer("weight_int8", T.tensor(
+            np.zeros((out_channels, in_channels // groups, *self.kernel_size), np.int8), device="hip"))
+
+    def _prepare_weight(self) -> None:
+        O, I, KD, KH, KW = self.weight_int8.shape
+        w = Tensor.empty((O, KD * KH * KW * I), T.int8, "hip")
+        _C.call("lq_repack_oihw_to_ohwi_i8", self.weight_int8.data_ptr, w.data_ptr, O, I, 1, KD * KH * KW, None)
+        self._w_ohwi = w
+        self._wsum = _ops.rowsum_i8(w)
+
+    def _resolve_pad3(self, sizes) -> list[tuple[int, int]]:
+        if self.padding_str == "valid":
+            return [(0, 0)] * 3
+        if self.padding_str == "same":
+            return [_same_pad_pair(n, k, s, d)
+                    for n, k, s, d in zip(sizes, self.kernel_size, self.stride, self.dilation)]
+        return [(p, p) for p in self.padding]
+
+    def forward(self, x: Tensor) -> Tensor:
+        name = type(self).__name__
+        g = input_grid(x, name)
+        if x.ndim != 5 or x.shape[1] != self.in_channels:
+            raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, D, H, W), got {x.shape}")
+        if self.padding_mode != "zeros":
+            raise NotImplementedError(f"{name}: padding_mode {self.padding_mode!r}; the hip backend pads "
+                                      "volumes with zeros only")
+        if g.zp_host is None:
+            raise NotImplementedError(
+                f"{name}: the input zero point is only known on the device; convolution needs it "
+                "on the host for the padding code (static quantization provides it)")
+        if g.layout != "plain":
+            raise _C.LucidError(f"{name}: 5-d activation codes must be stored in their own (B, C, D, H, W) order")
+        if self._w_ohwi is None:
+            self._prepare_weight()
+        if self._zp_host is None:
+            self._zp_host = int(host_scalar(self.zero_point))
+        pads = self._resolve_pad3(x.shape[2:])
+        return volumetric_gemm(name, x, g, self._w_ohwi, self._wsum, self.weight_scale, self.bias, self.kernel_size,
+                               self.stride, pads, self.dilation, (1, 1, 1), self.groups, self._fused_relu,
+                               self.scale, self.zero_point, self.out_qdtype, self._zp_host)
+
+    @classmethod
+    def from_float(cls, mod) -> "Conv3d":
+        """Quantize a calibrated float ``Conv3d`` (``conv.py:186-222``)."""
+        qmod = cls(mod.in_channels, mod.out_channels, mod.kernel_size, mod.stride, mod.padding,
+                   mod.dilation, mod.groups, bias=mod.bias is not None)
+        codes, w_scale, w_zp, ch_axis = quantize_weight(mod)
+        require_symmetric_weight(w_zp, cls.__name__)
+        qmod.register_buffer("weight_int8", codes)
+        qmod.register_buffer("weight_scale", w_scale)
+        qmod.register_buffer("weight_zero_point", w_zp)
+        qmod.weight_ch_axis = ch_axis
+        qmod.padding_str = getattr(mod, "_padding_str", None)
+        qmod.padding_mode = getattr(mod, "padding_mode", "zeros")
+        if mod.bias is not None:
+            qmod.register_buffer("bias", mod.bias.to("hip"))
+        a_scale, a_zp, a_qdtype = activation_qparams(mod)
+        qmod.register_buffer("scale", a_scale)
+        qmod.register_buffer("zero_point", a_zp)
+        qmod.out_qdtype = a_qdtype
+        return qmod

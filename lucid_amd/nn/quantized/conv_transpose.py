@@ -173,3 +173,54 @@ class ConvTranspose1d(ConvTranspose2d):
     def extra_repr(self) -> str:
         return (f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size[1]}, "
                 f"stride={self.stride[1]}, qdtype={self.out_qdtype.name}")
+
+
+class ConvTranspose3d(ConvTranspose2d):
+    """Quantized ``ConvTranspose3d`` (``lucid/nn/quantized/conv_transpose.py:484-640``):
+    ``weight_int8`` ``(in, out/groups, kd, kh, kw)``.  The same identity as the 2-d layer - a
+    stride-1 convolution of the zero-inserted input with the flipped kernel - on the
+    ``(B, C, D, H, W)`` codes through the explicit-GEMM route of ``Conv3d``; the zero insertion
+    happens inside the tap gather, nothing is materialised for it."""
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size, stride=1, padding=0,
+                 output_padding=0, dilation=1, groups: int = 1, bias: bool = True) -> None:
+        three = lambda v: (int(v),) * 3 if isinstance(v, int) else tuple(int(e) for e in v)
+        super().__init__(in_channels, out_channels, (1, 1), 1, 0, 0, 1, groups, bias)
+        self.kernel_size, self.stride, self.padding = three(kernel_size), three(stride), three(padding)
+        self.output_padding, self.dilation = three(output_padding), three(dilation)
+        self.register_buffer("weight_int8", T.tensor(
+            np.zeros((in_channels, out_channels // groups, *self.kernel_size), np.int8), device="hip"))
+
+    def _prepare_weight(self) -> None:
+        """The equivalent convolution's kernel rows ``[out, taps * in/groups]``: flipped in
+        space, channels swapped inside each group (one-off, on the host)."""
+        w = self.weight_int8.numpy()
+        cig = self.in_channels // self.groups
+        blocks = [np.transpose(w[g * cig:(g + 1) * cig, :, ::-1, ::-1, ::-1], (1, 2, 3, 4, 0))
+                  for g in range(self.groups)]
+        rows = np.concatenate(blocks, axis=0)
+        self._w_ohwi = T.tensor(np.ascontiguousarray(rows.reshape(rows.shape[0], -1)), device="hip")
+        self._wsum = _ops.rowsum_i8(self._w_ohwi)
+        self._w_scale_full = T.tensor(np.tile(self.weight_scale.numpy(), self.groups), device="hip")
+
+    def forward(self, x: Tensor) -> Tensor:
+        from .conv import volumetric_gemm
+        name = type(self).__name__
+        g = input_grid(x, name)
+        if x.ndim != 5 or x.shape[1] != self.in_channels:
+            raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, D, H, W), got {x.shape}")
+        if g.zp_host is None:
+            raise NotImplementedError(f"{name}: the input zero point must be known on the host")
+        if g.layout != "plain":
+            raise _C.LucidError(f"{name}: 5-d activation codes must be stored in their own (B, C, D, H, W) order")
+        lo = [d * (k - 1) - p for d, k, p in zip(self.dilation, self.kernel_size, self.padding)]
+        if min(lo) < 0:
+            raise NotImplementedError(f"{name}: padding larger than dilation * (kernel - 1) is not supported")
+        if self._w_ohwi is None:
+            self._prepare_weight()
+        if self._zp_host is None:
+            self._zp_host = int(host_scalar(self.zero_point))
+        pads = [(l, l + op) for l, op in zip(lo, self.output_padding)]
+        return volumetric_gemm(name, x, g, self._w_ohwi, self._wsum, self._w_scale_full, self.bias, self.kernel_size,
+                               (1, 1, 1), pads, self.dilation, self.stride, self.groups, False, self.scale,
+                               self.zero_point, self.out_qdtype, self._zp_host)

@@ -21,8 +21,8 @@ from .qconfig import QConfig, get_default_qconfig
 
 
 def _observed_types() -> tuple[type, ...]:
-    return (nn.Linear, nn.Conv1d, nn.Conv2d, nni.LinearReLU, nni.ConvReLU2d, nnq.QuantStub,
-            nnq.FloatFunctional, nn.ConvTranspose1d, nn.ConvTranspose2d, nn.Sigmoid, nn.Hardswish, nn.Hardsigmoid, nn.Tanh, nn.ELU, nn.LeakyReLU)
+    return (nn.Linear, nn.Conv1d, nn.Conv2d, nn.Conv3d, nni.LinearReLU, nni.ConvReLU2d, nnq.QuantStub,
+            nnq.FloatFunctional, nn.ConvTranspose1d, nn.ConvTranspose2d, nn.ConvTranspose3d, nn.Sigmoid, nn.Hardswish, nn.Hardsigmoid, nn.Tanh, nn.ELU, nn.LeakyReLU)
 
 
 def _quant_mapping() -> dict[type, object]:
@@ -34,6 +34,7 @@ def _quant_mapping() -> dict[type, object]:
         nnq.FloatFunctional: nnq.QFunctional.from_float,
         nn.ConvTranspose2d: nnq.ConvTranspose2d.from_float,
         nn.ConvTranspose1d: nnq.ConvTranspose1d.from_float,
+        nn.ConvTranspose3d: nnq.ConvTranspose3d.from_float,
         nn.Embedding: nnq.Embedding.from_float,
         nn.EmbeddingBag: nnq.EmbeddingBag.from_float,
         nn.Sigmoid: nnq.Sigmoid.from_float,
@@ -46,6 +47,7 @@ def _quant_mapping() -> dict[type, object]:
     if hasattr(nnq, "Conv2d"):
         m[nn.Conv2d] = nnq.Conv2d.from_float
         m[nn.Conv1d] = nnq.Conv1d.from_float
+        m[nn.Conv3d] = nnq.Conv3d.from_float
         m[nni.ConvReLU2d] = nnq.ConvReLU2d.from_float
     return m
 

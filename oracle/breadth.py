@@ -16,6 +16,14 @@ where the reference loops.
                      fake-quantize to the calibrated grid)
 * ``lstm``           ``CpuBackend.h:13394-13519`` on dequantized weights
                      (``lucid/nn/quantized/dynamic/rnn.py``)
+* ``qconv3d``        ``lucid/nn/quantized/conv.py:545-700`` (dequantize kernel, ``F.conv3d``,
+                     bias, fake-quantize) in the integer formulation of the 2-d layer: taps
+                     gathered with numpy slices, then the oracle's ``qlinear`` per group;
+                     ``tests/test_oracle_breadth.py`` pins the gather and the group
+                     bookkeeping against ``scipy.signal.correlate`` on the centred codes
+* ``qconv_transpose3d``  ``lucid/nn/quantized/conv_transpose.py:484-640`` as ``qconv3d`` of the
+                     zero-inserted codes with the flipped kernel; the same test file pins that
+                     identity against the scatter definition of a transposed convolution
 
 PARITY UNPINNED at the bit level for sigmoid, tanh, elu (the reference evaluates exp /
 tanh through Accelerate's vForce, whose last-bit behaviour is not published) and for the
@@ -156,3 +164,64 @@ def conv_transpose2d(x, w, bias, stride, padding, output_padding, dilation=(1, 1
     if bias is not None:
         out = out + np.asarray(bias, np.float64)[None, :, None, None]
     return out
+
+
+def qconv3d(x, w, a_zp, a_scale, w_scale, stride=(1, 1, 1), pad=((0, 0),) * 3, dilation=(1, 1, 1), groups=1,
+            bias=None, relu=False, **out):
+    """Integer-formulation Conv3d.  ``x`` int8 stored codes (B, C, D, H, W); ``w`` int8
+    (Cout, C/groups, KD, KH, KW); ``a_zp`` the input zero point as a stored code (what the
+    padding holds); ``pad`` = ((lo, hi),) * 3; ``out``: the ``qlinear`` output arguments
+    (``out_mode``, ``out_scale``, ...).  Returns (B, Cout, OD, OH, OW)."""
+    import oracle as O
+    x = np.asarray(x, np.int8)
+    w = np.asarray(w, np.int8)
+    B, C = x.shape[:2]
+    Co, Cg = w.shape[:2]
+    K3 = w.shape[2:]
+    assert Cg * groups == C and Co % groups == 0
+    xp = np.pad(x, ((0, 0), (0, 0), *pad), constant_values=np.int8(a_zp))
+    outs = [(n - d * (k - 1) - 1) // s + 1 for n, k, s, d in zip(xp.shape[2:], K3, stride, dilation)]
+    taps = []
+    for kd in range(K3[0]):
+        for kh in range(K3[1]):
+            for kw in range(K3[2]):
+                sl = tuple(slice(kk * d, kk * d + (o - 1) * s + 1, s)
+                           for kk, d, o, s in zip((kd, kh, kw), dilation, outs, stride))
+                taps.append(xp[(slice(None), slice(None), *sl)])          # (B, C, OD, OH, OW)
+    cols = np.stack(taps, axis=0)                                          # (taps, B, C, OD, OH, OW)
+    cols = np.transpose(cols, (1, 3, 4, 5, 0, 2))                          # (B, OD, OH, OW, taps, C)
+    M = B * outs[0] * outs[1] * outs[2]
+    Og = Co // groups
+    parts = []
+    for g in range(groups):
+        a = np.ascontiguousarray(cols[..., g * Cg:(g + 1) * Cg]).reshape(M, -1)
+        wg = w[g * Og:(g + 1) * Og].reshape(Og, Cg, -1)
+        wg = np.ascontiguousarray(np.transpose(wg, (0, 2, 1))).reshape(Og, -1)   # k = tap * Cg + c
+        ws = np.asarray(w_scale, np.float32)
+        parts.append(O.qlinear(a, wg, a_zp, a_scale, ws[g * Og:(g + 1) * Og] if ws.ndim else ws,
+                               bias=None if bias is None else np.asarray(bias)[g * Og:(g + 1) * Og],
+                               relu=relu, **out))
+    y = np.concatenate(parts, axis=1).reshape(B, *outs, Co)
+    return np.ascontiguousarray(np.moveaxis(y, -1, 1))
+
+
+def qconv_transpose3d(x, w, a_zp, a_scale, w_scale, stride=(1, 1, 1), padding=(0, 0, 0), output_padding=(0, 0, 0),
+                      dilation=(1, 1, 1), groups=1, bias=None, **out):
+    """Integer-formulation ConvTranspose3d.  ``x`` int8 stored codes (B, Cin, D, H, W); ``w``
+    int8 (Cin, Cout/groups, KD, KH, KW); ``w_scale`` per output channel of a group (Cout/groups,),
+    shared by the groups.  Zero-insert the codes (inserted codes = ``a_zp``), flip the kernel,
+    swap its channel axes inside each group, convolve with stride 1 and padding
+    ``dilation * (k - 1) - padding`` (``+ output_padding`` on the high side)."""
+    x = np.asarray(x, np.int8)
+    w = np.asarray(w, np.int8)
+    B, Cin = x.shape[:2]
+    K3 = w.shape[2:]
+    spread = np.full((B, Cin, *[(n - 1) * s + 1 for n, s in zip(x.shape[2:], stride)]), np.int8(a_zp), np.int8)
+    spread[(slice(None), slice(None), *[slice(None, None, s) for s in stride])] = x
+    cig = Cin // groups
+    wc = np.concatenate([np.transpose(w[g * cig:(g + 1) * cig, :, ::-1, ::-1, ::-1], (1, 0, 2, 3, 4))
+                         for g in range(groups)], axis=0)                       # (Cout, Cin/groups, K3)
+    lo = [d * (k - 1) - p for d, k, p in zip(dilation, K3, padding)]
+    pad = tuple((l, l + op) for l, op in zip(lo, output_padding))
+    return qconv3d(spread, wc, a_zp, a_scale, np.tile(np.asarray(w_scale, np.float32), groups), pad=pad,
+                   dilation=dilation, groups=groups, bias=bias, **out)

@@ -358,3 +358,99 @@ def test_conv_transpose1d(cin, cout, k, stride, padding, output_padding, dilatio
     lo = (21 - 1) * stride - 2 * padding + dilation * (k - 1) + output_padding + 1
     assert got.shape == (2, cout, lo) and np.array_equal(got, want)
     assert np.isfinite(qm(hip(x)).numpy()).all()
+
+
+# ---------------------------------------------------------------- Conv3d
+@pytest.mark.parametrize("cin,cout,k,stride,padding,dilation,groups,vol",
+                         [(16, 32, 3, 1, 1, 1, 1, (6, 10, 12)), (8, 24, (1, 3, 2), (1, 2, 1), (0, 1, 1), 1, 1, (4, 9, 7)),
+                          (32, 32, 3, (2, 1, 1), "same", (1, 2, 1), 2, (5, 8, 8)), (16, 16, 1, 1, 0, 1, 1, (3, 4, 5)),
+                          (48, 96, (2, 3, 3), 2, "valid", 1, 3, (6, 11, 9))])
+def test_conv3d_bit_exact_against_the_oracle(cin, cout, k, stride, padding, dilation, groups, vol):
+    """nnq.Conv3d (conv.py:545-700) == the oracle's integer Conv3d of the same codes, bit for
+    bit; the float view lies on the output grid."""
+    import oracle.breadth as Br
+    three = lambda v: (v,) * 3 if isinstance(v, int) else tuple(v)
+    rng = np.random.default_rng(cin * 3 + cout + sum(vol))
+    m = nn.Sequential(nnq.QuantStub(), nn.Conv3d(cin, cout, k, stride=stride, padding=padding, dilation=dilation,
+                                                 groups=groups), nnq.DeQuantStub())
+    prepared = Q.prepare(m, Q.get_default_qconfig())
+    for _ in range(4):
+        x = rng.standard_normal((2, cin, *vol)).astype(np.float32)
+        prepared[0].activation_post_process(hip(x))
+        prepared[1].activation_post_process(hip((rng.standard_normal((2, cout, 2, 2, 2)) * 1.5).astype(np.float32)))
+    qm = Q.convert(prepared)
+    c3 = qm[1]
+    assert isinstance(c3, nnq.Conv3d) and c3.weight_int8.shape == (cout, cin // groups, *three(k))
+    x = rng.standard_normal((2, cin, *vol)).astype(np.float32)
+    out = c3(qm[0](hip(x)))
+    s0, z0 = qm[0].scale.item(), qm[0].zero_point.item()
+    codes = O.quantize(x, s0, z0, 0, 255, code_offset=-128)
+    K3, S3, D3 = three(k), three(stride), three(dilation)
+    if padding == "same":
+        pad = []
+        for n, kk, ss, dd in zip(vol, K3, S3, D3):
+            total = max(0, (-(-n // ss) - 1) * ss + (kk - 1) * dd + 1 - n)
+            pad.append((total // 2, total - total // 2))
+    elif padding == "valid":
+        pad = [(0, 0)] * 3
+    else:
+        pad = [(p, p) for p in three(padding)]
+    want = Br.qconv3d(codes, c3.weight_int8.numpy(), int(z0) - 128, np.float32(s0), c3.weight_scale.numpy(),
+                      stride=S3, pad=tuple(pad), dilation=D3, groups=groups, bias=c3.bias.numpy(),
+                      out_mode=O.OUT_REQUANT_I8, out_scale=np.float32(c3.scale.item()),
+                      out_zp=np.float32(c3.zero_point.item()), out_qmin=0, out_qmax=255, out_offset=-128)
+    got = out._grid.codes.numpy()
+    assert got.shape == want.shape and np.array_equal(got, want)
+    assert len(np.unique(got)) > 20
+    y = qm(hip(x)).numpy()
+    exp_y = (want.astype(np.float32) + 128 - np.float32(c3.zero_point.item())) * np.float32(c3.scale.item())
+    assert np.array_equal(y, exp_y)
+
+
+def test_conv3d_refuses_what_it_does_not_do():
+    c3 = nnq.Conv3d(4, 4, 3)
+    c3.padding_mode = "reflect"
+    x = nnq.Quantize(hip(np.float32(0.1)), hip(np.float32(128.0)), Q.quint8)(hip(np.zeros((1, 4, 3, 3, 3), np.float32)))
+    with pytest.raises(NotImplementedError):
+        c3(x)
+    with pytest.raises(Exception):
+        nnq.Conv3d(4, 4, 3)(nnq.Quantize(hip(np.float32(0.1)), hip(np.float32(128.0)), Q.quint8)(
+            hip(np.zeros((1, 4, 3, 3), np.float32))))
+
+
+@pytest.mark.parametrize("cin,cout,k,stride,padding,output_padding,dilation,groups,vol",
+                         [(16, 32, 3, 2, 1, 1, 1, 1, (3, 5, 4)), (32, 32, (2, 3, 2), (1, 3, 2), (0, 1, 0), (0, 2, 1), 1, 2, (4, 3, 5)),
+                          (16, 16, 3, 1, 1, 0, (2, 1, 2), 1, (5, 4, 6))])
+def test_conv_transpose3d_bit_exact_against_the_oracle(cin, cout, k, stride, padding, output_padding, dilation, groups,
+                                                       vol):
+    """nnq.ConvTranspose3d (conv_transpose.py:484-640) == the oracle's integer formulation
+    (itself pinned against the scatter definition), codes bit for bit."""
+    import oracle.breadth as Br
+    three = lambda v: (v,) * 3 if isinstance(v, int) else tuple(v)
+    rng = np.random.default_rng(cin + cout + sum(vol))
+    m = nn.Sequential(nnq.QuantStub(), nn.ConvTranspose3d(cin, cout, k, stride=stride, padding=padding,
+                                                          output_padding=output_padding, groups=groups,
+                                                          dilation=dilation), nnq.DeQuantStub())
+    prepared = Q.prepare(m, Q.get_default_qconfig())
+    for _ in range(4):
+        prepared[0].activation_post_process(hip(rng.standard_normal((2, cin, *vol)).astype(np.float32)))
+        prepared[1].activation_post_process(hip((rng.standard_normal((2, cout, 2, 2, 2)) * 0.8).astype(np.float32)))
+    qm = Q.convert(prepared)
+    t3 = qm[1]
+    assert isinstance(t3, nnq.ConvTranspose3d) and t3.weight_int8.shape == (cin, cout // groups, *three(k))
+    x = rng.standard_normal((2, cin, *vol)).astype(np.float32)
+    out = t3(qm[0](hip(x)))
+    s0, z0 = qm[0].scale.item(), qm[0].zero_point.item()
+    codes = O.quantize(x, s0, z0, 0, 255, code_offset=-128)
+    want = Br.qconv_transpose3d(codes, t3.weight_int8.numpy(), int(z0) - 128, np.float32(s0), t3.weight_scale.numpy(),
+                                stride=three(stride), padding=three(padding), output_padding=three(output_padding),
+                                dilation=three(dilation), groups=groups, bias=t3.bias.numpy(),
+                                out_mode=O.OUT_REQUANT_I8, out_scale=np.float32(t3.scale.item()),
+                                out_zp=np.float32(t3.zero_point.item()), out_qmin=0, out_qmax=255, out_offset=-128)
+    got = out._grid.codes.numpy()
+    size = [(n - 1) * s - 2 * p + d * (kk - 1) + op + 1 for n, s, p, d, kk, op in
+            zip(vol, three(stride), three(padding), three(dilation), three(k), three(output_padding))]
+    assert got.shape == (2, cout, *size) == want.shape
+    assert np.array_equal(got, want)
+    assert len(np.unique(got)) > 20
+    assert np.isfinite(qm(hip(x)).numpy()).all()

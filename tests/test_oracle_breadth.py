@@ -137,3 +137,64 @@ def test_conv_transpose_scatter_form_against_the_direct_sum(stride, padding, out
                                     acc += x[b, ci, h, wd] * w[ci, co - g * cog, i, j]
                     want[b, co, oh, ow] = acc
     assert np.allclose(out, want, atol=1e-10)
+
+
+@pytest.mark.parametrize("stride,pad,dilation,groups", [
+    ((1, 1, 1), ((0, 0),) * 3, (1, 1, 1), 1), ((2, 1, 2), ((1, 1), (0, 2), (1, 0)), (1, 1, 1), 1),
+    ((1, 2, 1), ((1, 1),) * 3, (2, 1, 1), 2), ((1, 1, 1), ((2, 2), (1, 1), (0, 0)), (1, 2, 2), 4)])
+def test_qconv3d_accumulation_against_scipy_correlate(stride, pad, dilation, groups):
+    """The oracle's Conv3d (numpy tap gather + its qlinear per group) against an independent
+    routine: scipy's N-d cross-correlation of the centred codes with the (zero-dilated) kernel,
+    strided by slicing.  With unit scales and no bias the float32 output is the exact integer
+    sum of (x - zp) * w, so the comparison is exact; a wrong tap order, a transposed kernel, a
+    group mix-up or padding with anything but the zero point would show."""
+    from scipy.signal import correlate
+    rng = np.random.default_rng(11 + groups)
+    B, C, Co, K3 = 2, 8, 12, (3, 2, 3)
+    x = rng.integers(-128, 128, (B, C, 6, 7, 8)).astype(np.int8)
+    w = rng.integers(-127, 128, (Co, C // groups, *K3)).astype(np.int8)
+    zp = -37
+    got = Br.qconv3d(x, w, zp, np.float32(1.0), np.ones(Co, np.float32), stride=stride, pad=pad, dilation=dilation,
+                     groups=groups, out_mode=O.OUT_F32)
+    xc = np.pad(x.astype(np.int64) - zp, ((0, 0), (0, 0), *pad))            # padding = zero point -> 0
+    wd = np.zeros((Co, C // groups, *[d * (k - 1) + 1 for k, d in zip(K3, dilation)]), np.int64)
+    wd[(slice(None), slice(None), *[slice(None, None, d) for d in dilation])] = w
+    Cg, Og = C // groups, Co // groups
+    want = np.zeros(got.shape, np.int64)
+    for b in range(B):
+        for o in range(Co):
+            g = o // Og
+            full = sum(correlate(xc[b, g * Cg + c], wd[o, c], mode="valid", method="direct") for c in range(Cg))
+            want[b, o] = full[::stride[0], ::stride[1], ::stride[2]]
+    assert got.shape == want.shape and np.array_equal(got.astype(np.int64), want)
+
+
+@pytest.mark.parametrize("stride,padding,output_padding,dilation,groups", [
+    ((1, 1, 1), (0, 0, 0), (0, 0, 0), (1, 1, 1), 1), ((2, 3, 2), (1, 0, 1), (1, 2, 0), (1, 1, 1), 1),
+    ((2, 1, 2), (0, 1, 0), (0, 0, 1), (2, 1, 1), 2)])
+def test_qconv_transpose3d_against_the_scatter_definition(stride, padding, output_padding, dilation, groups):
+    """The oracle's ConvTranspose3d (zero insertion + flipped kernel + its Conv3d) against the
+    definition: every input sample adds sample * kernel into the output at stride * position
+    + dilation * tap - padding.  Unit scales, no bias: exact integers."""
+    rng = np.random.default_rng(5 + groups)
+    B, Cin, Cout, K3 = 2, 4, 6, (2, 3, 2)
+    x = rng.integers(-128, 128, (B, Cin, 3, 4, 3)).astype(np.int8)
+    w = rng.integers(-127, 128, (Cin, Cout // groups, *K3)).astype(np.int8)
+    zp = 21
+    got = Br.qconv_transpose3d(x, w, zp, np.float32(1.0), np.ones(Cout // groups, np.float32), stride=stride,
+                               padding=padding, output_padding=output_padding, dilation=dilation, groups=groups,
+                               out_mode=O.OUT_F32)
+    size = [(n - 1) * s - 2 * p + d * (k - 1) + op + 1
+            for n, s, p, d, k, op in zip(x.shape[2:], stride, padding, dilation, K3, output_padding)]
+    full = np.zeros((B, Cout, *[n + 2 * p for n, p in zip(size, padding)]), np.int64)
+    cig, cog = Cin // groups, Cout // groups
+    xc = x.astype(np.int64) - zp
+    for ci in range(Cin):
+        g = ci // cig
+        for idx in np.ndindex(*x.shape[2:]):
+            for tap in np.ndindex(*K3):
+                pos = tuple(i * s + t * d for i, s, t, d in zip(idx, stride, tap, dilation))
+                full[(slice(None), slice(g * cog, (g + 1) * cog), *pos)] += \
+                    xc[(slice(None), ci, *idx)][:, None] * w[(ci, slice(None), *tap)][None, :]
+    want = full[(slice(None), slice(None), *[slice(p, p + n) for p, n in zip(padding, size)])]
+    assert got.shape == want.shape and np.array_equal(got.astype(np.int64), want)
