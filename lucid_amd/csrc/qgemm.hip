@@ -490,8 +490,8 @@ namespace {
 
 // x = every float32 bit pattern of [first, first + count): the tile epilogue's requantize
 // (quant_fast: reciprocal multiply with a guard band, division for the rest), in its three
-// forms (the code, the code minus the zero point, the code shifted into 0..255), against the plain [floor at zero,]
-// divide-round-add-clamp, compared as the codes the two would store.
+// forms (the code, the code minus the zero point, the code shifted into 0..255), against the
+// plain [floor at zero,] divide-round-add-clamp, compared as the codes the two would store.
 __global__ __launch_bounds__(256) void quant_route_check_kernel(float s, float z, float lo, float hi, int relu,
                                                                 unsigned long long first,
                                                                 unsigned long long count,
