@@ -595,23 +595,25 @@ int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH
                               lq_stream stream);
 
 /* Quantized Conv3d (lucid/nn/quantized/conv.py:545-700: dequantize kernel -> F.conv3d ->
- * bias -> fake_quantize) as an explicit GEMM on codes: lq_im2col_ncdhw_i8 gathers the
- * taps of the channels [c0, c0 + Cg) of one group from codes stored in Lucid's own
- * (B, C, D, H, W) order into cols [B*OD*OH*OW, KD*KH*KW*Cg], k = ((kd*KH + kh)*KW + kw)*Cg + c,
- * taps in the padding reading pad_code (the input zero point's stored code);
- * lq_qlinear_i8 multiplies it with that group's kernel rows [Cout/groups, K] (the
- * (O, I, KD*KH*KW) buffer turned by lq_repack_oihw_to_ohwi_i8) with the usual fused
- * epilogue; lq_rows_to_channels_first_i8 writes the [B*L, Ng] result into channels
- * [c0, c0 + Ng) of the (B, Ctot, L) output.  insert > 1 reads the input as if
- * insert - 1 zero-point codes stood between neighbouring samples: the zero insertion
- * of ConvTranspose3d (lucid/nn/quantized/conv_transpose.py:484-640), which is then this
- * stride-1 convolution with the flipped kernel.  kernel / stride / pad_lo / dilation /
- * insert / out_size are host arrays of three ints (depth, height, width). */
-int lq_im2col_ncdhw_i8(const int8_t* x, int8_t* cols, int B, int C, int D, int H, int W, int c0, int Cg,
+ * bias -> fake_quantize) as an explicit GEMM on codes.  lq_transpose_i8 (batched byte
+ * transpose: src[b] R x Cn -> dst[b] Cn x R, batches src_stride / dst_stride bytes
+ * apart) turns Lucid's (B, C, D*H*W) codes channels-last; lq_im2col_ndhwc_i8 gathers the
+ * taps of the channels [c0, c0 + Cg) of one group from (B, D, H, W, C) codes into
+ * cols [B*OD*OH*OW, KD*KH*KW*Cg], k = ((kd*KH + kh)*KW + kw)*Cg + c, taps in the padding
+ * reading pad_code (the input zero point's stored code); lq_qlinear_i8 multiplies it
+ * with that group's kernel rows [Cout/groups, K] (the (O, I, KD*KH*KW) buffer turned by
+ * lq_repack_oihw_to_ohwi_i8) with the usual fused epilogue; lq_transpose_i8 again writes
+ * the [L, Cout/groups] result of each batch into its channel slice of the
+ * (B, Cout, L) output.  insert > 1 reads the input as if insert - 1 zero-point codes
+ * stood between neighbouring samples: the zero insertion of ConvTranspose3d
+ * (lucid/nn/quantized/conv_transpose.py:484-640), which is then this stride-1
+ * convolution with the flipped kernel.  kernel / stride / pad_lo / dilation / insert /
+ * out_size are host arrays of three ints (depth, height, width). */
+int lq_im2col_ndhwc_i8(const int8_t* x, int8_t* cols, int B, int D, int H, int W, int C, int c0, int Cg,
                        const int* kernel, const int* stride, const int* pad_lo, const int* dilation,
                        const int* insert, const int* out_size, int pad_code, lq_stream stream);
-int lq_rows_to_channels_first_i8(const int8_t* rows, int8_t* dst, int B, size_t L, int Ng, int c0, int Ctot,
-                                 lq_stream stream);
+int lq_transpose_i8(const int8_t* src, int8_t* dst, int batches, size_t R, size_t Cn, size_t src_stride,
+                    size_t dst_stride, lq_stream stream);
 
 /* F.pad with mode reflect (1) / replicate (2) / circular (3) on NHWC codes: how a
  * quantized convolution with padding_mode != "zeros" pads before convolving with

@@ -196,8 +196,8 @@ _SIGNATURES["lq_qconv2d_i8"] = [C.POINTER(QConv2dArgs), _vp]
 _SIGNATURES["lq_quantize_nchw_to_nhwc"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_dequantize_nhwc_to_nchw"] = [_vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp]
 _SIGNATURES["lq_repack_oihw_to_ohwi_i8"] = [_vp, _vp, _i, _i, _i, _i, _vp]
-_SIGNATURES["lq_im2col_ncdhw_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]
-_SIGNATURES["lq_rows_to_channels_first_i8"] = [_vp, _vp, _i, C.c_size_t, _i, _i, _i, _vp]
+_SIGNATURES["lq_im2col_ndhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]
+_SIGNATURES["lq_transpose_i8"] = [_vp, _vp, _i, _sz, _sz, _sz, _sz, _vp]
 _SIGNATURES["lq_maxpool2d_nhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 
 _RESTYPE = {"lq_last_error": C.c_char_p, "lq_range_buffer_bytes": C.c_size_t}

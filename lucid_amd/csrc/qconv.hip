@@ -219,26 +219,30 @@ __global__ void repack_oihw_to_ohwi_kernel(const int8_t* __restrict__ w, int8_t*
     }
 }
 
-// Volumetric convolution as an explicit GEMM.  x: codes in Lucid's own (B, C, D, H, W)
-// order; cols: [B*OD*OH*OW, KD*KH*KW*Cg] with k = ((kd*KH + kh)*KW + kw)*Cg + c over the
-// channels [c0, c0 + Cg) of one group; taps in the padding read pad_code (the zero point's
+// Volumetric convolution as an explicit GEMM.  x: codes in channels-last order
+// (B, D, H, W, C); cols: [B*OD*OH*OW, KD*KH*KW*Cg] with k = ((kd*KH + kh)*KW + kw)*Cg + c over
+// the channels [c0, c0 + Cg) of one group; taps in the padding read pad_code (the zero point's
 // stored code).  `ins` > 1 spreads the input over a grid with ins - 1 zero-point codes between
 // neighbours (the zero insertion of a transposed convolution) without materialising it.
-// One byte per lane: consecutive lanes write consecutive bytes.
+// A lane moves VEC consecutive channels of one tap (16 where the channel counts and pointers
+// allow, else 1), consecutive lanes consecutive chunks: reads and writes are contiguous runs.
 struct Vol3 {
     int d, h, w;
 };
 
-__global__ void im2col_ncdhw_i8_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ cols, int C, Vol3 in,
+template <int VEC>
+__global__ void im2col_ndhwc_i8_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ cols, int C, Vol3 in,
                                        int c0, int Cg, Vol3 kern, Vol3 stride, Vol3 pad, Vol3 dil, Vol3 ins,
-                                       Vol3 out, int pad_code, size_t total) {
-    const size_t K = size_t(kern.d) * kern.h * kern.w * Cg;
-    for (size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+                                       Vol3 out, int pad_code, size_t units) {
+    const int chunks = Cg / VEC;
+    const unsigned pad4 = unsigned(pad_code & 0xff) * 0x01010101u;
+    for (size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < units;
          idx += size_t(gridDim.x) * blockDim.x) {
-        const size_t k = idx % K;
-        size_t m = idx / K;
-        const int c = int(k % Cg);
-        int tap = int(k / Cg);
+        const int chunk = int(idx % chunks);
+        size_t r = idx / chunks;
+        const int taps = kern.d * kern.h * kern.w;
+        int tap = int(r % taps);
+        size_t m = r / taps;
         const int kw = tap % kern.w;
         tap /= kern.w;
         const int kh = tap % kern.h, kd = tap / kern.h;
@@ -252,27 +256,44 @@ __global__ void im2col_ncdhw_i8_kernel(const int8_t* __restrict__ x, int8_t* __r
         const int vd = od * stride.d - pad.d + kd * dil.d;
         const int vh = oh * stride.h - pad.h + kh * dil.h;
         const int vw = ow * stride.w - pad.w + kw * dil.w;
-        int v = pad_code;
+        const int8_t* src = nullptr;
         if (vd >= 0 && vh >= 0 && vw >= 0 && vd % ins.d == 0 && vh % ins.h == 0 && vw % ins.w == 0) {
             const int id = vd / ins.d, ih = vh / ins.h, iw = vw / ins.w;
             if (id < in.d && ih < in.h && iw < in.w)
-                v = x[(((b * C + c0 + c) * in.d + id) * in.h + ih) * size_t(in.w) + iw];
+                src = x + (((b * in.d + id) * in.h + ih) * size_t(in.w) + iw) * C + c0 + chunk * VEC;
         }
-        cols[idx] = int8_t(v);
+        int8_t* dst = cols + idx * VEC;  // (m, tap, chunk) in this order IS the matrix order
+        if (VEC == 16) {
+            uint4 v = {pad4, pad4, pad4, pad4};
+            if (src) v = *reinterpret_cast<const uint4*>(src);
+            *reinterpret_cast<uint4*>(dst) = v;
+        } else {
+            *dst = src ? *src : int8_t(pad_code);
+        }
     }
 }
 
-// GEMM result rows [B*L, Ng] (position-major) into channels [c0, c0 + Ng) of a
-// channels-first tensor (B, Ctot, L): one byte per lane, consecutive lanes along L.
-__global__ void rows_to_channels_first_i8_kernel(const int8_t* __restrict__ rows, int8_t* __restrict__ dst,
-                                                 size_t L, int Ng, int c0, int Ctot, size_t total) {
-    for (size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
-         idx += size_t(gridDim.x) * blockDim.x) {
-        const size_t l = idx % L;
-        const size_t r = idx / L;
-        const int n = int(r % Ng);
-        const size_t b = r / Ng;
-        dst[(b * Ctot + c0 + n) * L + l] = rows[(b * L + l) * Ng + n];
+// Batched byte transpose through LDS: src[b] is R x Cn (rows contiguous), dst[b] is Cn x R;
+// batches are src_stride / dst_stride bytes apart (so a destination may be a channel slice of
+// a larger tensor).  64 x 64 tiles; a wavefront reads and writes 64 consecutive bytes.
+__global__ __launch_bounds__(256) void transpose_i8_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst,
+                                                           size_t R, size_t Cn, size_t src_stride,
+                                                           size_t dst_stride, unsigned tiles_c) {
+    __shared__ int8_t tile[64][65];
+    const size_t r0 = size_t(blockIdx.x / tiles_c) * 64, c0 = size_t(blockIdx.x % tiles_c) * 64;
+    const int8_t* s = src + size_t(blockIdx.y) * src_stride;
+    int8_t* d = dst + size_t(blockIdx.y) * dst_stride;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const size_t r = r0 + j * 4 + w, c = c0 + lane;
+        if (r < R && c < Cn) tile[j * 4 + w][lane] = s[r * Cn + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const size_t c = c0 + j * 4 + w, r = r0 + lane;
+        if (r < R && c < Cn) d[c * R + r] = tile[lane][j * 4 + w];
     }
 }
 
@@ -611,44 +632,52 @@ int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH
     return LQ_OK;
 }
 
-int lq_im2col_ncdhw_i8(const int8_t* x, int8_t* cols, int B, int C, int D, int H, int W, int c0, int Cg,
+int lq_im2col_ndhwc_i8(const int8_t* x, int8_t* cols, int B, int D, int H, int W, int C, int c0, int Cg,
                        const int* kernel, const int* stride, const int* pad_lo, const int* dilation,
                        const int* insert, const int* out_size, int pad_code, lq_stream stream) {
     LQ_REQUIRE(kernel && stride && pad_lo && dilation && insert && out_size, LQ_ERR_VALUE,
-               "im2col_ncdhw: NULL geometry");
-    LQ_REQUIRE(B >= 0 && C > 0 && D > 0 && H > 0 && W > 0, LQ_ERR_SHAPE, "im2col_ncdhw: bad input shape");
-    LQ_REQUIRE(c0 >= 0 && Cg > 0 && c0 + Cg <= C, LQ_ERR_SHAPE, "im2col_ncdhw: channels [%d, %d) of %d", c0,
+               "im2col_ndhwc: NULL geometry");
+    LQ_REQUIRE(B >= 0 && C > 0 && D > 0 && H > 0 && W > 0, LQ_ERR_SHAPE, "im2col_ndhwc: bad input shape");
+    LQ_REQUIRE(c0 >= 0 && Cg > 0 && c0 + Cg <= C, LQ_ERR_SHAPE, "im2col_ndhwc: channels [%d, %d) of %d", c0,
                c0 + Cg, C);
-    LQ_REQUIRE(pad_code >= -128 && pad_code <= 127, LQ_ERR_VALUE, "im2col_ncdhw: padding code %d is no int8", pad_code);
+    LQ_REQUIRE(pad_code >= -128 && pad_code <= 127, LQ_ERR_VALUE, "im2col_ndhwc: padding code %d is no int8", pad_code);
     // any tap outside the spread input reads the padding code, so out_size needs no upper bound:
     // high-side padding, e.g. a transposed convolution's output_padding, is simply more outputs
     for (int i = 0; i < 3; ++i)
         LQ_REQUIRE(kernel[i] > 0 && stride[i] > 0 && dilation[i] > 0 && insert[i] > 0 && pad_lo[i] >= 0 &&
                        out_size[i] >= 0,
-                   LQ_ERR_VALUE, "im2col_ncdhw: bad geometry in dimension %d", i);
+                   LQ_ERR_VALUE, "im2col_ndhwc: bad geometry in dimension %d", i);
     const size_t M = size_t(B) * out_size[0] * out_size[1] * out_size[2];
     const size_t total = M * kernel[0] * kernel[1] * kernel[2] * Cg;
     if (total == 0) return LQ_OK;
-    LQ_REQUIRE(x && cols, LQ_ERR_VALUE, "im2col_ncdhw: NULL pointer");
-    hipLaunchKernelGGL(im2col_ncdhw_i8_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream), x, cols, C,
-                       Vol3{D, H, W}, c0, Cg, Vol3{kernel[0], kernel[1], kernel[2]},
-                       Vol3{stride[0], stride[1], stride[2]}, Vol3{pad_lo[0], pad_lo[1], pad_lo[2]},
-                       Vol3{dilation[0], dilation[1], dilation[2]}, Vol3{insert[0], insert[1], insert[2]},
-                       Vol3{out_size[0], out_size[1], out_size[2]}, pad_code, total);
-    LQ_CHECK_LAUNCH("im2col_ncdhw");
+    LQ_REQUIRE(x && cols, LQ_ERR_VALUE, "im2col_ndhwc: NULL pointer");
+    const bool vec = C % 16 == 0 && Cg % 16 == 0 && c0 % 16 == 0 && aligned16(x) && aligned16(cols);
+    const Vol3 in{D, H, W}, kn{kernel[0], kernel[1], kernel[2]}, st{stride[0], stride[1], stride[2]},
+        pd{pad_lo[0], pad_lo[1], pad_lo[2]}, dl{dilation[0], dilation[1], dilation[2]},
+        is{insert[0], insert[1], insert[2]}, ot{out_size[0], out_size[1], out_size[2]};
+    if (vec)
+        hipLaunchKernelGGL(im2col_ndhwc_i8_kernel<16>, dim3(grid_1d(total / 16)), dim3(256), 0, as_stream(stream), x,
+                           cols, C, in, c0, Cg, kn, st, pd, dl, is, ot, pad_code, total / 16);
+    else
+        hipLaunchKernelGGL(im2col_ndhwc_i8_kernel<1>, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream), x, cols,
+                           C, in, c0, Cg, kn, st, pd, dl, is, ot, pad_code, total);
+    LQ_CHECK_LAUNCH("im2col_ndhwc");
     return LQ_OK;
 }
 
-int lq_rows_to_channels_first_i8(const int8_t* rows, int8_t* dst, int B, size_t L, int Ng, int c0, int Ctot,
-                                 lq_stream stream) {
-    LQ_REQUIRE(B >= 0 && Ng > 0 && c0 >= 0 && c0 + Ng <= Ctot, LQ_ERR_SHAPE,
-               "rows_to_channels_first: channels [%d, %d) of %d", c0, c0 + Ng, Ctot);
-    const size_t total = size_t(B) * L * Ng;
-    if (total == 0) return LQ_OK;
-    LQ_REQUIRE(rows && dst, LQ_ERR_VALUE, "rows_to_channels_first: NULL pointer");
-    hipLaunchKernelGGL(rows_to_channels_first_i8_kernel, dim3(grid_1d(total)), dim3(256), 0, as_stream(stream), rows,
-                       dst, L, Ng, c0, Ctot, total);
-    LQ_CHECK_LAUNCH("rows_to_channels_first");
+int lq_transpose_i8(const int8_t* src, int8_t* dst, int batches, size_t R, size_t Cn, size_t src_stride,
+                    size_t dst_stride, lq_stream stream) {
+    LQ_REQUIRE(batches >= 0 && batches < 65536, LQ_ERR_SHAPE, "transpose_i8: %d batches (at most 65535)", batches);
+    if (batches == 0 || R == 0 || Cn == 0) return LQ_OK;
+    LQ_REQUIRE(src && dst, LQ_ERR_VALUE, "transpose_i8: NULL pointer");
+    LQ_REQUIRE(src_stride >= R * Cn && dst_stride >= R * Cn, LQ_ERR_SHAPE,
+               "transpose_i8: batch stride smaller than a %zu x %zu matrix", R, Cn);
+    const size_t tiles_r = (R + 63) / 64, tiles_c = (Cn + 63) / 64;
+    LQ_REQUIRE(tiles_r * tiles_c < 0x7fffffffull && tiles_c < 0x7fffffffull, LQ_ERR_SHAPE,
+               "transpose_i8: matrix too large");
+    hipLaunchKernelGGL(transpose_i8_kernel, dim3(unsigned(tiles_r * tiles_c), unsigned(batches)), dim3(256), 0,
+                       as_stream(stream), src, dst, R, Cn, src_stride, dst_stride, unsigned(tiles_c));
+    LQ_CHECK_LAUNCH("transpose_i8");
     return LQ_OK;
 }
 

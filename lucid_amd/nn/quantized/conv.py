@@ -256,7 +256,8 @@ def volumetric_gemm(name, x: Tensor, g, w_rows: Tensor, wsum: Tensor, w_scale: T
     """A 3-d convolution on codes as an explicit GEMM, group by group: gather the taps of
     ``x``'s ``(B, C, D, H, W)`` codes (``insert`` > 1: as if zero-point codes stood between
     neighbouring samples), multiply with the group's kernel rows ``[Cout/groups, taps * C/groups]``
-    through the fused int8 GEMM, write the result channels-first.  ``pads`` = ((lo, hi),) * 3."""
+    through the fused int8 GEMM, write the result channels-first.  The codes are turned
+    channels-last first, so that the gather moves contiguous runs.  ``pads`` = ((lo, hi),) * 3."""
     B, Cc, D, H, W = x.shape
     spread = [(n - 1) * i + 1 for n, i in zip((D, H, W), insert)]
     outs = [(n + lo + hi - d * (k - 1) - 1) // s + 1
@@ -269,17 +270,21 @@ def volumetric_gemm(name, x: Tensor, g, w_rows: Tensor, wsum: Tensor, w_scale: T
     a_zp = int(g.zp_host) + g.offset
     off = storage_offset(qdtype)
     i3 = lambda v: (C.c_int * 3)(*[int(e) for e in v])
+    vol = D * H * W
+    last = Tensor.empty((B, D, H, W, Cc), T.int8, "hip")      # channels-last copy of the input codes
+    _C.call("lq_transpose_i8", g.codes.data_ptr, last.data_ptr, B, Cc, vol, Cc * vol, Cc * vol, None)
     codes = Tensor.empty((B, Co, *outs), T.int8, "hip")
     cols = Tensor.empty((B * L, Cg * kernel[0] * kernel[1] * kernel[2]), T.int8, "hip")
     for grp in range(groups):
-        _C.call("lq_im2col_ncdhw_i8", g.codes.data_ptr, cols.data_ptr, B, Cc, D, H, W, grp * Cg, Cg, i3(kernel),
+        _C.call("lq_im2col_ndhwc_i8", last.data_ptr, cols.data_ptr, B, D, H, W, Cc, grp * Cg, Cg, i3(kernel),
                 i3(stride), i3([p[0] for p in pads]), i3(dilation), i3(insert), i3(outs), a_zp, None)
         part = lambda t: t.row_range(grp * Og, (grp + 1) * Og)
         y = _ops.qlinear_i8(cols, part(w_rows), a_zp=a_zp, a_scale=g.scale, w_scale=part(w_scale), wsum=part(wsum),
                             bias=None if bias is None else part(bias), relu=relu, out_mode=_ops.OUT_REQUANT_I8,
                             out_scale=scale, out_zp=zero_point, out_qmin=qdtype.quant_min,
                             out_qmax=qdtype.quant_max, out_offset=off)
-        _C.call("lq_rows_to_channels_first_i8", y.data_ptr, codes.data_ptr, B, L, Og, grp * Og, Co, None)
+        # each batch's [L, Og] block -> its (Og, L) channel slice of the (B, Co, L) output
+        _C.call("lq_transpose_i8", y.data_ptr, codes.data_ptr + grp * Og * L, B, L, Og, L * Og, Co * L, None)
     return Tensor.on_grid((B, Co, *outs), Grid(codes, scale, zero_point, qdtype, off, zp_host, "plain"))
 
 
