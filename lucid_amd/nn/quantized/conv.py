@@ -208,15 +208,15 @@ class Conv1d(Conv2d):
         if g.layout != "plain":
             raise _C.LucidError(f"{name}: 3-d activation codes must be stored in their own (B, C, L) order")
         B, Cc, Ln = x.shape
-        # (B, C, L) -> (B, 1, L, C): the weight repacker is a generic (O, I, K) -> (O, K, I) turn
+        # (B, C, L) -> (B, 1, L, C): a batched byte transpose
         nhwc = Tensor.empty((B, 1, Ln, Cc), T.int8, "hip")
-        _C.call("lq_repack_oihw_to_ohwi_i8", g.codes.data_ptr, nhwc.data_ptr, B, Cc, 1, Ln, None)
+        _C.call("lq_transpose_i8", g.codes.data_ptr, nhwc.data_ptr, B, Cc, Ln, Cc * Ln, Cc * Ln, None)
         x4 = Tensor.on_grid((B, Cc, 1, Ln), Grid(nhwc, g.scale, g.zero_point, g.qdtype, g.offset, g.zp_host, "nhwc"))
         y4 = super().forward(x4)
         gy = y4._grid
         _, Co, _, Lo = y4.shape
         plain = Tensor.empty((B, Co, Lo), T.int8, "hip")
-        _C.call("lq_repack_oihw_to_ohwi_i8", gy.codes.data_ptr, plain.data_ptr, B, Lo, 1, Co, None)
+        _C.call("lq_transpose_i8", gy.codes.data_ptr, plain.data_ptr, B, Lo, Co, Lo * Co, Lo * Co, None)
         return Tensor.on_grid((B, Co, Lo), Grid(plain, gy.scale, gy.zero_point, gy.qdtype, gy.offset, gy.zp_host,
                                                 "plain"))
 
