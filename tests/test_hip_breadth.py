@@ -454,3 +454,24 @@ def test_conv_transpose3d_bit_exact_against_the_oracle(cin, cout, k, stride, pad
     assert np.array_equal(got, want)
     assert len(np.unique(got)) > 20
     assert np.isfinite(qm(hip(x)).numpy()).all()
+
+
+@pytest.mark.parametrize("batches,R,Cn,pad_src,pad_dst", [(1, 64, 64, 0, 0), (3, 70, 130, 0, 0), (2, 1, 257, 5, 0),
+                                                           (4, 200, 3, 0, 96), (2, 129, 65, 7, 33)])
+def test_batched_byte_transpose(batches, R, Cn, pad_src, pad_dst):
+    """lq_transpose_i8: every batch's R x Cn matrix becomes Cn x R, batch strides respected on
+    both sides (the gap bytes of the destination keep what they held), edge tiles included."""
+    from lucid_amd import _C
+    rng = np.random.default_rng(R * 7 + Cn)
+    ss, ds = R * Cn + pad_src, R * Cn + pad_dst
+    src = rng.integers(-128, 128, batches * ss).astype(np.int8)
+    dst0 = rng.integers(-128, 128, batches * ds).astype(np.int8)
+    s, d = hip(src), hip(dst0)
+    _C.call("lq_transpose_i8", s.data_ptr, d.data_ptr, batches, R, Cn, ss, ds, None)
+    got = d.numpy()
+    want = dst0.copy()
+    for b in range(batches):
+        want[b * ds:b * ds + R * Cn] = src[b * ss:b * ss + R * Cn].reshape(R, Cn).T.ravel()
+    assert np.array_equal(got, want)
+    with pytest.raises(Exception):
+        _C.call("lq_transpose_i8", s.data_ptr, d.data_ptr, batches, R, Cn, R * Cn - 1, ds, None)
