@@ -24,8 +24,15 @@
  *     parameters use C = 1.
  *   - launches are asynchronous on `stream` (a hipStream_t; NULL = the default
  *     stream).  lq_sync / lq_d2h synchronise.
- *   - reductions and the split-K GEMM use a per-device workspace owned by the
- *     library; calls that overlap on one device on different streams race on it.
+ *   - reductions, gathered matrices and the split-K GEMM use scratch owned by
+ *     the library, one buffer per (device, stream): calls on different streams
+ *     do not share scratch and may overlap; calls on one stream are ordered by
+ *     it.  The functions are re-entrant (Lucid's dispatcher is read-only and
+ *     concurrent-safe after start-up, lucid/_C/backend/Dispatcher.h:49-52).
+ *   - an output that is also read by the same call (out == residual, or
+ *     out == join.q of lq_qlinear_i8 / lq_qconv2d_i8) is allowed: every element
+ *     is read before it is written by the same lane.  The first-call tile
+ *     tuner is skipped for such calls (it would apply the operand repeatedly).
  */
 #ifndef LUCID_HIP_H
 #define LUCID_HIP_H

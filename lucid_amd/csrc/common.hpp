@@ -35,9 +35,15 @@ int hip_fail(hipError_t e, const char* what);
         if (_e != hipSuccess) return lq::hip_fail(_e, "launch " name); \
     } while (0)
 
-// Per-device scratch for reduction partials and split-K partial sums.
-// Grown on demand; never shrunk.  Calls that overlap on one device race on it.
-int workspace(size_t nbytes, void** ptr);
+// Library-owned scratch for reduction partials, gathered matrices and split-K partial
+// sums: one buffer per (device, stream, kind), grown on demand and never shrunk, so calls
+// on different streams do not share scratch and calls on one stream are ordered by it.
+// A buffer that is outgrown stays allocated while any captured graph exists (its address
+// may be baked into the graph).  `fresh` reports that the buffer was (re)allocated by
+// this request and holds no defined contents.
+int stream_buffer(int kind, size_t nbytes, size_t min_bytes, hipStream_t stream, void** ptr, bool* fresh);
+// kind 0: the general workspace (at least 4 MiB)
+int workspace(size_t nbytes, hipStream_t stream, void** ptr);
 
 inline hipStream_t as_stream(lq_stream s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -453,7 +453,7 @@ int lq_histc_f32(const float* x, size_t n, double lo, double hi, int bins, float
     LQ_REQUIRE(n == 0 || x, LQ_ERR_VALUE, "histc: NULL input");
     hipStream_t st = as_stream(stream);
     void* ws = nullptr;
-    int rc = workspace(size_t(bins) * sizeof(unsigned long long), &ws);
+    int rc = workspace(size_t(bins) * sizeof(unsigned long long), as_stream(stream), &ws);
     if (rc) return rc;
     auto* counts = static_cast<unsigned long long*>(ws);
     rc = lq_fill_bytes(counts, 0, size_t(bins) * sizeof(unsigned long long), stream);

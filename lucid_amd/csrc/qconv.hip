@@ -514,7 +514,7 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
         const size_t flt_bytes = (size_t(p->Cout) * p->KH * KWp * 4 + 255) / 256 * 256;
         LQ_REQUIRE(size_t(p->B) * Hp * Wp * 4 < 0xffffffffull, LQ_ERR_SHAPE, "qconv2d_i8: padded image too large");
         void* ws = nullptr;
-        int rc = workspace(img_bytes + flt_bytes, &ws);
+        int rc = workspace(img_bytes + flt_bytes, st, &ws);
         if (rc) return rc;
         int8_t* img = static_cast<int8_t*>(ws);
         int8_t* flt = img + img_bytes;
@@ -556,7 +556,7 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
     const size_t cols_bytes = (M * Kp + 255) / 256 * 256;
     const size_t w_bytes = (size_t(Og) * Kp + 255) / 256 * 256;
     void* ws = nullptr;
-    int rc = workspace(cols_bytes + w_bytes, &ws);
+    int rc = workspace(cols_bytes + w_bytes, st, &ws);
     if (rc) return rc;
     int8_t* cols = static_cast<int8_t*>(ws);
     int8_t* wpad = cols + cols_bytes;

@@ -29,35 +29,25 @@
 using namespace lq;
 
 namespace lq {
-SkScratch g_sk[16];
-
-// Returns in *out the device's scratch grown to the requested sizes, or null
-// when it would have to grow and may not (the stream is being captured into a
-// graph: growing synchronizes the device).
-int sk_scratch(size_t counters, size_t slab_bytes, bool may_grow, SkScratch** out) {
-    int dev = 0;
-    LQ_HIP(hipGetDevice(&dev));
-    LQ_REQUIRE(dev >= 0 && dev < 16, LQ_ERR_DEVICE, "device index %d out of range", dev);
-    SkScratch& s = g_sk[dev];
-    *out = nullptr;
-    if ((s.counter_count < counters || s.slab_bytes < slab_bytes) && !may_grow) return LQ_OK;
-    if (s.counter_count < counters) {
-        LQ_HIP(hipDeviceSynchronize());
-        if (s.counters) LQ_HIP(hipFree(s.counters));
-        s.counters = nullptr;
-        const size_t want = counters < 65536 ? 65536 : counters;
-        LQ_HIP(hipMalloc(&s.counters, want * sizeof(int)));
-        LQ_HIP(hipMemset(s.counters, 0, want * sizeof(int)));
-        s.counter_count = want;
+// The stream's stream-K scratch, grown to the requested sizes: arrival counters (zero
+// between launches: freshly allocated ones are cleared by a kernel on the stream, which a
+// graph capture records like any other launch) and the accumulator slabs.
+int sk_scratch(size_t counters, size_t slab_bytes, hipStream_t st, SkScratch* out) {
+    void* c = nullptr;
+    bool fresh = false;
+    int rc = stream_buffer(1, counters * sizeof(int), size_t(65536) * sizeof(int), st, &c, &fresh);
+    if (rc) return rc;
+    if (fresh) {
+        const size_t bytes = counters * sizeof(int) < size_t(65536) * sizeof(int) ? size_t(65536) * sizeof(int)
+                                                                                : counters * sizeof(int);
+        rc = lq_fill_bytes(c, 0, bytes, reinterpret_cast<lq_stream>(st));
+        if (rc) return rc;
     }
-    if (s.slab_bytes < slab_bytes) {
-        LQ_HIP(hipDeviceSynchronize());
-        if (s.slabs) LQ_HIP(hipFree(s.slabs));
-        s.slabs = nullptr;
-        LQ_HIP(hipMalloc(&s.slabs, slab_bytes));
-        s.slab_bytes = slab_bytes;
-    }
-    *out = &s;
+    void* s = nullptr;
+    rc = stream_buffer(2, slab_bytes, 0, st, &s, nullptr);
+    if (rc) return rc;
+    out->counters = static_cast<int*>(c);
+    out->slabs = static_cast<int32_t*>(s);
     return LQ_OK;
 }
 
@@ -189,7 +179,12 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     LQ_HIP(hipStreamIsCapturing(st, &capturing));
     // too little work to be worth timing: a handful of tiles whatever the shape
     const double ops = 2.0 * g.M * double(g.N) * g.K * groups;
-    if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9) return LQ_OK;
+    // timing launches the candidates many times into the caller's output: not when that output
+    // is also an operand the epilogue reads (an in-place residual or join would be applied
+    // once per timing launch)
+    const bool in_place = (g.residual && static_cast<const void*>(g.residual) == g.out) ||
+                          (g.join_q && static_cast<const void*>(g.join_q) == g.out);
+    if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9 || in_place) return LQ_OK;
 
     // candidates are whole tile_config values (shape | schedule << 8)
     int cands[16], n = 0;

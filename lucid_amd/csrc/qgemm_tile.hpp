@@ -839,15 +839,13 @@ using CfgTall8 = TileCfg<128, 256, 64, 2, 4, 3, 2>;
 
 }  // namespace
 
-// Stream-K scratch per device: arrival counters (zero between launches: the
+// Stream-K scratch of one stream: arrival counters (zero between launches: the
 // finisher of a tile resets its counter) and two accumulator slabs per worker.
 struct SkScratch {
     int* counters = nullptr;
-    size_t counter_count = 0;
     int32_t* slabs = nullptr;
-    size_t slab_bytes = 0;
 };
-int sk_scratch(size_t counters, size_t slab_bytes, bool may_grow, SkScratch** out);
+int sk_scratch(size_t counters, size_t slab_bytes, hipStream_t st, SkScratch* out);
 
 namespace {
 
@@ -906,19 +904,12 @@ int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st
         if (split > nk / 4) split = nk / 4;
         workers = long(tiles) * (split < 1 ? 1 : split);
     }
-    SkScratch* s = nullptr;
+    SkScratch s;
     const size_t slab_words = size_t(Cfg::TM) * Cfg::TN * 16 * Cfg::THREADS;
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    LQ_HIP(hipStreamIsCapturing(st, &capturing));
-    int rc = sk_scratch(size_t(sk_tiles) * groups, size_t(groups) * workers * 2 * slab_words * 4,
-                        capturing == hipStreamCaptureStatusNone, &s);
+    int rc = sk_scratch(size_t(sk_tiles) * groups, size_t(groups) * workers * 2 * slab_words * 4, st, &s);
     if (rc) return rc;
-    if (!s) {  // scratch too small and the stream is being captured: one block per tile
-        LQ_HIP(hipLaunchKernel(fn_dp, dim3(tiles, groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
-        return LQ_OK;
-    }
-    copy.sk_counters = s->counters;
-    copy.sk_slabs = s->slabs;
+    copy.sk_counters = s.counters;
+    copy.sk_slabs = s.slabs;
     copy.sk_tiles = sk_tiles;
     LQ_HIP(hipLaunchKernel(fn_sk, dim3(unsigned(workers), groups), dim3(Cfg::THREADS), kargs, Cfg::SMEM, st));
     return LQ_OK;

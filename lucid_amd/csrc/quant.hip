@@ -651,6 +651,87 @@ __global__ __launch_bounds__(1024) void quantize_tensor_dynamic_kernel(
     for (size_t e = quads * 4 + threadIdx.x; e < n; e += 1024) op.scalar(e, s, z);
 }
 
+
+// min / max launch sequence.  `get_ws(nbytes, &ptr)`
+// supplies the memory for the partial results of a two-stage reduction; `ws_limit` is the
+// most it can supply: the number of slices per channel is cut down to fit (the result does
+// not depend on it: min and max are exact in any order).
+template <class GetWs>
+int minmax_launch(const float* x, size_t outer, size_t C, size_t inner, float* mn, float* mx, hipStream_t st,
+                  size_t ws_limit, GetWs get_ws) {
+    LQ_REQUIRE(mn && mx, LQ_ERR_VALUE, "minmax: output pointer is NULL");
+    LQ_REQUIRE(C >= 1, LQ_ERR_SHAPE, "minmax: C must be >= 1");
+    const size_t per_channel = outer * inner;
+    if (per_channel == 0) {  // empty reduction: identities (Reduce.cpp:95,107)
+        hipLaunchKernelGGL(minmax_identity_kernel, dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, mn,
+                           mx, C);
+        LQ_CHECK_LAUNCH("minmax_identity");
+        return LQ_OK;
+    }
+    LQ_REQUIRE(x, LQ_ERR_VALUE, "minmax: x is NULL");
+    LQ_REQUIRE(C <= 0x3fffffffull, LQ_ERR_SHAPE, "minmax: too many channels (%zu)", C);
+
+    if (inner < 64 && C > 1) {
+        const size_t cols = C * inner;
+        // enough row slices to occupy the chip, at least 32 rows each
+        size_t col_blocks = (cols + kThreads - 1) / kThreads;
+        size_t splits = 2048 / col_blocks;
+        if (splits > outer / 32) splits = outer / 32;
+        if (splits < 1) splits = 1;
+        if (splits > 65535) splits = 65535;
+        LQ_REQUIRE(2 * cols * sizeof(float) <= ws_limit, LQ_ERR_SHAPE,
+                   "minmax: %zu channel-inner columns need %zu bytes of partial results, more than the %zu available",
+                   cols, 2 * cols * sizeof(float), ws_limit);
+        if (splits > ws_limit / (2 * cols * sizeof(float))) splits = ws_limit / (2 * cols * sizeof(float));
+        void* ws = nullptr;
+        int rc = get_ws(2 * splits * cols * sizeof(float), &ws);
+        if (rc) return rc;
+        float* pmin = static_cast<float*>(ws);
+        float* pmax = pmin + splits * cols;
+        hipLaunchKernelGGL(minmax_col_kernel, dim3(unsigned(col_blocks), unsigned(splits)),
+                           dim3(kThreads), 0, st, x, outer, cols, unsigned(splits), pmin, pmax);
+        LQ_CHECK_LAUNCH("minmax_col");
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(256), 0, st, pmin, pmax, C,
+                           unsigned(splits), unsigned(inner), mn, mx);
+        LQ_CHECK_LAUNCH("minmax_finalize");
+        return LQ_OK;
+    }
+
+    // contiguous runs: aim for ~2048 blocks, each slice at least 4096 elements
+    size_t splits = 1;
+    if (C < 2048) {
+        splits = 2048 / C;
+        size_t max_splits = inner / 4096;
+        if (splits > max_splits) splits = max_splits;
+        if (splits < 1) splits = 1;
+    }
+    const bool vec = (inner % 4 == 0) && aligned16(x);
+    float *pmin = mn, *pmax = mx;
+    if (splits > ws_limit / (2 * C * sizeof(float))) splits = ws_limit / (2 * C * sizeof(float));
+    if (splits < 1) splits = 1;  // one block per channel writes mn / mx directly: no partials at all
+    if (splits > 1) {
+        void* ws = nullptr;
+        int rc = get_ws(2 * splits * C * sizeof(float), &ws);
+        if (rc) return rc;
+        pmin = static_cast<float*>(ws);
+        pmax = pmin + splits * C;
+    }
+    dim3 grid{unsigned(C * splits)}, block{kThreads};
+    if (vec)
+        hipLaunchKernelGGL((minmax_seg_kernel<true>), grid, block, 0, st, x, outer, C, inner,
+                           unsigned(splits), pmin, pmax);
+    else
+        hipLaunchKernelGGL((minmax_seg_kernel<false>), grid, block, 0, st, x, outer, C, inner,
+                           unsigned(splits), pmin, pmax);
+    LQ_CHECK_LAUNCH("minmax_seg");
+    if (splits > 1) {
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(256), 0, st, pmin, pmax, C,
+                           unsigned(splits), 1u, mn, mx);
+        LQ_CHECK_LAUNCH("minmax_finalize");
+    }
+    return LQ_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -703,72 +784,9 @@ int lq_quantize_rows_dynamic_i8(const float* x, size_t rows, size_t cols, int sy
 
 int lq_minmax(const float* x, size_t outer, size_t C, size_t inner, float* mn, float* mx,
               lq_stream stream) {
-    LQ_REQUIRE(mn && mx, LQ_ERR_VALUE, "minmax: output pointer is NULL");
-    LQ_REQUIRE(C >= 1, LQ_ERR_SHAPE, "minmax: C must be >= 1");
     hipStream_t st = as_stream(stream);
-    const size_t per_channel = outer * inner;
-    if (per_channel == 0) {  // empty reduction: identities (Reduce.cpp:95,107)
-        hipLaunchKernelGGL(minmax_identity_kernel, dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, mn,
-                           mx, C);
-        LQ_CHECK_LAUNCH("minmax_identity");
-        return LQ_OK;
-    }
-    LQ_REQUIRE(x, LQ_ERR_VALUE, "minmax: x is NULL");
-    LQ_REQUIRE(C <= 0x3fffffffull, LQ_ERR_SHAPE, "minmax: too many channels (%zu)", C);
-
-    if (inner < 64 && C > 1) {
-        const size_t cols = C * inner;
-        // enough row slices to occupy the chip, at least 32 rows each
-        size_t col_blocks = (cols + kThreads - 1) / kThreads;
-        size_t splits = 2048 / col_blocks;
-        if (splits > outer / 32) splits = outer / 32;
-        if (splits < 1) splits = 1;
-        if (splits > 65535) splits = 65535;
-        void* ws = nullptr;
-        int rc = workspace(2 * splits * cols * sizeof(float), &ws);
-        if (rc) return rc;
-        float* pmin = static_cast<float*>(ws);
-        float* pmax = pmin + splits * cols;
-        hipLaunchKernelGGL(minmax_col_kernel, dim3(unsigned(col_blocks), unsigned(splits)),
-                           dim3(kThreads), 0, st, x, outer, cols, unsigned(splits), pmin, pmax);
-        LQ_CHECK_LAUNCH("minmax_col");
-        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(256), 0, st, pmin, pmax, C,
-                           unsigned(splits), unsigned(inner), mn, mx);
-        LQ_CHECK_LAUNCH("minmax_finalize");
-        return LQ_OK;
-    }
-
-    // contiguous runs: aim for ~2048 blocks, each slice at least 4096 elements
-    size_t splits = 1;
-    if (C < 2048) {
-        splits = 2048 / C;
-        size_t max_splits = inner / 4096;
-        if (splits > max_splits) splits = max_splits;
-        if (splits < 1) splits = 1;
-    }
-    const bool vec = (inner % 4 == 0) && aligned16(x);
-    float *pmin = mn, *pmax = mx;
-    if (splits > 1) {
-        void* ws = nullptr;
-        int rc = workspace(2 * splits * C * sizeof(float), &ws);
-        if (rc) return rc;
-        pmin = static_cast<float*>(ws);
-        pmax = pmin + splits * C;
-    }
-    dim3 grid{unsigned(C * splits)}, block{kThreads};
-    if (vec)
-        hipLaunchKernelGGL((minmax_seg_kernel<true>), grid, block, 0, st, x, outer, C, inner,
-                           unsigned(splits), pmin, pmax);
-    else
-        hipLaunchKernelGGL((minmax_seg_kernel<false>), grid, block, 0, st, x, outer, C, inner,
-                           unsigned(splits), pmin, pmax);
-    LQ_CHECK_LAUNCH("minmax_seg");
-    if (splits > 1) {
-        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(unsigned(C)), dim3(256), 0, st, pmin, pmax, C,
-                           unsigned(splits), 1u, mn, mx);
-        LQ_CHECK_LAUNCH("minmax_finalize");
-    }
-    return LQ_OK;
+    return minmax_launch(x, outer, C, inner, mn, mx, st, ~size_t(0),
+                         [st](size_t nbytes, void** ws) { return workspace(nbytes, st, ws); });
 }
 
 int lq_calc_qparams(const float* mn, const float* mx, size_t C, int symmetric, int qmin, int qmax,

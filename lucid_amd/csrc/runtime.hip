@@ -34,32 +34,86 @@ int hip_fail(hipError_t e, const char* what) {
 
 namespace {
 constexpr int kMaxDevices = 16;
-struct Workspace {
+
+// One lock for the runtime's host-side state: the per-stream scratch buffers, the
+// caching pool and the graph tables (a scratch request asks whether graphs are
+// alive, and destroying a graph releases retired scratch, so separate locks
+// would have to nest both ways).
+std::recursive_mutex g_rt_mutex;
+
+// ---- per-(device, stream) scratch
+// Reduction partials, the im2col fallback's matrix and the split-K slabs live in
+// buffers owned by the library.  They are keyed by the stream the call runs on,
+// so calls on different streams never share one (calls that overlap on ONE
+// stream's buffer are ordered by that stream).  A buffer only ever grows.  The
+// block it outgrows is not freed on the spot: a captured graph may have its
+// address baked into kernel nodes, and freeing needs a device-wide
+// synchronisation that is illegal while a stream is capturing.  Outgrown blocks
+// are retired and released at the next moment when no graph exists and nothing
+// is being captured.
+struct StreamBuf {
     void* ptr = nullptr;
     size_t size = 0;
 };
-Workspace g_ws[kMaxDevices];
-std::mutex g_ws_mutex;
+struct BufKey {
+    int dev;
+    hipStream_t stream;
+    int kind;
+    bool operator<(const BufKey& o) const {
+        if (dev != o.dev) return dev < o.dev;
+        if (stream != o.stream) return stream < o.stream;
+        return kind < o.kind;
+    }
+};
+std::map<BufKey, StreamBuf> g_bufs;
+std::vector<void*> g_retired;
+
+// ---- graphs (tables; the entry points are further down)
+struct GraphRec {
+    hipGraph_t graph = nullptr;      // the captured template, kept until the exec is destroyed
+    hipGraphExec_t exec = nullptr;   // null while capturing or after a failed end
+    std::vector<std::pair<int, void*>> blocks;  // (device, block) allocated during capture
+};
+std::unordered_map<int, GraphRec> g_graphs;
+int g_captures_in_progress = 0;
+int g_next_graph_id = 1;
+thread_local int t_capturing_graph = 0;  // id of the graph this thread is capturing, 0 = none
+
+// caller holds g_rt_mutex
+bool graphs_quiescent() { return g_graphs.empty() && g_captures_in_progress == 0; }
+
+// caller holds g_rt_mutex.  Frees retired scratch when nothing can still refer to it.
+void drain_retired() {
+    if (g_retired.empty() || !graphs_quiescent()) return;
+    if (hipDeviceSynchronize() != hipSuccess) return;  // keep them; try again later
+    for (void* p : g_retired) (void)hipFree(p);
+    g_retired.clear();
+}
 }  // namespace
 
-int workspace(size_t nbytes, void** ptr) {
+int stream_buffer(int kind, size_t nbytes, size_t min_bytes, hipStream_t stream, void** ptr, bool* fresh) {
     int dev = 0;
     LQ_HIP(hipGetDevice(&dev));
     LQ_REQUIRE(dev >= 0 && dev < kMaxDevices, LQ_ERR_DEVICE, "device index %d out of range", dev);
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace& w = g_ws[dev];
-    if (w.size < nbytes) {
-        // finish whatever still reads the old block before it goes away
-        LQ_HIP(hipDeviceSynchronize());
-        if (w.ptr) LQ_HIP(hipFree(w.ptr));
-        w.ptr = nullptr;
-        w.size = 0;
-        size_t want = nbytes < (size_t(4) << 20) ? (size_t(4) << 20) : nbytes;
-        LQ_HIP(hipMalloc(&w.ptr, want));
-        w.size = want;
+    std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
+    StreamBuf& b = g_bufs[BufKey{dev, stream, kind}];
+    if (fresh) *fresh = false;
+    if (b.size < nbytes || b.ptr == nullptr) {
+        const size_t want = nbytes < min_bytes ? min_bytes : nbytes;
+        void* p = nullptr;
+        LQ_HIP(hipMalloc(&p, want));  // legal during a relaxed capture; no synchronisation here
+        if (b.ptr) g_retired.push_back(b.ptr);
+        b.ptr = p;
+        b.size = want;
+        if (fresh) *fresh = true;
+        drain_retired();
     }
-    *ptr = w.ptr;
+    *ptr = b.ptr;
     return LQ_OK;
+}
+
+int workspace(size_t nbytes, hipStream_t stream, void** ptr) {
+    return stream_buffer(0, nbytes, size_t(4) << 20, stream, ptr, nullptr);
 }
 
 }  // namespace lq
@@ -98,7 +152,7 @@ int lq_init(int device) {
         return fail(LQ_ERR_GPU_NOT_AVAILABLE, "device %d is %s; this library is built for gfx950 only",
                     device, prop.gcnArchName);
     void* ws = nullptr;
-    return workspace(size_t(4) << 20, &ws);
+    return workspace(size_t(4) << 20, nullptr, &ws);
 }
 
 int lq_device_name(char* buf, size_t buflen) {
@@ -118,22 +172,23 @@ int lq_device_name(char* buf, size_t buflen) {
 // Blocks are recycled in submission order, which is safe for work issued on
 // one stream; a caller that frees memory still in use on ANOTHER stream must
 // synchronise first (as with any pooled allocator).
-// While a graph is being captured (lq_graph_begin .. lq_graph_end) every block
-// allocated belongs to that graph: freeing it is deferred until the graph is
-// destroyed, so replays never write into memory that was handed to someone else.
+// While a thread captures a graph (lq_graph_begin .. lq_graph_end) every block
+// it allocates is pinned to that graph: replays write into it, so it cannot be
+// handed to anyone else before the graph is destroyed.  lq_free on a pinned
+// block only records that its owner is done with it; lq_graph_destroy releases
+// the blocks so marked and unpins the others, whose owners release them later.
 namespace {
+struct Pin {
+    int graph;
+    bool owner_freed;
+};
 struct Pool {
     std::multimap<size_t, void*> free_blocks;           // size -> block
     std::unordered_map<void*, size_t> live;              // block -> size
-    std::unordered_map<void*, int> graph_owner;          // block -> graph id (while pinned)
+    std::unordered_map<void*, Pin> pinned;               // block -> graph that replays into it
     size_t bytes_reserved = 0, bytes_in_use = 0;
 };
 Pool g_pool[kMaxDevices];
-std::mutex g_pool_mutex;
-int g_capturing_graph = 0;  // id of the graph being captured, 0 = none
-int g_next_graph_id = 1;
-std::unordered_map<int, std::vector<std::pair<int, void*>>> g_graph_blocks;  // id -> (dev, block)
-std::unordered_map<int, hipGraphExec_t> g_graph_exec;
 
 size_t round_size(size_t n) {
     if (n < 512) return 512;
@@ -149,7 +204,7 @@ extern "C" int lq_alloc(void** ptr, size_t nbytes) {
     LQ_HIP(hipGetDevice(&dev));
     LQ_REQUIRE(dev >= 0 && dev < kMaxDevices, LQ_ERR_DEVICE, "device index %d out of range", dev);
     const size_t size = round_size(nbytes);
-    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
     Pool& pool = g_pool[dev];
     void* p = nullptr;
     auto it = pool.free_blocks.lower_bound(size);
@@ -174,16 +229,16 @@ extern "C" int lq_alloc(void** ptr, size_t nbytes) {
         pool.bytes_reserved += size;
         pool.bytes_in_use += size;
     }
-    if (g_capturing_graph) {
-        pool.graph_owner[p] = g_capturing_graph;
-        g_graph_blocks[g_capturing_graph].push_back({dev, p});
+    if (t_capturing_graph) {
+        pool.pinned[p] = Pin{t_capturing_graph, false};
+        g_graphs[t_capturing_graph].blocks.push_back({dev, p});
     }
     *ptr = p;
     return LQ_OK;
 }
 
 namespace {
-// caller holds g_pool_mutex
+// caller holds g_rt_mutex
 void release_block(Pool& pool, void* p) {
     auto it = pool.live.find(p);
     if (it == pool.live.end()) return;
@@ -191,15 +246,33 @@ void release_block(Pool& pool, void* p) {
     pool.free_blocks.insert({it->second, p});
     pool.live.erase(it);
 }
+
+// caller holds g_rt_mutex.  The graph no longer replays into its blocks: those whose
+// owner has already freed them go back to the pool, the others are merely unpinned.
+void unpin_graph_blocks(GraphRec& rec) {
+    for (auto& db : rec.blocks) {
+        Pool& pool = g_pool[db.first];
+        auto it = pool.pinned.find(db.second);
+        if (it == pool.pinned.end()) continue;
+        const bool freed = it->second.owner_freed;
+        pool.pinned.erase(it);
+        if (freed) release_block(pool, db.second);
+    }
+    rec.blocks.clear();
+}
 }  // namespace
 
 extern "C" int lq_free(void* ptr) {
     if (!ptr) return LQ_OK;
-    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
     for (int dev = 0; dev < kMaxDevices; ++dev) {
         Pool& pool = g_pool[dev];
         if (!pool.live.count(ptr)) continue;
-        if (pool.graph_owner.count(ptr)) return LQ_OK;  // deferred until lq_graph_destroy
+        auto pin = pool.pinned.find(ptr);
+        if (pin != pool.pinned.end()) {
+            pin->second.owner_freed = true;  // released when its graph is destroyed
+            return LQ_OK;
+        }
         release_block(pool, ptr);
         return LQ_OK;
     }
@@ -208,7 +281,7 @@ extern "C" int lq_free(void* ptr) {
 
 extern "C" int lq_empty_cache(void) {
     LQ_HIP(hipDeviceSynchronize());
-    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
     int dev = 0;
     LQ_HIP(hipGetDevice(&dev));
     Pool& pool = g_pool[dev];
@@ -217,83 +290,99 @@ extern "C" int lq_empty_cache(void) {
         pool.bytes_reserved -= kv.first;
     }
     pool.free_blocks.clear();
+    drain_retired();
     return LQ_OK;
 }
 
 extern "C" int lq_memory_stats(size_t* bytes_in_use, size_t* bytes_reserved) {
     int dev = 0;
     LQ_HIP(hipGetDevice(&dev));
-    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
     if (bytes_in_use) *bytes_in_use = g_pool[dev].bytes_in_use;
     if (bytes_reserved) *bytes_reserved = g_pool[dev].bytes_reserved;
     return LQ_OK;
 }
 
 // ------------------------------------------------------------------ graphs
+// Capture state is per thread (the thread that begins a capture is the one that
+// launches into it), so allocations made meanwhile by other threads are not
+// pinned to the graph.
 extern "C" int lq_graph_begin(lq_stream stream, int* graph_id) {
     LQ_REQUIRE(stream, LQ_ERR_VALUE, "graph capture needs a created stream, not the default stream");
     LQ_REQUIRE(graph_id, LQ_ERR_VALUE, "graph_id is NULL");
+    LQ_REQUIRE(t_capturing_graph == 0, LQ_ERR_VALUE, "this thread is already capturing a graph");
+    int id = 0;
     {
-        std::lock_guard<std::mutex> lock(g_pool_mutex);
-        LQ_REQUIRE(g_capturing_graph == 0, LQ_ERR_VALUE, "a graph capture is already in progress");
-        g_capturing_graph = g_next_graph_id++;
-        *graph_id = g_capturing_graph;
-        g_graph_blocks[*graph_id];
+        std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
+        id = g_next_graph_id++;
+        g_graphs[id];
+        ++g_captures_in_progress;
     }
     hipError_t e = hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed);
     if (e != hipSuccess) {
-        std::lock_guard<std::mutex> lock(g_pool_mutex);
-        g_capturing_graph = 0;
+        std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
+        g_graphs.erase(id);
+        --g_captures_in_progress;
         return hip_fail(e, "hipStreamBeginCapture");
     }
+    t_capturing_graph = id;
+    *graph_id = id;
     return LQ_OK;
 }
 
+// On failure the graph id stays known (with no executable) until lq_graph_destroy,
+// but the blocks allocated during the capture are unpinned at once.
 extern "C" int lq_graph_end(lq_stream stream, int graph_id) {
     hipGraph_t graph = nullptr;
     hipError_t e = hipStreamEndCapture(as_stream(stream), &graph);
-    {
-        std::lock_guard<std::mutex> lock(g_pool_mutex);
-        g_capturing_graph = 0;
-    }
-    if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture");
+    if (t_capturing_graph == graph_id) t_capturing_graph = 0;
     hipGraphExec_t exec = nullptr;
-    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    (void)hipGraphDestroy(graph);
-    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
-    std::lock_guard<std::mutex> lock(g_pool_mutex);
-    g_graph_exec[graph_id] = exec;
+    hipError_t e2 = hipSuccess;
+    if (e == hipSuccess) e2 = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
+    if (g_captures_in_progress > 0) --g_captures_in_progress;
+    auto it = g_graphs.find(graph_id);
+    if (e != hipSuccess || e2 != hipSuccess || it == g_graphs.end()) {
+        if (graph) (void)hipGraphDestroy(graph);
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (it != g_graphs.end()) unpin_graph_blocks(it->second);
+        (void)hipGetLastError();
+        if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture");
+        if (e2 != hipSuccess) return hip_fail(e2, "hipGraphInstantiate");
+        return fail(LQ_ERR_VALUE, "unknown graph id %d", graph_id);
+    }
+    it->second.graph = graph;
+    it->second.exec = exec;
     return LQ_OK;
 }
 
 extern "C" int lq_graph_launch(int graph_id, lq_stream stream) {
     hipGraphExec_t exec = nullptr;
     {
-        std::lock_guard<std::mutex> lock(g_pool_mutex);
-        auto it = g_graph_exec.find(graph_id);
-        LQ_REQUIRE(it != g_graph_exec.end(), LQ_ERR_VALUE, "unknown graph id %d", graph_id);
-        exec = it->second;
+        std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
+        auto it = g_graphs.find(graph_id);
+        LQ_REQUIRE(it != g_graphs.end() && it->second.exec, LQ_ERR_VALUE, "graph id %d has no executable", graph_id);
+        exec = it->second.exec;
     }
     LQ_HIP(hipGraphLaunch(exec, as_stream(stream)));
     return LQ_OK;
 }
 
 extern "C" int lq_graph_destroy(int graph_id) {
-    std::lock_guard<std::mutex> lock(g_pool_mutex);
-    auto it = g_graph_exec.find(graph_id);
-    if (it != g_graph_exec.end()) {
-        LQ_HIP(hipGraphExecDestroy(it->second));
-        g_graph_exec.erase(it);
+    std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
+    auto it = g_graphs.find(graph_id);
+    if (it == g_graphs.end()) return LQ_OK;
+    if (t_capturing_graph == graph_id) {  // destroyed without an end: the capture is abandoned
+        t_capturing_graph = 0;
+        if (g_captures_in_progress > 0) --g_captures_in_progress;
     }
-    auto bt = g_graph_blocks.find(graph_id);
-    if (bt != g_graph_blocks.end()) {
-        for (auto& db : bt->second) {
-            Pool& pool = g_pool[db.first];
-            pool.graph_owner.erase(db.second);
-            release_block(pool, db.second);  // the Python owners are gone or will no-op
-        }
-        g_graph_blocks.erase(bt);
-    }
+    hipError_t e = hipSuccess;
+    if (it->second.exec) e = hipGraphExecDestroy(it->second.exec);
+    if (it->second.graph) (void)hipGraphDestroy(it->second.graph);
+    unpin_graph_blocks(it->second);
+    g_graphs.erase(it);
+    drain_retired();
+    if (e != hipSuccess) return hip_fail(e, "hipGraphExecDestroy");
     return LQ_OK;
 }
 
@@ -334,7 +423,22 @@ int lq_stream_create(lq_stream* stream) {
 }
 
 int lq_stream_destroy(lq_stream stream) {
-    if (stream) LQ_HIP(hipStreamDestroy(as_stream(stream)));
+    if (!stream) return LQ_OK;
+    {
+        // the stream's scratch goes with it (retired: a graph captured on it may still use it)
+        std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
+        for (auto it = g_bufs.begin(); it != g_bufs.end();) {
+            if (it->first.stream == as_stream(stream)) {
+                if (it->second.ptr) g_retired.push_back(it->second.ptr);
+                it = g_bufs.erase(it);
+            } else {
+                ++it;
+            }
+        }
+    }
+    LQ_HIP(hipStreamDestroy(as_stream(stream)));
+    std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
+    drain_retired();
     return LQ_OK;
 }
 

@@ -442,7 +442,7 @@ int launch_wq_mfma(const float* x, const uint32_t* packed, const float* scales, 
     constexpr int STEP = 512 / BITS;
     const int mblocks = (M + 15) / 16;
     void* ws = nullptr;
-    const int rc = workspace(size_t(mblocks) * 16 * K * sizeof(float), &ws);
+    const int rc = workspace(size_t(mblocks) * 16 * K * sizeof(float), st, &ws);
     if (rc) return rc;
     const int per_block = K / STEP * (32 / BITS) * 64;
     hipLaunchKernelGGL((wq_arrange_x_kernel<BITS>), dim3(unsigned((per_block + 255) / 256), unsigned(mblocks)),
@@ -535,7 +535,7 @@ int lq_wq_matmul(const float* x, const uint32_t* packed, const float* scales, co
     }
     // compute-bound shapes: decode once into the workspace, then the float32 MFMA GEMM
     void* ws = nullptr;
-    rc = workspace(size_t(N) * K * sizeof(float), &ws);
+    rc = workspace(size_t(N) * K * sizeof(float), st, &ws);
     if (rc) return rc;
     rc = lq_wq_dequantize(packed, scales, biases, N, K, group_size, bits, static_cast<float*>(ws), stream);
     if (rc) return rc;

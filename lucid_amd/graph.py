@@ -72,7 +72,14 @@ def capture():
             _C.call("lq_graph_end", stream, gid.value)
             g.id = gid.value
         except Exception:
+            # the capture was invalidated (or its body raised and left it unusable): drop the
+            # id so that the blocks allocated during the capture are unpinned
+            _C.load().lq_graph_destroy(gid.value)
+            g.destroy()
             if ok:
                 raise
-        if not ok and g.id is not None:
+        if not ok:
+            # the body raised: whatever was captured is not a usable graph
+            if g.id is None:
+                _C.load().lq_graph_destroy(gid.value)
             g.destroy()

@@ -70,3 +70,107 @@ def test_capture_needs_a_created_stream():
     gid = C.c_int()
     with pytest.raises(ValueError):
         _C.call("lq_graph_begin", None, C.byref(gid))
+
+
+def _stats():
+    used, res = C.c_size_t(), C.c_size_t()
+    _C.call("lq_memory_stats", C.byref(used), C.byref(res))
+    return used.value, res.value
+
+
+def test_scratch_growth_after_capture_keeps_the_graph_valid():
+    """A graph bakes the address of its stream's scratch into its kernel nodes.  A later call
+    on the same stream that needs more scratch must not free that block under the graph."""
+    _C.init()
+    rng = np.random.default_rng(3)
+    n = 1 << 22
+    x = L.tensor(rng.standard_normal(n).astype(np.float32), device="hip")
+    mn = L.Tensor.empty((1,), L.float32, "hip")
+    mx = L.Tensor.empty((1,), L.float32, "hip")
+    stream = C.c_void_p()
+    _C.call("lq_stream_create", C.byref(stream))
+    gid = C.c_int()
+    _C.call("lq_sync", None)
+    _C.call("lq_graph_begin", stream, C.byref(gid))
+    try:
+        # per-tensor min / max of 4 M elements: two stages, partial results in the stream's scratch
+        _C.call("lq_minmax", x.data_ptr, 1, 1, n, mn.data_ptr, mx.data_ptr, stream)
+    finally:
+        _C.call("lq_graph_end", stream, gid.value)
+    # eager work on the same stream that outgrows the 4 MiB scratch: the group-wise matmul with
+    # M > 64 decodes its weight into N * K floats of scratch (16 MiB here)
+    M, N, K = 65, 4096, 1024
+    xs = L.tensor(np.zeros((M, K), np.float32), device="hip")
+    packed = L.tensor(np.zeros((N, K // 4), np.int32), device="hip")
+    sc = L.tensor(np.ones((N, K // 64), np.float32), device="hip")
+    bi = L.tensor(np.zeros((N, K // 64), np.float32), device="hip")
+    out = L.Tensor.empty((M, N), L.float32, "hip")
+    _C.call("lq_wq_matmul", xs.data_ptr, packed.data_ptr, sc.data_ptr, bi.data_ptr, M, N, K, 64, 8,
+            out.data_ptr, stream)
+    _C.call("lq_sync", stream)
+    for rep in range(3):
+        data = rng.standard_normal(n).astype(np.float32) * (rep + 1)
+        x.copy_from(data)
+        _C.call("lq_graph_launch", gid.value, stream)
+        _C.call("lq_sync", stream)
+        assert mn.numpy()[0] == data.min() and mx.numpy()[0] == data.max(), rep
+        # and once more with eager scratch use on the stream between the replays
+        _C.call("lq_wq_matmul", xs.data_ptr, packed.data_ptr, sc.data_ptr, bi.data_ptr, M, N, K, 64, 8,
+                out.data_ptr, stream)
+    _C.call("lq_graph_destroy", gid.value)
+    _C.call("lq_stream_destroy", stream)
+
+
+def test_tensor_that_outlives_its_graph_keeps_its_memory():
+    """Blocks allocated during capture go back to the pool at destroy only if their owner has
+    freed them; a result tensor still alive keeps its block to itself."""
+    import gc
+    _C.init()
+    gc.collect()
+    _C.call("lq_empty_cache")  # so that the only cached block after destroy is the one released by it
+    x = L.tensor(np.arange(4096, dtype=np.float32), device="hip")
+    with L.graph.capture() as g:
+        y = L.Tensor.empty((4096,), L.float32, "hip")
+        _C.call("lq_relu_f32", x.data_ptr, y.data_ptr, 4096, None)
+        tmp = L.Tensor.empty((4096,), L.float32, "hip")  # dies before the graph does
+        _C.call("lq_relu_f32", x.data_ptr, tmp.data_ptr, 4096, None)
+        tmp_ptr = tmp.data_ptr
+        del tmp
+    g.replay()
+    L.synchronize()
+    g.destroy()
+    fresh = [L.Tensor.empty((4096,), L.float32, "hip") for _ in range(8)]
+    ptrs = [t.data_ptr for t in fresh]
+    assert y.data_ptr not in ptrs            # still owned by y
+    assert tmp_ptr in ptrs                   # its owner was gone: released with the graph
+    for t in fresh:
+        t.copy_from(np.full(4096, -1.0, np.float32))
+    L.synchronize()
+    assert np.array_equal(y.numpy(), np.arange(4096, dtype=np.float32))
+    used_before = _stats()[0]
+    del y
+    assert _stats()[0] < used_before         # y's own free released the block
+
+
+def test_failed_capture_releases_its_blocks():
+    import gc
+    _C.init()
+    gc.collect()
+    x = L.tensor(np.ones(1 << 16, np.float32), device="hip")
+    used0 = _stats()[0]
+    with pytest.raises(RuntimeError, match="boom"):
+        with L.graph.capture():
+            t = L.Tensor.empty((1 << 16,), L.float32, "hip")
+            _C.call("lq_relu_f32", x.data_ptr, t.data_ptr, 1 << 16, None)
+            raise RuntimeError("boom")
+    del t
+    gc.collect()
+    assert _stats()[0] == used0
+    # and the library still captures and replays afterwards
+    with L.graph.capture() as g:
+        y = L.Tensor.empty((1 << 16,), L.float32, "hip")
+        _C.call("lq_relu_f32", x.data_ptr, y.data_ptr, 1 << 16, None)
+    g.replay()
+    L.synchronize()
+    assert np.all(y.numpy() == 1.0)
+    g.destroy()
