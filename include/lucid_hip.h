@@ -214,6 +214,23 @@ int lq_copy_kernel(void* dst, const void* src, size_t nbytes, lq_stream stream);
 int lq_minmax(const float* x, size_t outer, size_t C, size_t inner, float* mn, float* mx,
               lq_stream stream);
 
+/* lq_minmax for callers that cannot allocate (code under HIP graph capture, serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in Lucid.  Same
+ * arguments, same results bit for bit; the partial results of the two-stage
+ * reduction live in a 1 MiB array that is part of the library's device image
+ * (one copy per GPU, held until the process ends), and the call makes no
+ * hipMalloc / hipFree.  Limit: a reduction over short runs (inner < 64, C > 1)
+ * needs 8 * C * inner bytes of partials and is refused with LQ_ERR_SHAPE beyond
+ * 1 MiB (C * inner > 131072); every other shape fits (fewer slices per channel
+ * are used when the usual number would not).  Nothing in the array has to be
+ * cleared between calls: every partial that is read has been written by the same
+ * call.  All calls on one GPU share the array, so calls that overlap on one GPU
+ * (different streams, or one stream and a graph replay on another) race.
+ * lq_init resolves the array's address for its device; without it the first call
+ * on a device does. */
+int lq_minmax_noalloc(const float* x, size_t outer, size_t C, size_t inner, float* mn, float* mx,
+                      lq_stream stream);
+
 /* calculate_qparams (lucid/quantization/_qparams.py:190-215) over C channels,
  * entirely on the device.  scale, zp: device f32[C]. */
 int lq_calc_qparams(const float* mn, const float* mx, size_t C, int symmetric, int qmin, int qmax,

@@ -111,6 +111,7 @@ _SIGNATURES = {
     "lq_probe_mfma_i8": [_vp, _vp, _sz, _i, _vp, C.POINTER(C.c_double), _vp],
     "lq_copy_kernel": [_vp, _vp, _sz, _vp],
     "lq_minmax": [_vp, _sz, _sz, _sz, _vp, _vp, _vp],
+    "lq_minmax_noalloc": [_vp, _sz, _sz, _sz, _vp, _vp, _vp],
     "lq_calc_qparams": [_vp, _vp, _sz, _i, _i, _i, _i, _f, _vp, _vp, _vp],
     "lq_quantize": [_vp, _vp, _i, _i, _sz, _sz, _sz, _vp, _vp, _i, _i, _i, _vp],
     "lq_dequantize": [_vp, _i, _i, _vp, _sz, _sz, _sz, _vp, _vp, _i, _vp],

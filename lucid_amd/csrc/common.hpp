@@ -44,6 +44,9 @@ int hip_fail(hipError_t e, const char* what);
 int stream_buffer(int kind, size_t nbytes, size_t min_bytes, hipStream_t stream, void** ptr, bool* fresh);
 // kind 0: the general workspace (at least 4 MiB)
 int workspace(size_t nbytes, hipStream_t stream, void** ptr);
+// Resolves, for the current device, the address of the static scratch array that
+// lq_minmax_noalloc uses (called by lq_init; the entry point does it on first use otherwise).
+int minmax_noalloc_init();
 
 inline hipStream_t as_stream(lq_stream s) { return reinterpret_cast<hipStream_t>(s); }
 

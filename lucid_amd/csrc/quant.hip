@@ -4,6 +4,7 @@
 // do the arithmetic in the order Lucid's CPU path does it
 // (lucid/quantization/_functional.py:180, 281, 311-313): IEEE division,
 // round-half-even, add zero point, clamp, cast.  No reciprocal, no FMA.
+#include <mutex>
 #include "common.hpp"
 #include "range_slots.hpp"
 
@@ -652,7 +653,32 @@ __global__ __launch_bounds__(1024) void quantize_tensor_dynamic_kernel(
 }
 
 
-// min / max launch sequence.  `get_ws(nbytes, &ptr)`
+// ---------------------------------------------------------------- static scratch (no-allocation entry point)
+// lq_minmax_noalloc keeps the partial results of its two-stage reduction here instead of in
+// the library's growable workspace, so that the call allocates nothing.  Each GPU holds its
+// own copy of the array at its own address; the name below is only the host-side handle of
+// the symbol, the device address comes from hipGetSymbolAddress, once per device.
+constexpr size_t kNoAllocScratchBytes = size_t(1) << 20;
+__device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+void* g_scratch_ptr[16] = {nullptr};
+std::mutex g_scratch_mutex;
+
+int noalloc_scratch_ptr(void** out) {
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    LQ_REQUIRE(dev >= 0 && dev < 16, LQ_ERR_DEVICE, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        LQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        LQ_REQUIRE(p != nullptr, LQ_ERR_INTERNAL, "hipGetSymbolAddress returned a null address for the static scratch");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return LQ_OK;
+}
+
+// min / max launch sequence shared by lq_minmax and lq_minmax_noalloc.  `get_ws(nbytes, &ptr)`
 // supplies the memory for the partial results of a two-stage reduction; `ws_limit` is the
 // most it can supply: the number of slices per channel is cut down to fit (the result does
 // not depend on it: min and max are exact in any order).
@@ -734,6 +760,13 @@ int minmax_launch(const float* x, size_t outer, size_t C, size_t inner, float* m
 
 }  // namespace
 
+namespace lq {
+int minmax_noalloc_init() {
+    void* p = nullptr;
+    return noalloc_scratch_ptr(&p);
+}
+}  // namespace lq
+
 extern "C" {
 
 int lq_quantize_tensor_dynamic_i8(const float* x, size_t n, int symmetric, int qmin, int qmax, int is_signed,
@@ -787,6 +820,22 @@ int lq_minmax(const float* x, size_t outer, size_t C, size_t inner, float* mn, f
     hipStream_t st = as_stream(stream);
     return minmax_launch(x, outer, C, inner, mn, mx, st, ~size_t(0),
                          [st](size_t nbytes, void** ws) { return workspace(nbytes, st, ws); });
+}
+
+int lq_minmax_noalloc(const float* x, size_t outer, size_t C, size_t inner, float* mn, float* mx,
+                      lq_stream stream) {
+    void* scratch = nullptr;
+    int rc = noalloc_scratch_ptr(&scratch);
+    if (rc) return rc;
+    return minmax_launch(x, outer, C, inner, mn, mx, as_stream(stream), kNoAllocScratchBytes,
+                         [scratch](size_t nbytes, void** ws) {
+                             // minmax_launch sizes its partials to the limit it was given
+                             LQ_REQUIRE(nbytes <= kNoAllocScratchBytes, LQ_ERR_SHAPE,
+                                        "minmax_noalloc: %zu bytes of partials exceed the %zu-byte static scratch",
+                                        nbytes, kNoAllocScratchBytes);
+                             *ws = scratch;
+                             return int(LQ_OK);
+                         });
 }
 
 int lq_calc_qparams(const float* mn, const float* mx, size_t C, int symmetric, int qmin, int qmax,

@@ -152,7 +152,9 @@ int lq_init(int device) {
         return fail(LQ_ERR_GPU_NOT_AVAILABLE, "device %d is %s; this library is built for gfx950 only",
                     device, prop.gcnArchName);
     void* ws = nullptr;
-    return workspace(size_t(4) << 20, nullptr, &ws);
+    int rc = workspace(size_t(4) << 20, nullptr, &ws);
+    if (rc) return rc;
+    return minmax_noalloc_init();  // resolves the static scratch of lq_minmax_noalloc on this device
 }
 
 int lq_device_name(char* buf, size_t buflen) {
