@@ -529,7 +529,9 @@ typedef struct {
     void* out;             /* [M, ldo] in the type out_mode implies          */
     long ldo;              /* output row stride in elements; 0 means N       */
     int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
-    int tile_config;       /* tuning: low byte 0 = choose, 1..12 = a tile shape;
+    int tile_config;       /* tuning: low byte 0 = choose, 1..12 = a tile shape of the
+                              four-wavefront kernel, 13 / 14 = 256x352 / 256x256 tiles of
+                              the eight-wavefront kernel (plain GEMM, K % 64 == 0);
                               next byte 0 = choose, 1 = one block per tile,
                               2 = stream-K work split, 3 = stream-K over the
                               leftover tiles of the last round only; bits 16..30

@@ -63,6 +63,7 @@ int launch_tile_c9(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c10(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c11(const GemmArgs&, bool, int, int, hipStream_t);
 int launch_tile_c12(const GemmArgs&, bool, int, int, hipStream_t);
+int launch_pp_shape(const GemmArgs&, int, hipStream_t);
 }  // namespace lq
 
 namespace {
@@ -81,6 +82,12 @@ int launch_tile_shape(const GemmArgs& g, bool conv, int groups, int cfg, int sch
     case 10: return launch_tile_c10(g, conv, groups, schedule, st);
     case 11: return launch_tile_c11(g, conv, groups, schedule, st);
     case 12: return launch_tile_c12(g, conv, groups, schedule, st);
+    case 13:
+    case 14:
+        // the eight-wavefront ping-pong kernel: plain GEMMs, one block per tile
+        LQ_REQUIRE(!conv && groups == 1, LQ_ERR_VALUE, "tile_config %d is for plain GEMMs", cfg);
+        LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
+        return launch_pp_shape(g, cfg - 13, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -187,13 +194,17 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
     if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9 || in_place) return LQ_OK;
 
     // candidates are whole tile_config values (shape | schedule << 8)
-    int cands[16], n = 0;
+    int cands[20], n = 0;
     if (g.N <= 64) cands[n++] = 6;
     cands[n++] = 5;
     if (g.K <= 256) cands[n++] = 8;  // one to four k-iterations: latency-bound tiles, four blocks per CU
     if (g.N > 64) cands[n++] = 3, cands[n++] = 4;
     if (g.N > 128 && g.M > 128) cands[n++] = 1, cands[n++] = 11;
     if (g.N > 128 && !conv) cands[n++] = 12;
+    // large plain GEMMs: the ping-pong kernel's 256 x 352 and 256 x 256 tiles
+    if (!conv && groups == 1 && g.K % 64 == 0 && g.M >= 256 && g.N >= 256 && !g.gelu && g.range == nullptr &&
+        size_t(g.M) * g.K < 0xffffffffull && size_t(g.N) * g.K < 0xffffffffull)
+        cands[n++] = 13, cands[n++] = 14;
     // a long K over few tiles (late convolution stages): split K between the idle CUs
     const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
     if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);

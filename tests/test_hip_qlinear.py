@@ -446,3 +446,79 @@ def test_fused_join_grid_variants(z1, z2, off2, Zj, qmin, qmax, offj, relu):
                         np.float32(Zj), qmin, qmax, offj)
     assert np.array_equal(fused, exp.reshape(M, N))
     assert len(np.unique(fused)) > 20
+
+
+PP_SHAPES = [(256, 256, 128), (300, 260, 192), (513, 1000, 576), (2048, 512, 4096), (1, 16, 64), (700, 130, 64),
+             (257, 353, 320), (2048, 1004, 256), (40, 1001, 128)]
+
+
+@pytest.mark.parametrize("cfg", [13, 14])
+@pytest.mark.parametrize("M,N,K", PP_SHAPES)
+def test_ping_pong_kernel_exact(cfg, M, N, K):
+    """The eight-wavefront kernel (tile_config 13 / 14): accumulators and the float16 epilogue
+    against the oracle on full, ragged and tiny shapes (edge tiles, rows read past the end of a
+    matrix, widths that rule out the vector and the paired stores)."""
+    rng = np.random.default_rng(cfg * 1000 + M + N + K)
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    ad, wd = hip(a), hip(w)
+    acc = _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, path=TILE, tile_config=cfg).numpy()
+    assert np.array_equal(acc, O.igemm(a, w))
+    a_scale = rng.uniform(0.005, 0.05, M).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    got = _ops.qlinear_i8(ad, wd, a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias),
+                          out_mode=_ops.OUT_F16, path=TILE, tile_config=cfg).numpy()
+    exp = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, out_mode=O.OUT_F16)
+    assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+
+
+@pytest.mark.parametrize("cfg", [13, 14])
+@pytest.mark.parametrize("M,N,K", [(512, 704, 256), (300, 260, 128), (129, 1001, 64)])
+def test_ping_pong_kernel_every_output_form(cfg, M, N, K):
+    """Every epilogue form of the eight-wavefront kernel equals the oracle: an activation zero
+    point with the row-sum correction, per-tensor and per-row activation scales, ReLU, float32
+    with a residual, requantized codes (both storage forms), fake-quantized float32, and the
+    fused join on codes."""
+    rng = np.random.default_rng(cfg * 77 + M + N + K)
+    a, w = codes(rng, (M, K), -100, 100), codes(rng, (N, K), -100, 100)
+    ad, wd = hip(a), hip(w)
+    wsum = _ops.rowsum_i8(wd)
+    a_zp = 7
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.3).astype(np.float32)
+    one = lambda v: hip(np.float32(v))
+    for per_row in (False, True):
+        a_scale = rng.uniform(0.005, 0.05, M if per_row else 1).astype(np.float32)
+        common = dict(a_zp=a_zp, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=wsum, bias=hip(bias), path=TILE,
+                      tile_config=cfg)
+        ocommon = dict(bias=bias)
+        res = rng.standard_normal((M, N)).astype(np.float32)
+        for relu in (False, True):
+            y = _ops.qlinear_i8(ad, wd, **common, relu=relu, out_mode=_ops.OUT_F32, residual=hip(res)).numpy()
+            exp = O.qlinear(a, w, a_zp, a_scale, w_scale, relu=relu, out_mode=O.OUT_F32, **ocommon) + res
+            assert np.array_equal(y.view(np.uint32), exp.astype(np.float32).view(np.uint32))
+            yf = O.qlinear(a, w, a_zp, a_scale, w_scale, relu=relu, out_mode=O.OUT_F32, **ocommon)
+            S = np.float32(np.abs(yf).max() / 100 + 1e-6)
+            for (Z, qmin, qmax, off) in ((np.float32(128.0 if not relu else 3.0), 0, 255, -128),
+                                         (np.float32(-7.0), -128, 127, 0)):
+                kw = dict(out_scale=one(S), out_zp=one(Z), out_qmin=qmin, out_qmax=qmax, out_offset=off)
+                okw = dict(out_scale=S, out_zp=Z, out_qmin=qmin, out_qmax=qmax, out_offset=off)
+                q = _ops.qlinear_i8(ad, wd, **common, relu=relu, out_mode=_ops.OUT_REQUANT_I8, **kw).numpy()
+                assert np.array_equal(q, O.qlinear(a, w, a_zp, a_scale, w_scale, relu=relu,
+                                                   out_mode=O.OUT_REQUANT_I8, **ocommon, **okw))
+                fq = _ops.qlinear_i8(ad, wd, **common, relu=relu, out_mode=_ops.OUT_FAKEQUANT_F32, **kw).numpy()
+                efq = O.qlinear(a, w, a_zp, a_scale, w_scale, relu=relu, out_mode=O.OUT_FAKEQUANT_F32, **ocommon, **okw)
+                assert np.array_equal(fq.view(np.uint32), efq.view(np.uint32))
+        # the fused join against the two-step form of the oracle
+        s1, z1, s2, z2, Sj, Zj = (np.float32(v) for v in (S, 3.0, 0.027, 131.0, S * 1.3, 64.0))
+        other = rng.integers(0, 256, (M, N)).astype(np.int64)
+        stored = (other - 128).astype(np.int8)
+        fused = _ops.qlinear_i8(ad, wd, **common, out_mode=_ops.OUT_REQUANT_I8, out_scale=one(s1), out_zp=one(z1),
+                                out_qmin=-128, out_qmax=127, out_offset=0,
+                                join=dict(q=hip(stored), offset=-128, scale=one(s2), zp=one(z2), relu=True,
+                                          out_scale=one(Sj), out_zp=one(Zj), out_qmin=0, out_qmax=255,
+                                          out_offset=-128)).numpy()
+        first = O.qlinear(a, w, a_zp, a_scale, w_scale, out_mode=O.OUT_REQUANT_I8, out_scale=s1, out_zp=z1,
+                          out_qmin=-128, out_qmax=127, out_offset=0, **ocommon)
+        expj = O.add_requant(first, 0, s1, z1, stored, -128, s2, z2, True, Sj, Zj, 0, 255, -128)
+        assert np.array_equal(fused, expj.reshape(M, N))
