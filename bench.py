@@ -44,12 +44,19 @@ PEAK_HBM_GBS = 8000.0     # MI355X published HBM3E bandwidth, GB/s
 # the library's plain 1 GiB copy kernel: fetch x2.000, write x1.000).  The runs
 # are summarised in profiles/hbm_traffic_qlinear_and_quantize.md.
 MEASURED_TRAFFIC_BYTES = {
-    # one 128x256-tiled launch / the column split (256x256 tiles over 8192 columns + 128x256 over 2816)
-    "linear_m2048": int((2.0 * 96504 + 44032) * 1024),
-    "linear_m2048_split": int((2.0 * (49357.0 + 30884.2) + 32768 + 11264) * 1024),
     "quantize_per_channel_i8": int((2.0 * 524577 + 262144) * 1024),
     "dequantize_per_channel_i8": int((2.0 * 131350 + 1048712) * 1024),
     "minmax_per_channel": int((2.0 * 524317 + 257) * 1024),
+}
+
+
+# The headline Linear's HBM traffic depends on the tile shape, so each figure is kept with the
+# tile_config (lq_last_tile_config) it was measured under and is reported only when the run
+# resolves to that same configuration (null otherwise: a stale figure would mislead).
+LINEAR_TRAFFIC_BY_TILE_CONFIG = {
+    0x10d: int((2.0 * 55349.4 + 60688.6) * 1024),                       # one launch of 256x352 tiles, eight wavefronts
+    0x104: int((2.0 * 96504 + 44032) * 1024),                           # one launch of 128x256 tiles
+    0x20010b: int((2.0 * (49357.0 + 30884.2) + 32768 + 11264) * 1024),  # 256x256 over 8192 columns + 128x256 over 2816
 }
 
 
@@ -116,6 +123,13 @@ def bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup, seed=1):
         _ops.qlinear_i8(t["xq"], t["wq"], a_scale=t["xs"], w_scale=t["ws"], bias=t["bias"],
                         out_mode=_ops.OUT_F16, out=t["out"], repeat=repeat)
 
+    # Let the clock settle first: after idling (the uploads and quantization above are light
+    # work) the part takes tens of milliseconds of load to reach the state it then holds, and
+    # a dozen 80 us warm-up launches end before that.  Untimed, like the warm-up steps.
+    step()
+    settle = 500
+    step(settle)
+    _C.call("lq_sync", None)
     # per-launch event pairs give the spread; the average launch duration comes
     # from `steps` launches issued back to back from native code between one
     # pair of events, so that no host-side gap is charged to the kernel
@@ -632,6 +646,9 @@ def main() -> int:
                     help="run just this end-to-end leg and print its figures")
     ap.add_argument("--vendor-child", default=None, help=argparse.SUPPRESS)
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also run the plain 1 GiB copy kernel a few times: the known-size dispatch that "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled by")
     ap.add_argument("--eager", action="store_true",
                     help="time Python-driven launches instead of HIP graph replays (for runs under a tracer)")
     ap.add_argument("--cpu-sample-rows", type=int, default=2048)
@@ -700,8 +717,8 @@ def main() -> int:
             "peak": PEAK_INT8_TOPS,
             "unit": "TOP/s",
             "frac": round(r["kernel_tops"] / PEAK_INT8_TOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES["linear_m2048_split" if r["split"] else "linear_m2048"],
-            "kernel": "qgemm_tile_kernel",
+            "traffic": LINEAR_TRAFFIC_BY_TILE_CONFIG.get(r["tile_config"]),
+            "kernel": "qgemm_pp_kernel" if (r["tile_config"] & 0xff) in (13, 14) else "qgemm_tile_kernel",
             "avg_kernel_us": round(r["avg_kernel_ms"] * 1e3, 2),
             "median_kernel_us": round(r["median_ms"] * 1e3, 2),
             "p95_kernel_us": round(r["p95_ms"] * 1e3, 2),
@@ -720,6 +737,14 @@ def main() -> int:
             "algorithmic_ops": sp["ops"], "avg_kernel_us": round(sp["avg_ms"] * 1e3, 2),
             "achieved": round(sp["ops"] / sp["avg_ms"] / 1e9, 2),
             "frac": round(sp["ops"] / sp["avg_ms"] / 1e9 / PEAK_INT8_TOPS, 4)}
+    if args.traffic_calibration:
+        n = 1 << 28
+        src, dst = L.Tensor.empty((n,), L.float32, "hip"), L.Tensor.empty((n,), L.float32, "hip")
+        _C.call("lq_fill_bytes", src.data_ptr, 1, 4 * n, None)
+        for _ in range(4):
+            _C.call("lq_copy_kernel", dst.data_ptr, src.data_ptr, 4 * n, None)
+        _C.call("lq_sync", None)
+        del src, dst
     # the same operand codes through a loop of MFMAs alone: the data-dependent ceiling
     ceiling = probe_mfma_ceiling(L, _C, r["tensors"]["xq"], r["tensors"]["wq"])
     line["roofline"]["mfma_only_same_operands_tops"] = round(ceiling, 1)

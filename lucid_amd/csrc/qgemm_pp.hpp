@@ -135,9 +135,12 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     const int nk = g.K / BK;
 
     // ---- global -> LDS: chunk c of an operand is its rows 16c .. 16c+15; lane l fills the slot
-    // of row 16c + l/4, physical 16-byte chunk l%4, with the logical chunk (l%4) ^ ((l/16)%4)
+    // of row 16c + l/4, physical 16-byte chunk l%4, with the logical chunk (l%4) ^ ((row/2)%4).
+    // (Measured: with this swizzle the fragment reads below - 16 rows x 4 chunks per instruction -
+    // run at the rate of a contiguous ds_read_b128; with (row/4)%4, which suits fragments of 32
+    // rows x 2 chunks, they take 40 % longer.)
     const int ld_row = lane >> 2;
-    const int ld_kc = (lane & 3) ^ ((lane >> 4) & 3);
+    const int ld_kc = (lane & 3) ^ ((lane >> 3) & 3);
     // The operands are read through buffer descriptors: one 32-bit offset register per lane, the
     // k position in a scalar offset, and rows past the end of a matrix (the last tile in m or n)
     // read as zeros instead of needing a clamp.
@@ -189,8 +192,8 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     };
 
     // ---- LDS -> registers: lane l of a 16 x 64 fragment holds row l%16, logical chunk l/16,
-    // which sits at physical chunk (l/16) ^ ((l/4)%4)
-    const int fr_off = (lane & 15) * BK + (((lane >> 4) ^ ((lane >> 2) & 3)) * 16);
+    // which sits at physical chunk (l/16) ^ ((row/2)%4)
+    const int fr_off = (lane & 15) * BK + (((lane >> 4) ^ ((lane >> 1) & 3)) * 16);
     const int a_frag0 = wm * (TM * 16) * BK + fr_off;
     const int b_frag0 = BM * BK + wn * (TN * 16) * BK + fr_off;
     pp_v4i af[TM], bf[TN];
@@ -234,22 +237,21 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
         }
         __builtin_amdgcn_s_setprio(0);
     };
-
-    // ---- prologue: STAGES-1 stages in flight; stage 0 complete before phase 0
-    // issue order per wavefront: A(0,1), B(0), B(1,2); then step u adds A(u+2,u+3) when u is
-    // even and B(u+2,u+3) when u is odd
-    pair_load_all(0, std::false_type{});
-    pp_static_for<LB>([&](auto c) { stage_load(0, std::integral_constant<int, LA + decltype(c)::value>{}); });
-    pair_load_all(1, std::true_type{});
-    // column parameters of the tile into LDS (the barriers of the main loop publish them)
+    // ---- prologue: the tile's column parameters are requested first (they go to LDS, where the
+    // barriers of the main loop publish them), then the first stages.  Issue order per
+    // wavefront: A(0,1), B(0), B(1,2); then step u adds A(u+2,u+3) when u is even and B(u+2,u+3)
+    // when u is odd.
     float* s_ws = reinterpret_cast<float*>(smem + Cfg::PARAM_OFF);
     float* s_bias = s_ws + BN;
     int32_t* s_corr = reinterpret_cast<int32_t*>(s_bias + BN);
-    if (tid < BN) {
-        const int n = n0 + tid;
-        const ColParams c = load_col(g, n < g.N ? n : g.N - 1);
-        s_ws[tid] = c.ws, s_bias[tid] = c.bias, s_corr[tid] = c.corr;
-    }
+    ColParams c_mine{1.0f, -0.0f, 0};
+    if (tid < BN) c_mine = load_col(g, n0 + tid < g.N ? n0 + tid : g.N - 1);
+    __builtin_amdgcn_sched_barrier(0);
+    pair_load_all(0, std::false_type{});
+    pp_static_for<LB>([&](auto c) { stage_load(0, std::integral_constant<int, LA + decltype(c)::value>{}); });
+    pair_load_all(1, std::true_type{});
+    __builtin_amdgcn_sched_barrier(0);
+    if (tid < BN) s_ws[tid] = c_mine.ws, s_bias[tid] = c_mine.bias, s_corr[tid] = c_mine.corr;
     __builtin_amdgcn_s_waitcnt(pp_vmcnt_imm(2 * LB));  // stage 0 has landed: only B(1,2) may be outstanding
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -266,8 +268,8 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     };
     // One k step of a wavefront.  Step u refills operand OP = u % 2 for stages u+2, u+3 (their
     // buffers held stages u-2 and u-1, whose last readers finished in phase 2u-1).  Group 0 issues
-    // the loads between the MFMAs of its phase 2u+1; group 1 at the start of its read phase, which
-    // is the same phase 2u+1.  Either way, when the wavefront then waits for its loads of stage
+    // the loads between the MFMAs of its phase 2u+1; group 1 behind the fragment reads of its read
+    // phase, which is the same phase 2u+1.  Either way, when the wavefront then waits for its loads of stage
     // u+1, what it issued later is one load of the pair's second stage plus this step's pair.
     auto step_g0 = [&](int u, auto op_tag) {
         constexpr int kAllowed = 1 + 2 * (decltype(op_tag)::value ? LB : LA);
@@ -284,8 +286,8 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     };
     auto step_g1 = [&](int u, auto op_tag) {
         constexpr int kAllowed = 1 + 2 * (decltype(op_tag)::value ? LB : LA);
-        pair_load_all(u + 2, op_tag);
         read_frags(u);
+        pair_load_all(u + 2, op_tag);
         if (u == nk - 1) fetch_params();
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(pp_vmcnt_imm(kAllowed));
@@ -313,11 +315,10 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
         }
         if (u < nk) step_g1(u, std::false_type{});
     }
-    // Both groups have passed the same number of barriers.  Group 0 arrives here one phase
-    // before group 1, whose last phase reads no LDS: the stage buffers are free for staging.
+    // Both groups have passed the same number of barriers.
     // ---- epilogue.  acc[i][j][r] is row wm0 + 16 i + lane % 16, column wn0 + 16 j + 4 (lane / 16) + r:
-    // four consecutive columns per lane and tile.  No LDS, no barrier: group 0 runs it while
-    // group 1 still issues its last MFMAs.
+    // four consecutive columns per lane and tile.  No staging through LDS and no barrier: group 0
+    // runs it while group 1 still issues its last MFMAs.
     __builtin_amdgcn_s_waitcnt(pp_vmcnt_imm(0));  // no direct load may land in LDS after this wavefront has ended
     if (wm0 >= g.M || wn0 >= g.N) return;
     float S = 1.0f, Z = 0.0f;
