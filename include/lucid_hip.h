@@ -44,7 +44,7 @@
 extern "C" {
 #endif
 
-#define LQ_VERSION 2
+#define LQ_VERSION 3
 
 typedef enum {
     LQ_OK = 0,
@@ -552,6 +552,16 @@ typedef struct {
                               receives the min / max of the stored output, for
                               lq_calc_qparams_from_range of the next dynamic
                               quantizer; mode F32, tile kernel only             */
+    const int32_t* w_zp;   /* optional [N] zero points of the weight rows, as stored
+                              codes (device): per-channel affine weights
+                              (lucid/quantization/_qscheme.py per_channel_affine, kept by
+                              from_float, lucid/nn/quantized/linear.py:217-236).  The
+                              effective accumulator is then
+                                sum_k (a[m,k] - a_zp) * (w[n,k] - w_zp[n])
+                                = acc - a_zp*wsum[n] - w_zp[n]*sum_k a[m,k] + K*a_zp*w_zp[n],
+                              exact in int32 (K <= 33025); the row sums of a are taken by
+                              the call, wsum is required.  NULL = symmetric weights;
+                              ignored in mode ACC_I32; not with range.            */
 } lq_qlinear_args;
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);
@@ -605,6 +615,11 @@ typedef struct {
     lq_join_args join;     /* optional join on codes (NHWC, ld = Cout): the residual
                               add of a bottleneck block fused into its last
                               convolution; mode REQUANT_I8 only                  */
+    const int32_t* w_zp;   /* optional [Cout] zero points of the filters' stored codes
+                              (device), as lq_qlinear_args.w_zp; the window sums of the
+                              image come from a convolution with an all-ones filter, so
+                              taps in the padding count as a_zp and cancel exactly.
+                              NULL = symmetric; ignored in mode ACC_I32            */
 } lq_qconv2d_args;
 
 int lq_qconv2d_i8(const lq_qconv2d_args* args, lq_stream stream);

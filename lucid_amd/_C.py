@@ -140,6 +140,7 @@ class QLinearArgs(C.Structure):
         ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
         ("out", _vp), ("ldo", C.c_long), ("force_path", _i), ("tile_config", _i),
         ("residual", _vp), ("ldr", C.c_long), ("join", JoinArgs), ("gelu", _i), ("range", _vp),
+        ("w_zp", _vp),
     ]
 
 
@@ -190,6 +191,7 @@ class QConv2dArgs(C.Structure):
         ("out_scale", _vp), ("out_zp", _vp),
         ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
         ("out", _vp), ("force_path", _i), ("tile_config", _i), ("join", JoinArgs),
+        ("w_zp", _vp),
     ]
 
 
@@ -208,7 +210,7 @@ _lib = None
 _initialised_device = None
 
 
-ABI_VERSION = 2  # LQ_VERSION of include/lucid_hip.h this binding was written against
+ABI_VERSION = 3  # LQ_VERSION of include/lucid_hip.h this binding was written against
 
 
 def load() -> C.CDLL:

@@ -45,9 +45,10 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
                out_qmax: int = 255, out_offset: int = 0, path: int = PATH_AUTO,
                tile_config: int = 0, out: Tensor | None = None, repeat: int = 1,
                residual: Tensor | None = None, join=None, gelu: bool = False,
-               range_buf: Tensor | None = None) -> Tensor:
+               range_buf: Tensor | None = None, w_zp: Tensor | None = None) -> Tensor:
     """Fused int8 GEMM + epilogue; see ``lq_qlinear_i8`` in ``lucid_hip.h``.
     ``a`` is int8 ``[M, K]``, ``w`` int8 ``[N, K]``; the result is ``[M, N]``.
+    ``w_zp`` (int32 ``[N]``) holds the zero points of affine weight rows.
     ``residual`` (float32, ``M*N`` elements) is added after the activation;
     ``join`` fuses a residual add on codes after the requantize (see ``_fill_join``)."""
     if a.ndim != 2 or w.ndim != 2 or a.shape[1] != w.shape[1]:
@@ -84,6 +85,9 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
     args.residual, args.ldr = _ptr(residual, "residual", T.float32), 0
     _fill_join(args.join, join, (M, N))
     args.gelu, args.range = int(gelu), _ptr(range_buf, "range", T.float32)
+    if w_zp is not None and w_zp.numel != N:
+        raise _C.ShapeMismatch(f"w_zp has {w_zp.numel} entries for N = {N}")
+    args.w_zp = _ptr(w_zp, "w_zp", T.int32)
     if repeat == 1:
         _C.call("lq_qlinear_i8", C.byref(args), None)
     else:
@@ -121,9 +125,10 @@ def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None
                groups: int = 1, relu: bool = False, out_mode: int = OUT_F32,
                out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
                out_qmax: int = 255, out_offset: int = 0, path: int = CONV_AUTO,
-               tile_config: int = 0, join=None) -> Tensor:
+               tile_config: int = 0, join=None, w_zp: Tensor | None = None) -> Tensor:
     """Fused int8 convolution; see ``lq_qconv2d_i8``.  ``x`` int8 NHWC, ``w``
-    int8 ``[Cout, KH, KW, Cin/groups]``, ``pad`` = (h_lo, h_hi, w_lo, w_hi).
+    int8 ``[Cout, KH, KW, Cin/groups]``, ``pad`` = (h_lo, h_hi, w_lo, w_hi);
+    ``w_zp`` (int32 ``[Cout]``) holds the zero points of affine filters.
     Returns NHWC ``[B, OH, OW, Cout]``."""
     if x.ndim != 4 or w.ndim != 4:
         raise _C.ShapeMismatch(f"qconv2d_i8: expected 4-d x and w, got {x.shape} and {w.shape}")
@@ -149,5 +154,8 @@ def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None
     a.out_qmin, a.out_qmax, a.out_offset = int(out_qmin), int(out_qmax), int(out_offset)
     a.out, a.force_path, a.tile_config = out.data_ptr, int(path), int(tile_config)
     _fill_join(a.join, join, out.shape)
+    if w_zp is not None and w_zp.numel != Cout:
+        raise _C.ShapeMismatch(f"w_zp has {w_zp.numel} entries for Cout = {Cout}")
+    a.w_zp = _ptr(w_zp, "w_zp", T.int32)
     _C.call("lq_qconv2d_i8", C.byref(a), None)
     return out

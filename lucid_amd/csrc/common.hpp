@@ -42,7 +42,8 @@ int hip_fail(hipError_t e, const char* what);
 // may be baked into the graph).  `fresh` reports that the buffer was (re)allocated by
 // this request and holds no defined contents.
 int stream_buffer(int kind, size_t nbytes, size_t min_bytes, hipStream_t stream, void** ptr, bool* fresh);
-// kind 0: the general workspace (at least 4 MiB)
+// kind 0: the general workspace (at least 4 MiB); 1 / 2: stream-K counters / slabs;
+// 3: raw accumulators and operand sums of a layer with affine weights
 int workspace(size_t nbytes, hipStream_t stream, void** ptr);
 // Resolves, for the current device, the address of the static scratch array that
 // lq_minmax_noalloc uses (called by lq_init; the entry point does it on first use otherwise).

@@ -485,6 +485,38 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
     const int jrc = set_join(g, p->join, p->out_mode, p->Cout, "qconv2d_i8");
     if (jrc) return jrc;
 
+    if (p->w_zp && p->out_mode != OUT_ACC_I32) {
+        // affine filters: the raw accumulators, then the window sums of the image as a
+        // convolution with one all-ones filter per group (taps in the padding read the
+        // code a_zp, as in the main pass), then the corrections and the epilogue proper
+        LQ_REQUIRE(p->wsum, LQ_ERR_VALUE, "qconv2d_i8: affine filters need the filter sums");
+        LQ_REQUIRE(K <= 33025, LQ_ERR_SHAPE,
+                   "qconv2d_i8: K = %ld overflows the int32 accumulator with affine filters", K);
+        const size_t acc_bytes = (M * p->Cout * 4 + 255) / 256 * 256;
+        const size_t sum_bytes = (M * p->groups * 4 + 255) / 256 * 256;
+        const size_t ones_bytes = size_t(p->groups) * K;
+        void* tmp = nullptr;
+        bool fresh = false;
+        int rc = stream_buffer(3, acc_bytes + sum_bytes + ones_bytes, 0, st, &tmp, &fresh);
+        if (rc) return rc;
+        int32_t* acc = static_cast<int32_t*>(tmp);
+        int32_t* asum = reinterpret_cast<int32_t*>(static_cast<char*>(tmp) + acc_bytes);
+        int8_t* ones = static_cast<int8_t*>(tmp) + acc_bytes + sum_bytes;
+        rc = lq_fill_bytes(ones, 1, ones_bytes, stream);
+        if (rc) return rc;
+        lq_qconv2d_args raw = *p;
+        raw.w_zp = nullptr; raw.out_mode = OUT_ACC_I32; raw.out = acc; raw.join = lq_join_args{};
+        raw.bias = nullptr; raw.relu = 0;
+        rc = lq_qconv2d_i8(&raw, stream);
+        if (rc) return rc;
+        lq_qconv2d_args win = raw;
+        win.w = ones; win.Cout = p->groups; win.out = asum; win.tile_config = 0;
+        rc = lq_qconv2d_i8(&win, stream);
+        if (rc) return rc;
+        g.N = p->Cout;
+        return launch_affine_fixup(g, acc, asum, p->groups, Og, p->w_zp, int(K), st);
+    }
+
     const bool is_gemm = p->KH == 1 && p->KW == 1 && p->stride_h == 1 && p->stride_w == 1 &&
                          p->pad_h_lo == 0 && p->pad_h_hi == 0 && p->pad_w_lo == 0 &&
                          p->pad_w_hi == 0 && p->groups == 1;

@@ -407,6 +407,33 @@ __global__ __launch_bounds__(256) void qgemm_naive_kernel(GemmArgs g) {
     }
 }
 
+// One thread per output element: the affine-weight corrections on the stored raw
+// accumulator, in wrapping 32-bit arithmetic (the true value fits int32, so every partial
+// wrap cancels), then the ordinary scalar epilogue.
+__global__ __launch_bounds__(256) void affine_fixup_kernel(GemmArgs g, const int32_t* __restrict__ acc,
+                                                           const int32_t* __restrict__ asum, int asum_ld,
+                                                           int n_per_group, const int32_t* __restrict__ w_zp,
+                                                           int kdot) {
+    const size_t total = size_t(g.M) * g.N;
+    float S = 1.0f, Z = 0.0f;
+    if (g.out_mode == OUT_REQUANT_I8 || g.out_mode == OUT_FAKEQUANT_F32) {
+        S = g.out_scale[0];
+        Z = g.out_zp[0];
+    }
+    const int za = g.a_zp_dev ? int(g.a_zp_dev[0]) + g.a_zp : g.a_zp;
+    for (size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x; idx < total;
+         idx += size_t(gridDim.x) * 256) {
+        const int m = int(idx / g.N), n = int(idx % g.N);
+        ColParams c = load_col(g, n);
+        const uint32_t zw = uint32_t(w_zp[n]);
+        const uint32_t rs = uint32_t(asum[size_t(m) * asum_ld + n / n_per_group]);
+        const uint32_t eff = uint32_t(acc[idx]) - uint32_t(c.corr) - zw * rs + uint32_t(kdot) * uint32_t(za) * zw;
+        c.corr = 0;
+        const float as = g.a_scale ? g.a_scale[g.a_scale_per_row ? m : 0] : 1.0f;
+        epilogue_store(g, m, n, int32_t(eff), as, c, S, Z);
+    }
+}
+
 __global__ void rowsum_i8_kernel(const int8_t* __restrict__ w, int32_t* __restrict__ out, int N,
                                  int K) {
     // one wavefront per row
@@ -547,6 +574,23 @@ int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, int rel
 
 int lq_last_tile_config(void) { return t_last_tile_config; }
 
+}  // extern "C"
+
+namespace lq {
+int launch_affine_fixup(const GemmArgs& g, const int32_t* acc, const int32_t* asum, int asum_ld,
+                        int n_per_group, const int32_t* w_zp, int kdot, hipStream_t st) {
+    const size_t total = size_t(g.M) * g.N;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(affine_fixup_kernel, dim3(unsigned(blocks)), dim3(256), 0, st, g, acc, asum, asum_ld,
+                       n_per_group, w_zp, kdot);
+    LQ_CHECK_LAUNCH("affine_fixup");
+    return LQ_OK;
+}
+}  // namespace lq
+
+extern "C" {
+
 int lq_rowsum_i8(const int8_t* w, int32_t* out, int N, int K, lq_stream stream) {
     if (N == 0) return LQ_OK;
     LQ_REQUIRE(w && out, LQ_ERR_VALUE, "rowsum_i8: NULL pointer");
@@ -621,6 +665,29 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
     g.gelu = p->gelu != 0;
     g.range = p->range;
 
+    if (p->w_zp && p->out_mode != OUT_ACC_I32) {
+        // affine weights: raw accumulators and the activation row sums into temporaries,
+        // then one elementwise pass with the corrections and the epilogue proper
+        LQ_REQUIRE(p->wsum, LQ_ERR_VALUE, "qlinear_i8: affine weights need the weight row sums");
+        LQ_REQUIRE(p->range == nullptr, LQ_ERR_VALUE, "qlinear_i8: a kept range is not available with affine weights");
+        LQ_REQUIRE(p->K <= 33025, LQ_ERR_SHAPE,
+                   "qlinear_i8: K = %d overflows the int32 accumulator with affine weights", p->K);
+        hipStream_t st = as_stream(stream);
+        void* tmp = nullptr;
+        bool fresh = false;
+        const size_t acc_bytes = (size_t(p->M) * p->N * 4 + 255) / 256 * 256;
+        int rc = stream_buffer(3, acc_bytes + size_t(p->M) * 4, 0, st, &tmp, &fresh);
+        if (rc) return rc;
+        int32_t* acc = static_cast<int32_t*>(tmp);
+        int32_t* asum = reinterpret_cast<int32_t*>(static_cast<char*>(tmp) + acc_bytes);
+        GemmArgs raw{};
+        raw.a = p->a; raw.w = p->w; raw.M = p->M; raw.N = p->N; raw.K = p->K;
+        raw.out_mode = OUT_ACC_I32; raw.out = acc; raw.ldo = p->N;
+        rc = run_gemm(raw, p->force_path, p->tile_config, st);
+        if (!rc) rc = lq_rowsum_i8(p->a, asum, p->M, p->K, stream);
+        if (!rc) rc = launch_affine_fixup(g, acc, asum, 1, p->N, p->w_zp, p->K, st);
+        return rc;
+    }
     return run_gemm(g, p->force_path, p->tile_config, as_stream(stream));
 }
 

@@ -94,4 +94,12 @@ int run_tile_kernel(const GemmArgs& g, bool conv, int groups, int tile_config, h
 // 1 = tile, 2 = skinny, 3 = naive) and launches.
 int run_gemm(const GemmArgs& g, int force_path, int tile_config, hipStream_t st);
 
+// Second pass of a layer whose weight codes are affine (zero points w_zp[n]).  acc is the
+// raw [M, N] sum_k a*w (contiguous), asum[m * asum_ld + n / n_per_group] the sum of the
+// activation codes that met column n's weights (kdot of them).  Forms
+//     acc - a_zp*wsum[n] - w_zp[n]*asum + kdot*a_zp*w_zp[n]
+// and stores it through the epilogue that g describes (g.out / g.ldo / g.out_mode ...).
+int launch_affine_fixup(const GemmArgs& g, const int32_t* acc, const int32_t* asum, int asum_ld,
+                        int n_per_group, const int32_t* w_zp, int kdot, hipStream_t st);
+
 }  // namespace lq

@@ -58,13 +58,33 @@ def activation_qparams(mod) -> tuple[Tensor, Tensor, QDtype]:
     return scale.to("hip"), zero_point.to("hip"), obs.qdtype
 
 
-def require_symmetric_weight(zero_point: Tensor, what: str) -> None:
-    """The int8 kernels fold the activation zero point only; a non-zero weight
-    zero point would also need activation row sums."""
-    if np.any(zero_point.numpy() != 0):
-        raise NotImplementedError(
-            f"{what}: affine (non-zero zero_point) weights are not supported by the hip int8 "
-            "kernels; use a symmetric weight observer (Lucid's default)")
+_UNSET = object()
+
+
+def weight_zero_points(mod, tile: int = 1) -> Tensor | None:
+    """The zero points of a module's weight rows as the int32 device vector the int8
+    kernels take, or ``None`` when every one is zero (symmetric weights, Lucid's default:
+    the kernels then skip the activation sums).  ``tile`` repeats the vector (the
+    per-group copies of a transposed convolution's channels).  Cached on the module until
+    ``weight_zero_point`` is loaded again."""
+    cached = mod.__dict__.get("_wzp", _UNSET)
+    if cached is not _UNSET:
+        return cached
+    z = mod.weight_zero_point.numpy().reshape(-1).astype(np.float64)
+    if not np.any(z != 0):
+        wzp = None
+    else:
+        zi = np.rint(z)
+        if np.any(zi != z) or zi.min() < -128 or zi.max() > 127:
+            raise ValueError(f"{type(mod).__name__}: weight zero points must be int8 codes, got "
+                             f"values in [{z.min()}, {z.max()}]")
+        wzp = T.tensor(np.tile(zi.astype(np.int32), tile), device="hip")
+    mod.__dict__["_wzp"] = wzp
+    return wzp
+
+
+def forget_weight_zero_points(mod) -> None:
+    mod.__dict__.pop("_wzp", None)
 
 
 def input_grid(x: Tensor, what: str) -> Grid:

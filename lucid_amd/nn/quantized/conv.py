@@ -23,7 +23,7 @@ from ..._tensor import Grid, Tensor
 from ...quantization._qscheme import QDtype, quint8
 from ..module import Module
 from ._utils import (activation_qparams, host_scalar, input_grid, quantize_weight,
-                     require_symmetric_weight, storage_offset)
+                     forget_weight_zero_points, storage_offset, weight_zero_points)
 
 
 _PAD_MODES = {"zeros": 0, "reflect": 1, "replicate": 2, "circular": 3}
@@ -74,7 +74,7 @@ class Conv2d(Module):
         if name == "zero_point":
             self._zp_host = None
         if name == "weight_zero_point":
-            require_symmetric_weight(self.weight_zero_point, type(self).__name__)
+            forget_weight_zero_points(self)
 
     def _resolve_pad(self, x: Tensor) -> tuple[int, int, int, int]:
         """(h_lo, h_hi, w_lo, w_hi), as ``conv.py:119-141``."""
@@ -145,7 +145,7 @@ class Conv2d(Module):
             pad=pad, dilation=self.dilation, groups=self.groups,
             relu=self._fused_relu, out_mode=_ops.OUT_REQUANT_I8, out_scale=self.scale,
             out_zp=self.zero_point, out_qmin=self.out_qdtype.quant_min,
-            out_qmax=self.out_qdtype.quant_max, out_offset=off, join=jarg)
+            out_qmax=self.out_qdtype.quant_max, out_offset=off, join=jarg, w_zp=weight_zero_points(self))
         B, OH, OW, Co = codes.shape
         if out_grid is not None:
             return Tensor.on_grid((B, Co, OH, OW), Grid(codes, *out_grid, "nhwc"))
@@ -158,7 +158,6 @@ class Conv2d(Module):
         qmod = cls(mod.in_channels, mod.out_channels, mod.kernel_size, mod.stride, mod.padding,
                    mod.dilation, mod.groups, bias=mod.bias is not None)
         codes, w_scale, w_zp, ch_axis = quantize_weight(mod)
-        require_symmetric_weight(w_zp, cls.__name__)
         qmod.register_buffer("weight_int8", codes)
         qmod.register_buffer("weight_scale", w_scale)
         qmod.register_buffer("weight_zero_point", w_zp)
@@ -226,7 +225,6 @@ class Conv1d(Conv2d):
         qmod = cls(mod.in_channels, mod.out_channels, mod.kernel_size, mod.stride, mod.padding,
                    mod.dilation, mod.groups, bias=mod.bias is not None)
         codes, w_scale, w_zp, ch_axis = quantize_weight(mod)
-        require_symmetric_weight(w_zp, cls.__name__)
         qmod.register_buffer("weight_int8", codes)
         qmod.register_buffer("weight_scale", w_scale)
         qmod.register_buffer("weight_zero_point", w_zp)
@@ -252,7 +250,7 @@ def _triple(v):
 
 def volumetric_gemm(name, x: Tensor, g, w_rows: Tensor, wsum: Tensor, w_scale: Tensor, bias, kernel, stride,
                     pads, dilation, insert, groups: int, relu: bool, scale: Tensor, zero_point: Tensor,
-                    qdtype: QDtype, zp_host: int) -> Tensor:
+                    qdtype: QDtype, zp_host: int, w_zp: Tensor | None = None) -> Tensor:
     """A 3-d convolution on codes as an explicit GEMM, group by group: gather the taps of
     ``x``'s ``(B, C, D, H, W)`` codes (``insert`` > 1: as if zero-point codes stood between
     neighbouring samples), multiply with the group's kernel rows ``[Cout/groups, taps * C/groups]``
@@ -282,7 +280,7 @@ def volumetric_gemm(name, x: Tensor, g, w_rows: Tensor, wsum: Tensor, w_scale: T
         y = _ops.qlinear_i8(cols, part(w_rows), a_zp=a_zp, a_scale=g.scale, w_scale=part(w_scale), wsum=part(wsum),
                             bias=None if bias is None else part(bias), relu=relu, out_mode=_ops.OUT_REQUANT_I8,
                             out_scale=scale, out_zp=zero_point, out_qmin=qdtype.quant_min,
-                            out_qmax=qdtype.quant_max, out_offset=off)
+                            out_qmax=qdtype.quant_max, out_offset=off, w_zp=None if w_zp is None else part(w_zp))
         # each batch's [L, Og] block -> its (Og, L) channel slice of the (B, Co, L) output
         _C.call("lq_transpose_i8", y.data_ptr, codes.data_ptr + grp * Og * L, B, L, Og, L * Og, Co * L, None)
     return Tensor.on_grid((B, Co, *outs), Grid(codes, scale, zero_point, qdtype, off, zp_host, "plain"))
@@ -343,7 +341,8 @@ class Conv3d(Conv2d):
         pads = self._resolve_pad3(x.shape[2:])
         return volumetric_gemm(name, x, g, self._w_ohwi, self._wsum, self.weight_scale, self.bias, self.kernel_size,
                                self.stride, pads, self.dilation, (1, 1, 1), self.groups, self._fused_relu,
-                               self.scale, self.zero_point, self.out_qdtype, self._zp_host)
+                               self.scale, self.zero_point, self.out_qdtype, self._zp_host,
+                               w_zp=weight_zero_points(self))
 
     @classmethod
     def from_float(cls, mod) -> "Conv3d":
@@ -351,7 +350,6 @@ class Conv3d(Conv2d):
         qmod = cls(mod.in_channels, mod.out_channels, mod.kernel_size, mod.stride, mod.padding,
                    mod.dilation, mod.groups, bias=mod.bias is not None)
         codes, w_scale, w_zp, ch_axis = quantize_weight(mod)
-        require_symmetric_weight(w_zp, cls.__name__)
         qmod.register_buffer("weight_int8", codes)
         qmod.register_buffer("weight_scale", w_scale)
         qmod.register_buffer("weight_zero_point", w_zp)

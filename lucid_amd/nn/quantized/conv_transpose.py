@@ -21,7 +21,7 @@ from ..._tensor import Grid, Tensor
 from ...quantization._functional import quantize
 from ...quantization._qscheme import QDtype, per_channel_symmetric, qint8, quint8
 from ..module import Module
-from ._utils import activation_qparams, host_scalar, input_grid, require_symmetric_weight, storage_offset
+from ._utils import activation_qparams, host_scalar, forget_weight_zero_points, input_grid, storage_offset, weight_zero_points
 
 
 def _pair(v):
@@ -54,7 +54,7 @@ class ConvTranspose2d(Module):
         if name == "zero_point":
             self._zp_host = None
         if name == "weight_zero_point":
-            require_symmetric_weight(self.weight_zero_point, type(self).__name__)
+            forget_weight_zero_points(self)
 
     def _prepare_weight(self) -> None:
         """The equivalent convolution's kernel, ``(out, kh, kw, in/groups)``: flipped in
@@ -98,7 +98,8 @@ class ConvTranspose2d(Module):
             w_scale=self._w_scale_full, wsum=self._wsum, bias=self.bias, stride=(1, 1),
             pad=(lo_h, lo_h + oph, lo_w, lo_w + opw), dilation=self.dilation, groups=self.groups,
             relu=False, out_mode=_ops.OUT_REQUANT_I8, out_scale=self.scale, out_zp=self.zero_point,
-            out_qmin=self.out_qdtype.quant_min, out_qmax=self.out_qdtype.quant_max, out_offset=off)
+            out_qmin=self.out_qdtype.quant_min, out_qmax=self.out_qdtype.quant_max, out_offset=off,
+            w_zp=weight_zero_points(self, self.groups))
         B, OH, OW, Co = codes.shape
         return Tensor.on_grid((B, Co, OH, OW), Grid(codes, self.scale, self.zero_point, self.out_qdtype, off,
                                                     self._zp_host, "nhwc"))
@@ -223,4 +224,5 @@ class ConvTranspose3d(ConvTranspose2d):
         pads = [(l, l + op) for l, op in zip(lo, self.output_padding)]
         return volumetric_gemm(name, x, g, self._w_ohwi, self._wsum, self._w_scale_full, self.bias, self.kernel_size,
                                (1, 1, 1), pads, self.dilation, self.stride, self.groups, False, self.scale,
-                               self.zero_point, self.out_qdtype, self._zp_host)
+                               self.zero_point, self.out_qdtype, self._zp_host,
+                               w_zp=weight_zero_points(self, self.groups))

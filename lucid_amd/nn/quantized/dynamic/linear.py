@@ -20,7 +20,7 @@ from ....quantization._functional import minmax, quantize
 from ....quantization._qparams import calculate_qparams
 from ....quantization._qscheme import QDtype, per_channel_symmetric, per_tensor_affine, qint8, quint8
 from ...module import Module
-from .._utils import require_symmetric_weight, storage_offset
+from .._utils import forget_weight_zero_points, storage_offset, weight_zero_points
 
 
 class Linear(Module):
@@ -43,7 +43,7 @@ class Linear(Module):
         if name == "weight_int8":
             self._wsum = None
         if name == "weight_zero_point":
-            require_symmetric_weight(self.weight_zero_point, "dynamic.Linear")
+            forget_weight_zero_points(self)
 
     def forward(self, x: Tensor, residual: Tensor | None = None, activation: str | None = None,
                 track_range: bool = False) -> Tensor:
@@ -97,13 +97,17 @@ class Linear(Module):
         if self._wsum is None:
             self._wsum = _ops.rowsum_i8(self.weight_int8)
         rng = None
+        w_zp = weight_zero_points(self)
+        if track_range and w_zp is not None:
+            raise NotImplementedError("dynamic.Linear: track_range (an extension of this backend) is "
+                                      "not available with affine weights")
         if track_range:
             from ...functional import _new_range
             rng = _new_range()
         y = _ops.qlinear_i8(xq, self.weight_int8, a_zp=off, a_zp_dev=x_zp, a_scale=x_scale,
                             w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias,
                             out_mode=_ops.OUT_F32, residual=residual, gelu=activation == "gelu",
-                            range_buf=rng)
+                            range_buf=rng, w_zp=w_zp)
         y = y.reshape(*lead_shape, N)
         y._range = rng
         return y

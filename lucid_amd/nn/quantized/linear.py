@@ -20,7 +20,7 @@ from ..._tensor import Grid, Tensor
 from ...quantization._qscheme import QDtype, quint8
 from ..module import Module
 from ._utils import (activation_qparams, host_scalar, input_grid, quantize_weight,
-                     require_symmetric_weight, storage_offset, zp_args)
+                     forget_weight_zero_points, storage_offset, weight_zero_points, zp_args)
 
 
 class Linear(Module):
@@ -50,7 +50,7 @@ class Linear(Module):
         if name == "zero_point":
             self._zp_host = None
         if name == "weight_zero_point":
-            require_symmetric_weight(self.weight_zero_point, type(self).__name__)
+            forget_weight_zero_points(self)
 
     def _activation(self, y: Tensor) -> Tensor:
         """Post-linear activation hook (identity; ReLU in the fused variant).
@@ -94,7 +94,7 @@ class Linear(Module):
             a_scale=g.scale, w_scale=self.weight_scale, wsum=self._wsum, bias=self.bias,
             relu=self._fused_relu, out_mode=_ops.OUT_REQUANT_I8, out_scale=self.scale,
             out_zp=self.zero_point, out_qmin=self.out_qdtype.quant_min,
-            out_qmax=self.out_qdtype.quant_max, out_offset=off)
+            out_qmax=self.out_qdtype.quant_max, out_offset=off, w_zp=weight_zero_points(self))
         shape = x.shape[:-1] + (N,)
         return Tensor.on_grid(shape, Grid(codes.reshape(shape), self.scale, self.zero_point,
                                           self.out_qdtype, off, self._zp_host))
@@ -105,7 +105,6 @@ class Linear(Module):
         has_bias = mod.bias is not None
         qmod = cls(mod.in_features, mod.out_features, bias=has_bias)
         codes, w_scale, w_zp, ch_axis = quantize_weight(mod)
-        require_symmetric_weight(w_zp, cls.__name__)
         qmod.register_buffer("weight_int8", codes)
         qmod.register_buffer("weight_scale", w_scale)
         qmod.register_buffer("weight_zero_point", w_zp)

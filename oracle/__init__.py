@@ -196,9 +196,10 @@ def _bias_kind(bias):
 
 
 def qlinear(a, w, a_zp, a_scale, w_scale, bias=None, relu=False, out_mode=OUT_F32,
-            out_scale=1.0, out_zp=0.0, out_qmin=0, out_qmax=255, out_offset=0):
+            out_scale=1.0, out_zp=0.0, out_qmin=0, out_qmax=255, out_offset=0, w_zp=None):
     """Integer-formulation quantized Linear.  ``a`` int8 [M,K] stored codes,
-    ``a_zp`` the zero point of the stored codes, ``a_scale`` scalar or [M]."""
+    ``a_zp`` the zero point of the stored codes, ``a_scale`` scalar or [M];
+    ``w_zp`` int [N] zero points of the weight rows (None: symmetric weights)."""
     a = np.ascontiguousarray(a, dtype=np.int8)
     w = np.ascontiguousarray(w, dtype=np.int8)
     M, K = a.shape
@@ -209,6 +210,13 @@ def qlinear(a, w, a_zp, a_scale, w_scale, bias=None, relu=False, out_mode=OUT_F3
     w_scale = _f32(w_scale).reshape(-1)
     bk, b = _bias_kind(bias)
     out = _out_array((M, N), out_mode)
+    if w_zp is not None:
+        zw = np.ascontiguousarray(np.broadcast_to(np.asarray(w_zp, dtype=np.int32).reshape(-1), (N,)))
+        lib().orc_qlinear_affine(_p(a), _p(w), _p(zw), M, N, K, int(a_zp), _p(a_scale), per_row,
+                                 _p(w_scale), bk, _p(b), int(relu), out_mode, C.c_float(out_scale),
+                                 C.c_float(out_zp), int(out_qmin), int(out_qmax), int(out_offset),
+                                 _p(out))
+        return out.view(np.float16) if out_mode == OUT_F16 else out
     lib().orc_qlinear(_p(a), _p(w), M, N, K, int(a_zp), _p(a_scale), per_row, _p(w_scale), bk,
                       _p(b), int(relu), out_mode, C.c_float(out_scale), C.c_float(out_zp),
                       int(out_qmin), int(out_qmax), int(out_offset), _p(out))
@@ -236,9 +244,10 @@ def conv_out_size(S, K, stride, pad_lo, pad_hi, dil):
 
 def qconv2d(x, w, a_zp, a_scale, w_scale, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1),
             groups=1, bias=None, relu=False, out_mode=OUT_F32, out_scale=1.0, out_zp=0.0,
-            out_qmin=0, out_qmax=255, out_offset=0):
+            out_qmin=0, out_qmax=255, out_offset=0, w_zp=None):
     """Integer-formulation Conv2d.  ``x`` int8 NHWC codes, ``w`` int8
-    [Cout,KH,KW,Cin/groups], ``pad`` = (h_lo, h_hi, w_lo, w_hi).  Output NHWC."""
+    [Cout,KH,KW,Cin/groups], ``pad`` = (h_lo, h_hi, w_lo, w_hi); ``w_zp`` int [Cout] zero
+    points of the filters (None: symmetric).  Output NHWC."""
     x = np.ascontiguousarray(x, dtype=np.int8)
     w = np.ascontiguousarray(w, dtype=np.int8)
     B, H, W, Cin = x.shape
@@ -248,6 +257,15 @@ def qconv2d(x, w, a_zp, a_scale, w_scale, stride=(1, 1), pad=(0, 0, 0, 0), dilat
     OW = conv_out_size(W, KW, stride[1], pad[2], pad[3], dilation[1])
     bk, b = _bias_kind(bias)
     out = _out_array((B, OH, OW, Cout), out_mode)
+    if w_zp is not None:
+        zw = np.ascontiguousarray(np.broadcast_to(np.asarray(w_zp, dtype=np.int32).reshape(-1), (Cout,)))
+        lib().orc_qconv2d_affine(_p(x), _p(w), _p(zw), B, H, W, Cin, Cout, KH, KW, stride[0],
+                                 stride[1], pad[0], pad[1], pad[2], pad[3], dilation[0],
+                                 dilation[1], groups, int(a_zp), C.c_float(a_scale),
+                                 _p(_f32(w_scale)), bk, _p(b), int(relu), out_mode,
+                                 C.c_float(out_scale), C.c_float(out_zp), int(out_qmin),
+                                 int(out_qmax), int(out_offset), _p(out))
+        return out.view(np.float16) if out_mode == OUT_F16 else out
     lib().orc_qconv2d(_p(x), _p(w), B, H, W, Cin, Cout, KH, KW, stride[0], stride[1], pad[0],
                       pad[1], pad[2], pad[3], dilation[0], dilation[1], groups, int(a_zp),
                       C.c_float(a_scale), _p(_f32(w_scale)), bk, _p(b), int(relu), out_mode,

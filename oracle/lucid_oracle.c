@@ -497,6 +497,35 @@ void orc_qlinear(const int8_t* a, const int8_t* w, int M, int N, int K, int a_zp
     free(wsum);
 }
 
+/* The same Linear with affine weight codes: row n of w carries the zero point w_zp[n]
+ * (per-channel affine weights, lucid/quantization/_qscheme.py per_channel_affine, as
+ * from_float stores them in nn/quantized/linear.py:217-236).  The float composite
+ * dequantizes both operands before the product (linear.py:199-215), so the exact
+ * integer value under the two scales is
+ *     eff[m,n] = sum_k (a[m,k] - a_zp) * (w[n,k] - w_zp[n]),
+ * taken here term by term in 64 bits; the epilogue is orc_qlinear's with the
+ * corrections already applied.  Mode ACC_I32 returns the raw sum_k a*w as before. */
+void orc_qlinear_affine(const int8_t* a, const int8_t* w, const int32_t* w_zp, int M, int N,
+                        int K, int a_zp, const float* a_scale, int a_scale_per_row,
+                        const float* w_scale, int bias_kind, const void* bias, int relu,
+                        int out_mode, float out_scale, float out_zp, int out_qmin,
+                        int out_qmax, int out_offset, void* out) {
+    int32_t* eff = (int32_t*)malloc((size_t)M * N * sizeof(int32_t));
+#pragma omp parallel for schedule(static)
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            int64_t s = 0;
+            const int64_t zw = (out_mode == ORC_OUT_ACC_I32 || !w_zp) ? 0 : w_zp[n];
+            const int64_t za = out_mode == ORC_OUT_ACC_I32 ? 0 : a_zp;
+            for (int k = 0; k < K; ++k)
+                s += ((int64_t)a[(size_t)m * K + k] - za) * ((int64_t)w[(size_t)n * K + k] - zw);
+            eff[(size_t)m * N + n] = (int32_t)s;
+        }
+    orc_qlinear_epilogue(eff, M, N, 0, NULL, a_scale, a_scale_per_row, w_scale, bias_kind, bias,
+                         relu, out_mode, out_scale, out_zp, out_qmin, out_qmax, out_offset, out);
+    free(eff);
+}
+
 /* ------------------------------------------------------------------ */
 /* float GEMM used by the faithful path:  c[m,n] = sum_k a[m,k]*b[n,k]  */
 /* (the reference calls cblas_sgemm with transB, CpuBackend.h:4493;    */
@@ -641,6 +670,53 @@ void orc_qconv2d(const int8_t* x, const int8_t* w, int B, int H, int W, int Cin,
         free(acc);
     }
     (void)esz;
+}
+
+/* orc_qconv2d with affine filter codes: filter co carries the zero point w_zp[co]
+ * (nn/quantized/conv.py from_float with a per-channel affine weight observer).  Taps in
+ * the padding hold the code a_zp, i.e. the float value 0 that zero padding of the
+ * dequantized image gives (Im2Col.cpp:59-100), so they contribute (a_zp - a_zp) * (...) = 0
+ * exactly as in the float composite. */
+void orc_qconv2d_affine(const int8_t* x, const int8_t* w, const int32_t* w_zp, int B, int H,
+                        int W, int Cin, int Cout, int KH, int KW, int sh, int sw, int ph_lo,
+                        int ph_hi, int pw_lo, int pw_hi, int dh, int dw, int groups, int a_zp,
+                        float a_scale, const float* w_scale, int bias_kind, const void* bias,
+                        int relu, int out_mode, float out_scale, float out_zp, int out_qmin,
+                        int out_qmax, int out_offset, void* out) {
+    int OH = orc_conv_out_size(H, KH, sh, ph_lo, ph_hi, dh);
+    int OW = orc_conv_out_size(W, KW, sw, pw_lo, pw_hi, dw);
+    int Cg = Cin / groups, Og = Cout / groups;
+#pragma omp parallel for schedule(static)
+    for (int b = 0; b < B; ++b)
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow)
+                for (int co = 0; co < Cout; ++co) {
+                    const int g = co / Og;
+                    const int64_t zw = (out_mode == ORC_OUT_ACC_I32 || !w_zp) ? 0 : w_zp[co];
+                    const int64_t za = out_mode == ORC_OUT_ACC_I32 ? 0 : a_zp;
+                    int64_t s = 0;
+                    for (int kh = 0; kh < KH; ++kh)
+                        for (int kw = 0; kw < KW; ++kw) {
+                            const int ih = oh * sh - ph_lo + kh * dh, iw = ow * sw - pw_lo + kw * dw;
+                            const int inside = ih >= 0 && ih < H && iw >= 0 && iw < W;
+                            for (int ci = 0; ci < Cg; ++ci) {
+                                const int64_t av =
+                                    inside ? x[(((size_t)b * H + ih) * W + iw) * Cin + g * Cg + ci]
+                                           : a_zp;
+                                const int64_t wv = w[(((size_t)co * KH + kh) * KW + kw) * Cg + ci];
+                                s += (av - za) * (wv - zw);
+                            }
+                        }
+                    size_t idx = (((size_t)b * OH + oh) * OW + ow) * Cout + co;
+                    if (out_mode == ORC_OUT_ACC_I32) {
+                        ((int32_t*)out)[idx] = (int32_t)s;
+                        continue;
+                    }
+                    float y = epi_value((int32_t)s, 0, 0, a_scale, w_scale[co], bias_kind, bias,
+                                        (size_t)co, relu);
+                    epilogue_store(y, out_mode, out, idx, out_scale, out_zp, out_qmin, out_qmax,
+                                   out_offset);
+                }
 }
 
 /* Float im2col for one image, one group, NCHW (Im2Col.cpp:59-100): rows are

@@ -19,7 +19,7 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_version_and_registry():
-    assert _C.load().lq_version() == _C.ABI_VERSION == 2
+    assert _C.load().lq_version() == _C.ABI_VERSION == 3
     ops = dict((n, (v, d)) for n, v, d in _C.op_registry())
     for name in ("quantize", "dequantize", "fake_quantize", "minmax", "calc_qparams"):
         assert ops[name] == (1, True)

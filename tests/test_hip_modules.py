@@ -278,6 +278,84 @@ class TestStaticPTQ:
         assert q(idx) is idx
 
 
+# ------------------------------------------------------------------ affine weights
+def _affine_qconfig():
+    from lucid_amd.quantization.observer import HistogramObserver, PerChannelMinMaxObserver
+    return Q.QConfig(activation=HistogramObserver.with_args(qscheme=Q.per_tensor_affine, qdtype=Q.quint8),
+                     weight=PerChannelMinMaxObserver.with_args(ch_axis=0, qscheme=Q.per_channel_affine,
+                                                               qdtype=Q.qint8))
+
+
+def _oracle_affine_weight(w):
+    mn, mx = O.minmax(w, ch_axis=0)
+    ws, wz = O.calc_qparams(mn, mx, False, -128, 127, True)
+    return O.quantize(w, ws, wz, -128, 127, ch_axis=0), ws, wz
+
+
+def test_static_ptq_with_per_channel_affine_weights():
+    """A weight observer with qscheme per_channel_affine gives non-zero weight zero points;
+    convert() keeps them and the int8 forward applies them: bit-exact against the oracle's
+    integer formulation, within a code of Lucid's float composite."""
+    rng = np.random.default_rng(4)
+    m, params = _static_model(rng)
+    w1, b1, w2, b2 = params
+    w1 = (w1 + rng.uniform(-0.5, 0.5, (32, 1))).astype(np.float32)   # rows off centre: zero points != 0
+    w2 = (w2 + rng.uniform(-0.5, 0.5, (8, 1))).astype(np.float32)
+    _set(m.fc1[0], w1, b1)
+    _set(m.fc2, w2, b2)
+    params = (w1, b1, w2, b2)
+    prepared = Q.prepare(m, _affine_qconfig())
+    _calibrate(prepared, params, rng)
+    qm = Q.convert(prepared)
+    assert np.any(qm.fc1.weight_zero_point.numpy() != 0) and np.any(qm.fc2.weight_zero_point.numpy() != 0)
+    x = rng.standard_normal((64, 16)).astype(np.float32)
+    y = qm(hip(x)).numpy()
+    s0, z0 = qm.quant.scale.item(), qm.quant.zero_point.item()
+    s1, z1 = qm.fc1.scale.item(), qm.fc1.zero_point.item()
+    s2, z2 = qm.fc2.scale.item(), qm.fc2.zero_point.item()
+    xq = O.quantize(x, s0, z0, 0, 255, code_offset=-128)
+    wq1, ws1, wz1 = _oracle_affine_weight(w1)
+    wq2, ws2, wz2 = _oracle_affine_weight(w2)
+    assert np.array_equal(qm.fc1.weight_int8.numpy(), wq1) and np.array_equal(qm.fc1.weight_zero_point.numpy(), wz1)
+    h = O.qlinear(xq, wq1, int(z0) - 128, s0, ws1, bias=b1, relu=True, out_mode=O.OUT_REQUANT_I8,
+                  out_scale=s1, out_zp=z1, out_offset=-128, w_zp=wz1.astype(np.int32))
+    yq = O.qlinear(h, wq2, int(z1) - 128, s1, ws2, bias=b2, out_mode=O.OUT_REQUANT_I8,
+                   out_scale=s2, out_zp=z2, out_offset=-128, w_zp=wz2.astype(np.int32))
+    assert np.array_equal(y.view(np.uint32), O.dequantize(yq, s2, z2, code_offset=-128).view(np.uint32))
+    xf = O.fake_quantize(x, s0, z0, 0, 255)
+    hf = O.linear_faithful(xf, wq1, ws1, wz1, bias=b1, relu=True, fq=(s1, z1, 0, 255))
+    yf = O.linear_faithful(hf, wq2, ws2, wz2, bias=b2, fq=(s2, z2, 0, 255))
+    assert np.abs(y - yf).max() <= s2 * 1.001 and (y != yf).mean() < 0.02
+    # a state_dict round trip keeps the zero points in force
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")  # the twin is converted uncalibrated on purpose
+        qm2 = Q.convert(Q.prepare(_static_model(np.random.default_rng(9))[0], _affine_qconfig()))
+    qm2.load_state_dict(qm.state_dict())
+    assert np.array_equal(qm2(hip(x)).numpy().view(np.uint32), y.view(np.uint32))
+
+
+def test_dynamic_linear_with_affine_weights():
+    rng = np.random.default_rng(6)
+    lin = nnqd.Linear(48, 24)
+    w = codes = rng.integers(-128, 128, (24, 48)).astype(np.int8)
+    zw = rng.integers(-60, 60, 24).astype(np.float32)
+    ws = rng.uniform(0.001, 0.004, 24).astype(np.float32)
+    b = rng.standard_normal(24).astype(np.float32)
+    lin.load_state_dict({"weight_int8": L.tensor(w), "weight_scale": L.tensor(ws), "weight_zero_point": L.tensor(zw),
+                         "bias": L.tensor(b)})
+    x = rng.standard_normal((10, 48)).astype(np.float32)
+    y = lin(hip(x)).numpy()
+    mn, mx = O.minmax(x)
+    xs, xz = O.calc_qparams(mn, mx, False, 0, 255, False)
+    xq = O.quantize(x, xs, xz, 0, 255, code_offset=-128)
+    exp = O.qlinear(xq, codes, int(xz[0]) - 128, xs, ws, bias=b, w_zp=zw.astype(np.int32))
+    assert np.array_equal(y.view(np.uint32), exp.view(np.uint32))
+    with pytest.raises(ValueError, match="int8 codes"):
+        lin.load_state_dict({"weight_int8": L.tensor(w), "weight_scale": L.tensor(ws),
+                             "weight_zero_point": L.tensor(zw + 0.5), "bias": L.tensor(b)})
+        lin(hip(x))
+
+
 # ------------------------------------------------------------------ residual join
 def test_qfunctional_add_relu_matches_oracle():
     rng = np.random.default_rng(5)

@@ -274,3 +274,112 @@ def test_packed_route_for_few_input_channels(B, H, W, Cin, Cout, KH, KW, stride,
                      out_scale=0.05, out_zp=0.0, out_qmin=0, out_qmax=255, out_offset=-128)
     assert np.array_equal(auto.numpy(), want)
     assert np.array_equal(_ops.qconv2d_i8(dx, dw, **kw, path=_ops.CONV_IM2COL).numpy(), want)
+
+
+# ------------------------------------------------------------------ affine filter codes
+@pytest.mark.parametrize("case", [CASES[0], CASES[1], CASES[2], CASES[4], CASES[5], CASES[6], CASES[8]])
+def test_affine_filter_zero_points_on_every_route(case):
+    """Per-channel affine filters (a zero point per output channel): every route and output
+    form equals the oracle's term-by-term sum of (x - za) * (w - zw[co]) over the window, with
+    taps in the padding contributing nothing, bit for bit."""
+    B, H, W, Cin, Cout, KH, KW, st, pad, dil, groups, routes = case
+    rng = np.random.default_rng(31 + sum(case[:7]))
+    x = codes(rng, (B, H, W, Cin))
+    w = codes(rng, (Cout, KH, KW, Cin // groups))
+    zw = rng.integers(-128, 128, Cout).astype(np.int32)
+    zw[::5] = 0
+    a_zp = int(rng.integers(-128, 128))
+    a_scale = np.float32(rng.uniform(0.005, 0.03))
+    w_scale = rng.uniform(0.0005, 0.004, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    kw = dict(stride=st, pad=pad, dilation=dil, groups=groups, bias=bias, relu=True)
+    y = O.qconv2d(x, w, a_zp, a_scale, w_scale, w_zp=zw, **kw)
+    S, Z = np.float32(y.max() / 250 + 1e-6), np.float32(1.0)
+    xd, wd = hip(x), hip(w)
+    dkw = dict(stride=st, pad=pad, dilation=dil, groups=groups, relu=True, a_zp=a_zp, a_scale=hip(a_scale),
+               w_scale=hip(w_scale), wsum=_ops.rowsum_i8(wd), bias=hip(bias), out_scale=hip(S), out_zp=hip(Z),
+               out_qmin=0, out_qmax=255, out_offset=-128, w_zp=hip(zw))
+    for route in routes + (0,):
+        for mode in (_ops.OUT_F32, _ops.OUT_REQUANT_I8):
+            got = _ops.qconv2d_i8(xd, wd, out_mode=mode, path=route, **dkw).numpy()
+            exp = O.qconv2d(x, w, a_zp, a_scale, w_scale, out_mode=mode, out_scale=S, out_zp=Z, out_qmin=0,
+                            out_qmax=255, out_offset=-128, w_zp=zw, **kw)
+            assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (route, mode)
+    sym = _ops.qconv2d_i8(xd, wd, out_mode=_ops.OUT_F32, **{**dkw, "w_zp": None}).numpy()
+    assert not np.array_equal(sym, O.qconv2d(x, w, a_zp, a_scale, w_scale, w_zp=zw, **kw))
+
+
+def test_affine_filters_with_the_fused_join():
+    B, H, W, Cin, Cout = 2, 10, 10, 32, 48
+    rng = np.random.default_rng(12)
+    x, w = codes(rng, (B, H, W, Cin)), codes(rng, (Cout, 3, 3, Cin))
+    zw = rng.integers(-90, 90, Cout).astype(np.int32)
+    other = codes(rng, (B, H, W, Cout))
+    a_scale, w_scale = np.float32(0.02), rng.uniform(0.0005, 0.004, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    xd, wd = hip(x), hip(w)
+    join = dict(q=hip(other), offset=-128, scale=hip(np.float32(0.04)), zp=hip(np.float32(131.0)), relu=True,
+                out_scale=hip(np.float32(0.06)), out_zp=hip(np.float32(0.0)), out_qmin=0, out_qmax=255,
+                out_offset=-128)
+    got = _ops.qconv2d_i8(xd, wd, a_zp=-3, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=_ops.rowsum_i8(wd),
+                          bias=hip(bias), pad=(1, 1, 1, 1), out_mode=_ops.OUT_REQUANT_I8,
+                          out_scale=hip(np.float32(0.05)), out_zp=hip(np.float32(120.0)), out_qmin=0,
+                          out_qmax=255, out_offset=-128, join=join, w_zp=hip(zw)).numpy()
+    c1 = O.qconv2d(x, w, -3, a_scale, w_scale, pad=(1, 1, 1, 1), bias=bias, out_mode=O.OUT_REQUANT_I8,
+                   out_scale=0.05, out_zp=120.0, out_offset=-128, w_zp=zw)
+    exp = O.add_requant(c1, -128, 0.05, 120.0, other, -128, 0.04, 131.0, True, 0.06, 0.0, 0, 255, -128)
+    assert np.array_equal(got, exp)
+
+
+@pytest.mark.parametrize("groups", [1, 2])
+def test_conv_module_with_affine_filters(groups):
+    """nnq.Conv2d and nnq.ConvTranspose2d loaded with non-zero weight zero points apply them:
+    bit-exact against the oracle on the equivalent convolution."""
+    import lucid_amd.nn.quantized as nnq
+    import lucid_amd.quantization as Q
+    from lucid_amd._tensor import Grid, Tensor
+
+    rng = np.random.default_rng(50 + groups)
+    B, H, W, Cin, Cout = 2, 9, 10, 16, 24
+    x = rng.integers(0, 256, (B, H, W, Cin)).astype(np.int16)
+    in_scale, in_zp = np.float32(0.02), 131
+    grid = Grid(hip((x - 128).astype(np.int8)), L.tensor(np.float32(in_scale), device="hip"),
+                L.tensor(np.float32(in_zp), device="hip"), Q.quint8, -128, in_zp, "nhwc")
+    xin = Tensor.on_grid((B, Cin, H, W), grid)
+
+    wq = codes(rng, (Cout, Cin // groups, 3, 3))
+    ws = rng.uniform(0.001, 0.01, Cout).astype(np.float32)
+    wz = rng.integers(-100, 100, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    conv = nnq.Conv2d(Cin, Cout, 3, padding=1, groups=groups)
+    state = {"weight_int8": wq, "weight_scale": ws, "weight_zero_point": wz, "bias": bias,
+             "scale": np.float32(0.05), "zero_point": np.float32(120.0)}
+    conv.load_state_dict({k: L.tensor(v, device="hip") for k, v in state.items()})
+    got = conv(xin)._grid.codes.numpy()
+    exp = O.qconv2d((x - 128).astype(np.int8), np.ascontiguousarray(wq.transpose(0, 2, 3, 1)), in_zp - 128, in_scale,
+                    ws, pad=(1, 1, 1, 1), groups=groups, bias=bias, out_mode=O.OUT_REQUANT_I8, out_scale=0.05,
+                    out_zp=120.0, out_qmin=0, out_qmax=255, out_offset=-128, w_zp=wz.astype(np.int32))
+    assert np.array_equal(got, exp)
+
+    # transposed: weight (Cin, Cout/groups, kh, kw), qparams per output channel within a group
+    og = Cout // groups
+    wt = codes(rng, (Cin, og, 3, 3))
+    wst = rng.uniform(0.001, 0.01, og).astype(np.float32)
+    wzt = rng.integers(-100, 100, og).astype(np.float32)
+    dec = nnq.ConvTranspose2d(Cin, Cout, 3, stride=2, padding=1, output_padding=1, groups=groups)
+    state = {"weight_int8": wt, "weight_scale": wst, "weight_zero_point": wzt, "bias": bias,
+             "scale": np.float32(0.05), "zero_point": np.float32(120.0)}
+    dec.load_state_dict({k: L.tensor(v, device="hip") for k, v in state.items()})
+    got = dec(xin)._grid.codes.numpy()
+    # the equivalent convolution: zero-point codes between the samples, flipped kernel, channels
+    # swapped inside each group, stride 1, padding k - 1 - p (+ output_padding at the high end)
+    spread = np.full((B, 2 * H - 1, 2 * W - 1, Cin), in_zp - 128, np.int8)
+    spread[:, ::2, ::2] = (x - 128).astype(np.int8)
+    cig = Cin // groups
+    weq = np.concatenate([np.transpose(wt[g * cig:(g + 1) * cig, :, ::-1, ::-1], (1, 2, 3, 0))
+                          for g in range(groups)], axis=0)
+    exp = O.qconv2d(spread, np.ascontiguousarray(weq), in_zp - 128, in_scale, np.tile(wst, groups),
+                    pad=(1, 2, 1, 2), groups=groups, bias=bias, out_mode=O.OUT_REQUANT_I8, out_scale=0.05,
+                    out_zp=120.0, out_qmin=0, out_qmax=255, out_offset=-128,
+                    w_zp=np.tile(wzt, groups).astype(np.int32))
+    assert np.array_equal(got, exp)

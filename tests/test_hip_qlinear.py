@@ -522,3 +522,92 @@ def test_ping_pong_kernel_every_output_form(cfg, M, N, K):
                           out_qmin=-128, out_qmax=127, out_offset=0, **ocommon)
         expj = O.add_requant(first, 0, s1, z1, stored, -128, s2, z2, True, Sj, Zj, 0, 255, -128)
         assert np.array_equal(fused, expj.reshape(M, N))
+
+
+# ------------------------------------------------------------------ affine weight codes
+AFFINE_CASES = [
+    # M, N, K, path
+    (64, 256, 784, TILE), (300, 260, 144, TILE), (2048, 512, 1024, TILE), (1, 11008, 4096, SKINNY),
+    (16, 1024, 4096, SKINNY), (17, 33, 784, SKINNY), (5, 7, 3, NAIVE), (64, 10, 250, NAIVE), (129, 77, 784, 0),
+]
+
+
+@pytest.mark.parametrize("M,N,K,path", AFFINE_CASES)
+def test_affine_weight_zero_points_every_output_form(M, N, K, path):
+    """Per-channel affine weights (a zero point per weight row): every output form equals the
+    oracle's term-by-term sum of (a - za) * (w - zw[n]) bit for bit."""
+    rng = np.random.default_rng(M * 5 + N * 11 + K)
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    zw = rng.integers(-128, 128, N).astype(np.int32)
+    zw[::7] = 0
+    za = int(rng.integers(-128, 128))
+    a_scale = rng.uniform(0.005, 0.05, M).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.5).astype(np.float32)
+    y = O.qlinear(a, w, za, a_scale, w_scale, bias=bias, relu=True, w_zp=zw)
+    S, Z = np.float32(y.max() / 250 + 1e-6), np.float32(2.0)
+    ad, wd = hip(a), hip(w)
+    dkw = dict(a_zp=za, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=_ops.rowsum_i8(wd), bias=hip(bias),
+               relu=True, out_scale=hip(S), out_zp=hip(Z), out_qmin=0, out_qmax=255, out_offset=-128,
+               w_zp=hip(zw), path=path)
+    okw = dict(bias=bias, relu=True, out_scale=S, out_zp=Z, out_qmin=0, out_qmax=255, out_offset=-128, w_zp=zw)
+    for mode in (_ops.OUT_F32, _ops.OUT_F16, _ops.OUT_REQUANT_I8, _ops.OUT_FAKEQUANT_F32):
+        got = _ops.qlinear_i8(ad, wd, out_mode=mode, **dkw).numpy()
+        exp = O.qlinear(a, w, za, a_scale, w_scale, out_mode=mode, **okw)
+        assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), mode
+    # raw accumulators are unchanged by the zero points
+    acc = _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, w_zp=hip(zw), wsum=_ops.rowsum_i8(wd), path=path)
+    assert np.array_equal(acc.numpy(), O.igemm(a, w))
+
+
+def test_affine_weights_with_device_zero_point_residual_and_join():
+    """The corrections compose with the other epilogue operands: a zero point that lives on
+    the device (dynamic quantization), a float residual, a GELU, and the join on codes."""
+    rng = np.random.default_rng(77)
+    M, N, K = 70, 96, 320
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    zw = rng.integers(-100, 100, N).astype(np.int32)
+    a_scale, w_scale = np.float32(0.02), rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    ad, wd = hip(a), hip(w)
+    wsum = _ops.rowsum_i8(wd)
+    # effective zero point = int(*a_zp_dev) + a_zp = 133 - 128
+    got = _ops.qlinear_i8(ad, wd, a_zp=-128, a_zp_dev=hip(np.float32(133.0)), a_scale=hip(a_scale),
+                          w_scale=hip(w_scale), wsum=wsum, bias=hip(bias), residual=hip(res), w_zp=hip(zw)).numpy()
+    exp = O.qlinear(a, w, 5, a_scale, w_scale, bias=bias, w_zp=zw) + res
+    assert np.array_equal(got.view(np.uint32), exp.astype(np.float32).view(np.uint32))
+    # the symmetric call with the same weights differs, so w_zp is really applied
+    sym = _ops.qlinear_i8(ad, wd, a_zp=5, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=wsum,
+                          bias=hip(bias)).numpy()
+    assert not np.array_equal(sym + res, got)
+    # join on codes: identical to the unfused pair on the affine layer's own codes
+    S1, Z1 = hip(np.float32(0.05)), hip(np.float32(120.0))
+    other = codes(rng, (M, N))
+    join = dict(q=hip(other), offset=-128, scale=hip(np.float32(0.04)), zp=hip(np.float32(131.0)), relu=True,
+                out_scale=hip(np.float32(0.06)), out_zp=hip(np.float32(0.0)), out_qmin=0, out_qmax=255,
+                out_offset=-128)
+    kw = dict(a_zp=5, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=wsum, bias=hip(bias),
+              out_mode=_ops.OUT_REQUANT_I8, out_scale=S1, out_zp=Z1, out_qmin=0, out_qmax=255, out_offset=-128)
+    fused_sym = _ops.qlinear_i8(ad, wd, join=join, **kw).numpy()
+    fused_aff = _ops.qlinear_i8(ad, wd, join=join, w_zp=hip(zw), **kw).numpy()
+    fused_zero = _ops.qlinear_i8(ad, wd, join=join, w_zp=hip(np.zeros(N, np.int32)), **kw).numpy()
+    assert np.array_equal(fused_zero, fused_sym)            # the two-pass route with zw = 0 is the one-pass result
+    assert not np.array_equal(fused_aff, fused_sym)
+    # fused_aff against the oracle composition: layer codes, then add_relu_requant
+    c1 = O.qlinear(a, w, 5, a_scale, w_scale, bias=bias, out_mode=O.OUT_REQUANT_I8, out_scale=0.05, out_zp=120.0,
+                   out_offset=-128, w_zp=zw)
+    exp = O.add_requant(c1, -128, 0.05, 120.0, other, -128, 0.04, 131.0, True, 0.06, 0.0, 0, 255, -128)
+    assert np.array_equal(fused_aff, exp)
+
+
+def test_affine_weights_reject_what_they_cannot_do():
+    rng = np.random.default_rng(1)
+    a, w = hip(codes(rng, (4, 64))), hip(codes(rng, (8, 64)))
+    zw = hip(np.ones(8, np.int32))
+    one = hip(np.float32(1.0))
+    with pytest.raises(ValueError, match="row sums"):
+        _ops.qlinear_i8(a, w, a_scale=one, w_scale=hip(np.ones(8, np.float32)), w_zp=zw)
+    with pytest.raises(L.ShapeMismatch):
+        _ops.qlinear_i8(a, w, a_scale=one, w_scale=hip(np.ones(8, np.float32)), wsum=_ops.rowsum_i8(w),
+                        w_zp=hip(np.ones(7, np.int32)))

@@ -285,3 +285,107 @@ def test_maxpool_on_codes_commutes_with_quantize():
     xt = torch.from_numpy(O.dequantize(q, s, z, code_offset=-128).transpose(0, 3, 1, 2).copy())
     ref = torch.nn.functional.max_pool2d(xt, 3, 2, 1).numpy().transpose(0, 2, 3, 1)
     assert np.array_equal(O.dequantize(pooled, s, z, code_offset=-128), ref)
+
+
+# ------------------------------------------------------------------ affine weights
+def _affine_weight_case(rng, N, K):
+    """Per-channel affine int8 weight codes the way from_float makes them: min / max per row,
+    affine qparams on [-128, 127], quantize."""
+    wf = (rng.standard_normal((N, K)) * 0.1 + rng.uniform(-0.15, 0.15, (N, 1))).astype(np.float32)
+    mn, mx = O.minmax(wf, ch_axis=0)
+    ws, wz = O.calc_qparams(mn, mx, False, -128, 127, True)
+    wq = O.quantize(wf, ws, wz, -128, 127, ch_axis=0)
+    return wf, wq, ws, wz
+
+
+@pytest.mark.parametrize("M,N,K", [(5, 7, 3), (33, 20, 147), (16, 48, 512)])
+def test_affine_weight_linear_is_the_exact_integer_sum(M, N, K):
+    """Accumulator under the scales = sum_k (a - za) * (w - zw[n]), checked through the
+    float32 output against an int64 numpy evaluation put through the same float steps, and
+    through the correction identity that the GPU path uses."""
+    rng = np.random.default_rng(M * N + K)
+    a, w = _codes(rng, (M, K)), _codes(rng, (N, K))
+    zw = rng.integers(-128, 128, N).astype(np.int32)
+    za = -37
+    a_scale = np.float32(0.0173)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    got = O.qlinear(a, w, za, a_scale, w_scale, bias=bias, out_mode=O.OUT_F32, w_zp=zw)
+    eff = (a.astype(np.int64) - za) @ (w.astype(np.int64) - zw[:, None]).T
+    exp = eff.astype(np.float32) * (a_scale * w_scale)[None, :] + bias[None, :]
+    assert np.array_equal(got.view(np.uint32), exp.astype(np.float32).view(np.uint32))
+    # acc - za*wsum - zw*asum + K*za*zw is the same integer
+    acc = O.igemm(a, w).astype(np.int64)
+    ident = (acc - za * w.astype(np.int64).sum(1)[None, :] - zw[None, :] * a.astype(np.int64).sum(1)[:, None]
+             + K * za * zw[None, :].astype(np.int64))
+    assert np.array_equal(ident, eff)
+    # zero weight zero points: the symmetric function, bit for bit, in every output form
+    for mode in (O.OUT_F32, O.OUT_F16, O.OUT_REQUANT_I8, O.OUT_FAKEQUANT_F32):
+        kw = dict(bias=bias, relu=True, out_mode=mode, out_scale=0.05, out_zp=3.0, out_offset=-128)
+        y0 = O.qlinear(a, w, za, a_scale, w_scale, **kw)
+        y1 = O.qlinear(a, w, za, a_scale, w_scale, w_zp=np.zeros(N, np.int32), **kw)
+        assert np.array_equal(y0.view(np.uint8), y1.view(np.uint8))
+
+
+def test_affine_weight_linear_special_cases():
+    rng = np.random.default_rng(8)
+    M, N, K = 9, 6, 40
+    a = _codes(rng, (M, K))
+    zw = np.array([-128, -5, 0, 17, 127, 64], np.int32)
+    # every code equal to its row's zero point = an all-zero float weight: output == bias
+    w = np.repeat(zw.astype(np.int8)[:, None], K, axis=1)
+    bias = rng.standard_normal(N).astype(np.float32)
+    y = O.qlinear(a, w, 11, 0.02, np.full(N, 0.003, np.float32), bias=bias, w_zp=zw)
+    assert np.array_equal(y, np.broadcast_to(bias, (M, N)))
+    # every activation code equal to its zero point = an all-zero input: output == bias
+    w = _codes(rng, (N, K))
+    y = O.qlinear(np.full((M, K), 11, np.int8), w, 11, 0.02, np.full(N, 0.003, np.float32), bias=bias, w_zp=zw)
+    assert np.array_equal(y, np.broadcast_to(bias, (M, N)))
+    # raw accumulators ignore both zero points
+    assert np.array_equal(O.qlinear(a, w, 11, 1.0, np.ones(N, np.float32), out_mode=O.OUT_ACC_I32, w_zp=zw),
+                          O.igemm(a, w))
+
+
+def test_affine_weight_linear_tracks_lucids_float_path():
+    """Against the float restatement of Lucid's composite (dequantize the affine weight, float
+    GEMM, lucid/nn/quantized/linear.py:199-215), which takes the weight zero points itself."""
+    rng = np.random.default_rng(21)
+    M, N, K = 32, 40, 256
+    wf, wq, ws, wz = _affine_weight_case(rng, N, K)
+    assert np.any(wz != 0)
+    x = rng.uniform(-1, 2, (M, K)).astype(np.float32)
+    mn, mx = O.minmax(x)
+    xs, xz = O.calc_qparams(mn, mx, False, 0, 255, False)
+    xq = O.quantize(x, xs, xz, 0, 255, code_offset=-128)
+    xg = O.fake_quantize(x, xs, xz, 0, 255)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    y_int = O.qlinear(xq, wq, int(xz[0]) - 128, xs, ws, bias=bias, w_zp=wz.astype(np.int32))
+    y_ref = O.linear_faithful(xg, wq, ws, wz, bias=bias)
+    assert np.abs(y_int - y_ref).max() <= 1e-3 * np.abs(y_ref).max()
+    # and ignoring the zero points is visibly wrong, so the check above has teeth
+    y_sym = O.qlinear(xq, wq, int(xz[0]) - 128, xs, ws, bias=bias)
+    assert np.abs(y_sym - y_ref).max() > 0.05 * np.abs(y_ref).max()
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_affine_weight_conv_is_the_exact_integer_sum(case):
+    B, H, W, Cin, Cout, KH, KW, st, pad, dil, groups = case
+    rng = np.random.default_rng(5 + sum(case[:7]))
+    x = _codes(rng, (B, H, W, Cin))
+    w = _codes(rng, (Cout, KH, KW, Cin // groups))
+    zw = rng.integers(-128, 128, Cout).astype(np.int32)
+    za = 23
+    a_scale = np.float32(0.021)
+    w_scale = rng.uniform(0.0005, 0.004, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    got = O.qconv2d(x, w, za, a_scale, w_scale, stride=st, pad=pad, dilation=dil, groups=groups,
+                    bias=bias, out_mode=O.OUT_F32, w_zp=zw)
+    # (x - za) conv (w - zw) with true zero padding, by the numpy accumulator on shifted operands
+    eff = _np_conv_acc(x.astype(np.int64) - za, w.astype(np.int64) - zw[:, None, None, None], st, pad, dil,
+                       groups, 0)
+    exp = eff.astype(np.float32) * (a_scale * w_scale) + bias
+    assert np.array_equal(got.view(np.uint32), exp.astype(np.float32).view(np.uint32))
+    y0 = O.qconv2d(x, w, za, a_scale, w_scale, stride=st, pad=pad, dilation=dil, groups=groups, bias=bias)
+    y1 = O.qconv2d(x, w, za, a_scale, w_scale, stride=st, pad=pad, dilation=dil, groups=groups, bias=bias,
+                   w_zp=np.zeros(Cout, np.int32))
+    assert np.array_equal(y0.view(np.uint32), y1.view(np.uint32))
