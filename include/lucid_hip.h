@@ -205,6 +205,58 @@ int lq_probe_mfma_i8(const int8_t* a, const int8_t* b, size_t nbytes, int iters,
  * workload for hardware-counter scaling. */
 int lq_copy_kernel(void* dst, const void* src, size_t nbytes, lq_stream stream);
 
+/* ---------------------------------------------------------- engine primitives */
+/* The IBackend calls that Lucid's quantization composites are written in, one kernel
+ * each, on contiguous device buffers of n elements - what an unmodified
+ * clip(round(x / s) + z, qmin, qmax).to(int8) (lucid/quantization/_functional.py:180),
+ * (q.to(float32) - z) * s (_functional.py:281) or an observer's min / max dispatches to
+ * when its tensors live on this device.  The fused lq_quantize / lq_dequantize /
+ * lq_fake_quantize / lq_minmax give the same bits in one pass and are what the modules
+ * use; these are the slow, call-for-call route and the specification of the fused ones.
+ *   lq_add/sub/mul/div_f32     IBackend::add/sub/mul/div (IBackend.h:370-373; IEEE float32,
+ *                              division as vDSP_vdiv, Vdsp.cpp:47-48); lq_add_f32 is declared
+ *                              with the float32 network kernels below
+ *   lq_maximum/minimum_f32     IBackend::maximum/minimum (IBackend.h:433-434): a NaN in either
+ *                              operand gives NaN (vDSP_vmax / vDSP_vmin, Vdsp.cpp:140-151)
+ *   lq_round_f32               IBackend::round (IBackend.h:474): ties to even (vvnintf,
+ *                              Vforce.cpp:136)
+ *   lq_clip_f32                IBackend::clip (IBackend.h:1232): bounds cast to float, NaN
+ *                              passes through (CpuBackend.h:6880-6891)
+ *   lq_astype                  IBackend::astype / cast (IBackend.h:2121,1235): static_cast
+ *                              between LQ_I8 / I16 / I32 / F16 / F32 (CpuBackend.h:6214-6236);
+ *                              float -> integer saturates at int32 and maps NaN to 0 (both
+ *                              undefined in C), then truncates to the width
+ *   lq_broadcast_f32           the materialised broadcast of a per-channel operand,
+ *                              out[o,c,i] = src[c] (kernel/BinaryKernel.h:591-606)
+ *   lq_reduce_minmax           IBackend::reduce_min + reduce_max over `axes` (IBackend.h:689-692;
+ *                              n_axes == 0 reduces everything), NaN-propagating
+ *                              (Reduce.cpp:87-125); mn / mx hold one float per kept
+ *                              element in row-major order.  The reduced axes must merge into
+ *                              one run of neighbouring dimensions or into the two ends of
+ *                              the shape (every call the observers make does);
+ *                              LQ_ERR_NOT_IMPLEMENTED otherwise. */
+int lq_sub_f32(const float* a, const float* b, float* out, size_t n, lq_stream stream);
+int lq_mul_f32(const float* a, const float* b, float* out, size_t n, lq_stream stream);
+int lq_div_f32(const float* a, const float* b, float* out, size_t n, lq_stream stream);
+int lq_maximum_f32(const float* a, const float* b, float* out, size_t n, lq_stream stream);
+int lq_minimum_f32(const float* a, const float* b, float* out, size_t n, lq_stream stream);
+int lq_round_f32(const float* x, float* out, size_t n, lq_stream stream);
+int lq_clip_f32(const float* x, float* out, size_t n, double min_v, double max_v, lq_stream stream);
+int lq_astype(const void* src, int src_dtype, void* dst, int dst_dtype, size_t n, lq_stream stream);
+int lq_broadcast_f32(const float* src, float* out, size_t outer, size_t C, size_t inner, lq_stream stream);
+int lq_reduce_minmax(const float* x, const int64_t* shape, int ndim, const int* axes, int n_axes, float* mn,
+                     float* mx, lq_stream stream);
+
+/* Eval-mode BatchNorm forward on (B, C, spatial) float32 (1-d / 2-d / 3-d alike):
+ *     rstd[c] = 1 / float(sqrt(double(var[c]) + eps))
+ *     y       = gamma[c] * (x - mean[c]) * rstd[c] + beta[c]        (float32, in that order)
+ * IBackend::batch_norm_eval_forward (CpuBackend.h:9163-9208), what F.batch_norm runs when
+ * not training (lucid/nn/functional/normalization.py:104-109).  gamma / beta NULL = 1 / 0.
+ * It lets an un-fused conv + BN model run on the device, e.g. to check fuse_modules
+ * against it (lucid/test/unit/quantization/test_static_ptq.py:90-99). */
+int lq_batchnorm_eval_f32(const float* x, float* out, size_t B, int C, size_t spatial, const float* mean,
+                          const float* var, const float* gamma, const float* beta, double eps, lq_stream stream);
+
 /* ------------------------------------------------------------ quantize family */
 /* min and max over everything but the channel axis, NaN-propagating.
  * Replaces reduce_min/reduce_max (IBackend.h:689-692; CpuBackend.h:12012,

@@ -173,6 +173,14 @@ _SIGNATURES["lq_wq_dequantize"] = [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]
 _SIGNATURES["lq_wq_matmul"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp]
 _SIGNATURES["lq_bias_act_f32"] = [_vp, _vp, _sz, _i, _i, _vp]
 _SIGNATURES["lq_rowsum_i8"] = [_vp, _vp, _i, _i, _vp]
+for _name in ("sub", "mul", "div", "maximum", "minimum"):
+    _SIGNATURES[f"lq_{_name}_f32"] = [_vp, _vp, _vp, _sz, _vp]
+_SIGNATURES["lq_round_f32"] = [_vp, _vp, _sz, _vp]
+_SIGNATURES["lq_clip_f32"] = [_vp, _vp, _sz, C.c_double, C.c_double, _vp]
+_SIGNATURES["lq_astype"] = [_vp, _i, _vp, _i, _sz, _vp]
+_SIGNATURES["lq_broadcast_f32"] = [_vp, _vp, _sz, _sz, _sz, _vp]
+_SIGNATURES["lq_reduce_minmax"] = [_vp, C.POINTER(C.c_int64), _i, C.POINTER(C.c_int), _i, _vp, _vp, _vp]
+_SIGNATURES["lq_batchnorm_eval_f32"] = [_vp, _vp, _sz, _i, _sz, _vp, _vp, _vp, _vp, C.c_double, _vp]
 _SIGNATURES["lq_qlinear_i8"] = [C.POINTER(QLinearArgs), _vp]
 _SIGNATURES["lq_qlinear_i8_n"] = [C.POINTER(QLinearArgs), _i, _vp]
 

@@ -31,6 +31,7 @@ from ._tensor import (
     synchronize,
     tensor,
 )
+from ._engine_ops import (add, amax, amin, clip, div, maximum, minimum, mul, round, sub)  # noqa: A004
 from . import quantization
 from . import nn
 from . import backends

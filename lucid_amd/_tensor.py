@@ -217,12 +217,15 @@ class Tensor:
         return out
 
     def to(self, target) -> "Tensor":
-        """``.to("hip")`` / ``.to("cpu")`` (``lucid/_tensor/_to.py:125-199``).
-        Dtype conversion is not part of this path and is rejected."""
+        """``.to("hip")`` / ``.to("cpu")`` (``lucid/_tensor/_to.py:125-199``), or ``.to(dtype)``:
+        the engine's ``astype`` on the device, numpy's on the host."""
         if isinstance(target, dtype):
             if target == self.dtype:
                 return self
-            raise NotImplementedError("dtype conversion is outside the hip quantized path")
+            if self.device == "cpu":
+                return Tensor(self.shape, target, "cpu", host=self._host.astype(target.np))
+            from ._engine_ops import astype
+            return astype(self, target)
         dev = _norm_device(target)
         if dev == self.device:
             return self
@@ -302,6 +305,51 @@ class Tensor:
 
     def detach(self) -> "Tensor":
         return self
+
+    # -- arithmetic: one engine call per operator, on float32 device tensors
+    def __add__(self, other):
+        from . import _engine_ops as E
+        return E.add(self, other)
+
+    __radd__ = __add__
+
+    def __sub__(self, other):
+        from . import _engine_ops as E
+        return E.sub(self, other)
+
+    def __rsub__(self, other):
+        from . import _engine_ops as E
+        return E.sub(other, self)
+
+    def __mul__(self, other):
+        from . import _engine_ops as E
+        return E.mul(self, other)
+
+    __rmul__ = __mul__
+
+    def __truediv__(self, other):
+        from . import _engine_ops as E
+        return E.div(self, other)
+
+    def __rtruediv__(self, other):
+        from . import _engine_ops as E
+        return E.div(other, self)
+
+    def min(self, dim=None, keepdim: bool = False) -> "Tensor":
+        from . import _engine_ops as E
+        return E.amin(self, dim, keepdim)
+
+    def max(self, dim=None, keepdim: bool = False) -> "Tensor":
+        from . import _engine_ops as E
+        return E.amax(self, dim, keepdim)
+
+    def round(self) -> "Tensor":
+        from . import _engine_ops as E
+        return E.round(self)
+
+    def clip(self, min_v, max_v) -> "Tensor":
+        from . import _engine_ops as E
+        return E.clip(self, min_v, max_v)
 
     def clone(self) -> "Tensor":
         if self.device == "cpu":

@@ -141,9 +141,23 @@ class Conv1d(Module):
             rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
 
     def forward(self, x):
-        raise NotImplementedError(
-            "float nn.Conv1d.forward is not part of the hip quantized-inference backend; "
-            "quantize the model (convert) first")
+        """Float32 convolution on the device: the 2-d kernel on a one-row image."""
+        if not isinstance(x, Tensor) or x.device != "hip":
+            raise NotImplementedError(
+                "float nn.Conv1d.forward runs on the 'hip' device only; the CPU float path is Lucid's")
+        if self.padding_mode != "zeros" or self._padding_str == "same":
+            raise NotImplementedError("float nn.Conv1d.forward: zero padding with a number (or 'valid') only")
+        if x.ndim != 3 or x.shape[1] != self.in_channels:
+            raise _C.ShapeMismatch(f"Conv1d: expected (B, {self.in_channels}, L), got {x.shape}")
+        from .functional import conv2d_f32
+        B, Cc, Ln = x.shape
+        w = self.weight if self.weight.device == "hip" else self.weight.to("hip")
+        b = self.bias
+        if b is not None and b.device != "hip":
+            b = b.to("hip")
+        y = conv2d_f32(x.reshape(B, Cc, 1, Ln), w.reshape(self.out_channels, Cc // self.groups, 1, self.kernel_size),
+                       b, (1, self.stride), (0, self.padding), (1, self.dilation), self.groups)
+        return y.reshape(B, self.out_channels, y.shape[3])
 
 
 class Conv3d(Module):
@@ -173,22 +187,51 @@ class Conv3d(Module):
             "quantize the model (convert) first")
 
 
-class BatchNorm2d(Module):
-    """Float BatchNorm2d as a parameter / statistics holder (folded into the
-    preceding convolution by ``fuse_modules`` before quantization)."""
+class _BatchNorm(Module):
+    """Float BatchNorm: the parameter / statistics holder that ``fuse_modules`` folds into the
+    preceding convolution, and the eval-mode forward on the device
+    (``lucid/nn/modules/normalization.py`` ``_BatchNormBase``; ``F.batch_norm`` with
+    ``training=False``).  Training-mode statistics are Lucid's."""
 
-    def __init__(self, num_features: int, eps: float = 1e-5, affine: bool = True) -> None:
+    _ndim = (4,)
+
+    def __init__(self, num_features: int, eps: float = 1e-5, momentum: float = 0.1, affine: bool = True) -> None:
         super().__init__()
-        self.num_features, self.eps, self.affine = num_features, eps, affine
+        self.num_features, self.eps, self.momentum, self.affine = num_features, eps, momentum, affine
         self.register_buffer("weight", T.tensor(np.ones(num_features, np.float32)) if affine else None)
         self.register_buffer("bias", T.tensor(np.zeros(num_features, np.float32)) if affine else None)
         self.register_buffer("running_mean", T.tensor(np.zeros(num_features, np.float32)))
         self.register_buffer("running_var", T.tensor(np.ones(num_features, np.float32)))
 
     def forward(self, x):
-        raise NotImplementedError(
-            "float nn.BatchNorm2d.forward is not part of the hip quantized-inference backend; "
-            "fold it into the convolution with quantization.fuse_modules")
+        if getattr(self, "training", False):
+            raise NotImplementedError(
+                f"float nn.{type(self).__name__}.forward in training mode (batch statistics) is Lucid's; "
+                "call .eval() - the hip backend runs the frozen-statistics forward")
+        if not isinstance(x, Tensor) or x.device != "hip":
+            raise NotImplementedError(
+                f"float nn.{type(self).__name__}.forward runs on the 'hip' device only; the CPU float path is Lucid's")
+        if x.ndim not in self._ndim or x.shape[1] != self.num_features:
+            raise _C.ShapeMismatch(f"{type(self).__name__}: expected {self._ndim}-d input with "
+                                   f"{self.num_features} channels, got {x.shape}")
+        from .._engine_ops import batch_norm_eval
+        return batch_norm_eval(x, self.running_mean, self.running_var, self.weight if self.affine else None,
+                               self.bias if self.affine else None, self.eps)
+
+    def extra_repr(self) -> str:
+        return f"{self.num_features}, eps={self.eps}, affine={self.affine}"
+
+
+class BatchNorm1d(_BatchNorm):
+    _ndim = (2, 3)
+
+
+class BatchNorm2d(_BatchNorm):
+    _ndim = (4,)
+
+
+class BatchNorm3d(_BatchNorm):
+    _ndim = (5,)
 
 
 def relu(x: Tensor) -> Tensor:

@@ -28,3 +28,11 @@ class LinearReLU(_Fused):
 
 class ConvReLU2d(_Fused):
     """``Conv2d`` followed by ``ReLU``."""
+
+
+class ConvReLU1d(_Fused):
+    """``Conv1d`` followed by ``ReLU``."""
+
+
+class ConvReLU3d(_Fused):
+    """``Conv3d`` followed by ``ReLU``."""

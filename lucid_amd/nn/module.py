@@ -99,8 +99,11 @@ class Module:
         """Called after a buffer was replaced by ``load_state_dict``."""
 
     def eval(self) -> "Module":
+        return self.train(False)
+
+    def train(self, mode: bool = True) -> "Module":
         for m in self.modules():
-            object.__setattr__(m, "training", False)
+            object.__setattr__(m, "training", bool(mode))
         return self
 
     def to(self, device) -> "Module":

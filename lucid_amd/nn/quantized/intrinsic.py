@@ -3,7 +3,7 @@ before the output requantize, inside the kernel epilogue."""
 
 from __future__ import annotations
 
-from .conv import Conv2d
+from .conv import Conv1d, Conv2d, Conv3d
 from .linear import Linear
 
 
@@ -46,3 +46,33 @@ class ConvReLU2d(Conv2d):
         inner.qconfig = mod.qconfig
         inner.activation_post_process = mod.activation_post_process
         return super().from_float(inner)
+
+
+def _unwrap_fused(mod):
+    """The weighted layer of a fused float pair, carrying the pair's qconfig and observer."""
+    if not hasattr(mod, "__getitem__"):
+        return mod
+    inner = mod[0]
+    inner.qconfig = mod.qconfig
+    inner.activation_post_process = mod.activation_post_process
+    return inner
+
+
+class ConvReLU1d(Conv1d):
+    """Quantized ``Conv1d`` + ``ReLU`` (``intrinsic.py:141-240``)."""
+
+    _fused_relu = True
+
+    @classmethod
+    def from_float(cls, mod) -> "ConvReLU1d":
+        return super().from_float(_unwrap_fused(mod))
+
+
+class ConvReLU3d(Conv3d):
+    """Quantized ``Conv3d`` + ``ReLU`` (``intrinsic.py:344-440``)."""
+
+    _fused_relu = True
+
+    @classmethod
+    def from_float(cls, mod) -> "ConvReLU3d":
+        return super().from_float(_unwrap_fused(mod))

@@ -19,18 +19,19 @@ from ... import _tensor as T
 
 def fuse_conv_bn_eval(conv, bn):
     """Return a copy of ``conv`` with ``bn``'s inference-time affine folded in."""
-    from .. import BatchNorm2d, Conv2d
+    from .. import BatchNorm1d, BatchNorm2d, BatchNorm3d, Conv1d, Conv2d, Conv3d
 
-    if not isinstance(conv, Conv2d):
-        raise TypeError(f"fuse_conv_bn_eval: conv must be Conv2d, got {type(conv).__name__}")
-    if not isinstance(bn, BatchNorm2d):
-        raise TypeError(f"fuse_conv_bn_eval: bn must be BatchNorm2d, got {type(bn).__name__}")
+    if not isinstance(conv, (Conv1d, Conv2d, Conv3d)):
+        raise TypeError(f"fuse_conv_bn_eval: conv must be Conv1d/2d/3d, got {type(conv).__name__}")
+    if not isinstance(bn, (BatchNorm1d, BatchNorm2d, BatchNorm3d)):
+        raise TypeError(f"fuse_conv_bn_eval: bn must be BatchNorm1d/2d/3d, got {type(bn).__name__}")
     fused = copy.deepcopy(conv)
     eps = np.float32(bn.eps)
     mean = bn.running_mean.numpy().astype(np.float32)
     var = bn.running_var.numpy().astype(np.float32)
-    gamma = bn.weight.numpy().astype(np.float32) if bn.weight is not None else None
-    beta = bn.bias.numpy().astype(np.float32) if bn.bias is not None else None
+    affine = getattr(bn, "affine", True)
+    gamma = bn.weight.numpy().astype(np.float32) if affine and bn.weight is not None else None
+    beta = bn.bias.numpy().astype(np.float32) if affine and bn.bias is not None else None
     inv_std = np.float32(1.0) / np.sqrt(var + eps)
     scale = inv_std if gamma is None else gamma * inv_std
     weight = fused.weight.numpy().astype(np.float32)

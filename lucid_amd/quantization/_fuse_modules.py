@@ -27,22 +27,32 @@ def _set(model, dotted: str, new) -> None:
     parent._modules[parts[-1]] = new
 
 
+_CONV_TYPES = (nn.Conv1d, nn.Conv2d, nn.Conv3d)
+_BN_TYPES = (nn.BatchNorm1d, nn.BatchNorm2d, nn.BatchNorm3d)
+
+
+def _conv_relu(conv, relu):
+    return {nn.Conv1d: nni.ConvReLU1d, nn.Conv2d: nni.ConvReLU2d, nn.Conv3d: nni.ConvReLU3d}[type(conv)](conv, relu)
+
+
 def _fuse_run(mods):
+    """Replacements for a fusible run: the fused module first, ``Identity`` for the rest
+    (``fuse_modules.py:60-84``)."""
     ids = [nn.Identity() for _ in range(len(mods) - 1)]
     first = mods[0]
-    if isinstance(first, nn.Conv2d):
+    if isinstance(first, _CONV_TYPES):
         rest = list(mods[1:])
         conv = first
-        if rest and isinstance(rest[0], nn.BatchNorm2d):
+        if rest and isinstance(rest[0], _BN_TYPES):
             conv = fuse_conv_bn_eval(first, rest.pop(0))
         if rest and isinstance(rest[0], nn.ReLU):
             rest.pop(0)
-            conv = nni.ConvReLU2d(conv, nn.ReLU())
+            conv = _conv_relu(conv, nn.ReLU())
         if not rest:
             return [conv, *ids]
     if isinstance(first, nn.Linear) and len(mods) == 2 and isinstance(mods[1], nn.ReLU):
         return [nni.LinearReLU(first, nn.ReLU()), *ids]
-    raise ValueError(f"fuse_modules: unsupported pattern {[type(m).__name__ for m in mods]}")
+    raise ValueError(f"fuse_modules: unsupported fusion pattern {[type(m).__name__ for m in mods]}")
 
 
 def fuse_modules(model, modules_to_fuse: Sequence[Sequence[str]], inplace: bool = False):

@@ -21,7 +21,7 @@ from .qconfig import QConfig, get_default_qconfig
 
 
 def _observed_types() -> tuple[type, ...]:
-    return (nn.Linear, nn.Conv1d, nn.Conv2d, nn.Conv3d, nni.LinearReLU, nni.ConvReLU2d, nnq.QuantStub,
+    return (nn.Linear, nn.Conv1d, nn.Conv2d, nn.Conv3d, nni.LinearReLU, nni.ConvReLU1d, nni.ConvReLU2d, nni.ConvReLU3d, nnq.QuantStub,
             nnq.FloatFunctional, nn.ConvTranspose1d, nn.ConvTranspose2d, nn.ConvTranspose3d, nn.Sigmoid, nn.Hardswish, nn.Hardsigmoid, nn.Tanh, nn.ELU, nn.LeakyReLU)
 
 
@@ -49,6 +49,8 @@ def _quant_mapping() -> dict[type, object]:
         m[nn.Conv1d] = nnq.Conv1d.from_float
         m[nn.Conv3d] = nnq.Conv3d.from_float
         m[nni.ConvReLU2d] = nnq.ConvReLU2d.from_float
+        m[nni.ConvReLU1d] = nnq.ConvReLU1d.from_float
+        m[nni.ConvReLU3d] = nnq.ConvReLU3d.from_float
     return m
 
 

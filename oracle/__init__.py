@@ -313,3 +313,16 @@ def maxpool2d_nhwc_i8(x, kernel, stride, pad):
     lib().orc_maxpool2d_nhwc_i8(_p(x), B, H, W, Cn, kernel[0], kernel[1], stride[0], stride[1],
                                 pad[0], pad[1], _p(out))
     return out
+
+
+def batchnorm_eval(x, mean, var, gamma=None, beta=None, eps=1e-5):
+    """Eval-mode BatchNorm on ``(B, C, *)`` float32 with frozen statistics."""
+    x = _f32(x)
+    B, Cn = x.shape[0], x.shape[1]
+    spatial = int(np.prod(x.shape[2:], dtype=np.int64))
+    out = np.empty_like(x)
+    g = None if gamma is None else _f32(gamma)
+    b = None if beta is None else _f32(beta)
+    lib().orc_batchnorm_eval(_p(x), _p(out), C.c_size_t(B), C.c_size_t(Cn), C.c_size_t(spatial),
+                             _p(_f32(mean)), _p(_f32(var)), _p(g), _p(b), C.c_double(eps))
+    return out

@@ -830,3 +830,22 @@ void orc_maxpool2d_nhwc_i8(const int8_t* x, int B, int H, int W, int C, int KH, 
                     out[(((size_t)b * OH + oh) * OW + ow) * C + c] = (int8_t)best;
                 }
 }
+
+/* ------------------------------------------------------------------ */
+/* Eval-mode BatchNorm forward, IBackend::batch_norm_eval_forward      */
+/* (lucid/_C/backend/cpu/CpuBackend.h:9163-9208): x is (B, C, spatial); */
+/*   rstd[c] = 1 / (float)sqrt((double)var[c] + eps)                   */
+/*   y       = g * (x - m) * r + b       float32, left to right        */
+/* gamma / beta NULL = ones / zeros (nn/functional/normalization.py:91-101). */
+void orc_batchnorm_eval(const float* x, float* y, size_t B, size_t C, size_t spatial,
+                        const float* mean, const float* var, const float* gamma,
+                        const float* beta, double eps) {
+    for (size_t b = 0; b < B; ++b)
+        for (size_t c = 0; c < C; ++c) {
+            const float r = 1.0f / (float)sqrt((double)var[c] + eps);
+            const float m = mean[c], g = gamma ? gamma[c] : 1.0f, bb = beta ? beta[c] : 0.0f;
+            const float* xr = x + (b * C + c) * spatial;
+            float* yr = y + (b * C + c) * spatial;
+            for (size_t s = 0; s < spatial; ++s) yr[s] = g * (xr[s] - m) * r + bb;
+        }
+}

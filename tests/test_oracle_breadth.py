@@ -198,3 +198,39 @@ def test_qconv_transpose3d_against_the_scatter_definition(stride, padding, outpu
                     xc[(slice(None), ci, *idx)][:, None] * w[(ci, slice(None), *tap)][None, :]
     want = full[(slice(None), slice(None), *[slice(p, p + n) for p, n in zip(padding, size)])]
     assert got.shape == want.shape and np.array_equal(got.astype(np.int64), want)
+
+
+# ------------------------------------------------------------------ eval-mode BatchNorm
+def test_batchnorm_eval_restates_the_reference_steps():
+    """rstd through double, then g * (x - m) * r + b in float32 left to right
+    (CpuBackend.h:9190-9198): pinned against the same steps in numpy float32, against torch's
+    batch_norm within rounding, and on closed forms a dropped or swapped term would break."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(0)
+    for shape in [(3, 5), (2, 4, 9), (2, 6, 7, 5), (2, 3, 4, 5, 6)]:
+        Cn = shape[1]
+        x = rng.standard_normal(shape).astype(np.float32) * 3
+        m = rng.standard_normal(Cn).astype(np.float32)
+        v = rng.uniform(0.1, 4.0, Cn).astype(np.float32)
+        g = rng.uniform(0.5, 1.5, Cn).astype(np.float32)
+        b = rng.standard_normal(Cn).astype(np.float32)
+        y = O.batchnorm_eval(x, m, v, g, b, 1e-5)
+        bc = (1, Cn) + (1,) * (len(shape) - 2)
+        r = (np.float32(1.0) / np.sqrt(v.astype(np.float64) + 1e-5).astype(np.float32)).astype(np.float32)
+        exp = ((g.reshape(bc) * (x - m.reshape(bc))).astype(np.float32) * r.reshape(bc)).astype(np.float32) \
+            + b.reshape(bc)
+        assert np.array_equal(y.view(np.uint32), exp.astype(np.float32).view(np.uint32))
+        t = torch.nn.functional.batch_norm(torch.from_numpy(x), torch.from_numpy(m), torch.from_numpy(v),
+                                           torch.from_numpy(g), torch.from_numpy(b), False, 0.0, 1e-5).numpy()
+        assert np.allclose(y, t, rtol=2e-6, atol=2e-6)
+        # no affine parameters = gamma 1, beta 0
+        assert np.array_equal(O.batchnorm_eval(x, m, v, None, None, 1e-5),
+                              O.batchnorm_eval(x, m, v, np.ones(Cn), np.zeros(Cn), 1e-5))
+    # mean 0, var 1 - eps, gamma 1, beta 0: the identity; x == mean: exactly beta
+    x = rng.standard_normal((2, 3, 8)).astype(np.float32)
+    one_minus = np.full(3, 1.0 - 1e-5, np.float64).astype(np.float32)
+    y = O.batchnorm_eval(x, np.zeros(3), one_minus, None, None, 1e-5)
+    assert np.allclose(y, x, rtol=1e-6)
+    y = O.batchnorm_eval(np.broadcast_to(np.float32([1, 2, 3])[None, :, None], (2, 3, 8)), [1, 2, 3], [4, 5, 6],
+                         [7, 8, 9], [0.5, -0.5, 0.25], 1e-5)
+    assert np.array_equal(y, np.broadcast_to(np.float32([0.5, -0.5, 0.25])[None, :, None], (2, 3, 8)))
