@@ -174,3 +174,32 @@ def test_failed_capture_releases_its_blocks():
     L.synchronize()
     assert np.all(y.numpy() == 1.0)
     g.destroy()
+
+
+def test_vit_b16_batch64_graph_replay_matches_eager():
+    """The serving configuration of the ViT bench: a captured forward of ViT-B/16 at batch 64
+    gives the eager logits bit for bit on every replay, for several batches, with eager work
+    and synchronisations in between (the dynamic quantizers' ranges live on the device, so
+    nothing in the forward talks to the host)."""
+    model = W.QViT(W.VIT_B16, seed=2)
+    rng = np.random.default_rng(9)
+    batches = [rng.uniform(0, 1, (64, 3, 224, 224)).astype(np.float32) for _ in range(3)]
+    x = L.tensor(batches[0], device="hip")
+    eager = []
+    for b in batches:
+        x.copy_from(b)
+        eager.append(model(x).numpy())
+    assert not np.array_equal(eager[0], eager[1])
+    with L.graph.capture() as g:
+        y = model(x)
+    for rep in range(2):
+        for i, b in enumerate(batches):
+            x.copy_from(b)
+            g.replay()
+            junk = model.blocks[0].fc1(L.tensor(rng.standard_normal((7, 768)).astype(np.float32), device="hip"))
+            L.synchronize()
+            assert junk.shape == (7, 3072)
+            assert np.array_equal(y.numpy().view(np.uint32), eager[i].view(np.uint32)), (rep, i)
+    g.destroy()
+    x.copy_from(batches[2])
+    assert np.array_equal(model(x).numpy().view(np.uint32), eager[2].view(np.uint32))

@@ -133,14 +133,16 @@ def test_vit_b16_block_stage_by_stage():
     assert np.array_equal(blk.fc2(hip(ge)).numpy(), V.dynamic_linear(ge, wq, ws, p[b + "fc2.bias"]))
 
 
-@pytest.mark.parametrize("cfg,batch", [(SMALL, 3), (workloads.VIT_B16, 2)])
-def test_vit_end_to_end_against_the_cpu_path(cfg, batch):
+# bound = twice the error measured on MI355X for that configuration (1.35e-7 and 1.82e-2)
+@pytest.mark.parametrize("cfg,batch,bound", [(SMALL, 3, 3e-7), (workloads.VIT_B16, 2, 3.7e-2)])
+def test_vit_end_to_end_against_the_cpu_path(cfg, batch, bound):
     """Free-running comparison.  A dynamic quantizer turns an input difference d
     (here float32 rounding order, 1e-7) into an RMS difference of sqrt(d * step)
     on the elements that cross a rounding tie, so after a few layers two correct
     implementations differ at the level of the quantization step itself
-    (~0.4 % of the activation range per layer); the bound below is that level,
-    not a rounding-error bound.  Stage-by-stage parity is the test above."""
+    (~0.4 % of the activation range per layer); the bound of the 12-layer model is that
+    level, not a rounding-error bound, while the 2-layer model stays at rounding level.
+    Stage-by-stage parity is the test above."""
     p = workloads.vit_float_params(cfg, seed=4)
     rng = np.random.default_rng(11)
     images = rng.uniform(0, 1, (batch, 3, cfg["image"], cfg["image"])).astype(np.float32)
@@ -150,7 +152,7 @@ def test_vit_end_to_end_against_the_cpu_path(cfg, batch):
     assert got.shape == exp.shape == (batch, cfg["classes"])
     err = rel(got, exp)
     print(f"ViT dim {cfg['dim']} depth {cfg['depth']} batch {batch}: end-to-end max error / max |logit| = {err:.2e}")
-    assert err < 4e-2
+    assert err < bound
 
 
 def _range_of(t):
