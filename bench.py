@@ -93,6 +93,21 @@ def time_launches(_C, fn, steps, warmup):
     return total, per
 
 
+def time_in_graph(L, _C, fn, steps, per_graph=20):
+    """Average milliseconds per call of `fn` when `per_graph` calls are captured into a HIP
+    graph and the graph is replayed `steps` times between one pair of events: the rate of
+    short kernels without the interpreter's gap between launches."""
+    fn()
+    with L.graph.capture() as g:
+        for _ in range(per_graph):
+            fn()
+    for _ in range(5):
+        g.replay()
+    total, _ = time_launches(_C, g.replay, steps, 2)
+    g.destroy()
+    return total / (steps * per_graph)
+
+
 def make_linear(L, Q, _C, _ops, M, K, N, seed):
     """Synthetic layer of the benchmark's shape, quantized on the device with
     the library's own kernels."""
@@ -163,6 +178,24 @@ def bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup, seed=1):
                 p95_ms=float(np.percentile(per, 95)), ops=ops, bytes=bytes_alg,
                 tops=ops / (total / steps) / 1e9, kernel_tops=ops / avg_ms / 1e9,
                 gbs=bytes_alg / avg_ms / 1e6, tensors=t)
+
+
+def bench_linear_cold_weights(L, _C, _ops, t, M, K, N, steps):
+    """The decode-shaped layer with weights that are NOT resident in the 256 MB last-level
+    cache: the launches cycle through enough copies of the weight matrix to exceed it, as the
+    layers of a real model do, replayed from a HIP graph so that no host gap is charged.
+    Returns the average microseconds per launch."""
+    copies = int(320e6 // (N * K)) + 2
+    ws = [t["wq"]] + [t["wq"].clone() for _ in range(copies - 1)]
+    with L.graph.capture() as g:
+        for w in ws:
+            _ops.qlinear_i8(t["xq"], w, a_scale=t["xs"], w_scale=t["ws"], bias=t["bias"],
+                            out_mode=_ops.OUT_F16, out=t["out"])
+    for _ in range(20):
+        g.replay()
+    total, _ = time_launches(_C, g.replay, steps, 3)
+    g.destroy()
+    return total / (steps * copies) * 1e3
 
 
 def probe_mfma_ceiling(L, _C, xq, wq, ms_target=40.0):
@@ -484,12 +517,16 @@ def bench_weight_only(L, _C, steps, warmup, K=4096, N=11008, gs=64):
         nbytes = N * K * bits // 8 + 2 * 4 * N * (K // gs)
         for m in (1, 16):
             x = L.tensor(rng.standard_normal((m, K)).astype(np.float32), device="hip")
-            fn = lambda: _qgemm.quantized_matmul(x, packed, scales, biases, True, gs, bits)
+            res = L.Tensor.empty((m, N), L.float32, "hip")
+            fn = lambda: _C.call("lq_wq_matmul", x.data_ptr, packed.data_ptr, scales.data_ptr, biases.data_ptr,
+                                 m, N, K, gs, bits, res.data_ptr, None)
+            # us: launches replayed back to back from a HIP graph (the kernel's own rate);
+            # bracketed_launch_median_us: each launch driven from Python between its own events
+            us = time_in_graph(L, _C, fn, max(10, steps // 2)) * 1e3
             _, per = time_launches(_C, fn, steps, warmup)
-            us = float(np.median(per)) * 1e3
             gbs = nbytes / (us * 1e-6) / 1e9
-            out[f"w{bits}_m{m}"] = {"us": round(us, 2), "GB/s": round(gbs, 1),
-                                    "frac_of_8TBs": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+            out[f"w{bits}_m{m}"] = {"us": round(us, 2), "bracketed_launch_median_us": round(float(np.median(per)) * 1e3, 2),
+                                    "GB/s": round(gbs, 1), "frac_of_8TBs": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
     return out
 
 
@@ -642,7 +679,7 @@ def main() -> int:
     ap.add_argument("--vendor-yardstick", action="store_true",
                     help="time the ROCm library's int8 GEMM (through torch._int_mm, if torch is importable) "
                          "on the same operand codes beside this library's; a yardstick, not a dependency")
-    ap.add_argument("--only", default=None, choices=["resnet50", "vit"],
+    ap.add_argument("--only", default=None, choices=["resnet50", "vit", "decode"],
                     help="run just this end-to-end leg and print its figures")
     ap.add_argument("--vendor-child", default=None, help=argparse.SUPPRESS)
     ap.add_argument("--no-extra", action="store_true")
@@ -685,6 +722,17 @@ def main() -> int:
         t = make_linear(L, Q, _C, _ops, M, K, N, 1)
         res["benchmark_codes"] = round(probe_mfma_ceiling(L, _C, t["xq"], t["wq"]), 1)
         print(json.dumps({"mfma_only_tops_by_operand_data": res, "datasheet_peak_tops": PEAK_INT8_TOPS}))
+        return 0
+    if args.only == "decode":
+        # the decode-shaped (HBM-bound) Linears alone: int8 at M = 1 / 16 and weight-only int4 / int8
+        res = {}
+        for m in (1, 16):
+            rs = bench_linear(L, Q, _C, _ops, m, K, N, args.steps, args.warmup, seed=3)
+            cold_us = bench_linear_cold_weights(L, _C, _ops, rs["tensors"], m, K, N, max(10, args.steps // 2))
+            res[f"linear_m{m}"] = {"us": round(rs["avg_kernel_ms"] * 1e3, 2), "frac_of_8TBs": round(rs["gbs"] / PEAK_HBM_GBS, 4),
+                                   "cold_weights_us": round(cold_us, 2)}
+        res["weight_only_group64_k4096_n11008"] = bench_weight_only(L, _C, args.steps, args.warmup)
+        print(json.dumps(res))
         return 0
     if args.only:
         # one of the end-to-end legs alone (a clean kernel trace of one network)
@@ -762,10 +810,16 @@ def main() -> int:
             rs = bench_linear(L, Q, _C, _ops, m, K, N, args.steps, args.warmup, seed=3)
             # us / GB/s: average of back-to-back launches between one pair of events (as the
             # headline); the median of individually bracketed launches, event cost included, beside it
+            # cold_*: the same launches cycling through weight copies that exceed the last-level
+            # cache, i.e. every byte from HBM (the back-to-back figure re-reads one 45 MB matrix,
+            # which stays in the 256 MB cache between launches)
+            cold_us = bench_linear_cold_weights(L, _C, _ops, rs["tensors"], m, K, N, max(10, args.steps // 2))
             extra[f"linear_m{m}"] = {"us": round(rs["avg_kernel_ms"] * 1e3, 2),
                                      "bracketed_launch_median_us": round(rs["median_ms"] * 1e3, 2),
                                      "GB/s": round(rs["gbs"], 1),
                                      "frac_of_8TBs": round(rs["gbs"] / PEAK_HBM_GBS, 4),
+                                     "cold_weights_us": round(cold_us, 2),
+                                     "cold_weights_frac_of_8TBs": round(rs["bytes"] / cold_us / 1e3 / PEAK_HBM_GBS, 4),
                                      "TOP/s": round(rs["kernel_tops"], 2), "bytes": rs["bytes"]}
             del rs["tensors"]
         # the same layer at a prefill-sized M: more tiles per CU, better-filled rounds

@@ -387,6 +387,163 @@ __global__ __launch_bounds__(256) void qgemm_skinny_kernel(GemmArgs g) {
         }
 }
 
+// ---------------------------------------------------------------- one activation row
+// M == 1: the weight matrix is read exactly once and nothing else of size moves, so the
+// kernel is a stream of 16-byte loads.  What the memory pipeline charges for is load
+// instructions, whatever their active lanes or bytes (measured: the same 45 MB through
+// 8-byte loads takes twice as long; an activation load with four active lanes costs as much
+// as a full one), so every weight instruction moves a full KiB of one row and the activation
+// row costs K / 1024 instructions per block: it is copied to LDS once and read from there.
+// A wavefront owns four consecutive rows and requests all of their bytes (16 loads for
+// K = 4096) before the first dot product; v_dot4_i32_i8 needs no operand layout, so there
+// is no transposition.  Sums over the 64 lanes are exact integer adds.
+__global__ __launch_bounds__(512) void qgemv1_kernel(GemmArgs g) {
+    extern __shared__ int8_t a_lds[];  // K bytes rounded up to a multiple of 4 KiB
+    constexpr int RW = 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const int kchunks = (g.K + 4095) / 4096;
+    // the activation row is requested first: loads return in order
+    for (int k = tid * 16; k < kchunks * 4096; k += blockDim.x * 16) {
+        const v4i v = k < g.K ? *reinterpret_cast<const v4i*>(g.a + k) : v4i{0, 0, 0, 0};
+        *reinterpret_cast<v4i*>(a_lds + k) = v;
+    }
+    float S = 1.0f, Z = 0.0f;
+    if (g.out_mode == OUT_REQUANT_I8 || g.out_mode == OUT_FAKEQUANT_F32) {
+        S = g.out_scale[0];
+        Z = g.out_zp[0];
+    }
+    const float as = g.a_scale ? g.a_scale[0] : 1.0f;
+    const int nb = (blockIdx.x * waves + wave) * RW;
+    // lane r finishes row nb + r: its column operands are requested before the weights
+    const int n_mine = nb + (lane < RW ? lane : 0);
+    ColParams cp{1.0f, -0.0f, 0};
+    if (lane < RW && n_mine < g.N) cp = load_col(g, n_mine);
+
+    int acc[RW];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) acc[r] = 0;
+    for (int kc = 0; kc < kchunks; ++kc) {
+        v4i wv[RW][4];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            const int n = nb + r;
+            const int8_t* row = g.w + size_t(n < g.N ? n : 0) * g.K;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int k = kc * 4096 + i * 1024 + lane * 16;
+                wv[r][i] = (n < g.N && k < g.K) ? *reinterpret_cast<const v4i*>(row + k) : v4i{0, 0, 0, 0};
+            }
+        }
+        if (kc == 0) __syncthreads();  // the activation row is in LDS (uniform: every wave runs chunk 0)
+        v4i av[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) av[i] = *reinterpret_cast<const v4i*>(a_lds + kc * 4096 + i * 1024 + lane * 16);
+#pragma unroll
+        for (int r = 0; r < RW; ++r)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[r] = __builtin_amdgcn_sdot4(wv[r][i].x, av[i].x, acc[r], false);
+                acc[r] = __builtin_amdgcn_sdot4(wv[r][i].y, av[i].y, acc[r], false);
+                acc[r] = __builtin_amdgcn_sdot4(wv[r][i].z, av[i].z, acc[r], false);
+                acc[r] = __builtin_amdgcn_sdot4(wv[r][i].w, av[i].w, acc[r], false);
+            }
+    }
+    // rotations inside each row of 16 lanes, then the four row totals through scalar registers
+    int mine = 0;
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        int v = acc[r];
+        v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false);
+        v += __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false);
+        v += __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false);
+        v += __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false);
+        v = __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) + __builtin_amdgcn_readlane(v, 32) +
+            __builtin_amdgcn_readlane(v, 48);
+        if (lane == r) mine = v;
+    }
+    if (lane < RW && n_mine < g.N) epilogue_store(g, 0, n_mine, mine, as, cp, S, Z);
+}
+
+// ---------------------------------------------------------------- up to 16 activation rows
+// 2 <= M <= 16, K >= 1024: one block of 16 wavefronts per compute unit's share of the rows
+// (rows_per_block <= 16 G), the wavefronts split the 256-byte K blocks.  A wavefront loads
+// the activation fragment of its K block once and uses it for all G row groups, so the
+// activation costs 4 load instructions per 4 G weight instructions instead of one per MFMA,
+// and all of a wavefront's weight bytes are requested before its first MFMA.  Partial sums
+// meet in LDS through integer atomic adds (order-independent, hence deterministic); the
+// wavefronts that finish early add theirs off the critical path.
+template <int G>
+__global__ __launch_bounds__(1024) void qgemm_skinny16_kernel(GemmArgs g, int rows_per_block) {
+    __shared__ int red[G * 4 * 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const int ln = lane & 15, lg = lane >> 4;
+    for (int i = tid; i < G * 4 * 64; i += blockDim.x) red[i] = 0;
+    const int n0 = blockIdx.x * rows_per_block;
+    const int n_end = n0 + rows_per_block < g.N ? n0 + rows_per_block : g.N;
+
+    // the epilogue's operands are requested first (wavefront j finishes row group j)
+    float S = 1.0f, Z = 0.0f, as_uniform = 1.0f;
+    ColParams cp{1.0f, -0.0f, 0};
+    const int n_mine = n0 + wave * 16 + ln;
+    if (wave < G && n_mine < n_end) {
+        if (g.out_mode == OUT_REQUANT_I8 || g.out_mode == OUT_FAKEQUANT_F32) {
+            S = g.out_scale[0];
+            Z = g.out_zp[0];
+        }
+        cp = load_col(g, n_mine);
+        as_uniform = g.a_scale ? g.a_scale[0] : 1.0f;
+    }
+    __syncthreads();  // the accumulators are zero before anyone adds to them
+
+    const int kblocks = (g.K + 255) / 256;
+    const bool m_ok = ln < g.M;
+    const int8_t* arow = g.a + size_t(m_ok ? ln : 0) * g.K;
+    v4i acc[G];
+#pragma unroll
+    for (int j = 0; j < G; ++j) acc[j] = v4i{0, 0, 0, 0};
+    for (int kb = wave; kb < kblocks; kb += waves) {
+        const int kbase = kb * 256 + lg * 16;
+        v4i af[4], wf[G][4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int k = kbase + c * 64;
+            af[c] = (m_ok && k < g.K) ? *reinterpret_cast<const v4i*>(arow + k) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < G; ++j) {
+            const int n = n0 + j * 16 + ln;
+            const int8_t* wrow = g.w + size_t(n < n_end ? n : n0) * g.K;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int k = kbase + c * 64;
+                wf[j][c] = (n < n_end && k < g.K) ? *reinterpret_cast<const v4i*>(wrow + k) : v4i{0, 0, 0, 0};
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int j = 0; j < G; ++j)
+                acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[c], wf[j][c], acc[j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < G; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            __hip_atomic_fetch_add(&red[(j * 4 + r) * 64 + lane], acc[j][r], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+    __syncthreads();
+    if (wave >= G || n_mine >= n_end) return;
+    // red[(j*4 + r)*64 + lane] is row 4*(lane>>4) + r of the activations, weight row n0 + 16 j + (lane&15)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int mm = 4 * lg + r;
+        if (mm < g.M) {
+            const float as = g.a_scale_per_row ? g.a_scale[mm] : as_uniform;
+            epilogue_store(g, mm, n_mine, red[(wave * 4 + r) * 64 + lane], as, cp, S, Z);
+        }
+    }
+}
+
 // ---------------------------------------------------------------- naive kernel
 __global__ __launch_bounds__(256) void qgemm_naive_kernel(GemmArgs g) {
     const size_t total = size_t(g.M) * g.N;
@@ -500,6 +657,30 @@ int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t 
         if (rc) return rc;
     } else if (path == 2) {
         LQ_REQUIRE(g.M <= 64, LQ_ERR_SHAPE, "qlinear_i8: skinny path needs M <= 64 (M = %d)", g.M);
+        if (g.M == 1 && g.K <= 65536) {
+            // four rows per wavefront; as many wavefronts per block (up to 8) as still leave 256 blocks
+            int waves = 8;
+            while (waves > 1 && (g.N + 4 * waves - 1) / (4 * waves) < 256) waves >>= 1;
+            const unsigned blocks = unsigned((g.N + 4 * waves - 1) / (4 * waves));
+            const size_t lds = size_t((g.K + 4095) / 4096) * 4096;
+            hipLaunchKernelGGL(qgemv1_kernel, dim3(blocks), dim3(waves * 64), lds, st, g);
+            LQ_CHECK_LAUNCH("qgemv1");
+            return LQ_OK;
+        }
+        if (g.M <= 16 && g.K >= 1024) {
+            int R = (g.N + 255) / 256;  // one block per compute unit when the rows allow it
+            R = R < 16 ? 16 : (R > 64 ? 64 : R);
+            const int G = (R + 15) / 16;
+            const dim3 grid16{unsigned((g.N + R - 1) / R)}, block16{1024};
+            switch (G) {
+            case 1: hipLaunchKernelGGL((qgemm_skinny16_kernel<1>), grid16, block16, 0, st, g, R); break;
+            case 2: hipLaunchKernelGGL((qgemm_skinny16_kernel<2>), grid16, block16, 0, st, g, R); break;
+            case 3: hipLaunchKernelGGL((qgemm_skinny16_kernel<3>), grid16, block16, 0, st, g, R); break;
+            default: hipLaunchKernelGGL((qgemm_skinny16_kernel<4>), grid16, block16, 0, st, g, R); break;
+            }
+            LQ_CHECK_LAUNCH("qgemm_skinny16");
+            return LQ_OK;
+        }
         dim3 grid{unsigned((g.N + 15) / 16)}, block{256};
         if (g.M <= 16)
             hipLaunchKernelGGL((qgemm_skinny_kernel<1>), grid, block, 0, st, g);

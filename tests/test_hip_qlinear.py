@@ -30,6 +30,12 @@ ACC_CASES = [
     (1, 11008, 4096, SKINNY), (16, 11008, 4096, SKINNY), (16, 1024, 4096, SKINNY),
     (3, 50, 48, SKINNY), (17, 33, 784, SKINNY), (33, 100, 272, SKINNY), (64, 256, 784, SKINNY),
     (64, 10, 256, SKINNY), (5, 7, 16, SKINNY),
+    # one activation row (dot-product kernel): ragged N, K tails, several 4 KiB chunks, few rows
+    (1, 50, 48, SKINNY), (1, 4096, 11008, SKINNY), (1, 77, 4112, SKINNY), (1, 3, 16, SKINNY), (1, 1031, 1024, SKINNY),
+    (1, 9000, 256, SKINNY), (1, 2, 65536, SKINNY),
+    # 2..16 rows with K >= 1024 (one block per compute unit's share of the rows)
+    (2, 11008, 4096, SKINNY), (7, 1000, 1040, SKINNY), (16, 4099, 2048, SKINNY), (9, 16400, 1024, SKINNY),
+    (13, 33, 8192, SKINNY), (5, 12000, 1296, SKINNY),
     (5, 7, 3, NAIVE), (17, 33, 147, NAIVE), (64, 10, 250, NAIVE),
 ]
 
@@ -145,6 +151,7 @@ MODES = [_ops.OUT_F32, _ops.OUT_F16, _ops.OUT_REQUANT_I8, _ops.OUT_FAKEQUANT_F32
 
 @pytest.mark.parametrize("path,M,N,K", [(TILE, 300, 260, 144), (TILE, 64, 256, 784),
                                          (SKINNY, 16, 272, 4096), (SKINNY, 37, 50, 64),
+                                         (SKINNY, 1, 1030, 4096), (SKINNY, 1, 45, 4112), (SKINNY, 11, 700, 2064),
                                          (NAIVE, 9, 21, 30)])
 @pytest.mark.parametrize("per_row,bias_kind,relu", [(False, "f32", False), (False, "f32", True),
                                                     (True, "f16", False), (False, None, True),
