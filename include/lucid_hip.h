@@ -84,6 +84,10 @@ int lq_memory_stats(size_t* bytes_in_use, size_t* bytes_reserved); /* MemoryStat
 int lq_h2d(void* dst_dev, const void* src_host, size_t nbytes, lq_stream stream);
 int lq_d2h(void* dst_host, const void* src_dev, size_t nbytes, lq_stream stream);
 int lq_d2d(void* dst_dev, const void* src_dev, size_t nbytes, lq_stream stream);
+/* `rows` rows of row_bytes each between two pitched device buffers (a column slice of a
+ * matrix: one direction's half of a bidirectional LSTM output, a channel slice). */
+int lq_d2d_rows(void* dst_dev, size_t dst_pitch, const void* src_dev, size_t src_pitch, size_t row_bytes,
+                size_t rows, lq_stream stream);
 int lq_fill_bytes(void* dst_dev, int value, size_t nbytes, lq_stream stream);
 int lq_sync(lq_stream stream);
 int lq_stream_create(lq_stream* stream);

@@ -82,6 +82,7 @@ _SIGNATURES = {
     "lq_h2d": [_vp, _vp, _sz, _vp],
     "lq_d2h": [_vp, _vp, _sz, _vp],
     "lq_d2d": [_vp, _vp, _sz, _vp],
+    "lq_d2d_rows": [_vp, _sz, _vp, _sz, _sz, _sz, _vp],
     "lq_fill_bytes": [_vp, _i, _sz, _vp],
     "lq_sync": [_vp],
     "lq_stream_create": [C.POINTER(_vp)],

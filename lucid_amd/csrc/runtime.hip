@@ -411,6 +411,16 @@ int lq_d2d(void* dst, const void* src, size_t nbytes, lq_stream stream) {
     return LQ_OK;
 }
 
+int lq_d2d_rows(void* dst, size_t dst_pitch, const void* src, size_t src_pitch, size_t row_bytes, size_t rows,
+                lq_stream stream) {
+    if (row_bytes == 0 || rows == 0) return LQ_OK;
+    LQ_REQUIRE(dst && src, LQ_ERR_VALUE, "NULL pointer in d2d_rows");
+    LQ_REQUIRE(dst_pitch >= row_bytes && src_pitch >= row_bytes, LQ_ERR_SHAPE, "d2d_rows: pitch smaller than a row");
+    LQ_HIP(hipMemcpy2DAsync(dst, dst_pitch, src, src_pitch, row_bytes, rows, hipMemcpyDeviceToDevice,
+                            as_stream(stream)));
+    return LQ_OK;
+}
+
 int lq_sync(lq_stream stream) {
     LQ_HIP(hipStreamSynchronize(as_stream(stream)));
     return LQ_OK;

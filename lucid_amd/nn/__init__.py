@@ -493,30 +493,33 @@ class ConvTranspose3d(Module):
 
 class LSTM(Module):
     """Float LSTM as a parameter holder: ``weight_ih_l{k}`` (4H, in), ``weight_hh_l{k}``
-    (4H, H), ``bias_ih_l{k}``, ``bias_hh_l{k}`` (and ``..._reverse`` when bidirectional),
-    gate order i, f, g, o."""
+    (4H, H or proj_size), ``bias_ih_l{k}``, ``bias_hh_l{k}``, ``weight_hr_l{k}`` (proj_size, H)
+    when ``proj_size > 0`` (and ``..._reverse`` when bidirectional), gate order i, f, g, o."""
 
     def __init__(self, input_size: int, hidden_size: int, num_layers: int = 1, bias: bool = True,
                  batch_first: bool = False, dropout: float = 0.0, bidirectional: bool = False,
                  proj_size: int = 0) -> None:
         super().__init__()
-        if proj_size:
-            raise NotImplementedError("LSTM: proj_size is not supported on the hip backend")
+        if proj_size < 0 or (proj_size > 0 and proj_size >= hidden_size):
+            raise ValueError(f"proj_size ({proj_size}) must be in [0, hidden_size = {hidden_size})")
         self.input_size, self.hidden_size, self.num_layers = input_size, hidden_size, num_layers
         self.bias, self.batch_first, self.dropout = bias, batch_first, dropout
-        self.bidirectional, self.proj_size = bidirectional, 0
+        self.bidirectional, self.proj_size = bidirectional, proj_size
+        rec = proj_size if proj_size > 0 else hidden_size  # what re-enters the recurrence
         bound = 1.0 / np.sqrt(hidden_size)
         rng = np.random.default_rng(input_size * 7919 + hidden_size * 31 + num_layers)
         dirs = 2 if bidirectional else 1
         for k in range(num_layers):
-            fan = input_size if k == 0 else hidden_size * dirs
+            fan = input_size if k == 0 else rec * dirs
             for suffix in ("", "_reverse")[:dirs]:
                 u = lambda *shape: T.tensor(rng.uniform(-bound, bound, shape).astype(np.float32))
                 self.register_buffer(f"weight_ih_l{k}{suffix}", u(4 * hidden_size, fan))
-                self.register_buffer(f"weight_hh_l{k}{suffix}", u(4 * hidden_size, hidden_size))
+                self.register_buffer(f"weight_hh_l{k}{suffix}", u(4 * hidden_size, rec))
                 if bias:
                     self.register_buffer(f"bias_ih_l{k}{suffix}", u(4 * hidden_size))
                     self.register_buffer(f"bias_hh_l{k}{suffix}", u(4 * hidden_size))
+                if proj_size > 0:  # W_hr: (proj_size, hidden_size), rnn.py:541-549
+                    self.register_buffer(f"weight_hr_l{k}{suffix}", u(proj_size, hidden_size))
 
     def named_parameters(self):
         return list(self.named_buffers())

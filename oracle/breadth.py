@@ -121,23 +121,35 @@ def quantized_act_codes(kind, q, in_offset, s, z, alpha, S, Z, qmin, qmax, out_o
     return O.quantize(act(kind, x, alpha), S, Z, qmin, qmax, code_offset=out_offset)
 
 
-def lstm(x, h0, c0, w_ih, w_hh, b_ih, b_hh):
-    """One layer, one direction, time-major ``x`` (T, B, I); returns (y, h_n, c_n)."""
+def lstm(x, h0, c0, w_ih, w_hh, b_ih, b_hh, w_hr=None, batch_sizes=None, reverse=False):
+    """One layer, one direction, time-major ``x`` (T, B, I); returns (y, h_n, c_n).
+
+    The recurrence of ``lstm_forward_train`` (CpuBackend.h:13394-13519): gates i, f, g, o;
+    with ``w_hr`` (P, H) the step's output and next hidden state are the projection
+    ``(o * tanh(c)) W_hr^T`` (lines 13503-13511).  ``batch_sizes`` (non-increasing, one per
+    step) is the active-set schedule of a packed batch (lucid/nn/modules/rnn.py:585-650):
+    at step t only the first ``batch_sizes[t]`` rows advance, the rest keep their state and
+    their output row is zero.  ``reverse`` walks the steps from the last to the first."""
     x = np.asarray(x, np.float32)
     T, B, _ = x.shape
-    H = h0.shape[-1]
+    H = c0.shape[-1]
+    R = H if w_hr is None else w_hr.shape[0]
     h, c = np.asarray(h0, np.float32).copy(), np.asarray(c0, np.float32).copy()
     bias = (np.asarray(b_ih, np.float32) + np.asarray(b_hh, np.float32)).astype(np.float32)
-    y = np.zeros((T, B, H), np.float32)
+    y = np.zeros((T, B, R), np.float32)
     sig = lambda v: (np.float32(1.0) / (np.float32(1.0) + np.exp(-v).astype(np.float32))).astype(np.float32)
-    for t in range(T):
-        raw = ((x[t] @ w_ih.T).astype(np.float32) + (h @ w_hh.T).astype(np.float32)).astype(np.float32)
+    for t in (range(T - 1, -1, -1) if reverse else range(T)):
+        n = B if batch_sizes is None else int(batch_sizes[t])
+        if n == 0:
+            continue
+        raw = ((x[t, :n] @ w_ih.T).astype(np.float32) + (h[:n] @ w_hh.T).astype(np.float32)).astype(np.float32)
         raw = (raw + bias).astype(np.float32)
         i, f = sig(raw[:, :H]), sig(raw[:, H:2 * H])
         g, o = np.tanh(raw[:, 2 * H:3 * H]).astype(np.float32), sig(raw[:, 3 * H:])
-        c = (f * c + i * g).astype(np.float32)
-        h = (o * np.tanh(c).astype(np.float32)).astype(np.float32)
-        y[t] = h
+        c[:n] = (f * c[:n] + i * g).astype(np.float32)
+        hr = (o * np.tanh(c[:n]).astype(np.float32)).astype(np.float32)
+        h[:n] = hr if w_hr is None else (hr @ np.asarray(w_hr, np.float32).T).astype(np.float32)
+        y[t, :n] = h[:n]
     return y, h, c
 
 

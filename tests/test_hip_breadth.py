@@ -284,6 +284,94 @@ def test_dynamic_lstm(layers, bidir, batch_first, bias, with_state):
     assert np.abs(yf - y.numpy()).mean() / (np.abs(yf).mean() + 1e-9) < 0.03
 
 
+def _deq(q, name):
+    return (getattr(q, name + "_int8").numpy().astype(np.float32) *
+            getattr(q, name + "_scale").numpy()[:, None]).astype(np.float32)
+
+
+@pytest.mark.parametrize("layers,bidir,proj,sorted_input", [(1, False, 0, True), (2, True, 0, False), (1, False, 6, True),
+                                                            (2, True, 5, False)])
+def test_dynamic_lstm_packed_sequences_and_projection(layers, bidir, proj, sorted_input):
+    """PackedSequence input and proj_size (lucid/nn/quantized/dynamic/rnn.py:66-84 hands both to
+    the float shell, lucid/nn/modules/rnn.py:585-795): against the oracle's recurrence run with
+    the packed active-set schedule, layer by layer and direction by direction."""
+    import lucid_amd.nn.quantized.dynamic as nnqd
+    from lucid_amd.nn.utils.rnn import PackedSequence, pack_padded_sequence, pad_packed_sequence
+    rng = np.random.default_rng(layers * 5 + bidir + proj)
+    I, H, Bn, Tn = 8, 16, 5, 7
+    R = proj if proj else H
+    dirs = 2 if bidir else 1
+    lengths = [7, 5, 5, 2, 1] if sorted_input else [2, 7, 1, 5, 5]
+    lstm = nn.LSTM(I, H, num_layers=layers, bidirectional=bidir, proj_size=proj)
+    qm = Q.quantize_dynamic(lstm)
+    assert isinstance(qm, nnqd.LSTM) and qm.proj_size == proj
+    if proj:
+        assert qm.weight_hr_l0_int8.shape == (proj, H) and qm.weight_hh_l0_int8.shape == (4 * H, proj)
+    x = rng.standard_normal((Tn, Bn, I)).astype(np.float32)
+    packed = pack_padded_sequence(hip(x), lengths, enforce_sorted=sorted_input)
+    assert isinstance(packed, PackedSequence) and packed.data.shape == (sum(lengths), I)
+    # the packing itself, against numpy
+    order = sorted(range(Bn), key=lambda i: -lengths[i])
+    slen = [lengths[i] for i in order]
+    bsz = [sum(1 for v in slen if v > t) for t in range(Tn)]
+    want = np.concatenate([x[t, order[:bs]] for t, bs in enumerate(bsz)])
+    assert np.array_equal(packed.data.numpy(), want) and packed.batch_sizes.numpy().tolist() == bsz
+    hx = (rng.standard_normal((layers * dirs, Bn, R)).astype(np.float32),
+          rng.standard_normal((layers * dirs, Bn, H)).astype(np.float32))
+    out, (hn, cn) = qm(packed, (hip(hx[0]), hip(hx[1])))
+    assert isinstance(out, PackedSequence) and out.data.shape == (sum(lengths), dirs * R)
+    # oracle: padded in packed order, the schedule, states as given; final states back in caller order
+    xs = np.zeros((Tn, Bn, I), np.float32)
+    off = 0
+    for t, bs in enumerate(bsz):
+        xs[t, :bs] = want[off:off + bs]
+        off += bs
+    hs, cs = [], []
+    for k in range(layers):
+        outs = []
+        for d, suffix in enumerate(("", "_reverse")[:dirs]):
+            idx = k * dirs + d
+            y, h, c = Br.lstm(xs, hx[0][idx], hx[1][idx], _deq(qm, f"weight_ih_l{k}{suffix}"),
+                              _deq(qm, f"weight_hh_l{k}{suffix}"), getattr(qm, f"bias_ih_l{k}{suffix}").numpy(),
+                              getattr(qm, f"bias_hh_l{k}{suffix}").numpy(),
+                              w_hr=_deq(qm, f"weight_hr_l{k}{suffix}") if proj else None, batch_sizes=bsz, reverse=d == 1)
+            outs.append(y)
+            hs.append(h)
+            cs.append(c)
+        xs = np.concatenate(outs, axis=-1)
+    wy = np.concatenate([xs[t, :bs] for t, bs in enumerate(bsz)])
+    inv = packed.unsorted_indices.numpy().tolist()
+    wh, wc = np.stack(hs)[:, inv], np.stack(cs)[:, inv]
+    for got, exp in ((out.data.numpy(), wy), (hn.numpy(), wh), (cn.numpy(), wc)):
+        assert got.shape == exp.shape and np.abs(got - exp).max() < 2e-5
+    # unpacking restores the caller's order and lengths
+    padded, lens = pad_packed_sequence(out, total_length=Tn)
+    assert lens.numpy().tolist() == lengths
+    for b, n in enumerate(lengths):
+        assert np.abs(padded.numpy()[:n, b] - xs[:n, inv[b]]).max() < 2e-5 and not padded.numpy()[n:, b].any()
+    # a dense tensor through the same module still takes the dense route
+    yd, _ = qm(hip(x))
+    assert yd.shape == (Tn, Bn, dirs * R)
+
+
+def test_pack_and_pad_round_trip_on_both_devices():
+    from lucid_amd.nn.utils.rnn import pack_padded_sequence, pack_sequence, pad_packed_sequence, pad_sequence
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((4, 6, 3)).astype(np.float32)            # batch-first (B, T, F)
+    lengths = [3, 6, 1, 4]
+    for dev in ("cpu", "hip"):
+        p = pack_padded_sequence(L.tensor(x, device=dev), lengths, batch_first=True, enforce_sorted=False)
+        back, lens = pad_packed_sequence(p, batch_first=True, padding_value=-1.0)
+        assert lens.numpy().tolist() == lengths and back.shape == (4, 6, 3) and back.device == dev
+        for b, n in enumerate(lengths):
+            assert np.array_equal(back.numpy()[b, :n], x[b, :n]) and (back.numpy()[b, n:] == -1.0).all()
+    with pytest.raises(ValueError, match="sorted"):
+        pack_padded_sequence(L.tensor(x), lengths, batch_first=True)
+    seqs = [L.tensor(rng.standard_normal((n, 2)).astype(np.float32)) for n in (5, 3, 2)]
+    assert pad_sequence(seqs).shape == (5, 3, 2)
+    assert pack_sequence(seqs).batch_sizes.numpy().tolist() == [3, 3, 2, 1, 1]
+
+
 # ---------------------------------------------------------------- Conv1d
 @pytest.mark.parametrize("cin,cout,k,stride,padding,dilation,groups,Ln",
                          [(16, 32, 3, 1, 1, 1, 1, 50), (32, 48, 5, 2, 2, 1, 1, 37), (32, 32, 3, 1, "same", 2, 2, 64),

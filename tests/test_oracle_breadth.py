@@ -104,6 +104,60 @@ def test_lstm_against_a_float64_recurrence():
     assert np.array_equal(y[-1], hn)
 
 
+@pytest.mark.parametrize("proj", [0, 4])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_lstm_projection_and_packed_schedule_against_torch(proj, reverse):
+    """The oracle's projection (W_hr) and packed active-set schedule against torch.nn.LSTM fed a
+    PackedSequence, and against running every sequence alone: a row's states must freeze at its
+    own last step, in both directions."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(11 + proj + reverse)
+    T, B, I, H = 6, 4, 5, 7
+    R = proj if proj else H
+    lengths = [6, 4, 4, 1]
+    batch_sizes = [sum(1 for v in lengths if v > t) for t in range(T)]
+    x = rng.standard_normal((T, B, I)).astype(np.float32)
+    for b, n in enumerate(lengths):
+        x[n:, b] = 0
+    wih = (rng.standard_normal((4 * H, I)) * 0.3).astype(np.float32)
+    whh = (rng.standard_normal((4 * H, R)) * 0.3).astype(np.float32)
+    whr = (rng.standard_normal((proj, H)) * 0.3).astype(np.float32) if proj else None
+    bih, bhh = ((rng.standard_normal(4 * H) * 0.1).astype(np.float32) for _ in range(2))
+    h0 = rng.standard_normal((B, R)).astype(np.float32)
+    c0 = rng.standard_normal((B, H)).astype(np.float32)
+    y, hn, cn = Br.lstm(x, h0, c0, wih, whh, bih, bhh, w_hr=whr, batch_sizes=batch_sizes, reverse=reverse)
+    # (1) every sequence on its own, dense
+    for b, n in enumerate(lengths):
+        xs = x[:n, b:b + 1]
+        ys, hs, cs = Br.lstm(xs[::-1] if reverse else xs, h0[b:b + 1], c0[b:b + 1], wih, whh, bih, bhh, w_hr=whr)
+        ys = ys[::-1] if reverse else ys
+        # (numpy's matmul may round the last bit differently for a batch of one)
+        assert np.allclose(y[:n, b], ys[:, 0], atol=1e-6) and not y[n:, b].any()
+        assert np.allclose(hn[b], hs[0], atol=1e-6) and np.allclose(cn[b], cs[0], atol=1e-6)
+    # (2) torch, the same weights, a packed batch (bidirectional: take the direction under test)
+    m = torch.nn.LSTM(I, H, bidirectional=True, proj_size=proj)
+    with torch.no_grad():
+        for suffix in ("", "_reverse"):
+            getattr(m, "weight_ih_l0" + suffix).copy_(torch.from_numpy(wih))
+            getattr(m, "weight_hh_l0" + suffix).copy_(torch.from_numpy(whh))
+            getattr(m, "bias_ih_l0" + suffix).copy_(torch.from_numpy(bih))
+            getattr(m, "bias_hh_l0" + suffix).copy_(torch.from_numpy(bhh))
+            if proj:
+                getattr(m, "weight_hr_l0" + suffix).copy_(torch.from_numpy(whr))
+        pk = torch.nn.utils.rnn.pack_padded_sequence(torch.from_numpy(x), lengths)
+        h0t = torch.from_numpy(np.stack([h0, h0]))
+        c0t = torch.from_numpy(np.stack([c0, c0]))
+        out, (hT, cT) = m(pk, (h0t, c0t))
+        out, _ = torch.nn.utils.rnn.pad_packed_sequence(out, total_length=T)
+    d = 1 if reverse else 0
+    assert np.allclose(y, out.numpy()[:, :, d * R:(d + 1) * R], atol=2e-6)
+    assert np.allclose(hn, hT.numpy()[d], atol=2e-6) and np.allclose(cn, cT.numpy()[d], atol=2e-6)
+    # a dense schedule is the plain recurrence
+    yd, hd, cd = Br.lstm(x, h0, c0, wih, whh, bih, bhh, w_hr=whr, batch_sizes=[B] * T)
+    y0, hh0, cc0 = Br.lstm(x, h0, c0, wih, whh, bih, bhh, w_hr=whr)
+    assert np.array_equal(yd, y0) and np.array_equal(hd, hh0) and np.array_equal(cd, cc0)
+
+
 @pytest.mark.parametrize("stride,padding,output_padding,dilation,groups",
                          [((2, 2), (1, 1), (1, 1), (1, 1), 1), ((1, 1), (0, 0), (0, 0), (1, 1), 1),
                           ((3, 2), (2, 0), (2, 1), (1, 1), 1), ((2, 2), (1, 1), (0, 0), (2, 1), 2)])
