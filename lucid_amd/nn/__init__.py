@@ -149,15 +149,12 @@ class Conv1d(Module):
             raise NotImplementedError("float nn.Conv1d.forward: zero padding with a number (or 'valid') only")
         if x.ndim != 3 or x.shape[1] != self.in_channels:
             raise _C.ShapeMismatch(f"Conv1d: expected (B, {self.in_channels}, L), got {x.shape}")
-        from .functional import conv2d_f32
-        B, Cc, Ln = x.shape
+        from .functional import conv1d_f32
         w = self.weight if self.weight.device == "hip" else self.weight.to("hip")
         b = self.bias
         if b is not None and b.device != "hip":
             b = b.to("hip")
-        y = conv2d_f32(x.reshape(B, Cc, 1, Ln), w.reshape(self.out_channels, Cc // self.groups, 1, self.kernel_size),
-                       b, (1, self.stride), (0, self.padding), (1, self.dilation), self.groups)
-        return y.reshape(B, self.out_channels, y.shape[3])
+        return conv1d_f32(x, w, b, self.stride, self.padding, self.dilation, self.groups)
 
 
 class Conv3d(Module):
@@ -182,9 +179,27 @@ class Conv3d(Module):
             rng.uniform(-bound, bound, out_channels).astype(np.float32)) if bias else None)
 
     def forward(self, x):
-        raise NotImplementedError(
-            "float nn.Conv3d.forward is not part of the hip quantized-inference backend; "
-            "quantize the model (convert) first")
+        """Float32 convolution on the device (depth taps summed over 2-d convolutions of depth
+        slices): calibration and QAT forwards of volumetric models.  Zero padding, symmetric."""
+        if not isinstance(x, Tensor) or x.device != "hip":
+            raise NotImplementedError(
+                "float nn.Conv3d.forward runs on the 'hip' device only; the CPU float path is Lucid's")
+        if self.padding_mode != "zeros":
+            raise NotImplementedError(f"float nn.Conv3d.forward: padding_mode {self.padding_mode!r} is not built")
+        pad = self.padding
+        if self._padding_str == "same":
+            from .quantized.conv import _same_pad_pair
+            pairs = [_same_pad_pair(n, k, s, d)
+                     for n, k, s, d in zip(x.shape[2:], self.kernel_size, self.stride, self.dilation)]
+            if any(lo != hi for lo, hi in pairs):
+                raise NotImplementedError("float nn.Conv3d.forward: asymmetric 'same' padding is not built")
+            pad = tuple(lo for lo, _ in pairs)
+        from .functional import conv3d_f32
+        w = self.weight if self.weight.device == "hip" else self.weight.to("hip")
+        b = self.bias
+        if b is not None and b.device != "hip":
+            b = b.to("hip")
+        return conv3d_f32(x, w, b, self.stride, pad, self.dilation, self.groups)
 
 
 class _BatchNorm(Module):

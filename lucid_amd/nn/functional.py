@@ -130,6 +130,72 @@ def conv2d_f32(x: Tensor, weight: Tensor, bias: Tensor | None = None, stride=(1,
     return out
 
 
+def conv1d_f32(x: Tensor, weight: Tensor, bias: Tensor | None = None, stride: int = 1, padding: int = 0,
+               dilation: int = 1, groups: int = 1) -> Tensor:
+    """``F.conv1d`` in float32: the 2-d kernel on a one-row image."""
+    _require_f32_hip("conv1d", x, weight)
+    if x.ndim != 3 or weight.ndim != 3:
+        raise _C.ShapeMismatch(f"conv1d: expected (B, C, L) input and (O, I, K) weight, got {x.shape} and {weight.shape}")
+    B, Cc, Ln = x.shape
+    O, I, K = weight.shape
+    y = conv2d_f32(x.reshape(B, Cc, 1, Ln), weight.reshape(O, I, 1, K), bias, (1, int(stride)), (0, int(padding)),
+                   (1, int(dilation)), groups)
+    return y.reshape(B, O, y.shape[3])
+
+
+def conv3d_f32(x: Tensor, weight: Tensor, bias: Tensor | None = None, stride=(1, 1, 1), padding=(0, 0, 0),
+               dilation=(1, 1, 1), groups: int = 1) -> Tensor:
+    """``F.conv3d`` in float32 with zero padding, for calibration and QAT forwards of volumetric
+    models: every output depth slice is the sum over the kernel's depth taps of a 2-d convolution
+    of one input depth slice (pitched device copies cut the slices out of ``(B, C, D, H, W)``).
+    The summation order differs from Lucid's im2col GEMM, so the result agrees with it to
+    float32 rounding, not bit for bit."""
+    _require_f32_hip("conv3d", x, weight)
+    if x.ndim != 5 or weight.ndim != 5 or weight.shape[1] * groups != x.shape[1]:
+        raise _C.ShapeMismatch(f"conv3d: input {x.shape} and weight {weight.shape} (groups={groups}) do not match")
+    B, Cin, D, H, W = x.shape
+    Cout, Cg, KD, KH, KW = weight.shape
+    (sd, sh, sw), (pd, ph, pw), (dd, dh, dw) = stride, padding, dilation
+    OD = (D + 2 * pd - dd * (KD - 1) - 1) // sd + 1
+    OH = (H + 2 * ph - dh * (KH - 1) - 1) // sh + 1
+    OW = (W + 2 * pw - dw * (KW - 1) - 1) // sw + 1
+    if min(OD, OH, OW) < 1:
+        raise _C.ShapeMismatch(f"conv3d: kernel {(KD, KH, KW)} does not fit input {x.shape}")
+    out = Tensor.empty((B, Cout, OD, OH, OW), T.float32, "hip")
+    # the kernel's depth taps as KD contiguous (Cout, Cg, KH, KW) filters
+    taps = []
+    for kd in range(KD):
+        wk = Tensor.empty((Cout, Cg, KH, KW), T.float32, "hip")
+        _C.call("lq_d2d_rows", wk.data_ptr, KH * KW * 4, weight.data_ptr + kd * KH * KW * 4, KD * KH * KW * 4,
+                KH * KW * 4, Cout * Cg, None)
+        taps.append(wk)
+    plane_in, plane_out = H * W * 4, OH * OW * 4
+    xs = Tensor.empty((B, Cin, H, W), T.float32, "hip")
+    for od in range(OD):
+        acc = None
+        for kd in range(KD):
+            z = od * sd - pd + kd * dd
+            if z < 0 or z >= D:
+                continue  # a tap in the zero padding
+            _C.call("lq_d2d_rows", xs.data_ptr, plane_in, x.data_ptr + z * plane_in, D * plane_in, plane_in, B * Cin, None)
+            part = conv2d_f32(xs, taps[kd], None, (sh, sw), (ph, pw), (dh, dw), groups)
+            if acc is None:
+                acc = part
+            else:
+                _C.call("lq_add_f32", acc.data_ptr, part.data_ptr, acc.data_ptr, acc.numel, None)
+        if acc is None:
+            acc = Tensor.empty((B, Cout, OH, OW), T.float32, "hip")
+            _C.call("lq_fill_bytes", acc.data_ptr, 0, acc.nbytes, None)
+        if bias is not None:
+            # y[b, c, :, :] + bias[c]: the bias as a (B * Cout, OH * OW) broadcast
+            full = Tensor.empty(acc.shape, T.float32, "hip")
+            _C.call("lq_broadcast_f32", bias.data_ptr, full.data_ptr, B, Cout, OH * OW, None)
+            _C.call("lq_add_f32", acc.data_ptr, full.data_ptr, acc.data_ptr, acc.numel, None)
+        _C.call("lq_d2d_rows", out.data_ptr + od * plane_out, OD * plane_out, acc.data_ptr, plane_out, plane_out,
+                B * Cout, None)
+    return out
+
+
 def linear_f32(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
     """``F.linear`` in float32 (``CpuBackend.h:4525``): ``x @ weight.T + bias``."""
     _require_f32_hip("linear", x, weight)

@@ -325,9 +325,8 @@ class Conv3d(Conv2d):
         g = input_grid(x, name)
         if x.ndim != 5 or x.shape[1] != self.in_channels:
             raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, D, H, W), got {x.shape}")
-        if self.padding_mode != "zeros":
-            raise NotImplementedError(f"{name}: padding_mode {self.padding_mode!r}; the hip backend pads "
-                                      "volumes with zeros only")
+        if self.padding_mode not in _PAD_MODES:
+            raise ValueError(f"{name}: unknown padding_mode {self.padding_mode!r}")
         if g.zp_host is None:
             raise NotImplementedError(
                 f"{name}: the input zero point is only known on the device; convolution needs it "
@@ -339,6 +338,24 @@ class Conv3d(Conv2d):
         if self._zp_host is None:
             self._zp_host = int(host_scalar(self.zero_point))
         pads = self._resolve_pad3(x.shape[2:])
+        if self.padding_mode != "zeros" and any(lo or hi for lo, hi in pads):
+            # pre-pad the codes, then convolve with padding 0 (nn/modules/conv.py:104-123).  F.pad's
+            # reflect / replicate / circular act on one axis at a time, so the volume is padded in
+            # two passes of the 2-d kernel: (H, W) with every (b, c, d) plane as an image of one
+            # channel, then D with every (b, c) volume as a one-column image whose "channels" are
+            # the padded planes.
+            B, Cc, D, H, W = x.shape
+            (d_lo, d_hi), (h_lo, h_hi), (w_lo, w_hi) = pads
+            Hp, Wp = H + h_lo + h_hi, W + w_lo + w_hi
+            mode = _PAD_MODES[self.padding_mode]
+            hw = Tensor.empty((B, Cc, D, Hp, Wp), T.int8, "hip")
+            _C.call("lq_pad_nhwc_i8", g.codes.data_ptr, hw.data_ptr, B * Cc * D, H, W, 1, h_lo, h_hi, w_lo, w_hi, mode,
+                    None)
+            full = Tensor.empty((B, Cc, D + d_lo + d_hi, Hp, Wp), T.int8, "hip")
+            _C.call("lq_pad_nhwc_i8", hw.data_ptr, full.data_ptr, B * Cc, D, 1, Hp * Wp, d_lo, d_hi, 0, 0, mode, None)
+            g = Grid(full, g.scale, g.zero_point, g.qdtype, g.offset, g.zp_host, "plain")
+            x = Tensor.on_grid(full.shape, g)
+            pads = [(0, 0)] * 3
         return volumetric_gemm(name, x, g, self._w_ohwi, self._wsum, self.weight_scale, self.bias, self.kernel_size,
                                self.stride, pads, self.dilation, (1, 1, 1), self.groups, self._fused_relu,
                                self.scale, self.zero_point, self.out_qdtype, self._zp_host,

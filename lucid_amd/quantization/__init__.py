@@ -32,16 +32,16 @@ def __getattr__(name):
     if name in ("prepare", "prepare_qat", "convert", "quantize_dynamic"):
         from . import _quantize
         return getattr(_quantize, name)
-    if name == "fuse_modules":
-        from ._fuse_modules import fuse_modules
-        return fuse_modules
+    if name in ("fuse_modules", "fuse_modules_qat"):
+        from . import _fuse_modules
+        return getattr(_fuse_modules, name)
     raise AttributeError(name)
 
 
 __all__ = [
     "ObserverBase", "MinMaxObserver", "PerChannelMinMaxObserver", "FixedQParamsObserver",
     "MovingAverageMinMaxObserver", "MovingAveragePerChannelMinMaxObserver", "HistogramObserver",
-    "QConfig", "get_default_qconfig", "prepare", "convert", "quantize_dynamic", "fuse_modules",
+    "QConfig", "get_default_qconfig", "prepare", "convert", "quantize_dynamic", "fuse_modules", "fuse_modules_qat",
     "QScheme", "per_tensor_affine", "per_tensor_symmetric", "per_channel_affine",
     "per_channel_symmetric", "QDtype", "qint8", "quint8", "qint32", "qint4", "QParams",
     "calculate_qparams", "quantize", "dequantize", "fake_quantize", "minmax", "quantize_rows_dynamic",

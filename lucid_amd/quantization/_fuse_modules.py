@@ -62,3 +62,38 @@ def fuse_modules(model, modules_to_fuse: Sequence[Sequence[str]], inplace: bool 
         for name, new in zip(group, _fuse_run(mods)):
             _set(model, name, new)
     return model
+
+
+def _fuse_run_qat(mods, qconfig):
+    """QAT replacements (``fuse_modules.py:186-216``): a Conv + BN (+ ReLU) run becomes the
+    ``nn.intrinsic.qat`` module that folds the BatchNorm on every forward; runs without a
+    BatchNorm become the plain fused marker that ``prepare_qat`` then swaps."""
+    from ..nn.intrinsic import qat as nniqat
+    ids = [nn.Identity() for _ in range(len(mods) - 1)]
+    first = mods[0]
+    if isinstance(first, _CONV_TYPES):
+        rank = _CONV_TYPES.index(type(first)) + 1
+        rest = list(mods[1:])
+        if rest and isinstance(rest[0], _BN_TYPES):
+            bn = rest.pop(0)
+            relu = bool(rest and isinstance(rest[0], nn.ReLU))
+            plain = (nniqat.ConvBn1d, nniqat.ConvBn2d, nniqat.ConvBn3d)[rank - 1]
+            fused = (nniqat.ConvBnReLU1d, nniqat.ConvBnReLU2d, nniqat.ConvBnReLU3d)[rank - 1]
+            return [(fused if relu else plain)(first, bn, qconfig=qconfig), *ids]
+        if rest and isinstance(rest[0], nn.ReLU):
+            return [_conv_relu(first, nn.ReLU()), *ids]
+        return [first, *ids]
+    if isinstance(first, nn.Linear) and len(mods) == 2 and isinstance(mods[1], nn.ReLU):
+        return [nni.LinearReLU(first, nn.ReLU()), *ids]
+    raise ValueError(f"fuse_modules_qat: unsupported pattern {[type(m).__name__ for m in mods]}")
+
+
+def fuse_modules_qat(model, modules_to_fuse: Sequence[Sequence[str]], qconfig, inplace: bool = False):
+    """``fuse_modules`` for the QAT workflow (``fuse_modules.py:219-330``), run before
+    ``prepare_qat``."""
+    model = model if inplace else copy.deepcopy(model)
+    for group in modules_to_fuse:
+        mods = [_get(model, name) for name in group]
+        for name, new in zip(group, _fuse_run_qat(mods, qconfig)):
+            _set(model, name, new)
+    return model

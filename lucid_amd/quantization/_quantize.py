@@ -138,11 +138,13 @@ def prepare(model, qconfig: QConfig | None = None, inplace: bool = False):
 
 
 def _qat_mapping() -> dict[type, object]:
-    """Float module type -> its QAT form (``_quantize.py:557-573``): Linear and Conv2d, plain
-    and fused with ReLU."""
+    """Float module type -> its QAT form (``_quantize.py:557-573``)."""
     import lucid_amd.nn.qat as nnqat
     return {nn.Linear: nnqat.Linear.from_float, nni.LinearReLU: nnqat.LinearReLU.from_float,
-            nn.Conv2d: nnqat.Conv2d.from_float, nni.ConvReLU2d: nnqat.ConvReLU2d.from_float}
+            nn.Conv1d: nnqat.Conv1d.from_float, nn.Conv2d: nnqat.Conv2d.from_float, nn.Conv3d: nnqat.Conv3d.from_float,
+            nn.Embedding: nnqat.Embedding.from_float,
+            nni.ConvReLU1d: nnqat.ConvReLU1d.from_float, nni.ConvReLU2d: nnqat.ConvReLU2d.from_float,
+            nni.ConvReLU3d: nnqat.ConvReLU3d.from_float}
 
 
 def _prepare_qat_recursive(module, qcfg, qat_map) -> int:
@@ -195,6 +197,15 @@ def convert(model, inplace: bool = False):
     mapping[nnqat.LinearReLU] = nnq.LinearReLU.from_float
     mapping[nnqat.Conv2d] = nnq.Conv2d.from_float
     mapping[nnqat.ConvReLU2d] = nnq.ConvReLU2d.from_float
+    mapping[nnqat.Conv1d] = nnq.Conv1d.from_float
+    mapping[nnqat.Conv3d] = nnq.Conv3d.from_float
+    mapping[nnqat.ConvReLU1d] = nnq.ConvReLU1d.from_float
+    mapping[nnqat.ConvReLU3d] = nnq.ConvReLU3d.from_float
+    mapping[nnqat.Embedding] = nnq.Embedding.from_float
+    import lucid_amd.nn.intrinsic.qat as nniqat
+    for _cls in (nniqat.ConvBn1d, nniqat.ConvBn2d, nniqat.ConvBn3d, nniqat.ConvBnReLU1d, nniqat.ConvBnReLU2d,
+                 nniqat.ConvBnReLU3d):
+        mapping[_cls] = nniqat.convbn_to_quantized
     if backends.quantized.use_mlx():
         mapping[nn.Linear] = _mlx_linear_builder(relu=False)
         mapping[nni.LinearReLU] = _mlx_linear_builder(relu=True)

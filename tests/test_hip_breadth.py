@@ -497,9 +497,9 @@ def test_conv3d_bit_exact_against_the_oracle(cin, cout, k, stride, padding, dila
 
 def test_conv3d_refuses_what_it_does_not_do():
     c3 = nnq.Conv3d(4, 4, 3)
-    c3.padding_mode = "reflect"
+    c3.padding_mode = "mirror"
     x = nnq.Quantize(hip(np.float32(0.1)), hip(np.float32(128.0)), Q.quint8)(hip(np.zeros((1, 4, 3, 3, 3), np.float32)))
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError, match="padding_mode"):
         c3(x)
     with pytest.raises(Exception):
         nnq.Conv3d(4, 4, 3)(nnq.Quantize(hip(np.float32(0.1)), hip(np.float32(128.0)), Q.quint8)(
@@ -563,3 +563,32 @@ def test_batched_byte_transpose(batches, R, Cn, pad_src, pad_dst):
     assert np.array_equal(got, want)
     with pytest.raises(Exception):
         _C.call("lq_transpose_i8", s.data_ptr, d.data_ptr, batches, R, Cn, R * Cn - 1, ds, None)
+
+
+@pytest.mark.parametrize("padding_mode", ["reflect", "replicate", "circular"])
+def test_conv3d_with_a_padding_mode(padding_mode):
+    """nnq.Conv3d with padding_mode != zeros (lucid/nn/quantized/conv.py:545; the float layer
+    pre-pads with F.pad and convolves with padding 0, nn/modules/conv.py:104-123): the padded
+    codes equal numpy's pad of the codes, the convolution equals the oracle on them."""
+    rng = np.random.default_rng(20)
+    B, Cc, D, H, W, Co = 2, 16, 4, 6, 5, 24
+    codes = rng.integers(0, 256, (B, Cc, D, H, W)).astype(np.int16)
+    wq = rng.integers(-127, 128, (Co, Cc, 3, 3, 3)).astype(np.int8)
+    ws = rng.uniform(0.001, 0.01, Co).astype(np.float32)
+    bias = rng.standard_normal(Co).astype(np.float32)
+    conv = nnq.Conv3d(Cc, Co, 3, padding=(1, 2, 1))
+    conv.padding_mode = padding_mode
+    state = {"weight_int8": wq, "weight_scale": ws, "weight_zero_point": np.zeros(Co, np.float32), "bias": bias,
+             "scale": np.float32(0.05), "zero_point": np.float32(120.0)}
+    conv.load_state_dict({k: L.tensor(v, device="hip") for k, v in state.items()})
+    from lucid_amd._tensor import Grid, Tensor
+    in_scale, in_zp = np.float32(0.02), 128
+    grid = Grid(hip((codes - 128).astype(np.int8)), hip(np.float32(in_scale)), hip(np.float32(in_zp)), Q.quint8, -128,
+                in_zp, "plain")
+    y = conv(Tensor.on_grid((B, Cc, D, H, W), grid))
+    got = y._grid.codes.numpy()
+    np_mode = {"reflect": "reflect", "replicate": "edge", "circular": "wrap"}[padding_mode]
+    xp = np.pad((codes - 128).astype(np.int8), ((0, 0), (0, 0), (1, 1), (2, 2), (1, 1)), mode=np_mode)
+    exp = Br.qconv3d(xp, wq, in_zp - 128, in_scale, ws, bias=bias, out_mode=O.OUT_REQUANT_I8, out_scale=0.05, out_zp=120.0,
+                     out_qmin=0, out_qmax=255, out_offset=-128)
+    assert got.shape == exp.shape and np.array_equal(got, exp)
