@@ -727,7 +727,7 @@ def main() -> int:
         # the decode-shaped (HBM-bound) Linears alone: int8 at M = 1 / 16 and weight-only int4 / int8
         res = {}
         for m in (1, 16):
-            rs = bench_linear(L, Q, _C, _ops, m, K, N, args.steps, args.warmup, seed=3)
+            rs = bench_linear(L, Q, _C, _ops, m, K, N, max(args.steps, 400), args.warmup, seed=3)
             cold_us = bench_linear_cold_weights(L, _C, _ops, rs["tensors"], m, K, N, max(10, args.steps // 2))
             res[f"linear_m{m}"] = {"us": round(rs["avg_kernel_ms"] * 1e3, 2), "frac_of_8TBs": round(rs["gbs"] / PEAK_HBM_GBS, 4),
                                    "cold_weights_us": round(cold_us, 2)}
@@ -807,7 +807,9 @@ def main() -> int:
             L, Q, _C, _ops, r["tensors"], M, K, N, 10)
         del r["tensors"]
         for m in (1, 16):
-            rs = bench_linear(L, Q, _C, _ops, m, K, N, args.steps, args.warmup, seed=3)
+            # at least 400 launches between the events: the ~50 us from the first event to the
+            # first kernel's start would otherwise be a tenth of 50 launches of 7 us
+            rs = bench_linear(L, Q, _C, _ops, m, K, N, max(args.steps, 400), args.warmup, seed=3)
             # us / GB/s: average of back-to-back launches between one pair of events (as the
             # headline); the median of individually bracketed launches, event cost included, beside it
             # cold_*: the same launches cycling through weight copies that exceed the last-level
