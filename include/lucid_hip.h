@@ -691,8 +691,46 @@ int lq_dequantize_nhwc_to_nchw(const int8_t* q, int code_offset, float* out, int
 int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH, int KW,
                               lq_stream stream);
 
+/* Quantized Conv3d forward as an implicit GEMM (lucid/nn/quantized/conv.py:545-700:
+ * dequantize kernel -> F.conv3d -> bias -> fake_quantize; IBackend::conv_nd_forward,
+ * IBackend.h:1469-1482, with three spatial dims), by the integer identity of
+ * lq_qconv2d_i8 with
+ *     m = (b, od, oh, ow),  n = cout,  k = (kd, kh, kw, cin_in_group).
+ * Activation codes are channels-last NDHWC [B,D,H,W,Cin], weight codes
+ * [Cout,KD,KH,KW,Cin/groups] (lq_transpose_i8 and lq_repack_oihw_to_ohwi_i8 with
+ * KH*KW := KD*KH*KW make them from Lucid's layouts); the taps are gathered by the
+ * GEMM's tile loader, so no patch matrix is written.  Zero padding becomes padding
+ * with the code a_zp; groups run in one launch.  stride / pad_lo / pad_hi /
+ * dilation are (depth, height, width).  Output: NDHWC [B,OD,OH,OW,Cout].
+ * Needs Cin/groups % 16 == 0 and 16-byte aligned tensors (LQ_ERR_NOT_IMPLEMENTED
+ * otherwise: use the explicit route below). */
+typedef struct {
+    const int8_t* x;       /* NDHWC codes as stored                          */
+    const int8_t* w;       /* [Cout,KD,KH,KW,Cin/groups] codes               */
+    int B, D, H, W, Cin, Cout, KD, KH, KW;
+    int stride[3], pad_lo[3], pad_hi[3], dilation[3], groups;
+    const int32_t* wsum;   /* [Cout] sum of each filter's codes              */
+    int a_zp;              /* zero point of the stored codes; also the pad code */
+    const float* a_scale;  /* [1]                                            */
+    const float* w_scale;  /* [Cout]                                         */
+    const void* bias;      /* [Cout] or NULL                                 */
+    int bias_dtype;
+    int relu;
+    int out_mode;          /* LQ_OUT_*                                       */
+    const float* out_scale;
+    const float* out_zp;
+    int out_qmin, out_qmax, out_offset;
+    void* out;             /* NDHWC [B,OD,OH,OW,Cout]                        */
+    int tile_config;       /* 0 = choose; shapes 3, 4, 5, 6, 9 have the gather */
+    const int32_t* w_zp;   /* optional [Cout] zero points of affine filters, as
+                              lq_qconv2d_args.w_zp                            */
+} lq_qconv3d_args;
+
+int lq_qconv3d_i8(const lq_qconv3d_args* args, lq_stream stream);
+
 /* Quantized Conv3d (lucid/nn/quantized/conv.py:545-700: dequantize kernel -> F.conv3d ->
- * bias -> fake_quantize) as an explicit GEMM on codes.  lq_transpose_i8 (batched byte
+ * bias -> fake_quantize) as an explicit GEMM on codes (any channel count; also what the
+ * transposed convolution uses).  lq_transpose_i8 (batched byte
  * transpose: src[b] R x Cn -> dst[b] Cn x R, batches src_stride / dst_stride bytes
  * apart) turns Lucid's (B, C, D*H*W) codes channels-last; lq_im2col_ndhwc_i8 gathers the
  * taps of the channels [c0, c0 + Cg) of one group from (B, D, H, W, C) codes into

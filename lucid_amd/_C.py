@@ -205,6 +205,24 @@ class QConv2dArgs(C.Structure):
 
 
 _SIGNATURES["lq_qconv2d_i8"] = [C.POINTER(QConv2dArgs), _vp]
+
+
+class QConv3dArgs(C.Structure):
+    """``lq_qconv3d_args`` of ``include/lucid_hip.h``."""
+
+    _fields_ = [
+        ("x", _vp), ("w", _vp),
+        ("B", _i), ("D", _i), ("H", _i), ("W", _i), ("Cin", _i), ("Cout", _i), ("KD", _i), ("KH", _i), ("KW", _i),
+        ("stride", _i * 3), ("pad_lo", _i * 3), ("pad_hi", _i * 3), ("dilation", _i * 3), ("groups", _i),
+        ("wsum", _vp), ("a_zp", _i), ("a_scale", _vp), ("w_scale", _vp),
+        ("bias", _vp), ("bias_dtype", _i), ("relu", _i), ("out_mode", _i),
+        ("out_scale", _vp), ("out_zp", _vp),
+        ("out_qmin", _i), ("out_qmax", _i), ("out_offset", _i),
+        ("out", _vp), ("tile_config", _i), ("w_zp", _vp),
+    ]
+
+
+_SIGNATURES["lq_qconv3d_i8"] = [C.POINTER(QConv3dArgs), _vp]
 _SIGNATURES["lq_quantize_nchw_to_nhwc"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]
 _SIGNATURES["lq_dequantize_nhwc_to_nchw"] = [_vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp]
 _SIGNATURES["lq_repack_oihw_to_ohwi_i8"] = [_vp, _vp, _i, _i, _i, _i, _vp]

@@ -159,3 +159,43 @@ def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None
     a.w_zp = _ptr(w_zp, "w_zp", T.int32)
     _C.call("lq_qconv2d_i8", C.byref(a), None)
     return out
+
+
+def qconv3d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None,
+               w_scale: Tensor | None = None, wsum: Tensor | None = None, bias: Tensor | None = None,
+               stride=(1, 1, 1), pad=((0, 0),) * 3, dilation=(1, 1, 1), groups: int = 1, relu: bool = False,
+               out_mode: int = OUT_F32, out_scale: Tensor | None = None, out_zp: Tensor | None = None,
+               out_qmin: int = 0, out_qmax: int = 255, out_offset: int = 0, tile_config: int = 0,
+               w_zp: Tensor | None = None) -> Tensor:
+    """Fused int8 volumetric convolution; see ``lq_qconv3d_i8``.  ``x`` int8 NDHWC, ``w`` int8
+    ``[Cout, KD, KH, KW, Cin/groups]``, ``pad`` = ((lo, hi),) * 3 for depth, height, width.
+    Returns NDHWC ``[B, OD, OH, OW, Cout]``."""
+    if x.ndim != 5 or w.ndim != 5:
+        raise _C.ShapeMismatch(f"qconv3d_i8: expected 5-d x and w, got {x.shape} and {w.shape}")
+    B, D, H, W, Cin = x.shape
+    Cout, KD, KH, KW, Cg = w.shape
+    if Cg * groups != Cin:
+        raise _C.ShapeMismatch(f"qconv3d_i8: weight {w.shape} does not match Cin={Cin}, groups={groups}")
+    outs = [conv_out_size(n, k, int(s), int(lo), int(hi), int(d))
+            for n, k, s, (lo, hi), d in zip((D, H, W), (KD, KH, KW), stride, pad, dilation)]
+    out = Tensor.empty((B, *[max(o, 0) for o in outs], Cout), _OUT_DTYPE[out_mode], "hip")
+    a = _C.QConv3dArgs()
+    a.x, a.w = _ptr(x, "x", T.int8), _ptr(w, "w", T.int8)
+    a.B, a.D, a.H, a.W, a.Cin, a.Cout, a.KD, a.KH, a.KW = B, D, H, W, Cin, Cout, KD, KH, KW
+    for i in range(3):
+        a.stride[i], a.dilation[i] = int(stride[i]), int(dilation[i])
+        a.pad_lo[i], a.pad_hi[i] = int(pad[i][0]), int(pad[i][1])
+    a.groups = int(groups)
+    a.wsum, a.a_zp = _ptr(wsum, "wsum", T.int32), int(a_zp)
+    a.a_scale, a.w_scale = _ptr(a_scale, "a_scale", T.float32), _ptr(w_scale, "w_scale", T.float32)
+    a.bias = _ptr(bias, "bias", (T.float32, T.float16))
+    a.bias_dtype = bias.dtype.code if bias is not None else 0
+    a.relu, a.out_mode = int(relu), int(out_mode)
+    a.out_scale, a.out_zp = _ptr(out_scale, "out_scale", T.float32), _ptr(out_zp, "out_zp", T.float32)
+    a.out_qmin, a.out_qmax, a.out_offset = int(out_qmin), int(out_qmax), int(out_offset)
+    a.out, a.tile_config = out.data_ptr, int(tile_config)
+    if w_zp is not None and w_zp.numel != Cout:
+        raise _C.ShapeMismatch(f"w_zp has {w_zp.numel} entries for Cout = {Cout}")
+    a.w_zp = _ptr(w_zp, "w_zp", T.int32)
+    _C.call("lq_qconv3d_i8", C.byref(a), None)
+    return out

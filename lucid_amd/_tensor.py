@@ -79,7 +79,7 @@ class Grid:
     asks for it.  ``offset`` is what was added to the code when storing it
     (-128 for ``quint8``, so the codes are valid signed MFMA operands).
     ``layout`` is "plain" (same element order as the float view) or "nhwc"
-    (codes of an NCHW float tensor kept channel-last for the conv kernels).
+    (codes of an NCHW / NCDHW float tensor kept channel-last for the conv kernels).
     """
 
     __slots__ = ("codes", "scale", "zero_point", "qdtype", "offset", "zp_host", "layout")
@@ -185,8 +185,10 @@ class Tensor:
             raise _C.LucidError("tensor has no storage")
         n = self.numel
         buf = DeviceBuffer(n * 4)
-        if g.layout == "nhwc" and len(self.shape) == 4:
-            B, Cc, H, W = self.shape
+        if g.layout == "nhwc" and len(self.shape) in (4, 5):
+            # (B, C, H, W) or (B, C, D, H, W): the kernel only needs the number of positions per image
+            B, Cc = self.shape[:2]
+            H, W = int(np.prod(self.shape[2:-1], dtype=np.int64)), self.shape[-1]
             _C.call("lq_dequantize_nhwc_to_nchw", g.codes.data_ptr, g.offset, buf.ptr, B, Cc, H, W,
                     g.scale.data_ptr, g.zero_point.data_ptr, None)
         else:

@@ -561,7 +561,7 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
         gg.w = flt; gg.K = p->KH * KWp * 4; gg.N = p->Cout;
         gg.cx = img; gg.cH = Hp; gg.cW = Wp; gg.cCin = 4; gg.cCg = 16; gg.cKW = KWp / 4;
         gg.cph = 0; gg.cpw = 0; gg.cdw = 4;  // a tap of the gather = four real pixels
-        return run_tile_kernel(gg, true, 1, p->tile_config, st);
+        return run_tile_kernel(gg, 1, 1, p->tile_config, st);
     }
     if (path == 1) {
         LQ_REQUIRE(is_gemm, LQ_ERR_VALUE, "qconv2d_i8: the gemm route needs a 1x1 stride-1 unpadded conv");
@@ -571,7 +571,7 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
     if (path == 2) {
         LQ_REQUIRE(Cg % 16 == 0 && aligned, LQ_ERR_VALUE,
                    "qconv2d_i8: the implicit route needs Cin/groups %% 16 == 0 and aligned tensors");
-        return run_tile_kernel(g, true, p->groups, p->tile_config, st);
+        return run_tile_kernel(g, 1, p->groups, p->tile_config, st);
     }
     if (path == 4) {
         ConvShape c{p->B, p->H, p->W, p->Cin, p->Cout, p->KH, p->KW, OH, OW, p->stride_h,
@@ -615,6 +615,101 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
         if (rc) return rc;
     }
     return LQ_OK;
+}
+
+int lq_qconv3d_i8(const lq_qconv3d_args* p, lq_stream stream) {
+    LQ_REQUIRE(p, LQ_ERR_VALUE, "qconv3d_i8: args is NULL");
+    LQ_REQUIRE(p->B >= 0 && p->D > 0 && p->H > 0 && p->W > 0 && p->Cin > 0 && p->Cout > 0 && p->KD > 0 &&
+                   p->KH > 0 && p->KW > 0,
+               LQ_ERR_SHAPE, "qconv3d_i8: non-positive extent");
+    LQ_REQUIRE(p->groups >= 1 && p->Cin % p->groups == 0 && p->Cout % p->groups == 0, LQ_ERR_SHAPE,
+               "qconv3d_i8: channels (%d -> %d) not divisible by groups %d", p->Cin, p->Cout, p->groups);
+    int out3[3];
+    const int in3[3] = {p->D, p->H, p->W}, k3[3] = {p->KD, p->KH, p->KW};
+    for (int i = 0; i < 3; ++i) {
+        LQ_REQUIRE(p->stride[i] >= 1 && p->dilation[i] >= 1 && p->pad_lo[i] >= 0 && p->pad_hi[i] >= 0, LQ_ERR_VALUE,
+                   "qconv3d_i8: bad stride / dilation / padding");
+        // output extent, lucid/_C/nn/ConvNd.cpp:56-59
+        out3[i] = (in3[i] + p->pad_lo[i] + p->pad_hi[i] - p->dilation[i] * (k3[i] - 1) - 1) / p->stride[i] + 1;
+        LQ_REQUIRE(out3[i] > 0, LQ_ERR_SHAPE, "qconv3d_i8: empty output");
+    }
+    if (p->B == 0) return LQ_OK;
+    LQ_REQUIRE(p->x && p->w && p->out, LQ_ERR_VALUE, "qconv3d_i8: NULL tensor pointer");
+    LQ_REQUIRE(p->out_mode >= OUT_ACC_I32 && p->out_mode <= OUT_FAKEQUANT_F32, LQ_ERR_VALUE,
+               "qconv3d_i8: unknown out_mode %d", p->out_mode);
+    LQ_REQUIRE(p->a_zp >= -128 && p->a_zp <= 127, LQ_ERR_VALUE,
+               "qconv3d_i8: activation zero point %d is not an int8 code", p->a_zp);
+    const int Cg = p->Cin / p->groups, Og = p->Cout / p->groups;
+    const long K = long(p->KD) * p->KH * p->KW * Cg;
+    LQ_REQUIRE(K <= 131071, LQ_ERR_SHAPE, "qconv3d_i8: K = %ld overflows the int32 accumulator", K);
+    const size_t M = size_t(p->B) * out3[0] * out3[1] * out3[2];
+    LQ_REQUIRE(M <= 0x7fffffffull && size_t(p->B) * p->D * p->H * p->W * p->Cin < 0x7fffffffull, LQ_ERR_SHAPE,
+               "qconv3d_i8: tensor too large for 32-bit indexing");
+    // the gather keeps a voxel's (h, w) origin in 16 bits each
+    LQ_REQUIRE(p->H + p->pad_lo[1] + p->pad_hi[1] < 32768 && p->W + p->pad_lo[2] + p->pad_hi[2] < 32768, LQ_ERR_SHAPE,
+               "qconv3d_i8: a padded plane of 32768 or more rows / columns");
+    LQ_REQUIRE(Cg % 16 == 0 && aligned16(p->x) && aligned16(p->w), LQ_ERR_NOT_IMPLEMENTED,
+               "qconv3d_i8: the gather needs Cin/groups %% 16 == 0 (got %d) and 16-byte aligned tensors; use "
+               "lq_im2col_ndhwc_i8 + lq_qlinear_i8",
+               Cg);
+    if (p->out_mode != OUT_ACC_I32) {
+        LQ_REQUIRE(p->w_scale && p->a_scale, LQ_ERR_VALUE, "qconv3d_i8: scale pointer is NULL");
+        LQ_REQUIRE(p->a_zp == 0 || p->wsum, LQ_ERR_VALUE,
+                   "qconv3d_i8: a non-zero activation zero point needs the filter sums");
+        LQ_REQUIRE(p->bias == nullptr || p->bias_dtype == LQ_F32 || p->bias_dtype == LQ_F16, LQ_ERR_DTYPE,
+                   "qconv3d_i8: bias must be float32 or float16");
+    }
+    if (p->out_mode == OUT_REQUANT_I8 || p->out_mode == OUT_FAKEQUANT_F32) {
+        LQ_REQUIRE(p->out_scale && p->out_zp, LQ_ERR_VALUE, "qconv3d_i8: output qparams are NULL");
+        if (p->out_mode == OUT_REQUANT_I8)
+            LQ_REQUIRE(p->out_qmin + p->out_offset >= -128 && p->out_qmax + p->out_offset <= 127, LQ_ERR_VALUE,
+                       "qconv3d_i8: output grid + offset does not fit int8");
+    }
+    hipStream_t st = as_stream(stream);
+    GemmArgs g{};
+    g.a = p->x; g.w = p->w; g.M = int(M); g.N = Og; g.K = int(K);
+    g.wsum = p->wsum; g.a_zp = p->a_zp; g.a_zp_dev = nullptr;
+    g.a_scale = p->a_scale; g.a_scale_per_row = 0; g.w_scale = p->w_scale;
+    g.bias = p->bias; g.bias_dtype = p->bias_dtype; g.relu = p->relu; g.out_mode = p->out_mode;
+    g.out_scale = p->out_scale; g.out_zp = p->out_zp;
+    g.out_qmin = p->out_qmin; g.out_qmax = p->out_qmax; g.out_offset = p->out_offset;
+    g.out = p->out; g.ldo = p->Cout;
+    g.cx = p->x; g.cD = p->D; g.cH = p->H; g.cW = p->W; g.cCin = p->Cin; g.cCg = Cg;
+    g.cOD = out3[0]; g.cOH = out3[1]; g.cOW = out3[2]; g.cKH = p->KH; g.cKW = p->KW;
+    g.csd = p->stride[0]; g.csh = p->stride[1]; g.csw = p->stride[2];
+    g.cpd = p->pad_lo[0]; g.cph = p->pad_lo[1]; g.cpw = p->pad_lo[2];
+    g.cdd = p->dilation[0]; g.cdh = p->dilation[1]; g.cdw = p->dilation[2];
+
+    if (p->w_zp && p->out_mode != OUT_ACC_I32) {
+        // affine filters, as in lq_qconv2d_i8: raw accumulators, the window sums of the volume
+        // from one all-ones filter per group, then the corrections and the epilogue proper
+        LQ_REQUIRE(p->wsum, LQ_ERR_VALUE, "qconv3d_i8: affine filters need the filter sums");
+        LQ_REQUIRE(K <= 33025, LQ_ERR_SHAPE, "qconv3d_i8: K = %ld overflows the int32 accumulator with affine filters",
+                   K);
+        const size_t acc_bytes = (M * p->Cout * 4 + 255) / 256 * 256;
+        const size_t sum_bytes = (M * p->groups * 4 + 255) / 256 * 256;
+        const size_t ones_bytes = size_t(p->groups) * K;
+        void* tmp = nullptr;
+        bool fresh = false;
+        int rc = stream_buffer(3, acc_bytes + sum_bytes + ones_bytes, 0, st, &tmp, &fresh);
+        if (rc) return rc;
+        int32_t* acc = static_cast<int32_t*>(tmp);
+        int32_t* asum = reinterpret_cast<int32_t*>(static_cast<char*>(tmp) + acc_bytes);
+        int8_t* ones = static_cast<int8_t*>(tmp) + acc_bytes + sum_bytes;
+        rc = lq_fill_bytes(ones, 1, ones_bytes, stream);
+        if (rc) return rc;
+        lq_qconv3d_args raw = *p;
+        raw.w_zp = nullptr; raw.out_mode = OUT_ACC_I32; raw.out = acc; raw.bias = nullptr; raw.relu = 0;
+        rc = lq_qconv3d_i8(&raw, stream);
+        if (rc) return rc;
+        lq_qconv3d_args win = raw;
+        win.w = ones; win.Cout = p->groups; win.out = asum; win.tile_config = 0;
+        rc = lq_qconv3d_i8(&win, stream);
+        if (rc) return rc;
+        g.N = p->Cout;
+        return launch_affine_fixup(g, acc, asum, p->groups, Og, p->w_zp, int(K), st);
+    }
+    return run_tile_kernel(g, 2, p->groups, p->tile_config, st);
 }
 
 int lq_quantize_nchw_to_nhwc(const float* x, int8_t* q, int code_offset, int B, int C, int H, int W,

@@ -51,24 +51,24 @@ int sk_scratch(size_t counters, size_t slab_bytes, hipStream_t st, SkScratch* ou
     return LQ_OK;
 }
 
-int launch_tile_c1(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c2(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c3(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c4(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c5(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c6(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c7(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c8(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c9(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c10(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c11(const GemmArgs&, bool, int, int, hipStream_t);
-int launch_tile_c12(const GemmArgs&, bool, int, int, hipStream_t);
+int launch_tile_c1(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c2(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c3(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c4(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c5(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c6(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c7(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c8(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c9(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c10(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c11(const GemmArgs&, int, int, int, hipStream_t);
+int launch_tile_c12(const GemmArgs&, int, int, int, hipStream_t);
 int launch_pp_shape(const GemmArgs&, int, hipStream_t);
 }  // namespace lq
 
 namespace {
 
-int launch_tile_shape(const GemmArgs& g, bool conv, int groups, int cfg, int schedule, hipStream_t st) {
+int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int schedule, hipStream_t st) {
     switch (cfg) {
     case 1: return launch_tile_c1(g, conv, groups, schedule, st);
     case 2: return launch_tile_c2(g, conv, groups, schedule, st);
@@ -102,7 +102,7 @@ int heuristic_tile_shape(const GemmArgs& g, int groups) {
     return 4;
 }
 
-int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st);
+int launch_tile_cfg(const GemmArgs& g, int conv, int groups, int tile_config, hipStream_t st);
 thread_local int t_last_tile_config = 0;  // what the last tile-kernel launch of this thread resolved to
 
 constexpr int kSplitShape = 11;  // 256 x 256 x 128 tiles, eight wavefronts
@@ -117,7 +117,7 @@ int launch_split(const GemmArgs& g, int a_tiles, hipStream_t st) {
     if (NA <= 0 || NA >= g.N) return fail(LQ_ERR_VALUE, "tile split: %ld columns of %d", NA, g.N);
     GemmArgs ga = g;
     ga.N = int(NA);
-    int rc = launch_tile_shape(ga, false, 1, kSplitShape, 1, st);
+    int rc = launch_tile_shape(ga, 0, 1, kSplitShape, 1, st);
     if (rc) return rc;
     GemmArgs gb = g;
     gb.N = g.N - int(NA);
@@ -129,7 +129,7 @@ int launch_split(const GemmArgs& g, int a_tiles, hipStream_t st) {
     gb.out = static_cast<char*>(g.out) + NA * esz;
     if (g.residual) gb.residual = g.residual + NA;
     if (g.join_q) gb.join_q = g.join_q + NA;
-    return launch_tile_cfg(gb, false, 1, 0, st);
+    return launch_tile_cfg(gb, 0, 1, 0, st);
 }
 
 // The best tile shape depends on how the tile count falls on the 256 CUs and on
@@ -139,7 +139,7 @@ int launch_split(const GemmArgs& g, int a_tiles, hipStream_t st) {
 // bit-identical results) and the choice is kept for the life of the process.
 // Not while the stream is being captured, and not when LQ_TILE_AUTOTUNE=0.
 struct TuneKey {
-    int M, N, K, mode, conv, groups, geom[8], flags;
+    int M, N, K, mode, conv, groups, geom[14], flags;
     bool operator==(const TuneKey& o) const { return std::memcmp(this, &o, sizeof(TuneKey)) == 0; }
 };
 struct TuneKeyHash {
@@ -161,7 +161,7 @@ bool autotune_enabled() {
     return on;
 }
 
-int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, int* cfg_out) {
+int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, int* cfg_out) {
     TuneKey key;
     std::memset(&key, 0, sizeof(key));
     key.M = g.M, key.N = g.N, key.K = g.K, key.mode = g.out_mode, key.conv = conv, key.groups = groups;
@@ -169,6 +169,10 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
         const int geom[8] = {g.cH, g.cW, g.cCin, g.cKW, g.csh * 16 + g.csw, g.cph * 256 + g.cpw,
                              g.cdh * 16 + g.cdw, g.cOW};
         std::memcpy(key.geom, geom, sizeof(geom));
+    }
+    if (conv == 2) {
+        const int geom3[6] = {g.cD, g.cOD, g.cKH, g.csd, g.cpd, g.cdd};
+        std::memcpy(key.geom + 8, geom3, sizeof(geom3));
     }
     key.flags = (g.residual ? 1 : 0) | (g.a_scale_per_row ? 2 : 0) | (g.bias ? 4 : 0) | (g.join_q ? 8 : 0) |
                 (g.gelu ? 16 : 0) | (g.range ? 32 : 0);
@@ -180,7 +184,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
             return LQ_OK;
         }
     }
-    const int fallback = heuristic_tile_shape(g, groups);
+    int fallback = heuristic_tile_shape(g, groups);
     *cfg_out = fallback;
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     LQ_HIP(hipStreamIsCapturing(st, &capturing));
@@ -195,28 +199,36 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
 
     // candidates are whole tile_config values (shape | schedule << 8)
     int cands[20], n = 0;
-    if (g.N <= 64) cands[n++] = 6;
-    cands[n++] = 5;
-    if (g.K <= 256) cands[n++] = 8;  // one to four k-iterations: latency-bound tiles, four blocks per CU
-    if (g.N > 64) cands[n++] = 3, cands[n++] = 4;
-    if (g.N > 128 && g.M > 128) cands[n++] = 1, cands[n++] = 11;
-    if (g.N > 128 && !conv) cands[n++] = 12;
-    // large plain GEMMs: the ping-pong kernel's 256 x 352 and 256 x 256 tiles
-    if (!conv && groups == 1 && g.K % 64 == 0 && g.M >= 256 && g.N >= 256 && !g.gelu && g.range == nullptr &&
-        size_t(g.M) * g.K < 0xffffffffull && size_t(g.N) * g.K < 0xffffffffull)
-        cands[n++] = 13, cands[n++] = 14;
-    // a long K over few tiles (late convolution stages): split K between the idle CUs
-    const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
-    if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
-    if (tiles128 < 256) cands[n++] = 9;  // ... or cover the chip with 64 x 64 tiles
-    if (tiles128 < 256 && g.K >= 1024) cands[n++] = 10;  // ... with 128-byte k-iterations
-    // whole rounds of 256 x 256 tiles plus a remainder (see launch_split)
-    if (!conv && groups == 1 && g.range == nullptr && g.M >= 256) {
-        const long tiles_m = (g.M + 255) / 256, tiles_n = g.N / 256;
-        const long rounds = tiles_m * tiles_n / 256;
-        const long a_tiles = rounds > 0 ? rounds * 256 / tiles_m : 0;
-        if (a_tiles > 0 && a_tiles * 256 < g.N && a_tiles < 32768)
-            cands[n++] = kSplitShape | (1 << 8) | int(a_tiles << 16);
+    if (conv == 2) {
+        // the shapes the volumetric gather is built for
+        if (g.N <= 64) cands[n++] = 6;
+        cands[n++] = 5;
+        if (g.N > 64) cands[n++] = 3, cands[n++] = 4;
+        if (long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups < 256) cands[n++] = 9;
+    } else {
+        if (g.N <= 64) cands[n++] = 6;
+        cands[n++] = 5;
+        if (g.K <= 256) cands[n++] = 8;  // one to four k-iterations: latency-bound tiles, four blocks per CU
+        if (g.N > 64) cands[n++] = 3, cands[n++] = 4;
+        if (g.N > 128 && g.M > 128) cands[n++] = 1, cands[n++] = 11;
+        if (g.N > 128 && !conv) cands[n++] = 12;
+        // large plain GEMMs: the ping-pong kernel's 256 x 352 and 256 x 256 tiles
+        if (!conv && groups == 1 && g.K % 64 == 0 && g.M >= 256 && g.N >= 256 && !g.gelu && g.range == nullptr &&
+            size_t(g.M) * g.K < 0xffffffffull && size_t(g.N) * g.K < 0xffffffffull)
+            cands[n++] = 13, cands[n++] = 14;
+        // a long K over few tiles (late convolution stages): split K between the idle CUs
+        const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
+        if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
+        if (tiles128 < 256) cands[n++] = 9;  // ... or cover the chip with 64 x 64 tiles
+        if (tiles128 < 256 && g.K >= 1024) cands[n++] = 10;  // ... with 128-byte k-iterations
+        // whole rounds of 256 x 256 tiles plus a remainder (see launch_split)
+        if (!conv && groups == 1 && g.range == nullptr && g.M >= 256) {
+            const long tiles_m = (g.M + 255) / 256, tiles_n = g.N / 256;
+            const long rounds = tiles_m * tiles_n / 256;
+            const long a_tiles = rounds > 0 ? rounds * 256 / tiles_m : 0;
+            if (a_tiles > 0 && a_tiles * 256 < g.N && a_tiles < 32768)
+                cands[n++] = kSplitShape | (1 << 8) | int(a_tiles << 16);
+        }
     }
     hipEvent_t e0, e1;
     LQ_HIP(hipEventCreate(&e0));
@@ -268,7 +280,7 @@ int tuned_tile_shape(const GemmArgs& g, bool conv, int groups, hipStream_t st, i
 // byte = schedule (0 = choose, 1 = block per tile, 2 = stream-K, 3 = stream-K over
 // the leftover tiles only), bits 16..30 = number of leading 256-column tiles given to
 // shape 1 with the remaining columns tuned separately (0 = no split).
-int launch_tile_cfg(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st) {
+int launch_tile_cfg(const GemmArgs& g, int conv, int groups, int tile_config, hipStream_t st) {
     int cfg = tile_config & 0xff;
     int schedule = (tile_config >> 8) & 0xff;
     int a_tiles = (tile_config >> 16) & 0x7fff;
@@ -628,7 +640,7 @@ int pad_table(const int8_t** table) {
     return LQ_OK;
 }
 
-int run_tile_kernel(const GemmArgs& g_in, bool conv, int groups, int tile_config, hipStream_t st) {
+int run_tile_kernel(const GemmArgs& g_in, int conv, int groups, int tile_config, hipStream_t st) {
     GemmArgs g = g_in;
     const int8_t* table = nullptr;
     int rc = pad_table(&table);
@@ -637,9 +649,9 @@ int run_tile_kernel(const GemmArgs& g_in, bool conv, int groups, int tile_config
     if (conv) {
         const int zp = g.a_zp;  // the stored code of real 0.0
         g.pad_src = table + size_t(uint8_t(int8_t(zp))) * 16;
-        return launch_tile_cfg(g, true, groups, tile_config, st);
+        return launch_tile_cfg(g, conv, groups, tile_config, st);
     }
-    return launch_tile_cfg(g, false, 1, tile_config, st);
+    return launch_tile_cfg(g, 0, 1, tile_config, st);
 }
 
 int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t st) {
@@ -653,7 +665,7 @@ int run_gemm(const GemmArgs& g_in, int force_path, int tile_config, hipStream_t 
     LQ_REQUIRE(path == 3 || vec_ok, LQ_ERR_VALUE,
                "qlinear_i8: MFMA paths need K %% 16 == 0 and 16-byte aligned operands");
     if (path == 1) {
-        int rc = run_tile_kernel(g, false, 1, tile_config, st);
+        int rc = run_tile_kernel(g, 0, 1, tile_config, st);
         if (rc) return rc;
     } else if (path == 2) {
         LQ_REQUIRE(g.M <= 64, LQ_ERR_SHAPE, "qlinear_i8: skinny path needs M <= 64 (M = %d)", g.M);

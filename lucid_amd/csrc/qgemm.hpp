@@ -48,13 +48,16 @@ struct GemmArgs {
     const float* join_out_zp;
     int join_out_qmin, join_out_qmax, join_out_offset;
     const int8_t* zeros;  // >= 16 zero bytes, source for K-tail chunks
-    // Implicit-GEMM convolution (tile kernel instantiated with CONV = true): the
+    // Implicit-GEMM convolution (tile kernel instantiated with CONV = 1): the
     // A operand is gathered from NHWC activation codes; row m is output pixel
     // (b, oh, ow), column k is ((kh*KW + kw)*Cg + ci).  N is then the output
     // channels of ONE group and blockIdx.y selects the group.
     const int8_t* cx;       // NHWC codes
     const int8_t* pad_src;  // 16 bytes holding the zero-point code (out-of-image taps)
     int cH, cW, cCin, cOH, cOW, cKW, cCg, csh, csw, cph, cpw, cdh, cdw;
+    // CONV = 2, volumetric: NDHWC codes, row m is output voxel (b, od, oh, ow), column k is
+    // (((kd*KH + kh)*KW + kw)*Cg + ci)
+    int cD, cOD, cKH, csd, cpd, cdd;
     // stream-K scratch (set by the launcher)
     int* sk_counters;
     int32_t* sk_slabs;
@@ -85,9 +88,10 @@ inline int set_join(GemmArgs& g, const lq_join_args& j, int out_mode, long n_col
 // convolution taps.
 int pad_table(const int8_t** table);
 
-// Launches the MFMA tile kernel on a filled-in GemmArgs.  conv = true gathers
-// the A operand from NHWC codes (cx / c* fields); `groups` becomes gridDim.y.
-int run_tile_kernel(const GemmArgs& g, bool conv, int groups, int tile_config, hipStream_t st);
+// Launches the MFMA tile kernel on a filled-in GemmArgs.  conv = 1 gathers the A operand
+// from NHWC codes, conv = 2 from NDHWC codes (cx / c* fields); `groups` becomes gridDim.y.
+// The volumetric gather is built for tile shapes 3, 5, 6 and 9, one block per tile.
+int run_tile_kernel(const GemmArgs& g, int conv, int groups, int tile_config, hipStream_t st);
 
 
 // Chooses between the tile, skinny and naive kernels (force_path: 0 = choose,

@@ -276,7 +276,7 @@ struct IterSplit {
 // arrival counter; whoever arrives last adds the other slabs to its registers
 // and runs the epilogue.  Integer partial sums add exactly, so the result does
 // not depend on who arrives when.
-template <class Cfg, int MODE, bool CONV, bool SK>
+template <class Cfg, int MODE, int CONV, bool SK>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel(GemmArgs g) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
     constexpr int C = Cfg::C, R = Cfg::R, PA = Cfg::PA, PB = Cfg::PB, STAGES = Cfg::STAGES;
@@ -336,12 +336,24 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         const int m0 = tm * BM, n0 = n_base + tn * BN;
         unsigned a_off[PA], b_off[PB];
         int a_hw[PA];  // CONV: top-left input coordinate of the pixel, (ih0 << 16) | (iw0 & 0xffff)
+        int a_d[CONV == 2 ? PA : 1];  // volumetric: its first depth slice
         const int a_rows = g.M - m0, b_rows = n_limit - n0;  // valid rows in this tile (>= 1)
 #pragma unroll
         for (int it = 0; it < PA; ++it) {
             int r = it * Cfg::ROWS_PER_PASS + row_in_pass;
             r = r < a_rows ? r : a_rows - 1;  // clamp: reads stay in bounds, rows are masked at the store
-            if (CONV) {
+            if constexpr (CONV == 2) {
+                const int m = m0 + r;
+                const int plane = g.cOH * g.cOW, vol = g.cOD * plane;
+                const int b = m / vol, rem = m - b * vol;
+                const int od = rem / plane, rem2 = rem - od * plane;
+                const int oh = rem2 / g.cOW, ow = rem2 - oh * g.cOW;
+                const int id0 = od * g.csd - g.cpd, ih0 = oh * g.csh - g.cph, iw0 = ow * g.csw - g.cpw;
+                a_hw[it] = (ih0 << 16) | (iw0 & 0xffff);
+                a_d[it] = id0;
+                a_off[it] = unsigned(((b * g.cD + id0) * g.cH + ih0) * g.cW + iw0) * unsigned(g.cCin) +
+                            unsigned(int(blockIdx.y) * g.cCg);
+            } else if (CONV) {
                 const int m = m0 + r;
                 const int pix = g.cOH * g.cOW;
                 const int b = m / pix, rem = m - b * pix;
@@ -370,11 +382,16 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
         // to be loaded.  Stages are loaded in k order, BK bytes apart, so the position is found
         // by division once per segment and then stepped (the divisions by run-time values cost
         // more than the MFMAs of a small tile's k-iteration).
-        int c_ci0 = 0, c_kh = 0, c_kw = 0;
+        int c_ci0 = 0, c_kh = 0, c_kw = 0, c_kd = 0;
         if (CONV) {
             const int k = kb * BK + kc * 16;
-            const int tap = k / g.cCg;
+            int tap = k / g.cCg;
             c_ci0 = k - tap * g.cCg;
+            if (CONV == 2) {
+                const int taps_hw = g.cKH * g.cKW;
+                c_kd = tap / taps_hw;
+                tap -= c_kd * taps_hw;
+            }
             c_kh = tap / g.cKW;
             c_kw = tap - c_kh * g.cKW;
         }
@@ -399,19 +416,23 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::MINWAVES) void qgemm_tile_kernel
             }
             if (CONV) {
                 // this lane's 16 bytes lie inside one filter tap (Cg % 16 == 0)
-                const int ci0 = c_ci0, kh = c_kh, kw = c_kw;
+                const int ci0 = c_ci0, kh = c_kh, kw = c_kw, kd = c_kd;
                 c_ci0 += BK;  // on to the next stage
                 while (c_ci0 >= g.cCg) {
                     c_ci0 -= g.cCg;
-                    if (++c_kw == g.cKW) c_kw = 0, ++c_kh;
+                    if (++c_kw == g.cKW) {
+                        c_kw = 0, ++c_kh;
+                        if (CONV == 2 && c_kh == g.cKH) c_kh = 0, ++c_kd;
+                    }
                 }
-                const int dh = kh * g.cdh, dw = kw * g.cdw;
-                const unsigned delta = unsigned(dh * g.cW + dw) * unsigned(g.cCin) + unsigned(ci0);
+                const int dh = kh * g.cdh, dw = kw * g.cdw, dd = CONV == 2 ? kd * g.cdd : 0;
+                const unsigned delta = unsigned((dd * g.cH + dh) * g.cW + dw) * unsigned(g.cCin) + unsigned(ci0);
 #pragma unroll
                 for (int it = 0; it < PA; ++it) {
                     const int ih = (a_hw[it] >> 16) + dh;
                     const int iw = int(short(a_hw[it] & 0xffff)) + dw;
-                    const bool ok = in_k && unsigned(ih) < unsigned(g.cH) && unsigned(iw) < unsigned(g.cW);
+                    bool ok = in_k && unsigned(ih) < unsigned(g.cH) && unsigned(iw) < unsigned(g.cW);
+                    if constexpr (CONV == 2) ok = ok && unsigned(a_d[it] + dd) < unsigned(g.cD);
                     const int8_t* src = ok ? a_tile + (a_off[it] + delta) : g.pad_src;
                     __builtin_amdgcn_global_load_lds(LQ_GPTR(src), LQ_LPTR(sa + it * (THREADS * 16)), 16, 0, 0);
                 }
@@ -849,10 +870,15 @@ int sk_scratch(size_t counters, size_t slab_bytes, hipStream_t st, SkScratch* ou
 
 namespace {
 
-template <class Cfg, int MODE, bool CONV>
+template <class Cfg, int MODE, int CONV>
 int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
     const void* fn_dp = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV, false>);
-    const void* fn_sk = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV, true>);
+    // the volumetric gather is built for one block per tile only
+    const void* fn_sk = reinterpret_cast<const void*>(qgemm_tile_kernel<Cfg, MODE, CONV, CONV != 2>);
+    if (CONV == 2) {
+        LQ_REQUIRE(schedule <= 1, LQ_ERR_NOT_IMPLEMENTED, "tile kernel: a volumetric convolution runs one block per tile");
+        schedule = 1;
+    }
     static bool attr_set = false;
     if (!attr_set) {
         LQ_HIP(hipFuncSetAttribute(fn_dp, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
@@ -915,7 +941,7 @@ int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st
     return LQ_OK;
 }
 
-template <class Cfg, bool CONV>
+template <class Cfg, int CONV>
 int launch_tile(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
     LQ_REQUIRE(size_t(Cfg::BM > Cfg::BN ? Cfg::BM : Cfg::BN) * g.K < 0xffffffffull, LQ_ERR_SHAPE,
                "tile kernel: K too large");
@@ -924,7 +950,7 @@ int launch_tile(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
     case OUT_F32:
         if (g.gelu || g.range != nullptr) {
             if (CONV) return fail(LQ_ERR_NOT_IMPLEMENTED, "tile kernel: GELU / kept range are not built for convolutions");
-            return launch_tile_mode<Cfg, OUT_F32X, false>(g, groups, schedule, st);
+            return launch_tile_mode<Cfg, OUT_F32X, 0>(g, groups, schedule, st);
         }
         return launch_tile_mode<Cfg, OUT_F32, CONV>(g, groups, schedule, st);
     case OUT_F16: return launch_tile_mode<Cfg, OUT_F16, CONV>(g, groups, schedule, st);
@@ -938,11 +964,16 @@ int launch_tile(const GemmArgs& g, int groups, int schedule, hipStream_t st) {
 }  // namespace
 }  // namespace lq
 
-// One per translation unit: the launcher of one tile shape.
-#define LQ_DEFINE_TILE_LAUNCHER(NAME, CFG)                                                      \
+// One per translation unit: the launcher of one tile shape.  conv: 0 = plain GEMM, 1 = gather
+// from NHWC codes, 2 = from NDHWC codes (only in the units that pass WITH_3D = true).
+#define LQ_DEFINE_TILE_LAUNCHER(NAME, CFG, WITH_3D)                                             \
     namespace lq {                                                                              \
-    int NAME(const GemmArgs& g, bool conv, int groups, int schedule, hipStream_t st) {          \
-        return conv ? launch_tile<CFG, true>(g, groups, schedule, st)                           \
-                    : launch_tile<CFG, false>(g, groups, schedule, st);                         \
+    int NAME(const GemmArgs& g, int conv, int groups, int schedule, hipStream_t st) {           \
+        if (conv == 2) {                                                                        \
+            if constexpr (WITH_3D) return launch_tile<CFG, 2>(g, groups, schedule, st);         \
+            return fail(LQ_ERR_NOT_IMPLEMENTED, "this tile shape has no volumetric gather");    \
+        }                                                                                       \
+        return conv ? launch_tile<CFG, 1>(g, groups, schedule, st)                              \
+                    : launch_tile<CFG, 0>(g, groups, schedule, st);                             \
     }                                                                                           \
     }

@@ -1,4 +1,4 @@
 // Tile kernel instances of one shape (CfgSmall); see qgemm_tile.hpp.
 #include "qgemm_tile.hpp"
 
-LQ_DEFINE_TILE_LAUNCHER(launch_tile_c9, CfgSmall)
+LQ_DEFINE_TILE_LAUNCHER(launch_tile_c9, CfgSmall, true)

@@ -99,6 +99,18 @@ def input_grid(x: Tensor, what: str) -> Grid:
     return x._grid
 
 
+def plain_volume_grid(x: Tensor, g: Grid) -> Grid:
+    """The grid of a 5-d activation with its codes in (B, C, D, H, W) order: channels-last
+    codes (layout "nhwc", what the volumetric convolution leaves) are transposed back."""
+    if g.layout == "plain":
+        return g
+    B, Cc = x.shape[0], x.shape[1]
+    vol = x.numel // max(B * Cc, 1)
+    codes = Tensor.empty(x.shape, T.int8, "hip")
+    _C.call("lq_transpose_i8", g.codes.data_ptr, codes.data_ptr, B, vol, Cc, vol * Cc, Cc * vol, None)
+    return Grid(codes, g.scale, g.zero_point, g.qdtype, g.offset, g.zp_host, "plain")
+
+
 def zp_args(g: Grid) -> tuple[int, Tensor | None]:
     """``(a_zp, a_zp_dev)`` for the GEMM / conv entry points: a host zero point
     when it is known, otherwise the device scalar plus the storage offset."""

@@ -22,7 +22,7 @@ from ... import _tensor as T
 from ..._tensor import Grid, Tensor
 from ...quantization._qscheme import QDtype, quint8
 from ..module import Module
-from ._utils import (activation_qparams, host_scalar, input_grid, quantize_weight,
+from ._utils import (activation_qparams, host_scalar, input_grid, plain_volume_grid, quantize_weight,
                      forget_weight_zero_points, storage_offset, weight_zero_points)
 
 
@@ -251,7 +251,10 @@ def _triple(v):
 def volumetric_gemm(name, x: Tensor, g, w_rows: Tensor, wsum: Tensor, w_scale: Tensor, bias, kernel, stride,
                     pads, dilation, insert, groups: int, relu: bool, scale: Tensor, zero_point: Tensor,
                     qdtype: QDtype, zp_host: int, w_zp: Tensor | None = None) -> Tensor:
-    """A 3-d convolution on codes as an explicit GEMM, group by group: gather the taps of
+    """A 3-d convolution on codes.  With ``C/groups`` a multiple of 16 and no insertion: one
+    fused launch whose loader gathers the taps (``lq_qconv3d_i8``), the result kept channels-last
+    (layout "nhwc").  Otherwise as an explicit
+    GEMM, group by group: gather the taps of
     ``x``'s ``(B, C, D, H, W)`` codes (``insert`` > 1: as if zero-point codes stood between
     neighbouring samples), multiply with the group's kernel rows ``[Cout/groups, taps * C/groups]``
     through the fused int8 GEMM, write the result channels-first.  The codes are turned
@@ -269,8 +272,20 @@ def volumetric_gemm(name, x: Tensor, g, w_rows: Tensor, wsum: Tensor, w_scale: T
     off = storage_offset(qdtype)
     i3 = lambda v: (C.c_int * 3)(*[int(e) for e in v])
     vol = D * H * W
-    last = Tensor.empty((B, D, H, W, Cc), T.int8, "hip")      # channels-last copy of the input codes
-    _C.call("lq_transpose_i8", g.codes.data_ptr, last.data_ptr, B, Cc, vol, Cc * vol, Cc * vol, None)
+    if g.layout == "nhwc":
+        last = g.codes                                        # already (B, D, H, W, C)
+    else:
+        last = Tensor.empty((B, D, H, W, Cc), T.int8, "hip")  # channels-last copy of the input codes
+        _C.call("lq_transpose_i8", g.codes.data_ptr, last.data_ptr, B, Cc, vol, Cc * vol, Cc * vol, None)
+    if Cg % 16 == 0 and tuple(insert) == (1, 1, 1):
+        # the taps are gathered by the GEMM's loader (no patch matrix), all groups in one launch
+        w5 = w_rows.reshape((Co, *[int(k) for k in kernel], Cg))
+        y = _ops.qconv3d_i8(last, w5, a_zp=a_zp, a_scale=g.scale, w_scale=w_scale, wsum=wsum, bias=bias,
+                            stride=stride, pad=pads, dilation=dilation, groups=groups, relu=relu,
+                            out_mode=_ops.OUT_REQUANT_I8, out_scale=scale, out_zp=zero_point,
+                            out_qmin=qdtype.quant_min, out_qmax=qdtype.quant_max, out_offset=off, w_zp=w_zp)
+        # the result stays channels-last: the next volumetric layer reads it as it is
+        return Tensor.on_grid((B, Co, *outs), Grid(y, scale, zero_point, qdtype, off, zp_host, "nhwc"))
     codes = Tensor.empty((B, Co, *outs), T.int8, "hip")
     cols = Tensor.empty((B * L, Cg * kernel[0] * kernel[1] * kernel[2]), T.int8, "hip")
     for grp in range(groups):
@@ -331,14 +346,13 @@ class Conv3d(Conv2d):
             raise NotImplementedError(
                 f"{name}: the input zero point is only known on the device; convolution needs it "
                 "on the host for the padding code (static quantization provides it)")
-        if g.layout != "plain":
-            raise _C.LucidError(f"{name}: 5-d activation codes must be stored in their own (B, C, D, H, W) order")
         if self._w_ohwi is None:
             self._prepare_weight()
         if self._zp_host is None:
             self._zp_host = int(host_scalar(self.zero_point))
         pads = self._resolve_pad3(x.shape[2:])
         if self.padding_mode != "zeros" and any(lo or hi for lo, hi in pads):
+            g = plain_volume_grid(x, g)
             # pre-pad the codes, then convolve with padding 0 (nn/modules/conv.py:104-123).  F.pad's
             # reflect / replicate / circular act on one axis at a time, so the volume is padded in
             # two passes of the 2-d kernel: (H, W) with every (b, c, d) plane as an image of one

@@ -212,8 +212,6 @@ class ConvTranspose3d(ConvTranspose2d):
             raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, D, H, W), got {x.shape}")
         if g.zp_host is None:
             raise NotImplementedError(f"{name}: the input zero point must be known on the host")
-        if g.layout != "plain":
-            raise _C.LucidError(f"{name}: 5-d activation codes must be stored in their own (B, C, D, H, W) order")
         lo = [d * (k - 1) - p for d, k, p in zip(self.dilation, self.kernel_size, self.padding)]
         if min(lo) < 0:
             raise NotImplementedError(f"{name}: padding larger than dilation * (kernel - 1) is not supported")

@@ -3,6 +3,8 @@
 
 from __future__ import annotations
 
+import numpy as np
+
 from ... import _C
 from ... import _tensor as T
 from ..._tensor import Grid, Tensor
@@ -56,10 +58,11 @@ class Quantize(Module):
         if self._zp_host is None:
             self._zp_host = int(host_scalar(self.zero_point))
         off = storage_offset(self.qdtype)
-        if x.ndim == 4:
-            # an image batch: codes go channel-last, the layout of the conv kernels
-            B, Cc, H, W = x.shape
-            codes = Tensor.empty((B, H, W, Cc), T.int8, "hip")
+        if x.ndim in (4, 5):
+            # an image or video batch: codes go channel-last, the layout of the conv kernels
+            B, Cc = x.shape[:2]
+            H, W = int(np.prod(x.shape[2:-1], dtype=np.int64)), x.shape[-1]
+            codes = Tensor.empty((B, *x.shape[2:], Cc), T.int8, "hip")
             _C.call("lq_quantize_nchw_to_nhwc", x.data_ptr, codes.data_ptr, off, B, Cc, H, W,
                     self.scale.data_ptr, self.zero_point.data_ptr, self.qdtype.quant_min,
                     self.qdtype.quant_max, None)

@@ -19,6 +19,12 @@ def hip(a, dtype=None):
     return L.tensor(a, device="hip") if dtype is None else L.tensor(np.asarray(a, dtype), device="hip")
 
 
+def volume_codes(t):
+    """Stored codes of a 5-d activation in (B, C, D, H, W) order, whichever layout it is kept in."""
+    codes = t._grid.codes.numpy()
+    return np.ascontiguousarray(np.moveaxis(codes, -1, 1)) if t._grid.layout == "nhwc" else codes
+
+
 # ---------------------------------------------------------------- embeddings
 @pytest.mark.parametrize("num,dim,idx_dtype", [(100, 32, np.int64), (257, 30, np.int32), (5000, 768, np.int64)])
 def test_embedding_bit_exact(num, dim, idx_dtype):
@@ -487,12 +493,92 @@ def test_conv3d_bit_exact_against_the_oracle(cin, cout, k, stride, padding, dila
                       stride=S3, pad=tuple(pad), dilation=D3, groups=groups, bias=c3.bias.numpy(),
                       out_mode=O.OUT_REQUANT_I8, out_scale=np.float32(c3.scale.item()),
                       out_zp=np.float32(c3.zero_point.item()), out_qmin=0, out_qmax=255, out_offset=-128)
-    got = out._grid.codes.numpy()
+    got = volume_codes(out)
+    assert out._grid.layout == ("nhwc" if (cin // groups) % 16 == 0 else "plain")
     assert got.shape == want.shape and np.array_equal(got, want)
     assert len(np.unique(got)) > 20
     y = qm(hip(x)).numpy()
     exp_y = (want.astype(np.float32) + 128 - np.float32(c3.zero_point.item())) * np.float32(c3.scale.item())
     assert np.array_equal(y, exp_y)
+
+
+GATHER3D_CASES = [
+    # B, C, Co, vol, kernel, stride, pads, dilation, groups, tile shape
+    (2, 16, 32, (5, 9, 11), (3, 3, 3), (1, 1, 1), ((1, 1), (1, 1), (1, 1)), (1, 1, 1), 1, 0),
+    (1, 32, 24, (4, 13, 7), (2, 3, 1), (2, 1, 2), ((0, 1), (2, 0), (0, 0)), (1, 2, 1), 1, 5),
+    (3, 64, 64, (6, 10, 10), (3, 3, 3), (1, 2, 1), ((1, 1), (0, 1), (2, 2)), (2, 1, 1), 1, 6),
+    (2, 96, 160, (3, 8, 9), (1, 3, 3), (1, 1, 1), ((0, 0), (1, 1), (1, 1)), (1, 1, 1), 2, 3),
+    (2, 48, 288, (4, 6, 6), (3, 1, 2), (1, 1, 1), ((2, 2), (0, 0), (1, 0)), (1, 1, 3), 3, 4),
+    (1, 16, 16, (2, 3, 3), (2, 2, 2), (1, 1, 1), ((0, 0), (0, 0), (0, 0)), (1, 1, 1), 1, 9),
+    (2, 32, 48, (7, 7, 7), (3, 3, 3), (2, 2, 2), ((1, 1), (1, 1), (1, 1)), (1, 1, 1), 1, 9),
+]
+
+
+@pytest.mark.parametrize("B,C,Co,vol,kernel,stride,pads,dilation,groups,shape", GATHER3D_CASES)
+def test_conv3d_loader_gather_exact(B, C, Co, vol, kernel, stride, pads, dilation, groups, shape):
+    """lq_qconv3d_i8 (taps gathered by the tile loader from NDHWC codes) against the oracle's
+    integer Conv3d: raw accumulators, the requantize epilogue with bias and ReLU, and float32
+    output, on strides, dilations, one-sided pads, groups and every tile shape that has the gather."""
+    from lucid_amd import _ops
+    rng = np.random.default_rng(B * 100 + C + Co + sum(vol) + shape)
+    Cg = C // groups
+    x = rng.integers(-128, 128, (B, C, *vol), dtype=np.int8)
+    w = rng.integers(-127, 128, (Co, Cg, *kernel), dtype=np.int8)
+    a_zp = int(rng.integers(-100, 100))
+    a_scale = np.float32(0.021)
+    w_scale = rng.uniform(0.001, 0.01, Co).astype(np.float32)
+    bias = (rng.standard_normal(Co) * 0.5).astype(np.float32)
+    xl = hip(np.ascontiguousarray(np.transpose(x, (0, 2, 3, 4, 1))))
+    wl = hip(np.ascontiguousarray(np.transpose(w, (0, 2, 3, 4, 1))))
+    wsum = hip(w.reshape(Co, -1).astype(np.int32).sum(1).astype(np.int32))
+    common = dict(stride=stride, pad=pads, dilation=dilation, groups=groups)
+    to_ncdhw = lambda t: np.ascontiguousarray(np.moveaxis(t.numpy(), -1, 1))
+    acc = _ops.qconv3d_i8(xl, wl, a_zp=a_zp, out_mode=_ops.OUT_ACC_I32, tile_config=shape, **common)
+    want_acc = Br.qconv3d(x, w, a_zp, a_scale, w_scale, out_mode=O.OUT_ACC_I32, **common)
+    assert np.array_equal(to_ncdhw(acc), want_acc)
+    k = Cg * kernel[0] * kernel[1] * kernel[2]
+    out_scale = np.float32(0.0135 * np.sqrt(k))  # ~6 standard deviations of the float result over the grid
+    got = _ops.qconv3d_i8(xl, wl, a_zp=a_zp, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=wsum, bias=hip(bias),
+                          relu=True, out_mode=_ops.OUT_REQUANT_I8, out_scale=hip(out_scale), out_zp=hip(np.float32(3.0)),
+                          out_qmin=0, out_qmax=255, out_offset=-128, tile_config=shape, **common)
+    want = Br.qconv3d(x, w, a_zp, a_scale, w_scale, bias=bias, relu=True, out_mode=O.OUT_REQUANT_I8, out_scale=out_scale,
+                      out_zp=np.float32(3.0), out_qmin=0, out_qmax=255, out_offset=-128, **common)
+    assert np.array_equal(to_ncdhw(got), want)
+    assert want.size < 1000 or len(np.unique(want)) > 20
+    f = _ops.qconv3d_i8(xl, wl, a_zp=a_zp, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=wsum, bias=hip(bias),
+                        out_mode=_ops.OUT_F32, tile_config=shape, **common)
+    want_f = Br.qconv3d(x, w, a_zp, a_scale, w_scale, bias=bias, out_mode=O.OUT_F32, **common)
+    assert np.array_equal(to_ncdhw(f).view(np.uint32), want_f.view(np.uint32))
+
+
+def test_conv3d_loader_gather_affine_filters_and_refusals():
+    """Affine filter codes through lq_qconv3d_i8 (window sums from an all-ones filter) against
+    the oracle; channel counts the gather is not built for are refused by name."""
+    from lucid_amd import _C, _ops
+    rng = np.random.default_rng(77)
+    B, C, Co, vol, kernel = 2, 32, 40, (4, 6, 5), (3, 2, 3)
+    x = rng.integers(-128, 128, (B, C, *vol), dtype=np.int8)
+    w = rng.integers(-128, 128, (Co, C, *kernel), dtype=np.int8)
+    w_zp = rng.integers(-20, 20, Co).astype(np.int32)
+    a_zp, a_scale = -7, np.float32(0.03)
+    w_scale = rng.uniform(0.001, 0.01, Co).astype(np.float32)
+    pads = ((1, 0), (0, 1), (1, 1))
+    xl = hip(np.ascontiguousarray(np.transpose(x, (0, 2, 3, 4, 1))))
+    wl = hip(np.ascontiguousarray(np.transpose(w, (0, 2, 3, 4, 1))))
+    wsum = hip(w.reshape(Co, -1).astype(np.int32).sum(1).astype(np.int32))
+    got = _ops.qconv3d_i8(xl, wl, a_zp=a_zp, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=wsum, pad=pads,
+                          out_mode=_ops.OUT_F32, w_zp=hip(w_zp))
+    want = Br.qconv3d(x, w, a_zp, a_scale, w_scale, pad=pads, out_mode=O.OUT_F32, w_zp=w_zp)
+    assert np.array_equal(np.moveaxis(got.numpy(), -1, 1).view(np.uint32), want.view(np.uint32))
+    with pytest.raises(NotImplementedError, match=r"Cin/groups % 16 == 0 \(got 8\)"):
+        _ops.qconv3d_i8(hip(np.zeros((1, 2, 2, 2, 8), np.int8)), hip(np.zeros((4, 1, 1, 1, 8), np.int8)), a_zp=0,
+                        out_mode=_ops.OUT_ACC_I32)
+    with pytest.raises(NotImplementedError, match="no volumetric gather"):
+        _ops.qconv3d_i8(hip(np.zeros((1, 2, 2, 2, 16), np.int8)), hip(np.zeros((4, 1, 1, 1, 16), np.int8)), a_zp=0,
+                        out_mode=_ops.OUT_ACC_I32, tile_config=1)
+    with pytest.raises(_C.ShapeMismatch, match="empty output"):
+        _ops.qconv3d_i8(hip(np.zeros((1, 2, 2, 2, 16), np.int8)), hip(np.zeros((4, 3, 1, 1, 16), np.int8)), a_zp=0,
+                        out_mode=_ops.OUT_ACC_I32)
 
 
 def test_conv3d_refuses_what_it_does_not_do():
@@ -535,7 +621,7 @@ def test_conv_transpose3d_bit_exact_against_the_oracle(cin, cout, k, stride, pad
                                 dilation=three(dilation), groups=groups, bias=t3.bias.numpy(),
                                 out_mode=O.OUT_REQUANT_I8, out_scale=np.float32(t3.scale.item()),
                                 out_zp=np.float32(t3.zero_point.item()), out_qmin=0, out_qmax=255, out_offset=-128)
-    got = out._grid.codes.numpy()
+    got = volume_codes(out)
     size = [(n - 1) * s - 2 * p + d * (kk - 1) + op + 1 for n, s, p, d, kk, op in
             zip(vol, three(stride), three(padding), three(dilation), three(k), three(output_padding))]
     assert got.shape == (2, cout, *size) == want.shape
@@ -586,9 +672,57 @@ def test_conv3d_with_a_padding_mode(padding_mode):
     grid = Grid(hip((codes - 128).astype(np.int8)), hip(np.float32(in_scale)), hip(np.float32(in_zp)), Q.quint8, -128,
                 in_zp, "plain")
     y = conv(Tensor.on_grid((B, Cc, D, H, W), grid))
-    got = y._grid.codes.numpy()
+    got = volume_codes(y)
     np_mode = {"reflect": "reflect", "replicate": "edge", "circular": "wrap"}[padding_mode]
     xp = np.pad((codes - 128).astype(np.int8), ((0, 0), (0, 0), (1, 1), (2, 2), (1, 1)), mode=np_mode)
     exp = Br.qconv3d(xp, wq, in_zp - 128, in_scale, ws, bias=bias, out_mode=O.OUT_REQUANT_I8, out_scale=0.05, out_zp=120.0,
                      out_qmin=0, out_qmax=255, out_offset=-128)
     assert got.shape == exp.shape and np.array_equal(got, exp)
+
+
+def test_volumes_stay_channels_last_between_layers():
+    """QuantStub -> Conv3d -> Conv3d (reflect padding) -> ConvTranspose3d -> DeQuantStub on a video
+    batch: the stub and the first convolution leave channels-last codes, the padded layer and the
+    transposed convolution take them in either order, the float view comes out in (B, C, D, H, W)
+    order - all equal to the oracle chained layer by layer."""
+    rng = np.random.default_rng(31)
+    m = nn.Sequential(nnq.QuantStub(), nn.Conv3d(16, 32, 3, padding=1), nn.Conv3d(32, 16, (1, 3, 3), padding=(0, 1, 1)),
+                      nn.ConvTranspose3d(16, 8, 2, stride=2), nnq.DeQuantStub())
+    prepared = Q.prepare(m, Q.get_default_qconfig())
+    for _ in range(3):
+        prepared[0].activation_post_process(hip(rng.standard_normal((2, 16, 4, 6, 5)).astype(np.float32)))
+        for i, c in ((1, 32), (2, 16), (3, 8)):
+            prepared[i].activation_post_process(hip((rng.standard_normal((2, c, 2, 2, 2)) * 1.2).astype(np.float32)))
+    qm = Q.convert(prepared)
+    qm[2].padding_mode = "reflect"
+    x = rng.standard_normal((2, 16, 4, 6, 5)).astype(np.float32)
+    q0 = qm[0](hip(x))
+    assert q0._grid.layout == "nhwc" and q0._grid.codes.shape == (2, 4, 6, 5, 16)
+    s0, z0 = qm[0].scale.item(), qm[0].zero_point.item()
+    codes = O.quantize(x, s0, z0, 0, 255, code_offset=-128)
+    assert np.array_equal(volume_codes(q0), codes)
+    assert np.array_equal(q0.numpy(), (codes.astype(np.float32) + 128 - np.float32(z0)) * np.float32(s0))
+
+    def req(mod):
+        return dict(out_mode=O.OUT_REQUANT_I8, out_scale=np.float32(mod.scale.item()),
+                    out_zp=np.float32(mod.zero_point.item()), out_qmin=0, out_qmax=255, out_offset=-128)
+
+    y1 = qm[1](q0)
+    assert y1._grid.layout == "nhwc"
+    w1 = Br.qconv3d(codes, qm[1].weight_int8.numpy(), int(z0) - 128, np.float32(s0), qm[1].weight_scale.numpy(),
+                    pad=((1, 1),) * 3, bias=qm[1].bias.numpy(), **req(qm[1]))
+    assert np.array_equal(volume_codes(y1), w1)
+    y2 = qm[2](y1)
+    z1 = int(qm[1].zero_point.item()) - 128
+    w1p = np.pad(w1, ((0, 0), (0, 0), (0, 0), (1, 1), (1, 1)), mode="reflect")
+    w2 = Br.qconv3d(w1p, qm[2].weight_int8.numpy(), z1, np.float32(qm[1].scale.item()), qm[2].weight_scale.numpy(),
+                    bias=qm[2].bias.numpy(), **req(qm[2]))
+    assert np.array_equal(volume_codes(y2), w2)
+    y3 = qm[3](y2)
+    w3 = Br.qconv_transpose3d(w2, qm[3].weight_int8.numpy(), int(qm[2].zero_point.item()) - 128,
+                              np.float32(qm[2].scale.item()), qm[3].weight_scale.numpy(), stride=(2, 2, 2),
+                              bias=qm[3].bias.numpy(), **req(qm[3]))
+    assert np.array_equal(volume_codes(y3), w3)
+    out = qm(hip(x)).numpy()
+    exp = (w3.astype(np.float32) + 128 - np.float32(qm[3].zero_point.item())) * np.float32(qm[3].scale.item())
+    assert out.shape == (2, 8, 8, 12, 10) and np.array_equal(out, exp)
