@@ -64,6 +64,8 @@ int launch_tile_c10(const GemmArgs&, int, int, int, hipStream_t);
 int launch_tile_c11(const GemmArgs&, int, int, int, hipStream_t);
 int launch_tile_c12(const GemmArgs&, int, int, int, hipStream_t);
 int launch_pp_shape(const GemmArgs&, int, hipStream_t);
+bool conv_halo_applies(const GemmArgs&, int conv);
+int launch_conv_halo(const GemmArgs&, int conv, int groups, hipStream_t);
 }  // namespace lq
 
 namespace {
@@ -88,6 +90,11 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
         LQ_REQUIRE(!conv && groups == 1, LQ_ERR_VALUE, "tile_config %d is for plain GEMMs", cfg);
         LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
         return launch_pp_shape(g, cfg - 13, st);
+    case 15:
+        // stride-1 convolution with the input halo held in LDS, one block per box of outputs
+        LQ_REQUIRE(conv, LQ_ERR_VALUE, "tile_config 15 is for convolutions");
+        LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config 15 runs one block per tile");
+        return launch_conv_halo(g, conv, groups, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -205,6 +212,7 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
         cands[n++] = 5;
         if (g.N > 64) cands[n++] = 3, cands[n++] = 4;
         if (long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups < 256) cands[n++] = 9;
+        if (conv_halo_applies(g, conv)) cands[n++] = 15;
     } else {
         if (g.N <= 64) cands[n++] = 6;
         cands[n++] = 5;
@@ -221,6 +229,8 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
         if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
         if (tiles128 < 256) cands[n++] = 9;  // ... or cover the chip with 64 x 64 tiles
         if (tiles128 < 256 && g.K >= 1024) cands[n++] = 10;  // ... with 128-byte k-iterations
+        // filters with several taps at stride 1: the input halo of a box of outputs held in LDS
+        if (conv && g.K > g.cCg && conv_halo_applies(g, conv)) cands[n++] = 15;
         // whole rounds of 256 x 256 tiles plus a remainder (see launch_split)
         if (!conv && groups == 1 && g.range == nullptr && g.M >= 256) {
             const long tiles_m = (g.M + 255) / 256, tiles_n = g.N / 256;

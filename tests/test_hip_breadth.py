@@ -511,6 +511,10 @@ GATHER3D_CASES = [
     (2, 48, 288, (4, 6, 6), (3, 1, 2), (1, 1, 1), ((2, 2), (0, 0), (1, 0)), (1, 1, 3), 3, 4),
     (1, 16, 16, (2, 3, 3), (2, 2, 2), (1, 1, 1), ((0, 0), (0, 0), (0, 0)), (1, 1, 1), 1, 9),
     (2, 32, 48, (7, 7, 7), (3, 3, 3), (2, 2, 2), ((1, 1), (1, 1), (1, 1)), (1, 1, 1), 1, 9),
+    # shape 15: the box-of-outputs kernel with the input halo in LDS (stride 1, 64-channel slices)
+    (2, 64, 64, (6, 10, 10), (3, 3, 3), (1, 1, 1), ((1, 1), (1, 1), (1, 1)), (1, 1, 1), 1, 15),
+    (1, 128, 80, (5, 9, 21), (2, 3, 3), (1, 1, 1), ((0, 1), (2, 0), (1, 1)), (2, 1, 2), 2, 15),
+    (2, 128, 32, (3, 5, 4), (3, 1, 2), (1, 1, 1), ((1, 1), (0, 0), (0, 1)), (1, 1, 1), 1, 15),
 ]
 
 

@@ -383,3 +383,59 @@ def test_conv_module_with_affine_filters(groups):
                     out_zp=120.0, out_qmin=0, out_qmax=255, out_offset=-128,
                     w_zp=np.tile(wzt, groups).astype(np.int32))
     assert np.array_equal(got, exp)
+
+
+HALO_CASES = [
+    # B, H, W, Cin, Cout, KH, KW, pad(hlo,hhi,wlo,whi), dil, groups
+    (2, 28, 28, 128, 128, 3, 3, (1, 1, 1, 1), (1, 1), 1),     # ResNet 3x3, two 64-channel slices
+    (2, 56, 56, 64, 64, 3, 3, (1, 1, 1, 1), (1, 1), 1),
+    (3, 17, 13, 64, 70, 3, 3, (1, 1, 1, 1), (1, 1), 1),       # ragged box, ragged columns
+    (1, 9, 20, 128, 48, 3, 2, (0, 2, 1, 0), (2, 3), 2),       # one-sided pads, dilation, groups
+    (2, 7, 7, 192, 256, 5, 5, (2, 2, 2, 2), (1, 1), 1),       # image smaller than a box
+    (1, 40, 6, 64, 33, 1, 3, (0, 0, 1, 1), (1, 1), 1),        # width below eight
+]
+
+
+@pytest.mark.parametrize("case", HALO_CASES)
+def test_halo_kernel_exact(case):
+    """tile_config 15 - the stride-1 convolution that keeps a box's input halo in LDS - against
+    the oracle: accumulators, and the requantize / float32 / float16 / fake-quantize epilogues."""
+    B, H, W, Cin, Cout, KH, KW, pad, dil, groups = case
+    rng = np.random.default_rng(sum(case[:7]) + 15)
+    x = codes(rng, (B, H, W, Cin))
+    w = codes(rng, (Cout, KH, KW, Cin // groups))
+    a_zp = int(rng.integers(-100, 100))
+    geo = dict(stride=(1, 1), pad=pad, dilation=dil, groups=groups)
+    xd, wd = hip(x), hip(w)
+    exp = O.qconv2d(x, w, a_zp, 1.0, np.ones(Cout, np.float32), out_mode=O.OUT_ACC_I32, **geo)
+    got = _ops.qconv2d_i8(xd, wd, a_zp=a_zp, out_mode=_ops.OUT_ACC_I32, path=IMPLICIT, tile_config=15, **geo).numpy()
+    assert got.shape == exp.shape and np.array_equal(got, exp)
+    a_scale = np.float32(0.02)
+    w_scale = rng.uniform(0.0005, 0.004, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    y = O.qconv2d(x, w, a_zp, a_scale, w_scale, bias=bias, out_mode=O.OUT_F32, **geo)
+    S, Z = np.float32(np.abs(y).max() / 200 + 1e-6), np.float32(0.0)
+    dkw = dict(a_zp=a_zp, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=_ops.rowsum_i8(wd), bias=hip(bias),
+               relu=True, out_scale=hip(S), out_zp=hip(Z), out_qmin=0, out_qmax=255, out_offset=-128,
+               path=IMPLICIT, tile_config=15, **geo)
+    for mode in (_ops.OUT_REQUANT_I8, _ops.OUT_F32, _ops.OUT_F16, _ops.OUT_FAKEQUANT_F32):
+        got = _ops.qconv2d_i8(xd, wd, out_mode=mode, **dkw).numpy()
+        exp = O.qconv2d(x, w, a_zp, a_scale, w_scale, bias=bias, relu=True, out_mode=mode, out_scale=S, out_zp=Z,
+                        out_qmin=0, out_qmax=255, out_offset=-128, **geo)
+        if mode in (_ops.OUT_REQUANT_I8,):
+            assert np.array_equal(got, exp), mode
+        elif mode == _ops.OUT_F16:
+            assert np.array_equal(got.view(np.uint16), exp.view(np.uint16)), mode
+        else:
+            assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), mode
+
+
+def test_halo_kernel_refuses_what_it_is_not_built_for():
+    rng = np.random.default_rng(3)
+    x, w = hip(codes(rng, (1, 8, 8, 64))), hip(codes(rng, (64, 3, 3, 64)))
+    with pytest.raises(NotImplementedError, match="stride 1"):
+        _ops.qconv2d_i8(x, w, a_zp=0, stride=(2, 2), pad=(1, 1, 1, 1), out_mode=_ops.OUT_ACC_I32, path=IMPLICIT,
+                        tile_config=15)
+    x32, w32 = hip(codes(rng, (1, 8, 8, 32))), hip(codes(rng, (64, 3, 3, 32)))
+    with pytest.raises(NotImplementedError, match="64 == 0"):
+        _ops.qconv2d_i8(x32, w32, a_zp=0, pad=(1, 1, 1, 1), out_mode=_ops.OUT_ACC_I32, path=IMPLICIT, tile_config=15)
