@@ -587,7 +587,10 @@ typedef struct {
     int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
     int tile_config;       /* tuning: low byte 0 = choose, 1..12 = a tile shape of the
                               four-wavefront kernel, 13 / 14 = 256x352 / 256x256 tiles of
-                              the eight-wavefront kernel (plain GEMM, K % 64 == 0);
+                              the eight-wavefront kernel (plain GEMM, K % 64 == 0),
+                              15 (convolutions only) = one block per box of 256 output
+                              positions x 64 channels with the box's input halo held in
+                              LDS (stride 1, Cin/groups % 64 == 0, no join);
                               next byte 0 = choose, 1 = one block per tile,
                               2 = stream-K work split, 3 = stream-K over the
                               leftover tiles of the last round only; bits 16..30
@@ -721,7 +724,8 @@ typedef struct {
     const float* out_zp;
     int out_qmin, out_qmax, out_offset;
     void* out;             /* NDHWC [B,OD,OH,OW,Cout]                        */
-    int tile_config;       /* 0 = choose; shapes 3, 4, 5, 6, 9 have the gather */
+    int tile_config;       /* 0 = choose; shapes 3, 4, 5, 6, 9 have the gather, 15 is
+                              the halo-in-LDS kernel (see lq_qlinear_args)       */
     const int32_t* w_zp;   /* optional [Cout] zero points of affine filters, as
                               lq_qconv2d_args.w_zp                            */
 } lq_qconv3d_args;
