@@ -35,7 +35,7 @@ ACC_CASES = [
     (1, 9000, 256, SKINNY), (1, 2, 65536, SKINNY),
     # 2..16 rows with K >= 1024 (one block per compute unit's share of the rows)
     (2, 11008, 4096, SKINNY), (7, 1000, 1040, SKINNY), (16, 4099, 2048, SKINNY), (9, 16400, 1024, SKINNY),
-    (13, 33, 8192, SKINNY), (5, 12000, 1296, SKINNY),
+    (13, 33, 8192, SKINNY), (5, 12000, 1296, SKINNY), (3, 31, 6144, SKINNY), (16, 64, 2048, SKINNY), (4, 70, 1280, SKINNY), (2, 40, 16384, SKINNY), (8, 300, 8192, SKINNY),
     (5, 7, 3, NAIVE), (17, 33, 147, NAIVE), (64, 10, 250, NAIVE),
 ]
 
