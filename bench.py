@@ -477,9 +477,9 @@ def bench_vit_b16(L, _C, steps, warmup):
 
 def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     """Dynamic-quantized MLP Linear(784,256)-ReLU-Linear(256,10), batch 64
-    (launch-latency bound: 0.43 MOP).  Eager = one Python-driven forward (5
-    launches: per layer one for the activation's min / max, qparams and codes and one
-    for the GEMM, and the ReLU between); graph = the same forward replayed from a HIP graph."""
+    (launch-latency bound: 0.43 MOP).  Eager = one Python-driven forward (3
+    launches: per layer one that takes the activation's min / max, qparams and codes and
+    multiplies, and the ReLU between); graph = the same forward replayed from a HIP graph."""
     import lucid_amd.nn as nn
 
     rng = np.random.default_rng(1)
@@ -500,7 +500,7 @@ def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     assert np.isfinite(y.numpy()).all()
     g.destroy()
     return {"eager_us_per_forward": round(eager_us, 1), "graph_us_per_forward": round(graph_us, 1),
-            "launches_per_forward": 5}
+            "launches_per_forward": 3}
 
 
 def bench_weight_only(L, _C, steps, warmup, K=4096, N=11008, gs=64):

@@ -393,6 +393,18 @@ int lq_quantize_tensor_dynamic_i8(const float* x, size_t n, int symmetric, int q
                                   float eps, int code_offset, float* scale, float* zp, float* mn_out,
                                   float* mx_out, int8_t* q, lq_stream stream);
 
+/* A dynamic-quantized Linear on a small activation in ONE launch: nnqd.Linear.forward
+ * (lucid/nn/quantized/dynamic/linear.py:87-99) for x [M, K] float32 with M <= 64,
+ * K % 16 == 0 and M * K <= 65536 - the tensor's min / max, calculate_qparams, the
+ * activation codes (kept in LDS), the integer GEMM against w [N, K] int8 codes with
+ * per-row scales w_scale [N] and code sums wsum [N], float32 bias [N] or NULL, optional
+ * ReLU; out [M, N] float32.  The bits of lq_quantize_tensor_dynamic_i8 followed by
+ * lq_qlinear_i8 (mode F32).  Symmetric weights only.  Anything else:
+ * LQ_ERR_NOT_IMPLEMENTED (use the two calls). */
+int lq_dynamic_linear_small_f32(const float* x, int M, int K, const int8_t* w, int N, const float* w_scale,
+                                const int32_t* wsum, const float* bias, int relu, int symmetric, int qmin, int qmax,
+                                int is_signed, float eps, int code_offset, float* out, lq_stream stream);
+
 /* Dynamic per-row quantization in one pass: for every row of x [rows, cols],
  * min / max of the row (PerChannelMinMaxObserver with ch_axis = 0,
  * observer.py:634-653), its qparams (calculate_qparams, _qparams.py:198-215) and

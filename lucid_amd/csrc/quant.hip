@@ -758,6 +758,107 @@ int minmax_launch(const float* x, size_t outer, size_t C, size_t inner, float* m
     return LQ_OK;
 }
 
+// A whole dynamic-quantized Linear on a small activation in one launch
+// (lucid/nn/quantized/dynamic/linear.py:87-99: x.min() / x.max(), calculate_qparams, quantize,
+// dequantize-free integer GEMM, bias): every block takes the tensor's min / max and qparams and
+// quantizes x into LDS itself - x is at most 65536 floats, so repeating that per block costs less
+// than a separate launch and its round trip - but only its own 16 rows, and then computes a
+// 16 x 16 block of the output: its 16 wavefronts split the k steps of v_mfma_i32_16x16x64_i8 (activation fragments from the LDS codes,
+// weight rows from global memory), meet through LDS atomics, and one lane per output applies
+// float(acc - zp * wsum[n]) * (s * w_scale[n]) + bias[n] (and the optional ReLU) in the order of
+// the GEMM's epilogue.  Same bits as lq_quantize_tensor_dynamic_i8 followed by lq_qlinear_i8.
+__global__ __launch_bounds__(1024) void dynamic_linear_small_kernel(
+    const float* __restrict__ x, int M, int K, const int8_t* __restrict__ w, int N, const float* __restrict__ w_scale,
+    const int32_t* __restrict__ wsum, const float* __restrict__ bias, int relu, int symmetric, int qmin, int qmax,
+    int is_signed, float eps, float half_range, int off, float* __restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) int8_t dl_smem[];
+    __shared__ float s_sz[2];
+    typedef int dl_v4i __attribute__((ext_vector_type(4)));
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int8_t* const codes = dl_smem;                                     // [16][K]: the block's rows
+    int* const red = reinterpret_cast<int*>(dl_smem + size_t(16) * K);  // [4][64]
+    constexpr int kKeep = 16;
+    const int quads = (M * K) >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    // What does not depend on x is requested first, so that it arrives under the quantization: the
+    // wavefront's first weight fragment and the output lane's column parameters.
+    const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+    const int ln = lane & 15, lg = lane >> 4;
+    const int8_t* wrow = w + size_t(n0 + ln < N ? n0 + ln : N - 1) * size_t(K);
+    const int ksteps = (K + 63) >> 6;
+    const bool first_in_k = wave < ksteps && wave * 64 + lg * 16 < K;
+    const dl_v4i wf_first = first_in_k ? *reinterpret_cast<const dl_v4i*>(wrow + wave * 64 + lg * 16) : dl_v4i{0, 0, 0, 0};
+    const int out_n = n0 + (tid & 15);
+    const bool out_lane = tid < 256 && out_n < N;
+    const float c_ws = (out_lane && w_scale) ? w_scale[out_n] : 1.0f;
+    const int c_wsum = (out_lane && wsum) ? wsum[out_n] : 0;
+    const float c_bias = (out_lane && bias) ? bias[out_n] : -0.0f;
+    MinMax m{__builtin_inff(), -__builtin_inff(), 0};
+    float4 v[kKeep];
+#pragma unroll
+    for (int u = 0; u < kKeep; ++u) {
+        const int i = u * 1024 + tid;
+        if (i < quads) v[u] = x4[i];
+    }
+    if (tid < 256) red[tid] = 0;
+    // the block's rows m0 .. m0+15 are a contiguous range of quads; rows past M (the last block's padding)
+    // feed accumulator rows that are never stored
+    const int q_lo = (m0 * K) >> 2;
+    const int q_hi = ((m0 + 16 < M ? m0 + 16 : M) * K) >> 2;
+    for (int i = q_hi - q_lo + tid; i < 4 * K; i += 1024) reinterpret_cast<unsigned*>(codes)[i] = 0u;
+#pragma unroll
+    for (int u = 0; u < kKeep; ++u)
+        if (u * 1024 + tid < quads) mm_update(m, v[u].x), mm_update(m, v[u].y), mm_update(m, v[u].z), mm_update(m, v[u].w);
+    m = mm_block_reduce(m);
+    if (tid == 0) {
+        const float qnan = __builtin_nanf("");
+        float s, z;
+        qparams_of(m.nan ? qnan : m.lo, m.nan ? qnan : m.hi, symmetric, qmin, qmax, is_signed, eps, half_range, &s, &z);
+        s_sz[0] = s, s_sz[1] = z;
+    }
+    __syncthreads();
+    const float s = s_sz[0], z = s_sz[1], r = 1.0f / s;
+    const QuantizeOp<int8_t> op{x4, reinterpret_cast<Code8x4*>(codes), float(double(qmin)), float(double(qmax)), off};
+#pragma unroll
+    for (int u = 0; u < kKeep; ++u) {
+        const int i = u * 1024 + tid;
+        if (i >= q_lo && i < q_hi) op.q[i - q_lo] = op.pack(v[u], s, z, r);
+    }
+    __syncthreads();
+
+    dl_v4i acc = dl_v4i{0, 0, 0, 0};
+    for (int ks = wave; ks < ksteps; ks += 16) {
+        const int k = ks * 64 + lg * 16;
+        const bool in_k = k < K;  // K % 16 == 0: a 16-byte chunk is inside or outside as a whole
+        const dl_v4i wf = ks == wave ? wf_first : (in_k ? *reinterpret_cast<const dl_v4i*>(wrow + k) : dl_v4i{0, 0, 0, 0});
+        const dl_v4i af = in_k ? *reinterpret_cast<const dl_v4i*>(codes + size_t(ln) * K + k) : dl_v4i{0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc, 0, 0, 0);
+    }
+    if (wave < ksteps) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            __hip_atomic_fetch_add(&red[q * 64 + lane], acc[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
+    // red[q * 64 + lane]: activation row m0 + 4 (lane / 16) + q, weight row n0 + lane % 16
+    if (tid < 256) {
+        const int q = tid >> 6, l = tid & 63;
+        const int mm = m0 + 4 * (l >> 4) + q, nn = n0 + (l & 15);
+        if (mm < M && nn < N) {
+            // GEMM epilogue, float32 output form: the zero point enters as an integer, the steps stay separate
+            const int zp = int(z) + off;
+            const int corr = (wsum != nullptr && zp != 0) ? zp * c_wsum : 0;
+            const float f = float(red[tid] - corr);
+            const float sc = s * c_ws;
+            float y = f * sc;
+            y = y + c_bias;
+            const float floor = relu ? 0.0f : -__builtin_inff();
+            y = (y < floor) ? floor : y;
+            out[size_t(mm) * N + nn] = y;
+        }
+    }
+}
+
 }  // namespace
 
 namespace lq {
@@ -782,6 +883,35 @@ int lq_quantize_tensor_dynamic_i8(const float* x, size_t n, int symmetric, int q
     hipLaunchKernelGGL(quantize_tensor_dynamic_kernel, dim3(1), dim3(1024), 0, as_stream(stream), x, n, symmetric,
                        qmin, qmax, is_signed, eps, half_range, code_offset, scale, zp, mn_out, mx_out, q);
     LQ_CHECK_LAUNCH("quantize_tensor_dynamic");
+    return LQ_OK;
+}
+
+int lq_dynamic_linear_small_f32(const float* x, int M, int K, const int8_t* w, int N, const float* w_scale,
+                                const int32_t* wsum, const float* bias, int relu, int symmetric, int qmin, int qmax,
+                                int is_signed, float eps, int code_offset, float* out, lq_stream stream) {
+    if (M == 0 || N == 0) return LQ_OK;
+    LQ_REQUIRE(x && w && out, LQ_ERR_VALUE, "dynamic_linear_small: NULL pointer");
+    LQ_REQUIRE(qmax > qmin && qmin + code_offset >= -128 && qmax + code_offset <= 127, LQ_ERR_VALUE,
+               "dynamic_linear_small: grid [%d,%d] + offset %d does not fit int8", qmin, qmax, code_offset);
+    LQ_REQUIRE(M > 0 && M <= 64 && K >= 16 && K % 16 == 0 && long(M) * K <= 65536 && K <= 33025 && N > 0 &&
+                   aligned16(x) && aligned16(w),
+               LQ_ERR_NOT_IMPLEMENTED,
+               "dynamic_linear_small: takes up to 64 rows, K %% 16 == 0, at most 65536 activations and 16-byte "
+               "aligned operands (got M = %d, K = %d); use lq_quantize_tensor_dynamic_i8 + lq_qlinear_i8", M, K);
+    const float half_range = float((double(qmax) - double(qmin)) / 2.0);
+    const int tiles = (M + 15) / 16;
+    const size_t lds = size_t(16) * K + 256 * sizeof(int);
+    static bool attr_set = false;
+    if (!attr_set) {
+        LQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dynamic_linear_small_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(dynamic_linear_small_kernel, dim3(unsigned((N + 15) / 16), unsigned(tiles)), dim3(1024), lds,
+                       as_stream(stream), x,
+                       M, K, w, N, w_scale, wsum, bias, relu, symmetric, qmin, qmax, is_signed, eps, half_range,
+                       code_offset, out);
+    LQ_CHECK_LAUNCH("dynamic_linear_small");
     return LQ_OK;
 }
 

@@ -63,6 +63,17 @@ class Linear(Module):
         M = x.numel // K
         qd = self.act_qdtype
         off = storage_offset(qd)
+        if (x._range is None and residual is None and activation is None and not track_range and 0 < M <= 64
+                and K % 16 == 0 and M * K <= 65536 and weight_zero_points(self) is None
+                and (self.bias is None or self.bias.dtype == T.float32)):
+            # a small activation: min / max, qparams, codes, GEMM and bias in one launch (same bits)
+            if self._wsum is None:
+                self._wsum = _ops.rowsum_i8(self.weight_int8)
+            y = Tensor.empty((M, N), T.float32, "hip")
+            _C.call("lq_dynamic_linear_small_f32", x.data_ptr, M, K, self.weight_int8.data_ptr, N,
+                    self.weight_scale.data_ptr, self._wsum.data_ptr, None if self.bias is None else self.bias.data_ptr,
+                    0, 0, qd.quant_min, qd.quant_max, int(qd.signed), 1e-8, off, y.data_ptr, None)
+            return y.reshape(*x.shape[:-1], N)
         xq = Tensor.empty((M, K), T.int8, "hip")
         small = x._range is None and x.numel <= (1 << 18)
         if small:

@@ -449,3 +449,46 @@ def test_engine_toggle():
         assert not backends.quantized.use_mlx()
     finally:
         backends.quantized.engine = prev
+
+
+@pytest.mark.parametrize("M,K,N", [(64, 784, 256), (64, 256, 10), (1, 16, 1), (17, 48, 33), (5, 1024, 70), (64, 1024, 16),
+                                   (33, 1040, 100)])
+@pytest.mark.parametrize("kind", ["normal", "constant", "nan"])
+def test_small_dynamic_linear_in_one_launch(M, K, N, kind):
+    """lq_dynamic_linear_small_f32 (min / max, qparams, codes, GEMM and bias of nnqd.Linear in one
+    launch) gives the bits of lq_quantize_tensor_dynamic_i8 followed by lq_qlinear_i8, and of the
+    oracle's integer formulation, on ragged shapes, a constant input (scale at eps) and a NaN."""
+    from lucid_amd import _C, _ops
+    rng = np.random.default_rng(M * 3 + K + N)
+    x = rng.standard_normal((M, K)).astype(np.float32) * 3
+    if kind == "constant":
+        x[:] = 0.0
+    elif kind == "nan":
+        x[M // 2, K // 3] = np.nan
+    w = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    xd, wd, wsd, bd = hip(x), hip(w), hip(ws), hip(b)
+    wsum = _ops.rowsum_i8(wd)
+    for relu, bias in ((0, bd), (1, bd), (0, None)):
+        y = L.Tensor.empty((M, N), L.float32, "hip")
+        _C.call("lq_dynamic_linear_small_f32", xd.data_ptr, M, K, wd.data_ptr, N, wsd.data_ptr, wsum.data_ptr,
+                None if bias is None else bias.data_ptr, relu, 0, 0, 255, 0, 1e-8, -128, y.data_ptr, None)
+        xq = L.Tensor.empty((M, K), L.int8, "hip")
+        s, z = L.Tensor.empty((), L.float32, "hip"), L.Tensor.empty((), L.float32, "hip")
+        _C.call("lq_quantize_tensor_dynamic_i8", xd.data_ptr, M * K, 0, 0, 255, 0, 1e-8, -128, s.data_ptr, z.data_ptr,
+                None, None, xq.data_ptr, None)
+        two = _ops.qlinear_i8(xq, wd, a_zp=-128, a_zp_dev=z, a_scale=s, w_scale=wsd, wsum=wsum, bias=bias,
+                              relu=bool(relu), out_mode=_ops.OUT_F32)
+        got, want = y.numpy(), two.numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(got[~np.isnan(got)].view(np.uint32), want[~np.isnan(want)].view(np.uint32))
+        if kind == "normal" and relu == 0 and bias is not None:
+            mn, mx = O.minmax(x)
+            xs, xz = O.calc_qparams(mn, mx, False, 0, 255, False)
+            codes = O.quantize(x, xs, xz, 0, 255, code_offset=-128)
+            exp = O.qlinear(codes, w, int(xz[0]) - 128, xs, ws, bias=b, out_mode=O.OUT_F32)
+            assert np.array_equal(got.view(np.uint32), exp.view(np.uint32))
+    with pytest.raises(NotImplementedError, match="up to 64 rows"):
+        _C.call("lq_dynamic_linear_small_f32", xd.data_ptr, 65, K, wd.data_ptr, N, wsd.data_ptr, wsum.data_ptr, None, 0, 0,
+                0, 255, 0, 1e-8, -128, y.data_ptr, None)
