@@ -91,10 +91,17 @@ int lq_d2d_rows(void* dst_dev, size_t dst_pitch, const void* src_dev, size_t src
 int lq_fill_bytes(void* dst_dev, int value, size_t nbytes, lq_stream stream);
 int lq_sync(lq_stream stream);
 int lq_stream_create(lq_stream* stream);
+/* A stream that does not synchronise implicitly with the default stream (hipStreamNonBlocking,
+ * default priority): work on several of them overlaps even while the default stream is in use;
+ * order them with events (lq_event_record / lq_stream_wait_event). */
+int lq_stream_create_nonblocking(lq_stream* stream);
 int lq_stream_destroy(lq_stream stream);
 int lq_event_create(lq_event* ev);
 int lq_event_destroy(lq_event ev);
 int lq_event_record(lq_event ev, lq_stream stream);
+/* Work queued on `stream` after this call waits for `ev` (hipStreamWaitEvent): the
+ * fork / join of forwards that run on several streams at once. */
+int lq_stream_wait_event(lq_stream stream, lq_event ev);
 int lq_event_sync(lq_event ev);
 int lq_event_elapsed_ms(lq_event start, lq_event stop, float* ms);
 

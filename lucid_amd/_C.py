@@ -86,11 +86,13 @@ _SIGNATURES = {
     "lq_fill_bytes": [_vp, _i, _sz, _vp],
     "lq_sync": [_vp],
     "lq_stream_create": [C.POINTER(_vp)],
+    "lq_stream_create_nonblocking": [C.POINTER(_vp)],
     "lq_stream_destroy": [_vp],
     "lq_event_create": [C.POINTER(_vp)],
     "lq_event_destroy": [_vp],
     "lq_event_record": [_vp, _vp],
     "lq_event_sync": [_vp],
+    "lq_stream_wait_event": [_vp, _vp],
     "lq_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "lq_op_count": [],
     "lq_op_info": [_i, C.POINTER(C.c_char_p), C.POINTER(_i), C.POINTER(_i)],

@@ -102,8 +102,11 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
 // Shape chosen from the problem size alone: 128 x 256 tiles keep two blocks per
 // CU busy; narrower tiles when N is small or when the wide ones would leave
 // most of the 256 CUs without work.
-int heuristic_tile_shape(const GemmArgs& g, int groups) {
+int heuristic_tile_shape(const GemmArgs& g, int conv, int groups) {
     const long mt128 = (g.M + 127) / 128;
+    // far fewer 128 x 128 tiles than CUs (a small batch in the late stages of a network): 64 x 64
+    // tiles, four blocks per CU, with 128-byte k steps when K is long (plain and 2-d only)
+    if (mt128 * ((g.N + 127) / 128) * groups < 128) return (g.K >= 1024 && conv != 2) ? 10 : 9;
     if (g.N <= 64) return 6;
     if (g.N <= 128 || mt128 * ((g.N + 255) / 256) * groups < 256) return 5;
     return 4;
@@ -191,7 +194,7 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
             return LQ_OK;
         }
     }
-    int fallback = heuristic_tile_shape(g, groups);
+    int fallback = heuristic_tile_shape(g, conv, groups);
     *cfg_out = fallback;
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     LQ_HIP(hipStreamIsCapturing(st, &capturing));
@@ -202,7 +205,7 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
     // once per timing launch)
     const bool in_place = (g.residual && static_cast<const void*>(g.residual) == g.out) ||
                           (g.join_q && static_cast<const void*>(g.join_q) == g.out);
-    if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 2e9 || in_place) return LQ_OK;
+    if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 5e8 || in_place) return LQ_OK;
 
     // candidates are whole tile_config values (shape | schedule << 8)
     int cands[20], n = 0;

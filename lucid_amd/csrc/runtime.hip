@@ -434,6 +434,14 @@ int lq_stream_create(lq_stream* stream) {
     return LQ_OK;
 }
 
+int lq_stream_create_nonblocking(lq_stream* stream) {
+    LQ_REQUIRE(stream, LQ_ERR_VALUE, "stream is NULL");
+    hipStream_t s;
+    LQ_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
+    *stream = s;
+    return LQ_OK;
+}
+
 int lq_stream_destroy(lq_stream stream) {
     if (!stream) return LQ_OK;
     {
@@ -469,6 +477,12 @@ int lq_event_destroy(lq_event ev) {
 
 int lq_event_record(lq_event ev, lq_stream stream) {
     LQ_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(ev), as_stream(stream)));
+    return LQ_OK;
+}
+
+int lq_stream_wait_event(lq_stream stream, lq_event ev) {
+    LQ_REQUIRE(ev, LQ_ERR_VALUE, "stream_wait_event: event is NULL");
+    LQ_HIP(hipStreamWaitEvent(as_stream(stream), reinterpret_cast<hipEvent_t>(ev), 0));
     return LQ_OK;
 }
 

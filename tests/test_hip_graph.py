@@ -66,6 +66,33 @@ def test_resnet50_graph_replay_matches_eager():
     assert np.array_equal(model(L.tensor(batches[1], device="hip")).numpy(), eager[1])
 
 
+@pytest.mark.parametrize("batch,parts", [(6, 2), (7, 3), (4, 4)])
+def test_batch_split_replay_on_several_streams_matches_eager(batch, parts):
+    """graph.capture_split: the forward captured once per slice of the batch, each on its own stream,
+    replayed together - the concatenated result equals one eager forward of the whole batch, replay
+    after replay, with eager work between the replays and with new input in the same buffer."""
+    model = W.QResNet50()
+    rng = np.random.default_rng(batch)
+    batches = [rng.uniform(0, 1, (batch, 3, 64, 64)).astype(np.float32) for _ in range(3)]
+    eager = [model(L.tensor(b, device="hip")).numpy() for b in batches]
+    x = L.tensor(batches[0], device="hip")
+    bounds = [batch * i // parts for i in range(parts + 1)]
+    for lo, hi in zip(bounds[:-1], bounds[1:]):
+        model(x.row_range(lo, hi))  # every slice size once, eagerly
+    sg = L.graph.capture_split(model, x, parts)
+    assert len(sg.graphs) == parts and sg.output.shape == eager[0].shape
+    for rep in range(2):
+        for i, b in enumerate(batches):
+            x.copy_from(b)
+            sg.replay()
+            junk = L.tensor(rng.standard_normal(30000).astype(np.float32), device="hip")
+            assert np.isfinite(junk.numpy()).all()
+            L.synchronize()
+            assert np.array_equal(sg.output.numpy(), eager[i]), (rep, i)
+    sg.destroy()
+    assert np.array_equal(model(L.tensor(batches[1], device="hip")).numpy(), eager[1])
+
+
 def test_capture_needs_a_created_stream():
     gid = C.c_int()
     with pytest.raises(ValueError):
