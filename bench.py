@@ -447,9 +447,9 @@ def bench_resnet50(L, _C, steps, warmup):
     assert np.isfinite(ref).all()
     g.destroy()
     if not EAGER_ONLY:
-        # the same batch as two halves, each captured into its own graph and replayed on its own
-        # stream at the same time: a forward is ~60 short dependent launches, and one half's
-        # ramp-up and drain gaps are filled by the other's kernels.  Same result, bit for bit
+        # the same batch as two halves, captured as two parallel branches of one graph: a forward is
+        # ~60 short dependent launches, and one half's ramp-up and drain gaps are filled by the
+        # other's kernels.  Same result, bit for bit
         # (static quantization: an image's result does not depend on its neighbours).
         model(x.row_range(0, batch // 2))
         sg = L.graph.capture_split(model, x, 2)
@@ -463,7 +463,7 @@ def bench_resnet50(L, _C, steps, warmup):
         if ms2 < ms:
             out.update({"images_per_s": round(batch / ms2 * 1e3, 1), "ms_per_batch": round(ms2, 4),
                         "int8_TOP/s": round(2 * gmacs / ms2, 2), "p95_ms": round(float(np.percentile(per2, 95)), 4),
-                        "launch": "two hip graphs (batch halves) replayed on two streams"})
+                        "launch": "hip graph replay, batch halves as two parallel branches"})
     return out
 
 

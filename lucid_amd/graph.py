@@ -86,46 +86,36 @@ def capture():
 
 
 class SplitGraph:
-    """A forward captured once per contiguous slice of the batch, each slice on a stream of its own,
-    replayed together.  A chain of short dependent kernels leaves most of the chip idle while each
-    kernel ramps up and drains; independent slices of the batch fill those gaps for one another.
+    """A forward captured once per contiguous slice of the batch, the slices as parallel branches of
+    ONE graph (each captured on a stream of its own, forked from and joined to the capture stream
+    by events).  A chain of short dependent kernels leaves most of the chip idle while each kernel
+    ramps up and drains; independent slices of the batch fill those gaps for one another.
 
     Only for forwards whose result for a row does not depend on the other rows of the batch
     (static quantization; NOT dynamic per-tensor quantization, whose ranges are taken over the
     whole batch).  ``output`` holds the slices' results, concatenated along axis 0."""
 
     def __init__(self) -> None:
-        self.graphs: list[Graph] = []
+        self.graph: Graph | None = None
+        self.branches = 0
         self.output = None
-        self._fork = None
-        self._joins: list = []
-        self._streams: list = []  # replay streams: non-blocking, so the slices overlap even next to the default stream
+        self._events: list = []
+        self._streams: list = []
 
     def replay(self) -> None:
-        """Launch every slice's graph on its own stream; work queued on the current stream
-        afterwards waits for all of them."""
-        cur = _C.current_stream()
-        _C.call("lq_event_record", self._fork, cur)
-        # every slice is launched before the current stream is touched again: when that is the
-        # default stream, each operation on it orders all the other streams' later work behind it
-        for g, st, ev in zip(self.graphs, self._streams, self._joins):
-            _C.call("lq_stream_wait_event", st, self._fork)
-            _C.call("lq_graph_launch", g.id, st)
-            _C.call("lq_event_record", ev, st)
-        for ev in self._joins:
-            _C.call("lq_stream_wait_event", cur, ev)
+        if self.graph is None:
+            raise _C.LucidError("graph was not captured")
+        self.graph.replay()
 
     def destroy(self) -> None:
-        for g in self.graphs:
-            g.destroy()
-        self.graphs = []
-        for ev in [self._fork, *self._joins]:
-            if ev is not None:
-                _C.call("lq_event_destroy", ev)
-        self._fork, self._joins = None, []
+        if self.graph is not None:
+            self.graph.destroy()
+            self.graph = None
+        for ev in self._events:
+            _C.call("lq_event_destroy", ev)
         for st in self._streams:
             _C.call("lq_stream_destroy", st)
-        self._streams = []
+        self._events, self._streams = [], []
 
     def __del__(self):
         try:
@@ -135,35 +125,55 @@ class SplitGraph:
 
 
 def capture_split(fn, x, parts: int = 2) -> SplitGraph:
-    """Capture ``fn`` on ``parts`` contiguous slices of ``x`` along axis 0 (see ``SplitGraph``).
-    ``fn(x_slice)`` returns one device tensor whose axis 0 is the slice's batch.  Run ``fn`` on
-    each slice size once before capturing (host-side scalars, kernel tuning)."""
+    """Capture ``fn`` on ``parts`` contiguous slices of ``x`` along axis 0 as parallel branches of one
+    graph (see ``SplitGraph``).  ``fn(x_slice)`` returns one device tensor whose axis 0 is the
+    slice's batch.  Run ``fn`` on each slice size once before capturing (host-side scalars, kernel
+    tuning)."""
     from ._tensor import Tensor
 
     batch = x.shape[0]
     parts = max(1, min(int(parts), batch))
     bounds = [batch * i // parts for i in range(parts + 1)]
     sg = SplitGraph()
-    ev = C.c_void_p()
-    _C.call("lq_event_create", C.byref(ev))
-    sg._fork = ev
+    sg.branches = parts
+
+    def new_event():
+        ev = C.c_void_p()
+        _C.call("lq_event_create", C.byref(ev))
+        sg._events.append(ev)
+        return ev
+
     try:
-        for lo, hi in zip(bounds[:-1], bounds[1:]):
-            xs = x.row_range(lo, hi)
-            with capture() as g:
-                y = fn(xs)
-                if sg.output is None:
-                    # allocated during the first capture, so it stays pinned like the other captured tensors
-                    sg.output = Tensor.empty((batch, *y.shape[1:]), y.dtype, "hip")
-                dst = sg.output.row_range(lo, hi)
-                _C.call("lq_d2d", dst.data_ptr, y.data_ptr, y.nbytes, _C.current_stream())
-            sg.graphs.append(g)
-            j = C.c_void_p()
-            _C.call("lq_event_create", C.byref(j))
-            sg._joins.append(j)
+        fork = new_event()
+        for _ in range(parts - 1):
             st = C.c_void_p()
-            _C.call("lq_stream_create_nonblocking", C.byref(st))
+            _C.call("lq_stream_create", C.byref(st))
             sg._streams.append(st)
+        with capture() as g:
+            main = _C.current_stream()
+            _C.call("lq_event_record", fork, main)
+            joins = []
+            try:
+                for i, (lo, hi) in enumerate(zip(bounds[:-1], bounds[1:])):
+                    st = main if i == 0 else sg._streams[i - 1]
+                    if i:
+                        _C.call("lq_stream_wait_event", st, fork)  # the stream joins the capture here
+                    _C.set_current_stream(st)
+                    y = fn(x.row_range(lo, hi))
+                    if sg.output is None:
+                        # allocated during the capture, so it stays pinned like the other captured tensors
+                        sg.output = Tensor.empty((batch, *y.shape[1:]), y.dtype, "hip")
+                    dst = sg.output.row_range(lo, hi)
+                    _C.call("lq_d2d", dst.data_ptr, y.data_ptr, y.nbytes, st)
+                    if i:
+                        join = new_event()
+                        _C.call("lq_event_record", join, st)
+                        joins.append(join)
+            finally:
+                _C.set_current_stream(main)
+            for join in joins:
+                _C.call("lq_stream_wait_event", main, join)
+        sg.graph = g
     except Exception:
         sg.destroy()
         raise

@@ -68,8 +68,8 @@ def test_resnet50_graph_replay_matches_eager():
 
 @pytest.mark.parametrize("batch,parts", [(6, 2), (7, 3), (4, 4)])
 def test_batch_split_replay_on_several_streams_matches_eager(batch, parts):
-    """graph.capture_split: the forward captured once per slice of the batch, each on its own stream,
-    replayed together - the concatenated result equals one eager forward of the whole batch, replay
+    """graph.capture_split: the forward captured once per slice of the batch, as parallel branches of
+    one graph - the concatenated result equals one eager forward of the whole batch, replay
     after replay, with eager work between the replays and with new input in the same buffer."""
     model = W.QResNet50()
     rng = np.random.default_rng(batch)
@@ -80,7 +80,7 @@ def test_batch_split_replay_on_several_streams_matches_eager(batch, parts):
     for lo, hi in zip(bounds[:-1], bounds[1:]):
         model(x.row_range(lo, hi))  # every slice size once, eagerly
     sg = L.graph.capture_split(model, x, parts)
-    assert len(sg.graphs) == parts and sg.output.shape == eager[0].shape
+    assert sg.branches == parts and sg.output.shape == eager[0].shape
     for rep in range(2):
         for i, b in enumerate(batches):
             x.copy_from(b)
