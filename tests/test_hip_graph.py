@@ -203,6 +203,39 @@ def test_failed_capture_releases_its_blocks():
     g.destroy()
 
 
+def test_failed_split_capture_releases_its_blocks_and_streams():
+    """capture_split whose forward raises on the second slice (a branch stream has joined the
+    capture and is never joined back): the error reaches the caller, the blocks allocated during
+    the capture are released, and a following capture_split works."""
+    import gc
+    _C.init()
+    gc.collect()
+    x = L.tensor(np.arange(8 * 4096, dtype=np.float32).reshape(8, 4096) - 9000.0, device="hip")
+    calls = []
+
+    def relu(xs, fail_on=None):
+        calls.append(xs.shape[0])
+        if fail_on is not None and len(calls) == fail_on:
+            raise RuntimeError("boom")
+        y = L.Tensor.empty(xs.shape, L.float32, "hip")
+        _C.call("lq_relu_f32", xs.data_ptr, y.data_ptr, xs.numel, None)
+        return y
+
+    used0 = _stats()[0]
+    with pytest.raises(RuntimeError, match="boom"):
+        L.graph.capture_split(lambda xs: relu(xs, fail_on=2), x, 2)
+    gc.collect()
+    assert _stats()[0] == used0
+    assert _C.current_stream() is None
+    calls.clear()
+    sg = L.graph.capture_split(relu, x, 3)
+    assert calls == [2, 3, 3]
+    sg.replay()
+    L.synchronize()
+    assert np.array_equal(sg.output.numpy(), np.maximum(x.numpy(), 0.0))
+    sg.destroy()
+
+
 def test_vit_b16_batch64_graph_replay_matches_eager():
     """The serving configuration of the ViT bench: a captured forward of ViT-B/16 at batch 64
     gives the eager logits bit for bit on every replay, for several batches, with eager work
