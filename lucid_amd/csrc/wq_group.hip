@@ -187,10 +187,21 @@ __global__ __launch_bounds__(256) void wq_gemv1_kernel(const float* x, const uin
         uint4 w[RW];
         float s[RW], b[RW];
     };
+    // Scales and biases of the wavefront's rows.  With at most 64 groups per row (and RW = 4) they
+    // come in two wavefront-wide direct loads into LDS - 16 lanes x 16 bytes per row and array -
+    // instead of two 4-byte loads per row and step: a load instruction costs the memory pipeline
+    // about the same whatever it carries.  Layout: sb[wave][array][row][64].
+    const bool sb_lds = RW == 4 && groups_per_row <= 64 && groups_per_row % 4 == 0 &&
+                        ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 15u) == 0;
+    float* const sb = sx + K + wave * 512;
     auto fetch = [&](int step, Operands& o) {
         const int L = step * 64 + lane, g = (L * CODES) >> gs_shift;  // group sizes are powers of two
 #pragma unroll
-        for (int r = 0; r < RW; ++r) o.w[r] = wrow[r][L], o.s[r] = srow[r][g], o.b[r] = brow[r][g];
+        for (int r = 0; r < RW; ++r) o.w[r] = wrow[r][L];
+        if (!sb_lds) {
+#pragma unroll
+            for (int r = 0; r < RW; ++r) o.s[r] = srow[r][g], o.b[r] = brow[r][g];
+        }
     };
     auto pin = [] {
         asm volatile("" ::: "memory");
@@ -198,18 +209,35 @@ __global__ __launch_bounds__(256) void wq_gemv1_kernel(const float* x, const uin
     };
     Operands o0, o1;
     fetch(0, o0);
+    if (sb_lds) {
+        const int r = lane >> 4;
+        int part = (lane & 15) * 4;
+        part = part < groups_per_row ? part : groups_per_row - 4;  // lanes past the row's groups repeat its last four
+        typedef __attribute__((address_space(1))) void* gptr;
+        typedef __attribute__((address_space(3))) void* lptr;
+        __builtin_amdgcn_global_load_lds((gptr)(srow[r % RW] + part), (lptr)(sb), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr)(brow[r % RW] + part), (lptr)(sb + 256), 16, 0, 0);
+    }
     pin();
     for (int i = tid * 4; i < K; i += 256 * 4) {
         const float4 v = *reinterpret_cast<const float4*>(x + i);
         const int L = i / CODES, j = (i % CODES) / 4;
         *reinterpret_cast<float4*>(sx + (j * chunks + L) * 4) = v;
     }
+    // the activation loads above are younger than the direct loads: once they have been consumed (they
+    // were, by the LDS stores), the scales and biases have landed as well
+    __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 8));  // vmcnt(0)
     __syncthreads();
     float acc[RW];
 #pragma unroll
     for (int r = 0; r < RW; ++r) acc[r] = 0.0f;
-    auto compute = [&](int step, const Operands& o) {
+    auto compute = [&](int step, Operands& o) {
         const int L = step * 64 + lane;
+        if (sb_lds) {
+            const int g = (L * CODES) >> gs_shift;
+#pragma unroll
+            for (int r = 0; r < RW; ++r) o.s[r] = sb[r * 64 + g], o.b[r] = sb[256 + r * 64 + g];
+        }
         float dot[RW], sum = 0.0f;
 #pragma unroll
         for (int r = 0; r < RW; ++r) dot[r] = 0.0f;
@@ -221,10 +249,21 @@ __global__ __launch_bounds__(256) void wq_gemv1_kernel(const float* x, const uin
             for (int r = 0; r < RW; ++r) {
                 const uint32_t words[4] = {o.w[r].x, o.w[r].y, o.w[r].z, o.w[r].w};
                 float c[4];
+                if (BITS == 4) {
+                    // the even nibbles of a word as the bytes of `lo`, the odd ones as the bytes of `hi`
+                    // (three instructions per eight codes), then one byte-to-float conversion per code:
+                    // five instructions less per word than a bit-field extract and a conversion per code
+                    const uint32_t word = words[quad >> 1];
+                    const uint32_t lo = word & 0x0f0f0f0fu, hi = (word >> 4) & 0x0f0f0f0fu;
+                    const int sh = (quad & 1) * 16;  // a constant once the quad loop is unrolled
+                    c[0] = float((lo >> sh) & 0xffu), c[1] = float((hi >> sh) & 0xffu);
+                    c[2] = float((lo >> (sh + 8)) & 0xffu), c[3] = float((hi >> (sh + 8)) & 0xffu);
+                } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int j = quad * 4 + e;  // code index inside the 16-byte load
-                    c[e] = float((words[j * BITS / 32] >> ((j * BITS) % 32)) & MASK);
+                    for (int e = 0; e < 4; ++e) {
+                        const int j = quad * 4 + e;  // code index inside the 16-byte load
+                        c[e] = float((words[j * BITS / 32] >> ((j * BITS) % 32)) & MASK);
+                    }
                 }
                 // fused multiply-adds by name (contraction is off for this library): the decode
                 // loop is bound by vector instructions, not by memory
@@ -264,7 +303,7 @@ __global__ __launch_bounds__(256) void wq_gemv1_kernel(const float* x, const uin
 template <int BITS>
 int launch_gemv1(const float* x, const uint32_t* packed, const float* scales, const float* biases, int N, int K,
                  int gs, float* out, hipStream_t st) {
-    const size_t smem = size_t(K) * sizeof(float);
+    const size_t smem = size_t(K) * sizeof(float) + 4 * 512 * sizeof(float);  // x, then scales / biases per wavefront
     const void* fn = reinterpret_cast<const void*>(wq_gemv1_kernel<BITS>);
     static size_t attr = 0;
     if (smem > attr) {
