@@ -61,3 +61,44 @@ def test_two_streams_share_no_scratch():
             assert mn.numpy()[0] == xs[i].min() and mx.numpy()[0] == xs[i].max(), i
     for s in streams:
         _C.call("lq_stream_destroy", s)
+
+
+def test_fork_and_join_with_events_on_non_blocking_streams():
+    """lq_stream_create_nonblocking + lq_event_record / lq_stream_wait_event: work forked from the
+    default stream onto two streams that do not synchronise with it implicitly, joined back by
+    events - the consumer on the default stream sees both results."""
+    _C.init()
+    rng = np.random.default_rng(5)
+    n = 1 << 20
+    x = L.tensor(rng.standard_normal(2 * n).astype(np.float32), device="hip")
+    y = L.Tensor.empty((2 * n,), L.float32, "hip")
+    streams, joins = [], []
+    for _ in range(2):
+        s, e = C.c_void_p(), C.c_void_p()
+        _C.call("lq_stream_create_nonblocking", C.byref(s))
+        _C.call("lq_event_create", C.byref(e))
+        streams.append(s)
+        joins.append(e)
+    fork = C.c_void_p()
+    _C.call("lq_event_create", C.byref(fork))
+    try:
+        for rep in range(3):
+            x.copy_from(rng.standard_normal(2 * n).astype(np.float32))   # on the default stream
+            _C.call("lq_event_record", fork, None)
+            for i, (s, e) in enumerate(zip(streams, joins)):
+                _C.call("lq_stream_wait_event", s, fork)
+                _C.call("lq_relu_f32", x.data_ptr + 4 * n * i, y.data_ptr + 4 * n * i, n, s)
+                _C.call("lq_event_record", e, s)
+            for e in joins:
+                _C.call("lq_stream_wait_event", None, e)
+            z = L.Tensor.empty((2 * n,), L.float32, "hip")
+            _C.call("lq_add_f32", y.data_ptr, y.data_ptr, z.data_ptr, 2 * n, None)  # consumer on the default stream
+            assert np.array_equal(z.numpy(), 2 * np.maximum(x.numpy(), 0.0)), rep
+    finally:
+        L.synchronize()
+        for s in streams:
+            _C.call("lq_stream_destroy", s)
+        for e in [fork, *joins]:
+            _C.call("lq_event_destroy", e)
+    with pytest.raises(ValueError, match="event is NULL"):
+        _C.call("lq_stream_wait_event", None, None)
