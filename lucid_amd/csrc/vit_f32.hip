@@ -495,18 +495,26 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
 #pragma unroll
         // (scale * log2 e: the scores are kept in the base-2 domain, so that the softmax
         // numerators are one v_exp_f32 each: 2^(s - max) = e^((s - max) ln 2))
-        for (int s = 0; s < AT_D / 4; ++s) qf[s] = qp[4 * s + g] * (scale * 1.4426950408889634f);
+        // MFMA s carries k = 16 (s / 4) + 4 g + s % 4 in lane group g: a lane's four consecutive
+        // instructions then need four consecutive floats of a K row - one 16-byte LDS read
+        for (int s = 0; s < AT_D / 4; ++s) qf[s] = qp[16 * (s >> 2) + 4 * g + (s & 3)] * (scale * 1.4426950408889634f);
     }
     constexpr int NT = AT_TMAX / 16;
     v4f st[NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        v4f a = {0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NT; ++t) st[t] = v4f{0.f, 0.f, 0.f, 0.f};
+    // k slice outermost: the 13 tiles' accumulators are independent chains, so consecutive MFMAs never
+    // wait for each other (per tile the order of the k slices - and with it every bit - is unchanged)
 #pragma unroll
-        for (int s = 0; s < AT_D / 4; ++s)
-            a = __builtin_amdgcn_mfma_f32_16x16x4f32(sk[16 * t + c][4 * s + g], qf[s], a, 0, 0, 0);
-        st[t] = a;
-    }
+    for (int u = 0; u < AT_D / 16; ++u)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const float4 kv = *reinterpret_cast<const float4*>(&sk[16 * t + c][16 * u + 4 * g]);
+            st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.x, qf[4 * u + 0], st[t], 0, 0, 0);
+            st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.y, qf[4 * u + 1], st[t], 0, 0, 0);
+            st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.z, qf[4 * u + 2], st[t], 0, 0, 0);
+            st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.w, qf[4 * u + 3], st[t], 0, 0, 0);
+        }
     // st[t][r] = S[query q0 + c][key 16t + 4g + r]
     float mx = -__builtin_inff();
 #pragma unroll
@@ -536,22 +544,26 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
 #pragma unroll
     for (int j = 0; j < AT_D / 16; ++j) o[j] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
+    // tile j of the output holds head-dim columns 4 c + j (not 16 j + c): a lane's four tiles then take four
+    // consecutive floats of a V row - one 16-byte LDS read - and store four consecutive floats
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const float p = st[t][r] * inv;
-#pragma unroll
-            for (int j = 0; j < AT_D / 16; ++j)
-                o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, sv[16 * t + 4 * g + r][16 * j + c], o[j], 0, 0, 0);
+            const float4 vv = *reinterpret_cast<const float4*>(&sv[16 * t + 4 * g + r][4 * c]);
+            o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, vv.x, o[0], 0, 0, 0);
+            o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, vv.y, o[1], 0, 0, 0);
+            o[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, vv.z, o[2], 0, 0, 0);
+            o[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, vv.w, o[3], 0, 0, 0);
         }
-    // result layout of the 16x16 MFMA: column = lane % 16, row = 4*(lane/16) + r
+    // result layout of the 16x16 MFMA: column slot = lane % 16, row = 4*(lane/16) + r
 #pragma unroll
-    for (int j = 0; j < AT_D / 16; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int q = q0 + 4 * g + r;
-            if (q < T) out[(size_t(b) * T + q) * (size_t(H) * AT_D) + size_t(h) * AT_D + 16 * j + c] = o[j][r];
-        }
+    for (int r = 0; r < 4; ++r) {
+        const int q = q0 + 4 * g + r;
+        if (q < T)
+            *reinterpret_cast<float4*>(out + (size_t(b) * T + q) * (size_t(H) * AT_D) + size_t(h) * AT_D + 4 * c) =
+                float4{o[0][r], o[1][r], o[2][r], o[3][r]};
+    }
     if (range) {
         float lo = __builtin_inff(), hi = -__builtin_inff();
         int nan = 0;
