@@ -23,6 +23,7 @@
 #include "qgemm.hpp"
 #include "qepilogue.hpp"
 
+#include <mutex>
 #include <utility>
 
 namespace lq {
@@ -42,7 +43,6 @@ struct PPCfg {
     // one wavefront-wide 16-byte direct load fills 1 KiB = 16 rows of 64 bytes
     static constexpr int A_CHUNKS = BM / 16, B_CHUNKS = BN / 16;
     static constexpr int LA = (A_CHUNKS + WAVES - 1) / WAVES, LB = (B_CHUNKS + WAVES - 1) / WAVES;
-    static constexpr int LOADS = LA + LB;  // direct loads per wavefront and stage (some may repeat a chunk)
     static constexpr int STAGE_BYTES = (BM + BN) * BK;
     // after the stage buffers: the block's column parameters (scale, bias, correction) as three
     // arrays of BN words, written once in the prologue and read by the epilogue
@@ -117,12 +117,255 @@ __device__ __forceinline__ void pp_pack(uint4 v, const CodePack& cpk, uint32_t* 
     }
 }
 
+// Which column tile a wavefront keeps in accumulator column j.  Normally tile j.  When the
+// wavefront has an odd number of column tiles and its first output column sits half a store
+// run off an aligned position in memory (the second half of a 352-column tile starts at column
+// 176; the epilogue stores pairs of tiles as runs of 32 columns, which for float16 are 64
+// bytes), the tiles are rotated by one: column j holds tile (j + 1) % TN.  The pairs
+// (0,1), (2,3), ... of accumulator columns are then the tiles (1,2), (3,4), ..., whose runs
+// start on a multiple of their size, and the lone last column is tile 0.  A run that
+// straddles two such segments reaches memory as two partial writes.  Only the LDS address
+// of a B fragment and the column an accumulator is stored to depend on it.
+template <int TN, int MODE>
+__device__ __forceinline__ int pp_rotation(const GemmArgs& g, int wn0) {
+    constexpr int esize = MODE == OUT_F16 ? 2 : ((MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) ? 1 : 4);
+    if (TN % 2 == 0 || g.ldo % 32 != 0 || reinterpret_cast<uintptr_t>(g.out) % (16 * esize) != 0) return 0;
+    return (reinterpret_cast<uintptr_t>(g.out) / esize + size_t(wn0)) % 32 == 16 ? 1 : 0;
+}
+
+// The register epilogue.  acc[i][j][r] is row wm0 + 16 i + lane % 16, column
+// wn0 + 16 t + 4 (lane / 16) + r with t = the column tile of j (pp_rotation): four consecutive
+// columns per lane and tile, so scale, bias, ReLU / requantize / join run on registers and the
+// packed values are stored directly.  s_ws / s_bias / s_corr: the block's column parameters in
+// LDS (column n0 first); as_row: this lane's row scales.
+template <int TM, int TN, int MODE>
+__device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM][TN], const float (&as_row)[TM],
+                                            const float* s_ws, const float* s_bias, const int32_t* s_corr, int n0,
+                                            int wm0, int wn0, int lane, int rot) {
+    if (wm0 >= g.M || wn0 >= g.N) return;
+    float S = 1.0f, Z = 0.0f;
+    constexpr bool kRequant = MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN || MODE == OUT_FAKEQUANT_F32;
+    if (kRequant) {
+        S = g.out_scale[0];
+        Z = g.out_zp[0];
+    }
+    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), kRequant, g.relu != 0, MODE == OUT_REQUANT_I8);
+    JoinParams jp;
+    if (MODE == OUT_REQUANT_JOIN) jp = load_join(g, G, true);
+    const CodePack cpk = make_code_pack<MODE>(g, MODE == OUT_REQUANT_JOIN ? jp.out : G);
+    constexpr int esize = MODE == OUT_F16 ? 2 : ((MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) ? 1 : 4);
+    constexpr bool kFloatOut = MODE == OUT_F32 || MODE == OUT_F16 || MODE == OUT_F32X;
+    const bool prescaled = (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) && !g.a_scale_per_row;
+    const bool cols_in = wn0 + TN * 16 <= g.N, rows_in = wm0 + TM * 16 <= g.M;
+    // uniform: every access of this wavefront may be a whole aligned vector
+    const bool vec_out = cols_in && g.ldo % 4 == 0 && reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0 &&
+                         (!kFloatOut || g.residual == nullptr || (g.ldr % 4 == 0 && aligned16(g.residual))) &&
+                         (MODE != OUT_REQUANT_JOIN ||
+                          (g.join_ld % 4 == 0 && reinterpret_cast<uintptr_t>(g.join_q) % 4 == 0 && jp.k2_exact));
+    // first column of the lane's four in the tile of accumulator column j: pairs are the
+    // columns j = 2x, 2x + 1 (tiles j + rot), the lone last column of an odd TN is tile
+    // rot ? 0 : TN - 1
+    const int pair0 = wn0 + 16 * rot;
+    const int last_tile = rot ? 0 : TN - 1;
+    const int lane_col = 4 * (lane >> 4);
+    // Wider stores for pairs of column tiles: the lanes of an even and the following odd row
+    // group (16 lanes each) exchange one tile's packed values (v_permlane16_swap), after which an
+    // even-group lane holds eight consecutive columns of the first tile and an odd-group lane
+    // eight of the second.  A row then receives 64 contiguous bytes of float16 (32 of int8
+    // codes, 128 of 32-bit values) from four lanes instead of half that.
+    constexpr int kDw = MODE == OUT_F16 ? 2 : ((MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) ? 1 : 4);
+    constexpr int kPairs = TN / 2;
+    constexpr bool kLone = TN % 2 == 1;
+    const bool wide = vec_out && g.ldo % 8 == 0 && reinterpret_cast<uintptr_t>(g.out) % 16 == 0;
+    const int g_odd = (lane >> 4) & 1;
+    const int swapped_col = 16 * g_odd + 4 * ((lane >> 4) & ~1);  // within a pair: first of the lane's 8 columns
+    typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
+    typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
+
+    // ---- the plain float forms on an interior sub-tile (every row and column inside the
+    // matrix, aligned, no residual, no ReLU, no zero-point correction): the same float steps -
+    // convert, as * ws, multiply, add the bias - and nothing else: row pointers are formed
+    // once and every store takes a constant offset from one of them.
+    if constexpr (MODE == OUT_F16 || MODE == OUT_F32) {
+        const int zp = g.a_zp_dev ? int(g.a_zp_dev[0]) + g.a_zp : g.a_zp;
+        const bool lean = wide && rows_in && g.residual == nullptr && !g.relu && (g.wsum == nullptr || zp == 0);
+        if (lean) {
+            char* rows[TM];  // the lane's position in a pair's run, row block by row block
+            rows[0] = static_cast<char*>(g.out) +
+                      (size_t(wm0 + (lane & 15)) * size_t(g.ldo) + size_t(pair0 + swapped_col)) * esize;
+            const size_t row_step = size_t(16) * size_t(g.ldo) * esize;
+#pragma unroll
+            for (int i = 1; i < TM; ++i) rows[i] = rows[i - 1] + row_step;
+            // from there to the lane's own four columns of the lone tile
+            const ptrdiff_t lone_delta = ptrdiff_t(16 * last_tile + lane_col - 16 * rot - swapped_col) * esize;
+            auto value4 = [&](const pp_v4i& a, const float4& ws, const float4& b, float as, uint4& v) {
+                v.x = __float_as_uint(float(a[0]) * (as * ws.x) + b.x);
+                v.y = __float_as_uint(float(a[1]) * (as * ws.y) + b.y);
+                v.z = __float_as_uint(float(a[2]) * (as * ws.z) + b.z);
+                v.w = __float_as_uint(float(a[3]) * (as * ws.w) + b.w);
+            };
+            pp_static_for<kPairs>([&](auto x_tag) {
+                constexpr int j = 2 * decltype(x_tag)::value;
+                const int cl = pair0 - n0 + 16 * j + lane_col;  // the lane's own columns of the pair's first tile
+                const float4 ws0 = *reinterpret_cast<const float4*>(s_ws + cl), b0 = *reinterpret_cast<const float4*>(s_bias + cl);
+                const float4 ws1 = *reinterpret_cast<const float4*>(s_ws + cl + 16),
+                             b1 = *reinterpret_cast<const float4*>(s_bias + cl + 16);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    uint4 v, w;
+                    value4(acc[i][j], ws0, b0, as_row[i], v);
+                    value4(acc[i][j + 1], ws1, b1, as_row[i], w);
+                    uint32_t p[kDw], q[kDw], lo[kDw], hi[kDw];
+                    pp_pack<MODE>(v, cpk, p);
+                    pp_pack<MODE>(w, cpk, q);
+#pragma unroll
+                    for (int d = 0; d < kDw; ++d) {
+                        const auto sw = __builtin_amdgcn_permlane16_swap(p[d], q[d], false, false);
+                        lo[d] = sw[0], hi[d] = sw[1];
+                    }
+                    char* dst = rows[i] + 16 * j * esize;
+                    if constexpr (kDw == 2) {
+                        *reinterpret_cast<v4u_t*>(dst) = v4u_t{lo[0], lo[1], hi[0], hi[1]};
+                    } else {
+                        *reinterpret_cast<v4u_t*>(dst) = v4u_t{lo[0], lo[1], lo[2], lo[3]};
+                        *reinterpret_cast<v4u_t*>(dst + 16) = v4u_t{hi[0], hi[1], hi[2], hi[3]};
+                    }
+                }
+            });
+            if constexpr (kLone) {
+                const int cl = wn0 - n0 + 16 * last_tile + lane_col;
+                const float4 ws = *reinterpret_cast<const float4*>(s_ws + cl), b = *reinterpret_cast<const float4*>(s_bias + cl);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    uint4 v;
+                    value4(acc[i][TN - 1], ws, b, as_row[i], v);
+                    uint32_t p[kDw];
+                    pp_pack<MODE>(v, cpk, p);
+                    char* dst = rows[i] + lone_delta;
+                    if constexpr (kDw == 2)
+                        *reinterpret_cast<v2u_t*>(dst) = v2u_t{p[0], p[1]};
+                    else
+                        *reinterpret_cast<v4u_t*>(dst) = v4u_t{p[0], p[1], p[2], p[3]};
+                }
+            }
+            return;
+        }
+    }
+
+    // ---- every other form.  values of one tile in the lane's own layout, residual / join applied
+    auto tile_values = [&](int m, const pp_v4i& a, const ColParams (&c4)[4], float as, int nq, uint4& v) {
+        if (prescaled) {
+            v.x = epilogue_value<MODE, true>(g, a[0], 1.0f, c4[0], G);
+            v.y = epilogue_value<MODE, true>(g, a[1], 1.0f, c4[1], G);
+            v.z = epilogue_value<MODE, true>(g, a[2], 1.0f, c4[2], G);
+            v.w = epilogue_value<MODE, true>(g, a[3], 1.0f, c4[3], G);
+        } else {
+            v.x = epilogue_value<MODE, false>(g, a[0], as, c4[0], G);
+            v.y = epilogue_value<MODE, false>(g, a[1], as, c4[1], G);
+            v.z = epilogue_value<MODE, false>(g, a[2], as, c4[2], G);
+            v.w = epilogue_value<MODE, false>(g, a[3], as, c4[3], G);
+        }
+        if (vec_out && (rows_in || m < g.M)) {
+            if (kFloatOut && g.residual != nullptr) {
+                const float4 rv = *reinterpret_cast<const float4*>(g.residual + size_t(m) * size_t(g.ldr) + size_t(nq));
+                v.x = __float_as_uint(__uint_as_float(v.x) + rv.x);
+                v.y = __float_as_uint(__uint_as_float(v.y) + rv.y);
+                v.z = __float_as_uint(__uint_as_float(v.z) + rv.z);
+                v.w = __float_as_uint(__uint_as_float(v.w) + rv.w);
+            }
+            if (MODE == OUT_REQUANT_JOIN) {
+                const uint32_t jb = *reinterpret_cast<const uint32_t*>(g.join_q + size_t(m) * size_t(g.join_ld) + size_t(nq)) ^
+                                    0x80808080u;  // stored bytes + 128, all four
+                v.x = join_code_biased(jp, v.x, float(jb & 0xffu));
+                v.y = join_code_biased(jp, v.y, float((jb >> 8) & 0xffu));
+                v.z = join_code_biased(jp, v.z, float((jb >> 16) & 0xffu));
+                v.w = join_code_biased(jp, v.w, float(jb >> 24));
+            }
+        }
+    };
+    auto load_c4 = [&](int nq, ColParams (&c4)[4]) {
+        const int cl = nq - n0;  // column within the block tile, a multiple of 4
+        const float4 ws = *reinterpret_cast<const float4*>(s_ws + cl);
+        const float4 b = *reinterpret_cast<const float4*>(s_bias + cl);
+        const int4 cr = *reinterpret_cast<const int4*>(s_corr + cl);
+        c4[0] = ColParams{ws.x, b.x, cr.x}, c4[1] = ColParams{ws.y, b.y, cr.y};
+        c4[2] = ColParams{ws.z, b.z, cr.z}, c4[3] = ColParams{ws.w, b.w, cr.w};
+        if (prescaled) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) c4[r].ws = as_row[0] * c4[r].ws;
+        }
+    };
+    // one tile stored from the lane's own layout (four consecutive columns)
+    auto store_own = [&](int m, int nq, uint4 v) {
+        if (!rows_in && m >= g.M) return;
+        const size_t idx = size_t(m) * size_t(g.ldo) + size_t(nq);
+        if (vec_out) {
+            store_vec4<MODE>(g, idx, v, cpk);
+        } else if (nq < g.N) {
+            store_scalar<MODE>(g, idx, finish_value<MODE>(g, v.x, m, nq, jp), cpk);
+            if (nq + 1 < g.N) store_scalar<MODE>(g, idx + 1, finish_value<MODE>(g, v.y, m, nq + 1, jp), cpk);
+            if (nq + 2 < g.N) store_scalar<MODE>(g, idx + 2, finish_value<MODE>(g, v.z, m, nq + 2, jp), cpk);
+            if (nq + 3 < g.N) store_scalar<MODE>(g, idx + 3, finish_value<MODE>(g, v.w, m, nq + 3, jp), cpk);
+        }
+    };
+    pp_static_for<kPairs>([&](auto x_tag) {
+        constexpr int j = 2 * decltype(x_tag)::value;
+        const int nq = pair0 + 16 * j + lane_col;
+        ColParams c4[4], d4[4];
+        load_c4(nq, c4);
+        load_c4(nq + 16, d4);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int m = wm0 + 16 * i + (lane & 15);
+            uint4 v, w;
+            tile_values(m, acc[i][j], c4, as_row[i], nq, v);
+            tile_values(m, acc[i][j + 1], d4, as_row[i], nq + 16, w);
+            if (!wide) {
+                store_own(m, nq, v);
+                store_own(m, nq + 16, w);
+                continue;
+            }
+            uint32_t p[kDw], q[kDw], lo[kDw], hi[kDw];
+            pp_pack<MODE>(v, cpk, p);
+            pp_pack<MODE>(w, cpk, q);
+#pragma unroll
+            for (int d = 0; d < kDw; ++d) {
+                const auto sw = __builtin_amdgcn_permlane16_swap(p[d], q[d], false, false);
+                lo[d] = sw[0], hi[d] = sw[1];
+            }
+            if (!rows_in && m >= g.M) continue;
+            char* dst = static_cast<char*>(g.out) +
+                        (size_t(m) * size_t(g.ldo) + size_t(pair0 + 16 * j + swapped_col)) * esize;
+            if constexpr (kDw == 1) {
+                *reinterpret_cast<v2u_t*>(dst) = v2u_t{lo[0], hi[0]};
+            } else if constexpr (kDw == 2) {
+                *reinterpret_cast<v4u_t*>(dst) = v4u_t{lo[0], lo[1], hi[0], hi[1]};
+            } else {
+                *reinterpret_cast<v4u_t*>(dst) = v4u_t{lo[0], lo[1], lo[2], lo[3]};
+                *reinterpret_cast<v4u_t*>(dst + 16) = v4u_t{hi[0], hi[1], hi[2], hi[3]};
+            }
+        }
+    });
+    if constexpr (kLone) {
+        const int nq = wn0 + 16 * last_tile + lane_col;
+        ColParams c4[4];
+        load_c4(nq, c4);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int m = wm0 + 16 * i + (lane & 15);
+            uint4 v;
+            tile_values(m, acc[i][TN - 1], c4, as_row[i], nq, v);
+            store_own(m, nq, v);
+        }
+    }
+}
+
 // K must be a multiple of 64 (the launcher checks); M and N are arbitrary: rows past
-// the end are clamped for the loads and masked at the store.
+// the end of an operand read as zeros and are masked at the store.
 template <class Cfg, int MODE>
 __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void qgemm_pp_kernel(GemmArgs g) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
-    constexpr int STAGES = Cfg::STAGES, LA = Cfg::LA, LB = Cfg::LB, LOADS = Cfg::LOADS;
+    constexpr int STAGES = Cfg::STAGES, LA = Cfg::LA, LB = Cfg::LB;
     extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -133,6 +376,8 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     pp_tile_coords(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int nk = g.K / BK;
+    const int wm0 = m0 + wm * (TM * 16), wn0 = n0 + wn * (TN * 16);  // this wavefront's sub-tile
+    const int rot = pp_rotation<TN, MODE>(g, wn0);
 
     // ---- global -> LDS: chunk c of an operand is its rows 16c .. 16c+15; lane l fills the slot
     // of row 16c + l/4, physical 16-byte chunk l%4, with the logical chunk (l%4) ^ ((row/2)%4).
@@ -161,7 +406,7 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     const __amdgpu_buffer_rsrc_t b_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.w), 0, unsigned(g.N) * unsigned(g.K), 0x00020000);
 
-    // Direct load x (0 .. LOADS-1) of this wavefront for stage s of the k loop.  Stages past the
+    // Direct load x (0 .. LA + LB - 1) of this wavefront for stage s of the k loop.  Stages past the
     // end reload the last one into a buffer nobody reads, which keeps the number of outstanding
     // loads - the vmcnt to wait for - the same throughout.
     auto stage_load = [&](int s, auto x_tag) {
@@ -180,29 +425,30 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // alternately so that the two 64-byte halves of each 128-byte line of a matrix row are
     // requested back to back: the second request finds the line the first one brought into the
     // CU's cache (loaded a whole stage apart, every line would be fetched from the L2 twice).
-    constexpr int kFirstB = LA;
-    auto pair_load = [&](int s, auto op_tag, auto c_tag) {  // c: 0 .. 2 * L - 1 within the pair
-        constexpr int first = decltype(op_tag)::value ? kFirstB : 0;
-        constexpr int c = decltype(c_tag)::value;
-        stage_load(s + (c & 1), std::integral_constant<int, first + c / 2>{});
-    };
     auto pair_load_all = [&](int s, auto op_tag) {
+        constexpr int first = decltype(op_tag)::value ? LA : 0;
         constexpr int n = 2 * (decltype(op_tag)::value ? LB : LA);
-        pp_static_for<n>([&](auto c) { pair_load(s, op_tag, c); });
+        pp_static_for<n>([&](auto c_tag) {
+            constexpr int c = decltype(c_tag)::value;
+            stage_load(s + (c & 1), std::integral_constant<int, first + c / 2>{});
+        });
     };
 
     // ---- LDS -> registers: lane l of a 16 x 64 fragment holds row l%16, logical chunk l/16,
-    // which sits at physical chunk (l/16) ^ ((row/2)%4)
+    // which sits at physical chunk (l/16) ^ ((row/2)%4).  B fragment j is the wavefront's column
+    // tile (j + rot) % TN.
     const int fr_off = (lane & 15) * BK + (((lane >> 4) ^ ((lane >> 1) & 3)) * 16);
     const int a_frag0 = wm * (TM * 16) * BK + fr_off;
-    const int b_frag0 = BM * BK + wn * (TN * 16) * BK + fr_off;
+    const int b_frag0 = BM * BK + wn * (TN * 16) * BK + fr_off + rot * 16 * BK;
+    const int b_frag_last = BM * BK + wn * (TN * 16) * BK + fr_off + (rot ? 0 : (TN - 1) * 16 * BK);
     pp_v4i af[TM], bf[TN];
     auto read_frags = [&](int s) {
-                const int8_t* buf = smem + (s % STAGES) * Cfg::STAGE_BYTES;
+        const int8_t* buf = smem + (s % STAGES) * Cfg::STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const pp_v4i*>(buf + a_frag0 + i * 16 * BK);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const pp_v4i*>(buf + b_frag0 + j * 16 * BK);
+        for (int j = 0; j < TN - 1; ++j) bf[j] = *reinterpret_cast<const pp_v4i*>(buf + b_frag0 + j * 16 * BK);
+        bf[TN - 1] = *reinterpret_cast<const pp_v4i*>(buf + b_frag_last);
     };
 
     pp_v4i acc[TM][TN];
@@ -211,30 +457,18 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = pp_v4i{0, 0, 0, 0};
 
-    // The MFMAs of one k step.  LOADER: this wavefront's pair of operand OP (0 = A, 1 = B) for
-    // stages s, s+1 is spread between them, so that the loads queue up behind the matrix
-    // instructions instead of in front of them.
+    // The MFMAs of one k step, column by column; within a column the row order alternates, so
+    // that only one operand changes from one instruction to the next (fewer operand bits
+    // toggle: the MFMA-only rate on the same codes is 2 % higher in this order, and the launch 1 us shorter).
     constexpr int kMfmas = TM * TN;
-    auto compute = [&](int s, auto op_tag, auto loader_tag) {
-        constexpr bool loader = decltype(loader_tag)::value;
-        constexpr int nl = loader ? 2 * (decltype(op_tag)::value ? LB : LA) : 0;
-        constexpr int gap = kMfmas / (nl + 1);
+    auto compute = [&]() {
         __builtin_amdgcn_s_setprio(2);
         pp_static_for<kMfmas>([&](auto x_tag) {
             constexpr int X = decltype(x_tag)::value;
-            constexpr int i = X % TM, j = X / TM;
+            constexpr int j = X / TM;
+            constexpr int i = (j & 1) ? TM - 1 - X % TM : X % TM;
             acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
-            if constexpr (nl > 0 && (X + 1) % gap == 0 && (X + 1) / gap <= nl)
-                pair_load(s, op_tag, std::integral_constant<int, (X + 1) / gap - 1>{});
         });
-        if (nl > 0) {
-#pragma unroll
-            for (int x = 0; x < nl; ++x) {
-                __builtin_amdgcn_sched_group_barrier(0x008, gap, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, kMfmas - nl * gap, 0);
-        }
         __builtin_amdgcn_s_setprio(0);
     };
     // ---- prologue: the tile's column parameters are requested first (they go to LDS, where the
@@ -257,7 +491,6 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     __builtin_amdgcn_sched_barrier(0);
 
     // Row scales of this lane's TM rows, fetched during the wavefront's last read phase.
-    const int wm0 = m0 + wm * (TM * 16), wn0 = n0 + wn * (TN * 16);  // this wavefront's sub-tile
     float as_row[TM];
     auto fetch_params = [&]() {
 #pragma unroll
@@ -266,25 +499,15 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
             as_row[i] = g.a_scale ? g.a_scale[(g.a_scale_per_row && m < g.M) ? m : 0] : 1.0f;
         }
     };
-    // One k step of a wavefront.  Step u refills operand OP = u % 2 for stages u+2, u+3 (their
-    // buffers held stages u-2 and u-1, whose last readers finished in phase 2u-1).  Group 0 issues
-    // the loads between the MFMAs of its phase 2u+1; group 1 behind the fragment reads of its read
-    // phase, which is the same phase 2u+1.  Either way, when the wavefront then waits for its loads of stage
-    // u+1, what it issued later is one load of the pair's second stage plus this step's pair.
-    auto step_g0 = [&](int u, auto op_tag) {
-        constexpr int kAllowed = 1 + 2 * (decltype(op_tag)::value ? LB : LA);
-        read_frags(u);
-        if (u == nk - 1) fetch_params();
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        compute(u + 2, op_tag, std::true_type{});
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(pp_vmcnt_imm(kAllowed));
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    auto step_g1 = [&](int u, auto op_tag) {
+    // One k step of a wavefront: a read phase (the step's fragments, then the refill of operand
+    // OP = u % 2 for the stages u+2, u+3, whose buffers held the stages u-2 and u-1: their last
+    // readers finished in phase 2u-1), the barrier, and an MFMA phase of nothing but the 44
+    // matrix instructions.  The direct loads are issued in the read phase by both groups: a
+    // load instruction between two MFMAs of the same wavefront holds up the second one by
+    // about 20 cycles (measured: 113 k cycles for the 64 steps with group 0's loads between its MFMAs,
+    // 98 k with them here; 92 k is the MFMAs alone).  When the wavefront waits for its loads of stage u+1, what
+    // it issued later is one load of the pair's second stage plus this step's pair.
+    auto step = [&](int u, auto op_tag, bool trailing_barrier) {
         constexpr int kAllowed = 1 + 2 * (decltype(op_tag)::value ? LB : LA);
         read_frags(u);
         pair_load_all(u + 2, op_tag);
@@ -293,173 +516,44 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
         __builtin_amdgcn_s_waitcnt(pp_vmcnt_imm(kAllowed));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        compute(u + 2, op_tag, std::false_type{});
+        compute();
         __builtin_amdgcn_sched_barrier(0);
-        if (u + 1 < nk) __builtin_amdgcn_s_barrier();
+        if (trailing_barrier) __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
     };
-    if (group == 0) {
-        int u = 0;
-        for (; u + 1 < nk; u += 2) {
-            step_g0(u, std::false_type{});
-            step_g0(u + 1, std::true_type{});
-        }
-        if (u < nk) step_g0(u, std::false_type{});
-    } else {
+    // Group 0 reads in the even phases and computes in the odd ones, group 1 one phase later;
+    // both pass the same number of barriers (group 1 skips the one after its last MFMAs).
+    if (group == 1) {
         __builtin_amdgcn_s_barrier();  // phase 0 belongs to group 0
         __builtin_amdgcn_sched_barrier(0);
+    }
+    {
         int u = 0;
         for (; u + 1 < nk; u += 2) {
-            step_g1(u, std::false_type{});
-            step_g1(u + 1, std::true_type{});
+            step(u, std::false_type{}, true);
+            step(u + 1, std::true_type{}, group == 0 || u + 2 < nk);
         }
-        if (u < nk) step_g1(u, std::false_type{});
+        if (u < nk) step(u, std::false_type{}, group == 0);
     }
-    // Both groups have passed the same number of barriers.
-    // ---- epilogue.  acc[i][j][r] is row wm0 + 16 i + lane % 16, column wn0 + 16 j + 4 (lane / 16) + r:
-    // four consecutive columns per lane and tile.  No staging through LDS and no barrier: group 0
-    // runs it while group 1 still issues its last MFMAs.
+    // ---- epilogue: no staging through LDS and no barrier; group 0 runs it while group 1 still
+    // issues its last MFMAs.
     __builtin_amdgcn_s_waitcnt(pp_vmcnt_imm(0));  // no direct load may land in LDS after this wavefront has ended
-    if (wm0 >= g.M || wn0 >= g.N) return;
-    float S = 1.0f, Z = 0.0f;
-    constexpr bool kRequant = MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN || MODE == OUT_FAKEQUANT_F32;
-    if (kRequant) {
-        S = g.out_scale[0];
-        Z = g.out_zp[0];
-    }
-    const QGrid G = make_qgrid(S, Z, float(g.out_qmin), float(g.out_qmax), kRequant, g.relu != 0, MODE == OUT_REQUANT_I8);
-    JoinParams jp;
-    if (MODE == OUT_REQUANT_JOIN) jp = load_join(g, G, true);
-    const CodePack cpk = make_code_pack<MODE>(g, MODE == OUT_REQUANT_JOIN ? jp.out : G);
-    constexpr int esize = MODE == OUT_F16 ? 2 : ((MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) ? 1 : 4);
-    constexpr bool kFloatOut = MODE == OUT_F32 || MODE == OUT_F16 || MODE == OUT_F32X;
-    const bool prescaled = (MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) && !g.a_scale_per_row;
-    const bool cols_in = wn0 + TN * 16 <= g.N, rows_in = wm0 + TM * 16 <= g.M;
-    // uniform: every access of this wavefront may be a whole aligned vector
-    const bool vec_out = cols_in && g.ldo % 4 == 0 && reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0 &&
-                         (!kFloatOut || g.residual == nullptr || (g.ldr % 4 == 0 && aligned16(g.residual))) &&
-                         (MODE != OUT_REQUANT_JOIN ||
-                          (g.join_ld % 4 == 0 && reinterpret_cast<uintptr_t>(g.join_q) % 4 == 0 && jp.k2_exact));
-    const int nq0 = wn0 + 4 * (lane >> 4);
-    // Wider stores for pairs of column tiles: the lanes of an even and the following odd row
-    // group (16 lanes each) exchange one tile's packed values (v_permlane16_swap), after which an
-    // even-group lane holds eight consecutive columns of tile j and an odd-group lane eight of
-    // tile j+1.  A row then receives 64 contiguous bytes of float16 (32 of int8 codes, 128 of
-    // 32-bit values) from four lanes instead of half that.
-    constexpr int kDw = MODE == OUT_F16 ? 2 : ((MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN) ? 1 : 4);
-    const bool wide = vec_out && g.ldo % 8 == 0 && reinterpret_cast<uintptr_t>(g.out) % 16 == 0;
-    const int g_odd = (lane >> 4) & 1;
-    const int col_swapped = wn0 + 16 * g_odd + 4 * ((lane >> 4) & ~1);  // + 16 j: first of the lane's 8 columns
-
-    // values of tile (i, j) in the lane's own layout, residual / join applied; false: row outside
-    auto tile_values = [&](int i_row_m, const v4i_t& a, const ColParams (&c4)[4], float as, int nq, uint4& v) {
-        if (prescaled) {
-            v.x = epilogue_value<MODE, true>(g, a[0], 1.0f, c4[0], G);
-            v.y = epilogue_value<MODE, true>(g, a[1], 1.0f, c4[1], G);
-            v.z = epilogue_value<MODE, true>(g, a[2], 1.0f, c4[2], G);
-            v.w = epilogue_value<MODE, true>(g, a[3], 1.0f, c4[3], G);
-        } else {
-            v.x = epilogue_value<MODE, false>(g, a[0], as, c4[0], G);
-            v.y = epilogue_value<MODE, false>(g, a[1], as, c4[1], G);
-            v.z = epilogue_value<MODE, false>(g, a[2], as, c4[2], G);
-            v.w = epilogue_value<MODE, false>(g, a[3], as, c4[3], G);
-        }
-        const int m = i_row_m;
-        if (vec_out && (rows_in || m < g.M)) {
-            if (kFloatOut && g.residual != nullptr) {
-                const float4 rv = *reinterpret_cast<const float4*>(g.residual + size_t(m) * size_t(g.ldr) + size_t(nq));
-                v.x = __float_as_uint(__uint_as_float(v.x) + rv.x);
-                v.y = __float_as_uint(__uint_as_float(v.y) + rv.y);
-                v.z = __float_as_uint(__uint_as_float(v.z) + rv.z);
-                v.w = __float_as_uint(__uint_as_float(v.w) + rv.w);
-            }
-            if (MODE == OUT_REQUANT_JOIN) {
-                const uint32_t jb = *reinterpret_cast<const uint32_t*>(g.join_q + size_t(m) * size_t(g.join_ld) + size_t(nq)) ^
-                                    0x80808080u;  // stored bytes + 128, all four
-                v.x = join_code_biased(jp, v.x, float(jb & 0xffu));
-                v.y = join_code_biased(jp, v.y, float((jb >> 8) & 0xffu));
-                v.z = join_code_biased(jp, v.z, float((jb >> 16) & 0xffu));
-                v.w = join_code_biased(jp, v.w, float(jb >> 24));
-            }
-        }
-    };
-    auto load_c4 = [&](int nq, ColParams (&c4)[4]) {
-        const int cl = nq - n0;  // column within the tile, a multiple of 4
-        const float4 ws = *reinterpret_cast<const float4*>(s_ws + cl);
-        const float4 b = *reinterpret_cast<const float4*>(s_bias + cl);
-        const int4 cr = *reinterpret_cast<const int4*>(s_corr + cl);
-        c4[0] = ColParams{ws.x, b.x, cr.x}, c4[1] = ColParams{ws.y, b.y, cr.y};
-        c4[2] = ColParams{ws.z, b.z, cr.z}, c4[3] = ColParams{ws.w, b.w, cr.w};
-        if (prescaled) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) c4[r].ws = as_row[0] * c4[r].ws;
-        }
-    };
-    // one tile stored from the lane's own layout (four consecutive columns)
-    auto store_own = [&](int m, int nq, uint4 v) {
-        if (!rows_in && m >= g.M) return;
-        const size_t idx = size_t(m) * size_t(g.ldo) + size_t(nq);
-        if (vec_out) {
-            store_vec4<MODE>(g, idx, v, cpk);
-        } else if (nq < g.N) {
-            store_scalar<MODE>(g, idx, finish_value<MODE>(g, v.x, m, nq, jp), cpk);
-            if (nq + 1 < g.N) store_scalar<MODE>(g, idx + 1, finish_value<MODE>(g, v.y, m, nq + 1, jp), cpk);
-            if (nq + 2 < g.N) store_scalar<MODE>(g, idx + 2, finish_value<MODE>(g, v.z, m, nq + 2, jp), cpk);
-            if (nq + 3 < g.N) store_scalar<MODE>(g, idx + 3, finish_value<MODE>(g, v.w, m, nq + 3, jp), cpk);
-        }
-    };
-#pragma unroll
-    for (int j = 0; j < TN; j += 2) {
-        const int nq = nq0 + 16 * j;
-        ColParams c4[4], d4[4];
-        load_c4(nq, c4);
-        if (j + 1 < TN) load_c4(nq + 16, d4);
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int m = wm0 + 16 * i + (lane & 15);
-            uint4 v, w;
-            tile_values(m, acc[i][j], c4, as_row[i], nq, v);
-            if (j + 1 >= TN) {
-                store_own(m, nq, v);
-                continue;
-            }
-            tile_values(m, acc[i][j + 1], d4, as_row[i], nq + 16, w);
-            if (!wide) {
-                store_own(m, nq, v);
-                store_own(m, nq + 16, w);
-                continue;
-            }
-            uint32_t p[kDw], q[kDw];
-            pp_pack<MODE>(v, cpk, p);
-            pp_pack<MODE>(w, cpk, q);
-            uint32_t lo[kDw], hi[kDw];
-#pragma unroll
-            for (int d = 0; d < kDw; ++d) {
-                const auto sw = __builtin_amdgcn_permlane16_swap(p[d], q[d], false, false);
-                lo[d] = sw[0], hi[d] = sw[1];
-            }
-            if (!rows_in && m >= g.M) continue;
-            char* dst = static_cast<char*>(g.out) + (size_t(m) * size_t(g.ldo) + size_t(col_swapped + 16 * j)) * esize;
-            if (kDw == 1) {
-                *reinterpret_cast<uint2*>(dst) = uint2{lo[0], hi[0]};
-            } else if (kDw == 2) {
-                *reinterpret_cast<uint4*>(dst) = uint4{lo[0], lo[1], hi[0], hi[1]};
-            } else {
-                *reinterpret_cast<uint4*>(dst) = uint4{lo[0], lo[1], lo[2], lo[3]};
-                *reinterpret_cast<uint4*>(dst + 16) = uint4{hi[0], hi[1], hi[2], hi[3]};
-            }
-        }
-    }
+    pp_epilogue<TM, TN, MODE>(g, acc, as_row, s_ws, s_bias, s_corr, n0, wm0, wn0, lane, rot);
 }
 
 template <class Cfg, int MODE>
 int launch_pp_mode(const GemmArgs& g, hipStream_t st) {
     const void* fn = reinterpret_cast<const void*>(qgemm_pp_kernel<Cfg, MODE>);
-    static bool attr_set = false;
-    if (!attr_set) {
-        LQ_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
-        attr_set = true;
-    }
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    LQ_REQUIRE(dev >= 0 && dev < 16, LQ_ERR_DEVICE, "device index %d out of range", dev);
+    // the dynamic LDS limit is a per-device attribute of the function: set once per device
+    static std::once_flag attr_once[16];
+    hipError_t attr_err = hipSuccess;
+    std::call_once(attr_once[dev], [&] {
+        attr_err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM);
+    });
+    LQ_HIP(attr_err);
     const int tiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
     GemmArgs copy = g;
     void* kargs[] = {&copy};
