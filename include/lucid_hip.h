@@ -402,8 +402,8 @@ int lq_quantize_tensor_dynamic_i8(const float* x, size_t n, int symmetric, int q
 
 /* A dynamic-quantized Linear on a small activation in ONE launch: nnqd.Linear.forward
  * (lucid/nn/quantized/dynamic/linear.py:87-99) for x [M, K] float32 with M <= 64,
- * K % 16 == 0 and M * K <= 65536 - the tensor's min / max, calculate_qparams, the
- * activation codes (kept in LDS), the integer GEMM against w [N, K] int8 codes with
+ * K % 16 == 0, K <= 6080 (16 rows of codes stay in LDS) and M * K <= 65536 - the tensor's
+ * min / max, calculate_qparams, the activation codes (kept in LDS), the integer GEMM against w [N, K] int8 codes with
  * per-row scales w_scale [N] and code sums wsum [N], float32 bias [N] or NULL, optional
  * ReLU; out [M, N] float32.  The bits of lq_quantize_tensor_dynamic_i8 followed by
  * lq_qlinear_i8 (mode F32).  Symmetric weights only.  Anything else:
@@ -648,6 +648,18 @@ int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);
  * tile-kernel launch resolved to - what the autotuner chose when 0 was passed.  For
  * benchmarks and tests; 0 before the first such launch.  No counterpart in Lucid. */
 int lq_last_tile_config(void);
+
+/* The tuner's choices as text, so that a deployment tunes once: one line per problem shape
+ * ("lq-tune-1", the shape key's integers, the chosen tile_config).  lq_tune_export writes what
+ * this process has chosen so far into buf (NUL-terminated); *needed receives the bytes
+ * required, and buf may be NULL to ask for that alone.  lq_tune_import adds the lines of
+ * `text` to the table (later launches of those shapes skip the timing; lines that do not
+ * start with "lq-tune-1" are skipped, a malformed one is LQ_ERR_VALUE); *accepted (may be
+ * NULL) receives the number of entries taken.  A file of such lines named by the environment
+ * variable LQ_TUNE_FILE is imported before the first lookup.  Results do not depend on the
+ * tile shape, only the time does.  No counterpart in Lucid. */
+int lq_tune_export(char* buf, size_t capacity, size_t* needed);
+int lq_tune_import(const char* text, int* accepted);
 
 /* The same forward launched n times back to back from native code: for
  * launch-bound callers (decode-shaped layers run for ~10 us, less than an

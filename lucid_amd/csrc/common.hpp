@@ -3,9 +3,11 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 #include <string>
 
 #include "../../include/lucid_hip.h"
@@ -48,6 +50,34 @@ int workspace(size_t nbytes, hipStream_t stream, void** ptr);
 // Resolves, for the current device, the address of the static scratch array that
 // lq_minmax_noalloc uses (called by lq_init; the entry point does it on first use otherwise).
 int minmax_noalloc_init();
+
+// A launch site's once-per-device set-up (the dynamic LDS limit of a kernel is a per-device
+// attribute of the function): one bit per device, taken under a mutex, so that the first calls
+// of two threads, or on two devices, neither race nor skip it.
+struct DeviceOnce {
+    std::atomic<uint32_t> done{0};
+    std::mutex mu;
+};
+template <class F>
+int device_once(DeviceOnce& o, F&& setup) {
+    int dev = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    LQ_REQUIRE(dev >= 0 && dev < 32, LQ_ERR_DEVICE, "device index %d out of range", dev);
+    const uint32_t bit = 1u << dev;
+    if (o.done.load(std::memory_order_acquire) & bit) return LQ_OK;
+    std::lock_guard<std::mutex> lock(o.mu);
+    if (o.done.load(std::memory_order_relaxed) & bit) return LQ_OK;
+    const int rc = setup();
+    if (rc == LQ_OK) o.done.fetch_or(bit, std::memory_order_release);
+    return rc;
+}
+// the common case: kernel `fn` may use up to `bytes` of dynamic LDS
+inline int allow_dynamic_lds(DeviceOnce& o, const void* fn, int bytes) {
+    return device_once(o, [&]() -> int {
+        LQ_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+        return LQ_OK;
+    });
+}
 
 inline hipStream_t as_stream(lq_stream s) { return reinterpret_cast<hipStream_t>(s); }
 

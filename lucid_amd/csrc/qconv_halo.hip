@@ -256,11 +256,8 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
 template <int MODE>
 int launch_mode(const GemmArgs& g, const HaloGeom& q, dim3 grid, size_t lds, hipStream_t st) {
     const void* fn = reinterpret_cast<const void*>(qconv_halo_kernel<MODE>);
-    static bool attr_set = false;
-    if (!attr_set) {
-        LQ_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        attr_set = true;
-    }
+    static DeviceOnce attr_once;
+    if (int rc = allow_dynamic_lds(attr_once, fn, 96 * 1024)) return rc;
     GemmArgs gc = g;
     HaloGeom qc = q;
     void* kargs[] = {&gc, &qc};

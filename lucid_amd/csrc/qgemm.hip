@@ -24,6 +24,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <string>
 #include <unordered_map>
 
 using namespace lq;
@@ -99,14 +100,32 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
     }
 }
 
-// Shape chosen from the problem size alone: 128 x 256 tiles keep two blocks per
-// CU busy; narrower tiles when N is small or when the wide ones would leave
-// most of the 256 CUs without work.
+// Whether the eight-wavefront ping-pong kernel (shapes 13 and 14) can run the problem.
+bool pp_applies(const GemmArgs& g, int conv, int groups) {
+    return !conv && groups == 1 && g.K > 0 && g.K % 64 == 0 && g.M >= 256 && g.N >= 256 && !g.gelu &&
+           g.range == nullptr && size_t(g.M) * g.K < 0xffffffffull && size_t(g.N) * g.K < 0xffffffffull;
+}
+
+// Shape chosen from the problem size alone (what a launch gets when the tuner may not run: a
+// stream under capture, LQ_TILE_AUTOTUNE=0, an in-place residual).  Large plain GEMMs go to
+// the ping-pong kernel, with the tile width that wastes less of the 256 CUs: the cost of a
+// shape is its rounds of 256 tiles times the tile's area.  Otherwise 128 x 256 tiles keep two
+// blocks per CU busy; narrower tiles when N is small or when the wide ones would leave most
+// of the CUs without work.
 int heuristic_tile_shape(const GemmArgs& g, int conv, int groups) {
     const long mt128 = (g.M + 127) / 128;
     // far fewer 128 x 128 tiles than CUs (a small batch in the late stages of a network): 64 x 64
     // tiles, four blocks per CU, with 128-byte k steps when K is long (plain and 2-d only)
     if (mt128 * ((g.N + 127) / 128) * groups < 128) return (g.K >= 1024 && conv != 2) ? 10 : 9;
+    if (pp_applies(g, conv, groups) && g.K >= 512) {
+        const long tm = (g.M + 255) / 256;
+        const long t352 = tm * ((g.N + 351) / 352), t256 = tm * ((g.N + 255) / 256);
+        // at least half a round of tiles, or the four-wavefront shapes below cover the chip better
+        if (t256 >= 128) {
+            const long c352 = ((t352 + 255) / 256) * 352, c256 = ((t256 + 255) / 256) * 256;
+            return c352 < c256 ? 13 : 14;
+        }
+    }
     if (g.N <= 64) return 6;
     if (g.N <= 128 || mt128 * ((g.N + 255) / 256) * groups < 256) return 5;
     return 4;
@@ -163,6 +182,60 @@ struct TuneKeyHash {
 std::mutex g_tune_mu;
 std::unordered_map<TuneKey, int, TuneKeyHash> g_tune;
 
+// One tuned choice as a line of text: "lq-tune-1" followed by the key's integers and the
+// chosen tile_config.  What lq_tune_export writes and lq_tune_import reads.
+constexpr int kTuneKeyInts = sizeof(TuneKey) / sizeof(int);
+static_assert(sizeof(TuneKey) == kTuneKeyInts * sizeof(int), "the key is all ints");
+
+int tune_import_text(const char* text, int* accepted) {
+    int n_ok = 0;
+    const char* p = text;
+    while (p && *p) {
+        const char* eol = std::strchr(p, '\n');
+        std::string line(p, eol ? size_t(eol - p) : std::strlen(p));
+        p = eol ? eol + 1 : nullptr;
+        if (line.compare(0, 10, "lq-tune-1 ") != 0) continue;  // blank lines, comments, other versions
+        int v[kTuneKeyInts + 1];
+        const char* q = line.c_str() + 10;
+        int got = 0;
+        while (got < kTuneKeyInts + 1) {
+            char* end = nullptr;
+            const long x = std::strtol(q, &end, 10);
+            if (end == q) break;
+            v[got++] = int(x);
+            q = end;
+        }
+        if (got != kTuneKeyInts + 1) return fail(LQ_ERR_VALUE, "tune_import: malformed line '%s'", line.c_str());
+        const int shape = v[kTuneKeyInts] & 0xff;
+        if (shape < 1 || shape > 15) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
+        TuneKey key;
+        std::memcpy(&key, v, sizeof(key));
+        std::lock_guard<std::mutex> lock(g_tune_mu);
+        g_tune[key] = v[kTuneKeyInts];
+        ++n_ok;
+    }
+    if (accepted) *accepted = n_ok;
+    return LQ_OK;
+}
+
+// LQ_TUNE_FILE names a file of such lines that is read before the first lookup, so that a
+// deployment pays for tuning once and not in every process (a missing file is not an error).
+void tune_import_env_file() {
+    static std::once_flag once;
+    std::call_once(once, [] {
+        const char* path = std::getenv("LQ_TUNE_FILE");
+        if (!path || !*path) return;
+        std::FILE* f = std::fopen(path, "r");
+        if (!f) return;
+        std::string text;
+        char buf[4096];
+        size_t n;
+        while ((n = std::fread(buf, 1, sizeof buf, f)) > 0) text.append(buf, n);
+        std::fclose(f);
+        (void)tune_import_text(text.c_str(), nullptr);
+    });
+}
+
 bool autotune_enabled() {
     static const bool on = [] {
         const char* e = std::getenv("LQ_TILE_AUTOTUNE");
@@ -186,6 +259,7 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
     }
     key.flags = (g.residual ? 1 : 0) | (g.a_scale_per_row ? 2 : 0) | (g.bias ? 4 : 0) | (g.join_q ? 8 : 0) |
                 (g.gelu ? 16 : 0) | (g.range ? 32 : 0);
+    tune_import_env_file();
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);
         auto it = g_tune.find(key);
@@ -224,9 +298,7 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
         if (g.N > 128 && g.M > 128) cands[n++] = 1, cands[n++] = 11;
         if (g.N > 128 && !conv) cands[n++] = 12;
         // large plain GEMMs: the ping-pong kernel's 256 x 352 and 256 x 256 tiles
-        if (!conv && groups == 1 && g.K % 64 == 0 && g.M >= 256 && g.N >= 256 && !g.gelu && g.range == nullptr &&
-            size_t(g.M) * g.K < 0xffffffffull && size_t(g.N) * g.K < 0xffffffffull)
-            cands[n++] = 13, cands[n++] = 14;
+        if (pp_applies(g, conv, groups)) cands[n++] = 13, cands[n++] = 14;
         // a long K over few tiles (late convolution stages): split K between the idle CUs
         const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
         if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);
@@ -637,9 +709,11 @@ namespace lq {
 
 int pad_table(const int8_t** table) {
     static void* tables[16] = {nullptr};
+    static std::mutex mu;
     int dev = 0;
     LQ_HIP(hipGetDevice(&dev));
     LQ_REQUIRE(dev >= 0 && dev < 16, LQ_ERR_DEVICE, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);  // two threads' first calls must not both build it
     if (!tables[dev]) {
         uint8_t host[256 * 16];
         for (int v = 0; v < 256; ++v)
@@ -779,6 +853,32 @@ int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, int rel
 }
 
 int lq_last_tile_config(void) { return t_last_tile_config; }
+
+int lq_tune_export(char* buf, size_t capacity, size_t* needed) {
+    LQ_REQUIRE(needed, LQ_ERR_VALUE, "tune_export: needed is NULL");
+    std::string text;
+    {
+        std::lock_guard<std::mutex> lock(g_tune_mu);
+        for (const auto& kv : g_tune) {
+            text += "lq-tune-1";
+            int v[kTuneKeyInts];
+            std::memcpy(v, &kv.first, sizeof(kv.first));
+            for (int i = 0; i < kTuneKeyInts; ++i) text += " " + std::to_string(v[i]);
+            text += " " + std::to_string(kv.second) + "\n";
+        }
+    }
+    *needed = text.size() + 1;
+    if (buf == nullptr) return LQ_OK;
+    LQ_REQUIRE(capacity >= text.size() + 1, LQ_ERR_VALUE, "tune_export: %zu bytes needed, %zu given", text.size() + 1,
+               capacity);
+    std::memcpy(buf, text.c_str(), text.size() + 1);
+    return LQ_OK;
+}
+
+int lq_tune_import(const char* text, int* accepted) {
+    LQ_REQUIRE(text, LQ_ERR_VALUE, "tune_import: text is NULL");
+    return tune_import_text(text, accepted);
+}
 
 }  // extern "C"
 

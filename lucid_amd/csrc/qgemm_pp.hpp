@@ -23,7 +23,6 @@
 #include "qgemm.hpp"
 #include "qepilogue.hpp"
 
-#include <mutex>
 #include <utility>
 
 namespace lq {
@@ -544,16 +543,8 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
 template <class Cfg, int MODE>
 int launch_pp_mode(const GemmArgs& g, hipStream_t st) {
     const void* fn = reinterpret_cast<const void*>(qgemm_pp_kernel<Cfg, MODE>);
-    int dev = 0;
-    LQ_HIP(hipGetDevice(&dev));
-    LQ_REQUIRE(dev >= 0 && dev < 16, LQ_ERR_DEVICE, "device index %d out of range", dev);
-    // the dynamic LDS limit is a per-device attribute of the function: set once per device
-    static std::once_flag attr_once[16];
-    hipError_t attr_err = hipSuccess;
-    std::call_once(attr_once[dev], [&] {
-        attr_err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM);
-    });
-    LQ_HIP(attr_err);
+    static DeviceOnce attr_once;
+    if (int rc = allow_dynamic_lds(attr_once, fn, Cfg::SMEM)) return rc;
     const int tiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
     GemmArgs copy = g;
     void* kargs[] = {&copy};

@@ -879,12 +879,13 @@ int launch_tile_mode(const GemmArgs& g, int groups, int schedule, hipStream_t st
         LQ_REQUIRE(schedule <= 1, LQ_ERR_NOT_IMPLEMENTED, "tile kernel: a volumetric convolution runs one block per tile");
         schedule = 1;
     }
-    static bool attr_set = false;
-    if (!attr_set) {
-        LQ_HIP(hipFuncSetAttribute(fn_dp, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
-        LQ_HIP(hipFuncSetAttribute(fn_sk, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
-        attr_set = true;
-    }
+    static DeviceOnce attr_once;
+    if (int rc = device_once(attr_once, [&]() -> int {
+            LQ_HIP(hipFuncSetAttribute(fn_dp, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
+            LQ_HIP(hipFuncSetAttribute(fn_sk, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM));
+            return LQ_OK;
+        }))
+        return rc;
     const int tiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
     const int nk = (g.K + Cfg::BK - 1) / Cfg::BK;
     // blocks that fit on the chip at once: 256 CUs x blocks per CU (LDS-bound)

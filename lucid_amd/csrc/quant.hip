@@ -893,20 +893,19 @@ int lq_dynamic_linear_small_f32(const float* x, int M, int K, const int8_t* w, i
     LQ_REQUIRE(x && w && out, LQ_ERR_VALUE, "dynamic_linear_small: NULL pointer");
     LQ_REQUIRE(qmax > qmin && qmin + code_offset >= -128 && qmax + code_offset <= 127, LQ_ERR_VALUE,
                "dynamic_linear_small: grid [%d,%d] + offset %d does not fit int8", qmin, qmax, code_offset);
-    LQ_REQUIRE(M > 0 && M <= 64 && K >= 16 && K % 16 == 0 && long(M) * K <= 65536 && K <= 33025 && N > 0 &&
+    // 16 rows of codes (16 K bytes) + 1 KiB of reduction scratch have to fit the 96 KiB of dynamic
+    // LDS the kernel is allowed: K <= 6080
+    LQ_REQUIRE(M > 0 && M <= 64 && K >= 16 && K % 16 == 0 && long(M) * K <= 65536 && K <= 6080 && N > 0 &&
                    aligned16(x) && aligned16(w),
                LQ_ERR_NOT_IMPLEMENTED,
-               "dynamic_linear_small: takes up to 64 rows, K %% 16 == 0, at most 65536 activations and 16-byte "
-               "aligned operands (got M = %d, K = %d); use lq_quantize_tensor_dynamic_i8 + lq_qlinear_i8", M, K);
+               "dynamic_linear_small: takes up to 64 rows, K %% 16 == 0 and K <= 6080, at most 65536 activations and "
+               "16-byte aligned operands (got M = %d, K = %d); use lq_quantize_tensor_dynamic_i8 + lq_qlinear_i8", M, K);
     const float half_range = float((double(qmax) - double(qmin)) / 2.0);
     const int tiles = (M + 15) / 16;
     const size_t lds = size_t(16) * K + 256 * sizeof(int);
-    static bool attr_set = false;
-    if (!attr_set) {
-        LQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dynamic_linear_small_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        attr_set = true;
-    }
+    static DeviceOnce attr_once;
+    if (int rc = allow_dynamic_lds(attr_once, reinterpret_cast<const void*>(dynamic_linear_small_kernel), 96 * 1024))
+        return rc;
     hipLaunchKernelGGL(dynamic_linear_small_kernel, dim3(unsigned((N + 15) / 16), unsigned(tiles)), dim3(1024), lds,
                        as_stream(stream), x,
                        M, K, w, N, w_scale, wsum, bias, relu, symmetric, qmin, qmax, is_signed, eps, half_range,

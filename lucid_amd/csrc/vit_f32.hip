@@ -716,12 +716,8 @@ int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, f
                "attention: too many (batch, head) pairs for a kept range");
     const int waves = (T + 15) / 16;
     constexpr size_t kSmem = size_t(2) * AT_TMAX * AT_LD * sizeof(float);
-    static bool attr_set = false;
-    if (!attr_set) {
-        LQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(kSmem)));
-        attr_set = true;
-    }
+    static DeviceOnce attr_once;
+    if (int rc = allow_dynamic_lds(attr_once, reinterpret_cast<const void*>(attention_kernel), int(kSmem))) return rc;
     attention_kernel<<<unsigned(B) * H, waves * 64, kSmem, as_stream(stream)>>>(qkv, out, B, T, H, scale,
                                                                                  range);
     LQ_CHECK_LAUNCH();

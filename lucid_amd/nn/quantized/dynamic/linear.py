@@ -23,6 +23,11 @@ from ...module import Module
 from .._utils import forget_weight_zero_points, storage_offset, weight_zero_points
 
 
+# The one-launch kernel keeps 16 rows of activation codes (16 K bytes) plus 1 KiB of scratch in
+# the 96 KiB of LDS it may use: wider layers take the two-launch route, whatever the batch.
+SMALL_LINEAR_MAX_K = 6080
+
+
 class Linear(Module):
     def __init__(self, in_features: int, out_features: int, bias: bool = True) -> None:
         super().__init__()
@@ -64,7 +69,7 @@ class Linear(Module):
         qd = self.act_qdtype
         off = storage_offset(qd)
         if (x._range is None and residual is None and activation is None and not track_range and 0 < M <= 64
-                and K % 16 == 0 and M * K <= 65536 and weight_zero_points(self) is None
+                and K % 16 == 0 and K <= SMALL_LINEAR_MAX_K and M * K <= 65536 and weight_zero_points(self) is None
                 and (self.bias is None or self.bias.dtype == T.float32)):
             # a small activation: min / max, qparams, codes, GEMM and bias in one launch (same bits)
             if self._wsum is None:

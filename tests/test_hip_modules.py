@@ -452,7 +452,7 @@ def test_engine_toggle():
 
 
 @pytest.mark.parametrize("M,K,N", [(64, 784, 256), (64, 256, 10), (1, 16, 1), (17, 48, 33), (5, 1024, 70), (64, 1024, 16),
-                                   (33, 1040, 100)])
+                                   (33, 1040, 100), (3, 6080, 40)])
 @pytest.mark.parametrize("kind", ["normal", "constant", "nan"])
 def test_small_dynamic_linear_in_one_launch(M, K, N, kind):
     """lq_dynamic_linear_small_f32 (min / max, qparams, codes, GEMM and bias of nnqd.Linear in one
@@ -492,3 +492,39 @@ def test_small_dynamic_linear_in_one_launch(M, K, N, kind):
     with pytest.raises(NotImplementedError, match="up to 64 rows"):
         _C.call("lq_dynamic_linear_small_f32", xd.data_ptr, 65, K, wd.data_ptr, N, wsd.data_ptr, wsum.data_ptr, None, 0, 0,
                 0, 255, 0, 1e-8, -128, y.data_ptr, None)
+
+
+@pytest.mark.parametrize("K", [6080, 6096, 8192, 11008, 16384])
+@pytest.mark.parametrize("M", [1, 4])
+def test_dynamic_linear_wide_layer_at_small_batch(M, K):
+    """nnqd.Linear on a layer too wide for the one-launch kernel (16 K bytes of codes must fit
+    96 KiB of LDS: K <= 6080) takes the two-launch route at any batch size, with the bits the
+    one-launch kernel would give: checked against the explicit quantize + GEMM pair."""
+    import lucid_amd.nn.quantized.dynamic as nnqd
+    from lucid_amd import _C, _ops
+    from lucid_amd.nn.quantized.dynamic.linear import SMALL_LINEAR_MAX_K
+    rng = np.random.default_rng(K + M)
+    N = 48
+    lin = nnqd.Linear(K, N)
+    w = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    lin.weight_int8 = hip(w)
+    lin.weight_scale = hip(rng.uniform(0.001, 0.01, N).astype(np.float32))
+    lin.bias = hip(rng.standard_normal(N).astype(np.float32))
+    lin._state_loaded("weight_int8")
+    x = (rng.standard_normal((M, K)) * 2).astype(np.float32)
+    xd = hip(x)
+    y = lin(xd).numpy()
+    xq = L.Tensor.empty((M, K), L.int8, "hip")
+    s, z = L.Tensor.empty((), L.float32, "hip"), L.Tensor.empty((), L.float32, "hip")
+    _C.call("lq_quantize_tensor_dynamic_i8", xd.data_ptr, M * K, 0, 0, 255, 0, 1e-8, -128, s.data_ptr, z.data_ptr,
+            None, None, xq.data_ptr, None)
+    want = _ops.qlinear_i8(xq, lin.weight_int8, a_zp=-128, a_zp_dev=z, a_scale=s, w_scale=lin.weight_scale,
+                           wsum=_ops.rowsum_i8(lin.weight_int8), bias=lin.bias, out_mode=_ops.OUT_F32).numpy()
+    assert y.shape == (M, N)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    if K > SMALL_LINEAR_MAX_K:
+        out = L.Tensor.empty((M, N), L.float32, "hip")
+        with pytest.raises(NotImplementedError, match="K <= 6080"):
+            _C.call("lq_dynamic_linear_small_f32", xd.data_ptr, M, K, lin.weight_int8.data_ptr, N,
+                    lin.weight_scale.data_ptr, _ops.rowsum_i8(lin.weight_int8).data_ptr, None, 0, 0, 0, 255, 0, 1e-8,
+                    -128, out.data_ptr, None)

@@ -618,3 +618,136 @@ def test_affine_weights_reject_what_they_cannot_do():
     with pytest.raises(L.ShapeMismatch):
         _ops.qlinear_i8(a, w, a_scale=one, w_scale=hip(np.ones(8, np.float32)), wsum=_ops.rowsum_i8(w),
                         w_zp=hip(np.ones(7, np.int32)))
+
+
+def _llm_layer(rng, M, K=4096, N=11008):
+    wf = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    mn, mx = O.minmax(wf, ch_axis=0)
+    ws, wz = O.calc_qparams(mn, mx, True, -128, 127, True)
+    wq = O.quantize(wf, ws, wz, -128, 127, ch_axis=0)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    mn, mx = O.minmax(x, ch_axis=0)
+    xs, xz = O.calc_qparams(mn, mx, True, -128, 127, True)
+    xq = O.quantize(x, xs, xz, -128, 127, ch_axis=0)
+    return xq, xs, wq, ws, bias
+
+
+def test_headline_shape_on_the_forced_ping_pong_kernel():
+    """M=2048, K=4096, N=11008 with tile_config 13 forced: the full grid of 8 x 32 tiles of
+    256 x 352 (one per compute unit, the last tile column mostly padding).  float16 output
+    against the oracle on rows sampled from every tile row; exact accumulators in full through
+    linearity, and a whole tile column (all 2048 rows x the last 96 real columns plus the
+    columns of the first tile) against the oracle's integer GEMM."""
+    from lucid_amd import _C
+    rng = np.random.default_rng(2048)
+    M, K, N = 2048, 4096, 11008
+    xq, xs, wq, ws, bias = _llm_layer(rng, M)
+    xd, wd = hip(xq), hip(wq)
+    got = _ops.qlinear_i8(xd, wd, a_scale=hip(xs), w_scale=hip(ws), bias=hip(bias), out_mode=_ops.OUT_F16,
+                          path=TILE, tile_config=13 | 0x100).numpy()
+    assert _C.load().lq_last_tile_config() == 0x10d
+    rows = np.unique(np.concatenate([rng.integers(0, M, 24), np.arange(0, M, 256), np.arange(255, M, 256)]))
+    exp = O.qlinear(xq[rows], wq, 0, xs[rows], ws, bias=bias, out_mode=O.OUT_F16)
+    assert np.array_equal(got[rows].view(np.uint16), exp.view(np.uint16))
+    acc = _ops.qlinear_i8(xd, wd, out_mode=_ops.OUT_ACC_I32, path=TILE, tile_config=13 | 0x100).numpy()
+    cols = np.concatenate([np.arange(0, 352), np.arange(31 * 352, N)])
+    assert np.array_equal(acc[:, cols], O.igemm(xq, wq[cols]))
+    xa, xb = codes(rng, (M, K), -60, 60), codes(rng, (M, K), -60, 60)
+    f = lambda t: _ops.qlinear_i8(hip(t), wd, out_mode=_ops.OUT_ACC_I32, path=TILE, tile_config=13 | 0x100).numpy()
+    assert np.array_equal(f(xa) + f(xb), f((xa + xb).astype(np.int8)))
+
+
+def test_first_call_under_capture_gets_the_ping_pong_kernel():
+    """The tuner may not time candidates on a stream that is being captured; the size rule it
+    falls back on must then give a large plain GEMM the eight-wavefront kernel (256 x 352 tiles
+    when they fit the 256 compute units better, 256 x 256 otherwise), not the four-wavefront
+    128 x 256 shape."""
+    from lucid_amd import _C
+    rng = np.random.default_rng(5)
+    for (M, K, N), want in (((2048, 4096, 11008), 0x10d), ((2048, 1024, 8192), 0x10e), ((4096, 576, 11008 - 352), 0x10d)):
+        a, w = codes(rng, (M, K)), codes(rng, (N, K))
+        ad, wd = hip(a), hip(w)
+        out = L.Tensor.empty((M, N), L.int32, "hip")
+        with L.graph.capture() as g:
+            _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, out=out)
+            cfg = _C.load().lq_last_tile_config()
+        assert cfg == want, hex(cfg)
+        g.replay()
+        _C.call("lq_sync", None)
+        rows = rng.integers(0, M, 16)
+        assert np.array_equal(out.numpy()[rows], O.igemm(a[rows], w))
+        g.destroy()
+
+
+def test_tuning_choices_export_and_import():
+    """lq_tune_export / lq_tune_import: a shape the tuner has timed appears in the exported text;
+    an imported line decides a shape this process has never run, without any timing (the
+    imported choice is what lq_last_tile_config reports), and the result is unchanged."""
+    import ctypes as C
+    from lucid_amd import _C
+    lib = _C.load()
+    rng = np.random.default_rng(9)
+    M, K, N = 640, 512, 768
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    ad, wd = hip(a), hip(w)
+    _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32)          # tuned here (0.5 GOP is the tuner's floor)
+    chosen = lib.lq_last_tile_config()
+    need = C.c_size_t()
+    _C.call("lq_tune_export", None, 0, C.byref(need))
+    buf = C.create_string_buffer(need.value)
+    _C.call("lq_tune_export", buf, need.value, C.byref(need))
+    lines = [ln for ln in buf.value.decode().splitlines() if ln.startswith("lq-tune-1 ")]
+    mine = [ln for ln in lines if ln.split()[1:4] == [str(M), str(N), str(K)]]
+    # the table keeps the tuner's candidate value (schedule 0 = one block per tile), the launch reports it resolved
+    assert len(mine) == 1 and int(mine[0].split()[-1]) & 0xff == chosen & 0xff
+    with pytest.raises(ValueError):
+        _C.call("lq_tune_export", buf, 1, C.byref(need))
+    # the same key with other extents and a shape the tuner would not pick first: 64 x 64 tiles
+    M2, N2 = 648, 776
+    fields = mine[0].split()
+    fields[1:4] = [str(M2), str(N2), str(K)]
+    fields[-1] = str(9 | 0x100)
+    taken = C.c_int()
+    _C.call("lq_tune_import", ("# a comment\n" + " ".join(fields) + "\n").encode(), C.byref(taken))
+    assert taken.value == 1
+    a2, w2 = codes(rng, (M2, K)), codes(rng, (N2, K))
+    acc = _ops.qlinear_i8(hip(a2), hip(w2), out_mode=_ops.OUT_ACC_I32).numpy()
+    assert lib.lq_last_tile_config() == (9 | 0x100)
+    assert np.array_equal(acc, O.igemm(a2, w2))
+    with pytest.raises(ValueError):
+        _C.call("lq_tune_import", b"lq-tune-1 1 2 3\n", None)
+
+
+def test_first_calls_from_two_threads():
+    """Two threads of a fresh process make their first launches at once (kernel attributes, the
+    padding table and the tuner's table are set up on first use): both get right results."""
+    import os, subprocess, sys, textwrap
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = textwrap.dedent("""
+        import sys, threading
+        import numpy as np
+        sys.path.insert(0, %r)
+        import lucid_amd as L
+        from lucid_amd import _C, _ops
+        import oracle as O
+        _C.init(0)
+        rng = np.random.default_rng(3)
+        M, K, N = 512, 256, 704
+        a = rng.integers(-128, 128, (M, K)).astype(np.int8)
+        w = rng.integers(-128, 128, (N, K)).astype(np.int8)
+        want = O.igemm(a, w)
+        ad, wd = L.tensor(a, device="hip"), L.tensor(w, device="hip")
+        go, bad = threading.Barrier(2), []
+        def run(cfg):
+            go.wait()
+            for _ in range(3):
+                got = _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, path=_ops.PATH_TILE, tile_config=cfg).numpy()
+                if not np.array_equal(got, want):
+                    bad.append(cfg)
+        ts = [threading.Thread(target=run, args=(c,)) for c in (13, 13)]
+        [t.start() for t in ts]; [t.join() for t in ts]
+        print("BAD" if bad else "OK", flush=True)
+    """ % root)
+    r = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and r.stdout.strip().endswith("OK"), r.stdout + r.stderr
