@@ -81,6 +81,9 @@ int lq_alloc(void** ptr, size_t nbytes);
 int lq_free(void* ptr);
 int lq_empty_cache(void);
 int lq_memory_stats(size_t* bytes_in_use, size_t* bytes_reserved); /* MemoryStats, bind_tensor.cpp */
+/* Free and total bytes of the current device as the driver reports them (hipMemGetInfo): unlike
+ * lq_memory_stats this sees every allocation, the library's own scratch included. */
+int lq_device_memory_info(size_t* free_bytes, size_t* total_bytes);
 int lq_h2d(void* dst_dev, const void* src_host, size_t nbytes, lq_stream stream);
 int lq_d2h(void* dst_host, const void* src_dev, size_t nbytes, lq_stream stream);
 int lq_d2d(void* dst_dev, const void* src_dev, size_t nbytes, lq_stream stream);
@@ -639,7 +642,8 @@ typedef struct {
                                 = acc - a_zp*wsum[n] - w_zp[n]*sum_k a[m,k] + K*a_zp*w_zp[n],
                               exact in int32 (K <= 33025); the row sums of a are taken by
                               the call, wsum is required.  NULL = symmetric weights;
-                              ignored in mode ACC_I32; not with range.            */
+                              LQ_ERR_VALUE with mode ACC_I32 (the raw sums a * w);
+                              not with range.                                      */
 } lq_qlinear_args;
 
 int lq_qlinear_i8(const lq_qlinear_args* args, lq_stream stream);
@@ -709,7 +713,7 @@ typedef struct {
                               (device), as lq_qlinear_args.w_zp; the window sums of the
                               image come from a convolution with an all-ones filter, so
                               taps in the padding count as a_zp and cancel exactly.
-                              NULL = symmetric; ignored in mode ACC_I32            */
+                              NULL = symmetric; LQ_ERR_VALUE with mode ACC_I32     */
 } lq_qconv2d_args;
 
 int lq_qconv2d_i8(const lq_qconv2d_args* args, lq_stream stream);

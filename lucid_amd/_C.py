@@ -67,6 +67,7 @@ _vp, _sz, _i, _f, _u64 = C.c_void_p, C.c_size_t, C.c_int, C.c_float, C.c_uint64
 _SIGNATURES = {
     "lq_version": [],
     "lq_last_tile_config": [],
+    "lq_device_memory_info": [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "lq_tune_export": [C.c_char_p, _sz, C.POINTER(C.c_size_t)],
     "lq_tune_import": [C.c_char_p, C.POINTER(C.c_int)],
     "lq_last_error": [],

@@ -485,7 +485,9 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
     const int jrc = set_join(g, p->join, p->out_mode, p->Cout, "qconv2d_i8");
     if (jrc) return jrc;
 
-    if (p->w_zp && p->out_mode != OUT_ACC_I32) {
+    LQ_REQUIRE(p->w_zp == nullptr || p->out_mode != OUT_ACC_I32, LQ_ERR_VALUE,
+               "qconv2d_i8: mode ACC_I32 returns the raw sums a * w; weight zero points cannot be applied to it");
+    if (p->w_zp) {
         // affine filters: the raw accumulators, then the window sums of the image as a
         // convolution with one all-ones filter per group (taps in the padding read the
         // code a_zp, as in the main pass), then the corrections and the epilogue proper
@@ -680,7 +682,9 @@ int lq_qconv3d_i8(const lq_qconv3d_args* p, lq_stream stream) {
     g.cpd = p->pad_lo[0]; g.cph = p->pad_lo[1]; g.cpw = p->pad_lo[2];
     g.cdd = p->dilation[0]; g.cdh = p->dilation[1]; g.cdw = p->dilation[2];
 
-    if (p->w_zp && p->out_mode != OUT_ACC_I32) {
+    LQ_REQUIRE(p->w_zp == nullptr || p->out_mode != OUT_ACC_I32, LQ_ERR_VALUE,
+               "qconv3d_i8: mode ACC_I32 returns the raw sums a * w; weight zero points cannot be applied to it");
+    if (p->w_zp) {
         // affine filters, as in lq_qconv2d_i8: raw accumulators, the window sums of the volume
         // from one all-ones filter per group, then the corrections and the epilogue proper
         LQ_REQUIRE(p->wsum, LQ_ERR_VALUE, "qconv3d_i8: affine filters need the filter sums");

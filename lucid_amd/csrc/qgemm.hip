@@ -971,7 +971,9 @@ int lq_qlinear_i8(const lq_qlinear_args* p, lq_stream stream) {
     g.gelu = p->gelu != 0;
     g.range = p->range;
 
-    if (p->w_zp && p->out_mode != OUT_ACC_I32) {
+    LQ_REQUIRE(p->w_zp == nullptr || p->out_mode != OUT_ACC_I32, LQ_ERR_VALUE,
+               "qlinear_i8: mode ACC_I32 returns the raw sums a * w; weight zero points cannot be applied to it");
+    if (p->w_zp) {
         // affine weights: raw accumulators and the activation row sums into temporaries,
         // then one elementwise pass with the corrections and the epilogue proper
         LQ_REQUIRE(p->wsum, LQ_ERR_VALUE, "qlinear_i8: affine weights need the weight row sums");

@@ -73,9 +73,10 @@ struct GraphRec {
     hipGraph_t graph = nullptr;      // the captured template, kept until the exec is destroyed
     hipGraphExec_t exec = nullptr;   // null while capturing or after a failed end
     std::vector<std::pair<int, void*>> blocks;  // (device, block) allocated during capture
+    bool capturing = false;          // between a successful begin and its end / destroy
 };
 std::unordered_map<int, GraphRec> g_graphs;
-int g_captures_in_progress = 0;
+int g_captures_in_progress = 0;  // records with `capturing` set; changed only together with that flag
 int g_next_graph_id = 1;
 thread_local int t_capturing_graph = 0;  // id of the graph this thread is capturing, 0 = none
 
@@ -296,6 +297,12 @@ extern "C" int lq_empty_cache(void) {
     return LQ_OK;
 }
 
+extern "C" int lq_device_memory_info(size_t* free_bytes, size_t* total_bytes) {
+    LQ_REQUIRE(free_bytes && total_bytes, LQ_ERR_VALUE, "device_memory_info: NULL pointer");
+    LQ_HIP(hipMemGetInfo(free_bytes, total_bytes));
+    return LQ_OK;
+}
+
 extern "C" int lq_memory_stats(size_t* bytes_in_use, size_t* bytes_reserved) {
     int dev = 0;
     LQ_HIP(hipGetDevice(&dev));
@@ -317,7 +324,7 @@ extern "C" int lq_graph_begin(lq_stream stream, int* graph_id) {
     {
         std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
         id = g_next_graph_id++;
-        g_graphs[id];
+        g_graphs[id].capturing = true;
         ++g_captures_in_progress;
     }
     hipError_t e = hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed);
@@ -342,8 +349,13 @@ extern "C" int lq_graph_end(lq_stream stream, int graph_id) {
     hipError_t e2 = hipSuccess;
     if (e == hipSuccess) e2 = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
-    if (g_captures_in_progress > 0) --g_captures_in_progress;
     auto it = g_graphs.find(graph_id);
+    // only this record's own capture ends here: a stray or repeated call for another id must not
+    // make a capture that is still running look finished
+    if (it != g_graphs.end() && it->second.capturing) {
+        it->second.capturing = false;
+        --g_captures_in_progress;
+    }
     if (e != hipSuccess || e2 != hipSuccess || it == g_graphs.end()) {
         if (graph) (void)hipGraphDestroy(graph);
         if (exec) (void)hipGraphExecDestroy(exec);
@@ -374,9 +386,10 @@ extern "C" int lq_graph_destroy(int graph_id) {
     std::lock_guard<std::recursive_mutex> lock(g_rt_mutex);
     auto it = g_graphs.find(graph_id);
     if (it == g_graphs.end()) return LQ_OK;
-    if (t_capturing_graph == graph_id) {  // destroyed without an end: the capture is abandoned
-        t_capturing_graph = 0;
-        if (g_captures_in_progress > 0) --g_captures_in_progress;
+    if (t_capturing_graph == graph_id) t_capturing_graph = 0;
+    if (it->second.capturing) {  // destroyed without an end (by whichever thread): the capture is abandoned
+        it->second.capturing = false;
+        --g_captures_in_progress;
     }
     hipError_t e = hipSuccess;
     if (it->second.exec) e = hipGraphExecDestroy(it->second.exec);

@@ -562,8 +562,10 @@ def test_affine_weight_zero_points_every_output_form(M, N, K, path):
         got = _ops.qlinear_i8(ad, wd, out_mode=mode, **dkw).numpy()
         exp = O.qlinear(a, w, za, a_scale, w_scale, out_mode=mode, **okw)
         assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), mode
-    # raw accumulators are unchanged by the zero points
-    acc = _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, w_zp=hip(zw), wsum=_ops.rowsum_i8(wd), path=path)
+    # the raw accumulators are the sums a * w: weight zero points cannot apply to them and are refused
+    with pytest.raises(ValueError, match="ACC_I32"):
+        _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, w_zp=hip(zw), wsum=_ops.rowsum_i8(wd), path=path)
+    acc = _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, path=path)
     assert np.array_equal(acc.numpy(), O.igemm(a, w))
 
 

@@ -89,3 +89,38 @@ def test_noalloc_makes_no_pool_allocation():
     _C.call("lq_memory_stats", C.byref(used1), C.byref(res1))
     assert (used1.value, res1.value) == (used0.value, res0.value)
     assert mn.numpy()[0] == 1.0 and mx.numpy()[0] == 1.0
+
+
+def test_noalloc_takes_no_device_memory_at_all():
+    """The pool's statistics do not see the library's own scratch (raw hipMalloc), so the contract
+    is checked against the driver's free-memory figure, on a stream that has never been used: there
+    lq_minmax has to allocate its 4 MiB workspace (which the figure shows), lq_minmax_noalloc
+    nothing."""
+    _C.init()
+    x = L.tensor(np.arange(1 << 22, dtype=np.float32), device="hip")
+    mn = L.Tensor.empty((1,), L.float32, "hip")
+    mx = L.Tensor.empty((1,), L.float32, "hip")
+
+    def free_bytes():
+        _C.call("lq_sync", None)
+        f, t = C.c_size_t(), C.c_size_t()
+        _C.call("lq_device_memory_info", C.byref(f), C.byref(t))
+        return f.value
+
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    _C.call("lq_stream_create", C.byref(s1))
+    _C.call("lq_stream_create", C.byref(s2))
+    _C.call("lq_minmax_noalloc", x.data_ptr, 1, 1, 1 << 22, mn.data_ptr, mx.data_ptr, None)  # first use is behind us
+    for s in (s1, s2):  # and so is whatever the runtime sets up at a stream's first launch
+        _C.call("lq_fill_bytes", mn.data_ptr, 0, 4, s)
+        _C.call("lq_sync", s)
+    before = free_bytes()
+    _C.call("lq_minmax_noalloc", x.data_ptr, 1, 1, 1 << 22, mn.data_ptr, mx.data_ptr, s1)
+    _C.call("lq_sync", s1)
+    assert free_bytes() == before
+    assert mn.numpy()[0] == 0.0 and mx.numpy()[0] == float((1 << 22) - 1)
+    # the allocating entry point on another fresh stream: the figure does see library scratch
+    _C.call("lq_minmax", x.data_ptr, 1, 1, 1 << 22, mn.data_ptr, mx.data_ptr, s2)
+    _C.call("lq_sync", s2)
+    assert free_bytes() <= before - (4 << 20)
+    assert mn.numpy()[0] == 0.0 and mx.numpy()[0] == float((1 << 22) - 1)
