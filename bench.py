@@ -131,7 +131,27 @@ def make_linear(L, Q, _C, _ops, M, K, N, seed):
     return dict(x=x, xq=xq, xs=xs, wq=wq, ws=ws, bias=bias, out=out)
 
 
-def bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup, seed=1):
+def sample_for_verification(t, M, N, seed, rows=32):
+    """Host copies of `rows` sampled rows of the timed output and of everything that determines
+    them (their activation codes and scales, the whole weight matrix, scales, bias)."""
+    rng = np.random.default_rng(seed + 100)
+    idx = np.unique(np.concatenate([rng.integers(0, M, rows), [0, M - 1]]))
+    out = t["out"].numpy()
+    return dict(rows=idx, out=out[idx].copy(), xq=t["xq"].numpy()[idx].copy(), xs=t["xs"].numpy()[idx].copy(),
+                wq=t["wq"].numpy(), ws=t["ws"].numpy(), bias=t["bias"].numpy())
+
+
+def verify_linear_sample(v):
+    """The sampled rows of the timed float16 output against the oracle's integer formulation
+    (bit for bit).  Called from the cpu_baseline leg only."""
+    import oracle as O
+
+    exp = O.qlinear(v["xq"], v["wq"], 0, v["xs"], v["ws"], bias=v["bias"], out_mode=O.OUT_F16)
+    same = np.array_equal(v["out"].view(np.uint16), exp.view(np.uint16))
+    return {"rows_checked": int(len(v["rows"])), "columns": int(exp.shape[1]), "bit_exact": bool(same)}
+
+
+def bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup, seed=1, keep_verify_sample=False):
     t = make_linear(L, Q, _C, _ops, M, K, N, seed)
 
     def step(repeat=1):
@@ -174,10 +194,36 @@ def bench_linear(L, Q, _C, _ops, M, K, N, steps, warmup, seed=1):
         first()
         tot_a, _ = time_launches(_C, lambda: first(steps), 1, 1)
         split = dict(columns=NA, ops=2.0 * M * K * NA, avg_ms=tot_a / steps)
-    return dict(tile_config=tile_config, split=split, total_ms=total, avg_kernel_ms=avg_ms, median_ms=float(np.median(per)),
+    verify = None
+    if keep_verify_sample:
+        # what the timed launches left in `out`, with the operands of the same rows: checked
+        # against the CPU restatement in the cpu_baseline leg (sample_for_verification)
+        verify = sample_for_verification(t, M, N, seed)
+    return dict(tile_config=tile_config, split=split, verify=verify, total_ms=total, avg_kernel_ms=avg_ms, median_ms=float(np.median(per)),
                 p95_ms=float(np.percentile(per, 95)), ops=ops, bytes=bytes_alg,
                 tops=ops / (total / steps) / 1e9, kernel_tops=ops / avg_ms / 1e9,
                 gbs=bytes_alg / avg_ms / 1e6, tensors=t)
+
+
+def zero_operand_rate(L, _C, _ops, t, M, K, N):
+    """TOP/s of the headline launch with every activation and weight code zero (scales, bias and
+    output form unchanged): how fast the kernel's structure runs when the matrix cores draw the
+    least power.  A diagnostic beside the timed figure."""
+    xz = L.Tensor.empty((M, K), L.int8, "hip")
+    wz = L.Tensor.empty((N, K), L.int8, "hip")
+    _C.call("lq_fill_bytes", xz.data_ptr, 0, M * K, None)
+    _C.call("lq_fill_bytes", wz.data_ptr, 0, N * K, None)
+    scratch = L.Tensor.empty((M, N), L.float16, "hip")
+
+    def step(repeat=1):
+        _ops.qlinear_i8(xz, wz, a_scale=t["xs"], w_scale=t["ws"], bias=t["bias"], out_mode=_ops.OUT_F16,
+                        out=scratch, repeat=repeat)
+
+    step()
+    step(300)
+    _C.call("lq_sync", None)
+    total, _ = time_launches(_C, lambda: step(200), 1, 1)
+    return 2.0 * M * K * N / (total / 200) / 1e9
 
 
 def bench_linear_cold_weights(L, _C, _ops, t, M, K, N, steps):
@@ -198,7 +244,7 @@ def bench_linear_cold_weights(L, _C, _ops, t, M, K, N, steps):
     return total / (steps * copies) * 1e3
 
 
-def probe_mfma_ceiling(L, _C, xq, wq, ms_target=40.0):
+def probe_mfma_ceiling(L, _C, xq, wq, ms_target=40.0, entry="lq_probe_mfma_i8"):
     """TOP/s of a loop of nothing but int8 MFMAs over register operands taken from
     the benchmark's own activation and weight codes (two wavefronts per SIMD, eight
     independent accumulators each): what the matrix cores sustain for this data under
@@ -211,7 +257,7 @@ def probe_mfma_ceiling(L, _C, xq, wq, ms_target=40.0):
     def run(iters):
         evs = _events(_C, 2)
         _C.call("lq_event_record", evs[0], None)
-        _C.call("lq_probe_mfma_i8", xq.data_ptr, wq.data_ptr, nbytes, iters, sink.data_ptr, C.byref(ops), None)
+        _C.call(entry, xq.data_ptr, wq.data_ptr, nbytes, iters, sink.data_ptr, C.byref(ops), None)
         _C.call("lq_event_record", evs[1], None)
         _C.call("lq_event_sync", evs[1])
         ms = _elapsed_ms(_C, evs[0], evs[1])
@@ -334,7 +380,31 @@ def bench_quant_roundtrip(L, Q, _C, steps, warmup):
         out[name] = {"us": round(med * 1e3, 1), "GB/s": round(nbytes / med / 1e6, 1),
                      "frac_of_8TBs": round(nbytes / med / 1e6 / PEAK_HBM_GBS, 4),
                      "bytes": nbytes, "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+    # a slice of what the timed kernels left behind (channel 1234: input, codes, the per-channel
+    # dequantization of those codes), checked against the CPU restatement in the cpu_baseline leg
+    ch = 1234
+    _C.call("lq_dequantize", q.data_ptr, _C.I8, 0, dq.data_ptr, 1, Cn, inner, s.data_ptr, z.data_ptr, 0, None)
+    _C.call("lq_sync", None)
+    QUANT_VERIFY.update(x=x.row_range(ch, ch + 1).numpy().reshape(-1), q=q.row_range(ch, ch + 1).numpy().reshape(-1),
+                        dq=dq.row_range(ch, ch + 1).numpy().reshape(-1), s=s.numpy()[ch:ch + 1], z=z.numpy()[ch:ch + 1])
     return out
+
+
+QUANT_VERIFY = {}
+
+
+def verify_quant_slice():
+    """One channel of the timed quantize / dequantize outputs against the oracle, bit for bit."""
+    import oracle as O
+
+    v = QUANT_VERIFY
+    if not v:
+        return None
+    codes = O.quantize(v["x"], v["s"], v["z"], -128, 127)
+    back = O.dequantize(codes, v["s"], v["z"])
+    return {"elements_checked": int(v["x"].size),
+            "bit_exact": bool(np.array_equal(codes.astype(np.int8), v["q"]) and
+                              np.array_equal(back.view(np.uint32), v["dq"].view(np.uint32)))}
 
 
 def _acc_digest(c):
@@ -544,8 +614,26 @@ def bench_weight_only(L, _C, steps, warmup, K=4096, N=11008, gs=64):
             us = time_in_graph(L, _C, fn, max(10, steps // 2)) * 1e3
             _, per = time_launches(_C, fn, steps, warmup)
             gbs = nbytes / (us * 1e-6) / 1e9
-            out[f"w{bits}_m{m}"] = {"us": round(us, 2), "bracketed_launch_median_us": round(float(np.median(per)) * 1e3, 2),
-                                    "GB/s": round(gbs, 1), "frac_of_8TBs": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+            # cold: the launches of one graph cycle through copies of the packed weight that together
+            # exceed the 256 MB last-level cache, so every byte comes from HBM (what a model's layers see)
+            copies = int(320e6 // nbytes) + 2
+            sets = [(packed, scales, biases)] + [(packed.clone(), scales.clone(), biases.clone()) for _ in range(copies - 1)]
+            with L.graph.capture() as g:
+                for (pk, sc, bi) in sets:
+                    _C.call("lq_wq_matmul", x.data_ptr, pk.data_ptr, sc.data_ptr, bi.data_ptr, m, N, K, gs, bits,
+                            res.data_ptr, None)
+            for _ in range(5):
+                g.replay()
+            tot, _ = time_launches(_C, g.replay, max(10, steps // 2), 2)
+            g.destroy()
+            cold_us = tot / (max(10, steps // 2) * copies) * 1e3
+            del sets
+            out[f"w{bits}_m{m}"] = {"us_weights_in_llc": round(us, 2),
+                                    "bracketed_launch_median_us": round(float(np.median(per)) * 1e3, 2),
+                                    "GB/s_weights_in_llc": round(gbs, 1),
+                                    "frac_of_8TBs_llc_resident": round(gbs / PEAK_HBM_GBS, 4),
+                                    "us": round(cold_us, 2), "GB/s": round(nbytes / cold_us / 1e3, 1),
+                                    "frac_of_8TBs": round(nbytes / cold_us / 1e3 / PEAK_HBM_GBS, 4), "bytes": nbytes}
     return out
 
 
@@ -737,9 +825,12 @@ def main() -> int:
                              ("uniform_-127..127", -127, 127)):
             _C.call("lq_fill_uniform_i8", a.data_ptr, n, 1, lo, hi, None)
             _C.call("lq_fill_uniform_i8", b.data_ptr, n, 2, lo, hi, None)
-            res[name] = round(probe_mfma_ceiling(L, _C, a, b), 1)
+            res[name] = {"32x32x32": round(probe_mfma_ceiling(L, _C, a, b), 1),
+                         "16x16x64": round(probe_mfma_ceiling(L, _C, a, b, entry="lq_probe_mfma_i8_k64"), 1)}
         t = make_linear(L, Q, _C, _ops, M, K, N, 1)
-        res["benchmark_codes"] = round(probe_mfma_ceiling(L, _C, t["xq"], t["wq"]), 1)
+        res["benchmark_codes"] = {"32x32x32": round(probe_mfma_ceiling(L, _C, t["xq"], t["wq"]), 1),
+                                  "16x16x64": round(probe_mfma_ceiling(L, _C, t["xq"], t["wq"],
+                                                                       entry="lq_probe_mfma_i8_k64"), 1)}
         print(json.dumps({"mfma_only_tops_by_operand_data": res, "datasheet_peak_tops": PEAK_INT8_TOPS}))
         return 0
     if args.only == "decode":
@@ -748,8 +839,10 @@ def main() -> int:
         for m in (1, 16):
             rs = bench_linear(L, Q, _C, _ops, m, K, N, max(args.steps, 400), args.warmup, seed=3)
             cold_us = bench_linear_cold_weights(L, _C, _ops, rs["tensors"], m, K, N, max(10, args.steps // 2))
-            res[f"linear_m{m}"] = {"us": round(rs["avg_kernel_ms"] * 1e3, 2), "frac_of_8TBs": round(rs["gbs"] / PEAK_HBM_GBS, 4),
-                                   "cold_weights_us": round(cold_us, 2)}
+            res[f"linear_m{m}"] = {"us": round(cold_us, 2),
+                                   "frac_of_8TBs": round(rs["bytes"] / cold_us / 1e3 / PEAK_HBM_GBS, 4),
+                                   "us_weights_in_llc": round(rs["avg_kernel_ms"] * 1e3, 2),
+                                   "frac_of_8TBs_llc_resident": round(rs["gbs"] / PEAK_HBM_GBS, 4)}
         res["weight_only_group64_k4096_n11008"] = bench_weight_only(L, _C, args.steps, args.warmup)
         print(json.dumps(res))
         return 0
@@ -761,7 +854,7 @@ def main() -> int:
     if args.vendor_yardstick:
         print(json.dumps(vendor_yardstick(L, Q, _C, _ops, args.steps, args.warmup)))
         return 0
-    r = bench_linear(L, Q, _C, _ops, M, K, N, args.steps, args.warmup)
+    r = bench_linear(L, Q, _C, _ops, M, K, N, args.steps, args.warmup, keep_verify_sample=True)
     line = {
         "metric": "quantized-Linear int8 TOPS & % MFMA peak; int8 ResNet-50 images/sec",
         "value": round(r["tops"], 2),
@@ -813,9 +906,16 @@ def main() -> int:
         _C.call("lq_sync", None)
         del src, dst
     # the same operand codes through a loop of MFMAs alone: the data-dependent ceiling
-    ceiling = probe_mfma_ceiling(L, _C, r["tensors"]["xq"], r["tensors"]["wq"])
+    # (v_mfma_i32_16x16x64_i8 in the kernel's own register walk: the instruction the kernel issues;
+    # the 32x32x32 form, which draws more power per operation, beside it)
+    ceiling = probe_mfma_ceiling(L, _C, r["tensors"]["xq"], r["tensors"]["wq"], entry="lq_probe_mfma_i8_k64")
     line["roofline"]["mfma_only_same_operands_tops"] = round(ceiling, 1)
     line["roofline"]["frac_of_mfma_only"] = round(r["kernel_tops"] / ceiling, 4)
+    line["roofline"]["mfma_only_same_operands_32x32x32_tops"] = round(
+        probe_mfma_ceiling(L, _C, r["tensors"]["xq"], r["tensors"]["wq"]), 1)
+    # diagnostic, never the headline: the same launch on all-zero operands.  No operand bit toggles,
+    # so the board's power limit does not pull the clock down and what is left is the kernel's structure.
+    line["roofline"]["zero_operands_diagnostic_tops"] = round(zero_operand_rate(L, _C, _ops, r["tensors"], M, K, N), 1)
     if not args.no_extra:
         extra = {}
         fused_tops, separate_tops = bench_act_quant_plus_linear(L, Q, _C, _ops, r["tensors"], M, K, N,
@@ -835,13 +935,16 @@ def main() -> int:
             # cache, i.e. every byte from HBM (the back-to-back figure re-reads one 45 MB matrix,
             # which stays in the 256 MB cache between launches)
             cold_us = bench_linear_cold_weights(L, _C, _ops, rs["tensors"], m, K, N, max(10, args.steps // 2))
-            extra[f"linear_m{m}"] = {"us": round(rs["avg_kernel_ms"] * 1e3, 2),
+            # us / GB/s / frac_of_8TBs: weights from HBM (the cycling copies); *_llc_resident / *_weights_in_llc:
+            # the back-to-back launches on one matrix, which is cache bandwidth, not HBM bandwidth
+            extra[f"linear_m{m}"] = {"us": round(cold_us, 2),
+                                     "GB/s": round(rs["bytes"] / cold_us / 1e3, 1),
+                                     "frac_of_8TBs": round(rs["bytes"] / cold_us / 1e3 / PEAK_HBM_GBS, 4),
+                                     "us_weights_in_llc": round(rs["avg_kernel_ms"] * 1e3, 2),
                                      "bracketed_launch_median_us": round(rs["median_ms"] * 1e3, 2),
-                                     "GB/s": round(rs["gbs"], 1),
-                                     "frac_of_8TBs": round(rs["gbs"] / PEAK_HBM_GBS, 4),
-                                     "cold_weights_us": round(cold_us, 2),
-                                     "cold_weights_frac_of_8TBs": round(rs["bytes"] / cold_us / 1e3 / PEAK_HBM_GBS, 4),
-                                     "TOP/s": round(rs["kernel_tops"], 2), "bytes": rs["bytes"]}
+                                     "GB/s_weights_in_llc": round(rs["gbs"], 1),
+                                     "frac_of_8TBs_llc_resident": round(rs["gbs"] / PEAK_HBM_GBS, 4),
+                                     "TOP/s_weights_in_llc": round(rs["kernel_tops"], 2), "bytes": rs["bytes"]}
             del rs["tensors"]
         # the same layer at a prefill-sized M: more tiles per CU, better-filled rounds
         rl = bench_linear(L, Q, _C, _ops, 8192, K, N, max(10, args.steps // 2), max(3, args.warmup // 2), seed=5)
@@ -872,7 +975,17 @@ def main() -> int:
                       f"({dt:.2f} s per call, {spent:.0f} s of CPU time in all)",
             "single_thread": single,
         }
+        # the timed outputs against the CPU restatement, in this leg only
+        checks = {"linear_m2048_fp16_output": verify_linear_sample(r["verify"])}
+        qv = verify_quant_slice()
+        if qv is not None:
+            checks["quantize_dequantize_per_channel_slice"] = qv
+        line["verified"] = all(c["bit_exact"] for c in checks.values())
+        line["verification"] = checks
     print(json.dumps(line))
+    if line.get("verified") is False:
+        print("bench.py: a timed output differs from the CPU restatement", file=sys.stderr)
+        return 1
     return 0
 
 

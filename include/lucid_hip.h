@@ -215,6 +215,12 @@ int lq_selftest_requant_route(float scale, float zp, int qmin, int qmax, int rel
  * counterpart in Lucid. */
 int lq_probe_mfma_i8(const int8_t* a, const int8_t* b, size_t nbytes, int iters, int* sink,
                      double* ops, lq_stream stream);
+/* The same probe with the instruction and the register walk of the large-GEMM kernel: each
+ * wavefront keeps 4 x 11 tiles of v_mfma_i32_16x16x64_i8 (2*16*16*64 operations each) and visits
+ * them column by column, alternating the row order; at least 44 KiB per operand.  The two
+ * instructions sustain different rates on the same operand data under the power limit. */
+int lq_probe_mfma_i8_k64(const int8_t* a, const int8_t* b, size_t nbytes, int iters, int* sink,
+                         double* ops, lq_stream stream);
 /* Plain device copy kernel (n bytes, 16-byte vectors): the calibration
  * workload for hardware-counter scaling. */
 int lq_copy_kernel(void* dst, const void* src, size_t nbytes, lq_stream stream);

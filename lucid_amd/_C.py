@@ -116,6 +116,7 @@ _SIGNATURES = {
     "lq_dynamic_linear_small_f32": [_vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _i, _vp, _vp],
     "lq_selftest_requant_route": [C.c_float, C.c_float, _i, _i, _i, C.c_ulonglong, C.c_ulonglong, _vp, _vp, _vp],
     "lq_probe_mfma_i8": [_vp, _vp, _sz, _i, _vp, C.POINTER(C.c_double), _vp],
+    "lq_probe_mfma_i8_k64": [_vp, _vp, _sz, _i, _vp, C.POINTER(C.c_double), _vp],
     "lq_copy_kernel": [_vp, _vp, _sz, _vp],
     "lq_minmax": [_vp, _sz, _sz, _sz, _vp, _vp, _vp],
     "lq_minmax_noalloc": [_vp, _sz, _sz, _sz, _vp, _vp, _vp],

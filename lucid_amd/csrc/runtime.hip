@@ -615,6 +615,40 @@ __global__ __launch_bounds__(256) void probe_mfma_i8_kernel(const int8_t* __rest
     if (threadIdx.x == 0) sink[0] = s;
 }
 
+// The same probe with the instruction and the walk of the large-GEMM kernel: a wavefront owns
+// 4 x 11 tiles of v_mfma_i32_16x16x64_i8, visits them column by column with the row order
+// alternating (one operand changes between neighbours), two wavefronts per SIMD.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void probe_mfma_i8_k64_kernel(
+    const int8_t* __restrict__ a, const int8_t* __restrict__ b, int iters, int* __restrict__ sink) {
+    probe_v4i acc[4][11];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 11; ++j) acc[i][j] = probe_v4i{0, 0, 0, 0};
+    probe_v4i ra[4], rb[11];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ra[i] = reinterpret_cast<const probe_v4i*>(a)[i * 256 + threadIdx.x];
+#pragma unroll
+    for (int j = 0; j < 11; ++j) rb[j] = reinterpret_cast<const probe_v4i*>(b)[j * 256 + threadIdx.x];
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 11; ++j)
+#pragma unroll
+            for (int ii = 0; ii < 4; ++ii) {
+                const int i = (j & 1) ? 3 - ii : ii;
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(rb[j], ra[i], acc[i][j], 0, 0, 0);
+            }
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 11; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s ^= acc[i][j][r];
+    if (threadIdx.x == 0) sink[0] = s;
+}
+
 __global__ void fill_bytes_kernel(uint8_t* x, size_t n, uint8_t v) {
     size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     size_t stride = size_t(gridDim.x) * blockDim.x;
@@ -677,6 +711,23 @@ int lq_probe_mfma_i8(const int8_t* a, const int8_t* b, size_t nbytes, int iters,
     hipLaunchKernelGGL(probe_mfma_i8_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), a, b, iters, sink);
     LQ_CHECK_LAUNCH("probe_mfma_i8");
     *ops = double(blocks) * 4.0 * double(iters) * 8.0 * (2.0 * 32 * 32 * 32);
+    return LQ_OK;
+}
+
+int lq_probe_mfma_i8_k64(const int8_t* a, const int8_t* b, size_t nbytes, int iters, int* sink, double* ops,
+                         lq_stream stream) {
+    LQ_REQUIRE(a && b && sink && ops, LQ_ERR_VALUE, "probe_mfma_i8_k64: NULL pointer");
+    LQ_REQUIRE(iters > 0, LQ_ERR_VALUE, "probe_mfma_i8_k64: iters must be positive");
+    LQ_REQUIRE(nbytes >= size_t(256) * 11 * 16, LQ_ERR_SHAPE, "probe_mfma_i8_k64: need at least 44 KiB of operand data");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0, LQ_ERR_VALUE,
+               "probe_mfma_i8_k64: operands must be 16-byte aligned");
+    int dev = 0, cus = 0;
+    LQ_HIP(hipGetDevice(&dev));
+    LQ_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int blocks = 2 * cus;  // two wavefronts per SIMD
+    hipLaunchKernelGGL(probe_mfma_i8_k64_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), a, b, iters, sink);
+    LQ_CHECK_LAUNCH("probe_mfma_i8_k64");
+    *ops = double(blocks) * 4.0 * double(iters) * 44.0 * (2.0 * 16 * 16 * 64);
     return LQ_OK;
 }
 
