@@ -795,6 +795,14 @@ int lq_im2col_ndhwc_i8(const int8_t* x, int8_t* cols, int B, int D, int H, int W
 int lq_transpose_i8(const int8_t* src, int8_t* dst, int batches, size_t R, size_t Cn, size_t src_stride,
                     size_t dst_stride, lq_stream stream);
 
+/* F.pad on the last two axes of a float32 tensor seen as `planes` images of H x W
+ * (lucid/nn/modules/conv.py:104-123 pre-pads this way for padding_mode != "zeros"; mode 0
+ * pads with zeros, for the uneven amounts of padding="same"): mode 1 reflect, 2 replicate,
+ * 3 circular.  out is [planes, H+top+bottom, W+left+right].  The float-input form of the
+ * quantized convolutions runs on it. */
+int lq_pad_planes_f32(const float* x, float* out, size_t planes, int H, int W, int pad_top, int pad_bottom,
+                      int pad_left, int pad_right, int mode, lq_stream stream);
+
 /* F.pad with mode reflect (1) / replicate (2) / circular (3) on NHWC codes: how a
  * quantized convolution with padding_mode != "zeros" pads before convolving with
  * padding 0 (lucid/nn/modules/conv.py:104-123).  The padded float image is a gather

@@ -331,6 +331,25 @@ __global__ __launch_bounds__(256) void pad_nhwc_i8_kernel(const int8_t* __restri
 }
 
 
+// F.pad on the last two axes of a float tensor viewed as `planes` images of H x W: mode 0 pads
+// with zeros, 1 / 2 / 3 are reflect / replicate / circular.  One lane per output element.
+__global__ __launch_bounds__(256) void pad_planes_f32_kernel(const float* __restrict__ x, float* __restrict__ out,
+                                                             size_t planes, int H, int W, int pt, int pl, int OH,
+                                                             int OW, int mode) {
+    const size_t total = planes * OH * OW;
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int ow = int(i % OW), oh = int((i / OW) % OH);
+    const size_t p = i / (size_t(OW) * OH);
+    const int ih0 = oh - pt, iw0 = ow - pl;
+    float v = 0.0f;
+    if (mode != 0 || (ih0 >= 0 && ih0 < H && iw0 >= 0 && iw0 < W)) {
+        const int ih = pad_source(ih0, H, mode), iw = pad_source(iw0, W, mode);
+        v = x[(p * H + ih) * W + iw];
+    }
+    out[i] = v;
+}
+
 // max-pool on codes, NHWC.  Quantisation is monotone, so the maximum of the
 // codes is the code of the maximum; padded taps never win.
 __global__ __launch_bounds__(256) void maxpool_nhwc_i8_kernel(const int8_t* __restrict__ x,
@@ -833,6 +852,28 @@ int lq_pad_nhwc_i8(const int8_t* x, int8_t* out, int B, int H, int W, int C, int
     hipLaunchKernelGGL(pad_nhwc_i8_kernel, dim3(unsigned((total + 255) / 256)), dim3(256), 0, as_stream(stream), x,
                        out, B, H, W, C, pad_top, pad_left, OH, OW, mode, vec);
     LQ_CHECK_LAUNCH("pad_nhwc_i8");
+    return LQ_OK;
+}
+
+int lq_pad_planes_f32(const float* x, float* out, size_t planes, int H, int W, int pad_top, int pad_bottom,
+                      int pad_left, int pad_right, int mode, lq_stream stream) {
+    LQ_REQUIRE(mode >= 0 && mode <= 3, LQ_ERR_VALUE, "pad_planes_f32: mode %d (0 zeros, 1 reflect, 2 replicate, 3 circular)", mode);
+    LQ_REQUIRE(H > 0 && W > 0 && pad_top >= 0 && pad_bottom >= 0 && pad_left >= 0 && pad_right >= 0, LQ_ERR_VALUE,
+               "pad_planes_f32: bad extents");
+    if (mode == 1)
+        LQ_REQUIRE(pad_top < H && pad_bottom < H && pad_left < W && pad_right < W, LQ_ERR_VALUE,
+                   "pad_planes_f32: reflect padding must be smaller than the image");
+    if (mode == 3)
+        LQ_REQUIRE(pad_top <= H && pad_bottom <= H && pad_left <= W && pad_right <= W, LQ_ERR_VALUE,
+                   "pad_planes_f32: circular padding must not exceed the image");
+    const int OH = H + pad_top + pad_bottom, OW = W + pad_left + pad_right;
+    const size_t total = planes * OH * OW;
+    if (total == 0) return LQ_OK;
+    LQ_REQUIRE(x && out, LQ_ERR_VALUE, "pad_planes_f32: NULL pointer");
+    LQ_REQUIRE((total + 255) / 256 < 0x7fffffffull, LQ_ERR_SHAPE, "pad_planes_f32: tensor too large");
+    hipLaunchKernelGGL(pad_planes_f32_kernel, dim3(unsigned((total + 255) / 256)), dim3(256), 0, as_stream(stream), x, out,
+                       planes, H, W, pad_top, pad_left, OH, OW, mode);
+    LQ_CHECK_LAUNCH("pad_planes_f32");
     return LQ_OK;
 }
 

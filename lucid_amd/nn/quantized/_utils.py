@@ -87,6 +87,60 @@ def forget_weight_zero_points(mod) -> None:
     mod.__dict__.pop("_wzp", None)
 
 
+def is_plain_float(x) -> bool:
+    """A float32 device tensor that carries no quantization grid: the input for which a quantized
+    layer takes Lucid's float formulation."""
+    return isinstance(x, Tensor) and x.device == "hip" and x._grid is None and x.dtype == T.float32
+
+
+def float_input_conv(mod, x: Tensor, nd: int, pads, relu: bool) -> Tensor:
+    """A quantized convolution on a plain float input, as Lucid writes it
+    (``lucid/nn/quantized/conv.py:168-184``): dequantize the weight, convolve in float32 with the
+    bias, optionally ReLU, fake-quantize the result to the layer's output grid - returned as a
+    tensor on that grid (its float view is the fake-quantized value).  ``pads`` = per spatial
+    axis ``(lo, hi)``; a padding mode other than zeros, or uneven amounts, pre-pad the input
+    (``lucid/nn/modules/conv.py:104-123``).  The float32 convolution sums in another order than
+    Lucid's GEMM, so codes can differ by one step where a value sits on a rounding tie."""
+    from ...quantization._functional import dequantize
+    from .. import functional as F
+    from .modules import Quantize
+
+    name = type(mod).__name__
+    w = mod.__dict__.get("_w_float")
+    if w is None:
+        w = dequantize(mod.weight_int8, mod.weight_scale, mod.weight_zero_point, ch_axis=0)
+        mod.__dict__["_w_float"] = w
+    mode = {"zeros": 0, "reflect": 1, "replicate": 2, "circular": 3}[mod.padding_mode]
+    sym = all(lo == hi for lo, hi in pads)
+    conv_pad = tuple(lo for lo, _ in pads)
+    if any(lo or hi for lo, hi in pads) and (mode != 0 or not sym):
+        if nd == 3 and (pads[0][0] or pads[0][1]):
+            raise NotImplementedError(f"{name}: a float input with padding_mode={mod.padding_mode!r} or uneven "
+                                      "padding along the depth axis; quantize the input first (QuantStub)")
+        lead = x.shape[:-2] if nd >= 2 else x.shape[:-1]
+        H = x.shape[-2] if nd >= 2 else 1
+        W = x.shape[-1]
+        (pt, pb) = pads[-2] if nd >= 2 else (0, 0)
+        (pl, pr) = pads[-1]
+        padded = Tensor.empty((*lead, *( [H + pt + pb] if nd >= 2 else []), W + pl + pr), T.float32, "hip")
+        _C.call("lq_pad_planes_f32", x.data_ptr, padded.data_ptr, int(np.prod(lead, dtype=np.int64)), H, W, pt, pb,
+                pl, pr, mode, None)
+        x, conv_pad = padded, (0,) * nd
+    if nd == 1:
+        y = F.conv1d_f32(x, w, mod.bias, mod.stride[-1], conv_pad[0], mod.dilation[-1], mod.groups)
+    elif nd == 2:
+        y = F.conv2d_f32(x, w, mod.bias, mod.stride, conv_pad, mod.dilation, mod.groups)
+    else:
+        y = F.conv3d_f32(x, w, mod.bias, mod.stride, conv_pad, mod.dilation, mod.groups)
+    if relu:
+        _C.call("lq_relu_f32", y.data_ptr, y.data_ptr, y.numel, None)
+    q = mod.__dict__.get("_out_quantize")
+    if q is None:
+        q = Quantize(mod.scale, mod.zero_point, mod.out_qdtype)
+        mod.__dict__["_out_quantize"] = q
+    return q(y)
+
+
 def input_grid(x: Tensor, what: str) -> Grid:
     if not isinstance(x, Tensor) or x.device != "hip":
         raise _C.DeviceMismatch(f"{what}: input must be a tensor on the 'hip' device")

@@ -22,7 +22,7 @@ from ... import _tensor as T
 from ..._tensor import Grid, Tensor
 from ...quantization._qscheme import QDtype, quint8
 from ..module import Module
-from ._utils import (activation_qparams, host_scalar, input_grid, plain_volume_grid, quantize_weight,
+from ._utils import (activation_qparams, float_input_conv, host_scalar, input_grid, is_plain_float, plain_volume_grid, quantize_weight,
                      forget_weight_zero_points, storage_offset, weight_zero_points)
 
 
@@ -75,6 +75,10 @@ class Conv2d(Module):
             self._zp_host = None
         if name == "weight_zero_point":
             forget_weight_zero_points(self)
+        if name in ("weight_int8", "weight_scale", "weight_zero_point"):
+            self.__dict__.pop("_w_float", None)      # the float-input form's dequantized weight
+        if name in ("scale", "zero_point"):
+            self.__dict__.pop("_out_quantize", None)
 
     def _resolve_pad(self, x: Tensor) -> tuple[int, int, int, int]:
         """(h_lo, h_hi, w_lo, w_hi), as ``conv.py:119-141``."""
@@ -102,6 +106,12 @@ class Conv2d(Module):
         into this layer's epilogue: the result is on the functional's grid, bit for bit what
         the two separate modules give, and the layer's own output is never stored."""
         name = type(self).__name__
+        if is_plain_float(x) and join is None:
+            # no grid on the input: Lucid's float formulation (conv.py:168-184)
+            if x.ndim != 4 or x.shape[1] != self.in_channels:
+                raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, H, W), got {x.shape}")
+            p = self._resolve_pad(x)
+            return float_input_conv(self, x, 2, ((p[0], p[1]), (p[2], p[3])), self._fused_relu)
         g = input_grid(x, name)
         if x.ndim != 4 or x.shape[1] != self.in_channels:
             raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, H, W), got {x.shape}")
@@ -201,6 +211,11 @@ class Conv1d(Conv2d):
 
     def forward(self, x: Tensor) -> Tensor:
         name = type(self).__name__
+        if is_plain_float(x):
+            if x.ndim != 3 or x.shape[1] != self.in_channels:
+                raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, L), got {x.shape}")
+            p = self._resolve_pad(x.reshape(x.shape[0], x.shape[1], 1, x.shape[2]))
+            return float_input_conv(self, x, 1, ((p[2], p[3]),), self._fused_relu)
         g = input_grid(x, name)
         if x.ndim != 3 or x.shape[1] != self.in_channels:
             raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, L), got {x.shape}")
@@ -337,6 +352,10 @@ class Conv3d(Conv2d):
 
     def forward(self, x: Tensor) -> Tensor:
         name = type(self).__name__
+        if is_plain_float(x):
+            if x.ndim != 5 or x.shape[1] != self.in_channels:
+                raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, D, H, W), got {x.shape}")
+            return float_input_conv(self, x, 3, self._resolve_pad3(x.shape[2:]), self._fused_relu)
         g = input_grid(x, name)
         if x.ndim != 5 or x.shape[1] != self.in_channels:
             raise _C.ShapeMismatch(f"{name}: expected (B, {self.in_channels}, D, H, W), got {x.shape}")

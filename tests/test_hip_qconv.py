@@ -439,3 +439,115 @@ def test_halo_kernel_refuses_what_it_is_not_built_for():
     x32, w32 = hip(codes(rng, (1, 8, 8, 32))), hip(codes(rng, (64, 3, 3, 32)))
     with pytest.raises(NotImplementedError, match="64 == 0"):
         _ops.qconv2d_i8(x32, w32, a_zp=0, pad=(1, 1, 1, 1), out_mode=_ops.OUT_ACC_I32, path=IMPLICIT, tile_config=15)
+
+
+def _loaded(conv, wq, ws, bias, S, Z):
+    state = {"weight_int8": wq, "weight_scale": ws, "weight_zero_point": np.zeros(len(ws), np.float32), "bias": bias,
+             "scale": np.float32(S), "zero_point": np.float32(Z)}
+    conv.load_state_dict({k: L.tensor(v, device="hip") for k, v in state.items()})
+    return conv
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("geom", [dict(k=3, stride=1, padding=1, dilation=1, groups=1),
+                                  dict(k=3, stride=2, padding=1, dilation=1, groups=2),
+                                  dict(k=(1, 3), stride=1, padding=(0, 2), dilation=(1, 2), groups=1),
+                                  dict(k=3, stride=2, padding="same", dilation=1, groups=1),
+                                  dict(k=5, stride=1, padding="valid", dilation=1, groups=1)])
+def test_float_input_form_of_quantized_conv2d(geom, relu):
+    """nnq.Conv2d / ConvReLU2d on a plain float tensor take Lucid's float formulation
+    (lucid/nn/quantized/conv.py:168-184): dequantized weight -> float32 convolution -> bias ->
+    [ReLU] -> fake_quantize.  Against the oracle's pass-for-pass restatement: the float32 sums run
+    in another order, so the tolerance is the reference's own (one quantization step where a value
+    sits on a rounding tie, equal elsewhere)."""
+    import lucid_amd.nn.quantized.intrinsic as nniq
+    import lucid_amd.nn.quantized as nnq
+
+    rng = np.random.default_rng(11)
+    B, Cin, Cout, H, W = 2, 8, 12, 11, 13
+    k = geom["k"] if isinstance(geom["k"], tuple) else (geom["k"], geom["k"])
+    x = rng.standard_normal((B, Cin, H, W)).astype(np.float32)
+    wq = codes(rng, (Cout, Cin // geom["groups"], *k), -127, 127)
+    ws = rng.uniform(0.002, 0.01, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    S, Z = 0.04, 128.0
+    cls = nniq.ConvReLU2d if relu else nnq.Conv2d
+    conv = _loaded(cls(Cin, Cout, k, stride=geom["stride"], padding=geom["padding"], dilation=geom["dilation"],
+                       groups=geom["groups"]), wq, ws, bias, S, Z)
+    y = conv(hip(x))
+    assert y._grid is not None and y.shape[:2] == (B, Cout)
+    got = y.numpy()
+    pad = geom["padding"]
+    xin = x
+    if pad == "same":   # uneven amounts: the odd unit on the high side (lucid/nn/modules/conv.py:44-55)
+        st = geom["stride"]
+        amounts = []
+        for n, kk in ((H, k[0]), (W, k[1])):
+            out = (n + st - 1) // st
+            tot = max(0, (out - 1) * st + kk - n)
+            amounts.append((tot // 2, tot - tot // 2))
+        xin = np.pad(x, ((0, 0), (0, 0), amounts[0], amounts[1]))
+        pad = (0, 0)
+    elif pad == "valid":
+        pad = (0, 0)
+    elif isinstance(pad, int):
+        pad = (pad, pad)
+    dil = geom["dilation"] if isinstance(geom["dilation"], tuple) else (geom["dilation"],) * 2
+    exp = O.conv2d_faithful(xin, wq, ws, np.zeros(Cout, np.float32), bias=bias, stride=(geom["stride"],) * 2, pad=pad,
+                            dilation=dil, groups=geom["groups"], relu=relu, fq=(S, Z, 0, 255))
+    assert got.shape == exp.shape
+    diff = np.abs(got - exp)
+    assert diff.max() <= S * 1.0001
+    assert np.mean(diff > 0) < 0.01
+
+
+@pytest.mark.parametrize("padding_mode", ["reflect", "replicate", "circular"])
+def test_float_input_form_with_a_padding_mode(padding_mode):
+    """The float-input form pre-pads the float image as the float layer does; checked against the
+    same layer fed the pre-padded image with padding 0."""
+    import lucid_amd.nn.quantized as nnq
+
+    rng = np.random.default_rng(12)
+    B, Cin, Cout, H, W = 2, 4, 6, 9, 10
+    x = rng.standard_normal((B, Cin, H, W)).astype(np.float32)
+    wq = codes(rng, (Cout, Cin, 3, 3), -127, 127)
+    ws = rng.uniform(0.002, 0.01, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    conv = _loaded(nnq.Conv2d(Cin, Cout, 3, padding=(1, 2)), wq, ws, bias, 0.05, 100.0)
+    conv.padding_mode = padding_mode
+    got = conv(hip(x)).numpy()
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (2, 2)), mode={"reflect": "reflect", "replicate": "edge", "circular": "wrap"}[padding_mode])
+    plain = _loaded(nnq.Conv2d(Cin, Cout, 3, padding=0), wq, ws, bias, 0.05, 100.0)
+    want = plain(hip(xp)).numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_float_input_form_of_quantized_conv1d_and_conv3d():
+    """Conv1d / Conv3d on plain floats: within one output step of the same layer fed the input
+    quantized on a fine grid (the int8 route), which the oracle pins bit for bit elsewhere."""
+    import lucid_amd.nn.quantized as nnq
+
+    rng = np.random.default_rng(13)
+    S = 0.05
+    # 1-d
+    B, Cin, Cout, Ln = 2, 16, 8, 33
+    x = (rng.integers(-100, 100, (B, Cin, Ln)) * 0.01).astype(np.float32)     # exactly on a 0.01 grid
+    wq = codes(rng, (Cout, Cin, 3), -127, 127)
+    ws = rng.uniform(0.002, 0.01, Cout).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    c1 = _loaded(nnq.Conv1d(Cin, Cout, 3, stride=2, padding=1), wq, ws, bias, S, 128.0)
+    got = c1(hip(x)).numpy()
+    xq = nnq.Quantize(L.tensor(np.float32(0.01), device="hip"), L.tensor(np.float32(128.0), device="hip"))(hip(x))
+    want = c1(xq).numpy()
+    assert got.shape == want.shape == (B, Cout, 17)
+    assert np.abs(got - want).max() <= S * 1.0001 and np.mean(got != want) < 0.02
+    # 3-d
+    B, Cin, Cout, D, H, W = 1, 16, 8, 5, 6, 7
+    x = (rng.integers(-100, 100, (B, Cin, D, H, W)) * 0.01).astype(np.float32)
+    wq = codes(rng, (Cout, Cin, 3, 3, 3), -127, 127)
+    c3 = _loaded(nnq.Conv3d(Cin, Cout, 3, padding=1), wq, ws, bias, S, 128.0)
+    got = c3(hip(x)).numpy()
+    want = c3(xq.__class__.on_grid(x.shape, nnq.Quantize(L.tensor(np.float32(0.01), device="hip"),
+                                                         L.tensor(np.float32(128.0), device="hip"))(hip(x))._grid)).numpy()
+    assert got.shape == want.shape == (B, Cout, D, H, W)
+    assert np.abs(got - want).max() <= S * 1.0001 and np.mean(got != want) < 0.02
