@@ -614,8 +614,9 @@ typedef struct {
     long ldo;              /* output row stride in elements; 0 means N       */
     int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
     int tile_config;       /* tuning: low byte 0 = choose, 1..12 = a tile shape of the
-                              four-wavefront kernel, 13 / 14 = 256x352 / 256x256 tiles of
-                              the eight-wavefront kernel (plain GEMM, K % 64 == 0),
+                              four-wavefront kernel, 13 / 14 / 16 = 256x352 / 256x256 /
+                              256x192 tiles of the eight-wavefront kernel (plain GEMM,
+                              K % 64 == 0),
                               15 (convolutions only) = one block per box of 256 output
                               positions x 64 channels with the box's input halo held in
                               LDS (stride 1, Cin/groups % 64 == 0, no join);

@@ -87,10 +87,12 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
     case 12: return launch_tile_c12(g, conv, groups, schedule, st);
     case 13:
     case 14:
-        // the eight-wavefront ping-pong kernel: plain GEMMs, one block per tile
+    case 16:
+        // the eight-wavefront ping-pong kernel (256 x 352 / 256 x 256 / 256 x 192 tiles): plain GEMMs,
+        // one block per tile
         LQ_REQUIRE(!conv && groups == 1, LQ_ERR_VALUE, "tile_config %d is for plain GEMMs", cfg);
         LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
-        return launch_pp_shape(g, cfg - 13, st);
+        return launch_pp_shape(g, cfg == 16 ? 2 : cfg - 13, st);
     case 15:
         // stride-1 convolution with the input halo held in LDS, one block per box of outputs
         LQ_REQUIRE(conv, LQ_ERR_VALUE, "tile_config 15 is for convolutions");
@@ -122,7 +124,10 @@ int heuristic_tile_shape(const GemmArgs& g, int conv, int groups) {
         const long t352 = tm * ((g.N + 351) / 352), t256 = tm * ((g.N + 255) / 256);
         // at least half a round of tiles, or the four-wavefront shapes below cover the chip better
         if (t256 >= 128) {
-            const long c352 = ((t352 + 255) / 256) * 352, c256 = ((t256 + 255) / 256) * 256;
+            const long t192 = tm * ((g.N + 191) / 192);
+            const long c352 = ((t352 + 255) / 256) * 352, c256 = ((t256 + 255) / 256) * 256,
+                       c192 = ((t192 + 255) / 256) * 192;
+            if (c192 < c256 && c192 < c352) return 16;
             return c352 < c256 ? 13 : 14;
         }
     }
@@ -207,7 +212,7 @@ int tune_import_text(const char* text, int* accepted) {
         }
         if (got != kTuneKeyInts + 1) return fail(LQ_ERR_VALUE, "tune_import: malformed line '%s'", line.c_str());
         const int shape = v[kTuneKeyInts] & 0xff;
-        if (shape < 1 || shape > 15) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
+        if (shape < 1 || shape > 16) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
         TuneKey key;
         std::memcpy(&key, v, sizeof(key));
         std::lock_guard<std::mutex> lock(g_tune_mu);
@@ -282,7 +287,7 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
     if (!autotune_enabled() || capturing != hipStreamCaptureStatusNone || ops < 5e8 || in_place) return LQ_OK;
 
     // candidates are whole tile_config values (shape | schedule << 8)
-    int cands[20], n = 0;
+    int cands[24], n = 0;
     if (conv == 2) {
         // the shapes the volumetric gather is built for
         if (g.N <= 64) cands[n++] = 6;
@@ -298,7 +303,7 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
         if (g.N > 128 && g.M > 128) cands[n++] = 1, cands[n++] = 11;
         if (g.N > 128 && !conv) cands[n++] = 12;
         // large plain GEMMs: the ping-pong kernel's 256 x 352 and 256 x 256 tiles
-        if (pp_applies(g, conv, groups)) cands[n++] = 13, cands[n++] = 14;
+        if (pp_applies(g, conv, groups)) cands[n++] = 13, cands[n++] = 14, cands[n++] = 16;
         // a long K over few tiles (late convolution stages): split K between the idle CUs
         const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
         if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);

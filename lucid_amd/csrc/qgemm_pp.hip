@@ -4,9 +4,14 @@
 namespace lq {
 
 // which: 0 = 256 x 352 tiles (N = 11008 is 32 of them wide less a sliver: with M = 2048 exactly
-// one tile per CU), 1 = 256 x 256 tiles
+// one tile per CU), 1 = 256 x 256 tiles, 2 = 256 x 192 tiles (N = 768 as four columns of tiles:
+// 200 tiles for 12 608 rows where 256-wide ones give 150 for the 256 CUs)
 int launch_pp_shape(const GemmArgs& g, int which, hipStream_t st) {
-    return which == 0 ? launch_pp<PPCfg352>(g, st) : launch_pp<PPCfg256>(g, st);
+    switch (which) {
+    case 0: return launch_pp<PPCfg352>(g, st);
+    case 1: return launch_pp<PPCfg256>(g, st);
+    default: return launch_pp<PPCfg192>(g, st);
+    }
 }
 
 }  // namespace lq

@@ -572,6 +572,7 @@ int launch_pp(const GemmArgs& g, hipStream_t st) {
 
 using PPCfg352 = PPCfg<256, 352, 4, 2, 4>;
 using PPCfg256 = PPCfg<256, 256, 4, 2, 4>;
+using PPCfg192 = PPCfg<256, 192, 4, 2, 4>;
 
 }  // namespace
 }  // namespace lq
