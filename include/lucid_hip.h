@@ -616,7 +616,9 @@ typedef struct {
     int tile_config;       /* tuning: low byte 0 = choose, 1..12 = a tile shape of the
                               four-wavefront kernel, 13 / 14 / 16 = 256x352 / 256x256 /
                               256x192 tiles of the eight-wavefront kernel (plain GEMM,
-                              K % 64 == 0),
+                              K % 64 == 0), 17 = 256x352 tiles with one wavefront per SIMD
+                              (plain GEMM, K % 128 == 0, K >= 256, float16 output or raw
+                              accumulators; never chosen automatically),
                               15 (convolutions only) = one block per box of 256 output
                               positions x 64 channels with the box's input halo held in
                               LDS (stride 1, Cin/groups % 64 == 0, no join);

@@ -65,6 +65,7 @@ int launch_tile_c10(const GemmArgs&, int, int, int, hipStream_t);
 int launch_tile_c11(const GemmArgs&, int, int, int, hipStream_t);
 int launch_tile_c12(const GemmArgs&, int, int, int, hipStream_t);
 int launch_pp_shape(const GemmArgs&, int, hipStream_t);
+int launch_bw_shape(const GemmArgs&, int, hipStream_t);
 bool conv_halo_applies(const GemmArgs&, int conv);
 int launch_conv_halo(const GemmArgs&, int conv, int groups, hipStream_t);
 }  // namespace lq
@@ -93,6 +94,11 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
         LQ_REQUIRE(!conv && groups == 1, LQ_ERR_VALUE, "tile_config %d is for plain GEMMs", cfg);
         LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
         return launch_pp_shape(g, cfg == 16 ? 2 : cfg - 13, st);
+    case 17:
+        // one wavefront per SIMD, 256 x 352 tiles (plain GEMMs, K % 128 == 0)
+        LQ_REQUIRE(!conv && groups == 1, LQ_ERR_VALUE, "tile_config %d is for plain GEMMs", cfg);
+        LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
+        return launch_bw_shape(g, 0, st);
     case 15:
         // stride-1 convolution with the input halo held in LDS, one block per box of outputs
         LQ_REQUIRE(conv, LQ_ERR_VALUE, "tile_config 15 is for convolutions");
@@ -212,7 +218,7 @@ int tune_import_text(const char* text, int* accepted) {
         }
         if (got != kTuneKeyInts + 1) return fail(LQ_ERR_VALUE, "tune_import: malformed line '%s'", line.c_str());
         const int shape = v[kTuneKeyInts] & 0xff;
-        if (shape < 1 || shape > 16) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
+        if (shape < 1 || shape > 17) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
         TuneKey key;
         std::memcpy(&key, v, sizeof(key));
         std::lock_guard<std::mutex> lock(g_tune_mu);

@@ -181,36 +181,68 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
     typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
     typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
 
-    // ---- the plain float forms on an interior sub-tile (every row and column inside the
-    // matrix, aligned, no residual, no ReLU, no zero-point correction): the same float steps -
-    // convert, as * ws, multiply, add the bias - and nothing else: row pointers are formed
-    // once and every store takes a constant offset from one of them.
+    // ---- the plain float forms (aligned output, no residual, no ReLU, no zero-point correction)
+    // when the matrix ends on a 16 x 16 tile boundary inside this sub-tile or beyond it: the same
+    // float steps - convert, as * ws, multiply, add the bias - and nothing else.  Row pointers are
+    // formed once and every store takes a constant offset from one of them; row blocks and column
+    // tiles past the end of the matrix are skipped whole (the last tile column of N = 11008 holds
+    // 96 real columns: without this its blocks, taking the element-wise route, finish many
+    // microseconds after everybody else).
     if constexpr (MODE == OUT_F16 || MODE == OUT_F32) {
         const int zp = g.a_zp_dev ? int(g.a_zp_dev[0]) + g.a_zp : g.a_zp;
-        const bool lean = wide && rows_in && g.residual == nullptr && !g.relu && (g.wsum == nullptr || zp == 0);
+        const int ncols = g.N - wn0, nrows = g.M - wm0;
+        const bool lean = g.ldo % 8 == 0 && reinterpret_cast<uintptr_t>(g.out) % 16 == 0 && g.residual == nullptr &&
+                          !g.relu && (g.wsum == nullptr || zp == 0) && (ncols >= TN * 16 || ncols % 16 == 0) &&
+                          (nrows >= TM * 16 || nrows % 16 == 0);
         if (lean) {
+            const int vt = ncols >= TN * 16 ? TN : ncols / 16;  // column tiles and row blocks inside the matrix
+            const int vr = nrows >= TM * 16 ? TM : nrows / 16;
             char* rows[TM];  // the lane's position in a pair's run, row block by row block
             rows[0] = static_cast<char*>(g.out) +
                       (size_t(wm0 + (lane & 15)) * size_t(g.ldo) + size_t(pair0 + swapped_col)) * esize;
             const size_t row_step = size_t(16) * size_t(g.ldo) * esize;
 #pragma unroll
             for (int i = 1; i < TM; ++i) rows[i] = rows[i - 1] + row_step;
-            // from there to the lane's own four columns of the lone tile
-            const ptrdiff_t lone_delta = ptrdiff_t(16 * last_tile + lane_col - 16 * rot - swapped_col) * esize;
             auto value4 = [&](const pp_v4i& a, const float4& ws, const float4& b, float as, uint4& v) {
                 v.x = __float_as_uint(float(a[0]) * (as * ws.x) + b.x);
                 v.y = __float_as_uint(float(a[1]) * (as * ws.y) + b.y);
                 v.z = __float_as_uint(float(a[2]) * (as * ws.z) + b.z);
                 v.w = __float_as_uint(float(a[3]) * (as * ws.w) + b.w);
             };
+            // accumulator column j, which is column tile t, from the lane's own layout (four columns)
+            auto single = [&](auto j_tag, int t) {
+                constexpr int j = decltype(j_tag)::value;
+                const int cl = wn0 - n0 + 16 * t + lane_col;
+                const float4 ws = *reinterpret_cast<const float4*>(s_ws + cl), b = *reinterpret_cast<const float4*>(s_bias + cl);
+                const ptrdiff_t delta = ptrdiff_t(16 * t + lane_col - 16 * rot - swapped_col) * esize;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    if (i >= vr) break;
+                    uint4 v;
+                    value4(acc[i][j], ws, b, as_row[i], v);
+                    uint32_t p[kDw];
+                    pp_pack<MODE>(v, cpk, p);
+                    char* dst = rows[i] + delta;
+                    if constexpr (kDw == 2)
+                        *reinterpret_cast<v2u_t*>(dst) = v2u_t{p[0], p[1]};
+                    else
+                        *reinterpret_cast<v4u_t*>(dst) = v4u_t{p[0], p[1], p[2], p[3]};
+                }
+            };
             pp_static_for<kPairs>([&](auto x_tag) {
                 constexpr int j = 2 * decltype(x_tag)::value;
+                const int ta = j + rot;  // the pair's column tiles: ta, ta + 1
+                if (ta + 1 >= vt) {
+                    if (ta < vt) single(std::integral_constant<int, j>{}, ta);
+                    return;
+                }
                 const int cl = pair0 - n0 + 16 * j + lane_col;  // the lane's own columns of the pair's first tile
                 const float4 ws0 = *reinterpret_cast<const float4*>(s_ws + cl), b0 = *reinterpret_cast<const float4*>(s_bias + cl);
                 const float4 ws1 = *reinterpret_cast<const float4*>(s_ws + cl + 16),
                              b1 = *reinterpret_cast<const float4*>(s_bias + cl + 16);
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
+                    if (i >= vr) break;
                     uint4 v, w;
                     value4(acc[i][j], ws0, b0, as_row[i], v);
                     value4(acc[i][j + 1], ws1, b1, as_row[i], w);
@@ -232,20 +264,7 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
                 }
             });
             if constexpr (kLone) {
-                const int cl = wn0 - n0 + 16 * last_tile + lane_col;
-                const float4 ws = *reinterpret_cast<const float4*>(s_ws + cl), b = *reinterpret_cast<const float4*>(s_bias + cl);
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    uint4 v;
-                    value4(acc[i][TN - 1], ws, b, as_row[i], v);
-                    uint32_t p[kDw];
-                    pp_pack<MODE>(v, cpk, p);
-                    char* dst = rows[i] + lone_delta;
-                    if constexpr (kDw == 2)
-                        *reinterpret_cast<v2u_t*>(dst) = v2u_t{p[0], p[1]};
-                    else
-                        *reinterpret_cast<v4u_t*>(dst) = v4u_t{p[0], p[1], p[2], p[3]};
-                }
+                if (last_tile < vt) single(std::integral_constant<int, TN - 1>{}, last_tile);
             }
             return;
         }

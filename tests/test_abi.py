@@ -18,6 +18,19 @@ def test_library_exports_every_declared_symbol():
     assert set(declared) == set(_C._SIGNATURES), "binding table and header disagree"
 
 
+def test_inline_assembly_mfma_loop_is_clean():
+    """The one-wavefront-per-SIMD GEMM kernel issues its MFMAs from inline assembly, so the
+    compiler must not touch an accumulator inside the k loop (it would read a register an MFMA is
+    still writing).  `make check` compiles the kernel to ISA (cached after a build) and verifies
+    that the loop holds no register move or spill."""
+    import os
+    import subprocess
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "lucid_amd", "csrc")
+    r = subprocess.run(["make", "-C", csrc, "check"], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("clean") >= 2 and "NOT CLEAN" not in r.stdout
+
+
 def test_version_and_registry():
     assert _C.load().lq_version() == _C.ABI_VERSION == 3
     ops = dict((n, (v, d)) for n, v, d in _C.op_registry())

@@ -753,3 +753,59 @@ def test_first_calls_from_two_threads():
     """ % root)
     r = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=110)
     assert r.returncode == 0 and r.stdout.strip().endswith("OK"), r.stdout + r.stderr
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 352, 1024), (300, 260, 256), (513, 1000, 384), (2048, 704, 4096), (40, 1001, 512),
+                                   (2048, 11008, 256)])
+def test_one_wavefront_per_simd_kernel_exact(M, N, K):
+    """tile_config 17 (four wavefronts with the whole register file each, MFMAs from inline
+    assembly): accumulators and the float16 epilogue against the oracle on full, ragged and edge
+    shapes, and the shapes it is not built for are refused."""
+    rng = np.random.default_rng(17000 + M + N + K)
+    a, w = codes(rng, (M, K)), codes(rng, (N, K))
+    ad, wd = hip(a), hip(w)
+    acc = _ops.qlinear_i8(ad, wd, out_mode=_ops.OUT_ACC_I32, path=TILE, tile_config=17).numpy()
+    assert np.array_equal(acc, O.igemm(a, w))
+    a_scale = rng.uniform(0.005, 0.05, M).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.02).astype(np.float16)
+    got = _ops.qlinear_i8(ad, wd, a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias),
+                          out_mode=_ops.OUT_F16, path=TILE, tile_config=17).numpy()
+    exp = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, out_mode=O.OUT_F16)
+    assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+    # with a ReLU (the general epilogue) as well
+    got = _ops.qlinear_i8(ad, wd, a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias), relu=True,
+                          out_mode=_ops.OUT_F16, path=TILE, tile_config=17).numpy()
+    exp = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, relu=True, out_mode=O.OUT_F16)
+    assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+
+
+def test_one_wavefront_per_simd_kernel_refusals():
+    rng = np.random.default_rng(1)
+    a, w = hip(codes(rng, (256, 192))), hip(codes(rng, (256, 192)))
+    with pytest.raises(L.ShapeMismatch, match="multiple of 128"):
+        _ops.qlinear_i8(a, w, out_mode=_ops.OUT_ACC_I32, path=TILE, tile_config=17)
+    a, w = hip(codes(rng, (256, 256))), hip(codes(rng, (256, 256)))
+    one = hip(np.ones(256, np.float32))
+    with pytest.raises(NotImplementedError, match="output mode"):
+        _ops.qlinear_i8(a, w, a_scale=one, w_scale=one, out_mode=_ops.OUT_F32, path=TILE, tile_config=17)
+
+
+def test_matrix_edges_on_tile_boundaries_take_the_fast_epilogue_and_stay_exact():
+    """The float16 / float32 epilogue of the large-GEMM kernels skips whole 16 x 16 tiles past the
+    end of the matrix (N = 11008 ends 96 columns into its last 352-wide tile; M = 12608 ends 64
+    rows into its last 256-high one): results against the oracle where M and N end on, next to
+    and off a tile boundary."""
+    rng = np.random.default_rng(33)
+    K = 128
+    for M, N in ((256 + 64, 352 + 96), (256 + 64, 352 + 100), (256 + 70, 352 + 96), (512 + 16, 704 + 176 + 16), (272, 256 + 48)):
+        a, w = codes(rng, (M, K)), codes(rng, (N, K))
+        a_scale = rng.uniform(0.005, 0.05, M).astype(np.float32)
+        w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+        bias = (rng.standard_normal(N) * 0.02).astype(np.float32)
+        for cfg in (13, 14, 16):
+            for mode, omode, dt in ((_ops.OUT_F16, O.OUT_F16, np.uint16), (_ops.OUT_F32, O.OUT_F32, np.uint32)):
+                got = _ops.qlinear_i8(hip(a), hip(w), a_scale=hip(a_scale), w_scale=hip(w_scale), bias=hip(bias),
+                                      out_mode=mode, path=TILE, tile_config=cfg).numpy()
+                exp = O.qlinear(a, w, 0, a_scale, w_scale, bias=bias, out_mode=omode)
+                assert np.array_equal(got.view(dt), exp.view(dt)), (M, N, cfg, mode)
