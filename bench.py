@@ -98,6 +98,12 @@ def time_in_graph(L, _C, fn, steps, per_graph=20):
     graph and the graph is replayed `steps` times between one pair of events: the rate of
     short kernels without the interpreter's gap between launches."""
     fn()
+    if EAGER_ONLY:  # no graph launch under a tracer: the same calls, driven from Python
+        def many():
+            for _ in range(per_graph):
+                fn()
+        total, _ = time_launches(_C, many, steps, 2)
+        return total / (steps * per_graph)
     with L.graph.capture() as g:
         for _ in range(per_graph):
             fn()
@@ -233,13 +239,16 @@ def bench_linear_cold_weights(L, _C, _ops, t, M, K, N, steps):
     Returns the average microseconds per launch."""
     copies = int(320e6 // (N * K)) + 2
     ws = [t["wq"]] + [t["wq"].clone() for _ in range(copies - 1)]
-    with L.graph.capture() as g:
+
+    def cycle():
         for w in ws:
             _ops.qlinear_i8(t["xq"], w, a_scale=t["xs"], w_scale=t["ws"], bias=t["bias"],
                             out_mode=_ops.OUT_F16, out=t["out"])
+
+    g = _Replay(L, cycle)  # a graph replay, or the same launches from Python under --eager
     for _ in range(20):
-        g.replay()
-    total, _ = time_launches(_C, g.replay, steps, 3)
+        g.run()
+    total, _ = time_launches(_C, g.run, steps, 3)
     g.destroy()
     return total / (steps * copies) * 1e3
 
@@ -566,9 +575,9 @@ def bench_vit_b16(L, _C, steps, warmup):
 
 def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     """Dynamic-quantized MLP Linear(784,256)-ReLU-Linear(256,10), batch 64
-    (launch-latency bound: 0.43 MOP).  Eager = one Python-driven forward (3
-    launches: per layer one that takes the activation's min / max, qparams and codes and
-    multiplies, and the ReLU between); graph = the same forward replayed from a HIP graph."""
+    (launch-latency bound: 0.43 MOP).  Eager = one Python-driven forward (ONE launch: a single
+    block takes each layer's min / max, qparams and codes, multiplies, and applies the ReLU
+    between them); graph = the same forward replayed from a HIP graph."""
     import lucid_amd.nn as nn
 
     rng = np.random.default_rng(1)
@@ -589,7 +598,7 @@ def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     assert np.isfinite(y.numpy()).all()
     g.destroy()
     return {"eager_us_per_forward": round(eager_us, 1), "graph_us_per_forward": round(graph_us, 1),
-            "launches_per_forward": 3}
+            "launches_per_forward": 1}
 
 
 def bench_weight_only(L, _C, steps, warmup, K=4096, N=11008, gs=64):
@@ -618,13 +627,15 @@ def bench_weight_only(L, _C, steps, warmup, K=4096, N=11008, gs=64):
             # exceed the 256 MB last-level cache, so every byte comes from HBM (what a model's layers see)
             copies = int(320e6 // nbytes) + 2
             sets = [(packed, scales, biases)] + [(packed.clone(), scales.clone(), biases.clone()) for _ in range(copies - 1)]
-            with L.graph.capture() as g:
+            def cycle():
                 for (pk, sc, bi) in sets:
                     _C.call("lq_wq_matmul", x.data_ptr, pk.data_ptr, sc.data_ptr, bi.data_ptr, m, N, K, gs, bits,
                             res.data_ptr, None)
+
+            g = _Replay(L, cycle)
             for _ in range(5):
-                g.replay()
-            tot, _ = time_launches(_C, g.replay, max(10, steps // 2), 2)
+                g.run()
+            tot, _ = time_launches(_C, g.run, max(10, steps // 2), 2)
             g.destroy()
             cold_us = tot / (max(10, steps // 2) * copies) * 1e3
             del sets

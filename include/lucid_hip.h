@@ -421,6 +421,20 @@ int lq_dynamic_linear_small_f32(const float* x, int M, int K, const int8_t* w, i
                                 const int32_t* wsum, const float* bias, int relu, int symmetric, int qmin, int qmax,
                                 int is_signed, float eps, int code_offset, float* out, lq_stream stream);
 
+/* Two dynamic-quantized Linears in ONE launch of one block: y = L2(act1(L1(x))) with each layer as
+ * lq_dynamic_linear_small_f32 computes it (the hidden activation's min / max, qparams and codes
+ * included: one block owns the batch, so that reduction is block-wide) and relu1 / relu2 the
+ * optional ReLU behind each.  x [M, K1] float32, w1 [N1, K1], w2 [N2, N1] int8 codes with their
+ * per-row scales, code sums and float32 biases (or NULL); out [M, N2] float32.  M <= 64,
+ * K1 % 16 == 0 and <= 1024, N1 % 16 == 0 and <= 256, N2 <= 64; anything else
+ * LQ_ERR_NOT_IMPLEMENTED.  Same bits as the separate calls (Linear, ReLU, Linear of a
+ * quantize_dynamic'd MLP: lucid/nn/quantized/dynamic/linear.py:84-99).  No counterpart in Lucid. */
+int lq_dynamic_mlp2_small_f32(const float* x, int M, int K1, const int8_t* w1, int N1, const float* w1_scale,
+                              const int32_t* w1sum, const float* bias1, int relu1, const int8_t* w2, int N2,
+                              const float* w2_scale, const int32_t* w2sum, const float* bias2, int relu2, int symmetric,
+                              int qmin, int qmax, int is_signed, float eps, int code_offset, float* out,
+                              lq_stream stream);
+
 /* Dynamic per-row quantization in one pass: for every row of x [rows, cols],
  * min / max of the row (PerChannelMinMaxObserver with ch_axis = 0,
  * observer.py:634-653), its qparams (calculate_qparams, _qparams.py:198-215) and

@@ -114,6 +114,8 @@ _SIGNATURES = {
     "lq_quantize_tensor_dynamic_i8": [_vp, _sz, _i, _i, _i, _i, C.c_float, _i, _vp, _vp, _vp, _vp, _vp, _vp],
     "lq_quantize_rows_dynamic_i8": [_vp, _sz, _sz, _i, _i, _i, _i, C.c_float, _i, _vp, _vp, _vp, _vp, _vp, _vp],
     "lq_dynamic_linear_small_f32": [_vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _i, _vp, _vp],
+    "lq_dynamic_mlp2_small_f32": [_vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i,
+                                  C.c_float, _i, _vp, _vp],
     "lq_selftest_requant_route": [C.c_float, C.c_float, _i, _i, _i, C.c_ulonglong, C.c_ulonglong, _vp, _vp, _vp],
     "lq_probe_mfma_i8": [_vp, _vp, _sz, _i, _vp, C.POINTER(C.c_double), _vp],
     "lq_probe_mfma_i8_k64": [_vp, _vp, _sz, _i, _vp, C.POINTER(C.c_double), _vp],

@@ -859,6 +859,170 @@ __global__ __launch_bounds__(1024) void dynamic_linear_small_kernel(
     }
 }
 
+// Two dynamic-quantized Linears with an optional ReLU after each, on a small activation, in ONE
+// launch of ONE block (the MLP Linear(784,256) -> ReLU -> Linear(256,10) at batch 64 is 0.43 MOP:
+// three launches cost three round trips).  The block does, in order, exactly what the separate
+// operators do - the tensor's min / max, calculate_qparams, the activation codes, the integer
+// GEMM, float(acc - zp * wsum[n]) * (s * w_scale[n]) + bias[n], ReLU - for the first layer, keeps
+// its float32 output in LDS, and repeats the sequence on it for the second: the hidden
+// activation's min / max is a block-wide reduction because one block owns the whole batch.  Same
+// bits as two lq_dynamic_linear_small_f32 calls (the ReLU in between folded into the first).
+// LDS: codes of x [64][K1] | hidden float32 [64][N1] | hidden codes [64][N1].
+__global__ __launch_bounds__(1024) void dynamic_mlp2_small_kernel(
+    const float* __restrict__ x, int M, int K1, const int8_t* __restrict__ w1, int N1, const float* __restrict__ ws1,
+    const int32_t* __restrict__ wsum1, const float* __restrict__ b1, int relu1, const int8_t* __restrict__ w2, int N2,
+    const float* __restrict__ ws2, const int32_t* __restrict__ wsum2, const float* __restrict__ b2, int relu2,
+    int symmetric, int qmin, int qmax, int is_signed, float eps, float half_range, int off, float* __restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) int8_t ml_smem[];
+    __shared__ float s_sz[4];
+    typedef int ml_v4i __attribute__((ext_vector_type(4)));
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ln = lane & 15, lg = lane >> 4;
+    int8_t* const codes1 = ml_smem;                                             // [64][K1]
+    float* const hid = reinterpret_cast<float*>(ml_smem + size_t(64) * K1);      // [64][N1]
+    int8_t* const codes2 = ml_smem + size_t(64) * K1 + size_t(64) * N1 * 4;      // [64][N1]
+    constexpr int kKeep = 16;
+    const float qnan = __builtin_nanf("");
+
+    // ---- layer 1: range, qparams and codes of x (all rows; rows past M are zero codes)
+    const int quads = (M * K1) >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    MinMax m{__builtin_inff(), -__builtin_inff(), 0};
+    float4 v[kKeep];
+#pragma unroll
+    for (int u = 0; u < kKeep; ++u) {
+        const int i = u * 1024 + tid;
+        if (i < quads) v[u] = x4[i];
+    }
+    for (int i = quads + tid; i < 16 * K1; i += 1024) reinterpret_cast<unsigned*>(codes1)[i] = 0u;
+    for (int i = ((M * N1) >> 2) + tid; i < 16 * N1; i += 1024) reinterpret_cast<unsigned*>(codes2)[i] = 0u;
+#pragma unroll
+    for (int u = 0; u < kKeep; ++u)
+        if (u * 1024 + tid < quads) mm_update(m, v[u].x), mm_update(m, v[u].y), mm_update(m, v[u].z), mm_update(m, v[u].w);
+    m = mm_block_reduce(m);
+    if (tid == 0) {
+        float s, z;
+        qparams_of(m.nan ? qnan : m.lo, m.nan ? qnan : m.hi, symmetric, qmin, qmax, is_signed, eps, half_range, &s, &z);
+        s_sz[0] = s, s_sz[1] = z;
+    }
+    __syncthreads();
+    {
+        const float s = s_sz[0], z = s_sz[1], r = 1.0f / s;
+        const QuantizeOp<int8_t> op{x4, reinterpret_cast<Code8x4*>(codes1), float(double(qmin)), float(double(qmax)), off};
+#pragma unroll
+        for (int u = 0; u < kKeep; ++u) {
+            const int i = u * 1024 + tid;
+            if (i < quads) op.q[i] = op.pack(v[u], s, z, r);
+        }
+    }
+    __syncthreads();
+
+    // ---- layer 1: GEMM.  A wavefront owns 16 output columns (a weight fragment is loaded once per
+    // k step and multiplied with the four row blocks of the batch) and applies the epilogue itself.
+    MinMax hm{__builtin_inff(), -__builtin_inff(), 0};
+    {
+        const float s = s_sz[0], z = s_sz[1];
+        const int zp = int(z) + off;
+        const int ksteps = (K1 + 63) >> 6;
+        for (int cb = wave; cb * 16 < N1; cb += 16) {
+            const int n = cb * 16 + ln;
+            const int nc = n < N1 ? n : N1 - 1;
+            const int8_t* wrow = w1 + size_t(nc) * size_t(K1);
+            const float c_ws = ws1 ? ws1[nc] : 1.0f;
+            const int c_wsum = wsum1 ? wsum1[nc] : 0;
+            const float c_bias = b1 ? b1[nc] : -0.0f;
+            ml_v4i acc[4];
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) acc[rb] = ml_v4i{0, 0, 0, 0};
+            ml_v4i wf = lg * 16 < K1 ? *reinterpret_cast<const ml_v4i*>(wrow + lg * 16) : ml_v4i{0, 0, 0, 0};
+            for (int ks = 0; ks < ksteps; ++ks) {
+                const int k = ks * 64 + lg * 16, kn = k + 64;
+                const bool in_k = k < K1;  // K1 % 16 == 0: a 16-byte chunk is inside or outside as a whole
+                const ml_v4i wnext = (ks + 1 < ksteps && kn < K1) ? *reinterpret_cast<const ml_v4i*>(wrow + kn) : ml_v4i{0, 0, 0, 0};
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb) {
+                    const ml_v4i af = in_k ? *reinterpret_cast<const ml_v4i*>(codes1 + size_t(16 * rb + ln) * K1 + k)
+                                           : ml_v4i{0, 0, 0, 0};
+                    acc[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc[rb], 0, 0, 0);
+                }
+                wf = wnext;
+            }
+            // acc[rb][q]: activation row 16 rb + 4 (lane / 16) + q, weight row n
+            const int corr = (wsum1 != nullptr && zp != 0) ? zp * c_wsum : 0;
+            const float sc = s * c_ws;
+            const float floor = relu1 ? 0.0f : -__builtin_inff();
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int mm = 16 * rb + 4 * lg + q;
+                    if (mm < M && n < N1) {
+                        const float f = float(acc[rb][q] - corr);
+                        float y = f * sc;
+                        y = y + c_bias;
+                        y = (y < floor) ? floor : y;
+                        hid[mm * N1 + n] = y;
+                        mm_update(hm, y);
+                    }
+                }
+        }
+    }
+    // ---- layer 2: range, qparams and codes of the hidden activation
+    hm = mm_block_reduce(hm);  // (its barrier also publishes hid)
+    if (tid == 0) {
+        float s, z;
+        qparams_of(hm.nan ? qnan : hm.lo, hm.nan ? qnan : hm.hi, symmetric, qmin, qmax, is_signed, eps, half_range, &s, &z);
+        s_sz[2] = s, s_sz[3] = z;
+    }
+    __syncthreads();
+    const float s2 = s_sz[2], z2 = s_sz[3];
+    {
+        const float r2 = 1.0f / s2;
+        const float4* h4 = reinterpret_cast<const float4*>(hid);
+        const QuantizeOp<int8_t> op{h4, reinterpret_cast<Code8x4*>(codes2), float(double(qmin)), float(double(qmax)), off};
+        const int quads2 = (M * N1) >> 2;
+        for (int i = tid; i < quads2; i += 1024) op.q[i] = op.pack(h4[i], s2, z2, r2);
+    }
+    __syncthreads();
+    // ---- layer 2: GEMM, one wavefront per 16 x 16 output tile
+    {
+        const int rb = wave & 3, cb = wave >> 2;
+        if (cb * 16 < N2 && rb * 16 < M) {
+            const int zp = int(z2) + off;
+            const int n = cb * 16 + ln;
+            const int nc = n < N2 ? n : N2 - 1;
+            const int8_t* wrow = w2 + size_t(nc) * size_t(N1);
+            const float c_ws = ws2 ? ws2[nc] : 1.0f;
+            const int c_wsum = wsum2 ? wsum2[nc] : 0;
+            const float c_bias = b2 ? b2[nc] : -0.0f;
+            ml_v4i acc = ml_v4i{0, 0, 0, 0};
+            const int ksteps = (N1 + 63) >> 6;
+            for (int ks = 0; ks < ksteps; ++ks) {
+                const int k = ks * 64 + lg * 16;
+                const bool in_k = k < N1;
+                const ml_v4i wf = in_k ? *reinterpret_cast<const ml_v4i*>(wrow + k) : ml_v4i{0, 0, 0, 0};
+                const ml_v4i af = in_k ? *reinterpret_cast<const ml_v4i*>(codes2 + size_t(16 * rb + ln) * N1 + k)
+                                       : ml_v4i{0, 0, 0, 0};
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc, 0, 0, 0);
+            }
+            const int corr = (wsum2 != nullptr && zp != 0) ? zp * c_wsum : 0;
+            const float sc = s2 * c_ws;
+            const float floor = relu2 ? 0.0f : -__builtin_inff();
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int mm = 16 * rb + 4 * lg + q;
+                if (mm < M && n < N2) {
+                    const float f = float(acc[q] - corr);
+                    float y = f * sc;
+                    y = y + c_bias;
+                    y = (y < floor) ? floor : y;
+                    out[size_t(mm) * N2 + n] = y;
+                }
+            }
+        }
+    }
+}
+
 }  // namespace
 
 namespace lq {
@@ -883,6 +1047,34 @@ int lq_quantize_tensor_dynamic_i8(const float* x, size_t n, int symmetric, int q
     hipLaunchKernelGGL(quantize_tensor_dynamic_kernel, dim3(1), dim3(1024), 0, as_stream(stream), x, n, symmetric,
                        qmin, qmax, is_signed, eps, half_range, code_offset, scale, zp, mn_out, mx_out, q);
     LQ_CHECK_LAUNCH("quantize_tensor_dynamic");
+    return LQ_OK;
+}
+
+int lq_dynamic_mlp2_small_f32(const float* x, int M, int K1, const int8_t* w1, int N1, const float* w1_scale,
+                              const int32_t* w1sum, const float* bias1, int relu1, const int8_t* w2, int N2,
+                              const float* w2_scale, const int32_t* w2sum, const float* bias2, int relu2, int symmetric,
+                              int qmin, int qmax, int is_signed, float eps, int code_offset, float* out,
+                              lq_stream stream) {
+    if (M == 0 || N2 == 0) return LQ_OK;
+    LQ_REQUIRE(x && w1 && w2 && out, LQ_ERR_VALUE, "dynamic_mlp2_small: NULL pointer");
+    LQ_REQUIRE(qmax > qmin && qmin + code_offset >= -128 && qmax + code_offset <= 127, LQ_ERR_VALUE,
+               "dynamic_mlp2_small: grid [%d,%d] + offset %d does not fit int8", qmin, qmax, code_offset);
+    // one block holds x's codes (64 K1 bytes), the hidden activation (256 N1 bytes) and its codes (64 N1 bytes)
+    LQ_REQUIRE(M > 0 && M <= 64 && K1 >= 16 && K1 % 16 == 0 && K1 <= 1024 && long(M) * K1 <= 65536 && N1 >= 16 &&
+                   N1 % 16 == 0 && N1 <= 256 && N2 > 0 && N2 <= 64 && aligned16(x) && aligned16(w1) && aligned16(w2),
+               LQ_ERR_NOT_IMPLEMENTED,
+               "dynamic_mlp2_small: takes up to 64 rows, K1 %% 16 == 0 up to 1024, a hidden width that is a multiple of "
+               "16 up to 256 and up to 64 outputs (got M = %d, K1 = %d, N1 = %d, N2 = %d); use two "
+               "lq_dynamic_linear_small_f32 calls", M, K1, N1, N2);
+    const float half_range = float((double(qmax) - double(qmin)) / 2.0);
+    const size_t lds = size_t(64) * K1 + size_t(64) * N1 * 5;
+    static DeviceOnce attr_once;
+    if (int rc = allow_dynamic_lds(attr_once, reinterpret_cast<const void*>(dynamic_mlp2_small_kernel), 152 * 1024))
+        return rc;
+    hipLaunchKernelGGL(dynamic_mlp2_small_kernel, dim3(1), dim3(1024), lds, as_stream(stream), x, M, K1, w1, N1, w1_scale,
+                       w1sum, bias1, relu1, w2, N2, w2_scale, w2sum, bias2, relu2, symmetric, qmin, qmax, is_signed, eps,
+                       half_range, code_offset, out);
+    LQ_CHECK_LAUNCH("dynamic_mlp2_small");
     return LQ_OK;
 }
 

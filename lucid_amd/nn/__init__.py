@@ -26,6 +26,25 @@ class Identity(Module):
         return x
 
 
+def _fused_dynamic_pair(mods, i, x):
+    """``(result, next index)`` when the modules at ``i`` are Linear [, ReLU], Linear from
+    ``nn.quantized.dynamic`` on an activation small enough for the one-launch kernel, else ``None``
+    (no hooks on the modules: a hook has to see each module's own output)."""
+    from .quantized.dynamic import linear as _dyn
+
+    first = mods[i]
+    if type(first) is not _dyn.Linear or i + 1 >= len(mods):
+        return None
+    relu = type(mods[i + 1]) is ReLU
+    j = i + 2 if relu else i + 1
+    if j >= len(mods) or type(mods[j]) is not _dyn.Linear:
+        return None
+    if any(getattr(m, "_forward_hooks", None) or getattr(m, "_forward_pre_hooks", None) for m in mods[i:j + 1]):
+        return None
+    y = _dyn.fused_pair(first, relu, mods[j], x)
+    return None if y is None else (y, j + 1)
+
+
 class Sequential(Module):
     def __init__(self, *mods) -> None:
         super().__init__()
@@ -39,8 +58,16 @@ class Sequential(Module):
         return len(self._modules)
 
     def forward(self, x):
-        for m in self._modules.values():
-            x = m(x)
+        mods = list(self._modules.values())
+        i = 0
+        while i < len(mods):
+            # two small dynamic-quantized Linears in a row, with or without a ReLU between: one launch
+            skip = _fused_dynamic_pair(mods, i, x)
+            if skip is not None:
+                x, i = skip
+                continue
+            x = mods[i](x)
+            i += 1
         return x
 
 

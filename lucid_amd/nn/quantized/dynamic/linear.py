@@ -28,6 +28,39 @@ from .._utils import forget_weight_zero_points, storage_offset, weight_zero_poin
 SMALL_LINEAR_MAX_K = 6080
 
 
+def fused_pair(first, relu_between: bool, second, x):
+    """``second(relu(first(x)))`` (or without the ReLU) for two dynamic ``Linear`` layers on a small
+    activation as ONE launch (``lq_dynamic_mlp2_small_f32``: one block owns the batch, so the hidden
+    activation's min / max is a block-wide reduction), or ``None`` when the shapes or operands do
+    not qualify.  Same bits as calling the modules one after the other."""
+    if not (isinstance(first, Linear) and isinstance(second, Linear) and isinstance(x, Tensor)):
+        return None
+    if x.device != "hip" or x.dtype != T.float32 or x._grid is not None or x._range is not None:
+        return None
+    K1, N1, N2 = first.in_features, first.out_features, second.out_features
+    if x.ndim < 1 or x.shape[-1] != K1 or second.in_features != N1:
+        return None
+    M = x.numel // K1
+    if not (0 < M <= 64 and K1 % 16 == 0 and 16 <= K1 <= 1024 and M * K1 <= 65536 and N1 % 16 == 0
+            and 16 <= N1 <= 256 and 0 < N2 <= 64):
+        return None
+    if first.act_qdtype is not second.act_qdtype:
+        return None
+    for lin in (first, second):
+        if weight_zero_points(lin) is not None or (lin.bias is not None and lin.bias.dtype != T.float32):
+            return None
+        if lin._wsum is None:
+            lin._wsum = _ops.rowsum_i8(lin.weight_int8)
+    qd = first.act_qdtype
+    y = Tensor.empty((M, N2), T.float32, "hip")
+    _C.call("lq_dynamic_mlp2_small_f32", x.data_ptr, M, K1, first.weight_int8.data_ptr, N1, first.weight_scale.data_ptr,
+            first._wsum.data_ptr, None if first.bias is None else first.bias.data_ptr, int(relu_between),
+            second.weight_int8.data_ptr, N2, second.weight_scale.data_ptr, second._wsum.data_ptr,
+            None if second.bias is None else second.bias.data_ptr, 0, 0, qd.quant_min, qd.quant_max, int(qd.signed),
+            1e-8, storage_offset(qd), y.data_ptr, None)
+    return y.reshape(*x.shape[:-1], N2)
+
+
 class Linear(Module):
     def __init__(self, in_features: int, out_features: int, bias: bool = True) -> None:
         super().__init__()

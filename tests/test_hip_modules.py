@@ -528,3 +528,87 @@ def test_dynamic_linear_wide_layer_at_small_batch(M, K):
             _C.call("lq_dynamic_linear_small_f32", xd.data_ptr, M, K, lin.weight_int8.data_ptr, N,
                     lin.weight_scale.data_ptr, _ops.rowsum_i8(lin.weight_int8).data_ptr, None, 0, 0, 0, 255, 0, 1e-8,
                     -128, out.data_ptr, None)
+
+
+class _recorded_calls:
+    """The names of the compute entry points called through the binding while the block runs."""
+
+    def __enter__(self):
+        from lucid_amd import _C
+        self._C, self._orig, self.names = _C, _C.call, []
+
+        def call(name, *args):
+            if name not in ("lq_alloc", "lq_free", "lq_sync", "lq_d2h", "lq_h2d", "lq_rowsum_i8"):  # one-off weight prep
+                self.names.append(name)
+            return self._orig(name, *args)
+
+        _C.call = call
+        return self.names
+
+    def __exit__(self, *exc):
+        self._C.call = self._orig
+        return False
+
+
+@pytest.mark.parametrize("M,K1,N1,N2", [(64, 784, 256, 10), (5, 64, 16, 1), (33, 1024, 240, 64), (17, 48, 32, 10)])
+@pytest.mark.parametrize("relu", [True, False])
+@pytest.mark.parametrize("kind", ["normal", "constant", "nan"])
+def test_two_dynamic_linears_in_one_launch(M, K1, N1, N2, relu, kind):
+    """A Sequential of nnqd.Linear [, ReLU], nnqd.Linear on a small batch runs as ONE launch
+    (lq_dynamic_mlp2_small_f32: the hidden activation's min / max is a reduction inside the one
+    block that owns the batch): bit for bit what the modules give one after the other, and what
+    the oracle's integer formulation gives."""
+    rng = np.random.default_rng(M + K1 + N1 + N2)
+    l1, l2 = nn.Linear(K1, N1), nn.Linear(N1, N2)
+    l1.register_buffer("weight", L.tensor((rng.standard_normal((N1, K1)) * 0.05).astype(np.float32)))
+    l1.register_buffer("bias", L.tensor((rng.standard_normal(N1) * 0.05).astype(np.float32)))
+    l2.register_buffer("weight", L.tensor((rng.standard_normal((N2, N1)) * 0.05).astype(np.float32)))
+    l2.register_buffer("bias", L.tensor((rng.standard_normal(N2) * 0.05).astype(np.float32)))
+    mods = [l1, nn.ReLU(), l2] if relu else [l1, l2]
+    model = Q.quantize_dynamic(nn.Sequential(*mods))
+    x = rng.standard_normal((M, K1)).astype(np.float32)
+    if kind == "constant":
+        x[:] = 0.25
+    elif kind == "nan":
+        x[M // 2, K1 // 3] = np.nan
+    xd = hip(x)
+    with _recorded_calls() as calls:
+        got_t = model(xd)
+    assert calls == ["lq_dynamic_mlp2_small_f32"]        # one kernel launch for the whole model
+    got = got_t.numpy()
+    h = model[0](xd)
+    if relu:
+        h = model[1](h)
+    want = model[-1](h).numpy()
+    assert got.shape == (M, N2)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~np.isnan(got)].view(np.uint32), want[~np.isnan(want)].view(np.uint32))
+    if kind == "normal":
+        q1, q2 = model[0], model[-1]
+        mn, mx = O.minmax(x)
+        xs, xz = O.calc_qparams(mn, mx, False, 0, 255, False)
+        c1 = O.quantize(x, xs, xz, 0, 255, code_offset=-128)
+        hh = O.qlinear(c1, q1.weight_int8.numpy(), int(xz[0]) - 128, xs, q1.weight_scale.numpy(), bias=q1.bias.numpy(),
+                       relu=relu, out_mode=O.OUT_F32)
+        mn, mx = O.minmax(hh)
+        hs, hz = O.calc_qparams(mn, mx, False, 0, 255, False)
+        c2 = O.quantize(hh, hs, hz, 0, 255, code_offset=-128)
+        exp = O.qlinear(c2, q2.weight_int8.numpy(), int(hz[0]) - 128, hs, q2.weight_scale.numpy(), bias=q2.bias.numpy(),
+                        out_mode=O.OUT_F32)
+        assert np.array_equal(got.view(np.uint32), exp.view(np.uint32))
+
+
+def test_two_dynamic_linears_keep_separate_launches_when_hooked_or_large():
+    """A forward hook has to see each module's own output, and a wide layer does not fit the one
+    block: the modules then run one after the other."""
+    rng = np.random.default_rng(3)
+    model = Q.quantize_dynamic(nn.Sequential(nn.Linear(64, 32), nn.ReLU(), nn.Linear(32, 8)))
+    x = hip(rng.standard_normal((4, 64)).astype(np.float32))
+    seen = []
+    model[0].register_forward_hook(lambda mod, inp, out: seen.append(out.shape))
+    y = model(x)
+    assert seen == [(4, 32)] and y.shape == (4, 8)
+    big = Q.quantize_dynamic(nn.Sequential(nn.Linear(64, 512), nn.Linear(512, 8)))
+    with _recorded_calls() as calls:
+        assert big(x).shape == (4, 8)
+    assert "lq_dynamic_mlp2_small_f32" not in calls and len(calls) >= 2
