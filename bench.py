@@ -54,7 +54,7 @@ MEASURED_TRAFFIC_BYTES = {
 # tile_config (lq_last_tile_config) it was measured under and is reported only when the run
 # resolves to that same configuration (null otherwise: a stale figure would mislead).
 LINEAR_TRAFFIC_BY_TILE_CONFIG = {
-    0x10d: int((2.0 * 55349.4 + 60688.6) * 1024),                       # one launch of 256x352 tiles, eight wavefronts
+    0x10d: int((2.0 * 57280.4 + 54085.0) * 1024),                       # one launch of 256x352 tiles, eight wavefronts
     0x104: int((2.0 * 96504 + 44032) * 1024),                           # one launch of 128x256 tiles
     0x20010b: int((2.0 * (49357.0 + 30884.2) + 32768 + 11264) * 1024),  # 256x256 over 8192 columns + 128x256 over 2816
 }
@@ -889,7 +889,8 @@ def main() -> int:
             "unit": "TOP/s",
             "frac": round(r["kernel_tops"] / PEAK_INT8_TOPS, 4),
             "traffic": LINEAR_TRAFFIC_BY_TILE_CONFIG.get(r["tile_config"]),
-            "kernel": "qgemm_pp_kernel" if (r["tile_config"] & 0xff) in (13, 14) else "qgemm_tile_kernel",
+            "kernel": {13: "qgemm_pp_kernel", 14: "qgemm_pp_kernel", 16: "qgemm_pp_kernel", 17: "qgemm_bw_kernel"}.get(
+                r["tile_config"] & 0xff, "qgemm_tile_kernel"),
             "avg_kernel_us": round(r["avg_kernel_ms"] * 1e3, 2),
             "median_kernel_us": round(r["median_ms"] * 1e3, 2),
             "p95_kernel_us": round(r["p95_ms"] * 1e3, 2),

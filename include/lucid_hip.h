@@ -383,7 +383,10 @@ int lq_global_avgpool_nhwc_i8(const int8_t* q, int code_offset, int B, int H, in
  * packed is [N, K*bits/32], scales and biases [N, K/group_size].  Decoding takes scales
  * and biases as given, so weights packed elsewhere under this contract load unchanged.
  * lq_wq_matmul: out[M,N] = x[M,K] . w_hat^T in float32 (transpose = True of
- * _qgemm.quantized_matmul); M <= 16 streams the packed weight once per four rows,
+ * _qgemm.quantized_matmul).  M = 1 streams the packed weight through a dot-product kernel;
+ * 2 <= M <= 64 (K a multiple of 512 / bits) runs on the matrix cores with the codes as one
+ * bfloat16 operand and x split exactly into three bfloat16 parts, per-group sums scaled in
+ * float32, partial sums of the k ranges added in a fixed order (results are reproducible);
  * larger M decodes into the workspace and runs the float32 GEMM. */
 int lq_wq_quantize(const float* w, int N, int K, int group_size, int bits, uint32_t* packed, float* scales,
                    float* biases, lq_stream stream);

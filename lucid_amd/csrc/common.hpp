@@ -47,6 +47,13 @@ int stream_buffer(int kind, size_t nbytes, size_t min_bytes, hipStream_t stream,
 // kind 0: the general workspace (at least 4 MiB); 1 / 2: stream-K counters / slabs;
 // 3: raw accumulators and operand sums of a layer with affine weights
 int workspace(size_t nbytes, hipStream_t stream, void** ptr);
+// Split-K scratch of one stream: arrival counters (zero between launches: the finisher of a
+// tile resets its counter) and slabs for the partial results, whose layout the kernel defines.
+struct SkScratch {
+    int* counters = nullptr;
+    int32_t* slabs = nullptr;
+};
+int sk_scratch(size_t counters, size_t slab_bytes, hipStream_t st, SkScratch* out);
 // Resolves, for the current device, the address of the static scratch array that
 // lq_minmax_noalloc uses (called by lq_init; the entry point does it on first use otherwise).
 int minmax_noalloc_init();

@@ -860,14 +860,6 @@ using CfgTall8 = TileCfg<128, 256, 64, 2, 4, 3, 2>;
 
 }  // namespace
 
-// Stream-K scratch of one stream: arrival counters (zero between launches: the
-// finisher of a tile resets its counter) and two accumulator slabs per worker.
-struct SkScratch {
-    int* counters = nullptr;
-    int32_t* slabs = nullptr;
-};
-int sk_scratch(size_t counters, size_t slab_bytes, hipStream_t st, SkScratch* out);
-
 namespace {
 
 template <class Cfg, int MODE, int CONV>

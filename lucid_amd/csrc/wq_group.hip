@@ -332,163 +332,380 @@ int launch_gemv(const float* x, const uint32_t* packed, const float* scales, con
     return LQ_OK;
 }
 
-// Small-batch matmul on the matrix cores: up to 16 activation rows against 32 weight
-// rows per block.  The weight is the A operand of v_mfma_f32_16x16x4_f32 and x^T the B
-// operand, so a lane holds one weight row r = lane % 16 (two row blocks) and one
-// activation row of the same index, and the four k slots of an instruction belong to
-// the four lane quarters q = lane / 16.  A quarter owns CODES consecutive k of a step -
-// exactly the codes of one 16-byte load, all in one group - so nothing is shuffled
-// between lanes: code j of the load meets x[k0 + j] in instruction j.  Weights are
-// decoded as c * s + b (the dequantize kernel's expression) right before use.  The four
-// eight wavefronts of a block take the k steps round-robin (two per SIMD, each with
-// four independent accumulator chains, so dependent MFMAs do not wait on each other)
-// and add their partial tiles through LDS in a fixed order.
+// Small-batch matmul on the matrix cores (2 .. 64 activation rows, 16 per block row).
 //
-// Read straight from x, a lane's 16-byte loads would touch 64 different cache lines per
-// instruction (16 rows x 4 quarters).  A pre-pass therefore lays x out in the order the
-// lanes consume it - float4 number (step * XV + j) * 64 + lane of a 16-row block - so
-// that every load of the main kernel is one contiguous KiB per wavefront; rows past M
-// are written as zeros there.
+// y[m, n] = sum over groups g of  s[n, g] * (sum_{k in g} c[n, k] x[m, k])  +  b[n, g] * (sum_{k in g} x[m, k]):
+// the inner sums run on v_mfma_f32_16x16x32_bf16 with the codes themselves as one operand -
+// an 8-bit code is exact in bfloat16, a 4-bit code c is formed as the bit pattern 0x4300 | c
+// = 128 + c (one AND-OR per two codes) and the 128 goes into the bias term - and x as the
+// other, split into three bfloat16 parts x = hi + mid + lo (exact: 8 + 8 + 8 significant
+// bits), one MFMA each.  Products are exact and accumulate in float32, so nothing of x or
+// of the weight is rounded before the sums.
+//
+// Operand layout of the instruction: lane = (row % 16) + 16 * quarter holds eight k of its
+// row, quarter q the k slots 8q .. 8q+7 of the instruction's 32.  x is the A operand (rows
+// m) and the codes the B operand (rows n), so an accumulator lane holds column n = lane % 16
+// and rows m = 4 * quarter + 0..3, and s, b are one value per lane.
+//
+// A lane streams its weight row with 16-byte loads (32 int4 / 16 int8 codes; the four
+// quarters of a row take consecutive loads: a "window" of 128 / 64 k, 1 KiB per wavefront
+// load over 16 rows).  An instruction must stay inside one group, because the scale is
+// applied to its sum.  With group_size >= the window that holds as loaded (register j of
+// every quarter feeds instruction j).  With two groups per window the registers are
+// exchanged between lane halves (v_permlane32_swap: instructions 0, 1 then hold the first
+// two quarters' k, instructions 2, 3 the last two), with four groups the 4 x 4 (register,
+// quarter) matrix is transposed (v_permlane32_swap + v_permlane16_swap), so instruction i
+// holds the k of quarter i.  Which k a slot of an instruction ends up with does not matter
+// as long as x follows: the block writes the three parts of its x range into LDS in exactly
+// that order.  The sum of x over a group segment comes from the same fragments against a
+// row of ones (one more accumulator tile per wavefront), already in the layout the lanes
+// need it in.
+//
+// Every block needs the x of its k range next to its weights (64 bytes of x per k against
+// rows / 2 or rows bytes of codes), and every block converts it again.  So a block takes
+// many rows (256: eight wavefronts with two 16-row tiles each) and a short k range (512),
+// keeps that range's fragments in LDS for all its wavefronts, and requests all its weights
+// at once when it starts.  The k ranges of a row tile are blocks of their own (grid.y); each
+// writes its partial sums to a slab, and the last one to arrive (an arrival counter per row
+// tile, reset by that block) adds the slabs in index order - the result does not depend on
+// the order of arrival - and stores.  One launch, no workspace besides the slabs.
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+// LDS a block may ask for: 48 KiB of x fragments and the tables of 256 rows x 16 groups
+constexpr int kWqMaxLds = 512 / 32 * 3 * 64 * 16 + 2 * 256 * 17 * 4;
 
 template <int BITS>
-__global__ __launch_bounds__(256) void wq_arrange_x_kernel(const float* __restrict__ x, int M, int K,
-                                                           float4* __restrict__ xt) {
-    constexpr int CODES = 128 / BITS, STEP = 4 * CODES, XV = CODES / 4;
-    const int per_block = K / STEP * XV * 64;  // float4 per 16-row block
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= per_block) return;
-    const int lane = idx & 63, sj = idx >> 6, j = sj % XV, step = sj / XV;
-    const int m = blockIdx.y * 16 + (lane & 15), k = step * STEP + (lane >> 4) * CODES + 4 * j;
-    float4 v = {0.f, 0.f, 0.f, 0.f};
-    if (m < M) v = *reinterpret_cast<const float4*>(x + size_t(m) * K + k);
-    xt[size_t(blockIdx.y) * per_block + idx] = v;
+struct WqGeom {
+    static constexpr int CODES = 128 / BITS;  // codes per 16-byte load: 32 or 16
+    static constexpr int WK = 4 * CODES;      // k per window: 128 or 64
+    static constexpr int NI = WK / 32;        // instructions (k steps of 32) per window: 4 or 2
+};
+
+// How the registers are exchanged for a group size: 0 = not at all, 1 = between lane halves,
+// 2 = transposed; the window then holds 1, 2 or 4 group segments.
+__host__ __device__ inline int wq_swap_mode(int bits, int gs) {
+    const int window = 512 / bits;
+    return gs >= window ? 0 : (gs * 2 == window ? 1 : 2);
 }
 
-template <int BITS>
-__global__ __launch_bounds__(512) void wq_mfma_kernel(const float4* xt, const uint32_t* packed, const float* scales,
-                                                      const float* biases, int M, int N, int K, int gs, float* out) {
-    constexpr int CODES = 128 / BITS;  // codes per 16-byte load: 32 or 16
-    constexpr int STEP = 4 * CODES;    // k covered by one wavefront step
-    constexpr int XV = CODES / 4;      // float4 loads of x per step
-    constexpr uint32_t MASK = (1u << BITS) - 1u;
-    constexpr int WAVES = 8;
-    __shared__ __attribute__((aligned(16))) float red[WAVES][2][64][4];
-    // the wavefront index as a scalar, so that the step loop branches uniformly
+// After the exchange, register rho of quarter q holds what quarter q_src loaded as register j_src.
+__host__ __device__ inline void wq_source(int sw, int rho, int q, int& q_src, int& j_src) {
+    q_src = q, j_src = rho;
+    if (sw == 1 && (rho < 2) != (q < 2)) {
+        q_src = rho < 2 ? q - 2 : q + 2;
+        j_src = rho < 2 ? rho + 2 : rho - 2;
+    } else if (sw == 2) {
+        q_src = rho, j_src = q;
+    }
+}
+
+// upper lane half of a <-> lower lane half of b
+__device__ __forceinline__ void wq_swap32(uint32_t& a, uint32_t& b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    a = r[0], b = r[1];
+}
+// odd 16-lane rows of a <-> even 16-lane rows of b
+__device__ __forceinline__ void wq_swap16(uint32_t& a, uint32_t& b) {
+    const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+    a = r[0], b = r[1];
+}
+
+// x = h + m + l with each part a bfloat16 (bit patterns in the low halves)
+__device__ __forceinline__ void wq_split3(float x, uint32_t& h, uint32_t& m, uint32_t& l) {
+    const uint32_t xb = __float_as_uint(x);
+    h = xb >> 16;  // truncated: the remainder keeps x's sign and has at most 16 significant bits
+    const float r1 = x - __uint_as_float(xb & 0xffff0000u);
+    const uint32_t rb = __float_as_uint(r1);
+    m = rb >> 16;
+    const float r2 = r1 - __uint_as_float(rb & 0xffff0000u);  // at most 8 significant bits: a bfloat16
+    l = __float_as_uint(r2) >> 16;
+    if ((xb & 0x7f800000u) == 0x7f800000u) m = l = 0;  // infinity / NaN stay in the first part alone
+}
+
+constexpr int kWqRows = 256;    // weight rows per block
+constexpr int kWqSliceK = 512;  // k per block
+
+template <int BITS, int SW>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void wq_mfma_kernel(
+    const float* x, const uint32_t* packed, const float* scales, const float* biases, int M, int N, int K,
+    int gs_shift, float* out, float* slabs, int* counters) {
+    using G = WqGeom<BITS>;
+    constexpr int CODES = G::CODES, WK = G::WK, NI = G::NI;
+    constexpr int GW = 1 << SW, SEG = WK / GW;  // group segments per window and their length
+    constexpr int IPS = NI / GW;                // instructions per segment
+    constexpr int RB = 2, WAVES = 8, WPS = kWqSliceK / WK;  // windows per block: 4 or 8
+    constexpr int UNITS = WPS * NI * 64;                    // (window, instruction, lane) triples of the block's x
+    static_assert(IPS >= 1, "a segment is at least one instruction");
+    static_assert(WAVES * RB * 16 == kWqRows && UNITS % 512 == 0, "");
+    // Dynamic LDS: the x fragments of the block's windows ([window][instruction][part][lane],
+    // 16 bytes each), then the block's rows of scales and of biases for the groups of those
+    // windows - each row padded by one float: lanes of a quarter read 16 different rows at the
+    // same group, and the odd stride spreads them over the banks.
+    extern __shared__ __attribute__((aligned(16))) uint4 wq_lds[];
+    __shared__ int s_arrived;
+    // the wavefront index as a scalar, so that branches on it are uniform
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, q = lane >> 4;
-    const int n_base = blockIdx.x * 32;
-    const int words_per_row = K * BITS / 32, groups_per_row = K / gs;
-    const int gs_shift = 31 - __builtin_clz(gs);  // group sizes are powers of two
-    const int m0 = blockIdx.y * 16;
-    const float4* xblk = xt + size_t(blockIdx.y) * (K / STEP * XV * 64) + lane;
-    const uint32_t* wrow[2];
-    const float* srow[2];
-    const float* brow[2];
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
-        int n = n_base + rb * 16 + r;
-        n = n < N ? n : N - 1;  // clamped rows are computed and dropped at the store
-        wrow[rb] = packed + size_t(n) * words_per_row;
-        srow[rb] = scales + size_t(n) * groups_per_row;
-        brow[rb] = biases + size_t(n) * groups_per_row;
-    }
-    v4f acc[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
-    const int steps = K / STEP;
+    const int tile = blockIdx.x, ks = blockIdx.y, mb = blockIdx.z, slices = gridDim.y;
+    const int n_base = tile * kWqRows + wave * (RB * 16), m0 = mb * 16;
+    const int words_per_row = K * BITS / 32, groups_per_row = K >> gs_shift;
+    const int windows = K / WK;
+    const int w0 = ks * WPS;
+    const int nw = windows - w0 < WPS ? windows - w0 : WPS;  // at least 1: the host sizes grid.y so
+    // groups of this block's windows, and the row stride of the tables
+    const int g0 = (w0 * WK) >> gs_shift;
+    const int ng = (((w0 + nw) * WK - 1) >> gs_shift) - g0 + 1;
+    const int gmax = kWqSliceK >> gs_shift, gp = (gmax < 1 ? 1 : gmax) + 1;
 
-    // Two register sets, named at compile time (a run-time buffer index would put the
-    // arrays in scratch memory): the loads of the next step are issued before this one
-    // is used.
-    struct Operands {
-        uint4 wv[2];
-        float sc[2], bi[2];
-        float4 xv[XV];
-    };
-    auto fetch = [&](int step, Operands& o) {
-        const int k0 = step * STEP + q * CODES;
+    // All the weights of this wavefront are requested now and used window by window.  For the
+    // request a lane takes quarter lane % 4 of row lane / 4 - four neighbouring lanes read 64
+    // contiguous bytes, where the operand layout (row lane % 16, quarter lane / 16) would make
+    // every lane a cache access of its own -; a lane permutation below puts each 16 bytes
+    // where the instruction wants them.
+    uint4 wv[WPS][RB];
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-            o.wv[rb] = *reinterpret_cast<const uint4*>(wrow[rb] + k0 * BITS / 32);
-            o.sc[rb] = srow[rb][k0 >> gs_shift];
-            o.bi[rb] = brow[rb][k0 >> gs_shift];
+    for (int rb = 0; rb < RB; ++rb) {
+        int n = n_base + rb * 16 + (lane >> 2);
+        n = n < N ? n : N - 1;  // clamped rows are computed and dropped at the store
+        const uint32_t* row = packed + size_t(n) * words_per_row + (lane & 3) * (CODES * BITS / 32);
+#pragma unroll
+        for (int wi = 0; wi < WPS; ++wi)
+            // past the last window every lane reads the same 16 bytes: one cache line, dropped later
+            wv[wi][rb] = *reinterpret_cast<const uint4*>(wi < nw ? row + (w0 + wi) * (WK * BITS / 32) : packed);
+    }
+    // x of the block's windows, split and laid out as fragments by the block itself.  A thread
+    // takes eight consecutive k of one row (a wavefront reads 2 KiB of a row) and finds the
+    // (instruction, quarter) that holds them: the exchange of registers is its own inverse.
+    uint4* x_lds = wq_lds;
+    {
+        constexpr int OCTS = kWqSliceK / 8;  // per row
+        static_assert(16 * OCTS == UNITS, "");
+        float4 raw[UNITS / 512][2];
+#pragma unroll
+        for (int u = 0; u < UNITS / 512; ++u) {
+            const int unit = u * 512 + threadIdx.x, m = m0 + unit / OCTS, kl = (unit % OCTS) * 8;
+            raw[u][0] = raw[u][1] = float4{0.f, 0.f, 0.f, 0.f};
+            if (m < M && kl < nw * WK) {
+                const float* src = x + size_t(m) * K + w0 * WK + kl;
+                raw[u][0] = *reinterpret_cast<const float4*>(src);
+                raw[u][1] = *reinterpret_cast<const float4*>(src + 4);
+            }
         }
 #pragma unroll
-        for (int j = 0; j < XV; ++j) o.xv[j] = xblk[(step * XV + j) * 64];
-    };
-    auto compute = [&](const Operands& o) {
+        for (int u = 0; u < UNITS / 512; ++u) {
+            const int unit = u * 512 + threadIdx.x, ml = unit / OCTS, kl = (unit % OCTS) * 8;
+            const int wi = kl / WK, off = kl % WK, qs = off / CODES, js = (off % CODES) / (32 / BITS);
+            int qd, rho;
+            wq_source(SW, js, qs, qd, rho);
+            const int i = BITS == 4 ? rho : rho / 2;
+            const float v[8] = {raw[u][0].x, raw[u][0].y, raw[u][0].z, raw[u][0].w,
+                                raw[u][1].x, raw[u][1].y, raw[u][1].z, raw[u][1].w};
+            uint32_t d3[3][4];
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-            const uint32_t words[4] = {o.wv[rb].x, o.wv[rb].y, o.wv[rb].z, o.wv[rb].w};
-            const float s = o.sc[rb], b = o.bi[rb];
+            for (int d = 0; d < 4; ++d) {
+                // slots 2d, 2d+1: the 4-bit decode pairs nibble d with nibble d + 4
+                const float e0 = BITS == 4 ? v[d] : v[2 * d], e1 = BITS == 4 ? v[d + 4] : v[2 * d + 1];
+                uint32_t h0, m0_, l0, h1, m1, l1;
+                wq_split3(e0, h0, m0_, l0);
+                wq_split3(e1, h1, m1, l1);
+                d3[0][d] = h0 | (h1 << 16), d3[1][d] = m0_ | (m1 << 16), d3[2][d] = l0 | (l1 << 16);
+            }
+            if (wi < nw) {
 #pragma unroll
-            for (int j = 0; j < CODES; ++j) {
-                const uint32_t code = (words[j * BITS / 32] >> ((j * BITS) % 32)) & MASK;
-                const float wval = float(code) * s + b;
-                const float4 xq = o.xv[j / 4];
-                const float xval = (j % 4) == 0 ? xq.x : ((j % 4) == 1 ? xq.y : ((j % 4) == 2 ? xq.z : xq.w));
-                acc[rb][j & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(wval, xval, acc[rb][j & 1], 0, 0, 0);
+                for (int p = 0; p < 3; ++p)
+                    x_lds[((wi * NI + i) * 3 + p) * 64 + ml + 16 * qd] = uint4{d3[p][0], d3[p][1], d3[p][2], d3[p][3]};
+            }
+        }
+    }
+    float* s_lds = reinterpret_cast<float*>(wq_lds + WPS * NI * 3 * 64);
+    float* b_lds = s_lds + kWqRows * gp;
+    {
+        const int row_first = tile * kWqRows;
+        for (int i = threadIdx.x; i < kWqRows * ng; i += 512) {
+            const int row = i / ng, g = i - row * ng;
+            const int n = row_first + row < N ? row_first + row : N - 1;
+            s_lds[row * gp + g] = scales[size_t(n) * groups_per_row + g0 + g];
+            b_lds[row * gp + g] = biases[size_t(n) * groups_per_row + g0 + g];
+        }
+    }
+    __syncthreads();
+
+    v4f y[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) y[rb] = v4f{0.f, 0.f, 0.f, 0.f};
+    const int row_in_tile = wave * (RB * 16) + r;
+    const uint4 ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};  // eight times 1.0
+#pragma unroll
+    for (int wi = 0; wi < WPS; ++wi) {
+        if (wi < nw) {
+            uint32_t wd[RB][4];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                // lane (row r, quarter q) takes what lane 4 r + q loaded
+                const int from = (4 * r + q) * 4;
+                wd[rb][0] = uint32_t(__builtin_amdgcn_ds_bpermute(from, int(wv[wi][rb].x)));
+                wd[rb][1] = uint32_t(__builtin_amdgcn_ds_bpermute(from, int(wv[wi][rb].y)));
+                wd[rb][2] = uint32_t(__builtin_amdgcn_ds_bpermute(from, int(wv[wi][rb].z)));
+                wd[rb][3] = uint32_t(__builtin_amdgcn_ds_bpermute(from, int(wv[wi][rb].w)));
+                if (SW >= 1) wq_swap32(wd[rb][0], wd[rb][2]), wq_swap32(wd[rb][1], wd[rb][3]);
+                if (SW == 2) wq_swap16(wd[rb][0], wd[rb][1]), wq_swap16(wd[rb][2], wd[rb][3]);
+            }
+#pragma unroll
+            for (int e = 0; e < GW; ++e) {
+                const int g = (((w0 + wi) * WK + e * SEG) >> gs_shift) - g0;
+                // acc[RB]: the segment's sum of x, from the same fragments against a row of ones (every
+                // column of that tile holds it: exactly the value each lane needs for its rows m)
+                v4f acc[RB + 1];
+#pragma unroll
+                for (int rb = 0; rb <= RB; ++rb) acc[rb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ii = 0; ii < IPS; ++ii) {
+                    const int i = e * IPS + ii;
+                    uint4 cf[RB];
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb) {
+                        if (BITS == 4) {
+                            const uint32_t c = wd[rb][i];
+                            cf[rb].x = (c & 0x000f000fu) | 0x43004300u;
+                            cf[rb].y = ((c >> 4) & 0x000f000fu) | 0x43004300u;
+                            cf[rb].z = ((c >> 8) & 0x000f000fu) | 0x43004300u;
+                            cf[rb].w = ((c >> 12) & 0x000f000fu) | 0x43004300u;
+                        } else {
+                            // a byte as a float has zeros below bit 16: its upper half is the bfloat16
+                            const uint32_t a = wd[rb][2 * i], b = wd[rb][2 * i + 1];
+                            const uint32_t a0 = __float_as_uint(float(a & 0xffu)), a1 = __float_as_uint(float((a >> 8) & 0xffu));
+                            const uint32_t a2 = __float_as_uint(float((a >> 16) & 0xffu)), a3 = __float_as_uint(float(a >> 24));
+                            const uint32_t b0 = __float_as_uint(float(b & 0xffu)), b1 = __float_as_uint(float((b >> 8) & 0xffu));
+                            const uint32_t b2 = __float_as_uint(float((b >> 16) & 0xffu)), b3 = __float_as_uint(float(b >> 24));
+                            cf[rb].x = __builtin_amdgcn_perm(a1, a0, 0x07060302u);
+                            cf[rb].y = __builtin_amdgcn_perm(a3, a2, 0x07060302u);
+                            cf[rb].z = __builtin_amdgcn_perm(b1, b0, 0x07060302u);
+                            cf[rb].w = __builtin_amdgcn_perm(b3, b2, 0x07060302u);
+                        }
+                    }
+#pragma unroll
+                    for (int p = 0; p < 3; ++p) {
+                        const v8bf xf = __builtin_bit_cast(v8bf, x_lds[((wi * NI + i) * 3 + p) * 64 + lane]);
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb)
+                            acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, __builtin_bit_cast(v8bf, cf[rb]),
+                                                                              acc[rb], 0, 0, 0);
+                        acc[RB] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, __builtin_bit_cast(v8bf, ones), acc[RB], 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    const float sc = s_lds[(row_in_tile + rb * 16) * gp + g];
+                    const float bi = b_lds[(row_in_tile + rb * 16) * gp + g];
+                    // the 4-bit codes entered as 128 + c
+                    const float bz = BITS == 4 ? bi - 128.0f * sc : bi;
+                    y[rb] = y[rb] + (acc[rb] * sc + acc[RB] * bz);
+                }
+            }
+        }
+    }
+
+    // accumulator element t of a lane: row m = 4 * quarter + t, column n = lane % 16
+    auto store_out = [&](const v4f (&v)[RB]) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int n = n_base + rb * 16 + r;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int mm = m0 + 4 * q + t;
+                if (n < N && mm < M) out[size_t(mm) * N + n] = v[rb][t];
             }
         }
     };
-    // The look-ahead fetch is unconditional (past the end it re-reads the last step and
-    // the result is dropped): a branch around it would make the compiler wait, at the
-    // join, as if the new loads had not been issued - that is, for them.
-    // keeps the look-ahead loads ahead of the MFMAs: neither the optimizer (memory clobber;
-    // the pointers are not __restrict__ for that reason) nor the instruction scheduler may
-    // move a load across this point
-    auto pin = [] {
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    Operands o0, o1;
-    int step = wave;
-    const int last = steps - 1;
-    if (step < steps) {
-        fetch(step, o0);
-        for (;;) {
-            fetch(step + WAVES < steps ? step + WAVES : last, o1);
-            pin();
-            compute(o0);
-            pin();
-            step += WAVES;
-            if (step >= steps) break;
-            fetch(step + WAVES < steps ? step + WAVES : last, o0);
-            pin();
-            compute(o1);
-            pin();
-            step += WAVES;
-            if (step >= steps) break;
-        }
+    if (slices == 1) {
+        store_out(y);
+        return;
     }
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb) *reinterpret_cast<v4f*>(red[wave][rb][lane]) = acc[rb][0] + acc[rb][1];
-    __syncthreads();
-    // D[i][j]: lane holds i = 4 * (lane / 16) + t, j = lane % 16  ->  out[m0 + j][n_base + rb*16 + i]
+    // slab of (row tile, k range): [wavefront][tile of 16 rows][lane] x 16 bytes, written through to
+    // device scope; then the arrival counter of the row tile
+    constexpr unsigned kScopeDevice = 16;  // "sc1" cache-policy bit of buffer accesses
+    constexpr unsigned kSlabBytes = WAVES * RB * 64 * 16;
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const size_t tile_index = size_t(mb) * gridDim.x + tile;
+    float* first_slab = slabs + tile_index * slices * (kSlabBytes / 4);
+    const unsigned my_off = unsigned((wave * RB) * 64 + lane) * 16;
     {
-        const int e = threadIdx.x;  // 2 * 64 * 4 = 512 values, one per thread
-        const int rb = e >> 8, l = (e >> 2) & 63, t = e & 3;
-        float v = red[0][rb][l][t];
+        const __amdgpu_buffer_rsrc_t mine =
+            __builtin_amdgcn_make_buffer_rsrc(first_slab + size_t(ks) * (kSlabBytes / 4), 0, kSlabBytes, 0x00020000);
 #pragma unroll
-        for (int w = 1; w < WAVES; ++w) v += red[w][rb][l][t];
-        const int n = n_base + rb * 16 + 4 * (l >> 4) + t, mm = m0 + (l & 15);
-        if (n < N && mm < M) out[size_t(mm) * N + n] = v;
+        for (int rb = 0; rb < RB; ++rb)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, y[rb]), mine, my_off + unsigned(rb * 64 * 16), 0,
+                                                   kScopeDevice);
     }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's partial sums have been written through
+    __syncthreads();                      // ... and so have the other wavefronts'
+    if (threadIdx.x == 0)
+        s_arrived = __hip_atomic_fetch_add(&counters[tile_index], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (__builtin_amdgcn_readfirstlane(s_arrived) != slices - 1) return;
+    v4f total[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) total[rb] = v4f{0.f, 0.f, 0.f, 0.f};
+    // eight slabs are requested together (one memory round trip, not eight); a slot past the
+    // last slab re-reads the last one and is not added, so that the loads stay unconditional
+    constexpr int kBatch = 8;
+    for (int k0 = 0; k0 < slices; k0 += kBatch) {
+        v4u part[kBatch][RB];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const int k = k0 + j < slices ? k0 + j : slices - 1;
+            const __amdgpu_buffer_rsrc_t other =
+                __builtin_amdgcn_make_buffer_rsrc(first_slab + size_t(k) * (kSlabBytes / 4), 0, kSlabBytes, 0x00020000);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+                part[j][rb] = __builtin_amdgcn_raw_buffer_load_b128(other, my_off + unsigned(rb * 64 * 16), 0, kScopeDevice);
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j)
+            if (k0 + j < slices) {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) total[rb] = total[rb] + __builtin_bit_cast(v4f, part[j][rb]);
+            }
+    }
+    store_out(total);
+    if (threadIdx.x == 0) counters[tile_index] = 0;  // ready for the next launch
 }
+
 
 template <int BITS>
 int launch_wq_mfma(const float* x, const uint32_t* packed, const float* scales, const float* biases, int M, int N,
                    int K, int gs, float* out, hipStream_t st) {
-    constexpr int STEP = 512 / BITS;
-    const int mblocks = (M + 15) / 16;
-    void* ws = nullptr;
-    const int rc = workspace(size_t(mblocks) * 16 * K * sizeof(float), st, &ws);
-    if (rc) return rc;
-    const int per_block = K / STEP * (32 / BITS) * 64;
-    hipLaunchKernelGGL((wq_arrange_x_kernel<BITS>), dim3(unsigned((per_block + 255) / 256), unsigned(mblocks)),
-                       dim3(256), 0, st, x, M, K, static_cast<float4*>(ws));
-    LQ_CHECK_LAUNCH("wq_arrange_x");
-    hipLaunchKernelGGL((wq_mfma_kernel<BITS>), dim3(unsigned((N + 31) / 32), unsigned(mblocks)), dim3(512), 0, st,
-                       static_cast<const float4*>(ws), packed, scales, biases, M, N, K, gs, out);
+    using G = WqGeom<BITS>;
+    constexpr int WPS = kWqSliceK / G::WK;
+    const int sw = wq_swap_mode(BITS, gs);
+    const int mblocks = (M + 15) / 16, windows = K / G::WK;
+    const int tiles = (N + kWqRows - 1) / kWqRows, slices = (windows + WPS - 1) / WPS;
+    SkScratch sk;
+    if (slices > 1) {
+        const int rc = sk_scratch(size_t(mblocks) * tiles, size_t(mblocks) * tiles * slices * (8 * 2 * 64 * 16), st, &sk);
+        if (rc) return rc;
+    }
+    const dim3 grid{unsigned(tiles), unsigned(slices), unsigned(mblocks)};
+    const int gs_shift = 31 - __builtin_clz(unsigned(gs));
+    const int gmax = kWqSliceK / gs;
+    const size_t lds = size_t(WPS) * G::NI * 3 * 64 * 16 + size_t(2) * kWqRows * ((gmax < 1 ? 1 : gmax) + 1) * 4;
+#define LQ_WQ_LAUNCH(SWM)                                                                                         \
+    do {                                                                                                          \
+        static DeviceOnce attr_once;                                                                              \
+        const int arc = allow_dynamic_lds(attr_once, reinterpret_cast<const void*>(wq_mfma_kernel<BITS, SWM>),    \
+                                          kWqMaxLds);                                                             \
+        if (arc) return arc;                                                                                      \
+        hipLaunchKernelGGL((wq_mfma_kernel<BITS, SWM>), grid, dim3(512), lds, st, x, packed, scales, biases, M,   \
+                           N, K, gs_shift, out, reinterpret_cast<float*>(sk.slabs), sk.counters);                 \
+    } while (0)
+    if (sw == 0)
+        LQ_WQ_LAUNCH(0);
+    else if (sw == 1)
+        LQ_WQ_LAUNCH(1);
+    else if constexpr (BITS == 4)
+        LQ_WQ_LAUNCH(2);
+#undef LQ_WQ_LAUNCH
     LQ_CHECK_LAUNCH("wq_mfma");
     return LQ_OK;
 }

@@ -56,6 +56,26 @@ def test_matmul_against_the_dequantize_path(bits, M, N, K, gs):
     assert np.allclose(y, y_deq, atol=1e-3)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_small_batch_matmul_is_reproducible_and_exact_on_exact_inputs(bits):
+    # the matrix-core path adds the partial sums of its k ranges in a fixed order: two calls
+    # agree bit for bit; and with x, scales and biases that keep every product and sum exact in
+    # float32 (small integers), the result equals the integer arithmetic exactly - x is split
+    # into bfloat16 parts without loss and the codes enter unrounded
+    rng = np.random.default_rng(bits)
+    M, N, K, gs = 16, 300, 1024, 64
+    packed = rng.integers(0, 2**32, (N, K * bits // 32), dtype=np.uint32).view(np.int32)
+    s = rng.integers(1, 3, (N, K // gs)).astype(np.float32)
+    b = rng.integers(-8, 9, (N, K // gs)).astype(np.float32)
+    x = rng.integers(-7, 8, (M, K)).astype(np.float32)  # every partial sum stays below 2^24
+    args = (hip(x), hip(packed), hip(s), hip(b), True, gs, bits)
+    y1 = _qgemm.quantized_matmul(*args).numpy()
+    y2 = _qgemm.quantized_matmul(*args).numpy()
+    assert np.array_equal(y1, y2)
+    w = W.dequantize(packed, s, b, gs, bits).astype(np.float64)
+    assert np.array_equal(y1.astype(np.float64), x.astype(np.float64) @ w.T)
+
+
 def test_decoding_takes_foreign_scales_and_biases_as_given():
     # a weight packed elsewhere under the same contract may carry negative scales
     rng = np.random.default_rng(1)
