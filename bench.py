@@ -577,7 +577,9 @@ def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     """Dynamic-quantized MLP Linear(784,256)-ReLU-Linear(256,10), batch 64
     (launch-latency bound: 0.43 MOP).  Eager = one Python-driven forward (ONE launch: a single
     block takes each layer's min / max, qparams and codes, multiplies, and applies the ReLU
-    between them); graph = the same forward replayed from a HIP graph."""
+    between them); graph = the forward replayed from a HIP graph, which holds the two layers as
+    two launches of many blocks (nn.Sequential does not fuse under capture: shorter on the GPU,
+    and a replay pays the launch cost once either way)."""
     import lucid_amd.nn as nn
 
     rng = np.random.default_rng(1)
@@ -598,7 +600,7 @@ def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     assert np.isfinite(y.numpy()).all()
     g.destroy()
     return {"eager_us_per_forward": round(eager_us, 1), "graph_us_per_forward": round(graph_us, 1),
-            "launches_per_forward": 1}
+            "launches_per_forward": {"eager": 1, "graph": 2}}
 
 
 def bench_weight_only(L, _C, steps, warmup, K=4096, N=11008, gs=64):
@@ -797,7 +799,7 @@ def main() -> int:
     ap.add_argument("--vendor-yardstick", action="store_true",
                     help="time the ROCm library's int8 GEMM (through torch._int_mm, if torch is importable) "
                          "on the same operand codes beside this library's; a yardstick, not a dependency")
-    ap.add_argument("--only", default=None, choices=["resnet50", "vit", "decode"],
+    ap.add_argument("--only", default=None, choices=["resnet50", "vit", "decode", "mlp"],
                     help="run just this end-to-end leg and print its figures")
     ap.add_argument("--vendor-child", default=None, help=argparse.SUPPRESS)
     ap.add_argument("--no-extra", action="store_true")
@@ -856,6 +858,9 @@ def main() -> int:
                                    "frac_of_8TBs_llc_resident": round(rs["gbs"] / PEAK_HBM_GBS, 4)}
         res["weight_only_group64_k4096_n11008"] = bench_weight_only(L, _C, args.steps, args.warmup)
         print(json.dumps(res))
+        return 0
+    if args.only == "mlp":
+        print(json.dumps({"dynamic_mlp_784_256_10_batch64": bench_dynamic_mlp(L, Q, _C, max(args.steps, 200), args.warmup)}))
         return 0
     if args.only:
         # one of the end-to-end legs alone (a clean kernel trace of one network)

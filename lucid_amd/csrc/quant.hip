@@ -784,10 +784,18 @@ __global__ __launch_bounds__(1024) void dynamic_linear_small_kernel(
     // wavefront's first weight fragment and the output lane's column parameters.
     const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
     const int ln = lane & 15, lg = lane >> 4;
-    const int8_t* wrow = w + size_t(n0 + ln < N ? n0 + ln : N - 1) * size_t(K);
+    // (requested with lane = 4 * row + chunk, so that four neighbouring lanes read 64 contiguous bytes,
+    // and handed to the lane that multiplies it - row lane % 16, chunk lane / 16 - by dl_place)
+    const int rq = lane >> 2, cq = lane & 3;
+    const int8_t* wrow = w + size_t(n0 + rq < N ? n0 + rq : N - 1) * size_t(K);
+    auto dl_place = [&](dl_v4i f) {
+        const int from = (4 * ln + lg) * 4;
+        return dl_v4i{__builtin_amdgcn_ds_bpermute(from, f[0]), __builtin_amdgcn_ds_bpermute(from, f[1]),
+                      __builtin_amdgcn_ds_bpermute(from, f[2]), __builtin_amdgcn_ds_bpermute(from, f[3])};
+    };
     const int ksteps = (K + 63) >> 6;
-    const bool first_in_k = wave < ksteps && wave * 64 + lg * 16 < K;
-    const dl_v4i wf_first = first_in_k ? *reinterpret_cast<const dl_v4i*>(wrow + wave * 64 + lg * 16) : dl_v4i{0, 0, 0, 0};
+    const bool first_in_k = wave < ksteps && wave * 64 + cq * 16 < K;
+    const dl_v4i wf_first = first_in_k ? *reinterpret_cast<const dl_v4i*>(wrow + wave * 64 + cq * 16) : dl_v4i{0, 0, 0, 0};
     const int out_n = n0 + (tid & 15);
     const bool out_lane = tid < 256 && out_n < N;
     const float c_ws = (out_lane && w_scale) ? w_scale[out_n] : 1.0f;
@@ -830,7 +838,9 @@ __global__ __launch_bounds__(1024) void dynamic_linear_small_kernel(
     for (int ks = wave; ks < ksteps; ks += 16) {
         const int k = ks * 64 + lg * 16;
         const bool in_k = k < K;  // K % 16 == 0: a 16-byte chunk is inside or outside as a whole
-        const dl_v4i wf = ks == wave ? wf_first : (in_k ? *reinterpret_cast<const dl_v4i*>(wrow + k) : dl_v4i{0, 0, 0, 0});
+        const int kq = ks * 64 + cq * 16;
+        const dl_v4i wf = dl_place(ks == wave ? wf_first
+                                              : (kq < K ? *reinterpret_cast<const dl_v4i*>(wrow + kq) : dl_v4i{0, 0, 0, 0}));
         const dl_v4i af = in_k ? *reinterpret_cast<const dl_v4i*>(codes + size_t(ln) * K + k) : dl_v4i{0, 0, 0, 0};
         acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc, 0, 0, 0);
     }
@@ -894,6 +904,33 @@ __global__ __launch_bounds__(1024) void dynamic_mlp2_small_kernel(
         const int i = u * 1024 + tid;
         if (i < quads) v[u] = x4[i];
     }
+    // A wavefront owns one block of 16 columns of layer 1 (N1 <= 256 = 16 wavefronts x 16) over
+    // at most 16 k steps, and one 16 x 16 tile of layer 2 over at most 4.  All its weight
+    // fragments of a layer are requested together - layer 2's here, behind x; layer 1's as soon as
+    // the registers that hold x are free - so each layer pays one memory round trip.  (Requested
+    // one k step ahead instead, the 13 dependent round trips of K1 = 784 were most of the time.)
+    constexpr int kSteps1 = 16, kSteps2 = 4;
+    const int n1 = wave * 16 + ln, nc1 = n1 < N1 ? n1 : N1 - 1;  // the column whose results this lane holds
+    const int rb2 = wave & 3, cb2 = wave >> 2;
+    const int n2 = cb2 * 16 + ln, nc2 = n2 < N2 ? n2 : N2 - 1;
+    // For the request a lane takes 16-byte chunk lane % 4 of row lane / 4, so that four
+    // neighbouring lanes read 64 contiguous bytes (with the operand layout - row lane % 16, chunk
+    // lane / 16 - every lane would be a cache access of its own: 64 per instruction on the one CU
+    // that runs this block); ml_place then hands each chunk to the lane that multiplies it.
+    const int rq = lane >> 2, cq = lane & 3;
+    auto ml_place = [&](ml_v4i f) {
+        const int from = (4 * ln + lg) * 4;
+        return ml_v4i{__builtin_amdgcn_ds_bpermute(from, f[0]), __builtin_amdgcn_ds_bpermute(from, f[1]),
+                      __builtin_amdgcn_ds_bpermute(from, f[2]), __builtin_amdgcn_ds_bpermute(from, f[3])};
+    };
+    ml_v4i w1f[kSteps1], w2f[kSteps2];
+    {
+        const int r2 = cb2 * 16 + rq;
+        const int8_t* wrow2 = w2 + size_t(r2 < N2 ? r2 : N2 - 1) * size_t(N1) + cq * 16;
+#pragma unroll
+        for (int ks = 0; ks < kSteps2; ++ks)  // N1 % 16 == 0: a 16-byte chunk is inside or outside as a whole
+            w2f[ks] = ks * 64 + cq * 16 < N1 ? *reinterpret_cast<const ml_v4i*>(wrow2 + ks * 64) : ml_v4i{0, 0, 0, 0};
+    }
     for (int i = quads + tid; i < 16 * K1; i += 1024) reinterpret_cast<unsigned*>(codes1)[i] = 0u;
     for (int i = ((M * N1) >> 2) + tid; i < 16 * N1; i += 1024) reinterpret_cast<unsigned*>(codes2)[i] = 0u;
 #pragma unroll
@@ -915,6 +952,13 @@ __global__ __launch_bounds__(1024) void dynamic_mlp2_small_kernel(
             if (i < quads) op.q[i] = op.pack(v[u], s, z, r);
         }
     }
+    {
+        const int r1 = wave * 16 + rq;
+        const int8_t* wrow1 = w1 + size_t(r1 < N1 ? r1 : N1 - 1) * size_t(K1) + cq * 16;
+#pragma unroll
+        for (int ks = 0; ks < kSteps1; ++ks)
+            w1f[ks] = ks * 64 + cq * 16 < K1 ? *reinterpret_cast<const ml_v4i*>(wrow1 + ks * 64) : ml_v4i{0, 0, 0, 0};
+    }
     __syncthreads();
 
     // ---- layer 1: GEMM.  A wavefront owns 16 output columns (a weight fragment is loaded once per
@@ -923,29 +967,27 @@ __global__ __launch_bounds__(1024) void dynamic_mlp2_small_kernel(
     {
         const float s = s_sz[0], z = s_sz[1];
         const int zp = int(z) + off;
-        const int ksteps = (K1 + 63) >> 6;
-        for (int cb = wave; cb * 16 < N1; cb += 16) {
-            const int n = cb * 16 + ln;
-            const int nc = n < N1 ? n : N1 - 1;
-            const int8_t* wrow = w1 + size_t(nc) * size_t(K1);
+        if (wave * 16 < N1) {
+            const int n = n1, nc = nc1;
             const float c_ws = ws1 ? ws1[nc] : 1.0f;
             const int c_wsum = wsum1 ? wsum1[nc] : 0;
             const float c_bias = b1 ? b1[nc] : -0.0f;
             ml_v4i acc[4];
 #pragma unroll
             for (int rb = 0; rb < 4; ++rb) acc[rb] = ml_v4i{0, 0, 0, 0};
-            ml_v4i wf = lg * 16 < K1 ? *reinterpret_cast<const ml_v4i*>(wrow + lg * 16) : ml_v4i{0, 0, 0, 0};
-            for (int ks = 0; ks < ksteps; ++ks) {
-                const int k = ks * 64 + lg * 16, kn = k + 64;
-                const bool in_k = k < K1;  // K1 % 16 == 0: a 16-byte chunk is inside or outside as a whole
-                const ml_v4i wnext = (ks + 1 < ksteps && kn < K1) ? *reinterpret_cast<const ml_v4i*>(wrow + kn) : ml_v4i{0, 0, 0, 0};
 #pragma unroll
-                for (int rb = 0; rb < 4; ++rb) {
-                    const ml_v4i af = in_k ? *reinterpret_cast<const ml_v4i*>(codes1 + size_t(16 * rb + ln) * K1 + k)
-                                           : ml_v4i{0, 0, 0, 0};
-                    acc[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc[rb], 0, 0, 0);
+            for (int ks = 0; ks < kSteps1; ++ks) {
+                const int k = ks * 64 + lg * 16;
+                if (ks * 64 < K1) {  // uniform
+                    const bool in_k = k < K1;
+                    const ml_v4i wf = ml_place(w1f[ks]);
+#pragma unroll
+                    for (int rb = 0; rb < 4; ++rb) {
+                        const ml_v4i af = in_k ? *reinterpret_cast<const ml_v4i*>(codes1 + size_t(16 * rb + ln) * K1 + k)
+                                               : ml_v4i{0, 0, 0, 0};
+                        acc[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc[rb], 0, 0, 0);
+                    }
                 }
-                wf = wnext;
             }
             // acc[rb][q]: activation row 16 rb + 4 (lane / 16) + q, weight row n
             const int corr = (wsum1 != nullptr && zp != 0) ? zp * c_wsum : 0;
@@ -986,24 +1028,22 @@ __global__ __launch_bounds__(1024) void dynamic_mlp2_small_kernel(
     __syncthreads();
     // ---- layer 2: GEMM, one wavefront per 16 x 16 output tile
     {
-        const int rb = wave & 3, cb = wave >> 2;
+        const int rb = rb2, cb = cb2;
         if (cb * 16 < N2 && rb * 16 < M) {
             const int zp = int(z2) + off;
-            const int n = cb * 16 + ln;
-            const int nc = n < N2 ? n : N2 - 1;
-            const int8_t* wrow = w2 + size_t(nc) * size_t(N1);
+            const int n = n2, nc = nc2;
             const float c_ws = ws2 ? ws2[nc] : 1.0f;
             const int c_wsum = wsum2 ? wsum2[nc] : 0;
             const float c_bias = b2 ? b2[nc] : -0.0f;
             ml_v4i acc = ml_v4i{0, 0, 0, 0};
-            const int ksteps = (N1 + 63) >> 6;
-            for (int ks = 0; ks < ksteps; ++ks) {
+#pragma unroll
+            for (int ks = 0; ks < kSteps2; ++ks) {
                 const int k = ks * 64 + lg * 16;
-                const bool in_k = k < N1;
-                const ml_v4i wf = in_k ? *reinterpret_cast<const ml_v4i*>(wrow + k) : ml_v4i{0, 0, 0, 0};
-                const ml_v4i af = in_k ? *reinterpret_cast<const ml_v4i*>(codes2 + size_t(16 * rb + ln) * N1 + k)
-                                       : ml_v4i{0, 0, 0, 0};
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc, 0, 0, 0);
+                if (ks * 64 < N1) {  // uniform
+                    const ml_v4i af = k < N1 ? *reinterpret_cast<const ml_v4i*>(codes2 + size_t(16 * rb + ln) * N1 + k)
+                                             : ml_v4i{0, 0, 0, 0};
+                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, ml_place(w2f[ks]), acc, 0, 0, 0);
+                }
             }
             const int corr = (wsum2 != nullptr && zp != 0) ? zp * c_wsum : 0;
             const float sc = s2 * c_ws;

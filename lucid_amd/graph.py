@@ -50,8 +50,17 @@ class Graph:
             pass
 
 
+_captures_open = 0
+
+
+def is_capturing() -> bool:
+    """True inside a ``capture()`` block of this module (what is launched now will be replayed)."""
+    return _captures_open > 0
+
+
 @contextlib.contextmanager
 def capture():
+    global _captures_open
     _C.init()
     g = Graph()
     stream = C.c_void_p()
@@ -63,10 +72,12 @@ def capture():
     _C.call("lq_graph_begin", stream, C.byref(gid))
     _C.set_current_stream(stream)
     ok = False
+    _captures_open += 1
     try:
         yield g
         ok = True
     finally:
+        _captures_open -= 1
         _C.set_current_stream(prev)
         try:
             _C.call("lq_graph_end", stream, gid.value)

@@ -29,9 +29,19 @@ class Identity(Module):
 def _fused_dynamic_pair(mods, i, x):
     """``(result, next index)`` when the modules at ``i`` are Linear [, ReLU], Linear from
     ``nn.quantized.dynamic`` on an activation small enough for the one-launch kernel, else ``None``
-    (no hooks on the modules: a hook has to see each module's own output)."""
-    from .quantized.dynamic import linear as _dyn
+    (no hooks on the modules: a hook has to see each module's own output).
 
+    Not while a graph is being captured.  The one launch is one block on one CU (21 us for
+    784-256-10 at batch 64: that CU's vector units quantize all 50 k inputs), the two separate
+    layers are two launches of many blocks (8 + 6 us).  Launched from Python the one launch wins,
+    27 against 53 us per forward, because each launch costs the host about as much as it runs; a
+    replayed graph pays its ~11 us once whichever it holds, and there the shorter kernels win,
+    25 against 33 us.  Same bits either way."""
+    from .quantized.dynamic import linear as _dyn
+    from .. import graph as _graph
+
+    if _graph.is_capturing():
+        return None
     first = mods[i]
     if type(first) is not _dyn.Linear or i + 1 >= len(mods):
         return None

@@ -612,3 +612,23 @@ def test_two_dynamic_linears_keep_separate_launches_when_hooked_or_large():
     with _recorded_calls() as calls:
         assert big(x).shape == (4, 8)
     assert "lq_dynamic_mlp2_small_f32" not in calls and len(calls) >= 2
+
+
+def test_two_dynamic_linears_are_captured_as_separate_launches_with_the_same_bits():
+    """Under graph capture the pair is not fused (two launches of many blocks replay sooner than one
+    block on one CU); the replayed result equals the eager, fused one bit for bit."""
+    rng = np.random.default_rng(5)
+    model = Q.quantize_dynamic(nn.Sequential(nn.Linear(784, 256), nn.ReLU(), nn.Linear(256, 10)))
+    x = hip(rng.standard_normal((64, 784)).astype(np.float32))
+    with _recorded_calls() as calls:
+        eager = model(x).numpy()
+    assert calls == ["lq_dynamic_mlp2_small_f32"]
+    with L.graph.capture() as g:
+        with _recorded_calls() as calls:
+            y = model(x)
+    assert "lq_dynamic_mlp2_small_f32" not in calls and calls.count("lq_dynamic_linear_small_f32") == 2
+    for _ in range(3):
+        g.replay()
+        L.synchronize()
+        assert np.array_equal(y.numpy().view(np.uint32), eager.view(np.uint32))
+    g.destroy()
