@@ -453,67 +453,128 @@ __global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__
 // most 208 tokens.  qkv is the packed activation [B, T, 3, H, 64] of the qkv
 // Linear; out is [B, T, H*64].
 //
-// Per wavefront: S^T = K . Q^T as 13 tiles of 16 keys x 16 queries
-// (v_mfma_f32_16x16x4_f32, accumulators stay in registers), softmax over the
-// keys of each query (a lane holds 52 of a query's keys, the other three lane
-// groups the rest), then O = P . V where the S^T accumulators ARE the A
-// operand: register r of a tile holds P[query = lane%16][key = 16t + 4*(lane/16) + r],
-// which is a valid k-slice assignment as long as V is read with the same one.
-constexpr int AT_D = 64, AT_TMAX = 208, AT_LD = AT_D + 4;  // row stride 68: 4*row + k hits all 64 banks
+// float32 operands on the bfloat16 matrix instruction.  A float32 is the exact sum of three
+// bfloat16 values (8 + 8 + 8 significant bits: at_split3x2), and a product a * b keeps 2^-24
+// relative accuracy with six of the nine part products (hi.hi, hi.mid, mid.hi, hi.lo, lo.hi,
+// mid.mid; the three left out are below 2^-24 of |a b|).  Part products are exact in float32
+// and accumulate in float32, so each dot product is as accurate as a float32 one, and
+// v_mfma_f32_16x16x32_bf16 runs sixteen times the rate of v_mfma_f32_16x16x4_f32: six
+// instructions of the one replace eight of the other at a sixth of the time each.
+//
+// Per wavefront: S^T = K . Q^T as 13 tiles of 16 keys x 16 queries (accumulators stay in
+// registers; K's three parts in LDS, split once per block), softmax over the keys of each
+// query (a lane holds 52 of a query's keys, the other three lane groups the rest), then
+// O = P . V where the S^T accumulators ARE the A operand: register r of tile t holds
+// P[query = lane%16][key = 16t + 4*(lane/16) + r], so two tiles give a lane the eight k slots
+// of an instruction, which is a valid k-slice assignment as long as V is read with the same
+// one: V^T's three parts replace K's in LDS after the scores ([column][key], so that a lane's
+// four keys of a tile are 8 contiguous bytes).
+constexpr int AT_D = 64, AT_TMAX = 208;
+constexpr int AT_KLD = AT_D + 8;          // bfloat16 per K row: 144 bytes, the 16 rows of a fragment on 16 bank groups
+constexpr int AT_KEYS = AT_TMAX + 16;     // keys of V^T: tiles pair up, the fourteenth is zero
+constexpr int AT_VLD = AT_KEYS + 4;       // bfloat16 per V^T row: 456 bytes
+constexpr int AT_PART_K = AT_TMAX * AT_KLD, AT_PART_V = AT_D * AT_VLD;  // elements of one part
+constexpr size_t AT_SMEM = size_t(3) * (AT_PART_K > AT_PART_V ? AT_PART_K : AT_PART_V) * 2;
+
+typedef __bf16 at_v8bf __attribute__((ext_vector_type(8)));
+
+// (e0, e1) = h + m + l part by part, each part a pair of bfloat16 (e0's in the low half): the
+// packed conversion rounds to nearest, the remainders are exact (8 + 8 + 8 significant bits with
+// signed remainders).  A NaN stays a NaN in every part; an infinity turns into a NaN in the
+// lower parts, so a non-finite input gives a non-finite output.
+typedef __bf16 at_bf2 __attribute__((ext_vector_type(2)));
+typedef float at_f2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t at_pk(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(at_f2{a, b}, at_bf2));
+}
+__device__ __forceinline__ void at_split3x2(float e0, float e1, uint32_t& h, uint32_t& m, uint32_t& l) {
+    h = at_pk(e0, e1);
+    e0 -= __uint_as_float(h << 16), e1 -= __uint_as_float(h & 0xffff0000u);
+    m = at_pk(e0, e1);
+    e0 -= __uint_as_float(m << 16), e1 -= __uint_as_float(m & 0xffff0000u);
+    l = at_pk(e0, e1);
+}
+
+// acc += a * b from the parts, smallest terms first
+__device__ __forceinline__ v4f at_mma6(const uint4 (&a)[3], const uint4 (&b)[3], v4f acc) {
+    auto mm = [&](const uint4& x, const uint4& y) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(at_v8bf, x), __builtin_bit_cast(at_v8bf, y), acc,
+                                                      0, 0, 0);
+    };
+    mm(a[1], b[1]);
+    mm(a[0], b[2]);
+    mm(a[2], b[0]);
+    mm(a[0], b[1]);
+    mm(a[1], b[0]);
+    mm(a[0], b[0]);
+    return acc;
+}
 
 __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict__ qkv, float* __restrict__ out,
                                                         int B, int T, int H, float scale, float* range) {
-    extern __shared__ __attribute__((aligned(16))) float at_smem[];
-    float (*sk)[AT_LD] = reinterpret_cast<float (*)[AT_LD]>(at_smem);
-    float (*sv)[AT_LD] = reinterpret_cast<float (*)[AT_LD]>(at_smem + AT_TMAX * AT_LD);
+    extern __shared__ __attribute__((aligned(16))) uint16_t at_smem[];
     const int b = blockIdx.x / H, h = blockIdx.x % H;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int nwaves = blockDim.x >> 6;
     const size_t tok_stride = size_t(3) * H * AT_D;
     const float* base = qkv + size_t(b) * T * tok_stride + size_t(h) * AT_D;
-    // K and V rows into LDS (rows past T are zero)
-    for (int i = tid; i < AT_TMAX * (AT_D / 4); i += blockDim.x) {
-        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
-        float4 kv = {0.f, 0.f, 0.f, 0.f}, vv = {0.f, 0.f, 0.f, 0.f};
-        if (row < T) {
-            const float* p = base + size_t(row) * tok_stride + c4;
-            kv = *reinterpret_cast<const float4*>(p + size_t(H) * AT_D);
-            vv = *reinterpret_cast<const float4*>(p + size_t(2) * H * AT_D);
-        }
-        *reinterpret_cast<float4*>(&sk[row][c4]) = kv;
-        *reinterpret_cast<float4*>(&sv[row][c4]) = vv;
+    // V is requested now (up to four 16-byte pieces per thread: all of it for 13 wavefronts) and laid
+    // out after the scores
+    constexpr int kPieces = AT_TMAX * (AT_D / 4), kHeld = 4;
+    float4 vheld[kHeld];
+#pragma unroll
+    for (int u = 0; u < kHeld; ++u) {
+        const int i = tid + u * int(blockDim.x), row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        vheld[u] = float4{0.f, 0.f, 0.f, 0.f};
+        if (i < kPieces && row < T) vheld[u] = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(2) * H * AT_D + c4);
     }
-    __syncthreads();
+    // K rows into LDS as three bfloat16 parts (rows past T are zero)
+    for (int i = tid; i < kPieces; i += blockDim.x) {
+        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        float4 kv = {0.f, 0.f, 0.f, 0.f};
+        if (row < T) kv = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(H) * AT_D + c4);
+        uint32_t lo[3], hi[3];
+        at_split3x2(kv.x, kv.y, lo[0], lo[1], lo[2]);
+        at_split3x2(kv.z, kv.w, hi[0], hi[1], hi[2]);
+#pragma unroll
+        for (int p = 0; p < 3; ++p)
+            *reinterpret_cast<uint2*>(at_smem + p * AT_PART_K + row * AT_KLD + c4) = uint2{lo[p], hi[p]};
+    }
     const int q0 = wave * 16;  // the launch has exactly ceil(T / 16) wavefronts, so q0 < T
-    (void)nwaves;
     const int g = lane >> 4, c = lane & 15;
-    // B operand of S^T: Q[q0 + c][4*s + g], pre-scaled so that S = scale * log2(e) * Q.K^T
-    float qf[AT_D / 4];
+    // B operand of S^T: Q[q0 + c][32 u + 8 g + 0..7], pre-scaled so that S = scale * log2(e) * Q.K^T
+    // (the scores are kept in the base-2 domain, so that the softmax numerators are one v_exp_f32 each)
+    uint4 qf[AT_D / 32][3];
     {
         const int q = q0 + c;
         const float* qp = base + size_t(q < T ? q : T - 1) * tok_stride;
+        const float qs = scale * 1.4426950408889634f;
 #pragma unroll
-        // (scale * log2 e: the scores are kept in the base-2 domain, so that the softmax
-        // numerators are one v_exp_f32 each: 2^(s - max) = e^((s - max) ln 2))
-        // MFMA s carries k = 16 (s / 4) + 4 g + s % 4 in lane group g: a lane's four consecutive
-        // instructions then need four consecutive floats of a K row - one 16-byte LDS read
-        for (int s = 0; s < AT_D / 4; ++s) qf[s] = qp[16 * (s >> 2) + 4 * g + (s & 3)] * (scale * 1.4426950408889634f);
+        for (int u = 0; u < AT_D / 32; ++u) {
+            const float4 a = *reinterpret_cast<const float4*>(qp + 32 * u + 8 * g);
+            const float4 bq = *reinterpret_cast<const float4*>(qp + 32 * u + 8 * g + 4);
+            const float v[8] = {a.x * qs, a.y * qs, a.z * qs, a.w * qs, bq.x * qs, bq.y * qs, bq.z * qs, bq.w * qs};
+            uint32_t d[3][4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) at_split3x2(v[2 * e], v[2 * e + 1], d[0][e], d[1][e], d[2][e]);
+#pragma unroll
+            for (int p = 0; p < 3; ++p) qf[u][p] = uint4{d[p][0], d[p][1], d[p][2], d[p][3]};
+        }
     }
+    __syncthreads();
     constexpr int NT = AT_TMAX / 16;
     v4f st[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) st[t] = v4f{0.f, 0.f, 0.f, 0.f};
-    // k slice outermost: the 13 tiles' accumulators are independent chains, so consecutive MFMAs never
-    // wait for each other (per tile the order of the k slices - and with it every bit - is unchanged)
+    // k slice outermost: the 13 tiles' accumulators are independent chains
 #pragma unroll
-    for (int u = 0; u < AT_D / 16; ++u)
+    for (int u = 0; u < AT_D / 32; ++u)
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const float4 kv = *reinterpret_cast<const float4*>(&sk[16 * t + c][16 * u + 4 * g]);
-            st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.x, qf[4 * u + 0], st[t], 0, 0, 0);
-            st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.y, qf[4 * u + 1], st[t], 0, 0, 0);
-            st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.z, qf[4 * u + 2], st[t], 0, 0, 0);
-            st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.w, qf[4 * u + 3], st[t], 0, 0, 0);
+            uint4 kf[3];
+#pragma unroll
+            for (int p = 0; p < 3; ++p)
+                kf[p] = *reinterpret_cast<const uint4*>(at_smem + p * AT_PART_K + (16 * t + c) * AT_KLD + 32 * u + 8 * g);
+            st[t] = at_mma6(kf, qf[u], st[t]);
         }
     // st[t][r] = S[query q0 + c][key 16t + 4g + r]
     float mx = -__builtin_inff();
@@ -539,23 +600,71 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
     const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
-    // O[q][n] = sum_key P[q][key] V[key][n], four 16-wide column tiles
+
+    // V^T's parts take K's place: [column][key], keys past T (and the fourteenth tile) zero
+    __syncthreads();  // every wavefront has read its K fragments
+    for (int i = tid; i < 3 * AT_D * (AT_KEYS - AT_TMAX) / 2; i += blockDim.x) {
+        const int p = i / (AT_D * (AT_KEYS - AT_TMAX) / 2), rest = i % (AT_D * (AT_KEYS - AT_TMAX) / 2);
+        const int n = rest / ((AT_KEYS - AT_TMAX) / 2), k2 = rest % ((AT_KEYS - AT_TMAX) / 2);
+        *reinterpret_cast<uint32_t*>(at_smem + p * AT_PART_V + n * AT_VLD + AT_TMAX + 2 * k2) = 0u;
+    }
+    auto place_v = [&](int i, float4 vv) {
+        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        uint32_t lo[3], hi[3];
+        at_split3x2(vv.x, vv.y, lo[0], lo[1], lo[2]);
+        at_split3x2(vv.z, vv.w, hi[0], hi[1], hi[2]);
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+            uint16_t* col = at_smem + p * AT_PART_V + c4 * AT_VLD + row;
+            col[0] = uint16_t(lo[p]), col[AT_VLD] = uint16_t(lo[p] >> 16);
+            col[2 * AT_VLD] = uint16_t(hi[p]), col[3 * AT_VLD] = uint16_t(hi[p] >> 16);
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < kHeld; ++u) {
+        const int i = tid + u * int(blockDim.x);
+        if (i < kPieces) place_v(i, vheld[u]);
+    }
+    for (int i = tid + kHeld * int(blockDim.x); i < kPieces; i += blockDim.x) {  // fewer than 13 wavefronts
+        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        float4 vv = {0.f, 0.f, 0.f, 0.f};
+        if (row < T) vv = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(2) * H * AT_D + c4);
+        place_v(i, vv);
+    }
+    __syncthreads();
+
+    // O[q][n] = sum_key P[q][key] V[key][n], four 16-wide column tiles; tile j of the output holds
+    // head-dim columns 4 c + j (not 16 j + c), so that a lane stores four consecutive floats
     v4f o[AT_D / 16];
 #pragma unroll
     for (int j = 0; j < AT_D / 16; ++j) o[j] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    // tile j of the output holds head-dim columns 4 c + j (not 16 j + c): a lane's four tiles then take four
-    // consecutive floats of a V row - one 16-byte LDS read - and store four consecutive floats
-    for (int t = 0; t < NT; ++t)
+    for (int tp = 0; tp < (NT + 1) / 2; ++tp) {
+        // the eight k slots of this lane: keys 32 tp + 4 g + 0..3 and 32 tp + 16 + 4 g + 0..3
+        float pv[8];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float p = st[t][r] * inv;
-            const float4 vv = *reinterpret_cast<const float4*>(&sv[16 * t + 4 * g + r][4 * c]);
-            o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, vv.x, o[0], 0, 0, 0);
-            o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, vv.y, o[1], 0, 0, 0);
-            o[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, vv.z, o[2], 0, 0, 0);
-            o[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(p, vv.w, o[3], 0, 0, 0);
+            pv[r] = st[2 * tp][r] * inv;
+            pv[4 + r] = 2 * tp + 1 < NT ? st[2 * tp + 1 < NT ? 2 * tp + 1 : 0][r] * inv : 0.0f;
         }
+        uint32_t d[3][4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) at_split3x2(pv[2 * e], pv[2 * e + 1], d[0][e], d[1][e], d[2][e]);
+        uint4 pf[3];
+#pragma unroll
+        for (int p = 0; p < 3; ++p) pf[p] = uint4{d[p][0], d[p][1], d[p][2], d[p][3]};
+#pragma unroll
+        for (int j = 0; j < AT_D / 16; ++j) {
+            uint4 vf[3];
+#pragma unroll
+            for (int p = 0; p < 3; ++p) {
+                const uint16_t* vrow = at_smem + p * AT_PART_V + (4 * c + j) * AT_VLD + 32 * tp + 4 * g;
+                const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
+                vf[p] = uint4{lo.x, lo.y, hi.x, hi.y};
+            }
+            o[j] = at_mma6(pf, vf, o[j]);
+        }
+    }
     // result layout of the 16x16 MFMA: column slot = lane % 16, row = 4*(lane/16) + r
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -715,7 +824,7 @@ int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, f
     LQ_REQUIRE(range == nullptr || long(B) * H <= kRangeSlots, LQ_ERR_SHAPE,
                "attention: too many (batch, head) pairs for a kept range");
     const int waves = (T + 15) / 16;
-    constexpr size_t kSmem = size_t(2) * AT_TMAX * AT_LD * sizeof(float);
+    constexpr size_t kSmem = AT_SMEM;
     static DeviceOnce attr_once;
     if (int rc = allow_dynamic_lds(attr_once, reinterpret_cast<const void*>(attention_kernel), int(kSmem))) return rc;
     attention_kernel<<<unsigned(B) * H, waves * 64, kSmem, as_stream(stream)>>>(qkv, out, B, T, H, scale,
