@@ -636,9 +636,10 @@ typedef struct {
                               K % 64 == 0), 17 = 256x352 tiles with one wavefront per SIMD
                               (plain GEMM, K % 128 == 0, K >= 256, float16 output or raw
                               accumulators; never chosen automatically),
-                              15 (convolutions only) = one block per box of 256 output
-                              positions x 64 channels with the box's input halo held in
-                              LDS (stride 1, Cin/groups % 64 == 0, no join);
+                              15 / 18 / 19 (convolutions only) = one block per box of
+                              256 / 128 / 64 output positions x 64 channels with the box's
+                              input halo held in LDS (stride 1, Cin/groups % 64 == 0, no
+                              join);
                               next byte 0 = choose, 1 = one block per tile,
                               2 = stream-K work split, 3 = stream-K over the
                               leftover tiles of the last round only; bits 16..30

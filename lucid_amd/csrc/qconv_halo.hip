@@ -1,5 +1,5 @@
 // Stride-1 int8 convolution (2-d or volumetric) on channels-last codes with the input held in
-// LDS: a block owns a box of 256 output positions and 64 output channels, loads the box's
+// LDS: a block owns a box of 256 (or 128, or 64) output positions and 64 output channels, loads the box's
 // input halo - (TD + (KD-1) dd) x (TH + (KH-1) dh) x (TW + (KW-1) dw) positions x 64 channels -
 // into LDS ONCE per 64-channel slice, and takes the A fragments of every filter tap from it
 // at a shifted row.  The gather of the tile GEMM's loader fetches every input position once
@@ -9,8 +9,10 @@
 //   LDS: halo rows of 64 bytes (one position's 64 channels), 16-byte chunk kc of row r at
 //        physical chunk kc ^ ((r/2) % 4); then NB stages of 64 filter rows x 64 bytes, same
 //        placement; then the block's 64 column parameter sets.
-//   wavefront w: positions 64w .. 64w+63 of the box (w fastest, then h, then d) x 64 channels,
-//        16 accumulator tiles of v_mfma_i32_16x16x64_i8 with the filter fragment as the first
+//   wavefront w: positions 16 TI w .. 16 TI (w+1) - 1 of the box (w fastest, then h, then d) x 64
+//        channels (TI = 4, 2 or 1 tiles of 16 positions: boxes of 256, 128 or 64 positions - the
+//        smaller boxes are for layers with too few positions to give 256 CUs a 256-position box
+//        each), TI x 4 accumulator tiles of v_mfma_i32_16x16x64_i8 with the filter fragment as the first
 //        operand, so a lane holds four consecutive output channels of one position and the
 //        epilogue runs on registers (the helpers of qepilogue.hpp: same bits as the tile kernel).
 #include "common.hpp"
@@ -33,7 +35,7 @@ constexpr int kRing = 6;  // filter stages in the ring
 struct HaloGeom {
     int D, H, W, OD, OH, OW;     // input and output extents (D = OD = 1 for a 2-d layer)
     int KD, KH, KW, pd, ph, pw, dd, dh, dw;
-    int ltd, lth, ltw;           // log2 of the box extents; their product is 256
+    int ltd, lth, ltw;           // log2 of the box extents; their product is the box (256, 128 or 64)
     int HD, HH, HW;              // halo extents
     int halo_rows;               // HD * HH * HW rounded up to a multiple of 64
     int tiles_d, tiles_h, tiles_w;
@@ -42,7 +44,7 @@ struct HaloGeom {
     int inv_hw, inv_hh;          // 2^20 / HW + 1, 2^20 / HH + 1
 };
 
-template <int MODE>
+template <int MODE, int TI>
 __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom q) {
     extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -100,10 +102,10 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
 
     // ---- LDS -> registers: lane l of a 16 x 64 fragment holds row l%16, logical chunk l/16
     const int fr = lane & 15, fc = lane >> 4;
-    int a_row[4];  // halo row of the lane's position in each of the wavefront's four 16-row tiles, tap (0, 0, 0)
+    int a_row[TI];  // halo row of the lane's position in each of the wavefront's 16-row tiles, tap (0, 0, 0)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int v = wave * 64 + i * 16 + fr;
+    for (int i = 0; i < TI; ++i) {
+        const int v = wave * (16 * TI) + i * 16 + fr;
         const int vw = v & ((1 << q.ltw) - 1), vh = (v >> q.ltw) & ((1 << q.lth) - 1), vd = v >> (q.ltw + q.lth);
         a_row[i] = (vd * q.HH + vh) * q.HW + vw;
     }
@@ -113,9 +115,9 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
         const int r = j * 16 + fr;
         b_off[j] = r * 64 + ((fc ^ ((r >> 1) & 3)) << 4);
     }
-    hv4i acc[4][4];
+    hv4i acc[TI][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = hv4i{0, 0, 0, 0};
 
@@ -124,11 +126,11 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
     if (tid < 64) c_mine = load_col(g, grp * Og + (n0 + tid < Og ? n0 + tid : Og - 1));
 
     // fragments of tap (kd, kh, kw), whose filter rows sit in ring stage `stage`
-    auto read_frags = [&](int kd, int kh, int kw, int stage, hv4i (&af)[4], hv4i (&bf)[4]) {
+    auto read_frags = [&](int kd, int kh, int kw, int stage, hv4i (&af)[TI], hv4i (&bf)[4]) {
         const int toff = ((kd * q.dd) * q.HH + kh * q.dh) * q.HW + kw * q.dw;
         const int8_t* st = ring + stage * 4096;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < TI; ++i) {
             const int hr = a_row[i] + toff;
             af[i] = *reinterpret_cast<const hv4i*>(halo + hr * 64 + ((fc ^ ((hr >> 1) & 3)) << 4));
         }
@@ -144,7 +146,7 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
     // One tap: wait for the NEXT tap's filter stage, meet the other wavefronts (they have all
     // consumed the stage that is refilled now), request the stage kRing-1 taps ahead, read the
     // next tap's fragments into the other register set, and issue this tap's MFMAs on top of them.
-    auto tap_step = [&](int cb, int tp, int& kd, int& kh, int& kw, hv4i (&af)[4], hv4i (&bf)[4], hv4i (&an)[4],
+    auto tap_step = [&](int cb, int tp, int& kd, int& kh, int& kw, hv4i (&af)[TI], hv4i (&bf)[4], hv4i (&an)[TI],
                         hv4i (&bn)[4]) {
         if (tp + 1 < taps) {
             if (tp + kRing - 1 <= taps)
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < TI; ++i)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
     };
 
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
         __builtin_amdgcn_s_waitcnt(halo_vmcnt_imm(0));
         __syncthreads();
         int kd = 0, kh = 0, kw = 0;
-        hv4i a0[4], b0[4], a1[4], b1[4];
+        hv4i a0[TI], b0[4], a1[TI], b1[4];
         read_frags(0, 0, 0, 0, a0, b0);
         int tp = 0;
         for (; tp + 1 < taps; tp += 2) {
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
         if (tp < taps) tap_step(cb, tp, kd, kh, kw, a0, b0, a1, b1);
     }
 
-    // ---- epilogue on registers.  acc[i][j][r]: position 64 wave + 16 i + lane%16 of the box,
+    // ---- epilogue on registers.  acc[i][j][r]: position 16 TI wave + 16 i + lane%16 of the box,
     // column n0 + 16 j + 4 (lane/16) + r of the group.
     float S = 1.0f, Z = 0.0f;
     constexpr bool kRequant = MODE == OUT_REQUANT_I8 || MODE == OUT_FAKEQUANT_F32;
@@ -201,10 +203,10 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
     const bool prescaled = MODE == OUT_REQUANT_I8;
     const bool cols_in = n0 + 64 <= Og;
     const bool vec_out = cols_in && g.ldo % 4 == 0 && Og % 4 == 0 && reinterpret_cast<uintptr_t>(g.out) % (4 * esize) == 0;
-    long m_row[4];  // output row (position index over the whole batch) of each tile's lane row, -1 outside
+    long m_row[TI];  // output row (position index over the whole batch) of each tile's lane row, -1 outside
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int v = wave * 64 + i * 16 + fr;
+    for (int i = 0; i < TI; ++i) {
+        const int v = wave * (16 * TI) + i * 16 + fr;
         const int vw = v & ((1 << q.ltw) - 1), vh = (v >> q.ltw) & ((1 << q.lth) - 1), vd = v >> (q.ltw + q.lth);
         const int od = od0 + vd, oh = oh0 + vh, ow = ow0 + vw;
         m_row[i] = (od < q.OD && oh < q.OH && ow < q.OW) ? (long((b * q.OD + od) * q.OH + oh) * q.OW + ow) : -1;
@@ -223,7 +225,7 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
         }
         const int nq = grp * Og + n0 + cl;  // global column of the lane's first value
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < TI; ++i) {
             if (m_row[i] < 0) continue;
             const hv4i a = acc[i][j];
             uint4 v;
@@ -253,9 +255,9 @@ __global__ __launch_bounds__(256, 2) void qconv_halo_kernel(GemmArgs g, HaloGeom
     }
 }
 
-template <int MODE>
+template <int MODE, int TI>
 int launch_mode(const GemmArgs& g, const HaloGeom& q, dim3 grid, size_t lds, hipStream_t st) {
-    const void* fn = reinterpret_cast<const void*>(qconv_halo_kernel<MODE>);
+    const void* fn = reinterpret_cast<const void*>(qconv_halo_kernel<MODE, TI>);
     static DeviceOnce attr_once;
     if (int rc = allow_dynamic_lds(attr_once, fn, 96 * 1024)) return rc;
     GemmArgs gc = g;
@@ -276,8 +278,9 @@ int ilog2(int v) {
 namespace lq {
 
 // Whether the halo kernel can run the convolution described by g (conv = 1: NHWC, 2: NDHWC
-// geometry in the c* fields; N = output channels of one group), and with which box.
-static bool plan_halo(const GemmArgs& g, int conv, HaloGeom* out) {
+// geometry in the c* fields; N = output channels of one group) with boxes of 2^lbox positions,
+// and with which box.
+static bool plan_halo(const GemmArgs& g, int conv, int lbox, HaloGeom* out) {
     if (conv != 1 && conv != 2) return false;
     HaloGeom q{};
     const bool vol = conv == 2;
@@ -302,11 +305,11 @@ static bool plan_halo(const GemmArgs& g, int conv, HaloGeom* out) {
     if (!aligned16(g.cx) || !aligned16(g.w)) return false;
     q.cblocks = Cg / 64;
     q.n_tiles = (g.N + 63) / 64;
-    // the box: powers of two with product 256; fewest boxes first, then the smallest halo, then the widest rows
+    // the box: powers of two with product 2^lbox; fewest boxes first, then the smallest halo, then the widest rows
     long best_cost = -1;
-    for (int ltw = 0; ltw <= 8; ++ltw)
-        for (int lth = 0; ltw + lth <= 8; ++lth) {
-            const int ltd = 8 - ltw - lth;
+    for (int ltw = 0; ltw <= lbox; ++ltw)
+        for (int lth = 0; ltw + lth <= lbox; ++lth) {
+            const int ltd = lbox - ltw - lth;
             const int tw = 1 << ltw, th = 1 << lth, td = 1 << ltd;
             if (td > 1 && !vol) continue;
             if (tw < 8 && q.OW >= 8) continue;  // fragment rows should be runs of consecutive halo rows
@@ -329,14 +332,14 @@ static bool plan_halo(const GemmArgs& g, int conv, HaloGeom* out) {
     return true;
 }
 
-bool conv_halo_applies(const GemmArgs& g, int conv) {
+bool conv_halo_applies(const GemmArgs& g, int conv, int lbox) {
     HaloGeom q;
-    return plan_halo(g, conv, &q);
+    return (lbox == 8 || lbox == 7 || lbox == 6) && plan_halo(g, conv, lbox, &q);
 }
 
-int launch_conv_halo(const GemmArgs& g, int conv, int groups, hipStream_t st) {
+int launch_conv_halo(const GemmArgs& g, int conv, int groups, int lbox, hipStream_t st) {
     HaloGeom q;
-    LQ_REQUIRE(plan_halo(g, conv, &q), LQ_ERR_NOT_IMPLEMENTED,
+    LQ_REQUIRE(conv_halo_applies(g, conv, lbox) && plan_halo(g, conv, lbox, &q), LQ_ERR_NOT_IMPLEMENTED,
                "halo convolution: needs stride 1, Cin/groups %% 64 == 0, no join and a halo of at most 1024 positions");
     const long batch = long(g.M) / (long(q.OD) * q.OH * q.OW);
     const long boxes = batch * q.tiles_d * q.tiles_h * q.tiles_w;
@@ -344,13 +347,21 @@ int launch_conv_halo(const GemmArgs& g, int conv, int groups, hipStream_t st) {
                "halo convolution: grid too large");
     const dim3 grid{unsigned(boxes), unsigned(q.n_tiles * groups)};
     const size_t lds = size_t(q.halo_rows) * 64 + kRing * 4096 + 3 * 64 * 4;
-    switch (g.out_mode) {
-    case OUT_ACC_I32: return launch_mode<OUT_ACC_I32>(g, q, grid, lds, st);
-    case OUT_F32: return launch_mode<OUT_F32>(g, q, grid, lds, st);
-    case OUT_F16: return launch_mode<OUT_F16>(g, q, grid, lds, st);
-    case OUT_REQUANT_I8: return launch_mode<OUT_REQUANT_I8>(g, q, grid, lds, st);
-    default: return launch_mode<OUT_FAKEQUANT_F32>(g, q, grid, lds, st);
+#define LQ_HALO_MODES(TI)                                                                   \
+    switch (g.out_mode) {                                                                   \
+    case OUT_ACC_I32: return launch_mode<OUT_ACC_I32, TI>(g, q, grid, lds, st);             \
+    case OUT_F32: return launch_mode<OUT_F32, TI>(g, q, grid, lds, st);                     \
+    case OUT_F16: return launch_mode<OUT_F16, TI>(g, q, grid, lds, st);                     \
+    case OUT_REQUANT_I8: return launch_mode<OUT_REQUANT_I8, TI>(g, q, grid, lds, st);       \
+    default: return launch_mode<OUT_FAKEQUANT_F32, TI>(g, q, grid, lds, st);                \
     }
+    if (lbox == 8) {
+        LQ_HALO_MODES(4)
+    } else if (lbox == 7) {
+        LQ_HALO_MODES(2)
+    }
+    LQ_HALO_MODES(1)
+#undef LQ_HALO_MODES
 }
 
 }  // namespace lq

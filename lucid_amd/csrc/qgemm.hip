@@ -66,8 +66,8 @@ int launch_tile_c11(const GemmArgs&, int, int, int, hipStream_t);
 int launch_tile_c12(const GemmArgs&, int, int, int, hipStream_t);
 int launch_pp_shape(const GemmArgs&, int, hipStream_t);
 int launch_bw_shape(const GemmArgs&, int, hipStream_t);
-bool conv_halo_applies(const GemmArgs&, int conv);
-int launch_conv_halo(const GemmArgs&, int conv, int groups, hipStream_t);
+bool conv_halo_applies(const GemmArgs&, int conv, int lbox = 8);
+int launch_conv_halo(const GemmArgs&, int conv, int groups, int lbox, hipStream_t);
 }  // namespace lq
 
 namespace {
@@ -100,10 +100,12 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
         LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
         return launch_bw_shape(g, 0, st);
     case 15:
-        // stride-1 convolution with the input halo held in LDS, one block per box of outputs
-        LQ_REQUIRE(conv, LQ_ERR_VALUE, "tile_config 15 is for convolutions");
-        LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config 15 runs one block per tile");
-        return launch_conv_halo(g, conv, groups, st);
+    case 18:
+    case 19:
+        // stride-1 convolution with the input halo held in LDS, one block per box of 256 / 128 / 64 outputs
+        LQ_REQUIRE(conv, LQ_ERR_VALUE, "tile_config %d is for convolutions", cfg);
+        LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
+        return launch_conv_halo(g, conv, groups, cfg == 15 ? 8 : (cfg == 18 ? 7 : 6), st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -218,7 +220,7 @@ int tune_import_text(const char* text, int* accepted) {
         }
         if (got != kTuneKeyInts + 1) return fail(LQ_ERR_VALUE, "tune_import: malformed line '%s'", line.c_str());
         const int shape = v[kTuneKeyInts] & 0xff;
-        if (shape < 1 || shape > 17) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
+        if (shape < 1 || shape > 19) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
         TuneKey key;
         std::memcpy(&key, v, sizeof(key));
         std::lock_guard<std::mutex> lock(g_tune_mu);
@@ -316,7 +318,13 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
         if (tiles128 < 256) cands[n++] = 9;  // ... or cover the chip with 64 x 64 tiles
         if (tiles128 < 256 && g.K >= 1024) cands[n++] = 10;  // ... with 128-byte k-iterations
         // filters with several taps at stride 1: the input halo of a box of outputs held in LDS
-        if (conv && g.K > g.cCg && conv_halo_applies(g, conv)) cands[n++] = 15;
+        if (conv && g.K > g.cCg && conv_halo_applies(g, conv)) {
+            cands[n++] = 15;
+            // smaller boxes where 256-position boxes leave CUs without one
+            const long boxes256 = (long(g.M) + 255) / 256 * ((g.N + 63) / 64) * groups;
+            if (boxes256 < 1024 && conv_halo_applies(g, conv, 7)) cands[n++] = 18;
+            if (boxes256 < 512 && conv_halo_applies(g, conv, 6)) cands[n++] = 19;
+        }
         // whole rounds of 256 x 256 tiles plus a remainder (see launch_split)
         if (!conv && groups == 1 && g.range == nullptr && g.M >= 256) {
             const long tiles_m = (g.M + 255) / 256, tiles_n = g.N / 256;

@@ -396,10 +396,12 @@ HALO_CASES = [
 ]
 
 
+@pytest.mark.parametrize("cfg", [15, 18, 19])
 @pytest.mark.parametrize("case", HALO_CASES)
-def test_halo_kernel_exact(case):
-    """tile_config 15 - the stride-1 convolution that keeps a box's input halo in LDS - against
-    the oracle: accumulators, and the requantize / float32 / float16 / fake-quantize epilogues."""
+def test_halo_kernel_exact(case, cfg):
+    """tile_config 15 / 18 / 19 - the stride-1 convolution that keeps the input halo of a box of
+    256 / 128 / 64 outputs in LDS - against the oracle: accumulators, and the requantize / float32 /
+    float16 / fake-quantize epilogues."""
     B, H, W, Cin, Cout, KH, KW, pad, dil, groups = case
     rng = np.random.default_rng(sum(case[:7]) + 15)
     x = codes(rng, (B, H, W, Cin))
@@ -408,7 +410,7 @@ def test_halo_kernel_exact(case):
     geo = dict(stride=(1, 1), pad=pad, dilation=dil, groups=groups)
     xd, wd = hip(x), hip(w)
     exp = O.qconv2d(x, w, a_zp, 1.0, np.ones(Cout, np.float32), out_mode=O.OUT_ACC_I32, **geo)
-    got = _ops.qconv2d_i8(xd, wd, a_zp=a_zp, out_mode=_ops.OUT_ACC_I32, path=IMPLICIT, tile_config=15, **geo).numpy()
+    got = _ops.qconv2d_i8(xd, wd, a_zp=a_zp, out_mode=_ops.OUT_ACC_I32, path=IMPLICIT, tile_config=cfg, **geo).numpy()
     assert got.shape == exp.shape and np.array_equal(got, exp)
     a_scale = np.float32(0.02)
     w_scale = rng.uniform(0.0005, 0.004, Cout).astype(np.float32)
@@ -417,7 +419,7 @@ def test_halo_kernel_exact(case):
     S, Z = np.float32(np.abs(y).max() / 200 + 1e-6), np.float32(0.0)
     dkw = dict(a_zp=a_zp, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=_ops.rowsum_i8(wd), bias=hip(bias),
                relu=True, out_scale=hip(S), out_zp=hip(Z), out_qmin=0, out_qmax=255, out_offset=-128,
-               path=IMPLICIT, tile_config=15, **geo)
+               path=IMPLICIT, tile_config=cfg, **geo)
     for mode in (_ops.OUT_REQUANT_I8, _ops.OUT_F32, _ops.OUT_F16, _ops.OUT_FAKEQUANT_F32):
         got = _ops.qconv2d_i8(xd, wd, out_mode=mode, **dkw).numpy()
         exp = O.qconv2d(x, w, a_zp, a_scale, w_scale, bias=bias, relu=True, out_mode=mode, out_scale=S, out_zp=Z,
