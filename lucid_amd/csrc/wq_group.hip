@@ -339,7 +339,7 @@ int launch_gemv(const float* x, const uint32_t* packed, const float* scales, con
 // an 8-bit code is exact in bfloat16, a 4-bit code c is formed as the bit pattern 0x4300 | c
 // = 128 + c (one AND-OR per two codes) and the 128 goes into the bias term - and x as the
 // other, split into three bfloat16 parts x = hi + mid + lo (exact: 8 + 8 + 8 significant
-// bits), one MFMA each.  Products are exact and accumulate in float32, so nothing of x or
+// bits, wq_split3x2), one MFMA each.  Products are exact and accumulate in float32, so nothing of x or
 // of the weight is rounded before the sums.
 //
 // Operand layout of the instruction: lane = (row % 16) + 16 * quarter holds eight k of its
@@ -411,16 +411,21 @@ __device__ __forceinline__ void wq_swap16(uint32_t& a, uint32_t& b) {
     a = r[0], b = r[1];
 }
 
-// x = h + m + l with each part a bfloat16 (bit patterns in the low halves)
-__device__ __forceinline__ void wq_split3(float x, uint32_t& h, uint32_t& m, uint32_t& l) {
-    const uint32_t xb = __float_as_uint(x);
-    h = xb >> 16;  // truncated: the remainder keeps x's sign and has at most 16 significant bits
-    const float r1 = x - __uint_as_float(xb & 0xffff0000u);
-    const uint32_t rb = __float_as_uint(r1);
-    m = rb >> 16;
-    const float r2 = r1 - __uint_as_float(rb & 0xffff0000u);  // at most 8 significant bits: a bfloat16
-    l = __float_as_uint(r2) >> 16;
-    if ((xb & 0x7f800000u) == 0x7f800000u) m = l = 0;  // infinity / NaN stay in the first part alone
+// (e0, e1) = h + m + l part by part, each part a pair of bfloat16 (e0's in the low half): the
+// packed conversion rounds to nearest, the remainders are exact (8 + 8 + 8 significant bits with
+// signed remainders).  A NaN stays a NaN in every part; an infinity turns into a NaN in the
+// lower parts, so a non-finite x gives a non-finite y.
+typedef __bf16 wq_bf2 __attribute__((ext_vector_type(2)));
+typedef float wq_f2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t wq_pk(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(wq_f2{a, b}, wq_bf2));
+}
+__device__ __forceinline__ void wq_split3x2(float e0, float e1, uint32_t& h, uint32_t& m, uint32_t& l) {
+    h = wq_pk(e0, e1);
+    e0 -= __uint_as_float(h << 16), e1 -= __uint_as_float(h & 0xffff0000u);
+    m = wq_pk(e0, e1);
+    e0 -= __uint_as_float(m << 16), e1 -= __uint_as_float(m & 0xffff0000u);
+    l = wq_pk(e0, e1);
 }
 
 constexpr int kWqRows = 256;    // weight rows per block
@@ -447,7 +452,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     // the wavefront index as a scalar, so that branches on it are uniform
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, q = lane >> 4;
-    const int tile = blockIdx.x, ks = blockIdx.y, mb = blockIdx.z, slices = gridDim.y;
+    // the k ranges of a row tile are neighbours in the grid: they are dispatched together, so the pieces of a
+    // weight row (one per k range) are requested at about the same time
+    const int tile = blockIdx.y, ks = blockIdx.x, mb = blockIdx.z, slices = gridDim.x;
     const int n_base = tile * kWqRows + wave * (RB * 16), m0 = mb * 16;
     const int words_per_row = K * BITS / 32, groups_per_row = K >> gs_shift;
     const int windows = K / WK;
@@ -458,6 +465,53 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int ng = (((w0 + nw) * WK - 1) >> gs_shift) - g0 + 1;
     const int gmax = kWqSliceK >> gs_shift, gp = (gmax < 1 ? 1 : gmax) + 1;
 
+    // Every global load of the block is requested before anything is consumed, in the order of
+    // consumption (the wait counter retires loads in order): the scale / bias tables (short, from
+    // the L2), x, the weights.
+    // Tables: 256 rows x gcap slots (gcap = the groups of a full k range, 4, 8 or 16), four slots per
+    // 16-byte load where the rows allow it (a dword per lane costs the vector cache as many cycles
+    // as 16 bytes per lane do).
+    constexpr int kTabVec = kWqRows * 16 / 4 / 512;  // 16-byte loads per thread and table, at 16 groups per k range
+    const int gcap = gp - 1, gsh = 31 - __builtin_clz(unsigned(gcap));  // a power of two: shifts, no division
+    const bool tab_vec = ng == gcap && (groups_per_row & 3) == 0 && aligned16(scales) && aligned16(biases);
+    float4 tab_s[kTabVec], tab_b[kTabVec];
+    {
+        const int row_first = tile * kWqRows;
+#pragma unroll
+        for (int u = 0; u < kTabVec; ++u) {
+            const int i = (threadIdx.x + u * 512) * 4, row = i >> gsh, g = i & (gcap - 1);
+            tab_s[u] = tab_b[u] = float4{0.f, 0.f, 0.f, 0.f};
+            if (i < kWqRows * gcap) {
+                const int n = row_first + row < N ? row_first + row : N - 1;
+                const size_t at = size_t(n) * groups_per_row + g0 + g;
+                if (tab_vec) {
+                    tab_s[u] = *reinterpret_cast<const float4*>(scales + at);
+                    tab_b[u] = *reinterpret_cast<const float4*>(biases + at);
+                } else {
+                    // ragged: the last k range of a K that is not a multiple of 512, or unaligned rows
+                    if (g < ng) tab_s[u].x = scales[at], tab_b[u].x = biases[at];
+                    if (g + 1 < ng) tab_s[u].y = scales[at + 1], tab_b[u].y = biases[at + 1];
+                    if (g + 2 < ng) tab_s[u].z = scales[at + 2], tab_b[u].z = biases[at + 2];
+                    if (g + 3 < ng) tab_s[u].w = scales[at + 3], tab_b[u].w = biases[at + 3];
+                }
+            }
+        }
+    }
+    // x of the block's windows: a thread takes eight consecutive k of one row (a wavefront reads
+    // 2 KiB of a row)
+    constexpr int OCTS = kWqSliceK / 8;  // per row
+    static_assert(16 * OCTS == UNITS, "");
+    float4 raw[UNITS / 512][2];
+#pragma unroll
+    for (int u = 0; u < UNITS / 512; ++u) {
+        const int unit = u * 512 + threadIdx.x, m = m0 + unit / OCTS, kl = (unit % OCTS) * 8;
+        raw[u][0] = raw[u][1] = float4{0.f, 0.f, 0.f, 0.f};
+        if (m < M && kl < nw * WK) {
+            const float* src = x + size_t(m) * K + w0 * WK + kl;
+            raw[u][0] = *reinterpret_cast<const float4*>(src);
+            raw[u][1] = *reinterpret_cast<const float4*>(src + 4);
+        }
+    }
     // All the weights of this wavefront are requested now and used window by window.  For the
     // request a lane takes quarter lane % 4 of row lane / 4 - four neighbouring lanes read 64
     // contiguous bytes, where the operand layout (row lane % 16, quarter lane / 16) would make
@@ -474,24 +528,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             // past the last window every lane reads the same 16 bytes: one cache line, dropped later
             wv[wi][rb] = *reinterpret_cast<const uint4*>(wi < nw ? row + (w0 + wi) * (WK * BITS / 32) : packed);
     }
-    // x of the block's windows, split and laid out as fragments by the block itself.  A thread
-    // takes eight consecutive k of one row (a wavefront reads 2 KiB of a row) and finds the
-    // (instruction, quarter) that holds them: the exchange of registers is its own inverse.
+    // The tables go to LDS, then x, split and laid out as fragments by the block itself: a thread
+    // finds the (instruction, quarter) that holds its eight k - the exchange of registers is its
+    // own inverse.
     uint4* x_lds = wq_lds;
-    {
-        constexpr int OCTS = kWqSliceK / 8;  // per row
-        static_assert(16 * OCTS == UNITS, "");
-        float4 raw[UNITS / 512][2];
+    float* s_lds = reinterpret_cast<float*>(wq_lds + WPS * NI * 3 * 64);
+    float* b_lds = s_lds + kWqRows * gp;
 #pragma unroll
-        for (int u = 0; u < UNITS / 512; ++u) {
-            const int unit = u * 512 + threadIdx.x, m = m0 + unit / OCTS, kl = (unit % OCTS) * 8;
-            raw[u][0] = raw[u][1] = float4{0.f, 0.f, 0.f, 0.f};
-            if (m < M && kl < nw * WK) {
-                const float* src = x + size_t(m) * K + w0 * WK + kl;
-                raw[u][0] = *reinterpret_cast<const float4*>(src);
-                raw[u][1] = *reinterpret_cast<const float4*>(src + 4);
-            }
+    for (int u = 0; u < kTabVec; ++u) {
+        const int i = (threadIdx.x + u * 512) * 4, row = i >> gsh, g = i & (gcap - 1);
+        if (i < kWqRows * gcap) {  // (slots past ng hold zeros and are never read)
+            float* sd = s_lds + row * gp + g;
+            float* bd = b_lds + row * gp + g;
+            sd[0] = tab_s[u].x, sd[1] = tab_s[u].y, sd[2] = tab_s[u].z, sd[3] = tab_s[u].w;
+            bd[0] = tab_b[u].x, bd[1] = tab_b[u].y, bd[2] = tab_b[u].z, bd[3] = tab_b[u].w;
         }
+    }
+    {
 #pragma unroll
         for (int u = 0; u < UNITS / 512; ++u) {
             const int unit = u * 512 + threadIdx.x, ml = unit / OCTS, kl = (unit % OCTS) * 8;
@@ -506,27 +559,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             for (int d = 0; d < 4; ++d) {
                 // slots 2d, 2d+1: the 4-bit decode pairs nibble d with nibble d + 4
                 const float e0 = BITS == 4 ? v[d] : v[2 * d], e1 = BITS == 4 ? v[d + 4] : v[2 * d + 1];
-                uint32_t h0, m0_, l0, h1, m1, l1;
-                wq_split3(e0, h0, m0_, l0);
-                wq_split3(e1, h1, m1, l1);
-                d3[0][d] = h0 | (h1 << 16), d3[1][d] = m0_ | (m1 << 16), d3[2][d] = l0 | (l1 << 16);
+                wq_split3x2(e0, e1, d3[0][d], d3[1][d], d3[2][d]);
             }
             if (wi < nw) {
 #pragma unroll
                 for (int p = 0; p < 3; ++p)
                     x_lds[((wi * NI + i) * 3 + p) * 64 + ml + 16 * qd] = uint4{d3[p][0], d3[p][1], d3[p][2], d3[p][3]};
             }
-        }
-    }
-    float* s_lds = reinterpret_cast<float*>(wq_lds + WPS * NI * 3 * 64);
-    float* b_lds = s_lds + kWqRows * gp;
-    {
-        const int row_first = tile * kWqRows;
-        for (int i = threadIdx.x; i < kWqRows * ng; i += 512) {
-            const int row = i / ng, g = i - row * ng;
-            const int n = row_first + row < N ? row_first + row : N - 1;
-            s_lds[row * gp + g] = scales[size_t(n) * groups_per_row + g0 + g];
-            b_lds[row * gp + g] = biases[size_t(n) * groups_per_row + g0 + g];
         }
     }
     __syncthreads();
@@ -627,7 +666,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     constexpr unsigned kScopeDevice = 16;  // "sc1" cache-policy bit of buffer accesses
     constexpr unsigned kSlabBytes = WAVES * RB * 64 * 16;
     typedef unsigned v4u __attribute__((ext_vector_type(4)));
-    const size_t tile_index = size_t(mb) * gridDim.x + tile;
+    const size_t tile_index = size_t(mb) * gridDim.y + tile;
     float* first_slab = slabs + tile_index * slices * (kSlabBytes / 4);
     const unsigned my_off = unsigned((wave * RB) * 64 + lane) * 16;
     {
@@ -686,7 +725,7 @@ int launch_wq_mfma(const float* x, const uint32_t* packed, const float* scales, 
         const int rc = sk_scratch(size_t(mblocks) * tiles, size_t(mblocks) * tiles * slices * (8 * 2 * 64 * 16), st, &sk);
         if (rc) return rc;
     }
-    const dim3 grid{unsigned(tiles), unsigned(slices), unsigned(mblocks)};
+    const dim3 grid{unsigned(slices), unsigned(tiles), unsigned(mblocks)};
     const int gs_shift = 31 - __builtin_clz(unsigned(gs));
     const int gmax = kWqSliceK / gs;
     const size_t lds = size_t(WPS) * G::NI * 3 * 64 * 16 + size_t(2) * kWqRows * ((gmax < 1 ? 1 : gmax) + 1) * 4;
