@@ -731,7 +731,9 @@ typedef struct {
     void* out;             /* NHWC [B,OH,OW,Cout]                            */
     int force_path;        /* 0 = choose; 1 = gemm (1x1), 2 = implicit GEMM,
                               3 = explicit im2col + GEMM, 4 = naive,
-                              5 = packed 4-channel image (Cin <= 4)          */
+                              5 = packed 4-channel image (Cin <= 4),
+                              6 = the same with x and w already packed
+                              (lq_quantize_nchw_to_packed4, lq_pack4_filter_i8)  */
     int tile_config;
     lq_join_args join;     /* optional join on codes (NHWC, ld = Cout): the residual
                               add of a bottleneck block fused into its last
@@ -753,6 +755,22 @@ int lq_quantize_nchw_to_nhwc(const float* x, int8_t* q, int code_offset, int B, 
                              lq_stream stream);
 int lq_dequantize_nhwc_to_nchw(const int8_t* q, int code_offset, float* out, int B, int C, int H,
                                int W, const float* scale, const float* zp, lq_stream stream);
+
+/* A first layer with at most four input channels (the RGB stem of a vision model,
+ * lucid/nn/quantized/modules.py:266-292 followed by conv.py:168-184) without the NHWC code
+ * tensor in between: lq_quantize_nchw_to_packed4 quantizes the float32 NCHW image straight
+ * into the four-channel, spatially pre-padded code image that the few-channel route of
+ * lq_qconv2d_i8 gathers from (padding and spare channels hold fill_code, the zero-point
+ * code as stored; extents from lq_qconv2d_packed4_geometry), lq_pack4_filter_i8 lays the
+ * filter codes out to match once ([Cout,KH,KW,Cin] -> [Cout,KH,KWp,4], zeros in the added
+ * taps and channels), and lq_qconv2d_i8 with force_path = 6 takes both as x and w (H, W,
+ * pads, KW, Cin still describe the logical layer).  Same codes as lq_quantize_nchw_to_nhwc
+ * + force_path 5. */
+int lq_qconv2d_packed4_geometry(const lq_qconv2d_args* args, int* Hp, int* Wp, int* KWp);
+int lq_quantize_nchw_to_packed4(const float* x, int8_t* out, int code_offset, int B, int C, int H, int W,
+                                int pad_h_lo, int pad_w_lo, int Hp, int Wp, const float* scale, const float* zp,
+                                int qmin, int qmax, int fill_code, lq_stream stream);
+int lq_pack4_filter_i8(const int8_t* w, int8_t* out, int Cout, int KH, int KW, int Cin, lq_stream stream);
 int lq_repack_oihw_to_ohwi_i8(const int8_t* w, int8_t* out, int O, int I, int KH, int KW,
                               lq_stream stream);
 

@@ -234,6 +234,9 @@ class QConv3dArgs(C.Structure):
 
 _SIGNATURES["lq_qconv3d_i8"] = [C.POINTER(QConv3dArgs), _vp]
 _SIGNATURES["lq_quantize_nchw_to_nhwc"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]
+_SIGNATURES["lq_qconv2d_packed4_geometry"] = [C.POINTER(QConv2dArgs), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]
+_SIGNATURES["lq_quantize_nchw_to_packed4"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _i, _vp]
+_SIGNATURES["lq_pack4_filter_i8"] = [_vp, _vp, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_dequantize_nhwc_to_nchw"] = [_vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp]
 _SIGNATURES["lq_repack_oihw_to_ohwi_i8"] = [_vp, _vp, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_im2col_ndhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]

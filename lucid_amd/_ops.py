@@ -95,7 +95,7 @@ def qlinear_i8(a: Tensor, w: Tensor, *, a_zp: int = 0, a_zp_dev: Tensor | None =
     return out
 
 
-CONV_AUTO, CONV_GEMM, CONV_IMPLICIT, CONV_IM2COL, CONV_NAIVE, CONV_PACKED4 = range(6)
+CONV_AUTO, CONV_GEMM, CONV_IMPLICIT, CONV_IM2COL, CONV_NAIVE, CONV_PACKED4, CONV_PREPACKED4 = range(7)
 
 
 def conv_out_size(size: int, k: int, stride: int, pad_lo: int, pad_hi: int, dil: int) -> int:
@@ -125,17 +125,30 @@ def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None
                groups: int = 1, relu: bool = False, out_mode: int = OUT_F32,
                out_scale: Tensor | None = None, out_zp: Tensor | None = None, out_qmin: int = 0,
                out_qmax: int = 255, out_offset: int = 0, path: int = CONV_AUTO,
-               tile_config: int = 0, join=None, w_zp: Tensor | None = None) -> Tensor:
+               tile_config: int = 0, join=None, w_zp: Tensor | None = None,
+               logical: tuple[int, int, int, int] | None = None) -> Tensor:
     """Fused int8 convolution; see ``lq_qconv2d_i8``.  ``x`` int8 NHWC, ``w``
     int8 ``[Cout, KH, KW, Cin/groups]``, ``pad`` = (h_lo, h_hi, w_lo, w_hi);
     ``w_zp`` (int32 ``[Cout]``) holds the zero points of affine filters.
-    Returns NHWC ``[B, OH, OW, Cout]``."""
+    With ``path=CONV_PREPACKED4`` ``x`` and ``w`` are the packed tensors of
+    ``quantize_nchw_to_packed4`` and ``pack4_filter_i8`` and ``logical`` = (H, W, Cin, KW)
+    of the layer they stand for.  Returns NHWC ``[B, OH, OW, Cout]``."""
     if x.ndim != 4 or w.ndim != 4:
         raise _C.ShapeMismatch(f"qconv2d_i8: expected 4-d x and w, got {x.shape} and {w.shape}")
-    B, H, W, Cin = x.shape
-    Cout, KH, KW, Cg = w.shape
-    if Cg * groups != Cin:
-        raise _C.ShapeMismatch(f"qconv2d_i8: weight {w.shape} does not match Cin={Cin}, groups={groups}")
+    if path == CONV_PREPACKED4:
+        if logical is None or groups != 1:
+            raise ValueError("qconv2d_i8: packed operands need logical=(H, W, Cin, KW) and groups == 1")
+        H, W, Cin, KW = (int(v) for v in logical)
+        Hp, Wp, KWp = packed4_geometry(H, W, Cin, KW, int(stride[1]), pad)
+        B, Cout, KH = x.shape[0], w.shape[0], w.shape[1]
+        if tuple(x.shape[1:]) != (Hp, Wp, 4) or tuple(w.shape[2:]) != (KWp, 4):
+            raise _C.ShapeMismatch(f"qconv2d_i8: packed x {x.shape} / w {w.shape} do not match the layer's "
+                                   f"[B, {Hp}, {Wp}, 4] / [Cout, KH, {KWp}, 4]")
+    else:
+        B, H, W, Cin = x.shape
+        Cout, KH, KW, Cg = w.shape
+        if Cg * groups != Cin:
+            raise _C.ShapeMismatch(f"qconv2d_i8: weight {w.shape} does not match Cin={Cin}, groups={groups}")
     OH = conv_out_size(H, KH, stride[0], pad[0], pad[1], dilation[0])
     OW = conv_out_size(W, KW, stride[1], pad[2], pad[3], dilation[1])
     out = Tensor.empty((B, max(OH, 0), max(OW, 0), Cout), _OUT_DTYPE[out_mode], "hip")
@@ -158,6 +171,41 @@ def qconv2d_i8(x: Tensor, w: Tensor, *, a_zp: int, a_scale: Tensor | None = None
         raise _C.ShapeMismatch(f"w_zp has {w_zp.numel} entries for Cout = {Cout}")
     a.w_zp = _ptr(w_zp, "w_zp", T.int32)
     _C.call("lq_qconv2d_i8", C.byref(a), None)
+    return out
+
+
+def packed4_geometry(H: int, W: int, Cin: int, KW: int, stride_w: int, pad) -> tuple[int, int, int]:
+    """(Hp, Wp, KWp) of the packed four-channel image and filter of a layer with at most four
+    input channels; see ``lq_qconv2d_packed4_geometry``."""
+    a = _C.QConv2dArgs()
+    a.H, a.W, a.Cin, a.KW, a.KH, a.B, a.Cout = int(H), int(W), int(Cin), int(KW), 1, 1, 1
+    a.stride_h, a.stride_w, a.dil_h, a.dil_w, a.groups = 1, int(stride_w), 1, 1, 1
+    a.pad_h_lo, a.pad_h_hi, a.pad_w_lo, a.pad_w_hi = (int(v) for v in pad)
+    hp, wp, kwp = C.c_int(), C.c_int(), C.c_int()
+    _C.call("lq_qconv2d_packed4_geometry", C.byref(a), C.byref(hp), C.byref(wp), C.byref(kwp))
+    return hp.value, wp.value, kwp.value
+
+
+def quantize_nchw_to_packed4(x: Tensor, scale: Tensor, zero_point: Tensor, qmin: int, qmax: int, offset: int,
+                             fill_code: int, pad, Hp: int, Wp: int) -> Tensor:
+    """float32 NCHW (C <= 4) -> int8 ``[B, Hp, Wp, 4]`` codes of the few-channel convolution
+    route; see ``lq_quantize_nchw_to_packed4``."""
+    if x.ndim != 4 or x.dtype != T.float32:
+        raise _C.ShapeMismatch(f"quantize_nchw_to_packed4: expected a float32 (B, C, H, W) tensor, got {x.shape}")
+    B, Cc, H, W = x.shape
+    out = Tensor.empty((B, Hp, Wp, 4), T.int8, "hip")
+    _C.call("lq_quantize_nchw_to_packed4", _ptr(x, "x", T.float32), out.data_ptr, int(offset), B, Cc, H, W,
+            int(pad[0]), int(pad[2]), int(Hp), int(Wp), _ptr(scale, "scale", T.float32),
+            _ptr(zero_point, "zero_point", T.float32), int(qmin), int(qmax), int(fill_code), None)
+    return out
+
+
+def pack4_filter_i8(w: Tensor) -> Tensor:
+    """int8 ``[Cout, KH, KW, Cin]`` (Cin <= 4) -> ``[Cout, KH, KWp, 4]`` with zeros in the added
+    taps and channels; see ``lq_pack4_filter_i8``."""
+    Cout, KH, KW, Cin = w.shape
+    out = Tensor.empty((Cout, KH, (KW + 3) // 4 * 4, 4), T.int8, "hip")
+    _C.call("lq_pack4_filter_i8", _ptr(w, "w", T.int8), out.data_ptr, Cout, KH, KW, Cin, None)
     return out
 
 

@@ -438,6 +438,48 @@ __global__ __launch_bounds__(256) void quantize_nchw_to_nhwc_small_c_kernel(
     }
 }
 
+// float32 NCHW (at most four channels) -> the packed four-channel, spatially pre-padded code
+// image of the few-channel route, in one pass: what lq_quantize_nchw_to_nhwc followed by
+// pack4_padded_kernel writes (the same quantization arithmetic; padding and spare channels hold
+// `fill`, the zero-point code).  One packed pixel per lane.
+__global__ __launch_bounds__(256) void quantize_nchw_to_packed4_kernel(
+    const float* __restrict__ x, int B, int C, int H, int W, int ph, int pw, int Hp, int Wp, const float* scale,
+    const float* zp, float lo, float hi, int off, int fill, uint32_t* __restrict__ out) {
+    const float s = scale[0], z = zp[0];
+    const size_t n = size_t(B) * Hp * Wp, stride = size_t(gridDim.x) * 256, HW = size_t(H) * W;
+    const uint32_t f = uint32_t(uint8_t(fill));
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+        const int wp = int(i % Wp);
+        const size_t r = i / Wp;
+        const int hp = int(r % Hp), b = int(r / Hp);
+        const int h = hp - ph, w = wp - pw;
+        uint32_t v = f | (f << 8) | (f << 16) | (f << 24);
+        if (h >= 0 && h < H && w >= 0 && w < W) {
+            v = 0;
+            for (int c = 0; c < 4; ++c) {
+                uint32_t code = f;
+                if (c < C) {
+                    const float u = q_core_local(x[(size_t(b) * C + c) * HW + size_t(h) * W + w], s, z, lo, hi);
+                    code = uint32_t(uint8_t(int8_t(((u != u) ? 0 : int(u)) + off)));
+                }
+                v |= code << (8 * c);
+            }
+        }
+        out[i] = v;
+    }
+}
+
+// Extents of the packed image of a few-channel layer: rows start 16-byte aligned and the last
+// output's window of KWp pixels lies inside the row.
+void packed4_geometry(const lq_qconv2d_args* p, int OW, int* KWp, int* Hp, int* Wp) {
+    *KWp = (p->KW + 3) / 4 * 4;
+    *Hp = p->H + p->pad_h_lo + p->pad_h_hi;
+    int wp = p->W + p->pad_w_lo + p->pad_w_hi;
+    const int need = (OW - 1) * p->stride_w + *KWp;
+    wp = wp > need ? wp : need;
+    *Wp = (wp + 3) / 4 * 4;
+}
+
 inline unsigned grid_1d(size_t n, unsigned per_block = 256) {
     size_t b = (n + per_block - 1) / per_block;
     if (b < 1) b = 1;
@@ -506,6 +548,8 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
 
     LQ_REQUIRE(p->w_zp == nullptr || p->out_mode != OUT_ACC_I32, LQ_ERR_VALUE,
                "qconv2d_i8: mode ACC_I32 returns the raw sums a * w; weight zero points cannot be applied to it");
+    LQ_REQUIRE(p->w_zp == nullptr || p->force_path != 6, LQ_ERR_VALUE,
+               "qconv2d_i8: affine filters take the NHWC image (the window sums are gathered from it), not the packed one");
     if (p->w_zp) {
         // affine filters: the raw accumulators, then the window sums of the image as a
         // convolution with one all-ones filter per group (taps in the padding read the
@@ -542,7 +586,8 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
                          p->pad_h_lo == 0 && p->pad_h_hi == 0 && p->pad_w_lo == 0 &&
                          p->pad_w_hi == 0 && p->groups == 1;
     const bool aligned = aligned16(p->x) && aligned16(p->w);
-    int path = p->force_path;  // 0 = choose, 1 = gemm, 2 = implicit, 3 = im2col, 4 = naive, 5 = packed 4-channel
+    int path = p->force_path;  // 0 = choose, 1 = gemm, 2 = implicit, 3 = im2col, 4 = naive, 5 = packed 4-channel,
+                               // 6 = packed 4-channel with x and w already packed
     const bool few_channels = p->Cin <= 4 && p->groups == 1 && p->dil_w == 1 && p->KH * ((p->KW + 3) / 4) * 16 <= 131071;
     if (path == 0) {
         if (is_gemm && p->Cin % 16 == 0 && aligned)
@@ -554,30 +599,34 @@ int lq_qconv2d_i8(const lq_qconv2d_args* p, lq_stream stream) {
         else
             path = 3;
     }
-    if (path == 5) {
+    if (path == 5 || path == 6) {
         LQ_REQUIRE(few_channels, LQ_ERR_VALUE,
                    "qconv2d_i8: the packed route needs Cin <= 4, groups == 1 and dilation_w == 1");
-        const int KWp = (p->KW + 3) / 4 * 4;
-        const int Hp = p->H + p->pad_h_lo + p->pad_h_hi;
-        int Wp = p->W + p->pad_w_lo + p->pad_w_hi;
-        const int need = (OW - 1) * p->stride_w + KWp;  // the last output's window of KWp pixels
-        Wp = Wp > need ? Wp : need;
-        Wp = (Wp + 3) / 4 * 4;                          // rows start 16-byte aligned
-        const size_t img_bytes = (size_t(p->B) * Hp * Wp * 4 + 255) / 256 * 256;
-        const size_t flt_bytes = (size_t(p->Cout) * p->KH * KWp * 4 + 255) / 256 * 256;
+        int KWp, Hp, Wp;
+        packed4_geometry(p, OW, &KWp, &Hp, &Wp);
         LQ_REQUIRE(size_t(p->B) * Hp * Wp * 4 < 0xffffffffull, LQ_ERR_SHAPE, "qconv2d_i8: padded image too large");
-        void* ws = nullptr;
-        int rc = workspace(img_bytes + flt_bytes, st, &ws);
-        if (rc) return rc;
-        int8_t* img = static_cast<int8_t*>(ws);
-        int8_t* flt = img + img_bytes;
-        hipLaunchKernelGGL(pack4_padded_kernel, dim3(grid_1d(size_t(p->B) * Hp * Wp)), dim3(256), 0, st, p->x, p->B,
-                           p->H, p->W, p->Cin, p->pad_h_lo, p->pad_w_lo, Hp, Wp, p->a_zp,
-                           reinterpret_cast<uint32_t*>(img));
-        LQ_CHECK_LAUNCH("pack4_padded");
-        hipLaunchKernelGGL(pack4_filter_kernel, dim3(grid_1d(size_t(p->Cout) * p->KH * KWp * 4)), dim3(256), 0, st,
-                           p->w, p->Cout, p->KH, p->KW, p->Cin, KWp, flt);
-        LQ_CHECK_LAUNCH("pack4_filter");
+        const int8_t* img = p->x;
+        const int8_t* flt = p->w;
+        if (path == 5) {
+            const size_t img_bytes = (size_t(p->B) * Hp * Wp * 4 + 255) / 256 * 256;
+            const size_t flt_bytes = (size_t(p->Cout) * p->KH * KWp * 4 + 255) / 256 * 256;
+            void* ws = nullptr;
+            int rc = workspace(img_bytes + flt_bytes, st, &ws);
+            if (rc) return rc;
+            int8_t* wimg = static_cast<int8_t*>(ws);
+            int8_t* wflt = wimg + img_bytes;
+            hipLaunchKernelGGL(pack4_padded_kernel, dim3(grid_1d(size_t(p->B) * Hp * Wp)), dim3(256), 0, st, p->x, p->B,
+                               p->H, p->W, p->Cin, p->pad_h_lo, p->pad_w_lo, Hp, Wp, p->a_zp,
+                               reinterpret_cast<uint32_t*>(wimg));
+            LQ_CHECK_LAUNCH("pack4_padded");
+            hipLaunchKernelGGL(pack4_filter_kernel, dim3(grid_1d(size_t(p->Cout) * p->KH * KWp * 4)), dim3(256), 0, st,
+                               p->w, p->Cout, p->KH, p->KW, p->Cin, KWp, wflt);
+            LQ_CHECK_LAUNCH("pack4_filter");
+            img = wimg, flt = wflt;
+        } else {
+            // x: [B, Hp, Wp, 4] from lq_quantize_nchw_to_packed4, w: [Cout, KH, KWp, 4] from lq_pack4_filter_i8
+            LQ_REQUIRE(aligned16(img) && aligned16(flt), LQ_ERR_VALUE, "qconv2d_i8: packed tensors must be 16-byte aligned");
+        }
         GemmArgs gg = g;
         gg.w = flt; gg.K = p->KH * KWp * 4; gg.N = p->Cout;
         gg.cx = img; gg.cH = Hp; gg.cW = Wp; gg.cCin = 4; gg.cCg = 16; gg.cKW = KWp / 4;
@@ -756,6 +805,49 @@ int lq_quantize_nchw_to_nhwc(const float* x, int8_t* q, int code_offset, int B, 
                        as_stream(stream), x, q, B, C, HW, scale, zp, float(qmin), float(qmax),
                        code_offset);
     LQ_CHECK_LAUNCH("quantize_nchw_to_nhwc");
+    return LQ_OK;
+}
+
+int lq_qconv2d_packed4_geometry(const lq_qconv2d_args* p, int* Hp, int* Wp, int* KWp) {
+    LQ_REQUIRE(p && Hp && Wp && KWp, LQ_ERR_VALUE, "qconv2d_packed4_geometry: NULL pointer");
+    LQ_REQUIRE(p->H > 0 && p->W > 0 && p->KW > 0 && p->stride_w >= 1 && p->dil_w == 1 && p->Cin >= 1 && p->Cin <= 4 &&
+                   p->groups == 1 && p->pad_h_lo >= 0 && p->pad_h_hi >= 0 && p->pad_w_lo >= 0 && p->pad_w_hi >= 0,
+               LQ_ERR_VALUE, "qconv2d_packed4_geometry: the packed route needs Cin <= 4, groups == 1 and dilation_w == 1");
+    const int OW = (p->W + p->pad_w_lo + p->pad_w_hi - (p->KW - 1) - 1) / p->stride_w + 1;
+    LQ_REQUIRE(OW > 0, LQ_ERR_SHAPE, "qconv2d_packed4_geometry: empty output");
+    packed4_geometry(p, OW, KWp, Hp, Wp);
+    return LQ_OK;
+}
+
+int lq_quantize_nchw_to_packed4(const float* x, int8_t* out, int code_offset, int B, int C, int H, int W,
+                                int pad_h_lo, int pad_w_lo, int Hp, int Wp, const float* scale, const float* zp,
+                                int qmin, int qmax, int fill_code, lq_stream stream) {
+    if (size_t(B) * Hp * Wp == 0) return LQ_OK;
+    LQ_REQUIRE(x && out && scale && zp, LQ_ERR_VALUE, "quantize_nchw_to_packed4: NULL pointer");
+    LQ_REQUIRE(C >= 1 && C <= 4 && H > 0 && W > 0 && pad_h_lo >= 0 && pad_w_lo >= 0 && Hp >= H + pad_h_lo &&
+                   Wp >= W + pad_w_lo && Wp % 4 == 0,
+               LQ_ERR_SHAPE, "quantize_nchw_to_packed4: the packed image [%d, %d] does not hold %d x %d at (%d, %d)", Hp,
+               Wp, H, W, pad_h_lo, pad_w_lo);
+    LQ_REQUIRE(qmin <= qmax && qmin + code_offset >= -128 && qmax + code_offset <= 127 && fill_code >= -128 &&
+                   fill_code <= 127,
+               LQ_ERR_VALUE, "quantize_nchw_to_packed4: grid [%d,%d] + offset %d does not fit int8", qmin, qmax,
+               code_offset);
+    LQ_REQUIRE(aligned16(out), LQ_ERR_VALUE, "quantize_nchw_to_packed4: out must be 16-byte aligned");
+    hipLaunchKernelGGL(quantize_nchw_to_packed4_kernel, dim3(grid_1d(size_t(B) * Hp * Wp)), dim3(256), 0,
+                       as_stream(stream), x, B, C, H, W, pad_h_lo, pad_w_lo, Hp, Wp, scale, zp, float(qmin), float(qmax),
+                       code_offset, fill_code, reinterpret_cast<uint32_t*>(out));
+    LQ_CHECK_LAUNCH("quantize_nchw_to_packed4");
+    return LQ_OK;
+}
+
+int lq_pack4_filter_i8(const int8_t* w, int8_t* out, int Cout, int KH, int KW, int Cin, lq_stream stream) {
+    if (size_t(Cout) * KH * KW == 0) return LQ_OK;
+    LQ_REQUIRE(w && out, LQ_ERR_VALUE, "pack4_filter_i8: NULL pointer");
+    LQ_REQUIRE(Cin >= 1 && Cin <= 4 && Cout > 0 && KH > 0 && KW > 0, LQ_ERR_SHAPE, "pack4_filter_i8: bad shape");
+    const int KWp = (KW + 3) / 4 * 4;
+    hipLaunchKernelGGL(pack4_filter_kernel, dim3(grid_1d(size_t(Cout) * KH * KWp * 4)), dim3(256), 0,
+                       as_stream(stream), w, Cout, KH, KW, Cin, KWp, out);
+    LQ_CHECK_LAUNCH("pack4_filter");
     return LQ_OK;
 }
 

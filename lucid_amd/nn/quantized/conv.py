@@ -71,6 +71,7 @@ class Conv2d(Module):
     def _state_loaded(self, name: str) -> None:
         if name == "weight_int8":
             self._w_ohwi = self._wsum = None
+            self.__dict__.pop("_w_packed4", None)
         if name == "zero_point":
             self._zp_host = None
         if name == "weight_zero_point":
@@ -101,10 +102,59 @@ class Conv2d(Module):
         self._w_ohwi = w
         self._wsum = _ops.rowsum_i8(w)
 
-    def forward(self, x: Tensor, join=None) -> Tensor:
+    def _forward_quantizing(self, x: Tensor, quantize) -> Tensor | None:
+        """``self(quantize(x))`` for a float image of at most four channels without the NHWC code
+        tensor in between: the image is quantized straight into the packed, pre-padded form the
+        few-channel kernel route gathers from (one pass instead of quantize + pack, and the
+        filter is packed once).  None where that route does not take the layer."""
+        KH, KW = self.kernel_size
+        if type(self).forward is not Conv2d.forward or not is_plain_float(x) \
+                or x.ndim != 4 or x.shape[1] != self.in_channels or x.dtype != T.float32 or x.device != "hip" \
+                or self.in_channels > 4 or self.groups != 1 or self.dilation[1] != 1 \
+                or self.padding_mode != "zeros" or KH * ((KW + 3) // 4) * 16 > 131071 \
+                or weight_zero_points(self) is not None or x.numel == 0:
+            return None
+        if self._w_ohwi is None:
+            self._prepare_weight()
+        if self.__dict__.get("_w_packed4") is None:
+            self._w_packed4 = _ops.pack4_filter_i8(self._w_ohwi)
+        if self._zp_host is None:
+            self._zp_host = int(host_scalar(self.zero_point))
+        if quantize._zp_host is None:
+            quantize._zp_host = int(host_scalar(quantize.zero_point))
+        qd, qoff = quantize.qdtype, storage_offset(quantize.qdtype)
+        pad = self._resolve_pad(x)
+        B, Cc, H, W = x.shape
+        if _ops.conv_out_size(H, KH, self.stride[0], pad[0], pad[1], self.dilation[0]) <= 0 or \
+                _ops.conv_out_size(W, KW, self.stride[1], pad[2], pad[3], 1) <= 0:
+            return None
+        Hp, Wp, _ = _ops.packed4_geometry(H, W, Cc, KW, self.stride[1], pad)
+        a_zp = quantize._zp_host + qoff
+        image = _ops.quantize_nchw_to_packed4(x, quantize.scale, quantize.zero_point, qd.quant_min, qd.quant_max,
+                                              qoff, a_zp, pad, Hp, Wp)
+        off = storage_offset(self.out_qdtype)
+        codes = _ops.qconv2d_i8(
+            image, self._w_packed4, a_zp=a_zp, a_scale=quantize.scale, w_scale=self.weight_scale, wsum=self._wsum,
+            bias=self.bias, stride=self.stride, pad=pad, dilation=self.dilation, relu=self._fused_relu,
+            out_mode=_ops.OUT_REQUANT_I8, out_scale=self.scale, out_zp=self.zero_point,
+            out_qmin=self.out_qdtype.quant_min, out_qmax=self.out_qdtype.quant_max, out_offset=off,
+            path=_ops.CONV_PREPACKED4, logical=(H, W, Cc, KW))
+        _, OH, OW, Co = codes.shape
+        return Tensor.on_grid((B, Co, OH, OW), Grid(codes, self.scale, self.zero_point,
+                                                    self.out_qdtype, off, self._zp_host, "nhwc"))
+
+    def forward(self, x: Tensor, join=None, quantize=None) -> Tensor:
         """``join = (other, qfunctional, relu)`` fuses ``qfunctional.add[_relu](self(x), other)``
         into this layer's epilogue: the result is on the functional's grid, bit for bit what
-        the two separate modules give, and the layer's own output is never stored."""
+        the two separate modules give, and the layer's own output is never stored.
+        ``quantize`` (a ``Quantize`` module) stands for ``self(quantize(x))`` on a float ``x``:
+        the same codes, and for a first layer of at most four channels one pass less."""
+        if quantize is not None:
+            if join is None:
+                fused = self._forward_quantizing(x, quantize)
+                if fused is not None:
+                    return fused
+            x = quantize(x)
         name = type(self).__name__
         if is_plain_float(x) and join is None:
             # no grid on the input: Lucid's float formulation (conv.py:168-184)

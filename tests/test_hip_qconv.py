@@ -276,6 +276,93 @@ def test_packed_route_for_few_input_channels(B, H, W, Cin, Cout, KH, KW, stride,
     assert np.array_equal(_ops.qconv2d_i8(dx, dw, **kw, path=_ops.CONV_IM2COL).numpy(), want)
 
 
+@pytest.mark.parametrize("B,H,W,Cin,Cout,KH,KW,stride,pad", [
+    (2, 224, 224, 3, 64, 7, 7, (2, 2), (3, 3, 3, 3)),   # the ResNet stem
+    (3, 17, 13, 3, 24, 3, 3, (1, 1), (1, 1, 1, 1)),
+    (2, 20, 9, 1, 16, 5, 2, (2, 1), (2, 1, 0, 1)),
+    (2, 11, 11, 4, 40, 3, 5, (1, 3), (0, 0, 2, 2)),
+])
+def test_float_image_quantized_into_the_packed_form(B, H, W, Cin, Cout, KH, KW, stride, pad):
+    """A float NCHW image quantized straight into the packed four-channel image, convolved with the
+    filter packed once: the codes of the oracle's quantize followed by its convolution, and the
+    packed image itself holds the oracle's codes inside and the zero-point code everywhere else."""
+    rng = np.random.default_rng(7 * B + H + Cout)
+    x = (rng.standard_normal((B, Cin, H, W)) * 1.3).astype(np.float32)
+    x.reshape(-1)[:6] = [np.nan, np.inf, -np.inf, 1e30, -1e30, 0.0125]
+    w = rng.integers(-127, 128, (Cout, KH, KW, Cin)).astype(np.int8)
+    ws = (rng.random(Cout).astype(np.float32) + 0.5) * 1e-3
+    bias = rng.standard_normal(Cout).astype(np.float32) * 0.1
+    s_in, z_in = np.float32(0.025), np.float32(119.0)
+    xq = np.ascontiguousarray(O.quantize(x, s_in, z_in, 0, 255, code_offset=-128).transpose(0, 2, 3, 1))
+    a_zp = 119 - 128
+    Hp, Wp, KWp = _ops.packed4_geometry(H, W, Cin, KW, stride[1], pad)
+    assert KWp == (KW + 3) // 4 * 4 and Hp == H + pad[0] + pad[1] and Wp % 4 == 0
+    OW = O.conv_out_size(W, KW, stride[1], pad[2], pad[3], 1)
+    assert Wp >= max(W + pad[2] + pad[3], (OW - 1) * stride[1] + KWp)
+    image = _ops.quantize_nchw_to_packed4(hip(x), hip(s_in), hip(z_in), 0, 255, -128, a_zp, pad, Hp, Wp)
+    want_image = np.full((B, Hp, Wp, 4), a_zp, np.int8)
+    want_image[:, pad[0]:pad[0] + H, pad[2]:pad[2] + W, :Cin] = xq
+    assert np.array_equal(image.numpy(), want_image)
+    dw = hip(w)
+    wp = _ops.pack4_filter_i8(dw)
+    want_w = np.zeros((Cout, KH, KWp, 4), np.int8)
+    want_w[:, :, :KW, :Cin] = w
+    assert np.array_equal(wp.numpy(), want_w)
+    kw = dict(a_zp=a_zp, a_scale=hip(s_in), w_scale=hip(ws), wsum=_ops.rowsum_i8(dw), bias=hip(bias),
+              stride=stride, pad=pad, relu=True, out_mode=_ops.OUT_REQUANT_I8, out_scale=hip(np.float32(0.05)),
+              out_zp=hip(np.float32(3.0)), out_qmin=0, out_qmax=255, out_offset=-128)
+    got = _ops.qconv2d_i8(image, wp, **kw, path=_ops.CONV_PREPACKED4, logical=(H, W, Cin, KW))
+    want = O.qconv2d(xq, w, a_zp, s_in, ws, stride=stride, pad=pad, bias=bias, relu=True, out_mode=O.OUT_REQUANT_I8,
+                     out_scale=0.05, out_zp=3.0, out_qmin=0, out_qmax=255, out_offset=-128)
+    assert np.array_equal(got.numpy(), want)
+    assert np.array_equal(_ops.qconv2d_i8(hip(xq), dw, **kw).numpy(), want)
+
+
+@pytest.mark.parametrize("cin,relu,wzp,padding", [(3, True, 0, 3), (1, False, 0, "same"), (4, True, 0, 0),
+                                                  (8, False, 0, 1), (3, False, 5, 1)])
+def test_conv_module_taking_the_quantize_module(cin, relu, wzp, padding):
+    """``conv(x, quantize=q)`` holds the codes of ``conv(q(x))``: through the packed image where the
+    layer has at most four channels and symmetric filters, through ``q`` itself otherwise."""
+    import lucid_amd.nn.quantized as nnq
+    import lucid_amd.quantization as Q
+
+    rng = np.random.default_rng(60 + cin)
+    B, H, W, Cout, k = 2, 19, 23, 24, 5
+    x = hip((rng.standard_normal((B, cin, H, W)) * 1.5).astype(np.float32))
+    conv = (nnq.ConvReLU2d if relu else nnq.Conv2d)(cin, Cout, k, stride=1 if padding == "same" else 2, padding=padding)
+    state = {"weight_int8": codes(rng, (Cout, cin, k, k), -127, 127),
+             "weight_scale": rng.uniform(0.001, 0.01, Cout).astype(np.float32),
+             "weight_zero_point": np.full(Cout, wzp, np.float32), "bias": rng.standard_normal(Cout).astype(np.float32),
+             "scale": np.float32(0.05), "zero_point": np.float32(17.0)}
+    conv.load_state_dict({k_: L.tensor(v, device="hip") for k_, v in state.items()})
+    q = nnq.Quantize(hip(np.float32(0.03)), hip(np.float32(121.0)), Q.quint8)
+    fused = conv(x, quantize=q)
+    two = conv(q(x))
+    assert fused.shape == two.shape and fused._grid.layout == two._grid.layout == "nhwc"
+    assert np.array_equal(fused._grid.codes.numpy(), two._grid.codes.numpy())
+    assert ("_w_packed4" in conv.__dict__) == (cin <= 4 and wzp == 0)
+    # new weights drop the packed filter
+    conv.load_state_dict({"weight_int8": L.tensor(-state["weight_int8"], device="hip")}, strict=False)
+    assert conv.__dict__.get("_w_packed4") is None
+    assert np.array_equal(conv(x, quantize=q)._grid.codes.numpy(), conv(q(x))._grid.codes.numpy())
+
+
+def test_packed_operands_are_checked():
+    one = hip(np.float32(1.0))
+    image, wp = hip(np.zeros((1, 8, 12, 4), np.int8)), hip(np.zeros((16, 3, 4, 4), np.int8))
+    kw = dict(a_zp=0, a_scale=one, w_scale=hip(np.ones(16, np.float32)), pad=(1, 1, 1, 1), path=_ops.CONV_PREPACKED4)
+    with pytest.raises(ValueError, match="logical"):
+        _ops.qconv2d_i8(image, wp, **kw)
+    with pytest.raises(_C.ShapeMismatch, match="packed"):
+        _ops.qconv2d_i8(image, wp, **kw, logical=(7, 7, 3, 3))        # the image of a 6 x 6 layer
+    assert _ops.qconv2d_i8(image, wp, **kw, logical=(6, 6, 3, 3)).shape == (1, 6, 6, 16)
+    with pytest.raises(ValueError, match="affine filters"):
+        _ops.qconv2d_i8(image, wp, **kw, logical=(6, 6, 3, 3), wsum=hip(np.zeros(16, np.int32)),
+                        w_zp=hip(np.ones(16, np.int32)))
+    with pytest.raises(ValueError, match="Cin <= 4"):
+        _ops.packed4_geometry(8, 8, 5, 3, 1, (0, 0, 0, 0))
+
+
 # ------------------------------------------------------------------ affine filter codes
 @pytest.mark.parametrize("case", [CASES[0], CASES[1], CASES[2], CASES[4], CASES[5], CASES[6], CASES[8]])
 def test_affine_filter_zero_points_on_every_route(case):

@@ -154,7 +154,7 @@ class QResNet50(nn.Module):
         self.dequant = nnq.DeQuantize()
 
     def forward(self, x):
-        x = self.maxpool(self.conv1(self.quant(x)))
+        x = self.maxpool(self.conv1(x, quantize=self.quant))  # = conv1(quant(x)), quantized into the stem's packed image
         x = self.blocks(x)
         return self.dequant(self.fc(self.flatten(self.avgpool(x))))
 
