@@ -639,7 +639,10 @@ typedef struct {
                               15 / 18 / 19 (convolutions only) = one block per box of
                               256 / 128 / 64 output positions x 64 channels with the box's
                               input halo held in LDS (stride 1, Cin/groups % 64 == 0, no
-                              join);
+                              join), 20 (the packed route of a convolution with at most four
+                              input channels, filter row of at most 256 bytes, no join) =
+                              boxes of 16 x 16 output positions x 64 channels with the
+                              filter in registers and the box's input halo in LDS;
                               next byte 0 = choose, 1 = one block per tile,
                               2 = stream-K work split, 3 = stream-K over the
                               leftover tiles of the last round only; bits 16..30

@@ -68,6 +68,8 @@ int launch_pp_shape(const GemmArgs&, int, hipStream_t);
 int launch_bw_shape(const GemmArgs&, int, hipStream_t);
 bool conv_halo_applies(const GemmArgs&, int conv, int lbox = 8);
 int launch_conv_halo(const GemmArgs&, int conv, int groups, int lbox, hipStream_t);
+bool conv_few_applies(const GemmArgs&, int conv, int groups);
+int launch_conv_few(const GemmArgs&, int conv, int groups, hipStream_t);
 }  // namespace lq
 
 namespace {
@@ -106,6 +108,11 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
         LQ_REQUIRE(conv, LQ_ERR_VALUE, "tile_config %d is for convolutions", cfg);
         LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
         return launch_conv_halo(g, conv, groups, cfg == 15 ? 8 : (cfg == 18 ? 7 : 6), st);
+    case 20:
+        // at most four input channels on the packed image: filter in registers, input halo of 16 x 16 boxes in LDS
+        LQ_REQUIRE(conv, LQ_ERR_VALUE, "tile_config %d is for convolutions", cfg);
+        LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
+        return launch_conv_few(g, conv, groups, st);
     default: return fail(LQ_ERR_VALUE, "unknown tile_config %d", cfg);
     }
 }
@@ -124,6 +131,8 @@ bool pp_applies(const GemmArgs& g, int conv, int groups) {
 // of the CUs without work.
 int heuristic_tile_shape(const GemmArgs& g, int conv, int groups) {
     const long mt128 = (g.M + 127) / 128;
+    // an image of at most four channels with a block's worth of 16 x 16 boxes for every CU
+    if (g.M >= 65536 && conv_few_applies(g, conv, groups)) return 20;
     // far fewer 128 x 128 tiles than CUs (a small batch in the late stages of a network): 64 x 64
     // tiles, four blocks per CU, with 128-byte k steps when K is long (plain and 2-d only)
     if (mt128 * ((g.N + 127) / 128) * groups < 128) return (g.K >= 1024 && conv != 2) ? 10 : 9;
@@ -220,7 +229,7 @@ int tune_import_text(const char* text, int* accepted) {
         }
         if (got != kTuneKeyInts + 1) return fail(LQ_ERR_VALUE, "tune_import: malformed line '%s'", line.c_str());
         const int shape = v[kTuneKeyInts] & 0xff;
-        if (shape < 1 || shape > 19) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
+        if (shape < 1 || shape > 20) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
         TuneKey key;
         std::memcpy(&key, v, sizeof(key));
         std::lock_guard<std::mutex> lock(g_tune_mu);
@@ -325,6 +334,7 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
             if (boxes256 < 1024 && conv_halo_applies(g, conv, 7)) cands[n++] = 18;
             if (boxes256 < 512 && conv_halo_applies(g, conv, 6)) cands[n++] = 19;
         }
+        if (conv_few_applies(g, conv, groups)) cands[n++] = 20;
         // whole rounds of 256 x 256 tiles plus a remainder (see launch_split)
         if (!conv && groups == 1 && g.range == nullptr && g.M >= 256) {
             const long tiles_m = (g.M + 255) / 256, tiles_n = g.N / 256;

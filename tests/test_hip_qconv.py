@@ -318,6 +318,55 @@ def test_float_image_quantized_into_the_packed_form(B, H, W, Cin, Cout, KH, KW, 
     assert np.array_equal(_ops.qconv2d_i8(hip(xq), dw, **kw).numpy(), want)
 
 
+@pytest.mark.parametrize("B,H,W,Cin,Cout,KH,KW,stride,pad,dil_h", [
+    (2, 224, 224, 3, 64, 7, 7, (2, 2), (3, 3, 3, 3), 1),    # the ResNet stem: whole 16-byte stores
+    (3, 17, 13, 3, 24, 3, 3, (1, 1), (1, 1, 1, 1), 1),      # one k step, a partial column tile
+    (2, 20, 9, 1, 16, 5, 2, (2, 1), (2, 1, 0, 1), 2),       # dilated rows, one channel
+    (2, 11, 11, 4, 40, 3, 5, (1, 3), (0, 0, 2, 2), 1),      # stride 3 along the row
+    (1, 40, 37, 3, 160, 5, 5, (1, 2), (2, 2, 2, 2), 1),     # three column tiles, the last one partial
+    (5, 33, 70, 2, 128, 8, 8, (3, 1), (1, 2, 3, 4), 1),     # K = 256, boxes past the right edge
+])
+def test_few_channel_kernel_with_the_filter_in_registers(B, H, W, Cin, Cout, KH, KW, stride, pad, dil_h):
+    """tile_config 20 on the packed route: accumulators and every output form equal the oracle's."""
+    rng = np.random.default_rng(11 * B + H + Cout)
+    x = rng.integers(-128, 128, (B, H, W, Cin)).astype(np.int8)
+    w = rng.integers(-127, 128, (Cout, KH, KW, Cin)).astype(np.int8)
+    ws = (rng.random(Cout).astype(np.float32) + 0.5) * 1e-3
+    bias = rng.standard_normal(Cout).astype(np.float32) * 0.1
+    dx, dw = hip(x), hip(w)
+    geo = dict(stride=stride, pad=pad, dilation=(dil_h, 1))
+    acc = _ops.qconv2d_i8(dx, dw, a_zp=0, **geo, out_mode=_ops.OUT_ACC_I32, path=_ops.CONV_PACKED4, tile_config=20)
+    assert _C.load().lq_last_tile_config() & 0xff == 20
+    assert np.array_equal(acc.numpy(), O.qconv2d(x, w, 0, 1.0, np.ones(Cout, np.float32), **geo, out_mode=O.OUT_ACC_I32))
+    common = dict(a_zp=-7, a_scale=hip(np.float32(0.02)), w_scale=hip(ws), wsum=_ops.rowsum_i8(dw), bias=hip(bias), **geo,
+                  relu=True, path=_ops.CONV_PACKED4, tile_config=20)
+    ocommon = dict(**geo, bias=bias, relu=True)
+    for mode, omode in ((_ops.OUT_F32, O.OUT_F32), (_ops.OUT_F16, O.OUT_F16)):
+        got = _ops.qconv2d_i8(dx, dw, **common, out_mode=mode).numpy()
+        assert np.array_equal(got, O.qconv2d(x, w, -7, 0.02, ws, **ocommon, out_mode=omode))
+    for mode, omode, okw in ((_ops.OUT_REQUANT_I8, O.OUT_REQUANT_I8, dict(out_offset=-128)),
+                             (_ops.OUT_FAKEQUANT_F32, O.OUT_FAKEQUANT_F32, {})):
+        got = _ops.qconv2d_i8(dx, dw, **common, out_mode=mode, out_scale=hip(np.float32(0.05)),
+                              out_zp=hip(np.float32(3.0)), out_qmin=0, out_qmax=255, **okw).numpy()
+        want = O.qconv2d(x, w, -7, 0.02, ws, **ocommon, out_mode=omode, out_scale=0.05, out_zp=3.0, out_qmin=0,
+                         out_qmax=255, **okw)
+        assert np.array_equal(got, want)
+    # a signed output grid: the codes are not packed through the unsigned-byte conversion
+    got = _ops.qconv2d_i8(dx, dw, **common, out_mode=_ops.OUT_REQUANT_I8, out_scale=hip(np.float32(0.05)),
+                          out_zp=hip(np.float32(-20.0)), out_qmin=-128, out_qmax=127).numpy()
+    assert np.array_equal(got, O.qconv2d(x, w, -7, 0.02, ws, **ocommon, out_mode=O.OUT_REQUANT_I8, out_scale=0.05,
+                                         out_zp=-20.0, out_qmin=-128, out_qmax=127))
+
+
+def test_few_channel_kernel_declines_long_filter_rows():
+    x, w = hip(np.zeros((1, 20, 20, 3), np.int8)), hip(np.zeros((16, 11, 11, 3), np.int8))
+    with pytest.raises(NotImplementedError, match="K <= 256"):          # 11 x 12 x 4 = 528 bytes
+        _ops.qconv2d_i8(x, w, a_zp=0, out_mode=_ops.OUT_ACC_I32, path=_ops.CONV_PACKED4, tile_config=20)
+    x16, w16 = hip(np.zeros((1, 8, 8, 16), np.int8)), hip(np.zeros((16, 3, 3, 16), np.int8))
+    with pytest.raises(NotImplementedError, match="packed four-channel image"):
+        _ops.qconv2d_i8(x16, w16, a_zp=0, out_mode=_ops.OUT_ACC_I32, tile_config=20)
+
+
 @pytest.mark.parametrize("cin,relu,wzp,padding", [(3, True, 0, 3), (1, False, 0, "same"), (4, True, 0, 0),
                                                   (8, False, 0, 1), (3, False, 5, 1)])
 def test_conv_module_taking_the_quantize_module(cin, relu, wzp, padding):
