@@ -461,22 +461,36 @@ __global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__
 // v_mfma_f32_16x16x32_bf16 runs sixteen times the rate of v_mfma_f32_16x16x4_f32: six
 // instructions of the one replace eight of the other at a sixth of the time each.
 //
+// The three parts of K (row-major) and of V^T ([column][key]) are both in LDS from the start -
+// 79 872 + 81 408 bytes of the CU's 160 KiB - so after the one barrier that follows the splits
+// a wavefront runs scores, softmax and P . V on its own, and the 13 wavefronts (four on one
+// SIMD, three on the others) drift apart instead of waiting for each other between phases.
+//
 // Per wavefront: S^T = K . Q^T as 13 tiles of 16 keys x 16 queries (accumulators stay in
-// registers; K's three parts in LDS, split once per block), softmax over the keys of each
-// query (a lane holds 52 of a query's keys, the other three lane groups the rest), then
-// O = P . V where the S^T accumulators ARE the A operand: register r of tile t holds
-// P[query = lane%16][key = 16t + 4*(lane/16) + r], so two tiles give a lane the eight k slots
-// of an instruction, which is a valid k-slice assignment as long as V is read with the same
-// one: V^T's three parts replace K's in LDS after the scores ([column][key], so that a lane's
-// four keys of a tile are 8 contiguous bytes).
+// registers), softmax over the keys of each query (a lane holds 52 of a query's keys, the other
+// three lane groups the rest), then O = P . V where the S^T accumulators ARE the A operand:
+// register r of tile t holds P[query = lane%16][key = 16t + 4*(lane/16) + r], so two tiles give
+// a lane the eight k slots of an instruction, which is a valid k-slice assignment as long as V
+// is read with the same one ([column][key] keeps a lane's four keys of a tile in 8 contiguous
+// bytes); the thirteenth tile goes through the 16-key form of the instruction alone.
 constexpr int AT_D = 64, AT_TMAX = 208;
-constexpr int AT_KLD = AT_D + 8;          // bfloat16 per K row: 144 bytes, the 16 rows of a fragment on 16 bank groups
-constexpr int AT_KEYS = AT_TMAX + 16;     // keys of V^T: tiles pair up, the fourteenth is zero
-constexpr int AT_VLD = AT_KEYS + 4;       // bfloat16 per V^T row: 456 bytes
-constexpr int AT_PART_K = AT_TMAX * AT_KLD, AT_PART_V = AT_D * AT_VLD;  // elements of one part
-constexpr size_t AT_SMEM = size_t(3) * (AT_PART_K > AT_PART_V ? AT_PART_K : AT_PART_V) * 2;
+// K: rows of 64 bfloat16 = 128 bytes = all 32 banks; the 16-byte chunk k of row r sits at chunk
+// k ^ (r % 8), so the 16 rows of a fragment (same logical chunk) cover every bank exactly twice
+constexpr int AT_PART_K = AT_TMAX * AT_D;
+// V^T: 106 dwords per row = 10 mod 32: the 16 rows a fragment reads (8 bytes each) fall on 16
+// different bank pairs
+constexpr int AT_VLD = AT_TMAX + 4;
+constexpr int AT_PART_V = AT_D * AT_VLD;  // elements of one part
+constexpr size_t AT_K_BYTES = size_t(3) * AT_PART_K * 2;
+constexpr size_t AT_SMEM = AT_K_BYTES + size_t(3) * AT_PART_V * 2;
+static_assert(AT_SMEM + 1024 <= 160 * 1024, "LDS of a CU, with the range reduction's few words");
 
 typedef __bf16 at_v8bf __attribute__((ext_vector_type(8)));
+typedef short at_v4s __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int at_k_index(int row, int col) {  // col a multiple of 4
+    return row * AT_D + ((((col >> 3) ^ (row & 7)) << 3) | (col & 7));
+}
 
 // (e0, e1) = h + m + l part by part, each part a pair of bfloat16 (e0's in the low half): the
 // packed conversion rounds to nearest, the remainders are exact (8 + 8 + 8 significant bits with
@@ -509,49 +523,116 @@ __device__ __forceinline__ v4f at_mma6(const uint4 (&a)[3], const uint4 (&b)[3],
     mm(a[0], b[0]);
     return acc;
 }
+// the same over 16 k slots (four per lane)
+__device__ __forceinline__ v4f at_mma6_k16(const uint2 (&a)[3], const uint2 (&b)[3], v4f acc) {
+    auto mm = [&](const uint2& x, const uint2& y) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(at_v4s, x), __builtin_bit_cast(at_v4s, y), acc,
+                                                        0, 0, 0);
+    };
+    mm(a[1], b[1]);
+    mm(a[0], b[2]);
+    mm(a[2], b[0]);
+    mm(a[0], b[1]);
+    mm(a[1], b[0]);
+    mm(a[0], b[0]);
+    return acc;
+}
 
 __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict__ qkv, float* __restrict__ out,
                                                         int B, int T, int H, float scale, float* range) {
     extern __shared__ __attribute__((aligned(16))) uint16_t at_smem[];
+    uint16_t* const k_lds = at_smem;
+    uint16_t* const v_lds = at_smem + 3 * AT_PART_K;
     const int b = blockIdx.x / H, h = blockIdx.x % H;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t tok_stride = size_t(3) * H * AT_D;
     const float* base = qkv + size_t(b) * T * tok_stride + size_t(h) * AT_D;
-    // V is requested now (up to four 16-byte pieces per thread: all of it for 13 wavefronts) and laid
-    // out after the scores
+    // K and V are requested before anything is used (a block of 13 wavefronts holds all of both: four
+    // 16-byte pieces of each per thread).  A thread's V pieces are two pairs of consecutive keys at the
+    // same four columns: V^T keeps a column's keys contiguous, so a pair of keys is one dword of each part
     constexpr int kPieces = AT_TMAX * (AT_D / 4), kHeld = 4;
-    float4 vheld[kHeld];
+    constexpr int kPairs = (AT_TMAX / 2) * (AT_D / 4);
+    float4 kheld[kHeld], vheld[kHeld];
 #pragma unroll
     for (int u = 0; u < kHeld; ++u) {
         const int i = tid + u * int(blockDim.x), row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
-        vheld[u] = float4{0.f, 0.f, 0.f, 0.f};
-        if (i < kPieces && row < T) vheld[u] = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(2) * H * AT_D + c4);
+        kheld[u] = float4{0.f, 0.f, 0.f, 0.f};
+        if (i < kPieces && row < T) kheld[u] = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(H) * AT_D + c4);
     }
-    // K rows into LDS as three bfloat16 parts (rows past T are zero)
-    for (int i = tid; i < kPieces; i += blockDim.x) {
-        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
-        float4 kv = {0.f, 0.f, 0.f, 0.f};
-        if (row < T) kv = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(H) * AT_D + c4);
-        uint32_t lo[3], hi[3];
-        at_split3x2(kv.x, kv.y, lo[0], lo[1], lo[2]);
-        at_split3x2(kv.z, kv.w, hi[0], hi[1], hi[2]);
 #pragma unroll
-        for (int p = 0; p < 3; ++p)
-            *reinterpret_cast<uint2*>(at_smem + p * AT_PART_K + row * AT_KLD + c4) = uint2{lo[p], hi[p]};
+    for (int u = 0; u < kHeld; ++u) {
+        const int i = tid + (u >> 1) * int(blockDim.x), row = 2 * (i / (AT_D / 4)) + (u & 1), c4 = (i % (AT_D / 4)) * 4;
+        vheld[u] = float4{0.f, 0.f, 0.f, 0.f};
+        if (i < kPairs && row < T) vheld[u] = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(2) * H * AT_D + c4);
     }
     const int q0 = wave * 16;  // the launch has exactly ceil(T / 16) wavefronts, so q0 < T
     const int g = lane >> 4, c = lane & 15;
-    // B operand of S^T: Q[q0 + c][32 u + 8 g + 0..7], pre-scaled so that S = scale * log2(e) * Q.K^T
-    // (the scores are kept in the base-2 domain, so that the softmax numerators are one v_exp_f32 each)
-    uint4 qf[AT_D / 32][3];
+    // the lane's slice of its query row: Q[q0 + c][32 u + 8 g + 0..7]
+    float4 qheld[2 * (AT_D / 32)];
     {
         const int q = q0 + c;
         const float* qp = base + size_t(q < T ? q : T - 1) * tok_stride;
+#pragma unroll
+        for (int u = 0; u < AT_D / 32; ++u) {
+            qheld[2 * u] = *reinterpret_cast<const float4*>(qp + 32 * u + 8 * g);
+            qheld[2 * u + 1] = *reinterpret_cast<const float4*>(qp + 32 * u + 8 * g + 4);
+        }
+    }
+    // K rows into LDS as three bfloat16 parts (rows past T are zero)
+    auto place_k = [&](int i, float4 kv) {
+        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        uint32_t lo[3], hi[3];
+        at_split3x2(kv.x, kv.y, lo[0], lo[1], lo[2]);
+        at_split3x2(kv.z, kv.w, hi[0], hi[1], hi[2]);
+        const int at = at_k_index(row, c4);
+#pragma unroll
+        for (int p = 0; p < 3; ++p) *reinterpret_cast<uint2*>(k_lds + p * AT_PART_K + at) = uint2{lo[p], hi[p]};
+    };
+#pragma unroll
+    for (int u = 0; u < kHeld; ++u) {
+        const int i = tid + u * int(blockDim.x);
+        if (i < kPieces) place_k(i, kheld[u]);
+    }
+    for (int i = tid + kHeld * int(blockDim.x); i < kPieces; i += blockDim.x) {  // fewer than 13 wavefronts
+        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        float4 kv = {0.f, 0.f, 0.f, 0.f};
+        if (row < T) kv = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(H) * AT_D + c4);
+        place_k(i, kv);
+    }
+    // V^T's parts: keys 2 pair and 2 pair + 1 at columns c4 .. c4 + 3 (keys past T are zero)
+    auto place_v = [&](int i, float4 v0, float4 v1) {
+        const int pair = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        const float a[4] = {v0.x, v0.y, v0.z, v0.w}, bb[4] = {v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            uint32_t d[3];
+            at_split3x2(a[e], bb[e], d[0], d[1], d[2]);
+#pragma unroll
+            for (int p = 0; p < 3; ++p)
+                *reinterpret_cast<uint32_t*>(v_lds + p * AT_PART_V + (c4 + e) * AT_VLD + 2 * pair) = d[p];
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < kHeld / 2; ++u) {
+        const int i = tid + u * int(blockDim.x);
+        if (i < kPairs) place_v(i, vheld[2 * u], vheld[2 * u + 1]);
+    }
+    for (int i = tid + (kHeld / 2) * int(blockDim.x); i < kPairs; i += blockDim.x) {  // fewer than 13 wavefronts
+        const int pair = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
+        float4 v0 = {0.f, 0.f, 0.f, 0.f}, v1 = {0.f, 0.f, 0.f, 0.f};
+        const float* vp = base + size_t(2) * H * AT_D + c4;
+        if (2 * pair < T) v0 = *reinterpret_cast<const float4*>(vp + size_t(2 * pair) * tok_stride);
+        if (2 * pair + 1 < T) v1 = *reinterpret_cast<const float4*>(vp + size_t(2 * pair + 1) * tok_stride);
+        place_v(i, v0, v1);
+    }
+    // B operand of S^T, pre-scaled so that S = scale * log2(e) * Q.K^T (the scores are kept in the
+    // base-2 domain, so that the softmax numerators are one v_exp_f32 each)
+    uint4 qf[AT_D / 32][3];
+    {
         const float qs = scale * 1.4426950408889634f;
 #pragma unroll
         for (int u = 0; u < AT_D / 32; ++u) {
-            const float4 a = *reinterpret_cast<const float4*>(qp + 32 * u + 8 * g);
-            const float4 bq = *reinterpret_cast<const float4*>(qp + 32 * u + 8 * g + 4);
+            const float4 a = qheld[2 * u], bq = qheld[2 * u + 1];
             const float v[8] = {a.x * qs, a.y * qs, a.z * qs, a.w * qs, bq.x * qs, bq.y * qs, bq.z * qs, bq.w * qs};
             uint32_t d[3][4];
 #pragma unroll
@@ -560,7 +641,7 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
             for (int p = 0; p < 3; ++p) qf[u][p] = uint4{d[p][0], d[p][1], d[p][2], d[p][3]};
         }
     }
-    __syncthreads();
+    __syncthreads();  // the only one before the range reduction: from here on a wavefront is on its own
     constexpr int NT = AT_TMAX / 16;
     v4f st[NT];
 #pragma unroll
@@ -571,9 +652,9 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             uint4 kf[3];
+            const int at = at_k_index(16 * t + c, 32 * u + 8 * g);
 #pragma unroll
-            for (int p = 0; p < 3; ++p)
-                kf[p] = *reinterpret_cast<const uint4*>(at_smem + p * AT_PART_K + (16 * t + c) * AT_KLD + 32 * u + 8 * g);
+            for (int p = 0; p < 3; ++p) kf[p] = *reinterpret_cast<const uint4*>(k_lds + p * AT_PART_K + at);
             st[t] = at_mma6(kf, qf[u], st[t]);
         }
     // st[t][r] = S[query q0 + c][key 16t + 4g + r]
@@ -601,51 +682,21 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
     sum += __shfl_xor(sum, 32, 64);
     const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
 
-    // V^T's parts take K's place: [column][key], keys past T (and the fourteenth tile) zero
-    __syncthreads();  // every wavefront has read its K fragments
-    for (int i = tid; i < 3 * AT_D * (AT_KEYS - AT_TMAX) / 2; i += blockDim.x) {
-        const int p = i / (AT_D * (AT_KEYS - AT_TMAX) / 2), rest = i % (AT_D * (AT_KEYS - AT_TMAX) / 2);
-        const int n = rest / ((AT_KEYS - AT_TMAX) / 2), k2 = rest % ((AT_KEYS - AT_TMAX) / 2);
-        *reinterpret_cast<uint32_t*>(at_smem + p * AT_PART_V + n * AT_VLD + AT_TMAX + 2 * k2) = 0u;
-    }
-    auto place_v = [&](int i, float4 vv) {
-        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
-        uint32_t lo[3], hi[3];
-        at_split3x2(vv.x, vv.y, lo[0], lo[1], lo[2]);
-        at_split3x2(vv.z, vv.w, hi[0], hi[1], hi[2]);
-#pragma unroll
-        for (int p = 0; p < 3; ++p) {
-            uint16_t* col = at_smem + p * AT_PART_V + c4 * AT_VLD + row;
-            col[0] = uint16_t(lo[p]), col[AT_VLD] = uint16_t(lo[p] >> 16);
-            col[2 * AT_VLD] = uint16_t(hi[p]), col[3 * AT_VLD] = uint16_t(hi[p] >> 16);
-        }
-    };
-#pragma unroll
-    for (int u = 0; u < kHeld; ++u) {
-        const int i = tid + u * int(blockDim.x);
-        if (i < kPieces) place_v(i, vheld[u]);
-    }
-    for (int i = tid + kHeld * int(blockDim.x); i < kPieces; i += blockDim.x) {  // fewer than 13 wavefronts
-        const int row = i / (AT_D / 4), c4 = (i % (AT_D / 4)) * 4;
-        float4 vv = {0.f, 0.f, 0.f, 0.f};
-        if (row < T) vv = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(2) * H * AT_D + c4);
-        place_v(i, vv);
-    }
-    __syncthreads();
-
     // O[q][n] = sum_key P[q][key] V[key][n], four 16-wide column tiles; tile j of the output holds
-    // head-dim columns 4 c + j (not 16 j + c), so that a lane stores four consecutive floats
+    // head-dim columns 16 j + c: the 16 lanes of a fragment read consecutive V^T rows (rows 4 c + j,
+    // which would let a lane store four consecutive floats, fall on four bank pairs only)
+    static_assert(NT % 2 == 1, "tile pairs and one single tile");
     v4f o[AT_D / 16];
 #pragma unroll
     for (int j = 0; j < AT_D / 16; ++j) o[j] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int tp = 0; tp < (NT + 1) / 2; ++tp) {
+    for (int tp = 0; tp < NT / 2; ++tp) {
         // the eight k slots of this lane: keys 32 tp + 4 g + 0..3 and 32 tp + 16 + 4 g + 0..3
         float pv[8];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             pv[r] = st[2 * tp][r] * inv;
-            pv[4 + r] = 2 * tp + 1 < NT ? st[2 * tp + 1 < NT ? 2 * tp + 1 : 0][r] * inv : 0.0f;
+            pv[4 + r] = st[2 * tp + 1][r] * inv;
         }
         uint32_t d[3][4];
 #pragma unroll
@@ -658,20 +709,43 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
             uint4 vf[3];
 #pragma unroll
             for (int p = 0; p < 3; ++p) {
-                const uint16_t* vrow = at_smem + p * AT_PART_V + (4 * c + j) * AT_VLD + 32 * tp + 4 * g;
+                const uint16_t* vrow = v_lds + p * AT_PART_V + (16 * j + c) * AT_VLD + 32 * tp + 4 * g;
                 const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
                 vf[p] = uint4{lo.x, lo.y, hi.x, hi.y};
             }
             o[j] = at_mma6(pf, vf, o[j]);
         }
     }
-    // result layout of the 16x16 MFMA: column slot = lane % 16, row = 4*(lane/16) + r
+    {
+        // the last tile: keys 16 (NT - 1) + 4 g + 0..3, four k slots per lane
+        float pv[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pv[r] = st[NT - 1][r] * inv;
+        uint32_t d[3][2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) at_split3x2(pv[2 * e], pv[2 * e + 1], d[0][e], d[1][e], d[2][e]);
+        uint2 pf[3];
+#pragma unroll
+        for (int p = 0; p < 3; ++p) pf[p] = uint2{d[p][0], d[p][1]};
+#pragma unroll
+        for (int j = 0; j < AT_D / 16; ++j) {
+            uint2 vf[3];
+#pragma unroll
+            for (int p = 0; p < 3; ++p)
+                vf[p] = *reinterpret_cast<const uint2*>(v_lds + p * AT_PART_V + (16 * j + c) * AT_VLD + 16 * (NT - 1) + 4 * g);
+            o[j] = at_mma6_k16(pf, vf, o[j]);
+        }
+    }
+    // result layout of the 16x16 MFMA: column slot = lane % 16, row = 4*(lane/16) + r; the 16 lanes
+    // of a row store 64 consecutive bytes
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int q = q0 + 4 * g + r;
-        if (q < T)
-            *reinterpret_cast<float4*>(out + (size_t(b) * T + q) * (size_t(H) * AT_D) + size_t(h) * AT_D + 4 * c) =
-                float4{o[0][r], o[1][r], o[2][r], o[3][r]};
+        if (q < T) {
+            float* orow = out + (size_t(b) * T + q) * (size_t(H) * AT_D) + size_t(h) * AT_D + c;
+#pragma unroll
+            for (int j = 0; j < AT_D / 16; ++j) orow[16 * j] = o[j][r];
+        }
     }
     if (range) {
         float lo = __builtin_inff(), hi = -__builtin_inff();
