@@ -339,22 +339,52 @@ __global__ __launch_bounds__(256) void assemble_tokens_kernel(const float* __res
     out[i] = v + pos[size_t(t) * D + d];
 }
 
-// ---------------------------------------------------------------- float32 GEMM, out = a . w^T + bias
-// 128 x 128 x 16 block tile, 4 wavefronts of 64 x 64, v_mfma_f32_32x32x2_f32.
-// LDS tiles are k-major ([k][row], rows padded) so that a fragment read takes
-// consecutive words.
-constexpr int SG_BM = 128, SG_BN = 128, SG_BK = 16, SG_LD = 128 + 4;
+// (e0, e1) = h + m + l part by part, each part a pair of bfloat16 (e0's in the low half): the
+// packed conversion rounds to nearest, the remainders are exact (8 + 8 + 8 significant bits with
+// signed remainders).  A NaN stays a NaN in every part; an infinity turns into a NaN in the
+// lower parts, so a non-finite input gives a non-finite output.
+typedef __bf16 at_bf2 __attribute__((ext_vector_type(2)));
+typedef float at_f2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t at_pk(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(at_f2{a, b}, at_bf2));
+}
+__device__ __forceinline__ void at_split3x2(float e0, float e1, uint32_t& h, uint32_t& m, uint32_t& l) {
+    h = at_pk(e0, e1);
+    e0 -= __uint_as_float(h << 16), e1 -= __uint_as_float(h & 0xffff0000u);
+    m = at_pk(e0, e1);
+    e0 -= __uint_as_float(m << 16), e1 -= __uint_as_float(m & 0xffff0000u);
+    l = at_pk(e0, e1);
+}
 
-__global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__ a, const float* __restrict__ w,
-                                                       const float* __restrict__ bias, float* __restrict__ out,
-                                                       int M, int N, int K) {
-    __shared__ float sa[2][SG_BK][SG_LD];
-    __shared__ float sb[2][SG_BK][SG_LD];
+typedef __bf16 sg_v8bf __attribute__((ext_vector_type(8)));
+
+// ---------------------------------------------------------------- float32 GEMM, out = a . w^T + bias
+// float32 operands on the bfloat16 matrix instruction: both operands are split into three
+// bfloat16 parts when a tile is written to LDS (at_split3x2), and six part products per k step
+// (hi.hi, hi.mid, mid.hi, hi.lo, lo.hi, mid.mid, smallest first, accumulated in float32) give
+// every product 2^-24 relative accuracy - a float32 GEMM at six instructions of
+// v_mfma_f32_32x32x16_bf16 per 16 k, against eight of v_mfma_f32_32x32x2_f32 at four times the
+// cycles each.
+//
+// 128 x 128 x 32 block tile, 4 wavefronts of 64 x 64; the next tile's operands wait in registers
+// while the current one is multiplied.  LDS: per part 256 rows (A's 128, then W's) of 32
+// bfloat16 = 64 bytes; the 16-byte chunk k of row r sits at chunk k ^ ((r / 4) % 4), which puts
+// the 16 rows of a fragment pass on 16 different bank groups.
+constexpr int SG_BM = 128, SG_BN = 128, SG_BK = 32, SG_ROWS = SG_BM + SG_BN;
+
+__device__ __forceinline__ int sg_index(int row, int k) {  // k a multiple of 4
+    return row * SG_BK + ((((k >> 3) ^ ((row >> 2) & 3)) << 3) | (k & 7));
+}
+
+__global__ __launch_bounds__(256, 2) void sgemm_nt_kernel(const float* __restrict__ a, const float* __restrict__ w,
+                                                          const float* __restrict__ bias, float* __restrict__ out,
+                                                          int M, int N, int K) {
+    __shared__ __attribute__((aligned(16))) uint16_t sp[3][SG_ROWS * SG_BK];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.y * SG_BM, n0 = blockIdx.x * SG_BN;
-    // loader: thread -> (row = tid / 4 (+64), 4 consecutive k at 4 * (tid % 4))
-    const int lrow = tid >> 2, lk = (tid & 3) * 4;
+    // loader: piece tid + 256 u = row (tid + 256 u) / 8 of either operand, four consecutive k at 4 * (tid % 8)
+    const int lrow = tid >> 3, lk = (tid & 7) * 4;
     const bool vec = (K % 4 == 0) && aligned16(a) && aligned16(w);
     v16f acc[2][2];
 #pragma unroll
@@ -364,73 +394,78 @@ __global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    float4 ra[2], rb[2];
+    float4 ra[4], rb[4];
+    auto fetch_row = [&](const float* base, int row, int rows, int k) {
+        float4 v = {0.f, 0.f, 0.f, 0.f};
+        if (row < rows) {
+            const float* p = base + size_t(row) * K + k;
+            if (vec && k + 3 < K) {
+                v = *reinterpret_cast<const float4*>(p);
+            } else {
+                if (k < K) v.x = p[0];
+                if (k + 1 < K) v.y = p[1];
+                if (k + 2 < K) v.z = p[2];
+                if (k + 3 < K) v.w = p[3];
+            }
+        }
+        return v;
+    };
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int m = m0 + lrow + 64 * h, n = n0 + lrow + 64 * h, k = k0 + lk;
-            float4 va = {0.f, 0.f, 0.f, 0.f}, vb = {0.f, 0.f, 0.f, 0.f};
-            if (m < M) {
-                const float* p = a + size_t(m) * K + k;
-                if (vec && k + 3 < K) {
-                    va = *reinterpret_cast<const float4*>(p);
-                } else {
-                    if (k < K) va.x = p[0];
-                    if (k + 1 < K) va.y = p[1];
-                    if (k + 2 < K) va.z = p[2];
-                    if (k + 3 < K) va.w = p[3];
-                }
-            }
-            if (n < N) {
-                const float* p = w + size_t(n) * K + k;
-                if (vec && k + 3 < K) {
-                    vb = *reinterpret_cast<const float4*>(p);
-                } else {
-                    if (k < K) vb.x = p[0];
-                    if (k + 1 < K) vb.y = p[1];
-                    if (k + 2 < K) vb.z = p[2];
-                    if (k + 3 < K) vb.w = p[3];
-                }
-            }
-            ra[h] = va;
-            rb[h] = vb;
+        for (int u = 0; u < 4; ++u) {
+            ra[u] = fetch_row(a, m0 + lrow + 32 * u, M, k0 + lk);
+            rb[u] = fetch_row(w, n0 + lrow + 32 * u, N, k0 + lk);
         }
     };
-    auto stash = [&](int buf) {
+    auto stash_one = [&](int row, float4 v) {
+        uint32_t lo[3], hi[3];
+        at_split3x2(v.x, v.y, lo[0], lo[1], lo[2]);
+        at_split3x2(v.z, v.w, hi[0], hi[1], hi[2]);
+        const int at = sg_index(row, lk);
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int r = lrow + 64 * h;
-            sa[buf][lk][r] = ra[h].x, sa[buf][lk + 1][r] = ra[h].y, sa[buf][lk + 2][r] = ra[h].z,
-            sa[buf][lk + 3][r] = ra[h].w;
-            sb[buf][lk][r] = rb[h].x, sb[buf][lk + 1][r] = rb[h].y, sb[buf][lk + 2][r] = rb[h].z,
-            sb[buf][lk + 3][r] = rb[h].w;
+        for (int p = 0; p < 3; ++p) *reinterpret_cast<uint2*>(&sp[p][at]) = uint2{lo[p], hi[p]};
+    };
+    auto stash = [&] {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            stash_one(lrow + 32 * u, ra[u]);
+            stash_one(SG_BM + lrow + 32 * u, rb[u]);
         }
     };
     const int nk = (K + SG_BK - 1) / SG_BK;
+    const int fr = lane & 31, kg = lane >> 5;
     fetch(0);
-    stash(0);
-    __syncthreads();
     for (int t = 0; t < nk; ++t) {
-        const int buf = t & 1;
+        stash();
+        __syncthreads();
         if (t + 1 < nk) fetch((t + 1) * SG_BK);
 #pragma unroll
-        for (int kk = 0; kk < SG_BK; kk += 2) {
-            const int kr = kk + (lane >> 5);
-            float fa[2], fb[2];
+        for (int ks = 0; ks < SG_BK / 16; ++ks) {
+            uint4 fa[2][3], fb[2][3];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) fa[i] = sa[buf][kr][wm * 64 + i * 32 + (lane & 31)];
+            for (int i = 0; i < 2; ++i) {
+                const int at = sg_index(wm * 64 + i * 32 + fr, 16 * ks + 8 * kg);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) fb[j] = sb[buf][kr][wn * 64 + j * 32 + (lane & 31)];
+                for (int p = 0; p < 3; ++p) fa[i][p] = *reinterpret_cast<const uint4*>(&sp[p][at]);
+            }
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int j = 0; j < 2; ++j) {
+                const int at = sg_index(SG_BM + wn * 64 + j * 32 + fr, 16 * ks + 8 * kg);
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                for (int p = 0; p < 3; ++p) fb[j][p] = *reinterpret_cast<const uint4*>(&sp[p][at]);
+            }
+            auto mm = [&](int pa, int pb) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(sg_v8bf, fa[i][pa]),
+                                                                            __builtin_bit_cast(sg_v8bf, fb[j][pb]),
+                                                                            acc[i][j], 0, 0, 0);
+            };
+            mm(1, 1), mm(0, 2), mm(2, 0), mm(0, 1), mm(1, 0), mm(0, 0);
         }
-        if (t + 1 < nk) {
-            stash(buf ^ 1);  // the other buffer was last read one iteration ago, behind a barrier
-            __syncthreads();
-        }
+        __syncthreads();  // the tile has been read: the next one may be written
     }
     // result layout of the 32x32 MFMA: column = lane % 32, row = 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
@@ -490,23 +525,6 @@ typedef short at_v4s __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int at_k_index(int row, int col) {  // col a multiple of 4
     return row * AT_D + ((((col >> 3) ^ (row & 7)) << 3) | (col & 7));
-}
-
-// (e0, e1) = h + m + l part by part, each part a pair of bfloat16 (e0's in the low half): the
-// packed conversion rounds to nearest, the remainders are exact (8 + 8 + 8 significant bits with
-// signed remainders).  A NaN stays a NaN in every part; an infinity turns into a NaN in the
-// lower parts, so a non-finite input gives a non-finite output.
-typedef __bf16 at_bf2 __attribute__((ext_vector_type(2)));
-typedef float at_f2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t at_pk(float a, float b) {
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(at_f2{a, b}, at_bf2));
-}
-__device__ __forceinline__ void at_split3x2(float e0, float e1, uint32_t& h, uint32_t& m, uint32_t& l) {
-    h = at_pk(e0, e1);
-    e0 -= __uint_as_float(h << 16), e1 -= __uint_as_float(h & 0xffff0000u);
-    m = at_pk(e0, e1);
-    e0 -= __uint_as_float(m << 16), e1 -= __uint_as_float(m & 0xffff0000u);
-    l = at_pk(e0, e1);
 }
 
 // acc += a * b from the parts, smallest terms first

@@ -431,6 +431,14 @@ __device__ __forceinline__ void wq_split3x2(float e0, float e1, uint32_t& h, uin
 constexpr int kWqRows = 256;    // weight rows per block
 constexpr int kWqSliceK = 512;  // k per block
 
+// Where the A fragment of row m, lane quarter qd of instruction block `blk` sits among the block's
+// 64 16-byte slots.  The threads of a wavefront that write the fragments share one m and differ in
+// (block, quarter): with the plain slot m + 16 qd they would all hit the same four banks (a
+// 64-way conflict: the writes took a tenth of the kernel); rotating m by 4 qd + blk spreads them
+// evenly over the 16 bank groups.  A bijection within the block, so the reads of a whole block
+// stay conflict-free.
+__device__ __forceinline__ int wq_x_slot(int m, int qd, int blk) { return ((m + 4 * qd + blk) & 15) + 16 * qd; }
+
 template <int BITS, int SW>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void wq_mfma_kernel(
     const float* x, const uint32_t* packed, const float* scales, const float* biases, int M, int N, int K,
@@ -564,7 +572,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             if (wi < nw) {
 #pragma unroll
                 for (int p = 0; p < 3; ++p)
-                    x_lds[((wi * NI + i) * 3 + p) * 64 + ml + 16 * qd] = uint4{d3[p][0], d3[p][1], d3[p][2], d3[p][3]};
+                    x_lds[((wi * NI + i) * 3 + p) * 64 + wq_x_slot(ml, qd, wi * NI + i)] = uint4{d3[p][0], d3[p][1], d3[p][2], d3[p][3]};
             }
         }
     }
@@ -625,7 +633,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                     }
 #pragma unroll
                     for (int p = 0; p < 3; ++p) {
-                        const v8bf xf = __builtin_bit_cast(v8bf, x_lds[((wi * NI + i) * 3 + p) * 64 + lane]);
+                        const v8bf xf = __builtin_bit_cast(v8bf, x_lds[((wi * NI + i) * 3 + p) * 64 + wq_x_slot(lane & 15, lane >> 4, wi * NI + i)]);
 #pragma unroll
                         for (int rb = 0; rb < RB; ++rb)
                             acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, __builtin_bit_cast(v8bf, cf[rb]),
