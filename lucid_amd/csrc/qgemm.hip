@@ -119,8 +119,11 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
 
 // Whether the eight-wavefront ping-pong kernel (shapes 13 and 14) can run the problem.
 bool pp_applies(const GemmArgs& g, int conv, int groups) {
-    return !conv && groups == 1 && g.K > 0 && g.K % 64 == 0 && g.M >= 256 && g.N >= 256 && !g.gelu &&
-           g.range == nullptr && size_t(g.M) * g.K < 0xffffffffull && size_t(g.N) * g.K < 0xffffffffull;
+    // (a kept range needs a slot per tile: the shapes' tiles are at least 256 x 192)
+    return !conv && groups == 1 && g.K > 0 && g.K % 64 == 0 && g.M >= 256 && g.N >= 256 &&
+           ((!g.gelu && g.range == nullptr) || g.out_mode == OUT_F32) &&
+           (g.range == nullptr || long((g.M + 255) / 256) * ((g.N + 191) / 192) <= 16384) &&
+           size_t(g.M) * g.K < 0xffffffffull && size_t(g.N) * g.K < 0xffffffffull;
 }
 
 // Shape chosen from the problem size alone (what a launch gets when the tuner may not run: a

@@ -211,7 +211,9 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(1,
     asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
     __builtin_amdgcn_s_waitcnt(pp_vmcnt_imm(0));  // no direct load may land in LDS after this wavefront has ended
     __builtin_amdgcn_sched_barrier(0);
-    pp_epilogue<TM, TN, MODE>(g, acc, as_row, s_ws, s_bias, s_corr, n0, wm0, wn0, lane, rot);
+    float r_lo = 0.0f, r_hi = 0.0f;  // (no kept range in this kernel's output forms)
+    int r_nan = 0;
+    pp_epilogue<TM, TN, MODE>(g, acc, as_row, s_ws, s_bias, s_corr, n0, wm0, wn0, lane, rot, r_lo, r_hi, r_nan);
 }
 
 template <class Cfg, int MODE>

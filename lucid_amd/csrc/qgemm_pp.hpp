@@ -22,6 +22,7 @@
 #include "common.hpp"
 #include "qgemm.hpp"
 #include "qepilogue.hpp"
+#include "range_slots.hpp"
 
 #include <utility>
 
@@ -140,8 +141,16 @@ __device__ __forceinline__ int pp_rotation(const GemmArgs& g, int wn0) {
 template <int TM, int TN, int MODE>
 __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM][TN], const float (&as_row)[TM],
                                             const float* s_ws, const float* s_bias, const int32_t* s_corr, int n0,
-                                            int wm0, int wn0, int lane, int rot) {
+                                            int wm0, int wn0, int lane, int rot, float& r_lo, float& r_hi, int& r_nan) {
     if (wm0 >= g.M || wn0 >= g.N) return;
+    // running range of what this lane stores (float32 output with a kept range only)
+    const bool keep = MODE == OUT_F32X && g.range != nullptr;
+    auto track = [&](uint32_t bits) {
+        const float y = __uint_as_float(bits);
+        r_nan |= (y != y);
+        r_lo = fminf(r_lo, y);
+        r_hi = fmaxf(r_hi, y);
+    };
     float S = 1.0f, Z = 0.0f;
     constexpr bool kRequant = MODE == OUT_REQUANT_I8 || MODE == OUT_REQUANT_JOIN || MODE == OUT_FAKEQUANT_F32;
     if (kRequant) {
@@ -319,11 +328,15 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
         const size_t idx = size_t(m) * size_t(g.ldo) + size_t(nq);
         if (vec_out) {
             store_vec4<MODE>(g, idx, v, cpk);
-        } else if (nq < g.N) {
-            store_scalar<MODE>(g, idx, finish_value<MODE>(g, v.x, m, nq, jp), cpk);
-            if (nq + 1 < g.N) store_scalar<MODE>(g, idx + 1, finish_value<MODE>(g, v.y, m, nq + 1, jp), cpk);
-            if (nq + 2 < g.N) store_scalar<MODE>(g, idx + 2, finish_value<MODE>(g, v.z, m, nq + 2, jp), cpk);
-            if (nq + 3 < g.N) store_scalar<MODE>(g, idx + 3, finish_value<MODE>(g, v.w, m, nq + 3, jp), cpk);
+        } else {
+            const uint32_t e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (nq + k < g.N) {
+                    const uint32_t f = finish_value<MODE>(g, e[k], m, nq + k, jp);
+                    if (MODE == OUT_F32X && keep) track(f);
+                    store_scalar<MODE>(g, idx + k, f, cpk);
+                }
         }
     };
     pp_static_for<kPairs>([&](auto x_tag) {
@@ -338,6 +351,10 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
             uint4 v, w;
             tile_values(m, acc[i][j], c4, as_row[i], nq, v);
             tile_values(m, acc[i][j + 1], d4, as_row[i], nq + 16, w);
+            if (MODE == OUT_F32X && keep && vec_out && (rows_in || m < g.M)) {
+                track(v.x), track(v.y), track(v.z), track(v.w);
+                track(w.x), track(w.y), track(w.z), track(w.w);
+            }
             if (!wide) {
                 store_own(m, nq, v);
                 store_own(m, nq + 16, w);
@@ -373,6 +390,7 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
             const int m = wm0 + 16 * i + (lane & 15);
             uint4 v;
             tile_values(m, acc[i][TN - 1], c4, as_row[i], nq, v);
+            if (MODE == OUT_F32X && keep && vec_out && (rows_in || m < g.M)) track(v.x), track(v.y), track(v.z), track(v.w);
             store_own(m, nq, v);
         }
     }
@@ -556,7 +574,12 @@ __global__ __launch_bounds__(Cfg::THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // ---- epilogue: no staging through LDS and no barrier; group 0 runs it while group 1 still
     // issues its last MFMAs.
     __builtin_amdgcn_s_waitcnt(pp_vmcnt_imm(0));  // no direct load may land in LDS after this wavefront has ended
-    pp_epilogue<TM, TN, MODE>(g, acc, as_row, s_ws, s_bias, s_corr, n0, wm0, wn0, lane, rot);
+    float r_lo = __builtin_inff(), r_hi = -__builtin_inff();
+    int r_nan = 0;
+    pp_epilogue<TM, TN, MODE>(g, acc, as_row, s_ws, s_bias, s_corr, n0, wm0, wn0, lane, rot, r_lo, r_hi, r_nan);
+    // one block per tile: the block's slot is the tile's (every wavefront has passed the same
+    // number of barriers by now)
+    if (MODE == OUT_F32X && g.range != nullptr) range_block_store(g.range, r_lo, r_hi, r_nan);
 }
 
 template <class Cfg, int MODE>
@@ -576,8 +599,13 @@ int launch_pp(const GemmArgs& g, hipStream_t st) {
     LQ_REQUIRE(g.K > 0 && g.K % 64 == 0, LQ_ERR_SHAPE, "ping-pong kernel: K = %d is not a multiple of 64", g.K);
     LQ_REQUIRE(size_t(g.M) * g.K < 0xffffffffull && size_t(g.N) * g.K < 0xffffffffull, LQ_ERR_SHAPE,
                "ping-pong kernel: an operand of 4 GiB or more");
-    LQ_REQUIRE(!g.gelu && g.range == nullptr, LQ_ERR_NOT_IMPLEMENTED,
-               "ping-pong kernel: GELU / kept range are not built for it");
+    if (g.gelu || g.range != nullptr) {
+        LQ_REQUIRE(g.out_mode == OUT_F32, LQ_ERR_VALUE, "ping-pong kernel: GELU / a kept range go with float32 output");
+        const long tiles = long((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
+        LQ_REQUIRE(g.range == nullptr || tiles <= kRangeSlots, LQ_ERR_SHAPE,
+                   "ping-pong kernel: %ld tiles are too many for a kept range", tiles);
+        return launch_pp_mode<Cfg, OUT_F32X>(g, st);
+    }
     switch (g.out_mode) {
     case OUT_ACC_I32: return launch_pp_mode<Cfg, OUT_ACC_I32>(g, st);
     case OUT_F32: return launch_pp_mode<Cfg, OUT_F32>(g, st);

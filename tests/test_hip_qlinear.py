@@ -531,6 +531,54 @@ def test_ping_pong_kernel_every_output_form(cfg, M, N, K):
         assert np.array_equal(fused, expj.reshape(M, N))
 
 
+@pytest.mark.parametrize("cfg", [13, 14, 16])
+@pytest.mark.parametrize("M,N,K", [(512, 704, 256), (300, 260, 128), (129, 1001, 64), (1576, 3072, 768)])
+def test_ping_pong_kernel_gelu_and_kept_range(cfg, M, N, K):
+    """GELU in the epilogue and the kept range of what is stored, on the eight-wavefront kernel:
+    the bits of the four-wavefront tile kernel (which the stand-alone GELU kernel is tested
+    against), with and without a residual, and exactly the minimum and maximum of the result -
+    rows and columns of edge tiles past the matrix do not count, a NaN does."""
+    from lucid_amd import _C
+    rng = np.random.default_rng(cfg * 31 + M + N + K)
+    a, w = codes(rng, (M, K), -100, 100), codes(rng, (N, K), -100, 100)
+    ad, wd = hip(a), hip(w)
+    per_row = cfg != 14
+    a_scale = rng.uniform(0.002, 0.01, M if per_row else 1).astype(np.float32)
+    w_scale = rng.uniform(0.0005, 0.004, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.3).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    common = dict(a_zp=5, a_scale=hip(a_scale), w_scale=hip(w_scale), wsum=_ops.rowsum_i8(wd), bias=hip(bias),
+                  out_mode=_ops.OUT_F32, path=TILE)
+
+    def kept(buf):
+        mn, mx = L.Tensor.empty((), L.float32, "hip"), L.Tensor.empty((), L.float32, "hip")
+        s, z = L.Tensor.empty((), L.float32, "hip"), L.Tensor.empty((), L.float32, "hip")
+        _C.call("lq_calc_qparams_from_range", buf.data_ptr, 0, 0, 255, 0, 1e-8, s.data_ptr, z.data_ptr, mn.data_ptr,
+                mx.data_ptr, None)
+        return float(mn.numpy()), float(mx.numpy())
+
+    for residual in (None, res):
+        kw = dict(common, residual=hip(residual) if residual is not None else None)
+        rb = L.Tensor.empty((_C.range_buffer_words(),), L.float32, "hip")
+        got = _ops.qlinear_i8(ad, wd, **kw, gelu=True, range_buf=rb, tile_config=cfg).numpy()
+        assert _C.load().lq_last_tile_config() & 0xff == cfg
+        want = _ops.qlinear_i8(ad, wd, **kw, gelu=True, tile_config=5).numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        assert kept(rb) == (float(want.min()), float(want.max()))
+        # a kept range without the GELU
+        rb2 = L.Tensor.empty((_C.range_buffer_words(),), L.float32, "hip")
+        plain = _ops.qlinear_i8(ad, wd, **kw, range_buf=rb2, tile_config=cfg).numpy()
+        assert np.array_equal(plain.view(np.uint32), _ops.qlinear_i8(ad, wd, **kw, tile_config=5).numpy().view(np.uint32))
+        assert kept(rb2) == (float(plain.min()), float(plain.max()))
+    # a NaN in one stored element reaches the range
+    bad = res.copy()
+    bad[M - 1, N - 1] = np.nan
+    rb = L.Tensor.empty((_C.range_buffer_words(),), L.float32, "hip")
+    _ops.qlinear_i8(ad, wd, **common, residual=hip(bad), gelu=True, range_buf=rb, tile_config=cfg)
+    mn, mx = kept(rb)
+    assert np.isnan(mn) and np.isnan(mx)
+
+
 # ------------------------------------------------------------------ affine weight codes
 AFFINE_CASES = [
     # M, N, K, path
