@@ -556,7 +556,7 @@ __device__ __forceinline__ v4f at_mma6_k16(const uint2 (&a)[3], const uint2 (&b)
     return acc;
 }
 
-__global__ __launch_bounds__(832) void attention_kernel(const float* __restrict__ qkv, float* __restrict__ out,
+__global__ __launch_bounds__(1024) void attention_kernel(const float* __restrict__ qkv, float* __restrict__ out,
                                                         int B, int T, int H, float scale, float* range) {
     extern __shared__ __attribute__((aligned(16))) uint16_t at_smem[];
     uint16_t* const k_lds = at_smem;
@@ -583,7 +583,13 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
         vheld[u] = float4{0.f, 0.f, 0.f, 0.f};
         if (i < kPairs && row < T) vheld[u] = *reinterpret_cast<const float4*>(base + size_t(row) * tok_stride + size_t(2) * H * AT_D + c4);
     }
-    const int q0 = wave * 16;  // the launch has exactly ceil(T / 16) wavefronts, so q0 < T
+    // One wavefront per tile of 16 queries.  With 4 n + 1 tiles one SIMD would hold a wavefront more
+    // than the others and everybody would wait for it: the launch then has three more wavefronts,
+    // and the last tile's four each compute its scores but only one 16-column tile of its output.
+    const int tiles = (T + 15) / 16;
+    const bool shared_last = int(blockDim.x) > tiles * 64;
+    const int q0 = (wave < tiles ? wave : tiles - 1) * 16;
+    const int only_j = (shared_last && wave >= tiles - 1) ? wave - (tiles - 1) : -1;  // wavefront-uniform
     const int g = lane >> 4, c = lane & 15;
     // the lane's slice of its query row: Q[q0 + c][32 u + 8 g + 0..7]
     float4 qheld[2 * (AT_D / 32)];
@@ -724,6 +730,7 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
         for (int p = 0; p < 3; ++p) pf[p] = uint4{d[p][0], d[p][1], d[p][2], d[p][3]};
 #pragma unroll
         for (int j = 0; j < AT_D / 16; ++j) {
+            if (only_j >= 0 && only_j != j) continue;
             uint4 vf[3];
 #pragma unroll
             for (int p = 0; p < 3; ++p) {
@@ -747,6 +754,7 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
         for (int p = 0; p < 3; ++p) pf[p] = uint2{d[p][0], d[p][1]};
 #pragma unroll
         for (int j = 0; j < AT_D / 16; ++j) {
+            if (only_j >= 0 && only_j != j) continue;
             uint2 vf[3];
 #pragma unroll
             for (int p = 0; p < 3; ++p)
@@ -762,7 +770,8 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
         if (q < T) {
             float* orow = out + (size_t(b) * T + q) * (size_t(H) * AT_D) + size_t(h) * AT_D + c;
 #pragma unroll
-            for (int j = 0; j < AT_D / 16; ++j) orow[16 * j] = o[j][r];
+            for (int j = 0; j < AT_D / 16; ++j)
+                if (only_j < 0 || only_j == j) orow[16 * j] = o[j][r];
         }
     }
     if (range) {
@@ -772,7 +781,7 @@ __global__ __launch_bounds__(832) void attention_kernel(const float* __restrict_
         for (int j = 0; j < AT_D / 16; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                if (q0 + 4 * g + r < T) {
+                if (q0 + 4 * g + r < T && (only_j < 0 || only_j == j)) {
                     nan |= (o[j][r] != o[j][r]);
                     lo = fminf(lo, o[j][r]);
                     hi = fmaxf(hi, o[j][r]);
@@ -915,7 +924,8 @@ int lq_attention_f32(const float* qkv, float* out, int B, int T, int H, int D, f
     if (B == 0) return LQ_OK;
     LQ_REQUIRE(range == nullptr || long(B) * H <= kRangeSlots, LQ_ERR_SHAPE,
                "attention: too many (batch, head) pairs for a kept range");
-    const int waves = (T + 15) / 16;
+    const int tiles = (T + 15) / 16;
+    const int waves = tiles + ((tiles > 1 && tiles % 4 == 1) ? 3 : 0);  // see the kernel: the last tile shared by four
     constexpr size_t kSmem = AT_SMEM;
     static DeviceOnce attr_once;
     if (int rc = allow_dynamic_lds(attr_once, reinterpret_cast<const void*>(attention_kernel), int(kSmem))) return rc;
