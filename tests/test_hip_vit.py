@@ -50,7 +50,8 @@ def test_gelu_and_add(n):
     assert np.array_equal(F.add(hip(x), hip(y)).numpy(), x + y)
 
 
-@pytest.mark.parametrize("B,T,H", [(2, 197, 12), (1, 1, 1), (3, 16, 2), (2, 17, 3), (1, 208, 2), (4, 50, 12)])
+@pytest.mark.parametrize("B,T,H", [(2, 197, 12), (1, 1, 1), (3, 16, 2), (2, 17, 3), (1, 208, 2), (4, 50, 12),
+                                   (2, 70, 3), (1, 130, 2), (1, 193, 1), (2, 144, 2)])   # 5, 9, 13 tiles: the last one shared
 def test_attention_on_packed_qkv(B, T, H):
     rng = np.random.default_rng(B * 1000 + T * 10 + H)
     qkv = rng.standard_normal((B, T, 3 * H * 64)).astype(np.float32)
