@@ -633,9 +633,9 @@ typedef struct {
     long ldo;              /* output row stride in elements; 0 means N       */
     int force_path;        /* 0 = choose; 1 = tile, 2 = skinny, 3 = naive    */
     int tile_config;       /* tuning: low byte 0 = choose, 1..12 = a tile shape of the
-                              four-wavefront kernel, 13 / 14 / 16 = 256x352 / 256x256 /
-                              256x192 tiles of the eight-wavefront kernel (plain GEMM,
-                              K % 64 == 0), 17 = 256x352 tiles with one wavefront per SIMD
+                              four-wavefront kernel, 13 / 14 / 16 / 21 / 22 = 256x352 /
+                              256x256 / 256x192 / 224x192 / 160x256 tiles of the
+                              eight-wavefront kernel (plain GEMM, K % 64 == 0), 17 = 256x352 tiles with one wavefront per SIMD
                               (plain GEMM, K % 128 == 0, K >= 256, float16 output or raw
                               accumulators; never chosen automatically),
                               15 / 18 / 19 (convolutions only) = one block per box of

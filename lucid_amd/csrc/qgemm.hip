@@ -91,11 +91,13 @@ int launch_tile_shape(const GemmArgs& g, int conv, int groups, int cfg, int sche
     case 13:
     case 14:
     case 16:
-        // the eight-wavefront ping-pong kernel (256 x 352 / 256 x 256 / 256 x 192 tiles): plain GEMMs,
-        // one block per tile
+    case 21:
+    case 22:
+        // the eight-wavefront ping-pong kernel (256 x 352 / 256 x 256 / 256 x 192 / 224 x 192 / 160 x 256
+        // tiles): plain GEMMs, one block per tile
         LQ_REQUIRE(!conv && groups == 1, LQ_ERR_VALUE, "tile_config %d is for plain GEMMs", cfg);
         LQ_REQUIRE(schedule <= 1, LQ_ERR_VALUE, "tile_config %d runs one block per tile", cfg);
-        return launch_pp_shape(g, cfg == 16 ? 2 : cfg - 13, st);
+        return launch_pp_shape(g, cfg == 16 ? 2 : (cfg >= 21 ? cfg - 18 : cfg - 13), st);
     case 17:
         // one wavefront per SIMD, 256 x 352 tiles (plain GEMMs, K % 128 == 0)
         LQ_REQUIRE(!conv && groups == 1, LQ_ERR_VALUE, "tile_config %d is for plain GEMMs", cfg);
@@ -232,7 +234,7 @@ int tune_import_text(const char* text, int* accepted) {
         }
         if (got != kTuneKeyInts + 1) return fail(LQ_ERR_VALUE, "tune_import: malformed line '%s'", line.c_str());
         const int shape = v[kTuneKeyInts] & 0xff;
-        if (shape < 1 || shape > 20) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
+        if (shape < 1 || shape > 22) return fail(LQ_ERR_VALUE, "tune_import: tile shape %d in '%s'", shape, line.c_str());
         TuneKey key;
         std::memcpy(&key, v, sizeof(key));
         std::lock_guard<std::mutex> lock(g_tune_mu);
@@ -323,7 +325,15 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
         if (g.N > 128 && g.M > 128) cands[n++] = 1, cands[n++] = 11;
         if (g.N > 128 && !conv) cands[n++] = 12;
         // large plain GEMMs: the ping-pong kernel's 256 x 352 and 256 x 256 tiles
-        if (pp_applies(g, conv, groups)) cands[n++] = 13, cands[n++] = 14, cands[n++] = 16;
+        if (pp_applies(g, conv, groups)) {
+            cands[n++] = 13, cands[n++] = 14, cands[n++] = 16;
+            // shorter tiles where they put a block on more of the CUs in one round
+            const long t192 = long((g.M + 255) / 256) * ((g.N + 191) / 192);
+            const long t224 = long((g.M + 223) / 224) * ((g.N + 191) / 192);
+            const long t160 = long((g.M + 159) / 160) * ((g.N + 255) / 256);
+            if (t192 < 256 && t224 > t192 && t224 <= 256) cands[n++] = 21;
+            if (t192 < 256 && t160 > t192 && t160 <= 256) cands[n++] = 22;
+        }
         // a long K over few tiles (late convolution stages): split K between the idle CUs
         const long tiles128 = long((g.M + 127) / 128) * ((g.N + 127) / 128) * groups;
         if (tiles128 * 2 <= 512 && g.K >= 2048) cands[n++] = 5 | (2 << 8);

@@ -620,6 +620,10 @@ int launch_pp(const GemmArgs& g, hipStream_t st) {
 using PPCfg352 = PPCfg<256, 352, 4, 2, 4>;
 using PPCfg256 = PPCfg<256, 256, 4, 2, 4>;
 using PPCfg192 = PPCfg<256, 192, 4, 2, 4>;
+// shorter tiles for row counts that 256-row tiles split badly over the 256 CUs (12 608 rows x 768
+// columns: 200 tiles of 256 x 192, but 228 of 224 x 192 and 237 of 160 x 256, each with less work)
+using PPCfg224x192 = PPCfg<224, 192, 2, 4, 4>;
+using PPCfg160x256 = PPCfg<160, 256, 2, 4, 4>;
 
 }  // namespace
 }  // namespace lq

@@ -459,7 +459,7 @@ PP_SHAPES = [(256, 256, 128), (300, 260, 192), (513, 1000, 576), (2048, 512, 409
              (257, 353, 320), (2048, 1004, 256), (40, 1001, 128)]
 
 
-@pytest.mark.parametrize("cfg", [13, 14, 16])
+@pytest.mark.parametrize("cfg", [13, 14, 16, 21, 22])
 @pytest.mark.parametrize("M,N,K", PP_SHAPES)
 def test_ping_pong_kernel_exact(cfg, M, N, K):
     """The eight-wavefront kernel (tile_config 13 / 14): accumulators and the float16 epilogue
@@ -479,7 +479,7 @@ def test_ping_pong_kernel_exact(cfg, M, N, K):
     assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
 
 
-@pytest.mark.parametrize("cfg", [13, 14, 16])
+@pytest.mark.parametrize("cfg", [13, 14, 16, 21, 22])
 @pytest.mark.parametrize("M,N,K", [(512, 704, 256), (300, 260, 128), (129, 1001, 64), (512, 768, 192)])
 def test_ping_pong_kernel_every_output_form(cfg, M, N, K):
     """Every epilogue form of the eight-wavefront kernel equals the oracle: an activation zero
@@ -531,7 +531,7 @@ def test_ping_pong_kernel_every_output_form(cfg, M, N, K):
         assert np.array_equal(fused, expj.reshape(M, N))
 
 
-@pytest.mark.parametrize("cfg", [13, 14, 16])
+@pytest.mark.parametrize("cfg", [13, 14, 16, 21, 22])
 @pytest.mark.parametrize("M,N,K", [(512, 704, 256), (300, 260, 128), (129, 1001, 64), (1576, 3072, 768)])
 def test_ping_pong_kernel_gelu_and_kept_range(cfg, M, N, K):
     """GELU in the epilogue and the kept range of what is stored, on the eight-wavefront kernel:
