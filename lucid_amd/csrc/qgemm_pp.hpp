@@ -279,8 +279,33 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
         }
     }
 
-    // ---- every other form.  values of one tile in the lane's own layout, residual / join applied
-    auto tile_values = [&](int m, const pp_v4i& a, const ColParams (&c4)[4], float as, int nq, uint4& v) {
+    // ---- every other form.  The residual operand of a float output is requested first, every
+    // tile of the wavefront at once: requested tile by tile, each of the TM * TN loads would be
+    // waited for on its own (the operand was last touched several kernels ago and comes from
+    // memory), which costs the ViT's proj and fc2 a third of their time.  In-place use
+    // (out == residual) is unaffected: an element is still read before it is written, by its own lane.
+    // (tiles of up to 24 sub-tiles per wavefront: the larger shapes have no registers to spare)
+    constexpr bool kResidualForm = (MODE == OUT_F32 || MODE == OUT_F16 || MODE == OUT_F32X) && TM * TN <= 24;
+    const bool res_ahead = kResidualForm && vec_out && g.residual != nullptr;
+    float4 rres[kResidualForm ? TM : 1][kResidualForm ? TN : 1];
+    if constexpr (kResidualForm) {
+        if (res_ahead) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int m = wm0 + 16 * i + (lane & 15);
+                const float* rp = g.residual + size_t(rows_in || m < g.M ? m : 0) * size_t(g.ldr) + size_t(lane_col);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    // accumulator column j is column tile j + rot (the lone last one: last_tile)
+                    const int t = (kLone && j == TN - 1) ? last_tile : j + rot;
+                    rres[i][j] = *reinterpret_cast<const float4*>(rp + wn0 + 16 * t);
+                }
+            }
+        }
+    }
+    // values of one tile in the lane's own layout, residual / join applied; (ri, rj): the tile's
+    // place among the wavefront's accumulators
+    auto tile_values = [&](int m, const pp_v4i& a, const ColParams (&c4)[4], float as, int nq, uint4& v, int ri, int rj) {
         if (prescaled) {
             v.x = epilogue_value<MODE, true>(g, a[0], 1.0f, c4[0], G);
             v.y = epilogue_value<MODE, true>(g, a[1], 1.0f, c4[1], G);
@@ -294,7 +319,9 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
         }
         if (vec_out && (rows_in || m < g.M)) {
             if (kFloatOut && g.residual != nullptr) {
-                const float4 rv = *reinterpret_cast<const float4*>(g.residual + size_t(m) * size_t(g.ldr) + size_t(nq));
+                const float4 rv = kResidualForm
+                                      ? rres[kResidualForm ? ri : 0][kResidualForm ? rj : 0]
+                                      : *reinterpret_cast<const float4*>(g.residual + size_t(m) * size_t(g.ldr) + size_t(nq));
                 v.x = __float_as_uint(__uint_as_float(v.x) + rv.x);
                 v.y = __float_as_uint(__uint_as_float(v.y) + rv.y);
                 v.z = __float_as_uint(__uint_as_float(v.z) + rv.z);
@@ -349,8 +376,8 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
         for (int i = 0; i < TM; ++i) {
             const int m = wm0 + 16 * i + (lane & 15);
             uint4 v, w;
-            tile_values(m, acc[i][j], c4, as_row[i], nq, v);
-            tile_values(m, acc[i][j + 1], d4, as_row[i], nq + 16, w);
+            tile_values(m, acc[i][j], c4, as_row[i], nq, v, i, j);
+            tile_values(m, acc[i][j + 1], d4, as_row[i], nq + 16, w, i, j + 1);
             if (MODE == OUT_F32X && keep && vec_out && (rows_in || m < g.M)) {
                 track(v.x), track(v.y), track(v.z), track(v.w);
                 track(w.x), track(w.y), track(w.z), track(w.w);
@@ -389,7 +416,7 @@ __device__ __forceinline__ void pp_epilogue(const GemmArgs& g, pp_v4i (&acc)[TM]
         for (int i = 0; i < TM; ++i) {
             const int m = wm0 + 16 * i + (lane & 15);
             uint4 v;
-            tile_values(m, acc[i][TN - 1], c4, as_row[i], nq, v);
+            tile_values(m, acc[i][TN - 1], c4, as_row[i], nq, v, i, TN - 1);
             if (MODE == OUT_F32X && keep && vec_out && (rows_in || m < g.M)) track(v.x), track(v.y), track(v.z), track(v.w);
             store_own(m, nq, v);
         }
