@@ -141,7 +141,8 @@ int heuristic_tile_shape(const GemmArgs& g, int conv, int groups) {
     // far fewer 128 x 128 tiles than CUs (a small batch in the late stages of a network): 64 x 64
     // tiles, four blocks per CU, with 128-byte k steps when K is long (plain and 2-d only)
     if (mt128 * ((g.N + 127) / 128) * groups < 128) return (g.K >= 1024 && conv != 2) ? 10 : 9;
-    if (pp_applies(g, conv, groups) && g.K >= 512) {
+    // (not with a GELU: its vector arithmetic needs a second block on the CU to overlap with)
+    if (pp_applies(g, conv, groups) && g.K >= 512 && !g.gelu) {
         const long tm = (g.M + 255) / 256;
         const long t352 = tm * ((g.N + 351) / 352), t256 = tm * ((g.N + 255) / 256);
         // at least half a round of tiles, or the four-wavefront shapes below cover the chip better
@@ -325,7 +326,9 @@ int tuned_tile_shape(const GemmArgs& g, int conv, int groups, hipStream_t st, in
         if (g.N > 128 && g.M > 128) cands[n++] = 1, cands[n++] = 11;
         if (g.N > 128 && !conv) cands[n++] = 12;
         // large plain GEMMs: the ping-pong kernel's 256 x 352 and 256 x 256 tiles
-        if (pp_applies(g, conv, groups)) {
+        // (with a GELU in the epilogue they lose in the network - ViT-B/16 fc1: 5.22 against 5.08 ms per
+        // batch - even where they tie in isolation: one block per CU, nothing overlaps its epilogue)
+        if (pp_applies(g, conv, groups) && !g.gelu) {
             cands[n++] = 13, cands[n++] = 14, cands[n++] = 16;
             // shorter tiles where they put a block on more of the CUs in one round
             const long t192 = long((g.M + 255) / 256) * ((g.N + 191) / 192);
