@@ -153,6 +153,7 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
 // expressions on the same inputs, so the same bits - and writes int8 codes.  x is read twice
 // and 1 byte per element written, where LayerNorm + quantize read it twice, write it once as
 // float32 and read that back.  Rows of up to 2048 floats, vector-aligned.
+template <int KEEP>  // float4 per lane held in registers: 4 for rows of up to 1024 floats, else KEEP
 __global__ __launch_bounds__(256) void layernorm_stats_kernel(const float* __restrict__ x,
                                                               const float* __restrict__ gamma,
                                                               const float* __restrict__ beta, long rows, int cols,
@@ -169,20 +170,29 @@ __global__ __launch_bounds__(256) void layernorm_stats_kernel(const float* __res
     const long row = long(blockIdx.x) * 4 + wave;
     if (row < rows) {
         const float* xr = x + row * cols;
-        float4 v[LN_KEEP];
+        float4 v[KEEP], gv[KEEP], bv[KEEP];
 #pragma unroll
-        for (int u = 0; u < LN_KEEP; ++u) {
+        for (int u = 0; u < KEEP; ++u) {
             const int c = lane * 4 + u * 256;
             if (c < cols) v[u] = *reinterpret_cast<const float4*>(xr + c);
         }
+        // gamma and beta are needed after the two reductions: requested now, they arrive under them
+#pragma unroll
+        for (int u = 0; u < KEEP; ++u) {
+            const int c = lane * 4 + u * 256;
+            if (c < cols) {
+                gv[u] = *reinterpret_cast<const float4*>(gamma + c);
+                bv[u] = *reinterpret_cast<const float4*>(beta + c);
+            }
+        }
         float s = 0.0f;
 #pragma unroll
-        for (int u = 0; u < LN_KEEP; ++u)
+        for (int u = 0; u < KEEP; ++u)
             if (lane * 4 + u * 256 < cols) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
         const float mean = wave_sum(s) * inv_n;
         float q = 0.0f;
 #pragma unroll
-        for (int u = 0; u < LN_KEEP; ++u)
+        for (int u = 0; u < KEEP; ++u)
             if (lane * 4 + u * 256 < cols) {
                 const float a = v[u].x - mean, b = v[u].y - mean, cc = v[u].z - mean, d = v[u].w - mean;
                 q += (a * a + b * b) + (cc * cc + d * d);
@@ -191,11 +201,10 @@ __global__ __launch_bounds__(256) void layernorm_stats_kernel(const float* __res
         const float rstd = 1.0f / sqrtf(var + eps);
         if (lane == 0) stats[2 * row] = mean, stats[2 * row + 1] = rstd;
 #pragma unroll
-        for (int u = 0; u < LN_KEEP; ++u) {
+        for (int u = 0; u < KEEP; ++u) {
             const int c = lane * 4 + u * 256;
             if (c < cols) {
-                const float4 g = *reinterpret_cast<const float4*>(gamma + c);
-                const float4 b = *reinterpret_cast<const float4*>(beta + c);
+                const float4 g = gv[u], b = bv[u];
                 track(((v[u].x - mean) * rstd) * g.x + b.x);
                 track(((v[u].y - mean) * rstd) * g.y + b.y);
                 track(((v[u].z - mean) * rstd) * g.z + b.z);
@@ -823,8 +832,11 @@ int lq_layernorm_stats_f32(const float* x, const float* gamma, const float* beta
     if (rows == 0) return LQ_OK;
     const long blocks = (rows + 3) / 4;
     LQ_REQUIRE(blocks <= kRangeSlots, LQ_ERR_SHAPE, "layernorm_stats: %ld rows are too many for a kept range", rows);
-    layernorm_stats_kernel<<<unsigned(blocks), 256, 0, as_stream(stream)>>>(x, gamma, beta, rows, cols, eps, stats,
-                                                                             range);
+    if (cols <= 4 * 256)
+        layernorm_stats_kernel<4><<<unsigned(blocks), 256, 0, as_stream(stream)>>>(x, gamma, beta, rows, cols, eps, stats, range);
+    else
+        layernorm_stats_kernel<LN_KEEP><<<unsigned(blocks), 256, 0, as_stream(stream)>>>(x, gamma, beta, rows, cols, eps, stats,
+                                                                                          range);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }
