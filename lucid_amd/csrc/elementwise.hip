@@ -210,8 +210,10 @@ __global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const int8_t* 
     const int part = threadIdx.x >> 6;  // 4 slices of the pixels
     __shared__ int red[4][64];
     int s = 0;
-    if (c < C)
-        for (int p = part; p < HW; p += 4) s += q[(size_t(b) * HW + p) * C + c];
+    if (c < C) {
+#pragma unroll 8
+        for (int p = part; p < HW; p += 4) s += q[(size_t(b) * HW + p) * C + c];  // (unrolled: the loads go out together)
+    }
     red[part][threadIdx.x & 63] = s;
     __syncthreads();
     if (part == 0 && c < C) {

@@ -417,6 +417,51 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_i8x16_kernel(const uint4* __
     }
 }
 
+// The same with the window size known at compile time: every tap's 16 bytes are requested before
+// the first maximum is taken (taps outside the image read a clamped address and are replaced by
+// -128).  With run-time loops and their bounds tests each tap's load was waited for before the next
+// one was requested: nine memory round trips in a row for a 3 x 3 window.
+template <int KH, int KW>
+__global__ __launch_bounds__(256) void maxpool_nhwc_i8x16_fixed_kernel(const uint4* __restrict__ x, uint4* __restrict__ out,
+                                                                       int B, int H, int W, int C16, int sh, int sw,
+                                                                       int ph, int pw, int OH, int OW) {
+    const size_t total = size_t(B) * OH * OW * C16;
+    for (size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += size_t(gridDim.x) * 256) {
+        const int c = int(idx % C16);
+        size_t p = idx / C16;
+        const int ow = int(p % OW);
+        p /= OW;
+        const int oh = int(p % OH), b = int(p / OH);
+        uint4 v[KH][KW];
+        bool ok[KH][KW];
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh) {
+            const int ih = oh * sh - ph + kh;
+            const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih);
+#pragma unroll
+            for (int kw = 0; kw < KW; ++kw) {
+                const int iw = ow * sw - pw + kw;
+                const int iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);
+                ok[kh][kw] = ih == ihc && iw == iwc;
+                v[kh][kw] = x[((size_t(b) * H + ihc) * W + iwc) * C16 + c];
+            }
+        }
+        uint4 best = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};  // -128 in every byte
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < KW; ++kw) {
+                const uint4 t = v[kh][kw];
+                const bool k = ok[kh][kw];
+                best.x = max_i8x4(best.x, k ? t.x : 0x80808080u);
+                best.y = max_i8x4(best.y, k ? t.y : 0x80808080u);
+                best.z = max_i8x4(best.z, k ? t.z : 0x80808080u);
+                best.w = max_i8x4(best.w, k ? t.w : 0x80808080u);
+            }
+        out[idx] = best;
+    }
+}
+
 // float32 NCHW -> int8 NHWC for at most four channels (an RGB image): one pixel per
 // lane, plane reads and pixel writes both contiguous across a wavefront.
 __global__ __launch_bounds__(256) void quantize_nchw_to_nhwc_small_c_kernel(
@@ -981,6 +1026,19 @@ int lq_maxpool2d_nhwc_i8(const int8_t* x, int8_t* out, int B, int H, int W, int 
     if (total == 0) return LQ_OK;
     LQ_REQUIRE(x && out, LQ_ERR_VALUE, "maxpool2d_nhwc_i8: NULL pointer");
     if (C % 16 == 0 && aligned16(x) && aligned16(out)) {
+        if ((KH == 3 && KW == 3) || (KH == 2 && KW == 2)) {
+            const dim3 grid{grid_1d(total / 16)};
+            const uint4* xi = reinterpret_cast<const uint4*>(x);
+            uint4* oi = reinterpret_cast<uint4*>(out);
+            if (KH == 3)
+                hipLaunchKernelGGL((maxpool_nhwc_i8x16_fixed_kernel<3, 3>), grid, dim3(256), 0, as_stream(stream), xi, oi,
+                                   B, H, W, C / 16, stride_h, stride_w, pad_h, pad_w, OH, OW);
+            else
+                hipLaunchKernelGGL((maxpool_nhwc_i8x16_fixed_kernel<2, 2>), grid, dim3(256), 0, as_stream(stream), xi, oi,
+                                   B, H, W, C / 16, stride_h, stride_w, pad_h, pad_w, OH, OW);
+            LQ_CHECK_LAUNCH("maxpool2d_nhwc_i8");
+            return LQ_OK;
+        }
         hipLaunchKernelGGL(maxpool_nhwc_i8x16_kernel, dim3(grid_1d(total / 16)), dim3(256), 0, as_stream(stream),
                            reinterpret_cast<const uint4*>(x), reinterpret_cast<uint4*>(out), B, H, W, C / 16, KH, KW,
                            stride_h, stride_w, pad_h, pad_w, OH, OW);

@@ -114,13 +114,19 @@ def test_layout_helpers_round_trip():
     assert np.array_equal(wo.numpy(), w.transpose(0, 2, 3, 1))
 
 
-def test_maxpool_on_codes():
-    rng = np.random.default_rng(4)
-    x = codes(rng, (2, 13, 12, 70))
-    out = L.Tensor.empty((2, 7, 6, 70), L.int8, "hip")
-    _C.call("lq_maxpool2d_nhwc_i8", hip(x).data_ptr, out.data_ptr, 2, 13, 12, 70, 3, 3, 2, 2, 1, 1,
-            None)
-    assert np.array_equal(out.numpy(), O.maxpool2d_nhwc_i8(x, (3, 3), (2, 2), (1, 1)))
+@pytest.mark.parametrize("C", [70, 64, 48])          # scalar kernel; 16-channel lanes
+@pytest.mark.parametrize("k,s,p", [((3, 3), (2, 2), (1, 1)), ((2, 2), (2, 2), (0, 0)), ((2, 2), (1, 2), (1, 1)),
+                                   ((3, 3), (1, 1), (0, 1)), ((3, 2), (2, 1), (1, 0)), ((5, 5), (3, 3), (2, 2))])
+def test_maxpool_on_codes(C, k, s, p):
+    """Windows with compile-time sizes (3 x 3, 2 x 2: every tap requested up front) and the general
+    loop, with and without padding: the oracle's maxima, code for code."""
+    rng = np.random.default_rng(4 + C + k[0])
+    B, H, W = 2, 13, 12
+    x = codes(rng, (B, H, W, C))
+    OH, OW = (H + 2 * p[0] - k[0]) // s[0] + 1, (W + 2 * p[1] - k[1]) // s[1] + 1
+    out = L.Tensor.empty((B, OH, OW, C), L.int8, "hip")
+    _C.call("lq_maxpool2d_nhwc_i8", hip(x).data_ptr, out.data_ptr, B, H, W, C, k[0], k[1], s[0], s[1], p[0], p[1], None)
+    assert np.array_equal(out.numpy(), O.maxpool2d_nhwc_i8(x, k, s, p))
 
 
 def test_argument_validation():
