@@ -537,6 +537,14 @@ int lq_gather_rows_f32(const float* src, size_t src_row_stride, float* dst, size
 int lq_assemble_tokens_f32(const float* patches, const float* cls, const float* pos, float* out, int B, int T,
                            int D, lq_stream stream);
 
+/* lq_patchify_f32, lq_sgemm_nt_f32 and lq_assemble_tokens_f32 in one launch, with the same
+ * arithmetic in the same order (vit/_model.py:62-69 and 452-454): the GEMM reads its rows
+ * straight from the image [B,C,H,W], adds bias[D] and then the position row, and writes
+ * token rows out[B, 1 + (H/p)*(W/p), D]; row 0 of every image is cls + pos[0].
+ * w: [D, C*p*p], cls: [D], pos: [1 + (H/p)*(W/p), D].  bias may be null. */
+int lq_patch_embed_f32(const float* img, const float* w, const float* bias, const float* cls, const float* pos,
+                       float* out, int B, int C, int H, int W, int patch, int D, lq_stream stream);
+
 /* The other merges of QFunctional (functional_module.py:220-246) on codes:
  * fq(act(x OP y)), OP = add (0) or mul (1), y a second code tensor or - when qb is
  * NULL - the float scalar (add_scalar / mul_scalar).  Each operand is dequantized

@@ -172,6 +172,7 @@ _SIGNATURES["lq_calc_qparams_from_range"] = [_vp, _i, _i, _i, _i, _f, _vp, _vp, 
 _SIGNATURES["lq_patchify_f32"] = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_sgemm_nt_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _SIGNATURES["lq_assemble_tokens_f32"] = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
+_SIGNATURES["lq_patch_embed_f32"] = [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_pad_nhwc_i8"] = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_pad_planes_f32"] = [_vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp]
 _SIGNATURES["lq_binary_requant_i8"] = [_i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _f, _sz, _i, _vp, _vp, _i, _i,

@@ -11,6 +11,7 @@
 //                           read straight from the packed qkv activation
 //   lq_patchify_f32 + lq_sgemm_nt_f32   the stride = kernel patch convolution as a GEMM
 //   lq_assemble_tokens_f32  class token + position table
+//   lq_patch_embed_f32      the three above in one launch: the GEMM gathers the patches itself
 //
 // Matrix products use the float32 MFMA instructions; results agree with a CPU
 // float32 evaluation to rounding-order differences (tested to 1e-4 relative).
@@ -385,16 +386,41 @@ __device__ __forceinline__ int sg_index(int row, int k) {  // k a multiple of 4
     return row * SG_BK + ((((k >> 3) ^ ((row >> 2) & 3)) << 3) | (k & 7));
 }
 
+// PATCH: the A operand is an image [B,C,H,W] read as the rows of its p x p patches (row = (b, gy,
+// gx), column = (c, ph, pw): four consecutive columns are four consecutive pixels of one image
+// row when p is a multiple of 4), and the result row (b, i) lands on token row 1 + i of image b
+// with the position table added; the blocks of the first row tile also write the class-token rows.
+struct PatchForm {
+    int C, H, W, p, gw, per_image;  // per_image = (H/p) * (W/p) patches
+    int B, log2p;                   // log2p = -1 when p is not a power of two
+    const float* cls;  // [N]
+    const float* pos;  // [(1 + per_image), N]
+};
+
+// PATCH 0: a is a plain [M,K] matrix.  1: patch rows with p a power of two and every group of
+// four columns one aligned 16-byte load (no branch and no division in the loop).  2: patch rows
+// of any geometry, element by element.
+template <int PATCH>
 __global__ __launch_bounds__(256, 2) void sgemm_nt_kernel(const float* __restrict__ a, const float* __restrict__ w,
                                                           const float* __restrict__ bias, float* __restrict__ out,
-                                                          int M, int N, int K) {
+                                                          int M, int N, int K, PatchForm pf) {
     __shared__ __attribute__((aligned(16))) uint16_t sp[3][SG_ROWS * SG_BK];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.y * SG_BM, n0 = blockIdx.x * SG_BN;
     // loader: piece tid + 256 u = row (tid + 256 u) / 8 of either operand, four consecutive k at 4 * (tid % 8)
     const int lrow = tid >> 3, lk = (tid & 7) * 4;
-    const bool vec = (K % 4 == 0) && aligned16(a) && aligned16(w);
+    const bool vec = (K % 4 == 0) && aligned16(w) && (PATCH != 0 || aligned16(a));
+    size_t patch_at[4];  // PATCH: where the patch of loader row u starts in the image
+    if constexpr (PATCH != 0) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int row = min(m0 + lrow + 32 * u, M - 1);
+            const int b = row / pf.per_image, i = row - b * pf.per_image;
+            const int gy = i / pf.gw, gx = i - gy * pf.gw;
+            patch_at[u] = (size_t(b) * pf.C * pf.H + size_t(gy) * pf.p) * pf.W + size_t(gx) * pf.p;
+        }
+    }
     v16f acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -419,11 +445,70 @@ __global__ __launch_bounds__(256, 2) void sgemm_nt_kernel(const float* __restric
         }
         return v;
     };
-    auto fetch = [&](int k0) {
+    // PATCH: column k of a patch row is pixel (c, ph, pw) of the patch.  Loads go to clamped
+    // (always valid) addresses and what lies past M or K is zeroed afterwards, so that the four
+    // loads of a fetch are issued back to back.
+    auto fetch_patches = [&](int k) {
+        if constexpr (PATCH == 1) {
+            const int kk = min(k, K - 4);
+            const int pw = kk & (pf.p - 1), ph = (kk >> pf.log2p) & (pf.p - 1), c = kk >> (2 * pf.log2p);
+            const size_t pixel = (size_t(c) * pf.H + ph) * pf.W + pw;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            ra[u] = fetch_row(a, m0 + lrow + 32 * u, M, k0 + lk);
-            rb[u] = fetch_row(w, n0 + lrow + 32 * u, N, k0 + lk);
+            for (int u = 0; u < 4; ++u) ra[u] = *reinterpret_cast<const float4*>(a + patch_at[u] + pixel);
+            if (k >= K) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) ra[u] = float4{0.f, 0.f, 0.f, 0.f};
+            }
+        } else {
+            const int pp = pf.p * pf.p;
+            size_t pixel[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int kk = min(k + e, K - 1);
+                const int c = kk / pp, r = kk - c * pp;
+                const int ph = r / pf.p, pw = r - ph * pf.p;
+                pixel[e] = (size_t(c) * pf.H + ph) * pf.W + pw;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const float* p = a + patch_at[u];
+                ra[u] = float4{p[pixel[0]], p[pixel[1]], p[pixel[2]], p[pixel[3]]};
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (k >= K) ra[u].x = 0.f;
+                if (k + 1 >= K) ra[u].y = 0.f;
+                if (k + 2 >= K) ra[u].z = 0.f;
+                if (k + 3 >= K) ra[u].w = 0.f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (m0 + lrow + 32 * u >= M) ra[u] = float4{0.f, 0.f, 0.f, 0.f};
+    };
+    // plain rows in the aligned case: the row is clamped instead of tested (a row past the end
+    // only feeds results that are never stored) and a k past the end is zeroed afterwards
+    auto fetch_rows_vec = [&](const float* base, int row0, int rows, int k, float4 (&r)[4]) {
+        const int kk = min(k, K - 4);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            r[u] = *reinterpret_cast<const float4*>(base + size_t(min(row0 + 32 * u, rows - 1)) * K + kk);
+        if (k >= K) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) r[u] = float4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    auto fetch = [&](int k0) {
+        if constexpr (PATCH != 0) fetch_patches(k0 + lk);
+        if (vec) {
+            if constexpr (PATCH == 0) fetch_rows_vec(a, m0 + lrow, M, k0 + lk, ra);
+            fetch_rows_vec(w, n0 + lrow, N, k0 + lk, rb);
+        } else {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if constexpr (PATCH == 0) ra[u] = fetch_row(a, m0 + lrow + 32 * u, M, k0 + lk);
+                rb[u] = fetch_row(w, n0 + lrow + 32 * u, N, k0 + lk);
+            }
         }
     };
     auto stash_one = [&](int row, float4 v) {
@@ -484,12 +569,45 @@ __global__ __launch_bounds__(256, 2) void sgemm_nt_kernel(const float* __restric
             const int n = n0 + wn * 64 + j * 32 + (lane & 31);
             if (n >= N) continue;
             const float bv = bias ? bias[n] : 0.0f;
+            if constexpr (PATCH != 0) {
+                // the sixteen position values are requested before the first store: a store
+                // between two loads would make each load wait for the one before it
+                float pv[16];
+                size_t at[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m < M) out[size_t(m) * N + n] = acc[i][j][r] + bv;
+                for (int q = 0; q < 4; ++q) {
+                    const int mq = m0 + wm * 64 + i * 32 + 8 * q + 4 * (lane >> 5);
+                    int b = mq / pf.per_image, t = mq - b * pf.per_image;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        at[4 * q + r] = (size_t(b) * (pf.per_image + 1) + 1 + t) * N + n;
+                        pv[4 * q + r] = mq + r < M ? pf.pos[size_t(1 + t) * N + n] : 0.0f;
+                        if (++t == pf.per_image) t = 0, ++b;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (m < M) out[at[r]] = (acc[i][j][r] + bv) + pv[r];
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (m < M) out[size_t(m) * N + n] = acc[i][j][r] + bv;
+                }
             }
         }
+    if constexpr (PATCH != 0) {
+        // class-token rows: token 0 of every image, this block's 128 columns
+        if (blockIdx.y == 0) {
+            const int n = n0 + (tid & 127);
+            if (n < N) {
+                const float v = pf.cls[n] + pf.pos[n];
+                for (int b = tid >> 7; b < pf.B; b += 2) out[size_t(b) * (pf.per_image + 1) * N + n] = v;
+            }
+        }
+    }
 }
 
 // ---------------------------------------------------------------- attention
@@ -911,7 +1029,31 @@ int lq_sgemm_nt_f32(const float* a, const float* w, const float* bias, float* ou
     if (M == 0 || N == 0) return LQ_OK;
     dim3 grid((N + SG_BN - 1) / SG_BN, (M + SG_BM - 1) / SG_BM);
     LQ_REQUIRE(grid.y < 65536, LQ_ERR_SHAPE, "sgemm: M too large");
-    sgemm_nt_kernel<<<grid, 256, 0, as_stream(stream)>>>(a, w, bias, out, M, N, K);
+    sgemm_nt_kernel<0><<<grid, 256, 0, as_stream(stream)>>>(a, w, bias, out, M, N, K, PatchForm{});
+    LQ_CHECK_LAUNCH();
+    return LQ_OK;
+}
+
+int lq_patch_embed_f32(const float* img, const float* w, const float* bias, const float* cls, const float* pos,
+                       float* out, int B, int C, int H, int W, int patch, int D, void* stream) {
+    LQ_REQUIRE(img && w && cls && pos && out, LQ_ERR_VALUE, "patch_embed: null pointer");
+    LQ_REQUIRE(B >= 0 && C > 0 && H > 0 && W > 0 && D > 0 && patch > 0 && H % patch == 0 && W % patch == 0,
+               LQ_ERR_SHAPE, "patch_embed: image %dx%dx%dx%d is not a whole number of %d-pixel patches", B, C, H, W,
+               patch);
+    const int per_image = (H / patch) * (W / patch);
+    const size_t rows = size_t(B) * per_image, K = size_t(C) * patch * patch;
+    LQ_REQUIRE(rows < (size_t(1) << 31) && K < (size_t(1) << 31), LQ_ERR_SHAPE, "patch_embed: too many patch rows");
+    if (B == 0) return LQ_OK;
+    dim3 grid((D + SG_BN - 1) / SG_BN, (unsigned(rows) + SG_BM - 1) / SG_BM);
+    LQ_REQUIRE(grid.y < 65536, LQ_ERR_SHAPE, "patch_embed: too many patch rows");
+    int log2p = -1;
+    for (int e = 0; e < 15; ++e)
+        if ((1 << e) == patch) log2p = e;
+    const PatchForm pf{C, H, W, patch, W / patch, per_image, B, log2p, cls, pos};
+    if (log2p >= 2 && W % 4 == 0 && aligned16(img))
+        sgemm_nt_kernel<1><<<grid, 256, 0, as_stream(stream)>>>(img, w, bias, out, int(rows), D, int(K), pf);
+    else
+        sgemm_nt_kernel<2><<<grid, 256, 0, as_stream(stream)>>>(img, w, bias, out, int(rows), D, int(K), pf);
     LQ_CHECK_LAUNCH();
     return LQ_OK;
 }

@@ -84,16 +84,54 @@ def test_patchify_and_token_assembly_are_exact():
     rng = np.random.default_rng(3)
     img = rng.standard_normal((3, 3, 32, 48)).astype(np.float32)
     rows = L.Tensor.empty((3 * 6, 3 * 256), L.float32, "hip")
-    _C.call("lq_patchify_f32", hip(img).data_ptr, rows.data_ptr, 3, 3, 32, 48, 16, None)
+    d_img = hip(img)
+    _C.call("lq_patchify_f32", d_img.data_ptr, rows.data_ptr, 3, 3, 32, 48, 16, None)
     assert np.array_equal(rows.numpy(), V.patch_rows(img, 16))
     emb = rng.standard_normal((3, 6, 40)).astype(np.float32)
     cls = rng.standard_normal(40).astype(np.float32)
     pos = rng.standard_normal((7, 40)).astype(np.float32)
     out = L.Tensor.empty((3, 7, 40), L.float32, "hip")
-    _C.call("lq_assemble_tokens_f32", hip(emb).data_ptr, hip(cls).data_ptr, hip(pos).data_ptr,
-            out.data_ptr, 3, 7, 40, None)
+    d_emb, d_cls, d_pos = hip(emb), hip(cls), hip(pos)  # held: a temporary's memory is reused at once
+    _C.call("lq_assemble_tokens_f32", d_emb.data_ptr, d_cls.data_ptr, d_pos.data_ptr, out.data_ptr, 3, 7, 40, None)
     exp = np.concatenate([np.broadcast_to(cls, (3, 1, 40)), emb], axis=1) + pos[None]
     assert np.array_equal(out.numpy(), exp.astype(np.float32))
+
+
+@pytest.mark.parametrize("B,C,H,W,p,D,bias", [
+    (3, 3, 32, 48, 16, 40, True),      # less than one tile either way
+    (5, 3, 96, 96, 16, 200, True),     # 180 patch rows: a ragged second row tile, images straddling tiles
+    (2, 1, 30, 18, 6, 130, False),     # patch not a multiple of 4: the element-by-element gather
+    (1, 2, 8, 8, 4, 8, True),
+    (64, 3, 224, 224, 16, 768, True),  # ViT-B/16 at the bench batch
+])
+def test_patch_embedding_in_one_launch_equals_the_three_steps(B, C, H, W, p, D, bias):
+    """lq_patch_embed_f32 against lq_patchify_f32 -> lq_sgemm_nt_f32 -> lq_assemble_tokens_f32
+    bit for bit (same products, same summation order), and the chain's gather and
+    assembly against numpy above."""
+    rng = np.random.default_rng(B * 1000 + D)
+    n, K = (H // p) * (W // p), C * p * p
+    img = hip(rng.standard_normal((B, C, H, W)).astype(np.float32))
+    w = hip((rng.standard_normal((D, K)) / np.sqrt(K)).astype(np.float32))
+    bv = hip(rng.standard_normal(D).astype(np.float32)) if bias else None
+    cls = hip(rng.standard_normal(D).astype(np.float32))
+    pos = hip(rng.standard_normal((n + 1, D)).astype(np.float32))
+    rows = L.Tensor.empty((B * n, K), L.float32, "hip")
+    _C.call("lq_patchify_f32", img.data_ptr, rows.data_ptr, B, C, H, W, p, None)
+    emb = F.linear_f32(rows, w, bv)
+    exp = L.Tensor.empty((B, n + 1, D), L.float32, "hip")
+    _C.call("lq_assemble_tokens_f32", emb.data_ptr, cls.data_ptr, pos.data_ptr, exp.data_ptr, B, n + 1, D, None)
+    got = L.tensor(np.full((B, n + 1, D), np.nan, np.float32), device="hip")
+    _C.call("lq_patch_embed_f32", img.data_ptr, w.data_ptr, bv.data_ptr if bias else None, cls.data_ptr,
+            pos.data_ptr, got.data_ptr, B, C, H, W, p, D, None)
+    assert np.array_equal(got.numpy(), exp.numpy())
+
+
+def test_patch_embedding_refuses_a_ragged_image():
+    z = L.Tensor.empty((1, 3, 20, 32), L.float32, "hip")
+    o = L.Tensor.empty((1, 3, 8), L.float32, "hip")
+    with pytest.raises(Exception, match="whole number"):
+        _C.call("lq_patch_embed_f32", z.data_ptr, z.data_ptr, None, z.data_ptr, z.data_ptr, o.data_ptr,
+                1, 3, 20, 32, 16, 8, None)
 
 
 SMALL = dict(image=64, patch=16, dim=128, depth=2, heads=2, mlp=256, classes=10)

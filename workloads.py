@@ -300,12 +300,10 @@ class QViT(nn.Module):
         B, C, H, W = x.shape
         ps, d = cfg["patch"], cfg["dim"]
         n = (H // ps) * (W // ps)
-        rows = L.Tensor.empty((B * n, C * ps * ps), L.float32, "hip")
-        _C.call("lq_patchify_f32", x.data_ptr, rows.data_ptr, B, C, H, W, ps, None)
-        emb = F.linear_f32(rows, self.patch_weight, self.patch_bias)
+        # patch rows, their Linear, the class token and the position table in one launch
         tok = L.Tensor.empty((B, n + 1, d), L.float32, "hip")
-        _C.call("lq_assemble_tokens_f32", emb.data_ptr, self.cls_token.data_ptr, self.pos_embed.data_ptr,
-                tok.data_ptr, B, n + 1, d, None)
+        _C.call("lq_patch_embed_f32", x.data_ptr, self.patch_weight.data_ptr, self.patch_bias.data_ptr,
+                self.cls_token.data_ptr, self.pos_embed.data_ptr, tok.data_ptr, B, C, H, W, ps, d, None)
         tok = self.norm(self.blocks(tok))
         # class-token pooling: row 0 of every image
         cls = L.Tensor.empty((B, d), L.float32, "hip")
