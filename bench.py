@@ -575,11 +575,12 @@ def bench_vit_b16(L, _C, steps, warmup):
 
 def bench_dynamic_mlp(L, Q, _C, steps, warmup):
     """Dynamic-quantized MLP Linear(784,256)-ReLU-Linear(256,10), batch 64
-    (launch-latency bound: 0.43 MOP).  Eager = one Python-driven forward (ONE launch: a single
-    block takes each layer's min / max, qparams and codes, multiplies, and applies the ReLU
-    between them); graph = the forward replayed from a HIP graph, which holds the two layers as
-    two launches of many blocks (nn.Sequential does not fuse under capture: shorter on the GPU,
-    and a replay pays the launch cost once either way)."""
+    (launch-latency bound: 0.43 MOP).  One forward is ONE launch (layer 1 as 64 blocks, each taking
+    the input's min / max, qparams and its rows' codes itself; the last block to finish reduces
+    the hidden activation's range and runs layer 2) when driven from Python, which is bound by
+    what a launch costs the host; a captured graph holds the two layers as two launches (shorter
+    kernels, and a replay pays the launch cost once either way).  Eager = Python-driven forwards
+    back to back; graph = the forward replayed from a HIP graph."""
     import lucid_amd.nn as nn
 
     rng = np.random.default_rng(1)

@@ -424,10 +424,10 @@ int lq_dynamic_linear_small_f32(const float* x, int M, int K, const int8_t* w, i
                                 const int32_t* wsum, const float* bias, int relu, int symmetric, int qmin, int qmax,
                                 int is_signed, float eps, int code_offset, float* out, lq_stream stream);
 
-/* Two dynamic-quantized Linears in ONE launch of one block: y = L2(act1(L1(x))) with each layer as
+/* Two dynamic-quantized Linears in ONE launch: y = L2(act1(L1(x))) with each layer as
  * lq_dynamic_linear_small_f32 computes it (the hidden activation's min / max, qparams and codes
- * included: one block owns the batch, so that reduction is block-wide) and relu1 / relu2 the
- * optional ReLU behind each.  x [M, K1] float32, w1 [N1, K1], w2 [N2, N1] int8 codes with their
+ * included: the blocks of layer 1 pass their tiles and ranges through the stream's scratch and
+ * the last of them to arrive runs layer 2) and relu1 / relu2 the optional ReLU behind each.  x [M, K1] float32, w1 [N1, K1], w2 [N2, N1] int8 codes with their
  * per-row scales, code sums and float32 biases (or NULL); out [M, N2] float32.  M <= 64,
  * K1 % 16 == 0 and <= 1024, N1 % 16 == 0 and <= 256, N2 <= 64; anything else
  * LQ_ERR_NOT_IMPLEMENTED.  Same bits as the separate calls (Linear, ReLU, Linear of a

@@ -13,6 +13,7 @@ in and out; every compute entry point requires ``device == "hip"`` and raises
 from __future__ import annotations
 
 import ctypes as C
+import math
 import weakref
 from dataclasses import dataclass
 
@@ -133,7 +134,7 @@ class Tensor:
     def empty(shape, dt=float32, device="hip") -> "Tensor":
         dt = as_dtype(dt)
         shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
-        n = int(np.prod(shape, dtype=np.int64))
+        n = math.prod(shape)
         if _norm_device(device) == "cpu":
             return Tensor(shape, dt, "cpu", host=np.empty(shape, dt.np))
         return Tensor(shape, dt, "hip", buf=DeviceBuffer(n * dt.itemsize))
@@ -157,7 +158,7 @@ class Tensor:
 
     @property
     def numel(self) -> int:
-        return int(np.prod(self.shape, dtype=np.int64))
+        return math.prod(self.shape)
 
     @property
     def nbytes(self) -> int:
@@ -267,9 +268,9 @@ class Tensor:
             shape = tuple(shape[0])
         shape = list(shape)
         if -1 in shape:
-            known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
+            known = math.prod(s for s in shape if s != -1)
             shape[shape.index(-1)] = self.numel // max(known, 1)
-        if int(np.prod(shape, dtype=np.int64)) != self.numel:
+        if math.prod(shape) != self.numel:
             raise _C.ShapeMismatch(f"cannot reshape {self.shape} to {tuple(shape)}")
         if self.device == "cpu":
             return Tensor(shape, self.dtype, "cpu", host=self._host.reshape(shape))

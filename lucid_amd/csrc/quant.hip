@@ -870,33 +870,58 @@ __global__ __launch_bounds__(1024) void dynamic_linear_small_kernel(
 }
 
 // Two dynamic-quantized Linears with an optional ReLU after each, on a small activation, in ONE
-// launch of ONE block (the MLP Linear(784,256) -> ReLU -> Linear(256,10) at batch 64 is 0.43 MOP:
-// three launches cost three round trips).  The block does, in order, exactly what the separate
-// operators do - the tensor's min / max, calculate_qparams, the activation codes, the integer
-// GEMM, float(acc - zp * wsum[n]) * (s * w_scale[n]) + bias[n], ReLU - for the first layer, keeps
-// its float32 output in LDS, and repeats the sequence on it for the second: the hidden
-// activation's min / max is a block-wide reduction because one block owns the whole batch.  Same
-// bits as two lq_dynamic_linear_small_f32 calls (the ReLU in between folded into the first).
-// LDS: codes of x [64][K1] | hidden float32 [64][N1] | hidden codes [64][N1].
-__global__ __launch_bounds__(1024) void dynamic_mlp2_small_kernel(
+// launch (the MLP Linear(784,256) -> ReLU -> Linear(256,10) at batch 64 is 0.43 MOP: three
+// launches cost three round trips).  Layer 1 runs exactly as dynamic_linear_small_kernel runs it -
+// a block per 16 x 16 tile of the hidden activation, so the 50 k inputs are quantized by 64 CUs
+// at once - with each block's tile (ReLU applied) and its min / max written through to device
+// scope; the block that arrives last (one counter, at most 64 arrivals) then owns the whole
+// hidden activation - 64 KB, one round trip - and does for layer 2 what the separate operators
+// do: the tensor's min / max (from the tiles'), calculate_qparams, the codes, the integer GEMM
+// (one wavefront per 16 x 16 output tile), float(acc - zp * wsum[n]) * (s * w_scale[n]) + bias[n],
+// ReLU.  Same bits as two lq_dynamic_linear_small_f32 calls (the ReLU between them folded into
+// the first).  15.7 us for that MLP; with ONE block doing both layers it was 21 us (one CU's
+// vector units quantized all 50 k inputs).  `hid`: [M][N1] float32, then 64 minima and 64 maxima;
+// `counter`: zero between launches (the last block resets it).
+__global__ __launch_bounds__(1024) void dynamic_mlp2_blocks_kernel(
     const float* __restrict__ x, int M, int K1, const int8_t* __restrict__ w1, int N1, const float* __restrict__ ws1,
     const int32_t* __restrict__ wsum1, const float* __restrict__ b1, int relu1, const int8_t* __restrict__ w2, int N2,
     const float* __restrict__ ws2, const int32_t* __restrict__ wsum2, const float* __restrict__ b2, int relu2,
-    int symmetric, int qmin, int qmax, int is_signed, float eps, float half_range, int off, float* __restrict__ out) {
-    extern __shared__ __attribute__((aligned(16))) int8_t ml_smem[];
+    int symmetric, int qmin, int qmax, int is_signed, float eps, float half_range, int off, float* __restrict__ out,
+    float* hid, int* counter) {
+    extern __shared__ __attribute__((aligned(16))) int8_t mb_smem[];
     __shared__ float s_sz[4];
-    typedef int ml_v4i __attribute__((ext_vector_type(4)));
+    __shared__ int s_arrived;
+    typedef int mb_v4i __attribute__((ext_vector_type(4)));
+    typedef unsigned mb_v4u __attribute__((ext_vector_type(4)));
+    constexpr unsigned kScopeDevice = 16;  // "sc1" cache-policy bit of buffer accesses
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int ln = lane & 15, lg = lane >> 4;
-    int8_t* const codes1 = ml_smem;                                             // [64][K1]
-    float* const hid = reinterpret_cast<float*>(ml_smem + size_t(64) * K1);      // [64][N1]
-    int8_t* const codes2 = ml_smem + size_t(64) * K1 + size_t(64) * N1 * 4;      // [64][N1]
+    int8_t* const codes = mb_smem;                                      // [16][K1]: the block's rows
+    int* const red = reinterpret_cast<int*>(mb_smem + size_t(16) * K1);  // [4][64]
+    int8_t* const codes2 = mb_smem + size_t(16) * K1 + 1024;             // [64][N1]: the last block's
     constexpr int kKeep = 16;
     const float qnan = __builtin_nanf("");
-
-    // ---- layer 1: range, qparams and codes of x (all rows; rows past M are zero codes)
     const int quads = (M * K1) >> 2;
     const float4* x4 = reinterpret_cast<const float4*>(x);
+    const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+    const int nblocks = gridDim.x * gridDim.y, bid = blockIdx.y * gridDim.x + blockIdx.x;
+    const int ln = lane & 15, lg = lane >> 4;
+    const int rq = lane >> 2, cq = lane & 3;
+    const int8_t* wrow = w1 + size_t(n0 + rq < N1 ? n0 + rq : N1 - 1) * size_t(K1);
+    auto place = [&](mb_v4i f) {
+        const int from = (4 * ln + lg) * 4;
+        return mb_v4i{__builtin_amdgcn_ds_bpermute(from, f[0]), __builtin_amdgcn_ds_bpermute(from, f[1]),
+                      __builtin_amdgcn_ds_bpermute(from, f[2]), __builtin_amdgcn_ds_bpermute(from, f[3])};
+    };
+    const size_t hid_bytes = size_t(M) * N1 * 4;
+    const __amdgpu_buffer_rsrc_t hbuf = __builtin_amdgcn_make_buffer_rsrc(hid, 0, int(hid_bytes) + 512, 0x00020000);
+    const int ksteps = (K1 + 63) >> 6;
+    const bool first_in_k = wave < ksteps && wave * 64 + cq * 16 < K1;
+    const mb_v4i wf_first = first_in_k ? *reinterpret_cast<const mb_v4i*>(wrow + wave * 64 + cq * 16) : mb_v4i{0, 0, 0, 0};
+    const int out_n = n0 + (tid & 15);
+    const bool out_lane = tid < 256 && out_n < N1;
+    const float c_ws = (out_lane && ws1) ? ws1[out_n] : 1.0f;
+    const int c_wsum = (out_lane && wsum1) ? wsum1[out_n] : 0;
+    const float c_bias = (out_lane && b1) ? b1[out_n] : -0.0f;
     MinMax m{__builtin_inff(), -__builtin_inff(), 0};
     float4 v[kKeep];
 #pragma unroll
@@ -904,35 +929,10 @@ __global__ __launch_bounds__(1024) void dynamic_mlp2_small_kernel(
         const int i = u * 1024 + tid;
         if (i < quads) v[u] = x4[i];
     }
-    // A wavefront owns one block of 16 columns of layer 1 (N1 <= 256 = 16 wavefronts x 16) over
-    // at most 16 k steps, and one 16 x 16 tile of layer 2 over at most 4.  All its weight
-    // fragments of a layer are requested together - layer 2's here, behind x; layer 1's as soon as
-    // the registers that hold x are free - so each layer pays one memory round trip.  (Requested
-    // one k step ahead instead, the 13 dependent round trips of K1 = 784 were most of the time.)
-    constexpr int kSteps1 = 16, kSteps2 = 4;
-    const int n1 = wave * 16 + ln, nc1 = n1 < N1 ? n1 : N1 - 1;  // the column whose results this lane holds
-    const int rb2 = wave & 3, cb2 = wave >> 2;
-    const int n2 = cb2 * 16 + ln, nc2 = n2 < N2 ? n2 : N2 - 1;
-    // For the request a lane takes 16-byte chunk lane % 4 of row lane / 4, so that four
-    // neighbouring lanes read 64 contiguous bytes (with the operand layout - row lane % 16, chunk
-    // lane / 16 - every lane would be a cache access of its own: 64 per instruction on the one CU
-    // that runs this block); ml_place then hands each chunk to the lane that multiplies it.
-    const int rq = lane >> 2, cq = lane & 3;
-    auto ml_place = [&](ml_v4i f) {
-        const int from = (4 * ln + lg) * 4;
-        return ml_v4i{__builtin_amdgcn_ds_bpermute(from, f[0]), __builtin_amdgcn_ds_bpermute(from, f[1]),
-                      __builtin_amdgcn_ds_bpermute(from, f[2]), __builtin_amdgcn_ds_bpermute(from, f[3])};
-    };
-    ml_v4i w1f[kSteps1], w2f[kSteps2];
-    {
-        const int r2 = cb2 * 16 + rq;
-        const int8_t* wrow2 = w2 + size_t(r2 < N2 ? r2 : N2 - 1) * size_t(N1) + cq * 16;
-#pragma unroll
-        for (int ks = 0; ks < kSteps2; ++ks)  // N1 % 16 == 0: a 16-byte chunk is inside or outside as a whole
-            w2f[ks] = ks * 64 + cq * 16 < N1 ? *reinterpret_cast<const ml_v4i*>(wrow2 + ks * 64) : ml_v4i{0, 0, 0, 0};
-    }
-    for (int i = quads + tid; i < 16 * K1; i += 1024) reinterpret_cast<unsigned*>(codes1)[i] = 0u;
-    for (int i = ((M * N1) >> 2) + tid; i < 16 * N1; i += 1024) reinterpret_cast<unsigned*>(codes2)[i] = 0u;
+    if (tid < 256) red[tid] = 0;
+    const int q_lo = (m0 * K1) >> 2;
+    const int q_hi = ((m0 + 16 < M ? m0 + 16 : M) * K1) >> 2;
+    for (int i = q_hi - q_lo + tid; i < 4 * K1; i += 1024) reinterpret_cast<unsigned*>(codes)[i] = 0u;
 #pragma unroll
     for (int u = 0; u < kKeep; ++u)
         if (u * 1024 + tid < quads) mm_update(m, v[u].x), mm_update(m, v[u].y), mm_update(m, v[u].z), mm_update(m, v[u].w);
@@ -943,121 +943,136 @@ __global__ __launch_bounds__(1024) void dynamic_mlp2_small_kernel(
         s_sz[0] = s, s_sz[1] = z;
     }
     __syncthreads();
+    const float s = s_sz[0], z = s_sz[1], r = 1.0f / s;
     {
-        const float s = s_sz[0], z = s_sz[1], r = 1.0f / s;
-        const QuantizeOp<int8_t> op{x4, reinterpret_cast<Code8x4*>(codes1), float(double(qmin)), float(double(qmax)), off};
+        const QuantizeOp<int8_t> op{x4, reinterpret_cast<Code8x4*>(codes), float(double(qmin)), float(double(qmax)), off};
 #pragma unroll
         for (int u = 0; u < kKeep; ++u) {
             const int i = u * 1024 + tid;
-            if (i < quads) op.q[i] = op.pack(v[u], s, z, r);
+            if (i >= q_lo && i < q_hi) op.q[i - q_lo] = op.pack(v[u], s, z, r);
         }
-    }
-    {
-        const int r1 = wave * 16 + rq;
-        const int8_t* wrow1 = w1 + size_t(r1 < N1 ? r1 : N1 - 1) * size_t(K1) + cq * 16;
-#pragma unroll
-        for (int ks = 0; ks < kSteps1; ++ks)
-            w1f[ks] = ks * 64 + cq * 16 < K1 ? *reinterpret_cast<const ml_v4i*>(wrow1 + ks * 64) : ml_v4i{0, 0, 0, 0};
     }
     __syncthreads();
-
-    // ---- layer 1: GEMM.  A wavefront owns 16 output columns (a weight fragment is loaded once per
-    // k step and multiplied with the four row blocks of the batch) and applies the epilogue itself.
+    mb_v4i acc = mb_v4i{0, 0, 0, 0};
+    for (int ks = wave; ks < ksteps; ks += 16) {
+        const int k = ks * 64 + lg * 16;
+        const bool in_k = k < K1;
+        const int kq = ks * 64 + cq * 16;
+        const mb_v4i wf = place(ks == wave ? wf_first
+                                           : (kq < K1 ? *reinterpret_cast<const mb_v4i*>(wrow + kq) : mb_v4i{0, 0, 0, 0}));
+        const mb_v4i af = in_k ? *reinterpret_cast<const mb_v4i*>(codes + size_t(ln) * K1 + k) : mb_v4i{0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc, 0, 0, 0);
+    }
+    if (wave < ksteps) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            __hip_atomic_fetch_add(&red[q * 64 + lane], acc[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
     MinMax hm{__builtin_inff(), -__builtin_inff(), 0};
-    {
-        const float s = s_sz[0], z = s_sz[1];
-        const int zp = int(z) + off;
-        if (wave * 16 < N1) {
-            const int n = n1, nc = nc1;
-            const float c_ws = ws1 ? ws1[nc] : 1.0f;
-            const int c_wsum = wsum1 ? wsum1[nc] : 0;
-            const float c_bias = b1 ? b1[nc] : -0.0f;
-            ml_v4i acc[4];
-#pragma unroll
-            for (int rb = 0; rb < 4; ++rb) acc[rb] = ml_v4i{0, 0, 0, 0};
-#pragma unroll
-            for (int ks = 0; ks < kSteps1; ++ks) {
-                const int k = ks * 64 + lg * 16;
-                if (ks * 64 < K1) {  // uniform
-                    const bool in_k = k < K1;
-                    const ml_v4i wf = ml_place(w1f[ks]);
-#pragma unroll
-                    for (int rb = 0; rb < 4; ++rb) {
-                        const ml_v4i af = in_k ? *reinterpret_cast<const ml_v4i*>(codes1 + size_t(16 * rb + ln) * K1 + k)
-                                               : ml_v4i{0, 0, 0, 0};
-                        acc[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, wf, acc[rb], 0, 0, 0);
-                    }
-                }
-            }
-            // acc[rb][q]: activation row 16 rb + 4 (lane / 16) + q, weight row n
+    if (tid < 256) {
+        const int q = tid >> 6, l = tid & 63;
+        const int mm = m0 + 4 * (l >> 4) + q, nn = n0 + (l & 15);
+        if (mm < M && nn < N1) {
+            const int zp = int(z) + off;
             const int corr = (wsum1 != nullptr && zp != 0) ? zp * c_wsum : 0;
+            const float f = float(red[tid] - corr);
             const float sc = s * c_ws;
+            float y = f * sc;
+            y = y + c_bias;
             const float floor = relu1 ? 0.0f : -__builtin_inff();
-#pragma unroll
-            for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int mm = 16 * rb + 4 * lg + q;
-                    if (mm < M && n < N1) {
-                        const float f = float(acc[rb][q] - corr);
-                        float y = f * sc;
-                        y = y + c_bias;
-                        y = (y < floor) ? floor : y;
-                        hid[mm * N1 + n] = y;
-                        mm_update(hm, y);
-                    }
-                }
+            y = (y < floor) ? floor : y;
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), hbuf, unsigned(mm * N1 + nn) * 4, 0, kScopeDevice);
+            mm_update(hm, y);
         }
     }
-    // ---- layer 2: range, qparams and codes of the hidden activation
-    hm = mm_block_reduce(hm);  // (its barrier also publishes hid)
+    hm = mm_block_reduce(hm);
     if (tid == 0) {
-        float s, z;
-        qparams_of(hm.nan ? qnan : hm.lo, hm.nan ? qnan : hm.hi, symmetric, qmin, qmax, is_signed, eps, half_range, &s, &z);
-        s_sz[2] = s, s_sz[3] = z;
+        const float lo = hm.nan ? qnan : hm.lo, hi = hm.nan ? qnan : hm.hi;
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(lo), hbuf, unsigned(hid_bytes) + bid * 4, 0, kScopeDevice);
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(hi), hbuf, unsigned(hid_bytes) + 256 + bid * 4, 0, kScopeDevice);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this thread's part of the tile has been written through
+    __syncthreads();
+    if (tid == 0) s_arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_arrived != nblocks - 1) return;
+
+    // ---- the last block: layer 2 on the whole hidden activation.  Everything it needs from
+    // memory is requested together: the tiles' ranges, the activation, its weight fragments.
+    float slot_lo = __builtin_inff(), slot_hi = -__builtin_inff();
+    if (tid < nblocks) {
+        slot_lo = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(hbuf, unsigned(hid_bytes) + tid * 4, 0, kScopeDevice));
+        slot_hi = __uint_as_float(
+            __builtin_amdgcn_raw_buffer_load_b32(hbuf, unsigned(hid_bytes) + 256 + tid * 4, 0, kScopeDevice));
+    }
+    const int quads2 = (M * N1) >> 2;  // at most 4096: four per thread
+    mb_v4u h[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = u * 1024 + tid;
+        h[u] = __builtin_amdgcn_raw_buffer_load_b128(hbuf, unsigned(i < quads2 ? i : 0) * 16, 0, kScopeDevice);
+    }
+    constexpr int kSteps2 = 4;
+    const int rb2 = wave & 3, cb2 = wave >> 2;
+    const int n2 = cb2 * 16 + ln, nc2 = n2 < N2 ? n2 : N2 - 1;
+    mb_v4i w2f[kSteps2];
+    {
+        const int r2 = cb2 * 16 + rq;
+        const int8_t* wrow2 = w2 + size_t(r2 < N2 ? r2 : N2 - 1) * size_t(N1) + cq * 16;
+#pragma unroll
+        for (int ks = 0; ks < kSteps2; ++ks)
+            w2f[ks] = ks * 64 + cq * 16 < N1 ? *reinterpret_cast<const mb_v4i*>(wrow2 + ks * 64) : mb_v4i{0, 0, 0, 0};
+    }
+    const float c_ws2 = ws2 ? ws2[nc2] : 1.0f;
+    const int c_wsum2 = wsum2 ? wsum2[nc2] : 0;
+    const float c_bias2 = b2 ? b2[nc2] : -0.0f;
+    for (int i = quads2 + tid; i < 16 * N1; i += 1024) reinterpret_cast<unsigned*>(codes2)[i] = 0u;
+    MinMax tm{slot_lo, slot_hi, int((slot_lo != slot_lo) | (slot_hi != slot_hi))};
+    if (tm.nan) tm.lo = __builtin_inff(), tm.hi = -__builtin_inff();
+    tm = mm_block_reduce(tm);
+    if (tid == 0) {
+        float s2, z2;
+        qparams_of(tm.nan ? qnan : tm.lo, tm.nan ? qnan : tm.hi, symmetric, qmin, qmax, is_signed, eps, half_range, &s2, &z2);
+        s_sz[2] = s2, s_sz[3] = z2;
+        *counter = 0;  // ready for the next launch
     }
     __syncthreads();
     const float s2 = s_sz[2], z2 = s_sz[3];
     {
         const float r2 = 1.0f / s2;
-        const float4* h4 = reinterpret_cast<const float4*>(hid);
-        const QuantizeOp<int8_t> op{h4, reinterpret_cast<Code8x4*>(codes2), float(double(qmin)), float(double(qmax)), off};
-        const int quads2 = (M * N1) >> 2;
-        for (int i = tid; i < quads2; i += 1024) op.q[i] = op.pack(h4[i], s2, z2, r2);
+        const QuantizeOp<int8_t> op{nullptr, reinterpret_cast<Code8x4*>(codes2), float(double(qmin)), float(double(qmax)), off};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = u * 1024 + tid;
+            if (i < quads2) op.q[i] = op.pack(__builtin_bit_cast(float4, h[u]), s2, z2, r2);
+        }
     }
     __syncthreads();
-    // ---- layer 2: GEMM, one wavefront per 16 x 16 output tile
-    {
-        const int rb = rb2, cb = cb2;
-        if (cb * 16 < N2 && rb * 16 < M) {
-            const int zp = int(z2) + off;
-            const int n = n2, nc = nc2;
-            const float c_ws = ws2 ? ws2[nc] : 1.0f;
-            const int c_wsum = wsum2 ? wsum2[nc] : 0;
-            const float c_bias = b2 ? b2[nc] : -0.0f;
-            ml_v4i acc = ml_v4i{0, 0, 0, 0};
+    if (cb2 * 16 < N2 && rb2 * 16 < M) {
+        const int zp = int(z2) + off;
+        mb_v4i acc2 = mb_v4i{0, 0, 0, 0};
 #pragma unroll
-            for (int ks = 0; ks < kSteps2; ++ks) {
-                const int k = ks * 64 + lg * 16;
-                if (ks * 64 < N1) {  // uniform
-                    const ml_v4i af = k < N1 ? *reinterpret_cast<const ml_v4i*>(codes2 + size_t(16 * rb + ln) * N1 + k)
-                                             : ml_v4i{0, 0, 0, 0};
-                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, ml_place(w2f[ks]), acc, 0, 0, 0);
-                }
+        for (int ks = 0; ks < kSteps2; ++ks) {
+            const int k = ks * 64 + lg * 16;
+            if (ks * 64 < N1) {  // uniform
+                const mb_v4i af = k < N1 ? *reinterpret_cast<const mb_v4i*>(codes2 + size_t(16 * rb2 + ln) * N1 + k)
+                                         : mb_v4i{0, 0, 0, 0};
+                acc2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, place(w2f[ks]), acc2, 0, 0, 0);
             }
-            const int corr = (wsum2 != nullptr && zp != 0) ? zp * c_wsum : 0;
-            const float sc = s2 * c_ws;
-            const float floor = relu2 ? 0.0f : -__builtin_inff();
+        }
+        const int corr = (wsum2 != nullptr && zp != 0) ? zp * c_wsum2 : 0;
+        const float sc = s2 * c_ws2;
+        const float floor = relu2 ? 0.0f : -__builtin_inff();
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int mm = 16 * rb + 4 * lg + q;
-                if (mm < M && n < N2) {
-                    const float f = float(acc[q] - corr);
-                    float y = f * sc;
-                    y = y + c_bias;
-                    y = (y < floor) ? floor : y;
-                    out[size_t(mm) * N2 + n] = y;
-                }
+        for (int q = 0; q < 4; ++q) {
+            const int mm = 16 * rb2 + 4 * lg + q;
+            if (mm < M && n2 < N2) {
+                const float f = float(acc2[q] - corr);
+                float y = f * sc;
+                y = y + c_bias2;
+                y = (y < floor) ? floor : y;
+                out[size_t(mm) * N2 + n2] = y;
             }
         }
     }
@@ -1099,7 +1114,7 @@ int lq_dynamic_mlp2_small_f32(const float* x, int M, int K1, const int8_t* w1, i
     LQ_REQUIRE(x && w1 && w2 && out, LQ_ERR_VALUE, "dynamic_mlp2_small: NULL pointer");
     LQ_REQUIRE(qmax > qmin && qmin + code_offset >= -128 && qmax + code_offset <= 127, LQ_ERR_VALUE,
                "dynamic_mlp2_small: grid [%d,%d] + offset %d does not fit int8", qmin, qmax, code_offset);
-    // one block holds x's codes (64 K1 bytes), the hidden activation (256 N1 bytes) and its codes (64 N1 bytes)
+    // a block holds 16 rows of x's codes; the last one also the hidden activation's codes (64 N1 bytes)
     LQ_REQUIRE(M > 0 && M <= 64 && K1 >= 16 && K1 % 16 == 0 && K1 <= 1024 && long(M) * K1 <= 65536 && N1 >= 16 &&
                    N1 % 16 == 0 && N1 <= 256 && N2 > 0 && N2 <= 64 && aligned16(x) && aligned16(w1) && aligned16(w2),
                LQ_ERR_NOT_IMPLEMENTED,
@@ -1107,13 +1122,18 @@ int lq_dynamic_mlp2_small_f32(const float* x, int M, int K1, const int8_t* w1, i
                "16 up to 256 and up to 64 outputs (got M = %d, K1 = %d, N1 = %d, N2 = %d); use two "
                "lq_dynamic_linear_small_f32 calls", M, K1, N1, N2);
     const float half_range = float((double(qmax) - double(qmin)) / 2.0);
-    const size_t lds = size_t(64) * K1 + size_t(64) * N1 * 5;
+    // the hidden activation and the tiles' ranges pass through the stream's split-K scratch
+    SkScratch sk;
+    const size_t hid_bytes = size_t(M) * N1 * 4;
+    if (int rc = sk_scratch(1, hid_bytes + 512, as_stream(stream), &sk)) return rc;
+    const size_t lds = size_t(16) * K1 + 1024 + size_t(64) * N1;
     static DeviceOnce attr_once;
-    if (int rc = allow_dynamic_lds(attr_once, reinterpret_cast<const void*>(dynamic_mlp2_small_kernel), 152 * 1024))
+    if (int rc = allow_dynamic_lds(attr_once, reinterpret_cast<const void*>(dynamic_mlp2_blocks_kernel), 64 * 1024))
         return rc;
-    hipLaunchKernelGGL(dynamic_mlp2_small_kernel, dim3(1), dim3(1024), lds, as_stream(stream), x, M, K1, w1, N1, w1_scale,
-                       w1sum, bias1, relu1, w2, N2, w2_scale, w2sum, bias2, relu2, symmetric, qmin, qmax, is_signed, eps,
-                       half_range, code_offset, out);
+    hipLaunchKernelGGL(dynamic_mlp2_blocks_kernel, dim3(unsigned(N1 / 16), unsigned((M + 15) / 16)), dim3(1024), lds,
+                       as_stream(stream), x, M, K1, w1, N1, w1_scale, w1sum, bias1, relu1, w2, N2, w2_scale, w2sum, bias2,
+                       relu2, symmetric, qmin, qmax, is_signed, eps, half_range, code_offset, out,
+                       reinterpret_cast<float*>(sk.slabs), sk.counters);
     LQ_CHECK_LAUNCH("dynamic_mlp2_small");
     return LQ_OK;
 }

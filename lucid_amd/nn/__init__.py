@@ -31,12 +31,11 @@ def _fused_dynamic_pair(mods, i, x):
     ``nn.quantized.dynamic`` on an activation small enough for the one-launch kernel, else ``None``
     (no hooks on the modules: a hook has to see each module's own output).
 
-    Not while a graph is being captured.  The one launch is one block on one CU (21 us for
-    784-256-10 at batch 64: that CU's vector units quantize all 50 k inputs), the two separate
-    layers are two launches of many blocks (8 + 6 us).  Launched from Python the one launch wins,
-    27 against 53 us per forward, because each launch costs the host about as much as it runs; a
-    replayed graph pays its ~11 us once whichever it holds, and there the shorter kernels win,
-    25 against 33 us.  Same bits either way."""
+    Not while a graph is being captured.  The one launch (15.7 us of kernel for 784-256-10 at
+    batch 64: layer 2 waits for the last block of layer 1 through device-scope memory) saves the
+    host a launch, which is what a Python-driven forward is bound by; the two separate layers are
+    8 + 6 us of kernels, and a replayed graph, which pays its launch cost once whichever it holds,
+    is shorter with those: 25 against 31 us.  Same bits either way."""
     from .quantized.dynamic import linear as _dyn
     from .. import graph as _graph
 
@@ -49,8 +48,10 @@ def _fused_dynamic_pair(mods, i, x):
     j = i + 2 if relu else i + 1
     if j >= len(mods) or type(mods[j]) is not _dyn.Linear:
         return None
-    if any(getattr(m, "_forward_hooks", None) or getattr(m, "_forward_pre_hooks", None) for m in mods[i:j + 1]):
-        return None
+    for m in mods[i:j + 1]:
+        d = m.__dict__  # (not getattr: a name a module lacks costs an exception inside Module.__getattr__)
+        if d.get("_forward_hooks") or d.get("_forward_pre_hooks"):
+            return None
     y = _dyn.fused_pair(first, relu, mods[j], x)
     return None if y is None else (y, j + 1)
 

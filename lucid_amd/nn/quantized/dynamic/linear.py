@@ -30,9 +30,9 @@ SMALL_LINEAR_MAX_K = 6080
 
 def fused_pair(first, relu_between: bool, second, x):
     """``second(relu(first(x)))`` (or without the ReLU) for two dynamic ``Linear`` layers on a small
-    activation as ONE launch (``lq_dynamic_mlp2_small_f32``: one block owns the batch, so the hidden
-    activation's min / max is a block-wide reduction), or ``None`` when the shapes or operands do
-    not qualify.  Same bits as calling the modules one after the other."""
+    activation as ONE launch (``lq_dynamic_mlp2_small_f32``: the last block of layer 1 to finish
+    reduces the hidden activation's min / max and runs layer 2), or ``None`` when the shapes or
+    operands do not qualify.  Same bits as calling the modules one after the other."""
     if not (isinstance(first, Linear) and isinstance(second, Linear) and isinstance(x, Tensor)):
         return None
     if x.device != "hip" or x.dtype != T.float32 or x._grid is not None or x._range is not None:
@@ -46,19 +46,22 @@ def fused_pair(first, relu_between: bool, second, x):
         return None
     if first.act_qdtype is not second.act_qdtype:
         return None
-    for lin in (first, second):
-        if weight_zero_points(lin) is not None or (lin.bias is not None and lin.bias.dtype != T.float32):
+    # (the buffers straight from the registries: this path is bound by what a forward costs the host)
+    b1, b2 = first._buffers, second._buffers
+    bias1, bias2 = b1.get("bias"), b2.get("bias")
+    for lin, bias in ((first, bias1), (second, bias2)):
+        if weight_zero_points(lin) is not None or (bias is not None and bias.dtype != T.float32):
             return None
         if lin._wsum is None:
             lin._wsum = _ops.rowsum_i8(lin.weight_int8)
     qd = first.act_qdtype
-    y = Tensor.empty((M, N2), T.float32, "hip")
-    _C.call("lq_dynamic_mlp2_small_f32", x.data_ptr, M, K1, first.weight_int8.data_ptr, N1, first.weight_scale.data_ptr,
-            first._wsum.data_ptr, None if first.bias is None else first.bias.data_ptr, int(relu_between),
-            second.weight_int8.data_ptr, N2, second.weight_scale.data_ptr, second._wsum.data_ptr,
-            None if second.bias is None else second.bias.data_ptr, 0, 0, qd.quant_min, qd.quant_max, int(qd.signed),
+    y = Tensor.empty((*x.shape[:-1], N2), T.float32, "hip")
+    _C.call("lq_dynamic_mlp2_small_f32", x.data_ptr, M, K1, b1["weight_int8"].data_ptr, N1, b1["weight_scale"].data_ptr,
+            first._wsum.data_ptr, None if bias1 is None else bias1.data_ptr, int(relu_between),
+            b2["weight_int8"].data_ptr, N2, b2["weight_scale"].data_ptr, second._wsum.data_ptr,
+            None if bias2 is None else bias2.data_ptr, 0, 0, qd.quant_min, qd.quant_max, int(qd.signed),
             1e-8, storage_offset(qd), y.data_ptr, None)
-    return y.reshape(*x.shape[:-1], N2)
+    return y
 
 
 class Linear(Module):

@@ -555,8 +555,8 @@ class _recorded_calls:
 @pytest.mark.parametrize("kind", ["normal", "constant", "nan"])
 def test_two_dynamic_linears_in_one_launch(M, K1, N1, N2, relu, kind):
     """A Sequential of nnqd.Linear [, ReLU], nnqd.Linear on a small batch runs as ONE launch
-    (lq_dynamic_mlp2_small_f32: the hidden activation's min / max is a reduction inside the one
-    block that owns the batch): bit for bit what the modules give one after the other, and what
+    (lq_dynamic_mlp2_small_f32: the last block of layer 1 to finish reduces the hidden activation's
+    min / max and runs layer 2): bit for bit what the modules give one after the other, and what
     the oracle's integer formulation gives."""
     rng = np.random.default_rng(M + K1 + N1 + N2)
     l1, l2 = nn.Linear(K1, N1), nn.Linear(N1, N2)
@@ -599,8 +599,8 @@ def test_two_dynamic_linears_in_one_launch(M, K1, N1, N2, relu, kind):
 
 
 def test_two_dynamic_linears_keep_separate_launches_when_hooked_or_large():
-    """A forward hook has to see each module's own output, and a wide layer does not fit the one
-    block: the modules then run one after the other."""
+    """A forward hook has to see each module's own output, and a wide layer is not what the one
+    launch takes: the modules then run one after the other."""
     rng = np.random.default_rng(3)
     model = Q.quantize_dynamic(nn.Sequential(nn.Linear(64, 32), nn.ReLU(), nn.Linear(32, 8)))
     x = hip(rng.standard_normal((4, 64)).astype(np.float32))
@@ -615,8 +615,9 @@ def test_two_dynamic_linears_keep_separate_launches_when_hooked_or_large():
 
 
 def test_two_dynamic_linears_are_captured_as_separate_launches_with_the_same_bits():
-    """Under graph capture the pair is not fused (two launches of many blocks replay sooner than one
-    block on one CU); the replayed result equals the eager, fused one bit for bit."""
+    """Under graph capture the pair is not fused (the two layers' own kernels are shorter than the
+    one launch, which only saves the host a launch); the replayed result equals the eager, fused
+    one bit for bit - also with fused launches on other inputs between the replays."""
     rng = np.random.default_rng(5)
     model = Q.quantize_dynamic(nn.Sequential(nn.Linear(784, 256), nn.ReLU(), nn.Linear(256, 10)))
     x = hip(rng.standard_normal((64, 784)).astype(np.float32))
@@ -627,8 +628,12 @@ def test_two_dynamic_linears_are_captured_as_separate_launches_with_the_same_bit
         with _recorded_calls() as calls:
             y = model(x)
     assert "lq_dynamic_mlp2_small_f32" not in calls and calls.count("lq_dynamic_linear_small_f32") == 2
+    other = hip(rng.standard_normal((7, 784)).astype(np.float32) * 3)
+    other_eager = model[2](model[1](model[0](other))).numpy()
     for _ in range(3):
         g.replay()
         L.synchronize()
         assert np.array_equal(y.numpy().view(np.uint32), eager.view(np.uint32))
+        # the one launch again, smaller: its arrival counter and scratch are the previous call's
+        assert np.array_equal(model(other).numpy().view(np.uint32), other_eager.view(np.uint32))
     g.destroy()
