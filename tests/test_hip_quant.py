@@ -312,7 +312,8 @@ def _slice_to_host(t, sl, np_dtype):
     return out
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 4), (7, 784), (64, 1024), (33, 4096), (5, 16384), (3, 4100), (2, 20000)])
+@pytest.mark.parametrize("rows,cols", [(1, 4), (7, 784), (64, 1024), (33, 4096), (5, 16384), (3, 4100), (2, 20000),
+                                       (9, 1028), (6, 2048), (2048, 4096)])
 @pytest.mark.parametrize("scheme", ["sym_i8", "affine_u8", "affine_i8"])
 def test_quantize_rows_dynamic_equals_the_three_calls_and_the_oracle(rows, cols, scheme):
     """One pass per row (min / max -> qparams -> codes) against minmax + calculate_qparams +
