@@ -102,6 +102,7 @@ def test_patchify_and_token_assembly_are_exact():
     (5, 3, 96, 96, 16, 200, True),     # 180 patch rows: a ragged second row tile, images straddling tiles
     (2, 1, 30, 18, 6, 130, False),     # patch not a multiple of 4: the element-by-element gather
     (1, 2, 8, 8, 4, 8, True),
+    (2, 3, 12, 20, 4, 24, True),       # K = 48: a partial k tile
     (64, 3, 224, 224, 16, 768, True),  # ViT-B/16 at the bench batch
 ])
 def test_patch_embedding_in_one_launch_equals_the_three_steps(B, C, H, W, p, D, bias):
@@ -124,6 +125,28 @@ def test_patch_embedding_in_one_launch_equals_the_three_steps(B, C, H, W, p, D, 
     _C.call("lq_patch_embed_f32", img.data_ptr, w.data_ptr, bv.data_ptr if bias else None, cls.data_ptr,
             pos.data_ptr, got.data_ptr, B, C, H, W, p, D, None)
     assert np.array_equal(got.numpy(), exp.numpy())
+
+
+def test_patch_embedding_of_an_image_that_is_not_16_byte_aligned():
+    """The aligned-load form needs a 16-byte aligned image; one that starts 4 bytes further takes
+    the element-by-element gather and gives the same bits."""
+    rng = np.random.default_rng(12)
+    B, C, H, W, p, D = 2, 3, 32, 32, 16, 40
+    n, K = 4, C * p * p
+    flat = hip(rng.standard_normal(B * C * H * W + 1).astype(np.float32))
+    shifted = L.Tensor((B, C, H, W), L.float32, "hip", buf=flat._buf, offset=flat._offset + 4)
+    aligned = hip(flat.numpy()[1:].reshape(B, C, H, W).copy())
+    w = hip((rng.standard_normal((D, K)) / np.sqrt(K)).astype(np.float32))
+    bv, cls = hip(rng.standard_normal(D).astype(np.float32)), hip(rng.standard_normal(D).astype(np.float32))
+    pos = hip(rng.standard_normal((n + 1, D)).astype(np.float32))
+    outs = []
+    for img in (shifted, aligned):
+        assert (img.data_ptr % 16 == 0) == (img is aligned)
+        out = L.tensor(np.full((B, n + 1, D), np.nan, np.float32), device="hip")
+        _C.call("lq_patch_embed_f32", img.data_ptr, w.data_ptr, bv.data_ptr, cls.data_ptr, pos.data_ptr, out.data_ptr,
+                B, C, H, W, p, D, None)
+        outs.append(out.numpy())
+    assert np.array_equal(outs[0], outs[1]) and np.isfinite(outs[0]).all()
 
 
 def test_patch_embedding_refuses_a_ragged_image():
