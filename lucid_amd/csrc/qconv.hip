@@ -486,32 +486,46 @@ __global__ __launch_bounds__(256) void quantize_nchw_to_nhwc_small_c_kernel(
 // float32 NCHW (at most four channels) -> the packed four-channel, spatially pre-padded code
 // image of the few-channel route, in one pass: what lq_quantize_nchw_to_nhwc followed by
 // pack4_padded_kernel writes (the same quantization arithmetic; padding and spare channels hold
-// `fill`, the zero-point code).  One packed pixel per lane.
+// `fill`, the zero-point code).  A lane writes four consecutive packed pixels of one row as one
+// 16-byte store (rows of the packed image are a multiple of four pixels); its up to twelve
+// inputs are loaded from clamped addresses, all before the first is used, and what lies in the
+// padding is replaced afterwards.  Block = 64 quads x 4 rows, grid = (quads, rows, images).
 __global__ __launch_bounds__(256) void quantize_nchw_to_packed4_kernel(
     const float* __restrict__ x, int B, int C, int H, int W, int ph, int pw, int Hp, int Wp, const float* scale,
-    const float* zp, float lo, float hi, int off, int fill, uint32_t* __restrict__ out) {
+    const float* zp, float lo, float hi, int off, int fill, uint4* __restrict__ out) {
+    const int qx = blockIdx.x * 64 + (threadIdx.x & 63), hp = blockIdx.y * 4 + (threadIdx.x >> 6), b = blockIdx.z;
+    if (qx * 4 >= Wp || hp >= Hp) return;
     const float s = scale[0], z = zp[0];
-    const size_t n = size_t(B) * Hp * Wp, stride = size_t(gridDim.x) * 256, HW = size_t(H) * W;
-    const uint32_t f = uint32_t(uint8_t(fill));
-    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
-        const int wp = int(i % Wp);
-        const size_t r = i / Wp;
-        const int hp = int(r % Hp), b = int(r / Hp);
-        const int h = hp - ph, w = wp - pw;
-        uint32_t v = f | (f << 8) | (f << 16) | (f << 24);
-        if (h >= 0 && h < H && w >= 0 && w < W) {
-            v = 0;
-            for (int c = 0; c < 4; ++c) {
-                uint32_t code = f;
-                if (c < C) {
-                    const float u = q_core_local(x[(size_t(b) * C + c) * HW + size_t(h) * W + w], s, z, lo, hi);
-                    code = uint32_t(uint8_t(int8_t(((u != u) ? 0 : int(u)) + off)));
-                }
-                v |= code << (8 * c);
-            }
+    const int h = hp - ph, w0 = qx * 4 - pw;
+    const bool row_in = h >= 0 && h < H;
+    const size_t HW = size_t(H) * W;
+    const float* xr = x + size_t(b) * C * HW + size_t(row_in ? h : 0) * W;
+    float v[4][4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int w = w0 + j;
+            v[c][j] = c < C ? xr[size_t(c) * HW + (w < 0 ? 0 : (w >= W ? W - 1 : w))] : 0.0f;
         }
-        out[i] = v;
+    const uint32_t f = uint32_t(uint8_t(fill));
+    uint32_t px[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int w = w0 + j;
+        uint32_t p = 0;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint32_t code = f;
+            if (c < C) {
+                const float u = q_core_local(v[c][j], s, z, lo, hi);
+                code = uint32_t(uint8_t(int8_t(((u != u) ? 0 : int(u)) + off)));
+            }
+            p |= code << (8 * c);
+        }
+        px[j] = (row_in && w >= 0 && w < W) ? p : (f | (f << 8) | (f << 16) | (f << 24));
     }
+    out[(size_t(b) * Hp + hp) * (Wp / 4) + qx] = uint4{px[0], px[1], px[2], px[3]};
 }
 
 // Extents of the packed image of a few-channel layer: rows start 16-byte aligned and the last
@@ -878,9 +892,11 @@ int lq_quantize_nchw_to_packed4(const float* x, int8_t* out, int code_offset, in
                LQ_ERR_VALUE, "quantize_nchw_to_packed4: grid [%d,%d] + offset %d does not fit int8", qmin, qmax,
                code_offset);
     LQ_REQUIRE(aligned16(out), LQ_ERR_VALUE, "quantize_nchw_to_packed4: out must be 16-byte aligned");
-    hipLaunchKernelGGL(quantize_nchw_to_packed4_kernel, dim3(grid_1d(size_t(B) * Hp * Wp)), dim3(256), 0,
-                       as_stream(stream), x, B, C, H, W, pad_h_lo, pad_w_lo, Hp, Wp, scale, zp, float(qmin), float(qmax),
-                       code_offset, fill_code, reinterpret_cast<uint32_t*>(out));
+    LQ_REQUIRE(Wp % 4 == 0 && B <= 65535 && (Hp + 3) / 4 <= 65535, LQ_ERR_SHAPE,
+               "quantize_nchw_to_packed4: packed rows must be a multiple of 4 pixels (Wp = %d); at most 65535 images", Wp);
+    hipLaunchKernelGGL(quantize_nchw_to_packed4_kernel, dim3(unsigned((Wp / 4 + 63) / 64), unsigned((Hp + 3) / 4), unsigned(B)),
+                       dim3(256), 0, as_stream(stream), x, B, C, H, W, pad_h_lo, pad_w_lo, Hp, Wp, scale, zp, float(qmin),
+                       float(qmax), code_offset, fill_code, reinterpret_cast<uint4*>(out));
     LQ_CHECK_LAUNCH("quantize_nchw_to_packed4");
     return LQ_OK;
 }
